@@ -1,0 +1,95 @@
+"""Seeded synthetic GGUF blocks, router matrices and activations.
+
+Every bit pattern is a valid IQ2_XXS / IQ3_S / Q6_K block (8-bit grid indices, 7-bit signs, 4-bit scales; 9-bit
+IQ3_S indices; int8 Q6_K scales), so a block is random bytes with its fp16 ``d`` field overwritten by a value drawn
+uniformly from a realistic range. The same seed gives the same bytes on every machine (numpy PCG64).
+"""
+import numpy as np
+
+TYPE_F32, TYPE_Q6_K, TYPE_IQ2_XXS, TYPE_IQ3_S = 0, 14, 16, 21
+BLOCK_BYTES = {TYPE_Q6_K: 210, TYPE_IQ2_XXS: 66, TYPE_IQ3_S: 110}
+D_OFFSET = {TYPE_Q6_K: 208, TYPE_IQ2_XXS: 0, TYPE_IQ3_S: 0}
+# default fp16 scale ranges: IQ formats as in the benchmark definition; Q6_K smaller because its integer part
+# (int8 scale x 6-bit quant) is ~70x larger
+D_RANGE = {TYPE_IQ2_XXS: (1e-3, 2e-2), TYPE_IQ3_S: (1e-3, 2e-2), TYPE_Q6_K: (1e-4, 5e-4)}
+
+
+def row_bytes(t, ncols):
+    if t == TYPE_F32:
+        return 4 * ncols
+    assert ncols % 256 == 0
+    return BLOCK_BYTES[t] * (ncols // 256)
+
+
+def quant_rows(rng, t, nrows, ncols, d_range=None):
+    """uint8 [nrows, row_bytes]: random-valid blocks of type t."""
+    bb = BLOCK_BYTES[t]
+    nb = nrows * (ncols // 256)
+    raw = rng.integers(0, 256, size=(nb, bb), dtype=np.uint8)
+    lo, hi = d_range or D_RANGE[t]
+    d = rng.uniform(lo, hi, size=nb).astype(np.float16).view(np.uint16)
+    raw[:, D_OFFSET[t]] = (d & 255).astype(np.uint8)
+    raw[:, D_OFFSET[t] + 1] = (d >> 8).astype(np.uint8)
+    return raw.reshape(nrows, -1)
+
+
+def normed_x(rng, ntok, hidden):
+    """x ~ N(0,1), RMS-normalised with eps 1e-6 (float32 [ntok, hidden])."""
+    x = rng.standard_normal((ntok, hidden)).astype(np.float32)
+    x = x / np.sqrt((x.astype(np.float64) ** 2).mean(axis=1, keepdims=True) + 1e-6)
+    return x.astype(np.float32)
+
+
+def layer_config(hidden=2048, ffn=512, n_expert=512, top_k=10, layout="iq2"):
+    """layout 'iq2': everything IQ2_XXS, F32 router. layout 'f2': gate/up IQ2_XXS, down IQ3_S, shared expert
+    and router Q6_K."""
+    cfg = dict(hidden=hidden, ffn=ffn, n_expert=n_expert, top_k=top_k)
+    if layout == "iq2":
+        cfg.update(router_type=TYPE_F32, gate_up_type=TYPE_IQ2_XXS, down_type=TYPE_IQ2_XXS,
+                   sh_gate_up_type=TYPE_IQ2_XXS, sh_down_type=TYPE_IQ2_XXS)
+    elif layout == "f2":
+        cfg.update(router_type=TYPE_Q6_K, gate_up_type=TYPE_IQ2_XXS, down_type=TYPE_IQ3_S,
+                   sh_gate_up_type=TYPE_Q6_K, sh_down_type=TYPE_Q6_K)
+    else:
+        raise ValueError(layout)
+    cfg["layout"] = layout
+    return cfg
+
+
+def make_layer(seed, cfg):
+    """dict of numpy arrays holding one MoE layer in raw GGUF block layout (expert-major)."""
+    rng = np.random.default_rng(seed)
+    H, F, E = cfg["hidden"], cfg["ffn"], cfg["n_expert"]
+    out = {}
+    if cfg["router_type"] == TYPE_F32:
+        out["router"] = (0.02 * rng.standard_normal((E, H))).astype(np.float32)
+    else:
+        # fp16-subnormal d keeps Q6_K router logits O(1); real files use subnormal d too
+        out["router"] = quant_rows(rng, cfg["router_type"], E, H, d_range=(1e-5, 3e-5))
+    out["gate"] = quant_rows(rng, cfg["gate_up_type"], E * F, H).reshape(E, -1)
+    out["up"] = quant_rows(rng, cfg["gate_up_type"], E * F, H).reshape(E, -1)
+    out["down"] = quant_rows(rng, cfg["down_type"], E * H, F).reshape(E, -1)
+    out["sh_gate"] = quant_rows(rng, cfg["sh_gate_up_type"], F, H)
+    out["sh_up"] = quant_rows(rng, cfg["sh_gate_up_type"], F, H)
+    out["sh_down"] = quant_rows(rng, cfg["sh_down_type"], H, F)
+    out["sh_gate_inp"] = (0.02 * rng.standard_normal(H)).astype(np.float32)
+    return out
+
+
+def hot_logits(rng, ntok, n_expert, n_hot=32, bias=2.0):
+    """Router logits N(0,1) with a bias on a fixed set of hot experts (tokens overlap in their experts)."""
+    l = rng.standard_normal((ntok, n_expert)).astype(np.float32)
+    hot = (np.arange(n_hot) * 37) % n_expert
+    l[:, hot] += np.float32(bias)
+    return l
+
+
+def zipf_topk(rng, ntok, n_expert, top_k, s=1.1):
+    """Per token, top_k distinct experts drawn without replacement from a Zipf(s) popularity."""
+    p = 1.0 / np.arange(1, n_expert + 1) ** s
+    p /= p.sum()
+    perm = rng.permutation(n_expert)
+    ids = np.empty((ntok, top_k), np.uint32)
+    for t in range(ntok):
+        ids[t] = perm[rng.choice(n_expert, size=top_k, replace=False, p=p)]
+    return ids

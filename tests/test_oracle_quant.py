@@ -1,0 +1,178 @@
+"""The CPU oracle against the reference's golden vectors and known answers (no GPU).
+
+Golden fixtures come from the reference's own C (tests/golden/make_golden.c). Known answers are the ones in
+the reference's model-free tests: native/redlite_native_shared_exec_offline_test.c:18-55,
+native/redlite_native_quant_cpu.c:364-393, tests/test_redmetal.py:25-29.
+"""
+import json
+import os
+import struct
+
+import numpy as np
+import pytest
+
+import oracle_lib as orc
+
+T_F32, T_Q6K, T_IQ2, T_IQ3 = 0, 14, 16, 21
+
+
+def unhex(s, dtype):
+    return np.frombuffer(bytes.fromhex(s), dtype=dtype).copy()
+
+
+def test_f16_exhaustive(golden_dir):
+    g = json.load(open(os.path.join(golden_dir, "f16.json")))
+    mine = np.empty(65536, np.float32)
+    orc.lib().orc_f16_all(mine.ctypes.data_as(orc.C.c_void_p))
+    assert "%08x" % orc.lib().orc_crc32(mine.ctypes.data, mine.nbytes) == g["crc32_of_f32_le"]
+    for k, v in g["spot"].items():
+        assert "%08x" % mine[int(k, 16)].view(np.uint32) == v
+    # independent of the reference: numpy's IEEE half conversion, all non-NaN patterns
+    ref = np.arange(65536, dtype=np.uint16).view(np.float16).astype(np.float32)
+    ok = ~np.isnan(ref)
+    assert np.array_equal(mine[ok].view(np.uint32), ref[ok].view(np.uint32))
+    assert mine[1] == 2.0 ** -24
+
+
+def test_codebooks():
+    L = orc.lib()
+    g2 = np.ctypeslib.as_array(L.orc_iq2xxs_grid(), (2048,))
+    g3 = np.ctypeslib.as_array(L.orc_iq3s_grid(), (512,))
+    assert "%08x" % L.orc_crc32(g2.ctypes.data, 2048) == "9924ff02"
+    assert "%08x" % L.orc_crc32(g3.ctypes.data, 2048) == "f576e4f3"
+    assert set(np.unique(g2)) == {8, 25, 43}
+    assert list(g2[:8]) == [8] * 8 and list(g2[8:16]) == [43] + [8] * 7
+    assert list(g2[255 * 8:]) == [8, 25, 8, 8, 25, 43, 43, 43]
+    # spot values the reference's IQ3 selftest checks (native/redlite_native_iq3.c:398)
+    assert g3[0] == 0x01010101 and g3[511] == 0x0f0f0101 and g3[1] == 0x01010103 and g3[256] == 0x05090507
+    b = g3.view(np.uint8)
+    assert np.all(b % 2 == 1) and b.max() == 15 and b.min() == 1
+
+
+def test_row_sizes():
+    assert orc.row_bytes(T_Q6K, 256) == 210 and orc.row_bytes(T_IQ2, 256) == 66 and orc.row_bytes(T_IQ3, 2048) == 880
+    assert orc.row_bytes(T_IQ2, 2048) == 528 and orc.row_bytes(T_IQ2, 512) == 132 and orc.row_bytes(T_F32, 2048) == 8192
+    assert orc.row_bytes(T_IQ2, 100) == 0 and orc.row_bytes(17, 256) == 0
+
+
+def test_golden_rows(golden_dir):
+    g = json.load(open(os.path.join(golden_dir, "quant_rows.json")))
+    seen = set()
+    for c in g["cases"]:
+        t, n = c["type"], c["ncols"]
+        row = unhex(c["row"], np.uint8)
+        x = unhex(c["x"], np.float32)
+        want = struct.unpack("<d", bytes.fromhex(c["dot"]))[0]
+        got = orc.row_dot(t, row, x)
+        assert got == want, (t, n, c["fill"], got, want)          # same order of double operations: bit-equal
+        if t != T_F32:
+            w = orc.dequant_rows(t, row, n)[0]
+            assert np.array_equal(w.view(np.uint32), unhex(c["dequant"], np.uint32)), (t, n, c["fill"])
+            assert "%08x" % orc.lib().orc_crc32(w.ctypes.data, w.nbytes) == c["dequant_crc32"]
+            # the digest check of the reference's offline test: double dot of the dequantised row agrees
+            brute = float(np.dot(w.astype(np.float64), x.astype(np.float64)))
+            assert abs(brute - want) <= 1e-9 * max(1.0, np.abs(w.astype(np.float64) * x).sum())
+        if "dot_d" in c:
+            xd = unhex(c["xd"], np.float64)
+            assert orc.row_dot(t, row, xd) == struct.unpack("<d", bytes.fromhex(c["dot_d"]))[0]
+        seen.add((t, c["fill"]))
+    assert {(16, 0), (21, 0), (14, 0), (0, 0), (16, 3), (21, 3), (14, 3)} <= seen
+
+
+def test_appendix_rows():
+    """Two-block rows with formula bytes; expected values were produced by the compiled reference."""
+    want = {
+        T_IQ2: ("d10d4eca", "877d1af2", -12.7415771484375, [-0.923828125, 0.923828125, 0.537109375, -0.537109375], -1.25976562, 0.421875),
+        T_IQ3: ("99a6997b", "30688e0b", 8.427734375, [-1.265625, 3.796875, -5.484375, -2.953125], 3.515625, -1.421875),
+        T_Q6K: ("9c223205", "47004699", 484.328125, [-22.359375, 26.5, 9.109375, -8.28125], -0.9375, -28.4375),
+    }
+    x = np.array([((i * 7 + 3) % 31 - 15) / 16.0 for i in range(512)], np.float32)
+    for t, (crc_row, crc_w, dot, w03, w255, w511) in want.items():
+        bb = orc.lib().orc_block_bytes(t)
+        row = np.zeros(2 * bb, np.uint8)
+        for b in range(2):
+            for i in range(bb):
+                row[b * bb + i] = (i * 37 + 11 + b * 101) & 255
+            off = 208 if t == T_Q6K else 0
+            row[b * bb + off], row[b * bb + off + 1] = 0x00, 0x24
+        assert "%08x" % orc.lib().orc_crc32(row.ctypes.data, row.nbytes) == crc_row
+        w = orc.dequant_rows(t, row, 512)[0]
+        assert "%08x" % orc.lib().orc_crc32(w.ctypes.data, w.nbytes) == crc_w
+        assert list(w[:4]) == w03 and abs(w[255] - w255) < 1e-7 and w[511] == w511
+        assert orc.row_dot(t, row, x) == dot
+
+
+def test_known_answer_blocks():
+    ones = np.ones(256, np.float32)
+    q6 = np.zeros(210, np.uint8)
+    q6[:128] = 0x11
+    q6[128:192] = 0xAA
+    q6[192:208] = 1
+    q6[208], q6[209] = 0x00, 0x3C
+    assert orc.row_dot(T_Q6K, q6, ones) == 256.0
+    assert np.all(orc.dequant_rows(T_Q6K, q6, 256) == 1.0)
+    q6[208], q6[209] = 0x01, 0x00                      # smallest fp16 subnormal
+    assert abs(orc.row_dot(T_Q6K, q6, ones) - 2.0 ** -16) < 1e-12
+    q6z = np.zeros(210, np.uint8)
+    q6z[192:208] = 1
+    q6z[209] = 0x3C
+    assert orc.row_dot(T_Q6K, q6z, ones) == -8192.0
+    assert np.all(orc.dequant_rows(T_Q6K, q6z, 256) == -32.0)
+    iq2 = np.zeros(66, np.uint8)
+    iq2[1] = 0x3C
+    assert orc.row_dot(T_IQ2, iq2, ones) == 256.0
+    x = np.array([((i * 17 + 3) % 61 - 30) / 32.0 for i in range(256)], np.float32)
+    assert abs(orc.row_dot(T_IQ2, iq2, x) - float(x.astype(np.float64).sum())) < 1e-9
+
+
+def test_iq2xxs_sign_parity_and_exactness():
+    rng = np.random.default_rng(5)
+    from dwarfstar_red_lite_amd import synth
+    rows = synth.quant_rows(rng, T_IQ2, 8, 512)
+    w = orc.dequant_rows(T_IQ2, rows, 512)
+    neg = (w < 0).reshape(8, 64, 8).sum(axis=2)
+    assert np.all(neg % 2 == 0)                         # each group of 8 holds an even number of minus signs
+    mags = np.abs(w).reshape(8, 2, 8, 32)
+    # |w| / db must be a grid magnitude: ratios within one 32-group are ratios of {8,25,43}
+    r = mags / mags.min(axis=3, keepdims=True)
+    allowed = np.array([1.0, 25 / 8, 43 / 8, 43 / 25, 25 / 25])
+    assert np.all(np.min(np.abs(r[..., None] - allowed), axis=-1) < 1e-6)
+
+
+def _py_iq3s_block(bp, grid):
+    """independent pure-python decoder of one IQ3_S block from the published ggml layout"""
+    d = np.frombuffer(bytes(bp[:2]), np.float16)[0].astype(np.float32)
+    qs, qh, signs, scales = bp[2:66], bp[66:74], bp[74:106], bp[106:110]
+    y = np.zeros(256, np.float32)
+    for ib32 in range(8):
+        nib = (int(scales[ib32 // 2]) >> (4 * (ib32 % 2))) & 15
+        db = np.float32(d * np.float32(1 + 2 * nib))
+        for l in range(4):
+            for half in range(2):
+                idx = int(qs[8 * ib32 + 2 * l + half]) | (((int(qh[ib32]) >> (2 * l + half)) & 1) << 8)
+                word = int(grid[idx])
+                for j in range(4):
+                    s = -1.0 if (int(signs[4 * ib32 + l]) >> (4 * half + j)) & 1 else 1.0
+                    y[32 * ib32 + 8 * l + 4 * half + j] = np.float32(db * np.float32((word >> (8 * j)) & 255)) * np.float32(s)
+    return y
+
+
+def test_iq3s_against_independent_decoder():
+    from dwarfstar_red_lite_amd import synth
+    rng = np.random.default_rng(9)
+    grid = np.ctypeslib.as_array(orc.lib().orc_iq3s_grid(), (512,))
+    rows = synth.quant_rows(rng, T_IQ3, 3, 256)
+    for r in rows:
+        assert np.array_equal(orc.dequant_rows(T_IQ3, r, 256)[0], _py_iq3s_block(r, grid))
+
+
+def test_matvec_threads_identical():
+    from dwarfstar_red_lite_amd import synth
+    rng = np.random.default_rng(2)
+    w = synth.quant_rows(rng, T_IQ2, 96, 512)
+    x = rng.standard_normal(512).astype(np.float32)
+    a = orc.matvec(T_IQ2, w, 512, x, threads=1)
+    b = orc.matvec(T_IQ2, w, 512, x, threads=5)
+    c = orc.matvec(T_IQ2, w, 512, x, row_start=10, row_count=20, threads=3)
+    assert np.array_equal(a, b) and np.array_equal(a[10:30], c)
+    assert a[7] == np.float32(orc.row_dot(T_IQ2, w[7], x))
