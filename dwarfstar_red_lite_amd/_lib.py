@@ -1,0 +1,86 @@
+"""Loads libredmetal_hip.so and declares the C ABI (include/*.h). There is no fallback: without the built HIP
+library every entry point of this package raises."""
+import ctypes as C
+import os
+
+HERE = os.path.dirname(os.path.abspath(__file__))
+LIB_PATH = os.path.join(HERE, "libredmetal_hip.so")
+
+
+class RedHipError(RuntimeError):
+    pass
+
+
+class RouterTensorInfo(C.Structure):      # include/redmetal_router.h
+    _fields_ = [("layer", C.c_uint32), ("ggml_type", C.c_uint32), ("n_dims", C.c_uint32), ("shape", C.c_uint64 * 8),
+                ("tensor_offset", C.c_uint64), ("tensor_span_bytes", C.c_uint64)]
+
+
+class RouterTelemetry(C.Structure):
+    _fields_ = [("read_ms", C.c_double), ("compute_ms", C.c_double)]
+
+
+class MoeConfig(C.Structure):             # include/redhip_moe.h
+    _fields_ = [(n, C.c_uint32) for n in ("hidden", "ffn", "n_expert", "top_k", "n_layer", "max_tokens", "router_type",
+                                          "expert_type_word", "shared_type_word", "reserved")]
+
+
+# every symbol the headers declare: name -> (restype, argtypes)
+u32, u64, vp, dbl, i32 = C.c_uint32, C.c_uint64, C.c_void_p, C.c_double, C.c_int
+ABI = {
+    "redmetal_ffn_abi_version": (u32, []),
+    "redmetal_ffn_last_error": (C.c_char_p, []),
+    "redmetal_ffn_pool_create": (vp, [C.c_char_p, u64, u64, u32, vp, u32, vp, u32]),
+    "redmetal_ffn_pool_destroy": (None, [vp]),
+    "redmetal_ffn_pool_capacity": (u32, [vp]),
+    "redmetal_ffn_pool_slab_count": (u32, [vp]),
+    "redmetal_ffn_pool_allocated_bytes": (u64, [vp]),
+    "redmetal_ffn_pool_bytes_read": (u64, [vp]),
+    "redmetal_ffn_pool_read_calls": (u64, [vp]),
+    "redmetal_ffn_pool_read_ms": (dbl, [vp]),
+    "redmetal_ffn_pool_slot_inflight": (i32, [vp, u32]),
+    "redmetal_ffn_pool_load_expert": (i32, [vp, u32, u64, u64, u64, u64, u64, u64, C.POINTER(u64), C.POINTER(dbl)]),
+    "redmetal_ffn_pool_slot_addresses": (i32, [vp, u32, u64, u64, u64, C.POINTER(u64), C.POINTER(u64), C.POINTER(u64)]),
+    "redmetal_ffn_pool_execute_expert": (i32, [vp, u32, u32, u64, u64, u64, u32, u32, u32, u32, vp, u32, vp, u32, C.POINTER(dbl)]),
+    "redmetal_quant_abi_version": (u32, []),
+    "redmetal_quant_last_error": (C.c_char_p, []),
+    "redmetal_quant_rows": (i32, [C.c_char_p, u64, u64, u32, u32, u32, u32, u32, vp, u32, vp, u32, vp, u32, C.POINTER(dbl), C.POINTER(dbl)]),
+    "rl_native_router_gpu_f32": (i32, [C.c_char_p, C.POINTER(RouterTensorInfo), vp, u32, vp, u32, C.POINTER(RouterTelemetry), C.c_char_p, C.c_size_t]),
+    "rl_native_router_select_softmax_topk": (i32, [vp, u32, u32, vp, vp, vp, C.c_char_p, C.c_size_t]),
+    "redhip_moe_abi_version": (u32, []),
+    "redhip_moe_last_error": (C.c_char_p, []),
+    "redhip_moe_create": (vp, [C.POINTER(MoeConfig)]),
+    "redhip_moe_destroy": (None, [vp]),
+    "redhip_moe_resident_bytes": (u64, [vp]),
+    "redhip_moe_load_router": (i32, [vp, u32, vp, u64]),
+    "redhip_moe_load_shared": (i32, [vp, u32, vp, vp, u64, vp, u64, vp, u64]),
+    "redhip_moe_load_experts": (i32, [vp, u32, u32, u32, vp, vp, vp]),
+    "redhip_moe_forward": (i32, [vp, u32, vp, u32, vp, vp]),
+    "redhip_moe_route": (i32, [vp, u32, vp, u32, vp, vp, vp, vp]),
+    "redhip_moe_experts": (i32, [vp, u32, vp, u32, vp, vp, vp, vp]),
+    "redhip_moe_last_route": (i32, [vp, u32, vp, vp, vp, vp]),
+    "redhip_moe_group": (i32, [vp, vp, vp, u32, vp, vp, vp, vp, vp, vp, vp]),
+    "redhip_dequant_rows": (i32, [u32, vp, u32, u32, vp, vp]),
+    "redhip_moe_dequant_resident": (i32, [vp, u32, u32, u32, vp, vp]),
+    "redhip_gemv_rows": (i32, [u32, vp, u32, u32, u32, vp, vp, vp]),
+}
+
+_lib = None
+
+
+def load():
+    """The shared library with argtypes set. Raises RedHipError when it has not been built."""
+    global _lib
+    if _lib is None:
+        if not os.path.isfile(LIB_PATH):
+            raise RedHipError("HIP library not found at %s: run `python -m dwarfstar_red_lite_amd.build`" % LIB_PATH)
+        lib = C.CDLL(LIB_PATH)
+        for name, (res, args) in ABI.items():
+            fn = getattr(lib, name)          # AttributeError here = header/library mismatch
+            fn.restype = res
+            fn.argtypes = args
+        for fam in ("redmetal_ffn", "redmetal_quant", "redhip_moe"):
+            if getattr(lib, fam + "_abi_version")() != 1:
+                raise RedHipError("unsupported %s ABI version" % fam)
+        _lib = lib
+    return _lib

@@ -1,0 +1,62 @@
+// Internal interface between the C-ABI front ends and the gfx950 kernels of libredmetal_hip.so.
+#pragma once
+#include <hip/hip_runtime.h>
+#include <stddef.h>
+#include <stdint.h>
+
+namespace redhip {
+
+enum : uint32_t { T_F32 = 0u, T_Q6_K = 14u, T_IQ2_XXS = 16u, T_IQ3_S = 21u };
+
+// bytes per 256 weights; 0 for a type this library does not decode
+inline uint32_t block_bytes(uint32_t t) { return t == T_Q6_K ? 210u : t == T_IQ2_XXS ? 66u : t == T_IQ3_S ? 110u : 0u; }
+inline uint64_t row_bytes(uint32_t t, uint32_t ncols) {
+    if (!ncols) return 0;
+    if (t == T_F32) return 4ull * ncols;
+    const uint32_t b = block_bytes(t);
+    return (b && ncols % 256u == 0u) ? (uint64_t)(ncols / 256u) * b : 0ull;
+}
+inline bool quant_supported(uint32_t t) { return block_bytes(t) != 0u; }
+// the reference's two-type word: gate/up in bits 0-7, down in bits 8-15 when it differs
+inline uint32_t word_gate_up(uint32_t w) { return w & 255u; }
+inline uint32_t word_down(uint32_t w) { return ((w >> 8) & 255u) ? ((w >> 8) & 255u) : (w & 255u); }
+
+// ---- launchers (enqueue only; return hipSuccess or the launch error) ----
+
+hipError_t launch_dequant_rows(uint32_t type, const void *rows, uint32_t nrows, uint32_t ncols, float *out, hipStream_t s);
+
+// out[r] = W[row_start + r] . x for r < row_count; raw GGUF rows
+hipError_t launch_gemv_rows(uint32_t type, const void *w, uint32_t ncols, uint32_t row_start, uint32_t row_count,
+                            const float *x, float *out, hipStream_t s);
+
+// act[i] = SiLU(gate[i]) * up[i]
+hipError_t launch_silu_mul(const float *gate, const float *up, float *act, uint32_t n, hipStream_t s);
+
+// per token: softmax over n_expert logits, top_k by probability (ties to lower index), renormalised weights;
+// optional probs [ntok][n_expert]; optional shared scalar gate sigmoid(gate_inp . x_t) -> scalar[t]
+hipError_t launch_route_select(const float *logits, uint32_t ntok, uint32_t n_expert, uint32_t top_k,
+                               uint32_t *ids, float *weights, float *probs,
+                               const float *gate_inp, const float *x, uint32_t hidden, float *scalar, hipStream_t s);
+
+struct ExpertSet {               // where the experts of one layer live (raw GGUF layout, gate|up|down per expert)
+    const uint8_t *base;         // expert e starts at base + e * stride
+    uint64_t stride;
+    uint64_t gate_bytes, up_bytes;
+    uint32_t gate_up_type, down_type;
+};
+
+// act[slot][r] = SiLU(gate_e[r] . x) * (up_e[r] . x) for slot < n_slot, e = ids ? ids[slot] : slot
+hipError_t launch_moe_gateup(const ExpertSet &ex, const uint32_t *ids, uint32_t n_slot, uint32_t hidden, uint32_t ffn,
+                             const float *x, float *act, hipStream_t s);
+
+// out[r] = sum_k weights[k] * (down_{ids[k]}[r] . act[k]) + scalar[0] * (shared_down[r] . shared_act), k in selection order
+hipError_t launch_moe_down_combine(const ExpertSet &ex, const uint32_t *ids, const float *weights, uint32_t top_k,
+                                   const ExpertSet &shared, const float *scalar, uint32_t hidden, uint32_t ffn,
+                                   const float *act, const float *shared_act, float *out, hipStream_t s);
+
+// pair sort of [ntok][top_k] ids: see redhip_moe_group in include/redhip_moe.h
+hipError_t launch_group_pairs(const uint32_t *ids, const float *weights, uint32_t ntok, uint32_t top_k, uint32_t n_expert,
+                              uint32_t *uid, uint32_t *expert_start, uint32_t *pair_token, float *pair_weight,
+                              uint32_t *tok_pair, uint32_t *n_unique, hipStream_t s);
+
+}  // namespace redhip

@@ -1,0 +1,469 @@
+// gfx950 kernels over raw GGUF rows: dequantisation, GEMV, router selection, token grouping, and the
+// single-token expert FFN (gate/up/SwiGLU, then down fused with the weighted combine and the shared expert).
+// Wavefronts are 64 wide; a row is split over LPR lanes (8..64), each lane taking 32-weight chunks, and the
+// partial sums meet in a butterfly of cross-lane shuffles.
+#include "redhip_decode.h"
+
+namespace redhip {
+
+__device__ uint64_t g_iq2xxs_grid[256];
+__device__ uint32_t g_iq3s_grid[512];
+
+static hipError_t ensure_tables() {
+    static hipError_t state = hipErrorNotInitialized;
+    static int device_done[64] = {0};
+    int dev = 0;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return e;
+    if (dev >= 0 && dev < 64 && device_done[dev]) return hipSuccess;
+    e = hipMemcpyToSymbol(HIP_SYMBOL(g_iq2xxs_grid), redhip_iq2xxs_grid, sizeof(redhip_iq2xxs_grid));
+    if (e == hipSuccess) e = hipMemcpyToSymbol(HIP_SYMBOL(g_iq3s_grid), redhip_iq3s_grid, sizeof(redhip_iq3s_grid));
+    if (e == hipSuccess && dev >= 0 && dev < 64) device_done[dev] = 1;
+    state = e;
+    return state;
+}
+
+static inline uint32_t lanes_per_row(uint32_t ncols) {
+    const uint32_t chunks = ncols / 32u;
+    return chunks >= 64u ? 64u : chunks >= 32u ? 32u : chunks >= 16u ? 16u : 8u;
+}
+// x staged in LDS with one pad word per 32 floats, so lanes that walk different chunks hit different banks
+__device__ __forceinline__ uint32_t pad32(uint32_t i) { return i + (i >> 5); }
+static inline uint32_t padded_floats(uint32_t n) { return n + (n >> 5); }
+
+template <uint32_t T>
+__device__ __forceinline__ float chunk_dot(const uint8_t *row, uint32_t chunk, const float *x33) {
+    float w[32];
+    decode32<T>(row, chunk, w);
+    float acc = 0.0f;
+#pragma unroll
+    for (int j = 0; j < 32; ++j) acc = fmaf(w[j], x33[j], acc);
+    return acc;
+}
+
+template <int LPR> __device__ __forceinline__ float sub_reduce(float v) {
+#pragma unroll
+    for (int o = LPR / 2; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+
+// ---------------------------------------------------------------- dequantisation (parity tap)
+
+template <uint32_t T>
+__global__ __launch_bounds__(256) void dequant_rows_kernel(const uint8_t *rows, uint64_t rb, uint32_t nrows, uint32_t chunks_per_row, float *out) {
+    const uint64_t gid = (uint64_t)blockIdx.x * 256u + threadIdx.x;
+    if (gid >= (uint64_t)nrows * chunks_per_row) return;
+    const uint32_t r = (uint32_t)(gid / chunks_per_row), c = (uint32_t)(gid % chunks_per_row);
+    float w[32];
+    decode32<T>(rows + (uint64_t)r * rb, c, w);
+    float4 *o = reinterpret_cast<float4 *>(out + ((uint64_t)r * chunks_per_row + c) * 32u);
+#pragma unroll
+    for (int i = 0; i < 8; ++i) o[i] = make_float4(w[4 * i], w[4 * i + 1], w[4 * i + 2], w[4 * i + 3]);
+}
+
+hipError_t launch_dequant_rows(uint32_t type, const void *rows, uint32_t nrows, uint32_t ncols, float *out, hipStream_t s) {
+    hipError_t e = ensure_tables();
+    if (e != hipSuccess) return e;
+    const uint64_t rb = row_bytes(type, ncols);
+    if (!rb || ncols % 32u || !nrows) return hipErrorInvalidValue;
+    const uint32_t cpr = ncols / 32u;
+    const uint64_t total = (uint64_t)nrows * cpr;
+    const dim3 grid((uint32_t)((total + 255u) / 256u));
+    const uint8_t *p = static_cast<const uint8_t *>(rows);
+    switch (type) {
+        case T_IQ2_XXS: dequant_rows_kernel<T_IQ2_XXS><<<grid, 256, 0, s>>>(p, rb, nrows, cpr, out); break;
+        case T_IQ3_S: dequant_rows_kernel<T_IQ3_S><<<grid, 256, 0, s>>>(p, rb, nrows, cpr, out); break;
+        case T_Q6_K: dequant_rows_kernel<T_Q6_K><<<grid, 256, 0, s>>>(p, rb, nrows, cpr, out); break;
+        case T_F32: dequant_rows_kernel<T_F32><<<grid, 256, 0, s>>>(p, rb, nrows, cpr, out); break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------- GEMV over raw rows
+
+template <uint32_t T, int LPR>
+__global__ __launch_bounds__(256) void gemv_rows_kernel(const uint8_t *w, uint64_t rb, uint32_t ncols, uint32_t row_start,
+                                                        uint32_t row_count, const float *x, float *out) {
+    extern __shared__ float xs[];
+    for (uint32_t i = threadIdx.x; i < ncols; i += 256u) xs[pad32(i)] = x[i];
+    __syncthreads();
+    const uint32_t sub = threadIdx.x % LPR, r = blockIdx.x * (256u / LPR) + threadIdx.x / LPR;
+    float acc = 0.0f;
+    if (r < row_count) {
+        const uint8_t *row = w + (uint64_t)(row_start + r) * rb;
+        for (uint32_t c = sub; c < ncols / 32u; c += LPR) acc += chunk_dot<T>(row, c, xs + 33u * c);
+    }
+    acc = sub_reduce<LPR>(acc);
+    if (sub == 0u && r < row_count) out[r] = acc;
+}
+
+template <uint32_t T>
+static hipError_t gemv_dispatch(const uint8_t *w, uint32_t ncols, uint32_t row_start, uint32_t row_count, const float *x, float *out, hipStream_t s) {
+    const uint64_t rb = row_bytes(T, ncols);
+    const uint32_t lpr = lanes_per_row(ncols);
+    const dim3 grid((row_count + 256u / lpr - 1u) / (256u / lpr));
+    const size_t lds = padded_floats(ncols) * sizeof(float);
+    switch (lpr) {
+        case 64: gemv_rows_kernel<T, 64><<<grid, 256, lds, s>>>(w, rb, ncols, row_start, row_count, x, out); break;
+        case 32: gemv_rows_kernel<T, 32><<<grid, 256, lds, s>>>(w, rb, ncols, row_start, row_count, x, out); break;
+        case 16: gemv_rows_kernel<T, 16><<<grid, 256, lds, s>>>(w, rb, ncols, row_start, row_count, x, out); break;
+        default: gemv_rows_kernel<T, 8><<<grid, 256, lds, s>>>(w, rb, ncols, row_start, row_count, x, out); break;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_gemv_rows(uint32_t type, const void *w, uint32_t ncols, uint32_t row_start, uint32_t row_count,
+                            const float *x, float *out, hipStream_t s) {
+    hipError_t e = ensure_tables();
+    if (e != hipSuccess) return e;
+    if (!row_bytes(type, ncols) || ncols % 256u || !row_count || padded_floats(ncols) * 4u > 160u * 1024u) return hipErrorInvalidValue;
+    const uint8_t *p = static_cast<const uint8_t *>(w);
+    switch (type) {
+        case T_IQ2_XXS: return gemv_dispatch<T_IQ2_XXS>(p, ncols, row_start, row_count, x, out, s);
+        case T_IQ3_S: return gemv_dispatch<T_IQ3_S>(p, ncols, row_start, row_count, x, out, s);
+        case T_Q6_K: return gemv_dispatch<T_Q6_K>(p, ncols, row_start, row_count, x, out, s);
+        case T_F32: return gemv_dispatch<T_F32>(p, ncols, row_start, row_count, x, out, s);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+// ---------------------------------------------------------------- SwiGLU
+
+__device__ __forceinline__ float silu_mul(float g, float u) { return (g / (1.0f + expf(-g))) * u; }
+
+__global__ void silu_mul_kernel(const float *gate, const float *up, float *act, uint32_t n) {
+    const uint32_t i = blockIdx.x * blockDim.x + threadIdx.x;
+    if (i < n) act[i] = silu_mul(gate[i], up[i]);
+}
+
+hipError_t launch_silu_mul(const float *gate, const float *up, float *act, uint32_t n, hipStream_t s) {
+    silu_mul_kernel<<<(n + 255u) / 256u, 256, 0, s>>>(gate, up, act, n);
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------- router selection
+
+// One workgroup of 256 lanes per token. Probabilities are formed exactly as the reference does
+// (expf(l - max), double sum, one float reciprocal), selection is on the probabilities with ties to the lower
+// index, and the k selected weights are renormalised with a double sum taken in selection order.
+__global__ __launch_bounds__(256) void route_select_kernel(const float *logits, uint32_t n_expert, uint32_t top_k,
+                                                           uint32_t *ids, float *weights, float *probs,
+                                                           const float *gate_inp, const float *x, uint32_t hidden, float *scalar) {
+    __shared__ float p[1024];
+    __shared__ float red_f[4];
+    __shared__ double red_d[4];
+    __shared__ uint32_t red_i[4];
+    __shared__ float sel_p[16];
+    __shared__ uint32_t sel_i[16];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, wave = tid >> 6, tok = blockIdx.x;
+    const float *l = logits + (uint64_t)tok * n_expert;
+
+    float m = -INFINITY;
+    for (uint32_t i = tid; i < n_expert; i += 256u) m = fmaxf(m, l[i]);
+    for (int o = 32; o > 0; o >>= 1) m = fmaxf(m, __shfl_xor(m, o, 64));
+    if (lane == 0u) red_f[wave] = m;
+    __syncthreads();
+    m = fmaxf(fmaxf(red_f[0], red_f[1]), fmaxf(red_f[2], red_f[3]));
+
+    double part = 0.0;
+    for (uint32_t i = tid; i < n_expert; i += 256u) {
+        const float e = expf(l[i] - m);
+        p[i] = e;
+        part += (double)e;
+    }
+    for (int o = 32; o > 0; o >>= 1) part += __shfl_xor(part, o, 64);
+    if (lane == 0u) red_d[wave] = part;
+    __syncthreads();
+    const double denom = (red_d[0] + red_d[1]) + (red_d[2] + red_d[3]);
+    const bool bad = !(denom > 0.0) || isinf(denom) || isnan(denom);
+    const float inv = bad ? 0.0f : (float)(1.0 / denom);
+    for (uint32_t i = tid; i < n_expert; i += 256u) {
+        const float v = p[i] * inv;
+        p[i] = v;
+        if (probs) probs[(uint64_t)tok * n_expert + i] = v;
+    }
+    __syncthreads();
+
+    for (uint32_t k = 0; k < top_k; ++k) {
+        float bp = -INFINITY;
+        uint32_t bi = 0xffffffffu;
+        for (uint32_t i = tid; i < n_expert; i += 256u) {
+            const float v = p[i];                       // taken entries hold -1
+            if (v >= 0.0f && (v > bp || (v == bp && i < bi))) { bp = v; bi = i; }
+        }
+        for (int o = 32; o > 0; o >>= 1) {
+            const float op = __shfl_xor(bp, o, 64);
+            const uint32_t oi = __shfl_xor(bi, o, 64);
+            if (oi != 0xffffffffu && (bi == 0xffffffffu || op > bp || (op == bp && oi < bi))) { bp = op; bi = oi; }
+        }
+        if (lane == 0u) { red_f[wave] = bp; red_i[wave] = bi; }
+        __syncthreads();
+        if (tid == 0u) {
+            float fp = red_f[0];
+            uint32_t fi = red_i[0];
+            for (int w = 1; w < 4; ++w) {
+                const float op = red_f[w];
+                const uint32_t oi = red_i[w];
+                if (oi != 0xffffffffu && (fi == 0xffffffffu || op > fp || (op == fp && oi < fi))) { fp = op; fi = oi; }
+            }
+            if (fi == 0xffffffffu) { fi = k; fp = 0.0f; }      // only when every probability is NaN: keep ids in range
+            sel_p[k] = fp;
+            sel_i[k] = fi;
+            p[fi] = -1.0f;
+        }
+        __syncthreads();
+    }
+    if (tid == 0u) {
+        double sum = 0.0;
+        for (uint32_t k = 0; k < top_k; ++k) sum += (double)sel_p[k];
+        const bool bad2 = bad || !(sum > 0.0) || isinf(sum) || isnan(sum);
+        const float invs = bad2 ? __uint_as_float(0x7fc00000u) : (float)(1.0 / sum);
+        for (uint32_t k = 0; k < top_k; ++k) {
+            ids[(uint64_t)tok * top_k + k] = sel_i[k];
+            weights[(uint64_t)tok * top_k + k] = sel_p[k] * invs;      // NaN weights flag an invalid softmax
+        }
+    }
+    if (scalar) {                                        // shared-expert scalar gate sigmoid(gate_inp . x_t)
+        const float *xt = x + (uint64_t)tok * hidden;
+        double acc = 0.0;
+        for (uint32_t i = tid; i < hidden; i += 256u) acc += (double)gate_inp[i] * (double)xt[i];
+        for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+        __syncthreads();
+        if (lane == 0u) red_d[wave] = acc;
+        __syncthreads();
+        if (tid == 0u) {
+            const double z = (red_d[0] + red_d[1]) + (red_d[2] + red_d[3]);
+            scalar[tok] = (float)(1.0 / (1.0 + exp(-z)));
+        }
+    }
+}
+
+hipError_t launch_route_select(const float *logits, uint32_t ntok, uint32_t n_expert, uint32_t top_k,
+                               uint32_t *ids, float *weights, float *probs,
+                               const float *gate_inp, const float *x, uint32_t hidden, float *scalar, hipStream_t s) {
+    if (!ntok || !n_expert || n_expert > 1024u || !top_k || top_k > 16u || top_k > n_expert) return hipErrorInvalidValue;
+    if (scalar && (!gate_inp || !x)) return hipErrorInvalidValue;
+    route_select_kernel<<<ntok, 256, 0, s>>>(logits, n_expert, top_k, ids, weights, probs, gate_inp, x, hidden, scalar);
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------- single-token expert FFN
+
+template <uint32_t T, int LPR>
+__global__ __launch_bounds__(256) void moe_gateup_kernel(const uint8_t *base, uint64_t stride, uint64_t gate_bytes,
+                                                         const uint32_t *ids, uint32_t hidden, uint32_t ffn,
+                                                         const float *x, float *act) {
+    extern __shared__ float xs[];
+    for (uint32_t i = threadIdx.x; i < hidden; i += 256u) xs[pad32(i)] = x[i];
+    __syncthreads();
+    const uint32_t slot = blockIdx.y, e = ids ? ids[slot] : slot;
+    const uint32_t sub = threadIdx.x % LPR, r = blockIdx.x * (256u / LPR) + threadIdx.x / LPR;
+    const uint64_t rb = (uint64_t)(hidden / 256u) * Fmt<T>::kBlock;
+    float g = 0.0f, u = 0.0f;
+    if (r < ffn) {
+        const uint8_t *grow = base + (uint64_t)e * stride + (uint64_t)r * rb;
+        const uint8_t *urow = grow + gate_bytes;
+        for (uint32_t c = sub; c < hidden / 32u; c += LPR) {
+            g += chunk_dot<T>(grow, c, xs + 33u * c);
+            u += chunk_dot<T>(urow, c, xs + 33u * c);
+        }
+    }
+    g = sub_reduce<LPR>(g);
+    u = sub_reduce<LPR>(u);
+    if (sub == 0u && r < ffn) act[(uint64_t)slot * ffn + r] = silu_mul(g, u);
+}
+
+template <uint32_t T>
+static hipError_t gateup_dispatch(const ExpertSet &ex, const uint32_t *ids, uint32_t n_slot, uint32_t hidden, uint32_t ffn,
+                                  const float *x, float *act, hipStream_t s) {
+    const uint32_t lpr = lanes_per_row(hidden);
+    const dim3 grid((ffn + 256u / lpr - 1u) / (256u / lpr), n_slot);
+    const size_t lds = padded_floats(hidden) * sizeof(float);
+    switch (lpr) {
+        case 64: moe_gateup_kernel<T, 64><<<grid, 256, lds, s>>>(ex.base, ex.stride, ex.gate_bytes, ids, hidden, ffn, x, act); break;
+        case 32: moe_gateup_kernel<T, 32><<<grid, 256, lds, s>>>(ex.base, ex.stride, ex.gate_bytes, ids, hidden, ffn, x, act); break;
+        case 16: moe_gateup_kernel<T, 16><<<grid, 256, lds, s>>>(ex.base, ex.stride, ex.gate_bytes, ids, hidden, ffn, x, act); break;
+        default: moe_gateup_kernel<T, 8><<<grid, 256, lds, s>>>(ex.base, ex.stride, ex.gate_bytes, ids, hidden, ffn, x, act); break;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_moe_gateup(const ExpertSet &ex, const uint32_t *ids, uint32_t n_slot, uint32_t hidden, uint32_t ffn,
+                             const float *x, float *act, hipStream_t s) {
+    hipError_t e = ensure_tables();
+    if (e != hipSuccess) return e;
+    if (!n_slot || hidden % 256u || ffn % 256u) return hipErrorInvalidValue;
+    switch (ex.gate_up_type) {
+        case T_IQ2_XXS: return gateup_dispatch<T_IQ2_XXS>(ex, ids, n_slot, hidden, ffn, x, act, s);
+        case T_IQ3_S: return gateup_dispatch<T_IQ3_S>(ex, ids, n_slot, hidden, ffn, x, act, s);
+        case T_Q6_K: return gateup_dispatch<T_Q6_K>(ex, ids, n_slot, hidden, ffn, x, act, s);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+// down projection of the selected experts fused with the weighted sum (selection order) and the shared expert
+template <uint32_t TD, uint32_t TS, int LPR>
+__global__ __launch_bounds__(256) void moe_down_combine_kernel(const uint8_t *base, uint64_t stride, uint64_t down_off,
+                                                               const uint32_t *ids, const float *weights, uint32_t top_k,
+                                                               const uint8_t *sh_down, const float *scalar,
+                                                               uint32_t hidden, uint32_t ffn,
+                                                               const float *act, const float *sh_act, float *out) {
+    extern __shared__ float as[];                          // [top_k + 1][padded ffn]
+    const uint32_t fp = ffn + (ffn >> 5);
+    for (uint32_t i = threadIdx.x; i < top_k * ffn; i += 256u) as[(i / ffn) * fp + pad32(i % ffn)] = act[i];
+    if (sh_down) for (uint32_t i = threadIdx.x; i < ffn; i += 256u) as[top_k * fp + pad32(i)] = sh_act[i];
+    __syncthreads();
+    const uint32_t sub = threadIdx.x % LPR, r = blockIdx.x * (256u / LPR) + threadIdx.x / LPR;
+    const uint64_t rbd = (uint64_t)(ffn / 256u) * Fmt<TD>::kBlock, rbs = (uint64_t)(ffn / 256u) * Fmt<TS>::kBlock;
+    float total = 0.0f;
+    for (uint32_t k = 0; k < top_k; ++k) {
+        float part = 0.0f;
+        if (r < hidden) {
+            const uint8_t *row = base + (uint64_t)ids[k] * stride + down_off + (uint64_t)r * rbd;
+            for (uint32_t c = sub; c < ffn / 32u; c += LPR) part += chunk_dot<TD>(row, c, as + k * fp + 33u * c);
+        }
+        part = sub_reduce<LPR>(part);
+        total = fmaf(weights[k], part, total);
+    }
+    if (sh_down) {
+        float part = 0.0f;
+        if (r < hidden) {
+            const uint8_t *row = sh_down + (uint64_t)r * rbs;
+            for (uint32_t c = sub; c < ffn / 32u; c += LPR) part += chunk_dot<TS>(row, c, as + top_k * fp + 33u * c);
+        }
+        part = sub_reduce<LPR>(part);
+        total = fmaf(scalar[0], part, total);
+    }
+    if (sub == 0u && r < hidden) out[r] = total;
+}
+
+template <uint32_t TD, uint32_t TS>
+static hipError_t down_dispatch(const ExpertSet &ex, const uint32_t *ids, const float *weights, uint32_t top_k,
+                                const ExpertSet &sh, const float *scalar, uint32_t hidden, uint32_t ffn,
+                                const float *act, const float *sh_act, float *out, hipStream_t s) {
+    const uint32_t lpr = lanes_per_row(ffn);
+    const dim3 grid((hidden + 256u / lpr - 1u) / (256u / lpr));
+    const size_t lds = (size_t)(top_k + 1u) * padded_floats(ffn) * sizeof(float);
+    const uint8_t *shd = sh.base ? sh.base + sh.gate_bytes + sh.up_bytes : nullptr;
+    const uint64_t off = ex.gate_bytes + ex.up_bytes;
+#define REDHIP_DOWN(L) moe_down_combine_kernel<TD, TS, L><<<grid, 256, lds, s>>>(ex.base, ex.stride, off, ids, weights, top_k, shd, scalar, hidden, ffn, act, sh_act, out)
+    switch (lpr) {
+        case 64: REDHIP_DOWN(64); break;
+        case 32: REDHIP_DOWN(32); break;
+        case 16: REDHIP_DOWN(16); break;
+        default: REDHIP_DOWN(8); break;
+    }
+#undef REDHIP_DOWN
+    return hipGetLastError();
+}
+
+template <uint32_t TD>
+static hipError_t down_dispatch_shared(const ExpertSet &ex, const uint32_t *ids, const float *weights, uint32_t top_k,
+                                       const ExpertSet &sh, const float *scalar, uint32_t hidden, uint32_t ffn,
+                                       const float *act, const float *sh_act, float *out, hipStream_t s) {
+    switch (sh.base ? sh.down_type : TD) {
+        case T_IQ2_XXS: return down_dispatch<TD, T_IQ2_XXS>(ex, ids, weights, top_k, sh, scalar, hidden, ffn, act, sh_act, out, s);
+        case T_IQ3_S: return down_dispatch<TD, T_IQ3_S>(ex, ids, weights, top_k, sh, scalar, hidden, ffn, act, sh_act, out, s);
+        case T_Q6_K: return down_dispatch<TD, T_Q6_K>(ex, ids, weights, top_k, sh, scalar, hidden, ffn, act, sh_act, out, s);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+hipError_t launch_moe_down_combine(const ExpertSet &ex, const uint32_t *ids, const float *weights, uint32_t top_k,
+                                   const ExpertSet &shared, const float *scalar, uint32_t hidden, uint32_t ffn,
+                                   const float *act, const float *shared_act, float *out, hipStream_t s) {
+    hipError_t e = ensure_tables();
+    if (e != hipSuccess) return e;
+    if (hidden % 256u || ffn % 256u || (size_t)(top_k + 1u) * padded_floats(ffn) * 4u > 160u * 1024u) return hipErrorInvalidValue;
+    switch (ex.down_type) {
+        case T_IQ2_XXS: return down_dispatch_shared<T_IQ2_XXS>(ex, ids, weights, top_k, shared, scalar, hidden, ffn, act, shared_act, out, s);
+        case T_IQ3_S: return down_dispatch_shared<T_IQ3_S>(ex, ids, weights, top_k, shared, scalar, hidden, ffn, act, shared_act, out, s);
+        case T_Q6_K: return down_dispatch_shared<T_Q6_K>(ex, ids, weights, top_k, shared, scalar, hidden, ffn, act, shared_act, out, s);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+// ---------------------------------------------------------------- token grouping (pair sort)
+
+// One workgroup. For every (token, k) pair p = t * top_k + k:
+//   first[e]   = smallest p that names expert e            -> experts numbered in first-appearance order
+//   member[e]  = bitmap over tokens that selected e        -> rank of a pair inside its expert = popcount below t
+// which gives the stable counting sort of the host loop it replaces without a serial pass.
+__global__ __launch_bounds__(1024) void group_pairs_kernel(const uint32_t *ids, const float *weights, uint32_t ntok, uint32_t top_k,
+                                                           uint32_t n_expert, uint32_t *uid, uint32_t *expert_start,
+                                                           uint32_t *pair_token, float *pair_weight, uint32_t *tok_pair,
+                                                           uint32_t *n_unique) {
+    extern __shared__ uint32_t sm[];
+    const uint32_t words = (ntok + 31u) / 32u, P = ntok * top_k, tid = threadIdx.x;
+    uint32_t *first = sm;                          // [n_expert]
+    uint32_t *count = first + n_expert;            // [n_expert]
+    uint32_t *dense = count + n_expert;            // [n_expert]
+    uint32_t *start = dense + n_expert;            // [n_expert + 1] by dense index
+    uint32_t *scan = start + n_expert + 1u;        // [1024 + 1]
+    uint32_t *member = scan + 1025u;               // [n_expert][words]
+    for (uint32_t i = tid; i < n_expert; i += 1024u) { first[i] = 0xffffffffu; count[i] = 0u; dense[i] = 0u; }
+    for (uint32_t i = tid; i < n_expert * words; i += 1024u) member[i] = 0u;
+    __syncthreads();
+    for (uint32_t p = tid; p < P; p += 1024u) {
+        const uint32_t e = ids[p], t = p / top_k;
+        atomicMin(&first[e], p);
+        atomicAdd(&count[e], 1u);
+        atomicOr(&member[e * words + (t >> 5)], 1u << (t & 31u));
+    }
+    __syncthreads();
+    // exclusive scan of "pair p is the first appearance of its expert", P elements in chunks of per-thread runs
+    const uint32_t per = (P + 1023u) / 1024u;
+    uint32_t mine = 0u;
+    for (uint32_t j = 0; j < per; ++j) { const uint32_t p = tid * per + j; if (p < P && first[ids[p]] == p) ++mine; }
+    scan[tid + 1u] = mine;
+    if (tid == 0u) scan[0] = 0u;
+    __syncthreads();
+    if (tid == 0u) for (uint32_t i = 1; i <= 1024u; ++i) scan[i] += scan[i - 1u];       // 1024 adds: negligible
+    __syncthreads();
+    uint32_t run = scan[tid];
+    for (uint32_t j = 0; j < per; ++j) {
+        const uint32_t p = tid * per + j;
+        if (p < P && first[ids[p]] == p) { dense[ids[p]] = run; uid[run] = ids[p]; ++run; }
+    }
+    const uint32_t U = scan[1024];
+    __syncthreads();
+    // exclusive scan of the per-expert pair counts in dense order
+    if (tid == 0u) {
+        uint32_t acc = 0u;
+        for (uint32_t u = 0; u < U; ++u) { start[u] = acc; acc += count[uid[u]]; }
+        start[U] = acc;
+        n_unique[0] = U;
+    }
+    __syncthreads();
+    for (uint32_t u = tid; u <= U; u += 1024u) expert_start[u] = start[u];
+    for (uint32_t p = tid; p < P; p += 1024u) {
+        const uint32_t e = ids[p], t = p / top_k;
+        const uint32_t *bits = member + e * words;
+        uint32_t rank = __popc(bits[t >> 5] & ((1u << (t & 31u)) - 1u));
+        for (uint32_t w = 0; w < (t >> 5); ++w) rank += __popc(bits[w]);
+        const uint32_t pos = start[dense[e]] + rank;
+        pair_token[pos] = t;
+        pair_weight[pos] = weights[p];
+        tok_pair[p] = pos;
+    }
+}
+
+hipError_t launch_group_pairs(const uint32_t *ids, const float *weights, uint32_t ntok, uint32_t top_k, uint32_t n_expert,
+                              uint32_t *uid, uint32_t *expert_start, uint32_t *pair_token, float *pair_weight,
+                              uint32_t *tok_pair, uint32_t *n_unique, hipStream_t s) {
+    if (!ntok || !top_k || !n_expert || n_expert > 1024u) return hipErrorInvalidValue;
+    const uint32_t words = (ntok + 31u) / 32u;
+    const size_t lds = sizeof(uint32_t) * ((size_t)4u * n_expert + 1u + 1025u + (size_t)n_expert * words);
+    if (lds > 160u * 1024u) return hipErrorInvalidValue;
+    static bool attr_set = false;
+    if (!attr_set) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(group_pairs_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e != hipSuccess) return e;
+        attr_set = true;
+    }
+    group_pairs_kernel<<<1, 1024, lds, s>>>(ids, weights, ntok, top_k, n_expert, uid, expert_start, pair_token, pair_weight, tok_pair, n_unique);
+    return hipGetLastError();
+}
+
+}  // namespace redhip

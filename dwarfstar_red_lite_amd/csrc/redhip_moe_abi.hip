@@ -1,0 +1,304 @@
+// Resident MoE FFN layers: every expert of every layer stays in HBM, one call runs a layer's FFN on a stream.
+// See include/redhip_moe.h for the contract.
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+
+#include <vector>
+
+#include "../../include/redhip_moe.h"
+#include "redhip_internal.h"
+
+using namespace redhip;
+
+namespace {
+
+thread_local char g_moe_error[512];
+void moe_err(const char *fmt, ...) {
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(g_moe_error, sizeof(g_moe_error), fmt, ap);
+    va_end(ap);
+}
+#define HIP_OK(call, what)                                                            \
+    do {                                                                              \
+        const hipError_t e_ = (call);                                                 \
+        if (e_ != hipSuccess) { moe_err("%s: %s", what, hipGetErrorString(e_)); return 0; } \
+    } while (0)
+
+struct Layer {
+    uint8_t *router = nullptr;       // [n_expert] rows of `hidden` weights (F32 or Q6_K)
+    uint8_t *shared = nullptr;       // gate | up | down of the shared expert
+    float *gate_inp = nullptr;       // [hidden]
+    uint8_t *experts = nullptr;      // n_expert slots of expert_stride bytes, each gate | up | down
+};
+
+struct Moe {
+    redhip_moe_config cfg;
+    uint32_t gu_type, dn_type, sh_gu_type, sh_dn_type;
+    uint64_t gate_bytes, down_bytes, expert_stride;          // routed expert
+    uint64_t sh_gate_bytes, sh_down_bytes;                   // shared expert
+    uint64_t router_bytes;
+    uint64_t resident = 0;
+    std::vector<Layer> layers;
+    // workspace (device), sized for max_tokens
+    float *logits = nullptr, *weights = nullptr, *scalar = nullptr, *act = nullptr, *sh_act = nullptr;
+    uint32_t *ids = nullptr;
+    uint8_t *ws = nullptr;
+
+    ExpertSet routed(uint32_t l) const { return ExpertSet{layers[l].experts, expert_stride, gate_bytes, gate_bytes, gu_type, dn_type}; }
+    ExpertSet shared(uint32_t l) const { return ExpertSet{layers[l].shared, 0, sh_gate_bytes, sh_gate_bytes, sh_gu_type, sh_dn_type}; }
+};
+
+Moe *moe_of(redhip_moe_t h) { return static_cast<Moe *>(h); }
+
+size_t align256(size_t n) { return (n + 255u) & ~(size_t)255u; }
+
+bool check_layer(Moe *m, uint32_t layer) {
+    if (!m) { moe_err("null MoE handle"); return false; }
+    if (layer >= m->cfg.n_layer) { moe_err("layer %u out of range (%u layers)", layer, m->cfg.n_layer); return false; }
+    return true;
+}
+
+__global__ __launch_bounds__(256) void scalar_gate_kernel(const float *gate_inp, const float *x, uint32_t hidden, float *scalar) {
+    __shared__ double red[4];
+    const float *xt = x + (uint64_t)blockIdx.x * hidden;
+    double acc = 0.0;
+    for (uint32_t i = threadIdx.x; i < hidden; i += 256u) acc += (double)gate_inp[i] * (double)xt[i];
+    for (int o = 32; o > 0; o >>= 1) acc += __shfl_xor(acc, o, 64);
+    if ((threadIdx.x & 63u) == 0u) red[threadIdx.x >> 6] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0u) scalar[blockIdx.x] = (float)(1.0 / (1.0 + exp(-((red[0] + red[1]) + (red[2] + red[3])))));
+}
+
+int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const uint32_t *ids, const float *weights,
+                    float *out, hipStream_t s) {
+    const redhip_moe_config &c = m->cfg;
+    if (ntok != 1u) { moe_err("batched expert execution is not available in this build (ntok=%u)", ntok); return 0; }
+    const ExpertSet ex = m->routed(layer), sh = m->shared(layer);
+    HIP_OK(launch_moe_gateup(ex, ids, c.top_k, c.hidden, c.ffn, x, m->act, s), "routed gate/up launch");
+    HIP_OK(launch_moe_gateup(sh, nullptr, 1u, c.hidden, c.ffn, x, m->sh_act, s), "shared gate/up launch");
+    HIP_OK(launch_moe_down_combine(ex, ids, weights, c.top_k, sh, m->scalar, c.hidden, c.ffn, m->act, m->sh_act, out, s), "down/combine launch");
+    return 1;
+}
+
+}  // namespace
+
+extern "C" {
+
+uint32_t redhip_moe_abi_version(void) { return 1u; }
+const char *redhip_moe_last_error(void) { return g_moe_error[0] ? g_moe_error : "unknown redhip MoE error"; }
+
+redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
+    g_moe_error[0] = '\0';
+    if (!cfg) { moe_err("null MoE config"); return nullptr; }
+    const redhip_moe_config c = *cfg;
+    const uint32_t gu = word_gate_up(c.expert_type_word), dn = word_down(c.expert_type_word);
+    const uint32_t sgu = word_gate_up(c.shared_type_word), sdn = word_down(c.shared_type_word);
+    if (!c.hidden || c.hidden % 256u || !c.ffn || c.ffn % 256u || !c.n_expert || c.n_expert > 1024u || !c.top_k || c.top_k > 16u ||
+        c.top_k > c.n_expert || !c.n_layer || !c.max_tokens) {
+        moe_err("invalid MoE shape hidden=%u ffn=%u experts=%u top_k=%u layers=%u max_tokens=%u", c.hidden, c.ffn, c.n_expert, c.top_k, c.n_layer, c.max_tokens);
+        return nullptr;
+    }
+    if (!quant_supported(gu) || !quant_supported(dn) || !quant_supported(sgu) || !quant_supported(sdn) ||
+        (c.router_type != T_F32 && c.router_type != T_Q6_K) || (c.expert_type_word >> 16) || (c.shared_type_word >> 16)) {
+        moe_err("unsupported MoE types router=%u experts=0x%x shared=0x%x", c.router_type, c.expert_type_word, c.shared_type_word);
+        return nullptr;
+    }
+    int ndev = 0;
+    if (hipGetDeviceCount(&ndev) != hipSuccess || ndev < 1) { moe_err("no HIP device available"); return nullptr; }
+    Moe *m = new Moe();
+    m->cfg = c;
+    m->gu_type = gu; m->dn_type = dn; m->sh_gu_type = sgu; m->sh_dn_type = sdn;
+    m->gate_bytes = (uint64_t)c.ffn * row_bytes(gu, c.hidden);
+    m->down_bytes = (uint64_t)c.hidden * row_bytes(dn, c.ffn);
+    m->expert_stride = align256(2u * m->gate_bytes + m->down_bytes);
+    m->sh_gate_bytes = (uint64_t)c.ffn * row_bytes(sgu, c.hidden);
+    m->sh_down_bytes = (uint64_t)c.hidden * row_bytes(sdn, c.ffn);
+    m->router_bytes = (uint64_t)c.n_expert * row_bytes(c.router_type, c.hidden);
+    m->layers.resize(c.n_layer);
+    bool ok = true;
+    for (uint32_t l = 0; l < c.n_layer && ok; ++l) {
+        Layer &L = m->layers[l];
+        const size_t small = align256(m->router_bytes) + align256(2u * m->sh_gate_bytes + m->sh_down_bytes) + align256(4u * c.hidden);
+        uint8_t *p = nullptr;
+        ok = hipMalloc(reinterpret_cast<void **>(&p), small) == hipSuccess &&
+             hipMalloc(reinterpret_cast<void **>(&L.experts), (size_t)c.n_expert * m->expert_stride) == hipSuccess;
+        if (!ok) { if (p) (void)hipFree(p); break; }
+        L.router = p;
+        L.shared = p + align256(m->router_bytes);
+        L.gate_inp = reinterpret_cast<float *>(L.shared + align256(2u * m->sh_gate_bytes + m->sh_down_bytes));
+        m->resident += small + (uint64_t)c.n_expert * m->expert_stride;
+    }
+    const size_t T = c.max_tokens;
+    const size_t ws_bytes = align256(T * c.n_expert * 4u) + 2u * align256(T * c.top_k * 4u) + align256(T * 4u) +
+                            align256(T * c.top_k * c.ffn * 4u) + align256(T * c.ffn * 4u);
+    ok = ok && hipMalloc(reinterpret_cast<void **>(&m->ws), ws_bytes) == hipSuccess;
+    if (!ok) {
+        moe_err("failed to allocate resident MoE memory (%llu bytes so far)", (unsigned long long)m->resident);
+        redhip_moe_destroy(m);
+        return nullptr;
+    }
+    uint8_t *w = m->ws;
+    m->logits = reinterpret_cast<float *>(w); w += align256(T * c.n_expert * 4u);
+    m->ids = reinterpret_cast<uint32_t *>(w); w += align256(T * c.top_k * 4u);
+    m->weights = reinterpret_cast<float *>(w); w += align256(T * c.top_k * 4u);
+    m->scalar = reinterpret_cast<float *>(w); w += align256(T * 4u);
+    m->act = reinterpret_cast<float *>(w); w += align256(T * c.top_k * c.ffn * 4u);
+    m->sh_act = reinterpret_cast<float *>(w);
+    // first launches copy the codebooks to the device; do it here so that forward never synchronises
+    if (launch_dequant_rows(T_F32, m->ws, 1u, 32u, m->logits, nullptr) != hipSuccess || hipDeviceSynchronize() != hipSuccess) {
+        moe_err("failed to initialise device codebooks");
+        redhip_moe_destroy(m);
+        return nullptr;
+    }
+    return m;
+}
+
+void redhip_moe_destroy(redhip_moe_t h) {
+    Moe *m = moe_of(h);
+    if (!m) return;
+    (void)hipDeviceSynchronize();
+    for (Layer &L : m->layers) {
+        if (L.router) (void)hipFree(L.router);
+        if (L.experts) (void)hipFree(L.experts);
+    }
+    if (m->ws) (void)hipFree(m->ws);
+    delete m;
+}
+
+uint64_t redhip_moe_resident_bytes(redhip_moe_t h) { return h ? moe_of(h)->resident : 0u; }
+
+int redhip_moe_load_router(redhip_moe_t h, uint32_t layer, const void *weights, uint64_t bytes) {
+    Moe *m = moe_of(h);
+    if (!check_layer(m, layer)) return 0;
+    if (!weights || bytes != m->router_bytes) { moe_err("router byte size mismatch: got %llu expected %llu", (unsigned long long)bytes, (unsigned long long)m->router_bytes); return 0; }
+    HIP_OK(hipMemcpy(m->layers[layer].router, weights, (size_t)bytes, hipMemcpyDefault), "router upload");
+    return 1;
+}
+
+int redhip_moe_load_shared(redhip_moe_t h, uint32_t layer, const float *gate_inp, const void *gate, uint64_t gate_bytes,
+                           const void *up, uint64_t up_bytes, const void *down, uint64_t down_bytes) {
+    Moe *m = moe_of(h);
+    if (!check_layer(m, layer)) return 0;
+    if (!gate_inp || !gate || !up || !down || gate_bytes != m->sh_gate_bytes || up_bytes != m->sh_gate_bytes || down_bytes != m->sh_down_bytes) {
+        moe_err("shared expert byte size mismatch gate=%llu/%llu up=%llu/%llu down=%llu/%llu", (unsigned long long)gate_bytes,
+                (unsigned long long)m->sh_gate_bytes, (unsigned long long)up_bytes, (unsigned long long)m->sh_gate_bytes,
+                (unsigned long long)down_bytes, (unsigned long long)m->sh_down_bytes);
+        return 0;
+    }
+    Layer &L = m->layers[layer];
+    HIP_OK(hipMemcpy(L.gate_inp, gate_inp, 4u * (size_t)m->cfg.hidden, hipMemcpyDefault), "shared gate vector upload");
+    HIP_OK(hipMemcpy(L.shared, gate, (size_t)gate_bytes, hipMemcpyDefault), "shared gate upload");
+    HIP_OK(hipMemcpy(L.shared + gate_bytes, up, (size_t)up_bytes, hipMemcpyDefault), "shared up upload");
+    HIP_OK(hipMemcpy(L.shared + 2u * gate_bytes, down, (size_t)down_bytes, hipMemcpyDefault), "shared down upload");
+    return 1;
+}
+
+int redhip_moe_load_experts(redhip_moe_t h, uint32_t layer, uint32_t first, uint32_t count, const void *gate, const void *up, const void *down) {
+    Moe *m = moe_of(h);
+    if (!check_layer(m, layer)) return 0;
+    if (!gate || !up || !down || !count || first >= m->cfg.n_expert || count > m->cfg.n_expert - first) {
+        moe_err("invalid expert range first=%u count=%u of %u", first, count, m->cfg.n_expert);
+        return 0;
+    }
+    uint8_t *dst = m->layers[layer].experts + (uint64_t)first * m->expert_stride;
+    // 2-D copies place the tightly packed source matrices into the gate | up | down slots
+    HIP_OK(hipMemcpy2D(dst, m->expert_stride, gate, m->gate_bytes, m->gate_bytes, count, hipMemcpyDefault), "expert gate upload");
+    HIP_OK(hipMemcpy2D(dst + m->gate_bytes, m->expert_stride, up, m->gate_bytes, m->gate_bytes, count, hipMemcpyDefault), "expert up upload");
+    HIP_OK(hipMemcpy2D(dst + 2u * m->gate_bytes, m->expert_stride, down, m->down_bytes, m->down_bytes, count, hipMemcpyDefault), "expert down upload");
+    return 1;
+}
+
+int redhip_moe_route(redhip_moe_t h, uint32_t layer, const float *x_dev, uint32_t ntok, uint32_t *ids_dev, float *weights_dev,
+                     float *logits_dev, void *stream) {
+    Moe *m = moe_of(h);
+    if (!check_layer(m, layer)) return 0;
+    const redhip_moe_config &c = m->cfg;
+    if (!x_dev || !ntok || ntok > c.max_tokens) { moe_err("invalid token count %u (max %u)", ntok, c.max_tokens); return 0; }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    float *lg = logits_dev ? logits_dev : m->logits;
+    for (uint32_t t = 0; t < ntok; ++t)
+        HIP_OK(launch_gemv_rows(c.router_type, m->layers[layer].router, c.hidden, 0u, c.n_expert, x_dev + (size_t)t * c.hidden,
+                                lg + (size_t)t * c.n_expert, s), "router GEMV launch");
+    HIP_OK(launch_route_select(lg, ntok, c.n_expert, c.top_k, ids_dev ? ids_dev : m->ids, weights_dev ? weights_dev : m->weights, nullptr,
+                               m->layers[layer].gate_inp, x_dev, c.hidden, m->scalar, s), "router selection launch");
+    return 1;
+}
+
+int redhip_moe_experts(redhip_moe_t h, uint32_t layer, const float *x_dev, uint32_t ntok, const uint32_t *ids_dev,
+                       const float *weights_dev, float *out_dev, void *stream) {
+    Moe *m = moe_of(h);
+    if (!check_layer(m, layer)) return 0;
+    if (!x_dev || !ids_dev || !weights_dev || !out_dev || !ntok || ntok > m->cfg.max_tokens) { moe_err("invalid expert execution arguments"); return 0; }
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    scalar_gate_kernel<<<ntok, 256, 0, s>>>(m->layers[layer].gate_inp, x_dev, m->cfg.hidden, m->scalar);
+    HIP_OK(hipGetLastError(), "scalar gate launch");
+    return experts_enqueue(m, layer, x_dev, ntok, ids_dev, weights_dev, out_dev, s);
+}
+
+int redhip_moe_forward(redhip_moe_t h, uint32_t layer, const float *x_dev, uint32_t ntok, float *out_dev, void *stream) {
+    Moe *m = moe_of(h);
+    if (!check_layer(m, layer)) return 0;
+    if (!x_dev || !out_dev) { moe_err("null activation pointer"); return 0; }
+    if (!redhip_moe_route(h, layer, x_dev, ntok, nullptr, nullptr, nullptr, stream)) return 0;
+    return experts_enqueue(m, layer, x_dev, ntok, m->ids, m->weights, out_dev, static_cast<hipStream_t>(stream));
+}
+
+int redhip_moe_last_route(redhip_moe_t h, uint32_t ntok, uint32_t *ids, float *weights, float *logits, void *stream) {
+    Moe *m = moe_of(h);
+    if (!m || !ntok || ntok > m->cfg.max_tokens) { moe_err("invalid last-route request"); return 0; }
+    HIP_OK(hipStreamSynchronize(static_cast<hipStream_t>(stream)), "stream synchronise");
+    const redhip_moe_config &c = m->cfg;
+    if (ids) HIP_OK(hipMemcpy(ids, m->ids, (size_t)ntok * c.top_k * 4u, hipMemcpyDeviceToHost), "ids download");
+    if (weights) HIP_OK(hipMemcpy(weights, m->weights, (size_t)ntok * c.top_k * 4u, hipMemcpyDeviceToHost), "weights download");
+    if (logits) HIP_OK(hipMemcpy(logits, m->logits, (size_t)ntok * c.n_expert * 4u, hipMemcpyDeviceToHost), "logits download");
+    return 1;
+}
+
+int redhip_moe_group(redhip_moe_t h, const uint32_t *ids_dev, const float *weights_dev, uint32_t ntok, uint32_t *uid_dev,
+                     uint32_t *expert_start_dev, uint32_t *pair_token_dev, float *pair_weight_dev, uint32_t *tok_pair_dev,
+                     uint32_t *n_unique_dev, void *stream) {
+    Moe *m = moe_of(h);
+    if (!m) { moe_err("null MoE handle"); return 0; }
+    if (!ids_dev || !weights_dev || !uid_dev || !expert_start_dev || !pair_token_dev || !pair_weight_dev || !tok_pair_dev || !n_unique_dev || !ntok) {
+        moe_err("invalid grouping arguments");
+        return 0;
+    }
+    HIP_OK(launch_group_pairs(ids_dev, weights_dev, ntok, m->cfg.top_k, m->cfg.n_expert, uid_dev, expert_start_dev, pair_token_dev,
+                              pair_weight_dev, tok_pair_dev, n_unique_dev, static_cast<hipStream_t>(stream)), "grouping launch");
+    return 1;
+}
+
+int redhip_dequant_rows(uint32_t ggml_type, const void *rows_dev, uint32_t nrows, uint32_t ncols, float *out_dev, void *stream) {
+    if (!rows_dev || !out_dev) { moe_err("null dequant pointer"); return 0; }
+    HIP_OK(launch_dequant_rows(ggml_type, rows_dev, nrows, ncols, out_dev, static_cast<hipStream_t>(stream)), "dequant launch");
+    return 1;
+}
+
+int redhip_moe_dequant_resident(redhip_moe_t h, uint32_t layer, uint32_t expert, uint32_t which, float *out_dev, void *stream) {
+    Moe *m = moe_of(h);
+    if (!check_layer(m, layer)) return 0;
+    const redhip_moe_config &c = m->cfg;
+    if (!out_dev || which > 3u || (which < 3u && expert > c.n_expert)) { moe_err("invalid resident matrix request"); return 0; }
+    const Layer &L = m->layers[layer];
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    if (which == 3u) { HIP_OK(launch_dequant_rows(c.router_type, L.router, c.n_expert, c.hidden, out_dev, s), "router dequant"); return 1; }
+    const bool sh = expert == c.n_expert;
+    const uint8_t *base = sh ? L.shared : L.experts + (uint64_t)expert * m->expert_stride;
+    const uint64_t gb = sh ? m->sh_gate_bytes : m->gate_bytes;
+    const uint32_t gu = sh ? m->sh_gu_type : m->gu_type, dn = sh ? m->sh_dn_type : m->dn_type;
+    if (which == 0u) HIP_OK(launch_dequant_rows(gu, base, c.ffn, c.hidden, out_dev, s), "gate dequant");
+    else if (which == 1u) HIP_OK(launch_dequant_rows(gu, base + gb, c.ffn, c.hidden, out_dev, s), "up dequant");
+    else HIP_OK(launch_dequant_rows(dn, base + 2u * gb, c.hidden, c.ffn, out_dev, s), "down dequant");
+    return 1;
+}
+
+int redhip_gemv_rows(uint32_t ggml_type, const void *matrix_dev, uint32_t ncols, uint32_t row_start, uint32_t row_count,
+                     const float *x_dev, float *out_dev, void *stream) {
+    if (!matrix_dev || !x_dev || !out_dev) { moe_err("null GEMV pointer"); return 0; }
+    HIP_OK(launch_gemv_rows(ggml_type, matrix_dev, ncols, row_start, row_count, x_dev, out_dev, static_cast<hipStream_t>(stream)), "GEMV launch");
+    return 1;
+}
+
+}  // extern "C"

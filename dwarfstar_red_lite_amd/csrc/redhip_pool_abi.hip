@@ -1,0 +1,439 @@
+// C-ABI front ends that keep the reference's call surface: the single-expert FFN pool (redmetal_ffn_*), the
+// one-shot quantised GEMV (redmetal_quant_rows) and the router entry points. Host pointers in, host pointers
+// out, synchronous; the arithmetic runs in the gfx950 kernels of redhip_kernels.hip.
+#include <errno.h>
+#include <fcntl.h>
+#include <limits.h>
+#include <stdarg.h>
+#include <stdio.h>
+#include <string.h>
+#include <sys/stat.h>
+#include <time.h>
+#include <unistd.h>
+
+#include <mutex>
+#include <vector>
+
+#include "../../include/redmetal_ffn.h"
+#include "../../include/redmetal_quant.h"
+#include "../../include/redmetal_router.h"
+#include "redhip_internal.h"
+
+using namespace redhip;
+
+namespace {
+
+double now_ms() {
+    struct timespec ts;
+    clock_gettime(CLOCK_MONOTONIC, &ts);
+    return (double)ts.tv_sec * 1000.0 + (double)ts.tv_nsec / 1.0e6;
+}
+
+thread_local char g_ffn_error[512];
+thread_local char g_quant_error[512];
+
+void set_err(char *dst, size_t cap, const char *fmt, ...) {
+    if (!dst || !cap) return;
+    va_list ap;
+    va_start(ap, fmt);
+    vsnprintf(dst, cap, fmt, ap);
+    va_end(ap);
+}
+#define FFN_ERR(...) set_err(g_ffn_error, sizeof(g_ffn_error), __VA_ARGS__)
+#define QUANT_ERR(...) set_err(g_quant_error, sizeof(g_quant_error), __VA_ARGS__)
+
+// whole-range pread with EINTR retry; counts calls and bytes
+bool pread_range(int fd, uint64_t file_size, uint64_t offset, uint64_t len, uint8_t *dst, uint64_t *bytes, uint64_t *calls,
+                 char *err, size_t cap) {
+    if (!dst || offset > file_size || len > file_size - offset) {
+        set_err(err, cap, "invalid pread range offset=%llu len=%llu file_size=%llu", (unsigned long long)offset,
+                (unsigned long long)len, (unsigned long long)file_size);
+        return false;
+    }
+    uint64_t pos = 0;
+    while (pos < len) {
+        const uint64_t rem = len - pos;
+        const size_t want = rem > (uint64_t)SSIZE_MAX ? (size_t)SSIZE_MAX : (size_t)rem;
+        ssize_t n;
+        do { n = pread(fd, dst + pos, want, (off_t)(offset + pos)); } while (n < 0 && errno == EINTR);
+        if (calls) ++*calls;
+        if (n <= 0) {
+            set_err(err, cap, n < 0 ? "pread failed: %s" : "unexpected end of file%s", n < 0 ? strerror(errno) : "");
+            return false;
+        }
+        pos += (uint64_t)n;
+    }
+    if (bytes) *bytes += len;
+    return true;
+}
+
+struct DevBuf {                       // grow-only device scratch
+    void *p = nullptr;
+    size_t cap = 0;
+    bool reserve(size_t n) {
+        if (n <= cap) return true;
+        if (p) (void)hipFree(p);
+        p = nullptr;
+        cap = 0;
+        if (hipMalloc(&p, n) != hipSuccess) { p = nullptr; return false; }
+        cap = n;
+        return true;
+    }
+    ~DevBuf() { if (p) (void)hipFree(p); }
+};
+
+struct FfnPool {
+    int fd = -1;
+    uint64_t file_size = 0, slot_bytes = 0, budget = 0, allocated = 0;
+    uint32_t capacity = 0, slots_per_slab = 0;
+    std::vector<uint8_t *> slabs;                 // device memory, created on first use of a slot in the slab
+    std::vector<uint32_t> inflight;
+    std::mutex mu;                                // counters, slab creation, in-flight marks
+    std::mutex exec_mu;                           // the scratch below serves one execute at a time
+    DevBuf scratch;
+    uint64_t bytes_read = 0, read_calls = 0;
+    double read_ms = 0.0;
+
+    uint8_t *slot_base(uint32_t slot) {           // nullptr + message on failure
+        if (slot >= capacity) { FFN_ERR("FFN slot %u exceeds capacity %u", slot, capacity); return nullptr; }
+        const uint32_t slab = slot / slots_per_slab;
+        std::lock_guard<std::mutex> lk(mu);
+        while (slabs.size() <= slab) {
+            const uint32_t idx = (uint32_t)slabs.size();
+            const uint32_t first = idx * slots_per_slab;
+            const uint32_t n = capacity - first < slots_per_slab ? capacity - first : slots_per_slab;
+            void *p = nullptr;
+            const hipError_t e = hipMalloc(&p, (size_t)n * slot_bytes);
+            if (e != hipSuccess) { FFN_ERR("failed to allocate FFN slab %u (%llu bytes): %s", idx, (unsigned long long)n * slot_bytes, hipGetErrorString(e)); return nullptr; }
+            slabs.push_back(static_cast<uint8_t *>(p));
+            allocated += (uint64_t)n * slot_bytes;
+        }
+        return slabs[slab] + (uint64_t)(slot % slots_per_slab) * slot_bytes;
+    }
+    void mark(uint32_t slot, int delta) {
+        std::lock_guard<std::mutex> lk(mu);
+        if (delta > 0) inflight[slot] += (uint32_t)delta;
+        else if (inflight[slot]) inflight[slot] -= 1u;
+    }
+};
+
+FfnPool *pool_of(redmetal_ffn_pool_t h) { return static_cast<FfnPool *>(h); }
+
+bool sizes_overflow(uint64_t a, uint64_t b, uint64_t c) { return a > UINT64_MAX - b || a + b > UINT64_MAX - c; }
+
+}  // namespace
+
+extern "C" {
+
+// ------------------------------------------------------------------ redmetal_ffn
+
+uint32_t redmetal_ffn_abi_version(void) { return 1u; }
+const char *redmetal_ffn_last_error(void) { return g_ffn_error[0] ? g_ffn_error : "unknown Red Metal FFN error"; }
+
+redmetal_ffn_pool_t redmetal_ffn_pool_create(const char *model_path, uint64_t budget_bytes, uint64_t slot_bytes,
+        uint32_t slots_per_slab, const int8_t *iq2_xs_grid, uint32_t iq2_xs_grid_count,
+        const int8_t *iq1_m_grid, uint32_t iq1_m_grid_count) {
+    g_ffn_error[0] = '\0';
+    if (!model_path || !model_path[0] || !budget_bytes || !slot_bytes || !iq2_xs_grid || !iq1_m_grid ||
+        iq2_xs_grid_count != 512u * 8u || iq1_m_grid_count != 2048u * 8u) {
+        FFN_ERR("invalid Red Metal FFN pool arguments");
+        return nullptr;
+    }
+    if (slot_bytes > UINT64_MAX - 4095u) { FFN_ERR("FFN slot size overflow"); return nullptr; }
+    const uint64_t aligned = (slot_bytes + 4095u) & ~4095ull;
+    if (!aligned || aligned > budget_bytes) { FFN_ERR("FFN cache budget cannot fit one aligned expert slot"); return nullptr; }
+    int ndev = 0;
+    if (hipGetDeviceCount(&ndev) != hipSuccess || ndev < 1) { FFN_ERR("no HIP device available"); return nullptr; }
+    FfnPool *p = new FfnPool();
+    p->slot_bytes = aligned;
+    p->budget = budget_bytes;
+    const uint64_t cap64 = budget_bytes / aligned;
+    p->capacity = cap64 > 0xffffffffull ? 0xffffffffu : (uint32_t)cap64;
+    p->slots_per_slab = slots_per_slab ? slots_per_slab : 64u;
+    if (p->slots_per_slab > p->capacity) p->slots_per_slab = p->capacity;
+    p->fd = open(model_path, O_RDONLY);
+    if (p->fd < 0) { FFN_ERR("open(%s) failed: %s", model_path, strerror(errno)); delete p; return nullptr; }
+    struct stat st;
+    if (fstat(p->fd, &st) != 0 || st.st_size <= 0) {
+        FFN_ERR("failed to stat model file: %s", strerror(errno));
+        close(p->fd);
+        delete p;
+        return nullptr;
+    }
+    p->file_size = (uint64_t)st.st_size;
+    p->inflight.assign(p->capacity, 0u);
+    return p;
+}
+
+void redmetal_ffn_pool_destroy(redmetal_ffn_pool_t handle) {
+    FfnPool *p = pool_of(handle);
+    if (!p) return;
+    (void)hipDeviceSynchronize();
+    for (uint8_t *s : p->slabs) (void)hipFree(s);
+    if (p->fd >= 0) close(p->fd);
+    delete p;
+}
+
+uint32_t redmetal_ffn_pool_capacity(redmetal_ffn_pool_t h) { return h ? pool_of(h)->capacity : 0u; }
+uint32_t redmetal_ffn_pool_slab_count(redmetal_ffn_pool_t h) {
+    if (!h) return 0u;
+    std::lock_guard<std::mutex> lk(pool_of(h)->mu);
+    return (uint32_t)pool_of(h)->slabs.size();
+}
+uint64_t redmetal_ffn_pool_allocated_bytes(redmetal_ffn_pool_t h) {
+    if (!h) return 0u;
+    std::lock_guard<std::mutex> lk(pool_of(h)->mu);
+    return pool_of(h)->allocated;
+}
+uint64_t redmetal_ffn_pool_bytes_read(redmetal_ffn_pool_t h) {
+    if (!h) return 0u;
+    std::lock_guard<std::mutex> lk(pool_of(h)->mu);
+    return pool_of(h)->bytes_read;
+}
+uint64_t redmetal_ffn_pool_read_calls(redmetal_ffn_pool_t h) {
+    if (!h) return 0u;
+    std::lock_guard<std::mutex> lk(pool_of(h)->mu);
+    return pool_of(h)->read_calls;
+}
+double redmetal_ffn_pool_read_ms(redmetal_ffn_pool_t h) {
+    if (!h) return 0.0;
+    std::lock_guard<std::mutex> lk(pool_of(h)->mu);
+    return pool_of(h)->read_ms;
+}
+int redmetal_ffn_pool_slot_inflight(redmetal_ffn_pool_t h, uint32_t slot_id) {
+    FfnPool *p = pool_of(h);
+    if (!p || slot_id >= p->capacity) return 0;
+    std::lock_guard<std::mutex> lk(p->mu);
+    return p->inflight[slot_id] != 0u;
+}
+
+int redmetal_ffn_pool_load_expert(redmetal_ffn_pool_t h, uint32_t slot_id,
+        uint64_t gate_file_offset, uint64_t gate_bytes, uint64_t up_file_offset, uint64_t up_bytes,
+        uint64_t down_file_offset, uint64_t down_bytes, uint64_t *bytes_read, double *elapsed_ms) {
+    FfnPool *p = pool_of(h);
+    if (!p || slot_id >= p->capacity) return 0;
+    if (redmetal_ffn_pool_slot_inflight(h, slot_id)) { FFN_ERR("refusing to overwrite in-flight FFN slot %u", slot_id); return 0; }
+    if (sizes_overflow(gate_bytes, up_bytes, down_bytes)) { FFN_ERR("FFN expert payload size overflow"); return 0; }
+    const uint64_t payload = gate_bytes + up_bytes + down_bytes;
+    if (payload > p->slot_bytes) { FFN_ERR("FFN expert payload exceeds slot size"); return 0; }
+    uint8_t *base = p->slot_base(slot_id);
+    if (!base) return 0;
+    std::vector<uint8_t> host((size_t)payload);
+    uint64_t local_bytes = 0, local_calls = 0;
+    const double t0 = now_ms();
+    const bool ok =
+        pread_range(p->fd, p->file_size, gate_file_offset, gate_bytes, host.data(), &local_bytes, &local_calls, g_ffn_error, sizeof(g_ffn_error)) &&
+        pread_range(p->fd, p->file_size, up_file_offset, up_bytes, host.data() + gate_bytes, &local_bytes, &local_calls, g_ffn_error, sizeof(g_ffn_error)) &&
+        pread_range(p->fd, p->file_size, down_file_offset, down_bytes, host.data() + gate_bytes + up_bytes, &local_bytes, &local_calls, g_ffn_error, sizeof(g_ffn_error));
+    if (!ok) return 0;
+    if (payload) {
+        const hipError_t e = hipMemcpy(base, host.data(), (size_t)payload, hipMemcpyHostToDevice);
+        if (e != hipSuccess) { FFN_ERR("FFN slot upload failed: %s", hipGetErrorString(e)); return 0; }
+    }
+    const double ms = now_ms() - t0;
+    {
+        std::lock_guard<std::mutex> lk(p->mu);
+        p->bytes_read += local_bytes;
+        p->read_calls += local_calls;
+        p->read_ms += ms;
+    }
+    if (bytes_read) *bytes_read = local_bytes;
+    if (elapsed_ms) *elapsed_ms = ms;
+    return 1;
+}
+
+int redmetal_ffn_pool_slot_addresses(redmetal_ffn_pool_t h, uint32_t slot_id, uint64_t gate_bytes, uint64_t up_bytes,
+        uint64_t down_bytes, uint64_t *gate_address, uint64_t *up_address, uint64_t *down_address) {
+    FfnPool *p = pool_of(h);
+    if (!p || slot_id >= p->capacity) return 0;
+    if (sizes_overflow(gate_bytes, up_bytes, down_bytes) || gate_bytes + up_bytes + down_bytes > p->slot_bytes) return 0;
+    uint8_t *base = p->slot_base(slot_id);
+    if (!base) return 0;
+    const uint64_t a = (uint64_t)(uintptr_t)base;
+    if (gate_address) *gate_address = a;
+    if (up_address) *up_address = a + gate_bytes;
+    if (down_address) *down_address = a + gate_bytes + up_bytes;
+    return 1;
+}
+
+int redmetal_ffn_pool_execute_expert(redmetal_ffn_pool_t h, uint32_t slot_id, uint32_t ggml_type,
+        uint64_t gate_bytes, uint64_t up_bytes, uint64_t down_bytes, uint32_t hidden_size, uint32_t ffn_size,
+        uint32_t output_row_start, uint32_t output_row_count, const float *input, uint32_t input_count,
+        float *output, uint32_t output_count, double *elapsed_ms) {
+    FfnPool *p = pool_of(h);
+    if (!p || !input || !output || slot_id >= p->capacity) return 0;
+    const uint32_t gu = word_gate_up(ggml_type), dn = word_down(ggml_type);
+    if (!quant_supported(gu) || !quant_supported(dn) || (ggml_type >> 16)) {
+        FFN_ERR("unsupported FFN GGML type word 0x%x (supported: IQ2_XXS 16, IQ3_S 21, Q6_K 14)", ggml_type);
+        return 0;
+    }
+    if (!hidden_size || hidden_size % 256u || !ffn_size || ffn_size % 256u || input_count != hidden_size ||
+        !output_row_count || output_row_start >= hidden_size || output_row_count > hidden_size - output_row_start ||
+        output_count < output_row_count) {
+        FFN_ERR("invalid FFN dimensions hidden=%u ffn=%u start=%u count=%u", hidden_size, ffn_size, output_row_start, output_row_count);
+        return 0;
+    }
+    const uint64_t expect_gate = (uint64_t)ffn_size * row_bytes(gu, hidden_size);
+    const uint64_t expect_down = (uint64_t)hidden_size * row_bytes(dn, ffn_size);
+    if (gate_bytes != expect_gate || up_bytes != expect_gate || down_bytes != expect_down) {
+        FFN_ERR("FFN matrix byte mismatch gate=%llu/%llu up=%llu/%llu down=%llu/%llu", (unsigned long long)gate_bytes,
+                (unsigned long long)expect_gate, (unsigned long long)up_bytes, (unsigned long long)expect_gate,
+                (unsigned long long)down_bytes, (unsigned long long)expect_down);
+        return 0;
+    }
+    if (sizes_overflow(gate_bytes, up_bytes, down_bytes) || gate_bytes + up_bytes + down_bytes > p->slot_bytes) {
+        FFN_ERR("FFN resident expert exceeds slot bounds");
+        return 0;
+    }
+    uint8_t *base = p->slot_base(slot_id);
+    if (!base) return 0;
+
+    std::lock_guard<std::mutex> exec(p->exec_mu);
+    const size_t n_x = hidden_size, n_act = ffn_size, n_out = output_row_count;
+    if (!p->scratch.reserve((n_x + n_act + n_out) * sizeof(float))) { FFN_ERR("failed to allocate FFN activation buffers"); return 0; }
+    float *dx = static_cast<float *>(p->scratch.p), *dact = dx + n_x, *dout = dact + n_act;
+    hipError_t e = hipMemcpy(dx, input, n_x * sizeof(float), hipMemcpyHostToDevice);
+    if (e != hipSuccess) { FFN_ERR("FFN input upload failed: %s", hipGetErrorString(e)); return 0; }
+    p->mark(slot_id, 1);
+    const double t0 = now_ms();
+    ExpertSet ex{base, 0, gate_bytes, up_bytes, gu, dn};
+    e = launch_moe_gateup(ex, nullptr, 1u, hidden_size, ffn_size, dx, dact, nullptr);
+    if (e == hipSuccess) e = launch_gemv_rows(dn, base + gate_bytes + up_bytes, ffn_size, output_row_start, output_row_count, dact, dout, nullptr);
+    if (e == hipSuccess) e = hipStreamSynchronize(nullptr);
+    const double ms = now_ms() - t0;
+    p->mark(slot_id, -1);
+    if (e != hipSuccess) { FFN_ERR("FFN HIP command failed: %s", hipGetErrorString(e)); return 0; }
+    e = hipMemcpy(output, dout, n_out * sizeof(float), hipMemcpyDeviceToHost);
+    if (e != hipSuccess) { FFN_ERR("FFN output download failed: %s", hipGetErrorString(e)); return 0; }
+    if (elapsed_ms) *elapsed_ms = ms;
+    return 1;
+}
+
+// ------------------------------------------------------------------ redmetal_quant
+
+uint32_t redmetal_quant_abi_version(void) { return 1u; }
+const char *redmetal_quant_last_error(void) { return g_quant_error[0] ? g_quant_error : "unknown Red Metal quant error"; }
+
+int redmetal_quant_rows(const char *model_path, uint64_t matrix_file_offset, uint64_t matrix_bytes, uint32_t ggml_type,
+        uint32_t ncols, uint32_t nrows, uint32_t row_start, uint32_t row_count, const float *input, uint32_t input_count,
+        const int8_t *grid, uint32_t grid_count, float *output, uint32_t output_count, double *io_ms, double *gpu_ms) {
+    (void)grid;
+    (void)grid_count;
+    g_quant_error[0] = '\0';
+    if (!model_path || !model_path[0] || !input || !output) { QUANT_ERR("invalid Red Metal mixed-quant arguments"); return 0; }
+    if (ggml_type != T_F32 && !quant_supported(ggml_type)) { QUANT_ERR("unsupported GGML type %u", ggml_type); return 0; }
+    if (!ncols || ncols % 256u || !nrows || !row_count || row_start >= nrows || row_count > nrows - row_start ||
+        input_count != ncols || output_count < row_count) {
+        QUANT_ERR("invalid mixed-quant dimensions cols=%u rows=%u start=%u count=%u", ncols, nrows, row_start, row_count);
+        return 0;
+    }
+    const uint64_t rb = row_bytes(ggml_type, ncols);
+    if (!rb || (uint64_t)nrows > UINT64_MAX / rb || matrix_bytes != (uint64_t)nrows * rb) {
+        QUANT_ERR("matrix byte size mismatch: got %llu expected %llu", (unsigned long long)matrix_bytes, (unsigned long long)((uint64_t)nrows * rb));
+        return 0;
+    }
+    const int fd = open(model_path, O_RDONLY);
+    if (fd < 0) { QUANT_ERR("open(%s) failed: %s", model_path, strerror(errno)); return 0; }
+    struct stat st;
+    if (fstat(fd, &st) != 0 || st.st_size <= 0) { QUANT_ERR("failed to stat model file: %s", strerror(errno)); close(fd); return 0; }
+    std::vector<uint8_t> host((size_t)matrix_bytes);
+    const double t_io = now_ms();
+    const bool ok = pread_range(fd, (uint64_t)st.st_size, matrix_file_offset, matrix_bytes, host.data(), nullptr, nullptr, g_quant_error, sizeof(g_quant_error));
+    const double io = now_ms() - t_io;
+    close(fd);
+    if (!ok) return 0;
+    DevBuf buf;
+    const size_t w_bytes = ((size_t)matrix_bytes + 255u) & ~(size_t)255u;
+    if (!buf.reserve(w_bytes + ((size_t)ncols + row_count) * sizeof(float))) { QUANT_ERR("failed to allocate mixed quant device buffers"); return 0; }
+    uint8_t *dw = static_cast<uint8_t *>(buf.p);
+    float *dx = reinterpret_cast<float *>(dw + w_bytes), *dout = dx + ncols;
+    hipError_t e = hipMemcpy(dw, host.data(), (size_t)matrix_bytes, hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMemcpy(dx, input, (size_t)ncols * sizeof(float), hipMemcpyHostToDevice);
+    if (e != hipSuccess) { QUANT_ERR("mixed quant upload failed: %s", hipGetErrorString(e)); return 0; }
+    const double t_gpu = now_ms();
+    e = launch_gemv_rows(ggml_type, dw, ncols, row_start, row_count, dx, dout, nullptr);
+    if (e == hipSuccess) e = hipStreamSynchronize(nullptr);
+    const double gpu = now_ms() - t_gpu;
+    if (e != hipSuccess) { QUANT_ERR("mixed quant HIP command failed: %s", hipGetErrorString(e)); return 0; }
+    e = hipMemcpy(output, dout, (size_t)row_count * sizeof(float), hipMemcpyDeviceToHost);
+    if (e != hipSuccess) { QUANT_ERR("mixed quant download failed: %s", hipGetErrorString(e)); return 0; }
+    if (io_ms) *io_ms = io;
+    if (gpu_ms) *gpu_ms = gpu;
+    return 1;
+}
+
+// ------------------------------------------------------------------ router
+
+int rl_native_router_gpu_f32(const char *model_path, const rl_router_tensor_info *router, const float *input,
+        uint32_t input_count, float *logits, uint32_t logits_count, rl_native_router_telemetry *telemetry,
+        char *error, size_t error_cap) {
+    if (!model_path || !router || !input || !logits || (router->ggml_type != T_F32 && router->ggml_type != T_Q6_K) ||
+        router->n_dims != 2u || router->shape[0] > UINT32_MAX || router->shape[1] > UINT32_MAX) {
+        set_err(error, error_cap, "invalid HIP router arguments");
+        return 0;
+    }
+    const uint32_t hidden = (uint32_t)router->shape[0], experts = (uint32_t)router->shape[1];
+    const uint64_t rb = row_bytes(router->ggml_type, hidden);
+    const uint64_t weight_bytes = rb * experts;
+    if (!hidden || !experts || !rb || hidden % 256u || input_count != hidden || logits_count < experts ||
+        router->tensor_span_bytes < weight_bytes) {
+        set_err(error, error_cap, "HIP router shape/span mismatch");
+        return 0;
+    }
+    const int fd = open(model_path, O_RDONLY);
+    if (fd < 0) { set_err(error, error_cap, "open GGUF for HIP router failed"); return 0; }
+    struct stat st;
+    if (fstat(fd, &st) != 0) { close(fd); set_err(error, error_cap, "stat GGUF for HIP router failed"); return 0; }
+    std::vector<uint8_t> host((size_t)weight_bytes);
+    const double r0 = now_ms();
+    char msg[256];
+    const bool ok = pread_range(fd, (uint64_t)st.st_size, router->tensor_offset, weight_bytes, host.data(), nullptr, nullptr, msg, sizeof(msg));
+    const double r1 = now_ms();
+    close(fd);
+    if (!ok) { set_err(error, error_cap, "pread router weights failed"); return 0; }
+    DevBuf buf;
+    const size_t w_bytes = ((size_t)weight_bytes + 255u) & ~(size_t)255u;
+    if (!buf.reserve(w_bytes + ((size_t)hidden + experts) * sizeof(float))) { set_err(error, error_cap, "failed to allocate HIP router buffers"); return 0; }
+    uint8_t *dw = static_cast<uint8_t *>(buf.p);
+    float *dx = reinterpret_cast<float *>(dw + w_bytes), *dl = dx + hidden;
+    hipError_t e = hipMemcpy(dw, host.data(), (size_t)weight_bytes, hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = hipMemcpy(dx, input, (size_t)hidden * sizeof(float), hipMemcpyHostToDevice);
+    const double g0 = now_ms();
+    if (e == hipSuccess) e = launch_gemv_rows(router->ggml_type, dw, hidden, 0u, experts, dx, dl, nullptr);
+    if (e == hipSuccess) e = hipStreamSynchronize(nullptr);
+    const double g1 = now_ms();
+    if (e == hipSuccess) e = hipMemcpy(logits, dl, (size_t)experts * sizeof(float), hipMemcpyDeviceToHost);
+    if (e != hipSuccess) { set_err(error, error_cap, "HIP router command failed: %s", hipGetErrorString(e)); return 0; }
+    if (telemetry) { telemetry->read_ms = r1 - r0; telemetry->compute_ms = g1 - g0; }
+    if (error && error_cap) error[0] = '\0';
+    return 1;
+}
+
+int rl_native_router_select_softmax_topk(const float *logits, uint32_t expert_count, uint32_t top_k,
+        uint32_t *expert_ids, float *router_weights, float *probabilities, char *error, size_t error_cap) {
+    if (!logits || !expert_ids || !router_weights || !expert_count || !top_k || top_k > expert_count) {
+        set_err(error, error_cap, "invalid router top-k selection arguments");
+        return 0;
+    }
+    if (expert_count > 1024u || top_k > 16u) { set_err(error, error_cap, "router selection supports at most 1024 experts and top-16"); return 0; }
+    DevBuf buf;
+    const size_t n_f = (size_t)expert_count * 2u + 2u * top_k;
+    if (!buf.reserve(n_f * sizeof(float))) { set_err(error, error_cap, "out of memory for router probabilities"); return 0; }
+    float *dl = static_cast<float *>(buf.p), *dp = dl + expert_count, *dwt = dp + expert_count;
+    uint32_t *dids = reinterpret_cast<uint32_t *>(dwt + top_k);
+    hipError_t e = hipMemcpy(dl, logits, (size_t)expert_count * sizeof(float), hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = launch_route_select(dl, 1u, expert_count, top_k, dids, dwt, dp, nullptr, nullptr, 0u, nullptr, nullptr);
+    if (e == hipSuccess) e = hipMemcpy(router_weights, dwt, (size_t)top_k * sizeof(float), hipMemcpyDeviceToHost);
+    if (e == hipSuccess) e = hipMemcpy(expert_ids, dids, (size_t)top_k * sizeof(uint32_t), hipMemcpyDeviceToHost);
+    if (e == hipSuccess && probabilities) e = hipMemcpy(probabilities, dp, (size_t)expert_count * sizeof(float), hipMemcpyDeviceToHost);
+    if (e != hipSuccess) { set_err(error, error_cap, "router selection HIP command failed: %s", hipGetErrorString(e)); return 0; }
+    for (uint32_t k = 0; k < top_k; ++k)
+        if (router_weights[k] != router_weights[k]) {       // NaN marks a softmax whose denominator or selected sum is not finite
+            set_err(error, error_cap, "invalid router softmax denominator");
+            return 0;
+        }
+    if (error && error_cap) error[0] = '\0';
+    return 1;
+}
+
+}  // extern "C"

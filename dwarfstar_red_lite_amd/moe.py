@@ -1,0 +1,150 @@
+"""Resident MoE FFN layers (include/redhip_moe.h). torch owns the activation buffers and the stream; weights are
+uploaded once and stay in HBM."""
+import ctypes as C
+
+import numpy as np
+import torch
+
+from . import expert_type_word
+from ._lib import MoeConfig, RedHipError, load
+
+
+def _ptr(t):
+    if t is None:
+        return None
+    if isinstance(t, torch.Tensor):
+        assert t.is_contiguous()
+        return t.data_ptr()
+    return np.ascontiguousarray(t).ctypes.data
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+class ResidentMoe:
+    def __init__(self, cfg, n_layer=1, max_tokens=1):
+        """cfg: dict as produced by synth.layer_config (hidden, ffn, n_expert, top_k and the five type fields)."""
+        self.lib = load()
+        self.cfg = dict(cfg)
+        self.n_layer, self.max_tokens = n_layer, max_tokens
+        c = MoeConfig(cfg["hidden"], cfg["ffn"], cfg["n_expert"], cfg["top_k"], n_layer, max_tokens, cfg["router_type"],
+                      expert_type_word(cfg["gate_up_type"], cfg["down_type"]),
+                      expert_type_word(cfg["sh_gate_up_type"], cfg["sh_down_type"]), 0)
+        torch.cuda.init()
+        self.handle = self.lib.redhip_moe_create(C.byref(c))
+        if not self.handle:
+            raise RedHipError(self._err())
+
+    def _err(self):
+        raw = self.lib.redhip_moe_last_error()
+        return raw.decode("utf-8", errors="replace") if raw else "unknown redhip MoE error"
+
+    def _check(self, ok):
+        if not ok:
+            raise RedHipError(self._err())
+
+    def close(self):
+        if self.handle:
+            self.lib.redhip_moe_destroy(self.handle)
+            self.handle = None
+
+    def __del__(self):
+        try:
+            self.close()
+        except Exception:
+            pass
+
+    @property
+    def resident_bytes(self):
+        return int(self.lib.redhip_moe_resident_bytes(self.handle))
+
+    # ---- uploads (numpy arrays or torch tensors, host or device) ----
+    def load_layer(self, layer, arrays):
+        """arrays: dict with router, gate, up, down, sh_gate, sh_up, sh_down, sh_gate_inp (raw GGUF bytes)."""
+        a = arrays
+        nbytes = lambda t: t.numel() * t.element_size() if isinstance(t, torch.Tensor) else np.asarray(t).nbytes
+        self._check(self.lib.redhip_moe_load_router(self.handle, layer, _ptr(a["router"]), nbytes(a["router"])))
+        self._check(self.lib.redhip_moe_load_shared(self.handle, layer, _ptr(a["sh_gate_inp"]), _ptr(a["sh_gate"]), nbytes(a["sh_gate"]),
+                                                    _ptr(a["sh_up"]), nbytes(a["sh_up"]), _ptr(a["sh_down"]), nbytes(a["sh_down"])))
+        self.load_experts(layer, 0, self.cfg["n_expert"], a["gate"], a["up"], a["down"])
+
+    def load_experts(self, layer, first, count, gate, up, down):
+        self._check(self.lib.redhip_moe_load_experts(self.handle, layer, first, count, _ptr(gate), _ptr(up), _ptr(down)))
+
+    # ---- execution (torch CUDA tensors, current stream) ----
+    def forward(self, layer, x, out=None):
+        x = x.reshape(-1, self.cfg["hidden"])
+        assert x.is_cuda and x.dtype == torch.float32 and x.is_contiguous()
+        if out is None:
+            out = torch.empty_like(x)
+        self._check(self.lib.redhip_moe_forward(self.handle, layer, x.data_ptr(), x.shape[0], out.data_ptr(), _stream()))
+        return out
+
+    def route(self, layer, x):
+        x = x.reshape(-1, self.cfg["hidden"])
+        n, K, E = x.shape[0], self.cfg["top_k"], self.cfg["n_expert"]
+        ids = torch.empty((n, K), dtype=torch.int32, device=x.device)
+        w = torch.empty((n, K), dtype=torch.float32, device=x.device)
+        logits = torch.empty((n, E), dtype=torch.float32, device=x.device)
+        self._check(self.lib.redhip_moe_route(self.handle, layer, x.data_ptr(), n, ids.data_ptr(), w.data_ptr(), logits.data_ptr(), _stream()))
+        return ids, w, logits
+
+    def experts(self, layer, x, ids, weights, out=None):
+        x = x.reshape(-1, self.cfg["hidden"])
+        if out is None:
+            out = torch.empty_like(x)
+        self._check(self.lib.redhip_moe_experts(self.handle, layer, x.data_ptr(), x.shape[0], ids.data_ptr(), weights.data_ptr(),
+                                                out.data_ptr(), _stream()))
+        return out
+
+    def last_route(self, ntok):
+        K, E = self.cfg["top_k"], self.cfg["n_expert"]
+        ids = np.empty((ntok, K), np.uint32)
+        w = np.empty((ntok, K), np.float32)
+        logits = np.empty((ntok, E), np.float32)
+        self._check(self.lib.redhip_moe_last_route(self.handle, ntok, ids.ctypes.data, w.ctypes.data, logits.ctypes.data, _stream()))
+        return ids, w, logits
+
+    def group(self, ids, weights):
+        n, K = ids.shape
+        P, dev = n * K, ids.device
+        U_cap = min(P, self.cfg["n_expert"])
+        uid = torch.zeros(U_cap, dtype=torch.int32, device=dev)
+        start = torch.zeros(U_cap + 1, dtype=torch.int32, device=dev)
+        ptok = torch.zeros(P, dtype=torch.int32, device=dev)
+        pw = torch.zeros(P, dtype=torch.float32, device=dev)
+        tp = torch.zeros(P, dtype=torch.int32, device=dev)
+        nu = torch.zeros(1, dtype=torch.int32, device=dev)
+        self._check(self.lib.redhip_moe_group(self.handle, ids.data_ptr(), weights.data_ptr(), n, uid.data_ptr(), start.data_ptr(),
+                                              ptok.data_ptr(), pw.data_ptr(), tp.data_ptr(), nu.data_ptr(), _stream()))
+        U = int(nu.item())
+        return uid[:U], start[:U + 1], ptok, pw, tp
+
+    def dequant_resident(self, layer, expert, which):
+        H, F, E = self.cfg["hidden"], self.cfg["ffn"], self.cfg["n_expert"]
+        shape = (E, H) if which == 3 else ((F, H) if which < 2 else (H, F))
+        out = torch.empty(shape, dtype=torch.float32, device="cuda")
+        self._check(self.lib.redhip_moe_dequant_resident(self.handle, layer, expert, which, out.data_ptr(), _stream()))
+        return out
+
+
+def dequant_rows(ggml_type, rows, ncols):
+    """rows: uint8 CUDA tensor [nrows, row_bytes] of raw GGUF blocks -> float32 [nrows, ncols]."""
+    lib = load()
+    rows = rows.contiguous()
+    out = torch.empty((rows.shape[0], ncols), dtype=torch.float32, device=rows.device)
+    if not lib.redhip_dequant_rows(ggml_type, rows.data_ptr(), rows.shape[0], ncols, out.data_ptr(), _stream()):
+        raise RedHipError(lib.redhip_moe_last_error().decode())
+    return out
+
+
+def gemv_rows(ggml_type, matrix, ncols, x, row_start=0, row_count=None):
+    lib = load()
+    nrows = matrix.shape[0]
+    if row_count is None:
+        row_count = nrows - row_start
+    out = torch.empty(row_count, dtype=torch.float32, device=x.device)
+    if not lib.redhip_gemv_rows(ggml_type, matrix.data_ptr(), ncols, row_start, row_count, x.data_ptr(), out.data_ptr(), _stream()):
+        raise RedHipError(lib.redhip_moe_last_error().decode())
+    return out

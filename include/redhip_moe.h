@@ -1,0 +1,88 @@
+/*
+ * Resident MoE FFN layers - C ABI of libredmetal_hip.so (MI355X / gfx950).
+ *
+ * The production path: every expert of every layer stays in HBM, and one call runs the whole FFN of a layer
+ * for 1..max_tokens tokens on a HIP stream without touching the host:
+ *   router GEMV -> softmax top-k -> (token grouping) -> routed experts -> shared expert -> combine.
+ * It stands where the reference has the resident top-k pool with its residency table and stream-encoded
+ * execution (native/redmetal_topk.h:107-170, encode_device / encode_device_tail / encode_batched) driven by
+ * emit_ffn_pre_opt + emit_layer_experts (native/redmetal_engine.m:1733-1765,1800-1863) and, for chunks,
+ * prefill_chunk (native/redmetal_engine_prefill.m:1238-1300). The opaque Metal objects of those calls
+ * (id<MTLCommandBuffer>, id<MTLBuffer>) become a hipStream_t and device pointers.
+ *
+ * Conventions follow the pool families: int 1 = success / 0 = failure, message via redhip_moe_last_error()
+ * (thread-local), abi_version() == 1, handles made and destroyed by the caller, destroy(NULL) is a no-op.
+ * `*_dev` arguments are device pointers; `stream` is a hipStream_t (NULL = the default stream). Calls that
+ * take a stream only enqueue work. One forward at a time per handle: the handle owns the workspace.
+ */
+#pragma once
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *redhip_moe_t;
+
+typedef struct {
+    uint32_t hidden;            /* multiple of 256 */
+    uint32_t ffn;               /* multiple of 256 */
+    uint32_t n_expert;          /* <= 1024 */
+    uint32_t top_k;             /* <= 16 */
+    uint32_t n_layer;
+    uint32_t max_tokens;        /* largest ntok of redhip_moe_forward */
+    uint32_t router_type;       /* 0 (F32) or 14 (Q6_K) */
+    uint32_t expert_type_word;  /* gate_up | down << 8, as native/redlite_native_metal.h:69-73; types 16, 21, 14 */
+    uint32_t shared_type_word;  /* same encoding for the shared expert */
+    uint32_t reserved;
+} redhip_moe_config;
+
+uint32_t redhip_moe_abi_version(void);
+const char *redhip_moe_last_error(void);
+
+redhip_moe_t redhip_moe_create(const redhip_moe_config *config);
+void redhip_moe_destroy(redhip_moe_t moe);
+uint64_t redhip_moe_resident_bytes(redhip_moe_t moe);     /* weight bytes held in HBM */
+
+/* One-time uploads of raw GGUF blocks (the layout of native/redlite_native_gguf.c:402-440: rows back to back,
+ * experts contiguous). Sources may be host or device memory. Synchronous. */
+int redhip_moe_load_router(redhip_moe_t moe, uint32_t layer, const void *weights, uint64_t bytes);
+int redhip_moe_load_shared(redhip_moe_t moe, uint32_t layer, const float *gate_inp,
+    const void *gate, uint64_t gate_bytes, const void *up, uint64_t up_bytes, const void *down, uint64_t down_bytes);
+int redhip_moe_load_experts(redhip_moe_t moe, uint32_t layer, uint32_t first_expert, uint32_t count,
+    const void *gate, const void *up, const void *down);   /* count experts, each tightly packed */
+
+/* out_dev[t][hidden] = routed(x_t) + shared(x_t) * sigmoid(gate_inp . x_t), t < ntok. x_dev is [ntok][hidden]
+ * f32. Stream-ordered, no host synchronisation. */
+int redhip_moe_forward(redhip_moe_t moe, uint32_t layer, const float *x_dev, uint32_t ntok, float *out_dev, void *stream);
+
+/* Stream-ordered pieces of the same path (what forward chains), for callers that interleave their own work and
+ * for parity taps. ids_dev [ntok][top_k] u32, weights_dev [ntok][top_k] f32, logits_dev [ntok][n_expert] f32. */
+int redhip_moe_route(redhip_moe_t moe, uint32_t layer, const float *x_dev, uint32_t ntok,
+    uint32_t *ids_dev, float *weights_dev, float *logits_dev, void *stream);
+int redhip_moe_experts(redhip_moe_t moe, uint32_t layer, const float *x_dev, uint32_t ntok,
+    const uint32_t *ids_dev, const float *weights_dev, float *out_dev, void *stream);
+
+/* Routing of the last forward / route on this handle, copied to host after synchronising `stream`. Any may be NULL. */
+int redhip_moe_last_route(redhip_moe_t moe, uint32_t ntok, uint32_t *ids, float *weights, float *logits, void *stream);
+
+/* Token grouping of [ntok][top_k] ids (device), the GPU form of the pair sort in
+ * native/redmetal_engine_prefill.m:1246-1276: uid_dev[U] in first-appearance order, expert_start_dev[U+1],
+ * pair_token_dev[P], pair_weight_dev[P], tok_pair_dev[P], n_unique_dev[1]; P = ntok * top_k. */
+int redhip_moe_group(redhip_moe_t moe, const uint32_t *ids_dev, const float *weights_dev, uint32_t ntok,
+    uint32_t *uid_dev, uint32_t *expert_start_dev, uint32_t *pair_token_dev, float *pair_weight_dev,
+    uint32_t *tok_pair_dev, uint32_t *n_unique_dev, void *stream);
+
+/* Parity tap: f32 dequantisation of `rows` rows of `ncols` weights of raw GGUF blocks (device pointers). */
+int redhip_dequant_rows(uint32_t ggml_type, const void *rows_dev, uint32_t nrows, uint32_t ncols, float *out_dev, void *stream);
+/* Parity tap: dequantise one resident matrix (which: 0 gate, 1 up, 2 down; expert == n_expert: shared expert;
+ * which == 3: the router) from the layout the kernels read. out_dev holds rows x cols floats. */
+int redhip_moe_dequant_resident(redhip_moe_t moe, uint32_t layer, uint32_t expert, uint32_t which, float *out_dev, void *stream);
+
+/* GEMV on device memory: out_dev[r] = W[row_start + r] . x_dev, raw GGUF rows. */
+int redhip_gemv_rows(uint32_t ggml_type, const void *matrix_dev, uint32_t ncols, uint32_t row_start, uint32_t row_count,
+    const float *x_dev, float *out_dev, void *stream);
+
+#ifdef __cplusplus
+}
+#endif

@@ -1,0 +1,64 @@
+/*
+ * Single-expert FFN pool - C ABI of libredmetal_hip.so (MI355X / gfx950).
+ *
+ * Replaces the pool the reference declares in native/redmetal_ffn.h:9-70 and implements in
+ * native/redmetal_ffn.m:425-706. Names, argument meaning, return convention (1 = success, 0 = failure,
+ * message through redmetal_ffn_last_error(), thread-local) and the slot layout gate|up|down are kept, so a
+ * caller of the reference binds this library unchanged. Differences, all additive:
+ *   - ggml_type accepts IQ2_XXS (16), IQ3_S (21), Q6_K (14) and the reference's two-type word
+ *     gate_up | down << 8 (native/redlite_native_metal.h:69-73). IQ2_XS (17) / IQ1_M (29) are rejected with
+ *     a message: they are outside this path.
+ *   - the two grid arguments of pool_create are accepted as the reference requires them (non-NULL, exact
+ *     counts, native/redmetal_ffn.m:223-227) and otherwise unused: the codebooks are built in.
+ *   - slots live in device memory (HBM); load_expert reads the file into pinned host memory and copies.
+ * All pointers are host pointers; every call is synchronous.
+ */
+#pragma once
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+typedef void *redmetal_ffn_pool_t;
+
+/* native/redmetal_ffn.h:11-12, native/redmetal_ffn.m:424-427 */
+uint32_t redmetal_ffn_abi_version(void);
+const char *redmetal_ffn_last_error(void);
+
+/* native/redmetal_ffn.h:14-22, native/redmetal_ffn.m:211-316,429-450. slot size is rounded up to 4096;
+ * capacity = budget / slot size; slabs of slots_per_slab (0 = 64) slots are allocated on first use. */
+redmetal_ffn_pool_t redmetal_ffn_pool_create(const char *model_path, uint64_t budget_bytes, uint64_t slot_bytes,
+    uint32_t slots_per_slab, const int8_t *iq2_xs_grid, uint32_t iq2_xs_grid_count,
+    const int8_t *iq1_m_grid, uint32_t iq1_m_grid_count);
+
+/* native/redmetal_ffn.h:24-31, native/redmetal_ffn.m:452-482 */
+void redmetal_ffn_pool_destroy(redmetal_ffn_pool_t pool);
+uint32_t redmetal_ffn_pool_capacity(redmetal_ffn_pool_t pool);
+uint32_t redmetal_ffn_pool_slab_count(redmetal_ffn_pool_t pool);
+uint64_t redmetal_ffn_pool_allocated_bytes(redmetal_ffn_pool_t pool);
+uint64_t redmetal_ffn_pool_bytes_read(redmetal_ffn_pool_t pool);
+uint64_t redmetal_ffn_pool_read_calls(redmetal_ffn_pool_t pool);
+double redmetal_ffn_pool_read_ms(redmetal_ffn_pool_t pool);
+int redmetal_ffn_pool_slot_inflight(redmetal_ffn_pool_t pool, uint32_t slot_id);
+
+/* native/redmetal_ffn.h:33-43, native/redmetal_ffn.m:484-539: three preads into gate|up|down of the slot */
+int redmetal_ffn_pool_load_expert(redmetal_ffn_pool_t pool, uint32_t slot_id,
+    uint64_t gate_file_offset, uint64_t gate_bytes, uint64_t up_file_offset, uint64_t up_bytes,
+    uint64_t down_file_offset, uint64_t down_bytes, uint64_t *bytes_read, double *elapsed_ms);
+
+/* native/redmetal_ffn.h:45-53, native/redmetal_ffn.m:541-569: device virtual addresses of the three matrices */
+int redmetal_ffn_pool_slot_addresses(redmetal_ffn_pool_t pool, uint32_t slot_id,
+    uint64_t gate_bytes, uint64_t up_bytes, uint64_t down_bytes,
+    uint64_t *gate_address, uint64_t *up_address, uint64_t *down_address);
+
+/* native/redmetal_ffn.h:55-70, native/redmetal_ffn.m:571-706:
+ * output[i] = down[output_row_start + i] . (SiLU(gate . x) * (up . x)), no router weight. */
+int redmetal_ffn_pool_execute_expert(redmetal_ffn_pool_t pool, uint32_t slot_id, uint32_t ggml_type,
+    uint64_t gate_bytes, uint64_t up_bytes, uint64_t down_bytes, uint32_t hidden_size, uint32_t ffn_size,
+    uint32_t output_row_start, uint32_t output_row_count, const float *input, uint32_t input_count,
+    float *output, uint32_t output_count, double *elapsed_ms);
+
+#ifdef __cplusplus
+}
+#endif

@@ -1,0 +1,45 @@
+"""The C-ABI library loads and exports every symbol include/*.h declares (no GPU, no compute calls)."""
+import ctypes
+import glob
+import os
+import re
+
+import pytest
+
+from dwarfstar_red_lite_amd import _lib
+
+ROOT = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+
+
+def declared_symbols():
+    names = set()
+    for h in glob.glob(os.path.join(ROOT, "include", "*.h")):
+        text = re.sub(r"/\*.*?\*/", "", open(h).read(), flags=re.S)
+        text = re.sub(r"//.*", "", text)
+        for m in re.finditer(r"\b((?:redmetal|redhip|rl_native)_[a-z0-9_]+)\s*\(", text):
+            names.add(m.group(1))
+    return names
+
+
+def test_headers_and_library_agree():
+    if not os.path.isfile(_lib.LIB_PATH):
+        pytest.fail("libredmetal_hip.so is not built: run python -m dwarfstar_red_lite_amd.build")
+    names = declared_symbols()
+    assert len(names) >= 35
+    lib = ctypes.CDLL(_lib.LIB_PATH)
+    for n in sorted(names):
+        assert hasattr(lib, n), "library does not export " + n
+    assert names == set(_lib.ABI), names ^ set(_lib.ABI)
+    assert _lib.load().redmetal_ffn_abi_version() == 1
+
+
+def test_error_strings_without_device_work():
+    lib = _lib.load()
+    assert lib.redmetal_ffn_pool_create(None, 0, 0, 0, None, 0, None, 0) is None
+    assert b"invalid Red Metal FFN pool arguments" in lib.redmetal_ffn_last_error()
+    lib.redmetal_ffn_pool_destroy(None)
+    lib.redhip_moe_destroy(None)
+    assert lib.redhip_moe_create(None) is None
+    assert b"null MoE config" in lib.redhip_moe_last_error()
+    assert lib.redmetal_quant_rows(None, 0, 0, 16, 256, 1, 0, 1, None, 256, None, 0, None, 1, None, None) == 0
+    assert b"invalid Red Metal mixed-quant arguments" in lib.redmetal_quant_last_error()
