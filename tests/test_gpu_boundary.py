@@ -73,7 +73,7 @@ def test_ffn_pool(model_file):
     from dwarfstar_red_lite_amd import RedHipError
     path, blob, index, H, F = model_file
     x = synth.normed_x(np.random.default_rng(2), 1, H)[0]
-    slot_bytes = 2 * index["f2.gate.0"][1] + index["f2.down.0"][1]
+    slot_bytes = 2 * index["q6.gate"][1] + index["q6.down"][1]      # the largest of the three families
     aligned = (slot_bytes + 4095) // 4096 * 4096
     with RedMetalFfnPool(path, 5 * aligned + 100, slot_bytes, slots_per_slab=2) as pool:
         assert pool.capacity == 5 and pool.telemetry()["slab_count"] == 0
@@ -81,7 +81,7 @@ def test_ffn_pool(model_file):
             for e in range(3 if fam != "q6" else 1):
                 sfx = ".%d" % e if fam != "q6" else ""
                 lay = ExpertLayout(*index[fam + ".gate" + sfx], *index[fam + ".up" + sfx], *index[fam + ".down" + sfx])
-                slot = (e + 1) % 5
+                slot = 4 if fam == "q6" else (e + 1) % 5      # slots 1..4: three slabs of two slots, the last one short
                 info = pool.load(slot, lay)
                 assert info["bytes_read"] == lay.gate_bytes + lay.up_bytes + lay.down_bytes
                 g, u, d = pool.addresses(slot, lay)
