@@ -1,0 +1,229 @@
+#!/usr/bin/env python3
+"""MoE FFN layer benchmark on one MI355X.
+
+A step is one pass of the hot path over one batch: router GEMV -> softmax top-k -> routed experts -> shared expert
+-> combine for `--batch` tokens through ONE resident MoE layer. Steps cycle through `--layers` resident layers
+(distinct weights, so the 256 MB Infinity Cache cannot hold the working set) and through a pool of activations, so
+the router picks different experts every step. Inputs are resident in HBM before the timed region starts.
+
+Prints one JSON line (metric: microseconds per token for one MoE layer; lower is better), with
+  roofline      the dominant kernel's algorithmic bytes per launch / its measured launch duration, vs 8 TB/s
+  cpu_baseline  the CPU oracle (a port of the reference's scalar double-accumulating path) on this host's cores
+"""
+import argparse
+import ctypes as C
+import json
+import os
+import sys
+import time
+
+ROOT = os.path.dirname(os.path.abspath(__file__))
+for p in (ROOT, os.path.join(ROOT, "oracle")):
+    if p not in sys.path:
+        sys.path.insert(0, p)
+
+HBM_PEAK_GBS = 8000.0
+
+
+def parse():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=480)
+    ap.add_argument("--warmup", type=int, default=96)
+    ap.add_argument("--layout", choices=["iq2", "f2"], default="iq2", help="iq2: BASELINE config 1 (all IQ2_XXS, F32 router); f2: config 2 layout")
+    ap.add_argument("--layers", type=int, default=48, help="resident layers the steps cycle through")
+    ap.add_argument("--batch", type=int, default=1)
+    ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
+    return ap.parse_args()
+
+
+def synth_layer_on_gpu(torch, gen, cfg):
+    """Random-valid blocks generated on the GPU (same construction as dwarfstar_red_lite_amd.synth, torch RNG)."""
+    from dwarfstar_red_lite_amd import synth
+
+    def rows(t, nrows, ncols, d_range=None):
+        bb, off = synth.BLOCK_BYTES[t], synth.D_OFFSET[t]
+        nb = nrows * (ncols // 256)
+        raw = torch.randint(0, 256, (nb, bb), dtype=torch.uint8, device="cuda", generator=gen)
+        lo, hi = d_range or synth.D_RANGE[t]
+        d = (lo + (hi - lo) * torch.rand(nb, device="cuda", generator=gen)).to(torch.float16).view(torch.uint8).reshape(nb, 2)
+        raw[:, off:off + 2] = d
+        return raw.reshape(nrows, -1)
+
+    H, F, E = cfg["hidden"], cfg["ffn"], cfg["n_expert"]
+    a = {}
+    if cfg["router_type"] == 0:
+        a["router"] = 0.02 * torch.randn((E, H), device="cuda", generator=gen)
+    else:
+        a["router"] = rows(cfg["router_type"], E, H, d_range=(1e-5, 3e-5))
+    a["gate"] = rows(cfg["gate_up_type"], E * F, H).reshape(E, -1)
+    a["up"] = rows(cfg["gate_up_type"], E * F, H).reshape(E, -1)
+    a["down"] = rows(cfg["down_type"], E * H, F).reshape(E, -1)
+    a["sh_gate"] = rows(cfg["sh_gate_up_type"], F, H)
+    a["sh_up"] = rows(cfg["sh_gate_up_type"], F, H)
+    a["sh_down"] = rows(cfg["sh_down_type"], H, F)
+    a["sh_gate_inp"] = 0.02 * torch.randn(H, device="cuda", generator=gen)
+    return a
+
+
+def layer_bytes(cfg, distinct_experts, batch):
+    """Algorithmic bytes of one step: weights that must be read once + activations in and out."""
+    from dwarfstar_red_lite_amd import synth
+    H, F, E = cfg["hidden"], cfg["ffn"], cfg["n_expert"]
+    expert = 2 * F * synth.row_bytes(cfg["gate_up_type"], H) + H * synth.row_bytes(cfg["down_type"], F)
+    shared = 2 * F * synth.row_bytes(cfg["sh_gate_up_type"], H) + H * synth.row_bytes(cfg["sh_down_type"], F)
+    router = E * synth.row_bytes(cfg["router_type"], H)
+    return {"expert_bytes": distinct_experts * expert + shared, "router_bytes": router, "gate_inp_bytes": 4 * H,
+            "act_bytes": 2 * 4 * H * batch, "one_expert": expert, "shared": shared}
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    import numpy as np
+    import torch
+
+    from dwarfstar_red_lite_amd import load, synth
+    from dwarfstar_red_lite_amd.moe import ResidentMoe
+
+    lib = load()
+    torch.cuda.init()
+    cfg = synth.layer_config(layout=args.layout)
+    B, NL = args.batch, args.layers
+    moe = ResidentMoe(cfg, n_layer=NL, max_tokens=B)
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(20241125)
+    layer0 = None
+    for l in range(NL):
+        a = synth_layer_on_gpu(torch, gen, cfg)
+        moe.load_layer(l, a)
+        if l == 0:
+            layer0 = {k: v.cpu().numpy() for k, v in a.items()}
+            if cfg["router_type"] != 0:
+                layer0["router"] = layer0["router"].view(np.uint8)
+        del a
+    torch.cuda.synchronize()
+
+    NX = 64
+    xs_host = synth.normed_x(np.random.default_rng(99), NX * B, cfg["hidden"]).reshape(NX, B, cfg["hidden"])
+    xs = torch.from_numpy(xs_host).cuda()
+    outs = torch.empty_like(xs)
+    stream = torch.cuda.Stream()
+
+    def step(i):
+        moe.forward(i % NL, xs[i % NX], outs[i % NX])
+
+    # ---- parity gate on the very tensors the timed steps use (layer 0, CPU oracle) ----
+    import oracle_lib as orc
+    ref = orc.Layer(cfg, **layer0)
+    with torch.cuda.stream(stream):
+        step(0)
+        gids, _, _ = moe.last_route(B)
+    want, cids, _, _ = ref.forward(xs_host[0], threads=os.cpu_count() or 1)
+    got = outs[0].cpu().numpy()
+    rel = float(np.linalg.norm(got - want) / np.linalg.norm(want))
+    ids_ok = bool(np.array_equal(gids, cids))
+    if rel > 1e-3:
+        print("PARITY FAILURE: rel L2 %.3g vs the CPU oracle" % rel, file=sys.stderr)
+        sys.exit(1)
+
+    # ---- timed region ----
+    K, W = args.steps, args.warmup
+    with torch.cuda.stream(stream):
+        for i in range(W):
+            step(i)
+        stream.synchronize()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        for i in range(K):
+            step(W + i)
+        stream.synchronize()
+        torch.cuda.synchronize()
+        t1 = time.perf_counter()
+        ms_per_step = (t1 - t0) * 1e3 / K
+
+        # the same K steps again with per-kernel begin/end timestamps (HIP events on the launch stream)
+        n_stage = lib.redhip_profile_stage_count()
+        lib.redhip_profile_begin()
+        for i in range(K):
+            step(W + i)
+        stage_ms = (C.c_double * n_stage)()
+        stage_n = (C.c_uint32 * n_stage)()
+        lib.redhip_profile_end(stage_ms, stage_n, n_stage)
+        # distinct routed experts per step (B > 1 shares experts between tokens)
+        distinct = []
+        for i in range(min(K, NX)):
+            step(W + i)
+            ids, _, _ = moe.last_route(B)
+            distinct.append(len(set(ids.ravel().tolist())))
+    stages = {lib.redhip_profile_stage_name(s).decode(): {"ms_total": stage_ms[s], "launches": int(stage_n[s]),
+                                                        "us_avg": 1e3 * stage_ms[s] / stage_n[s]}
+              for s in range(n_stage) if stage_n[s]}
+    mean_distinct = float(np.mean(distinct))
+    lb = layer_bytes(cfg, mean_distinct, B)
+
+    # dominant kernel = the stage with the largest total time; its algorithmic bytes per launch
+    dom = max(stages, key=lambda k: stages[k]["ms_total"])
+    H, F = cfg["hidden"], cfg["ffn"]
+    gate_up = lb["one_expert"] - H * synth.row_bytes(cfg["down_type"], F)
+    per_launch = {
+        "router_gemv": lb["router_bytes"] / 1 + 4 * H + 4 * cfg["n_expert"],
+        "gateup": mean_distinct * gate_up + 4 * H,
+        "shared_gateup": 2 * F * synth.row_bytes(cfg["sh_gate_up_type"], H) + 4 * H,
+        "down_combine": mean_distinct * (lb["one_expert"] - gate_up) + H * synth.row_bytes(cfg["sh_down_type"], F) + 4 * H,
+        "fused_experts": lb["expert_bytes"] + 2 * 4 * H,
+    }
+    dom_bytes = per_launch.get(dom)
+    dom_us = stages[dom]["us_avg"] * (stages[dom]["launches"] / K)        # per step, if launched more than once per step
+    roofline = None
+    if dom_bytes:
+        achieved = dom_bytes / (dom_us * 1e-6) / 1e9
+        roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                    "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                    "bytes_per_launch": int(dom_bytes), "launch_us": round(dom_us, 3)}
+
+    us_per_token = ms_per_step * 1e3 / B
+    total_bytes = lb["expert_bytes"] + lb["router_bytes"] + lb["gate_inp_bytes"] + lb["act_bytes"]
+    result = {
+        "metric": "moe_ffn_layer_us_per_token", "value": round(us_per_token, 3), "unit": "us/token", "n_gpus": 1,
+        "steps": K, "warmup": W, "ms_per_step": round(ms_per_step, 6), "higher_is_better": False, "scaling": "weak",
+        "vs_baseline": None, "dtype": "f32", "data": "synthetic",
+        "config": {"workload": "config1: one MoE FFN layer, B=%d decode token(s), hidden 2048, 512 experts top-10 + shared, ffn 512, layout %s, "
+                               "all experts of %d layers resident" % (B, args.layout, NL),
+                   "layout": args.layout, "batch": B, "resident_layers": NL, "resident_gb": round(moe.resident_bytes / 1e9, 2),
+                   "mean_distinct_routed_experts": mean_distinct},
+        "layer_gbps": {"expert_bytes": int(lb["expert_bytes"]), "layer_bytes": int(total_bytes),
+                       "expert_gbps": round(lb["expert_bytes"] / (ms_per_step * 1e-3) / 1e9, 1),
+                       "layer_gbps": round(total_bytes / (ms_per_step * 1e-3) / 1e9, 1),
+                       "frac_of_peak_on_expert_bytes": round(lb["expert_bytes"] / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
+        "stages_us": {k: round(v["us_avg"] * v["launches"] / K, 3) for k, v in stages.items()},
+        "parity": {"rel_l2_vs_cpu_oracle": rel, "router_ids_identical": ids_ok},
+        "roofline": roofline,
+    }
+
+    # ---- CPU baseline: the oracle on this host's cores, layer 0, same activations ----
+    if not args.no_cpu:
+        cores = min(os.cpu_count() or 1, 64)
+        reps, t_cpu, budget = 0, 0.0, 12.0
+        while t_cpu < budget and reps < 400:
+            tc = time.perf_counter()
+            ref.forward(xs_host[reps % NX], threads=cores)
+            t_cpu += time.perf_counter() - tc
+            reps += 1
+        cpu_us = t_cpu * 1e6 / (reps * B)
+        t1c = time.perf_counter()
+        ref.forward(xs_host[0], threads=1)
+        one_us = (time.perf_counter() - t1c) * 1e6 / B
+        result["cpu_baseline"] = {"value": round(cpu_us, 1), "unit": "us/token", "cores": cores, "kind": "port",
+                                  "sample": "%d forwards of layer 0 (same weights and activations as the GPU run), rows split over %d pthreads "
+                                            "per matvec like the reference; 1 thread: %.0f us/token" % (reps, cores, one_us),
+                                  "gpu_speedup": round(cpu_us / us_per_token, 1)}
+    print(json.dumps(result))
+    moe.close()
+
+
+if __name__ == "__main__":
+    main()

@@ -63,6 +63,10 @@ ABI = {
     "redhip_dequant_rows": (i32, [u32, vp, u32, u32, vp, vp]),
     "redhip_moe_dequant_resident": (i32, [vp, u32, u32, u32, vp, vp]),
     "redhip_gemv_rows": (i32, [u32, vp, u32, u32, u32, vp, vp, vp]),
+    "redhip_profile_stage_count": (u32, []),
+    "redhip_profile_stage_name": (C.c_char_p, [u32]),
+    "redhip_profile_begin": (i32, []),
+    "redhip_profile_end": (i32, [C.POINTER(dbl), C.POINTER(u32), u32]),
 }
 
 _lib = None

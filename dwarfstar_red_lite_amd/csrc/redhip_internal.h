@@ -1,6 +1,7 @@
 // Internal interface between the C-ABI front ends and the gfx950 kernels of libredmetal_hip.so.
 #pragma once
 #include <hip/hip_runtime.h>
+#include <hip/hip_ext.h>
 #include <stddef.h>
 #include <stdint.h>
 
@@ -20,6 +21,23 @@ inline bool quant_supported(uint32_t t) { return block_bytes(t) != 0u; }
 // the reference's two-type word: gate/up in bits 0-7, down in bits 8-15 when it differs
 inline uint32_t word_gate_up(uint32_t w) { return w & 255u; }
 inline uint32_t word_down(uint32_t w) { return ((w >> 8) & 255u) ? ((w >> 8) & 255u) : (w & 255u); }
+
+// ---- per-stage kernel timing (off unless redhip_profile_begin was called) ----
+// When on, every kernel launch carries a start and a stop event whose timestamps are the dispatch's own begin
+// and end, so a stage's time is kernel execution only, not launch latency.
+enum Stage : uint32_t {
+    ST_OTHER = 0, ST_ROUTER_GEMV, ST_ROUTE_SELECT, ST_GROUP, ST_GATEUP, ST_SHARED_GATEUP, ST_DOWN_COMBINE,
+    ST_FUSED_EXPERTS, ST_BATCH_GATEUP, ST_BATCH_DOWN, ST_BATCH_COMBINE, ST_PREFILL_GATEUP, ST_PREFILL_DOWN, ST_COUNT
+};
+void prof_set_stage(uint32_t stage);                       // label of the launches that follow (calling thread)
+void prof_events(hipEvent_t *start, hipEvent_t *stop);     // both nullptr when profiling is off
+
+#define REDHIP_LAUNCH(kern, grid, block, lds, stream, ...)                                         \
+    do {                                                                                           \
+        hipEvent_t ev_a_ = nullptr, ev_b_ = nullptr;                                               \
+        ::redhip::prof_events(&ev_a_, &ev_b_);                                                     \
+        hipExtLaunchKernelGGL(kern, grid, block, lds, stream, ev_a_, ev_b_, 0u, __VA_ARGS__);      \
+    } while (0)
 
 // ---- launchers (enqueue only; return hipSuccess or the launch error) ----
 

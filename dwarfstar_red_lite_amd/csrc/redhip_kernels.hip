@@ -71,10 +71,10 @@ hipError_t launch_dequant_rows(uint32_t type, const void *rows, uint32_t nrows, 
     const dim3 grid((uint32_t)((total + 255u) / 256u));
     const uint8_t *p = static_cast<const uint8_t *>(rows);
     switch (type) {
-        case T_IQ2_XXS: dequant_rows_kernel<T_IQ2_XXS><<<grid, 256, 0, s>>>(p, rb, nrows, cpr, out); break;
-        case T_IQ3_S: dequant_rows_kernel<T_IQ3_S><<<grid, 256, 0, s>>>(p, rb, nrows, cpr, out); break;
-        case T_Q6_K: dequant_rows_kernel<T_Q6_K><<<grid, 256, 0, s>>>(p, rb, nrows, cpr, out); break;
-        case T_F32: dequant_rows_kernel<T_F32><<<grid, 256, 0, s>>>(p, rb, nrows, cpr, out); break;
+        case T_IQ2_XXS: REDHIP_LAUNCH(dequant_rows_kernel<T_IQ2_XXS>, dim3(grid), dim3(256), 0, s, p, rb, nrows, cpr, out); break;
+        case T_IQ3_S: REDHIP_LAUNCH(dequant_rows_kernel<T_IQ3_S>, dim3(grid), dim3(256), 0, s, p, rb, nrows, cpr, out); break;
+        case T_Q6_K: REDHIP_LAUNCH(dequant_rows_kernel<T_Q6_K>, dim3(grid), dim3(256), 0, s, p, rb, nrows, cpr, out); break;
+        case T_F32: REDHIP_LAUNCH(dequant_rows_kernel<T_F32>, dim3(grid), dim3(256), 0, s, p, rb, nrows, cpr, out); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
@@ -105,10 +105,10 @@ static hipError_t gemv_dispatch(const uint8_t *w, uint32_t ncols, uint32_t row_s
     const dim3 grid((row_count + 256u / lpr - 1u) / (256u / lpr));
     const size_t lds = padded_floats(ncols) * sizeof(float);
     switch (lpr) {
-        case 64: gemv_rows_kernel<T, 64><<<grid, 256, lds, s>>>(w, rb, ncols, row_start, row_count, x, out); break;
-        case 32: gemv_rows_kernel<T, 32><<<grid, 256, lds, s>>>(w, rb, ncols, row_start, row_count, x, out); break;
-        case 16: gemv_rows_kernel<T, 16><<<grid, 256, lds, s>>>(w, rb, ncols, row_start, row_count, x, out); break;
-        default: gemv_rows_kernel<T, 8><<<grid, 256, lds, s>>>(w, rb, ncols, row_start, row_count, x, out); break;
+        case 64: REDHIP_LAUNCH((gemv_rows_kernel<T, 64>), dim3(grid), dim3(256), lds, s, w, rb, ncols, row_start, row_count, x, out); break;
+        case 32: REDHIP_LAUNCH((gemv_rows_kernel<T, 32>), dim3(grid), dim3(256), lds, s, w, rb, ncols, row_start, row_count, x, out); break;
+        case 16: REDHIP_LAUNCH((gemv_rows_kernel<T, 16>), dim3(grid), dim3(256), lds, s, w, rb, ncols, row_start, row_count, x, out); break;
+        default: REDHIP_LAUNCH((gemv_rows_kernel<T, 8>), dim3(grid), dim3(256), lds, s, w, rb, ncols, row_start, row_count, x, out); break;
     }
     return hipGetLastError();
 }
@@ -138,7 +138,7 @@ __global__ void silu_mul_kernel(const float *gate, const float *up, float *act, 
 }
 
 hipError_t launch_silu_mul(const float *gate, const float *up, float *act, uint32_t n, hipStream_t s) {
-    silu_mul_kernel<<<(n + 255u) / 256u, 256, 0, s>>>(gate, up, act, n);
+    REDHIP_LAUNCH(silu_mul_kernel, dim3((n + 255u) / 256u), dim3(256), 0, s, gate, up, act, n);
     return hipGetLastError();
 }
 
@@ -244,7 +244,7 @@ hipError_t launch_route_select(const float *logits, uint32_t ntok, uint32_t n_ex
                                const float *gate_inp, const float *x, uint32_t hidden, float *scalar, hipStream_t s) {
     if (!ntok || !n_expert || n_expert > 1024u || !top_k || top_k > 16u || top_k > n_expert) return hipErrorInvalidValue;
     if (scalar && (!gate_inp || !x)) return hipErrorInvalidValue;
-    route_select_kernel<<<ntok, 256, 0, s>>>(logits, n_expert, top_k, ids, weights, probs, gate_inp, x, hidden, scalar);
+    REDHIP_LAUNCH(route_select_kernel, dim3(ntok), dim3(256), 0, s, logits, n_expert, top_k, ids, weights, probs, gate_inp, x, hidden, scalar);
     return hipGetLastError();
 }
 
@@ -281,10 +281,10 @@ static hipError_t gateup_dispatch(const ExpertSet &ex, const uint32_t *ids, uint
     const dim3 grid((ffn + 256u / lpr - 1u) / (256u / lpr), n_slot);
     const size_t lds = padded_floats(hidden) * sizeof(float);
     switch (lpr) {
-        case 64: moe_gateup_kernel<T, 64><<<grid, 256, lds, s>>>(ex.base, ex.stride, ex.gate_bytes, ids, hidden, ffn, x, act); break;
-        case 32: moe_gateup_kernel<T, 32><<<grid, 256, lds, s>>>(ex.base, ex.stride, ex.gate_bytes, ids, hidden, ffn, x, act); break;
-        case 16: moe_gateup_kernel<T, 16><<<grid, 256, lds, s>>>(ex.base, ex.stride, ex.gate_bytes, ids, hidden, ffn, x, act); break;
-        default: moe_gateup_kernel<T, 8><<<grid, 256, lds, s>>>(ex.base, ex.stride, ex.gate_bytes, ids, hidden, ffn, x, act); break;
+        case 64: REDHIP_LAUNCH((moe_gateup_kernel<T, 64>), dim3(grid), dim3(256), lds, s, ex.base, ex.stride, ex.gate_bytes, ids, hidden, ffn, x, act); break;
+        case 32: REDHIP_LAUNCH((moe_gateup_kernel<T, 32>), dim3(grid), dim3(256), lds, s, ex.base, ex.stride, ex.gate_bytes, ids, hidden, ffn, x, act); break;
+        case 16: REDHIP_LAUNCH((moe_gateup_kernel<T, 16>), dim3(grid), dim3(256), lds, s, ex.base, ex.stride, ex.gate_bytes, ids, hidden, ffn, x, act); break;
+        default: REDHIP_LAUNCH((moe_gateup_kernel<T, 8>), dim3(grid), dim3(256), lds, s, ex.base, ex.stride, ex.gate_bytes, ids, hidden, ffn, x, act); break;
     }
     return hipGetLastError();
 }
@@ -347,7 +347,7 @@ static hipError_t down_dispatch(const ExpertSet &ex, const uint32_t *ids, const 
     const size_t lds = (size_t)(top_k + 1u) * padded_floats(ffn) * sizeof(float);
     const uint8_t *shd = sh.base ? sh.base + sh.gate_bytes + sh.up_bytes : nullptr;
     const uint64_t off = ex.gate_bytes + ex.up_bytes;
-#define REDHIP_DOWN(L) moe_down_combine_kernel<TD, TS, L><<<grid, 256, lds, s>>>(ex.base, ex.stride, off, ids, weights, top_k, shd, scalar, hidden, ffn, act, sh_act, out)
+#define REDHIP_DOWN(L) REDHIP_LAUNCH((moe_down_combine_kernel<TD, TS, L>), dim3(grid), dim3(256), lds, s, ex.base, ex.stride, off, ids, weights, top_k, shd, scalar, hidden, ffn, act, sh_act, out)
     switch (lpr) {
         case 64: REDHIP_DOWN(64); break;
         case 32: REDHIP_DOWN(32); break;
@@ -462,7 +462,7 @@ hipError_t launch_group_pairs(const uint32_t *ids, const float *weights, uint32_
         if (e != hipSuccess) return e;
         attr_set = true;
     }
-    group_pairs_kernel<<<1, 1024, lds, s>>>(ids, weights, ntok, top_k, n_expert, uid, expert_start, pair_token, pair_weight, tok_pair, n_unique);
+    REDHIP_LAUNCH(group_pairs_kernel, dim3(1), dim3(1024), lds, s, ids, weights, ntok, top_k, n_expert, uid, expert_start, pair_token, pair_weight, tok_pair, n_unique);
     return hipGetLastError();
 }
 

@@ -76,9 +76,13 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
     const redhip_moe_config &c = m->cfg;
     if (ntok != 1u) { moe_err("batched expert execution is not available in this build (ntok=%u)", ntok); return 0; }
     const ExpertSet ex = m->routed(layer), sh = m->shared(layer);
+    prof_set_stage(ST_GATEUP);
     HIP_OK(launch_moe_gateup(ex, ids, c.top_k, c.hidden, c.ffn, x, m->act, s), "routed gate/up launch");
+    prof_set_stage(ST_SHARED_GATEUP);
     HIP_OK(launch_moe_gateup(sh, nullptr, 1u, c.hidden, c.ffn, x, m->sh_act, s), "shared gate/up launch");
+    prof_set_stage(ST_DOWN_COMBINE);
     HIP_OK(launch_moe_down_combine(ex, ids, weights, c.top_k, sh, m->scalar, c.hidden, c.ffn, m->act, m->sh_act, out, s), "down/combine launch");
+    prof_set_stage(ST_OTHER);
     return 1;
 }
 
@@ -218,11 +222,14 @@ int redhip_moe_route(redhip_moe_t h, uint32_t layer, const float *x_dev, uint32_
     if (!x_dev || !ntok || ntok > c.max_tokens) { moe_err("invalid token count %u (max %u)", ntok, c.max_tokens); return 0; }
     hipStream_t s = static_cast<hipStream_t>(stream);
     float *lg = logits_dev ? logits_dev : m->logits;
+    prof_set_stage(ST_ROUTER_GEMV);
     for (uint32_t t = 0; t < ntok; ++t)
         HIP_OK(launch_gemv_rows(c.router_type, m->layers[layer].router, c.hidden, 0u, c.n_expert, x_dev + (size_t)t * c.hidden,
                                 lg + (size_t)t * c.n_expert, s), "router GEMV launch");
+    prof_set_stage(ST_ROUTE_SELECT);
     HIP_OK(launch_route_select(lg, ntok, c.n_expert, c.top_k, ids_dev ? ids_dev : m->ids, weights_dev ? weights_dev : m->weights, nullptr,
                                m->layers[layer].gate_inp, x_dev, c.hidden, m->scalar, s), "router selection launch");
+    prof_set_stage(ST_OTHER);
     return 1;
 }
 
@@ -265,6 +272,7 @@ int redhip_moe_group(redhip_moe_t h, const uint32_t *ids_dev, const float *weigh
         moe_err("invalid grouping arguments");
         return 0;
     }
+    prof_set_stage(ST_GROUP);
     HIP_OK(launch_group_pairs(ids_dev, weights_dev, ntok, m->cfg.top_k, m->cfg.n_expert, uid_dev, expert_start_dev, pair_token_dev,
                               pair_weight_dev, tok_pair_dev, n_unique_dev, static_cast<hipStream_t>(stream)), "grouping launch");
     return 1;

@@ -83,6 +83,15 @@ int redhip_moe_dequant_resident(redhip_moe_t moe, uint32_t layer, uint32_t exper
 int redhip_gemv_rows(uint32_t ggml_type, const void *matrix_dev, uint32_t ncols, uint32_t row_start, uint32_t row_count,
     const float *x_dev, float *out_dev, void *stream);
 
+/* Per-stage kernel timing, the counterpart of the reference's RL_ENGINE_PROFILE stage timers
+ * (native/redmetal_engine.m:1150-1164). Between begin and end every kernel this library launches is bracketed
+ * by events that take the dispatch's own begin/end timestamps; end synchronises the device and returns, per
+ * stage, the summed kernel time in ms and the number of launches. Process-wide, for benchmarks. */
+uint32_t redhip_profile_stage_count(void);
+const char *redhip_profile_stage_name(uint32_t stage);
+int redhip_profile_begin(void);
+int redhip_profile_end(double *stage_ms, uint32_t *stage_launches, uint32_t n_stage);
+
 #ifdef __cplusplus
 }
 #endif
