@@ -7,13 +7,11 @@
 #include <stdint.h>
 
 #include "redhip_internal.h"
+#define REDHIP_TABLE_ATTR __device__
 #include "redhip_tables.h"
 
 namespace redhip {
 
-// codebooks in device memory (filled from redhip_tables.h at load time; read through the vector L1 or copied to LDS)
-extern __device__ uint64_t g_iq2xxs_grid[256];
-extern __device__ uint32_t g_iq3s_grid[512];
 
 __device__ __forceinline__ uint32_t ld_u16(const uint8_t *p) { return *reinterpret_cast<const uint16_t *>(p); }
 __device__ __forceinline__ uint32_t ld_u32_a2(const uint8_t *p) {   // 4 bytes at a 2-byte aligned address
@@ -58,7 +56,7 @@ template <> __device__ __forceinline__ void decode32<T_IQ2_XXS>(const uint8_t *r
     const float db = d * (0.5f + (float)(aux >> 28)) * 0.25f;
 #pragma unroll
     for (uint32_t l = 0; l < 4u; ++l) {
-        const uint64_t mag = g_iq2xxs_grid[(idx4 >> (8u * l)) & 255u];
+        const uint64_t mag = redhip_iq2xxs_grid[(idx4 >> (8u * l)) & 255u];
         const uint32_t s7 = (aux >> (7u * l)) & 127u;
         const uint32_t s8 = s7 | ((__popc(s7) & 1u) << 7);
 #pragma unroll
@@ -81,7 +79,7 @@ template <> __device__ __forceinline__ void decode32<T_IQ3_S>(const uint8_t *row
         const uint32_t pair = (l < 2u ? qs_lo >> (16u * l) : qs_hi >> (16u * (l - 2u))) & 0xffffu;
         const uint32_t ia = (pair & 255u) | ((qh << (8u - 2u * l)) & 256u);
         const uint32_t ib = (pair >> 8) | ((qh << (7u - 2u * l)) & 256u);
-        const uint32_t wa = g_iq3s_grid[ia], wb = g_iq3s_grid[ib];
+        const uint32_t wa = redhip_iq3s_grid[ia], wb = redhip_iq3s_grid[ib];
         const uint32_t sg = (sg4 >> (8u * l)) & 255u;
 #pragma unroll
         for (uint32_t j = 0; j < 4u; ++j) {

@@ -1,0 +1,665 @@
+// Decode path over packed IQ2_XXS, three launches per layer, no atomics and no device-scope fences (on this
+// hardware a grid-wide __threadfence costs tens of microseconds and same-address float atomics serialise):
+//
+//   router_*_kernel        logits of every expert (plus the shared expert's gate logit) and the fp16 split of x
+//   gateup_select_kernel   every workgroup repeats the cheap softmax top-k from the logits, then computes 32 gate
+//                          rows + 32 up rows of one selected expert (or the shared expert) -> SwiGLU -> fp16 halves
+//   down_combine_kernel    8 output rows per workgroup, one wave per selected expert; weighted sum in selection
+//                          order + shared expert * scalar gate: deterministic
+//
+// Arithmetic: a weight is (sign * magnitude * (2*scale+1)) * d/8 with sign*magnitude looked up as eight exact
+// fp16 values from LDS tables; an activation vector is split into two fp16 halves (hi + lo*2^-11, after a
+// power-of-two pre-scale), and v_mfma_f32_4x4x4_16B_f16 multiplies four weights of four rows by both halves per
+// lane with fp32 accumulation. Per-group scales and d are applied to the fp32 sums.
+//
+// Layout ("packed IQ2_XXS"): the 66-byte blocks are split at upload into an 8-byte stream [row][group] (4 grid
+// indices + 28 sign bits + 4 scale bits per 32 weights) and an fp16 stream [row][block] (d per 256 weights), both
+// naturally aligned. Same total bytes as the GGUF blocks.
+#include <hip/hip_fp16.h>
+
+#include "redhip_decode.h"
+
+namespace redhip {
+
+typedef _Float16 half4_t __attribute__((ext_vector_type(4)));
+typedef float float4_t __attribute__((ext_vector_type(4)));
+
+// ---------------------------------------------------------------- repacking (upload time)
+
+// raw rows [nrows][K/256 blocks of 66 B] -> qs [nrows][K/32] uint2, ds [nrows][K/256] u16      (col_major = 0)
+//                                        -> qs [K/32][nrows] uint2, ds [K/256][nrows] u16      (col_major = 1)
+__global__ void repack_iq2xxs_kernel(const uint8_t *raw0, uint64_t raw_stride, uint32_t nrows, uint32_t K, int col_major,
+                                     uint8_t *packed0, uint64_t packed_stride) {
+    const uint32_t groups = K / 32u, blocks = K / 256u;
+    const uint8_t *raw = raw0 + (uint64_t)blockIdx.y * raw_stride;          // blockIdx.y = matrix of the batch
+    uint2 *qs = reinterpret_cast<uint2 *>(packed0 + (uint64_t)blockIdx.y * packed_stride);
+    uint16_t *ds = reinterpret_cast<uint16_t *>(packed0 + (uint64_t)blockIdx.y * packed_stride + (uint64_t)nrows * groups * 8u);
+    const uint64_t gid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= (uint64_t)nrows * groups) return;
+    const uint32_t r = (uint32_t)(gid / groups), g = (uint32_t)(gid % groups);
+    const uint8_t *bp = raw + ((uint64_t)r * blocks + (g >> 3)) * 66u;
+    const uint2 v = make_uint2(ld_u32_a2(bp + 2u + 8u * (g & 7u)), ld_u32_a2(bp + 6u + 8u * (g & 7u)));
+    if (col_major) qs[(uint64_t)g * nrows + r] = v; else qs[(uint64_t)r * groups + g] = v;
+    if ((g & 7u) == 0u) {
+        const uint16_t d = (uint16_t)ld_u16(bp);
+        if (col_major) ds[(uint64_t)(g >> 3) * nrows + r] = d; else ds[(uint64_t)r * blocks + (g >> 3)] = d;
+    }
+}
+
+hipError_t launch_repack_iq2xxs(const void *raw, uint64_t raw_stride, uint32_t count, uint32_t nrows, uint32_t K, bool col_major,
+                                void *packed, uint64_t packed_stride, hipStream_t s) {
+    if (!nrows || !K || K % 256u || !count || count > 65535u) return hipErrorInvalidValue;
+    const uint64_t total = (uint64_t)nrows * (K / 32u);
+    REDHIP_LAUNCH(repack_iq2xxs_kernel, dim3((uint32_t)((total + 255u) / 256u), count), dim3(256), 0, s,
+                  static_cast<const uint8_t *>(raw), raw_stride, nrows, K, col_major ? 1 : 0, static_cast<uint8_t *>(packed), packed_stride);
+    return hipGetLastError();
+}
+
+// parity tap: f32 dequantisation straight from the packed streams (row-major output [nrows][K])
+__global__ void dequant_packed_iq2xxs_kernel(const uint2 *qs, const uint16_t *ds, uint32_t nrows, uint32_t K, int col_major, float *out) {
+    const uint32_t groups = K / 32u, blocks = K / 256u;
+    const uint64_t gid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= (uint64_t)nrows * groups) return;
+    const uint32_t r = (uint32_t)(gid / groups), g = (uint32_t)(gid % groups);
+    const uint2 v = col_major ? qs[(uint64_t)g * nrows + r] : qs[(uint64_t)r * groups + g];
+    const uint32_t dbits = col_major ? ds[(uint64_t)(g >> 3) * nrows + r] : ds[(uint64_t)r * blocks + (g >> 3)];
+    const float db = half_bits_to_f32(dbits) * (0.5f + (float)(v.y >> 28)) * 0.25f;
+    float *o = out + (uint64_t)r * K + 32u * g;
+    for (uint32_t l = 0; l < 4u; ++l) {
+        const uint64_t mag = redhip_iq2xxs_grid[(v.x >> (8u * l)) & 255u];
+        const uint32_t s7 = (v.y >> (7u * l)) & 127u, s8 = s7 | ((__popc(s7) & 1u) << 7);
+        for (uint32_t j = 0; j < 8u; ++j) o[8u * l + j] = apply_sign(db * (float)((uint32_t)(mag >> (8u * j)) & 255u), (s8 >> j) & 1u);
+    }
+}
+
+hipError_t launch_dequant_packed_iq2xxs(const void *packed, uint32_t nrows, uint32_t K, bool col_major, float *out, hipStream_t s) {
+    if (!nrows || !K || K % 256u) return hipErrorInvalidValue;
+    const uint2 *qs = static_cast<const uint2 *>(packed);
+    const uint16_t *ds = reinterpret_cast<const uint16_t *>(static_cast<const uint8_t *>(packed) + (uint64_t)nrows * (K / 32u) * 8u);
+    const uint64_t total = (uint64_t)nrows * (K / 32u);
+    REDHIP_LAUNCH(dequant_packed_iq2xxs_kernel, dim3((uint32_t)((total + 255u) / 256u)), dim3(256), 0, s, qs, ds, nrows, K, col_major ? 1 : 0, out);
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------- router GEMV + tail
+
+__device__ __forceinline__ float wave_sum(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ double wave_sum_d(double v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
+    return v;
+}
+__device__ __forceinline__ float wave_max(float v) {
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
+    return v;
+}
+// LDS written by some lanes of a wave becomes readable by its other lanes (one wave, no workgroup barrier)
+__device__ __forceinline__ void wave_lds_sync() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "wavefront");
+    __builtin_amdgcn_wave_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
+}
+__device__ __forceinline__ uint32_t wave_count(bool pred) { return (uint32_t)__popcll(__ballot(pred)); }
+
+// power-of-two pre-scale: largest |v| lands in [2^13, 2^14)
+__device__ __forceinline__ int prescale_exp(float amax) {
+    if (!(amax > 0.0f) || isinf(amax) || isnan(amax)) return 0;
+    return (int)((__float_as_uint(amax) >> 23) & 255u) - 127 - 13;
+}
+__device__ __forceinline__ float exp2i(int e) { return __uint_as_float((uint32_t)(e + 127) << 23); }   // e in [-126, 127]
+
+// v = hi + lo * 2^-11 (to 22 significant bits) after scaling by 2^-e
+__device__ __forceinline__ void split_hi_lo(float v, float inv_scale, _Float16 *hi, _Float16 *lo) {
+    const float t = v * inv_scale;
+    const _Float16 h = (_Float16)t;
+    *hi = h;
+    *lo = (_Float16)((t - (float)h) * 2048.0f);
+}
+
+// ---------------------------------------------------------------- router GEMV
+
+struct RouterArgs {
+    const float *x;            // [ntok][hidden]
+    const float *gate_inp;     // [hidden]
+    float *logits;             // [ntok][n_expert + 1]; the extra entry is gate_inp . x (shared expert's gate logit)
+    _Float16 *xh, *xl;         // [ntok][hidden] fp16 halves of x * 2^-xexp
+    int *xexp;                 // [ntok]
+    uint32_t hidden, n_expert;
+};
+
+// fp16 split of x, spread over the whole grid (every workgroup knows the largest |x| of its token)
+__device__ __forceinline__ void split_x_job(const RouterArgs &a, uint32_t tok, float amax) {
+    const uint32_t gt = blockIdx.x * blockDim.x + threadIdx.x, nt = gridDim.x * blockDim.x;
+    const int e = prescale_exp(amax);
+    const float inv = exp2i(-e);
+    const float *x = a.x + (uint64_t)tok * a.hidden;
+    for (uint32_t i = gt; i < a.hidden; i += nt) split_hi_lo(x[i], inv, a.xh + (uint64_t)tok * a.hidden + i, a.xl + (uint64_t)tok * a.hidden + i);
+    if (gt == 0u) a.xexp[tok] = e;
+}
+
+// F32 router: one wave per row (row n_expert is the shared expert's gate vector), the row and x read as float4
+// with lanes interleaved; every wave sees all of x, so the pre-scale exponent needs no extra pass. blockIdx.y = token.
+template <int NV>          // float4 per lane: hidden = 256 * NV
+__global__ __launch_bounds__(256) void router_f32_kernel(const float *w, RouterArgs a) {
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63u, H = a.hidden, tok = blockIdx.y;
+    const uint32_t r = blockIdx.x * 4u + wave;
+    const float4 *wr = reinterpret_cast<const float4 *>(r < a.n_expert ? w + (uint64_t)r * H : a.gate_inp);
+    const float4 *xv = reinterpret_cast<const float4 *>(a.x + (uint64_t)tok * H);
+    float4 wv[NV], xq[NV];
+    if (r <= a.n_expert) {
+#pragma unroll
+        for (int k = 0; k < NV; ++k) wv[k] = wr[lane + 64u * k];
+    }
+#pragma unroll
+    for (int k = 0; k < NV; ++k) xq[k] = xv[lane + 64u * k];
+    float acc = 0.0f, amax = 0.0f;
+#pragma unroll
+    for (int k = 0; k < NV; ++k) {
+        amax = fmaxf(fmaxf(amax, fmaxf(fabsf(xq[k].x), fabsf(xq[k].y))), fmaxf(fabsf(xq[k].z), fabsf(xq[k].w)));
+        if (r <= a.n_expert) {
+            acc = fmaf(wv[k].x, xq[k].x, acc); acc = fmaf(wv[k].y, xq[k].y, acc);
+            acc = fmaf(wv[k].z, xq[k].z, acc); acc = fmaf(wv[k].w, xq[k].w, acc);
+        }
+    }
+    acc = wave_sum(acc);
+    if (lane == 0u && r <= a.n_expert) a.logits[(uint64_t)tok * (a.n_expert + 1u) + r] = acc;
+    split_x_job(a, tok, wave_max(amax));
+}
+
+// quantised router: rows decoded 32 weights per lane from the raw blocks, x staged in LDS
+template <uint32_t T>
+__global__ __launch_bounds__(256) void router_quant_kernel(const uint8_t *w, RouterArgs a) {
+    __shared__ float lds_amax[4];
+    extern __shared__ float xs[];
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63u, H = a.hidden, tok = blockIdx.y;
+    const float *x = a.x + (uint64_t)tok * H;
+    float amax = 0.0f;
+    for (uint32_t i = threadIdx.x; i < H; i += 256u) { const float v = x[i]; xs[i + (i >> 5)] = v; amax = fmaxf(amax, fabsf(v)); }
+    amax = wave_max(amax);
+    if (lane == 0u) lds_amax[wave] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(lds_amax[0], lds_amax[1]), fmaxf(lds_amax[2], lds_amax[3]));
+    const uint32_t r = blockIdx.x * 4u + wave;
+    if (r <= a.n_expert) {
+        float acc = 0.0f;
+        if (r < a.n_expert) {
+            const uint8_t *row = w + (uint64_t)r * (H / 256u) * Fmt<T>::kBlock;
+            for (uint32_t c = lane; c < H / 32u; c += 64u) {
+                float wv[32];
+                decode32<T>(row, c, wv);
+                float s = 0.0f;
+#pragma unroll
+                for (int j = 0; j < 32; ++j) s = fmaf(wv[j], xs[33u * c + j], s);
+                acc += s;
+            }
+        } else {
+            for (uint32_t i = lane; i < H; i += 64u) acc = fmaf(a.gate_inp[i], xs[i + (i >> 5)], acc);
+        }
+        acc = wave_sum(acc);
+        if (lane == 0u) a.logits[(uint64_t)tok * (a.n_expert + 1u) + r] = acc;
+    }
+    split_x_job(a, tok, amax);
+}
+
+hipError_t launch_router_gemv(uint32_t router_type, const void *w, const float *x, const float *gate_inp, uint32_t ntok, uint32_t hidden,
+                              uint32_t n_expert, float *logits, void *xh, void *xl, int *xexp, hipStream_t s) {
+    if (!ntok || !hidden || hidden % 256u || !n_expert || n_expert > 1024u) return hipErrorInvalidValue;
+    RouterArgs a{x, gate_inp, logits, static_cast<_Float16 *>(xh), static_cast<_Float16 *>(xl), xexp, hidden, n_expert};
+    const dim3 grid((n_expert + 1u + 3u) / 4u, ntok);
+    if (router_type == T_F32) {
+        const float *wf = static_cast<const float *>(w);
+        switch (hidden / 256u) {
+            case 2: REDHIP_LAUNCH(router_f32_kernel<2>, grid, dim3(256), 0, s, wf, a); break;
+            case 4: REDHIP_LAUNCH(router_f32_kernel<4>, grid, dim3(256), 0, s, wf, a); break;
+            case 8: REDHIP_LAUNCH(router_f32_kernel<8>, grid, dim3(256), 0, s, wf, a); break;
+            case 16: REDHIP_LAUNCH(router_f32_kernel<16>, grid, dim3(256), 0, s, wf, a); break;
+            default: return hipErrorInvalidValue;
+        }
+    } else if (router_type == T_Q6_K) {
+        const size_t lds = (size_t)(hidden + hidden / 32u) * sizeof(float);
+        REDHIP_LAUNCH(router_quant_kernel<T_Q6_K>, grid, dim3(256), lds, s, static_cast<const uint8_t *>(w), a);
+    } else {
+        return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------- softmax top-k selection by one wave
+
+// Probabilities exactly as the CPU path forms them (expf(l - max), double sum, one float reciprocal). The wave
+// holds all n_expert probabilities in registers (PER per lane, element i = lane + 64 * s). Non-negative floats
+// order like their bit patterns, so the k-th largest probability is found by bisection on the bits with
+// ballot/popcount; ties at the threshold are then taken in index order: exactly the set and order of an argmax
+// loop with ties to the lower index. The k winners end up one per lane and are ranked against each other with
+// lane broadcasts.
+struct SelectOut {
+    uint32_t ids[16];
+    float w[16];
+    float scalar;
+    uint32_t tmp[16];
+    float tmp_p[16];
+};
+
+template <int PER>
+__device__ void wave_select_topk(const float *logits, uint32_t E, uint32_t K, SelectOut *out, float *probs = nullptr) {
+    const uint32_t lane = threadIdx.x & 63u;
+    float l[PER];
+    float m = -INFINITY;
+#pragma unroll
+    for (int s = 0; s < PER; ++s) {
+        const uint32_t i = lane + 64u * s;
+        l[s] = i < E ? logits[i] : -INFINITY;
+        m = fmaxf(m, l[s]);
+    }
+    const float gate_logit = logits[E];                      // shared expert's gate logit rides along
+    m = wave_max(m);
+    float p[PER];
+    double part = 0.0;
+#pragma unroll
+    for (int s = 0; s < PER; ++s) {
+        p[s] = lane + 64u * s < E ? expf(l[s] - m) : 0.0f;
+        part += (double)p[s];
+    }
+    const double denom = wave_sum_d(part);
+    const bool bad = !(denom > 0.0) || isinf(denom) || isnan(denom);
+    const float inv = bad ? 0.0f : (float)(1.0 / denom);
+    uint32_t key[PER];
+#pragma unroll
+    for (int s = 0; s < PER; ++s) {
+        p[s] *= inv;
+        key[s] = lane + 64u * s < E ? (__float_as_uint(p[s]) | 0x80000000u) : 0u;   // valid keys have the top bit set: padding never counts
+        if (probs && lane + 64u * s < E) probs[lane + 64u * s] = p[s];
+    }
+    // largest T with count(key >= T) >= K; bit 31 is set in every valid key
+    uint32_t T = 0x80000000u;
+#pragma unroll 1
+    for (int bit = 30; bit >= 0; --bit) {
+        const uint32_t cand = T | (1u << bit);
+        uint32_t c = 0u;
+#pragma unroll
+        for (int s = 0; s < PER; ++s) c += wave_count(key[s] >= cand);
+        T = c >= K ? cand : T;
+    }
+    uint32_t above = 0u;
+#pragma unroll
+    for (int s = 0; s < PER; ++s) above += wave_count(key[s] > T);
+    const uint32_t need_ties = K - above;                    // >= 1
+    // winners to LDS, one slot each: everything above T, then the first need_ties equal to T in index order
+    uint32_t n_sel = 0u, ties_seen = 0u;
+#pragma unroll
+    for (int s = 0; s < PER; ++s) {                          // index order = s-major over lanes
+        const bool gt = key[s] > T, eq = key[s] == T;
+        const uint64_t eq_mask = __ballot(eq);
+        const uint32_t eq_before = ties_seen + (uint32_t)__popcll(eq_mask & ((1ull << lane) - 1ull));
+        const bool take = gt || (eq && eq_before < need_ties);
+        const uint64_t take_mask = __ballot(take);
+        if (take) {
+            const uint32_t pos = n_sel + (uint32_t)__popcll(take_mask & ((1ull << lane) - 1ull));
+            out->tmp[pos] = lane + 64u * s;
+            out->tmp_p[pos] = p[s];
+        }
+        n_sel += (uint32_t)__popcll(take_mask);
+        ties_seen += (uint32_t)__popcll(eq_mask);
+    }
+    wave_lds_sync();
+    // lane q < K owns winner q; order by (p desc, index asc) with lane broadcasts
+    const uint32_t mine = lane < K ? out->tmp[lane] : 0xffffffffu;
+    const float pm = lane < K ? out->tmp_p[lane] : -1.0f;
+    uint32_t rank = 0u;
+    for (uint32_t q = 0; q < K; ++q) {
+        const uint32_t o = __shfl(mine, (int)q, 64);
+        const float po = __shfl(pm, (int)q, 64);
+        rank += (po > pm || (po == pm && o < mine)) ? 1u : 0u;
+    }
+    const double sum = wave_sum_d(lane < K ? (double)pm : 0.0);
+    const bool bad2 = bad || !(sum > 0.0) || isinf(sum) || isnan(sum);
+    const float invs = bad2 ? __uint_as_float(0x7fc00000u) : (float)(1.0 / sum);     // NaN weights flag an invalid softmax
+    if (lane < K) {
+        out->ids[rank] = mine < E ? mine : rank;
+        out->w[rank] = pm * invs;
+    }
+    if (lane == 0u) out->scalar = 1.0f / (1.0f + expf(-gate_logit));
+}
+
+// stand-alone selection (one wave per token): ids / weights [ntok][top_k], scalar [ntok]
+__global__ __launch_bounds__(64) void select_kernel(const float *logits, uint32_t E, uint32_t K, uint32_t *ids, float *weights, float *scalar,
+                                                    float *probs) {
+    __shared__ SelectOut sel;
+    const float *l = logits + (uint64_t)blockIdx.x * (E + 1u);
+    float *pr = probs ? probs + (uint64_t)blockIdx.x * E : nullptr;
+    if (E <= 512u) wave_select_topk<8>(l, E, K, &sel, pr); else wave_select_topk<16>(l, E, K, &sel, pr);
+    wave_lds_sync();
+    if (threadIdx.x < K) {
+        ids[(uint64_t)blockIdx.x * K + threadIdx.x] = sel.ids[threadIdx.x];
+        weights[(uint64_t)blockIdx.x * K + threadIdx.x] = sel.w[threadIdx.x];
+    }
+    if (threadIdx.x == 0u && scalar) scalar[blockIdx.x] = sel.scalar;
+}
+
+hipError_t launch_select(const float *logits, uint32_t ntok, uint32_t n_expert, uint32_t top_k, uint32_t *ids, float *weights, float *scalar,
+                         float *probs, hipStream_t s) {
+    if (!ntok || !n_expert || n_expert > 1024u || !top_k || top_k > 16u || top_k > n_expert) return hipErrorInvalidValue;
+    REDHIP_LAUNCH(select_kernel, dim3(ntok), dim3(64), 0, s, logits, n_expert, top_k, ids, weights, scalar, probs);
+    return hipGetLastError();
+}
+
+// without a router (callers that bring their own routing): fp16 split of x and the scalar gate, one workgroup per token
+__global__ __launch_bounds__(256) void prep_kernel(const float *x, const float *gate_inp, uint32_t H, _Float16 *xh, _Float16 *xl, int *xexp, float *scalar) {
+    __shared__ float red[4];
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63u, tok = blockIdx.x;
+    const float *xt = x + (uint64_t)tok * H;
+    float amax = 0.0f, acc = 0.0f;
+    for (uint32_t i = threadIdx.x; i < H; i += 256u) { const float v = xt[i]; amax = fmaxf(amax, fabsf(v)); acc = fmaf(gate_inp[i], v, acc); }
+    amax = wave_max(amax);
+    acc = wave_sum(acc);
+    if (lane == 0u) red[wave] = amax;
+    __syncthreads();
+    amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
+    __syncthreads();
+    if (lane == 0u) red[wave] = acc;
+    __syncthreads();
+    if (threadIdx.x == 0u) scalar[tok] = 1.0f / (1.0f + expf(-((red[0] + red[1]) + (red[2] + red[3]))));
+    const int e = prescale_exp(amax);
+    const float inv = exp2i(-e);
+    for (uint32_t i = threadIdx.x; i < H; i += 256u) split_hi_lo(xt[i], inv, xh + (uint64_t)tok * H + i, xl + (uint64_t)tok * H + i);
+    if (threadIdx.x == 0u) xexp[tok] = e;
+}
+
+hipError_t launch_prep(const float *x, const float *gate_inp, uint32_t ntok, uint32_t hidden, void *xh, void *xl, int *xexp, float *scalar, hipStream_t s) {
+    REDHIP_LAUNCH(prep_kernel, dim3(ntok), dim3(256), 0, s, x, gate_inp, hidden, static_cast<_Float16 *>(xh), static_cast<_Float16 *>(xl), xexp, scalar);
+    return hipGetLastError();
+}
+
+// ---------------------------------------------------------------- gate/up + SwiGLU and down + combine
+
+constexpr int kWaves = 16;                      // 1024 lanes per gate/up workgroup
+constexpr uint32_t kMagBytes = 256u * 16u;      // eight fp16 magnitudes per grid entry
+constexpr uint32_t kSignBytes = 128u * 16u;     // eight fp16 sign masks per 7-bit sign field
+
+// LDS decode tables, built by the first 384 lanes of a workgroup
+__device__ __forceinline__ void build_tables(uint8_t *lds, uint32_t tid, uint64_t grid_entry) {
+    if (tid < 256u) {
+        uint32_t w4[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const _Float16 lo = (_Float16)(float)((uint32_t)(grid_entry >> (16 * i)) & 255u), hi = (_Float16)(float)((uint32_t)(grid_entry >> (16 * i + 8)) & 255u);
+            w4[i] = (uint32_t)__builtin_bit_cast(uint16_t, lo) | ((uint32_t)__builtin_bit_cast(uint16_t, hi) << 16);
+        }
+        *reinterpret_cast<uint4 *>(lds + (size_t)tid * 16u) = make_uint4(w4[0], w4[1], w4[2], w4[3]);
+    } else if (tid < 384u) {
+        const uint32_t s7 = tid - 256u, s8 = s7 | ((__popc(s7) & 1u) << 7);
+        uint32_t w4[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w4[i] = (((s8 >> (2 * i)) & 1u) << 15) | (((s8 >> (2 * i + 1)) & 1u) << 31);
+        *reinterpret_cast<uint4 *>(lds + kMagBytes + (size_t)s7 * 16u) = make_uint4(w4[0], w4[1], w4[2], w4[3]);
+    }
+}
+
+template <int N, int OFF>
+__device__ __forceinline__ void halve_step(float *v, uint32_t lane) {      // N live values -> N / 2
+    const bool upper = (lane & (uint32_t)OFF) != 0u;
+#pragma unroll
+    for (int i = 0; i < N / 2; ++i) {
+        const float keep = upper ? v[N / 2 + i] : v[i];
+        const float give = upper ? v[i] : v[N / 2 + i];
+        v[i] = keep + __shfl_xor(give, OFF, 64);
+    }
+}
+// sum of `v` over the 16 lanes that share lane % 4, for UPW values at once
+template <int UPW>
+__device__ __forceinline__ float quad_column_reduce(float *v, uint32_t lane) {
+    static_assert(UPW == 1 || UPW == 2 || UPW == 4 || UPW == 8, "units per wave");
+    if constexpr (UPW >= 2) halve_step<UPW, 32>(v, lane);
+    if constexpr (UPW >= 4) halve_step<UPW / 2, 16>(v, lane);
+    if constexpr (UPW >= 8) halve_step<UPW / 4, 8>(v, lane);
+    constexpr int kFirstPlain = UPW >= 8 ? 4 : UPW >= 4 ? 8 : UPW >= 2 ? 16 : 32;
+    float r = v[0];
+#pragma unroll
+    for (int off = kFirstPlain; off >= 4; off >>= 1) r += __shfl_xor(r, off, 64);
+    return r;
+}
+// the unit whose total a lane holds after quad_column_reduce, and whether this lane is the one that stores it
+template <int UPW> __device__ __forceinline__ uint32_t reduced_unit(uint32_t lane) {
+    uint32_t u = 0u;
+    if constexpr (UPW >= 2) u += (lane & 32u) ? UPW / 2 : 0;
+    if constexpr (UPW >= 4) u += (lane & 16u) ? UPW / 4 : 0;
+    if constexpr (UPW >= 8) u += (lane & 8u) ? UPW / 8 : 0;
+    return u;
+}
+template <int UPW> __device__ __forceinline__ bool reduced_writer(uint32_t lane) {
+    constexpr uint32_t kPlainBits = UPW >= 8 ? 4u : UPW >= 4 ? 12u : UPW >= 2 ? 28u : 60u;   // lane bits folded by plain steps
+    return (lane & kPlainBits) == 0u;
+}
+
+// 32 weights of one group against the lane's activation operand: (hi . w + lo . w * 2^-11) * (2 * scale + 1).
+// v_mfma_f32_4x4x4_16B_f16: lanes 4b..4b+3 form block b; lane j of a block supplies row j of A (the activation
+// halves: j = 0 hi, j = 1 lo, others zero) and column j of B (its own four weights), and receives column j of
+// A x B: acc[0] = hi . w, acc[1] = lo . w.
+__device__ __forceinline__ float group_dot(uint2 q, const half4_t *ax, const uint8_t *lds) {
+    float4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (uint32_t l = 0; l < 4u; ++l) {
+        const uint32_t idx = (q.x >> (8u * l)) & 255u, s7 = (q.y >> (7u * l)) & 127u;
+        const uint4 m = *reinterpret_cast<const uint4 *>(lds + (idx << 4));
+        const uint4 sg = *reinterpret_cast<const uint4 *>(lds + kMagBytes + (s7 << 4));
+        union { uint32_t u[2]; half4_t h; } b0, b1;
+        b0.u[0] = m.x ^ sg.x; b0.u[1] = m.y ^ sg.y;
+        b1.u[0] = m.z ^ sg.z; b1.u[1] = m.w ^ sg.w;
+        acc = __builtin_amdgcn_mfma_f32_4x4x4f16(ax[2u * l], b0.h, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_4x4x4f16(ax[2u * l + 1u], b1.h, acc, 0, 0, 0);
+    }
+    return (acc[0] + acc[1] * 4.8828125e-4f) * (float)(2u * (q.y >> 28) + 1u);
+}
+
+// the lane's activation operand: 32 values starting at src (fp16), lanes j = 0 / 1 carry hi / lo, others zero
+__device__ __forceinline__ void load_act_operand(half4_t *ax, const _Float16 *hi, const _Float16 *lo, uint32_t j) {
+    const _Float16 *src = j == 0u ? hi : lo;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+        half4_t v = {(_Float16)0, (_Float16)0, (_Float16)0, (_Float16)0};
+        if (j < 2u) v = *reinterpret_cast<const half4_t *>(src + 4 * s);
+        ax[s] = v;
+    }
+}
+
+struct GateUpArgs {
+    const uint8_t *experts;    // packed experts of the layer, expert e at experts + e * stride
+    uint64_t stride;
+    const uint8_t *shared;     // packed shared expert
+    const float *logits;       // [n_expert + 1] (selection happens here) or nullptr: ids come from `ids_in`
+    const uint32_t *ids_in;    // [top_k] when logits == nullptr
+    uint32_t *ids_out;         // [top_k]   written by workgroup (0, 0) when selecting
+    float *weights_out;        // [top_k]
+    float *scalar_out;         // [1]
+    const _Float16 *xh, *xl;   // [hidden]
+    const int *xexp;           // [1]
+    _Float16 *act_h, *act_l;   // [top_k + 1][ffn]
+    int *act_exp;              // [top_k + 1][ffn / 32]
+    uint32_t hidden, ffn, n_expert, top_k;
+};
+
+template <int NKC>        // K chunks of 512 columns in a gate/up row: hidden = 512 * NKC
+__global__ __launch_bounds__(kWaves * 64) void gateup_select_kernel(GateUpArgs a) {
+    constexpr int NW = kWaves;
+    constexpr int UPW = 16 * NKC / NW;                 // (row-quad, K-chunk) units per wave
+    static_assert(UPW >= 1 && UPW * NW == 16 * NKC, "waves must tile the 16 row-quads x NKC chunks");
+    __shared__ __attribute__((aligned(16))) uint8_t lds[kMagBytes + kSignBytes];
+    __shared__ float part[NKC * 64];
+    __shared__ SelectOut sel;
+
+    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
+    const uint32_t H = a.hidden, F = a.ffn, HG = H / 32u, HB = H / 256u;
+    const uint32_t g = blockIdx.x;                     // FFN column group: act values [32 g, 32 g + 32)
+    const uint32_t slot = blockIdx.y;
+    const bool is_shared = slot >= a.top_k;
+    const uint64_t grid_entry = tid < 256u ? redhip_iq2xxs_grid[tid] : 0ull;
+
+    // activation operand: independent of the routing, requested before the selection
+    const uint32_t kc = wave % NKC, q0 = wave / NKC;
+    const uint32_t G = 16u * kc + blk;                 // this lane's group inside the gate/up rows
+    half4_t ax[8];
+    load_act_operand(ax, a.xh + 32u * G, a.xl + 32u * G, j);
+    build_tables(lds, tid, grid_entry);
+
+    uint32_t expert = 0u;
+    if (a.logits) {
+        if (wave == 0u) {        // the other waves have nothing to do until the expert is known
+            if (a.n_expert <= 512u) wave_select_topk<8>(a.logits, a.n_expert, a.top_k, &sel);
+            else wave_select_topk<16>(a.logits, a.n_expert, a.top_k, &sel);
+        }
+        __syncthreads();
+        if (!is_shared) expert = sel.ids[slot];
+        if (g == 0u && slot == 0u) {
+            if (tid < a.top_k) { a.ids_out[tid] = sel.ids[tid]; a.weights_out[tid] = sel.w[tid]; }
+            if (tid == 0u) a.scalar_out[0] = sel.scalar;
+        }
+    } else {
+        if (!is_shared) expert = a.ids_in[slot];
+        __syncthreads();                               // tables
+    }
+    const uint8_t *ex = is_shared ? a.shared : a.experts + (uint64_t)expert * a.stride;
+    const uint64_t gate_bytes = (uint64_t)F * HG * 8u + (uint64_t)F * HB * 2u;
+    const uint2 *gate_qs = reinterpret_cast<const uint2 *>(ex);
+    const uint16_t *gate_ds = reinterpret_cast<const uint16_t *>(ex + (uint64_t)F * HG * 8u);
+    const uint2 *up_qs = reinterpret_cast<const uint2 *>(ex + gate_bytes);
+    const uint16_t *up_ds = reinterpret_cast<const uint16_t *>(ex + gate_bytes + (uint64_t)F * HG * 8u);
+
+    uint2 wq[UPW];
+    uint32_t wd[UPW];
+#pragma unroll
+    for (int u = 0; u < UPW; ++u) {
+        const uint32_t quad = q0 + (NW / NKC) * u;     // 0..7 gate, 8..15 up
+        const uint32_t r = 32u * g + 4u * (quad & 7u) + j;
+        const uint2 *qs = quad < 8u ? gate_qs : up_qs;
+        const uint16_t *ds = quad < 8u ? gate_ds : up_ds;
+        wq[u] = qs[(uint64_t)r * HG + G];
+        wd[u] = ds[(uint64_t)r * HB + (G >> 3)];
+    }
+    float v[UPW];
+#pragma unroll
+    for (int u = 0; u < UPW; ++u) v[u] = group_dot(wq[u], ax, lds) * half_bits_to_f32(wd[u]);
+    const float tot = quad_column_reduce<UPW>(v, lane);
+    if (reduced_writer<UPW>(lane)) {
+        const uint32_t quad = q0 + (NW / NKC) * reduced_unit<UPW>(lane);
+        part[kc * 64u + 4u * quad + j] = tot;
+    }
+    __syncthreads();
+    if (tid < 32u) {
+        float gsum = 0.0f, usum = 0.0f;
+#pragma unroll
+        for (int c = 0; c < NKC; ++c) { gsum += part[c * 64 + tid]; usum += part[c * 64 + 32 + tid]; }
+        const float xs = 0.125f * exp2i(a.xexp[0]);                  // d/8 and the pre-scale of x
+        gsum *= xs;
+        usum *= xs;
+        const float act = (gsum / (1.0f + expf(-gsum))) * usum;
+        float amax = fabsf(act);
+#pragma unroll
+        for (int o = 16; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+        const int e = prescale_exp(amax);
+        split_hi_lo(act, exp2i(-e), a.act_h + (uint64_t)slot * F + 32u * g + tid, a.act_l + (uint64_t)slot * F + 32u * g + tid);
+        if (tid == 0u) a.act_exp[slot * (F / 32u) + g] = e;
+    }
+}
+
+struct DownArgs {
+    const uint8_t *experts;
+    uint64_t stride;
+    const uint8_t *shared;
+    const uint32_t *ids;       // [top_k]
+    const float *weights;      // [top_k]
+    const float *scalar;       // [1]
+    const _Float16 *act_h, *act_l;
+    const int *act_exp;
+    float *out;                // [hidden]
+    uint32_t hidden, ffn, top_k;
+};
+
+// 8 output rows per workgroup; wave s (< top_k + 1) owns slot s: both row quads of the workgroup against all
+// ffn columns (ffn = 512: 16 groups = the 16 lane blocks of a wave). Slots are then added in selection order.
+__global__ __launch_bounds__(kWaves * 64) void down_combine_kernel(DownArgs a) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds[kMagBytes + kSignBytes];
+    __shared__ float part[17 * 8];
+    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
+    const uint32_t H = a.hidden, F = a.ffn, FG = F / 32u, FB = F / 256u, n_slot = a.top_k + 1u;
+    const uint64_t grid_entry = tid < 256u ? redhip_iq2xxs_grid[tid] : 0ull;
+    const uint32_t row0 = 8u * blockIdx.x;
+    float tot[2] = {0.0f, 0.0f};
+    uint2 dq[2][2];            // [row quad][column chunk of 16 groups] (ffn <= 1024)
+    uint32_t dd[2][2];
+    const uint32_t n_chunk = (FG + 15u) / 16u;
+    const bool active = wave < n_slot;
+    const uint8_t *ex = nullptr;
+    if (active) {
+        ex = wave < a.top_k ? a.experts + (uint64_t)a.ids[wave] * a.stride : a.shared;
+        const uint64_t gate_bytes = (uint64_t)F * (H / 32u) * 8u + (uint64_t)F * (H / 256u) * 2u;
+        const uint2 *qs = reinterpret_cast<const uint2 *>(ex + 2u * gate_bytes);                         // [hidden][FG]
+        const uint16_t *ds = reinterpret_cast<const uint16_t *>(ex + 2u * gate_bytes + (uint64_t)H * FG * 8u);   // [hidden][FB]
+#pragma unroll
+        for (int q = 0; q < 2; ++q)
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+                const uint32_t r = row0 + 4u * q + j, G = 16u * c + blk;
+                if ((uint32_t)c < n_chunk && G < FG) { dq[q][c] = qs[(uint64_t)r * FG + G]; dd[q][c] = ds[(uint64_t)r * FB + (G >> 3)]; }
+            }
+    }
+    build_tables(lds, tid, grid_entry);
+    __syncthreads();
+    if (active) {
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            const uint32_t G = 16u * c + blk;
+            if ((uint32_t)c < n_chunk && G < FG) {
+                half4_t ax[8];
+                load_act_operand(ax, a.act_h + (uint64_t)wave * F + 32u * G, a.act_l + (uint64_t)wave * F + 32u * G, j);
+                const float sc = exp2i(a.act_exp[wave * FG + G]);
+#pragma unroll
+                for (int q = 0; q < 2; ++q) tot[q] += group_dot(dq[q][c], ax, lds) * half_bits_to_f32(dd[q][c]) * sc;
+            }
+        }
+        const float r = quad_column_reduce<2>(tot, lane);
+        if (reduced_writer<2>(lane)) part[wave * 8u + 4u * reduced_unit<2>(lane) + j] = r;
+    }
+    __syncthreads();
+    if (tid < 8u) {
+        float sum = 0.0f;
+        for (uint32_t s = 0; s < a.top_k; ++s) sum = fmaf(a.weights[s] * 0.125f, part[s * 8u + tid], sum);
+        sum = fmaf(a.scalar[0] * 0.125f, part[a.top_k * 8u + tid], sum);
+        a.out[row0 + tid] = sum;
+    }
+}
+
+hipError_t launch_gateup_select(const void *experts, uint64_t stride, const void *shared, const float *logits, const uint32_t *ids_in,
+                                uint32_t *ids_out, float *weights_out, float *scalar_out, const void *xh, const void *xl, const int *xexp,
+                                void *act_h, void *act_l, int *act_exp, uint32_t hidden, uint32_t ffn, uint32_t n_expert, uint32_t top_k,
+                                hipStream_t s) {
+    if (!fused_iq2_supported(hidden, ffn)) return hipErrorInvalidValue;
+    GateUpArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(shared), logits, ids_in, ids_out, weights_out,
+                 scalar_out, static_cast<const _Float16 *>(xh), static_cast<const _Float16 *>(xl), xexp, static_cast<_Float16 *>(act_h),
+                 static_cast<_Float16 *>(act_l), act_exp, hidden, ffn, n_expert, top_k};
+    const dim3 grid(ffn / 32u, top_k + 1u);
+    switch (hidden / 512u) {
+        case 1: REDHIP_LAUNCH(gateup_select_kernel<1>, grid, dim3(kWaves * 64), 0, s, a); break;
+        case 2: REDHIP_LAUNCH(gateup_select_kernel<2>, grid, dim3(kWaves * 64), 0, s, a); break;
+        case 4: REDHIP_LAUNCH(gateup_select_kernel<4>, grid, dim3(kWaves * 64), 0, s, a); break;
+        case 8: REDHIP_LAUNCH(gateup_select_kernel<8>, grid, dim3(kWaves * 64), 0, s, a); break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_down_combine(const void *experts, uint64_t stride, const void *shared, const uint32_t *ids, const float *weights,
+                               const float *scalar, const void *act_h, const void *act_l, const int *act_exp, float *out,
+                               uint32_t hidden, uint32_t ffn, uint32_t top_k, hipStream_t s) {
+    if (!fused_iq2_supported(hidden, ffn) || top_k + 1u > (uint32_t)kWaves) return hipErrorInvalidValue;
+    DownArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(shared), ids, weights, scalar,
+               static_cast<const _Float16 *>(act_h), static_cast<const _Float16 *>(act_l), act_exp, out, hidden, ffn, top_k};
+    REDHIP_LAUNCH(down_combine_kernel, dim3(hidden / 8u), dim3(kWaves * 64), 0, s, a);
+    return hipGetLastError();
+}
+
+}  // namespace redhip

@@ -77,4 +77,37 @@ hipError_t launch_group_pairs(const uint32_t *ids, const float *weights, uint32_
                               uint32_t *uid, uint32_t *expert_start, uint32_t *pair_token, float *pair_weight,
                               uint32_t *tok_pair, uint32_t *n_unique, hipStream_t s);
 
+// ---- decode path over packed IQ2_XXS (redhip_fused.hip) ----
+
+// shapes the packed kernels tile: gate/up rows in chunks of 512 columns over 16 waves; down rows of <= 1024 columns
+inline bool fused_iq2_supported(uint32_t hidden, uint32_t ffn) {
+    const uint32_t nkc = hidden / 512u;
+    return hidden % 512u == 0u && (nkc == 1u || nkc == 2u || nkc == 4u || nkc == 8u) && ffn && ffn % 256u == 0u && ffn <= 1024u;
+}
+
+// `count` matrices, raw_stride / packed_stride bytes apart; packed = qs [nrows][K/32] uint2 then ds [nrows][K/256] fp16
+hipError_t launch_repack_iq2xxs(const void *raw, uint64_t raw_stride, uint32_t count, uint32_t nrows, uint32_t K, bool col_major,
+                                void *packed, uint64_t packed_stride, hipStream_t s);
+hipError_t launch_dequant_packed_iq2xxs(const void *packed, uint32_t nrows, uint32_t K, bool col_major, float *out, hipStream_t s);
+
+// logits [ntok][n_expert + 1] (entry n_expert = gate_inp . x) and the fp16 split of x: xh, xl [ntok][hidden], xexp [ntok]
+hipError_t launch_router_gemv(uint32_t router_type, const void *w, const float *x, const float *gate_inp, uint32_t ntok, uint32_t hidden,
+                              uint32_t n_expert, float *logits, void *xh, void *xl, int *xexp, hipStream_t s);
+// softmax top-k of logits [ntok][n_expert + 1]; scalar[t] = sigmoid(logits[t][n_expert]); optional probs [ntok][n_expert]
+hipError_t launch_select(const float *logits, uint32_t ntok, uint32_t n_expert, uint32_t top_k, uint32_t *ids, float *weights, float *scalar,
+                         float *probs, hipStream_t s);
+// fp16 split of x and the scalar gate without a router
+hipError_t launch_prep(const float *x, const float *gate_inp, uint32_t ntok, uint32_t hidden, void *xh, void *xl, int *xexp, float *scalar, hipStream_t s);
+
+// single token: act[slot] = SwiGLU(gate . x, up . x) as fp16 halves with one exponent per 32 values. With `logits` the
+// kernel selects the experts itself (and writes ids / weights / scalar); with logits == nullptr it takes ids_in.
+hipError_t launch_gateup_select(const void *experts, uint64_t stride, const void *shared, const float *logits, const uint32_t *ids_in,
+                                uint32_t *ids_out, float *weights_out, float *scalar_out, const void *xh, const void *xl, const int *xexp,
+                                void *act_h, void *act_l, int *act_exp, uint32_t hidden, uint32_t ffn, uint32_t n_expert, uint32_t top_k,
+                                hipStream_t s);
+// single token: out[r] = sum_k weights[k] * down_{ids[k]}[r] . act[k] + scalar * shared_down[r] . act[top_k], k in order
+hipError_t launch_down_combine(const void *experts, uint64_t stride, const void *shared, const uint32_t *ids, const float *weights,
+                               const float *scalar, const void *act_h, const void *act_l, const int *act_exp, float *out,
+                               uint32_t hidden, uint32_t ffn, uint32_t top_k, hipStream_t s);
+
 }  // namespace redhip

@@ -6,22 +6,8 @@
 
 namespace redhip {
 
-__device__ uint64_t g_iq2xxs_grid[256];
-__device__ uint32_t g_iq3s_grid[512];
-
-static hipError_t ensure_tables() {
-    static hipError_t state = hipErrorNotInitialized;
-    static int device_done[64] = {0};
-    int dev = 0;
-    hipError_t e = hipGetDevice(&dev);
-    if (e != hipSuccess) return e;
-    if (dev >= 0 && dev < 64 && device_done[dev]) return hipSuccess;
-    e = hipMemcpyToSymbol(HIP_SYMBOL(g_iq2xxs_grid), redhip_iq2xxs_grid, sizeof(redhip_iq2xxs_grid));
-    if (e == hipSuccess) e = hipMemcpyToSymbol(HIP_SYMBOL(g_iq3s_grid), redhip_iq3s_grid, sizeof(redhip_iq3s_grid));
-    if (e == hipSuccess && dev >= 0 && dev < 64) device_done[dev] = 1;
-    state = e;
-    return state;
-}
+// the codebooks are constant device arrays of this translation unit (redhip_tables.h): nothing to upload
+static inline hipError_t ensure_tables() { return hipSuccess; }
 
 static inline uint32_t lanes_per_row(uint32_t ncols) {
     const uint32_t chunks = ncols / 32u;

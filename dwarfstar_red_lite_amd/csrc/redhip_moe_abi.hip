@@ -1,6 +1,7 @@
 // Resident MoE FFN layers: every expert of every layer stays in HBM, one call runs a layer's FFN on a stream.
 // See include/redhip_moe.h for the contract.
 #include <stdarg.h>
+#include <stdlib.h>
 #include <stdio.h>
 #include <string.h>
 
@@ -31,6 +32,8 @@ struct Layer {
     uint8_t *shared = nullptr;       // gate | up | down of the shared expert
     float *gate_inp = nullptr;       // [hidden]
     uint8_t *experts = nullptr;      // n_expert slots of expert_stride bytes, each gate | up | down
+    uint8_t *packed = nullptr;       // same slots in the packed IQ2_XXS layout of the fused kernel (fused path only)
+    uint8_t *shared_packed = nullptr;
 };
 
 struct Moe {
@@ -45,6 +48,13 @@ struct Moe {
     float *logits = nullptr, *weights = nullptr, *scalar = nullptr, *act = nullptr, *sh_act = nullptr;
     uint32_t *ids = nullptr;
     uint8_t *ws = nullptr;
+    // single-token fused path (all matrices IQ2_XXS, shapes the fused kernel tiles)
+    bool fused = false;
+    void *xh = nullptr, *xl = nullptr;       // fp16 [hidden] each
+    int *xexp = nullptr;
+    bool skip_select = false;                // forward(): the gate/up kernel selects, route() skips its own selection
+    void *act_h = nullptr, *act_l = nullptr; // fp16 [top_k + 1][ffn] each
+    int *act_exp = nullptr;                  // [top_k + 1][ffn / 32]
 
     ExpertSet routed(uint32_t l) const { return ExpertSet{layers[l].experts, expert_stride, gate_bytes, gate_bytes, gu_type, dn_type}; }
     ExpertSet shared(uint32_t l) const { return ExpertSet{layers[l].shared, 0, sh_gate_bytes, sh_gate_bytes, sh_gu_type, sh_dn_type}; }
@@ -71,10 +81,23 @@ __global__ __launch_bounds__(256) void scalar_gate_kernel(const float *gate_inp,
     if (threadIdx.x == 0u) scalar[blockIdx.x] = (float)(1.0 / (1.0 + exp(-((red[0] + red[1]) + (red[2] + red[3])))));
 }
 
+// select_here: the gate/up kernel selects the experts from m->logits itself (ids / weights are then outputs)
 int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const uint32_t *ids, const float *weights,
-                    float *out, hipStream_t s) {
+                    float *out, hipStream_t s, bool select_here = false) {
     const redhip_moe_config &c = m->cfg;
     if (ntok != 1u) { moe_err("batched expert execution is not available in this build (ntok=%u)", ntok); return 0; }
+    if (m->fused) {          // xh / xl / scalar come from the router kernel or the prep kernel
+        const Layer &L = m->layers[layer];
+        prof_set_stage(ST_GATEUP);
+        HIP_OK(launch_gateup_select(L.packed, m->expert_stride, L.shared_packed, select_here ? m->logits : nullptr, ids, m->ids, m->weights,
+                                    m->scalar, m->xh, m->xl, m->xexp, m->act_h, m->act_l, m->act_exp, c.hidden, c.ffn, c.n_expert, c.top_k, s),
+               "gate/up launch");
+        prof_set_stage(ST_DOWN_COMBINE);
+        HIP_OK(launch_down_combine(L.packed, m->expert_stride, L.shared_packed, select_here ? m->ids : ids, select_here ? m->weights : weights,
+                                   m->scalar, m->act_h, m->act_l, m->act_exp, out, c.hidden, c.ffn, c.top_k, s), "down/combine launch");
+        prof_set_stage(ST_OTHER);
+        return 1;
+    }
     const ExpertSet ex = m->routed(layer), sh = m->shared(layer);
     prof_set_stage(ST_GATEUP);
     HIP_OK(launch_moe_gateup(ex, ids, c.top_k, c.hidden, c.ffn, x, m->act, s), "routed gate/up launch");
@@ -121,6 +144,7 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
     m->sh_down_bytes = (uint64_t)c.hidden * row_bytes(sdn, c.ffn);
     m->router_bytes = (uint64_t)c.n_expert * row_bytes(c.router_type, c.hidden);
     m->layers.resize(c.n_layer);
+    m->fused = gu == T_IQ2_XXS && dn == T_IQ2_XXS && sgu == T_IQ2_XXS && sdn == T_IQ2_XXS && fused_iq2_supported(c.hidden, c.ffn);
     bool ok = true;
     for (uint32_t l = 0; l < c.n_layer && ok; ++l) {
         Layer &L = m->layers[l];
@@ -133,10 +157,17 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
         L.shared = p + align256(m->router_bytes);
         L.gate_inp = reinterpret_cast<float *>(L.shared + align256(2u * m->sh_gate_bytes + m->sh_down_bytes));
         m->resident += small + (uint64_t)c.n_expert * m->expert_stride;
+        if (m->fused) {
+            ok = hipMalloc(reinterpret_cast<void **>(&L.packed), (size_t)c.n_expert * m->expert_stride) == hipSuccess &&
+                 hipMalloc(reinterpret_cast<void **>(&L.shared_packed), align256(2u * m->sh_gate_bytes + m->sh_down_bytes)) == hipSuccess;
+            m->resident += (uint64_t)c.n_expert * m->expert_stride + align256(2u * m->sh_gate_bytes + m->sh_down_bytes);
+        }
     }
     const size_t T = c.max_tokens;
-    const size_t ws_bytes = align256(T * c.n_expert * 4u) + 2u * align256(T * c.top_k * 4u) + align256(T * 4u) +
-                            align256(T * c.top_k * c.ffn * 4u) + align256(T * c.ffn * 4u);
+    const size_t ws_bytes = align256(T * (c.n_expert + 1u) * 4u) + 2u * align256(T * c.top_k * 4u) + align256(T * 4u) +
+                            align256(T * c.top_k * c.ffn * 4u) + align256(T * c.ffn * 4u) +
+                            2u * align256(2u * T * c.hidden) + align256(4u * T) + 2u * align256(2u * (c.top_k + 1u) * c.ffn) +
+                            align256(4u * (c.top_k + 1u) * (c.ffn / 32u));
     ok = ok && hipMalloc(reinterpret_cast<void **>(&m->ws), ws_bytes) == hipSuccess;
     if (!ok) {
         moe_err("failed to allocate resident MoE memory (%llu bytes so far)", (unsigned long long)m->resident);
@@ -144,12 +175,19 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
         return nullptr;
     }
     uint8_t *w = m->ws;
-    m->logits = reinterpret_cast<float *>(w); w += align256(T * c.n_expert * 4u);
+    m->logits = reinterpret_cast<float *>(w); w += align256(T * (c.n_expert + 1u) * 4u);
     m->ids = reinterpret_cast<uint32_t *>(w); w += align256(T * c.top_k * 4u);
     m->weights = reinterpret_cast<float *>(w); w += align256(T * c.top_k * 4u);
     m->scalar = reinterpret_cast<float *>(w); w += align256(T * 4u);
     m->act = reinterpret_cast<float *>(w); w += align256(T * c.top_k * c.ffn * 4u);
-    m->sh_act = reinterpret_cast<float *>(w);
+    m->sh_act = reinterpret_cast<float *>(w); w += align256(T * c.ffn * 4u);
+    m->xh = w; w += align256(2u * T * c.hidden);
+    m->xl = w; w += align256(2u * T * c.hidden);
+    m->xexp = reinterpret_cast<int *>(w); w += align256(4u * T);
+    m->act_h = w; w += align256(2u * (c.top_k + 1u) * c.ffn);
+    m->act_l = w; w += align256(2u * (c.top_k + 1u) * c.ffn);
+    m->act_exp = reinterpret_cast<int *>(w);
+    if (hipMemset(m->ws, 0, ws_bytes) != hipSuccess) { moe_err("failed to clear the MoE workspace"); redhip_moe_destroy(m); return nullptr; }
     // first launches copy the codebooks to the device; do it here so that forward never synchronises
     if (launch_dequant_rows(T_F32, m->ws, 1u, 32u, m->logits, nullptr) != hipSuccess || hipDeviceSynchronize() != hipSuccess) {
         moe_err("failed to initialise device codebooks");
@@ -166,6 +204,8 @@ void redhip_moe_destroy(redhip_moe_t h) {
     for (Layer &L : m->layers) {
         if (L.router) (void)hipFree(L.router);
         if (L.experts) (void)hipFree(L.experts);
+        if (L.packed) (void)hipFree(L.packed);
+        if (L.shared_packed) (void)hipFree(L.shared_packed);
     }
     if (m->ws) (void)hipFree(m->ws);
     delete m;
@@ -196,6 +236,12 @@ int redhip_moe_load_shared(redhip_moe_t h, uint32_t layer, const float *gate_inp
     HIP_OK(hipMemcpy(L.shared, gate, (size_t)gate_bytes, hipMemcpyDefault), "shared gate upload");
     HIP_OK(hipMemcpy(L.shared + gate_bytes, up, (size_t)up_bytes, hipMemcpyDefault), "shared up upload");
     HIP_OK(hipMemcpy(L.shared + 2u * gate_bytes, down, (size_t)down_bytes, hipMemcpyDefault), "shared down upload");
+    if (m->fused) {
+        const redhip_moe_config &c = m->cfg;
+        HIP_OK(launch_repack_iq2xxs(L.shared, gate_bytes, 2u, c.ffn, c.hidden, false, L.shared_packed, gate_bytes, nullptr), "shared gate/up repack");
+        HIP_OK(launch_repack_iq2xxs(L.shared + 2u * gate_bytes, 0u, 1u, c.hidden, c.ffn, false, L.shared_packed + 2u * gate_bytes, 0u, nullptr), "shared down repack");
+        HIP_OK(hipStreamSynchronize(nullptr), "shared repack");
+    }
     return 1;
 }
 
@@ -211,6 +257,14 @@ int redhip_moe_load_experts(redhip_moe_t h, uint32_t layer, uint32_t first, uint
     HIP_OK(hipMemcpy2D(dst, m->expert_stride, gate, m->gate_bytes, m->gate_bytes, count, hipMemcpyDefault), "expert gate upload");
     HIP_OK(hipMemcpy2D(dst + m->gate_bytes, m->expert_stride, up, m->gate_bytes, m->gate_bytes, count, hipMemcpyDefault), "expert up upload");
     HIP_OK(hipMemcpy2D(dst + 2u * m->gate_bytes, m->expert_stride, down, m->down_bytes, m->down_bytes, count, hipMemcpyDefault), "expert down upload");
+    if (m->fused) {
+        const redhip_moe_config &c = m->cfg;
+        uint8_t *pk = m->layers[layer].packed + (uint64_t)first * m->expert_stride;
+        HIP_OK(launch_repack_iq2xxs(dst, m->expert_stride, count, c.ffn, c.hidden, false, pk, m->expert_stride, nullptr), "expert gate repack");
+        HIP_OK(launch_repack_iq2xxs(dst + m->gate_bytes, m->expert_stride, count, c.ffn, c.hidden, false, pk + m->gate_bytes, m->expert_stride, nullptr), "expert up repack");
+        HIP_OK(launch_repack_iq2xxs(dst + 2u * m->gate_bytes, m->expert_stride, count, c.hidden, c.ffn, false, pk + 2u * m->gate_bytes, m->expert_stride, nullptr), "expert down repack");
+        HIP_OK(hipStreamSynchronize(nullptr), "expert repack");
+    }
     return 1;
 }
 
@@ -222,6 +276,20 @@ int redhip_moe_route(redhip_moe_t h, uint32_t layer, const float *x_dev, uint32_
     if (!x_dev || !ntok || ntok > c.max_tokens) { moe_err("invalid token count %u (max %u)", ntok, c.max_tokens); return 0; }
     hipStream_t s = static_cast<hipStream_t>(stream);
     float *lg = logits_dev ? logits_dev : m->logits;
+    if (m->fused) {
+        prof_set_stage(ST_ROUTER_GEMV);
+        HIP_OK(launch_router_gemv(c.router_type, m->layers[layer].router, x_dev, m->layers[layer].gate_inp, ntok, c.hidden, c.n_expert,
+                                  m->logits, m->xh, m->xl, m->xexp, s), "router launch");
+        if (!m->skip_select) {
+            prof_set_stage(ST_ROUTE_SELECT);
+            HIP_OK(launch_select(m->logits, ntok, c.n_expert, c.top_k, ids_dev ? ids_dev : m->ids, weights_dev ? weights_dev : m->weights,
+                                 m->scalar, nullptr, s), "selection launch");
+        }
+        prof_set_stage(ST_OTHER);
+        if (logits_dev) HIP_OK(hipMemcpy2DAsync(logits_dev, 4u * (size_t)c.n_expert, m->logits, 4u * (size_t)(c.n_expert + 1u), 4u * (size_t)c.n_expert,
+                                                ntok, hipMemcpyDeviceToDevice, s), "logits copy");
+        return 1;
+    }
     prof_set_stage(ST_ROUTER_GEMV);
     for (uint32_t t = 0; t < ntok; ++t)
         HIP_OK(launch_gemv_rows(c.router_type, m->layers[layer].router, c.hidden, 0u, c.n_expert, x_dev + (size_t)t * c.hidden,
@@ -239,6 +307,11 @@ int redhip_moe_experts(redhip_moe_t h, uint32_t layer, const float *x_dev, uint3
     if (!check_layer(m, layer)) return 0;
     if (!x_dev || !ids_dev || !weights_dev || !out_dev || !ntok || ntok > m->cfg.max_tokens) { moe_err("invalid expert execution arguments"); return 0; }
     hipStream_t s = static_cast<hipStream_t>(stream);
+    if (m->fused && ntok == 1u) {
+        prof_set_stage(ST_OTHER);
+        HIP_OK(launch_prep(x_dev, m->layers[layer].gate_inp, ntok, m->cfg.hidden, m->xh, m->xl, m->xexp, m->scalar, s), "prep launch");
+        return experts_enqueue(m, layer, x_dev, ntok, ids_dev, weights_dev, out_dev, s);
+    }
     scalar_gate_kernel<<<ntok, 256, 0, s>>>(m->layers[layer].gate_inp, x_dev, m->cfg.hidden, m->scalar);
     HIP_OK(hipGetLastError(), "scalar gate launch");
     return experts_enqueue(m, layer, x_dev, ntok, ids_dev, weights_dev, out_dev, s);
@@ -248,8 +321,13 @@ int redhip_moe_forward(redhip_moe_t h, uint32_t layer, const float *x_dev, uint3
     Moe *m = moe_of(h);
     if (!check_layer(m, layer)) return 0;
     if (!x_dev || !out_dev) { moe_err("null activation pointer"); return 0; }
-    if (!redhip_moe_route(h, layer, x_dev, ntok, nullptr, nullptr, nullptr, stream)) return 0;
-    return experts_enqueue(m, layer, x_dev, ntok, m->ids, m->weights, out_dev, static_cast<hipStream_t>(stream));
+    static const bool sep_sel = getenv("REDHIP_SEPSEL") != nullptr;   // experiment: selection as its own launch
+    const bool select_in_gateup = m->fused && ntok == 1u && !sep_sel;
+    m->skip_select = select_in_gateup;
+    const int routed = redhip_moe_route(h, layer, x_dev, ntok, nullptr, nullptr, nullptr, stream);
+    m->skip_select = false;
+    if (!routed) return 0;
+    return experts_enqueue(m, layer, x_dev, ntok, m->ids, m->weights, out_dev, static_cast<hipStream_t>(stream), select_in_gateup);
 }
 
 int redhip_moe_last_route(redhip_moe_t h, uint32_t ntok, uint32_t *ids, float *weights, float *logits, void *stream) {
@@ -259,7 +337,10 @@ int redhip_moe_last_route(redhip_moe_t h, uint32_t ntok, uint32_t *ids, float *w
     const redhip_moe_config &c = m->cfg;
     if (ids) HIP_OK(hipMemcpy(ids, m->ids, (size_t)ntok * c.top_k * 4u, hipMemcpyDeviceToHost), "ids download");
     if (weights) HIP_OK(hipMemcpy(weights, m->weights, (size_t)ntok * c.top_k * 4u, hipMemcpyDeviceToHost), "weights download");
-    if (logits) HIP_OK(hipMemcpy(logits, m->logits, (size_t)ntok * c.n_expert * 4u, hipMemcpyDeviceToHost), "logits download");
+    if (logits) {
+        const size_t pitch = 4u * (size_t)(c.n_expert + (m->fused ? 1u : 0u));
+        HIP_OK(hipMemcpy2D(logits, 4u * (size_t)c.n_expert, m->logits, pitch, 4u * (size_t)c.n_expert, ntok, hipMemcpyDeviceToHost), "logits download");
+    }
     return 1;
 }
 
@@ -293,6 +374,13 @@ int redhip_moe_dequant_resident(redhip_moe_t h, uint32_t layer, uint32_t expert,
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (which == 3u) { HIP_OK(launch_dequant_rows(c.router_type, L.router, c.n_expert, c.hidden, out_dev, s), "router dequant"); return 1; }
     const bool sh = expert == c.n_expert;
+    if (m->fused) {        // the layout the fused kernel reads
+        const uint8_t *pk = sh ? L.shared_packed : L.packed + (uint64_t)expert * m->expert_stride;
+        const uint64_t gbytes = m->gate_bytes;
+        if (which < 2u) HIP_OK(launch_dequant_packed_iq2xxs(pk + which * gbytes, c.ffn, c.hidden, false, out_dev, s), "packed gate/up dequant");
+        else HIP_OK(launch_dequant_packed_iq2xxs(pk + 2u * gbytes, c.hidden, c.ffn, false, out_dev, s), "packed down dequant");
+        return 1;
+    }
     const uint8_t *base = sh ? L.shared : L.experts + (uint64_t)expert * m->expert_stride;
     const uint64_t gb = sh ? m->sh_gate_bytes : m->gate_bytes;
     const uint32_t gu = sh ? m->sh_gu_type : m->gu_type, dn = sh ? m->sh_dn_type : m->dn_type;

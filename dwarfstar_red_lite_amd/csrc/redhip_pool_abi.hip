@@ -417,12 +417,13 @@ int rl_native_router_select_softmax_topk(const float *logits, uint32_t expert_co
     }
     if (expert_count > 1024u || top_k > 16u) { set_err(error, error_cap, "router selection supports at most 1024 experts and top-16"); return 0; }
     DevBuf buf;
-    const size_t n_f = (size_t)expert_count * 2u + 2u * top_k;
+    const size_t n_f = (size_t)expert_count * 2u + 1u + 2u * top_k;          // the selection kernel reads one extra logit (the shared gate's)
     if (!buf.reserve(n_f * sizeof(float))) { set_err(error, error_cap, "out of memory for router probabilities"); return 0; }
-    float *dl = static_cast<float *>(buf.p), *dp = dl + expert_count, *dwt = dp + expert_count;
+    float *dl = static_cast<float *>(buf.p), *dp = dl + expert_count + 1u, *dwt = dp + expert_count;
     uint32_t *dids = reinterpret_cast<uint32_t *>(dwt + top_k);
-    hipError_t e = hipMemcpy(dl, logits, (size_t)expert_count * sizeof(float), hipMemcpyHostToDevice);
-    if (e == hipSuccess) e = launch_route_select(dl, 1u, expert_count, top_k, dids, dwt, dp, nullptr, nullptr, 0u, nullptr, nullptr);
+    hipError_t e = hipMemset(dl + expert_count, 0, sizeof(float));
+    if (e == hipSuccess) e = hipMemcpy(dl, logits, (size_t)expert_count * sizeof(float), hipMemcpyHostToDevice);
+    if (e == hipSuccess) e = launch_select(dl, 1u, expert_count, top_k, dids, dwt, nullptr, dp, nullptr);
     if (e == hipSuccess) e = hipMemcpy(router_weights, dwt, (size_t)top_k * sizeof(float), hipMemcpyDeviceToHost);
     if (e == hipSuccess) e = hipMemcpy(expert_ids, dids, (size_t)top_k * sizeof(uint32_t), hipMemcpyDeviceToHost);
     if (e == hipSuccess && probabilities) e = hipMemcpy(probabilities, dp, (size_t)expert_count * sizeof(float), hipMemcpyDeviceToHost);

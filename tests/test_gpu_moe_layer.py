@@ -73,5 +73,6 @@ def test_layer_full_size_config0():
         x = torch.from_numpy(xs[t:t + 1]).cuda()
         ids, w, logits = m.route(0, x)
         out2 = m.experts(0, x, ids, w).cpu().numpy()[0]
-        assert np.array_equal(out2, out)
+        # the fused kernel accumulates expert slices with float atomics: same terms, order of addition may differ
+        assert rel_l2(out2, out) <= 1e-5
     m.close()
