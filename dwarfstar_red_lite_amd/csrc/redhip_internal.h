@@ -72,6 +72,19 @@ hipError_t launch_moe_down_combine(const ExpertSet &ex, const uint32_t *ids, con
                                    const ExpertSet &shared, const float *scalar, uint32_t hidden, uint32_t ffn,
                                    const float *act, const float *shared_act, float *out, hipStream_t s);
 
+// batched experts over pairs sorted by expert (the grouping below). uid / expert_start / n_unique on the device; n_groups
+// is the launch bound on the number of groups (groups >= *n_unique exit at once). With uid == nullptr and
+// expert_start == nullptr there is a single group (expert 0 of `ex`) whose pairs are tokens 0..n_pairs_total-1.
+hipError_t launch_batch_gateup(const ExpertSet &ex, const uint32_t *uid, const uint32_t *expert_start, const uint32_t *pair_token,
+                               const uint32_t *n_unique, uint32_t n_groups, uint32_t n_pairs_total, uint32_t hidden, uint32_t ffn,
+                               const float *x, float *act, hipStream_t s);                     // act [pairs][ffn]
+hipError_t launch_batch_down(const ExpertSet &ex, const uint32_t *uid, const uint32_t *expert_start, const uint32_t *n_unique,
+                             uint32_t n_groups, uint32_t n_pairs_total, uint32_t hidden, uint32_t ffn, const float *act, float *tmp,
+                             hipStream_t s);                                                    // tmp [pairs][hidden]
+// out[t] = sum_k pair_weight[tok_pair[t][k]] * tmp[tok_pair[t][k]] (k in selection order) + scalar[t] * sh_tmp[t]
+hipError_t launch_batch_combine(const float *tmp, const float *pair_weight, const uint32_t *tok_pair, uint32_t ntok, uint32_t top_k,
+                                const float *sh_tmp, const float *scalar, uint32_t hidden, float *out, hipStream_t s);
+
 // pair sort of [ntok][top_k] ids: see redhip_moe_group in include/redhip_moe.h
 hipError_t launch_group_pairs(const uint32_t *ids, const float *weights, uint32_t ntok, uint32_t top_k, uint32_t n_expert,
                               uint32_t *uid, uint32_t *expert_start, uint32_t *pair_token, float *pair_weight,

@@ -370,6 +370,205 @@ hipError_t launch_moe_down_combine(const ExpertSet &ex, const uint32_t *ids, con
     }
 }
 
+// ---------------------------------------------------------------- batched experts over grouped (expert, token) pairs
+
+// Pairs are sorted by expert (expert_start[u] .. expert_start[u+1]); a workgroup takes one expert and a tile of
+// rows, decodes every weight once per slice of up to kPairTile pairs and applies it to each pair's activations,
+// so an expert's bytes are read once however many tokens selected it. The shared expert runs through the same
+// kernels as a single "expert" whose pairs are all the tokens.
+constexpr int kPairTile = 8;
+
+struct PairArgs {
+    const uint8_t *base;           // expert e at base + e * stride
+    uint64_t stride, matrix_off, second_off;      // gate (or down) at matrix_off, up at second_off
+    const uint32_t *uid;           // [U] expert of group u, or nullptr: expert 0
+    const uint32_t *expert_start;  // [U + 1]
+    const uint32_t *pair_token;    // [P] token of each pair, or nullptr: pair p is token p
+    const uint32_t *n_unique;      // [1] number of groups, or nullptr: one group
+    uint32_t n_pairs_total;        // used when expert_start == nullptr: one group of this many pairs
+};
+
+template <uint32_t T, int LPR>
+__global__ __launch_bounds__(256) void batch_gateup_kernel(PairArgs a, uint32_t hidden, uint32_t ffn, const float *x, float *act) {
+    extern __shared__ float xs[];                                     // [kPairTile][padded hidden]
+    const uint32_t u = blockIdx.y;
+    if (a.n_unique && u >= a.n_unique[0]) return;
+    const uint32_t e = a.uid ? a.uid[u] : 0u;
+    const uint32_t p0 = a.expert_start ? a.expert_start[u] : 0u, p1 = a.expert_start ? a.expert_start[u + 1u] : a.n_pairs_total;
+    const uint32_t hp = hidden + (hidden >> 5);
+    const uint32_t sub = threadIdx.x % LPR, r = blockIdx.x * (256u / LPR) + threadIdx.x / LPR;
+    const uint64_t rb = (uint64_t)(hidden / 256u) * Fmt<T>::kBlock;
+    const uint8_t *grow = a.base + (uint64_t)e * a.stride + a.matrix_off + (uint64_t)r * rb;
+    const uint8_t *urow = a.base + (uint64_t)e * a.stride + a.second_off + (uint64_t)r * rb;
+    for (uint32_t c0 = p0; c0 < p1; c0 += kPairTile) {
+        const uint32_t nb = p1 - c0 < (uint32_t)kPairTile ? p1 - c0 : (uint32_t)kPairTile;
+        __syncthreads();
+        for (uint32_t i = threadIdx.x; i < nb * hidden; i += 256u) {
+            const uint32_t pi = i / hidden, col = i % hidden;
+            const uint32_t tok = a.pair_token ? a.pair_token[c0 + pi] : c0 + pi;
+            xs[pi * hp + pad32(col)] = x[(uint64_t)tok * hidden + col];
+        }
+        __syncthreads();
+        float g[kPairTile], v[kPairTile];
+#pragma unroll
+        for (int i = 0; i < kPairTile; ++i) { g[i] = 0.0f; v[i] = 0.0f; }
+        if (r < ffn) {
+            for (uint32_t c = sub; c < hidden / 32u; c += LPR) {
+                float wg[32], wu[32];
+                decode32<T>(grow, c, wg);
+                decode32<T>(urow, c, wu);
+#pragma unroll
+                for (int i = 0; i < kPairTile; ++i) {
+                    if ((uint32_t)i < nb) {
+                        const float *xv = xs + i * hp + 33u * c;
+                        float sg = 0.0f, su = 0.0f;
+#pragma unroll
+                        for (int j = 0; j < 32; ++j) { sg = fmaf(wg[j], xv[j], sg); su = fmaf(wu[j], xv[j], su); }
+                        g[i] += sg;
+                        v[i] += su;
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kPairTile; ++i) {
+            if ((uint32_t)i < nb) {
+                const float gs = sub_reduce<LPR>(g[i]), us = sub_reduce<LPR>(v[i]);
+                if (sub == 0u && r < ffn) act[(uint64_t)(c0 + i) * ffn + r] = silu_mul(gs, us);
+            }
+        }
+    }
+}
+
+template <uint32_t T, int LPR>
+__global__ __launch_bounds__(256) void batch_down_kernel(PairArgs a, uint32_t hidden, uint32_t ffn, const float *act, float *tmp) {
+    extern __shared__ float as[];                                     // [kPairTile][padded ffn]
+    const uint32_t u = blockIdx.y;
+    if (a.n_unique && u >= a.n_unique[0]) return;
+    const uint32_t e = a.uid ? a.uid[u] : 0u;
+    const uint32_t p0 = a.expert_start ? a.expert_start[u] : 0u, p1 = a.expert_start ? a.expert_start[u + 1u] : a.n_pairs_total;
+    const uint32_t fp = ffn + (ffn >> 5);
+    const uint32_t sub = threadIdx.x % LPR, r = blockIdx.x * (256u / LPR) + threadIdx.x / LPR;
+    const uint64_t rb = (uint64_t)(ffn / 256u) * Fmt<T>::kBlock;
+    const uint8_t *row = a.base + (uint64_t)e * a.stride + a.matrix_off + (uint64_t)r * rb;
+    for (uint32_t c0 = p0; c0 < p1; c0 += kPairTile) {
+        const uint32_t nb = p1 - c0 < (uint32_t)kPairTile ? p1 - c0 : (uint32_t)kPairTile;
+        __syncthreads();
+        for (uint32_t i = threadIdx.x; i < nb * ffn; i += 256u) as[(i / ffn) * fp + pad32(i % ffn)] = act[(uint64_t)c0 * ffn + i];
+        __syncthreads();
+        float s[kPairTile];
+#pragma unroll
+        for (int i = 0; i < kPairTile; ++i) s[i] = 0.0f;
+        if (r < hidden) {
+            for (uint32_t c = sub; c < ffn / 32u; c += LPR) {
+                float w[32];
+                decode32<T>(row, c, w);
+#pragma unroll
+                for (int i = 0; i < kPairTile; ++i) {
+                    if ((uint32_t)i < nb) {
+                        const float *av = as + i * fp + 33u * c;
+                        float t = 0.0f;
+#pragma unroll
+                        for (int j = 0; j < 32; ++j) t = fmaf(w[j], av[j], t);
+                        s[i] += t;
+                    }
+                }
+            }
+        }
+#pragma unroll
+        for (int i = 0; i < kPairTile; ++i) {
+            if ((uint32_t)i < nb) {
+                const float t = sub_reduce<LPR>(s[i]);
+                if (sub == 0u && r < hidden) tmp[(uint64_t)(c0 + i) * hidden + r] = t;
+            }
+        }
+    }
+}
+
+// out[t][r] = sum_k pair_weight[p_k] * tmp[p_k][r] (p_k = tok_pair[t][k], selection order) + scalar[t] * sh_tmp[t][r]
+__global__ __launch_bounds__(256) void batch_combine_kernel(const float *tmp, const float *pair_weight, const uint32_t *tok_pair, uint32_t top_k,
+                                                            const float *sh_tmp, const float *scalar, uint32_t hidden, float *out) {
+    const uint32_t r = blockIdx.x * 256u + threadIdx.x, t = blockIdx.y;
+    if (r >= hidden) return;
+    float acc = 0.0f;
+    for (uint32_t k = 0; k < top_k; ++k) {
+        const uint32_t p = tok_pair[(uint64_t)t * top_k + k];
+        acc = fmaf(pair_weight[p], tmp[(uint64_t)p * hidden + r], acc);
+    }
+    if (sh_tmp) acc = fmaf(scalar[t], sh_tmp[(uint64_t)t * hidden + r], acc);
+    out[(uint64_t)t * hidden + r] = acc;
+}
+
+template <uint32_t T>
+static hipError_t batch_gateup_dispatch(const PairArgs &a, uint32_t n_groups, uint32_t hidden, uint32_t ffn, const float *x, float *act, hipStream_t s) {
+    const uint32_t lpr = lanes_per_row(hidden);
+    const dim3 grid((ffn + 256u / lpr - 1u) / (256u / lpr), n_groups);
+    const size_t lds = (size_t)kPairTile * padded_floats(hidden) * sizeof(float);
+#define REDHIP_BGU(L)                                                                                                              \
+    do {                                                                                                                           \
+        static bool attr = false;                                                                                                  \
+        if (!attr) {                                                                                                               \
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(batch_gateup_kernel<T, L>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
+            if (e != hipSuccess) return e;                                                                                         \
+            attr = true;                                                                                                           \
+        }                                                                                                                          \
+        REDHIP_LAUNCH((batch_gateup_kernel<T, L>), grid, dim3(256), lds, s, a, hidden, ffn, x, act);                               \
+    } while (0)
+    switch (lpr) {
+        case 64: REDHIP_BGU(64); break;
+        case 32: REDHIP_BGU(32); break;
+        case 16: REDHIP_BGU(16); break;
+        default: REDHIP_BGU(8); break;
+    }
+#undef REDHIP_BGU
+    return hipGetLastError();
+}
+
+template <uint32_t T>
+static hipError_t batch_down_dispatch(const PairArgs &a, uint32_t n_groups, uint32_t hidden, uint32_t ffn, const float *act, float *tmp, hipStream_t s) {
+    const uint32_t lpr = lanes_per_row(ffn);
+    const dim3 grid((hidden + 256u / lpr - 1u) / (256u / lpr), n_groups);
+    const size_t lds = (size_t)kPairTile * padded_floats(ffn) * sizeof(float);
+    switch (lpr) {
+        case 64: REDHIP_LAUNCH((batch_down_kernel<T, 64>), grid, dim3(256), lds, s, a, hidden, ffn, act, tmp); break;
+        case 32: REDHIP_LAUNCH((batch_down_kernel<T, 32>), grid, dim3(256), lds, s, a, hidden, ffn, act, tmp); break;
+        case 16: REDHIP_LAUNCH((batch_down_kernel<T, 16>), grid, dim3(256), lds, s, a, hidden, ffn, act, tmp); break;
+        default: REDHIP_LAUNCH((batch_down_kernel<T, 8>), grid, dim3(256), lds, s, a, hidden, ffn, act, tmp); break;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_batch_gateup(const ExpertSet &ex, const uint32_t *uid, const uint32_t *expert_start, const uint32_t *pair_token,
+                               const uint32_t *n_unique, uint32_t n_groups, uint32_t n_pairs_total, uint32_t hidden, uint32_t ffn,
+                               const float *x, float *act, hipStream_t s) {
+    if (!n_groups || hidden % 256u || ffn % 256u || (size_t)kPairTile * padded_floats(hidden) * 4u > 160u * 1024u || n_groups > 65535u) return hipErrorInvalidValue;
+    const PairArgs a{ex.base, ex.stride, 0u, ex.gate_bytes, uid, expert_start, pair_token, n_unique, n_pairs_total};
+    switch (ex.gate_up_type) {
+        case T_IQ2_XXS: return batch_gateup_dispatch<T_IQ2_XXS>(a, n_groups, hidden, ffn, x, act, s);
+        case T_IQ3_S: return batch_gateup_dispatch<T_IQ3_S>(a, n_groups, hidden, ffn, x, act, s);
+        case T_Q6_K: return batch_gateup_dispatch<T_Q6_K>(a, n_groups, hidden, ffn, x, act, s);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+hipError_t launch_batch_down(const ExpertSet &ex, const uint32_t *uid, const uint32_t *expert_start, const uint32_t *n_unique,
+                             uint32_t n_groups, uint32_t n_pairs_total, uint32_t hidden, uint32_t ffn, const float *act, float *tmp, hipStream_t s) {
+    if (!n_groups || hidden % 256u || ffn % 256u || n_groups > 65535u) return hipErrorInvalidValue;
+    const PairArgs a{ex.base, ex.stride, ex.gate_bytes + ex.up_bytes, 0u, uid, expert_start, nullptr, n_unique, n_pairs_total};
+    switch (ex.down_type) {
+        case T_IQ2_XXS: return batch_down_dispatch<T_IQ2_XXS>(a, n_groups, hidden, ffn, act, tmp, s);
+        case T_IQ3_S: return batch_down_dispatch<T_IQ3_S>(a, n_groups, hidden, ffn, act, tmp, s);
+        case T_Q6_K: return batch_down_dispatch<T_Q6_K>(a, n_groups, hidden, ffn, act, tmp, s);
+        default: return hipErrorInvalidValue;
+    }
+}
+
+hipError_t launch_batch_combine(const float *tmp, const float *pair_weight, const uint32_t *tok_pair, uint32_t ntok, uint32_t top_k,
+                                const float *sh_tmp, const float *scalar, uint32_t hidden, float *out, hipStream_t s) {
+    REDHIP_LAUNCH(batch_combine_kernel, dim3((hidden + 255u) / 256u, ntok), dim3(256), 0, s, tmp, pair_weight, tok_pair, top_k, sh_tmp, scalar, hidden, out);
+    return hipGetLastError();
+}
+
 // ---------------------------------------------------------------- token grouping (pair sort)
 
 // One workgroup. For every (token, k) pair p = t * top_k + k:

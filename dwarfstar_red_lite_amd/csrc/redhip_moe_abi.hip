@@ -53,6 +53,9 @@ struct Moe {
     void *xh = nullptr, *xl = nullptr;       // fp16 [hidden] each
     int *xexp = nullptr;
     bool skip_select = false;                // forward(): the gate/up kernel selects, route() skips its own selection
+    // batched path (ntok > 1): pairs grouped by expert
+    uint32_t *uid = nullptr, *expert_start = nullptr, *pair_token = nullptr, *tok_pair = nullptr, *n_unique = nullptr;
+    float *pair_weight = nullptr, *tmp = nullptr, *sh_tmp = nullptr;
     void *act_h = nullptr, *act_l = nullptr; // fp16 [top_k + 1][ffn] each
     int *act_exp = nullptr;                  // [top_k + 1][ffn / 32]
 
@@ -85,7 +88,23 @@ __global__ __launch_bounds__(256) void scalar_gate_kernel(const float *gate_inp,
 int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const uint32_t *ids, const float *weights,
                     float *out, hipStream_t s, bool select_here = false) {
     const redhip_moe_config &c = m->cfg;
-    if (ntok != 1u) { moe_err("batched expert execution is not available in this build (ntok=%u)", ntok); return 0; }
+    if (ntok > 1u) {       // group the (token, expert) pairs by expert, run each distinct expert once over its tokens
+        const uint32_t P = ntok * c.top_k, n_groups = P < c.n_expert ? P : c.n_expert;
+        const ExpertSet ex = m->routed(layer), sh = m->shared(layer);
+        prof_set_stage(ST_GROUP);
+        HIP_OK(launch_group_pairs(ids, weights, ntok, c.top_k, c.n_expert, m->uid, m->expert_start, m->pair_token, m->pair_weight,
+                                  m->tok_pair, m->n_unique, s), "grouping launch");
+        prof_set_stage(ST_BATCH_GATEUP);
+        HIP_OK(launch_batch_gateup(ex, m->uid, m->expert_start, m->pair_token, m->n_unique, n_groups, P, c.hidden, c.ffn, x, m->act, s), "batched gate/up launch");
+        HIP_OK(launch_batch_gateup(sh, nullptr, nullptr, nullptr, nullptr, 1u, ntok, c.hidden, c.ffn, x, m->sh_act, s), "batched shared gate/up launch");
+        prof_set_stage(ST_BATCH_DOWN);
+        HIP_OK(launch_batch_down(ex, m->uid, m->expert_start, m->n_unique, n_groups, P, c.hidden, c.ffn, m->act, m->tmp, s), "batched down launch");
+        HIP_OK(launch_batch_down(sh, nullptr, nullptr, nullptr, 1u, ntok, c.hidden, c.ffn, m->sh_act, m->sh_tmp, s), "batched shared down launch");
+        prof_set_stage(ST_BATCH_COMBINE);
+        HIP_OK(launch_batch_combine(m->tmp, m->pair_weight, m->tok_pair, ntok, c.top_k, m->sh_tmp, m->scalar, c.hidden, out, s), "batched combine launch");
+        prof_set_stage(ST_OTHER);
+        return 1;
+    }
     if (m->fused) {          // xh / xl / scalar come from the router kernel or the prep kernel
         const Layer &L = m->layers[layer];
         prof_set_stage(ST_GATEUP);
@@ -167,7 +186,8 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
     const size_t ws_bytes = align256(T * (c.n_expert + 1u) * 4u) + 2u * align256(T * c.top_k * 4u) + align256(T * 4u) +
                             align256(T * c.top_k * c.ffn * 4u) + align256(T * c.ffn * 4u) +
                             2u * align256(2u * T * c.hidden) + align256(4u * T) + 2u * align256(2u * (c.top_k + 1u) * c.ffn) +
-                            align256(4u * (c.top_k + 1u) * (c.ffn / 32u));
+                            align256(4u * (c.top_k + 1u) * (c.ffn / 32u)) +
+                            (T > 1u ? 6u * align256(4u * (T * c.top_k + 2u)) + align256(4u * T * c.top_k * c.hidden) + align256(4u * T * c.hidden) : 0u);
     ok = ok && hipMalloc(reinterpret_cast<void **>(&m->ws), ws_bytes) == hipSuccess;
     if (!ok) {
         moe_err("failed to allocate resident MoE memory (%llu bytes so far)", (unsigned long long)m->resident);
@@ -186,7 +206,18 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
     m->xexp = reinterpret_cast<int *>(w); w += align256(4u * T);
     m->act_h = w; w += align256(2u * (c.top_k + 1u) * c.ffn);
     m->act_l = w; w += align256(2u * (c.top_k + 1u) * c.ffn);
-    m->act_exp = reinterpret_cast<int *>(w);
+    m->act_exp = reinterpret_cast<int *>(w); w += align256(4u * (c.top_k + 1u) * (c.ffn / 32u));
+    if (T > 1u) {
+        const size_t pw = align256(4u * (T * c.top_k + 2u));
+        m->uid = reinterpret_cast<uint32_t *>(w); w += pw;
+        m->expert_start = reinterpret_cast<uint32_t *>(w); w += pw;
+        m->pair_token = reinterpret_cast<uint32_t *>(w); w += pw;
+        m->tok_pair = reinterpret_cast<uint32_t *>(w); w += pw;
+        m->n_unique = reinterpret_cast<uint32_t *>(w); w += pw;
+        m->pair_weight = reinterpret_cast<float *>(w); w += pw;
+        m->tmp = reinterpret_cast<float *>(w); w += align256(4u * T * c.top_k * c.hidden);
+        m->sh_tmp = reinterpret_cast<float *>(w);
+    }
     if (hipMemset(m->ws, 0, ws_bytes) != hipSuccess) { moe_err("failed to clear the MoE workspace"); redhip_moe_destroy(m); return nullptr; }
     // first launches copy the codebooks to the device; do it here so that forward never synchronises
     if (launch_dequant_rows(T_F32, m->ws, 1u, 32u, m->logits, nullptr) != hipSuccess || hipDeviceSynchronize() != hipSuccess) {
