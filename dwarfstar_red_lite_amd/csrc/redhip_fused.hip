@@ -241,13 +241,21 @@ struct SelectOut {
     uint32_t ids[16];
     float w[16];
     float scalar;
-    uint32_t tmp[16];
-    float tmp_p[16];
+    uint32_t tmp[64];
+    float tmp_p[64];
 };
+
+#ifdef REDHIP_SEL_TS
+__device__ unsigned long long g_sel_ts[16];
+#define SEL_TS(i) do { if (threadIdx.x == 0u) g_sel_ts[i] = wall_clock64(); } while (0)
+#else
+#define SEL_TS(i) do {} while (0)
+#endif
 
 template <int PER>
 __device__ void wave_select_topk(const float *logits, uint32_t E, uint32_t K, SelectOut *out, float *probs = nullptr) {
     const uint32_t lane = threadIdx.x & 63u;
+    SEL_TS(0);
     float l[PER];
     float m = -INFINITY;
 #pragma unroll
@@ -258,6 +266,7 @@ __device__ void wave_select_topk(const float *logits, uint32_t E, uint32_t K, Se
     }
     const float gate_logit = logits[E];                      // shared expert's gate logit rides along
     m = wave_max(m);
+    SEL_TS(1);
     float p[PER];
     double part = 0.0;
 #pragma unroll
@@ -265,9 +274,11 @@ __device__ void wave_select_topk(const float *logits, uint32_t E, uint32_t K, Se
         p[s] = lane + 64u * s < E ? expf(l[s] - m) : 0.0f;
         part += (double)p[s];
     }
+    SEL_TS(2);
     const double denom = wave_sum_d(part);
     const bool bad = !(denom > 0.0) || isinf(denom) || isnan(denom);
     const float inv = bad ? 0.0f : (float)(1.0 / denom);
+    SEL_TS(3);
     uint32_t key[PER];
 #pragma unroll
     for (int s = 0; s < PER; ++s) {
@@ -275,55 +286,98 @@ __device__ void wave_select_topk(const float *logits, uint32_t E, uint32_t K, Se
         key[s] = lane + 64u * s < E ? (__float_as_uint(p[s]) | 0x80000000u) : 0u;   // valid keys have the top bit set: padding never counts
         if (probs && lane + 64u * s < E) probs[lane + 64u * s] = p[s];
     }
-    // largest T with count(key >= T) >= K; bit 31 is set in every valid key
-    uint32_t T = 0x80000000u;
+    SEL_TS(4);
+    // Level 1: the K-th largest of the 64 per-lane maxima (tau) is a lower bound of the K-th largest key, so the
+    // winners are among the keys >= tau - usually a dozen of them. Bisection on one value per lane is cheap.
+    uint32_t lm = key[0];
+#pragma unroll
+    for (int s = 1; s < PER; ++s) lm = lm > key[s] ? lm : key[s];
+    uint32_t tau = 0x80000000u;                          // bit 31 is set in every valid key
 #pragma unroll 1
     for (int bit = 30; bit >= 0; --bit) {
-        const uint32_t cand = T | (1u << bit);
-        uint32_t c = 0u;
-#pragma unroll
-        for (int s = 0; s < PER; ++s) c += wave_count(key[s] >= cand);
-        T = c >= K ? cand : T;
+        const uint32_t cand = tau | (1u << bit);
+        tau = wave_count(lm >= cand) >= K ? cand : tau;
     }
-    uint32_t above = 0u;
+    SEL_TS(5);
+    uint32_t n_c = 0u;
 #pragma unroll
-    for (int s = 0; s < PER; ++s) above += wave_count(key[s] > T);
-    const uint32_t need_ties = K - above;                    // >= 1
-    // winners to LDS, one slot each: everything above T, then the first need_ties equal to T in index order
-    uint32_t n_sel = 0u, ties_seen = 0u;
+    for (int s = 0; s < PER; ++s) n_c += wave_count(key[s] >= tau);
+    SEL_TS(6);
+    uint32_t mine = 0xffffffffu, kmine = 0u, rank = 0u;
+    if (n_c <= 64u) {
+        // Level 2: candidates to LDS in index order, one per lane, ranked against each other with lane broadcasts:
+        // rank = number of candidates that beat this one under (p desc, index asc). rank < K <=> selected, and the
+        // rank is the position in selection order.
+        uint32_t n = 0u;
 #pragma unroll
-    for (int s = 0; s < PER; ++s) {                          // index order = s-major over lanes
-        const bool gt = key[s] > T, eq = key[s] == T;
-        const uint64_t eq_mask = __ballot(eq);
-        const uint32_t eq_before = ties_seen + (uint32_t)__popcll(eq_mask & ((1ull << lane) - 1ull));
-        const bool take = gt || (eq && eq_before < need_ties);
-        const uint64_t take_mask = __ballot(take);
-        if (take) {
-            const uint32_t pos = n_sel + (uint32_t)__popcll(take_mask & ((1ull << lane) - 1ull));
-            out->tmp[pos] = lane + 64u * s;
-            out->tmp_p[pos] = p[s];
+        for (int s = 0; s < PER; ++s) {
+            const bool take = key[s] >= tau;
+            const uint64_t mask = __ballot(take);
+            if (take) {
+                const uint32_t pos = n + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
+                out->tmp[pos] = lane + 64u * s;
+                out->tmp_p[pos] = p[s];
+            }
+            n += (uint32_t)__popcll(mask);
         }
-        n_sel += (uint32_t)__popcll(take_mask);
-        ties_seen += (uint32_t)__popcll(eq_mask);
+        wave_lds_sync();
+        if (lane < n_c) { mine = out->tmp[lane]; kmine = __float_as_uint(out->tmp_p[lane]) | 0x80000000u; }
+        for (uint32_t q = 0; q < n_c; ++q) {
+            const uint32_t o = __shfl(mine, (int)q, 64), ko = __shfl(kmine, (int)q, 64);
+            rank += (ko > kmine || (ko == kmine && o < mine)) ? 1u : 0u;
+        }
+        if (lane >= n_c) rank = 0xffffffffu;
+    } else {
+        // Heavy ties (more than 64 keys at or above tau): bisection over all keys, ties at the threshold in index order.
+        uint32_t T = 0x80000000u;
+#pragma unroll 1
+        for (int bit = 30; bit >= 0; --bit) {
+            const uint32_t cand = T | (1u << bit);
+            uint32_t c = 0u;
+#pragma unroll
+            for (int s = 0; s < PER; ++s) c += wave_count(key[s] >= cand);
+            T = c >= K ? cand : T;
+        }
+        uint32_t above = 0u;
+#pragma unroll
+        for (int s = 0; s < PER; ++s) above += wave_count(key[s] > T);
+        const uint32_t need_ties = K - above;                    // >= 1
+        uint32_t n_sel = 0u, ties_seen = 0u;
+#pragma unroll
+        for (int s = 0; s < PER; ++s) {                          // index order = s-major over lanes
+            const bool gt = key[s] > T, eq = key[s] == T;
+            const uint64_t eq_mask = __ballot(eq);
+            const uint32_t eq_before = ties_seen + (uint32_t)__popcll(eq_mask & ((1ull << lane) - 1ull));
+            const bool take = gt || (eq && eq_before < need_ties);
+            const uint64_t take_mask = __ballot(take);
+            if (take) {
+                const uint32_t pos = n_sel + (uint32_t)__popcll(take_mask & ((1ull << lane) - 1ull));
+                out->tmp[pos] = lane + 64u * s;
+                out->tmp_p[pos] = p[s];
+            }
+            n_sel += (uint32_t)__popcll(take_mask);
+            ties_seen += (uint32_t)__popcll(eq_mask);
+        }
+        wave_lds_sync();
+        if (lane < K) { mine = out->tmp[lane]; kmine = __float_as_uint(out->tmp_p[lane]) | 0x80000000u; }
+        for (uint32_t q = 0; q < K; ++q) {
+            const uint32_t o = __shfl(mine, (int)q, 64), ko = __shfl(kmine, (int)q, 64);
+            rank += (ko > kmine || (ko == kmine && o < mine)) ? 1u : 0u;
+        }
+        if (lane >= K) rank = 0xffffffffu;
     }
-    wave_lds_sync();
-    // lane q < K owns winner q; order by (p desc, index asc) with lane broadcasts
-    const uint32_t mine = lane < K ? out->tmp[lane] : 0xffffffffu;
-    const float pm = lane < K ? out->tmp_p[lane] : -1.0f;
-    uint32_t rank = 0u;
-    for (uint32_t q = 0; q < K; ++q) {
-        const uint32_t o = __shfl(mine, (int)q, 64);
-        const float po = __shfl(pm, (int)q, 64);
-        rank += (po > pm || (po == pm && o < mine)) ? 1u : 0u;
-    }
-    const double sum = wave_sum_d(lane < K ? (double)pm : 0.0);
+    SEL_TS(7);
+    const bool selected = rank < K;
+    const float pm = __uint_as_float(kmine & 0x7fffffffu);
+    const double sum = wave_sum_d(selected ? (double)pm : 0.0);
     const bool bad2 = bad || !(sum > 0.0) || isinf(sum) || isnan(sum);
     const float invs = bad2 ? __uint_as_float(0x7fc00000u) : (float)(1.0 / sum);     // NaN weights flag an invalid softmax
-    if (lane < K) {
+    if (selected) {
         out->ids[rank] = mine < E ? mine : rank;
         out->w[rank] = pm * invs;
     }
     if (lane == 0u) out->scalar = 1.0f / (1.0f + expf(-gate_logit));
+    SEL_TS(8);
 }
 
 // stand-alone selection (one wave per token): ids / weights [ntok][top_k], scalar [ntok]
