@@ -245,11 +245,12 @@ struct SelectOut {
     float tmp_p[64];
 };
 
-#ifdef REDHIP_SEL_TS
-__device__ unsigned long long g_sel_ts[16];
-#define SEL_TS(i) do { if (threadIdx.x == 0u) g_sel_ts[i] = wall_clock64(); } while (0)
-#else
 #define SEL_TS(i) do {} while (0)
+#ifdef REDHIP_KTS
+__device__ unsigned long long g_kts[256 * 32], g_kts2[256 * 32];
+#define KTS(i) do { if (threadIdx.x == 0u && blockIdx.x < 256u && (i) < 32u) { g_kts[blockIdx.x * 32u + (i)] = wall_clock64(); g_kts2[blockIdx.x * 32u + (i)] = clock64(); } } while (0)
+#else
+#define KTS(i) do {} while (0)
 #endif
 
 template <int PER>
@@ -431,11 +432,13 @@ hipError_t launch_prep(const float *x, const float *gate_inp, uint32_t ntok, uin
 
 // ---------------------------------------------------------------- gate/up + SwiGLU and down + combine
 
+// block scale d of a packed row: one conversion instruction (fp16 subnormals are exact, a NaN stays a NaN)
+__device__ __forceinline__ float scale_to_f32(uint32_t h) { return (float)__builtin_bit_cast(_Float16, (uint16_t)h); }
+
 constexpr int kWaves = 16;                      // 1024 lanes per gate/up workgroup
 constexpr uint32_t kMagBytes = 256u * 16u;      // eight fp16 magnitudes per grid entry
-constexpr uint32_t kSignBytes = 128u * 16u;     // eight fp16 sign masks per 7-bit sign field
 
-// LDS decode tables, built by the first 384 lanes of a workgroup
+// LDS decode table (eight fp16 magnitudes per grid entry), built by the first 256 lanes of a workgroup
 __device__ __forceinline__ void build_tables(uint8_t *lds, uint32_t tid, uint64_t grid_entry) {
     if (tid < 256u) {
         uint32_t w4[4];
@@ -445,12 +448,6 @@ __device__ __forceinline__ void build_tables(uint8_t *lds, uint32_t tid, uint64_
             w4[i] = (uint32_t)__builtin_bit_cast(uint16_t, lo) | ((uint32_t)__builtin_bit_cast(uint16_t, hi) << 16);
         }
         *reinterpret_cast<uint4 *>(lds + (size_t)tid * 16u) = make_uint4(w4[0], w4[1], w4[2], w4[3]);
-    } else if (tid < 384u) {
-        const uint32_t s7 = tid - 256u, s8 = s7 | ((__popc(s7) & 1u) << 7);
-        uint32_t w4[4];
-#pragma unroll
-        for (int i = 0; i < 4; ++i) w4[i] = (((s8 >> (2 * i)) & 1u) << 15) | (((s8 >> (2 * i + 1)) & 1u) << 31);
-        *reinterpret_cast<uint4 *>(lds + kMagBytes + (size_t)s7 * 16u) = make_uint4(w4[0], w4[1], w4[2], w4[3]);
     }
 }
 
@@ -464,18 +461,40 @@ __device__ __forceinline__ void halve_step(float *v, uint32_t lane) {      // N 
         v[i] = keep + __shfl_xor(give, OFF, 64);
     }
 }
-// sum of `v` over the 16 lanes that share lane % 4, for UPW values at once
+// sum of `v` over the 16 lanes that share lane % 4, for UPW values at once. A lane is (row = lane / 16, b = lane / 4 % 4,
+// j = lane % 4). Swapping the upper 32 lanes of one value with the lower 32 of another and adding leaves each half of
+// the wave with one value summed over both halves; the same with odd and even rows of 16 leaves row r with value r
+// summed over all rows; two rotating adds inside the row finish the sum over b.
+__device__ __forceinline__ float swap_add_32(float a, float b) {
+    const auto r = __builtin_amdgcn_permlane32_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float swap_add_16(float a, float b) {
+    const auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(a), __float_as_uint(b), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
+}
+__device__ __forceinline__ float row_sum_b(float s) {
+    s += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(s), 0x128, 0xf, 0xf, false));   // row_ror:8
+    s += __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(s), 0x124, 0xf, 0xf, false));   // row_ror:4
+    return s;
+}
 template <int UPW>
 __device__ __forceinline__ float quad_column_reduce(float *v, uint32_t lane) {
     static_assert(UPW == 1 || UPW == 2 || UPW == 4 || UPW == 8, "units per wave");
-    if constexpr (UPW >= 2) halve_step<UPW, 32>(v, lane);
-    if constexpr (UPW >= 4) halve_step<UPW / 2, 16>(v, lane);
-    if constexpr (UPW >= 8) halve_step<UPW / 4, 8>(v, lane);
-    constexpr int kFirstPlain = UPW >= 8 ? 4 : UPW >= 4 ? 8 : UPW >= 2 ? 16 : 32;
-    float r = v[0];
-#pragma unroll
-    for (int off = kFirstPlain; off >= 4; off >>= 1) r += __shfl_xor(r, off, 64);
-    return r;
+    if constexpr (UPW == 8) {
+        halve_step<8, 32>(v, lane);
+        halve_step<4, 16>(v, lane);
+        halve_step<2, 8>(v, lane);
+        return v[0] + __shfl_xor(v[0], 4, 64);
+    } else if constexpr (UPW == 4) {
+        return row_sum_b(swap_add_16(swap_add_32(v[0], v[2]), swap_add_32(v[1], v[3])));
+    } else if constexpr (UPW == 2) {
+        const float h = swap_add_32(v[0], v[1]);
+        return row_sum_b(swap_add_16(h, h));
+    } else {
+        const float h = swap_add_32(v[0], v[0]);
+        return row_sum_b(swap_add_16(h, h));
+    }
 }
 // the unit whose total a lane holds after quad_column_reduce, and whether this lane is the one that stores it
 template <int UPW> __device__ __forceinline__ uint32_t reduced_unit(uint32_t lane) {
@@ -490,6 +509,22 @@ template <int UPW> __device__ __forceinline__ bool reduced_writer(uint32_t lane)
     return (lane & kPlainBits) == 0u;
 }
 
+// Eight signed fp16 weights of one grid entry: magnitudes from the LDS table, signs placed by integer arithmetic.
+// s8 = s7 | parity << 7 holds one sign bit per weight; weight 2i sits in bits 0..15 of word i, weight 2i + 1 in
+// bits 16..31, so word i needs bit 2i of s8 at bit 15 and bit 2i + 1 at bit 31: one 24-bit multiply by
+// 2^(7 - 2i) + 2^(22 - 2i) of s8 << 8 puts both there (the two shifted copies do not overlap).
+union WeightQuad { uint32_t u[2]; half4_t h; };
+__device__ __forceinline__ void place_signs(uint4 m, uint32_t s7, WeightQuad &b0, WeightQuad &b1) {
+    const uint32_t s8s = (s7 << 8) | ((__popc(s7) & 1u) << 15);
+    b0.u[0] = (__umul24(s8s, (1u << 7) | (1u << 22)) & 0x80008000u) | m.x;
+    b0.u[1] = (__umul24(s8s, (1u << 5) | (1u << 20)) & 0x80008000u) | m.y;
+    b1.u[0] = (__umul24(s8s, (1u << 3) | (1u << 18)) & 0x80008000u) | m.z;
+    b1.u[1] = (__umul24(s8s, (1u << 1) | (1u << 16)) & 0x80008000u) | m.w;
+}
+__device__ __forceinline__ void signed_weights(const uint8_t *lds, uint32_t idx, uint32_t s7, WeightQuad &b0, WeightQuad &b1) {
+    place_signs(*reinterpret_cast<const uint4 *>(lds + (idx << 4)), s7, b0, b1);
+}
+
 // 32 weights of one group against the lane's activation operand: (hi . w + lo . w * 2^-11) * (2 * scale + 1).
 // v_mfma_f32_4x4x4_16B_f16: lanes 4b..4b+3 form block b; lane j of a block supplies row j of A (the activation
 // halves: j = 0 hi, j = 1 lo, others zero) and column j of B (its own four weights), and receives column j of
@@ -499,11 +534,8 @@ __device__ __forceinline__ float group_dot(uint2 q, const half4_t *ax, const uin
 #pragma unroll
     for (uint32_t l = 0; l < 4u; ++l) {
         const uint32_t idx = (q.x >> (8u * l)) & 255u, s7 = (q.y >> (7u * l)) & 127u;
-        const uint4 m = *reinterpret_cast<const uint4 *>(lds + (idx << 4));
-        const uint4 sg = *reinterpret_cast<const uint4 *>(lds + kMagBytes + (s7 << 4));
-        union { uint32_t u[2]; half4_t h; } b0, b1;
-        b0.u[0] = m.x ^ sg.x; b0.u[1] = m.y ^ sg.y;
-        b1.u[0] = m.z ^ sg.z; b1.u[1] = m.w ^ sg.w;
+        WeightQuad b0, b1;
+        signed_weights(lds, idx, s7, b0, b1);
         acc = __builtin_amdgcn_mfma_f32_4x4x4f16(ax[2u * l], b0.h, acc, 0, 0, 0);
         acc = __builtin_amdgcn_mfma_f32_4x4x4f16(ax[2u * l + 1u], b1.h, acc, 0, 0, 0);
     }
@@ -542,7 +574,7 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_select_kernel(GateUpArgs a
     constexpr int NW = kWaves;
     constexpr int UPW = 16 * NKC / NW;                 // (row-quad, K-chunk) units per wave
     static_assert(UPW >= 1 && UPW * NW == 16 * NKC, "waves must tile the 16 row-quads x NKC chunks");
-    __shared__ __attribute__((aligned(16))) uint8_t lds[kMagBytes + kSignBytes];
+    __shared__ __attribute__((aligned(16))) uint8_t lds[kMagBytes];
     __shared__ float part[NKC * 64];
     __shared__ SelectOut sel;
 
@@ -596,7 +628,7 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_select_kernel(GateUpArgs a
     }
     float v[UPW];
 #pragma unroll
-    for (int u = 0; u < UPW; ++u) v[u] = group_dot(wq[u], ax, lds) * half_bits_to_f32(wd[u]);
+    for (int u = 0; u < UPW; ++u) v[u] = group_dot(wq[u], ax, lds) * scale_to_f32(wd[u]);
     const float tot = quad_column_reduce<UPW>(v, lane);
     if (reduced_writer<UPW>(lane)) {
         const uint32_t quad = q0 + (NW / NKC) * reduced_unit<UPW>(lane);
@@ -636,7 +668,7 @@ struct DownArgs {
 // 8 output rows per workgroup; wave s (< top_k + 1) owns slot s: both row quads of the workgroup against all
 // ffn columns (ffn = 512: 16 groups = the 16 lane blocks of a wave). Slots are then added in selection order.
 __global__ __launch_bounds__(kWaves * 64) void down_combine_kernel(DownArgs a) {
-    __shared__ __attribute__((aligned(16))) uint8_t lds[kMagBytes + kSignBytes];
+    __shared__ __attribute__((aligned(16))) uint8_t lds[kMagBytes];
     __shared__ float part[17 * 8];
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
     const uint32_t H = a.hidden, F = a.ffn, FG = F / 32u, FB = F / 256u, n_slot = a.top_k + 1u;
@@ -672,7 +704,7 @@ __global__ __launch_bounds__(kWaves * 64) void down_combine_kernel(DownArgs a) {
                 load_act_operand(ax, a.act_h + (uint64_t)wave * F + 32u * G, a.act_l + (uint64_t)wave * F + 32u * G, j);
                 const float sc = exp2i(a.act_exp[wave * FG + G]);
 #pragma unroll
-                for (int q = 0; q < 2; ++q) tot[q] += group_dot(dq[q][c], ax, lds) * half_bits_to_f32(dd[q][c]) * sc;
+                for (int q = 0; q < 2; ++q) tot[q] += group_dot(dq[q][c], ax, lds) * scale_to_f32(dd[q][c]) * sc;
             }
         }
         const float r = quad_column_reduce<2>(tot, lane);
@@ -685,6 +717,408 @@ __global__ __launch_bounds__(kWaves * 64) void down_combine_kernel(DownArgs a) {
         sum = fmaf(a.scalar[0] * 0.125f, part[a.top_k * 8u + tid], sum);
         a.out[row0 + tid] = sum;
     }
+}
+
+// ---------------------------------------------------------------- small batches (2..16 tokens): select + group, batched gate/up, batched down
+
+// One workgroup: wave t selects the experts of token t, then wave 0 sorts the (token, k) pairs by expert. Same
+// outputs as the host pair sort it replaces: groups in first-appearance order, pairs of a group in token order.
+// Pairs sit two per lane (p = lane, lane + 64), so at most 128 pairs (e.g. 8 tokens x top-16, 12 x top-10).
+__global__ __launch_bounds__(1024) void select_group_kernel(const float *logits, uint32_t ntok, uint32_t E, uint32_t K,
+                                                            uint32_t *ids, float *weights, float *scalar, uint32_t *uid,
+                                                            uint32_t *expert_start, uint32_t *pair_token, float *pair_weight,
+                                                            uint32_t *tok_pair, uint32_t *n_unique) {
+    __shared__ SelectOut sel[16];
+    __shared__ uint32_t group_of_first[128];
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63u;
+    if (wave < ntok) {
+        const float *l = logits + (uint64_t)wave * (E + 1u);
+        if (E <= 512u) wave_select_topk<8>(l, E, K, &sel[wave]); else wave_select_topk<16>(l, E, K, &sel[wave]);
+        wave_lds_sync();
+        if (lane < K) { ids[wave * K + lane] = sel[wave].ids[lane]; weights[wave * K + lane] = sel[wave].w[lane]; }
+        if (lane == 0u) scalar[wave] = sel[wave].scalar;
+    }
+    __syncthreads();
+    if (wave != 0u) return;
+    const uint32_t P = ntok * K;
+    uint32_t e[2], first[2], before[2];
+    float w[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const uint32_t p = lane + 64u * h;
+        e[h] = p < P ? sel[p / K].ids[p % K] : 0xffffffffu - p;      // padding never matches anything
+        w[h] = p < P ? sel[p / K].w[p % K] : 0.0f;
+        first[h] = p;
+        before[h] = 0u;
+    }
+    for (uint32_t q = 0; q < P; ++q) {                              // q-th pair broadcast to all lanes
+        const uint32_t eq = __shfl(q < 64u ? e[0] : e[1], (int)(q & 63u), 64);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const uint32_t p = lane + 64u * h;
+            if (eq == e[h]) { first[h] = first[h] < q ? first[h] : q; before[h] += q < p ? 1u : 0u; }
+        }
+    }
+    // groups are numbered by the order of their first pair
+    uint32_t grp[2];
+    const bool is_first0 = lane < P && first[0] == lane, is_first1 = lane + 64u < P && first[1] == lane + 64u;
+    const uint64_t f0 = __ballot(is_first0), f1 = __ballot(is_first1);
+    const uint32_t U = (uint32_t)__popcll(f0) + (uint32_t)__popcll(f1);
+    if (is_first0) group_of_first[lane] = (uint32_t)__popcll(f0 & ((1ull << lane) - 1ull));
+    if (is_first1) group_of_first[lane + 64u] = (uint32_t)__popcll(f0) + (uint32_t)__popcll(f1 & ((1ull << lane) - 1ull));
+    wave_lds_sync();
+#pragma unroll
+    for (int h = 0; h < 2; ++h) grp[h] = lane + 64u * h < P ? group_of_first[first[h]] : 0xffffffffu;
+    // start of a group = number of pairs in earlier groups
+    uint32_t start[2] = {0u, 0u};
+    for (uint32_t q = 0; q < P; ++q) {
+        const uint32_t gq = __shfl(q < 64u ? grp[0] : grp[1], (int)(q & 63u), 64);
+#pragma unroll
+        for (int h = 0; h < 2; ++h) start[h] += gq < grp[h] ? 1u : 0u;
+    }
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const uint32_t p = lane + 64u * h;
+        if (p < P) {
+            const uint32_t pos = start[h] + before[h];
+            pair_token[pos] = p / K;
+            pair_weight[pos] = w[h];
+            tok_pair[p] = pos;
+            if (first[h] == p) { uid[grp[h]] = e[h]; expert_start[grp[h]] = start[h]; }
+        }
+    }
+    if (lane == 0u) { expert_start[U] = P; n_unique[0] = U; }
+}
+
+hipError_t launch_select_group(const float *logits, uint32_t ntok, uint32_t n_expert, uint32_t top_k, uint32_t *ids, float *weights,
+                               float *scalar, uint32_t *uid, uint32_t *expert_start, uint32_t *pair_token, float *pair_weight,
+                               uint32_t *tok_pair, uint32_t *n_unique, hipStream_t s) {
+    if (!ntok || ntok > 16u || ntok * top_k > 128u || !n_expert || n_expert > 1024u || !top_k || top_k > 16u || top_k > n_expert) return hipErrorInvalidValue;
+    REDHIP_LAUNCH(select_group_kernel, dim3(1), dim3(1024), 0, s, logits, ntok, n_expert, top_k, ids, weights, scalar, uid, expert_start,
+                  pair_token, pair_weight, tok_pair, n_unique);
+    return hipGetLastError();
+}
+
+// 32 weights of one group against NTP activation operands, each carrying two tokens (rows 0,1 = hi,lo of the
+// first, rows 2,3 of the second): the table lookups are done once, the MFMAs once per token pair. The lookups are
+// a separate step so that a caller can have those of several groups in flight before it consumes the first.
+__device__ __forceinline__ void group_lookup(uint2 q, const uint8_t *lds, uint4 *m) {
+#pragma unroll
+    for (uint32_t l = 0; l < 4u; ++l) m[l] = *reinterpret_cast<const uint4 *>(lds + (((q.x >> (8u * l)) & 255u) << 4));
+}
+template <int NTP>
+__device__ __forceinline__ void group_consume(uint2 q, const uint4 *m, const half4_t (*ax)[8], float *va, float *vb) {
+    float4_t acc[NTP];
+#pragma unroll
+    for (int t = 0; t < NTP; ++t) acc[t] = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (uint32_t l = 0; l < 4u; ++l) {
+        WeightQuad b0, b1;
+        place_signs(m[l], (q.y >> (7u * l)) & 127u, b0, b1);
+#pragma unroll
+        for (int t = 0; t < NTP; ++t) {
+            acc[t] = __builtin_amdgcn_mfma_f32_4x4x4f16(ax[t][2u * l], b0.h, acc[t], 0, 0, 0);
+            acc[t] = __builtin_amdgcn_mfma_f32_4x4x4f16(ax[t][2u * l + 1u], b1.h, acc[t], 0, 0, 0);
+        }
+    }
+    const float sc = (float)(2u * (q.y >> 28) + 1u);
+#pragma unroll
+    for (int t = 0; t < NTP; ++t) {
+        va[t] = (acc[t][0] + acc[t][1] * 4.8828125e-4f) * sc;
+        vb[t] = (acc[t][2] + acc[t][3] * 4.8828125e-4f) * sc;
+    }
+}
+template <int NTP>
+__device__ __forceinline__ void group_dot_multi(uint2 q, const half4_t (*ax)[8], const uint8_t *lds, float *va, float *vb) {
+    uint4 m[4];
+    group_lookup(q, lds, m);
+    group_consume<NTP>(q, m, ax, va, vb);
+}
+
+// activation operand for two tokens: lanes j = 0,1 carry hi,lo of token a; j = 2,3 of token b (32 values at `off`)
+__device__ __forceinline__ void load_act_operand2(half4_t *ax, const _Float16 *hi, const _Float16 *lo, uint64_t row_a, uint64_t row_b,
+                                                  bool have_b, uint32_t off, uint32_t j) {
+    const _Float16 *src = ((j & 1u) ? lo : hi) + ((j & 2u) ? row_b : row_a) + off;
+    const bool live = j < 2u || have_b;
+#pragma unroll
+    for (int s = 0; s < 8; ++s) {
+        half4_t v = {(_Float16)0, (_Float16)0, (_Float16)0, (_Float16)0};
+        if (live) v = *reinterpret_cast<const half4_t *>(src + 4 * s);
+        ax[s] = v;
+    }
+}
+
+struct BatchArgs {
+    const uint8_t *experts;
+    uint64_t stride;
+    const uint8_t *shared;
+    const uint32_t *uid, *expert_start, *pair_token, *n_unique;     // grouping (device)
+    const float *pair_weight;
+    const uint32_t *tok_pair;
+    const float *scalar;           // [ntok]
+    const _Float16 *xh, *xl;       // [ntok][hidden]
+    const int *xexp;               // [ntok]
+    _Float16 *act_h, *act_l;       // [P + ntok][ffn]: routed pairs, then the shared expert's pairs (token t at P + t)
+    int *act_exp;                  // [P + ntok][ffn / 32]
+    float *out;                    // [ntok][hidden]
+    uint32_t hidden, ffn, top_k, ntok;
+};
+
+// Persistent workgroups walk the units (u, g) = (group of pairs, 32 FFN columns): 32 gate + 32 up rows of the
+// group's expert (u == U: the shared expert, all tokens) for every token that selected it, NTP token pairs per
+// pass. The fp16 halves of all tokens sit in LDS, the routing metadata of the workgroup's units too, and the
+// weights of the next unit are requested while the current one is computed.
+constexpr int kMaxUnits = 16;      // units per workgroup
+constexpr int kMaxTok = 8;         // tokens of a small batch
+
+template <int NKC, int NTP>
+__global__ __launch_bounds__(kWaves * 64) void gateup_batch_kernel(BatchArgs a) {
+    constexpr int NW = kWaves;
+    constexpr int UPW = 16 * NKC / NW;
+    extern __shared__ __attribute__((aligned(16))) uint8_t dyn[];                  // activation planes of all tokens
+    __shared__ __attribute__((aligned(16))) uint8_t lds[kMagBytes];
+    __shared__ float part[2][2 * NTP][NKC * 64];                                   // alternating between passes
+    __shared__ uint32_t meta_expert[kMaxUnits], meta_p0[kMaxUnits], meta_n[kMaxUnits];
+    __shared__ uint8_t meta_tok[kMaxUnits][kMaxTok];
+    __shared__ float tok_scale[kMaxTok];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t H = a.hidden, F = a.ffn, HG = H / 32u, HB = H / 256u, FG = F / 32u, P = a.ntok * a.top_k;
+    const uint64_t grid_entry = tid < 256u ? redhip_iq2xxs_grid[tid] : 0ull;
+    const uint32_t U = a.n_unique[0], n_units = (U + 1u) * FG;
+    uint32_t count = 0u;
+    if (blockIdx.x < n_units) count = (n_units - blockIdx.x + gridDim.x - 1u) / gridDim.x;
+    if (count > (uint32_t)kMaxUnits) count = kMaxUnits;
+    if (count == 0u) return;
+    KTS(0);
+    // x operand in LDS as [piece s of 8 bytes][plane][group], plane = 2 * token + (hi, lo) and one more plane of
+    // zeros for lanes without a token: the 64 lanes of a wave read the same piece of consecutive groups, and the
+    // plane stride of HG + 8 keeps the hi and lo planes on different banks
+    const uint32_t PLS = HG + 8u, ZP = 2u * a.ntok, SS = (ZP + 1u) * PLS;
+    uint2 *xs = reinterpret_cast<uint2 *>(dyn);
+    if (tid < count) {
+        const uint32_t u = (blockIdx.x + tid * gridDim.x) / FG;
+        const bool sh = u == U;
+        meta_expert[tid] = sh ? 0xffffffffu : a.uid[u];
+        const uint32_t p0 = sh ? P : a.expert_start[u], p1 = sh ? P + a.ntok : a.expert_start[u + 1u];
+        meta_p0[tid] = p0;
+        meta_n[tid] = p1 - p0;
+        for (uint32_t i = 0; i < p1 - p0 && i < (uint32_t)kMaxTok; ++i) meta_tok[tid][i] = (uint8_t)(sh ? i : a.pair_token[p0 + i]);
+    }
+    if (tid >= 64u && tid < 64u + a.ntok) tok_scale[tid - 64u] = 0.125f * exp2i(a.xexp[tid - 64u]);
+    for (uint32_t i = tid; i < a.ntok * H / 8u; i += NW * 64u) {
+        const uint32_t t = i / (H / 8u), c = i % (H / 8u), at = (2u * (c & 3u)) * SS + 2u * t * PLS + (c >> 2);
+        const uint4 vh = reinterpret_cast<const uint4 *>(a.xh)[i], vl = reinterpret_cast<const uint4 *>(a.xl)[i];
+        xs[at] = make_uint2(vh.x, vh.y);
+        xs[at + SS] = make_uint2(vh.z, vh.w);
+        xs[at + PLS] = make_uint2(vl.x, vl.y);
+        xs[at + PLS + SS] = make_uint2(vl.z, vl.w);
+    }
+    for (uint32_t i = tid; i < 8u * PLS; i += NW * 64u) xs[(i / PLS) * SS + ZP * PLS + i % PLS] = make_uint2(0u, 0u);
+    build_tables(lds, tid, grid_entry);
+    __syncthreads();
+    KTS(1);
+
+    const uint64_t qs_bytes = (uint64_t)F * HG * 8u, gate_bytes = qs_bytes + (uint64_t)F * HB * 2u;
+    const uint32_t kc = wave % NKC, q0 = wave / NKC;              // wave-uniform: they stay in scalar registers
+    const uint32_t G = 16u * kc + blk;
+    const uint32_t lane_q = (j * HG + blk) * 8u, lane_d = (j * HB + (blk >> 3)) * 2u;
+    uint2 wq[UPW], wq_next[UPW];
+    uint32_t wd[UPW], wd_next[UPW];
+    // uniform row base + one lane offset for all units of the wave
+    auto load_weights = [&](uint32_t k, uint2 *q, uint32_t *d) {
+        const uint32_t g = (blockIdx.x + k * gridDim.x) % FG;
+        const uint32_t e = __builtin_amdgcn_readfirstlane(meta_expert[k]);
+        const uint8_t *ex = e == 0xffffffffu ? a.shared : a.experts + (uint64_t)e * a.stride;
+#pragma unroll
+        for (int un = 0; un < UPW; ++un) {
+            const uint32_t quad = q0 + (NW / NKC) * un;
+            const uint32_t row = 32u * g + 4u * (quad & 7u);
+            const uint8_t *mat = ex + (quad < 8u ? 0u : gate_bytes);
+            q[un] = *reinterpret_cast<const uint2 *>(mat + ((uint64_t)row * HG + 16u * kc) * 8u + lane_q);
+            d[un] = *reinterpret_cast<const uint16_t *>(mat + qs_bytes + ((uint64_t)row * HB + 2u * kc) * 2u + lane_d);
+        }
+    };
+    load_weights(0u, wq, wd);
+    uint32_t pass = 0u;
+    for (uint32_t k = 0; k < count; ++k) {
+        // always issued (the last unit asks for its own weights again): a conditional request would make the
+        // compiler wait for it before the first use of the current weights
+        load_weights(k + 1u < count ? k + 1u : k, wq_next, wd_next);
+        const uint32_t g = (blockIdx.x + k * gridDim.x) % FG, n = meta_n[k], p0 = meta_p0[k];
+        for (uint32_t pp = 0; pp < n; pp += 2u * NTP, ++pass) {
+            float (*pbuf)[NKC * 64] = part[pass & 1u];
+            half4_t ax[NTP][8];
+#pragma unroll
+            for (int t = 0; t < NTP; ++t) {
+                const uint32_t ip = pp + 2u * t + (j >> 1);
+                const uint32_t plane = ip < n ? 2u * meta_tok[k][ip] + (j & 1u) : ZP;
+                const uint2 *src = xs + plane * PLS + G;
+#pragma unroll
+                for (int s = 0; s < 8; ++s) {
+                    union { uint2 u; half4_t h; } v4;
+                    v4.u = src[(uint32_t)s * SS];
+                    ax[t][s] = v4.h;
+                }
+            }
+            float v[2 * NTP][UPW];
+            // one lookup round trip costs far more than its issue slot: the table reads run kAhead groups ahead
+            constexpr int kAhead = UPW < 2 ? UPW : 2;
+            uint4 m[UPW][4];
+            uint2 q[UPW];
+#pragma unroll
+            for (int un = 0; un < UPW; ++un) {
+                q[un] = wq[un];
+                asm volatile("" : "+v"(q[un].x), "+v"(q[un].y));   // table addresses are formed here, not hoisted out of the pass loop
+            }
+#pragma unroll
+            for (int un = 0; un < kAhead; ++un) group_lookup(q[un], lds, m[un]);
+#pragma unroll
+            for (int un = 0; un < UPW; ++un) {
+                if (un + kAhead < UPW) group_lookup(q[un + kAhead], lds, m[un + kAhead]);
+                float va[NTP], vb[NTP];
+                group_consume<NTP>(q[un], m[un], ax, va, vb);
+                const float d = scale_to_f32(wd[un]);
+#pragma unroll
+                for (int t = 0; t < NTP; ++t) { v[2 * t][un] = va[t] * d; v[2 * t + 1][un] = vb[t] * d; }
+            }
+#pragma unroll
+            for (int t = 0; t < 2 * NTP; ++t) {
+                const float tot = quad_column_reduce<UPW>(v[t], lane);
+                if (reduced_writer<UPW>(lane)) pbuf[t][kc * 64u + 4u * (q0 + (NW / NKC) * reduced_unit<UPW>(lane)) + j] = tot;
+            }
+            KTS(2u + 2u * k);
+            // the only barrier of a pass: the next pass writes the other half of `part`, and the one after that
+            // comes behind the next barrier, which the lanes below reach only after they have read this half
+            __syncthreads();
+            KTS(3u + 2u * k);
+            if (tid < 32u * 2u * NTP) {
+                const uint32_t t = tid >> 5, c = tid & 31u, ip = pp + t;
+                if (ip < n) {
+                    float gsum = 0.0f, usum = 0.0f;
+#pragma unroll
+                    for (int kk = 0; kk < NKC; ++kk) { gsum += pbuf[t][kk * 64 + c]; usum += pbuf[t][kk * 64 + 32 + c]; }
+                    const float xs = tok_scale[meta_tok[k][ip]];
+                    gsum *= xs;
+                    usum *= xs;
+                    const float act = (gsum / (1.0f + expf(-gsum))) * usum;
+                    float amax = fabsf(act);
+#pragma unroll
+                    for (int o = 16; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+                    const int e = prescale_exp(amax);
+                    const uint64_t pr = p0 + ip;
+                    split_hi_lo(act, exp2i(-e), a.act_h + pr * F + 32u * g + c, a.act_l + pr * F + 32u * g + c);
+                    if (c == 0u) a.act_exp[pr * FG + g] = e;
+                }
+            }
+        }
+#pragma unroll
+        for (int un = 0; un < UPW; ++un) { wq[un] = wq_next[un]; wd[un] = wd_next[un]; }
+    }
+}
+
+// Workgroup = 8 output rows; wave w walks the groups u = w, w + 16, ... (the last one is the shared expert) and,
+// for each, every pair of tokens that selected it. Per-pair partial rows meet in LDS and each token's sum is taken
+// in its own selection order.
+template <int MAXPAIR>
+__global__ __launch_bounds__(kWaves * 64) void down_batch_kernel(BatchArgs a) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds[kMagBytes];
+    __shared__ float part[MAXPAIR * 8];
+    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
+    const uint32_t H = a.hidden, F = a.ffn, FG = F / 32u, FB = F / 256u, P = a.ntok * a.top_k;
+    const uint64_t grid_entry = tid < 256u ? redhip_iq2xxs_grid[tid] : 0ull;
+    const uint32_t row0 = 8u * blockIdx.x, U = a.n_unique[0];
+    const uint64_t gate_bytes = (uint64_t)F * (H / 32u) * 8u + (uint64_t)F * (H / 256u) * 2u;
+    build_tables(lds, tid, grid_entry);
+    __syncthreads();
+    const uint32_t n_chunk = (FG + 15u) / 16u;
+    for (uint32_t u = wave; u <= U; u += kWaves) {
+        const bool is_shared = u == U;
+        const uint8_t *ex = is_shared ? a.shared : a.experts + (uint64_t)a.uid[u] * a.stride;
+        const uint32_t p0 = is_shared ? P : a.expert_start[u], p1 = is_shared ? P + a.ntok : a.expert_start[u + 1u];
+        const uint2 *qs = reinterpret_cast<const uint2 *>(ex + 2u * gate_bytes);
+        const uint16_t *ds = reinterpret_cast<const uint16_t *>(ex + 2u * gate_bytes + (uint64_t)H * FG * 8u);
+        for (uint32_t pp = p0; pp < p1; pp += 2u) {
+            const bool have_b = pp + 1u < p1;
+            float tot_a[2] = {0.0f, 0.0f}, tot_b[2] = {0.0f, 0.0f};
+            for (uint32_t c = 0; c < n_chunk; ++c) {
+                const uint32_t G = 16u * c + blk;
+                if (G < FG) {
+                    half4_t ax[1][8];
+                    load_act_operand2(ax[0], a.act_h, a.act_l, (uint64_t)pp * F, (uint64_t)(pp + 1u) * F, have_b, 32u * G, j);
+                    const float sa = exp2i(a.act_exp[pp * FG + G]), sb = have_b ? exp2i(a.act_exp[(pp + 1u) * FG + G]) : 0.0f;
+#pragma unroll
+                    for (int q = 0; q < 2; ++q) {
+                        const uint32_t r = row0 + 4u * q + j;
+                        const uint2 w = qs[(uint64_t)r * FG + G];
+                        const float d = scale_to_f32(ds[(uint64_t)r * FB + (G >> 3)]);
+                        float va[1], vb[1];
+                        group_dot_multi<1>(w, ax, lds, va, vb);
+                        tot_a[q] += va[0] * d * sa;
+                        tot_b[q] += vb[0] * d * sb;
+                    }
+                }
+            }
+            const float ra = quad_column_reduce<2>(tot_a, lane), rb = quad_column_reduce<2>(tot_b, lane);
+            if (reduced_writer<2>(lane)) {
+                const uint32_t rr = 4u * reduced_unit<2>(lane) + j;
+                part[pp * 8u + rr] = ra;
+                if (have_b) part[(pp + 1u) * 8u + rr] = rb;
+            }
+        }
+    }
+    __syncthreads();
+    for (uint32_t i = tid; i < a.ntok * 8u; i += kWaves * 64u) {
+        const uint32_t t = i >> 3, r = i & 7u;
+        float sum = 0.0f;
+        for (uint32_t k = 0; k < a.top_k; ++k) {
+            const uint32_t p = a.tok_pair[t * a.top_k + k];
+            sum = fmaf(a.pair_weight[p] * 0.125f, part[p * 8u + r], sum);
+        }
+        sum = fmaf(a.scalar[t] * 0.125f, part[(P + t) * 8u + r], sum);
+        a.out[(uint64_t)t * H + row0 + r] = sum;
+    }
+}
+
+hipError_t launch_batch_packed(const void *experts, uint64_t stride, const void *shared, const uint32_t *uid, const uint32_t *expert_start,
+                               const uint32_t *pair_token, const uint32_t *n_unique, const float *pair_weight, const uint32_t *tok_pair,
+                               const float *scalar, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l, int *act_exp,
+                               float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s) {
+    if (!fused_iq2_supported(hidden, ffn) || !ntok || ntok > (uint32_t)kMaxTok || ntok * top_k + ntok > 144u) return hipErrorInvalidValue;
+    BatchArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(shared), uid, expert_start, pair_token, n_unique,
+                pair_weight, tok_pair, scalar, static_cast<const _Float16 *>(xh), static_cast<const _Float16 *>(xl), xexp,
+                static_cast<_Float16 *>(act_h), static_cast<_Float16 *>(act_l), act_exp, out, hidden, ffn, top_k, ntok};
+    const uint32_t P = ntok * top_k, n_groups = (P < n_expert ? P : n_expert) + 1u;
+    const uint32_t unit_bound = n_groups * (ffn / 32u);
+    const dim3 grid(256u * ((unit_bound + 256u * kMaxUnits - 1u) / (256u * kMaxUnits)));
+    const size_t dyn_lds = (size_t)(2u * ntok + 1u) * (hidden / 32u + 8u) * 64u;   // hi and lo plane per token + a zero plane, 8 pieces of 8 bytes per group
+    prof_set_stage(ST_BATCH_GATEUP);
+#define REDHIP_GUB(NKC)                                                                                                   \
+    do {                                                                                                                  \
+        /* two token pairs per pass keep the kernel inside 128 VGPRs; larger groups take more passes */                  \
+        static bool attr = false;                                                                                          \
+        if (!attr) {                                                                                                       \
+            hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void *>(gateup_batch_kernel<NKC, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024); \
+            hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void *>(gateup_batch_kernel<NKC, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024); \
+            if (e1 != hipSuccess) return e1;                                                                               \
+            if (e2 != hipSuccess) return e2;                                                                               \
+            attr = true;                                                                                                   \
+        }                                                                                                                  \
+        if (ntok <= 8u) REDHIP_LAUNCH((gateup_batch_kernel<NKC, 1>), grid, dim3(kWaves * 64), dyn_lds, s, a);              \
+        else REDHIP_LAUNCH((gateup_batch_kernel<NKC, 2>), grid, dim3(kWaves * 64), dyn_lds, s, a);                         \
+    } while (0)
+    switch (hidden / 512u) {
+        case 1: REDHIP_GUB(1); break;
+        case 2: REDHIP_GUB(2); break;
+        case 4: REDHIP_GUB(4); break;
+        default: return hipErrorInvalidValue;
+    }
+#undef REDHIP_GUB
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    prof_set_stage(ST_BATCH_DOWN);
+    REDHIP_LAUNCH(down_batch_kernel<144>, dim3(hidden / 8u), dim3(kWaves * 64), 0, s, a);
+    return hipGetLastError();
 }
 
 hipError_t launch_gateup_select(const void *experts, uint64_t stride, const void *shared, const float *logits, const uint32_t *ids_in,
@@ -717,3 +1151,12 @@ hipError_t launch_down_combine(const void *experts, uint64_t stride, const void 
 }
 
 }  // namespace redhip
+
+#ifdef REDHIP_KTS
+extern "C" int redhip_debug_kts(unsigned long long *out) {
+    return hipMemcpyFromSymbol(out, HIP_SYMBOL(redhip::g_kts), sizeof(unsigned long long) * 256 * 32) == hipSuccess;
+}
+extern "C" int redhip_debug_kts2(unsigned long long *out) {
+    return hipMemcpyFromSymbol(out, HIP_SYMBOL(redhip::g_kts2), sizeof(unsigned long long) * 256 * 32) == hipSuccess;
+}
+#endif

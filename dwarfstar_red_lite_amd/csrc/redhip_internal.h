@@ -112,6 +112,17 @@ hipError_t launch_select(const float *logits, uint32_t ntok, uint32_t n_expert, 
 // fp16 split of x and the scalar gate without a router
 hipError_t launch_prep(const float *x, const float *gate_inp, uint32_t ntok, uint32_t hidden, void *xh, void *xl, int *xexp, float *scalar, hipStream_t s);
 
+// 2..16 tokens (at most 128 pairs): per-token selection and the pair sort in one launch
+hipError_t launch_select_group(const float *logits, uint32_t ntok, uint32_t n_expert, uint32_t top_k, uint32_t *ids, float *weights,
+                               float *scalar, uint32_t *uid, uint32_t *expert_start, uint32_t *pair_token, float *pair_weight,
+                               uint32_t *tok_pair, uint32_t *n_unique, hipStream_t s);
+// batched gate/up + down/combine over grouped pairs, packed IQ2_XXS, small batches (ntok * (top_k + 1) <= 144).
+// act buffers hold ntok * (top_k + 1) rows (routed pairs, then one row per token for the shared expert).
+hipError_t launch_batch_packed(const void *experts, uint64_t stride, const void *shared, const uint32_t *uid, const uint32_t *expert_start,
+                               const uint32_t *pair_token, const uint32_t *n_unique, const float *pair_weight, const uint32_t *tok_pair,
+                               const float *scalar, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l, int *act_exp,
+                               float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s);
+
 // single token: act[slot] = SwiGLU(gate . x, up . x) as fp16 halves with one exponent per 32 values. With `logits` the
 // kernel selects the experts itself (and writes ids / weights / scalar); with logits == nullptr it takes ids_in.
 hipError_t launch_gateup_select(const void *experts, uint64_t stride, const void *shared, const float *logits, const uint32_t *ids_in,

@@ -52,6 +52,7 @@ struct Moe {
     bool fused = false;
     void *xh = nullptr, *xl = nullptr;       // fp16 [hidden] each
     int *xexp = nullptr;
+    bool select_and_group = false;           // forward() of a small batch: one launch selects and sorts the pairs
     bool skip_select = false;                // forward(): the gate/up kernel selects, route() skips its own selection
     // batched path (ntok > 1): pairs grouped by expert
     uint32_t *uid = nullptr, *expert_start = nullptr, *pair_token = nullptr, *tok_pair = nullptr, *n_unique = nullptr;
@@ -59,6 +60,10 @@ struct Moe {
     void *act_h = nullptr, *act_l = nullptr; // fp16 [top_k + 1][ffn] each
     int *act_exp = nullptr;                  // [top_k + 1][ffn / 32]
 
+    // batches the packed MFMA kernels take: 2..16 tokens, at most 128 pairs
+    bool small_batch(uint32_t ntok) const {
+        return fused && ntok >= 2u && ntok <= 8u && ntok * cfg.top_k <= 128u && ntok * (cfg.top_k + 1u) <= 144u && cfg.hidden / 512u <= 4u;
+    }
     ExpertSet routed(uint32_t l) const { return ExpertSet{layers[l].experts, expert_stride, gate_bytes, gate_bytes, gu_type, dn_type}; }
     ExpertSet shared(uint32_t l) const { return ExpertSet{layers[l].shared, 0, sh_gate_bytes, sh_gate_bytes, sh_gu_type, sh_dn_type}; }
 };
@@ -85,15 +90,26 @@ __global__ __launch_bounds__(256) void scalar_gate_kernel(const float *gate_inp,
 }
 
 // select_here: the gate/up kernel selects the experts from m->logits itself (ids / weights are then outputs)
+// grouped: the pair sort of (ids, weights) is already in the workspace
 int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const uint32_t *ids, const float *weights,
-                    float *out, hipStream_t s, bool select_here = false) {
+                    float *out, hipStream_t s, bool select_here = false, bool grouped = false) {
     const redhip_moe_config &c = m->cfg;
     if (ntok > 1u) {       // group the (token, expert) pairs by expert, run each distinct expert once over its tokens
         const uint32_t P = ntok * c.top_k, n_groups = P < c.n_expert ? P : c.n_expert;
         const ExpertSet ex = m->routed(layer), sh = m->shared(layer);
-        prof_set_stage(ST_GROUP);
-        HIP_OK(launch_group_pairs(ids, weights, ntok, c.top_k, c.n_expert, m->uid, m->expert_start, m->pair_token, m->pair_weight,
-                                  m->tok_pair, m->n_unique, s), "grouping launch");
+        if (!grouped) {
+            prof_set_stage(ST_GROUP);
+            HIP_OK(launch_group_pairs(ids, weights, ntok, c.top_k, c.n_expert, m->uid, m->expert_start, m->pair_token, m->pair_weight,
+                                      m->tok_pair, m->n_unique, s), "grouping launch");
+        }
+        if (m->small_batch(ntok)) {     // packed IQ2_XXS, MFMA kernels; xh / xl / xexp / scalar come from the router or prep kernel
+            const Layer &L = m->layers[layer];
+            HIP_OK(launch_batch_packed(L.packed, m->expert_stride, L.shared_packed, m->uid, m->expert_start, m->pair_token, m->n_unique,
+                                       m->pair_weight, m->tok_pair, m->scalar, m->xh, m->xl, m->xexp, m->act_h, m->act_l, m->act_exp, out,
+                                       c.hidden, c.ffn, c.top_k, ntok, c.n_expert, s), "batched packed launch");
+            prof_set_stage(ST_OTHER);
+            return 1;
+        }
         prof_set_stage(ST_BATCH_GATEUP);
         HIP_OK(launch_batch_gateup(ex, m->uid, m->expert_start, m->pair_token, m->n_unique, n_groups, P, c.hidden, c.ffn, x, m->act, s), "batched gate/up launch");
         HIP_OK(launch_batch_gateup(sh, nullptr, nullptr, nullptr, nullptr, 1u, ntok, c.hidden, c.ffn, x, m->sh_act, s), "batched shared gate/up launch");
@@ -185,8 +201,8 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
     const size_t T = c.max_tokens;
     const size_t ws_bytes = align256(T * (c.n_expert + 1u) * 4u) + 2u * align256(T * c.top_k * 4u) + align256(T * 4u) +
                             align256(T * c.top_k * c.ffn * 4u) + align256(T * c.ffn * 4u) +
-                            2u * align256(2u * T * c.hidden) + align256(4u * T) + 2u * align256(2u * (c.top_k + 1u) * c.ffn) +
-                            align256(4u * (c.top_k + 1u) * (c.ffn / 32u)) +
+                            2u * align256(2u * T * c.hidden) + align256(4u * T) + 2u * align256(2u * T * (c.top_k + 1u) * c.ffn) +
+                            align256(4u * T * (c.top_k + 1u) * (c.ffn / 32u)) +
                             (T > 1u ? 6u * align256(4u * (T * c.top_k + 2u)) + align256(4u * T * c.top_k * c.hidden) + align256(4u * T * c.hidden) : 0u);
     ok = ok && hipMalloc(reinterpret_cast<void **>(&m->ws), ws_bytes) == hipSuccess;
     if (!ok) {
@@ -204,9 +220,9 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
     m->xh = w; w += align256(2u * T * c.hidden);
     m->xl = w; w += align256(2u * T * c.hidden);
     m->xexp = reinterpret_cast<int *>(w); w += align256(4u * T);
-    m->act_h = w; w += align256(2u * (c.top_k + 1u) * c.ffn);
-    m->act_l = w; w += align256(2u * (c.top_k + 1u) * c.ffn);
-    m->act_exp = reinterpret_cast<int *>(w); w += align256(4u * (c.top_k + 1u) * (c.ffn / 32u));
+    m->act_h = w; w += align256(2u * T * (c.top_k + 1u) * c.ffn);
+    m->act_l = w; w += align256(2u * T * (c.top_k + 1u) * c.ffn);
+    m->act_exp = reinterpret_cast<int *>(w); w += align256(4u * T * (c.top_k + 1u) * (c.ffn / 32u));
     if (T > 1u) {
         const size_t pw = align256(4u * (T * c.top_k + 2u));
         m->uid = reinterpret_cast<uint32_t *>(w); w += pw;
@@ -311,7 +327,11 @@ int redhip_moe_route(redhip_moe_t h, uint32_t layer, const float *x_dev, uint32_
         prof_set_stage(ST_ROUTER_GEMV);
         HIP_OK(launch_router_gemv(c.router_type, m->layers[layer].router, x_dev, m->layers[layer].gate_inp, ntok, c.hidden, c.n_expert,
                                   m->logits, m->xh, m->xl, m->xexp, s), "router launch");
-        if (!m->skip_select) {
+        if (m->select_and_group) {
+            prof_set_stage(ST_ROUTE_SELECT);
+            HIP_OK(launch_select_group(m->logits, ntok, c.n_expert, c.top_k, m->ids, m->weights, m->scalar, m->uid, m->expert_start,
+                                       m->pair_token, m->pair_weight, m->tok_pair, m->n_unique, s), "selection + grouping launch");
+        } else if (!m->skip_select) {
             prof_set_stage(ST_ROUTE_SELECT);
             HIP_OK(launch_select(m->logits, ntok, c.n_expert, c.top_k, ids_dev ? ids_dev : m->ids, weights_dev ? weights_dev : m->weights,
                                  m->scalar, nullptr, s), "selection launch");
@@ -338,7 +358,7 @@ int redhip_moe_experts(redhip_moe_t h, uint32_t layer, const float *x_dev, uint3
     if (!check_layer(m, layer)) return 0;
     if (!x_dev || !ids_dev || !weights_dev || !out_dev || !ntok || ntok > m->cfg.max_tokens) { moe_err("invalid expert execution arguments"); return 0; }
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (m->fused && ntok == 1u) {
+    if (m->fused && (ntok == 1u || m->small_batch(ntok))) {
         prof_set_stage(ST_OTHER);
         HIP_OK(launch_prep(x_dev, m->layers[layer].gate_inp, ntok, m->cfg.hidden, m->xh, m->xl, m->xexp, m->scalar, s), "prep launch");
         return experts_enqueue(m, layer, x_dev, ntok, ids_dev, weights_dev, out_dev, s);
@@ -354,11 +374,14 @@ int redhip_moe_forward(redhip_moe_t h, uint32_t layer, const float *x_dev, uint3
     if (!x_dev || !out_dev) { moe_err("null activation pointer"); return 0; }
     static const bool sep_sel = getenv("REDHIP_SEPSEL") != nullptr;   // experiment: selection as its own launch
     const bool select_in_gateup = m->fused && ntok == 1u && !sep_sel;
+    const bool group_in_select = m->small_batch(ntok);
     m->skip_select = select_in_gateup;
+    m->select_and_group = group_in_select;
     const int routed = redhip_moe_route(h, layer, x_dev, ntok, nullptr, nullptr, nullptr, stream);
     m->skip_select = false;
+    m->select_and_group = false;
     if (!routed) return 0;
-    return experts_enqueue(m, layer, x_dev, ntok, m->ids, m->weights, out_dev, static_cast<hipStream_t>(stream), select_in_gateup);
+    return experts_enqueue(m, layer, x_dev, ntok, m->ids, m->weights, out_dev, static_cast<hipStream_t>(stream), select_in_gateup, group_in_select);
 }
 
 int redhip_moe_last_route(redhip_moe_t h, uint32_t ntok, uint32_t *ids, float *weights, float *logits, void *stream) {
