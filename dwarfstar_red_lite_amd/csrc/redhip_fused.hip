@@ -245,12 +245,13 @@ struct SelectOut {
     float tmp_p[64];
 };
 
-#define SEL_TS(i) do {} while (0)
 #ifdef REDHIP_KTS
 __device__ unsigned long long g_kts[256 * 32], g_kts2[256 * 32];
 #define KTS(i) do { if (threadIdx.x == 0u && blockIdx.x < 256u && (i) < 32u) { g_kts[blockIdx.x * 32u + (i)] = wall_clock64(); g_kts2[blockIdx.x * 32u + (i)] = clock64(); } } while (0)
+#define SEL_TS(i) KTS(16u + (i))
 #else
 #define KTS(i) do {} while (0)
+#define SEL_TS(i) do {} while (0)
 #endif
 
 template <int PER>
@@ -588,6 +589,7 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_select_kernel(GateUpArgs a
     // activation operand: independent of the routing, requested before the selection
     const uint32_t kc = wave % NKC, q0 = wave / NKC;
     const uint32_t G = 16u * kc + blk;                 // this lane's group inside the gate/up rows
+    KTS(0);
     half4_t ax[8];
     load_act_operand(ax, a.xh + 32u * G, a.xl + 32u * G, j);
     build_tables(lds, tid, grid_entry);
@@ -608,6 +610,7 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_select_kernel(GateUpArgs a
         if (!is_shared) expert = a.ids_in[slot];
         __syncthreads();                               // tables
     }
+    KTS(1);
     const uint8_t *ex = is_shared ? a.shared : a.experts + (uint64_t)expert * a.stride;
     const uint64_t gate_bytes = (uint64_t)F * HG * 8u + (uint64_t)F * HB * 2u;
     const uint2 *gate_qs = reinterpret_cast<const uint2 *>(ex);
@@ -634,7 +637,9 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_select_kernel(GateUpArgs a
         const uint32_t quad = q0 + (NW / NKC) * reduced_unit<UPW>(lane);
         part[kc * 64u + 4u * quad + j] = tot;
     }
+    KTS(2);
     __syncthreads();
+    KTS(3);
     if (tid < 32u) {
         float gsum = 0.0f, usum = 0.0f;
 #pragma unroll
