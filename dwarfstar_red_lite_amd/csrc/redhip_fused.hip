@@ -83,20 +83,58 @@ hipError_t launch_dequant_packed_iq2xxs(const void *packed, uint32_t nrows, uint
 
 // ---------------------------------------------------------------- router GEMV + tail
 
-__device__ __forceinline__ float wave_sum(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-    return v;
+// Wave-wide reductions without LDS traffic: quad permutes and row rotations (DPP) inside rows of 16 lanes, then
+// swaps of odd/even rows and of the two halves of the wave. Every lane ends with the result.
+template <int CTRL> __device__ __forceinline__ float dpp_f32(float v) {
+    return __uint_as_float(__builtin_amdgcn_update_dpp(0u, __float_as_uint(v), CTRL, 0xf, 0xf, false));
 }
-__device__ __forceinline__ double wave_sum_d(double v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, 64);
-    return v;
+template <int CTRL> __device__ __forceinline__ double dpp_f64(double v) {
+    const uint64_t b = __builtin_bit_cast(uint64_t, v);
+    const uint32_t lo = __builtin_amdgcn_update_dpp(0u, (uint32_t)b, CTRL, 0xf, 0xf, false);
+    const uint32_t hi = __builtin_amdgcn_update_dpp(0u, (uint32_t)(b >> 32), CTRL, 0xf, 0xf, false);
+    return __builtin_bit_cast(double, (uint64_t)lo | ((uint64_t)hi << 32));
+}
+constexpr int kDppXor1 = 0xB1, kDppXor2 = 0x4E, kDppRor4 = 0x124, kDppRor8 = 0x128;   // quad_perm [1,0,3,2], [2,3,0,1]; row_ror
+__device__ __forceinline__ float wave_sum(float v) {
+    v += dpp_f32<kDppXor1>(v);
+    v += dpp_f32<kDppXor2>(v);
+    v += dpp_f32<kDppRor4>(v);
+    v += dpp_f32<kDppRor8>(v);
+    auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = __uint_as_float(r[0]) + __uint_as_float(r[1]);
+    r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return __uint_as_float(r[0]) + __uint_as_float(r[1]);
 }
 __device__ __forceinline__ float wave_max(float v) {
-#pragma unroll
-    for (int o = 32; o > 0; o >>= 1) v = fmaxf(v, __shfl_xor(v, o, 64));
-    return v;
+    v = fmaxf(v, dpp_f32<kDppXor1>(v));
+    v = fmaxf(v, dpp_f32<kDppXor2>(v));
+    v = fmaxf(v, dpp_f32<kDppRor4>(v));
+    v = fmaxf(v, dpp_f32<kDppRor8>(v));
+    auto r = __builtin_amdgcn_permlane16_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    v = fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+    r = __builtin_amdgcn_permlane32_swap(__float_as_uint(v), __float_as_uint(v), false, false);
+    return fmaxf(__uint_as_float(r[0]), __uint_as_float(r[1]));
+}
+__device__ __forceinline__ double swap_halves_add(double v, bool rows) {
+    const uint64_t b = __builtin_bit_cast(uint64_t, v);
+    const uint32_t lo = (uint32_t)b, hi = (uint32_t)(b >> 32);
+    uint64_t x, y;
+    if (rows) {
+        const auto a = __builtin_amdgcn_permlane16_swap(lo, lo, false, false), c = __builtin_amdgcn_permlane16_swap(hi, hi, false, false);
+        x = (uint64_t)a[0] | ((uint64_t)c[0] << 32); y = (uint64_t)a[1] | ((uint64_t)c[1] << 32);
+    } else {
+        const auto a = __builtin_amdgcn_permlane32_swap(lo, lo, false, false), c = __builtin_amdgcn_permlane32_swap(hi, hi, false, false);
+        x = (uint64_t)a[0] | ((uint64_t)c[0] << 32); y = (uint64_t)a[1] | ((uint64_t)c[1] << 32);
+    }
+    return __builtin_bit_cast(double, x) + __builtin_bit_cast(double, y);
+}
+__device__ __forceinline__ double wave_sum_d(double v) {
+    v += dpp_f64<kDppXor1>(v);
+    v += dpp_f64<kDppXor2>(v);
+    v += dpp_f64<kDppRor4>(v);
+    v += dpp_f64<kDppRor8>(v);
+    v = swap_halves_add(v, true);
+    return swap_halves_add(v, false);
 }
 // LDS written by some lanes of a wave becomes readable by its other lanes (one wave, no workgroup barrier)
 __device__ __forceinline__ void wave_lds_sync() {
@@ -243,19 +281,28 @@ struct SelectOut {
     float scalar;
     uint32_t tmp[64];
     float tmp_p[64];
+    uint64_t cand[64];        // candidates: key << 32 | ~index
 };
 
 #ifdef REDHIP_KTS
 __device__ unsigned long long g_kts[256 * 32], g_kts2[256 * 32];
 #define KTS(i) do { if (threadIdx.x == 0u && blockIdx.x < 256u && (i) < 32u) { g_kts[blockIdx.x * 32u + (i)] = wall_clock64(); g_kts2[blockIdx.x * 32u + (i)] = clock64(); } } while (0)
-#define SEL_TS(i) KTS(16u + (i))
+#define SEL_TS(i) do {} while (0)
 #else
 #define KTS(i) do {} while (0)
 #define SEL_TS(i) do {} while (0)
 #endif
 
+// (float)(1.0 / d) for finite d > 0 without the double division: a float reciprocal refined by two double FMAs is
+// good to 2^-45, which rounds to the same float except in about one case in 2^20
+__device__ __forceinline__ float reciprocal_as_float(double d) {
+    const double r0 = (double)__builtin_amdgcn_rcpf((float)d);
+    const double e = __builtin_fma(-d, r0, 1.0);
+    return (float)__builtin_fma(r0, e, r0);
+}
+
 template <int PER>
-__device__ void wave_select_topk(const float *logits, uint32_t E, uint32_t K, SelectOut *out, float *probs = nullptr) {
+__device__ __forceinline__ void wave_select_topk(const float *logits, uint32_t E, uint32_t K, SelectOut *out, float *probs = nullptr) {
     const uint32_t lane = threadIdx.x & 63u;
     SEL_TS(0);
     float l[PER];
@@ -279,7 +326,7 @@ __device__ void wave_select_topk(const float *logits, uint32_t E, uint32_t K, Se
     SEL_TS(2);
     const double denom = wave_sum_d(part);
     const bool bad = !(denom > 0.0) || isinf(denom) || isnan(denom);
-    const float inv = bad ? 0.0f : (float)(1.0 / denom);
+    const float inv = bad ? 0.0f : reciprocal_as_float(denom);
     SEL_TS(3);
     uint32_t key[PER];
 #pragma unroll
@@ -294,11 +341,14 @@ __device__ void wave_select_topk(const float *logits, uint32_t E, uint32_t K, Se
     uint32_t lm = key[0];
 #pragma unroll
     for (int s = 1; s < PER; ++s) lm = lm > key[s] ? lm : key[s];
+    // Only the upper 16 bits of tau are searched (two per step): a smaller tau is still a lower bound, it only lets a
+    // few more candidates through.
     uint32_t tau = 0x80000000u;                          // bit 31 is set in every valid key
 #pragma unroll 1
-    for (int bit = 30; bit >= 0; --bit) {
-        const uint32_t cand = tau | (1u << bit);
-        tau = wave_count(lm >= cand) >= K ? cand : tau;
+    for (int bit = 29; bit >= 15; bit -= 2) {
+        const uint32_t c1 = tau | (1u << bit), c2 = tau | (2u << bit), c3 = tau | (3u << bit);
+        const uint32_t n1 = wave_count(lm >= c1), n2 = wave_count(lm >= c2), n3 = wave_count(lm >= c3);
+        tau = n3 >= K ? c3 : n2 >= K ? c2 : n1 >= K ? c1 : tau;
     }
     SEL_TS(5);
     uint32_t n_c = 0u;
@@ -310,25 +360,32 @@ __device__ void wave_select_topk(const float *logits, uint32_t E, uint32_t K, Se
         // Level 2: candidates to LDS in index order, one per lane, ranked against each other with lane broadcasts:
         // rank = number of candidates that beat this one under (p desc, index asc). rank < K <=> selected, and the
         // rank is the position in selection order.
+        // A candidate is one 64-bit word, key above the complemented index: larger word <=> earlier in selection order.
         uint32_t n = 0u;
 #pragma unroll
         for (int s = 0; s < PER; ++s) {
             const bool take = key[s] >= tau;
             const uint64_t mask = __ballot(take);
             if (take) {
-                const uint32_t pos = n + (uint32_t)__popcll(mask & ((1ull << lane) - 1ull));
-                out->tmp[pos] = lane + 64u * s;
-                out->tmp_p[pos] = p[s];
+                const uint32_t pos = n + __builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u));
+                out->cand[pos] = ((uint64_t)key[s] << 32) | (uint64_t)(~(lane + 64u * s));
             }
             n += (uint32_t)__popcll(mask);
         }
+        if (lane >= n_c) out->cand[lane] = 0ull;                      // beats nobody
         wave_lds_sync();
-        if (lane < n_c) { mine = out->tmp[lane]; kmine = __float_as_uint(out->tmp_p[lane]) | 0x80000000u; }
-        for (uint32_t q = 0; q < n_c; ++q) {
-            const uint32_t o = __shfl(mine, (int)q, 64), ko = __shfl(kmine, (int)q, 64);
-            rank += (ko > kmine || (ko == kmine && o < mine)) ? 1u : 0u;
+        const uint64_t me = out->cand[lane];
+        kmine = (uint32_t)(me >> 32);
+        mine = lane < n_c ? ~(uint32_t)me : 0xffffffffu;
+        // every lane reads the same entry (an LDS broadcast), 16 reads in flight at a time
+        for (uint32_t base = 0; base < n_c; base += 16u) {
+            uint64_t o[16];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) o[i] = out->cand[base + i];
+#pragma unroll
+            for (int i = 0; i < 16; ++i) rank += o[i] > me ? 1u : 0u;
         }
-        if (lane >= n_c) rank = 0xffffffffu;
+        if (lane >= n_c) { rank = 0xffffffffu; kmine = 0u; }
     } else {
         // Heavy ties (more than 64 keys at or above tau): bisection over all keys, ties at the threshold in index order.
         uint32_t T = 0x80000000u;
@@ -363,7 +420,7 @@ __device__ void wave_select_topk(const float *logits, uint32_t E, uint32_t K, Se
         wave_lds_sync();
         if (lane < K) { mine = out->tmp[lane]; kmine = __float_as_uint(out->tmp_p[lane]) | 0x80000000u; }
         for (uint32_t q = 0; q < K; ++q) {
-            const uint32_t o = __shfl(mine, (int)q, 64), ko = __shfl(kmine, (int)q, 64);
+            const uint32_t o = __builtin_amdgcn_readlane(mine, q), ko = __builtin_amdgcn_readlane(kmine, q);
             rank += (ko > kmine || (ko == kmine && o < mine)) ? 1u : 0u;
         }
         if (lane >= K) rank = 0xffffffffu;
@@ -373,7 +430,7 @@ __device__ void wave_select_topk(const float *logits, uint32_t E, uint32_t K, Se
     const float pm = __uint_as_float(kmine & 0x7fffffffu);
     const double sum = wave_sum_d(selected ? (double)pm : 0.0);
     const bool bad2 = bad || !(sum > 0.0) || isinf(sum) || isnan(sum);
-    const float invs = bad2 ? __uint_as_float(0x7fc00000u) : (float)(1.0 / sum);     // NaN weights flag an invalid softmax
+    const float invs = bad2 ? __uint_as_float(0x7fc00000u) : reciprocal_as_float(sum);     // NaN weights flag an invalid softmax
     if (selected) {
         out->ids[rank] = mine < E ? mine : rank;
         out->w[rank] = pm * invs;
@@ -584,7 +641,8 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_select_kernel(GateUpArgs a
     const uint32_t g = blockIdx.x;                     // FFN column group: act values [32 g, 32 g + 32)
     const uint32_t slot = blockIdx.y;
     const bool is_shared = slot >= a.top_k;
-    const uint64_t grid_entry = tid < 256u ? redhip_iq2xxs_grid[tid] : 0ull;
+    const uint32_t tb = tid - 256u;                     // waves 4..7 build the table: wave 0 goes straight to the selection
+    const uint64_t grid_entry = tb < 256u ? redhip_iq2xxs_grid[tb] : 0ull;
 
     // activation operand: independent of the routing, requested before the selection
     const uint32_t kc = wave % NKC, q0 = wave / NKC;
@@ -592,7 +650,7 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_select_kernel(GateUpArgs a
     KTS(0);
     half4_t ax[8];
     load_act_operand(ax, a.xh + 32u * G, a.xl + 32u * G, j);
-    build_tables(lds, tid, grid_entry);
+    build_tables(lds, tb, grid_entry);
 
     uint32_t expert = 0u;
     if (a.logits) {
