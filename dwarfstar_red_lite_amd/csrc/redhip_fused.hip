@@ -784,16 +784,20 @@ __global__ __launch_bounds__(kWaves * 64) void down_combine_kernel(DownArgs a) {
 
 // ---------------------------------------------------------------- small batches (2..16 tokens): select + group, batched gate/up, batched down
 
-// One workgroup: wave t selects the experts of token t, then wave 0 sorts the (token, k) pairs by expert. Same
+// One workgroup: wave t selects the experts of token t, then the (token, k) pairs are grouped by expert. Same
 // outputs as the host pair sort it replaces: groups in first-appearance order, pairs of a group in token order.
-// Pairs sit two per lane (p = lane, lane + 64), so at most 128 pairs (e.g. 8 tokens x top-16, 12 x top-10).
+// A table in LDS holds, per expert, the set of tokens that selected it (a token selects an expert at most once): the
+// position of a pair inside its group and the group's size are bit counts of that set, the order of the groups a
+// bit count over the "first pair of its expert" flags, the group offsets one prefix sum. At most 128 pairs.
 __global__ __launch_bounds__(1024) void select_group_kernel(const float *logits, uint32_t ntok, uint32_t E, uint32_t K,
                                                             uint32_t *ids, float *weights, float *scalar, uint32_t *uid,
                                                             uint32_t *expert_start, uint32_t *pair_token, float *pair_weight,
                                                             uint32_t *tok_pair, uint32_t *n_unique) {
     __shared__ SelectOut sel[16];
-    __shared__ uint32_t group_of_first[128];
-    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63u;
+    __shared__ uint32_t token_set[1024];                 // per expert: bit t = token t selected it; later the group's offset
+    __shared__ uint32_t first_count[2], size_total[2];
+    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
+    if (tid < E) token_set[tid] = 0u;
     if (wave < ntok) {
         const float *l = logits + (uint64_t)wave * (E + 1u);
         if (E <= 512u) wave_select_topk<8>(l, E, K, &sel[wave]); else wave_select_topk<16>(l, E, K, &sel[wave]);
@@ -802,55 +806,38 @@ __global__ __launch_bounds__(1024) void select_group_kernel(const float *logits,
         if (lane == 0u) scalar[wave] = sel[wave].scalar;
     }
     __syncthreads();
-    if (wave != 0u) return;
-    const uint32_t P = ntok * K;
-    uint32_t e[2], first[2], before[2];
-    float w[2];
+    const uint32_t P = ntok * K, pr = tid;               // pair index (waves 0 and 1)
+    const bool live = pr < P;
+    const uint32_t t = live ? pr / K : 0u;
+    const uint32_t e = live ? sel[t].ids[pr % K] : 0u;
+    if (live) atomicOr(&token_set[e], 1u << t);
+    __syncthreads();
+    const uint32_t set = live ? token_set[e] : 0u;
+    const uint32_t n = (uint32_t)__popc(set), before = (uint32_t)__popc(set & ((1u << t) - 1u));
+    const bool first = live && before == 0u;
+    uint32_t scan = first ? n : 0u;                      // inclusive prefix sum of the group sizes in pair order
+    if (wave < 2u) {
 #pragma unroll
-    for (int h = 0; h < 2; ++h) {
-        const uint32_t p = lane + 64u * h;
-        e[h] = p < P ? sel[p / K].ids[p % K] : 0xffffffffu - p;      // padding never matches anything
-        w[h] = p < P ? sel[p / K].w[p % K] : 0.0f;
-        first[h] = p;
-        before[h] = 0u;
-    }
-    for (uint32_t q = 0; q < P; ++q) {                              // q-th pair broadcast to all lanes
-        const uint32_t eq = __shfl(q < 64u ? e[0] : e[1], (int)(q & 63u), 64);
-#pragma unroll
-        for (int h = 0; h < 2; ++h) {
-            const uint32_t p = lane + 64u * h;
-            if (eq == e[h]) { first[h] = first[h] < q ? first[h] : q; before[h] += q < p ? 1u : 0u; }
+        for (int o = 1; o < 64; o <<= 1) {
+            const uint32_t up = __shfl_up(scan, o, 64);
+            if (lane >= (uint32_t)o) scan += up;
         }
+        const uint64_t fm = __ballot(first);
+        if (lane == 63u) { first_count[wave] = (uint32_t)__popcll(fm); size_total[wave] = scan; }
     }
-    // groups are numbered by the order of their first pair
-    uint32_t grp[2];
-    const bool is_first0 = lane < P && first[0] == lane, is_first1 = lane + 64u < P && first[1] == lane + 64u;
-    const uint64_t f0 = __ballot(is_first0), f1 = __ballot(is_first1);
-    const uint32_t U = (uint32_t)__popcll(f0) + (uint32_t)__popcll(f1);
-    if (is_first0) group_of_first[lane] = (uint32_t)__popcll(f0 & ((1ull << lane) - 1ull));
-    if (is_first1) group_of_first[lane + 64u] = (uint32_t)__popcll(f0) + (uint32_t)__popcll(f1 & ((1ull << lane) - 1ull));
-    wave_lds_sync();
-#pragma unroll
-    for (int h = 0; h < 2; ++h) grp[h] = lane + 64u * h < P ? group_of_first[first[h]] : 0xffffffffu;
-    // start of a group = number of pairs in earlier groups
-    uint32_t start[2] = {0u, 0u};
-    for (uint32_t q = 0; q < P; ++q) {
-        const uint32_t gq = __shfl(q < 64u ? grp[0] : grp[1], (int)(q & 63u), 64);
-#pragma unroll
-        for (int h = 0; h < 2; ++h) start[h] += gq < grp[h] ? 1u : 0u;
+    const uint64_t first_mask = __ballot(first);
+    __syncthreads();
+    const uint32_t grp = (wave == 1u ? first_count[0] : 0u) + __builtin_amdgcn_mbcnt_hi((uint32_t)(first_mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)first_mask, 0u));
+    const uint32_t start = (wave == 1u ? size_total[0] : 0u) + scan - (first ? n : 0u);
+    if (first) { token_set[e] = start; uid[grp] = e; expert_start[grp] = start; }
+    if (tid == 0u) { const uint32_t U = first_count[0] + first_count[1]; expert_start[U] = P; n_unique[0] = U; }
+    __syncthreads();
+    if (live) {
+        const uint32_t pos = token_set[e] + before;
+        pair_token[pos] = t;
+        pair_weight[pos] = sel[t].w[pr % K];
+        tok_pair[pr] = pos;
     }
-#pragma unroll
-    for (int h = 0; h < 2; ++h) {
-        const uint32_t p = lane + 64u * h;
-        if (p < P) {
-            const uint32_t pos = start[h] + before[h];
-            pair_token[pos] = p / K;
-            pair_weight[pos] = w[h];
-            tok_pair[p] = pos;
-            if (first[h] == p) { uid[grp[h]] = e[h]; expert_start[grp[h]] = start[h]; }
-        }
-    }
-    if (lane == 0u) { expert_start[U] = P; n_unique[0] = U; }
 }
 
 hipError_t launch_select_group(const float *logits, uint32_t ntok, uint32_t n_expert, uint32_t top_k, uint32_t *ids, float *weights,
@@ -1080,53 +1067,97 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_batch_kernel(BatchArgs a) 
     }
 }
 
-// Workgroup = 8 output rows; wave w walks the groups u = w, w + 16, ... (the last one is the shared expert) and,
-// for each, every pair of tokens that selected it. Per-pair partial rows meet in LDS and each token's sum is taken
-// in its own selection order.
-template <int MAXPAIR>
+// Workgroup = 8 output rows; wave w owns the groups u = w, w + 16, ... (the last one is the shared expert) and,
+// for each, every pair of tokens that selected it. All weights of the wave's groups are requested at once, right at
+// the start, and the activations of a group while the one before it is computed, so the memory round trips overlap
+// instead of adding up. Per-pair partial rows meet in LDS and each token's sum is taken in its own selection order.
+template <int MAXPAIR, int NCH, int GPW>     // GPW: groups of a wave whose weights are in registers at once
 __global__ __launch_bounds__(kWaves * 64) void down_batch_kernel(BatchArgs a) {
     __shared__ __attribute__((aligned(16))) uint8_t lds[kMagBytes];
     __shared__ float part[MAXPAIR * 8];
-    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t H = a.hidden, F = a.ffn, FG = F / 32u, FB = F / 256u, P = a.ntok * a.top_k;
     const uint64_t grid_entry = tid < 256u ? redhip_iq2xxs_grid[tid] : 0ull;
-    const uint32_t row0 = 8u * blockIdx.x, U = a.n_unique[0];
-    const uint64_t gate_bytes = (uint64_t)F * (H / 32u) * 8u + (uint64_t)F * (H / 256u) * 2u;
+    const uint32_t row0 = 8u * blockIdx.x, U = __builtin_amdgcn_readfirstlane(a.n_unique[0]);
+    const uint64_t down_off = 2u * ((uint64_t)F * (H / 32u) * 8u + (uint64_t)F * (H / 256u) * 2u), qs_bytes = (uint64_t)H * FG * 8u;
+
+    uint2 wq[GPW][NCH][2];
+    uint32_t wd[GPW][NCH], gp0[GPW], gp1[GPW];      // wd: the two rows' block scales, 16 bits each
+    // metadata and weights of groups first, first + 16, ...; indices are clamped so that every request is valid
+    auto request = [&](uint32_t first) {
+#pragma unroll
+        for (int i = 0; i < GPW; ++i) {
+            const uint32_t u = first + 16u * (uint32_t)i, uc = u < U ? u : U;
+            const bool sh = uc == U;
+            // wave-uniform values: kept in scalar registers
+            const uint32_t e = __builtin_amdgcn_readfirstlane(a.uid[sh ? 0u : uc]), es0 = __builtin_amdgcn_readfirstlane(a.expert_start[uc]),
+                           es1 = __builtin_amdgcn_readfirstlane(a.expert_start[sh ? U : uc + 1u]);
+            gp0[i] = sh ? P : es0;
+            gp1[i] = u > U ? gp0[i] : sh ? P + a.ntok : es1;
+            const uint8_t *dn = (sh ? a.shared : a.experts + (uint64_t)e * a.stride) + down_off;
+#pragma unroll
+            for (int c = 0; c < NCH; ++c) {
+                const uint32_t G = 16u * (uint32_t)c + blk, Gc = G < FG ? G : FG - 1u;
+                uint32_t d2 = 0u;
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {
+                    const uint32_t r = row0 + 4u * (uint32_t)q + j;
+                    wq[i][c][q] = reinterpret_cast<const uint2 *>(dn)[(uint64_t)r * FG + Gc];
+                    d2 |= (uint32_t)reinterpret_cast<const uint16_t *>(dn + qs_bytes)[(uint64_t)r * FB + (Gc >> 3)] << (16 * q);
+                }
+                wd[i][c] = d2;
+            }
+        }
+    };
+    struct Pass { half4_t ax[NCH][8]; float sa[NCH], sb[NCH]; };
+    // activations of pairs pp (and pp + 1 if it belongs to the group); pp is clamped into the buffer
+    auto load_pass = [&](uint32_t pp, uint32_t p1, Pass &ps) {
+        const uint32_t last = P + a.ntok - 1u, pa = pp < last ? pp : last, pb = pa + 1u < p1 ? pa + 1u : pa;
+        const bool have_b = pp + 1u < p1;
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            const uint32_t G = 16u * (uint32_t)c + blk, Gc = G < FG ? G : FG - 1u;
+            load_act_operand2(ps.ax[c], a.act_h, a.act_l, (uint64_t)pa * F, (uint64_t)pb * F, true, 32u * Gc, j);
+            const float live = G < FG ? 1.0f : 0.0f;
+            ps.sa[c] = live * exp2i(a.act_exp[pa * FG + Gc]);
+            ps.sb[c] = have_b ? live * exp2i(a.act_exp[pb * FG + Gc]) : 0.0f;
+        }
+    };
+    request(wave);
     build_tables(lds, tid, grid_entry);
     __syncthreads();
-    const uint32_t n_chunk = (FG + 15u) / 16u;
-    for (uint32_t u = wave; u <= U; u += kWaves) {
-        const bool is_shared = u == U;
-        const uint8_t *ex = is_shared ? a.shared : a.experts + (uint64_t)a.uid[u] * a.stride;
-        const uint32_t p0 = is_shared ? P : a.expert_start[u], p1 = is_shared ? P + a.ntok : a.expert_start[u + 1u];
-        const uint2 *qs = reinterpret_cast<const uint2 *>(ex + 2u * gate_bytes);
-        const uint16_t *ds = reinterpret_cast<const uint16_t *>(ex + 2u * gate_bytes + (uint64_t)H * FG * 8u);
-        for (uint32_t pp = p0; pp < p1; pp += 2u) {
-            const bool have_b = pp + 1u < p1;
-            float tot_a[2] = {0.0f, 0.0f}, tot_b[2] = {0.0f, 0.0f};
-            for (uint32_t c = 0; c < n_chunk; ++c) {
-                const uint32_t G = 16u * c + blk;
-                if (G < FG) {
-                    half4_t ax[1][8];
-                    load_act_operand2(ax[0], a.act_h, a.act_l, (uint64_t)pp * F, (uint64_t)(pp + 1u) * F, have_b, 32u * G, j);
-                    const float sa = exp2i(a.act_exp[pp * FG + G]), sb = have_b ? exp2i(a.act_exp[(pp + 1u) * FG + G]) : 0.0f;
+
+    for (uint32_t first = wave; first <= U; first += 16u * GPW) {
+        if (first != wave) request(first);
+        Pass buf[2];                                     // activations of the current and of the next group
+        load_pass(gp0[0], gp1[0], buf[0]);
+#pragma unroll
+        for (int i = 0; i < GPW; ++i) {
+            Pass &cur = buf[NCH == 1 ? i & 1 : 0];
+            if (NCH == 1 && i + 1 < GPW) load_pass(gp0[i + 1 < GPW ? i + 1 : i], gp1[i + 1 < GPW ? i + 1 : i], buf[(i + 1) & 1]);
+            if (NCH != 1 && i > 0) load_pass(gp0[i], gp1[i], cur);
+            for (uint32_t pp = gp0[i]; pp < gp1[i]; pp += 2u) {
+                if (pp != gp0[i]) load_pass(pp, gp1[i], cur);            // further passes of a large group
+                const bool have_b = pp + 1u < gp1[i];
+                float tot_a[2] = {0.0f, 0.0f}, tot_b[2] = {0.0f, 0.0f};
+#pragma unroll
+                for (int c = 0; c < NCH; ++c) {
 #pragma unroll
                     for (int q = 0; q < 2; ++q) {
-                        const uint32_t r = row0 + 4u * q + j;
-                        const uint2 w = qs[(uint64_t)r * FG + G];
-                        const float d = scale_to_f32(ds[(uint64_t)r * FB + (G >> 3)]);
+                        const float d = scale_to_f32(wd[i][c] >> (16 * q));
                         float va[1], vb[1];
-                        group_dot_multi<1>(w, ax, lds, va, vb);
-                        tot_a[q] += va[0] * d * sa;
-                        tot_b[q] += vb[0] * d * sb;
+                        group_dot_multi<1>(wq[i][c][q], reinterpret_cast<const half4_t (*)[8]>(cur.ax[c]), lds, va, vb);
+                        tot_a[q] += va[0] * d * cur.sa[c];
+                        tot_b[q] += vb[0] * d * cur.sb[c];
                     }
                 }
-            }
-            const float ra = quad_column_reduce<2>(tot_a, lane), rb = quad_column_reduce<2>(tot_b, lane);
-            if (reduced_writer<2>(lane)) {
-                const uint32_t rr = 4u * reduced_unit<2>(lane) + j;
-                part[pp * 8u + rr] = ra;
-                if (have_b) part[(pp + 1u) * 8u + rr] = rb;
+                const float ra = quad_column_reduce<2>(tot_a, lane), rb = quad_column_reduce<2>(tot_b, lane);
+                if (reduced_writer<2>(lane)) {
+                    const uint32_t rr = 4u * reduced_unit<2>(lane) + j;
+                    part[pp * 8u + rr] = ra;
+                    if (have_b) part[(pp + 1u) * 8u + rr] = rb;
+                }
             }
         }
     }
@@ -1180,7 +1211,13 @@ hipError_t launch_batch_packed(const void *experts, uint64_t stride, const void 
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     prof_set_stage(ST_BATCH_DOWN);
-    REDHIP_LAUNCH(down_batch_kernel<144>, dim3(hidden / 8u), dim3(kWaves * 64), 0, s, a);
+    const uint32_t groups_per_wave = (n_groups + kWaves - 1u) / kWaves;     // bound known on the host: min(pairs, experts) + 1 groups
+    const dim3 dgrid(hidden / 8u), dblock(kWaves * 64);
+    if (ffn > 512u) REDHIP_LAUNCH((down_batch_kernel<144, 2, 2>), dgrid, dblock, 0, s, a);
+    else if (groups_per_wave <= 2u) REDHIP_LAUNCH((down_batch_kernel<144, 1, 2>), dgrid, dblock, 0, s, a);
+    else if (groups_per_wave <= 3u) REDHIP_LAUNCH((down_batch_kernel<144, 1, 3>), dgrid, dblock, 0, s, a);
+    else if (groups_per_wave <= 4u) REDHIP_LAUNCH((down_batch_kernel<144, 1, 4>), dgrid, dblock, 0, s, a);
+    else REDHIP_LAUNCH((down_batch_kernel<144, 1, 6>), dgrid, dblock, 0, s, a);
     return hipGetLastError();
 }
 
