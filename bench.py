@@ -144,7 +144,30 @@ def main():
         stream.synchronize()
         torch.cuda.synchronize()
         t1 = time.perf_counter()
-        ms_per_step = (t1 - t0) * 1e3 / K
+        eager_ms_per_step = (t1 - t0) * 1e3 / K
+    ms_per_step, launch_mode = eager_ms_per_step, "eager"
+    if not args.no_graph:
+        # the same K steps recorded once into a HIP graph (kernel launches only, no memset nodes) and replayed: this
+        # is how a decode loop would issue them; the replay is checked against the eager outputs before it is timed
+        eager_out = outs.clone()
+        graph = torch.cuda.CUDAGraph()
+        with torch.cuda.graph(graph, stream=stream):
+            for i in range(K):
+                step(W + i)
+        for _ in range(2):                      # untimed replays (the first one uploads the graph)
+            graph.replay()
+            torch.cuda.synchronize()
+            if not torch.equal(outs, eager_out):
+                print("GRAPH REPLAY MISMATCH: falling back to eager timing", file=sys.stderr)
+                break
+        else:
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            graph.replay()
+            torch.cuda.synchronize()
+            t1 = time.perf_counter()
+            ms_per_step, launch_mode = (t1 - t0) * 1e3 / K, "hip_graph"
+    with torch.cuda.stream(stream):
 
         # the same K steps again with per-kernel begin/end timestamps (HIP events on the launch stream)
         n_stage = lib.redhip_profile_stage_count()
@@ -170,12 +193,20 @@ def main():
     dom = max(stages, key=lambda k: stages[k]["ms_total"])
     H, F = cfg["hidden"], cfg["ffn"]
     gate_up = lb["one_expert"] - H * synth.row_bytes(cfg["down_type"], F)
+    sh_gate_up = 2 * F * synth.row_bytes(cfg["sh_gate_up_type"], H)
+    sh_down = H * synth.row_bytes(cfg["sh_down_type"], F)
+    down = lb["one_expert"] - gate_up
+    # weights each kernel has to read once + its activations in and out (f32 x, fp16 hi/lo activations)
     per_launch = {
-        "router_gemv": lb["router_bytes"] / 1 + 4 * H + 4 * cfg["n_expert"],
-        "gateup": mean_distinct * gate_up + 4 * H,
-        "shared_gateup": 2 * F * synth.row_bytes(cfg["sh_gate_up_type"], H) + 4 * H,
-        "down_combine": mean_distinct * (lb["one_expert"] - gate_up) + H * synth.row_bytes(cfg["sh_down_type"], F) + 4 * H,
+        "router_gemv": lb["router_bytes"] + 4 * H + B * (4 * H + 4 * cfg["n_expert"]),
+        # the packed path computes the shared expert's gate/up in the same launch; the generic one has its own stage
+        "gateup": mean_distinct * gate_up + (0 if "shared_gateup" in stages else sh_gate_up) + 4 * H,
+        "shared_gateup": sh_gate_up + 4 * H,
+        "down_combine": mean_distinct * down + sh_down + 4 * H,
         "fused_experts": lb["expert_bytes"] + 2 * 4 * H,
+        "batch_gateup": mean_distinct * gate_up + sh_gate_up + B * 4 * H,
+        "batch_down": mean_distinct * down + sh_down + B * 4 * H,
+        "route_select": B * 4 * (cfg["n_expert"] + 1),
     }
     dom_bytes = per_launch.get(dom)
     dom_us = stages[dom]["us_avg"] * (stages[dom]["launches"] / K)        # per step, if launched more than once per step
@@ -190,7 +221,8 @@ def main():
     total_bytes = lb["expert_bytes"] + lb["router_bytes"] + lb["gate_inp_bytes"] + lb["act_bytes"]
     result = {
         "metric": "moe_ffn_layer_us_per_token", "value": round(us_per_token, 3), "unit": "us/token", "n_gpus": 1,
-        "steps": K, "warmup": W, "ms_per_step": round(ms_per_step, 6), "higher_is_better": False, "scaling": "weak",
+        "steps": K, "warmup": W, "ms_per_step": round(ms_per_step, 6), "launch_mode": launch_mode,
+        "eager_ms_per_step": round(eager_ms_per_step, 6), "higher_is_better": False, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "config1: one MoE FFN layer, B=%d decode token(s), hidden 2048, 512 experts top-10 + shared, ffn 512, layout %s, "
                                "all experts of %d layers resident" % (B, args.layout, NL),

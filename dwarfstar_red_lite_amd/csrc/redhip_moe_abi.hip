@@ -372,8 +372,7 @@ int redhip_moe_forward(redhip_moe_t h, uint32_t layer, const float *x_dev, uint3
     Moe *m = moe_of(h);
     if (!check_layer(m, layer)) return 0;
     if (!x_dev || !out_dev) { moe_err("null activation pointer"); return 0; }
-    static const bool sep_sel = getenv("REDHIP_SEPSEL") != nullptr;   // experiment: selection as its own launch
-    const bool select_in_gateup = m->fused && ntok == 1u && !sep_sel;
+    const bool select_in_gateup = m->fused && ntok == 1u;
     const bool group_in_select = m->small_batch(ntok);
     m->skip_select = select_in_gateup;
     m->select_and_group = group_in_select;
