@@ -86,6 +86,18 @@ hipError_t launch_batch_combine(const float *tmp, const float *pair_weight, cons
                                 const float *sh_tmp, const float *scalar, uint32_t hidden, float *out, hipStream_t s);
 
 // pair sort of [ntok][top_k] ids: see redhip_moe_group in include/redhip_moe.h
+// prefill chunk on packed IQ2_XXS experts: tiles of 16 pairs per distinct expert, 16x16x16 fp16 MFMA. Needs the pair
+// grouping (uid, expert_start, pair_token, n_unique); writes tmp [pairs][hidden] and sh_tmp [ntok][hidden] for
+// launch_batch_combine. tile_* hold prefill_tile_bound() entries.
+inline uint32_t prefill_tile_bound(uint32_t ntok, uint32_t top_k, uint32_t n_expert) {
+    const uint32_t P = ntok * top_k;
+    return (P < n_expert ? P : n_expert) + P / 16u + (ntok + 15u) / 16u + 1u;
+}
+hipError_t launch_prefill_packed(const void *experts, uint64_t stride, const void *shared, const uint32_t *uid, const uint32_t *expert_start,
+                                 const uint32_t *pair_token, const uint32_t *n_unique, uint32_t *tile_group, uint32_t *tile_pair0,
+                                 uint32_t *tile_n, uint32_t *n_tiles, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l,
+                                 int *act_exp, float *tmp, float *sh_tmp, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok,
+                                 uint32_t n_expert, hipStream_t s);
 hipError_t launch_group_pairs(const uint32_t *ids, const float *weights, uint32_t ntok, uint32_t top_k, uint32_t n_expert,
                               uint32_t *uid, uint32_t *expert_start, uint32_t *pair_token, float *pair_weight,
                               uint32_t *tok_pair, uint32_t *n_unique, hipStream_t s);

@@ -56,6 +56,7 @@ struct Moe {
     bool skip_select = false;                // forward(): the gate/up kernel selects, route() skips its own selection
     // batched path (ntok > 1): pairs grouped by expert
     uint32_t *uid = nullptr, *expert_start = nullptr, *pair_token = nullptr, *tok_pair = nullptr, *n_unique = nullptr;
+    uint32_t *tile_group = nullptr, *tile_pair0 = nullptr, *tile_n = nullptr, *n_tiles = nullptr;      // prefill tiles
     float *pair_weight = nullptr, *tmp = nullptr, *sh_tmp = nullptr;
     void *act_h = nullptr, *act_l = nullptr; // fp16 [top_k + 1][ffn] each
     int *act_exp = nullptr;                  // [top_k + 1][ffn / 32]
@@ -64,6 +65,8 @@ struct Moe {
     bool small_batch(uint32_t ntok) const {
         return fused && ntok >= 2u && ntok <= 8u && ntok * cfg.top_k <= 128u && ntok * (cfg.top_k + 1u) <= 144u && cfg.hidden / 512u <= 4u;
     }
+    // every batch size runs on the packed layout when the layer has one (decode kernel, small-batch kernels, prefill tiles)
+    bool packed_path(uint32_t ntok) const { return fused && (ntok == 1u || small_batch(ntok) || cfg.hidden / 512u <= 4u); }
     ExpertSet routed(uint32_t l) const { return ExpertSet{layers[l].experts, expert_stride, gate_bytes, gate_bytes, gu_type, dn_type}; }
     ExpertSet shared(uint32_t l) const { return ExpertSet{layers[l].shared, 0, sh_gate_bytes, sh_gate_bytes, sh_gu_type, sh_dn_type}; }
 };
@@ -107,6 +110,16 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
             HIP_OK(launch_batch_packed(L.packed, m->expert_stride, L.shared_packed, m->uid, m->expert_start, m->pair_token, m->n_unique,
                                        m->pair_weight, m->tok_pair, m->scalar, m->xh, m->xl, m->xexp, m->act_h, m->act_l, m->act_exp, out,
                                        c.hidden, c.ffn, c.top_k, ntok, c.n_expert, s), "batched packed launch");
+            prof_set_stage(ST_OTHER);
+            return 1;
+        }
+        if (m->packed_path(ntok)) {     // prefill chunk: tiles of 16 pairs per expert on the MFMA units
+            const Layer &L = m->layers[layer];
+            HIP_OK(launch_prefill_packed(L.packed, m->expert_stride, L.shared_packed, m->uid, m->expert_start, m->pair_token, m->n_unique,
+                                         m->tile_group, m->tile_pair0, m->tile_n, m->n_tiles, m->xh, m->xl, m->xexp, m->act_h, m->act_l,
+                                         m->act_exp, m->tmp, m->sh_tmp, c.hidden, c.ffn, c.top_k, ntok, c.n_expert, s), "prefill launch");
+            prof_set_stage(ST_BATCH_COMBINE);
+            HIP_OK(launch_batch_combine(m->tmp, m->pair_weight, m->tok_pair, ntok, c.top_k, m->sh_tmp, m->scalar, c.hidden, out, s), "batched combine launch");
             prof_set_stage(ST_OTHER);
             return 1;
         }
@@ -203,7 +216,8 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
                             align256(T * c.top_k * c.ffn * 4u) + align256(T * c.ffn * 4u) +
                             2u * align256(2u * T * c.hidden) + align256(4u * T) + 2u * align256(2u * T * (c.top_k + 1u) * c.ffn) +
                             align256(4u * T * (c.top_k + 1u) * (c.ffn / 32u)) +
-                            (T > 1u ? 6u * align256(4u * (T * c.top_k + 2u)) + align256(4u * T * c.top_k * c.hidden) + align256(4u * T * c.hidden) : 0u);
+                            (T > 1u ? 6u * align256(4u * (T * c.top_k + 2u)) + align256(4u * T * c.top_k * c.hidden) + align256(4u * T * c.hidden) +
+                                          4u * align256(4u * (size_t)prefill_tile_bound(c.max_tokens, c.top_k, c.n_expert)) : 0u);
     ok = ok && hipMalloc(reinterpret_cast<void **>(&m->ws), ws_bytes) == hipSuccess;
     if (!ok) {
         moe_err("failed to allocate resident MoE memory (%llu bytes so far)", (unsigned long long)m->resident);
@@ -232,7 +246,12 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
         m->n_unique = reinterpret_cast<uint32_t *>(w); w += pw;
         m->pair_weight = reinterpret_cast<float *>(w); w += pw;
         m->tmp = reinterpret_cast<float *>(w); w += align256(4u * T * c.top_k * c.hidden);
-        m->sh_tmp = reinterpret_cast<float *>(w);
+        m->sh_tmp = reinterpret_cast<float *>(w); w += align256(4u * T * c.hidden);
+        const size_t tw = align256(4u * (size_t)prefill_tile_bound(c.max_tokens, c.top_k, c.n_expert));
+        m->tile_group = reinterpret_cast<uint32_t *>(w); w += tw;
+        m->tile_pair0 = reinterpret_cast<uint32_t *>(w); w += tw;
+        m->tile_n = reinterpret_cast<uint32_t *>(w); w += tw;
+        m->n_tiles = reinterpret_cast<uint32_t *>(w);
     }
     if (hipMemset(m->ws, 0, ws_bytes) != hipSuccess) { moe_err("failed to clear the MoE workspace"); redhip_moe_destroy(m); return nullptr; }
     // first launches copy the codebooks to the device; do it here so that forward never synchronises
@@ -358,7 +377,7 @@ int redhip_moe_experts(redhip_moe_t h, uint32_t layer, const float *x_dev, uint3
     if (!check_layer(m, layer)) return 0;
     if (!x_dev || !ids_dev || !weights_dev || !out_dev || !ntok || ntok > m->cfg.max_tokens) { moe_err("invalid expert execution arguments"); return 0; }
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (m->fused && (ntok == 1u || m->small_batch(ntok))) {
+    if (m->packed_path(ntok)) {
         prof_set_stage(ST_OTHER);
         HIP_OK(launch_prep(x_dev, m->layers[layer].gate_inp, ntok, m->cfg.hidden, m->xh, m->xl, m->xexp, m->scalar, s), "prep launch");
         return experts_enqueue(m, layer, x_dev, ntok, ids_dev, weights_dev, out_dev, s);

@@ -1,0 +1,367 @@
+// Prefill chunk (tens to hundreds of tokens) on packed IQ2_XXS experts: the (token, expert) pairs of one expert are cut
+// into tiles of 16 pairs, and a tile against 16 weight rows is one v_mfma_f32_16x16x16_f16 per 16 columns.
+//
+// Operand mapping (lane l, r = l % 16, q = l / 16), checked on gfx950:
+//   A[i = r][k = 4q .. 4q + 3]   activations of tile pair r
+//   B[k = 4q .. 4q + 3][j = r]   weights of row r
+//   D[i = 4q .. 4q + 3][j = r]   the lane receives ITS OWN row against four pairs
+// One IQ2_XXS group (32 weights, 4 grid entries) is two MFMAs: lane (r, q) decodes grid entry q of row r and feeds its
+// first four weights to the first MFMA and the other four to the second; the activation operand uses the same k order
+// (columns 8q .. 8q + 3, then 8q + 4 .. 8q + 7 of the group). Because D's column is the lane's own row, the group scale
+// (2 s + 1) and the block scale d are applied to the accumulator, per group, in f32. Activations are fp16 hi + lo
+// halves (22 bits) as everywhere else, so a group costs four MFMAs.
+//
+// Reference behaviour this replaces: native/redmetal_engine_prefill.m:1246-1330 (grouped GEMM over expert slices)
+// with the arithmetic of native/redlite_native_reference.c:251-382.
+#include <hip/hip_runtime.h>
+
+#include "redhip_mfma.h"
+
+namespace redhip {
+
+constexpr uint32_t kTile = 16u;                 // pairs per tile
+constexpr uint32_t kRowPad = 32u;               // fp16 elements of padding per staged activation row (64 B: spreads the rows over the banks)
+
+// ---------------------------------------------------------------- tile list
+
+// groups 0..U-1 are the distinct routed experts (pairs expert_start[u] .. expert_start[u + 1]), group U is the shared
+// expert with pairs P .. P + ntok. One workgroup: exclusive prefix sum of the tiles per group, then every group writes
+// its tiles: (group, first pair, number of pairs).
+__global__ __launch_bounds__(1024) void build_tiles_kernel(const uint32_t *expert_start, const uint32_t *n_unique, uint32_t P, uint32_t ntok,
+                                                           uint32_t *tile_group, uint32_t *tile_pair0, uint32_t *tile_n, uint32_t *n_tiles) {
+    __shared__ uint32_t wave_total[16];
+    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
+    const uint32_t U = n_unique[0];
+    uint32_t p0 = 0u, n = 0u;
+    if (tid < U) { p0 = expert_start[tid]; n = expert_start[tid + 1u] - p0; }
+    const uint32_t mine = (n + kTile - 1u) / kTile;
+    uint32_t scan = mine;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) {
+        const uint32_t up = __shfl_up(scan, o, 64);
+        if (lane >= (uint32_t)o) scan += up;
+    }
+    if (lane == 63u) wave_total[wave] = scan;
+    __syncthreads();
+    uint32_t base = 0u, routed_tiles = 0u;
+    for (uint32_t w = 0; w < 16u; ++w) { if (w < wave) base += wave_total[w]; routed_tiles += wave_total[w]; }
+    const uint32_t first = base + scan - mine;
+    for (uint32_t t = 0; t < mine; ++t) {
+        tile_group[first + t] = tid;
+        tile_pair0[first + t] = p0 + kTile * t;
+        tile_n[first + t] = n - kTile * t < kTile ? n - kTile * t : kTile;
+    }
+    const uint32_t shared_tiles = (ntok + kTile - 1u) / kTile;
+    for (uint32_t t = tid; t < shared_tiles; t += 1024u) {
+        tile_group[routed_tiles + t] = U;
+        tile_pair0[routed_tiles + t] = P + kTile * t;
+        tile_n[routed_tiles + t] = ntok - kTile * t < kTile ? ntok - kTile * t : kTile;
+    }
+    if (tid == 0u) n_tiles[0] = routed_tiles + shared_tiles;
+}
+
+struct PrefillArgs {
+    const uint8_t *experts;
+    uint64_t stride;
+    const uint8_t *shared;
+    const uint32_t *uid, *pair_token, *n_unique;
+    const uint32_t *tile_group, *tile_pair0, *tile_n, *n_tiles;
+    const _Float16 *xh, *xl;       // [ntok][hidden]
+    const int *xexp;               // [ntok]
+    _Float16 *act_h, *act_l;       // [P + ntok][ffn]
+    int *act_exp;                  // [P + ntok][ffn / 32]
+    float *tmp, *sh_tmp;           // down outputs: [P][hidden] routed pairs, [ntok][hidden] shared expert
+    uint32_t hidden, ffn, top_k, ntok;
+};
+
+// signed weights of grid entry q of a group word, and the group scale 2 s + 1
+__device__ __forceinline__ void decode_entry(uint2 w, uint32_t q, const uint8_t *lds, WeightQuad &b0, WeightQuad &b1) {
+    const uint32_t idx = (w.x >> (8u * q)) & 255u, s7 = (w.y >> (7u * q)) & 127u;
+    place_signs(*reinterpret_cast<const uint4 *>(lds + (idx << 4)), s7, b0, b1);
+}
+
+union Half8 { uint4 u; half4_t h[2]; };
+
+// one group of 32 columns: acc = A x B over the group's 32 k, activations hi and lo; returns the four f32 sums of this
+// lane's row against pairs 4q .. 4q + 3, without the scales
+__device__ __forceinline__ float4_t group_mfma(const Half8 &xa, const Half8 &xb, const WeightQuad &b0, const WeightQuad &b1) {
+    float4_t hi = {0.0f, 0.0f, 0.0f, 0.0f}, lo = {0.0f, 0.0f, 0.0f, 0.0f};
+    hi = __builtin_amdgcn_mfma_f32_16x16x16f16(xa.h[0], b0.h, hi, 0, 0, 0);
+    lo = __builtin_amdgcn_mfma_f32_16x16x16f16(xb.h[0], b0.h, lo, 0, 0, 0);
+    hi = __builtin_amdgcn_mfma_f32_16x16x16f16(xa.h[1], b1.h, hi, 0, 0, 0);
+    lo = __builtin_amdgcn_mfma_f32_16x16x16f16(xb.h[1], b1.h, lo, 0, 0, 0);
+    float4_t r;
+#pragma unroll
+    for (int t = 0; t < 4; ++t) r[t] = fmaf(lo[t], 4.8828125e-4f, hi[t]);
+    return r;
+}
+
+// ---------------------------------------------------------------- gate/up + SwiGLU
+
+// A workgroup takes whole tiles: the fp16 halves of the tile's 16 tokens are staged in LDS once, then the 32-column
+// groups g of the FFN are walked. Wave = (row tile rt: gate rows 0..15, gate 16..31, up 0..15, up 16..31 of the
+// group; K quarter kc). The four K quarters meet in LDS, SwiGLU and the fp16 split of the activation follow.
+template <int NKC>          // hidden = 512 * NKC
+__global__ __launch_bounds__(kWaves * 64) void prefill_gateup_kernel(PrefillArgs a) {
+    constexpr uint32_t H = 512u * NKC, HG = H / 32u, HB = H / 256u, GPW = HG / 4u, ROW = H + kRowPad;   // GPW: groups per wave
+    extern __shared__ __attribute__((aligned(16))) uint8_t dyn[];          // xs_h | xs_l: [16][ROW] fp16
+    __shared__ __attribute__((aligned(16))) uint8_t lds[kMagBytes];
+    __shared__ float part[4][kTile][68];                   // [K quarter][pair][row of the unit], rows padded off the bank stride
+    __shared__ float tok_scale[kTile];
+    __shared__ uint32_t tok_of[kTile];
+    _Float16 *xs_h = reinterpret_cast<_Float16 *>(dyn), *xs_l = xs_h + kTile * ROW;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, r = lane & 15u, q = lane >> 4;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6), rt = wave & 3u, kc = wave >> 2;
+    const uint32_t F = a.ffn, FG = F / 32u, P = a.ntok * a.top_k;
+    const uint64_t grid_entry = tid < 256u ? redhip_iq2xxs_grid[tid] : 0ull;
+    build_tables(lds, tid, grid_entry);
+    const uint32_t T = a.n_tiles[0], U = a.n_unique[0];
+    const uint64_t qs_bytes = (uint64_t)F * HG * 8u, gate_bytes = qs_bytes + (uint64_t)F * HB * 2u;
+
+    for (uint32_t tile = blockIdx.x; tile < T; tile += gridDim.x) {
+        const uint32_t u = a.tile_group[tile], p0 = a.tile_pair0[tile], n = a.tile_n[tile];
+        const uint8_t *ex = u == U ? a.shared : a.experts + (uint64_t)a.uid[u] * a.stride;
+        __syncthreads();                                   // the previous tile's readers are done with xs / tok_of
+        if (tid < kTile) {
+            const uint32_t p = p0 + tid, tok = tid < n ? (p < P ? a.pair_token[p] : p - P) : 0u;
+            tok_of[tid] = tok;
+            tok_scale[tid] = tid < n ? 0.125f * exp2i(a.xexp[tok]) : 0.0f;
+        }
+        __syncthreads();
+        {   // stage: 64 lanes per token, 16 bytes at a time
+            const uint32_t i = tid >> 6, tok = tok_of[i];
+            const bool live = i < n;
+            for (uint32_t c = lane; c < H / 8u; c += 64u) {
+                uint4 vh = make_uint4(0u, 0u, 0u, 0u), vl = vh;
+                if (live) {
+                    vh = reinterpret_cast<const uint4 *>(a.xh + (uint64_t)tok * H)[c];
+                    vl = reinterpret_cast<const uint4 *>(a.xl + (uint64_t)tok * H)[c];
+                }
+                *reinterpret_cast<uint4 *>(xs_h + i * ROW + 8u * c) = vh;
+                *reinterpret_cast<uint4 *>(xs_l + i * ROW + 8u * c) = vl;
+            }
+        }
+        __syncthreads();
+
+        // The wave's weights arrive in chunks of four groups (32 bytes of a row); the chunk after the current one, in
+        // the same unit or the next, is always in flight.
+        constexpr uint32_t CPU = GPW / 4u;                 // chunks per unit
+        const uint8_t *mat = ex + (rt < 2u ? 0u : gate_bytes);
+        auto chunk_ptr = [&](uint32_t it) {
+            const uint32_t g = it / CPU, c = it % CPU, row = 32u * g + 16u * (rt & 1u) + r;
+            return reinterpret_cast<const uint4 *>(mat + ((uint64_t)row * HG + kc * GPW + 4u * c) * 8u);
+        };
+        auto scale_ptr = [&](uint32_t it) {
+            const uint32_t g = it / CPU, c = it % CPU, row = 32u * g + 16u * (rt & 1u) + r;
+            return reinterpret_cast<const uint16_t *>(mat + qs_bytes) + (uint64_t)row * HB + (kc * GPW + 4u * c) / 8u;
+        };
+        const uint32_t n_it = FG * CPU;
+        uint4 wa = chunk_ptr(0u)[0], wb = chunk_ptr(0u)[1];
+        uint32_t dcur = *scale_ptr(0u);
+        float4_t tot = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll 1
+        for (uint32_t it = 0; it < n_it; ++it) {
+            const uint32_t nx = it + 1u < n_it ? it + 1u : it;
+            const uint4 na = chunk_ptr(nx)[0], nb = chunk_ptr(nx)[1];
+            const uint32_t dnext = *scale_ptr(nx);
+            const uint32_t g = it / CPU, c = it % CPU;
+            const uint2 w4[4] = {make_uint2(wa.x, wa.y), make_uint2(wa.z, wa.w), make_uint2(wb.x, wb.y), make_uint2(wb.z, wb.w)};
+            const uint32_t lane_off = r * ROW + 32u * (kc * GPW + 4u * c) + 8u * q;
+            float4_t blk = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (uint32_t k = 0; k < 4u; ++k) {
+                Half8 xa, xb;
+                xa.u = *reinterpret_cast<const uint4 *>(xs_h + lane_off + 32u * k);
+                xb.u = *reinterpret_cast<const uint4 *>(xs_l + lane_off + 32u * k);
+                WeightQuad b0, b1;
+                decode_entry(w4[k], q, lds, b0, b1);
+                const float4_t sm = group_mfma(xa, xb, b0, b1);
+                const float f = (float)(2u * (w4[k].y >> 28) + 1u);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) blk[t] = fmaf(sm[t], f, blk[t]);
+            }
+            const float d = scale_to_f32(dcur);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) tot[t] = fmaf(blk[t], d, tot[t]);
+            wa = na; wb = nb; dcur = dnext;
+            if (c + 1u < CPU) continue;
+            // end of the unit (g): the K quarters meet
+#pragma unroll
+            for (int t = 0; t < 4; ++t) part[kc][4u * q + (uint32_t)t][16u * rt + r] = tot[t];
+            __syncthreads();
+            if (tid < 512u) {                              // (pair i, column c): lanes 0..31 of a half wave share a pair
+                const uint32_t i = tid >> 5, c = tid & 31u;
+                float gsum = 0.0f, usum = 0.0f;
+#pragma unroll
+                for (int k4 = 0; k4 < 4; ++k4) { gsum += part[k4][i][c]; usum += part[k4][i][32u + c]; }
+                const float xs = tok_scale[i];
+                gsum *= xs;
+                usum *= xs;
+                const float act = (gsum / (1.0f + expf(-gsum))) * usum;
+                float amax = fabsf(act);
+#pragma unroll
+                for (int o = 16; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+                if (i < n) {
+                    const int e = prescale_exp(amax);
+                    const uint64_t pr = p0 + i;
+                    split_hi_lo(act, exp2i(-e), a.act_h + pr * F + 32u * g + c, a.act_l + pr * F + 32u * g + c);
+                    if (c == 0u) a.act_exp[pr * FG + g] = e;
+                }
+            }
+            __syncthreads();
+            tot = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        }
+    }
+}
+
+// ---------------------------------------------------------------- down
+
+// A workgroup takes whole tiles: the tile's activations (fp16 halves and the per-group exponents) are staged in LDS,
+// then wave w computes rows 256 c + 16 w .. + 15 for c = 0, 1, ... against all ffn columns. No reduction across
+// waves: every lane ends with its row against four pairs and stores them.
+template <int NFG>          // ffn = 32 * NFG
+__global__ __launch_bounds__(kWaves * 64) void prefill_down_kernel(PrefillArgs a) {
+    constexpr uint32_t F = 32u * NFG, FB = F / 256u, ROW = F + kRowPad;
+    extern __shared__ __attribute__((aligned(16))) uint8_t dyn[];          // as_h | as_l: [16][ROW] fp16
+    _Float16 *as_h = reinterpret_cast<_Float16 *>(dyn), *as_l = as_h + kTile * ROW;
+    __shared__ __attribute__((aligned(16))) float as_scale[NFG][kTile];     // 2^exponent of (group, pair)
+    __shared__ __attribute__((aligned(16))) uint8_t lds[kMagBytes];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, r = lane & 15u, q = lane >> 4;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t H = a.hidden, P = a.ntok * a.top_k;
+    const uint64_t grid_entry = tid < 256u ? redhip_iq2xxs_grid[tid] : 0ull;
+    build_tables(lds, tid, grid_entry);
+    const uint32_t T = a.n_tiles[0], U = a.n_unique[0];
+    const uint64_t down_off = 2u * ((uint64_t)F * (H / 32u) * 8u + (uint64_t)F * (H / 256u) * 2u), qs_bytes = (uint64_t)H * NFG * 8u;
+
+    for (uint32_t tile = blockIdx.x; tile < T; tile += gridDim.x) {
+        const uint32_t u = a.tile_group[tile], p0 = a.tile_pair0[tile], n = a.tile_n[tile];
+        const uint8_t *dn = (u == U ? a.shared : a.experts + (uint64_t)a.uid[u] * a.stride) + down_off;
+        __syncthreads();
+        {
+            const uint32_t i = tid >> 6;
+            const bool live = i < n;
+            for (uint32_t c = lane; c < F / 8u; c += 64u) {
+                uint4 vh = make_uint4(0u, 0u, 0u, 0u), vl = vh;
+                if (live) {
+                    vh = reinterpret_cast<const uint4 *>(a.act_h + (uint64_t)(p0 + i) * F)[c];
+                    vl = reinterpret_cast<const uint4 *>(a.act_l + (uint64_t)(p0 + i) * F)[c];
+                }
+                *reinterpret_cast<uint4 *>(as_h + i * ROW + 8u * c) = vh;
+                *reinterpret_cast<uint4 *>(as_l + i * ROW + 8u * c) = vl;
+            }
+            if (lane < NFG) as_scale[lane][i] = live ? exp2i(a.act_exp[(uint64_t)(p0 + i) * NFG + lane]) : 0.0f;
+        }
+        __syncthreads();
+        // Rows 256 b + 16 w + r for b = 0, 1, ...; the weights of a row arrive in chunks of four groups and the chunk after
+        // the current one (same row block or the next) is always in flight.
+        constexpr uint32_t NCK = NFG / 4u;
+        const uint8_t *lane_rows = dn + (uint64_t)(16u * wave + r) * NFG * 8u;
+        const uint16_t *lane_ds = reinterpret_cast<const uint16_t *>(dn + qs_bytes) + (uint64_t)(16u * wave + r) * FB;
+        auto chunk_ptr = [&](uint32_t it) {
+            return reinterpret_cast<const uint4 *>(lane_rows + (uint64_t)(it / NCK) * (16u * kWaves) * NFG * 8u + (it % NCK) * 32u);
+        };
+        auto scale_ptr = [&](uint32_t it) { return lane_ds + (uint64_t)(it / NCK) * (16u * kWaves) * FB + (it % NCK) / 2u; };
+        const uint32_t n_it = (H / (16u * kWaves)) * NCK;
+        uint4 wa = chunk_ptr(0u)[0], wb = chunk_ptr(0u)[1];
+        uint32_t dcur = *scale_ptr(0u);
+        float4_t tot = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll 1
+        for (uint32_t it = 0; it < n_it; ++it) {
+            const uint32_t nx = it + 1u < n_it ? it + 1u : it;
+            const uint4 na = chunk_ptr(nx)[0], nb = chunk_ptr(nx)[1];
+            const uint32_t dnext = *scale_ptr(nx);
+            const uint32_t c = it % NCK;
+            const uint2 w4[4] = {make_uint2(wa.x, wa.y), make_uint2(wa.z, wa.w), make_uint2(wb.x, wb.y), make_uint2(wb.z, wb.w)};
+            const uint32_t lane_off = r * ROW + 128u * c + 8u * q;
+            float4_t blk = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (uint32_t k = 0; k < 4u; ++k) {
+                Half8 xa, xb;
+                xa.u = *reinterpret_cast<const uint4 *>(as_h + lane_off + 32u * k);
+                xb.u = *reinterpret_cast<const uint4 *>(as_l + lane_off + 32u * k);
+                WeightQuad b0, b1;
+                decode_entry(w4[k], q, lds, b0, b1);
+                const float4_t sm = group_mfma(xa, xb, b0, b1);
+                const float4_t sc = *reinterpret_cast<const float4_t *>(&as_scale[4u * c + k][4u * q]);
+                const float f = (float)(2u * (w4[k].y >> 28) + 1u);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) blk[t] = fmaf(sm[t] * sc[t], f, blk[t]);
+            }
+            const float d = scale_to_f32(dcur);
+#pragma unroll
+            for (int t = 0; t < 4; ++t) tot[t] = fmaf(blk[t], d, tot[t]);
+            wa = na; wb = nb; dcur = dnext;
+            if (c + 1u < NCK) continue;
+            const uint32_t row = (it / NCK) * (16u * kWaves) + 16u * wave + r;
+#pragma unroll
+            for (uint32_t t = 0; t < 4u; ++t) {
+                const uint32_t i = 4u * q + t, p = p0 + i;
+                if (i < n) (p < P ? a.tmp + (uint64_t)p * H : a.sh_tmp + (uint64_t)(p - P) * H)[row] = 0.125f * tot[t];
+            }
+            tot = float4_t{0.0f, 0.0f, 0.0f, 0.0f};
+        }
+    }
+}
+
+hipError_t launch_prefill_packed(const void *experts, uint64_t stride, const void *shared, const uint32_t *uid, const uint32_t *expert_start,
+                                 const uint32_t *pair_token, const uint32_t *n_unique, uint32_t *tile_group, uint32_t *tile_pair0,
+                                 uint32_t *tile_n, uint32_t *n_tiles, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l,
+                                 int *act_exp, float *tmp, float *sh_tmp, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok,
+                                 uint32_t n_expert, hipStream_t s) {
+    if (!fused_iq2_supported(hidden, ffn) || hidden / 512u > 4u || !ntok) return hipErrorInvalidValue;
+    const uint32_t P = ntok * top_k;
+    prof_set_stage(ST_GROUP);
+    REDHIP_LAUNCH(build_tiles_kernel, dim3(1), dim3(1024), 0, s, expert_start, n_unique, P, ntok, tile_group, tile_pair0, tile_n, n_tiles);
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    PrefillArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(shared), uid, pair_token, n_unique,
+                  tile_group, tile_pair0, tile_n, n_tiles, static_cast<const _Float16 *>(xh), static_cast<const _Float16 *>(xl), xexp,
+                  static_cast<_Float16 *>(act_h), static_cast<_Float16 *>(act_l), act_exp, tmp, sh_tmp, hidden, ffn, top_k, ntok};
+    const uint32_t tile_bound = prefill_tile_bound(ntok, top_k, n_expert);
+    const dim3 grid(tile_bound < 256u ? tile_bound : 256u), block(kWaves * 64);
+    const size_t dyn_lds = (size_t)2u * kTile * (hidden + kRowPad) * 2u;
+    prof_set_stage(ST_PREFILL_GATEUP);
+#define REDHIP_PGU(NKC)                                                                                                                   \
+    do {                                                                                                                                  \
+        static bool attr = false;                                                                                                          \
+        if (!attr) {                                                                                                                       \
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(prefill_gateup_kernel<NKC>), hipFuncAttributeMaxDynamicSharedMemorySize, 136 * 1024); \
+            if (e != hipSuccess) return e;                                                                                                 \
+            attr = true;                                                                                                                   \
+        }                                                                                                                                  \
+        REDHIP_LAUNCH(prefill_gateup_kernel<NKC>, grid, block, dyn_lds, s, a);                                                             \
+    } while (0)
+    switch (hidden / 512u) {
+        case 1: REDHIP_PGU(1); break;
+        case 2: REDHIP_PGU(2); break;
+        case 4: REDHIP_PGU(4); break;
+        default: return hipErrorInvalidValue;
+    }
+#undef REDHIP_PGU
+    e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    prof_set_stage(ST_PREFILL_DOWN);
+    const size_t down_lds = (size_t)2u * kTile * (ffn + kRowPad) * 2u;
+#define REDHIP_PDN(NFG)                                                                                                                   \
+    do {                                                                                                                                  \
+        static bool attr = false;                                                                                                          \
+        if (!attr) {                                                                                                                       \
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(prefill_down_kernel<NFG>), hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024); \
+            if (e != hipSuccess) return e;                                                                                                 \
+            attr = true;                                                                                                                   \
+        }                                                                                                                                  \
+        REDHIP_LAUNCH(prefill_down_kernel<NFG>, grid, block, down_lds, s, a);                                                              \
+    } while (0)
+    switch (ffn / 256u) {
+        case 1: REDHIP_PDN(8); break;
+        case 2: REDHIP_PDN(16); break;
+        case 3: REDHIP_PDN(24); break;
+        case 4: REDHIP_PDN(32); break;
+        default: return hipErrorInvalidValue;
+    }
+#undef REDHIP_PDN
+    return hipGetLastError();
+}
+
+}  // namespace redhip

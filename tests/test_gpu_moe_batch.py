@@ -82,3 +82,43 @@ def test_prefill_sized_chunk_zipf():
     want = oracle_tokens(cfg, lay, x, ids, w)
     assert max(rel_l2(got[t], want[t]) for t in range(ntok)) <= REL_L2_TOL
     m.close()
+
+
+@pytest.mark.parametrize("hidden,ffn,ntok", [(1024, 512, 96), (512, 256, 40), (2048, 768, 33)])
+def test_prefill_chunk_packed_tiles(hidden, ffn, ntok):
+    """Prefill chunk on the packed IQ2_XXS layout (tiles of 16 pairs per expert on the 16x16x16 MFMA): Zipf routing, so
+    one expert fills several tiles, others have a single pair, some none; the last tile of a group is partial."""
+    from dwarfstar_red_lite_amd.moe import ResidentMoe
+    cfg = synth.layer_config(hidden=hidden, ffn=ffn, n_expert=64, top_k=4, layout="iq2")
+    lay = synth.make_layer(6, cfg)
+    m = ResidentMoe(cfg, n_layer=1, max_tokens=ntok)
+    m.load_layer(0, lay)
+    rng = np.random.default_rng(9)
+    x = synth.normed_x(rng, ntok, hidden)
+    ids = synth.zipf_topk(rng, ntok, 64, 4)
+    w = rng.random((ntok, 4)).astype(np.float32)
+    w /= w.sum(axis=1, keepdims=True)
+    counts = np.bincount(ids.ravel(), minlength=64)
+    assert counts.max() > 16 and counts.min() < 4
+    got = m.experts(0, torch.from_numpy(x).cuda(), torch.from_numpy(ids.astype(np.int32)).cuda(), torch.from_numpy(w).cuda()).cpu().numpy()
+    want = oracle_tokens(cfg, lay, x, ids, w)
+    assert max(rel_l2(got[t], want[t]) for t in range(ntok)) <= REL_L2_TOL
+    m.close()
+
+
+def test_prefill_chunk_forward_config_shape():
+    """A 24-token chunk at the benchmark shape through forward(): router, selection, grouping, tiles, combine."""
+    from dwarfstar_red_lite_amd.moe import ResidentMoe
+    cfg = synth.layer_config(layout="iq2")
+    lay = synth.make_layer(78, cfg)
+    ntok = 24
+    m = ResidentMoe(cfg, n_layer=1, max_tokens=ntok)
+    m.load_layer(0, lay)
+    x = synth.normed_x(np.random.default_rng(32), ntok, cfg["hidden"])
+    got = m.forward(0, torch.from_numpy(x).cuda()).cpu().numpy()
+    gids, gw, _ = m.last_route(ntok)
+    want, cids, cw, _ = orc.Layer(cfg, **lay).forward(x, threads=8)
+    assert np.array_equal(gids, cids)
+    assert np.abs(gw - cw).max() <= 1e-5
+    assert max(rel_l2(got[t], want[t]) for t in range(ntok)) <= REL_L2_TOL
+    m.close()
