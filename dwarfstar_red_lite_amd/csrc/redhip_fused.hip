@@ -22,6 +22,17 @@
 
 namespace redhip {
 
+#ifdef REDHIP_KTS
+__device__ unsigned long long g_kts[256 * 32], g_kts2[256 * 32];
+#define KTS(i) do { if (threadIdx.x == 0u && blockIdx.x < 256u && (i) < 32u) { g_kts[blockIdx.x * 32u + (i)] = wall_clock64(); g_kts2[blockIdx.x * 32u + (i)] = clock64(); } } while (0)
+#define SEL_TS(i) do {} while (0)
+#define KTSY(i) do { const uint32_t wg_ = blockIdx.x + gridDim.x * blockIdx.y; if (threadIdx.x == 0u && wg_ < 256u) { g_kts[wg_ * 32u + (i)] = wall_clock64(); } } while (0)
+#else
+#define KTSY(i) do {} while (0)
+#define KTS(i) do {} while (0)
+#define SEL_TS(i) do {} while (0)
+#endif
+
 
 // ---------------------------------------------------------------- repacking (upload time)
 
@@ -142,6 +153,43 @@ __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
 __device__ __forceinline__ uint32_t wave_count(bool pred) { return (uint32_t)__popcll(__ballot(pred)); }
+// Raw GGUF rows are decoded from LDS: a wave copies `bytes` (a multiple of 16, both addresses 16-byte aligned) with
+// coalesced 16-byte loads, so the many one- and two-byte fields of a block never go to memory one by one.
+__device__ __forceinline__ void wave_stage(uint8_t *dst, const uint8_t *src, uint32_t bytes, uint32_t lane) {
+    if (((uint32_t)(uintptr_t)src | bytes) % 16u == 0u) {
+        for (uint32_t i = lane; i < bytes / 16u; i += 64u) reinterpret_cast<uint4 *>(dst)[i] = reinterpret_cast<const uint4 *>(src)[i];
+    } else {                                             // GGUF blocks are always a multiple of two bytes
+        for (uint32_t i = lane; i < bytes / 2u; i += 64u) reinterpret_cast<uint16_t *>(dst)[i] = reinterpret_cast<const uint16_t *>(src)[i];
+    }
+}
+
+// One chunk of 32 Q6_K weights against 32 activations held in registers; sx0 / sx1 are the sums of the first and the
+// second 16 activations. The 6-bit quants are unpacked four at a time with byte-parallel integer operations and enter
+// the FMAs as unsigned bytes; the offset of 32 comes back through the activation sums:
+//   sum (q - 32) d s x = d s (sum q x - 32 sum x).  Layout as native/redlite_native_quant_cpu.c:130-153 reads it.
+__device__ __forceinline__ float q6k_dot32(const uint8_t *row, uint32_t chunk, const float *xv, float sx0, float sx1) {
+    const uint8_t *bp = row + (size_t)(chunk >> 3) * 210u;
+    const uint32_t sub = chunk & 7u, half = sub >> 2, q = sub & 3u;
+    const uint8_t *ql = bp + 64u * half + 32u * (q & 1u), *qh = bp + 128u + 32u * half;
+    const uint32_t scs = ld_u16(bp + 192u + 8u * half + 2u * q);
+    const float d = half_bits_to_f32(ld_u16(bp + 208u));
+    const float s0 = (float)(int)(int8_t)(scs & 255u), s1 = (float)(int)(int8_t)(scs >> 8);
+    const uint32_t nib_shift = (q >> 1) * 4u, hi_shift = 2u * q;
+    float acc0 = 0.0f, acc1 = 0.0f;
+#pragma unroll
+    for (uint32_t v = 0; v < 8u; ++v) {
+        uint32_t lo4, hi4;                               // 2-byte aligned: odd blocks of a row start at 2 mod 4
+        __builtin_memcpy(&lo4, __builtin_assume_aligned(ql + 4u * v, 2), 4);
+        __builtin_memcpy(&hi4, __builtin_assume_aligned(qh + 4u * v, 2), 4);
+        const uint32_t q4 = ((lo4 >> nib_shift) & 0x0f0f0f0fu) | (((hi4 >> hi_shift) & 0x03030303u) << 4);
+        float &acc = v < 4u ? acc0 : acc1;
+        acc = fmaf((float)(q4 & 255u), xv[4u * v], acc);
+        acc = fmaf((float)((q4 >> 8) & 255u), xv[4u * v + 1u], acc);
+        acc = fmaf((float)((q4 >> 16) & 255u), xv[4u * v + 2u], acc);
+        acc = fmaf((float)(q4 >> 24), xv[4u * v + 3u], acc);
+    }
+    return d * (s0 * fmaf(-32.0f, sx0, acc0) + s1 * fmaf(-32.0f, sx1, acc1));
+}
 
 // ---------------------------------------------------------------- router GEMV
 
@@ -152,6 +200,11 @@ struct RouterArgs {
     _Float16 *xh, *xl;         // [ntok][hidden] fp16 halves of x * 2^-xexp
     int *xexp;                 // [ntok]
     uint32_t hidden, n_expert;
+    // Q6_K shared expert of a mixed-precision layout (single token): its gate and up rows (2 * ffn rows, the up matrix
+    // right behind the gate matrix) are multiplied here, by workgroups behind the router's, into sh_gu [2 * ffn]
+    const uint8_t *sh_q6k;
+    float *sh_gu;
+    uint32_t ffn;
 };
 
 // fp16 split of x, spread over the whole grid (every workgroup knows the largest |x| of its token)
@@ -197,41 +250,92 @@ __global__ __launch_bounds__(256) void router_f32_kernel(const float *w, RouterA
 template <uint32_t T>
 __global__ __launch_bounds__(256) void router_quant_kernel(const uint8_t *w, RouterArgs a) {
     __shared__ float lds_amax[4];
-    extern __shared__ float xs[];
+    extern __shared__ float xs[];                        // x (padded), then the four raw rows of the workgroup
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63u, H = a.hidden, tok = blockIdx.y;
+    const uint32_t row_bytes = (H / 256u) * Fmt<T>::kBlock;
+    const uint32_t n_router_wg = (a.n_expert + 1u + 3u) / 4u;
+    const bool shared_wg = blockIdx.x >= n_router_wg;                   // only launched when a.sh_q6k is set
+    const uint32_t sh_row_bytes = (H / 256u) * 210u, sh_row0 = 8u * (blockIdx.x - n_router_wg) + 2u * wave;
+    uint8_t *my_row = reinterpret_cast<uint8_t *>(xs + H + H / 32u) + wave * (shared_wg ? 2u * sh_row_bytes : ((row_bytes + 15u) & ~15u));
+    if (shared_wg) wave_stage(my_row, a.sh_q6k + (uint64_t)sh_row0 * sh_row_bytes, 2u * sh_row_bytes, lane);      // the wave's two rows
+    else if (blockIdx.x * 4u + wave < a.n_expert) wave_stage(my_row, w + (uint64_t)(blockIdx.x * 4u + wave) * row_bytes, row_bytes, lane);
     const float *x = a.x + (uint64_t)tok * H;
+    KTS(12);
     float amax = 0.0f;
     for (uint32_t i = threadIdx.x; i < H; i += 256u) { const float v = x[i]; xs[i + (i >> 5)] = v; amax = fmaxf(amax, fabsf(v)); }
     amax = wave_max(amax);
     if (lane == 0u) lds_amax[wave] = amax;
+    KTS(13);
     __syncthreads();
+    KTS(14);
     amax = fmaxf(fmaxf(lds_amax[0], lds_amax[1]), fmaxf(lds_amax[2], lds_amax[3]));
     const uint32_t r = blockIdx.x * 4u + wave;
-    if (r <= a.n_expert) {
+    if (shared_wg) {
+        // 32 lanes per row, every 32nd chunk of 32 columns; the halves of the wave then add up separately
+        const uint8_t *row = my_row + (lane >> 5) * sh_row_bytes;
+        float acc = 0.0f;
+        for (uint32_t c = lane & 31u; c < H / 32u; c += 32u) {
+            float xv[32], sx0 = 0.0f, sx1 = 0.0f;
+#pragma unroll
+            for (int j = 0; j < 32; ++j) { xv[j] = xs[33u * c + j]; if (j < 16) sx0 += xv[j]; else sx1 += xv[j]; }
+            acc += q6k_dot32(row, c, xv, sx0, sx1);
+        }
+        acc += dpp_f32<kDppXor1>(acc);
+        acc += dpp_f32<kDppXor2>(acc);
+        acc += dpp_f32<kDppRor4>(acc);
+        acc += dpp_f32<kDppRor8>(acc);
+        const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(acc), __float_as_uint(acc), false, false);
+        acc = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);           // rows of 16 lanes: 0 + 1 and 2 + 3
+        if ((lane & 31u) == 0u && tok == 0u) a.sh_gu[sh_row0 + (lane >> 5)] = acc;
+    } else if (r <= a.n_expert) {
         float acc = 0.0f;
         if (r < a.n_expert) {
-            const uint8_t *row = w + (uint64_t)r * (H / 256u) * Fmt<T>::kBlock;
             for (uint32_t c = lane; c < H / 32u; c += 64u) {
-                float wv[32];
-                decode32<T>(row, c, wv);
-                float s = 0.0f;
+                if constexpr (T == T_Q6_K) {
+                    float xv[32], sx0 = 0.0f, sx1 = 0.0f;
 #pragma unroll
-                for (int j = 0; j < 32; ++j) s = fmaf(wv[j], xs[33u * c + j], s);
-                acc += s;
+                    for (int j = 0; j < 32; ++j) { xv[j] = xs[33u * c + j]; if (j < 16) sx0 += xv[j]; else sx1 += xv[j]; }
+                    acc += q6k_dot32(my_row, c, xv, sx0, sx1);
+                } else {
+                    float wv[32];
+                    decode32<T>(my_row, c, wv);
+                    float s = 0.0f;
+#pragma unroll
+                    for (int j = 0; j < 32; ++j) s = fmaf(wv[j], xs[33u * c + j], s);
+                    acc += s;
+                }
             }
         } else {
-            for (uint32_t i = lane; i < H; i += 64u) acc = fmaf(a.gate_inp[i], xs[i + (i >> 5)], acc);
+            const float4 *gp = reinterpret_cast<const float4 *>(a.gate_inp);
+            for (uint32_t i0 = 0; i0 < H / 4u; i0 += 256u) {              // four float4 per lane in flight
+                float4 gv[4];
+#pragma unroll
+                for (uint32_t k = 0; k < 4u; ++k) { const uint32_t i = i0 + 64u * k + lane; gv[k] = i < H / 4u ? gp[i] : make_float4(0.0f, 0.0f, 0.0f, 0.0f); }
+#pragma unroll
+                for (uint32_t k = 0; k < 4u; ++k) {
+                    const uint32_t i = 4u * (i0 + 64u * k + lane);
+                    if (i < H) {
+                        const float *xp = xs + i + (i >> 5);
+                        acc = fmaf(gv[k].x, xp[0], acc); acc = fmaf(gv[k].y, xp[1], acc); acc = fmaf(gv[k].z, xp[2], acc); acc = fmaf(gv[k].w, xp[3], acc);
+                    }
+                }
+            }
         }
         acc = wave_sum(acc);
         if (lane == 0u) a.logits[(uint64_t)tok * (a.n_expert + 1u) + r] = acc;
     }
+    KTS(15);
     split_x_job(a, tok, amax);
+    KTS(16);
 }
 
 hipError_t launch_router_gemv(uint32_t router_type, const void *w, const float *x, const float *gate_inp, uint32_t ntok, uint32_t hidden,
-                              uint32_t n_expert, float *logits, void *xh, void *xl, int *xexp, hipStream_t s) {
+                              uint32_t n_expert, float *logits, void *xh, void *xl, int *xexp, const void *sh_q6k, float *sh_gu, uint32_t ffn,
+                              hipStream_t s) {
     if (!ntok || !hidden || hidden % 256u || !n_expert || n_expert > 1024u) return hipErrorInvalidValue;
-    RouterArgs a{x, gate_inp, logits, static_cast<_Float16 *>(xh), static_cast<_Float16 *>(xl), xexp, hidden, n_expert};
+    const bool with_shared = sh_q6k && sh_gu && router_type == T_Q6_K && ntok == 1u && ffn % 4u == 0u;
+    RouterArgs a{x, gate_inp, logits, static_cast<_Float16 *>(xh), static_cast<_Float16 *>(xl), xexp, hidden, n_expert,
+                 with_shared ? static_cast<const uint8_t *>(sh_q6k) : nullptr, sh_gu, ffn};
     const dim3 grid((n_expert + 1u + 3u) / 4u, ntok);
     if (router_type == T_F32) {
         const float *wf = static_cast<const float *>(w);
@@ -243,8 +347,9 @@ hipError_t launch_router_gemv(uint32_t router_type, const void *w, const float *
             default: return hipErrorInvalidValue;
         }
     } else if (router_type == T_Q6_K) {
-        const size_t lds = (size_t)(hidden + hidden / 32u) * sizeof(float);
-        REDHIP_LAUNCH(router_quant_kernel<T_Q6_K>, grid, dim3(256), lds, s, static_cast<const uint8_t *>(w), a);
+        const size_t lds = (size_t)(hidden + hidden / 32u) * sizeof(float) + 8u * (((size_t)(hidden / 256u) * 210u + 15u) & ~(size_t)15u);
+        const dim3 qgrid(grid.x + (with_shared ? 2u * ffn / 8u : 0u), ntok);
+        REDHIP_LAUNCH(router_quant_kernel<T_Q6_K>, qgrid, dim3(256), lds, s, static_cast<const uint8_t *>(w), a);
     } else {
         return hipErrorInvalidValue;
     }
@@ -268,14 +373,6 @@ struct SelectOut {
     uint64_t cand[64];        // candidates: key << 32 | ~index
 };
 
-#ifdef REDHIP_KTS
-__device__ unsigned long long g_kts[256 * 32], g_kts2[256 * 32];
-#define KTS(i) do { if (threadIdx.x == 0u && blockIdx.x < 256u && (i) < 32u) { g_kts[blockIdx.x * 32u + (i)] = wall_clock64(); g_kts2[blockIdx.x * 32u + (i)] = clock64(); } } while (0)
-#define SEL_TS(i) do {} while (0)
-#else
-#define KTS(i) do {} while (0)
-#define SEL_TS(i) do {} while (0)
-#endif
 
 // (float)(1.0 / d) for finite d > 0 without the double division: a float reciprocal refined by two double FMAs is
 // good to 2^-45, which rounds to the same float except in about one case in 2^20
@@ -563,7 +660,10 @@ __device__ __forceinline__ void load_act_operand(half4_t *ax, const _Float16 *hi
 struct GateUpArgs {
     const uint8_t *experts;    // packed experts of the layer, expert e at experts + e * stride
     uint64_t stride;
-    const uint8_t *shared;     // packed shared expert
+    const uint8_t *shared;     // packed shared expert, or nullptr when it is not IQ2_XXS
+    const uint8_t *shared_q6k; // then: its raw Q6_K rows, gate matrix then up matrix
+    const float *x;            // [hidden] f32 activations (Q6_K shared expert only)
+    const float *shared_gu;    // or, instead of the two above: gate . x and up . x of the shared expert, [2 * ffn], already computed
     const float *logits;       // [n_expert + 1] (selection happens here) or nullptr: ids come from `ids_in`
     const uint32_t *ids_in;    // [top_k] when logits == nullptr
     uint32_t *ids_out;         // [top_k]   written by workgroup (0, 0) when selecting
@@ -597,27 +697,95 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_select_kernel(GateUpArgs a
     const uint32_t kc = wave % NKC, q0 = wave / NKC;
     const uint32_t G = 16u * kc + blk;                 // this lane's group inside the gate/up rows
     KTS(0);
+    KTSY(20);
     half4_t ax[8];
     load_act_operand(ax, a.xh + 32u * G, a.xl + 32u * G, j);
     build_tables(lds, tb, grid_entry);
 
     uint32_t expert = 0u;
-    if (a.logits) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t raw_rows[];      // Q6_K shared expert only: the unit's 64 raw rows, then x
+    if (is_shared) {
+        if (!a.shared && !a.shared_gu) {
+            // wave w copies its rows 4 w .. 4 w + 3 of the unit (0..31 gate, 32..63 up; contiguous in their matrix) and a
+            // share of x into LDS with wide loads, requested before anything else happens in this workgroup
+            const uint32_t row_bytes = HB * 210u;
+            const uint8_t *src = a.shared_q6k + (wave < 8u ? 0u : (uint64_t)F * row_bytes) + (uint64_t)(32u * g + 4u * (wave & 7u)) * row_bytes;
+            wave_stage(raw_rows + 4u * wave * row_bytes, src, 4u * row_bytes, lane);
+            float *xs = reinterpret_cast<float *>(raw_rows + 64u * row_bytes), *xsum = xs + H + H / 32u;
+            for (uint32_t i = tid; i < H; i += NW * 64u) xs[i + (i >> 5)] = a.x[i];
+            if (tid < H / 16u) {                             // sums of 16 consecutive activations (the Q6_K offset term)
+                const float4 *xp = reinterpret_cast<const float4 *>(a.x + 16u * tid);
+                const float4 v0 = xp[0], v1 = xp[1], v2 = xp[2], v3 = xp[3];
+                xsum[tid] = (((v0.x + v0.y) + (v0.z + v0.w)) + ((v1.x + v1.y) + (v1.z + v1.w))) + (((v2.x + v2.y) + (v2.z + v2.w)) + ((v3.x + v3.y) + (v3.z + v3.w)));
+            }
+        }
+        __syncthreads();                                   // tables; the shared expert does not depend on the routing
+    } else if (a.logits) {
         if (wave == 0u) {        // the other waves have nothing to do until the expert is known
             if (a.n_expert <= 512u) wave_select_topk<8>(a.logits, a.n_expert, a.top_k, &sel);
             else wave_select_topk<16>(a.logits, a.n_expert, a.top_k, &sel);
         }
         __syncthreads();
-        if (!is_shared) expert = sel.ids[slot];
+        expert = sel.ids[slot];
         if (g == 0u && slot == 0u) {
             if (tid < a.top_k) { a.ids_out[tid] = sel.ids[tid]; a.weights_out[tid] = sel.w[tid]; }
             if (tid == 0u) a.scalar_out[0] = sel.scalar;
         }
     } else {
-        if (!is_shared) expert = a.ids_in[slot];
+        expert = a.ids_in[slot];
         __syncthreads();                               // tables
     }
     KTS(1);
+    if (is_shared && !a.shared && a.shared_gu) {           // the router launch has already multiplied the shared expert's rows
+        if (tid < 32u) {
+            const float gsum = a.shared_gu[32u * g + tid], usum = a.shared_gu[F + 32u * g + tid];
+            const float act = (gsum / (1.0f + expf(-gsum))) * usum;
+            float amax = fabsf(act);
+#pragma unroll
+            for (int o = 16; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+            const int e = prescale_exp(amax);
+            split_hi_lo(act, exp2i(-e), a.act_h + (uint64_t)slot * F + 32u * g + tid, a.act_l + (uint64_t)slot * F + 32u * g + tid);
+            if (tid == 0u) a.act_exp[slot * (F / 32u) + g] = e;
+        }
+        return;
+    }
+    if (is_shared && !a.shared) {
+        // Q6_K shared expert: plain decode and f32 FMAs; wave w takes rows 4 w .. 4 w + 3 of the unit (0..31 gate, 32..63 up),
+        // the 16 lanes of a row take every 16th chunk of 32 columns and meet by row-wide adds
+        KTS(8);
+        const uint32_t urow = 4u * wave + (lane >> 4), row_bytes = HB * 210u;
+        const float *xs = reinterpret_cast<const float *>(raw_rows + 64u * row_bytes), *xsum = xs + H + H / 32u;   // x, one float of padding per 32
+        KTS(9);
+        const uint8_t *rowp = raw_rows + urow * row_bytes;
+        float acc = 0.0f;
+        for (uint32_t c = lane & 15u; c < HG; c += 16u) {
+            float xv[32];
+#pragma unroll
+            for (int i = 0; i < 32; ++i) xv[i] = xs[33u * c + i];
+            acc += q6k_dot32(rowp, c, xv, xsum[2u * c], xsum[2u * c + 1u]);
+        }
+        KTS(10);
+        acc += dpp_f32<kDppXor1>(acc);
+        acc += dpp_f32<kDppXor2>(acc);
+        acc += dpp_f32<kDppRor4>(acc);
+        acc += dpp_f32<kDppRor8>(acc);
+        if ((lane & 15u) < (uint32_t)NKC) part[(lane & 15u) * 64u + urow] = (lane & 15u) == 0u ? acc : 0.0f;
+        __syncthreads();
+        if (tid < 32u) {
+            float gsum = 0.0f, usum = 0.0f;
+#pragma unroll
+            for (int c = 0; c < NKC; ++c) { gsum += part[c * 64 + tid]; usum += part[c * 64 + 32 + tid]; }
+            const float act = (gsum / (1.0f + expf(-gsum))) * usum;
+            float amax = fabsf(act);
+#pragma unroll
+            for (int o = 16; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+            const int e = prescale_exp(amax);
+            split_hi_lo(act, exp2i(-e), a.act_h + (uint64_t)slot * F + 32u * g + tid, a.act_l + (uint64_t)slot * F + 32u * g + tid);
+            if (tid == 0u) a.act_exp[slot * (F / 32u) + g] = e;
+        }
+        KTSY(21);
+        return;
+    }
     const uint8_t *ex = is_shared ? a.shared : a.experts + (uint64_t)expert * a.stride;
     const uint64_t gate_bytes = (uint64_t)F * HG * 8u + (uint64_t)F * HB * 2u;
     const uint2 *gate_qs = reinterpret_cast<const uint2 *>(ex);
@@ -662,6 +830,7 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_select_kernel(GateUpArgs a
         split_hi_lo(act, exp2i(-e), a.act_h + (uint64_t)slot * F + 32u * g + tid, a.act_l + (uint64_t)slot * F + 32u * g + tid);
         if (tid == 0u) a.act_exp[slot * (F / 32u) + g] = e;
     }
+    KTSY(21);
 }
 
 struct DownArgs {
@@ -728,6 +897,110 @@ __global__ __launch_bounds__(kWaves * 64) void down_combine_kernel(DownArgs a) {
         for (uint32_t s = 0; s < a.top_k; ++s) sum = fmaf(a.weights[s] * 0.125f, part[s * 8u + tid], sum);
         sum = fmaf(a.scalar[0] * 0.125f, part[a.top_k * 8u + tid], sum);
         a.out[row0 + tid] = sum;
+    }
+}
+
+// Down + combine when the down matrices are not IQ2_XXS (mixed-precision layouts: IQ3_S routed, Q6_K shared): same
+// work split as down_combine_kernel (8 rows per workgroup, wave = slot, lane = (32-column chunk, row)), weights
+// decoded from the raw GGUF rows and multiplied in f32 against the activation rebuilt from its fp16 halves.
+struct DownRawArgs {
+    const uint8_t *experts;    // expert e's raw down rows at experts + e * stride
+    uint64_t stride;
+    const uint8_t *shared;     // raw down rows of the shared expert
+    const uint32_t *ids;
+    const float *weights, *scalar;
+    const _Float16 *act_h, *act_l;
+    const int *act_exp;
+    float *out;
+    uint32_t hidden, ffn, top_k;
+};
+
+template <uint32_t T>
+__device__ __forceinline__ float chunk_dot(const uint8_t *row, uint32_t chunk, const float *av) {
+    if constexpr (T == T_Q6_K) {
+        float sx0 = 0.0f, sx1 = 0.0f;
+#pragma unroll
+        for (int i = 0; i < 16; ++i) { sx0 += av[i]; sx1 += av[16 + i]; }
+        return q6k_dot32(row, chunk, av, sx0, sx1);
+    }
+    float w[32];
+    decode32<T>(row, chunk, w);
+    float acc = 0.0f;
+#pragma unroll
+    for (int i = 0; i < 32; ++i) acc = fmaf(w[i], av[i], acc);
+    return acc;
+}
+
+template <uint32_t TD, uint32_t TS>
+__global__ __launch_bounds__(kWaves * 64) void down_combine_raw_kernel(DownRawArgs a) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t raw_rows[];     // [slot][8 rows of the slot's matrix]
+    __shared__ float part[17 * 8];
+    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
+    const uint32_t F = a.ffn, FG = F / 32u, FB = F / 256u, n_slot = a.top_k + 1u;
+    const uint32_t row0 = 8u * blockIdx.x;
+    constexpr uint32_t kMaxBlock = Fmt<TD>::kBlock > Fmt<TS>::kBlock ? Fmt<TD>::kBlock : Fmt<TS>::kBlock;
+    if (wave < n_slot) {
+        const bool is_shared = wave == a.top_k;
+        const uint32_t row_bytes = FB * (is_shared ? Fmt<TS>::kBlock : Fmt<TD>::kBlock);
+        const uint8_t *rows = (is_shared ? a.shared : a.experts + (uint64_t)a.ids[wave] * a.stride) + (uint64_t)row0 * row_bytes;
+        uint8_t *mine = raw_rows + wave * 8u * FB * kMaxBlock;
+        wave_stage(mine, rows, 8u * row_bytes, lane);          // 8 rows x FB blocks of 66 / 110 / 210 bytes: a multiple of 16
+        float tot[2] = {0.0f, 0.0f};
+        for (uint32_t G = blk; G < FG; G += 16u) {
+            float av[32];
+            const float sc = exp2i(a.act_exp[wave * FG + G]);
+            const uint4 *ph = reinterpret_cast<const uint4 *>(a.act_h + (uint64_t)wave * F + 32u * G), *pl = reinterpret_cast<const uint4 *>(a.act_l + (uint64_t)wave * F + 32u * G);
+#pragma unroll
+            for (int v = 0; v < 4; ++v) {
+                union { uint4 u; _Float16 h[8]; } hh, ll;
+                hh.u = ph[v];
+                ll.u = pl[v];
+#pragma unroll
+                for (int i = 0; i < 8; ++i) av[8 * v + i] = fmaf((float)ll.h[i], 4.8828125e-4f, (float)hh.h[i]) * sc;
+            }
+            if (G == blk) wave_lds_sync();                       // the staged rows are visible to the whole wave
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                const uint8_t *row = mine + (4u * q + j) * row_bytes;
+                tot[q] += is_shared ? chunk_dot<TS>(row, G, av) : chunk_dot<TD>(row, G, av);
+            }
+        }
+        const float r = quad_column_reduce<2>(tot, lane);
+        if (reduced_writer<2>(lane)) part[wave * 8u + 4u * reduced_unit<2>(lane) + j] = r;
+    }
+    __syncthreads();
+    if (tid < 8u) {
+        float sum = 0.0f;
+        for (uint32_t s = 0; s < a.top_k; ++s) sum = fmaf(a.weights[s], part[s * 8u + tid], sum);
+        sum = fmaf(a.scalar[0], part[a.top_k * 8u + tid], sum);
+        a.out[row0 + tid] = sum;
+    }
+}
+
+template <uint32_t TD>
+static hipError_t launch_down_raw_shared(uint32_t ts, const DownRawArgs &a, hipStream_t s) {
+    const dim3 grid(a.hidden / 8u), block(kWaves * 64);
+    const size_t lds = (size_t)(a.top_k + 1u) * 8u * (a.ffn / 256u) * 210u;       // sized for the largest block type; at most 17 x 8 x 4 x 210 bytes
+    switch (ts) {
+        case T_IQ2_XXS: REDHIP_LAUNCH((down_combine_raw_kernel<TD, T_IQ2_XXS>), grid, block, lds, s, a); break;
+        case T_IQ3_S: REDHIP_LAUNCH((down_combine_raw_kernel<TD, T_IQ3_S>), grid, block, lds, s, a); break;
+        case T_Q6_K: REDHIP_LAUNCH((down_combine_raw_kernel<TD, T_Q6_K>), grid, block, lds, s, a); break;
+        default: return hipErrorInvalidValue;
+    }
+    return hipGetLastError();
+}
+
+hipError_t launch_down_combine_raw(uint32_t down_type, uint32_t shared_down_type, const void *experts, uint64_t stride, const void *shared,
+                                   const uint32_t *ids, const float *weights, const float *scalar, const void *act_h, const void *act_l,
+                                   const int *act_exp, float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, hipStream_t s) {
+    if (!hidden || hidden % 8u || !ffn || ffn % 256u || top_k + 1u > (uint32_t)kWaves) return hipErrorInvalidValue;
+    const DownRawArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(shared), ids, weights, scalar,
+                        static_cast<const _Float16 *>(act_h), static_cast<const _Float16 *>(act_l), act_exp, out, hidden, ffn, top_k};
+    switch (down_type) {
+        case T_IQ2_XXS: return launch_down_raw_shared<T_IQ2_XXS>(shared_down_type, a, s);
+        case T_IQ3_S: return launch_down_raw_shared<T_IQ3_S>(shared_down_type, a, s);
+        case T_Q6_K: return launch_down_raw_shared<T_Q6_K>(shared_down_type, a, s);
+        default: return hipErrorInvalidValue;
     }
 }
 
@@ -1170,22 +1443,35 @@ hipError_t launch_batch_packed(const void *experts, uint64_t stride, const void 
     return hipGetLastError();
 }
 
-hipError_t launch_gateup_select(const void *experts, uint64_t stride, const void *shared, const float *logits, const uint32_t *ids_in,
-                                uint32_t *ids_out, float *weights_out, float *scalar_out, const void *xh, const void *xl, const int *xexp,
-                                void *act_h, void *act_l, int *act_exp, uint32_t hidden, uint32_t ffn, uint32_t n_expert, uint32_t top_k,
-                                hipStream_t s) {
-    if (!fused_iq2_supported(hidden, ffn)) return hipErrorInvalidValue;
-    GateUpArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(shared), logits, ids_in, ids_out, weights_out,
-                 scalar_out, static_cast<const _Float16 *>(xh), static_cast<const _Float16 *>(xl), xexp, static_cast<_Float16 *>(act_h),
-                 static_cast<_Float16 *>(act_l), act_exp, hidden, ffn, n_expert, top_k};
+hipError_t launch_gateup_select(const void *experts, uint64_t stride, const void *shared, const void *shared_q6k, const float *x,
+                                const float *shared_gu, const float *logits, const uint32_t *ids_in, uint32_t *ids_out, float *weights_out,
+                                float *scalar_out, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l, int *act_exp,
+                                uint32_t hidden, uint32_t ffn, uint32_t n_expert, uint32_t top_k, hipStream_t s) {
+    if (!fused_iq2_supported(hidden, ffn) || (!shared && !shared_gu && (!shared_q6k || !x))) return hipErrorInvalidValue;
+    GateUpArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(shared), static_cast<const uint8_t *>(shared_q6k), x,
+                 shared_gu, logits, ids_in, ids_out, weights_out, scalar_out, static_cast<const _Float16 *>(xh), static_cast<const _Float16 *>(xl),
+                 xexp, static_cast<_Float16 *>(act_h), static_cast<_Float16 *>(act_l), act_exp, hidden, ffn, n_expert, top_k};
     const dim3 grid(ffn / 32u, top_k + 1u);
+    const size_t dyn = shared || shared_gu ? 0u : (size_t)64u * (hidden / 256u) * 210u + (size_t)(hidden + hidden / 32u + hidden / 16u) * 4u;   // raw Q6_K rows of one unit of the shared expert, x, sums of 16 x
+#define REDHIP_GUS(NKC)                                                                                                                \
+    do {                                                                                                                               \
+        static bool attr = false;                                                                                                       \
+        if (dyn && !attr) {                                                                                                             \
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gateup_select_kernel<NKC>), hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024); \
+            if (e != hipSuccess) return e;                                                                                              \
+            attr = true;                                                                                                                \
+        }                                                                                                                               \
+        REDHIP_LAUNCH(gateup_select_kernel<NKC>, grid, dim3(kWaves * 64), dyn, s, a);                                                   \
+    } while (0)
+    if (dyn > 144u * 1024u) return hipErrorInvalidValue;
     switch (hidden / 512u) {
-        case 1: REDHIP_LAUNCH(gateup_select_kernel<1>, grid, dim3(kWaves * 64), 0, s, a); break;
-        case 2: REDHIP_LAUNCH(gateup_select_kernel<2>, grid, dim3(kWaves * 64), 0, s, a); break;
-        case 4: REDHIP_LAUNCH(gateup_select_kernel<4>, grid, dim3(kWaves * 64), 0, s, a); break;
-        case 8: REDHIP_LAUNCH(gateup_select_kernel<8>, grid, dim3(kWaves * 64), 0, s, a); break;
+        case 1: REDHIP_GUS(1); break;
+        case 2: REDHIP_GUS(2); break;
+        case 4: REDHIP_GUS(4); break;
+        case 8: REDHIP_GUS(8); break;
         default: return hipErrorInvalidValue;
     }
+#undef REDHIP_GUS
     return hipGetLastError();
 }
 

@@ -117,7 +117,8 @@ hipError_t launch_dequant_packed_iq2xxs(const void *packed, uint32_t nrows, uint
 
 // logits [ntok][n_expert + 1] (entry n_expert = gate_inp . x) and the fp16 split of x: xh, xl [ntok][hidden], xexp [ntok]
 hipError_t launch_router_gemv(uint32_t router_type, const void *w, const float *x, const float *gate_inp, uint32_t ntok, uint32_t hidden,
-                              uint32_t n_expert, float *logits, void *xh, void *xl, int *xexp, hipStream_t s);
+                              uint32_t n_expert, float *logits, void *xh, void *xl, int *xexp, const void *sh_q6k, float *sh_gu, uint32_t ffn,
+                              hipStream_t s);
 // softmax top-k of logits [ntok][n_expert + 1]; scalar[t] = sigmoid(logits[t][n_expert]); optional probs [ntok][n_expert]
 hipError_t launch_select(const float *logits, uint32_t ntok, uint32_t n_expert, uint32_t top_k, uint32_t *ids, float *weights, float *scalar,
                          float *probs, hipStream_t s);
@@ -137,10 +138,14 @@ hipError_t launch_batch_packed(const void *experts, uint64_t stride, const void 
 
 // single token: act[slot] = SwiGLU(gate . x, up . x) as fp16 halves with one exponent per 32 values. With `logits` the
 // kernel selects the experts itself (and writes ids / weights / scalar); with logits == nullptr it takes ids_in.
-hipError_t launch_gateup_select(const void *experts, uint64_t stride, const void *shared, const float *logits, const uint32_t *ids_in,
-                                uint32_t *ids_out, float *weights_out, float *scalar_out, const void *xh, const void *xl, const int *xexp,
-                                void *act_h, void *act_l, int *act_exp, uint32_t hidden, uint32_t ffn, uint32_t n_expert, uint32_t top_k,
-                                hipStream_t s);
+hipError_t launch_gateup_select(const void *experts, uint64_t stride, const void *shared, const void *shared_q6k, const float *x,
+                                const float *shared_gu, const float *logits, const uint32_t *ids_in, uint32_t *ids_out, float *weights_out,
+                                float *scalar_out, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l, int *act_exp,
+                                uint32_t hidden, uint32_t ffn, uint32_t n_expert, uint32_t top_k, hipStream_t s);
+// down + weighted combine for layouts whose down matrices are raw GGUF rows of any supported type
+hipError_t launch_down_combine_raw(uint32_t down_type, uint32_t shared_down_type, const void *experts, uint64_t stride, const void *shared,
+                                   const uint32_t *ids, const float *weights, const float *scalar, const void *act_h, const void *act_l,
+                                   const int *act_exp, float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, hipStream_t s);
 // single token: out[r] = sum_k weights[k] * down_{ids[k]}[r] . act[k] + scalar * shared_down[r] . act[top_k], k in order
 hipError_t launch_down_combine(const void *experts, uint64_t stride, const void *shared, const uint32_t *ids, const float *weights,
                                const float *scalar, const void *act_h, const void *act_l, const int *act_exp, float *out,

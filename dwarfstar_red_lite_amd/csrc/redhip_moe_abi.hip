@@ -50,10 +50,16 @@ struct Moe {
     uint8_t *ws = nullptr;
     // single-token fused path (all matrices IQ2_XXS, shapes the fused kernel tiles)
     bool fused = false;
+    // mixed-precision layouts (gate/up IQ2_XXS, other matrices of other types): the routed gate/up matrices are packed
+    // for the MFMA gate/up kernel, the down matrices stay raw GGUF rows; one token at a time
+    bool mixed = false;
+    uint64_t packed_stride = 0;              // bytes between experts in `packed`
+    bool packed_gu() const { return fused || mixed; }
     void *xh = nullptr, *xl = nullptr;       // fp16 [hidden] each
     int *xexp = nullptr;
     bool select_and_group = false;           // forward() of a small batch: one launch selects and sorts the pairs
     bool skip_select = false;                // forward(): the gate/up kernel selects, route() skips its own selection
+    bool shared_gu_ready = false;            // the router launch of this forward() has left the shared expert's gate / up products in `act`
     // batched path (ntok > 1): pairs grouped by expert
     uint32_t *uid = nullptr, *expert_start = nullptr, *pair_token = nullptr, *tok_pair = nullptr, *n_unique = nullptr;
     uint32_t *tile_group = nullptr, *tile_pair0 = nullptr, *tile_n = nullptr, *n_tiles = nullptr;      // prefill tiles
@@ -66,7 +72,7 @@ struct Moe {
         return fused && ntok >= 2u && ntok <= 8u && ntok * cfg.top_k <= 128u && ntok * (cfg.top_k + 1u) <= 144u && cfg.hidden / 512u <= 4u;
     }
     // every batch size runs on the packed layout when the layer has one (decode kernel, small-batch kernels, prefill tiles)
-    bool packed_path(uint32_t ntok) const { return fused && (ntok == 1u || small_batch(ntok) || cfg.hidden / 512u <= 4u); }
+    bool packed_path(uint32_t ntok) const { return (fused && (ntok == 1u || small_batch(ntok) || cfg.hidden / 512u <= 4u)) || (mixed && ntok == 1u); }
     ExpertSet routed(uint32_t l) const { return ExpertSet{layers[l].experts, expert_stride, gate_bytes, gate_bytes, gu_type, dn_type}; }
     ExpertSet shared(uint32_t l) const { return ExpertSet{layers[l].shared, 0, sh_gate_bytes, sh_gate_bytes, sh_gu_type, sh_dn_type}; }
 };
@@ -134,15 +140,21 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
         prof_set_stage(ST_OTHER);
         return 1;
     }
-    if (m->fused) {          // xh / xl / scalar come from the router kernel or the prep kernel
+    if (m->packed_gu()) {    // xh / xl / scalar come from the router kernel or the prep kernel
         const Layer &L = m->layers[layer];
         prof_set_stage(ST_GATEUP);
-        HIP_OK(launch_gateup_select(L.packed, m->expert_stride, L.shared_packed, select_here ? m->logits : nullptr, ids, m->ids, m->weights,
-                                    m->scalar, m->xh, m->xl, m->xexp, m->act_h, m->act_l, m->act_exp, c.hidden, c.ffn, c.n_expert, c.top_k, s),
-               "gate/up launch");
+        HIP_OK(launch_gateup_select(L.packed, m->packed_stride, L.shared_packed, L.shared, x, select_here && m->shared_gu_ready ? m->act : nullptr,
+                                    select_here ? m->logits : nullptr, ids, m->ids,
+                                    m->weights, m->scalar, m->xh, m->xl, m->xexp, m->act_h, m->act_l, m->act_exp, c.hidden, c.ffn, c.n_expert,
+                                    c.top_k, s), "gate/up launch");
         prof_set_stage(ST_DOWN_COMBINE);
-        HIP_OK(launch_down_combine(L.packed, m->expert_stride, L.shared_packed, select_here ? m->ids : ids, select_here ? m->weights : weights,
-                                   m->scalar, m->act_h, m->act_l, m->act_exp, out, c.hidden, c.ffn, c.top_k, s), "down/combine launch");
+        if (m->fused)
+            HIP_OK(launch_down_combine(L.packed, m->expert_stride, L.shared_packed, select_here ? m->ids : ids, select_here ? m->weights : weights,
+                                       m->scalar, m->act_h, m->act_l, m->act_exp, out, c.hidden, c.ffn, c.top_k, s), "down/combine launch");
+        else
+            HIP_OK(launch_down_combine_raw(m->dn_type, m->sh_dn_type, L.experts + 2u * m->gate_bytes, m->expert_stride, L.shared + 2u * m->sh_gate_bytes,
+                                           select_here ? m->ids : ids, select_here ? m->weights : weights, m->scalar, m->act_h, m->act_l,
+                                           m->act_exp, out, c.hidden, c.ffn, c.top_k, s), "down/combine launch");
         prof_set_stage(ST_OTHER);
         return 1;
     }
@@ -193,6 +205,10 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
     m->router_bytes = (uint64_t)c.n_expert * row_bytes(c.router_type, c.hidden);
     m->layers.resize(c.n_layer);
     m->fused = gu == T_IQ2_XXS && dn == T_IQ2_XXS && sgu == T_IQ2_XXS && sdn == T_IQ2_XXS && fused_iq2_supported(c.hidden, c.ffn);
+    // (the raw-row down kernel stages 8 rows per slot in LDS: keep that within the default 64 KB)
+    m->mixed = !m->fused && gu == T_IQ2_XXS && (sgu == T_IQ2_XXS || sgu == T_Q6_K) && fused_iq2_supported(c.hidden, c.ffn) &&
+               (size_t)(c.top_k + 1u) * 8u * (c.ffn / 256u) * 210u <= 64u * 1024u && (sgu != T_Q6_K || (size_t)64u * (c.hidden / 256u) * 210u + (size_t)(c.hidden + c.hidden / 32u + c.hidden / 16u) * 4u <= 144u * 1024u);
+    m->packed_stride = m->fused ? m->expert_stride : align256(2u * m->gate_bytes);
     bool ok = true;
     for (uint32_t l = 0; l < c.n_layer && ok; ++l) {
         Layer &L = m->layers[l];
@@ -205,10 +221,11 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
         L.shared = p + align256(m->router_bytes);
         L.gate_inp = reinterpret_cast<float *>(L.shared + align256(2u * m->sh_gate_bytes + m->sh_down_bytes));
         m->resident += small + (uint64_t)c.n_expert * m->expert_stride;
-        if (m->fused) {
-            ok = hipMalloc(reinterpret_cast<void **>(&L.packed), (size_t)c.n_expert * m->expert_stride) == hipSuccess &&
-                 hipMalloc(reinterpret_cast<void **>(&L.shared_packed), align256(2u * m->sh_gate_bytes + m->sh_down_bytes)) == hipSuccess;
-            m->resident += (uint64_t)c.n_expert * m->expert_stride + align256(2u * m->sh_gate_bytes + m->sh_down_bytes);
+        if (m->packed_gu()) {
+            const bool sh_packed = m->sh_gu_type == T_IQ2_XXS;       // otherwise the shared expert is read from its raw rows
+            ok = hipMalloc(reinterpret_cast<void **>(&L.packed), (size_t)c.n_expert * m->packed_stride) == hipSuccess &&
+                 (!sh_packed || hipMalloc(reinterpret_cast<void **>(&L.shared_packed), align256(2u * m->sh_gate_bytes + m->sh_down_bytes)) == hipSuccess);
+            m->resident += (uint64_t)c.n_expert * m->packed_stride + (sh_packed ? align256(2u * m->sh_gate_bytes + m->sh_down_bytes) : 0u);
         }
     }
     const size_t T = c.max_tokens;
@@ -302,10 +319,11 @@ int redhip_moe_load_shared(redhip_moe_t h, uint32_t layer, const float *gate_inp
     HIP_OK(hipMemcpy(L.shared, gate, (size_t)gate_bytes, hipMemcpyDefault), "shared gate upload");
     HIP_OK(hipMemcpy(L.shared + gate_bytes, up, (size_t)up_bytes, hipMemcpyDefault), "shared up upload");
     HIP_OK(hipMemcpy(L.shared + 2u * gate_bytes, down, (size_t)down_bytes, hipMemcpyDefault), "shared down upload");
-    if (m->fused) {
+    if (L.shared_packed) {
         const redhip_moe_config &c = m->cfg;
         HIP_OK(launch_repack_iq2xxs(L.shared, gate_bytes, 2u, c.ffn, c.hidden, false, L.shared_packed, gate_bytes, nullptr), "shared gate/up repack");
-        HIP_OK(launch_repack_iq2xxs(L.shared + 2u * gate_bytes, 0u, 1u, c.hidden, c.ffn, false, L.shared_packed + 2u * gate_bytes, 0u, nullptr), "shared down repack");
+        if (m->fused)
+            HIP_OK(launch_repack_iq2xxs(L.shared + 2u * gate_bytes, 0u, 1u, c.hidden, c.ffn, false, L.shared_packed + 2u * gate_bytes, 0u, nullptr), "shared down repack");
         HIP_OK(hipStreamSynchronize(nullptr), "shared repack");
     }
     return 1;
@@ -323,12 +341,13 @@ int redhip_moe_load_experts(redhip_moe_t h, uint32_t layer, uint32_t first, uint
     HIP_OK(hipMemcpy2D(dst, m->expert_stride, gate, m->gate_bytes, m->gate_bytes, count, hipMemcpyDefault), "expert gate upload");
     HIP_OK(hipMemcpy2D(dst + m->gate_bytes, m->expert_stride, up, m->gate_bytes, m->gate_bytes, count, hipMemcpyDefault), "expert up upload");
     HIP_OK(hipMemcpy2D(dst + 2u * m->gate_bytes, m->expert_stride, down, m->down_bytes, m->down_bytes, count, hipMemcpyDefault), "expert down upload");
-    if (m->fused) {
+    if (m->packed_gu()) {
         const redhip_moe_config &c = m->cfg;
-        uint8_t *pk = m->layers[layer].packed + (uint64_t)first * m->expert_stride;
-        HIP_OK(launch_repack_iq2xxs(dst, m->expert_stride, count, c.ffn, c.hidden, false, pk, m->expert_stride, nullptr), "expert gate repack");
-        HIP_OK(launch_repack_iq2xxs(dst + m->gate_bytes, m->expert_stride, count, c.ffn, c.hidden, false, pk + m->gate_bytes, m->expert_stride, nullptr), "expert up repack");
-        HIP_OK(launch_repack_iq2xxs(dst + 2u * m->gate_bytes, m->expert_stride, count, c.hidden, c.ffn, false, pk + 2u * m->gate_bytes, m->expert_stride, nullptr), "expert down repack");
+        uint8_t *pk = m->layers[layer].packed + (uint64_t)first * m->packed_stride;
+        HIP_OK(launch_repack_iq2xxs(dst, m->expert_stride, count, c.ffn, c.hidden, false, pk, m->packed_stride, nullptr), "expert gate repack");
+        HIP_OK(launch_repack_iq2xxs(dst + m->gate_bytes, m->expert_stride, count, c.ffn, c.hidden, false, pk + m->gate_bytes, m->packed_stride, nullptr), "expert up repack");
+        if (m->fused)
+            HIP_OK(launch_repack_iq2xxs(dst + 2u * m->gate_bytes, m->expert_stride, count, c.hidden, c.ffn, false, pk + 2u * m->gate_bytes, m->packed_stride, nullptr), "expert down repack");
         HIP_OK(hipStreamSynchronize(nullptr), "expert repack");
     }
     return 1;
@@ -342,10 +361,13 @@ int redhip_moe_route(redhip_moe_t h, uint32_t layer, const float *x_dev, uint32_
     if (!x_dev || !ntok || ntok > c.max_tokens) { moe_err("invalid token count %u (max %u)", ntok, c.max_tokens); return 0; }
     hipStream_t s = static_cast<hipStream_t>(stream);
     float *lg = logits_dev ? logits_dev : m->logits;
-    if (m->fused) {
+    if (m->packed_gu()) {
         prof_set_stage(ST_ROUTER_GEMV);
+        // a Q6_K shared expert of a mixed layout rides along: its gate / up products land in m->act (otherwise unused on this path)
+        m->shared_gu_ready = m->mixed && m->sh_gu_type == T_Q6_K && c.router_type == T_Q6_K && ntok == 1u && c.top_k >= 2u;
         HIP_OK(launch_router_gemv(c.router_type, m->layers[layer].router, x_dev, m->layers[layer].gate_inp, ntok, c.hidden, c.n_expert,
-                                  m->logits, m->xh, m->xl, m->xexp, s), "router launch");
+                                  m->logits, m->xh, m->xl, m->xexp, m->shared_gu_ready ? m->layers[layer].shared : nullptr, m->act, c.ffn, s),
+               "router launch");
         if (m->select_and_group) {
             prof_set_stage(ST_ROUTE_SELECT);
             HIP_OK(launch_select_group(m->logits, ntok, c.n_expert, c.top_k, m->ids, m->weights, m->scalar, m->uid, m->expert_start,
@@ -391,7 +413,7 @@ int redhip_moe_forward(redhip_moe_t h, uint32_t layer, const float *x_dev, uint3
     Moe *m = moe_of(h);
     if (!check_layer(m, layer)) return 0;
     if (!x_dev || !out_dev) { moe_err("null activation pointer"); return 0; }
-    const bool select_in_gateup = m->fused && ntok == 1u;
+    const bool select_in_gateup = m->packed_gu() && ntok == 1u;
     const bool group_in_select = m->small_batch(ntok);
     m->skip_select = select_in_gateup;
     m->select_and_group = group_in_select;
@@ -410,7 +432,7 @@ int redhip_moe_last_route(redhip_moe_t h, uint32_t ntok, uint32_t *ids, float *w
     if (ids) HIP_OK(hipMemcpy(ids, m->ids, (size_t)ntok * c.top_k * 4u, hipMemcpyDeviceToHost), "ids download");
     if (weights) HIP_OK(hipMemcpy(weights, m->weights, (size_t)ntok * c.top_k * 4u, hipMemcpyDeviceToHost), "weights download");
     if (logits) {
-        const size_t pitch = 4u * (size_t)(c.n_expert + (m->fused ? 1u : 0u));
+        const size_t pitch = 4u * (size_t)(c.n_expert + (m->packed_gu() ? 1u : 0u));
         HIP_OK(hipMemcpy2D(logits, 4u * (size_t)c.n_expert, m->logits, pitch, 4u * (size_t)c.n_expert, ntok, hipMemcpyDeviceToHost), "logits download");
     }
     return 1;
@@ -446,8 +468,8 @@ int redhip_moe_dequant_resident(redhip_moe_t h, uint32_t layer, uint32_t expert,
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (which == 3u) { HIP_OK(launch_dequant_rows(c.router_type, L.router, c.n_expert, c.hidden, out_dev, s), "router dequant"); return 1; }
     const bool sh = expert == c.n_expert;
-    if (m->fused) {        // the layout the fused kernel reads
-        const uint8_t *pk = sh ? L.shared_packed : L.packed + (uint64_t)expert * m->expert_stride;
+    if (m->fused || (m->mixed && which < 2u && (!sh || L.shared_packed))) {        // the layout the MFMA kernels read
+        const uint8_t *pk = sh ? L.shared_packed : L.packed + (uint64_t)expert * m->packed_stride;
         const uint64_t gbytes = m->gate_bytes;
         if (which < 2u) HIP_OK(launch_dequant_packed_iq2xxs(pk + which * gbytes, c.ffn, c.hidden, false, out_dev, s), "packed gate/up dequant");
         else HIP_OK(launch_dequant_packed_iq2xxs(pk + 2u * gbytes, c.hidden, c.ffn, false, out_dev, s), "packed down dequant");
