@@ -22,7 +22,9 @@ for p in (ROOT, os.path.join(ROOT, "oracle")):
     if p not in sys.path:
         sys.path.insert(0, p)
 
+CAL_BYTES = 256 << 20
 HBM_PEAK_GBS = 8000.0
+MFMA_F16_PEAK_TFLOPS = 2500.0
 
 
 def parse():
@@ -36,6 +38,7 @@ def parse():
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-parity", action="store_true", help="kernel experiments only: do not stop when the parity gate fails")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
+    ap.add_argument("--calibrate", action="store_true", help="also run the plain copy kernel of known size (for rocprofv3 --pmc runs)")
     return ap.parse_args()
 
 
@@ -183,6 +186,12 @@ def main():
             step(W + i)
             ids, _, _ = moe.last_route(B)
             distinct.append(len(set(ids.ravel().tolist())))
+    if args.calibrate:         # yardstick for FETCH_SIZE / WRITE_SIZE: copies of exactly CAL_BYTES in, CAL_BYTES out
+        cal_src = torch.empty(CAL_BYTES, dtype=torch.uint8, device="cuda").random_(0, 256)
+        cal_dst = torch.empty_like(cal_src)
+        for _ in range(4):
+            assert lib.redhip_calibration_copy(cal_dst.data_ptr(), cal_src.data_ptr(), CAL_BYTES, None)
+        torch.cuda.synchronize()
     stages = {lib.redhip_profile_stage_name(s).decode(): {"ms_total": stage_ms[s], "launches": int(stage_n[s]),
                                                         "us_avg": 1e3 * stage_ms[s] / stage_n[s]}
               for s in range(n_stage) if stage_n[s]}
@@ -210,11 +219,30 @@ def main():
     }
     dom_bytes = per_launch.get(dom)
     dom_us = stages[dom]["us_avg"] * (stages[dom]["launches"] / K)        # per step, if launched more than once per step
+    # HBM bytes per launch of the dominant kernel, from the rocprofv3 --pmc FETCH_SIZE / WRITE_SIZE runs recorded under
+    # profiles/ (counters cannot be collected from inside this process); null for workloads that were not profiled
+    traffic = None
+    try:
+        with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as fh:
+            rec = json.load(fh).get("%s_b%d" % (args.layout, B), {}).get("stages", {}).get(dom)
+        if rec:
+            traffic = int(rec["fetch_bytes"] + rec["write_bytes"])
+    except (OSError, ValueError, KeyError):
+        traffic = None
     roofline = None
-    if dom_bytes:
+    if dom in ("prefill_gateup", "prefill_down"):
+        # prefill tiles run on the MFMA units: algorithmic flops of the stage (2 per multiply-add, every (token, expert) pair
+        # and every token's shared expert once; the fp16 hi/lo split that doubles the issued MFMAs is not counted)
+        pairs = B * (cfg["top_k"] + 1)
+        flops = pairs * 2.0 * H * F * (2 if dom == "prefill_gateup" else 1)
+        achieved = flops / (dom_us * 1e-6) / 1e12
+        roofline = {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 2), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                    "frac": round(achieved / MFMA_F16_PEAK_TFLOPS, 4), "traffic": traffic, "flops_per_launch": int(flops),
+                    "launch_us": round(dom_us, 3)}
+    elif dom_bytes:
         achieved = dom_bytes / (dom_us * 1e-6) / 1e9
         roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                    "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": None,
+                    "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
                     "bytes_per_launch": int(dom_bytes), "launch_us": round(dom_us, 3)}
 
     us_per_token = ms_per_step * 1e3 / B

@@ -67,6 +67,7 @@ ABI = {
     "redhip_profile_stage_name": (C.c_char_p, [u32]),
     "redhip_profile_begin": (i32, []),
     "redhip_profile_end": (i32, [C.POINTER(dbl), C.POINTER(u32), u32]),
+    "redhip_calibration_copy": (i32, [vp, vp, u64, vp]),
 }
 
 _lib = None

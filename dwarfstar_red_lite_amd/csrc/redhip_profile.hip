@@ -46,6 +46,13 @@ void prof_events(hipEvent_t *start, hipEvent_t *stop) {
 
 using namespace redhip;
 
+namespace redhip {
+// plain copy of known size: the yardstick for memory-traffic counters
+__global__ __launch_bounds__(256) void calibration_copy_kernel(uint4 *dst, const uint4 *src, uint64_t n16) {
+    for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (uint64_t)gridDim.x * blockDim.x) dst[i] = src[i];
+}
+}  // namespace redhip
+
 extern "C" {
 
 uint32_t redhip_profile_stage_count(void) { return ST_COUNT; }
@@ -79,6 +86,14 @@ int redhip_profile_end(double *stage_ms, uint32_t *stage_launches, uint32_t n_st
     g_prof.recs.clear();
     g_prof.next = 0;
     return ok;
+}
+
+int redhip_calibration_copy(void *dst_dev, const void *src_dev, uint64_t bytes, void *stream) {
+    if (!dst_dev || !src_dev || !bytes || bytes % 16u) return 0;
+    redhip::prof_set_stage(redhip::ST_OTHER);
+    REDHIP_LAUNCH(redhip::calibration_copy_kernel, dim3(2048), dim3(256), 0, static_cast<hipStream_t>(stream), static_cast<uint4 *>(dst_dev),
+                  static_cast<const uint4 *>(src_dev), bytes / 16u);
+    return hipGetLastError() == hipSuccess;
 }
 
 }  // extern "C"

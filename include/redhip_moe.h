@@ -91,6 +91,10 @@ uint32_t redhip_profile_stage_count(void);
 const char *redhip_profile_stage_name(uint32_t stage);
 int redhip_profile_begin(void);
 int redhip_profile_end(double *stage_ms, uint32_t *stage_launches, uint32_t n_stage);
+/* Counter calibration (no counterpart in the reference): one plain copy kernel, dst_dev[i] = src_dev[i] for
+ * `bytes` bytes (a multiple of 16), reading and writing exactly that much. Memory-traffic counters collected for
+ * the kernels above are scaled by what they read for this kernel of known size. */
+int redhip_calibration_copy(void *dst_dev, const void *src_dev, uint64_t bytes, void *stream);
 
 #ifdef __cplusplus
 }
