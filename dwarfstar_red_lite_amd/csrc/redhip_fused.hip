@@ -22,16 +22,6 @@
 
 namespace redhip {
 
-#ifdef REDHIP_KTS
-__device__ unsigned long long g_kts[256 * 32], g_kts2[256 * 32];
-#define KTS(i) do { if (threadIdx.x == 0u && blockIdx.x < 256u && (i) < 32u) { g_kts[blockIdx.x * 32u + (i)] = wall_clock64(); g_kts2[blockIdx.x * 32u + (i)] = clock64(); } } while (0)
-#define SEL_TS(i) do {} while (0)
-#define KTSY(i) do { const uint32_t wg_ = blockIdx.x + gridDim.x * blockIdx.y; if (threadIdx.x == 0u && wg_ < 256u) { g_kts[wg_ * 32u + (i)] = wall_clock64(); } } while (0)
-#else
-#define KTSY(i) do {} while (0)
-#define KTS(i) do {} while (0)
-#define SEL_TS(i) do {} while (0)
-#endif
 
 
 // ---------------------------------------------------------------- repacking (upload time)
@@ -260,14 +250,11 @@ __global__ __launch_bounds__(256) void router_quant_kernel(const uint8_t *w, Rou
     if (shared_wg) wave_stage(my_row, a.sh_q6k + (uint64_t)sh_row0 * sh_row_bytes, 2u * sh_row_bytes, lane);      // the wave's two rows
     else if (blockIdx.x * 4u + wave < a.n_expert) wave_stage(my_row, w + (uint64_t)(blockIdx.x * 4u + wave) * row_bytes, row_bytes, lane);
     const float *x = a.x + (uint64_t)tok * H;
-    KTS(12);
     float amax = 0.0f;
     for (uint32_t i = threadIdx.x; i < H; i += 256u) { const float v = x[i]; xs[i + (i >> 5)] = v; amax = fmaxf(amax, fabsf(v)); }
     amax = wave_max(amax);
     if (lane == 0u) lds_amax[wave] = amax;
-    KTS(13);
     __syncthreads();
-    KTS(14);
     amax = fmaxf(fmaxf(lds_amax[0], lds_amax[1]), fmaxf(lds_amax[2], lds_amax[3]));
     const uint32_t r = blockIdx.x * 4u + wave;
     if (shared_wg) {
@@ -324,9 +311,7 @@ __global__ __launch_bounds__(256) void router_quant_kernel(const uint8_t *w, Rou
         acc = wave_sum(acc);
         if (lane == 0u) a.logits[(uint64_t)tok * (a.n_expert + 1u) + r] = acc;
     }
-    KTS(15);
     split_x_job(a, tok, amax);
-    KTS(16);
 }
 
 hipError_t launch_router_gemv(uint32_t router_type, const void *w, const float *x, const float *gate_inp, uint32_t ntok, uint32_t hidden,
@@ -385,7 +370,6 @@ __device__ __forceinline__ float reciprocal_as_float(double d) {
 template <int PER>
 __device__ __forceinline__ void wave_select_topk(const float *logits, uint32_t E, uint32_t K, SelectOut *out, float *probs = nullptr) {
     const uint32_t lane = threadIdx.x & 63u;
-    SEL_TS(0);
     float l[PER];
     float m = -INFINITY;
 #pragma unroll
@@ -396,7 +380,6 @@ __device__ __forceinline__ void wave_select_topk(const float *logits, uint32_t E
     }
     const float gate_logit = logits[E];                      // shared expert's gate logit rides along
     m = wave_max(m);
-    SEL_TS(1);
     float p[PER];
     double part = 0.0;
 #pragma unroll
@@ -404,11 +387,9 @@ __device__ __forceinline__ void wave_select_topk(const float *logits, uint32_t E
         p[s] = lane + 64u * s < E ? expf(l[s] - m) : 0.0f;
         part += (double)p[s];
     }
-    SEL_TS(2);
     const double denom = wave_sum_d(part);
     const bool bad = !(denom > 0.0) || isinf(denom) || isnan(denom);
     const float inv = bad ? 0.0f : reciprocal_as_float(denom);
-    SEL_TS(3);
     uint32_t key[PER];
 #pragma unroll
     for (int s = 0; s < PER; ++s) {
@@ -416,7 +397,6 @@ __device__ __forceinline__ void wave_select_topk(const float *logits, uint32_t E
         key[s] = lane + 64u * s < E ? (__float_as_uint(p[s]) | 0x80000000u) : 0u;   // valid keys have the top bit set: padding never counts
         if (probs && lane + 64u * s < E) probs[lane + 64u * s] = p[s];
     }
-    SEL_TS(4);
     // Level 1: the K-th largest of the 64 per-lane maxima (tau) is a lower bound of the K-th largest key, so the
     // winners are among the keys >= tau - usually a dozen of them. Bisection on one value per lane is cheap.
     uint32_t lm = key[0];
@@ -431,11 +411,9 @@ __device__ __forceinline__ void wave_select_topk(const float *logits, uint32_t E
         const uint32_t n1 = wave_count(lm >= c1), n2 = wave_count(lm >= c2), n3 = wave_count(lm >= c3);
         tau = n3 >= K ? c3 : n2 >= K ? c2 : n1 >= K ? c1 : tau;
     }
-    SEL_TS(5);
     uint32_t n_c = 0u;
 #pragma unroll
     for (int s = 0; s < PER; ++s) n_c += wave_count(key[s] >= tau);
-    SEL_TS(6);
     uint32_t mine = 0xffffffffu, kmine = 0u, rank = 0u;
     if (n_c <= 64u) {
         // Level 2: candidates to LDS in index order, one per lane, ranked against each other with lane broadcasts:
@@ -506,7 +484,6 @@ __device__ __forceinline__ void wave_select_topk(const float *logits, uint32_t E
         }
         if (lane >= K) rank = 0xffffffffu;
     }
-    SEL_TS(7);
     const bool selected = rank < K;
     const float pm = __uint_as_float(kmine & 0x7fffffffu);
     const double sum = wave_sum_d(selected ? (double)pm : 0.0);
@@ -517,7 +494,6 @@ __device__ __forceinline__ void wave_select_topk(const float *logits, uint32_t E
         out->w[rank] = pm * invs;
     }
     if (lane == 0u) out->scalar = 1.0f / (1.0f + expf(-gate_logit));
-    SEL_TS(8);
 }
 
 // stand-alone selection (one wave per token): ids / weights [ntok][top_k], scalar [ntok]
@@ -696,8 +672,6 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_select_kernel(GateUpArgs a
     // activation operand: independent of the routing, requested before the selection
     const uint32_t kc = wave % NKC, q0 = wave / NKC;
     const uint32_t G = 16u * kc + blk;                 // this lane's group inside the gate/up rows
-    KTS(0);
-    KTSY(20);
     half4_t ax[8];
     load_act_operand(ax, a.xh + 32u * G, a.xl + 32u * G, j);
     build_tables(lds, tb, grid_entry);
@@ -735,7 +709,6 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_select_kernel(GateUpArgs a
         expert = a.ids_in[slot];
         __syncthreads();                               // tables
     }
-    KTS(1);
     if (is_shared && !a.shared && a.shared_gu) {           // the router launch has already multiplied the shared expert's rows
         if (tid < 32u) {
             const float gsum = a.shared_gu[32u * g + tid], usum = a.shared_gu[F + 32u * g + tid];
@@ -752,10 +725,8 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_select_kernel(GateUpArgs a
     if (is_shared && !a.shared) {
         // Q6_K shared expert: plain decode and f32 FMAs; wave w takes rows 4 w .. 4 w + 3 of the unit (0..31 gate, 32..63 up),
         // the 16 lanes of a row take every 16th chunk of 32 columns and meet by row-wide adds
-        KTS(8);
         const uint32_t urow = 4u * wave + (lane >> 4), row_bytes = HB * 210u;
         const float *xs = reinterpret_cast<const float *>(raw_rows + 64u * row_bytes), *xsum = xs + H + H / 32u;   // x, one float of padding per 32
-        KTS(9);
         const uint8_t *rowp = raw_rows + urow * row_bytes;
         float acc = 0.0f;
         for (uint32_t c = lane & 15u; c < HG; c += 16u) {
@@ -764,7 +735,6 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_select_kernel(GateUpArgs a
             for (int i = 0; i < 32; ++i) xv[i] = xs[33u * c + i];
             acc += q6k_dot32(rowp, c, xv, xsum[2u * c], xsum[2u * c + 1u]);
         }
-        KTS(10);
         acc += dpp_f32<kDppXor1>(acc);
         acc += dpp_f32<kDppXor2>(acc);
         acc += dpp_f32<kDppRor4>(acc);
@@ -783,7 +753,6 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_select_kernel(GateUpArgs a
             split_hi_lo(act, exp2i(-e), a.act_h + (uint64_t)slot * F + 32u * g + tid, a.act_l + (uint64_t)slot * F + 32u * g + tid);
             if (tid == 0u) a.act_exp[slot * (F / 32u) + g] = e;
         }
-        KTSY(21);
         return;
     }
     const uint8_t *ex = is_shared ? a.shared : a.experts + (uint64_t)expert * a.stride;
@@ -812,9 +781,7 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_select_kernel(GateUpArgs a
         const uint32_t quad = q0 + (NW / NKC) * reduced_unit<UPW>(lane);
         part[kc * 64u + 4u * quad + j] = tot;
     }
-    KTS(2);
     __syncthreads();
-    KTS(3);
     if (tid < 32u) {
         float gsum = 0.0f, usum = 0.0f;
 #pragma unroll
@@ -830,7 +797,6 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_select_kernel(GateUpArgs a
         split_hi_lo(act, exp2i(-e), a.act_h + (uint64_t)slot * F + 32u * g + tid, a.act_l + (uint64_t)slot * F + 32u * g + tid);
         if (tid == 0u) a.act_exp[slot * (F / 32u) + g] = e;
     }
-    KTSY(21);
 }
 
 struct DownArgs {
@@ -850,7 +816,7 @@ struct DownArgs {
 // ffn columns (ffn = 512: 16 groups = the 16 lane blocks of a wave). Slots are then added in selection order.
 __global__ __launch_bounds__(kWaves * 64) void down_combine_kernel(DownArgs a) {
     __shared__ __attribute__((aligned(16))) uint8_t lds[kMagBytes];
-    __shared__ float part[17 * 8];
+    __shared__ float part[17 * 8], comb[17];
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
     const uint32_t H = a.hidden, F = a.ffn, FG = F / 32u, FB = F / 256u, n_slot = a.top_k + 1u;
     const uint64_t grid_entry = tid < 256u ? redhip_iq2xxs_grid[tid] : 0ull;
@@ -874,6 +840,20 @@ __global__ __launch_bounds__(kWaves * 64) void down_combine_kernel(DownArgs a) {
                 if ((uint32_t)c < n_chunk && G < FG) { dq[q][c] = qs[(uint64_t)r * FG + G]; dd[q][c] = ds[(uint64_t)r * FB + (G >> 3)]; }
             }
     }
+    // activations and combine weights are requested before the table barrier: nothing below waits for memory twice
+    half4_t ax[2][8];
+    float sc[2] = {0.0f, 0.0f};
+    if (active) {
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            const uint32_t G = 16u * c + blk;
+            if ((uint32_t)c < n_chunk && G < FG) {
+                load_act_operand(ax[c], a.act_h + (uint64_t)wave * F + 32u * G, a.act_l + (uint64_t)wave * F + 32u * G, j);
+                sc[c] = exp2i(a.act_exp[wave * FG + G]);
+            }
+        }
+    }
+    if (tid < n_slot) comb[tid] = 0.125f * (tid < a.top_k ? a.weights[tid] : a.scalar[0]);
     build_tables(lds, tid, grid_entry);
     __syncthreads();
     if (active) {
@@ -881,11 +861,8 @@ __global__ __launch_bounds__(kWaves * 64) void down_combine_kernel(DownArgs a) {
         for (int c = 0; c < 2; ++c) {
             const uint32_t G = 16u * c + blk;
             if ((uint32_t)c < n_chunk && G < FG) {
-                half4_t ax[8];
-                load_act_operand(ax, a.act_h + (uint64_t)wave * F + 32u * G, a.act_l + (uint64_t)wave * F + 32u * G, j);
-                const float sc = exp2i(a.act_exp[wave * FG + G]);
 #pragma unroll
-                for (int q = 0; q < 2; ++q) tot[q] += group_dot(dq[q][c], ax, lds) * scale_to_f32(dd[q][c]) * sc;
+                for (int q = 0; q < 2; ++q) tot[q] += group_dot(dq[q][c], ax[c], lds) * scale_to_f32(dd[q][c]) * sc[c];
             }
         }
         const float r = quad_column_reduce<2>(tot, lane);
@@ -894,8 +871,7 @@ __global__ __launch_bounds__(kWaves * 64) void down_combine_kernel(DownArgs a) {
     __syncthreads();
     if (tid < 8u) {
         float sum = 0.0f;
-        for (uint32_t s = 0; s < a.top_k; ++s) sum = fmaf(a.weights[s] * 0.125f, part[s * 8u + tid], sum);
-        sum = fmaf(a.scalar[0] * 0.125f, part[a.top_k * 8u + tid], sum);
+        for (uint32_t s = 0; s < n_slot; ++s) sum = fmaf(comb[s], part[s * 8u + tid], sum);      // selection order, the shared expert last
         a.out[row0 + tid] = sum;
     }
 }
@@ -1162,7 +1138,6 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_batch_kernel(BatchArgs a) 
     if (blockIdx.x < n_units) count = (n_units - blockIdx.x + gridDim.x - 1u) / gridDim.x;
     if (count > (uint32_t)kMaxUnits) count = kMaxUnits;
     if (count == 0u) return;
-    KTS(0);
     // x operand in LDS as [piece s of 8 bytes][plane][group], plane = 2 * token + (hi, lo) and one more plane of
     // zeros for lanes without a token: the 64 lanes of a wave read the same piece of consecutive groups, and the
     // plane stride of HG + 8 keeps the hi and lo planes on different banks
@@ -1189,7 +1164,6 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_batch_kernel(BatchArgs a) 
     for (uint32_t i = tid; i < 8u * PLS; i += NW * 64u) xs[(i / PLS) * SS + ZP * PLS + i % PLS] = make_uint2(0u, 0u);
     build_tables(lds, tid, grid_entry);
     __syncthreads();
-    KTS(1);
 
     const uint64_t qs_bytes = (uint64_t)F * HG * 8u, gate_bytes = qs_bytes + (uint64_t)F * HB * 2u;
     const uint32_t kc = wave % NKC, q0 = wave / NKC;              // wave-uniform: they stay in scalar registers
@@ -1259,11 +1233,9 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_batch_kernel(BatchArgs a) 
                 const float tot = quad_column_reduce<UPW>(v[t], lane);
                 if (reduced_writer<UPW>(lane)) pbuf[t][kc * 64u + 4u * (q0 + (NW / NKC) * reduced_unit<UPW>(lane)) + j] = tot;
             }
-            KTS(2u + 2u * k);
             // the only barrier of a pass: the next pass writes the other half of `part`, and the one after that
             // comes behind the next barrier, which the lanes below reach only after they have read this half
             __syncthreads();
-            KTS(3u + 2u * k);
             if (tid < 32u * 2u * NTP) {
                 const uint32_t t = tid >> 5, c = tid & 31u, ip = pp + t;
                 if (ip < n) {
@@ -1486,12 +1458,3 @@ hipError_t launch_down_combine(const void *experts, uint64_t stride, const void 
 }
 
 }  // namespace redhip
-
-#ifdef REDHIP_KTS
-extern "C" int redhip_debug_kts(unsigned long long *out) {
-    return hipMemcpyFromSymbol(out, HIP_SYMBOL(redhip::g_kts), sizeof(unsigned long long) * 256 * 32) == hipSuccess;
-}
-extern "C" int redhip_debug_kts2(unsigned long long *out) {
-    return hipMemcpyFromSymbol(out, HIP_SYMBOL(redhip::g_kts2), sizeof(unsigned long long) * 256 * 32) == hipSuccess;
-}
-#endif
