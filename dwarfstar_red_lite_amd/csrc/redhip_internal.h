@@ -86,6 +86,10 @@ hipError_t launch_batch_combine(const float *tmp, const float *pair_weight, cons
                                 const float *sh_tmp, const float *scalar, uint32_t hidden, float *out, hipStream_t s);
 
 // pair sort of [ntok][top_k] ids: see redhip_moe_group in include/redhip_moe.h
+// f32 router logits of a chunk of tokens as a tiled fp32 MFMA product (every router row read once per 32 tokens), plus the
+// fp16 split of the activations; same outputs as launch_router_gemv
+hipError_t launch_router_f32_tiles(const float *w, const float *gate_inp, const float *x, uint32_t ntok, uint32_t hidden, uint32_t n_expert,
+                                   float *logits, void *xh, void *xl, int *xexp, hipStream_t s);
 // prefill chunk on packed IQ2_XXS experts: tiles of 16 pairs per distinct expert, 16x16x16 fp16 MFMA. Needs the pair
 // grouping (uid, expert_start, pair_token, n_unique); writes tmp [pairs][hidden] and sh_tmp [ntok][hidden] for
 // launch_batch_combine. tile_* hold prefill_tile_bound() entries.

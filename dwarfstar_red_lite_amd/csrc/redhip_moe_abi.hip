@@ -365,9 +365,13 @@ int redhip_moe_route(redhip_moe_t h, uint32_t layer, const float *x_dev, uint32_
         prof_set_stage(ST_ROUTER_GEMV);
         // a Q6_K shared expert of a mixed layout rides along: its gate / up products land in m->act (otherwise unused on this path)
         m->shared_gu_ready = m->mixed && m->sh_gu_type == T_Q6_K && c.router_type == T_Q6_K && ntok == 1u && c.top_k >= 2u;
-        HIP_OK(launch_router_gemv(c.router_type, m->layers[layer].router, x_dev, m->layers[layer].gate_inp, ntok, c.hidden, c.n_expert,
-                                  m->logits, m->xh, m->xl, m->xexp, m->shared_gu_ready ? m->layers[layer].shared : nullptr, m->act, c.ffn, s),
-               "router launch");
+        if (c.router_type == T_F32 && ntok >= 16u)
+            HIP_OK(launch_router_f32_tiles(reinterpret_cast<const float *>(m->layers[layer].router), m->layers[layer].gate_inp, x_dev, ntok, c.hidden,
+                                           c.n_expert, m->logits, m->xh, m->xl, m->xexp, s), "router tile launch");
+        else
+            HIP_OK(launch_router_gemv(c.router_type, m->layers[layer].router, x_dev, m->layers[layer].gate_inp, ntok, c.hidden, c.n_expert,
+                                      m->logits, m->xh, m->xl, m->xexp, m->shared_gu_ready ? m->layers[layer].shared : nullptr, m->act, c.ffn, s),
+                   "router launch");
         if (m->select_and_group) {
             prof_set_stage(ST_ROUTE_SELECT);
             HIP_OK(launch_select_group(m->logits, ntok, c.n_expert, c.top_k, m->ids, m->weights, m->scalar, m->uid, m->expert_start,
