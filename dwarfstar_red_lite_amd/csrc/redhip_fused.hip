@@ -1,16 +1,23 @@
-// Decode path over packed IQ2_XXS, three launches per layer, no atomics and no device-scope fences (on this
-// hardware a grid-wide __threadfence costs tens of microseconds and same-address float atomics serialise):
+// Kernels on packed IQ2_XXS rows for one token and for small batches; no atomics and no device-scope fences (on this
+// hardware a grid-wide __threadfence costs tens of microseconds and same-address float atomics serialise), so kernel
+// boundaries are the only grid-wide synchronisation.
 //
-//   router_*_kernel        logits of every expert (plus the shared expert's gate logit) and the fp16 split of x
-//   gateup_select_kernel   every workgroup repeats the cheap softmax top-k from the logits, then computes 32 gate
-//                          rows + 32 up rows of one selected expert (or the shared expert) -> SwiGLU -> fp16 halves
+// One token, three launches per layer:
+//   router_*_kernel        logits of every expert (plus the shared expert's gate logit) and the fp16 split of x; for a
+//                          Q6_K shared expert also its gate and up products, in extra workgroups
+//   gateup_select_kernel   every routed workgroup repeats the cheap softmax top-k from the logits on one wave, then
+//                          computes 32 gate rows + 32 up rows of one selected expert (or the shared expert) ->
+//                          SwiGLU -> fp16 halves
 //   down_combine_kernel    8 output rows per workgroup, one wave per selected expert; weighted sum in selection
-//                          order + shared expert * scalar gate: deterministic
+//                          order + shared expert * scalar gate: deterministic (down_combine_raw_kernel when the down
+//                          matrices are raw IQ3_S / Q6_K rows)
+// Two to eight tokens: select_group_kernel (selection per token + pair sort), gateup_batch_kernel (persistent
+// workgroups, every distinct expert read once), down_batch_kernel.
 //
-// Arithmetic: a weight is (sign * magnitude * (2*scale+1)) * d/8 with sign*magnitude looked up as eight exact
-// fp16 values from LDS tables; an activation vector is split into two fp16 halves (hi + lo*2^-11, after a
-// power-of-two pre-scale), and v_mfma_f32_4x4x4_16B_f16 multiplies four weights of four rows by both halves per
-// lane with fp32 accumulation. Per-group scales and d are applied to the fp32 sums.
+// Arithmetic: a weight is (sign * magnitude * (2*scale+1)) * d/8; the eight magnitudes of a grid entry are exact fp16
+// values from an LDS table, the sign bits are placed by integer arithmetic; an activation vector is split into two
+// fp16 halves (hi + lo*2^-11, after a power-of-two pre-scale), and v_mfma_f32_4x4x4_16B_f16 multiplies four weights of
+// four rows by both halves per lane with fp32 accumulation. Per-group scales and d are applied to the fp32 sums.
 //
 // Layout ("packed IQ2_XXS"): the 66-byte blocks are split at upload into an 8-byte stream [row][group] (4 grid
 // indices + 28 sign bits + 4 scale bits per 32 weights) and an fp16 stream [row][block] (d per 256 weights), both
