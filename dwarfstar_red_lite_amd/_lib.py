@@ -56,6 +56,7 @@ ABI = {
     "redhip_moe_load_shared": (i32, [vp, u32, vp, vp, u64, vp, u64, vp, u64]),
     "redhip_moe_load_experts": (i32, [vp, u32, u32, u32, vp, vp, vp]),
     "redhip_moe_forward": (i32, [vp, u32, vp, u32, vp, vp]),
+    "redhip_moe_forward_block": (i32, [vp, u32, vp, vp, vp, C.c_float, u32, vp, vp]),
     "redhip_moe_route": (i32, [vp, u32, vp, u32, vp, vp, vp, vp]),
     "redhip_moe_experts": (i32, [vp, u32, vp, u32, vp, vp, vp, vp]),
     "redhip_moe_last_route": (i32, [vp, u32, vp, vp, vp, vp]),

@@ -202,17 +202,30 @@ struct RouterArgs {
     const uint8_t *sh_q6k;
     float *sh_gu;
     uint32_t ffn;
+    // block step: the activations are (x + branch) * rsqrt(mean((x + branch)^2) + eps) * norm_w, written to xn_out
+    const float *branch, *norm_w;
+    float eps;
+    float *xn_out;             // [ntok][hidden]
 };
 
 // fp16 split of x, spread over the whole grid (every workgroup knows the largest |x| of its token)
-__device__ __forceinline__ void split_x_job(const RouterArgs &a, uint32_t tok, float amax) {
+__device__ __forceinline__ void split_x_job(const RouterArgs &a, uint32_t tok, float amax, float norm_inv) {
     const uint32_t gt = blockIdx.x * blockDim.x + threadIdx.x, nt = gridDim.x * blockDim.x;
     const int e = prescale_exp(amax);
     const float inv = exp2i(-e);
-    const float *x = a.x + (uint64_t)tok * a.hidden;
-    for (uint32_t i = gt; i < a.hidden; i += nt) split_hi_lo(x[i], inv, a.xh + (uint64_t)tok * a.hidden + i, a.xl + (uint64_t)tok * a.hidden + i);
+    const uint64_t base = (uint64_t)tok * a.hidden;
+    for (uint32_t i = gt; i < a.hidden; i += nt) {
+        float v = a.x[base + i];
+        if (a.branch) {                                    // same expression as in the kernels: ((x + branch) * inv) * w
+            v = ((v + a.branch[base + i]) * norm_inv) * a.norm_w[i];
+            a.xn_out[base + i] = v;
+        }
+        split_hi_lo(v, inv, a.xh + base + i, a.xl + base + i);
+    }
     if (gt == 0u) a.xexp[tok] = e;
 }
+// 1 / sqrt(mean of squares + eps) from a wave's (or workgroup's) sum of squares
+__device__ __forceinline__ float norm_scale(double ss, uint32_t n, float eps) { return (float)(1.0 / sqrt(ss / (double)n + (double)eps)); }
 
 // F32 router: one wave per row (row n_expert is the shared expert's gate vector), the row and x read as float4
 // with lanes interleaved; every wave sees all of x, so the pre-scale exponent needs no extra pass. blockIdx.y = token.
@@ -229,6 +242,25 @@ __global__ __launch_bounds__(256) void router_f32_kernel(const float *w, RouterA
     }
 #pragma unroll
     for (int k = 0; k < NV; ++k) xq[k] = xv[lane + 64u * k];
+    float norm_inv = 1.0f;
+    if (a.branch) {                                        // every wave holds the whole vector: the norm needs no workgroup barrier
+        const float4 *bv = reinterpret_cast<const float4 *>(a.branch + (uint64_t)tok * H), *nw = reinterpret_cast<const float4 *>(a.norm_w);
+        float4 wn[NV];
+        double ss = 0.0;
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            const float4 b = bv[lane + 64u * k];
+            wn[k] = nw[lane + 64u * k];
+            xq[k].x += b.x; xq[k].y += b.y; xq[k].z += b.z; xq[k].w += b.w;
+            ss += ((double)xq[k].x * xq[k].x + (double)xq[k].y * xq[k].y) + ((double)xq[k].z * xq[k].z + (double)xq[k].w * xq[k].w);
+        }
+        norm_inv = norm_scale(wave_sum_d(ss), H, a.eps);
+#pragma unroll
+        for (int k = 0; k < NV; ++k) {
+            xq[k].x = (xq[k].x * norm_inv) * wn[k].x; xq[k].y = (xq[k].y * norm_inv) * wn[k].y;
+            xq[k].z = (xq[k].z * norm_inv) * wn[k].z; xq[k].w = (xq[k].w * norm_inv) * wn[k].w;
+        }
+    }
     float acc = 0.0f, amax = 0.0f;
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
@@ -240,13 +272,14 @@ __global__ __launch_bounds__(256) void router_f32_kernel(const float *w, RouterA
     }
     acc = wave_sum(acc);
     if (lane == 0u && r <= a.n_expert) a.logits[(uint64_t)tok * (a.n_expert + 1u) + r] = acc;
-    split_x_job(a, tok, wave_max(amax));
+    split_x_job(a, tok, wave_max(amax), norm_inv);
 }
 
 // quantised router: rows decoded 32 weights per lane from the raw blocks, x staged in LDS
 template <uint32_t T>
 __global__ __launch_bounds__(256) void router_quant_kernel(const uint8_t *w, RouterArgs a) {
     __shared__ float lds_amax[4];
+    __shared__ double lds_ss[4];
     extern __shared__ float xs[];                        // x (padded), then the four raw rows of the workgroup
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63u, H = a.hidden, tok = blockIdx.y;
     const uint32_t row_bytes = (H / 256u) * Fmt<T>::kBlock;
@@ -257,8 +290,19 @@ __global__ __launch_bounds__(256) void router_quant_kernel(const uint8_t *w, Rou
     if (shared_wg) wave_stage(my_row, a.sh_q6k + (uint64_t)sh_row0 * sh_row_bytes, 2u * sh_row_bytes, lane);      // the wave's two rows
     else if (blockIdx.x * 4u + wave < a.n_expert) wave_stage(my_row, w + (uint64_t)(blockIdx.x * 4u + wave) * row_bytes, row_bytes, lane);
     const float *x = a.x + (uint64_t)tok * H;
-    float amax = 0.0f;
-    for (uint32_t i = threadIdx.x; i < H; i += 256u) { const float v = x[i]; xs[i + (i >> 5)] = v; amax = fmaxf(amax, fabsf(v)); }
+    float amax = 0.0f, norm_inv = 1.0f;
+    if (a.branch) {                                      // two passes over the staged vector: sum of squares, then scale
+        const float *br = a.branch + (uint64_t)tok * H;
+        double ss = 0.0;
+        for (uint32_t i = threadIdx.x; i < H; i += 256u) { const float v = x[i] + br[i]; xs[i + (i >> 5)] = v; ss += (double)v * v; }
+        ss = wave_sum_d(ss);
+        if (lane == 0u) lds_ss[wave] = ss;
+        __syncthreads();
+        norm_inv = norm_scale((lds_ss[0] + lds_ss[1]) + (lds_ss[2] + lds_ss[3]), H, a.eps);
+        for (uint32_t i = threadIdx.x; i < H; i += 256u) { const float v = (xs[i + (i >> 5)] * norm_inv) * a.norm_w[i]; xs[i + (i >> 5)] = v; amax = fmaxf(amax, fabsf(v)); }
+    } else {
+        for (uint32_t i = threadIdx.x; i < H; i += 256u) { const float v = x[i]; xs[i + (i >> 5)] = v; amax = fmaxf(amax, fabsf(v)); }
+    }
     amax = wave_max(amax);
     if (lane == 0u) lds_amax[wave] = amax;
     __syncthreads();
@@ -318,7 +362,7 @@ __global__ __launch_bounds__(256) void router_quant_kernel(const uint8_t *w, Rou
         acc = wave_sum(acc);
         if (lane == 0u) a.logits[(uint64_t)tok * (a.n_expert + 1u) + r] = acc;
     }
-    split_x_job(a, tok, amax);
+    split_x_job(a, tok, amax, norm_inv);
 }
 
 hipError_t launch_router_gemv(uint32_t router_type, const void *w, const float *x, const float *gate_inp, uint32_t ntok, uint32_t hidden,
@@ -326,8 +370,10 @@ hipError_t launch_router_gemv(uint32_t router_type, const void *w, const float *
                               hipStream_t s) {
     if (!ntok || !hidden || hidden % 256u || !n_expert || n_expert > 1024u) return hipErrorInvalidValue;
     const bool with_shared = sh_q6k && sh_gu && router_type == T_Q6_K && ntok == 1u && ffn % 4u == 0u;
+    const BlockContext &bc = block_context();
+    if (bc.branch && (!bc.norm_w || !bc.xn_out)) return hipErrorInvalidValue;
     RouterArgs a{x, gate_inp, logits, static_cast<_Float16 *>(xh), static_cast<_Float16 *>(xl), xexp, hidden, n_expert,
-                 with_shared ? static_cast<const uint8_t *>(sh_q6k) : nullptr, sh_gu, ffn};
+                 with_shared ? static_cast<const uint8_t *>(sh_q6k) : nullptr, sh_gu, ffn, bc.branch, bc.norm_w, bc.eps, bc.xn_out};
     const dim3 grid((n_expert + 1u + 3u) / 4u, ntok);
     if (router_type == T_F32) {
         const float *wf = static_cast<const float *>(w);
@@ -817,6 +863,7 @@ struct DownArgs {
     const int *act_exp;
     float *out;                // [hidden]
     uint32_t hidden, ffn, top_k;
+    const float *resid_a, *resid_b;     // when set: out[i] = (resid_a[i] + resid_b[i]) + layer output
 };
 
 // 8 output rows per workgroup; wave s (< top_k + 1) owns slot s: both row quads of the workgroup against all
@@ -879,7 +926,7 @@ __global__ __launch_bounds__(kWaves * 64) void down_combine_kernel(DownArgs a) {
     if (tid < 8u) {
         float sum = 0.0f;
         for (uint32_t s = 0; s < n_slot; ++s) sum = fmaf(comb[s], part[s * 8u + tid], sum);      // selection order, the shared expert last
-        a.out[row0 + tid] = sum;
+        a.out[row0 + tid] = a.resid_a ? (a.resid_a[row0 + tid] + a.resid_b[row0 + tid]) + sum : sum;
     }
 }
 
@@ -896,6 +943,7 @@ struct DownRawArgs {
     const int *act_exp;
     float *out;
     uint32_t hidden, ffn, top_k;
+    const float *resid_a, *resid_b;
 };
 
 template <uint32_t T>
@@ -956,7 +1004,7 @@ __global__ __launch_bounds__(kWaves * 64) void down_combine_raw_kernel(DownRawAr
         float sum = 0.0f;
         for (uint32_t s = 0; s < a.top_k; ++s) sum = fmaf(a.weights[s], part[s * 8u + tid], sum);
         sum = fmaf(a.scalar[0], part[a.top_k * 8u + tid], sum);
-        a.out[row0 + tid] = sum;
+        a.out[row0 + tid] = a.resid_a ? (a.resid_a[row0 + tid] + a.resid_b[row0 + tid]) + sum : sum;
     }
 }
 
@@ -978,7 +1026,8 @@ hipError_t launch_down_combine_raw(uint32_t down_type, uint32_t shared_down_type
                                    const int *act_exp, float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, hipStream_t s) {
     if (!hidden || hidden % 8u || !ffn || ffn % 256u || top_k + 1u > (uint32_t)kWaves) return hipErrorInvalidValue;
     const DownRawArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(shared), ids, weights, scalar,
-                        static_cast<const _Float16 *>(act_h), static_cast<const _Float16 *>(act_l), act_exp, out, hidden, ffn, top_k};
+                        static_cast<const _Float16 *>(act_h), static_cast<const _Float16 *>(act_l), act_exp, out, hidden, ffn, top_k,
+                        block_context().resid_a, block_context().resid_b};
     switch (down_type) {
         case T_IQ2_XXS: return launch_down_raw_shared<T_IQ2_XXS>(shared_down_type, a, s);
         case T_IQ3_S: return launch_down_raw_shared<T_IQ3_S>(shared_down_type, a, s);
@@ -1117,6 +1166,7 @@ struct BatchArgs {
     int *act_exp;                  // [P + ntok][ffn / 32]
     float *out;                    // [ntok][hidden]
     uint32_t hidden, ffn, top_k, ntok;
+    const float *resid_a, *resid_b;     // when set: out = (resid_a + resid_b) + layer output, [ntok][hidden] each
 };
 
 // Persistent workgroups walk the units (u, g) = (group of pairs, 32 FFN columns): 32 gate + 32 up rows of the
@@ -1371,7 +1421,8 @@ __global__ __launch_bounds__(kWaves * 64) void down_batch_kernel(BatchArgs a) {
             sum = fmaf(a.pair_weight[p] * 0.125f, part[p * 8u + r], sum);
         }
         sum = fmaf(a.scalar[t] * 0.125f, part[(P + t) * 8u + r], sum);
-        a.out[(uint64_t)t * H + row0 + r] = sum;
+        const uint64_t at = (uint64_t)t * H + row0 + r;
+        a.out[at] = a.resid_a ? (a.resid_a[at] + a.resid_b[at]) + sum : sum;
     }
 }
 
@@ -1382,7 +1433,8 @@ hipError_t launch_batch_packed(const void *experts, uint64_t stride, const void 
     if (!fused_iq2_supported(hidden, ffn) || !ntok || ntok > (uint32_t)kMaxTok || ntok * top_k + ntok > 144u) return hipErrorInvalidValue;
     BatchArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(shared), uid, expert_start, pair_token, n_unique,
                 pair_weight, tok_pair, scalar, static_cast<const _Float16 *>(xh), static_cast<const _Float16 *>(xl), xexp,
-                static_cast<_Float16 *>(act_h), static_cast<_Float16 *>(act_l), act_exp, out, hidden, ffn, top_k, ntok};
+                static_cast<_Float16 *>(act_h), static_cast<_Float16 *>(act_l), act_exp, out, hidden, ffn, top_k, ntok,
+                block_context().resid_a, block_context().resid_b};
     const uint32_t P = ntok * top_k, n_groups = (P < n_expert ? P : n_expert) + 1u;
     const uint32_t unit_bound = n_groups * (ffn / 32u);
     const dim3 grid(256u * ((unit_bound + 256u * kMaxUnits - 1u) / (256u * kMaxUnits)));
@@ -1459,7 +1511,8 @@ hipError_t launch_down_combine(const void *experts, uint64_t stride, const void 
                                uint32_t hidden, uint32_t ffn, uint32_t top_k, hipStream_t s) {
     if (!fused_iq2_supported(hidden, ffn) || top_k + 1u > (uint32_t)kWaves) return hipErrorInvalidValue;
     DownArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(shared), ids, weights, scalar,
-               static_cast<const _Float16 *>(act_h), static_cast<const _Float16 *>(act_l), act_exp, out, hidden, ffn, top_k};
+               static_cast<const _Float16 *>(act_h), static_cast<const _Float16 *>(act_l), act_exp, out, hidden, ffn, top_k,
+               block_context().resid_a, block_context().resid_b};
     REDHIP_LAUNCH(down_combine_kernel, dim3(hidden / 8u), dim3(kWaves * 64), 0, s, a);
     return hipGetLastError();
 }

@@ -30,6 +30,18 @@ enum Stage : uint32_t {
     ST_FUSED_EXPERTS, ST_BATCH_GATEUP, ST_BATCH_DOWN, ST_BATCH_COMBINE, ST_PREFILL_GATEUP, ST_PREFILL_DOWN, ST_COUNT
 };
 void prof_set_stage(uint32_t stage);                       // label of the launches that follow (calling thread)
+
+// The step around the layer (native/redlite_native_engine_cpu.c:418-427): the layer's input is the RMS-norm of x + branch,
+// and x + branch is added to its output. Both are context of the calling thread, picked up by the launchers below:
+// the router launchers normalise on the fly and write the normalised activations to xn_out, the launchers of a path's
+// last kernel add resid_a[i] + resid_b[i] to out[i]. All null outside redhip_moe_forward_block.
+struct BlockContext {
+    const float *branch = nullptr, *norm_w = nullptr;      // router side: x := (x + branch) * rsqrt(mean((x + branch)^2) + eps) * norm_w
+    float eps = 0.0f;
+    float *xn_out = nullptr;
+    const float *resid_a = nullptr, *resid_b = nullptr;   // output side
+};
+BlockContext &block_context();
 void prof_events(hipEvent_t *start, hipEvent_t *stop);     // both nullptr when profiling is off
 
 #define REDHIP_LAUNCH(kern, grid, block, lds, stream, ...)                                         \

@@ -294,7 +294,8 @@ __global__ __launch_bounds__(256) void moe_down_combine_kernel(const uint8_t *ba
                                                                const uint32_t *ids, const float *weights, uint32_t top_k,
                                                                const uint8_t *sh_down, const float *scalar,
                                                                uint32_t hidden, uint32_t ffn,
-                                                               const float *act, const float *sh_act, float *out) {
+                                                               const float *act, const float *sh_act, float *out,
+                                                               const float *resid_a, const float *resid_b) {
     extern __shared__ float as[];                          // [top_k + 1][padded ffn]
     const uint32_t fp = ffn + (ffn >> 5);
     for (uint32_t i = threadIdx.x; i < top_k * ffn; i += 256u) as[(i / ffn) * fp + pad32(i % ffn)] = act[i];
@@ -321,7 +322,7 @@ __global__ __launch_bounds__(256) void moe_down_combine_kernel(const uint8_t *ba
         part = sub_reduce<LPR>(part);
         total = fmaf(scalar[0], part, total);
     }
-    if (sub == 0u && r < hidden) out[r] = total;
+    if (sub == 0u && r < hidden) out[r] = resid_a ? (resid_a[r] + resid_b[r]) + total : total;      // block step: residual added here
 }
 
 template <uint32_t TD, uint32_t TS>
@@ -333,7 +334,7 @@ static hipError_t down_dispatch(const ExpertSet &ex, const uint32_t *ids, const 
     const size_t lds = (size_t)(top_k + 1u) * padded_floats(ffn) * sizeof(float);
     const uint8_t *shd = sh.base ? sh.base + sh.gate_bytes + sh.up_bytes : nullptr;
     const uint64_t off = ex.gate_bytes + ex.up_bytes;
-#define REDHIP_DOWN(L) REDHIP_LAUNCH((moe_down_combine_kernel<TD, TS, L>), dim3(grid), dim3(256), lds, s, ex.base, ex.stride, off, ids, weights, top_k, shd, scalar, hidden, ffn, act, sh_act, out)
+#define REDHIP_DOWN(L) REDHIP_LAUNCH((moe_down_combine_kernel<TD, TS, L>), dim3(grid), dim3(256), lds, s, ex.base, ex.stride, off, ids, weights, top_k, shd, scalar, hidden, ffn, act, sh_act, out, block_context().resid_a, block_context().resid_b)
     switch (lpr) {
         case 64: REDHIP_DOWN(64); break;
         case 32: REDHIP_DOWN(32); break;
@@ -487,7 +488,8 @@ __global__ __launch_bounds__(256) void batch_down_kernel(PairArgs a, uint32_t hi
 
 // out[t][r] = sum_k pair_weight[p_k] * tmp[p_k][r] (p_k = tok_pair[t][k], selection order) + scalar[t] * sh_tmp[t][r]
 __global__ __launch_bounds__(256) void batch_combine_kernel(const float *tmp, const float *pair_weight, const uint32_t *tok_pair, uint32_t top_k,
-                                                            const float *sh_tmp, const float *scalar, uint32_t hidden, float *out) {
+                                                            const float *sh_tmp, const float *scalar, uint32_t hidden, float *out,
+                                                            const float *resid_a, const float *resid_b) {
     const uint32_t r = blockIdx.x * 256u + threadIdx.x, t = blockIdx.y;
     if (r >= hidden) return;
     float acc = 0.0f;
@@ -496,7 +498,8 @@ __global__ __launch_bounds__(256) void batch_combine_kernel(const float *tmp, co
         acc = fmaf(pair_weight[p], tmp[(uint64_t)p * hidden + r], acc);
     }
     if (sh_tmp) acc = fmaf(scalar[t], sh_tmp[(uint64_t)t * hidden + r], acc);
-    out[(uint64_t)t * hidden + r] = acc;
+    const uint64_t at = (uint64_t)t * hidden + r;
+    out[at] = resid_a ? (resid_a[at] + resid_b[at]) + acc : acc;
 }
 
 template <uint32_t T>
@@ -565,7 +568,7 @@ hipError_t launch_batch_down(const ExpertSet &ex, const uint32_t *uid, const uin
 
 hipError_t launch_batch_combine(const float *tmp, const float *pair_weight, const uint32_t *tok_pair, uint32_t ntok, uint32_t top_k,
                                 const float *sh_tmp, const float *scalar, uint32_t hidden, float *out, hipStream_t s) {
-    REDHIP_LAUNCH(batch_combine_kernel, dim3((hidden + 255u) / 256u, ntok), dim3(256), 0, s, tmp, pair_weight, tok_pair, top_k, sh_tmp, scalar, hidden, out);
+    REDHIP_LAUNCH(batch_combine_kernel, dim3((hidden + 255u) / 256u, ntok), dim3(256), 0, s, tmp, pair_weight, tok_pair, top_k, sh_tmp, scalar, hidden, out, block_context().resid_a, block_context().resid_b);
     return hipGetLastError();
 }
 

@@ -46,6 +46,7 @@ struct Moe {
     std::vector<Layer> layers;
     // workspace (device), sized for max_tokens
     float *logits = nullptr, *weights = nullptr, *scalar = nullptr, *act = nullptr, *sh_act = nullptr;
+    float *xn = nullptr;                     // [max_tokens][hidden]: normalised activations of redhip_moe_forward_block
     uint32_t *ids = nullptr;
     uint8_t *ws = nullptr;
     // single-token fused path (all matrices IQ2_XXS, shapes the fused kernel tiles)
@@ -96,6 +97,20 @@ __global__ __launch_bounds__(256) void scalar_gate_kernel(const float *gate_inp,
     if ((threadIdx.x & 63u) == 0u) red[threadIdx.x >> 6] = acc;
     __syncthreads();
     if (threadIdx.x == 0u) scalar[blockIdx.x] = (float)(1.0 / (1.0 + exp(-((red[0] + red[1]) + (red[2] + red[3])))));
+}
+
+// resid = x + branch, xn = resid * rsqrt(mean(resid^2) + eps) * w (native/redlite_native_engine_cpu.c:418-424); one workgroup per
+// token. Used when the router kernel of the path cannot normalise on the fly.
+__global__ __launch_bounds__(256) void resid_rms_kernel(const float *x, const float *branch, const float *w, float eps, uint32_t hidden, float *xn) {
+    __shared__ double red[4];
+    const uint64_t base = (uint64_t)blockIdx.x * hidden;
+    double ss = 0.0;
+    for (uint32_t i = threadIdx.x; i < hidden; i += 256u) { const float v = x[base + i] + branch[base + i]; ss += (double)v * v; }
+    for (int o = 32; o > 0; o >>= 1) ss += __shfl_xor(ss, o, 64);
+    if ((threadIdx.x & 63u) == 0u) red[threadIdx.x >> 6] = ss;
+    __syncthreads();
+    const float inv = (float)(1.0 / sqrt(((red[0] + red[1]) + (red[2] + red[3])) / (double)hidden + (double)eps));
+    for (uint32_t i = threadIdx.x; i < hidden; i += 256u) xn[base + i] = ((x[base + i] + branch[base + i]) * inv) * w[i];
 }
 
 // select_here: the gate/up kernel selects the experts from m->logits itself (ids / weights are then outputs)
@@ -229,7 +244,7 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
         }
     }
     const size_t T = c.max_tokens;
-    const size_t ws_bytes = align256(T * (c.n_expert + 1u) * 4u) + 2u * align256(T * c.top_k * 4u) + align256(T * 4u) +
+    const size_t ws_bytes = align256(T * c.hidden * 4u) + align256(T * (c.n_expert + 1u) * 4u) + 2u * align256(T * c.top_k * 4u) + align256(T * 4u) +
                             align256(T * c.top_k * c.ffn * 4u) + align256(T * c.ffn * 4u) +
                             2u * align256(2u * T * c.hidden) + align256(4u * T) + 2u * align256(2u * T * (c.top_k + 1u) * c.ffn) +
                             align256(4u * T * (c.top_k + 1u) * (c.ffn / 32u)) +
@@ -242,6 +257,7 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
         return nullptr;
     }
     uint8_t *w = m->ws;
+    m->xn = reinterpret_cast<float *>(w); w += align256(T * c.hidden * 4u);
     m->logits = reinterpret_cast<float *>(w); w += align256(T * (c.n_expert + 1u) * 4u);
     m->ids = reinterpret_cast<uint32_t *>(w); w += align256(T * c.top_k * 4u);
     m->weights = reinterpret_cast<float *>(w); w += align256(T * c.top_k * 4u);
@@ -426,6 +442,44 @@ int redhip_moe_forward(redhip_moe_t h, uint32_t layer, const float *x_dev, uint3
     m->select_and_group = false;
     if (!routed) return 0;
     return experts_enqueue(m, layer, x_dev, ntok, m->ids, m->weights, out_dev, static_cast<hipStream_t>(stream), select_in_gateup, group_in_select);
+}
+
+int redhip_moe_forward_block(redhip_moe_t h, uint32_t layer, const float *x_dev, const float *branch_dev, const float *post_norm_dev, float eps,
+                             uint32_t ntok, float *x_out_dev, void *stream) {
+    Moe *m = moe_of(h);
+    if (!check_layer(m, layer)) return 0;
+    if (!x_dev || !branch_dev || !post_norm_dev || !x_out_dev || !ntok || ntok > m->cfg.max_tokens) { moe_err("invalid block step arguments"); return 0; }
+    const redhip_moe_config &c = m->cfg;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    BlockContext &bc = block_context();
+    bc = BlockContext{};
+    // the per-token router kernels of the packed paths normalise on the fly; everything else gets a kernel of its own
+    const bool in_router = m->packed_gu() && !(c.router_type == T_F32 && ntok >= 16u);
+    int ok = 1;
+    if (!in_router) {
+        prof_set_stage(ST_OTHER);
+        resid_rms_kernel<<<ntok, 256, 0, s>>>(x_dev, branch_dev, post_norm_dev, eps, c.hidden, m->xn);
+        if (hipGetLastError() != hipSuccess) { moe_err("residual + norm launch failed"); ok = 0; }
+    }
+    if (ok) {
+        const bool select_in_gateup = m->packed_gu() && ntok == 1u;
+        const bool group_in_select = m->small_batch(ntok);
+        m->skip_select = select_in_gateup;
+        m->select_and_group = group_in_select;
+        if (in_router) { bc.branch = branch_dev; bc.norm_w = post_norm_dev; bc.eps = eps; bc.xn_out = m->xn; }
+        ok = redhip_moe_route(h, layer, in_router ? x_dev : m->xn, ntok, nullptr, nullptr, nullptr, stream);
+        bc.branch = bc.norm_w = nullptr;
+        bc.xn_out = nullptr;
+        m->skip_select = false;
+        m->select_and_group = false;
+        if (ok) {
+            bc.resid_a = x_dev;                              // the path's last kernel adds x + branch to its output
+            bc.resid_b = branch_dev;
+            ok = experts_enqueue(m, layer, m->xn, ntok, m->ids, m->weights, x_out_dev, s, select_in_gateup, group_in_select);
+        }
+    }
+    bc = BlockContext{};
+    return ok;
 }
 
 int redhip_moe_last_route(redhip_moe_t h, uint32_t ntok, uint32_t *ids, float *weights, float *logits, void *stream) {

@@ -27,6 +27,11 @@ const char *const kStageNames[ST_COUNT] = {
 
 void prof_set_stage(uint32_t stage) { t_stage = stage < ST_COUNT ? stage : ST_OTHER; }
 
+BlockContext &block_context() {
+    static thread_local BlockContext ctx;
+    return ctx;
+}
+
 void prof_events(hipEvent_t *start, hipEvent_t *stop) {
     *start = *stop = nullptr;
     if (!g_prof.on) return;

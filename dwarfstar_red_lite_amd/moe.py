@@ -81,6 +81,19 @@ class ResidentMoe:
         self._check(self.lib.redhip_moe_forward(self.handle, layer, x.data_ptr(), x.shape[0], out.data_ptr(), _stream()))
         return out
 
+    def forward_block(self, layer, x, branch, post_norm, eps=1e-6, out=None):
+        """x_out = (x + branch) + layer(rmsnorm(x + branch) * post_norm): the layer with the residual steps around it."""
+        x = x.reshape(-1, self.cfg["hidden"])
+        branch = branch.reshape(-1, self.cfg["hidden"])
+        for t in (x, branch, post_norm):
+            assert t.is_cuda and t.dtype == torch.float32 and t.is_contiguous()
+        assert branch.shape == x.shape and post_norm.numel() == self.cfg["hidden"]
+        if out is None:
+            out = torch.empty_like(x)
+        self._check(self.lib.redhip_moe_forward_block(self.handle, layer, x.data_ptr(), branch.data_ptr(), post_norm.data_ptr(), float(eps),
+                                                      x.shape[0], out.data_ptr(), _stream()))
+        return out
+
     def route(self, layer, x):
         x = x.reshape(-1, self.cfg["hidden"])
         n, K, E = x.shape[0], self.cfg["top_k"], self.cfg["n_expert"]

@@ -66,6 +66,16 @@ int redhip_moe_experts(redhip_moe_t moe, uint32_t layer, const float *x_dev, uin
 /* Routing of the last forward / route on this handle, copied to host after synchronising `stream`. Any may be NULL. */
 int redhip_moe_last_route(redhip_moe_t moe, uint32_t ntok, uint32_t *ids, float *weights, float *logits, void *stream);
 
+/* The layer with the steps on either side of it, one call per layer and token batch
+ * (native/redlite_native_engine_cpu.c:418-427; Metal rl_resid_rms native/redmetal_engine.m:95-105 in front and
+ * rl_moe_tail :61-69 behind): resid = x + branch (the attention / DeltaNet branch output), the layer's input is
+ * resid * rsqrt(mean(resid^2) + eps) * post_norm, and x_out = resid + layer output. All pointers are device
+ * memory, [ntok][hidden] except post_norm_dev [hidden]; x_out_dev may be x_dev. Enqueues kernels only. Where the
+ * path allows, the norm is computed inside the router launch and the residual is added by the last kernel, so the
+ * two extra launches of the reference disappear. */
+int redhip_moe_forward_block(redhip_moe_t moe, uint32_t layer, const float *x_dev, const float *branch_dev,
+    const float *post_norm_dev, float eps, uint32_t ntok, float *x_out_dev, void *stream);
+
 /* Token grouping of [ntok][top_k] ids (device), the GPU form of the pair sort in
  * native/redmetal_engine_prefill.m:1246-1276: uid_dev[U] in first-appearance order, expert_start_dev[U+1],
  * pair_token_dev[P], pair_weight_dev[P], tok_pair_dev[P], n_unique_dev[1]; P = ntok * top_k. */
