@@ -55,6 +55,9 @@ ABI = {
     "redhip_moe_load_router": (i32, [vp, u32, vp, u64]),
     "redhip_moe_load_shared": (i32, [vp, u32, vp, vp, u64, vp, u64, vp, u64]),
     "redhip_moe_load_experts": (i32, [vp, u32, u32, u32, vp, vp, vp]),
+    "redhip_gguf_last_error": (C.c_char_p, []),
+    "redhip_gguf_moe_config": (i32, [C.c_char_p, u32, C.POINTER(MoeConfig)]),
+    "redhip_moe_load_gguf": (i32, [vp, C.c_char_p, u32, u32, C.POINTER(MoeConfig)]),
     "redhip_moe_forward": (i32, [vp, u32, vp, u32, vp, vp]),
     "redhip_moe_forward_block": (i32, [vp, u32, vp, vp, vp, C.c_float, u32, vp, vp]),
     "redhip_moe_route": (i32, [vp, u32, vp, u32, vp, vp, vp, vp]),

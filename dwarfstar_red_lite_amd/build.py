@@ -6,7 +6,7 @@ import subprocess
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
 LIB = os.path.join(HERE, "libredmetal_hip.so")
-SOURCES = ["redhip_kernels.hip", "redhip_fused.hip", "redhip_prefill.hip", "redhip_pool_abi.hip", "redhip_moe_abi.hip", "redhip_profile.hip"]
+SOURCES = ["redhip_kernels.hip", "redhip_fused.hip", "redhip_prefill.hip", "redhip_pool_abi.hip", "redhip_moe_abi.hip", "redhip_gguf.hip", "redhip_profile.hip"]
 # -packed-fp32-ops off: v_pk_*_f32 forms are not used on this pool of machines
 FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-shared", "-std=c++17",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-Wextra", "-Wno-unused-parameter"]

@@ -1,6 +1,7 @@
 """Resident MoE FFN layers (include/redhip_moe.h). torch owns the activation buffers and the stream; weights are
 uploaded once and stay in HBM."""
 import ctypes as C
+import os
 
 import numpy as np
 import torch
@@ -35,6 +36,23 @@ class ResidentMoe:
         self.handle = self.lib.redhip_moe_create(C.byref(c))
         if not self.handle:
             raise RedHipError(self._err())
+
+    @classmethod
+    def from_gguf(cls, path, first_layer=0, n_layer=None, max_tokens=1):
+        """Resident layers straight from a GGUF file: shapes, types and top_k come from the file."""
+        cfg, in_file = gguf_moe_config(path, first_layer)
+        n = in_file if n_layer is None else n_layer
+        m = cls(cfg, n_layer=n, max_tokens=max_tokens)
+        m.load_gguf(path, first_layer, n)
+        return m
+
+    def load_gguf(self, path, first_layer=0, n_layer=None):
+        cfg = self.cfg
+        c = MoeConfig(cfg["hidden"], cfg["ffn"], cfg["n_expert"], cfg["top_k"], self.n_layer, self.max_tokens, cfg["router_type"],
+                      expert_type_word(cfg["gate_up_type"], cfg["down_type"]),
+                      expert_type_word(cfg["sh_gate_up_type"], cfg["sh_down_type"]), 0)
+        if not self.lib.redhip_moe_load_gguf(self.handle, os.fsencode(path), first_layer, self.n_layer if n_layer is None else n_layer, C.byref(c)):
+            raise RedHipError(self.lib.redhip_gguf_last_error().decode("utf-8", errors="replace"))
 
     def _err(self):
         raw = self.lib.redhip_moe_last_error()
@@ -140,6 +158,19 @@ class ResidentMoe:
         out = torch.empty(shape, dtype=torch.float32, device="cuda")
         self._check(self.lib.redhip_moe_dequant_resident(self.handle, layer, expert, which, out.data_ptr(), _stream()))
         return out
+
+
+def gguf_moe_config(path, first_layer=0):
+    """(cfg dict as synth.layer_config gives it, number of consecutive MoE layers from first_layer) of a GGUF file. Host only."""
+    lib = load()
+    c = MoeConfig()
+    if not lib.redhip_gguf_moe_config(os.fsencode(path), first_layer, C.byref(c)):
+        raise RedHipError(lib.redhip_gguf_last_error().decode("utf-8", errors="replace"))
+    gu, dn = c.expert_type_word & 255, (c.expert_type_word >> 8) or (c.expert_type_word & 255)
+    sgu, sdn = c.shared_type_word & 255, (c.shared_type_word >> 8) or (c.shared_type_word & 255)
+    cfg = dict(hidden=c.hidden, ffn=c.ffn, n_expert=c.n_expert, top_k=c.top_k, router_type=c.router_type, gate_up_type=gu, down_type=dn,
+               sh_gate_up_type=sgu, sh_down_type=sdn)
+    return cfg, c.n_layer
 
 
 def dequant_rows(ggml_type, rows, ncols):

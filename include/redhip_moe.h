@@ -66,6 +66,18 @@ int redhip_moe_experts(redhip_moe_t moe, uint32_t layer, const float *x_dev, uin
 /* Routing of the last forward / route on this handle, copied to host after synchronising `stream`. Any may be NULL. */
 int redhip_moe_last_route(redhip_moe_t moe, uint32_t ntok, uint32_t *ids, float *weights, float *logits, void *stream);
 
+/* GGUF side (the role of native/redlite_native_gguf.c:196-440 and the tensor checks of
+ * native/redlite_native_engine.c:170-179): the MoE tensors of layer `first_layer + l` are blk.N.ffn_gate_inp.weight
+ * (router, (hidden, experts)), ffn_gate_inp_shexp.weight (F32 [hidden]), ffn_{gate,up,down}_shexp.weight and the
+ * expert-major ffn_{gate,up,down}_exps.weight ((hidden, ffn, experts) resp. (ffn, hidden, experts)).
+ * redhip_gguf_moe_config fills hidden / ffn / n_expert / top_k (from <arch>.expert_used_count) / types / n_layer (the
+ * run of consecutive MoE layers from first_layer) and max_tokens = 1 from a GGUF v2 / v3 file;
+ * redhip_moe_load_gguf uploads layers first_layer .. first_layer + n_layer - 1 of the file into layers 0 .. of a
+ * handle created with `cfg`. Errors: return 0 and redhip_gguf_last_error() (thread-local). */
+const char *redhip_gguf_last_error(void);
+int redhip_gguf_moe_config(const char *path, uint32_t first_layer, redhip_moe_config *out);
+int redhip_moe_load_gguf(redhip_moe_t moe, const char *path, uint32_t first_layer, uint32_t n_layer, const redhip_moe_config *cfg);
+
 /* The layer with the steps on either side of it, one call per layer and token batch
  * (native/redlite_native_engine_cpu.c:418-427; Metal rl_resid_rms native/redmetal_engine.m:95-105 in front and
  * rl_moe_tail :61-69 behind): resid = x + branch (the attention / DeltaNet branch output), the layer's input is

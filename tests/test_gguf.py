@@ -1,0 +1,67 @@
+"""GGUF side: directory parsing and configuration probe on the host; upload from a file on the GPU, where the layer loaded from
+the file must behave exactly as the same layer uploaded from memory."""
+import numpy as np
+import pytest
+
+from dwarfstar_red_lite_amd import synth
+from dwarfstar_red_lite_amd._lib import RedHipError
+from gguf_writer import write_moe_gguf
+
+
+def small_cfg(layout):
+    return synth.layer_config(hidden=512, ffn=256, n_expert=16, top_k=4, layout=layout)
+
+
+@pytest.mark.parametrize("layout", ["iq2", "f2"])
+def test_config_probe(tmp_path, layout):
+    from dwarfstar_red_lite_amd.moe import gguf_moe_config
+    cfg = small_cfg(layout)
+    layers = [synth.make_layer(40 + i, cfg) for i in range(3)]
+    path = tmp_path / "moe.gguf"
+    write_moe_gguf(path, cfg, layers, first_layer=2, extra_tensors=[("token_embd.weight", np.arange(100, dtype=np.float32))])
+    got, n = gguf_moe_config(str(path), first_layer=2)
+    assert n == 3
+    for k in ("hidden", "ffn", "n_expert", "top_k", "router_type", "gate_up_type", "down_type", "sh_gate_up_type", "sh_down_type"):
+        assert got[k] == cfg[k], k
+    with pytest.raises(RedHipError, match="lacks one of the MoE tensors"):
+        gguf_moe_config(str(path), first_layer=0)
+
+
+def test_rejects_broken_files(tmp_path):
+    from dwarfstar_red_lite_amd.moe import gguf_moe_config
+    p = tmp_path / "bad.gguf"
+    p.write_bytes(b"GGML" + b"\0" * 64)
+    with pytest.raises(RedHipError, match="invalid or unsupported GGUF header"):
+        gguf_moe_config(str(p))
+    cfg = small_cfg("iq2")
+    good = tmp_path / "good.gguf"
+    write_moe_gguf(good, cfg, [synth.make_layer(1, cfg)])
+    cut = tmp_path / "cut.gguf"
+    cut.write_bytes(good.read_bytes()[:-1000])
+    with pytest.raises(RedHipError, match="beyond the end of the file"):
+        gguf_moe_config(str(cut))
+    with pytest.raises(RedHipError, match="open .* failed"):
+        gguf_moe_config(str(tmp_path / "missing.gguf"))
+
+
+@pytest.mark.gpu
+@pytest.mark.parametrize("layout", ["iq2", "f2"])
+def test_load_from_file_equals_load_from_memory(tmp_path, layout):
+    torch = pytest.importorskip("torch")
+    from dwarfstar_red_lite_amd.moe import ResidentMoe
+    cfg = small_cfg(layout)
+    layers = [synth.make_layer(50 + i, cfg) for i in range(2)]
+    path = tmp_path / "moe.gguf"
+    write_moe_gguf(path, cfg, layers, first_layer=5)
+    a = ResidentMoe.from_gguf(str(path), first_layer=5, max_tokens=3)
+    assert a.n_layer == 2 and a.cfg["top_k"] == 4
+    b = ResidentMoe(cfg, n_layer=2, max_tokens=3)
+    x = torch.from_numpy(synth.normed_x(np.random.default_rng(3), 3, cfg["hidden"])).cuda()
+    for l in range(2):
+        b.load_layer(l, layers[l])
+        for nt in (1, 3):
+            assert torch.equal(a.forward(l, x[:nt]), b.forward(l, x[:nt]))
+        for which in range(3):
+            assert torch.equal(a.dequant_resident(l, 3, which), b.dequant_resident(l, 3, which))
+    a.close()
+    b.close()
