@@ -64,6 +64,7 @@ ABI = {
     "redhip_moe_experts": (i32, [vp, u32, vp, u32, vp, vp, vp, vp]),
     "redhip_moe_last_route": (i32, [vp, u32, vp, vp, vp, vp]),
     "redhip_moe_group": (i32, [vp, vp, vp, u32, vp, vp, vp, vp, vp, vp, vp]),
+    "redhip_set_codebooks": (i32, [vp, u32, vp, u32]),
     "redhip_dequant_rows": (i32, [u32, vp, u32, u32, vp, vp]),
     "redhip_moe_dequant_resident": (i32, [vp, u32, u32, u32, vp, vp]),
     "redhip_gemv_rows": (i32, [u32, vp, u32, u32, u32, vp, vp, vp]),

@@ -7,10 +7,23 @@
 
 namespace redhip {
 
-enum : uint32_t { T_F32 = 0u, T_Q6_K = 14u, T_IQ2_XXS = 16u, T_IQ3_S = 21u };
+enum : uint32_t { T_F32 = 0u, T_Q6_K = 14u, T_IQ2_XXS = 16u, T_IQ2_XS = 17u, T_IQ3_S = 21u, T_IQ1_M = 29u };
 
-// bytes per 256 weights; 0 for a type this library does not decode
+// bytes per 256 weights; 0 for a type this library does not decode. IQ2_XS and IQ1_M (the reference's current routed
+// formats, codebooks supplied by the caller) are decoded by the pool and one-shot GEMV surfaces only.
 inline uint32_t block_bytes(uint32_t t) { return t == T_Q6_K ? 210u : t == T_IQ2_XXS ? 66u : t == T_IQ3_S ? 110u : 0u; }
+inline uint32_t pool_block_bytes(uint32_t t) { return t == T_IQ2_XS ? 74u : t == T_IQ1_M ? 56u : block_bytes(t); }
+inline uint64_t pool_row_bytes(uint32_t t, uint32_t ncols) {
+    if (t == T_F32) return 4ull * ncols;
+    const uint32_t b = pool_block_bytes(t);
+    return (b && ncols && ncols % 256u == 0u) ? (uint64_t)(ncols / 256u) * b : 0ull;
+}
+inline bool pool_quant_supported(uint32_t t) { return pool_block_bytes(t) != 0u; }
+// device copies of the caller's IQ2_XS (512 x 8) / IQ1_M (2048 x 8) int8 codebooks; either may be null (left as is).
+// One copy per process: `owner` (a pool) makes a repeated call by the same owner free, so each pool can ask for its own
+// tables before every launch; callers whose tables differ must not run at the same time
+hipError_t set_caller_grids(const int8_t *iq2_xs, const int8_t *iq1_m, const void *owner = nullptr);
+void forget_caller_grids(const void *owner);
 inline uint64_t row_bytes(uint32_t t, uint32_t ncols) {
     if (!ncols) return 0;
     if (t == T_F32) return 4ull * ncols;

@@ -4,6 +4,8 @@
 // partial sums meet in a butterfly of cross-lane shuffles.
 #include "redhip_decode.h"
 
+#include <mutex>
+
 namespace redhip {
 
 // the codebooks are constant device arrays of this translation unit (redhip_tables.h): nothing to upload
@@ -16,6 +18,76 @@ static inline uint32_t lanes_per_row(uint32_t ncols) {
 // x staged in LDS with one pad word per 32 floats, so lanes that walk different chunks hit different banks
 __device__ __forceinline__ uint32_t pad32(uint32_t i) { return i + (i >> 5); }
 static inline uint32_t padded_floats(uint32_t n) { return n + (n >> 5); }
+
+// ---------------------------------------------------------------- IQ2_XS / IQ1_M (caller-supplied codebooks)
+
+// The reference hands these codebooks to its kernels as arguments (native/redmetal_ffn.m:223-227); here they live in
+// device memory of this translation unit, uploaded by the pool / one-shot surfaces before they launch.
+__device__ int8_t g_iq2xs_grid[512 * 8];
+__device__ int8_t g_iq1m_grid[2048 * 8];
+
+static std::mutex g_grid_mu;
+static const void *g_grid_owner = nullptr;      // whose tables the device holds; nullptr: nobody's in particular
+
+hipError_t set_caller_grids(const int8_t *iq2_xs, const int8_t *iq1_m, const void *owner) {
+    std::lock_guard<std::mutex> lk(g_grid_mu);
+    if (owner && owner == g_grid_owner) return hipSuccess;
+    hipError_t e = hipSuccess;
+    if (iq2_xs) e = hipMemcpyToSymbol(HIP_SYMBOL(g_iq2xs_grid), iq2_xs, sizeof(g_iq2xs_grid));
+    if (e == hipSuccess && iq1_m) e = hipMemcpyToSymbol(HIP_SYMBOL(g_iq1m_grid), iq1_m, sizeof(g_iq1m_grid));
+    g_grid_owner = e == hipSuccess ? owner : nullptr;
+    return e;
+}
+
+void forget_caller_grids(const void *owner) {
+    std::lock_guard<std::mutex> lk(g_grid_mu);
+    if (g_grid_owner == owner) g_grid_owner = nullptr;
+}
+
+template <> struct Fmt<T_IQ2_XS> { static constexpr uint32_t kBlock = 74u; };
+template <> struct Fmt<T_IQ1_M> { static constexpr uint32_t kBlock = 56u; };
+
+// IQ2_XS, native/redlite_native_reference.c:116-142: block = f16 d, 32 x u16 (9-bit codebook index + 7 sign bits, the
+// eighth sign is their parity), 8 bytes of 4-bit scales (one per 16 weights); weight = d * (0.5 + scale) * 0.25 * entry * sign
+template <> __device__ __forceinline__ void decode32<T_IQ2_XS>(const uint8_t *row, uint32_t chunk, float *w) {
+    const uint8_t *bp = row + (size_t)(chunk >> 3) * 74u;
+    const uint32_t cb = chunk & 7u;
+    const float d = half_bits_to_f32(ld_u16(bp));
+    const uint32_t sc = bp[66u + cb];
+    const float db0 = d * (0.5f + (float)(sc & 15u)) * 0.25f, db1 = d * (0.5f + (float)(sc >> 4)) * 0.25f;
+#pragma unroll
+    for (uint32_t k = 0; k < 4u; ++k) {
+        const uint32_t q = ld_u16(bp + 2u + 2u * (4u * cb + k));
+        const int8_t *entry = g_iq2xs_grid + (q & 511u) * 8u;
+        const uint32_t s7 = (q >> 9) & 127u, s8 = s7 | ((__popc(s7) & 1u) << 7);
+        const float db = k < 2u ? db0 : db1;
+#pragma unroll
+        for (uint32_t j = 0; j < 8u; ++j) w[8u * k + j] = apply_sign(db * (float)entry[j], (s8 >> j) & 1u);
+    }
+}
+
+// IQ1_M, native/redlite_native_reference.c:149-170: block = 32 index bytes, 16 bytes of nibbles (3 high index bits + the
+// sign of the 1/8 offset), four u16 with 3-bit scales (one per 16 weights) and the f16 d spread over their top nibbles;
+// weight = d * (2 * scale + 1) * (entry + or - 0.125), entry in {-1, 0, 1}
+template <> __device__ __forceinline__ void decode32<T_IQ1_M>(const uint8_t *row, uint32_t chunk, float *w) {
+    const uint8_t *bp = row + (size_t)(chunk >> 3) * 56u;
+    const uint32_t cb = chunk & 7u;
+    uint32_t sc[4];
+#pragma unroll
+    for (uint32_t i = 0; i < 4u; ++i) sc[i] = ld_u16(bp + 48u + 2u * i);
+    const float d = half_bits_to_f32((sc[0] >> 12) | ((sc[1] >> 8) & 0x00f0u) | ((sc[2] >> 4) & 0x0f00u) | (sc[3] & 0xf000u));
+#pragma unroll
+    for (uint32_t k = 0; k < 4u; ++k) {
+        const uint32_t group = 4u * cb + k;
+        const uint32_t nibble = ((uint32_t)bp[32u + (group >> 1)] >> (4u * (group & 1u))) & 15u;
+        const int8_t *entry = g_iq1m_grid + ((uint32_t)bp[group] | ((nibble & 7u) << 8)) * 8u;
+        const float delta = (nibble & 8u) ? -0.125f : 0.125f;
+        const uint32_t si = group >> 1;
+        const float dl = d * (float)(2u * ((sc[si >> 2] >> (3u * (si & 3u))) & 7u) + 1u);
+#pragma unroll
+        for (uint32_t j = 0; j < 8u; ++j) w[8u * k + j] = dl * ((float)entry[j] + delta);
+    }
+}
 
 template <uint32_t T>
 __device__ __forceinline__ float chunk_dot(const uint8_t *row, uint32_t chunk, const float *x33) {
@@ -50,7 +122,7 @@ __global__ __launch_bounds__(256) void dequant_rows_kernel(const uint8_t *rows, 
 hipError_t launch_dequant_rows(uint32_t type, const void *rows, uint32_t nrows, uint32_t ncols, float *out, hipStream_t s) {
     hipError_t e = ensure_tables();
     if (e != hipSuccess) return e;
-    const uint64_t rb = row_bytes(type, ncols);
+    const uint64_t rb = pool_row_bytes(type, ncols);
     if (!rb || ncols % 32u || !nrows) return hipErrorInvalidValue;
     const uint32_t cpr = ncols / 32u;
     const uint64_t total = (uint64_t)nrows * cpr;
@@ -61,6 +133,8 @@ hipError_t launch_dequant_rows(uint32_t type, const void *rows, uint32_t nrows, 
         case T_IQ3_S: REDHIP_LAUNCH(dequant_rows_kernel<T_IQ3_S>, dim3(grid), dim3(256), 0, s, p, rb, nrows, cpr, out); break;
         case T_Q6_K: REDHIP_LAUNCH(dequant_rows_kernel<T_Q6_K>, dim3(grid), dim3(256), 0, s, p, rb, nrows, cpr, out); break;
         case T_F32: REDHIP_LAUNCH(dequant_rows_kernel<T_F32>, dim3(grid), dim3(256), 0, s, p, rb, nrows, cpr, out); break;
+        case T_IQ2_XS: REDHIP_LAUNCH(dequant_rows_kernel<T_IQ2_XS>, dim3(grid), dim3(256), 0, s, p, rb, nrows, cpr, out); break;
+        case T_IQ1_M: REDHIP_LAUNCH(dequant_rows_kernel<T_IQ1_M>, dim3(grid), dim3(256), 0, s, p, rb, nrows, cpr, out); break;
         default: return hipErrorInvalidValue;
     }
     return hipGetLastError();
@@ -86,7 +160,7 @@ __global__ __launch_bounds__(256) void gemv_rows_kernel(const uint8_t *w, uint64
 
 template <uint32_t T>
 static hipError_t gemv_dispatch(const uint8_t *w, uint32_t ncols, uint32_t row_start, uint32_t row_count, const float *x, float *out, hipStream_t s) {
-    const uint64_t rb = row_bytes(T, ncols);
+    const uint64_t rb = pool_row_bytes(T, ncols);
     const uint32_t lpr = lanes_per_row(ncols);
     const dim3 grid((row_count + 256u / lpr - 1u) / (256u / lpr));
     const size_t lds = padded_floats(ncols) * sizeof(float);
@@ -103,13 +177,15 @@ hipError_t launch_gemv_rows(uint32_t type, const void *w, uint32_t ncols, uint32
                             const float *x, float *out, hipStream_t s) {
     hipError_t e = ensure_tables();
     if (e != hipSuccess) return e;
-    if (!row_bytes(type, ncols) || ncols % 256u || !row_count || padded_floats(ncols) * 4u > 160u * 1024u) return hipErrorInvalidValue;
+    if (!pool_row_bytes(type, ncols) || ncols % 256u || !row_count || padded_floats(ncols) * 4u > 160u * 1024u) return hipErrorInvalidValue;
     const uint8_t *p = static_cast<const uint8_t *>(w);
     switch (type) {
         case T_IQ2_XXS: return gemv_dispatch<T_IQ2_XXS>(p, ncols, row_start, row_count, x, out, s);
         case T_IQ3_S: return gemv_dispatch<T_IQ3_S>(p, ncols, row_start, row_count, x, out, s);
         case T_Q6_K: return gemv_dispatch<T_Q6_K>(p, ncols, row_start, row_count, x, out, s);
         case T_F32: return gemv_dispatch<T_F32>(p, ncols, row_start, row_count, x, out, s);
+        case T_IQ2_XS: return gemv_dispatch<T_IQ2_XS>(p, ncols, row_start, row_count, x, out, s);
+        case T_IQ1_M: return gemv_dispatch<T_IQ1_M>(p, ncols, row_start, row_count, x, out, s);
         default: return hipErrorInvalidValue;
     }
 }
@@ -284,6 +360,8 @@ hipError_t launch_moe_gateup(const ExpertSet &ex, const uint32_t *ids, uint32_t 
         case T_IQ2_XXS: return gateup_dispatch<T_IQ2_XXS>(ex, ids, n_slot, hidden, ffn, x, act, s);
         case T_IQ3_S: return gateup_dispatch<T_IQ3_S>(ex, ids, n_slot, hidden, ffn, x, act, s);
         case T_Q6_K: return gateup_dispatch<T_Q6_K>(ex, ids, n_slot, hidden, ffn, x, act, s);
+        case T_IQ2_XS: return gateup_dispatch<T_IQ2_XS>(ex, ids, n_slot, hidden, ffn, x, act, s);
+        case T_IQ1_M: return gateup_dispatch<T_IQ1_M>(ex, ids, n_slot, hidden, ffn, x, act, s);
         default: return hipErrorInvalidValue;
     }
 }

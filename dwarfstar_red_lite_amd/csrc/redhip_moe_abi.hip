@@ -511,6 +511,15 @@ int redhip_moe_group(redhip_moe_t h, const uint32_t *ids_dev, const float *weigh
     return 1;
 }
 
+int redhip_set_codebooks(const int8_t *iq2_xs_grid, uint32_t iq2_xs_count, const int8_t *iq1_m_grid, uint32_t iq1_m_count) {
+    if ((iq2_xs_grid && iq2_xs_count != 512u * 8u) || (iq1_m_grid && iq1_m_count != 2048u * 8u)) {
+        moe_err("codebook size mismatch: IQ2_XS takes 4096 values, IQ1_M 16384");
+        return 0;
+    }
+    HIP_OK(set_caller_grids(iq2_xs_grid, iq1_m_grid), "codebook upload");
+    return 1;
+}
+
 int redhip_dequant_rows(uint32_t ggml_type, const void *rows_dev, uint32_t nrows, uint32_t ncols, float *out_dev, void *stream) {
     if (!rows_dev || !out_dev) { moe_err("null dequant pointer"); return 0; }
     HIP_OK(launch_dequant_rows(ggml_type, rows_dev, nrows, ncols, out_dev, static_cast<hipStream_t>(stream)), "dequant launch");

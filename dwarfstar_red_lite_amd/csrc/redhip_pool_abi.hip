@@ -93,6 +93,7 @@ struct FfnPool {
     DevBuf scratch;
     uint64_t bytes_read = 0, read_calls = 0;
     double read_ms = 0.0;
+    std::vector<int8_t> iq2_xs, iq1_m;            // the caller's codebooks (the reference keeps them in two device buffers per pool)
 
     uint8_t *slot_base(uint32_t slot) {           // nullptr + message on failure
         if (slot >= capacity) { FFN_ERR("FFN slot %u exceeds capacity %u", slot, capacity); return nullptr; }
@@ -145,6 +146,8 @@ redmetal_ffn_pool_t redmetal_ffn_pool_create(const char *model_path, uint64_t bu
     int ndev = 0;
     if (hipGetDeviceCount(&ndev) != hipSuccess || ndev < 1) { FFN_ERR("no HIP device available"); return nullptr; }
     FfnPool *p = new FfnPool();
+    p->iq2_xs.assign(iq2_xs_grid, iq2_xs_grid + iq2_xs_grid_count);      // uploaded when an IQ2_XS / IQ1_M expert is executed
+    p->iq1_m.assign(iq1_m_grid, iq1_m_grid + iq1_m_grid_count);
     p->slot_bytes = aligned;
     p->budget = budget_bytes;
     const uint64_t cap64 = budget_bytes / aligned;
@@ -171,6 +174,7 @@ void redmetal_ffn_pool_destroy(redmetal_ffn_pool_t handle) {
     (void)hipDeviceSynchronize();
     for (uint8_t *s : p->slabs) (void)hipFree(s);
     if (p->fd >= 0) close(p->fd);
+    forget_caller_grids(p);
     delete p;
 }
 
@@ -263,8 +267,8 @@ int redmetal_ffn_pool_execute_expert(redmetal_ffn_pool_t h, uint32_t slot_id, ui
     FfnPool *p = pool_of(h);
     if (!p || !input || !output || slot_id >= p->capacity) return 0;
     const uint32_t gu = word_gate_up(ggml_type), dn = word_down(ggml_type);
-    if (!quant_supported(gu) || !quant_supported(dn) || (ggml_type >> 16)) {
-        FFN_ERR("unsupported FFN GGML type word 0x%x (supported: IQ2_XXS 16, IQ3_S 21, Q6_K 14)", ggml_type);
+    if (!pool_quant_supported(gu) || !pool_quant_supported(dn) || (ggml_type >> 16)) {
+        FFN_ERR("unsupported FFN GGML type word 0x%x (supported: IQ2_XS 17, IQ1_M 29, IQ2_XXS 16, IQ3_S 21, Q6_K 14)", ggml_type);
         return 0;
     }
     if (!hidden_size || hidden_size % 256u || !ffn_size || ffn_size % 256u || input_count != hidden_size ||
@@ -273,8 +277,8 @@ int redmetal_ffn_pool_execute_expert(redmetal_ffn_pool_t h, uint32_t slot_id, ui
         FFN_ERR("invalid FFN dimensions hidden=%u ffn=%u start=%u count=%u", hidden_size, ffn_size, output_row_start, output_row_count);
         return 0;
     }
-    const uint64_t expect_gate = (uint64_t)ffn_size * row_bytes(gu, hidden_size);
-    const uint64_t expect_down = (uint64_t)hidden_size * row_bytes(dn, ffn_size);
+    const uint64_t expect_gate = (uint64_t)ffn_size * pool_row_bytes(gu, hidden_size);
+    const uint64_t expect_down = (uint64_t)hidden_size * pool_row_bytes(dn, ffn_size);
     if (gate_bytes != expect_gate || up_bytes != expect_gate || down_bytes != expect_down) {
         FFN_ERR("FFN matrix byte mismatch gate=%llu/%llu up=%llu/%llu down=%llu/%llu", (unsigned long long)gate_bytes,
                 (unsigned long long)expect_gate, (unsigned long long)up_bytes, (unsigned long long)expect_gate,
@@ -294,6 +298,10 @@ int redmetal_ffn_pool_execute_expert(redmetal_ffn_pool_t h, uint32_t slot_id, ui
     float *dx = static_cast<float *>(p->scratch.p), *dact = dx + n_x, *dout = dact + n_act;
     hipError_t e = hipMemcpy(dx, input, n_x * sizeof(float), hipMemcpyHostToDevice);
     if (e != hipSuccess) { FFN_ERR("FFN input upload failed: %s", hipGetErrorString(e)); return 0; }
+    if (gu == T_IQ2_XS || gu == T_IQ1_M || dn == T_IQ2_XS || dn == T_IQ1_M) {      // this pool's codebooks on the device (free when they already are)
+        e = set_caller_grids(p->iq2_xs.data(), p->iq1_m.data(), p);
+        if (e != hipSuccess) { FFN_ERR("failed to upload the IQ2_XS / IQ1_M codebooks: %s", hipGetErrorString(e)); return 0; }
+    }
     p->mark(slot_id, 1);
     const double t0 = now_ms();
     ExpertSet ex{base, 0, gate_bytes, up_bytes, gu, dn};
@@ -317,17 +325,23 @@ const char *redmetal_quant_last_error(void) { return g_quant_error[0] ? g_quant_
 int redmetal_quant_rows(const char *model_path, uint64_t matrix_file_offset, uint64_t matrix_bytes, uint32_t ggml_type,
         uint32_t ncols, uint32_t nrows, uint32_t row_start, uint32_t row_count, const float *input, uint32_t input_count,
         const int8_t *grid, uint32_t grid_count, float *output, uint32_t output_count, double *io_ms, double *gpu_ms) {
-    (void)grid;
-    (void)grid_count;
     g_quant_error[0] = '\0';
     if (!model_path || !model_path[0] || !input || !output) { QUANT_ERR("invalid Red Metal mixed-quant arguments"); return 0; }
-    if (ggml_type != T_F32 && !quant_supported(ggml_type)) { QUANT_ERR("unsupported GGML type %u", ggml_type); return 0; }
+    if (ggml_type != T_F32 && !pool_quant_supported(ggml_type)) { QUANT_ERR("unsupported GGML type %u", ggml_type); return 0; }
+    if (ggml_type == T_IQ2_XS || ggml_type == T_IQ1_M) {      // these two decode through the caller's codebook, as in the reference
+        const uint32_t want = ggml_type == T_IQ2_XS ? 512u * 8u : 2048u * 8u;
+        if (!grid || grid_count != want) { QUANT_ERR("mixed-quant grid size mismatch: got %u expected %u", grid_count, want); return 0; }
+        if (set_caller_grids(ggml_type == T_IQ2_XS ? grid : nullptr, ggml_type == T_IQ1_M ? grid : nullptr) != hipSuccess) {
+            QUANT_ERR("failed to upload the codebook");
+            return 0;
+        }
+    }
     if (!ncols || ncols % 256u || !nrows || !row_count || row_start >= nrows || row_count > nrows - row_start ||
         input_count != ncols || output_count < row_count) {
         QUANT_ERR("invalid mixed-quant dimensions cols=%u rows=%u start=%u count=%u", ncols, nrows, row_start, row_count);
         return 0;
     }
-    const uint64_t rb = row_bytes(ggml_type, ncols);
+    const uint64_t rb = pool_row_bytes(ggml_type, ncols);
     if (!rb || (uint64_t)nrows > UINT64_MAX / rb || matrix_bytes != (uint64_t)nrows * rb) {
         QUANT_ERR("matrix byte size mismatch: got %llu expected %llu", (unsigned long long)matrix_bytes, (unsigned long long)((uint64_t)nrows * rb));
         return 0;

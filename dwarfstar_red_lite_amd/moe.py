@@ -173,6 +173,16 @@ def gguf_moe_config(path, first_layer=0):
     return cfg, c.n_layer
 
 
+def set_codebooks(iq2_xs_grid=None, iq1_m_grid=None):
+    """upload the int8 codebooks (512 x 8 and 2048 x 8 values) that IQ2_XS / IQ1_M rows decode through."""
+    lib = load()
+    a = np.ascontiguousarray(iq2_xs_grid, np.int8).ravel() if iq2_xs_grid is not None else None
+    b = np.ascontiguousarray(iq1_m_grid, np.int8).ravel() if iq1_m_grid is not None else None
+    if not lib.redhip_set_codebooks(a.ctypes.data if a is not None else None, a.size if a is not None else 0,
+                                    b.ctypes.data if b is not None else None, b.size if b is not None else 0):
+        raise RedHipError(lib.redhip_moe_last_error().decode())
+
+
 def dequant_rows(ggml_type, rows, ncols):
     """rows: uint8 CUDA tensor [nrows, row_bytes] of raw GGUF blocks -> float32 [nrows, ncols]."""
     lib = load()

@@ -13,14 +13,16 @@ ExpertLayout = namedtuple("ExpertLayout", "gate_offset gate_bytes up_offset up_b
 
 
 class RedMetalFfnPool:
-    def __init__(self, model, budget_bytes, slot_bytes, *, slots_per_slab=64):
+    def __init__(self, model, budget_bytes, slot_bytes, *, slots_per_slab=64, iq2_xs_grid=None, iq1_m_grid=None):
         if budget_bytes <= 0 or slot_bytes <= 0:
             raise ValueError("budget_bytes and slot_bytes must be positive")
         self.lib = load()
-        # the pool keeps the reference's signature: two codebook arguments with exact element counts; the HIP
-        # library carries its own codebooks and ignores their contents
-        self._iq2 = (C.c_int8 * (512 * 8))()
-        self._iq1 = (C.c_int8 * (2048 * 8))()
+        # the reference's signature: two int8 codebooks with exact element counts (it reads them from a llama.cpp checkout,
+        # redlite/quant_tables.py). The caller passes them here; without them the pool still serves the formats that carry
+        # their own tables, and execute() refuses IQ2_XS / IQ1_M
+        self._have_grids = iq2_xs_grid is not None and iq1_m_grid is not None
+        self._iq2 = (C.c_int8 * (512 * 8))(*(np.asarray(iq2_xs_grid, np.int8).ravel().tolist() if iq2_xs_grid is not None else ()))
+        self._iq1 = (C.c_int8 * (2048 * 8))(*(np.asarray(iq1_m_grid, np.int8).ravel().tolist() if iq1_m_grid is not None else ()))
         self.model = os.path.abspath(os.path.expanduser(str(model)))
         self.handle = self.lib.redmetal_ffn_pool_create(os.fsencode(self.model), int(budget_bytes), int(slot_bytes),
                                                         int(slots_per_slab), self._iq2, len(self._iq2), self._iq1, len(self._iq1))
@@ -69,6 +71,8 @@ class RedMetalFfnPool:
         x = np.ascontiguousarray(input_values, np.float32)
         if x.size != hidden_size:
             raise ValueError("input has %d values, expected %d" % (x.size, hidden_size))
+        if not self._have_grids and {ggml_type & 255, (ggml_type >> 8) & 255} & {17, 29}:
+            raise ValueError("IQ2_XS / IQ1_M experts need the pool created with iq2_xs_grid and iq1_m_grid")
         out = np.zeros(max(output_row_count, 1), np.float32)
         ms = C.c_double()
         ok = self.lib.redmetal_ffn_pool_execute_expert(self.handle, slot_id, int(ggml_type), layout.gate_bytes, layout.up_bytes,

@@ -6,12 +6,12 @@ uniformly from a realistic range. The same seed gives the same bytes on every ma
 """
 import numpy as np
 
-TYPE_F32, TYPE_Q6_K, TYPE_IQ2_XXS, TYPE_IQ3_S = 0, 14, 16, 21
-BLOCK_BYTES = {TYPE_Q6_K: 210, TYPE_IQ2_XXS: 66, TYPE_IQ3_S: 110}
-D_OFFSET = {TYPE_Q6_K: 208, TYPE_IQ2_XXS: 0, TYPE_IQ3_S: 0}
+TYPE_F32, TYPE_Q6_K, TYPE_IQ2_XXS, TYPE_IQ2_XS, TYPE_IQ3_S, TYPE_IQ1_M = 0, 14, 16, 17, 21, 29
+BLOCK_BYTES = {TYPE_Q6_K: 210, TYPE_IQ2_XXS: 66, TYPE_IQ3_S: 110, TYPE_IQ2_XS: 74, TYPE_IQ1_M: 56}
+D_OFFSET = {TYPE_Q6_K: 208, TYPE_IQ2_XXS: 0, TYPE_IQ3_S: 0, TYPE_IQ2_XS: 0}
 # default fp16 scale ranges: IQ formats as in the benchmark definition; Q6_K smaller because its integer part
 # (int8 scale x 6-bit quant) is ~70x larger
-D_RANGE = {TYPE_IQ2_XXS: (1e-3, 2e-2), TYPE_IQ3_S: (1e-3, 2e-2), TYPE_Q6_K: (1e-4, 5e-4)}
+D_RANGE = {TYPE_IQ2_XXS: (1e-3, 2e-2), TYPE_IQ3_S: (1e-3, 2e-2), TYPE_Q6_K: (1e-4, 5e-4), TYPE_IQ2_XS: (1e-3, 2e-2), TYPE_IQ1_M: (1e-3, 2e-2)}
 
 
 def row_bytes(t, ncols):
@@ -28,6 +28,10 @@ def quant_rows(rng, t, nrows, ncols, d_range=None):
     raw = rng.integers(0, 256, size=(nb, bb), dtype=np.uint8)
     lo, hi = d_range or D_RANGE[t]
     d = rng.uniform(lo, hi, size=nb).astype(np.float16).view(np.uint16)
+    if t == TYPE_IQ1_M:          # d is spread over the top nibbles of the four 16-bit scale words (bytes 48..55)
+        for i in range(4):
+            raw[:, 49 + 2 * i] = (raw[:, 49 + 2 * i] & 0x0f) | ((((d >> (4 * i)) & 15) << 4).astype(np.uint8))
+        return raw.reshape(nrows, -1)
     raw[:, D_OFFSET[t]] = (d & 255).astype(np.uint8)
     raw[:, D_OFFSET[t] + 1] = (d >> 8).astype(np.uint8)
     return raw.reshape(nrows, -1)

@@ -95,6 +95,12 @@ int redhip_moe_group(redhip_moe_t moe, const uint32_t *ids_dev, const float *wei
     uint32_t *uid_dev, uint32_t *expert_start_dev, uint32_t *pair_token_dev, float *pair_weight_dev,
     uint32_t *tok_pair_dev, uint32_t *n_unique_dev, void *stream);
 
+/* The int8 codebooks of IQ2_XS (512 x 8) and IQ1_M (2048 x 8) that type 17 / 29 rows decode through, copied to the device
+ * for the taps below; either may be NULL to keep what is there. The reference hands the same two tables to
+ * redmetal_ffn_pool_create and redmetal_quant_rows (native/redmetal_ffn.h:9-18, native/redmetal_quant.h:9-27), which upload
+ * them too. Process-wide; synchronous. */
+int redhip_set_codebooks(const int8_t *iq2_xs_grid, uint32_t iq2_xs_count, const int8_t *iq1_m_grid, uint32_t iq1_m_count);
+
 /* Parity tap: f32 dequantisation of `rows` rows of `ncols` weights of raw GGUF blocks (device pointers). */
 int redhip_dequant_rows(uint32_t ggml_type, const void *rows_dev, uint32_t nrows, uint32_t ncols, float *out_dev, void *stream);
 /* Parity tap: dequantise one resident matrix (which: 0 gate, 1 up, 2 down; expert == n_expert: shared expert;

@@ -136,6 +136,52 @@ static void deq_q6k_block(const uint8_t *bp, float *y) {
     }
 }
 
+/* ---- IQ2_XS / IQ1_M, native/redlite_native_reference.c:60-172 ---- */
+
+static uint32_t rd16(const uint8_t *p) { return (uint32_t)p[0] | ((uint32_t)p[1] << 8); }
+
+/* weight i (0..255) of one block as the double the reference multiplies the activation with */
+static double xs_m_weight(uint32_t type, const uint8_t *bp, const int8_t *grid, uint32_t i) {
+    if (type == 17u) {                                             /* :122-142 */
+        const double d = (double)orc_f16_to_f32((uint16_t)rd16(bp));
+        const uint32_t group = i >> 4, part = (i >> 3) & 1u, j = i & 7u;
+        const uint32_t scale = (bp[66u + (group >> 1)] >> (4u * (group & 1u))) & 0x0fu;
+        const double db = d * (0.5 + (double)scale) * 0.25;
+        const uint32_t q = rd16(bp + 2u + 2u * (2u * group + part));
+        uint32_t s7 = (q >> 9) & 0x7fu, parity = 0u;
+        for (uint32_t v = s7; v; v >>= 1) parity ^= v & 1u;       /* sign_byte, :60-69 */
+        const uint32_t signs = s7 | (parity << 7);
+        return db * (double)grid[(q & 0x01ffu) * 8u + j] * ((signs >> j) & 1u ? -1.0 : 1.0);
+    }
+    /* IQ1_M, :149-170 */
+    uint32_t sc[4];
+    for (uint32_t k = 0; k < 4u; ++k) sc[k] = rd16(bp + 48u + 2u * k);
+    const uint32_t d_bits = (sc[0] >> 12) | ((sc[1] >> 8) & 0x00f0u) | ((sc[2] >> 4) & 0x0f00u) | (sc[3] & 0xf000u);
+    const double d = (double)orc_f16_to_f32((uint16_t)d_bits);
+    const uint32_t group = i >> 3, j = i & 7u;
+    const uint32_t nibble = (bp[32u + (group >> 1)] >> (4u * (group & 1u))) & 0x0fu;
+    const uint32_t grid_index = (uint32_t)bp[group] | ((nibble & 7u) << 8);
+    const double delta = (nibble & 8u) ? -0.125 : 0.125;
+    const uint32_t scale_index = group >> 1, scale = (sc[scale_index >> 2] >> (3u * (scale_index & 3u))) & 7u;
+    return d * (double)(2u * scale + 1u) * ((double)grid[grid_index * 8u + j] + delta);
+}
+
+int orc_dequant_row_grid(uint32_t type, const uint8_t *row, uint32_t ncols, const int8_t *grid, float *out) {
+    if (!row || !grid || !out || !ncols || ncols % QK || (type != 17u && type != 29u)) return 0;
+    const size_t bb = type == 17u ? 74u : 56u;
+    for (uint32_t i = 0; i < ncols; ++i) out[i] = (float)xs_m_weight(type, row + (size_t)(i / QK) * bb, grid, i % QK);
+    return 1;
+}
+
+int orc_row_dot_grid(uint32_t type, const uint8_t *row, const float *x, uint32_t ncols, const int8_t *grid, double *out) {
+    if (!row || !grid || !x || !out || !ncols || ncols % QK || (type != 17u && type != 29u)) return 0;
+    const size_t bb = type == 17u ? 74u : 56u;
+    double acc = 0.0;
+    for (uint32_t i = 0; i < ncols; ++i) acc += (double)x[i] * xs_m_weight(type, row + (size_t)(i / QK) * bb, grid, i % QK);
+    *out = acc;
+    return 1;
+}
+
 /* native/redlite_native_quant_cpu.c:155-196 (types 0, 14, 16 and the IQ3 delegation) */
 int orc_dequant_row(uint32_t type, const uint8_t *row, uint32_t ncols, float *out) {
     if (!row || !out || !ncols) return 0;
@@ -417,6 +463,47 @@ static int routed_topk_mt(uint32_t gu_type, uint32_t dn_type,
         if (ok) for (uint32_t r = 0; r < hidden; ++r) out[r] += (double)weights[k] * tmp[r];
     }
     free(tmp);
+    return ok;
+}
+
+/* one row dot for any pool type: the two codebook formats go through the caller's grids (native/redlite_native_reference.c:78-172,
+ * float or double activations), the rest through dot_any */
+static int pool_row_dot(uint32_t type, const uint8_t *row, const float *xf, const double *xd, uint32_t ncols,
+                        const int8_t *xs_grid, const int8_t *m_grid, double *out) {
+    if (type != 17u && type != 29u) return dot_any(type, row, xf, xd, ncols, out);
+    const int8_t *grid = type == 17u ? xs_grid : m_grid;
+    if (!grid || ncols % QK) return 0;
+    const size_t bb = type == 17u ? 74u : 56u;
+    double acc = 0.0;
+    for (uint32_t i = 0; i < ncols; ++i)
+        acc += (xd ? xd[i] : (double)xf[i]) * xs_m_weight(type, row + (size_t)(i / QK) * bb, grid, i % QK);
+    *out = acc;
+    return 1;
+}
+
+static size_t pool_row_bytes(uint32_t type, uint32_t ncols) {
+    if (type == 17u || type == 29u) return ncols % QK ? 0u : (size_t)(ncols / QK) * (type == 17u ? 74u : 56u);
+    return orc_row_bytes(type, ncols);
+}
+
+/* native/redlite_native_reference.c:267-305 with the codebook formats (types 17 and 29) allowed on either side */
+int orc_expert_ffn_grid(uint32_t gate_up_type, uint32_t down_type, const uint8_t *gate, const uint8_t *up, const uint8_t *down,
+                        uint32_t hidden, uint32_t ffn, uint32_t row_start, uint32_t row_count, const float *x,
+                        const int8_t *xs_grid, const int8_t *m_grid, double *out) {
+    const size_t grb = pool_row_bytes(gate_up_type, hidden), drb = pool_row_bytes(down_type, ffn);
+    if (!gate || !up || !down || !x || !out || !grb || !drb || !row_count || row_start >= hidden || row_count > hidden - row_start) return 0;
+    double *a = (double *)malloc(sizeof(double) * (size_t)ffn);
+    if (!a) return 0;
+    int ok = 1;
+    for (uint32_t i = 0; i < ffn && ok; ++i) {
+        double g = 0.0, u = 0.0;
+        ok = pool_row_dot(gate_up_type, gate + (size_t)i * grb, x, NULL, hidden, xs_grid, m_grid, &g) &&
+             pool_row_dot(gate_up_type, up + (size_t)i * grb, x, NULL, hidden, xs_grid, m_grid, &u);
+        a[i] = orc_silu_mul(g, u);
+    }
+    for (uint32_t r = 0; r < row_count && ok; ++r)
+        ok = pool_row_dot(down_type, down + (size_t)(row_start + r) * drb, NULL, a, ffn, xs_grid, m_grid, &out[r]);
+    free(a);
     return ok;
 }
 

@@ -41,6 +41,15 @@ size_t orc_row_bytes(uint32_t type, uint32_t ncols);   /* 0 = unsupported */
 int orc_dequant_row(uint32_t type, const uint8_t *row, uint32_t ncols, float *out);
 int orc_row_dot(uint32_t type, const uint8_t *row, const float *x, uint32_t ncols, double *out);
 int orc_row_dot_d(uint32_t type, const uint8_t *row, const double *x, uint32_t ncols, double *out);
+/* IQ2_XS (17, 74-byte blocks) and IQ1_M (29, 56-byte blocks): the reference's current routed-expert formats. Their
+ * codebooks are arguments, as in the reference (512 x 8 resp. 2048 x 8 int8 values, native/redlite_native_tables.c).
+ * Dequantised weights (exact in f32) and the double-accumulated row dot of native/redlite_native_reference.c:116-172. */
+int orc_dequant_row_grid(uint32_t type, const uint8_t *row, uint32_t ncols, const int8_t *grid, float *out);
+int orc_row_dot_grid(uint32_t type, const uint8_t *row, const float *x, uint32_t ncols, const int8_t *grid, double *out);
+/* single-expert FFN where either side may be a codebook format (17 / 29); other types as orc_expert_ffn */
+int orc_expert_ffn_grid(uint32_t gate_up_type, uint32_t down_type, const uint8_t *gate, const uint8_t *up, const uint8_t *down,
+                        uint32_t hidden, uint32_t ffn, uint32_t row_start, uint32_t row_count, const float *x,
+                        const int8_t *xs_grid, const int8_t *m_grid, double *out);
 
 /* out[r] = (float) row_dot(W[row_start + r], x); rows split over `threads` pthreads like the reference's matvec */
 int orc_matvec(uint32_t type, const uint8_t *w, uint32_t ncols, uint32_t row_start, uint32_t row_count,

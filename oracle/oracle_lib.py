@@ -57,6 +57,10 @@ def lib():
         L.orc_dequant_row.argtypes = [C.c_uint32, C.c_void_p, C.c_uint32, C.c_void_p]
         L.orc_row_dot.argtypes = [C.c_uint32, C.c_void_p, C.c_void_p, C.c_uint32, f64p]
         L.orc_row_dot_d.argtypes = [C.c_uint32, C.c_void_p, C.c_void_p, C.c_uint32, f64p]
+        L.orc_dequant_row_grid.argtypes = [C.c_uint32, C.c_void_p, C.c_uint32, C.c_void_p, C.c_void_p]
+        L.orc_row_dot_grid.argtypes = [C.c_uint32, C.c_void_p, C.c_void_p, C.c_uint32, C.c_void_p, f64p]
+        L.orc_expert_ffn_grid.argtypes = [C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32,
+                                          C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
         L.orc_matvec.argtypes = [C.c_uint32, C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p, C.c_int]
         L.orc_rmsnorm.restype = None
         L.orc_rmsnorm.argtypes = [C.c_void_p, C.c_void_p, C.c_uint32, C.c_float, C.c_void_p]
@@ -216,3 +220,31 @@ def group_pairs(ids, weights, n_expert):
     if U < 0:
         raise ValueError("bad grouping arguments")
     return uid[:U].copy(), start[:U + 1].copy(), ptok, pw, tp
+
+
+def dequant_rows_grid(t, rows, ncols, grid):
+    """float32 [nrows, ncols] of IQ2_XS (17) / IQ1_M (29) rows; grid: int8 codebook of the type."""
+    rows = np.ascontiguousarray(rows, np.uint8).reshape(-1, rows.shape[-1])
+    grid = np.ascontiguousarray(grid, np.int8)
+    out = np.empty((rows.shape[0], ncols), np.float32)
+    for r in range(rows.shape[0]):
+        assert lib().orc_dequant_row_grid(t, _p(rows[r]), ncols, _p(grid), _p(out[r]))
+    return out
+
+
+def row_dot_grid(t, row, x, grid):
+    row, x, grid = np.ascontiguousarray(row, np.uint8), np.ascontiguousarray(x, np.float32), np.ascontiguousarray(grid, np.int8)
+    d = C.c_double()
+    assert lib().orc_row_dot_grid(t, _p(row), _p(x), x.size, _p(grid), C.byref(d))
+    return d.value
+
+
+def expert_ffn_grid(gu_t, dn_t, gate, up, down, hidden, ffn, x, xs_grid, m_grid, row_start=0, row_count=None):
+    """single-expert FFN in double where either side may be IQ2_XS (17) / IQ1_M (29)."""
+    row_count = hidden - row_start if row_count is None else row_count
+    x = np.ascontiguousarray(x, np.float32)
+    xs_grid, m_grid = np.ascontiguousarray(xs_grid, np.int8), np.ascontiguousarray(m_grid, np.int8)
+    out = np.zeros(row_count, np.float64)
+    assert lib().orc_expert_ffn_grid(gu_t, dn_t, _p(_bytes(gate)), _p(_bytes(up)), _p(_bytes(down)), hidden, ffn, row_start, row_count,
+                                     _p(x), _p(xs_grid), _p(m_grid), _p(out))
+    return out

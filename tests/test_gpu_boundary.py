@@ -61,7 +61,7 @@ def test_quant_rows(model_file):
     with pytest.raises(RedHipError, match="matrix byte size mismatch"):
         br.rows(path, off, n - 66, T_IQ2, H, F, 0, 1, x)
     with pytest.raises(RedHipError, match="unsupported GGML type"):
-        br.rows(path, off, n, 17, H, F, 0, 1, x)
+        br.rows(path, off, n, 18, H, F, 0, 1, x)
     with pytest.raises(RedHipError, match="invalid mixed-quant dimensions"):
         br.rows(path, off, n, T_IQ2, H, F, F, 1, x)
     with pytest.raises(RedHipError, match="invalid pread range"):
@@ -98,7 +98,7 @@ def test_ffn_pool(model_file):
         assert tel["slab_count"] == 3 and tel["allocated_bytes"] == 5 * aligned and tel["read_calls"] >= 21
         lay = ExpertLayout(*index["iq2.gate.0"], *index["iq2.up.0"], *index["iq2.down.0"])
         with pytest.raises(RedHipError, match="unsupported FFN GGML type"):
-            pool.execute(1, lay, 17, H, F, 0, H, x)
+            pool.execute(1, lay, 18, H, F, 0, H, x)
         with pytest.raises(RedHipError, match="FFN matrix byte mismatch"):
             pool.execute(1, lay._replace(gate_bytes=lay.gate_bytes - 66), T_IQ2, H, F, 0, H, x)
         with pytest.raises(RedHipError, match="invalid FFN dimensions"):

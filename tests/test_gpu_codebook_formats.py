@@ -1,0 +1,164 @@
+"""GPU parity of the two formats that decode through caller-supplied codebooks, IQ2_XS (type 17) and IQ1_M (type 29), on the
+surfaces that accept them: the dequantisation / GEMV taps, redmetal_quant_rows and the single-expert pool. The codebooks are the
+reference's own tables (golden fixture), handed over the way the reference hands them."""
+import json
+import os
+import struct
+
+import numpy as np
+import pytest
+
+import oracle_lib as orc
+from dwarfstar_red_lite_amd import expert_type_word, synth
+from gpu_common import REL_L2_TOL, T_IQ2, rel_l2
+
+pytestmark = pytest.mark.gpu
+torch = pytest.importorskip("torch")
+
+T_XS, T_M = 17, 29
+
+
+def dev(a):
+    return torch.from_numpy(np.array(a, copy=True)).cuda()
+
+
+@pytest.fixture(scope="module")
+def grids(golden_dir):
+    from dwarfstar_red_lite_amd import moe
+    g = json.load(open(os.path.join(golden_dir, "iq_grids.json")))
+    xs = np.frombuffer(bytes.fromhex(g["iq2_xs"]), np.int8)
+    m = np.frombuffer(bytes.fromhex(g["iq1_m"]), np.int8)
+    moe.set_codebooks(xs, m)
+    return xs, m
+
+
+def edge_rows(t, ncols):
+    """all-zero, all-one and extreme-scale blocks beside seeded ones"""
+    rng = np.random.default_rng(4321 + t)
+    rows = synth.quant_rows(rng, t, 6, ncols)
+    bb = synth.BLOCK_BYTES[t]
+    r = rows.reshape(6, -1, bb)
+    r[1] = 0
+    r[2] = 0xFF                  # every index, sign and scale bit set; d = NaN pattern for IQ2_XS is avoided below
+    if t == T_XS:
+        r[2, :, 0], r[2, :, 1] = 0x00, 0x3C          # d = 1
+        r[3, :, 0], r[3, :, 1] = 0x01, 0x00          # smallest subnormal d
+        r[4, :, 1] |= 0x80                           # negative d
+        r[5, :, 0], r[5, :, 1] = 0xFF, 0x7B          # 65504
+    else:
+        for i, nib in enumerate((0x0, 0x0, 0xC, 0x3)):          # d = 1.0 spread over the four top nibbles
+            r[2, :, 49 + 2 * i] = (r[2, :, 49 + 2 * i] & 0x0F) | (nib << 4)
+        r[3, :, 49::2] &= 0x0F                        # d = 0
+        r[3, :, 49] |= 0x10                           # ... then the smallest subnormal
+        r[4, :, 55] |= 0x80                           # negative d
+        for i, nib in enumerate((0xF, 0xF, 0xB, 0x7)):          # 65504
+            r[5, :, 49 + 2 * i] = (r[5, :, 49 + 2 * i] & 0x0F) | (nib << 4)
+    return rows
+
+
+@pytest.mark.parametrize("t", [T_XS, T_M])
+def test_dequant_bit_exact(t, grids):
+    from dwarfstar_red_lite_amd import moe
+    grid = grids[0] if t == T_XS else grids[1]
+    rng = np.random.default_rng(300 + t)
+    for ncols in (256, 512, 2048):
+        rows = np.concatenate([synth.quant_rows(rng, t, 37, ncols), edge_rows(t, ncols)])
+        got = moe.dequant_rows(t, dev(rows), ncols).cpu().numpy()
+        want = orc.dequant_rows_grid(t, rows, ncols, grid)
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (t, ncols)
+
+
+def test_golden_rows(golden_dir, grids):
+    """the rows the compiled reference was run on: dequantisation against the oracle, the dot against the reference's own"""
+    from dwarfstar_red_lite_amd import moe
+    g = json.load(open(os.path.join(golden_dir, "quant_rows_xs_m.json")))
+    for c in g["cases"]:
+        t, n = c["type"], c["ncols"]
+        row = np.frombuffer(bytes.fromhex(c["row"]), np.uint8).reshape(1, -1)
+        x = np.frombuffer(bytes.fromhex(c["x"]), np.float32)
+        want = struct.unpack("<d", bytes.fromhex(c["dot"]))[0]
+        w = orc.dequant_rows_grid(t, row, n, grids[0] if t == T_XS else grids[1])
+        got_w = moe.dequant_rows(t, dev(row), n).cpu().numpy()
+        assert np.array_equal(got_w.view(np.uint32), w.view(np.uint32)), (t, n, c["fill"])
+        got = float(moe.gemv_rows(t, dev(row), n, dev(x)).cpu().numpy()[0])
+        scale = float(np.abs(w.astype(np.float64) * x).sum())
+        assert abs(got - want) <= 2e-5 * scale + 1e-30, (t, n, c["fill"], got, want)
+
+
+@pytest.mark.parametrize("t", [T_XS, T_M])
+def test_gemv_rows(t, grids):
+    from dwarfstar_red_lite_amd import moe
+    grid = grids[0] if t == T_XS else grids[1]
+    rng = np.random.default_rng(400 + t)
+    for ncols in (256, 512, 1024, 2048):
+        nrows = 37
+        w = synth.quant_rows(rng, t, nrows, ncols)
+        x = rng.standard_normal(ncols).astype(np.float32)
+        want = np.array([orc.row_dot_grid(t, w[r], x, grid) for r in range(nrows)])
+        got = moe.gemv_rows(t, dev(w), ncols, dev(x)).cpu().numpy()
+        scale = np.abs(orc.dequant_rows_grid(t, w, ncols, grid).astype(np.float64) * x).sum(axis=1)
+        assert np.max(np.abs(got - want) / scale) <= 2e-5, (t, ncols)
+        assert rel_l2(got, want) <= REL_L2_TOL
+        part = moe.gemv_rows(t, dev(w), ncols, dev(x), row_start=5, row_count=9).cpu().numpy()
+        assert np.array_equal(part, got[5:14])
+
+
+@pytest.fixture(scope="module")
+def model_file(tmp_path_factory):
+    H, F = 512, 256
+    rng = np.random.default_rng(78)
+    parts, off, index = [np.zeros(10, np.uint8)], 10, {}
+    for fam, gu, dn in (("xs", T_XS, T_XS), ("m", T_M, T_M), ("m_xs", T_M, T_XS), ("xs_iq2", T_XS, T_IQ2)):
+        for name, t, nr, nc in (("gate", gu, F, H), ("up", gu, F, H), ("down", dn, H, F)):
+            b = synth.quant_rows(rng, t, nr, nc).ravel()
+            index[fam + "." + name] = (off, b.size)
+            parts.append(b)
+            off += b.size
+    blob = np.concatenate(parts)
+    path = tmp_path_factory.mktemp("model_xs_m") / "raw_blocks.bin"
+    blob.tofile(path)
+    return str(path), blob, index, H, F
+
+
+def test_quant_rows(model_file, grids):
+    from dwarfstar_red_lite_amd import RedHipError
+    from dwarfstar_red_lite_amd.redmetal_quant import RedMetalQuantBridge
+    path, blob, index, H, F = model_file
+    br = RedMetalQuantBridge()
+    x = synth.normed_x(np.random.default_rng(5), 1, H)[0]
+    for name, t, ncols, nrows, grid in (("xs.gate", T_XS, H, F, grids[0]), ("m.down", T_M, F, H, grids[1])):
+        off, n = index[name]
+        xin = x[:ncols]
+        out, _, _ = br.rows(path, off, n, t, ncols, nrows, 3, 11, xin, grid=grid)
+        w = blob[off:off + n].reshape(nrows, -1)
+        want = np.array([orc.row_dot_grid(t, w[r], xin, grid) for r in range(3, 14)])
+        assert rel_l2(out, want) <= REL_L2_TOL, name
+        with pytest.raises(RedHipError, match="grid size mismatch"):
+            br.rows(path, off, n, t, ncols, nrows, 0, 1, xin)
+        with pytest.raises(RedHipError, match="grid size mismatch"):
+            br.rows(path, off, n, t, ncols, nrows, 0, 1, xin, grid=grid[:-8])
+
+
+def test_ffn_pool(model_file, grids):
+    from dwarfstar_red_lite_amd.redmetal_ffn import ExpertLayout, RedMetalFfnPool
+    path, blob, index, H, F = model_file
+    xs, m = grids
+    x = synth.normed_x(np.random.default_rng(6), 1, H)[0]
+    slot_bytes = max(sum(index[f + "." + n][1] for n in ("gate", "up", "down")) for f in ("xs", "m", "m_xs", "xs_iq2"))
+    sl = lambda o, n: blob[o:o + n]
+    with RedMetalFfnPool(path, 8 * (slot_bytes + 4096), slot_bytes, iq2_xs_grid=xs, iq1_m_grid=m) as pool:
+        for slot, (fam, gu, dn) in enumerate((("xs", T_XS, T_XS), ("m", T_M, T_M), ("m_xs", T_M, T_XS), ("xs_iq2", T_XS, T_IQ2))):
+            lay = ExpertLayout(*index[fam + ".gate"], *index[fam + ".up"], *index[fam + ".down"])
+            pool.load(slot, lay)
+            want = orc.expert_ffn_grid(gu, dn, sl(lay.gate_offset, lay.gate_bytes), sl(lay.up_offset, lay.up_bytes),
+                                       sl(lay.down_offset, lay.down_bytes), H, F, x, xs, m)
+            out, _ = pool.execute(slot, lay, expert_type_word(gu, dn), H, F, 0, H, x)
+            assert rel_l2(out, want) <= REL_L2_TOL, fam
+            win, _ = pool.execute(slot, lay, expert_type_word(gu, dn), H, F, 500, 12, x)
+            assert np.array_equal(win, out[500:])
+    # a pool made without codebooks serves the other formats and says so for these two
+    with RedMetalFfnPool(path, 2 * (slot_bytes + 4096), slot_bytes) as pool:
+        lay = ExpertLayout(*index["xs.gate"], *index["xs.up"], *index["xs.down"])
+        pool.load(0, lay)
+        with pytest.raises(ValueError, match="need the pool created with"):
+            pool.execute(0, lay, T_XS, H, F, 0, H, x)

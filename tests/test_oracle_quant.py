@@ -176,3 +176,97 @@ def test_matvec_threads_identical():
     c = orc.matvec(T_IQ2, w, 512, x, row_start=10, row_count=20, threads=3)
     assert np.array_equal(a, b) and np.array_equal(a[10:30], c)
     assert a[7] == np.float32(orc.row_dot(T_IQ2, w[7], x))
+
+
+def load_iq_grids(golden_dir):
+    g = json.load(open(os.path.join(golden_dir, "iq_grids.json")))
+    return np.frombuffer(bytes.fromhex(g["iq2_xs"]), np.int8), np.frombuffer(bytes.fromhex(g["iq1_m"]), np.int8), g
+
+
+def fnv1a64(data):
+    h = 1469598103934665603          # the reference's offset basis (native/redlite_native_tables.c:272), not the textbook one
+    for b in data.tobytes():
+        h = ((h ^ b) * 0x100000001b3) & 0xffffffffffffffff
+    return h
+
+
+def test_iq2xs_iq1m_codebooks(golden_dir):
+    xs, m, g = load_iq_grids(golden_dir)
+    assert xs.size == 512 * 8 and m.size == 2048 * 8
+    assert set(np.unique(xs).tolist()) == {8, 25, 43} and set(np.unique(m).tolist()) == {-1, 0, 1}
+    # the digests the reference computes over the same tables (rl_native_quant_table_fnv1a)
+    assert "%016x" % fnv1a64(xs) == g["iq2_xs_fnv1a"] and "%016x" % fnv1a64(m) == g["iq1_m_fnv1a"]
+    assert len({xs[8 * i:8 * i + 8].tobytes() for i in range(512)}) == 512          # a codebook has no repeated entry
+    assert len({m[8 * i:8 * i + 8].tobytes() for i in range(2048)}) == 2048
+
+
+def test_golden_rows_iq2xs_iq1m(golden_dir):
+    """the reference's own row dot (rl_native_quant_row_dot) on seeded rows, bit for bit; the dequantised row is exact in
+    f32, so its double dot with x must agree with the reference's to rounding"""
+    xs, m, _ = load_iq_grids(golden_dir)
+    g = json.load(open(os.path.join(golden_dir, "quant_rows_xs_m.json")))
+    seen = set()
+    for c in g["cases"]:
+        t, n = c["type"], c["ncols"]
+        grid = xs if t == 17 else m
+        row = unhex(c["row"], np.uint8)
+        x = unhex(c["x"], np.float32)
+        want = struct.unpack("<d", bytes.fromhex(c["dot"]))[0]
+        assert orc.row_dot_grid(t, row, x, grid) == want, (t, n, c["fill"])
+        w = orc.dequant_rows_grid(t, row, n, grid)[0]
+        brute = float(np.dot(w.astype(np.float64), x.astype(np.float64)))
+        assert abs(brute - want) <= 1e-9 * max(1.0, np.abs(w.astype(np.float64) * x).sum())
+        seen.add((t, c["fill"]))
+    assert {(17, 0), (29, 0), (17, 3), (29, 3), (17, 4), (29, 4)} <= seen
+
+
+def test_iq2xs_iq1m_known_blocks(golden_dir):
+    """hand-built blocks: every field decoded where the format says it is"""
+    xs, m, _ = load_iq_grids(golden_dir)
+    blk = np.zeros(74, np.uint8)
+    blk[0:2] = np.frombuffer(np.float16(2.0).tobytes(), np.uint8)
+    q = 5 | (0b0000011 << 9)                    # entry 5, signs on weights 0 and 1, even parity: weight 7 positive
+    blk[2 + 2 * 3:2 + 2 * 3 + 2] = [q & 255, q >> 8]         # group 1, part 1 -> weights 24..31
+    blk[66] = 0x70                              # scale 7 for group 1 (high nibble of byte 0)
+    w = orc.dequant_rows_grid(17, blk[None, :], 256, xs)[0]
+    db = 2.0 * (0.5 + 7) * 0.25
+    want = db * xs[40:48].astype(np.float64) * np.array([-1, -1, 1, 1, 1, 1, 1, 1])
+    assert np.array_equal(w[24:32], want.astype(np.float32))
+    assert np.array_equal(w[0:8], (2.0 * 0.5 * 0.25 * xs[0:8]).astype(np.float32))      # entry 0, scale 0, no signs
+    blk = np.zeros(56, np.uint8)
+    d = int(np.frombuffer(np.float16(0.5).tobytes(), np.uint16)[0])
+    sc = [((d >> (4 * i)) & 15) << 12 for i in range(4)]
+    sc[0] |= 3 << 3                             # scale index 1 (groups 2, 3) = 3
+    for i in range(4):
+        blk[48 + 2 * i] = sc[i] & 255
+        blk[49 + 2 * i] = sc[i] >> 8
+    blk[2] = 0x34                               # group 2: low grid bits
+    blk[32 + 1] = 0x0a                          # group 2 nibble: delta negative, high grid bits 2
+    w = orc.dequant_rows_grid(29, blk[None, :], 256, m)[0]
+    gi = 0x34 | (2 << 8)
+    want = 0.5 * 7 * (m[8 * gi:8 * gi + 8].astype(np.float64) - 0.125)
+    assert np.array_equal(w[16:24], want.astype(np.float32))
+    assert np.array_equal(w[0:8], (0.5 * 1 * (m[0:8].astype(np.float64) + 0.125)).astype(np.float32))
+
+
+def test_expert_ffn_grid_composition(golden_dir):
+    """orc_expert_ffn_grid: the other formats give orc_expert_ffn bit for bit; with a codebook format on either side gate/up are
+    the pinned row dots and the down rows agree with a numpy double product over the exactly dequantised weights."""
+    from dwarfstar_red_lite_amd import synth
+    xs, m, _ = load_iq_grids(golden_dir)
+    H, F = 512, 256
+    rng = np.random.default_rng(91)
+    x = synth.normed_x(rng, 1, H)[0]
+    gate, up, down = synth.quant_rows(rng, 16, F, H), synth.quant_rows(rng, 16, F, H), synth.quant_rows(rng, 21, H, F)
+    assert np.array_equal(orc.expert_ffn_grid(16, 21, gate, up, down, H, F, x, xs, m), orc.expert_ffn(16, 21, gate, up, down, H, F, x))
+    for gu, dn in ((17, 17), (29, 29), (29, 17), (17, 16)):
+        gate, up, down = synth.quant_rows(rng, gu, F, H), synth.quant_rows(rng, gu, F, H), synth.quant_rows(rng, dn, H, F)
+        ggrid = xs if gu == 17 else m
+        act = np.array([orc.lib().orc_silu_mul(orc.row_dot_grid(gu, gate[r], x, ggrid), orc.row_dot_grid(gu, up[r], x, ggrid)) for r in range(F)])
+        wd = orc.dequant_rows_grid(dn, down, F, xs if dn == 17 else m) if dn in (17, 29) else orc.dequant_rows(dn, down, F)
+        want = wd.astype(np.float64) @ act
+        got = orc.expert_ffn_grid(gu, dn, gate, up, down, H, F, x, xs, m)
+        bound = 1e-12 * (np.abs(wd.astype(np.float64)) @ np.abs(act))
+        assert np.all(np.abs(got - want) <= bound + 1e-300), (gu, dn)
+        win = orc.expert_ffn_grid(gu, dn, gate, up, down, H, F, x, xs, m, row_start=500, row_count=12)
+        assert np.array_equal(win, got[500:])
