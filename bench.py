@@ -32,7 +32,9 @@ def parse():
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=480)
     ap.add_argument("--warmup", type=int, default=96)
-    ap.add_argument("--layout", choices=["iq2", "f2"], default="iq2", help="iq2: BASELINE config 1 (all IQ2_XXS, F32 router); f2: config 2 layout")
+    ap.add_argument("--layout", choices=["iq2", "f2", "xs", "m"], default="iq2",
+                    help="iq2: BASELINE config 1 (all IQ2_XXS, F32 router); f2: config 2 layout; xs / m: routed experts IQ2_XS / IQ1_M "
+                         "(the formats of the reference's target file), Q6_K shared expert")
     ap.add_argument("--layers", type=int, default=48, help="resident layers the steps cycle through")
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
@@ -46,12 +48,18 @@ def synth_layer_on_gpu(torch, gen, cfg):
     from dwarfstar_red_lite_amd import synth
 
     def rows(t, nrows, ncols, d_range=None):
-        bb, off = synth.BLOCK_BYTES[t], synth.D_OFFSET[t]
+        bb = synth.BLOCK_BYTES[t]
         nb = nrows * (ncols // 256)
         raw = torch.randint(0, 256, (nb, bb), dtype=torch.uint8, device="cuda", generator=gen)
         lo, hi = d_range or synth.D_RANGE[t]
         d = (lo + (hi - lo) * torch.rand(nb, device="cuda", generator=gen)).to(torch.float16).view(torch.uint8).reshape(nb, 2)
-        raw[:, off:off + 2] = d
+        if t == synth.TYPE_IQ1_M:          # d sits in the top nibbles of the four 16-bit scale words (bytes 48..55)
+            for i in range(4):
+                nib = (d[:, i // 2] >> (4 * (i % 2))) & 15
+                raw[:, 49 + 2 * i] = (raw[:, 49 + 2 * i] & 0x0F) | (nib << 4)
+        else:
+            off = synth.D_OFFSET[t]
+            raw[:, off:off + 2] = d
         return raw.reshape(nrows, -1)
 
     H, F, E = cfg["hidden"], cfg["ffn"], cfg["n_expert"]
@@ -96,6 +104,14 @@ def main():
     torch.cuda.init()
     cfg = synth.layer_config(layout=args.layout)
     B, NL = args.batch, args.layers
+    if args.layout in ("xs", "m"):          # these two decode through codebooks the caller supplies: the reference's, from the fixture
+        import json
+        import oracle_lib as orc
+        from dwarfstar_red_lite_amd import moe as moe_api
+        g = json.load(open(os.path.join(ROOT, "tests", "golden", "iq_grids.json")))
+        grids = [np.frombuffer(bytes.fromhex(g[k]), np.int8) for k in ("iq2_xs", "iq1_m")]
+        moe_api.set_codebooks(*grids)
+        orc.set_codebooks(*grids)
     moe = ResidentMoe(cfg, n_layer=NL, max_tokens=B)
     gen = torch.Generator(device="cuda")
     gen.manual_seed(20241125)
@@ -251,8 +267,9 @@ def main():
         "steps": K, "warmup": W, "ms_per_step": round(ms_per_step, 6), "launch_mode": launch_mode,
         "eager_ms_per_step": round(eager_ms_per_step, 6), "higher_is_better": False, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
-        "config": {"workload": "config1: one MoE FFN layer, B=%d decode token(s), hidden 2048, 512 experts top-10 + shared, ffn 512, layout %s, "
-                               "all experts of %d layers resident" % (B, args.layout, NL),
+        "config": {"workload": "%s: one MoE FFN layer, B=%d decode token(s), hidden 2048, 512 experts top-10 + shared, ffn 512, layout %s, "
+                               "all experts of %d layers resident" % ({"iq2": "config1", "f2": "config2"}.get(args.layout, "target-file expert format"),
+                                                                      B, args.layout, NL),
                    "layout": args.layout, "batch": B, "resident_layers": NL, "resident_gb": round(moe.resident_bytes / 1e9, 2),
                    "mean_distinct_routed_experts": mean_distinct},
         "layer_gbps": {"expert_bytes": int(lb["expert_bytes"]), "layer_bytes": int(total_bytes),

@@ -106,8 +106,8 @@ uint64_t tensor_bytes(uint32_t type, const uint64_t *dims, uint32_t n_dims) {
     uint64_t rows = 1;
     for (uint32_t i = 1; i < n_dims; ++i) rows *= dims[i];
     if (type == T_F32) return dims[0] * rows * 4u;
-    if (!quant_supported(type) || dims[0] % 256u) return 0;
-    return rows * row_bytes(type, (uint32_t)dims[0]);
+    if (!pool_quant_supported(type) || dims[0] % 256u) return 0;
+    return rows * pool_row_bytes(type, (uint32_t)dims[0]);
 }
 
 bool parse(const char *path, File &f, Directory &d) {
@@ -225,9 +225,14 @@ int redhip_gguf_moe_config(const char *path, uint32_t first_layer, redhip_moe_co
         const std::string &k = kv.first;
         if (k.size() > 18 && k.compare(k.size() - 18, 18, ".expert_used_count") == 0) out->top_k = (uint32_t)kv.second;
     }
+    // the run of layers from first_layer that share its shapes and types: a file whose layers differ in their expert format (the
+    // reference's target file holds IQ2_XS in its first and last layers and IQ1_M between) is walked as one run per format
     uint32_t n = 0;
     LayerTensors probe;
-    while (find(d, first_layer + n, "ffn_gate_exps.weight") && layer_tensors(d, first_layer + n, probe)) ++n;
+    while (find(d, first_layer + n, "ffn_gate_exps.weight") && layer_tensors(d, first_layer + n, probe) &&
+           probe.gate->type == t.gate->type && probe.down->type == t.down->type && probe.sh_gate->type == t.sh_gate->type &&
+           probe.sh_down->type == t.sh_down->type && probe.router->type == t.router->type && probe.router->dims[0] == t.router->dims[0] &&
+           probe.router->dims[1] == t.router->dims[1] && probe.gate->dims[1] == t.gate->dims[1]) ++n;
     g_gguf_error[0] = '\0';
     out->n_layer = n;
     out->max_tokens = 1;

@@ -24,6 +24,7 @@ inline bool pool_quant_supported(uint32_t t) { return pool_block_bytes(t) != 0u;
 // tables before every launch; callers whose tables differ must not run at the same time
 hipError_t set_caller_grids(const int8_t *iq2_xs, const int8_t *iq1_m, const void *owner = nullptr);
 void forget_caller_grids(const void *owner);
+bool caller_grid_present(uint32_t type);       // true for the formats that carry their own tables
 inline uint64_t row_bytes(uint32_t t, uint32_t ncols) {
     if (!ncols) return 0;
     if (t == T_F32) return 4ull * ncols;

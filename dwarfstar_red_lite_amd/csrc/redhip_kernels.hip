@@ -28,6 +28,12 @@ __device__ int8_t g_iq1m_grid[2048 * 8];
 
 static std::mutex g_grid_mu;
 static const void *g_grid_owner = nullptr;      // whose tables the device holds; nullptr: nobody's in particular
+static bool g_grid_have[2] = {false, false};    // IQ2_XS, IQ1_M uploaded at least once
+
+bool caller_grid_present(uint32_t type) {
+    std::lock_guard<std::mutex> lk(g_grid_mu);
+    return type == T_IQ2_XS ? g_grid_have[0] : type == T_IQ1_M ? g_grid_have[1] : true;
+}
 
 hipError_t set_caller_grids(const int8_t *iq2_xs, const int8_t *iq1_m, const void *owner) {
     std::lock_guard<std::mutex> lk(g_grid_mu);
@@ -36,6 +42,7 @@ hipError_t set_caller_grids(const int8_t *iq2_xs, const int8_t *iq1_m, const voi
     if (iq2_xs) e = hipMemcpyToSymbol(HIP_SYMBOL(g_iq2xs_grid), iq2_xs, sizeof(g_iq2xs_grid));
     if (e == hipSuccess && iq1_m) e = hipMemcpyToSymbol(HIP_SYMBOL(g_iq1m_grid), iq1_m, sizeof(g_iq1m_grid));
     g_grid_owner = e == hipSuccess ? owner : nullptr;
+    if (e == hipSuccess) { g_grid_have[0] |= iq2_xs != nullptr; g_grid_have[1] |= iq1_m != nullptr; }
     return e;
 }
 
@@ -366,7 +373,9 @@ hipError_t launch_moe_gateup(const ExpertSet &ex, const uint32_t *ids, uint32_t 
     }
 }
 
-// down projection of the selected experts fused with the weighted sum (selection order) and the shared expert
+// down projection of the selected experts fused with the weighted sum and the shared expert. A workgroup owns 64 / LPR output
+// rows; its four waves split the top_k + 1 matrices between them (slot k goes to wave k % 4, the shared expert is slot top_k), each
+// stages only its own slots' activations, and wave 0 adds the four partial sums in a fixed order.
 template <uint32_t TD, uint32_t TS, int LPR>
 __global__ __launch_bounds__(256) void moe_down_combine_kernel(const uint8_t *base, uint64_t stride, uint64_t down_off,
                                                                const uint32_t *ids, const float *weights, uint32_t top_k,
@@ -374,33 +383,40 @@ __global__ __launch_bounds__(256) void moe_down_combine_kernel(const uint8_t *ba
                                                                uint32_t hidden, uint32_t ffn,
                                                                const float *act, const float *sh_act, float *out,
                                                                const float *resid_a, const float *resid_b) {
-    extern __shared__ float as[];                          // [top_k + 1][padded ffn]
+    extern __shared__ float as[];                          // [top_k + 1][padded ffn], then [4][64 / LPR] partial sums
+    constexpr uint32_t kRows = 64u / LPR;
     const uint32_t fp = ffn + (ffn >> 5);
-    for (uint32_t i = threadIdx.x; i < top_k * ffn; i += 256u) as[(i / ffn) * fp + pad32(i % ffn)] = act[i];
-    if (sh_down) for (uint32_t i = threadIdx.x; i < ffn; i += 256u) as[top_k * fp + pad32(i)] = sh_act[i];
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63u;
+    const uint32_t n_slot = top_k + (sh_down ? 1u : 0u);
+    float *partial = as + (size_t)(top_k + 1u) * fp;
+    for (uint32_t k = wave; k < n_slot; k += 4u) {
+        const float *src = k < top_k ? act + (size_t)k * ffn : sh_act;
+        for (uint32_t i = lane; i < ffn; i += 64u) as[k * fp + pad32(i)] = src[i];
+    }
     __syncthreads();
-    const uint32_t sub = threadIdx.x % LPR, r = blockIdx.x * (256u / LPR) + threadIdx.x / LPR;
+    const uint32_t sub = lane % LPR, rl = lane / LPR, r = blockIdx.x * kRows + rl;
     const uint64_t rbd = (uint64_t)(ffn / 256u) * Fmt<TD>::kBlock, rbs = (uint64_t)(ffn / 256u) * Fmt<TS>::kBlock;
     float total = 0.0f;
-    for (uint32_t k = 0; k < top_k; ++k) {
+    for (uint32_t k = wave; k < n_slot; k += 4u) {
         float part = 0.0f;
         if (r < hidden) {
-            const uint8_t *row = base + (uint64_t)ids[k] * stride + down_off + (uint64_t)r * rbd;
-            for (uint32_t c = sub; c < ffn / 32u; c += LPR) part += chunk_dot<TD>(row, c, as + k * fp + 33u * c);
+            if (k < top_k) {
+                const uint8_t *row = base + (uint64_t)ids[k] * stride + down_off + (uint64_t)r * rbd;
+                for (uint32_t c = sub; c < ffn / 32u; c += LPR) part += chunk_dot<TD>(row, c, as + k * fp + 33u * c);
+            } else {
+                const uint8_t *row = sh_down + (uint64_t)r * rbs;
+                for (uint32_t c = sub; c < ffn / 32u; c += LPR) part += chunk_dot<TS>(row, c, as + k * fp + 33u * c);
+            }
         }
         part = sub_reduce<LPR>(part);
-        total = fmaf(weights[k], part, total);
+        total = fmaf(k < top_k ? weights[k] : scalar[0], part, total);
     }
-    if (sh_down) {
-        float part = 0.0f;
-        if (r < hidden) {
-            const uint8_t *row = sh_down + (uint64_t)r * rbs;
-            for (uint32_t c = sub; c < ffn / 32u; c += LPR) part += chunk_dot<TS>(row, c, as + top_k * fp + 33u * c);
-        }
-        part = sub_reduce<LPR>(part);
-        total = fmaf(scalar[0], part, total);
+    if (sub == 0u) partial[wave * kRows + rl] = total;
+    __syncthreads();
+    if (wave == 0u && sub == 0u && r < hidden) {
+        const float sum = (partial[rl] + partial[kRows + rl]) + (partial[2u * kRows + rl] + partial[3u * kRows + rl]);
+        out[r] = resid_a ? (resid_a[r] + resid_b[r]) + sum : sum;      // block step: residual added here
     }
-    if (sub == 0u && r < hidden) out[r] = resid_a ? (resid_a[r] + resid_b[r]) + total : total;      // block step: residual added here
 }
 
 template <uint32_t TD, uint32_t TS>
@@ -408,8 +424,8 @@ static hipError_t down_dispatch(const ExpertSet &ex, const uint32_t *ids, const 
                                 const ExpertSet &sh, const float *scalar, uint32_t hidden, uint32_t ffn,
                                 const float *act, const float *sh_act, float *out, hipStream_t s) {
     const uint32_t lpr = lanes_per_row(ffn);
-    const dim3 grid((hidden + 256u / lpr - 1u) / (256u / lpr));
-    const size_t lds = (size_t)(top_k + 1u) * padded_floats(ffn) * sizeof(float);
+    const dim3 grid((hidden + 64u / lpr - 1u) / (64u / lpr));
+    const size_t lds = ((size_t)(top_k + 1u) * padded_floats(ffn) + 4u * (64u / lpr)) * sizeof(float);
     const uint8_t *shd = sh.base ? sh.base + sh.gate_bytes + sh.up_bytes : nullptr;
     const uint64_t off = ex.gate_bytes + ex.up_bytes;
 #define REDHIP_DOWN(L) REDHIP_LAUNCH((moe_down_combine_kernel<TD, TS, L>), dim3(grid), dim3(256), lds, s, ex.base, ex.stride, off, ids, weights, top_k, shd, scalar, hidden, ffn, act, sh_act, out, block_context().resid_a, block_context().resid_b)
@@ -427,7 +443,7 @@ template <uint32_t TD>
 static hipError_t down_dispatch_shared(const ExpertSet &ex, const uint32_t *ids, const float *weights, uint32_t top_k,
                                        const ExpertSet &sh, const float *scalar, uint32_t hidden, uint32_t ffn,
                                        const float *act, const float *sh_act, float *out, hipStream_t s) {
-    switch (sh.base ? sh.down_type : TD) {
+    switch (sh.base ? sh.down_type : (TD == T_IQ2_XS || TD == T_IQ1_M) ? T_IQ2_XXS : TD) {      // without a shared expert TS is never read
         case T_IQ2_XXS: return down_dispatch<TD, T_IQ2_XXS>(ex, ids, weights, top_k, sh, scalar, hidden, ffn, act, sh_act, out, s);
         case T_IQ3_S: return down_dispatch<TD, T_IQ3_S>(ex, ids, weights, top_k, sh, scalar, hidden, ffn, act, sh_act, out, s);
         case T_Q6_K: return down_dispatch<TD, T_Q6_K>(ex, ids, weights, top_k, sh, scalar, hidden, ffn, act, sh_act, out, s);
@@ -440,11 +456,13 @@ hipError_t launch_moe_down_combine(const ExpertSet &ex, const uint32_t *ids, con
                                    const float *act, const float *shared_act, float *out, hipStream_t s) {
     hipError_t e = ensure_tables();
     if (e != hipSuccess) return e;
-    if (hidden % 256u || ffn % 256u || (size_t)(top_k + 1u) * padded_floats(ffn) * 4u > 160u * 1024u) return hipErrorInvalidValue;
+    if (hidden % 256u || ffn % 256u || ((size_t)(top_k + 1u) * padded_floats(ffn) + 32u) * 4u > 64u * 1024u) return hipErrorInvalidValue;
     switch (ex.down_type) {
         case T_IQ2_XXS: return down_dispatch_shared<T_IQ2_XXS>(ex, ids, weights, top_k, shared, scalar, hidden, ffn, act, shared_act, out, s);
         case T_IQ3_S: return down_dispatch_shared<T_IQ3_S>(ex, ids, weights, top_k, shared, scalar, hidden, ffn, act, shared_act, out, s);
         case T_Q6_K: return down_dispatch_shared<T_Q6_K>(ex, ids, weights, top_k, shared, scalar, hidden, ffn, act, shared_act, out, s);
+        case T_IQ2_XS: return down_dispatch_shared<T_IQ2_XS>(ex, ids, weights, top_k, shared, scalar, hidden, ffn, act, shared_act, out, s);
+        case T_IQ1_M: return down_dispatch_shared<T_IQ1_M>(ex, ids, weights, top_k, shared, scalar, hidden, ffn, act, shared_act, out, s);
         default: return hipErrorInvalidValue;
     }
 }
@@ -628,6 +646,8 @@ hipError_t launch_batch_gateup(const ExpertSet &ex, const uint32_t *uid, const u
         case T_IQ2_XXS: return batch_gateup_dispatch<T_IQ2_XXS>(a, n_groups, hidden, ffn, x, act, s);
         case T_IQ3_S: return batch_gateup_dispatch<T_IQ3_S>(a, n_groups, hidden, ffn, x, act, s);
         case T_Q6_K: return batch_gateup_dispatch<T_Q6_K>(a, n_groups, hidden, ffn, x, act, s);
+        case T_IQ2_XS: return batch_gateup_dispatch<T_IQ2_XS>(a, n_groups, hidden, ffn, x, act, s);
+        case T_IQ1_M: return batch_gateup_dispatch<T_IQ1_M>(a, n_groups, hidden, ffn, x, act, s);
         default: return hipErrorInvalidValue;
     }
 }
@@ -640,6 +660,8 @@ hipError_t launch_batch_down(const ExpertSet &ex, const uint32_t *uid, const uin
         case T_IQ2_XXS: return batch_down_dispatch<T_IQ2_XXS>(a, n_groups, hidden, ffn, act, tmp, s);
         case T_IQ3_S: return batch_down_dispatch<T_IQ3_S>(a, n_groups, hidden, ffn, act, tmp, s);
         case T_Q6_K: return batch_down_dispatch<T_Q6_K>(a, n_groups, hidden, ffn, act, tmp, s);
+        case T_IQ2_XS: return batch_down_dispatch<T_IQ2_XS>(a, n_groups, hidden, ffn, act, tmp, s);
+        case T_IQ1_M: return batch_down_dispatch<T_IQ1_M>(a, n_groups, hidden, ffn, act, tmp, s);
         default: return hipErrorInvalidValue;
     }
 }

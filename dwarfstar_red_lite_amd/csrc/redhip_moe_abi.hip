@@ -56,6 +56,12 @@ struct Moe {
     bool mixed = false;
     uint64_t packed_stride = 0;              // bytes between experts in `packed`
     bool packed_gu() const { return fused || mixed; }
+    // the one-launch router kernels (logits of every expert + the shared expert's gate logit, optional residual + norm) and the
+    // one-wave selection serve every layout whose router they tile; the per-row GEMV + generic selection are what is left
+    bool fast_route() const {
+        const uint32_t nv = cfg.hidden / 256u;
+        return packed_gu() || cfg.router_type == T_Q6_K || (cfg.router_type == T_F32 && (nv == 2u || nv == 4u || nv == 8u || nv == 16u));
+    }
     void *xh = nullptr, *xl = nullptr;       // fp16 [hidden] each
     int *xexp = nullptr;
     bool select_and_group = false;           // forward() of a small batch: one launch selects and sorts the pairs
@@ -202,9 +208,13 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
         moe_err("invalid MoE shape hidden=%u ffn=%u experts=%u top_k=%u layers=%u max_tokens=%u", c.hidden, c.ffn, c.n_expert, c.top_k, c.n_layer, c.max_tokens);
         return nullptr;
     }
-    if (!quant_supported(gu) || !quant_supported(dn) || !quant_supported(sgu) || !quant_supported(sdn) ||
+    if (!pool_quant_supported(gu) || !pool_quant_supported(dn) || !quant_supported(sgu) || !quant_supported(sdn) ||
         (c.router_type != T_F32 && c.router_type != T_Q6_K) || (c.expert_type_word >> 16) || (c.shared_type_word >> 16)) {
         moe_err("unsupported MoE types router=%u experts=0x%x shared=0x%x", c.router_type, c.expert_type_word, c.shared_type_word);
+        return nullptr;
+    }
+    if (!caller_grid_present(gu) || !caller_grid_present(dn)) {
+        moe_err("IQ2_XS / IQ1_M experts decode through the caller's codebooks: call redhip_set_codebooks first");
         return nullptr;
     }
     int ndev = 0;
@@ -212,8 +222,8 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
     Moe *m = new Moe();
     m->cfg = c;
     m->gu_type = gu; m->dn_type = dn; m->sh_gu_type = sgu; m->sh_dn_type = sdn;
-    m->gate_bytes = (uint64_t)c.ffn * row_bytes(gu, c.hidden);
-    m->down_bytes = (uint64_t)c.hidden * row_bytes(dn, c.ffn);
+    m->gate_bytes = (uint64_t)c.ffn * pool_row_bytes(gu, c.hidden);
+    m->down_bytes = (uint64_t)c.hidden * pool_row_bytes(dn, c.ffn);
     m->expert_stride = align256(2u * m->gate_bytes + m->down_bytes);
     m->sh_gate_bytes = (uint64_t)c.ffn * row_bytes(sgu, c.hidden);
     m->sh_down_bytes = (uint64_t)c.hidden * row_bytes(sdn, c.ffn);
@@ -377,11 +387,11 @@ int redhip_moe_route(redhip_moe_t h, uint32_t layer, const float *x_dev, uint32_
     if (!x_dev || !ntok || ntok > c.max_tokens) { moe_err("invalid token count %u (max %u)", ntok, c.max_tokens); return 0; }
     hipStream_t s = static_cast<hipStream_t>(stream);
     float *lg = logits_dev ? logits_dev : m->logits;
-    if (m->packed_gu()) {
+    if (m->fast_route()) {
         prof_set_stage(ST_ROUTER_GEMV);
         // a Q6_K shared expert of a mixed layout rides along: its gate / up products land in m->act (otherwise unused on this path)
         m->shared_gu_ready = m->mixed && m->sh_gu_type == T_Q6_K && c.router_type == T_Q6_K && ntok == 1u && c.top_k >= 2u;
-        if (c.router_type == T_F32 && ntok >= 16u)
+        if (m->packed_gu() && c.router_type == T_F32 && ntok >= 16u)
             HIP_OK(launch_router_f32_tiles(reinterpret_cast<const float *>(m->layers[layer].router), m->layers[layer].gate_inp, x_dev, ntok, c.hidden,
                                            c.n_expert, m->logits, m->xh, m->xl, m->xexp, s), "router tile launch");
         else
@@ -454,7 +464,7 @@ int redhip_moe_forward_block(redhip_moe_t h, uint32_t layer, const float *x_dev,
     BlockContext &bc = block_context();
     bc = BlockContext{};
     // the per-token router kernels of the packed paths normalise on the fly; everything else gets a kernel of its own
-    const bool in_router = m->packed_gu() && !(c.router_type == T_F32 && ntok >= 16u);
+    const bool in_router = m->fast_route() && !(m->packed_gu() && c.router_type == T_F32 && ntok >= 16u);
     int ok = 1;
     if (!in_router) {
         prof_set_stage(ST_OTHER);
@@ -490,7 +500,7 @@ int redhip_moe_last_route(redhip_moe_t h, uint32_t ntok, uint32_t *ids, float *w
     if (ids) HIP_OK(hipMemcpy(ids, m->ids, (size_t)ntok * c.top_k * 4u, hipMemcpyDeviceToHost), "ids download");
     if (weights) HIP_OK(hipMemcpy(weights, m->weights, (size_t)ntok * c.top_k * 4u, hipMemcpyDeviceToHost), "weights download");
     if (logits) {
-        const size_t pitch = 4u * (size_t)(c.n_expert + (m->packed_gu() ? 1u : 0u));
+        const size_t pitch = 4u * (size_t)(c.n_expert + (m->fast_route() ? 1u : 0u));
         HIP_OK(hipMemcpy2D(logits, 4u * (size_t)c.n_expert, m->logits, pitch, 4u * (size_t)c.n_expert, ntok, hipMemcpyDeviceToHost), "logits download");
     }
     return 1;

@@ -46,7 +46,8 @@ def normed_x(rng, ntok, hidden):
 
 def layer_config(hidden=2048, ffn=512, n_expert=512, top_k=10, layout="iq2"):
     """layout 'iq2': everything IQ2_XXS, F32 router. layout 'f2': gate/up IQ2_XXS, down IQ3_S, shared expert
-    and router Q6_K."""
+    and router Q6_K. layouts 'xs' / 'm': routed experts IQ2_XS / IQ1_M (what the reference's target file holds per
+    layer), F32 router, Q6_K shared expert."""
     cfg = dict(hidden=hidden, ffn=ffn, n_expert=n_expert, top_k=top_k)
     if layout == "iq2":
         cfg.update(router_type=TYPE_F32, gate_up_type=TYPE_IQ2_XXS, down_type=TYPE_IQ2_XXS,
@@ -54,6 +55,9 @@ def layer_config(hidden=2048, ffn=512, n_expert=512, top_k=10, layout="iq2"):
     elif layout == "f2":
         cfg.update(router_type=TYPE_Q6_K, gate_up_type=TYPE_IQ2_XXS, down_type=TYPE_IQ3_S,
                    sh_gate_up_type=TYPE_Q6_K, sh_down_type=TYPE_Q6_K)
+    elif layout in ("xs", "m"):
+        t = TYPE_IQ2_XS if layout == "xs" else TYPE_IQ1_M
+        cfg.update(router_type=TYPE_F32, gate_up_type=t, down_type=t, sh_gate_up_type=TYPE_Q6_K, sh_down_type=TYPE_Q6_K)
     else:
         raise ValueError(layout)
     cfg["layout"] = layout

@@ -71,7 +71,9 @@ int redhip_moe_last_route(redhip_moe_t moe, uint32_t ntok, uint32_t *ids, float 
  * (router, (hidden, experts)), ffn_gate_inp_shexp.weight (F32 [hidden]), ffn_{gate,up,down}_shexp.weight and the
  * expert-major ffn_{gate,up,down}_exps.weight ((hidden, ffn, experts) resp. (ffn, hidden, experts)).
  * redhip_gguf_moe_config fills hidden / ffn / n_expert / top_k (from <arch>.expert_used_count) / types / n_layer (the
- * run of consecutive MoE layers from first_layer) and max_tokens = 1 from a GGUF v2 / v3 file;
+ * run of consecutive MoE layers from first_layer that share its shapes and quantisation types: a file that changes its
+ * expert format between layers is walked as one run, and one handle, per format) and max_tokens = 1 from a GGUF v2 /
+ * v3 file;
  * redhip_moe_load_gguf uploads layers first_layer .. first_layer + n_layer - 1 of the file into layers 0 .. of a
  * handle created with `cfg`. Errors: return 0 and redhip_gguf_last_error() (thread-local). */
 const char *redhip_gguf_last_error(void);

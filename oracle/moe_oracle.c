@@ -62,6 +62,8 @@ size_t orc_block_bytes(uint32_t type) {
         case ORC_TYPE_Q6_K: return BLK_Q6K;
         case ORC_TYPE_IQ2_XXS: return BLK_IQ2XXS;
         case ORC_TYPE_IQ3_S: return BLK_IQ3S;
+        case 17u: return 74u;       /* IQ2_XS, native/redlite_native_reference.c:116 */
+        case 29u: return 56u;       /* IQ1_M, native/redlite_native_reference.c:144 */
         default: return 0;
     }
 }
@@ -173,6 +175,20 @@ int orc_dequant_row_grid(uint32_t type, const uint8_t *row, uint32_t ncols, cons
     return 1;
 }
 
+/* The caller's codebooks kept for the functions that take no grid argument (row dots, matvec, expert and layer forward), the way
+ * the reference keeps rl_native_quant_tables beside its model (native/redlite_native_reference.c:343). */
+static int8_t g_xs_grid[512 * 8], g_m_grid[2048 * 8];
+static int g_have_xs = 0, g_have_m = 0;
+
+void orc_set_codebooks(const int8_t *iq2_xs, const int8_t *iq1_m) {
+    if (iq2_xs) { memcpy(g_xs_grid, iq2_xs, sizeof(g_xs_grid)); g_have_xs = 1; }
+    if (iq1_m) { memcpy(g_m_grid, iq1_m, sizeof(g_m_grid)); g_have_m = 1; }
+}
+
+static const int8_t *kept_grid(uint32_t type) {
+    return type == 17u ? (g_have_xs ? g_xs_grid : NULL) : type == 29u ? (g_have_m ? g_m_grid : NULL) : NULL;
+}
+
 int orc_row_dot_grid(uint32_t type, const uint8_t *row, const float *x, uint32_t ncols, const int8_t *grid, double *out) {
     if (!row || !grid || !x || !out || !ncols || ncols % QK || (type != 17u && type != 29u)) return 0;
     const size_t bb = type == 17u ? 74u : 56u;
@@ -187,6 +203,7 @@ int orc_dequant_row(uint32_t type, const uint8_t *row, uint32_t ncols, float *ou
     if (!row || !out || !ncols) return 0;
     if (type == ORC_TYPE_F32) { memcpy(out, row, (size_t)ncols * 4u); return 1; }
     if (ncols % QK || !orc_block_bytes(type)) return 0;
+    if (type == 17u || type == 29u) return orc_dequant_row_grid(type, row, ncols, kept_grid(type), out);
     for (uint32_t b = 0; b < ncols / QK; ++b) {
         float *y = out + (size_t)b * QK;
         if (type == ORC_TYPE_IQ2_XXS) deq_iq2xxs_block(row + (size_t)b * BLK_IQ2XXS, y);
@@ -280,7 +297,15 @@ static int dot_any(uint32_t type, const uint8_t *row, const float *xf, const dou
     if (type == ORC_TYPE_IQ2_XXS) *out = dot_iq2xxs(row, xf, xd, ncols);
     else if (type == ORC_TYPE_Q6_K) *out = dot_q6k(row, xf, xd, ncols);
     else if (type == ORC_TYPE_IQ3_S) *out = dot_iq3s(row, xf, xd, ncols);
-    else return 0;
+    else if (type == 17u || type == 29u) {       /* native/redlite_native_reference.c:78-172 */
+        const int8_t *grid = kept_grid(type);
+        if (!grid) return 0;
+        const size_t bb = orc_block_bytes(type);
+        double acc = 0.0;
+        for (uint32_t i = 0; i < ncols; ++i)
+            acc += (xd ? xd[i] : (double)xf[i]) * xs_m_weight(type, row + (size_t)(i / QK) * bb, grid, i % QK);
+        *out = acc;
+    } else return 0;
     return 1;
 }
 

@@ -45,6 +45,8 @@ int orc_row_dot_d(uint32_t type, const uint8_t *row, const double *x, uint32_t n
  * codebooks are arguments, as in the reference (512 x 8 resp. 2048 x 8 int8 values, native/redlite_native_tables.c).
  * Dequantised weights (exact in f32) and the double-accumulated row dot of native/redlite_native_reference.c:116-172. */
 int orc_dequant_row_grid(uint32_t type, const uint8_t *row, uint32_t ncols, const int8_t *grid, float *out);
+/* keep copies of the IQ2_XS (512 x 8) / IQ1_M (2048 x 8) codebooks for the functions without a grid argument; NULL: unchanged */
+void orc_set_codebooks(const int8_t *iq2_xs, const int8_t *iq1_m);
 int orc_row_dot_grid(uint32_t type, const uint8_t *row, const float *x, uint32_t ncols, const int8_t *grid, double *out);
 /* single-expert FFN where either side may be a codebook format (17 / 29); other types as orc_expert_ffn */
 int orc_expert_ffn_grid(uint32_t gate_up_type, uint32_t down_type, const uint8_t *gate, const uint8_t *up, const uint8_t *down,

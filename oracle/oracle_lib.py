@@ -58,6 +58,8 @@ def lib():
         L.orc_row_dot.argtypes = [C.c_uint32, C.c_void_p, C.c_void_p, C.c_uint32, f64p]
         L.orc_row_dot_d.argtypes = [C.c_uint32, C.c_void_p, C.c_void_p, C.c_uint32, f64p]
         L.orc_dequant_row_grid.argtypes = [C.c_uint32, C.c_void_p, C.c_uint32, C.c_void_p, C.c_void_p]
+        L.orc_set_codebooks.argtypes = [C.c_void_p, C.c_void_p]
+        L.orc_set_codebooks.restype = None
         L.orc_row_dot_grid.argtypes = [C.c_uint32, C.c_void_p, C.c_void_p, C.c_uint32, C.c_void_p, f64p]
         L.orc_expert_ffn_grid.argtypes = [C.c_uint32, C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_uint32, C.c_uint32, C.c_uint32,
                                           C.c_uint32, C.c_void_p, C.c_void_p, C.c_void_p, C.c_void_p]
@@ -248,3 +250,11 @@ def expert_ffn_grid(gu_t, dn_t, gate, up, down, hidden, ffn, x, xs_grid, m_grid,
     assert lib().orc_expert_ffn_grid(gu_t, dn_t, _p(_bytes(gate)), _p(_bytes(up)), _p(_bytes(down)), hidden, ffn, row_start, row_count,
                                      _p(x), _p(xs_grid), _p(m_grid), _p(out))
     return out
+
+
+def set_codebooks(iq2_xs=None, iq1_m=None):
+    """keep the codebooks for the functions that take no grid (row_dot, matvec, expert_ffn, Layer.forward on types 17 / 29)."""
+    a = np.ascontiguousarray(iq2_xs, np.int8) if iq2_xs is not None else None
+    b = np.ascontiguousarray(iq1_m, np.int8) if iq1_m is not None else None
+    assert (a is None or a.size == 4096) and (b is None or b.size == 16384)
+    lib().orc_set_codebooks(_p(a), _p(b))

@@ -13,12 +13,15 @@ def _s(b):
 
 
 def write_moe_gguf(path, cfg, layers, first_layer=0, alignment=32, arch="qwen3next", extra_tensors=()):
-    """layers: list of dicts from synth.make_layer. Tensors per layer: router, sh_gate_inp, shared gate/up/down, routed
+    """layers: list of dicts from synth.make_layer; cfg: their configuration, or a list with one per layer. Tensors per layer: router, sh_gate_inp, shared gate/up/down, routed
     gate/up/down (expert-major). extra_tensors: (name, np.ndarray) pairs placed first (other model tensors)."""
+    cfgs = list(cfg) if isinstance(cfg, (list, tuple)) else [cfg] * len(layers)      # one dict, or one per layer (mixed formats)
+    cfg = cfgs[0]
     H, F, E = cfg["hidden"], cfg["ffn"], cfg["n_expert"]
     tensors = list((n, a, (a.size,), 0) for n, a in extra_tensors)
     for i, lay in enumerate(layers):
         l = first_layer + i
+        cfg = cfgs[i]
         tensors += [
             ("blk.%d.ffn_gate_inp.weight" % l, lay["router"], (H, E), cfg["router_type"]),
             ("blk.%d.ffn_gate_inp_shexp.weight" % l, lay["sh_gate_inp"], (H,), 0),

@@ -43,3 +43,16 @@ def test_error_strings_without_device_work():
     assert b"null MoE config" in lib.redhip_moe_last_error()
     assert lib.redmetal_quant_rows(None, 0, 0, 16, 256, 1, 0, 1, None, 256, None, 0, None, 1, None, None) == 0
     assert b"invalid Red Metal mixed-quant arguments" in lib.redmetal_quant_last_error()
+
+
+def test_codebook_formats_refused_before_codebooks():
+    """this process never uploads a codebook: a resident layer with IQ2_XS / IQ1_M experts is refused, not decoded through zeros;
+    wrong codebook sizes are refused too"""
+    lib = _lib.load()
+    cfg = _lib.MoeConfig(hidden=512, ffn=256, n_expert=16, top_k=4, router_type=0, expert_type_word=17, shared_type_word=14,
+                         n_layer=1, max_tokens=1)
+    assert lib.redhip_moe_create(ctypes.byref(cfg)) is None
+    assert b"redhip_set_codebooks" in lib.redhip_moe_last_error()
+    buf = (ctypes.c_int8 * 4096)()
+    assert lib.redhip_set_codebooks(buf, 4000, None, 0) == 0
+    assert b"codebook size mismatch" in lib.redhip_moe_last_error()

@@ -65,3 +65,43 @@ def test_load_from_file_equals_load_from_memory(tmp_path, layout):
             assert torch.equal(a.dequant_resident(l, 3, which), b.dequant_resident(l, 3, which))
     a.close()
     b.close()
+
+
+def test_config_probe_walks_format_runs(tmp_path):
+    """layers 0-1 IQ2_XS, 2-4 IQ1_M, 5 IQ2_XS (the reference's target file changes its expert format this way): one run per format"""
+    from dwarfstar_red_lite_amd.moe import gguf_moe_config
+    cx, cm = small_cfg("xs"), small_cfg("m")
+    cfgs = [cx, cx, cm, cm, cm, cx]
+    layers = [synth.make_layer(70 + i, c) for i, c in enumerate(cfgs)]
+    path = tmp_path / "mixed.gguf"
+    write_moe_gguf(path, cfgs, layers)
+    for first, n, t in ((0, 2, 17), (1, 1, 17), (2, 3, 29), (5, 1, 17)):
+        cfg, n_layer = gguf_moe_config(str(path), first)
+        assert n_layer == n and cfg["gate_up_type"] == t and cfg["down_type"] == t and cfg["sh_gate_up_type"] == 14
+
+
+@pytest.mark.gpu
+def test_load_format_runs_from_file(tmp_path, golden_dir):
+    import json
+    import os
+    torch = pytest.importorskip("torch")
+    from dwarfstar_red_lite_amd import moe
+    from dwarfstar_red_lite_amd.moe import ResidentMoe
+    g = json.load(open(os.path.join(golden_dir, "iq_grids.json")))
+    moe.set_codebooks(np.frombuffer(bytes.fromhex(g["iq2_xs"]), np.int8), np.frombuffer(bytes.fromhex(g["iq1_m"]), np.int8))
+    cx, cm = small_cfg("xs"), small_cfg("m")
+    cfgs = [cx, cm, cm]
+    layers = [synth.make_layer(80 + i, c) for i, c in enumerate(cfgs)]
+    path = tmp_path / "mixed.gguf"
+    write_moe_gguf(path, cfgs, layers)
+    x = torch.from_numpy(synth.normed_x(np.random.default_rng(4), 3, cx["hidden"])).cuda()
+    for first, n, cfg in ((0, 1, cx), (1, 2, cm)):
+        a = ResidentMoe.from_gguf(str(path), first_layer=first, max_tokens=3)
+        assert a.n_layer == n and a.cfg["gate_up_type"] == cfg["gate_up_type"]
+        b = ResidentMoe(cfg, n_layer=n, max_tokens=3)
+        for l in range(n):
+            b.load_layer(l, layers[first + l])
+            for nt in (1, 3):
+                assert torch.equal(a.forward(l, x[:nt]), b.forward(l, x[:nt]))
+        a.close()
+        b.close()

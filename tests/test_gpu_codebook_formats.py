@@ -162,3 +162,33 @@ def test_ffn_pool(model_file, grids):
         pool.load(0, lay)
         with pytest.raises(ValueError, match="need the pool created with"):
             pool.execute(0, lay, T_XS, H, F, 0, H, x)
+
+
+@pytest.mark.parametrize("layout", ["xs", "m"])
+@pytest.mark.parametrize("shape", [(512, 256, 16, 4), (2048, 512, 64, 10)])
+def test_resident_layer(layout, shape, grids):
+    """the resident layer with IQ2_XS / IQ1_M routed experts (what the reference's target file holds): one token, a ragged small
+    batch and a chunk, against the oracle's layer forward"""
+    from dwarfstar_red_lite_amd.moe import ResidentMoe
+    from test_gpu_moe_layer import ids_match_up_to_ties
+    orc.set_codebooks(*grids)
+    H, F, E, K = shape
+    cfg = synth.layer_config(hidden=H, ffn=F, n_expert=E, top_k=K, layout=layout)
+    m = ResidentMoe(cfg, n_layer=1, max_tokens=24)
+    lay = synth.make_layer(60 + H, cfg)
+    m.load_layer(0, lay)
+    ref = orc.Layer(cfg, **lay)
+    t = cfg["gate_up_type"]
+    for e, which in ((0, 0), (E - 1, 1), (E // 2, 2)):
+        want = orc.dequant_rows(t, lay[("gate", "up", "down")[which]][e].reshape(-1), H if which < 2 else F)
+        got = m.dequant_resident(0, e, which).cpu().numpy()
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+    xs = synth.normed_x(np.random.default_rng(8), 24, H)
+    for ntok in (1, 5, 24):
+        out = m.forward(0, torch.from_numpy(xs[:ntok].copy()).cuda()).cpu().numpy()
+        gids, gw, glog = m.last_route(ntok)
+        want, cids, cw, clog = ref.forward(xs[:ntok], threads=8)
+        for i in range(ntok):
+            assert ids_match_up_to_ties(gids[i], cids[i], clog[i])
+            assert rel_l2(out[i], want[i]) <= REL_L2_TOL, (layout, shape, ntok, i)
+    m.close()

@@ -52,7 +52,7 @@ def test_codebooks():
 def test_row_sizes():
     assert orc.row_bytes(T_Q6K, 256) == 210 and orc.row_bytes(T_IQ2, 256) == 66 and orc.row_bytes(T_IQ3, 2048) == 880
     assert orc.row_bytes(T_IQ2, 2048) == 528 and orc.row_bytes(T_IQ2, 512) == 132 and orc.row_bytes(T_F32, 2048) == 8192
-    assert orc.row_bytes(T_IQ2, 100) == 0 and orc.row_bytes(17, 256) == 0
+    assert orc.row_bytes(T_IQ2, 100) == 0 and orc.row_bytes(18, 256) == 0
 
 
 def test_golden_rows(golden_dir):
@@ -270,3 +270,20 @@ def test_expert_ffn_grid_composition(golden_dir):
         assert np.all(np.abs(got - want) <= bound + 1e-300), (gu, dn)
         win = orc.expert_ffn_grid(gu, dn, gate, up, down, H, F, x, xs, m, row_start=500, row_count=12)
         assert np.array_equal(win, got[500:])
+
+
+def test_kept_codebooks_match_grid_arguments(golden_dir):
+    """the functions without a grid argument, after set_codebooks, give what the grid-taking ones give, bit for bit"""
+    from dwarfstar_red_lite_amd import synth
+    xs, m, _ = load_iq_grids(golden_dir)
+    orc.set_codebooks(xs, m)
+    H, F = 512, 256
+    rng = np.random.default_rng(92)
+    x = synth.normed_x(rng, 1, H)[0]
+    for t, grid in ((17, xs), (29, m)):
+        rows = synth.quant_rows(rng, t, 5, H)
+        assert orc.row_bytes(t, H) == rows.shape[1]
+        assert np.array_equal(orc.dequant_rows(t, rows, H), orc.dequant_rows_grid(t, rows, H, grid))
+        assert [orc.row_dot(t, rows[r], x) for r in range(5)] == [orc.row_dot_grid(t, rows[r], x, grid) for r in range(5)]
+        gate, up, down = synth.quant_rows(rng, t, F, H), synth.quant_rows(rng, t, F, H), synth.quant_rows(rng, t, H, F)
+        assert np.array_equal(orc.expert_ffn(t, t, gate, up, down, H, F, x), orc.expert_ffn_grid(t, t, gate, up, down, H, F, x, xs, m))
