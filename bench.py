@@ -38,6 +38,7 @@ def parse():
     ap.add_argument("--layers", type=int, default=48, help="resident layers the steps cycle through")
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
+    ap.add_argument("--no-micro", action="store_true", help="skip the single-GEMV microbench (only run for --layout iq2 --batch 1)")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--calibrate", action="store_true", help="also run the plain copy kernel of known size (for rocprofv3 --pmc runs)")
     return ap.parse_args()
@@ -105,7 +106,6 @@ def main():
     cfg = synth.layer_config(layout=args.layout)
     B, NL = args.batch, args.layers
     if args.layout in ("xs", "m"):          # these two decode through codebooks the caller supplies: the reference's, from the fixture
-        import json
         import oracle_lib as orc
         from dwarfstar_red_lite_amd import moe as moe_api
         g = json.load(open(os.path.join(ROOT, "tests", "golden", "iq_grids.json")))
@@ -145,7 +145,7 @@ def main():
     got = outs[0].cpu().numpy()
     rel = float(np.linalg.norm(got - want) / np.linalg.norm(want))
     ids_ok = bool(np.array_equal(gids, cids))
-    if rel > 1e-3 or not ids_ok:
+    if not rel <= 1e-3 or not ids_ok:
         print("PARITY FAILURE: rel L2 %.3g vs the CPU oracle, router ids identical: %s" % (rel, ids_ok), file=sys.stderr)
         sys.exit(1)
 
@@ -280,6 +280,57 @@ def main():
         "parity": {"rel_l2_vs_cpu_oracle": rel, "router_ids_identical": ids_ok},
         "roofline": roofline,
     }
+
+    # ---- per-kernel microbench of config 1: one IQ2_XXS dequant-GEMV [512 x 2048] x [2048] on raw GGUF rows ----
+    if args.layout == "iq2" and B == 1 and not args.no_micro:
+        NM, reps = 1024, 2048                   # 1024 distinct matrices = 277 MB, more than the 256 MB last-level cache
+        mats = torch.randint(0, 256, (NM, F * synth.row_bytes(synth.TYPE_IQ2_XXS, H)), dtype=torch.uint8, device="cuda", generator=gen)
+        mats.view(NM * F * (H // 256), 66)[:, 1] = 0x1E            # d in [2^-8, 2^-7): finite whatever the random low byte
+        yv = torch.empty((NM, F), dtype=torch.float32, device="cuda")
+        xg = xs[0, 0].contiguous()
+        torch.cuda.synchronize()                # the matrices were filled on the default stream, the launches go to `stream`
+
+        def gemv(i):
+            ok = lib.redhip_gemv_rows(synth.TYPE_IQ2_XXS, mats[i % NM].data_ptr(), H, 0, F, xg.data_ptr(), yv[i % NM].data_ptr(),
+                                      stream.cuda_stream)
+            assert ok
+        with torch.cuda.stream(stream):
+            for i in range(64):
+                gemv(i)
+            stream.synchronize()
+            want_row = orc.matvec(synth.TYPE_IQ2_XXS, mats[5].cpu().numpy(), H, xs_host[0, 0])
+            got_row = yv[5].cpu().numpy()
+            micro_rel = float(np.linalg.norm(got_row - want_row) / np.linalg.norm(want_row))
+            g2 = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g2, stream=stream):
+                for i in range(reps):
+                    gemv(i)
+            g2.replay()
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            g2.replay()
+            torch.cuda.synchronize()
+            gemv_us = (time.perf_counter() - t0) * 1e6 / reps
+            lib.redhip_profile_begin()
+            for i in range(reps):
+                gemv(i)
+            sm, sn = (C.c_double * n_stage)(), (C.c_uint32 * n_stage)()
+            lib.redhip_profile_end(sm, sn, n_stage)
+        kern_us = 1e3 * sum(sm) / max(sum(sn), 1)
+        gemv_bytes = F * synth.row_bytes(synth.TYPE_IQ2_XXS, H) + 4 * H + 4 * F
+        fused_us = sum(v for k, v in result["stages_us"].items() if k in ("gateup", "down_combine", "fused_experts"))
+        result["microbench"] = {
+            "iq2_xxs_gemv_512x2048": {"us_back_to_back": round(gemv_us, 3), "kernel_us": round(kern_us, 3), "bytes": gemv_bytes,
+                                      "gbps_back_to_back": round(gemv_bytes / gemv_us / 1e3, 1), "gbps_kernel": round(gemv_bytes / kern_us / 1e3, 1),
+                                      "rel_l2_vs_cpu_oracle": micro_rel,
+                                      "note": "%d launches replayed from one HIP graph over %d distinct matrices; kernel_us = the dispatches' own "
+                                              "begin/end timestamps" % (reps, NM)},
+            "fused_experts_10_routed_1_shared": {"us": round(fused_us, 3), "bytes": int(lb["expert_bytes"]),
+                                                 "gbps": round(lb["expert_bytes"] / fused_us / 1e3, 1),
+                                                 "note": "gate/up/SwiGLU launch + down/combine launch of the timed steps"}}
+        if not micro_rel <= 1e-3:
+            print("PARITY FAILURE in the GEMV microbench: rel L2 %.3g" % micro_rel, file=sys.stderr)
+            sys.exit(1)
 
     # ---- CPU baseline: the oracle on this host's cores, layer 0, same activations ----
     if not args.no_cpu:

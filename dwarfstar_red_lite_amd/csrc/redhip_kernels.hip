@@ -149,17 +149,22 @@ hipError_t launch_dequant_rows(uint32_t type, const void *rows, uint32_t nrows, 
 
 // ---------------------------------------------------------------- GEMV over raw rows
 
+// x is read straight from global memory: the lanes of a row take consecutive 128-byte pieces, so a wave's read is one contiguous
+// run, it is issued together with the weight loads, and there is no staging barrier in front of the first decode
 template <uint32_t T, int LPR>
 __global__ __launch_bounds__(256) void gemv_rows_kernel(const uint8_t *w, uint64_t rb, uint32_t ncols, uint32_t row_start,
                                                         uint32_t row_count, const float *x, float *out) {
-    extern __shared__ float xs[];
-    for (uint32_t i = threadIdx.x; i < ncols; i += 256u) xs[pad32(i)] = x[i];
-    __syncthreads();
-    const uint32_t sub = threadIdx.x % LPR, r = blockIdx.x * (256u / LPR) + threadIdx.x / LPR;
+    const uint32_t sub = threadIdx.x % LPR, r = blockIdx.x * (blockDim.x / LPR) + threadIdx.x / LPR;
     float acc = 0.0f;
     if (r < row_count) {
         const uint8_t *row = w + (uint64_t)(row_start + r) * rb;
-        for (uint32_t c = sub; c < ncols / 32u; c += LPR) acc += chunk_dot<T>(row, c, xs + 33u * c);
+        for (uint32_t c = sub; c < ncols / 32u; c += LPR) {
+            float xv[32];
+            const float4 *xp = reinterpret_cast<const float4 *>(x + 32u * c);
+#pragma unroll
+            for (int i = 0; i < 8; ++i) { const float4 v = xp[i]; xv[4 * i] = v.x; xv[4 * i + 1] = v.y; xv[4 * i + 2] = v.z; xv[4 * i + 3] = v.w; }
+            acc += chunk_dot<T>(row, c, xv);
+        }
     }
     acc = sub_reduce<LPR>(acc);
     if (sub == 0u && r < row_count) out[r] = acc;
@@ -169,13 +174,14 @@ template <uint32_t T>
 static hipError_t gemv_dispatch(const uint8_t *w, uint32_t ncols, uint32_t row_start, uint32_t row_count, const float *x, float *out, hipStream_t s) {
     const uint64_t rb = pool_row_bytes(T, ncols);
     const uint32_t lpr = lanes_per_row(ncols);
-    const dim3 grid((row_count + 256u / lpr - 1u) / (256u / lpr));
-    const size_t lds = padded_floats(ncols) * sizeof(float);
+    // one wave per workgroup while that still leaves fewer workgroups than twice the compute units
+    const uint32_t nt = (row_count + 256u / lpr - 1u) / (256u / lpr) < 512u ? 64u : 256u;
+    const dim3 grid((row_count + nt / lpr - 1u) / (nt / lpr));
     switch (lpr) {
-        case 64: REDHIP_LAUNCH((gemv_rows_kernel<T, 64>), dim3(grid), dim3(256), lds, s, w, rb, ncols, row_start, row_count, x, out); break;
-        case 32: REDHIP_LAUNCH((gemv_rows_kernel<T, 32>), dim3(grid), dim3(256), lds, s, w, rb, ncols, row_start, row_count, x, out); break;
-        case 16: REDHIP_LAUNCH((gemv_rows_kernel<T, 16>), dim3(grid), dim3(256), lds, s, w, rb, ncols, row_start, row_count, x, out); break;
-        default: REDHIP_LAUNCH((gemv_rows_kernel<T, 8>), dim3(grid), dim3(256), lds, s, w, rb, ncols, row_start, row_count, x, out); break;
+        case 64: REDHIP_LAUNCH((gemv_rows_kernel<T, 64>), dim3(grid), dim3(nt), 0, s, w, rb, ncols, row_start, row_count, x, out); break;
+        case 32: REDHIP_LAUNCH((gemv_rows_kernel<T, 32>), dim3(grid), dim3(nt), 0, s, w, rb, ncols, row_start, row_count, x, out); break;
+        case 16: REDHIP_LAUNCH((gemv_rows_kernel<T, 16>), dim3(grid), dim3(nt), 0, s, w, rb, ncols, row_start, row_count, x, out); break;
+        default: REDHIP_LAUNCH((gemv_rows_kernel<T, 8>), dim3(grid), dim3(nt), 0, s, w, rb, ncols, row_start, row_count, x, out); break;
     }
     return hipGetLastError();
 }
@@ -184,7 +190,7 @@ hipError_t launch_gemv_rows(uint32_t type, const void *w, uint32_t ncols, uint32
                             const float *x, float *out, hipStream_t s) {
     hipError_t e = ensure_tables();
     if (e != hipSuccess) return e;
-    if (!pool_row_bytes(type, ncols) || ncols % 256u || !row_count || padded_floats(ncols) * 4u > 160u * 1024u) return hipErrorInvalidValue;
+    if (!pool_row_bytes(type, ncols) || ncols % 256u || !row_count || (reinterpret_cast<uintptr_t>(x) & 15u)) return hipErrorInvalidValue;      // x is read as float4
     const uint8_t *p = static_cast<const uint8_t *>(w);
     switch (type) {
         case T_IQ2_XXS: return gemv_dispatch<T_IQ2_XXS>(p, ncols, row_start, row_count, x, out, s);
