@@ -680,6 +680,27 @@ hipError_t launch_batch_combine(const float *tmp, const float *pair_weight, cons
 
 // ---------------------------------------------------------------- token grouping (pair sort)
 
+// exclusive prefix sum over the 1024 threads of a workgroup (16 waves): in-wave shuffles, then the 16 wave totals
+__device__ __forceinline__ uint32_t block_scan_1024(uint32_t v, uint32_t *wave_tot /* [17] */, uint32_t &total) {
+    const uint32_t lane = threadIdx.x & 63u, wave = threadIdx.x >> 6;
+    uint32_t inc = v;
+#pragma unroll
+    for (int o = 1; o < 64; o <<= 1) { const uint32_t n = __shfl_up(inc, o, 64); if (lane >= (uint32_t)o) inc += n; }
+    if (lane == 63u) wave_tot[wave] = inc;
+    __syncthreads();
+    if (threadIdx.x == 0u) {
+        uint32_t acc = 0u;
+#pragma unroll
+        for (int w = 0; w < 16; ++w) { const uint32_t t = wave_tot[w]; wave_tot[w] = acc; acc += t; }
+        wave_tot[16] = acc;
+    }
+    __syncthreads();
+    total = wave_tot[16];
+    const uint32_t ex = wave_tot[wave] + inc - v;
+    __syncthreads();                               // wave_tot may be reused right away
+    return ex;
+}
+
 // One workgroup. For every (token, k) pair p = t * top_k + k:
 //   first[e]   = smallest p that names expert e            -> experts numbered in first-appearance order
 //   member[e]  = bitmap over tokens that selected e        -> rank of a pair inside its expert = popcount below t
@@ -694,8 +715,9 @@ __global__ __launch_bounds__(1024) void group_pairs_kernel(const uint32_t *ids, 
     uint32_t *count = first + n_expert;            // [n_expert]
     uint32_t *dense = count + n_expert;            // [n_expert]
     uint32_t *start = dense + n_expert;            // [n_expert + 1] by dense index
-    uint32_t *scan = start + n_expert + 1u;        // [1024 + 1]
-    uint32_t *member = scan + 1025u;               // [n_expert][words]
+    uint32_t *uid_l = start + n_expert + 1u;       // [1024] experts by dense index (n_expert <= 1024)
+    uint32_t *wave_tot = uid_l + 1024u;            // [17]
+    uint32_t *member = wave_tot + 17u;             // [n_expert][words]
     for (uint32_t i = tid; i < n_expert; i += 1024u) { first[i] = 0xffffffffu; count[i] = 0u; dense[i] = 0u; }
     for (uint32_t i = tid; i < n_expert * words; i += 1024u) member[i] = 0u;
     __syncthreads();
@@ -706,31 +728,23 @@ __global__ __launch_bounds__(1024) void group_pairs_kernel(const uint32_t *ids, 
         atomicOr(&member[e * words + (t >> 5)], 1u << (t & 31u));
     }
     __syncthreads();
-    // exclusive scan of "pair p is the first appearance of its expert", P elements in chunks of per-thread runs
+    // exclusive scan of "pair p is the first appearance of its expert", P elements in per-thread runs
     const uint32_t per = (P + 1023u) / 1024u;
     uint32_t mine = 0u;
     for (uint32_t j = 0; j < per; ++j) { const uint32_t p = tid * per + j; if (p < P && first[ids[p]] == p) ++mine; }
-    scan[tid + 1u] = mine;
-    if (tid == 0u) scan[0] = 0u;
-    __syncthreads();
-    if (tid == 0u) for (uint32_t i = 1; i <= 1024u; ++i) scan[i] += scan[i - 1u];       // 1024 adds: negligible
-    __syncthreads();
-    uint32_t run = scan[tid];
+    uint32_t U = 0u;
+    uint32_t run = block_scan_1024(mine, wave_tot, U);
     for (uint32_t j = 0; j < per; ++j) {
         const uint32_t p = tid * per + j;
-        if (p < P && first[ids[p]] == p) { dense[ids[p]] = run; uid[run] = ids[p]; ++run; }
-    }
-    const uint32_t U = scan[1024];
-    __syncthreads();
-    // exclusive scan of the per-expert pair counts in dense order
-    if (tid == 0u) {
-        uint32_t acc = 0u;
-        for (uint32_t u = 0; u < U; ++u) { start[u] = acc; acc += count[uid[u]]; }
-        start[U] = acc;
-        n_unique[0] = U;
+        if (p < P && first[ids[p]] == p) { const uint32_t e = ids[p]; dense[e] = run; uid_l[run] = e; uid[run] = e; ++run; }
     }
     __syncthreads();
-    for (uint32_t u = tid; u <= U; u += 1024u) expert_start[u] = start[u];
+    // exclusive scan of the per-expert pair counts in dense order (U <= n_expert <= 1024: one per thread)
+    uint32_t all = 0u;
+    const uint32_t my_start = block_scan_1024(tid < U ? count[uid_l[tid]] : 0u, wave_tot, all);
+    if (tid < U) { start[tid] = my_start; expert_start[tid] = my_start; }
+    if (tid == 0u) { start[U] = all; expert_start[U] = all; n_unique[0] = U; }
+    __syncthreads();
     for (uint32_t p = tid; p < P; p += 1024u) {
         const uint32_t e = ids[p], t = p / top_k;
         const uint32_t *bits = member + e * words;
@@ -748,7 +762,7 @@ hipError_t launch_group_pairs(const uint32_t *ids, const float *weights, uint32_
                               uint32_t *tok_pair, uint32_t *n_unique, hipStream_t s) {
     if (!ntok || !top_k || !n_expert || n_expert > 1024u) return hipErrorInvalidValue;
     const uint32_t words = (ntok + 31u) / 32u;
-    const size_t lds = sizeof(uint32_t) * ((size_t)4u * n_expert + 1u + 1025u + (size_t)n_expert * words);
+    const size_t lds = sizeof(uint32_t) * ((size_t)4u * n_expert + 1u + 1024u + 17u + (size_t)n_expert * words);
     if (lds > 160u * 1024u) return hipErrorInvalidValue;
     static bool attr_set = false;
     if (!attr_set) {

@@ -307,14 +307,16 @@ __global__ __launch_bounds__(kWaves * 64) void prefill_down_kernel(PrefillArgs a
 // ---------------------------------------------------------------- router logits of a token chunk
 
 // logits[tok][e] = W[e] . x[tok] for an f32 router as a tiled product on v_mfma_f32_16x16x4_f32 (full fp32
-// multiply-add): a workgroup owns 32 router rows x 32 tokens, each of its four waves a 16 x 16 corner. Lane (r = l % 16,
-// q = l / 16) loads four consecutive k of row r and of token r per 16 k and feeds them to four MFMAs (A[i = r][k = q],
-// B[k = q][j = r], D[i = 4q .. 4q + 3][j = r]); row n_expert is the shared expert's gate vector. A second kind of
-// workgroup (blockIdx.x beyond the row tiles) does the fp16 split of its tokens' activations.
+// multiply-add): a workgroup owns 16 router rows x 16 tokens and its four waves each take a quarter of the hidden dimension,
+// so that a compute unit holds enough waves to cover the load latency; the four partial tiles meet in LDS and are added in a
+// fixed order. Lane (r = l % 16, q = l / 16) loads four consecutive k of row r and of token r per 16 k and feeds them to four
+// MFMAs (A[i = r][k = q], B[k = q][j = r], D[i = 4q .. 4q + 3][j = r]); row n_expert is the shared expert's gate vector. A
+// second kind of workgroup (blockIdx.x beyond the row tiles) does the fp16 split of its tokens' activations.
 __global__ __launch_bounds__(256) void router_f32_tile_kernel(const float *w, const float *gate_inp, const float *x, float *logits,
                                                               _Float16 *xh, _Float16 *xl, int *xexp, uint32_t H, uint32_t E, uint32_t ntok) {
+    __shared__ float part[4][16][17];
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, r = lane & 15u, q = lane >> 4;
-    const uint32_t row_tiles = (E + 1u + 31u) / 32u;
+    const uint32_t row_tiles = (E + 1u + 15u) / 16u;
     if (blockIdx.x >= row_tiles) {                         // split job: one wave per token, 4 tokens per workgroup
         const uint32_t tok = 4u * (blockIdx.y * (gridDim.x - row_tiles) + (blockIdx.x - row_tiles)) + wave;
         if (tok >= ntok) return;
@@ -329,9 +331,9 @@ __global__ __launch_bounds__(256) void router_f32_tile_kernel(const float *w, co
         if (lane == 0u) xexp[tok] = e;
         return;
     }
-    const uint32_t row = 32u * blockIdx.x + 16u * (wave & 1u) + r, tok = 32u * blockIdx.y + 16u * (wave >> 1) + r;
-    const float *wr = row < E ? w + (uint64_t)row * H : gate_inp;          // rows beyond E + 1 repeat the gate vector and are not stored
-    const float *xt = x + (uint64_t)(tok < ntok ? tok : ntok - 1u) * H;
+    const uint32_t row = 16u * blockIdx.x + r, tok = 16u * blockIdx.y + r, kq = H / 4u;          // this wave: k in [wave * kq, (wave + 1) * kq)
+    const float *wr = (row < E ? w + (uint64_t)row * H : gate_inp) + wave * kq;          // rows beyond E + 1 repeat the gate vector and are not stored
+    const float *xt = x + (uint64_t)(tok < ntok ? tok : ntok - 1u) * H + wave * kq;
     // 64 k per step: four loads of 16 bytes per operand, those of the next step in flight while this one is multiplied;
     // two accumulators halve the chain of dependent MFMAs
     float4_t acc0 = {0.0f, 0.0f, 0.0f, 0.0f}, acc1 = acc0;
@@ -341,8 +343,8 @@ __global__ __launch_bounds__(256) void router_f32_tile_kernel(const float *w, co
         av[u] = *reinterpret_cast<const float4 *>(wr + 16u * u + 4u * q);
         bv[u] = *reinterpret_cast<const float4 *>(xt + 16u * u + 4u * q);
     }
-    for (uint32_t k0 = 0; k0 < H; k0 += 64u) {
-        const uint32_t kn = k0 + 64u < H ? k0 + 64u : k0;          // the last step reloads itself: no branch around the loads
+    for (uint32_t k0 = 0; k0 < kq; k0 += 64u) {
+        const uint32_t kn = k0 + 64u < kq ? k0 + 64u : k0;          // the last step reloads itself: no branch around the loads
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             an[u] = *reinterpret_cast<const float4 *>(wr + kn + 16u * u + 4u * q);
@@ -358,22 +360,20 @@ __global__ __launch_bounds__(256) void router_f32_tile_kernel(const float *w, co
 #pragma unroll
         for (int u = 0; u < 4; ++u) { av[u] = an[u]; bv[u] = bn[u]; }
     }
-    float4_t acc;
 #pragma unroll
-    for (int t = 0; t < 4; ++t) acc[t] = acc0[t] + acc1[t];
-    if (tok < ntok) {
-#pragma unroll
-        for (uint32_t t = 0; t < 4u; ++t) {
-            const uint32_t out_row = 32u * blockIdx.x + 16u * (wave & 1u) + 4u * q + t;
-            if (out_row <= E) logits[(uint64_t)tok * (E + 1u) + out_row] = acc[t];
-        }
-    }
+    for (uint32_t t = 0; t < 4u; ++t) part[wave][r][4u * q + t] = acc0[t] + acc1[t];          // [token j][row i]
+    __syncthreads();
+    const uint32_t i = tid & 15u, j = tid >> 4;             // consecutive threads store consecutive rows of one token
+    const uint32_t out_row = 16u * blockIdx.x + i, out_tok = 16u * blockIdx.y + j;
+    if (out_tok < ntok && out_row <= E)
+        logits[(uint64_t)out_tok * (E + 1u) + out_row] = (part[0][j][i] + part[1][j][i]) + (part[2][j][i] + part[3][j][i]);
 }
 
 hipError_t launch_router_f32_tiles(const float *w, const float *gate_inp, const float *x, uint32_t ntok, uint32_t hidden, uint32_t n_expert,
                                    float *logits, void *xh, void *xl, int *xexp, hipStream_t s) {
-    if (!ntok || !hidden || hidden % 64u || !n_expert) return hipErrorInvalidValue;
-    const uint32_t row_tiles = (n_expert + 1u + 31u) / 32u, tok_tiles = (ntok + 31u) / 32u;
+    if (!ntok || !hidden || hidden % 256u || !n_expert) return hipErrorInvalidValue;
+    const uint32_t row_tiles = (n_expert + 1u + 15u) / 16u, tok_tiles = (ntok + 15u) / 16u;
+    if (tok_tiles > 65535u) return hipErrorInvalidValue;
     const uint32_t split_wgs = ((ntok + 3u) / 4u + tok_tiles - 1u) / tok_tiles;            // per blockIdx.y
     REDHIP_LAUNCH(router_f32_tile_kernel, dim3(row_tiles + split_wgs, tok_tiles), dim3(256), 0, s, w, gate_inp, x, logits,
                   static_cast<_Float16 *>(xh), static_cast<_Float16 *>(xl), xexp, hidden, n_expert, ntok);
