@@ -123,7 +123,12 @@ inline uint32_t prefill_tile_bound(uint32_t ntok, uint32_t top_k, uint32_t n_exp
     const uint32_t P = ntok * top_k;
     return (P < n_expert ? P : n_expert) + P / 16u + (ntok + 15u) / 16u + 1u;
 }
-hipError_t launch_prefill_packed(const void *experts, uint64_t stride, const void *shared, const uint32_t *uid, const uint32_t *expert_start,
+// tiled_experts / tiled_shared: optional tile-major copies (launch_tile_packed) of the same matrices, same stride and offsets; with
+// them and ffn <= 512 the kernels that keep a tile's activations in registers run.
+hipError_t launch_tile_packed(const void *packed, uint64_t packed_stride, uint32_t count, uint32_t nrows, uint32_t K, void *tiled, uint64_t tiled_stride,
+                              hipStream_t s);
+hipError_t launch_prefill_packed(const void *experts, uint64_t stride, const void *shared, const void *tiled_experts, const void *tiled_shared,
+                                 const uint32_t *uid, const uint32_t *expert_start,
                                  const uint32_t *pair_token, const uint32_t *n_unique, uint32_t *tile_group, uint32_t *tile_pair0,
                                  uint32_t *tile_n, uint32_t *n_tiles, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l,
                                  int *act_exp, float *tmp, float *sh_tmp, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok,

@@ -34,6 +34,8 @@ struct Layer {
     uint8_t *experts = nullptr;      // n_expert slots of expert_stride bytes, each gate | up | down
     uint8_t *packed = nullptr;       // same slots in the packed IQ2_XXS layout of the fused kernel (fused path only)
     uint8_t *shared_packed = nullptr;
+    uint8_t *tiled = nullptr;        // third copy, tile-major, read by the prefill kernels (handles that take chunks only)
+    uint8_t *shared_tiled = nullptr;
 };
 
 struct Moe {
@@ -56,6 +58,8 @@ struct Moe {
     bool mixed = false;
     uint64_t packed_stride = 0;              // bytes between experts in `packed`
     bool packed_gu() const { return fused || mixed; }
+    // handles that can be given chunks keep a tile-major copy for the prefill kernels that hold a tile's activations in registers
+    bool tiles_resident() const { return fused && cfg.max_tokens > 8u && cfg.ffn <= 512u && cfg.hidden / 512u <= 4u; }
     // the one-launch router kernels (logits of every expert + the shared expert's gate logit, optional residual + norm) and the
     // one-wave selection serve every layout whose router they tile; the per-row GEMV + generic selection are what is left
     bool fast_route() const {
@@ -142,7 +146,7 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
         }
         if (m->packed_path(ntok)) {     // prefill chunk: tiles of 16 pairs per expert on the MFMA units
             const Layer &L = m->layers[layer];
-            HIP_OK(launch_prefill_packed(L.packed, m->expert_stride, L.shared_packed, m->uid, m->expert_start, m->pair_token, m->n_unique,
+            HIP_OK(launch_prefill_packed(L.packed, m->expert_stride, L.shared_packed, L.tiled, L.shared_tiled, m->uid, m->expert_start, m->pair_token, m->n_unique,
                                          m->tile_group, m->tile_pair0, m->tile_n, m->n_tiles, m->xh, m->xl, m->xexp, m->act_h, m->act_l,
                                          m->act_exp, m->tmp, m->sh_tmp, c.hidden, c.ffn, c.top_k, ntok, c.n_expert, s), "prefill launch");
             prof_set_stage(ST_BATCH_COMBINE);
@@ -252,6 +256,11 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
                  (!sh_packed || hipMalloc(reinterpret_cast<void **>(&L.shared_packed), align256(2u * m->sh_gate_bytes + m->sh_down_bytes)) == hipSuccess);
             m->resident += (uint64_t)c.n_expert * m->packed_stride + (sh_packed ? align256(2u * m->sh_gate_bytes + m->sh_down_bytes) : 0u);
         }
+        if (ok && m->tiles_resident()) {
+            ok = hipMalloc(reinterpret_cast<void **>(&L.tiled), (size_t)c.n_expert * m->expert_stride) == hipSuccess &&
+                 hipMalloc(reinterpret_cast<void **>(&L.shared_tiled), align256(2u * m->sh_gate_bytes + m->sh_down_bytes)) == hipSuccess;
+            m->resident += (uint64_t)c.n_expert * m->expert_stride + align256(2u * m->sh_gate_bytes + m->sh_down_bytes);
+        }
     }
     const size_t T = c.max_tokens;
     const size_t ws_bytes = align256(T * c.hidden * 4u) + align256(T * (c.n_expert + 1u) * 4u) + 2u * align256(T * c.top_k * 4u) + align256(T * 4u) +
@@ -315,6 +324,8 @@ void redhip_moe_destroy(redhip_moe_t h) {
         if (L.experts) (void)hipFree(L.experts);
         if (L.packed) (void)hipFree(L.packed);
         if (L.shared_packed) (void)hipFree(L.shared_packed);
+        if (L.tiled) (void)hipFree(L.tiled);
+        if (L.shared_tiled) (void)hipFree(L.shared_tiled);
     }
     if (m->ws) (void)hipFree(m->ws);
     delete m;
@@ -350,6 +361,10 @@ int redhip_moe_load_shared(redhip_moe_t h, uint32_t layer, const float *gate_inp
         HIP_OK(launch_repack_iq2xxs(L.shared, gate_bytes, 2u, c.ffn, c.hidden, false, L.shared_packed, gate_bytes, nullptr), "shared gate/up repack");
         if (m->fused)
             HIP_OK(launch_repack_iq2xxs(L.shared + 2u * gate_bytes, 0u, 1u, c.hidden, c.ffn, false, L.shared_packed + 2u * gate_bytes, 0u, nullptr), "shared down repack");
+        if (L.shared_tiled) {
+            HIP_OK(launch_tile_packed(L.shared_packed, gate_bytes, 2u, c.ffn, c.hidden, L.shared_tiled, gate_bytes, nullptr), "shared gate/up tiling");
+            HIP_OK(launch_tile_packed(L.shared_packed + 2u * gate_bytes, 0u, 1u, c.hidden, c.ffn, L.shared_tiled + 2u * gate_bytes, 0u, nullptr), "shared down tiling");
+        }
         HIP_OK(hipStreamSynchronize(nullptr), "shared repack");
     }
     return 1;
@@ -374,6 +389,12 @@ int redhip_moe_load_experts(redhip_moe_t h, uint32_t layer, uint32_t first, uint
         HIP_OK(launch_repack_iq2xxs(dst + m->gate_bytes, m->expert_stride, count, c.ffn, c.hidden, false, pk + m->gate_bytes, m->packed_stride, nullptr), "expert up repack");
         if (m->fused)
             HIP_OK(launch_repack_iq2xxs(dst + 2u * m->gate_bytes, m->expert_stride, count, c.hidden, c.ffn, false, pk + 2u * m->gate_bytes, m->packed_stride, nullptr), "expert down repack");
+        if (m->layers[layer].tiled) {
+            uint8_t *tl = m->layers[layer].tiled + (uint64_t)first * m->expert_stride;
+            HIP_OK(launch_tile_packed(pk, m->packed_stride, count, c.ffn, c.hidden, tl, m->expert_stride, nullptr), "expert gate tiling");
+            HIP_OK(launch_tile_packed(pk + m->gate_bytes, m->packed_stride, count, c.ffn, c.hidden, tl + m->gate_bytes, m->expert_stride, nullptr), "expert up tiling");
+            HIP_OK(launch_tile_packed(pk + 2u * m->gate_bytes, m->packed_stride, count, c.hidden, c.ffn, tl + 2u * m->gate_bytes, m->expert_stride, nullptr), "expert down tiling");
+        }
         HIP_OK(hipStreamSynchronize(nullptr), "expert repack");
     }
     return 1;

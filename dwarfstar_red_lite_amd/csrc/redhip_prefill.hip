@@ -80,7 +80,8 @@ __device__ __forceinline__ void decode_entry(uint2 w, uint32_t q, const uint8_t 
     place_signs(*reinterpret_cast<const uint4 *>(lds + (idx << 4)), s7, b0, b1);
 }
 
-union Half8 { uint4 u; half4_t h[2]; };
+typedef _Float16 half8_t __attribute__((ext_vector_type(8)));
+union Half8 { uint4 u; half4_t h[2]; half8_t v; };
 
 // one group of 32 columns: acc = A x B over the group's 32 k, activations hi and lo; returns the four f32 sums of this
 // lane's row against pairs 4q .. 4q + 3, without the scales
@@ -304,6 +305,286 @@ __global__ __launch_bounds__(kWaves * 64) void prefill_down_kernel(PrefillArgs a
     }
 }
 
+// ---------------------------------------------------------------- register-resident tiles on the tile-major layout (ffn <= 512)
+
+// The two kernels above read a tile's activations from LDS again for every 16 weight rows and gather their weights 16 bytes
+// per row. These keep the activations in registers instead: a wave owns a fixed slice of the contraction dimension for the
+// whole tile, so the MFMA A operands (fp16 hi and lo halves, 16 bytes each per group of 32 columns) are loaded once per tile.
+// The weights come from a second, tile-major copy of the packed matrices in which the 32-byte chunks (four groups) of 16
+// consecutive rows lie next to each other, so that one wave-wide load is 512 contiguous bytes:
+//   chunk (row, c)  at ((row / 16 * (K / 128) + c) * 16 + row % 16) * 32          c = chunk of four groups along K
+//   scale (row, b)  at qs_bytes + ((row / 16 * (K / 256) + b) * 16 + row % 16) * 2
+// Decode: a 64 KB LDS table holds the eight fp16 magnitudes of every grid entry times every group scale 2 s + 1 (exact in
+// fp16), a 2 KB table the eight sign masks of every 7-bit sign field, so a lane's eight weights are two table reads and four
+// XORs, and with the group scale folded into the weights the groups of a chunk accumulate in the matrix units
+// (v_mfma_f32_16x16x32_f16: one instruction per group and activation half). The SwiGLU activations of a tile are collected
+// in LDS as f32 and split into fp16 halves with ONE exponent per pair at the end of the tile, so the down kernel scales its
+// sums once per output (22 bits below a pair's largest activation is ample for a dot product).
+constexpr int kRegWaves = 8;
+constexpr uint32_t kScaledMagBytes = 16u * 256u * 16u;      // [group scale s][grid entry]
+constexpr uint32_t kSignBytes = 128u * 16u;                 // [seven sign bits] (the eighth sign is their parity)
+
+// row-major packed matrix -> tile-major copy; one thread per 32-byte chunk, the scales ride along
+__global__ void tile_packed_kernel(const uint8_t *packed, uint64_t packed_stride, uint32_t nrows, uint32_t K, uint8_t *tiled, uint64_t tiled_stride) {
+    const uint32_t NC = K / 128u, NB = K / 256u;
+    const uint64_t gid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= (uint64_t)nrows * NC) return;
+    const uint32_t row = (uint32_t)(gid / NC), c = (uint32_t)(gid % NC);
+    const uint8_t *src = packed + (uint64_t)blockIdx.y * packed_stride;
+    uint8_t *dst = tiled + (uint64_t)blockIdx.y * tiled_stride;
+    const uint64_t qs_bytes = (uint64_t)nrows * (K / 32u) * 8u;
+    const uint4 *sp = reinterpret_cast<const uint4 *>(src + ((uint64_t)row * (K / 32u) + 4u * c) * 8u);
+    uint4 *dp = reinterpret_cast<uint4 *>(dst + (((uint64_t)(row / 16u) * NC + c) * 16u + row % 16u) * 32u);
+    dp[0] = sp[0];
+    dp[1] = sp[1];
+    if ((c & 1u) == 0u) {
+        const uint32_t b = c / 2u;
+        reinterpret_cast<uint16_t *>(dst + qs_bytes)[((uint64_t)(row / 16u) * NB + b) * 16u + row % 16u] =
+            reinterpret_cast<const uint16_t *>(src + qs_bytes)[(uint64_t)row * NB + b];
+    }
+}
+
+hipError_t launch_tile_packed(const void *packed, uint64_t packed_stride, uint32_t count, uint32_t nrows, uint32_t K, void *tiled, uint64_t tiled_stride,
+                              hipStream_t s) {
+    if (!nrows || nrows % 16u || !K || K % 256u || !count || count > 65535u) return hipErrorInvalidValue;
+    const uint64_t total = (uint64_t)nrows * (K / 128u);
+    REDHIP_LAUNCH(tile_packed_kernel, dim3((uint32_t)((total + 255u) / 256u), count), dim3(256), 0, s, static_cast<const uint8_t *>(packed), packed_stride,
+                  nrows, K, static_cast<uint8_t *>(tiled), tiled_stride);
+    return hipGetLastError();
+}
+
+// both decode tables, built once per workgroup
+__device__ __forceinline__ void build_scaled_tables(uint8_t *mag, uint8_t *sgn, uint32_t tid, uint32_t nthreads) {
+    for (uint32_t e = tid; e < 16u * 256u; e += nthreads) {
+        const uint64_t grid_entry = redhip_iq2xxs_grid[e & 255u];
+        const float f = (float)(2u * (e >> 8) + 1u);
+        uint32_t w4[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const _Float16 lo = (_Float16)(f * (float)((uint32_t)(grid_entry >> (16 * i)) & 255u)), hi = (_Float16)(f * (float)((uint32_t)(grid_entry >> (16 * i + 8)) & 255u));
+            w4[i] = (uint32_t)__builtin_bit_cast(uint16_t, lo) | ((uint32_t)__builtin_bit_cast(uint16_t, hi) << 16);
+        }
+        *reinterpret_cast<uint4 *>(mag + (size_t)e * 16u) = make_uint4(w4[0], w4[1], w4[2], w4[3]);
+    }
+    for (uint32_t s7 = tid; s7 < 128u; s7 += nthreads) {
+        const uint32_t s8 = s7 | ((__popc(s7) & 1u) << 7);
+        uint32_t w4[4];
+#pragma unroll
+        for (uint32_t i = 0; i < 4u; ++i) w4[i] = (((s8 >> (2u * i)) & 1u) << 15) | (((s8 >> (2u * i + 1u)) & 1u) << 31);
+        *reinterpret_cast<uint4 *>(sgn + (size_t)s7 * 16u) = make_uint4(w4[0], w4[1], w4[2], w4[3]);
+    }
+}
+
+// the eight signed fp16 weights of grid entry q of a group word, times the group's 2 s + 1
+__device__ __forceinline__ half8_t decode_scaled(uint2 w, uint32_t q, const uint8_t *mag, const uint8_t *sgn) {
+    const uint32_t idx = (w.x >> (8u * q)) & 255u, s7 = (w.y >> (7u * q)) & 127u;
+    const uint4 m = *reinterpret_cast<const uint4 *>(mag + ((((w.y >> 28) << 8) | idx) << 4));
+    const uint4 g = *reinterpret_cast<const uint4 *>(sgn + (s7 << 4));
+    Half8 r;
+    r.u = make_uint4(m.x ^ g.x, m.y ^ g.y, m.z ^ g.z, m.w ^ g.w);
+    return r.v;
+}
+
+struct RowChunk { uint4 a, b; uint32_t d; };      // four groups (32 bytes) of one packed row and the block scale over them
+
+struct TiledArgs {
+    PrefillArgs p;
+    const uint8_t *experts, *shared;      // tile-major copies; same expert stride and matrix offsets as the packed layout
+};
+
+// gate/up + SwiGLU. Wave = (K quarter kc, column half rh): for the unit of 32 FFN columns j it computes the gate row and the
+// up row of column 32 j + 16 rh + r against its quarter of the hidden dimension; the quarters meet in LDS (double-buffered:
+// one barrier per unit).
+template <int NKC>          // hidden = 512 * NKC
+__global__ __launch_bounds__(kRegWaves * 64) void prefill_gateup_reg_kernel(TiledArgs ta) {
+    const PrefillArgs &a = ta.p;
+    constexpr uint32_t H = 512u * NKC, HG = H / 32u, HB = H / 256u, GQ = HG / 4u, NC = H / 128u;   // GQ: groups per K quarter = 4 NKC
+    extern __shared__ __attribute__((aligned(16))) uint8_t dyn[];          // scaled magnitude table | sign table | acts: [16][F + 4] f32
+    __shared__ float part[2][4][kTile][68];                // [unit parity][K quarter][pair][gate 0..31 | up 0..31], padded
+    __shared__ float tok_scale[kTile];
+    __shared__ uint32_t tok_of[kTile];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, r = lane & 15u, q = lane >> 4;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6), kc = wave & 3u, rh = wave >> 2;
+    const uint32_t F = a.ffn, FG = F / 32u, P = a.ntok * a.top_k, AROW = F + 4u;
+    const uint8_t *mag = dyn, *sgn = dyn + kScaledMagBytes;
+    float *acts = reinterpret_cast<float *>(dyn + kScaledMagBytes + kSignBytes);
+    build_scaled_tables(dyn, dyn + kScaledMagBytes, tid, kRegWaves * 64u);
+    const uint32_t T = a.n_tiles[0], U = a.n_unique[0];
+    const uint64_t qs_bytes = (uint64_t)F * HG * 8u, gate_bytes = qs_bytes + (uint64_t)F * HB * 2u;
+
+    for (uint32_t tile = blockIdx.x; tile < T; tile += gridDim.x) {
+        const uint32_t u = a.tile_group[tile], p0 = a.tile_pair0[tile], n = a.tile_n[tile];
+        const uint8_t *ex = u == U ? ta.shared : ta.experts + (uint64_t)a.uid[u] * a.stride;
+        __syncthreads();                                   // the previous tile's readers are done with acts / tok_of; tables are built
+        if (tid < kTile) {
+            const uint32_t p = p0 + tid, tok = tid < n ? (p < P ? a.pair_token[p] : p - P) : 0u;
+            tok_of[tid] = tok;
+            tok_scale[tid] = tid < n ? 0.125f * exp2i(a.xexp[tok]) : 0.0f;
+        }
+        __syncthreads();
+        // this lane's A operands for the whole tile: token of pair r, columns 8 q .. 8 q + 7 of each group of the wave's quarter
+        Half8 xa[GQ], xb[GQ];
+        {
+            const uint64_t base = (uint64_t)tok_of[r] * H + 32u * (kc * GQ) + 8u * q;
+            const bool live = r < n;
+#pragma unroll
+            for (uint32_t g = 0; g < GQ; ++g) {
+                xa[g].u = make_uint4(0u, 0u, 0u, 0u);
+                xb[g].u = xa[g].u;
+                if (live) {
+                    xa[g].u = *reinterpret_cast<const uint4 *>(a.xh + base + 32u * g);
+                    xb[g].u = *reinterpret_cast<const uint4 *>(a.xl + base + 32u * g);
+                }
+            }
+        }
+        auto load_chunk = [&](const uint8_t *mat, uint32_t j, uint32_t c) {
+            const uint32_t rtile = 2u * j + rh, chunk = kc * NKC + c;
+            const uint4 *qp = reinterpret_cast<const uint4 *>(mat + (((uint64_t)rtile * NC + chunk) * 16u + r) * 32u);
+            const uint16_t *dp = reinterpret_cast<const uint16_t *>(mat + qs_bytes) + ((uint64_t)rtile * HB + chunk / 2u) * 16u + r;
+            return RowChunk{qp[0], qp[1], *dp};
+        };
+        const uint8_t *gmat = ex, *umat = ex + gate_bytes;
+        RowChunk cg = load_chunk(gmat, 0u, 0u), cu = load_chunk(umat, 0u, 0u);
+#pragma unroll 1
+        for (uint32_t j = 0; j < FG; ++j) {
+            float4_t totg = {0.0f, 0.0f, 0.0f, 0.0f}, totu = totg;
+#pragma unroll
+            for (uint32_t c = 0; c < (uint32_t)NKC; ++c) {
+                // the chunk after this one (same unit, or the first of the next unit; the last unit reloads itself) is in flight
+                const uint32_t nj = c + 1u < (uint32_t)NKC ? j : (j + 1u < FG ? j + 1u : j), nc = c + 1u < (uint32_t)NKC ? c + 1u : 0u;
+                const RowChunk ng = load_chunk(gmat, nj, nc), nu = load_chunk(umat, nj, nc);
+                const uint2 wg4[4] = {make_uint2(cg.a.x, cg.a.y), make_uint2(cg.a.z, cg.a.w), make_uint2(cg.b.x, cg.b.y), make_uint2(cg.b.z, cg.b.w)};
+                const uint2 wu4[4] = {make_uint2(cu.a.x, cu.a.y), make_uint2(cu.a.z, cu.a.w), make_uint2(cu.b.x, cu.b.y), make_uint2(cu.b.z, cu.b.w)};
+                // the four groups of the chunk share the block scale d: their products add up in the matrix units, activations
+                // hi and lo in accumulators of their own
+                float4_t gh = {0.0f, 0.0f, 0.0f, 0.0f}, gl = gh, uh = gh, ul = gh;
+#pragma unroll
+                for (uint32_t k = 0; k < 4u; ++k) {
+                    const uint32_t g = 4u * c + k;
+                    const half8_t bg = decode_scaled(wg4[k], q, mag, sgn), bu = decode_scaled(wu4[k], q, mag, sgn);
+                    gh = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[g].v, bg, gh, 0, 0, 0);
+                    gl = __builtin_amdgcn_mfma_f32_16x16x32_f16(xb[g].v, bg, gl, 0, 0, 0);
+                    uh = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[g].v, bu, uh, 0, 0, 0);
+                    ul = __builtin_amdgcn_mfma_f32_16x16x32_f16(xb[g].v, bu, ul, 0, 0, 0);
+                }
+                const float dg = scale_to_f32(cg.d), du = scale_to_f32(cu.d);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) {
+                    totg[t] = fmaf(fmaf(gl[t], 4.8828125e-4f, gh[t]), dg, totg[t]);
+                    totu[t] = fmaf(fmaf(ul[t], 4.8828125e-4f, uh[t]), du, totu[t]);
+                }
+                cg = ng;
+                cu = nu;
+            }
+            float (*pt)[kTile][68] = part[j & 1u];
+#pragma unroll
+            for (uint32_t t = 0; t < 4u; ++t) {
+                pt[kc][4u * q + t][16u * rh + r] = totg[t];
+                pt[kc][4u * q + t][32u + 16u * rh + r] = totu[t];
+            }
+            __syncthreads();
+            {   // (pair i, column c) per thread: the four quarters, the token's scale, SwiGLU
+                const uint32_t i = tid >> 5, c = tid & 31u;
+                const float gsum = ((pt[0][i][c] + pt[1][i][c]) + (pt[2][i][c] + pt[3][i][c])) * tok_scale[i];
+                const float usum = ((pt[0][i][32u + c] + pt[1][i][32u + c]) + (pt[2][i][32u + c] + pt[3][i][32u + c])) * tok_scale[i];
+                acts[i * AROW + 32u * j + c] = (gsum / (1.0f + expf(-gsum))) * usum;
+            }
+        }
+        __syncthreads();
+        // one exponent per pair, then the fp16 halves: wave w takes pairs 2 w and 2 w + 1
+#pragma unroll
+        for (uint32_t h = 0; h < 2u; ++h) {
+            const uint32_t i = 2u * wave + h;
+            if (i >= n) continue;                          // wave-uniform
+            float amax = 0.0f;
+            for (uint32_t c = lane; c < F; c += 64u) amax = fmaxf(amax, fabsf(acts[i * AROW + c]));
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+            const int e = prescale_exp(amax);
+            const float inv = exp2i(-e);
+            const uint64_t pr = p0 + i;
+            for (uint32_t c = lane; c < F; c += 64u) split_hi_lo(acts[i * AROW + c], inv, a.act_h + pr * F + c, a.act_l + pr * F + c);
+            if (lane == 0u) a.act_exp[pr] = e;
+        }
+    }
+}
+
+// down. Wave w computes rows 128 b + 16 w + r for b = 0, 1, ... against all ffn columns of the tile; no reduction across waves.
+template <int NFG>          // ffn = 32 * NFG, NFG <= 16
+__global__ __launch_bounds__(kRegWaves * 64) void prefill_down_reg_kernel(TiledArgs ta) {
+    const PrefillArgs &a = ta.p;
+    constexpr uint32_t F = 32u * NFG, FB = F / 256u, NCK = NFG / 4u;
+    extern __shared__ __attribute__((aligned(16))) uint8_t dyn[];          // scaled magnitude table | sign table
+    __shared__ __attribute__((aligned(16))) float pair_scale[kTile];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, r = lane & 15u, q = lane >> 4;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t H = a.hidden, P = a.ntok * a.top_k;
+    const uint8_t *mag = dyn, *sgn = dyn + kScaledMagBytes;
+    build_scaled_tables(dyn, dyn + kScaledMagBytes, tid, kRegWaves * 64u);
+    const uint32_t T = a.n_tiles[0], U = a.n_unique[0];
+    const uint64_t down_off = 2u * ((uint64_t)F * (H / 32u) * 8u + (uint64_t)F * (H / 256u) * 2u), qs_bytes = (uint64_t)H * NFG * 8u;
+    constexpr uint32_t kRowsPerPass = 16u * kRegWaves;
+
+    for (uint32_t tile = blockIdx.x; tile < T; tile += gridDim.x) {
+        const uint32_t u = a.tile_group[tile], p0 = a.tile_pair0[tile], n = a.tile_n[tile];
+        const uint8_t *dn = (u == U ? ta.shared : ta.experts + (uint64_t)a.uid[u] * a.stride) + down_off;
+        __syncthreads();
+        if (tid < kTile) pair_scale[tid] = tid < n ? 0.125f * exp2i(a.act_exp[p0 + tid]) : 0.0f;
+        __syncthreads();
+        Half8 xa[NFG], xb[NFG];
+        {
+            const uint64_t base = (uint64_t)(p0 + r) * F + 8u * q;
+            const bool live = r < n;
+#pragma unroll
+            for (uint32_t g = 0; g < (uint32_t)NFG; ++g) {
+                xa[g].u = make_uint4(0u, 0u, 0u, 0u);
+                xb[g].u = xa[g].u;
+                if (live) {
+                    xa[g].u = *reinterpret_cast<const uint4 *>(a.act_h + base + 32u * g);
+                    xb[g].u = *reinterpret_cast<const uint4 *>(a.act_l + base + 32u * g);
+                }
+            }
+        }
+        const float4_t ps = *reinterpret_cast<const float4_t *>(&pair_scale[4u * q]);
+        auto load_chunk = [&](uint32_t b, uint32_t c) {
+            const uint32_t rtile = kRegWaves * b + wave;
+            const uint4 *qp = reinterpret_cast<const uint4 *>(dn + (((uint64_t)rtile * NCK + c) * 16u + r) * 32u);
+            const uint16_t *dp = reinterpret_cast<const uint16_t *>(dn + qs_bytes) + ((uint64_t)rtile * FB + c / 2u) * 16u + r;
+            return RowChunk{qp[0], qp[1], *dp};
+        };
+        const uint32_t n_pass = H / kRowsPerPass;
+        RowChunk cw = load_chunk(0u, 0u);
+#pragma unroll 1
+        for (uint32_t b = 0; b < n_pass; ++b) {
+            float4_t tot = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+            for (uint32_t c = 0; c < NCK; ++c) {
+                const uint32_t nb = c + 1u < NCK ? b : (b + 1u < n_pass ? b + 1u : b), nc = c + 1u < NCK ? c + 1u : 0u;
+                const RowChunk nw = load_chunk(nb, nc);
+                const uint2 w4[4] = {make_uint2(cw.a.x, cw.a.y), make_uint2(cw.a.z, cw.a.w), make_uint2(cw.b.x, cw.b.y), make_uint2(cw.b.z, cw.b.w)};
+                float4_t hi = {0.0f, 0.0f, 0.0f, 0.0f}, lo = hi;
+#pragma unroll
+                for (uint32_t k = 0; k < 4u; ++k) {
+                    const uint32_t g = 4u * c + k;
+                    const half8_t bw = decode_scaled(w4[k], q, mag, sgn);
+                    hi = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[g].v, bw, hi, 0, 0, 0);
+                    lo = __builtin_amdgcn_mfma_f32_16x16x32_f16(xb[g].v, bw, lo, 0, 0, 0);
+                }
+                const float d = scale_to_f32(cw.d);
+#pragma unroll
+                for (int t = 0; t < 4; ++t) tot[t] = fmaf(fmaf(lo[t], 4.8828125e-4f, hi[t]), d, tot[t]);
+                cw = nw;
+            }
+            const uint32_t row = kRowsPerPass * b + 16u * wave + r;
+#pragma unroll
+            for (uint32_t t = 0; t < 4u; ++t) {
+                const uint32_t i = 4u * q + t, p = p0 + i;
+                if (i < n) (p < P ? a.tmp + (uint64_t)p * H : a.sh_tmp + (uint64_t)(p - P) * H)[row] = ps[t] * tot[t];
+            }
+        }
+    }
+}
+
 // ---------------------------------------------------------------- router logits of a token chunk
 
 // logits[tok][e] = W[e] . x[tok] for an f32 router as a tiled product on v_mfma_f32_16x16x4_f32 (full fp32
@@ -380,7 +661,8 @@ hipError_t launch_router_f32_tiles(const float *w, const float *gate_inp, const 
     return hipGetLastError();
 }
 
-hipError_t launch_prefill_packed(const void *experts, uint64_t stride, const void *shared, const uint32_t *uid, const uint32_t *expert_start,
+hipError_t launch_prefill_packed(const void *experts, uint64_t stride, const void *shared, const void *tiled_experts, const void *tiled_shared,
+                                 const uint32_t *uid, const uint32_t *expert_start,
                                  const uint32_t *pair_token, const uint32_t *n_unique, uint32_t *tile_group, uint32_t *tile_pair0,
                                  uint32_t *tile_n, uint32_t *n_tiles, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l,
                                  int *act_exp, float *tmp, float *sh_tmp, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok,
@@ -396,6 +678,42 @@ hipError_t launch_prefill_packed(const void *experts, uint64_t stride, const voi
                   static_cast<_Float16 *>(act_h), static_cast<_Float16 *>(act_l), act_exp, tmp, sh_tmp, hidden, ffn, top_k, ntok};
     const uint32_t tile_bound = prefill_tile_bound(ntok, top_k, n_expert);
     const dim3 grid(tile_bound < 256u ? tile_bound : 256u), block(kWaves * 64);
+    if (tiled_experts && tiled_shared && ffn <= 512u) {          // tile-major copy present: activations of a tile in registers
+        const TiledArgs ta{a, static_cast<const uint8_t *>(tiled_experts), static_cast<const uint8_t *>(tiled_shared)};
+        const dim3 rblock(kRegWaves * 64);
+        const size_t tab_lds = kScaledMagBytes + kSignBytes, acts_lds = tab_lds + (size_t)kTile * (ffn + 4u) * sizeof(float);
+        prof_set_stage(ST_PREFILL_GATEUP);
+#define REDHIP_PGR(NKC)                                                                                                                   \
+    do {                                                                                                                                  \
+        static bool attr = false;                                                                                                          \
+        if (!attr) {                                                                                                                       \
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(prefill_gateup_reg_kernel<NKC>), hipFuncAttributeMaxDynamicSharedMemorySize, 112 * 1024); \
+            if (e != hipSuccess) return e;                                                                                                 \
+            attr = true;                                                                                                                   \
+        }                                                                                                                                  \
+        REDHIP_LAUNCH(prefill_gateup_reg_kernel<NKC>, grid, rblock, acts_lds, s, ta);                                                      \
+    } while (0)
+        switch (hidden / 512u) {
+            case 1: REDHIP_PGR(1); break;
+            case 2: REDHIP_PGR(2); break;
+            case 4: REDHIP_PGR(4); break;
+            default: return hipErrorInvalidValue;
+        }
+#undef REDHIP_PGR
+        e = hipGetLastError();
+        if (e != hipSuccess) return e;
+        prof_set_stage(ST_PREFILL_DOWN);
+        static bool down_attr = false;
+        if (!down_attr) {
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(prefill_down_reg_kernel<8>), hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
+            if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void *>(prefill_down_reg_kernel<16>), hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
+            if (e != hipSuccess) return e;
+            down_attr = true;
+        }
+        if (ffn == 256u) REDHIP_LAUNCH(prefill_down_reg_kernel<8>, grid, rblock, tab_lds, s, ta);
+        else REDHIP_LAUNCH(prefill_down_reg_kernel<16>, grid, rblock, tab_lds, s, ta);
+        return hipGetLastError();
+    }
     const size_t dyn_lds = (size_t)2u * kTile * (hidden + kRowPad) * 2u;
     prof_set_stage(ST_PREFILL_GATEUP);
 #define REDHIP_PGU(NKC)                                                                                                                   \
