@@ -399,16 +399,16 @@ template <int NKC>          // hidden = 512 * NKC
 __global__ __launch_bounds__(kRegWaves * 64) void prefill_gateup_reg_kernel(TiledArgs ta) {
     const PrefillArgs &a = ta.p;
     constexpr uint32_t H = 512u * NKC, HG = H / 32u, HB = H / 256u, GQ = HG / 4u, NC = H / 128u;   // GQ: groups per K quarter = 4 NKC
-    extern __shared__ __attribute__((aligned(16))) uint8_t dyn[];          // scaled magnitude table | sign table | acts: [16][F + 4] f32
+    extern __shared__ __attribute__((aligned(16))) uint8_t dyn[];          // sign table | scaled magnitude table | acts: [16][F + 4] f32
     __shared__ float part[2][4][kTile][68];                // [unit parity][K quarter][pair][gate 0..31 | up 0..31], padded
     __shared__ float tok_scale[kTile];
     __shared__ uint32_t tok_of[kTile];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, r = lane & 15u, q = lane >> 4;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6), kc = wave & 3u, rh = wave >> 2;
     const uint32_t F = a.ffn, FG = F / 32u, P = a.ntok * a.top_k, AROW = F + 4u;
-    const uint8_t *mag = dyn, *sgn = dyn + kScaledMagBytes;
+    const uint8_t *sgn = dyn, *mag = dyn + kSignBytes;
     float *acts = reinterpret_cast<float *>(dyn + kScaledMagBytes + kSignBytes);
-    build_scaled_tables(dyn, dyn + kScaledMagBytes, tid, kRegWaves * 64u);
+    build_scaled_tables(dyn + kSignBytes, dyn, tid, kRegWaves * 64u);
     const uint32_t T = a.n_tiles[0], U = a.n_unique[0];
     const uint64_t qs_bytes = (uint64_t)F * HG * 8u, gate_bytes = qs_bytes + (uint64_t)F * HB * 2u;
 
@@ -453,6 +453,7 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_gateup_reg_kernel(Tile
                 // the chunk after this one (same unit, or the first of the next unit; the last unit reloads itself) is in flight
                 const uint32_t nj = c + 1u < (uint32_t)NKC ? j : (j + 1u < FG ? j + 1u : j), nc = c + 1u < (uint32_t)NKC ? c + 1u : 0u;
                 const RowChunk ng = load_chunk(gmat, nj, nc), nu = load_chunk(umat, nj, nc);
+                __builtin_amdgcn_sched_barrier(0);         // keeps the loads ahead of the chunk's arithmetic
                 const uint2 wg4[4] = {make_uint2(cg.a.x, cg.a.y), make_uint2(cg.a.z, cg.a.w), make_uint2(cg.b.x, cg.b.y), make_uint2(cg.b.z, cg.b.w)};
                 const uint2 wu4[4] = {make_uint2(cu.a.x, cu.a.y), make_uint2(cu.a.z, cu.a.w), make_uint2(cu.b.x, cu.b.y), make_uint2(cu.b.z, cu.b.w)};
                 // the four groups of the chunk share the block scale d: their products add up in the matrix units, activations
@@ -514,25 +515,33 @@ template <int NFG>          // ffn = 32 * NFG, NFG <= 16
 __global__ __launch_bounds__(kRegWaves * 64) void prefill_down_reg_kernel(TiledArgs ta) {
     const PrefillArgs &a = ta.p;
     constexpr uint32_t F = 32u * NFG, FB = F / 256u, NCK = NFG / 4u;
-    extern __shared__ __attribute__((aligned(16))) uint8_t dyn[];          // scaled magnitude table | sign table
+    extern __shared__ __attribute__((aligned(16))) uint8_t dyn[];          // sign table | scaled magnitude table
     __shared__ __attribute__((aligned(16))) float pair_scale[kTile];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, r = lane & 15u, q = lane >> 4;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t H = a.hidden, P = a.ntok * a.top_k;
-    const uint8_t *mag = dyn, *sgn = dyn + kScaledMagBytes;
-    build_scaled_tables(dyn, dyn + kScaledMagBytes, tid, kRegWaves * 64u);
+    const uint8_t *sgn = dyn, *mag = dyn + kSignBytes;
+    build_scaled_tables(dyn + kSignBytes, dyn, tid, kRegWaves * 64u);
     const uint32_t T = a.n_tiles[0], U = a.n_unique[0];
     const uint64_t down_off = 2u * ((uint64_t)F * (H / 32u) * 8u + (uint64_t)F * (H / 256u) * 2u), qs_bytes = (uint64_t)H * NFG * 8u;
     constexpr uint32_t kRowsPerPass = 16u * kRegWaves;
 
-    for (uint32_t tile = blockIdx.x; tile < T; tile += gridDim.x) {
+    // Work items are half tiles (the row passes of a tile cut in two) so that the last round of the persistent workgroups is
+    // short; a workgroup takes a contiguous range of items and keeps the activations when two of them share a tile.
+    const uint32_t n_pass_tile = H / kRowsPerPass, parts = n_pass_tile % 2u == 0u ? 2u : 1u, n_pass = n_pass_tile / parts;
+    const uint32_t items = T * parts;
+    const uint32_t item_begin = (uint32_t)(((uint64_t)blockIdx.x * items) / gridDim.x), item_end = (uint32_t)(((uint64_t)(blockIdx.x + 1u) * items) / gridDim.x);
+    Half8 xa[NFG], xb[NFG];
+    uint32_t have_tile = 0xffffffffu;
+    for (uint32_t item = item_begin; item < item_end; ++item) {
+        const uint32_t tile = item / parts, pass0 = (item % parts) * n_pass;
         const uint32_t u = a.tile_group[tile], p0 = a.tile_pair0[tile], n = a.tile_n[tile];
         const uint8_t *dn = (u == U ? ta.shared : ta.experts + (uint64_t)a.uid[u] * a.stride) + down_off;
-        __syncthreads();
-        if (tid < kTile) pair_scale[tid] = tid < n ? 0.125f * exp2i(a.act_exp[p0 + tid]) : 0.0f;
-        __syncthreads();
-        Half8 xa[NFG], xb[NFG];
-        {
+        if (tile != have_tile) {
+            have_tile = tile;
+            __syncthreads();
+            if (tid < kTile) pair_scale[tid] = tid < n ? 0.125f * exp2i(a.act_exp[p0 + tid]) : 0.0f;
+            __syncthreads();
             const uint64_t base = (uint64_t)(p0 + r) * F + 8u * q;
             const bool live = r < n;
 #pragma unroll
@@ -547,35 +556,47 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_down_reg_kernel(TiledA
         }
         const float4_t ps = *reinterpret_cast<const float4_t *>(&pair_scale[4u * q]);
         auto load_chunk = [&](uint32_t b, uint32_t c) {
-            const uint32_t rtile = kRegWaves * b + wave;
+            const uint32_t rtile = kRegWaves * (pass0 + b) + wave;
             const uint4 *qp = reinterpret_cast<const uint4 *>(dn + (((uint64_t)rtile * NCK + c) * 16u + r) * 32u);
             const uint16_t *dp = reinterpret_cast<const uint16_t *>(dn + qs_bytes) + ((uint64_t)rtile * FB + c / 2u) * 16u + r;
             return RowChunk{qp[0], qp[1], *dp};
         };
-        const uint32_t n_pass = H / kRowsPerPass;
-        RowChunk cw = load_chunk(0u, 0u);
+        // One buffer per chunk of a pass, reloaded with the same chunk of the next pass as soon as it has been decoded: every load
+        // has a whole pass of work to arrive. Inside a chunk all eight table reads are issued before the first XOR, so their
+        // latency is paid once per chunk.
+        RowChunk cw[NCK];
+#pragma unroll
+        for (uint32_t c = 0; c < NCK; ++c) cw[c] = load_chunk(0u, c);
 #pragma unroll 1
         for (uint32_t b = 0; b < n_pass; ++b) {
             float4_t tot = {0.0f, 0.0f, 0.0f, 0.0f};
+            const uint32_t nb = b + 1u < n_pass ? b + 1u : b;          // the last pass reloads itself: no branch around the loads
 #pragma unroll
             for (uint32_t c = 0; c < NCK; ++c) {
-                const uint32_t nb = c + 1u < NCK ? b : (b + 1u < n_pass ? b + 1u : b), nc = c + 1u < NCK ? c + 1u : 0u;
-                const RowChunk nw = load_chunk(nb, nc);
-                const uint2 w4[4] = {make_uint2(cw.a.x, cw.a.y), make_uint2(cw.a.z, cw.a.w), make_uint2(cw.b.x, cw.b.y), make_uint2(cw.b.z, cw.b.w)};
+                const uint2 w4[4] = {make_uint2(cw[c].a.x, cw[c].a.y), make_uint2(cw[c].a.z, cw[c].a.w), make_uint2(cw[c].b.x, cw[c].b.y), make_uint2(cw[c].b.z, cw[c].b.w)};
+                const float d = scale_to_f32(cw[c].d);
+                cw[c] = load_chunk(nb, c);
+                uint4 tm[4], ts[4];
+#pragma unroll
+                for (uint32_t k = 0; k < 4u; ++k) {
+                    const uint32_t idx = (w4[k].x >> (8u * q)) & 255u, s7 = (w4[k].y >> (7u * q)) & 127u;
+                    tm[k] = *reinterpret_cast<const uint4 *>(mag + ((((w4[k].y >> 28) << 8) | idx) << 4));
+                    ts[k] = *reinterpret_cast<const uint4 *>(sgn + (s7 << 4));
+                }
+                __builtin_amdgcn_sched_barrier(0);         // loads and table reads stay ahead of the arithmetic
                 float4_t hi = {0.0f, 0.0f, 0.0f, 0.0f}, lo = hi;
 #pragma unroll
                 for (uint32_t k = 0; k < 4u; ++k) {
                     const uint32_t g = 4u * c + k;
-                    const half8_t bw = decode_scaled(w4[k], q, mag, sgn);
-                    hi = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[g].v, bw, hi, 0, 0, 0);
-                    lo = __builtin_amdgcn_mfma_f32_16x16x32_f16(xb[g].v, bw, lo, 0, 0, 0);
+                    Half8 bw;
+                    bw.u = make_uint4(tm[k].x ^ ts[k].x, tm[k].y ^ ts[k].y, tm[k].z ^ ts[k].z, tm[k].w ^ ts[k].w);
+                    hi = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[g].v, bw.v, hi, 0, 0, 0);
+                    lo = __builtin_amdgcn_mfma_f32_16x16x32_f16(xb[g].v, bw.v, lo, 0, 0, 0);
                 }
-                const float d = scale_to_f32(cw.d);
 #pragma unroll
                 for (int t = 0; t < 4; ++t) tot[t] = fmaf(fmaf(lo[t], 4.8828125e-4f, hi[t]), d, tot[t]);
-                cw = nw;
             }
-            const uint32_t row = kRowsPerPass * b + 16u * wave + r;
+            const uint32_t row = kRowsPerPass * (pass0 + b) + 16u * wave + r;
 #pragma unroll
             for (uint32_t t = 0; t < 4u; ++t) {
                 const uint32_t i = 4u * q + t, p = p0 + i;
