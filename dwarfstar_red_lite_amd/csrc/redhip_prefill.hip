@@ -318,8 +318,9 @@ __global__ __launch_bounds__(kWaves * 64) void prefill_down_kernel(PrefillArgs a
 // fp16), a 2 KB table the eight sign masks of every 7-bit sign field, so a lane's eight weights are two table reads and four
 // XORs, and with the group scale folded into the weights the groups of a chunk accumulate in the matrix units
 // (v_mfma_f32_16x16x32_f16: one instruction per group and activation half). The SwiGLU activations of a tile are collected
-// in LDS as f32 and split into fp16 halves with ONE exponent per pair at the end of the tile, so the down kernel scales its
-// sums once per output (22 bits below a pair's largest activation is ample for a dot product).
+// in LDS as f32 and split into fp16 halves with one exponent per pair and half of the FFN columns, so the down kernel
+// scales its sums once per chunk instead of once per group (22 bits below the largest activation of 256 columns is ample
+// for a dot product).
 constexpr int kRegWaves = 8;
 constexpr uint32_t kScaledMagBytes = 16u * 256u * 16u;      // [group scale s][grid entry]
 constexpr uint32_t kSignBytes = 128u * 16u;                 // [seven sign bits] (the eighth sign is their parity)
@@ -412,19 +413,27 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_gateup_reg_kernel(Tile
     const uint32_t T = a.n_tiles[0], U = a.n_unique[0];
     const uint64_t qs_bytes = (uint64_t)F * HG * 8u, gate_bytes = qs_bytes + (uint64_t)F * HB * 2u;
 
-    for (uint32_t tile = blockIdx.x; tile < T; tile += gridDim.x) {
+    // Work items are half tiles (one half of the FFN columns, with an activation exponent of its own) so that the last round of
+    // the persistent workgroups is short; a workgroup takes a contiguous range of items and keeps its A operands when two of
+    // them share a tile.
+    const uint32_t items = 2u * T, FGH = FG / 2u;
+    const uint32_t item_begin = (uint32_t)(((uint64_t)blockIdx.x * items) / gridDim.x), item_end = (uint32_t)(((uint64_t)(blockIdx.x + 1u) * items) / gridDim.x);
+    Half8 xa[GQ], xb[GQ];
+    uint32_t have_tile = 0xffffffffu;
+    for (uint32_t item = item_begin; item < item_end; ++item) {
+        const uint32_t tile = item >> 1, half = item & 1u, j0 = half * FGH;
         const uint32_t u = a.tile_group[tile], p0 = a.tile_pair0[tile], n = a.tile_n[tile];
         const uint8_t *ex = u == U ? ta.shared : ta.experts + (uint64_t)a.uid[u] * a.stride;
-        __syncthreads();                                   // the previous tile's readers are done with acts / tok_of; tables are built
-        if (tid < kTile) {
-            const uint32_t p = p0 + tid, tok = tid < n ? (p < P ? a.pair_token[p] : p - P) : 0u;
-            tok_of[tid] = tok;
-            tok_scale[tid] = tid < n ? 0.125f * exp2i(a.xexp[tok]) : 0.0f;
-        }
-        __syncthreads();
-        // this lane's A operands for the whole tile: token of pair r, columns 8 q .. 8 q + 7 of each group of the wave's quarter
-        Half8 xa[GQ], xb[GQ];
-        {
+        __syncthreads();                                   // the previous item's readers are done with acts / tok_of; tables are built
+        if (tile != have_tile) {
+            have_tile = tile;
+            if (tid < kTile) {
+                const uint32_t p = p0 + tid, tok = tid < n ? (p < P ? a.pair_token[p] : p - P) : 0u;
+                tok_of[tid] = tok;
+                tok_scale[tid] = tid < n ? 0.125f * exp2i(a.xexp[tok]) : 0.0f;
+            }
+            __syncthreads();
+            // this lane's A operands for the whole tile: token of pair r, columns 8 q .. 8 q + 7 of each group of the wave's quarter
             const uint64_t base = (uint64_t)tok_of[r] * H + 32u * (kc * GQ) + 8u * q;
             const bool live = r < n;
 #pragma unroll
@@ -444,14 +453,14 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_gateup_reg_kernel(Tile
             return RowChunk{qp[0], qp[1], *dp};
         };
         const uint8_t *gmat = ex, *umat = ex + gate_bytes;
-        RowChunk cg = load_chunk(gmat, 0u, 0u), cu = load_chunk(umat, 0u, 0u);
+        RowChunk cg = load_chunk(gmat, j0, 0u), cu = load_chunk(umat, j0, 0u);
 #pragma unroll 1
-        for (uint32_t j = 0; j < FG; ++j) {
+        for (uint32_t j = j0; j < j0 + FGH; ++j) {
             float4_t totg = {0.0f, 0.0f, 0.0f, 0.0f}, totu = totg;
 #pragma unroll
             for (uint32_t c = 0; c < (uint32_t)NKC; ++c) {
                 // the chunk after this one (same unit, or the first of the next unit; the last unit reloads itself) is in flight
-                const uint32_t nj = c + 1u < (uint32_t)NKC ? j : (j + 1u < FG ? j + 1u : j), nc = c + 1u < (uint32_t)NKC ? c + 1u : 0u;
+                const uint32_t nj = c + 1u < (uint32_t)NKC ? j : (j + 1u < j0 + FGH ? j + 1u : j), nc = c + 1u < (uint32_t)NKC ? c + 1u : 0u;
                 const RowChunk ng = load_chunk(gmat, nj, nc), nu = load_chunk(umat, nj, nc);
                 __builtin_amdgcn_sched_barrier(0);         // keeps the loads ahead of the chunk's arithmetic
                 const uint2 wg4[4] = {make_uint2(cg.a.x, cg.a.y), make_uint2(cg.a.z, cg.a.w), make_uint2(cg.b.x, cg.b.y), make_uint2(cg.b.z, cg.b.w)};
@@ -492,20 +501,21 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_gateup_reg_kernel(Tile
             }
         }
         __syncthreads();
-        // one exponent per pair, then the fp16 halves: wave w takes pairs 2 w and 2 w + 1
+        // one exponent per pair and column half, then the fp16 halves: wave w takes pairs 2 w and 2 w + 1
+        const uint32_t c0 = 32u * j0, c1 = c0 + 32u * FGH;
 #pragma unroll
         for (uint32_t h = 0; h < 2u; ++h) {
             const uint32_t i = 2u * wave + h;
             if (i >= n) continue;                          // wave-uniform
             float amax = 0.0f;
-            for (uint32_t c = lane; c < F; c += 64u) amax = fmaxf(amax, fabsf(acts[i * AROW + c]));
+            for (uint32_t c = c0 + lane; c < c1; c += 64u) amax = fmaxf(amax, fabsf(acts[i * AROW + c]));
 #pragma unroll
             for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
             const int e = prescale_exp(amax);
             const float inv = exp2i(-e);
             const uint64_t pr = p0 + i;
-            for (uint32_t c = lane; c < F; c += 64u) split_hi_lo(acts[i * AROW + c], inv, a.act_h + pr * F + c, a.act_l + pr * F + c);
-            if (lane == 0u) a.act_exp[pr] = e;
+            for (uint32_t c = c0 + lane; c < c1; c += 64u) split_hi_lo(acts[i * AROW + c], inv, a.act_h + pr * F + c, a.act_l + pr * F + c);
+            if (lane == 0u) a.act_exp[2u * pr + half] = e;
         }
     }
 }
@@ -516,7 +526,7 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_down_reg_kernel(TiledA
     const PrefillArgs &a = ta.p;
     constexpr uint32_t F = 32u * NFG, FB = F / 256u, NCK = NFG / 4u;
     extern __shared__ __attribute__((aligned(16))) uint8_t dyn[];          // sign table | scaled magnitude table
-    __shared__ __attribute__((aligned(16))) float pair_scale[kTile];
+    __shared__ __attribute__((aligned(16))) float pair_scale[2][kTile];      // per column half of the activations
     const uint32_t tid = threadIdx.x, lane = tid & 63u, r = lane & 15u, q = lane >> 4;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t H = a.hidden, P = a.ntok * a.top_k;
@@ -540,7 +550,7 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_down_reg_kernel(TiledA
         if (tile != have_tile) {
             have_tile = tile;
             __syncthreads();
-            if (tid < kTile) pair_scale[tid] = tid < n ? 0.125f * exp2i(a.act_exp[p0 + tid]) : 0.0f;
+            if (tid < 2u * kTile) pair_scale[tid & 1u][tid >> 1] = (tid >> 1) < n ? 0.125f * exp2i(a.act_exp[2u * p0 + tid]) : 0.0f;
             __syncthreads();
             const uint64_t base = (uint64_t)(p0 + r) * F + 8u * q;
             const bool live = r < n;
@@ -554,7 +564,7 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_down_reg_kernel(TiledA
                 }
             }
         }
-        const float4_t ps = *reinterpret_cast<const float4_t *>(&pair_scale[4u * q]);
+        const float4_t ps0 = *reinterpret_cast<const float4_t *>(&pair_scale[0][4u * q]), ps1 = *reinterpret_cast<const float4_t *>(&pair_scale[1][4u * q]);
         auto load_chunk = [&](uint32_t b, uint32_t c) {
             const uint32_t rtile = kRegWaves * (pass0 + b) + wave;
             const uint4 *qp = reinterpret_cast<const uint4 *>(dn + (((uint64_t)rtile * NCK + c) * 16u + r) * 32u);
@@ -562,8 +572,7 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_down_reg_kernel(TiledA
             return RowChunk{qp[0], qp[1], *dp};
         };
         // One buffer per chunk of a pass, reloaded with the same chunk of the next pass as soon as it has been decoded: every load
-        // has a whole pass of work to arrive. Inside a chunk all eight table reads are issued before the first XOR, so their
-        // latency is paid once per chunk.
+        // has a whole pass of work to arrive.
         RowChunk cw[NCK];
 #pragma unroll
         for (uint32_t c = 0; c < NCK; ++c) cw[c] = load_chunk(0u, c);
@@ -576,31 +585,23 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_down_reg_kernel(TiledA
                 const uint2 w4[4] = {make_uint2(cw[c].a.x, cw[c].a.y), make_uint2(cw[c].a.z, cw[c].a.w), make_uint2(cw[c].b.x, cw[c].b.y), make_uint2(cw[c].b.z, cw[c].b.w)};
                 const float d = scale_to_f32(cw[c].d);
                 cw[c] = load_chunk(nb, c);
-                uint4 tm[4], ts[4];
-#pragma unroll
-                for (uint32_t k = 0; k < 4u; ++k) {
-                    const uint32_t idx = (w4[k].x >> (8u * q)) & 255u, s7 = (w4[k].y >> (7u * q)) & 127u;
-                    tm[k] = *reinterpret_cast<const uint4 *>(mag + ((((w4[k].y >> 28) << 8) | idx) << 4));
-                    ts[k] = *reinterpret_cast<const uint4 *>(sgn + (s7 << 4));
-                }
-                __builtin_amdgcn_sched_barrier(0);         // loads and table reads stay ahead of the arithmetic
+                __builtin_amdgcn_sched_barrier(0);         // keeps the loads here: the scheduler otherwise sinks them to the end of the pass
                 float4_t hi = {0.0f, 0.0f, 0.0f, 0.0f}, lo = hi;
 #pragma unroll
                 for (uint32_t k = 0; k < 4u; ++k) {
                     const uint32_t g = 4u * c + k;
-                    Half8 bw;
-                    bw.u = make_uint4(tm[k].x ^ ts[k].x, tm[k].y ^ ts[k].y, tm[k].z ^ ts[k].z, tm[k].w ^ ts[k].w);
-                    hi = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[g].v, bw.v, hi, 0, 0, 0);
-                    lo = __builtin_amdgcn_mfma_f32_16x16x32_f16(xb[g].v, bw.v, lo, 0, 0, 0);
+                    const half8_t bw = decode_scaled(w4[k], q, mag, sgn);
+                    hi = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[g].v, bw, hi, 0, 0, 0);
+                    lo = __builtin_amdgcn_mfma_f32_16x16x32_f16(xb[g].v, bw, lo, 0, 0, 0);
                 }
 #pragma unroll
-                for (int t = 0; t < 4; ++t) tot[t] = fmaf(fmaf(lo[t], 4.8828125e-4f, hi[t]), d, tot[t]);
+                for (int t = 0; t < 4; ++t) tot[t] = fmaf(fmaf(lo[t], 4.8828125e-4f, hi[t]) * d, 2u * c < NCK ? ps0[t] : ps1[t], tot[t]);
             }
             const uint32_t row = kRowsPerPass * (pass0 + b) + 16u * wave + r;
 #pragma unroll
             for (uint32_t t = 0; t < 4u; ++t) {
                 const uint32_t i = 4u * q + t, p = p0 + i;
-                if (i < n) (p < P ? a.tmp + (uint64_t)p * H : a.sh_tmp + (uint64_t)(p - P) * H)[row] = ps[t] * tot[t];
+                if (i < n) (p < P ? a.tmp + (uint64_t)p * H : a.sh_tmp + (uint64_t)(p - P) * H)[row] = tot[t];
             }
         }
     }
