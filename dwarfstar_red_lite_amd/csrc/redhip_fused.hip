@@ -1167,6 +1167,7 @@ struct BatchArgs {
     float *out;                    // [ntok][hidden]
     uint32_t hidden, ffn, top_k, ntok;
     const float *resid_a, *resid_b;     // when set: out = (resid_a + resid_b) + layer output, [ntok][hidden] each
+    float *act_f32;                // gate/up kernel: when set, the SwiGLU activations go here as f32 [P][ffn] (a down kernel on raw rows follows)
 };
 
 // Persistent workgroups walk the units (u, g) = (group of pairs, 32 FFN columns): 32 gate + 32 up rows of the
@@ -1190,7 +1191,7 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_batch_kernel(BatchArgs a) 
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t H = a.hidden, F = a.ffn, HG = H / 32u, HB = H / 256u, FG = F / 32u, P = a.ntok * a.top_k;
     const uint64_t grid_entry = tid < 256u ? redhip_iq2xxs_grid[tid] : 0ull;
-    const uint32_t U = a.n_unique[0], n_units = (U + 1u) * FG;
+    const uint32_t U = a.n_unique[0], n_units = (U + (a.shared ? 1u : 0u)) * FG;       // without a packed shared expert: routed groups only
     uint32_t count = 0u;
     if (blockIdx.x < n_units) count = (n_units - blockIdx.x + gridDim.x - 1u) / gridDim.x;
     if (count > (uint32_t)kMaxUnits) count = kMaxUnits;
@@ -1308,8 +1309,12 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_batch_kernel(BatchArgs a) 
                     for (int o = 16; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
                     const int e = prescale_exp(amax);
                     const uint64_t pr = p0 + ip;
-                    split_hi_lo(act, exp2i(-e), a.act_h + pr * F + 32u * g + c, a.act_l + pr * F + 32u * g + c);
-                    if (c == 0u) a.act_exp[pr * FG + g] = e;
+                    if (a.act_f32) {
+                        a.act_f32[pr * F + 32u * g + c] = act;
+                    } else {
+                        split_hi_lo(act, exp2i(-e), a.act_h + pr * F + 32u * g + c, a.act_l + pr * F + 32u * g + c);
+                        if (c == 0u) a.act_exp[pr * FG + g] = e;
+                    }
                 }
             }
         }
@@ -1426,6 +1431,8 @@ __global__ __launch_bounds__(kWaves * 64) void down_batch_kernel(BatchArgs a) {
     }
 }
 
+static hipError_t launch_gateup_batch_kernel(const BatchArgs &a, uint32_t n_groups, hipStream_t s);
+
 hipError_t launch_batch_packed(const void *experts, uint64_t stride, const void *shared, const uint32_t *uid, const uint32_t *expert_start,
                                const uint32_t *pair_token, const uint32_t *n_unique, const float *pair_weight, const uint32_t *tok_pair,
                                const float *scalar, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l, int *act_exp,
@@ -1434,8 +1441,24 @@ hipError_t launch_batch_packed(const void *experts, uint64_t stride, const void 
     BatchArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(shared), uid, expert_start, pair_token, n_unique,
                 pair_weight, tok_pair, scalar, static_cast<const _Float16 *>(xh), static_cast<const _Float16 *>(xl), xexp,
                 static_cast<_Float16 *>(act_h), static_cast<_Float16 *>(act_l), act_exp, out, hidden, ffn, top_k, ntok,
-                block_context().resid_a, block_context().resid_b};
+                block_context().resid_a, block_context().resid_b, nullptr};
     const uint32_t P = ntok * top_k, n_groups = (P < n_expert ? P : n_expert) + 1u;
+    hipError_t e = launch_gateup_batch_kernel(a, n_groups, s);
+    if (e != hipSuccess) return e;
+    prof_set_stage(ST_BATCH_DOWN);
+    const uint32_t groups_per_wave = (n_groups + kWaves - 1u) / kWaves;     // bound known on the host: min(pairs, experts) + 1 groups
+    const dim3 dgrid(hidden / 8u), dblock(kWaves * 64);
+    if (ffn > 512u) REDHIP_LAUNCH((down_batch_kernel<144, 2, 2>), dgrid, dblock, 0, s, a);
+    else if (groups_per_wave <= 2u) REDHIP_LAUNCH((down_batch_kernel<144, 1, 2>), dgrid, dblock, 0, s, a);
+    else if (groups_per_wave <= 3u) REDHIP_LAUNCH((down_batch_kernel<144, 1, 3>), dgrid, dblock, 0, s, a);
+    else if (groups_per_wave <= 4u) REDHIP_LAUNCH((down_batch_kernel<144, 1, 4>), dgrid, dblock, 0, s, a);
+    else REDHIP_LAUNCH((down_batch_kernel<144, 1, 6>), dgrid, dblock, 0, s, a);
+    return hipGetLastError();
+}
+
+// the persistent gate/up kernel of a small batch over n_groups groups of pairs (the shared expert included when a.shared is set)
+static hipError_t launch_gateup_batch_kernel(const BatchArgs &a, uint32_t n_groups, hipStream_t s) {
+    const uint32_t hidden = a.hidden, ffn = a.ffn, ntok = a.ntok;
     const uint32_t unit_bound = n_groups * (ffn / 32u);
     const dim3 grid(256u * ((unit_bound + 256u * kMaxUnits - 1u) / (256u * kMaxUnits)));
     const size_t dyn_lds = (size_t)(2u * ntok + 1u) * (hidden / 32u + 8u) * 64u;   // hi and lo plane per token + a zero plane, 8 pieces of 8 bytes per group
@@ -1461,18 +1484,22 @@ hipError_t launch_batch_packed(const void *experts, uint64_t stride, const void 
         default: return hipErrorInvalidValue;
     }
 #undef REDHIP_GUB
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return e;
-    prof_set_stage(ST_BATCH_DOWN);
-    const uint32_t groups_per_wave = (n_groups + kWaves - 1u) / kWaves;     // bound known on the host: min(pairs, experts) + 1 groups
-    const dim3 dgrid(hidden / 8u), dblock(kWaves * 64);
-    if (ffn > 512u) REDHIP_LAUNCH((down_batch_kernel<144, 2, 2>), dgrid, dblock, 0, s, a);
-    else if (groups_per_wave <= 2u) REDHIP_LAUNCH((down_batch_kernel<144, 1, 2>), dgrid, dblock, 0, s, a);
-    else if (groups_per_wave <= 3u) REDHIP_LAUNCH((down_batch_kernel<144, 1, 3>), dgrid, dblock, 0, s, a);
-    else if (groups_per_wave <= 4u) REDHIP_LAUNCH((down_batch_kernel<144, 1, 4>), dgrid, dblock, 0, s, a);
-    else REDHIP_LAUNCH((down_batch_kernel<144, 1, 6>), dgrid, dblock, 0, s, a);
     return hipGetLastError();
 }
+
+// gate/up + SwiGLU of the routed pairs of a small batch on packed IQ2_XXS gate/up matrices, activations written as f32 [pairs][ffn]:
+// the front half of a layer whose down matrices (and shared expert) are of other types and are read as raw rows afterwards
+hipError_t launch_batch_gateup_packed(const void *experts, uint64_t stride, const uint32_t *uid, const uint32_t *expert_start, const uint32_t *pair_token,
+                                      const uint32_t *n_unique, const void *xh, const void *xl, const int *xexp, float *act, uint32_t hidden,
+                                      uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s) {
+    if (!fused_iq2_supported(hidden, ffn) || !ntok || ntok > (uint32_t)kMaxTok || ntok * top_k + ntok > 144u || !act) return hipErrorInvalidValue;
+    BatchArgs a{static_cast<const uint8_t *>(experts), stride, nullptr, uid, expert_start, pair_token, n_unique, nullptr, nullptr, nullptr,
+                static_cast<const _Float16 *>(xh), static_cast<const _Float16 *>(xl), xexp, nullptr, nullptr, nullptr, nullptr, hidden, ffn, top_k, ntok,
+                nullptr, nullptr, act};
+    const uint32_t P = ntok * top_k;
+    return launch_gateup_batch_kernel(a, P < n_expert ? P : n_expert, s);
+}
+
 
 hipError_t launch_gateup_select(const void *experts, uint64_t stride, const void *shared, const void *shared_q6k, const float *x,
                                 const float *shared_gu, const float *logits, const uint32_t *ids_in, uint32_t *ids_out, float *weights_out,

@@ -166,6 +166,10 @@ hipError_t launch_select_group(const float *logits, uint32_t ntok, uint32_t n_ex
                                uint32_t *tok_pair, uint32_t *n_unique, hipStream_t s);
 // batched gate/up + down/combine over grouped pairs, packed IQ2_XXS, small batches (ntok * (top_k + 1) <= 144).
 // act buffers hold ntok * (top_k + 1) rows (routed pairs, then one row per token for the shared expert).
+// gate/up + SwiGLU of the routed pairs of a small batch (2..8 tokens) on packed IQ2_XXS gate/up matrices; act: f32 [pairs][ffn]
+hipError_t launch_batch_gateup_packed(const void *experts, uint64_t stride, const uint32_t *uid, const uint32_t *expert_start, const uint32_t *pair_token,
+                                      const uint32_t *n_unique, const void *xh, const void *xl, const int *xexp, float *act, uint32_t hidden,
+                                      uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s);
 hipError_t launch_batch_packed(const void *experts, uint64_t stride, const void *shared, const uint32_t *uid, const uint32_t *expert_start,
                                const uint32_t *pair_token, const uint32_t *n_unique, const float *pair_weight, const uint32_t *tok_pair,
                                const float *scalar, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l, int *act_exp,

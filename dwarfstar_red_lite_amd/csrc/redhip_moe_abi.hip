@@ -82,6 +82,10 @@ struct Moe {
     bool small_batch(uint32_t ntok) const {
         return fused && ntok >= 2u && ntok <= 8u && ntok * cfg.top_k <= 128u && ntok * (cfg.top_k + 1u) <= 144u && cfg.hidden / 512u <= 4u;
     }
+    // the same batches on a mixed layout: packed gate/up kernel for the routed pairs, raw-row kernels for the rest
+    bool small_batch_mixed(uint32_t ntok) const {
+        return mixed && ntok >= 2u && ntok <= 8u && ntok * cfg.top_k <= 128u && ntok * (cfg.top_k + 1u) <= 144u && cfg.hidden / 512u <= 4u;
+    }
     // every batch size runs on the packed layout when the layer has one (decode kernel, small-batch kernels, prefill tiles)
     bool packed_path(uint32_t ntok) const { return (fused && (ntok == 1u || small_batch(ntok) || cfg.hidden / 512u <= 4u)) || (mixed && ntok == 1u); }
     ExpertSet routed(uint32_t l) const { return ExpertSet{layers[l].experts, expert_stride, gate_bytes, gate_bytes, gu_type, dn_type}; }
@@ -155,7 +159,11 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
             return 1;
         }
         prof_set_stage(ST_BATCH_GATEUP);
-        HIP_OK(launch_batch_gateup(ex, m->uid, m->expert_start, m->pair_token, m->n_unique, n_groups, P, c.hidden, c.ffn, x, m->act, s), "batched gate/up launch");
+        if (m->small_batch_mixed(ntok))     // xh / xl / xexp come from the router kernel
+            HIP_OK(launch_batch_gateup_packed(m->layers[layer].packed, m->packed_stride, m->uid, m->expert_start, m->pair_token, m->n_unique, m->xh, m->xl,
+                                              m->xexp, m->act, c.hidden, c.ffn, c.top_k, ntok, c.n_expert, s), "batched packed gate/up launch");
+        else
+            HIP_OK(launch_batch_gateup(ex, m->uid, m->expert_start, m->pair_token, m->n_unique, n_groups, P, c.hidden, c.ffn, x, m->act, s), "batched gate/up launch");
         HIP_OK(launch_batch_gateup(sh, nullptr, nullptr, nullptr, nullptr, 1u, ntok, c.hidden, c.ffn, x, m->sh_act, s), "batched shared gate/up launch");
         prof_set_stage(ST_BATCH_DOWN);
         HIP_OK(launch_batch_down(ex, m->uid, m->expert_start, m->n_unique, n_groups, P, c.hidden, c.ffn, m->act, m->tmp, s), "batched down launch");
@@ -450,7 +458,7 @@ int redhip_moe_experts(redhip_moe_t h, uint32_t layer, const float *x_dev, uint3
     if (!check_layer(m, layer)) return 0;
     if (!x_dev || !ids_dev || !weights_dev || !out_dev || !ntok || ntok > m->cfg.max_tokens) { moe_err("invalid expert execution arguments"); return 0; }
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (m->packed_path(ntok)) {
+    if (m->packed_path(ntok) || m->small_batch_mixed(ntok)) {
         prof_set_stage(ST_OTHER);
         HIP_OK(launch_prep(x_dev, m->layers[layer].gate_inp, ntok, m->cfg.hidden, m->xh, m->xl, m->xexp, m->scalar, s), "prep launch");
         return experts_enqueue(m, layer, x_dev, ntok, ids_dev, weights_dev, out_dev, s);
@@ -465,7 +473,7 @@ int redhip_moe_forward(redhip_moe_t h, uint32_t layer, const float *x_dev, uint3
     if (!check_layer(m, layer)) return 0;
     if (!x_dev || !out_dev) { moe_err("null activation pointer"); return 0; }
     const bool select_in_gateup = m->packed_gu() && ntok == 1u;
-    const bool group_in_select = m->small_batch(ntok);
+    const bool group_in_select = m->small_batch(ntok) || m->small_batch_mixed(ntok);
     m->skip_select = select_in_gateup;
     m->select_and_group = group_in_select;
     const int routed = redhip_moe_route(h, layer, x_dev, ntok, nullptr, nullptr, nullptr, stream);
@@ -494,7 +502,7 @@ int redhip_moe_forward_block(redhip_moe_t h, uint32_t layer, const float *x_dev,
     }
     if (ok) {
         const bool select_in_gateup = m->packed_gu() && ntok == 1u;
-        const bool group_in_select = m->small_batch(ntok);
+        const bool group_in_select = m->small_batch(ntok) || m->small_batch_mixed(ntok);
         m->skip_select = select_in_gateup;
         m->select_and_group = group_in_select;
         if (in_router) { bc.branch = branch_dev; bc.norm_w = post_norm_dev; bc.eps = eps; bc.xn_out = m->xn; }
