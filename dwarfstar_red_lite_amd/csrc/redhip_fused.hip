@@ -324,7 +324,7 @@ __global__ __launch_bounds__(256) void router_quant_kernel(const uint8_t *w, Rou
         acc += dpp_f32<kDppRor8>(acc);
         const auto sw = __builtin_amdgcn_permlane16_swap(__float_as_uint(acc), __float_as_uint(acc), false, false);
         acc = __uint_as_float(sw[0]) + __uint_as_float(sw[1]);           // rows of 16 lanes: 0 + 1 and 2 + 3
-        if ((lane & 31u) == 0u && tok == 0u) a.sh_gu[sh_row0 + (lane >> 5)] = acc;
+        if ((lane & 31u) == 0u) a.sh_gu[(uint64_t)tok * 2u * a.ffn + sh_row0 + (lane >> 5)] = acc;
     } else if (r <= a.n_expert) {
         float acc = 0.0f;
         if (r < a.n_expert) {
@@ -369,7 +369,7 @@ hipError_t launch_router_gemv(uint32_t router_type, const void *w, const float *
                               uint32_t n_expert, float *logits, void *xh, void *xl, int *xexp, const void *sh_q6k, float *sh_gu, uint32_t ffn,
                               hipStream_t s) {
     if (!ntok || !hidden || hidden % 256u || !n_expert || n_expert > 1024u) return hipErrorInvalidValue;
-    const bool with_shared = sh_q6k && sh_gu && router_type == T_Q6_K && ntok == 1u && ffn % 4u == 0u;
+    const bool with_shared = sh_q6k && sh_gu && router_type == T_Q6_K && ntok <= 8u && ffn % 4u == 0u;      // sh_gu: [ntok][2 * ffn]
     const BlockContext &bc = block_context();
     if (bc.branch && (!bc.norm_w || !bc.xn_out)) return hipErrorInvalidValue;
     RouterArgs a{x, gate_inp, logits, static_cast<_Float16 *>(xh), static_cast<_Float16 *>(xl), xexp, hidden, n_expert,
@@ -716,6 +716,22 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_select_kernel(GateUpArgs a
 
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
     const uint32_t H = a.hidden, F = a.ffn, HG = H / 32u, HB = H / 256u;
+    if (const uint32_t tok = blockIdx.z) {             // several tokens in one launch: every token is a layer of the grid with buffers of its own
+        const uint64_t t = tok;
+        if (a.x) a.x += t * H;
+        if (a.shared_gu) a.shared_gu += t * 2u * F;
+        if (a.logits) a.logits += t * (a.n_expert + 1u);
+        if (a.ids_in) a.ids_in += t * a.top_k;
+        a.ids_out += t * a.top_k;
+        a.weights_out += t * a.top_k;
+        a.scalar_out += t;
+        a.xh += t * H;
+        a.xl += t * H;
+        a.xexp += t;
+        a.act_h += t * (a.top_k + 1u) * F;
+        a.act_l += t * (a.top_k + 1u) * F;
+        a.act_exp += t * (a.top_k + 1u) * (F / 32u);
+    }
     const uint32_t g = blockIdx.x;                     // FFN column group: act values [32 g, 32 g + 32)
     const uint32_t slot = blockIdx.y;
     const bool is_shared = slot >= a.top_k;
@@ -968,6 +984,17 @@ __global__ __launch_bounds__(kWaves * 64) void down_combine_raw_kernel(DownRawAr
     __shared__ float part[17 * 8];
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
     const uint32_t F = a.ffn, FG = F / 32u, FB = F / 256u, n_slot = a.top_k + 1u;
+    if (const uint32_t tok = blockIdx.y) {             // several tokens in one launch
+        const uint64_t t = tok;
+        a.ids += t * a.top_k;
+        a.weights += t * a.top_k;
+        a.scalar += t;
+        a.act_h += t * n_slot * F;
+        a.act_l += t * n_slot * F;
+        a.act_exp += t * n_slot * FG;
+        a.out += t * a.hidden;
+        if (a.resid_a) { a.resid_a += t * a.hidden; a.resid_b += t * a.hidden; }
+    }
     const uint32_t row0 = 8u * blockIdx.x;
     constexpr uint32_t kMaxBlock = Fmt<TD>::kBlock > Fmt<TS>::kBlock ? Fmt<TD>::kBlock : Fmt<TS>::kBlock;
     if (wave < n_slot) {
@@ -1009,8 +1036,8 @@ __global__ __launch_bounds__(kWaves * 64) void down_combine_raw_kernel(DownRawAr
 }
 
 template <uint32_t TD>
-static hipError_t launch_down_raw_shared(uint32_t ts, const DownRawArgs &a, hipStream_t s) {
-    const dim3 grid(a.hidden / 8u), block(kWaves * 64);
+static hipError_t launch_down_raw_shared(uint32_t ts, const DownRawArgs &a, uint32_t ntok, hipStream_t s) {
+    const dim3 grid(a.hidden / 8u, ntok), block(kWaves * 64);
     const size_t lds = (size_t)(a.top_k + 1u) * 8u * (a.ffn / 256u) * 210u;       // sized for the largest block type; at most 17 x 8 x 4 x 210 bytes
     switch (ts) {
         case T_IQ2_XXS: REDHIP_LAUNCH((down_combine_raw_kernel<TD, T_IQ2_XXS>), grid, block, lds, s, a); break;
@@ -1023,15 +1050,15 @@ static hipError_t launch_down_raw_shared(uint32_t ts, const DownRawArgs &a, hipS
 
 hipError_t launch_down_combine_raw(uint32_t down_type, uint32_t shared_down_type, const void *experts, uint64_t stride, const void *shared,
                                    const uint32_t *ids, const float *weights, const float *scalar, const void *act_h, const void *act_l,
-                                   const int *act_exp, float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, hipStream_t s) {
-    if (!hidden || hidden % 8u || !ffn || ffn % 256u || top_k + 1u > (uint32_t)kWaves) return hipErrorInvalidValue;
+                                   const int *act_exp, float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, hipStream_t s, uint32_t ntok) {
+    if (!hidden || hidden % 8u || !ffn || ffn % 256u || top_k + 1u > (uint32_t)kWaves || !ntok || ntok > 65535u) return hipErrorInvalidValue;
     const DownRawArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(shared), ids, weights, scalar,
                         static_cast<const _Float16 *>(act_h), static_cast<const _Float16 *>(act_l), act_exp, out, hidden, ffn, top_k,
                         block_context().resid_a, block_context().resid_b};
     switch (down_type) {
-        case T_IQ2_XXS: return launch_down_raw_shared<T_IQ2_XXS>(shared_down_type, a, s);
-        case T_IQ3_S: return launch_down_raw_shared<T_IQ3_S>(shared_down_type, a, s);
-        case T_Q6_K: return launch_down_raw_shared<T_Q6_K>(shared_down_type, a, s);
+        case T_IQ2_XXS: return launch_down_raw_shared<T_IQ2_XXS>(shared_down_type, a, ntok, s);
+        case T_IQ3_S: return launch_down_raw_shared<T_IQ3_S>(shared_down_type, a, ntok, s);
+        case T_Q6_K: return launch_down_raw_shared<T_Q6_K>(shared_down_type, a, ntok, s);
         default: return hipErrorInvalidValue;
     }
 }
@@ -1167,7 +1194,6 @@ struct BatchArgs {
     float *out;                    // [ntok][hidden]
     uint32_t hidden, ffn, top_k, ntok;
     const float *resid_a, *resid_b;     // when set: out = (resid_a + resid_b) + layer output, [ntok][hidden] each
-    float *act_f32;                // gate/up kernel: when set, the SwiGLU activations go here as f32 [P][ffn] (a down kernel on raw rows follows)
 };
 
 // Persistent workgroups walk the units (u, g) = (group of pairs, 32 FFN columns): 32 gate + 32 up rows of the
@@ -1191,7 +1217,7 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_batch_kernel(BatchArgs a) 
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t H = a.hidden, F = a.ffn, HG = H / 32u, HB = H / 256u, FG = F / 32u, P = a.ntok * a.top_k;
     const uint64_t grid_entry = tid < 256u ? redhip_iq2xxs_grid[tid] : 0ull;
-    const uint32_t U = a.n_unique[0], n_units = (U + (a.shared ? 1u : 0u)) * FG;       // without a packed shared expert: routed groups only
+    const uint32_t U = a.n_unique[0], n_units = (U + 1u) * FG;
     uint32_t count = 0u;
     if (blockIdx.x < n_units) count = (n_units - blockIdx.x + gridDim.x - 1u) / gridDim.x;
     if (count > (uint32_t)kMaxUnits) count = kMaxUnits;
@@ -1309,12 +1335,8 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_batch_kernel(BatchArgs a) 
                     for (int o = 16; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
                     const int e = prescale_exp(amax);
                     const uint64_t pr = p0 + ip;
-                    if (a.act_f32) {
-                        a.act_f32[pr * F + 32u * g + c] = act;
-                    } else {
-                        split_hi_lo(act, exp2i(-e), a.act_h + pr * F + 32u * g + c, a.act_l + pr * F + 32u * g + c);
-                        if (c == 0u) a.act_exp[pr * FG + g] = e;
-                    }
+                    split_hi_lo(act, exp2i(-e), a.act_h + pr * F + 32u * g + c, a.act_l + pr * F + 32u * g + c);
+                    if (c == 0u) a.act_exp[pr * FG + g] = e;
                 }
             }
         }
@@ -1441,7 +1463,7 @@ hipError_t launch_batch_packed(const void *experts, uint64_t stride, const void 
     BatchArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(shared), uid, expert_start, pair_token, n_unique,
                 pair_weight, tok_pair, scalar, static_cast<const _Float16 *>(xh), static_cast<const _Float16 *>(xl), xexp,
                 static_cast<_Float16 *>(act_h), static_cast<_Float16 *>(act_l), act_exp, out, hidden, ffn, top_k, ntok,
-                block_context().resid_a, block_context().resid_b, nullptr};
+                block_context().resid_a, block_context().resid_b};
     const uint32_t P = ntok * top_k, n_groups = (P < n_expert ? P : n_expert) + 1u;
     hipError_t e = launch_gateup_batch_kernel(a, n_groups, s);
     if (e != hipSuccess) return e;
@@ -1487,29 +1509,16 @@ static hipError_t launch_gateup_batch_kernel(const BatchArgs &a, uint32_t n_grou
     return hipGetLastError();
 }
 
-// gate/up + SwiGLU of the routed pairs of a small batch on packed IQ2_XXS gate/up matrices, activations written as f32 [pairs][ffn]:
-// the front half of a layer whose down matrices (and shared expert) are of other types and are read as raw rows afterwards
-hipError_t launch_batch_gateup_packed(const void *experts, uint64_t stride, const uint32_t *uid, const uint32_t *expert_start, const uint32_t *pair_token,
-                                      const uint32_t *n_unique, const void *xh, const void *xl, const int *xexp, float *act, uint32_t hidden,
-                                      uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s) {
-    if (!fused_iq2_supported(hidden, ffn) || !ntok || ntok > (uint32_t)kMaxTok || ntok * top_k + ntok > 144u || !act) return hipErrorInvalidValue;
-    BatchArgs a{static_cast<const uint8_t *>(experts), stride, nullptr, uid, expert_start, pair_token, n_unique, nullptr, nullptr, nullptr,
-                static_cast<const _Float16 *>(xh), static_cast<const _Float16 *>(xl), xexp, nullptr, nullptr, nullptr, nullptr, hidden, ffn, top_k, ntok,
-                nullptr, nullptr, act};
-    const uint32_t P = ntok * top_k;
-    return launch_gateup_batch_kernel(a, P < n_expert ? P : n_expert, s);
-}
-
 
 hipError_t launch_gateup_select(const void *experts, uint64_t stride, const void *shared, const void *shared_q6k, const float *x,
                                 const float *shared_gu, const float *logits, const uint32_t *ids_in, uint32_t *ids_out, float *weights_out,
                                 float *scalar_out, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l, int *act_exp,
-                                uint32_t hidden, uint32_t ffn, uint32_t n_expert, uint32_t top_k, hipStream_t s) {
-    if (!fused_iq2_supported(hidden, ffn) || (!shared && !shared_gu && (!shared_q6k || !x))) return hipErrorInvalidValue;
+                                uint32_t hidden, uint32_t ffn, uint32_t n_expert, uint32_t top_k, hipStream_t s, uint32_t ntok) {
+    if (!fused_iq2_supported(hidden, ffn) || (!shared && !shared_gu && (!shared_q6k || !x)) || !ntok || ntok > 64u) return hipErrorInvalidValue;
     GateUpArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(shared), static_cast<const uint8_t *>(shared_q6k), x,
                  shared_gu, logits, ids_in, ids_out, weights_out, scalar_out, static_cast<const _Float16 *>(xh), static_cast<const _Float16 *>(xl),
                  xexp, static_cast<_Float16 *>(act_h), static_cast<_Float16 *>(act_l), act_exp, hidden, ffn, n_expert, top_k};
-    const dim3 grid(ffn / 32u, top_k + 1u);
+    const dim3 grid(ffn / 32u, top_k + 1u, ntok);
     const size_t dyn = shared || shared_gu ? 0u : (size_t)64u * (hidden / 256u) * 210u + (size_t)(hidden + hidden / 32u + hidden / 16u) * 4u;   // raw Q6_K rows of one unit of the shared expert, x, sums of 16 x
 #define REDHIP_GUS(NKC)                                                                                                                \
     do {                                                                                                                               \

@@ -166,10 +166,6 @@ hipError_t launch_select_group(const float *logits, uint32_t ntok, uint32_t n_ex
                                uint32_t *tok_pair, uint32_t *n_unique, hipStream_t s);
 // batched gate/up + down/combine over grouped pairs, packed IQ2_XXS, small batches (ntok * (top_k + 1) <= 144).
 // act buffers hold ntok * (top_k + 1) rows (routed pairs, then one row per token for the shared expert).
-// gate/up + SwiGLU of the routed pairs of a small batch (2..8 tokens) on packed IQ2_XXS gate/up matrices; act: f32 [pairs][ffn]
-hipError_t launch_batch_gateup_packed(const void *experts, uint64_t stride, const uint32_t *uid, const uint32_t *expert_start, const uint32_t *pair_token,
-                                      const uint32_t *n_unique, const void *xh, const void *xl, const int *xexp, float *act, uint32_t hidden,
-                                      uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s);
 hipError_t launch_batch_packed(const void *experts, uint64_t stride, const void *shared, const uint32_t *uid, const uint32_t *expert_start,
                                const uint32_t *pair_token, const uint32_t *n_unique, const float *pair_weight, const uint32_t *tok_pair,
                                const float *scalar, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l, int *act_exp,
@@ -180,11 +176,11 @@ hipError_t launch_batch_packed(const void *experts, uint64_t stride, const void 
 hipError_t launch_gateup_select(const void *experts, uint64_t stride, const void *shared, const void *shared_q6k, const float *x,
                                 const float *shared_gu, const float *logits, const uint32_t *ids_in, uint32_t *ids_out, float *weights_out,
                                 float *scalar_out, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l, int *act_exp,
-                                uint32_t hidden, uint32_t ffn, uint32_t n_expert, uint32_t top_k, hipStream_t s);
+                                uint32_t hidden, uint32_t ffn, uint32_t n_expert, uint32_t top_k, hipStream_t s, uint32_t ntok = 1u);
 // down + weighted combine for layouts whose down matrices are raw GGUF rows of any supported type
 hipError_t launch_down_combine_raw(uint32_t down_type, uint32_t shared_down_type, const void *experts, uint64_t stride, const void *shared,
                                    const uint32_t *ids, const float *weights, const float *scalar, const void *act_h, const void *act_l,
-                                   const int *act_exp, float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, hipStream_t s);
+                                   const int *act_exp, float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, hipStream_t s, uint32_t ntok = 1u);
 // single token: out[r] = sum_k weights[k] * down_{ids[k]}[r] . act[k] + scalar * shared_down[r] . act[top_k], k in order
 hipError_t launch_down_combine(const void *experts, uint64_t stride, const void *shared, const uint32_t *ids, const float *weights,
                                const float *scalar, const void *act_h, const void *act_l, const int *act_exp, float *out,

@@ -82,7 +82,8 @@ struct Moe {
     bool small_batch(uint32_t ntok) const {
         return fused && ntok >= 2u && ntok <= 8u && ntok * cfg.top_k <= 128u && ntok * (cfg.top_k + 1u) <= 144u && cfg.hidden / 512u <= 4u;
     }
-    // the same batches on a mixed layout: packed gate/up kernel for the routed pairs, raw-row kernels for the rest
+    // the same batches on a mixed layout run on the single-token kernels, one grid layer per token (tokens rarely share an
+    // expert at these sizes, so reading a shared expert twice costs less than the pair sort and the per-pair kernels)
     bool small_batch_mixed(uint32_t ntok) const {
         return mixed && ntok >= 2u && ntok <= 8u && ntok * cfg.top_k <= 128u && ntok * (cfg.top_k + 1u) <= 144u && cfg.hidden / 512u <= 4u;
     }
@@ -132,7 +133,7 @@ __global__ __launch_bounds__(256) void resid_rms_kernel(const float *x, const fl
 int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const uint32_t *ids, const float *weights,
                     float *out, hipStream_t s, bool select_here = false, bool grouped = false) {
     const redhip_moe_config &c = m->cfg;
-    if (ntok > 1u) {       // group the (token, expert) pairs by expert, run each distinct expert once over its tokens
+    if (ntok > 1u && !m->small_batch_mixed(ntok)) {       // group the (token, expert) pairs by expert, run each distinct expert once over its tokens
         const uint32_t P = ntok * c.top_k, n_groups = P < c.n_expert ? P : c.n_expert;
         const ExpertSet ex = m->routed(layer), sh = m->shared(layer);
         if (!grouped) {
@@ -159,11 +160,7 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
             return 1;
         }
         prof_set_stage(ST_BATCH_GATEUP);
-        if (m->small_batch_mixed(ntok))     // xh / xl / xexp come from the router kernel
-            HIP_OK(launch_batch_gateup_packed(m->layers[layer].packed, m->packed_stride, m->uid, m->expert_start, m->pair_token, m->n_unique, m->xh, m->xl,
-                                              m->xexp, m->act, c.hidden, c.ffn, c.top_k, ntok, c.n_expert, s), "batched packed gate/up launch");
-        else
-            HIP_OK(launch_batch_gateup(ex, m->uid, m->expert_start, m->pair_token, m->n_unique, n_groups, P, c.hidden, c.ffn, x, m->act, s), "batched gate/up launch");
+        HIP_OK(launch_batch_gateup(ex, m->uid, m->expert_start, m->pair_token, m->n_unique, n_groups, P, c.hidden, c.ffn, x, m->act, s), "batched gate/up launch");
         HIP_OK(launch_batch_gateup(sh, nullptr, nullptr, nullptr, nullptr, 1u, ntok, c.hidden, c.ffn, x, m->sh_act, s), "batched shared gate/up launch");
         prof_set_stage(ST_BATCH_DOWN);
         HIP_OK(launch_batch_down(ex, m->uid, m->expert_start, m->n_unique, n_groups, P, c.hidden, c.ffn, m->act, m->tmp, s), "batched down launch");
@@ -179,7 +176,7 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
         HIP_OK(launch_gateup_select(L.packed, m->packed_stride, L.shared_packed, L.shared, x, select_here && m->shared_gu_ready ? m->act : nullptr,
                                     select_here ? m->logits : nullptr, ids, m->ids,
                                     m->weights, m->scalar, m->xh, m->xl, m->xexp, m->act_h, m->act_l, m->act_exp, c.hidden, c.ffn, c.n_expert,
-                                    c.top_k, s), "gate/up launch");
+                                    c.top_k, s, ntok), "gate/up launch");      // ntok > 1: a small batch on a mixed layout, one grid layer per token
         prof_set_stage(ST_DOWN_COMBINE);
         if (m->fused)
             HIP_OK(launch_down_combine(L.packed, m->expert_stride, L.shared_packed, select_here ? m->ids : ids, select_here ? m->weights : weights,
@@ -187,7 +184,7 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
         else
             HIP_OK(launch_down_combine_raw(m->dn_type, m->sh_dn_type, L.experts + 2u * m->gate_bytes, m->expert_stride, L.shared + 2u * m->sh_gate_bytes,
                                            select_here ? m->ids : ids, select_here ? m->weights : weights, m->scalar, m->act_h, m->act_l,
-                                           m->act_exp, out, c.hidden, c.ffn, c.top_k, s), "down/combine launch");
+                                           m->act_exp, out, c.hidden, c.ffn, c.top_k, s, ntok), "down/combine launch");
         prof_set_stage(ST_OTHER);
         return 1;
     }
@@ -419,7 +416,7 @@ int redhip_moe_route(redhip_moe_t h, uint32_t layer, const float *x_dev, uint32_
     if (m->fast_route()) {
         prof_set_stage(ST_ROUTER_GEMV);
         // a Q6_K shared expert of a mixed layout rides along: its gate / up products land in m->act (otherwise unused on this path)
-        m->shared_gu_ready = m->mixed && m->sh_gu_type == T_Q6_K && c.router_type == T_Q6_K && ntok == 1u && c.top_k >= 2u;
+        m->shared_gu_ready = m->mixed && m->sh_gu_type == T_Q6_K && c.router_type == T_Q6_K && (ntok == 1u || m->small_batch_mixed(ntok)) && c.top_k >= 2u;
         if (m->packed_gu() && c.router_type == T_F32 && ntok >= 16u)
             HIP_OK(launch_router_f32_tiles(reinterpret_cast<const float *>(m->layers[layer].router), m->layers[layer].gate_inp, x_dev, ntok, c.hidden,
                                            c.n_expert, m->logits, m->xh, m->xl, m->xexp, s), "router tile launch");
@@ -472,8 +469,8 @@ int redhip_moe_forward(redhip_moe_t h, uint32_t layer, const float *x_dev, uint3
     Moe *m = moe_of(h);
     if (!check_layer(m, layer)) return 0;
     if (!x_dev || !out_dev) { moe_err("null activation pointer"); return 0; }
-    const bool select_in_gateup = m->packed_gu() && ntok == 1u;
-    const bool group_in_select = m->small_batch(ntok) || m->small_batch_mixed(ntok);
+    const bool select_in_gateup = m->packed_gu() && (ntok == 1u || m->small_batch_mixed(ntok));
+    const bool group_in_select = m->small_batch(ntok);
     m->skip_select = select_in_gateup;
     m->select_and_group = group_in_select;
     const int routed = redhip_moe_route(h, layer, x_dev, ntok, nullptr, nullptr, nullptr, stream);
@@ -501,8 +498,8 @@ int redhip_moe_forward_block(redhip_moe_t h, uint32_t layer, const float *x_dev,
         if (hipGetLastError() != hipSuccess) { moe_err("residual + norm launch failed"); ok = 0; }
     }
     if (ok) {
-        const bool select_in_gateup = m->packed_gu() && ntok == 1u;
-        const bool group_in_select = m->small_batch(ntok) || m->small_batch_mixed(ntok);
+        const bool select_in_gateup = m->packed_gu() && (ntok == 1u || m->small_batch_mixed(ntok));
+        const bool group_in_select = m->small_batch(ntok);
         m->skip_select = select_in_gateup;
         m->select_and_group = group_in_select;
         if (in_router) { bc.branch = branch_dev; bc.norm_w = post_norm_dev; bc.eps = eps; bc.xn_out = m->xn; }
