@@ -127,6 +127,11 @@ inline uint32_t prefill_tile_bound(uint32_t ntok, uint32_t top_k, uint32_t n_exp
 // them and ffn <= 512 the kernels that keep a tile's activations in registers run.
 hipError_t launch_tile_packed(const void *packed, uint64_t packed_stride, uint32_t count, uint32_t nrows, uint32_t K, void *tiled, uint64_t tiled_stride,
                               hipStream_t s);
+// routed gate/up + SwiGLU of a chunk on the tile-major copy of packed IQ2_XXS gate/up matrices; act: f32 [pairs][ffn] (mixed layouts)
+hipError_t launch_prefill_gateup_tiled(const void *tiled_experts, uint64_t stride, const uint32_t *uid, const uint32_t *expert_start,
+                                       const uint32_t *pair_token, const uint32_t *n_unique, uint32_t *tile_group, uint32_t *tile_pair0, uint32_t *tile_n,
+                                       uint32_t *n_tiles, const void *xh, const void *xl, const int *xexp, float *act, uint32_t hidden, uint32_t ffn,
+                                       uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s);
 hipError_t launch_prefill_packed(const void *experts, uint64_t stride, const void *shared, const void *tiled_experts, const void *tiled_shared,
                                  const uint32_t *uid, const uint32_t *expert_start,
                                  const uint32_t *pair_token, const uint32_t *n_unique, uint32_t *tile_group, uint32_t *tile_pair0,

@@ -59,7 +59,9 @@ struct Moe {
     uint64_t packed_stride = 0;              // bytes between experts in `packed`
     bool packed_gu() const { return fused || mixed; }
     // handles that can be given chunks keep a tile-major copy for the prefill kernels that hold a tile's activations in registers
-    bool tiles_resident() const { return fused && cfg.max_tokens > 8u && cfg.ffn <= 512u && cfg.hidden / 512u <= 4u; }
+    bool tiles_resident() const { return packed_gu() && cfg.max_tokens > 8u && cfg.ffn <= 512u && cfg.hidden / 512u <= 4u; }
+    // a chunk on a mixed layout: the routed gate/up matrices (packed IQ2_XXS) run on the prefill tiles, the rest on raw rows
+    bool mixed_chunk(uint32_t ntok) const { return mixed && ntok > 8u && tiles_resident(); }
     // the one-launch router kernels (logits of every expert + the shared expert's gate logit, optional residual + norm) and the
     // one-wave selection serve every layout whose router they tile; the per-row GEMV + generic selection are what is left
     bool fast_route() const {
@@ -160,7 +162,13 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
             return 1;
         }
         prof_set_stage(ST_BATCH_GATEUP);
-        HIP_OK(launch_batch_gateup(ex, m->uid, m->expert_start, m->pair_token, m->n_unique, n_groups, P, c.hidden, c.ffn, x, m->act, s), "batched gate/up launch");
+        if (m->mixed_chunk(ntok))      // xh / xl / xexp come from the router kernel or the prep kernel
+            HIP_OK(launch_prefill_gateup_tiled(m->layers[layer].tiled, m->packed_stride, m->uid, m->expert_start, m->pair_token, m->n_unique, m->tile_group,
+                                               m->tile_pair0, m->tile_n, m->n_tiles, m->xh, m->xl, m->xexp, m->act, c.hidden, c.ffn, c.top_k, ntok,
+                                               c.n_expert, s), "tiled gate/up launch");
+        else
+            HIP_OK(launch_batch_gateup(ex, m->uid, m->expert_start, m->pair_token, m->n_unique, n_groups, P, c.hidden, c.ffn, x, m->act, s), "batched gate/up launch");
+        prof_set_stage(ST_BATCH_GATEUP);
         HIP_OK(launch_batch_gateup(sh, nullptr, nullptr, nullptr, nullptr, 1u, ntok, c.hidden, c.ffn, x, m->sh_act, s), "batched shared gate/up launch");
         prof_set_stage(ST_BATCH_DOWN);
         HIP_OK(launch_batch_down(ex, m->uid, m->expert_start, m->n_unique, n_groups, P, c.hidden, c.ffn, m->act, m->tmp, s), "batched down launch");
@@ -262,9 +270,9 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
             m->resident += (uint64_t)c.n_expert * m->packed_stride + (sh_packed ? align256(2u * m->sh_gate_bytes + m->sh_down_bytes) : 0u);
         }
         if (ok && m->tiles_resident()) {
-            ok = hipMalloc(reinterpret_cast<void **>(&L.tiled), (size_t)c.n_expert * m->expert_stride) == hipSuccess &&
-                 hipMalloc(reinterpret_cast<void **>(&L.shared_tiled), align256(2u * m->sh_gate_bytes + m->sh_down_bytes)) == hipSuccess;
-            m->resident += (uint64_t)c.n_expert * m->expert_stride + align256(2u * m->sh_gate_bytes + m->sh_down_bytes);
+            ok = hipMalloc(reinterpret_cast<void **>(&L.tiled), (size_t)c.n_expert * m->packed_stride) == hipSuccess &&
+                 (!m->fused || hipMalloc(reinterpret_cast<void **>(&L.shared_tiled), align256(2u * m->sh_gate_bytes + m->sh_down_bytes)) == hipSuccess);
+            m->resident += (uint64_t)c.n_expert * m->packed_stride + (m->fused ? align256(2u * m->sh_gate_bytes + m->sh_down_bytes) : 0u);
         }
     }
     const size_t T = c.max_tokens;
@@ -395,10 +403,11 @@ int redhip_moe_load_experts(redhip_moe_t h, uint32_t layer, uint32_t first, uint
         if (m->fused)
             HIP_OK(launch_repack_iq2xxs(dst + 2u * m->gate_bytes, m->expert_stride, count, c.hidden, c.ffn, false, pk + 2u * m->gate_bytes, m->packed_stride, nullptr), "expert down repack");
         if (m->layers[layer].tiled) {
-            uint8_t *tl = m->layers[layer].tiled + (uint64_t)first * m->expert_stride;
-            HIP_OK(launch_tile_packed(pk, m->packed_stride, count, c.ffn, c.hidden, tl, m->expert_stride, nullptr), "expert gate tiling");
-            HIP_OK(launch_tile_packed(pk + m->gate_bytes, m->packed_stride, count, c.ffn, c.hidden, tl + m->gate_bytes, m->expert_stride, nullptr), "expert up tiling");
-            HIP_OK(launch_tile_packed(pk + 2u * m->gate_bytes, m->packed_stride, count, c.hidden, c.ffn, tl + 2u * m->gate_bytes, m->expert_stride, nullptr), "expert down tiling");
+            uint8_t *tl = m->layers[layer].tiled + (uint64_t)first * m->packed_stride;
+            HIP_OK(launch_tile_packed(pk, m->packed_stride, count, c.ffn, c.hidden, tl, m->packed_stride, nullptr), "expert gate tiling");
+            HIP_OK(launch_tile_packed(pk + m->gate_bytes, m->packed_stride, count, c.ffn, c.hidden, tl + m->gate_bytes, m->packed_stride, nullptr), "expert up tiling");
+            if (m->fused)
+                HIP_OK(launch_tile_packed(pk + 2u * m->gate_bytes, m->packed_stride, count, c.hidden, c.ffn, tl + 2u * m->gate_bytes, m->packed_stride, nullptr), "expert down tiling");
         }
         HIP_OK(hipStreamSynchronize(nullptr), "expert repack");
     }
@@ -455,7 +464,7 @@ int redhip_moe_experts(redhip_moe_t h, uint32_t layer, const float *x_dev, uint3
     if (!check_layer(m, layer)) return 0;
     if (!x_dev || !ids_dev || !weights_dev || !out_dev || !ntok || ntok > m->cfg.max_tokens) { moe_err("invalid expert execution arguments"); return 0; }
     hipStream_t s = static_cast<hipStream_t>(stream);
-    if (m->packed_path(ntok) || m->small_batch_mixed(ntok)) {
+    if (m->packed_path(ntok) || m->small_batch_mixed(ntok) || m->mixed_chunk(ntok)) {
         prof_set_stage(ST_OTHER);
         HIP_OK(launch_prep(x_dev, m->layers[layer].gate_inp, ntok, m->cfg.hidden, m->xh, m->xl, m->xexp, m->scalar, s), "prep launch");
         return experts_enqueue(m, layer, x_dev, ntok, ids_dev, weights_dev, out_dev, s);

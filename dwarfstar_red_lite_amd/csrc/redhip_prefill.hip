@@ -391,6 +391,7 @@ struct RowChunk { uint4 a, b; uint32_t d; };      // four groups (32 bytes) of o
 struct TiledArgs {
     PrefillArgs p;
     const uint8_t *experts, *shared;      // tile-major copies; same expert stride and matrix offsets as the packed layout
+    float *act_f32;                       // gate/up kernel: when set, the SwiGLU activations go here as f32 [pairs][ffn] (kernels on raw rows follow)
 };
 
 // gate/up + SwiGLU. Wave = (K quarter kc, column half rh): for the unit of 32 FFN columns j it computes the gate row and the
@@ -507,6 +508,10 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_gateup_reg_kernel(Tile
         for (uint32_t h = 0; h < 2u; ++h) {
             const uint32_t i = 2u * wave + h;
             if (i >= n) continue;                          // wave-uniform
+            if (ta.act_f32) {
+                for (uint32_t c = c0 + lane; c < c1; c += 64u) ta.act_f32[(uint64_t)(p0 + i) * F + c] = acts[i * AROW + c];
+                continue;
+            }
             float amax = 0.0f;
             for (uint32_t c = c0 + lane; c < c1; c += 64u) amax = fmaxf(amax, fabsf(acts[i * AROW + c]));
 #pragma unroll
@@ -683,6 +688,50 @@ hipError_t launch_router_f32_tiles(const float *w, const float *gate_inp, const 
     return hipGetLastError();
 }
 
+static hipError_t launch_gateup_reg(const TiledArgs &ta, dim3 grid, hipStream_t s) {
+    const uint32_t hidden = ta.p.hidden, ffn = ta.p.ffn;
+    const size_t acts_lds = kScaledMagBytes + kSignBytes + (size_t)kTile * (ffn + 4u) * sizeof(float);
+    hipError_t e = hipSuccess;
+    prof_set_stage(ST_PREFILL_GATEUP);
+#define REDHIP_PGR(NKC)                                                                                                                   \
+    do {                                                                                                                                  \
+        static bool attr = false;                                                                                                          \
+        if (!attr) {                                                                                                                       \
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(prefill_gateup_reg_kernel<NKC>), hipFuncAttributeMaxDynamicSharedMemorySize, 112 * 1024); \
+            if (e != hipSuccess) return e;                                                                                                 \
+            attr = true;                                                                                                                   \
+        }                                                                                                                                  \
+        REDHIP_LAUNCH(prefill_gateup_reg_kernel<NKC>, grid, dim3(kRegWaves * 64), acts_lds, s, ta);                                        \
+    } while (0)
+    switch (hidden / 512u) {
+        case 1: REDHIP_PGR(1); break;
+        case 2: REDHIP_PGR(2); break;
+        case 4: REDHIP_PGR(4); break;
+        default: return hipErrorInvalidValue;
+    }
+#undef REDHIP_PGR
+    return hipGetLastError();
+}
+
+// routed gate/up + SwiGLU of a chunk on the tile-major copy of packed IQ2_XXS gate/up matrices, activations out as f32 [pairs][ffn]:
+// the front half of a layer whose other matrices are of other types. Needs the pair grouping; the shared expert is not touched.
+hipError_t launch_prefill_gateup_tiled(const void *tiled_experts, uint64_t stride, const uint32_t *uid, const uint32_t *expert_start,
+                                       const uint32_t *pair_token, const uint32_t *n_unique, uint32_t *tile_group, uint32_t *tile_pair0, uint32_t *tile_n,
+                                       uint32_t *n_tiles, const void *xh, const void *xl, const int *xexp, float *act, uint32_t hidden, uint32_t ffn,
+                                       uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s) {
+    if (!fused_iq2_supported(hidden, ffn) || hidden / 512u > 4u || ffn > 512u || !ntok || !tiled_experts || !act) return hipErrorInvalidValue;
+    const uint32_t P = ntok * top_k;
+    prof_set_stage(ST_GROUP);
+    REDHIP_LAUNCH(build_tiles_kernel, dim3(1), dim3(1024), 0, s, expert_start, n_unique, P, 0u, tile_group, tile_pair0, tile_n, n_tiles);      // no shared tiles
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    PrefillArgs a{nullptr, stride, nullptr, uid, pair_token, n_unique, tile_group, tile_pair0, tile_n, n_tiles, static_cast<const _Float16 *>(xh),
+                  static_cast<const _Float16 *>(xl), xexp, nullptr, nullptr, nullptr, nullptr, nullptr, hidden, ffn, top_k, ntok};
+    const TiledArgs ta{a, static_cast<const uint8_t *>(tiled_experts), nullptr, act};
+    const uint32_t tile_bound = prefill_tile_bound(ntok, top_k, n_expert);
+    return launch_gateup_reg(ta, dim3(tile_bound < 256u ? tile_bound : 256u), s);
+}
+
 hipError_t launch_prefill_packed(const void *experts, uint64_t stride, const void *shared, const void *tiled_experts, const void *tiled_shared,
                                  const uint32_t *uid, const uint32_t *expert_start,
                                  const uint32_t *pair_token, const uint32_t *n_unique, uint32_t *tile_group, uint32_t *tile_pair0,
@@ -701,28 +750,10 @@ hipError_t launch_prefill_packed(const void *experts, uint64_t stride, const voi
     const uint32_t tile_bound = prefill_tile_bound(ntok, top_k, n_expert);
     const dim3 grid(tile_bound < 256u ? tile_bound : 256u), block(kWaves * 64);
     if (tiled_experts && tiled_shared && ffn <= 512u) {          // tile-major copy present: activations of a tile in registers
-        const TiledArgs ta{a, static_cast<const uint8_t *>(tiled_experts), static_cast<const uint8_t *>(tiled_shared)};
+        const TiledArgs ta{a, static_cast<const uint8_t *>(tiled_experts), static_cast<const uint8_t *>(tiled_shared), nullptr};
         const dim3 rblock(kRegWaves * 64);
-        const size_t tab_lds = kScaledMagBytes + kSignBytes, acts_lds = tab_lds + (size_t)kTile * (ffn + 4u) * sizeof(float);
-        prof_set_stage(ST_PREFILL_GATEUP);
-#define REDHIP_PGR(NKC)                                                                                                                   \
-    do {                                                                                                                                  \
-        static bool attr = false;                                                                                                          \
-        if (!attr) {                                                                                                                       \
-            e = hipFuncSetAttribute(reinterpret_cast<const void *>(prefill_gateup_reg_kernel<NKC>), hipFuncAttributeMaxDynamicSharedMemorySize, 112 * 1024); \
-            if (e != hipSuccess) return e;                                                                                                 \
-            attr = true;                                                                                                                   \
-        }                                                                                                                                  \
-        REDHIP_LAUNCH(prefill_gateup_reg_kernel<NKC>, grid, rblock, acts_lds, s, ta);                                                      \
-    } while (0)
-        switch (hidden / 512u) {
-            case 1: REDHIP_PGR(1); break;
-            case 2: REDHIP_PGR(2); break;
-            case 4: REDHIP_PGR(4); break;
-            default: return hipErrorInvalidValue;
-        }
-#undef REDHIP_PGR
-        e = hipGetLastError();
+        const size_t tab_lds = kScaledMagBytes + kSignBytes;
+        e = launch_gateup_reg(ta, grid, s);
         if (e != hipSuccess) return e;
         prof_set_stage(ST_PREFILL_DOWN);
         static bool down_attr = false;
