@@ -114,6 +114,10 @@ hipError_t launch_batch_combine(const float *tmp, const float *pair_weight, cons
 // pair sort of [ntok][top_k] ids: see redhip_moe_group in include/redhip_moe.h
 // f32 router logits of a chunk of tokens as a tiled fp32 MFMA product (every router row read once per 32 tokens), plus the
 // fp16 split of the activations; same outputs as launch_router_gemv
+// out[tok][row] = W[row] . x[tok] on the fp32 matrix units: W f32 [n_rows][K] (+ one optional extra row), x f32 [ntok][K]
+hipError_t launch_f32_tiles(const float *w, const float *extra_row, const float *x, uint32_t ntok, uint32_t K, uint32_t n_rows, float *out,
+                            uint32_t out_stride, void *xh, void *xl, int *xexp, hipStream_t s);
+hipError_t launch_swiglu_rows(const float *gu, uint32_t gu_stride, uint32_t ntok, uint32_t ffn, float *act, hipStream_t s);
 hipError_t launch_router_f32_tiles(const float *w, const float *gate_inp, const float *x, uint32_t ntok, uint32_t hidden, uint32_t n_expert,
                                    float *logits, void *xh, void *xl, int *xexp, hipStream_t s);
 // prefill chunk on packed IQ2_XXS experts: tiles of 16 pairs per distinct expert, 16x16x16 fp16 MFMA. Needs the pair

@@ -36,6 +36,9 @@ struct Layer {
     uint8_t *shared_packed = nullptr;
     uint8_t *tiled = nullptr;        // third copy, tile-major, read by the prefill kernels (handles that take chunks only)
     uint8_t *shared_tiled = nullptr;
+    // mixed layouts that take chunks: f32 copies of the small dense matrices (dequantised once at upload) for the fp32 tile
+    // kernel: router [n_expert][hidden] (when it is quantised), shared gate | up [2 ffn][hidden], shared down [hidden][ffn]
+    float *dense_router = nullptr, *dense_gu = nullptr, *dense_down = nullptr;
 };
 
 struct Moe {
@@ -59,6 +62,10 @@ struct Moe {
     uint64_t packed_stride = 0;              // bytes between experts in `packed`
     bool packed_gu() const { return fused || mixed; }
     // handles that can be given chunks keep a tile-major copy for the prefill kernels that hold a tile's activations in registers
+    // chunks of 16 tokens and more take the router as a tiled f32 product (a quantised router through its f32 copy)
+    bool tiled_router(uint32_t ntok) const {
+        return packed_gu() && ntok >= 16u && (cfg.router_type == T_F32 || (mixed && tiles_resident()));
+    }
     bool tiles_resident() const { return packed_gu() && cfg.max_tokens > 8u && cfg.ffn <= 512u && cfg.hidden / 512u <= 4u; }
     // a chunk on a mixed layout: the routed gate/up matrices (packed IQ2_XXS) run on the prefill tiles, the rest on raw rows
     bool mixed_chunk(uint32_t ntok) const { return mixed && ntok > 8u && tiles_resident(); }
@@ -169,10 +176,21 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
         else
             HIP_OK(launch_batch_gateup(ex, m->uid, m->expert_start, m->pair_token, m->n_unique, n_groups, P, c.hidden, c.ffn, x, m->act, s), "batched gate/up launch");
         prof_set_stage(ST_BATCH_GATEUP);
-        HIP_OK(launch_batch_gateup(sh, nullptr, nullptr, nullptr, nullptr, 1u, ntok, c.hidden, c.ffn, x, m->sh_act, s), "batched shared gate/up launch");
+        const Layer &Ld = m->layers[layer];
+        const bool dense_shared = m->mixed_chunk(ntok) && Ld.dense_gu;      // the shared expert as two dense f32 products on the fp32 matrix units
+        if (dense_shared) {
+            float *gu = m->tmp;                          // [ntok][2 ffn]; free until the routed down kernel writes tmp (2 ffn <= top_k * hidden)
+            HIP_OK(launch_f32_tiles(Ld.dense_gu, nullptr, x, ntok, c.hidden, 2u * c.ffn, gu, 2u * c.ffn, nullptr, nullptr, nullptr, s), "shared gate/up tiles");
+            HIP_OK(launch_swiglu_rows(gu, 2u * c.ffn, ntok, c.ffn, m->sh_act, s), "shared SwiGLU");
+        } else {
+            HIP_OK(launch_batch_gateup(sh, nullptr, nullptr, nullptr, nullptr, 1u, ntok, c.hidden, c.ffn, x, m->sh_act, s), "batched shared gate/up launch");
+        }
         prof_set_stage(ST_BATCH_DOWN);
         HIP_OK(launch_batch_down(ex, m->uid, m->expert_start, m->n_unique, n_groups, P, c.hidden, c.ffn, m->act, m->tmp, s), "batched down launch");
-        HIP_OK(launch_batch_down(sh, nullptr, nullptr, nullptr, 1u, ntok, c.hidden, c.ffn, m->sh_act, m->sh_tmp, s), "batched shared down launch");
+        if (dense_shared)
+            HIP_OK(launch_f32_tiles(Ld.dense_down, nullptr, m->sh_act, ntok, c.ffn, c.hidden, m->sh_tmp, c.hidden, nullptr, nullptr, nullptr, s), "shared down tiles");
+        else
+            HIP_OK(launch_batch_down(sh, nullptr, nullptr, nullptr, 1u, ntok, c.hidden, c.ffn, m->sh_act, m->sh_tmp, s), "batched shared down launch");
         prof_set_stage(ST_BATCH_COMBINE);
         HIP_OK(launch_batch_combine(m->tmp, m->pair_weight, m->tok_pair, ntok, c.top_k, m->sh_tmp, m->scalar, c.hidden, out, s), "batched combine launch");
         prof_set_stage(ST_OTHER);
@@ -269,6 +287,17 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
                  (!sh_packed || hipMalloc(reinterpret_cast<void **>(&L.shared_packed), align256(2u * m->sh_gate_bytes + m->sh_down_bytes)) == hipSuccess);
             m->resident += (uint64_t)c.n_expert * m->packed_stride + (sh_packed ? align256(2u * m->sh_gate_bytes + m->sh_down_bytes) : 0u);
         }
+        if (ok && m->mixed && m->tiles_resident()) {
+            const size_t rb = c.router_type == T_F32 ? 0u : (size_t)c.n_expert * c.hidden * 4u, gb = (size_t)2u * c.ffn * c.hidden * 4u, db = (size_t)c.hidden * c.ffn * 4u;
+            float *d = nullptr;
+            ok = hipMalloc(reinterpret_cast<void **>(&d), align256(rb) + align256(gb) + align256(db)) == hipSuccess;
+            if (ok) {
+                L.dense_router = rb ? d : nullptr;
+                L.dense_gu = reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(d) + align256(rb));
+                L.dense_down = reinterpret_cast<float *>(reinterpret_cast<uint8_t *>(L.dense_gu) + align256(gb));
+                m->resident += align256(rb) + align256(gb) + align256(db);
+            }
+        }
         if (ok && m->tiles_resident()) {
             ok = hipMalloc(reinterpret_cast<void **>(&L.tiled), (size_t)c.n_expert * m->packed_stride) == hipSuccess &&
                  (!m->fused || hipMalloc(reinterpret_cast<void **>(&L.shared_tiled), align256(2u * m->sh_gate_bytes + m->sh_down_bytes)) == hipSuccess);
@@ -337,6 +366,7 @@ void redhip_moe_destroy(redhip_moe_t h) {
         if (L.experts) (void)hipFree(L.experts);
         if (L.packed) (void)hipFree(L.packed);
         if (L.shared_packed) (void)hipFree(L.shared_packed);
+        if (L.dense_gu) (void)hipFree(L.dense_router ? L.dense_router : L.dense_gu);
         if (L.tiled) (void)hipFree(L.tiled);
         if (L.shared_tiled) (void)hipFree(L.shared_tiled);
     }
@@ -351,6 +381,10 @@ int redhip_moe_load_router(redhip_moe_t h, uint32_t layer, const void *weights, 
     if (!check_layer(m, layer)) return 0;
     if (!weights || bytes != m->router_bytes) { moe_err("router byte size mismatch: got %llu expected %llu", (unsigned long long)bytes, (unsigned long long)m->router_bytes); return 0; }
     HIP_OK(hipMemcpy(m->layers[layer].router, weights, (size_t)bytes, hipMemcpyDefault), "router upload");
+    if (m->layers[layer].dense_router) {
+        HIP_OK(launch_dequant_rows(m->cfg.router_type, m->layers[layer].router, m->cfg.n_expert, m->cfg.hidden, m->layers[layer].dense_router, nullptr), "router dequant");
+        HIP_OK(hipStreamSynchronize(nullptr), "router dequant");
+    }
     return 1;
 }
 
@@ -369,6 +403,12 @@ int redhip_moe_load_shared(redhip_moe_t h, uint32_t layer, const float *gate_inp
     HIP_OK(hipMemcpy(L.shared, gate, (size_t)gate_bytes, hipMemcpyDefault), "shared gate upload");
     HIP_OK(hipMemcpy(L.shared + gate_bytes, up, (size_t)up_bytes, hipMemcpyDefault), "shared up upload");
     HIP_OK(hipMemcpy(L.shared + 2u * gate_bytes, down, (size_t)down_bytes, hipMemcpyDefault), "shared down upload");
+    if (L.dense_gu) {
+        const redhip_moe_config &c = m->cfg;
+        HIP_OK(launch_dequant_rows(m->sh_gu_type, L.shared, 2u * c.ffn, c.hidden, L.dense_gu, nullptr), "shared gate/up dequant");
+        HIP_OK(launch_dequant_rows(m->sh_dn_type, L.shared + 2u * gate_bytes, c.hidden, c.ffn, L.dense_down, nullptr), "shared down dequant");
+        HIP_OK(hipStreamSynchronize(nullptr), "shared dequant");
+    }
     if (L.shared_packed) {
         const redhip_moe_config &c = m->cfg;
         HIP_OK(launch_repack_iq2xxs(L.shared, gate_bytes, 2u, c.ffn, c.hidden, false, L.shared_packed, gate_bytes, nullptr), "shared gate/up repack");
@@ -426,8 +466,9 @@ int redhip_moe_route(redhip_moe_t h, uint32_t layer, const float *x_dev, uint32_
         prof_set_stage(ST_ROUTER_GEMV);
         // a Q6_K shared expert of a mixed layout rides along: its gate / up products land in m->act (otherwise unused on this path)
         m->shared_gu_ready = m->mixed && m->sh_gu_type == T_Q6_K && c.router_type == T_Q6_K && (ntok == 1u || m->small_batch_mixed(ntok)) && c.top_k >= 2u;
-        if (m->packed_gu() && c.router_type == T_F32 && ntok >= 16u)
-            HIP_OK(launch_router_f32_tiles(reinterpret_cast<const float *>(m->layers[layer].router), m->layers[layer].gate_inp, x_dev, ntok, c.hidden,
+        const float *router_f32 = c.router_type == T_F32 ? reinterpret_cast<const float *>(m->layers[layer].router) : m->layers[layer].dense_router;
+        if (m->tiled_router(ntok))
+            HIP_OK(launch_router_f32_tiles(router_f32, m->layers[layer].gate_inp, x_dev, ntok, c.hidden,
                                            c.n_expert, m->logits, m->xh, m->xl, m->xexp, s), "router tile launch");
         else
             HIP_OK(launch_router_gemv(c.router_type, m->layers[layer].router, x_dev, m->layers[layer].gate_inp, ntok, c.hidden, c.n_expert,
@@ -499,7 +540,7 @@ int redhip_moe_forward_block(redhip_moe_t h, uint32_t layer, const float *x_dev,
     BlockContext &bc = block_context();
     bc = BlockContext{};
     // the per-token router kernels of the packed paths normalise on the fly; everything else gets a kernel of its own
-    const bool in_router = m->fast_route() && !(m->packed_gu() && c.router_type == T_F32 && ntok >= 16u);
+    const bool in_router = m->fast_route() && !m->tiled_router(ntok);
     int ok = 1;
     if (!in_router) {
         prof_set_stage(ST_OTHER);

@@ -618,13 +618,14 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_down_reg_kernel(TiledA
 // multiply-add): a workgroup owns 16 router rows x 16 tokens and its four waves each take a quarter of the hidden dimension,
 // so that a compute unit holds enough waves to cover the load latency; the four partial tiles meet in LDS and are added in a
 // fixed order. Lane (r = l % 16, q = l / 16) loads four consecutive k of row r and of token r per 16 k and feeds them to four
-// MFMAs (A[i = r][k = q], B[k = q][j = r], D[i = 4q .. 4q + 3][j = r]); row n_expert is the shared expert's gate vector. A
-// second kind of workgroup (blockIdx.x beyond the row tiles) does the fp16 split of its tokens' activations.
-__global__ __launch_bounds__(256) void router_f32_tile_kernel(const float *w, const float *gate_inp, const float *x, float *logits,
+// MFMAs (A[i = r][k = q], B[k = q][j = r], D[i = 4q .. 4q + 3][j = r]); with `gate_inp` set, row E is that vector (the shared
+// expert's gate). A second kind of workgroup (blockIdx.x beyond the row tiles, launched when xh is set) does the fp16 split of
+// its tokens' activations. The same kernel multiplies any f32 matrix [E][H] with a chunk of activations (dense shared expert).
+__global__ __launch_bounds__(256) void router_f32_tile_kernel(const float *w, const float *gate_inp, const float *x, float *logits, uint32_t out_stride,
                                                               _Float16 *xh, _Float16 *xl, int *xexp, uint32_t H, uint32_t E, uint32_t ntok) {
     __shared__ float part[4][16][17];
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, r = lane & 15u, q = lane >> 4;
-    const uint32_t row_tiles = (E + 1u + 15u) / 16u;
+    const uint32_t n_rows = E + (gate_inp ? 1u : 0u), row_tiles = (n_rows + 15u) / 16u;
     if (blockIdx.x >= row_tiles) {                         // split job: one wave per token, 4 tokens per workgroup
         const uint32_t tok = 4u * (blockIdx.y * (gridDim.x - row_tiles) + (blockIdx.x - row_tiles)) + wave;
         if (tok >= ntok) return;
@@ -640,7 +641,7 @@ __global__ __launch_bounds__(256) void router_f32_tile_kernel(const float *w, co
         return;
     }
     const uint32_t row = 16u * blockIdx.x + r, tok = 16u * blockIdx.y + r, kq = H / 4u;          // this wave: k in [wave * kq, (wave + 1) * kq)
-    const float *wr = (row < E ? w + (uint64_t)row * H : gate_inp) + wave * kq;          // rows beyond E + 1 repeat the gate vector and are not stored
+    const float *wr = (row < E ? w + (uint64_t)row * H : gate_inp ? gate_inp : w) + wave * kq;      // rows beyond the last one repeat another and are not stored
     const float *xt = x + (uint64_t)(tok < ntok ? tok : ntok - 1u) * H + wave * kq;
     // 64 k per step: four loads of 16 bytes per operand, those of the next step in flight while this one is multiplied;
     // two accumulators halve the chain of dependent MFMAs
@@ -673,18 +674,38 @@ __global__ __launch_bounds__(256) void router_f32_tile_kernel(const float *w, co
     __syncthreads();
     const uint32_t i = tid & 15u, j = tid >> 4;             // consecutive threads store consecutive rows of one token
     const uint32_t out_row = 16u * blockIdx.x + i, out_tok = 16u * blockIdx.y + j;
-    if (out_tok < ntok && out_row <= E)
-        logits[(uint64_t)out_tok * (E + 1u) + out_row] = (part[0][j][i] + part[1][j][i]) + (part[2][j][i] + part[3][j][i]);
+    if (out_tok < ntok && out_row < n_rows)
+        logits[(uint64_t)out_tok * out_stride + out_row] = (part[0][j][i] + part[1][j][i]) + (part[2][j][i] + part[3][j][i]);
+}
+
+// out[tok][row] = W[row] . x[tok] for an f32 matrix W [n_rows][K] and a chunk of activations x [ntok][K]; extra_row (optional) is one more
+// row behind the matrix; xh / xl / xexp (optional): also write the fp16 halves of x
+hipError_t launch_f32_tiles(const float *w, const float *extra_row, const float *x, uint32_t ntok, uint32_t K, uint32_t n_rows, float *out,
+                            uint32_t out_stride, void *xh, void *xl, int *xexp, hipStream_t s) {
+    if (!ntok || !K || K % 256u || !n_rows || !w || !x || !out) return hipErrorInvalidValue;
+    const uint32_t row_tiles = (n_rows + (extra_row ? 1u : 0u) + 15u) / 16u, tok_tiles = (ntok + 15u) / 16u;
+    if (tok_tiles > 65535u) return hipErrorInvalidValue;
+    const uint32_t split_wgs = xh ? ((ntok + 3u) / 4u + tok_tiles - 1u) / tok_tiles : 0u;            // per blockIdx.y
+    REDHIP_LAUNCH(router_f32_tile_kernel, dim3(row_tiles + split_wgs, tok_tiles), dim3(256), 0, s, w, extra_row, x, out, out_stride,
+                  static_cast<_Float16 *>(xh), static_cast<_Float16 *>(xl), xexp, K, n_rows, ntok);
+    return hipGetLastError();
 }
 
 hipError_t launch_router_f32_tiles(const float *w, const float *gate_inp, const float *x, uint32_t ntok, uint32_t hidden, uint32_t n_expert,
                                    float *logits, void *xh, void *xl, int *xexp, hipStream_t s) {
-    if (!ntok || !hidden || hidden % 256u || !n_expert) return hipErrorInvalidValue;
-    const uint32_t row_tiles = (n_expert + 1u + 15u) / 16u, tok_tiles = (ntok + 15u) / 16u;
-    if (tok_tiles > 65535u) return hipErrorInvalidValue;
-    const uint32_t split_wgs = ((ntok + 3u) / 4u + tok_tiles - 1u) / tok_tiles;            // per blockIdx.y
-    REDHIP_LAUNCH(router_f32_tile_kernel, dim3(row_tiles + split_wgs, tok_tiles), dim3(256), 0, s, w, gate_inp, x, logits,
-                  static_cast<_Float16 *>(xh), static_cast<_Float16 *>(xl), xexp, hidden, n_expert, ntok);
+    return launch_f32_tiles(w, gate_inp, x, ntok, hidden, n_expert, logits, n_expert + 1u, xh, xl, xexp, s);
+}
+
+// act[tok][c] = silu(gu[tok][c]) * gu[tok][ffn + c]
+__global__ void swiglu_rows_kernel(const float *gu, uint32_t gu_stride, uint32_t ffn, float *act) {
+    const uint32_t c = blockIdx.x * blockDim.x + threadIdx.x, tok = blockIdx.y;
+    if (c >= ffn) return;
+    const float g = gu[(uint64_t)tok * gu_stride + c], u = gu[(uint64_t)tok * gu_stride + ffn + c];
+    act[(uint64_t)tok * ffn + c] = (g / (1.0f + expf(-g))) * u;
+}
+
+hipError_t launch_swiglu_rows(const float *gu, uint32_t gu_stride, uint32_t ntok, uint32_t ffn, float *act, hipStream_t s) {
+    REDHIP_LAUNCH(swiglu_rows_kernel, dim3((ffn + 255u) / 256u, ntok), dim3(256), 0, s, gu, gu_stride, ffn, act);
     return hipGetLastError();
 }
 
