@@ -131,11 +131,18 @@ inline uint32_t prefill_tile_bound(uint32_t ntok, uint32_t top_k, uint32_t n_exp
 // them and ffn <= 512 the kernels that keep a tile's activations in registers run.
 hipError_t launch_tile_packed(const void *packed, uint64_t packed_stride, uint32_t count, uint32_t nrows, uint32_t K, void *tiled, uint64_t tiled_stride,
                               hipStream_t s);
-// routed gate/up + SwiGLU of a chunk on the tile-major copy of packed IQ2_XXS gate/up matrices; act: f32 [pairs][ffn] (mixed layouts)
+// routed gate/up + SwiGLU of a chunk on the tile-major copy of packed IQ2_XXS gate/up matrices (mixed layouts); act: f32 [pairs][ffn], or
+// nullptr for fp16 halves + two exponents per pair in act_h / act_l / act_exp
 hipError_t launch_prefill_gateup_tiled(const void *tiled_experts, uint64_t stride, const uint32_t *uid, const uint32_t *expert_start,
                                        const uint32_t *pair_token, const uint32_t *n_unique, uint32_t *tile_group, uint32_t *tile_pair0, uint32_t *tile_n,
-                                       uint32_t *n_tiles, const void *xh, const void *xl, const int *xexp, float *act, uint32_t hidden, uint32_t ffn,
-                                       uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s);
+                                       uint32_t *n_tiles, const void *xh, const void *xl, const int *xexp, float *act, void *act_h, void *act_l,
+                                       int *act_exp, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s);
+// tile-major IQ3_S matrices (one 32-bit word per eight weights) from raw GGUF rows, and the routed down projection of a chunk on them
+hipError_t launch_tile_iq3s(const void *raw, uint64_t raw_stride, uint32_t count, uint32_t nrows, uint32_t K, void *tiled, uint64_t tiled_stride, hipStream_t s);
+hipError_t launch_prefill_down_iq3s(const void *tiled_down, uint64_t stride, const uint32_t *uid, const uint32_t *n_unique, const uint32_t *tile_group,
+                                    const uint32_t *tile_pair0, const uint32_t *tile_n, const uint32_t *n_tiles, const void *act_h, const void *act_l,
+                                    const int *act_exp, float *tmp, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert,
+                                    hipStream_t s);
 hipError_t launch_prefill_packed(const void *experts, uint64_t stride, const void *shared, const void *tiled_experts, const void *tiled_shared,
                                  const uint32_t *uid, const uint32_t *expert_start,
                                  const uint32_t *pair_token, const uint32_t *n_unique, uint32_t *tile_group, uint32_t *tile_pair0,

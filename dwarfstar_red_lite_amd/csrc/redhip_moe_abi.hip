@@ -39,6 +39,7 @@ struct Layer {
     // mixed layouts that take chunks: f32 copies of the small dense matrices (dequantised once at upload) for the fp32 tile
     // kernel: router [n_expert][hidden] (when it is quantised), shared gate | up [2 ffn][hidden], shared down [hidden][ffn]
     float *dense_router = nullptr, *dense_gu = nullptr, *dense_down = nullptr;
+    uint8_t *tiled_down = nullptr;   // mixed layouts with IQ3_S down matrices that take chunks: their tile-major copy
 };
 
 struct Moe {
@@ -69,6 +70,7 @@ struct Moe {
     bool tiles_resident() const { return packed_gu() && cfg.max_tokens > 8u && cfg.ffn <= 512u && cfg.hidden / 512u <= 4u; }
     // a chunk on a mixed layout: the routed gate/up matrices (packed IQ2_XXS) run on the prefill tiles, the rest on raw rows
     bool mixed_chunk(uint32_t ntok) const { return mixed && ntok > 8u && tiles_resident(); }
+    uint64_t tiled_down_stride() const { return ((uint64_t)cfg.hidden * (cfg.ffn / 32u) * 16u + (uint64_t)cfg.hidden * (cfg.ffn / 256u) * 2u + 255u) & ~255ull; }
     // the one-launch router kernels (logits of every expert + the shared expert's gate logit, optional residual + norm) and the
     // one-wave selection serve every layout whose router they tile; the per-row GEMV + generic selection are what is left
     bool fast_route() const {
@@ -169,10 +171,11 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
             return 1;
         }
         prof_set_stage(ST_BATCH_GATEUP);
+        const bool tiled_down = m->mixed_chunk(ntok) && m->layers[layer].tiled_down;      // then the activations stay fp16 halves for the IQ3_S tile kernel
         if (m->mixed_chunk(ntok))      // xh / xl / xexp come from the router kernel or the prep kernel
             HIP_OK(launch_prefill_gateup_tiled(m->layers[layer].tiled, m->packed_stride, m->uid, m->expert_start, m->pair_token, m->n_unique, m->tile_group,
-                                               m->tile_pair0, m->tile_n, m->n_tiles, m->xh, m->xl, m->xexp, m->act, c.hidden, c.ffn, c.top_k, ntok,
-                                               c.n_expert, s), "tiled gate/up launch");
+                                               m->tile_pair0, m->tile_n, m->n_tiles, m->xh, m->xl, m->xexp, tiled_down ? nullptr : m->act, m->act_h, m->act_l,
+                                               m->act_exp, c.hidden, c.ffn, c.top_k, ntok, c.n_expert, s), "tiled gate/up launch");
         else
             HIP_OK(launch_batch_gateup(ex, m->uid, m->expert_start, m->pair_token, m->n_unique, n_groups, P, c.hidden, c.ffn, x, m->act, s), "batched gate/up launch");
         prof_set_stage(ST_BATCH_GATEUP);
@@ -186,7 +189,12 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
             HIP_OK(launch_batch_gateup(sh, nullptr, nullptr, nullptr, nullptr, 1u, ntok, c.hidden, c.ffn, x, m->sh_act, s), "batched shared gate/up launch");
         }
         prof_set_stage(ST_BATCH_DOWN);
-        HIP_OK(launch_batch_down(ex, m->uid, m->expert_start, m->n_unique, n_groups, P, c.hidden, c.ffn, m->act, m->tmp, s), "batched down launch");
+        if (tiled_down)
+            HIP_OK(launch_prefill_down_iq3s(Ld.tiled_down, m->tiled_down_stride(), m->uid, m->n_unique, m->tile_group, m->tile_pair0, m->tile_n, m->n_tiles,
+                                            m->act_h, m->act_l, m->act_exp, m->tmp, c.hidden, c.ffn, c.top_k, ntok, c.n_expert, s), "tiled IQ3_S down launch");
+        else
+            HIP_OK(launch_batch_down(ex, m->uid, m->expert_start, m->n_unique, n_groups, P, c.hidden, c.ffn, m->act, m->tmp, s), "batched down launch");
+        prof_set_stage(ST_BATCH_DOWN);
         if (dense_shared)
             HIP_OK(launch_f32_tiles(Ld.dense_down, nullptr, m->sh_act, ntok, c.ffn, c.hidden, m->sh_tmp, c.hidden, nullptr, nullptr, nullptr, s), "shared down tiles");
         else
@@ -298,6 +306,10 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
                 m->resident += align256(rb) + align256(gb) + align256(db);
             }
         }
+        if (ok && m->mixed && m->tiles_resident() && dn == T_IQ3_S) {
+            ok = hipMalloc(reinterpret_cast<void **>(&L.tiled_down), (size_t)c.n_expert * m->tiled_down_stride()) == hipSuccess;
+            m->resident += (uint64_t)c.n_expert * m->tiled_down_stride();
+        }
         if (ok && m->tiles_resident()) {
             ok = hipMalloc(reinterpret_cast<void **>(&L.tiled), (size_t)c.n_expert * m->packed_stride) == hipSuccess &&
                  (!m->fused || hipMalloc(reinterpret_cast<void **>(&L.shared_tiled), align256(2u * m->sh_gate_bytes + m->sh_down_bytes)) == hipSuccess);
@@ -368,6 +380,7 @@ void redhip_moe_destroy(redhip_moe_t h) {
         if (L.shared_packed) (void)hipFree(L.shared_packed);
         if (L.dense_gu) (void)hipFree(L.dense_router ? L.dense_router : L.dense_gu);
         if (L.tiled) (void)hipFree(L.tiled);
+        if (L.tiled_down) (void)hipFree(L.tiled_down);
         if (L.shared_tiled) (void)hipFree(L.shared_tiled);
     }
     if (m->ws) (void)hipFree(m->ws);
@@ -449,6 +462,9 @@ int redhip_moe_load_experts(redhip_moe_t h, uint32_t layer, uint32_t first, uint
             if (m->fused)
                 HIP_OK(launch_tile_packed(pk + 2u * m->gate_bytes, m->packed_stride, count, c.hidden, c.ffn, tl + 2u * m->gate_bytes, m->packed_stride, nullptr), "expert down tiling");
         }
+        if (m->layers[layer].tiled_down)
+            HIP_OK(launch_tile_iq3s(dst + 2u * m->gate_bytes, m->expert_stride, count, c.hidden, c.ffn,
+                                    m->layers[layer].tiled_down + (uint64_t)first * m->tiled_down_stride(), m->tiled_down_stride(), nullptr), "expert down tiling");
         HIP_OK(hipStreamSynchronize(nullptr), "expert repack");
     }
     return 1;

@@ -612,6 +612,163 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_down_reg_kernel(TiledA
     }
 }
 
+// ---------------------------------------------------------------- IQ3_S down projection on tiles (mixed layouts)
+
+// Tile-major IQ3_S (built once at upload from the raw 110-byte blocks): per group of 32 weights four 32-bit words, one per eight
+// weights l: bits 0-8 the first grid index, 9-17 the second (each with its ninth bit from qh), 18-25 the eight sign bits, 26-29 the
+// group's scale nibble. A row's chunk of four groups is stored as [l][group] so that lane (r, l) reads its own four words as one
+// 16-byte load, and the chunks of 16 consecutive rows lie next to each other (a wave-wide load is 1024 contiguous bytes):
+//   chunk (row, c)  at ((row / 16 * (K / 128) + c) * 16 + row % 16) * 64,   lane l adds 16 l
+//   scale (row, b)  at qs_bytes + ((row / 16 * (K / 256) + b) * 16 + row % 16) * 2
+__global__ void tile_iq3s_kernel(const uint8_t *raw, uint64_t raw_stride, uint32_t nrows, uint32_t K, uint8_t *tiled, uint64_t tiled_stride) {
+    const uint32_t NG = K / 32u, NC = K / 128u, NB = K / 256u;
+    const uint64_t gid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= (uint64_t)nrows * NG) return;
+    const uint32_t row = (uint32_t)(gid / NG), g = (uint32_t)(gid % NG), sub = g & 7u;
+    const uint8_t *bp = raw + (uint64_t)blockIdx.y * raw_stride + ((uint64_t)row * NB + (g >> 3)) * 110u;
+    uint8_t *dst = tiled + (uint64_t)blockIdx.y * tiled_stride;
+    const uint32_t nib = ((uint32_t)bp[106u + (sub >> 1)] >> (4u * (sub & 1u))) & 15u, qh = bp[66u + sub];
+    uint32_t *out = reinterpret_cast<uint32_t *>(dst + (((uint64_t)(row / 16u) * NC + (g >> 2)) * 16u + row % 16u) * 64u);
+    for (uint32_t l = 0; l < 4u; ++l) {
+        const uint32_t ia = (uint32_t)bp[2u + 8u * sub + 2u * l] | ((qh << (8u - 2u * l)) & 256u);
+        const uint32_t ib = (uint32_t)bp[3u + 8u * sub + 2u * l] | ((qh << (7u - 2u * l)) & 256u);
+        out[4u * l + (g & 3u)] = ia | (ib << 9) | ((uint32_t)bp[74u + 4u * sub + l] << 18) | (nib << 26);
+    }
+    if (sub == 0u)
+        reinterpret_cast<uint16_t *>(dst + (uint64_t)nrows * NG * 16u)[((uint64_t)(row / 16u) * NB + (g >> 3)) * 16u + row % 16u] = (uint16_t)ld_u16(bp);
+}
+
+hipError_t launch_tile_iq3s(const void *raw, uint64_t raw_stride, uint32_t count, uint32_t nrows, uint32_t K, void *tiled, uint64_t tiled_stride, hipStream_t s) {
+    if (!nrows || nrows % 16u || !K || K % 256u || !count || count > 65535u) return hipErrorInvalidValue;
+    const uint64_t total = (uint64_t)nrows * (K / 32u);
+    REDHIP_LAUNCH(tile_iq3s_kernel, dim3((uint32_t)((total + 255u) / 256u), count), dim3(256), 0, s, static_cast<const uint8_t *>(raw), raw_stride, nrows, K,
+                  static_cast<uint8_t *>(tiled), tiled_stride);
+    return hipGetLastError();
+}
+
+constexpr uint32_t kIq3SignBytes = 256u * 16u;              // [eight sign bits]: eight fp16 sign masks
+constexpr uint32_t kIq3MagBytes = 16u * 512u * 8u;          // [scale nibble][grid entry]: four fp16 magnitudes times 1 + 2 nibble (at most 15 * 31: exact)
+
+__device__ __forceinline__ void build_iq3s_tables(uint8_t *sgn, uint8_t *mag, uint32_t tid, uint32_t nthreads) {
+    for (uint32_t e = tid; e < 16u * 512u; e += nthreads) {
+        const uint32_t gw = redhip_iq3s_grid[e & 511u];
+        const float f = (float)(1u + 2u * (e >> 9));
+        uint32_t w2[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const _Float16 lo = (_Float16)(f * (float)((gw >> (16 * i)) & 255u)), hi = (_Float16)(f * (float)((gw >> (16 * i + 8)) & 255u));
+            w2[i] = (uint32_t)__builtin_bit_cast(uint16_t, lo) | ((uint32_t)__builtin_bit_cast(uint16_t, hi) << 16);
+        }
+        *reinterpret_cast<uint2 *>(mag + (size_t)e * 8u) = make_uint2(w2[0], w2[1]);
+    }
+    for (uint32_t s8 = tid; s8 < 256u; s8 += nthreads) {
+        uint32_t w4[4];
+#pragma unroll
+        for (uint32_t i = 0; i < 4u; ++i) w4[i] = (((s8 >> (2u * i)) & 1u) << 15) | (((s8 >> (2u * i + 1u)) & 1u) << 31);
+        *reinterpret_cast<uint4 *>(sgn + (size_t)s8 * 16u) = make_uint4(w4[0], w4[1], w4[2], w4[3]);
+    }
+}
+
+// the eight signed, scaled fp16 weights of one word of the tile-major layout
+__device__ __forceinline__ half8_t decode_iq3s(uint32_t w, const uint8_t *sgn, const uint8_t *mag) {
+    const uint32_t t = (w >> 14) & 0xf000u;                   // scale nibble * 512 entries * 8 bytes
+    const uint2 ma = *reinterpret_cast<const uint2 *>(mag + (((w << 3) & 0xff8u) | t));
+    const uint2 mb = *reinterpret_cast<const uint2 *>(mag + (((w >> 6) & 0xff8u) | t));
+    const uint4 g = *reinterpret_cast<const uint4 *>(sgn + ((w >> 14) & 0xff0u));
+    Half8 r;
+    r.u = make_uint4(ma.x ^ g.x, ma.y ^ g.y, mb.x ^ g.z, mb.y ^ g.w);
+    return r.v;
+}
+
+struct Iq3DownArgs {
+    PrefillArgs p;                 // act_h / act_l / act_exp (two exponents per pair) from the gate/up kernel, tmp out; routed tiles only
+    const uint8_t *experts;        // tile-major IQ3_S down matrices
+    uint64_t stride;
+};
+
+// Same structure as prefill_down_reg_kernel: wave w computes rows 128 b + 16 w + r of the pass, a tile's activations stay in registers.
+template <int NFG>          // ffn = 32 * NFG, NFG <= 16
+__global__ __launch_bounds__(kRegWaves * 64) void prefill_down_iq3s_kernel(Iq3DownArgs da) {
+    const PrefillArgs &a = da.p;
+    constexpr uint32_t F = 32u * NFG, FB = F / 256u, NCK = NFG / 4u;
+    extern __shared__ __attribute__((aligned(16))) uint8_t dyn[];          // sign table | scaled magnitude table
+    __shared__ __attribute__((aligned(16))) float pair_scale[2][kTile];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, r = lane & 15u, q = lane >> 4;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t H = a.hidden;
+    const uint8_t *sgn = dyn, *mag = dyn + kIq3SignBytes;
+    build_iq3s_tables(dyn, dyn + kIq3SignBytes, tid, kRegWaves * 64u);
+    const uint32_t T = a.n_tiles[0];
+    const uint64_t qs_bytes = (uint64_t)H * NFG * 16u;
+    constexpr uint32_t kRowsPerPass = 16u * kRegWaves;
+    const uint32_t n_pass_tile = H / kRowsPerPass, parts = n_pass_tile % 2u == 0u ? 2u : 1u, n_pass = n_pass_tile / parts;
+    const uint32_t items = T * parts;
+    const uint32_t item_begin = (uint32_t)(((uint64_t)blockIdx.x * items) / gridDim.x), item_end = (uint32_t)(((uint64_t)(blockIdx.x + 1u) * items) / gridDim.x);
+    Half8 xa[NFG], xb[NFG];
+    uint32_t have_tile = 0xffffffffu;
+    for (uint32_t item = item_begin; item < item_end; ++item) {
+        const uint32_t tile = item / parts, pass0 = (item % parts) * n_pass;
+        const uint32_t u = a.tile_group[tile], p0 = a.tile_pair0[tile], n = a.tile_n[tile];
+        const uint8_t *dn = da.experts + (uint64_t)a.uid[u] * da.stride;
+        if (tile != have_tile) {
+            have_tile = tile;
+            __syncthreads();
+            if (tid < 2u * kTile) pair_scale[tid & 1u][tid >> 1] = (tid >> 1) < n ? exp2i(a.act_exp[2u * p0 + tid]) : 0.0f;      // IQ3_S: weight = d (1 + 2 nibble) grid, no 1/8
+            __syncthreads();
+            const uint64_t base = (uint64_t)(p0 + r) * F + 8u * q;
+            const bool live = r < n;
+#pragma unroll
+            for (uint32_t g = 0; g < (uint32_t)NFG; ++g) {
+                xa[g].u = make_uint4(0u, 0u, 0u, 0u);
+                xb[g].u = xa[g].u;
+                if (live) {
+                    xa[g].u = *reinterpret_cast<const uint4 *>(a.act_h + base + 32u * g);
+                    xb[g].u = *reinterpret_cast<const uint4 *>(a.act_l + base + 32u * g);
+                }
+            }
+        }
+        const float4_t ps0 = *reinterpret_cast<const float4_t *>(&pair_scale[0][4u * q]), ps1 = *reinterpret_cast<const float4_t *>(&pair_scale[1][4u * q]);
+        struct Chunk { uint4 w; uint32_t d; };
+        auto load_chunk = [&](uint32_t b, uint32_t c) {
+            const uint32_t rtile = kRegWaves * (pass0 + b) + wave;
+            const uint4 *qp = reinterpret_cast<const uint4 *>(dn + (((uint64_t)rtile * NCK + c) * 16u + r) * 64u + 16u * q);
+            const uint16_t *dp = reinterpret_cast<const uint16_t *>(dn + qs_bytes) + ((uint64_t)rtile * FB + c / 2u) * 16u + r;
+            return Chunk{qp[0], *dp};
+        };
+        Chunk cw[NCK];
+#pragma unroll
+        for (uint32_t c = 0; c < NCK; ++c) cw[c] = load_chunk(0u, c);
+#pragma unroll 1
+        for (uint32_t b = 0; b < n_pass; ++b) {
+            float4_t tot = {0.0f, 0.0f, 0.0f, 0.0f};
+            const uint32_t nb = b + 1u < n_pass ? b + 1u : b;          // the last pass reloads itself: no branch around the loads
+#pragma unroll
+            for (uint32_t c = 0; c < NCK; ++c) {
+                const uint32_t w4[4] = {cw[c].w.x, cw[c].w.y, cw[c].w.z, cw[c].w.w};
+                const float d = scale_to_f32(cw[c].d);
+                cw[c] = load_chunk(nb, c);
+                __builtin_amdgcn_sched_barrier(0);         // keeps the loads here: the scheduler otherwise sinks them to the end of the pass
+                float4_t hi = {0.0f, 0.0f, 0.0f, 0.0f}, lo = hi;
+#pragma unroll
+                for (uint32_t k = 0; k < 4u; ++k) {
+                    const uint32_t g = 4u * c + k;
+                    const half8_t bw = decode_iq3s(w4[k], sgn, mag);
+                    hi = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[g].v, bw, hi, 0, 0, 0);
+                    lo = __builtin_amdgcn_mfma_f32_16x16x32_f16(xb[g].v, bw, lo, 0, 0, 0);
+                }
+#pragma unroll
+                for (int t = 0; t < 4; ++t) tot[t] = fmaf(fmaf(lo[t], 4.8828125e-4f, hi[t]) * d, 2u * c < NCK ? ps0[t] : ps1[t], tot[t]);
+            }
+            const uint32_t row = kRowsPerPass * (pass0 + b) + 16u * wave + r;
+#pragma unroll
+            for (uint32_t t = 0; t < 4u; ++t) {
+                const uint32_t i = 4u * q + t;
+                if (i < n) a.tmp[(uint64_t)(p0 + i) * H + row] = tot[t];
+            }
+        }
+    }
+}
+
 // ---------------------------------------------------------------- router logits of a token chunk
 
 // logits[tok][e] = W[e] . x[tok] for an f32 router as a tiled product on v_mfma_f32_16x16x4_f32 (full fp32
@@ -734,23 +891,52 @@ static hipError_t launch_gateup_reg(const TiledArgs &ta, dim3 grid, hipStream_t 
     return hipGetLastError();
 }
 
-// routed gate/up + SwiGLU of a chunk on the tile-major copy of packed IQ2_XXS gate/up matrices, activations out as f32 [pairs][ffn]:
-// the front half of a layer whose other matrices are of other types. Needs the pair grouping; the shared expert is not touched.
+// routed gate/up + SwiGLU of a chunk on the tile-major copy of packed IQ2_XXS gate/up matrices: the front half of a layer whose other
+// matrices are of other types. Activations out as f32 [pairs][ffn] (`act`, for kernels on raw rows) or, with act == nullptr, as fp16 halves
+// with two exponents per pair (for launch_prefill_down_iq3s). Needs the pair grouping; builds the tile list; the shared expert is not touched.
 hipError_t launch_prefill_gateup_tiled(const void *tiled_experts, uint64_t stride, const uint32_t *uid, const uint32_t *expert_start,
                                        const uint32_t *pair_token, const uint32_t *n_unique, uint32_t *tile_group, uint32_t *tile_pair0, uint32_t *tile_n,
-                                       uint32_t *n_tiles, const void *xh, const void *xl, const int *xexp, float *act, uint32_t hidden, uint32_t ffn,
-                                       uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s) {
-    if (!fused_iq2_supported(hidden, ffn) || hidden / 512u > 4u || ffn > 512u || !ntok || !tiled_experts || !act) return hipErrorInvalidValue;
+                                       uint32_t *n_tiles, const void *xh, const void *xl, const int *xexp, float *act, void *act_h, void *act_l,
+                                       int *act_exp, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s) {
+    if (!fused_iq2_supported(hidden, ffn) || hidden / 512u > 4u || ffn > 512u || !ntok || !tiled_experts || (!act && (!act_h || !act_l || !act_exp)))
+        return hipErrorInvalidValue;
     const uint32_t P = ntok * top_k;
     prof_set_stage(ST_GROUP);
     REDHIP_LAUNCH(build_tiles_kernel, dim3(1), dim3(1024), 0, s, expert_start, n_unique, P, 0u, tile_group, tile_pair0, tile_n, n_tiles);      // no shared tiles
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     PrefillArgs a{nullptr, stride, nullptr, uid, pair_token, n_unique, tile_group, tile_pair0, tile_n, n_tiles, static_cast<const _Float16 *>(xh),
-                  static_cast<const _Float16 *>(xl), xexp, nullptr, nullptr, nullptr, nullptr, nullptr, hidden, ffn, top_k, ntok};
+                  static_cast<const _Float16 *>(xl), xexp, static_cast<_Float16 *>(act_h), static_cast<_Float16 *>(act_l), act_exp, nullptr, nullptr, hidden,
+                  ffn, top_k, ntok};
     const TiledArgs ta{a, static_cast<const uint8_t *>(tiled_experts), nullptr, act};
     const uint32_t tile_bound = prefill_tile_bound(ntok, top_k, n_expert);
     return launch_gateup_reg(ta, dim3(tile_bound < 256u ? tile_bound : 256u), s);
+}
+
+// routed down projection of a chunk on tile-major IQ3_S matrices, behind launch_prefill_gateup_tiled (its tile list and fp16 activations)
+hipError_t launch_prefill_down_iq3s(const void *tiled_down, uint64_t stride, const uint32_t *uid, const uint32_t *n_unique, const uint32_t *tile_group,
+                                    const uint32_t *tile_pair0, const uint32_t *tile_n, const uint32_t *n_tiles, const void *act_h, const void *act_l,
+                                    const int *act_exp, float *tmp, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert,
+                                    hipStream_t s) {
+    if (!tiled_down || !hidden || hidden % 128u || (ffn != 256u && ffn != 512u) || !ntok) return hipErrorInvalidValue;
+    PrefillArgs a{nullptr, stride, nullptr, uid, nullptr, n_unique, tile_group, tile_pair0, tile_n, n_tiles, nullptr, nullptr, nullptr,
+                  static_cast<_Float16 *>(const_cast<void *>(act_h)), static_cast<_Float16 *>(const_cast<void *>(act_l)), const_cast<int *>(act_exp), tmp,
+                  nullptr, hidden, ffn, top_k, ntok};
+    const Iq3DownArgs da{a, static_cast<const uint8_t *>(tiled_down), stride};
+    const uint32_t tile_bound = prefill_tile_bound(ntok, top_k, n_expert);
+    const dim3 grid(tile_bound < 256u ? tile_bound : 256u);
+    const size_t lds = kIq3SignBytes + kIq3MagBytes;
+    static bool attr = false;
+    if (!attr) {
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(prefill_down_iq3s_kernel<8>), hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
+        if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void *>(prefill_down_iq3s_kernel<16>), hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
+        if (e != hipSuccess) return e;
+        attr = true;
+    }
+    prof_set_stage(ST_PREFILL_DOWN);
+    if (ffn == 256u) REDHIP_LAUNCH(prefill_down_iq3s_kernel<8>, grid, dim3(kRegWaves * 64), lds, s, da);
+    else REDHIP_LAUNCH(prefill_down_iq3s_kernel<16>, grid, dim3(kRegWaves * 64), lds, s, da);
+    return hipGetLastError();
 }
 
 hipError_t launch_prefill_packed(const void *experts, uint64_t stride, const void *shared, const void *tiled_experts, const void *tiled_shared,
