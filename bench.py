@@ -36,6 +36,10 @@ def parse():
                     help="iq2: BASELINE config 1 (all IQ2_XXS, F32 router); f2: config 2 layout; xs / m: routed experts IQ2_XS / IQ1_M "
                          "(the formats of the reference's target file), Q6_K shared expert")
     ap.add_argument("--layers", type=int, default=48, help="resident layers the steps cycle through")
+    ap.add_argument("--routing", choices=["router", "hot", "zipf"], default="router",
+                    help="router: the layer's own router on the activations (router GEMV + selection inside the timed step); hot: drawn logits N(0,1) + 2.0 on "
+                         "32 hot experts (BASELINE config 3); zipf: top-k drawn from a Zipf(1.1) expert popularity (config 4). hot / zipf: the routing is "
+                         "an input, the timed step is grouping + experts + combine")
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")
     ap.add_argument("--no-micro", action="store_true", help="skip the single-GEMV microbench (only run for --layout iq2 --batch 1)")
@@ -90,6 +94,24 @@ def layer_bytes(cfg, distinct_experts, batch):
             "act_bytes": 2 * 4 * H * batch, "one_expert": expert, "shared": shared}
 
 
+def oracle_given_routing(orc, cfg, lay, x, ids, w, threads):
+    """CPU oracle of the experts behind a given routing: routed experts in selection order (double) + the gated shared expert"""
+    import numpy as np
+    H, F = cfg["hidden"], cfg["ffn"]
+    L = orc.lib()
+    p = lambda a: a.ctypes.data_as(orc.C.c_void_p)
+    out = np.empty((x.shape[0], H), np.float32)
+    for t in range(x.shape[0]):
+        routed = np.empty(H, np.float64)
+        idt, wt = np.ascontiguousarray(ids[t], np.uint32), np.ascontiguousarray(w[t], np.float32)
+        assert L.orc_routed_topk(cfg["gate_up_type"], cfg["down_type"], p(lay["gate"]), p(lay["up"]), p(lay["down"]), lay["gate"][0].nbytes,
+                                 lay["up"][0].nbytes, lay["down"][0].nbytes, p(idt), p(wt), idt.size, H, F, p(np.ascontiguousarray(x[t])), p(routed))
+        sh, sc = orc.shared_expert(cfg["sh_gate_up_type"], cfg["sh_down_type"], lay["sh_gate"], lay["sh_up"], lay["sh_down"], lay["sh_gate_inp"],
+                                   H, F, x[t], threads=threads)
+        out[t] = (routed + sh.astype(np.float64) * sc).astype(np.float32)
+    return out
+
+
 def main():
     args = parse()
     if args.gpus != 1:
@@ -132,19 +154,49 @@ def main():
     outs = torch.empty_like(xs)
     stream = torch.cuda.Stream()
 
+    # drawn routing (configs 3 and 4): ids / weights per activation set, made on the host
+    route_ids = route_w = None
+    if args.routing != "router":
+        import oracle_lib as orc
+        rr = np.random.default_rng(7)
+        K_, E_ = cfg["top_k"], cfg["n_expert"]
+        ids_h = np.empty((NX, B, K_), np.uint32)
+        w_h = np.empty((NX, B, K_), np.float32)
+        for i in range(NX):
+            if args.routing == "hot":
+                lg = synth.hot_logits(rr, B, E_)
+                for t in range(B):
+                    ids_h[i, t], w_h[i, t] = orc.router_select(lg[t], K_)
+            else:
+                ids_h[i] = synth.zipf_topk(rr, B, E_, K_)
+                ww = rr.random((B, K_)).astype(np.float32) + 0.1
+                w_h[i] = ww / ww.sum(axis=1, keepdims=True)
+        route_ids = torch.from_numpy(ids_h.astype(np.int32)).cuda()
+        route_w = torch.from_numpy(w_h).cuda()
+
     def step(i):
-        moe.forward(i % NL, xs[i % NX], outs[i % NX])
+        if route_ids is None:
+            moe.forward(i % NL, xs[i % NX], outs[i % NX])
+        else:
+            moe.experts(i % NL, xs[i % NX], route_ids[i % NX], route_w[i % NX], outs[i % NX])
 
     # ---- parity gate on the very tensors the timed steps use (layer 0, CPU oracle) ----
     import oracle_lib as orc
     ref = orc.Layer(cfg, **layer0)
     with torch.cuda.stream(stream):
         step(0)
-        gids, _, _ = moe.last_route(B)
-    want, cids, _, _ = ref.forward(xs_host[0], threads=os.cpu_count() or 1)
-    got = outs[0].cpu().numpy()
+        if route_ids is None:
+            gids, _, _ = moe.last_route(B)
+    if route_ids is None:
+        want, cids, _, _ = ref.forward(xs_host[0], threads=os.cpu_count() or 1)
+        got = outs[0].cpu().numpy()
+        ids_ok = bool(np.array_equal(gids, cids))
+    else:           # drawn routing: the oracle's routed experts + gated shared expert for the first tokens of the step
+        n_chk = min(B, 8)
+        want = oracle_given_routing(orc, cfg, layer0, xs_host[0][:n_chk], ids_h[0][:n_chk], w_h[0][:n_chk], os.cpu_count() or 1)
+        got = outs[0][:n_chk].cpu().numpy()
+        ids_ok = True
     rel = float(np.linalg.norm(got - want) / np.linalg.norm(want))
-    ids_ok = bool(np.array_equal(gids, cids))
     if not rel <= 1e-3 or not ids_ok:
         print("PARITY FAILURE: rel L2 %.3g vs the CPU oracle, router ids identical: %s" % (rel, ids_ok), file=sys.stderr)
         sys.exit(1)
@@ -198,8 +250,11 @@ def main():
         # distinct routed experts per step (B > 1 shares experts between tokens)
         distinct = []
         for i in range(min(K, NX)):
-            step(W + i)
-            ids, _, _ = moe.last_route(B)
+            if route_ids is None:
+                step(W + i)
+                ids, _, _ = moe.last_route(B)
+            else:
+                ids = ids_h[(W + i) % NX]
             distinct.append(len(set(ids.ravel().tolist())))
     if args.calibrate:         # yardstick for FETCH_SIZE / WRITE_SIZE: copies of exactly CAL_BYTES in, CAL_BYTES out
         cal_src = torch.empty(CAL_BYTES, dtype=torch.uint8, device="cuda").random_(0, 256)
@@ -270,7 +325,7 @@ def main():
         "config": {"workload": "%s: one MoE FFN layer, B=%d decode token(s), hidden 2048, 512 experts top-10 + shared, ffn 512, layout %s, "
                                "all experts of %d layers resident" % ({"iq2": "config1", "f2": "config2"}.get(args.layout, "target-file expert format"),
                                                                       B, args.layout, NL),
-                   "layout": args.layout, "batch": B, "resident_layers": NL, "resident_gb": round(moe.resident_bytes / 1e9, 2),
+                   "layout": args.layout, "batch": B, "routing": args.routing, "resident_layers": NL, "resident_gb": round(moe.resident_bytes / 1e9, 2),
                    "mean_distinct_routed_experts": mean_distinct},
         "layer_gbps": {"expert_bytes": int(lb["expert_bytes"]), "layer_bytes": int(total_bytes),
                        "expert_gbps": round(lb["expert_bytes"] / (ms_per_step * 1e-3) / 1e9, 1),
