@@ -15,7 +15,7 @@ torch = pytest.importorskip("torch")
 
 
 def dev(a):
-    return torch.from_numpy(np.ascontiguousarray(a)).cuda()
+    return torch.from_numpy(np.array(a, copy=True)).cuda()
 
 
 @pytest.mark.parametrize("t", [T_IQ2, T_IQ3, T_Q6K])

@@ -63,21 +63,22 @@ def test_ragged_small_batches_hot_experts(layout):
     m.close()
 
 
-def test_prefill_sized_chunk_zipf():
-    """BASELINE config 4 shape of routing: Zipf(1.1) expert popularity, variable token count per expert (small dims)."""
+@pytest.mark.parametrize("hidden,ffn,ntok", [(512, 256, 96), (1024, 512, 40), (2048, 512, 33), (1024, 768, 24)])
+def test_prefill_sized_chunk_zipf(hidden, ffn, ntok):
+    """BASELINE config 4 on the mixed layout: Zipf(1.1) expert popularity, variable token count per expert. Routed gate/up tiles on
+    packed IQ2_XXS, routed IQ3_S down tiles, the Q6_K shared expert as dense f32 products; ffn 768 takes the raw-row kernels."""
     from dwarfstar_red_lite_amd.moe import ResidentMoe
-    cfg = synth.layer_config(hidden=512, ffn=256, n_expert=64, top_k=4, layout="f2")
+    cfg = synth.layer_config(hidden=hidden, ffn=ffn, n_expert=64, top_k=4, layout="f2")
     lay = synth.make_layer(5, cfg)
-    ntok = 96
     m = ResidentMoe(cfg, n_layer=1, max_tokens=ntok)
     m.load_layer(0, lay)
     rng = np.random.default_rng(8)
-    x = synth.normed_x(rng, ntok, 512)
+    x = synth.normed_x(rng, ntok, hidden)
     ids = synth.zipf_topk(rng, ntok, 64, 4)
     w = rng.random((ntok, 4)).astype(np.float32)
     w /= w.sum(axis=1, keepdims=True)
     counts = np.bincount(ids.ravel(), minlength=64)
-    assert counts.max() > 16 and (counts == 0).any() or counts.min() < 4          # ragged: some experts busy, some nearly idle
+    assert counts.max() > 8 and counts.min() < 4          # ragged: some experts busy, some nearly idle
     got = m.experts(0, torch.from_numpy(x).cuda(), torch.from_numpy(ids.astype(np.int32)).cuda(), torch.from_numpy(w).cuda()).cpu().numpy()
     want = oracle_tokens(cfg, lay, x, ids, w)
     assert max(rel_l2(got[t], want[t]) for t in range(ntok)) <= REL_L2_TOL
@@ -106,10 +107,12 @@ def test_prefill_chunk_packed_tiles(hidden, ffn, ntok):
     m.close()
 
 
-def test_prefill_chunk_forward_config_shape():
-    """A 24-token chunk at the benchmark shape through forward(): router, selection, grouping, tiles, combine."""
+@pytest.mark.parametrize("layout", ["iq2", "f2"])
+def test_prefill_chunk_forward_config_shape(layout):
+    """A 24-token chunk at the benchmark shape through forward(): router (tiled, a Q6_K router through its f32 copy), selection, grouping,
+    tiles, combine."""
     from dwarfstar_red_lite_amd.moe import ResidentMoe
-    cfg = synth.layer_config(layout="iq2")
+    cfg = synth.layer_config(layout=layout)
     lay = synth.make_layer(78, cfg)
     ntok = 24
     m = ResidentMoe(cfg, n_layer=1, max_tokens=ntok)
@@ -117,8 +120,9 @@ def test_prefill_chunk_forward_config_shape():
     x = synth.normed_x(np.random.default_rng(32), ntok, cfg["hidden"])
     got = m.forward(0, torch.from_numpy(x).cuda()).cpu().numpy()
     gids, gw, _ = m.last_route(ntok)
-    want, cids, cw, _ = orc.Layer(cfg, **lay).forward(x, threads=8)
-    assert np.array_equal(gids, cids)
+    want, cids, cw, clog = orc.Layer(cfg, **lay).forward(x, threads=8)
+    from test_gpu_moe_layer import ids_match_up_to_ties
+    assert all(ids_match_up_to_ties(gids[t], cids[t], clog[t]) for t in range(ntok))
     assert np.abs(gw - cw).max() <= 1e-5
     assert max(rel_l2(got[t], want[t]) for t in range(ntok)) <= REL_L2_TOL
     m.close()
