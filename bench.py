@@ -33,12 +33,12 @@ def parse():
     ap.add_argument("--steps", type=int, default=480)
     ap.add_argument("--warmup", type=int, default=96)
     ap.add_argument("--layout", choices=["iq2", "f2", "xs", "m"], default="iq2",
-                    help="iq2: BASELINE config 1 (all IQ2_XXS, F32 router); f2: config 2 layout; xs / m: routed experts IQ2_XS / IQ1_M "
+                    help="iq2: the benchmark definition's config 1 (all IQ2_XXS, F32 router); f2: its config 2 layout; xs / m: routed experts IQ2_XS / IQ1_M "
                          "(the formats of the reference's target file), Q6_K shared expert")
     ap.add_argument("--layers", type=int, default=48, help="resident layers the steps cycle through")
     ap.add_argument("--routing", choices=["router", "hot", "zipf"], default="router",
                     help="router: the layer's own router on the activations (router GEMV + selection inside the timed step); hot: drawn logits N(0,1) + 2.0 on "
-                         "32 hot experts (BASELINE config 3); zipf: top-k drawn from a Zipf(1.1) expert popularity (config 4). hot / zipf: the routing is "
+                         "32 hot experts (the ragged small-batch config); zipf: top-k drawn from a Zipf(1.1) expert popularity (the prefill-chunk config). hot / zipf: the routing is "
                          "an input, the timed step is grouping + experts + combine")
     ap.add_argument("--batch", type=int, default=1)
     ap.add_argument("--no-cpu", action="store_true", help="skip the CPU baseline leg")

@@ -3,7 +3,7 @@ import numpy as np
 
 T_F32, T_Q6K, T_IQ2, T_IQ3 = 0, 14, 16, 21
 
-# BASELINE tolerance: GEMV / FFN outputs within 1e-3 relative L2 of the double-accumulating CPU path
+# parity tolerance: GEMV / FFN outputs within 1e-3 relative L2 of the double-accumulating CPU path
 REL_L2_TOL = 1e-3
 
 

@@ -32,7 +32,7 @@ def oracle_tokens(cfg, lay, x, ids, w):
 
 @pytest.mark.parametrize("layout", ["iq2", "f2"])
 def test_ragged_small_batches_hot_experts(layout):
-    """BASELINE config 3: 2..8 tokens, logits N(0,1) + 2.0 on 32 hot experts, shapes of config 0."""
+    """Ragged small batches: 2..8 tokens, logits N(0,1) + 2.0 on 32 hot experts, benchmark layer shape."""
     from dwarfstar_red_lite_amd.moe import ResidentMoe
     cfg = synth.layer_config(layout=layout)
     lay = synth.make_layer(77, cfg)
@@ -65,7 +65,7 @@ def test_ragged_small_batches_hot_experts(layout):
 
 @pytest.mark.parametrize("hidden,ffn,ntok", [(512, 256, 96), (1024, 512, 40), (2048, 512, 33), (1024, 768, 24)])
 def test_prefill_sized_chunk_zipf(hidden, ffn, ntok):
-    """BASELINE config 4 on the mixed layout: Zipf(1.1) expert popularity, variable token count per expert. Routed gate/up tiles on
+    """Prefill chunk on the mixed layout: Zipf(1.1) expert popularity, variable token count per expert. Routed gate/up tiles on
     packed IQ2_XXS, routed IQ3_S down tiles, the Q6_K shared expert as dense f32 products; ffn 768 takes the raw-row kernels."""
     from dwarfstar_red_lite_amd.moe import ResidentMoe
     cfg = synth.layer_config(hidden=hidden, ffn=ffn, n_expert=64, top_k=4, layout="f2")

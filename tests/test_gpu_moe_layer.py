@@ -55,7 +55,7 @@ def test_layer_single_token(layout, shape):
 
 
 def test_layer_full_size_config0():
-    """BASELINE config 0 at its real shape: hidden 2048, 512 experts, top-10 + shared, ffn 512, all IQ2_XXS, F32 router."""
+    """The benchmark layer at its real shape: hidden 2048, 512 experts, top-10 + shared, ffn 512, all IQ2_XXS, F32 router."""
     from dwarfstar_red_lite_amd.moe import ResidentMoe
     cfg = synth.layer_config()
     m = ResidentMoe(cfg, n_layer=1, max_tokens=1)
