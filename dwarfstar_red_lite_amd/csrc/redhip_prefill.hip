@@ -378,7 +378,7 @@ __device__ __forceinline__ void build_scaled_tables(uint8_t *mag, uint8_t *sgn, 
 
 // the eight signed fp16 weights of grid entry q of a group word, times the group's 2 s + 1
 __device__ __forceinline__ half8_t decode_scaled(uint2 w, uint32_t q, const uint8_t *mag, const uint8_t *sgn) {
-    const uint32_t idx = (w.x >> (8u * q)) & 255u, s7 = (w.y >> (7u * q)) & 127u;
+    const uint32_t idx = __builtin_amdgcn_ubfe(w.x, 8u * q, 8u), s7 = __builtin_amdgcn_ubfe(w.y, 7u * q, 7u);
     const uint4 m = *reinterpret_cast<const uint4 *>(mag + ((((w.y >> 28) << 8) | idx) << 4));
     const uint4 g = *reinterpret_cast<const uint4 *>(sgn + (s7 << 4));
     Half8 r;
@@ -401,16 +401,17 @@ template <int NKC>          // hidden = 512 * NKC
 __global__ __launch_bounds__(kRegWaves * 64) void prefill_gateup_reg_kernel(TiledArgs ta) {
     const PrefillArgs &a = ta.p;
     constexpr uint32_t H = 512u * NKC, HG = H / 32u, HB = H / 256u, GQ = HG / 4u, NC = H / 128u;   // GQ: groups per K quarter = 4 NKC
-    extern __shared__ __attribute__((aligned(16))) uint8_t dyn[];          // sign table | scaled magnitude table | acts: [16][F + 4] f32
+    extern __shared__ __attribute__((aligned(16))) uint8_t dyn[];          // acts: [16][F + 4] f32
+    __shared__ __attribute__((aligned(16))) uint8_t tables[kSignBytes + kScaledMagBytes];      // static: table reads take immediate offsets
     __shared__ float part[2][4][kTile][68];                // [unit parity][K quarter][pair][gate 0..31 | up 0..31], padded
     __shared__ float tok_scale[kTile];
     __shared__ uint32_t tok_of[kTile];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, r = lane & 15u, q = lane >> 4;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6), kc = wave & 3u, rh = wave >> 2;
     const uint32_t F = a.ffn, FG = F / 32u, P = a.ntok * a.top_k, AROW = F + 4u;
-    const uint8_t *sgn = dyn, *mag = dyn + kSignBytes;
-    float *acts = reinterpret_cast<float *>(dyn + kScaledMagBytes + kSignBytes);
-    build_scaled_tables(dyn + kSignBytes, dyn, tid, kRegWaves * 64u);
+    const uint8_t *sgn = tables, *mag = tables + kSignBytes;
+    float *acts = reinterpret_cast<float *>(dyn);
+    build_scaled_tables(tables + kSignBytes, tables, tid, kRegWaves * 64u);
     const uint32_t T = a.n_tiles[0], U = a.n_unique[0];
     const uint64_t qs_bytes = (uint64_t)F * HG * 8u, gate_bytes = qs_bytes + (uint64_t)F * HB * 2u;
 
@@ -530,13 +531,13 @@ template <int NFG>          // ffn = 32 * NFG, NFG <= 16
 __global__ __launch_bounds__(kRegWaves * 64) void prefill_down_reg_kernel(TiledArgs ta) {
     const PrefillArgs &a = ta.p;
     constexpr uint32_t F = 32u * NFG, FB = F / 256u, NCK = NFG / 4u;
-    extern __shared__ __attribute__((aligned(16))) uint8_t dyn[];          // sign table | scaled magnitude table
+    __shared__ __attribute__((aligned(16))) uint8_t tables[kSignBytes + kScaledMagBytes];      // static: table reads take immediate offsets
     __shared__ __attribute__((aligned(16))) float pair_scale[2][kTile];      // per column half of the activations
     const uint32_t tid = threadIdx.x, lane = tid & 63u, r = lane & 15u, q = lane >> 4;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t H = a.hidden, P = a.ntok * a.top_k;
-    const uint8_t *sgn = dyn, *mag = dyn + kSignBytes;
-    build_scaled_tables(dyn + kSignBytes, dyn, tid, kRegWaves * 64u);
+    const uint8_t *sgn = tables, *mag = tables + kSignBytes;
+    build_scaled_tables(tables + kSignBytes, tables, tid, kRegWaves * 64u);
     const uint32_t T = a.n_tiles[0], U = a.n_unique[0];
     const uint64_t down_off = 2u * ((uint64_t)F * (H / 32u) * 8u + (uint64_t)F * (H / 256u) * 2u), qs_bytes = (uint64_t)H * NFG * 8u;
     constexpr uint32_t kRowsPerPass = 16u * kRegWaves;
@@ -691,13 +692,13 @@ template <int NFG>          // ffn = 32 * NFG, NFG <= 16
 __global__ __launch_bounds__(kRegWaves * 64) void prefill_down_iq3s_kernel(Iq3DownArgs da) {
     const PrefillArgs &a = da.p;
     constexpr uint32_t F = 32u * NFG, FB = F / 256u, NCK = NFG / 4u;
-    extern __shared__ __attribute__((aligned(16))) uint8_t dyn[];          // sign table | scaled magnitude table
+    __shared__ __attribute__((aligned(16))) uint8_t tables[kIq3SignBytes + kIq3MagBytes];      // static: table reads take immediate offsets
     __shared__ __attribute__((aligned(16))) float pair_scale[2][kTile];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, r = lane & 15u, q = lane >> 4;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t H = a.hidden;
-    const uint8_t *sgn = dyn, *mag = dyn + kIq3SignBytes;
-    build_iq3s_tables(dyn, dyn + kIq3SignBytes, tid, kRegWaves * 64u);
+    const uint8_t *sgn = tables, *mag = tables + kIq3SignBytes;
+    build_iq3s_tables(tables, tables + kIq3SignBytes, tid, kRegWaves * 64u);
     const uint32_t T = a.n_tiles[0];
     const uint64_t qs_bytes = (uint64_t)H * NFG * 16u;
     constexpr uint32_t kRowsPerPass = 16u * kRegWaves;
@@ -868,14 +869,14 @@ hipError_t launch_swiglu_rows(const float *gu, uint32_t gu_stride, uint32_t ntok
 
 static hipError_t launch_gateup_reg(const TiledArgs &ta, dim3 grid, hipStream_t s) {
     const uint32_t hidden = ta.p.hidden, ffn = ta.p.ffn;
-    const size_t acts_lds = kScaledMagBytes + kSignBytes + (size_t)kTile * (ffn + 4u) * sizeof(float);
+    const size_t acts_lds = (size_t)kTile * (ffn + 4u) * sizeof(float);
     hipError_t e = hipSuccess;
     prof_set_stage(ST_PREFILL_GATEUP);
 #define REDHIP_PGR(NKC)                                                                                                                   \
     do {                                                                                                                                  \
         static bool attr = false;                                                                                                          \
         if (!attr) {                                                                                                                       \
-            e = hipFuncSetAttribute(reinterpret_cast<const void *>(prefill_gateup_reg_kernel<NKC>), hipFuncAttributeMaxDynamicSharedMemorySize, 112 * 1024); \
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(prefill_gateup_reg_kernel<NKC>), hipFuncAttributeMaxDynamicSharedMemorySize, 40 * 1024); \
             if (e != hipSuccess) return e;                                                                                                 \
             attr = true;                                                                                                                   \
         }                                                                                                                                  \
@@ -925,17 +926,9 @@ hipError_t launch_prefill_down_iq3s(const void *tiled_down, uint64_t stride, con
     const Iq3DownArgs da{a, static_cast<const uint8_t *>(tiled_down), stride};
     const uint32_t tile_bound = prefill_tile_bound(ntok, top_k, n_expert);
     const dim3 grid(tile_bound < 256u ? tile_bound : 256u);
-    const size_t lds = kIq3SignBytes + kIq3MagBytes;
-    static bool attr = false;
-    if (!attr) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(prefill_down_iq3s_kernel<8>), hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
-        if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void *>(prefill_down_iq3s_kernel<16>), hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
-        if (e != hipSuccess) return e;
-        attr = true;
-    }
     prof_set_stage(ST_PREFILL_DOWN);
-    if (ffn == 256u) REDHIP_LAUNCH(prefill_down_iq3s_kernel<8>, grid, dim3(kRegWaves * 64), lds, s, da);
-    else REDHIP_LAUNCH(prefill_down_iq3s_kernel<16>, grid, dim3(kRegWaves * 64), lds, s, da);
+    if (ffn == 256u) REDHIP_LAUNCH(prefill_down_iq3s_kernel<8>, grid, dim3(kRegWaves * 64), 0, s, da);
+    else REDHIP_LAUNCH(prefill_down_iq3s_kernel<16>, grid, dim3(kRegWaves * 64), 0, s, da);
     return hipGetLastError();
 }
 
@@ -959,19 +952,11 @@ hipError_t launch_prefill_packed(const void *experts, uint64_t stride, const voi
     if (tiled_experts && tiled_shared && ffn <= 512u) {          // tile-major copy present: activations of a tile in registers
         const TiledArgs ta{a, static_cast<const uint8_t *>(tiled_experts), static_cast<const uint8_t *>(tiled_shared), nullptr};
         const dim3 rblock(kRegWaves * 64);
-        const size_t tab_lds = kScaledMagBytes + kSignBytes;
         e = launch_gateup_reg(ta, grid, s);
         if (e != hipSuccess) return e;
         prof_set_stage(ST_PREFILL_DOWN);
-        static bool down_attr = false;
-        if (!down_attr) {
-            e = hipFuncSetAttribute(reinterpret_cast<const void *>(prefill_down_reg_kernel<8>), hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
-            if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void *>(prefill_down_reg_kernel<16>), hipFuncAttributeMaxDynamicSharedMemorySize, 80 * 1024);
-            if (e != hipSuccess) return e;
-            down_attr = true;
-        }
-        if (ffn == 256u) REDHIP_LAUNCH(prefill_down_reg_kernel<8>, grid, rblock, tab_lds, s, ta);
-        else REDHIP_LAUNCH(prefill_down_reg_kernel<16>, grid, rblock, tab_lds, s, ta);
+        if (ffn == 256u) REDHIP_LAUNCH(prefill_down_reg_kernel<8>, grid, rblock, 0, s, ta);
+        else REDHIP_LAUNCH(prefill_down_reg_kernel<16>, grid, rblock, 0, s, ta);
         return hipGetLastError();
     }
     const size_t dyn_lds = (size_t)2u * kTile * (hidden + kRowPad) * 2u;
