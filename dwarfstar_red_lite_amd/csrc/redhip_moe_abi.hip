@@ -62,6 +62,11 @@ struct Moe {
     bool mixed = false;
     uint64_t packed_stride = 0;              // bytes between experts in `packed`
     bool packed_gu() const { return fused || mixed; }
+    // every path of an all-IQ2_XXS handle of these shapes reads the packed copies: the raw GGUF rows of the routed experts only pass
+    // through a staging buffer at upload
+    bool keep_raw() const { return !(fused && cfg.hidden / 512u <= 4u); }
+    uint8_t *stage = nullptr;                // upload staging for handles that do not keep the raw rows: kStageExperts slots
+    static constexpr uint32_t kStageExperts = 64u;
     // handles that can be given chunks keep a tile-major copy for the prefill kernels that hold a tile's activations in registers
     // chunks of 16 tokens and more take the router as a tiled f32 product (a quantised router through its f32 copy)
     bool tiled_router(uint32_t ntok) const {
@@ -283,12 +288,12 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
         const size_t small = align256(m->router_bytes) + align256(2u * m->sh_gate_bytes + m->sh_down_bytes) + align256(4u * c.hidden);
         uint8_t *p = nullptr;
         ok = hipMalloc(reinterpret_cast<void **>(&p), small) == hipSuccess &&
-             hipMalloc(reinterpret_cast<void **>(&L.experts), (size_t)c.n_expert * m->expert_stride) == hipSuccess;
+             (!m->keep_raw() || hipMalloc(reinterpret_cast<void **>(&L.experts), (size_t)c.n_expert * m->expert_stride) == hipSuccess);
         if (!ok) { if (p) (void)hipFree(p); break; }
         L.router = p;
         L.shared = p + align256(m->router_bytes);
         L.gate_inp = reinterpret_cast<float *>(L.shared + align256(2u * m->sh_gate_bytes + m->sh_down_bytes));
-        m->resident += small + (uint64_t)c.n_expert * m->expert_stride;
+        m->resident += small + (m->keep_raw() ? (uint64_t)c.n_expert * m->expert_stride : 0u);
         if (m->packed_gu()) {
             const bool sh_packed = m->sh_gu_type == T_IQ2_XXS;       // otherwise the shared expert is read from its raw rows
             ok = hipMalloc(reinterpret_cast<void **>(&L.packed), (size_t)c.n_expert * m->packed_stride) == hipSuccess &&
@@ -384,6 +389,7 @@ void redhip_moe_destroy(redhip_moe_t h) {
         if (L.shared_tiled) (void)hipFree(L.shared_tiled);
     }
     if (m->ws) (void)hipFree(m->ws);
+    if (m->stage) (void)hipFree(m->stage);
     delete m;
 }
 
@@ -436,6 +442,8 @@ int redhip_moe_load_shared(redhip_moe_t h, uint32_t layer, const float *gate_inp
     return 1;
 }
 
+static int stage_and_pack(Moe *m, uint32_t layer, uint32_t first, uint32_t count, uint8_t *dst, const uint8_t *gate, const uint8_t *up, const uint8_t *down);
+
 int redhip_moe_load_experts(redhip_moe_t h, uint32_t layer, uint32_t first, uint32_t count, const void *gate, const void *up, const void *down) {
     Moe *m = moe_of(h);
     if (!check_layer(m, layer)) return 0;
@@ -443,7 +451,25 @@ int redhip_moe_load_experts(redhip_moe_t h, uint32_t layer, uint32_t first, uint
         moe_err("invalid expert range first=%u count=%u of %u", first, count, m->cfg.n_expert);
         return 0;
     }
-    uint8_t *dst = m->layers[layer].experts + (uint64_t)first * m->expert_stride;
+    if (!m->keep_raw()) {           // through the staging buffer, a few experts at a time
+        if (!m->stage) {
+            HIP_OK(hipMalloc(reinterpret_cast<void **>(&m->stage), (size_t)Moe::kStageExperts * m->expert_stride), "staging allocation");
+            m->resident += (uint64_t)Moe::kStageExperts * m->expert_stride;
+        }
+        for (uint32_t done = 0; done < count; done += Moe::kStageExperts) {
+            const uint32_t n = count - done < Moe::kStageExperts ? count - done : Moe::kStageExperts;
+            if (!stage_and_pack(m, layer, first + done, n, m->stage, static_cast<const uint8_t *>(gate) + (uint64_t)done * m->gate_bytes,
+                                static_cast<const uint8_t *>(up) + (uint64_t)done * m->gate_bytes, static_cast<const uint8_t *>(down) + (uint64_t)done * m->down_bytes))
+                return 0;
+        }
+        return 1;
+    }
+    return stage_and_pack(m, layer, first, count, m->layers[layer].experts + (uint64_t)first * m->expert_stride, static_cast<const uint8_t *>(gate),
+                          static_cast<const uint8_t *>(up), static_cast<const uint8_t *>(down));
+}
+
+// raw rows of `count` experts into the gate | up | down slots at dst, then the packed / tile-major copies of experts first .. first + count - 1
+static int stage_and_pack(Moe *m, uint32_t layer, uint32_t first, uint32_t count, uint8_t *dst, const uint8_t *gate, const uint8_t *up, const uint8_t *down) {
     // 2-D copies place the tightly packed source matrices into the gate | up | down slots
     HIP_OK(hipMemcpy2D(dst, m->expert_stride, gate, m->gate_bytes, m->gate_bytes, count, hipMemcpyDefault), "expert gate upload");
     HIP_OK(hipMemcpy2D(dst + m->gate_bytes, m->expert_stride, up, m->gate_bytes, m->gate_bytes, count, hipMemcpyDefault), "expert up upload");
