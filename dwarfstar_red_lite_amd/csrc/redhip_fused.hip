@@ -978,8 +978,8 @@ __device__ __forceinline__ float chunk_dot(const uint8_t *row, uint32_t chunk, c
     return acc;
 }
 
-template <uint32_t TD, uint32_t TS>
-__global__ __launch_bounds__(kWaves * 64) void down_combine_raw_kernel(DownRawArgs a) {
+template <uint32_t TD, uint32_t TS, int NW>      // NW waves: 12 when the slots fit (a third more registers per lane: no spills), else 16
+__global__ __launch_bounds__(NW * 64) void down_combine_raw_kernel(DownRawArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t raw_rows[];     // [slot][8 rows of the slot's matrix]
     __shared__ float part[17 * 8];
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
@@ -1037,14 +1037,17 @@ __global__ __launch_bounds__(kWaves * 64) void down_combine_raw_kernel(DownRawAr
 
 template <uint32_t TD>
 static hipError_t launch_down_raw_shared(uint32_t ts, const DownRawArgs &a, uint32_t ntok, hipStream_t s) {
-    const dim3 grid(a.hidden / 8u, ntok), block(kWaves * 64);
+    const bool narrow = a.top_k + 1u <= 12u;
+    const dim3 grid(a.hidden / 8u, ntok), block(narrow ? 12 * 64 : kWaves * 64);
     const size_t lds = (size_t)(a.top_k + 1u) * 8u * (a.ffn / 256u) * 210u;       // sized for the largest block type; at most 17 x 8 x 4 x 210 bytes
+#define REDHIP_DRAW(TSV) do { if (narrow) REDHIP_LAUNCH((down_combine_raw_kernel<TD, TSV, 12>), grid, block, lds, s, a); else REDHIP_LAUNCH((down_combine_raw_kernel<TD, TSV, kWaves>), grid, block, lds, s, a); } while (0)
     switch (ts) {
-        case T_IQ2_XXS: REDHIP_LAUNCH((down_combine_raw_kernel<TD, T_IQ2_XXS>), grid, block, lds, s, a); break;
-        case T_IQ3_S: REDHIP_LAUNCH((down_combine_raw_kernel<TD, T_IQ3_S>), grid, block, lds, s, a); break;
-        case T_Q6_K: REDHIP_LAUNCH((down_combine_raw_kernel<TD, T_Q6_K>), grid, block, lds, s, a); break;
+        case T_IQ2_XXS: REDHIP_DRAW(T_IQ2_XXS); break;
+        case T_IQ3_S: REDHIP_DRAW(T_IQ3_S); break;
+        case T_Q6_K: REDHIP_DRAW(T_Q6_K); break;
         default: return hipErrorInvalidValue;
     }
+#undef REDHIP_DRAW
     return hipGetLastError();
 }
 
