@@ -200,6 +200,7 @@ struct RouterArgs {
     // Q6_K shared expert of a mixed-precision layout (single token): its gate and up rows (2 * ffn rows, the up matrix
     // right behind the gate matrix) are multiplied here, by workgroups behind the router's, into sh_gu [2 * ffn]
     const uint8_t *sh_q6k;
+    const float *sh_dense;     // or the same 2 * ffn rows as f32 [2 * ffn][hidden] (f32 router kernel): rows behind the gate vector's
     float *sh_gu;
     uint32_t ffn;
     // block step: the activations are (x + branch) * rsqrt(mean((x + branch)^2) + eps) * norm_w, written to xn_out
@@ -233,10 +234,12 @@ template <int NV>          // float4 per lane: hidden = 256 * NV
 __global__ __launch_bounds__(256) void router_f32_kernel(const float *w, RouterArgs a) {
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63u, H = a.hidden, tok = blockIdx.y;
     const uint32_t r = blockIdx.x * 4u + wave;
-    const float4 *wr = reinterpret_cast<const float4 *>(r < a.n_expert ? w + (uint64_t)r * H : a.gate_inp);
+    const uint32_t n_rows = a.n_expert + 1u + (a.sh_dense ? 2u * a.ffn : 0u);      // router rows, the gate vector, then the shared expert's gate | up rows
+    const float4 *wr = reinterpret_cast<const float4 *>(r < a.n_expert ? w + (uint64_t)r * H : r == a.n_expert ? a.gate_inp
+                                                        : a.sh_dense + (uint64_t)(r < n_rows ? r - a.n_expert - 1u : 0u) * H);
     const float4 *xv = reinterpret_cast<const float4 *>(a.x + (uint64_t)tok * H);
     float4 wv[NV], xq[NV];
-    if (r <= a.n_expert) {
+    if (r < n_rows) {
 #pragma unroll
         for (int k = 0; k < NV; ++k) wv[k] = wr[lane + 64u * k];
     }
@@ -265,13 +268,14 @@ __global__ __launch_bounds__(256) void router_f32_kernel(const float *w, RouterA
 #pragma unroll
     for (int k = 0; k < NV; ++k) {
         amax = fmaxf(fmaxf(amax, fmaxf(fabsf(xq[k].x), fabsf(xq[k].y))), fmaxf(fabsf(xq[k].z), fabsf(xq[k].w)));
-        if (r <= a.n_expert) {
+        if (r < n_rows) {
             acc = fmaf(wv[k].x, xq[k].x, acc); acc = fmaf(wv[k].y, xq[k].y, acc);
             acc = fmaf(wv[k].z, xq[k].z, acc); acc = fmaf(wv[k].w, xq[k].w, acc);
         }
     }
     acc = wave_sum(acc);
     if (lane == 0u && r <= a.n_expert) a.logits[(uint64_t)tok * (a.n_expert + 1u) + r] = acc;
+    else if (lane == 0u && r < n_rows) a.sh_gu[(uint64_t)tok * 2u * a.ffn + (r - a.n_expert - 1u)] = acc;
     split_x_job(a, tok, wave_max(amax), norm_inv);
 }
 
@@ -367,14 +371,16 @@ __global__ __launch_bounds__(256) void router_quant_kernel(const uint8_t *w, Rou
 
 hipError_t launch_router_gemv(uint32_t router_type, const void *w, const float *x, const float *gate_inp, uint32_t ntok, uint32_t hidden,
                               uint32_t n_expert, float *logits, void *xh, void *xl, int *xexp, const void *sh_q6k, float *sh_gu, uint32_t ffn,
-                              hipStream_t s) {
+                              hipStream_t s, const float *sh_dense) {
     if (!ntok || !hidden || hidden % 256u || !n_expert || n_expert > 1024u) return hipErrorInvalidValue;
     const bool with_shared = sh_q6k && sh_gu && router_type == T_Q6_K && ntok <= 8u && ffn % 4u == 0u;      // sh_gu: [ntok][2 * ffn]
     const BlockContext &bc = block_context();
     if (bc.branch && (!bc.norm_w || !bc.xn_out)) return hipErrorInvalidValue;
+    const bool with_dense = sh_dense && sh_gu && router_type == T_F32 && ntok <= 8u;      // sh_gu: [ntok][2 * ffn]
     RouterArgs a{x, gate_inp, logits, static_cast<_Float16 *>(xh), static_cast<_Float16 *>(xl), xexp, hidden, n_expert,
-                 with_shared ? static_cast<const uint8_t *>(sh_q6k) : nullptr, sh_gu, ffn, bc.branch, bc.norm_w, bc.eps, bc.xn_out};
-    const dim3 grid((n_expert + 1u + 3u) / 4u, ntok);
+                 with_shared ? static_cast<const uint8_t *>(sh_q6k) : nullptr, with_dense ? sh_dense : nullptr, sh_gu, ffn, bc.branch, bc.norm_w, bc.eps,
+                 bc.xn_out};
+    const dim3 grid((n_expert + 1u + (with_dense ? 2u * ffn : 0u) + 3u) / 4u, ntok);
     if (router_type == T_F32) {
         const float *wf = static_cast<const float *>(w);
         switch (hidden / 256u) {

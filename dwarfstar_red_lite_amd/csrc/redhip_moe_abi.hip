@@ -70,7 +70,7 @@ struct Moe {
     // handles that can be given chunks keep a tile-major copy for the prefill kernels that hold a tile's activations in registers
     // chunks of 16 tokens and more take the router as a tiled f32 product (a quantised router through its f32 copy)
     bool tiled_router(uint32_t ntok) const {
-        return packed_gu() && ntok >= 16u && (cfg.router_type == T_F32 || (mixed && tiles_resident()));
+        return packed_gu() && ntok >= 16u && (cfg.router_type == T_F32 || mixed);
     }
     bool tiles_resident() const { return packed_gu() && cfg.max_tokens > 8u && cfg.ffn <= 512u && cfg.hidden / 512u <= 4u; }
     // a chunk on a mixed layout: the routed gate/up matrices (packed IQ2_XXS) run on the prefill tiles, the rest on raw rows
@@ -300,7 +300,7 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
                  (!sh_packed || hipMalloc(reinterpret_cast<void **>(&L.shared_packed), align256(2u * m->sh_gate_bytes + m->sh_down_bytes)) == hipSuccess);
             m->resident += (uint64_t)c.n_expert * m->packed_stride + (sh_packed ? align256(2u * m->sh_gate_bytes + m->sh_down_bytes) : 0u);
         }
-        if (ok && m->mixed && m->tiles_resident()) {
+        if (ok && m->mixed) {
             const size_t rb = c.router_type == T_F32 ? 0u : (size_t)c.n_expert * c.hidden * 4u, gb = (size_t)2u * c.ffn * c.hidden * 4u, db = (size_t)c.hidden * c.ffn * 4u;
             float *d = nullptr;
             ok = hipMalloc(reinterpret_cast<void **>(&d), align256(rb) + align256(gb) + align256(db)) == hipSuccess;
@@ -507,11 +507,20 @@ int redhip_moe_route(redhip_moe_t h, uint32_t layer, const float *x_dev, uint32_
     if (m->fast_route()) {
         prof_set_stage(ST_ROUTER_GEMV);
         // a Q6_K shared expert of a mixed layout rides along: its gate / up products land in m->act (otherwise unused on this path)
-        m->shared_gu_ready = m->mixed && m->sh_gu_type == T_Q6_K && c.router_type == T_Q6_K && (ntok == 1u || m->small_batch_mixed(ntok)) && c.top_k >= 2u;
         const float *router_f32 = c.router_type == T_F32 ? reinterpret_cast<const float *>(m->layers[layer].router) : m->layers[layer].dense_router;
+        // one token or a small batch on a mixed layout: the router and the shared expert's gate | up rows as one f32 GEMV over their f32 copies
+        // (4.5 times the bytes of the Q6_K rows, none of their decode arithmetic)
+        const uint32_t nv = c.hidden / 256u;
+        const bool dense_small = m->mixed && router_f32 && m->layers[layer].dense_gu && (ntok == 1u || m->small_batch_mixed(ntok)) && c.top_k >= 2u &&
+                                 (nv == 2u || nv == 4u || nv == 8u || nv == 16u);
+        m->shared_gu_ready = dense_small ||
+                             (m->mixed && m->sh_gu_type == T_Q6_K && c.router_type == T_Q6_K && (ntok == 1u || m->small_batch_mixed(ntok)) && c.top_k >= 2u);
         if (m->tiled_router(ntok))
             HIP_OK(launch_router_f32_tiles(router_f32, m->layers[layer].gate_inp, x_dev, ntok, c.hidden,
                                            c.n_expert, m->logits, m->xh, m->xl, m->xexp, s), "router tile launch");
+        else if (dense_small)
+            HIP_OK(launch_router_gemv(T_F32, router_f32, x_dev, m->layers[layer].gate_inp, ntok, c.hidden, c.n_expert, m->logits, m->xh, m->xl, m->xexp,
+                                      nullptr, m->act, c.ffn, s, m->layers[layer].dense_gu), "router launch");
         else
             HIP_OK(launch_router_gemv(c.router_type, m->layers[layer].router, x_dev, m->layers[layer].gate_inp, ntok, c.hidden, c.n_expert,
                                       m->logits, m->xh, m->xl, m->xexp, m->shared_gu_ready ? m->layers[layer].shared : nullptr, m->act, c.ffn, s),
