@@ -37,6 +37,12 @@ template <> struct Fmt<T_IQ2_XXS> { static constexpr uint32_t kBlock = 66u; };
 template <> struct Fmt<T_IQ3_S> { static constexpr uint32_t kBlock = 110u; };
 template <> struct Fmt<T_Q6_K> { static constexpr uint32_t kBlock = 210u; };
 template <> struct Fmt<T_F32> { static constexpr uint32_t kBlock = 1024u; };   // 256 floats
+template <> struct Fmt<T_IQ2_XS> { static constexpr uint32_t kBlock = 74u; };
+template <> struct Fmt<T_IQ1_M> { static constexpr uint32_t kBlock = 56u; };
+// bytes of the caller-supplied codebook a format decodes through (int8 [entries][8]); 0: the codebook is built in
+template <uint32_t T> struct Codebook { static constexpr uint32_t kBytes = 0u; };
+template <> struct Codebook<T_IQ2_XS> { static constexpr uint32_t kBytes = 512u * 8u; };
+template <> struct Codebook<T_IQ1_M> { static constexpr uint32_t kBytes = 2048u * 8u; };
 
 // w[0..32) = weights [32*chunk, 32*chunk + 32) of the row starting at `row`
 template <uint32_t T> __device__ __forceinline__ void decode32(const uint8_t *row, uint32_t chunk, float *w);
@@ -108,6 +114,54 @@ template <> __device__ __forceinline__ void decode32<T_Q6_K>(const uint8_t *row,
             const uint32_t l = 2u * i + b;
             w[l] = (l < 16u ? d0 : d1) * (float)v;
         }
+    }
+}
+
+// Formats that decode through a caller-supplied codebook: `grid` is that codebook, in global memory or a copy in LDS.
+template <uint32_t T> __device__ __forceinline__ void decode32_cb(const uint8_t *row, uint32_t chunk, float *w, const int8_t *grid) {
+    (void)grid;
+    decode32<T>(row, chunk, w);
+}
+
+// IQ2_XS, native/redlite_native_reference.c:116-142: block = f16 d, 32 x u16 (9-bit codebook index + 7 sign bits, the
+// eighth sign is their parity), 8 bytes of 4-bit scales (one per 16 weights); weight = d * (0.5 + scale) * 0.25 * entry * sign
+template <> __device__ __forceinline__ void decode32_cb<T_IQ2_XS>(const uint8_t *row, uint32_t chunk, float *w, const int8_t *grid) {
+    const uint8_t *bp = row + (size_t)(chunk >> 3) * 74u;
+    const uint32_t cb = chunk & 7u;
+    const float d = half_bits_to_f32(ld_u16(bp));
+    const uint32_t sc = bp[66u + cb];
+    const float db0 = d * (0.5f + (float)(sc & 15u)) * 0.25f, db1 = d * (0.5f + (float)(sc >> 4)) * 0.25f;
+#pragma unroll
+    for (uint32_t k = 0; k < 4u; ++k) {
+        const uint32_t q = ld_u16(bp + 2u + 2u * (4u * cb + k));
+        const int8_t *entry = grid + (q & 511u) * 8u;
+        const uint32_t s7 = (q >> 9) & 127u, s8 = s7 | ((__popc(s7) & 1u) << 7);
+        const float db = k < 2u ? db0 : db1;
+#pragma unroll
+        for (uint32_t j = 0; j < 8u; ++j) w[8u * k + j] = apply_sign(db * (float)entry[j], (s8 >> j) & 1u);
+    }
+}
+
+// IQ1_M, native/redlite_native_reference.c:149-170: block = 32 index bytes, 16 bytes of nibbles (3 high index bits + the
+// sign of the 1/8 offset), four u16 with 3-bit scales (one per 16 weights) and the f16 d spread over their top nibbles;
+// weight = d * (2 * scale + 1) * (entry + or - 0.125), entry in {-1, 0, 1}
+template <> __device__ __forceinline__ void decode32_cb<T_IQ1_M>(const uint8_t *row, uint32_t chunk, float *w, const int8_t *grid) {
+    const uint8_t *bp = row + (size_t)(chunk >> 3) * 56u;
+    const uint32_t cb = chunk & 7u;
+    uint32_t sc[4];
+#pragma unroll
+    for (uint32_t i = 0; i < 4u; ++i) sc[i] = ld_u16(bp + 48u + 2u * i);
+    const float d = half_bits_to_f32((sc[0] >> 12) | ((sc[1] >> 8) & 0x00f0u) | ((sc[2] >> 4) & 0x0f00u) | (sc[3] & 0xf000u));
+#pragma unroll
+    for (uint32_t k = 0; k < 4u; ++k) {
+        const uint32_t group = 4u * cb + k;
+        const uint32_t nibble = ((uint32_t)bp[32u + (group >> 1)] >> (4u * (group & 1u))) & 15u;
+        const int8_t *entry = grid + ((uint32_t)bp[group] | ((nibble & 7u) << 8)) * 8u;
+        const float delta = (nibble & 8u) ? -0.125f : 0.125f;
+        const uint32_t si = group >> 1;
+        const float dl = d * (float)(2u * ((sc[si >> 2] >> (3u * (si & 3u))) & 7u) + 1u);
+#pragma unroll
+        for (uint32_t j = 0; j < 8u; ++j) w[8u * k + j] = dl * ((float)entry[j] + delta);
     }
 }
 

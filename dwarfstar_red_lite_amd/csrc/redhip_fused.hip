@@ -62,6 +62,54 @@ hipError_t launch_repack_iq2xxs(const void *raw, uint64_t raw_stride, uint32_t c
     return hipGetLastError();
 }
 
+// The same split for the two formats that decode through caller-supplied codebooks, row-major only:
+//   IQ2_XS (74-byte blocks): qs [nrows][K/32] uint2 = the group's four u16 (9-bit index + 7 sign bits each), ds [nrows][K/256] u16,
+//                            sc [nrows][K/32] u8 = the group's two 4-bit scales (one per 16 weights)
+//   IQ1_M (56-byte blocks):  qs [nrows][K/32] uint2: x = the group's four low index bytes, y = its four nibbles (3 high index bits +
+//                            offset sign) | scale of the first 16 weights << 16 | scale of the second 16 << 19; ds [nrows][K/256] u16 = d
+//                            gathered from the top nibbles of the block's four scale words
+template <uint32_t T>
+__global__ void repack_codebook_kernel(const uint8_t *raw0, uint64_t raw_stride, uint32_t nrows, uint32_t K, uint8_t *packed0, uint64_t packed_stride) {
+    const uint32_t groups = K / 32u, blocks = K / 256u;
+    const uint8_t *raw = raw0 + (uint64_t)blockIdx.y * raw_stride;
+    uint8_t *pk = packed0 + (uint64_t)blockIdx.y * packed_stride;
+    uint2 *qs = reinterpret_cast<uint2 *>(pk);
+    uint16_t *ds = reinterpret_cast<uint16_t *>(pk + (uint64_t)nrows * groups * 8u);
+    uint8_t *sc = pk + (uint64_t)nrows * groups * 8u + (uint64_t)nrows * blocks * 2u;
+    const uint64_t gid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= (uint64_t)nrows * groups) return;
+    const uint32_t r = (uint32_t)(gid / groups), g = (uint32_t)(gid % groups), gb = g & 7u;
+    const uint8_t *bp = raw + ((uint64_t)r * blocks + (g >> 3)) * Fmt<T>::kBlock;
+    if constexpr (T == T_IQ2_XS) {
+        qs[gid] = make_uint2(ld_u32_a2(bp + 2u + 8u * gb), ld_u32_a2(bp + 6u + 8u * gb));
+        sc[gid] = bp[66u + gb];
+        if (gb == 0u) ds[(uint64_t)r * blocks + (g >> 3)] = (uint16_t)ld_u16(bp);
+    } else {
+        const uint32_t word = ld_u16(bp + 48u + 2u * (gb >> 1)), sh = 6u * (gb & 1u);
+        qs[gid] = make_uint2(ld_u32_a2(bp + 4u * gb), ld_u16(bp + 32u + 2u * gb) | (((word >> sh) & 7u) << 16) | (((word >> (sh + 3u)) & 7u) << 19));
+        if (gb == 0u) {
+            const uint32_t s0 = ld_u16(bp + 48u), s1 = ld_u16(bp + 50u), s2 = ld_u16(bp + 52u), s3 = ld_u16(bp + 54u);
+            ds[(uint64_t)r * blocks + (g >> 3)] = (uint16_t)((s0 >> 12) | ((s1 >> 8) & 0x00f0u) | ((s2 >> 4) & 0x0f00u) | (s3 & 0xf000u));
+        }
+    }
+}
+
+// gate / up matrices of `type` (IQ2_XXS, IQ2_XS, IQ1_M) into the streams the one-token gate/up kernel reads; packed_matrix_bytes() each
+hipError_t launch_repack_gateup(uint32_t type, const void *raw, uint64_t raw_stride, uint32_t count, uint32_t nrows, uint32_t K,
+                                void *packed, uint64_t packed_stride, hipStream_t s) {
+    if (type == T_IQ2_XXS) return launch_repack_iq2xxs(raw, raw_stride, count, nrows, K, false, packed, packed_stride, s);
+    if (!nrows || !K || K % 256u || !count || count > 65535u) return hipErrorInvalidValue;
+    const uint64_t total = (uint64_t)nrows * (K / 32u);
+    const dim3 grid((uint32_t)((total + 255u) / 256u), count);
+    if (type == T_IQ2_XS)
+        REDHIP_LAUNCH(repack_codebook_kernel<T_IQ2_XS>, grid, dim3(256), 0, s, static_cast<const uint8_t *>(raw), raw_stride, nrows, K, static_cast<uint8_t *>(packed), packed_stride);
+    else if (type == T_IQ1_M)
+        REDHIP_LAUNCH(repack_codebook_kernel<T_IQ1_M>, grid, dim3(256), 0, s, static_cast<const uint8_t *>(raw), raw_stride, nrows, K, static_cast<uint8_t *>(packed), packed_stride);
+    else
+        return hipErrorInvalidValue;
+    return hipGetLastError();
+}
+
 // parity tap: f32 dequantisation straight from the packed streams (row-major output [nrows][K])
 __global__ void dequant_packed_iq2xxs_kernel(const uint2 *qs, const uint16_t *ds, uint32_t nrows, uint32_t K, int col_major, float *out) {
     const uint32_t groups = K / 32u, blocks = K / 256u;
@@ -85,6 +133,46 @@ hipError_t launch_dequant_packed_iq2xxs(const void *packed, uint32_t nrows, uint
     const uint16_t *ds = reinterpret_cast<const uint16_t *>(static_cast<const uint8_t *>(packed) + (uint64_t)nrows * (K / 32u) * 8u);
     const uint64_t total = (uint64_t)nrows * (K / 32u);
     REDHIP_LAUNCH(dequant_packed_iq2xxs_kernel, dim3((uint32_t)((total + 255u) / 256u)), dim3(256), 0, s, qs, ds, nrows, K, col_major ? 1 : 0, out);
+    return hipGetLastError();
+}
+
+// the same tap for the packed IQ2_XS / IQ1_M streams; arithmetic as decode32_cb
+template <uint32_t T>
+__global__ void dequant_packed_codebook_kernel(const uint8_t *pk, uint32_t nrows, uint32_t K, const int8_t *grid, float *out) {
+    const uint32_t groups = K / 32u, blocks = K / 256u;
+    const uint64_t gid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= (uint64_t)nrows * groups) return;
+    const uint32_t r = (uint32_t)(gid / groups), g = (uint32_t)(gid % groups);
+    const uint2 v = reinterpret_cast<const uint2 *>(pk)[gid];
+    const float d = half_bits_to_f32(reinterpret_cast<const uint16_t *>(pk + (uint64_t)nrows * groups * 8u)[(uint64_t)r * blocks + (g >> 3)]);
+    float *o = out + (uint64_t)r * K + 32u * g;
+    if constexpr (T == T_IQ2_XS) {
+        const uint32_t sc = (pk + (uint64_t)nrows * groups * 8u + (uint64_t)nrows * blocks * 2u)[gid];
+        for (uint32_t l = 0; l < 4u; ++l) {
+            const uint32_t w16 = ((l < 2u ? v.x : v.y) >> (16u * (l & 1u))) & 0xffffu;
+            const int8_t *entry = grid + (w16 & 511u) * 8u;
+            const uint32_t s7 = w16 >> 9, s8 = s7 | ((__popc(s7) & 1u) << 7);
+            const float db = d * (0.5f + (float)(l < 2u ? (sc & 15u) : (sc >> 4))) * 0.25f;
+            for (uint32_t j = 0; j < 8u; ++j) o[8u * l + j] = apply_sign(db * (float)entry[j], (s8 >> j) & 1u);
+        }
+    } else {
+        for (uint32_t l = 0; l < 4u; ++l) {
+            const int8_t *entry = grid + (((v.x >> (8u * l)) & 255u) | (((v.y >> (4u * l)) & 7u) << 8)) * 8u;
+            const float delta = ((v.y >> (4u * l + 3u)) & 1u) ? -0.125f : 0.125f;
+            const float dl = d * (float)(2u * ((v.y >> (l < 2u ? 16u : 19u)) & 7u) + 1u);
+            for (uint32_t j = 0; j < 8u; ++j) o[8u * l + j] = dl * ((float)entry[j] + delta);
+        }
+    }
+}
+
+hipError_t launch_dequant_packed(uint32_t type, const void *packed, uint32_t nrows, uint32_t K, const int8_t *grid, float *out, hipStream_t s) {
+    if (type == T_IQ2_XXS) return launch_dequant_packed_iq2xxs(packed, nrows, K, false, out, s);
+    if (!nrows || !K || K % 256u || !grid) return hipErrorInvalidValue;
+    const uint64_t total = (uint64_t)nrows * (K / 32u);
+    const dim3 grid_dim((uint32_t)((total + 255u) / 256u));
+    if (type == T_IQ2_XS) REDHIP_LAUNCH(dequant_packed_codebook_kernel<T_IQ2_XS>, grid_dim, dim3(256), 0, s, static_cast<const uint8_t *>(packed), nrows, K, grid, out);
+    else if (type == T_IQ1_M) REDHIP_LAUNCH(dequant_packed_codebook_kernel<T_IQ1_M>, grid_dim, dim3(256), 0, s, static_cast<const uint8_t *>(packed), nrows, K, grid, out);
+    else return hipErrorInvalidValue;
     return hipGetLastError();
 }
 
@@ -681,6 +769,55 @@ __device__ __forceinline__ float group_dot(uint2 q, const half4_t *ax, const uin
     return (acc[0] + acc[1] * 4.8828125e-4f) * (float)(2u * (q.y >> 28) + 1u);
 }
 
+// The same product for the packed IQ2_XS group (FMT 1: 9-bit indices into the caller's 512-entry codebook, one scale per 16 weights in
+// `sc`) and the packed IQ1_M group (FMT 2: 11-bit indices into the caller's 2048-entry codebook of -1 / 0 / 1, plus or minus 1/8 per
+// eight weights added as packed fp16, exact; 3-bit scales per 16 weights in q.y). `lds` is the fp16 copy of the codebook.
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+template <int FMT>
+__device__ __forceinline__ float group_dot_fmt(uint2 q, uint32_t sc, const half4_t *ax, const uint8_t *lds) {
+    if constexpr (FMT == 0) {
+        return group_dot(q, ax, lds);
+    } else {
+        float4_t acc[2] = {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}};
+#pragma unroll
+        for (uint32_t l = 0; l < 4u; ++l) {
+            WeightQuad b0, b1;
+            if constexpr (FMT == 1) {
+                const uint32_t w16 = ((l < 2u ? q.x : q.y) >> (16u * (l & 1u))) & 0xffffu;
+                signed_weights(lds, w16 & 511u, w16 >> 9, b0, b1);
+            } else {
+                const uint32_t idx = ((q.x >> (8u * l)) & 255u) | (((q.y >> (4u * l)) & 7u) << 8);
+                const uint4 m = *reinterpret_cast<const uint4 *>(lds + (idx << 4));
+                const half2_t delta = __builtin_bit_cast(half2_t, 0x30003000u | (((q.y >> (4u * l + 3u)) & 1u) * 0x80008000u));
+                b0.u[0] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, m.x) + delta);
+                b0.u[1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, m.y) + delta);
+                b1.u[0] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, m.z) + delta);
+                b1.u[1] = __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, m.w) + delta);
+            }
+            acc[l >> 1] = __builtin_amdgcn_mfma_f32_4x4x4f16(ax[2u * l], b0.h, acc[l >> 1], 0, 0, 0);
+            acc[l >> 1] = __builtin_amdgcn_mfma_f32_4x4x4f16(ax[2u * l + 1u], b1.h, acc[l >> 1], 0, 0, 0);
+        }
+        const uint32_t s0 = FMT == 1 ? (sc & 15u) : ((q.y >> 16) & 7u), s1 = FMT == 1 ? (sc >> 4) : ((q.y >> 19) & 7u);
+        return (acc[0][0] + acc[0][1] * 4.8828125e-4f) * (float)(2u * s0 + 1u) + (acc[1][0] + acc[1][1] * 4.8828125e-4f) * (float)(2u * s1 + 1u);
+    }
+}
+
+// fp16 copy of a caller-supplied codebook (int8 [entries][8]) in LDS, 16 bytes per entry; built by every wave but the first
+template <int FMT>
+__device__ __forceinline__ void build_codebook_table(uint8_t *lds, uint32_t tid, const int8_t *grid) {
+    constexpr uint32_t kEntries = FMT == 1 ? 512u : 2048u;
+    for (uint32_t i = tid - 64u; i < kEntries; i += (kWaves - 1) * 64u) {      // tid < 64 wraps past the bound
+        const uint64_t e = reinterpret_cast<const uint64_t *>(grid)[i];
+        uint32_t w4[4];
+#pragma unroll
+        for (int k = 0; k < 4; ++k) {
+            const _Float16 lo = (_Float16)(float)(int8_t)(e >> (16 * k)), hi = (_Float16)(float)(int8_t)(e >> (16 * k + 8));
+            w4[k] = (uint32_t)__builtin_bit_cast(uint16_t, lo) | ((uint32_t)__builtin_bit_cast(uint16_t, hi) << 16);
+        }
+        *reinterpret_cast<uint4 *>(lds + (size_t)i * 16u) = make_uint4(w4[0], w4[1], w4[2], w4[3]);
+    }
+}
+
 // the lane's activation operand: 32 values starting at src (fp16), lanes j = 0 / 1 carry hi / lo, others zero
 __device__ __forceinline__ void load_act_operand(half4_t *ax, const _Float16 *hi, const _Float16 *lo, uint32_t j) {
     const _Float16 *src = j == 0u ? hi : lo;
@@ -695,6 +832,7 @@ __device__ __forceinline__ void load_act_operand(half4_t *ax, const _Float16 *hi
 struct GateUpArgs {
     const uint8_t *experts;    // packed experts of the layer, expert e at experts + e * stride
     uint64_t stride;
+    const int8_t *grid;        // the caller's codebook of the routed experts' format (IQ2_XS, IQ1_M) or nullptr
     const uint8_t *shared;     // packed shared expert, or nullptr when it is not IQ2_XXS
     const uint8_t *shared_q6k; // then: its raw Q6_K rows, gate matrix then up matrix
     const float *x;            // [hidden] f32 activations (Q6_K shared expert only)
@@ -711,12 +849,13 @@ struct GateUpArgs {
     uint32_t hidden, ffn, n_expert, top_k;
 };
 
-template <int NKC>        // K chunks of 512 columns in a gate/up row: hidden = 512 * NKC
+// FMT: format of the routed (and a packed shared) expert's gate / up matrices: 0 IQ2_XXS, 1 IQ2_XS, 2 IQ1_M
+template <int NKC, int FMT>        // K chunks of 512 columns in a gate/up row: hidden = 512 * NKC
 __global__ __launch_bounds__(kWaves * 64) void gateup_select_kernel(GateUpArgs a) {
     constexpr int NW = kWaves;
     constexpr int UPW = 16 * NKC / NW;                 // (row-quad, K-chunk) units per wave
     static_assert(UPW >= 1 && UPW * NW == 16 * NKC, "waves must tile the 16 row-quads x NKC chunks");
-    __shared__ __attribute__((aligned(16))) uint8_t lds[kMagBytes];
+    __shared__ __attribute__((aligned(16))) uint8_t lds[FMT == 0 ? kMagBytes : FMT == 1 ? 512u * 16u : 2048u * 16u];
     __shared__ float part[NKC * 64];
     __shared__ SelectOut sel;
 
@@ -742,14 +881,15 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_select_kernel(GateUpArgs a
     const uint32_t slot = blockIdx.y;
     const bool is_shared = slot >= a.top_k;
     const uint32_t tb = tid - 256u;                     // waves 4..7 build the table: wave 0 goes straight to the selection
-    const uint64_t grid_entry = tb < 256u ? redhip_iq2xxs_grid[tb] : 0ull;
+    const uint64_t grid_entry = FMT == 0 && tb < 256u ? redhip_iq2xxs_grid[tb] : 0ull;
 
     // activation operand: independent of the routing, requested before the selection
     const uint32_t kc = wave % NKC, q0 = wave / NKC;
     const uint32_t G = 16u * kc + blk;                 // this lane's group inside the gate/up rows
     half4_t ax[8];
     load_act_operand(ax, a.xh + 32u * G, a.xl + 32u * G, j);
-    build_tables(lds, tb, grid_entry);
+    if constexpr (FMT == 0) build_tables(lds, tb, grid_entry);
+    else if (!is_shared) build_codebook_table<FMT>(lds, tid, a.grid);      // a shared expert beside these formats is never packed
 
     uint32_t expert = 0u;
     extern __shared__ __attribute__((aligned(16))) uint8_t raw_rows[];      // Q6_K shared expert only: the unit's 64 raw rows, then x
@@ -831,14 +971,15 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_select_kernel(GateUpArgs a
         return;
     }
     const uint8_t *ex = is_shared ? a.shared : a.experts + (uint64_t)expert * a.stride;
-    const uint64_t gate_bytes = (uint64_t)F * HG * 8u + (uint64_t)F * HB * 2u;
+    const uint64_t sc_off = (uint64_t)F * HG * 8u + (uint64_t)F * HB * 2u;       // IQ2_XS: the scale bytes follow the two other streams
+    const uint64_t gate_bytes = sc_off + (FMT == 1 ? (uint64_t)F * HG : 0u);
     const uint2 *gate_qs = reinterpret_cast<const uint2 *>(ex);
     const uint16_t *gate_ds = reinterpret_cast<const uint16_t *>(ex + (uint64_t)F * HG * 8u);
     const uint2 *up_qs = reinterpret_cast<const uint2 *>(ex + gate_bytes);
     const uint16_t *up_ds = reinterpret_cast<const uint16_t *>(ex + gate_bytes + (uint64_t)F * HG * 8u);
 
     uint2 wq[UPW];
-    uint32_t wd[UPW];
+    uint32_t wd[UPW], wsc[UPW];
 #pragma unroll
     for (int u = 0; u < UPW; ++u) {
         const uint32_t quad = q0 + (NW / NKC) * u;     // 0..7 gate, 8..15 up
@@ -847,10 +988,11 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_select_kernel(GateUpArgs a
         const uint16_t *ds = quad < 8u ? gate_ds : up_ds;
         wq[u] = qs[(uint64_t)r * HG + G];
         wd[u] = ds[(uint64_t)r * HB + (G >> 3)];
+        wsc[u] = FMT == 1 ? (uint32_t)(ex + (quad < 8u ? 0u : gate_bytes) + sc_off)[(uint64_t)r * HG + G] : 0u;
     }
     float v[UPW];
 #pragma unroll
-    for (int u = 0; u < UPW; ++u) v[u] = group_dot(wq[u], ax, lds) * scale_to_f32(wd[u]);
+    for (int u = 0; u < UPW; ++u) v[u] = group_dot_fmt<FMT>(wq[u], wsc[u], ax, lds) * scale_to_f32(wd[u]);
     const float tot = quad_column_reduce<UPW>(v, lane);
     if (reduced_writer<UPW>(lane)) {
         const uint32_t quad = q0 + (NW / NKC) * reduced_unit<UPW>(lane);
@@ -861,7 +1003,7 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_select_kernel(GateUpArgs a
         float gsum = 0.0f, usum = 0.0f;
 #pragma unroll
         for (int c = 0; c < NKC; ++c) { gsum += part[c * 64 + tid]; usum += part[c * 64 + 32 + tid]; }
-        const float xs = 0.125f * exp2i(a.xexp[0]);                  // d/8 and the pre-scale of x
+        const float xs = (FMT == 2 ? 1.0f : 0.125f) * exp2i(a.xexp[0]);      // d/8 (IQ1_M: d) and the pre-scale of x
         gsum *= xs;
         usum *= xs;
         const float act = (gsum / (1.0f + expf(-gsum))) * usum;
@@ -966,10 +1108,11 @@ struct DownRawArgs {
     float *out;
     uint32_t hidden, ffn, top_k;
     const float *resid_a, *resid_b;
+    const int8_t *grid;        // the caller's codebook of the routed down format (IQ2_XS, IQ1_M) or nullptr
 };
 
 template <uint32_t T>
-__device__ __forceinline__ float chunk_dot(const uint8_t *row, uint32_t chunk, const float *av) {
+__device__ __forceinline__ float chunk_dot(const uint8_t *row, uint32_t chunk, const float *av, const int8_t *grid = nullptr) {
     if constexpr (T == T_Q6_K) {
         float sx0 = 0.0f, sx1 = 0.0f;
 #pragma unroll
@@ -977,7 +1120,7 @@ __device__ __forceinline__ float chunk_dot(const uint8_t *row, uint32_t chunk, c
         return q6k_dot32(row, chunk, av, sx0, sx1);
     }
     float w[32];
-    decode32<T>(row, chunk, w);
+    decode32_cb<T>(row, chunk, w, grid);
     float acc = 0.0f;
 #pragma unroll
     for (int i = 0; i < 32; ++i) acc = fmaf(w[i], av[i], acc);
@@ -988,8 +1131,16 @@ template <uint32_t TD, uint32_t TS, int NW>      // NW waves: 12 when the slots 
 __global__ __launch_bounds__(NW * 64) void down_combine_raw_kernel(DownRawArgs a) {
     extern __shared__ __attribute__((aligned(16))) uint8_t raw_rows[];     // [slot][8 rows of the slot's matrix]
     __shared__ float part[17 * 8];
+    constexpr uint32_t kGridBytes = Codebook<TD>::kBytes;                  // routed format's codebook, copied to LDS (the shared expert never has one)
+    __shared__ __attribute__((aligned(16))) int8_t cb[kGridBytes ? kGridBytes : 16u];
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
     const uint32_t F = a.ffn, FG = F / 32u, FB = F / 256u, n_slot = a.top_k + 1u;
+    uint4 cbv[2] = {};                                 // requested first, stored once the wave's rows are on their way
+    if constexpr (kGridBytes != 0u) {
+#pragma unroll
+        for (uint32_t i = 0; i < 2u; ++i)
+            if (tid + i * NW * 64u < kGridBytes / 16u) cbv[i] = reinterpret_cast<const uint4 *>(a.grid)[tid + i * NW * 64u];
+    }
     if (const uint32_t tok = blockIdx.y) {             // several tokens in one launch
         const uint64_t t = tok;
         a.ids += t * a.top_k;
@@ -1003,12 +1154,20 @@ __global__ __launch_bounds__(NW * 64) void down_combine_raw_kernel(DownRawArgs a
     }
     const uint32_t row0 = 8u * blockIdx.x;
     constexpr uint32_t kMaxBlock = Fmt<TD>::kBlock > Fmt<TS>::kBlock ? Fmt<TD>::kBlock : Fmt<TS>::kBlock;
+    const bool is_shared = wave == a.top_k;
+    const uint32_t row_bytes = FB * (is_shared ? Fmt<TS>::kBlock : Fmt<TD>::kBlock);
+    uint8_t *mine = raw_rows + wave * 8u * FB * kMaxBlock;
     if (wave < n_slot) {
-        const bool is_shared = wave == a.top_k;
-        const uint32_t row_bytes = FB * (is_shared ? Fmt<TS>::kBlock : Fmt<TD>::kBlock);
         const uint8_t *rows = (is_shared ? a.shared : a.experts + (uint64_t)a.ids[wave] * a.stride) + (uint64_t)row0 * row_bytes;
-        uint8_t *mine = raw_rows + wave * 8u * FB * kMaxBlock;
-        wave_stage(mine, rows, 8u * row_bytes, lane);          // 8 rows x FB blocks of 66 / 110 / 210 bytes: a multiple of 16
+        wave_stage(mine, rows, 8u * row_bytes, lane);          // 8 rows x FB blocks of 56 .. 210 bytes: a multiple of 16
+    }
+    if constexpr (kGridBytes != 0u) {
+#pragma unroll
+        for (uint32_t i = 0; i < 2u; ++i)
+            if (tid + i * NW * 64u < kGridBytes / 16u) reinterpret_cast<uint4 *>(cb)[tid + i * NW * 64u] = cbv[i];
+        __syncthreads();
+    }
+    if (wave < n_slot) {
         float tot[2] = {0.0f, 0.0f};
         for (uint32_t G = blk; G < FG; G += 16u) {
             float av[32];
@@ -1026,7 +1185,7 @@ __global__ __launch_bounds__(NW * 64) void down_combine_raw_kernel(DownRawArgs a
 #pragma unroll
             for (int q = 0; q < 2; ++q) {
                 const uint8_t *row = mine + (4u * q + j) * row_bytes;
-                tot[q] += is_shared ? chunk_dot<TS>(row, G, av) : chunk_dot<TD>(row, G, av);
+                tot[q] += is_shared ? chunk_dot<TS>(row, G, av) : chunk_dot<TD>(row, G, av, cb);
             }
         }
         const float r = quad_column_reduce<2>(tot, lane);
@@ -1059,15 +1218,19 @@ static hipError_t launch_down_raw_shared(uint32_t ts, const DownRawArgs &a, uint
 
 hipError_t launch_down_combine_raw(uint32_t down_type, uint32_t shared_down_type, const void *experts, uint64_t stride, const void *shared,
                                    const uint32_t *ids, const float *weights, const float *scalar, const void *act_h, const void *act_l,
-                                   const int *act_exp, float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, hipStream_t s, uint32_t ntok) {
+                                   const int *act_exp, float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, hipStream_t s, uint32_t ntok,
+                                   const int8_t *grid) {
     if (!hidden || hidden % 8u || !ffn || ffn % 256u || top_k + 1u > (uint32_t)kWaves || !ntok || ntok > 65535u) return hipErrorInvalidValue;
+    if ((down_type == T_IQ2_XS || down_type == T_IQ1_M) && !grid) return hipErrorInvalidValue;
     const DownRawArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(shared), ids, weights, scalar,
                         static_cast<const _Float16 *>(act_h), static_cast<const _Float16 *>(act_l), act_exp, out, hidden, ffn, top_k,
-                        block_context().resid_a, block_context().resid_b};
+                        block_context().resid_a, block_context().resid_b, grid};
     switch (down_type) {
         case T_IQ2_XXS: return launch_down_raw_shared<T_IQ2_XXS>(shared_down_type, a, ntok, s);
         case T_IQ3_S: return launch_down_raw_shared<T_IQ3_S>(shared_down_type, a, ntok, s);
         case T_Q6_K: return launch_down_raw_shared<T_Q6_K>(shared_down_type, a, ntok, s);
+        case T_IQ2_XS: return launch_down_raw_shared<T_IQ2_XS>(shared_down_type, a, ntok, s);
+        case T_IQ1_M: return launch_down_raw_shared<T_IQ1_M>(shared_down_type, a, ntok, s);
         default: return hipErrorInvalidValue;
     }
 }
@@ -1522,31 +1685,42 @@ static hipError_t launch_gateup_batch_kernel(const BatchArgs &a, uint32_t n_grou
 hipError_t launch_gateup_select(const void *experts, uint64_t stride, const void *shared, const void *shared_q6k, const float *x,
                                 const float *shared_gu, const float *logits, const uint32_t *ids_in, uint32_t *ids_out, float *weights_out,
                                 float *scalar_out, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l, int *act_exp,
-                                uint32_t hidden, uint32_t ffn, uint32_t n_expert, uint32_t top_k, hipStream_t s, uint32_t ntok) {
+                                uint32_t hidden, uint32_t ffn, uint32_t n_expert, uint32_t top_k, hipStream_t s, uint32_t ntok,
+                                uint32_t gate_up_type, const int8_t *grid) {
     if (!fused_iq2_supported(hidden, ffn) || (!shared && !shared_gu && (!shared_q6k || !x)) || !ntok || ntok > 64u) return hipErrorInvalidValue;
-    GateUpArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(shared), static_cast<const uint8_t *>(shared_q6k), x,
+    const bool codebook = gate_up_type == T_IQ2_XS || gate_up_type == T_IQ1_M;
+    if ((gate_up_type != T_IQ2_XXS && !codebook) || (codebook && (!grid || shared))) return hipErrorInvalidValue;
+    GateUpArgs a{static_cast<const uint8_t *>(experts), stride, grid, static_cast<const uint8_t *>(shared), static_cast<const uint8_t *>(shared_q6k), x,
                  shared_gu, logits, ids_in, ids_out, weights_out, scalar_out, static_cast<const _Float16 *>(xh), static_cast<const _Float16 *>(xl),
                  xexp, static_cast<_Float16 *>(act_h), static_cast<_Float16 *>(act_l), act_exp, hidden, ffn, n_expert, top_k};
-    const dim3 grid(ffn / 32u, top_k + 1u, ntok);
+    const dim3 grid_dim(ffn / 32u, top_k + 1u, ntok);
     const size_t dyn = shared || shared_gu ? 0u : (size_t)64u * (hidden / 256u) * 210u + (size_t)(hidden + hidden / 32u + hidden / 16u) * 4u;   // raw Q6_K rows of one unit of the shared expert, x, sums of 16 x
-#define REDHIP_GUS(NKC)                                                                                                                \
+    const size_t dyn_max = gate_up_type == T_IQ1_M ? 120u * 1024u : 144u * 1024u;      // beside the static decode table (32 KB for IQ1_M)
+#define REDHIP_GUS(NKC, FMT)                                                                                                           \
     do {                                                                                                                               \
         static bool attr = false;                                                                                                       \
         if (dyn && !attr) {                                                                                                             \
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gateup_select_kernel<NKC>), hipFuncAttributeMaxDynamicSharedMemorySize, 144 * 1024); \
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(gateup_select_kernel<NKC, FMT>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn_max); \
             if (e != hipSuccess) return e;                                                                                              \
             attr = true;                                                                                                                \
         }                                                                                                                               \
-        REDHIP_LAUNCH(gateup_select_kernel<NKC>, grid, dim3(kWaves * 64), dyn, s, a);                                                   \
+        REDHIP_LAUNCH((gateup_select_kernel<NKC, FMT>), grid_dim, dim3(kWaves * 64), dyn, s, a);                                          \
     } while (0)
-    if (dyn > 144u * 1024u) return hipErrorInvalidValue;
+#define REDHIP_GUS_FMT(NKC)                                                                                                            \
+    do {                                                                                                                               \
+        if (gate_up_type == T_IQ2_XS) REDHIP_GUS(NKC, 1);                                                                               \
+        else if (gate_up_type == T_IQ1_M) REDHIP_GUS(NKC, 2);                                                                           \
+        else REDHIP_GUS(NKC, 0);                                                                                                        \
+    } while (0)
+    if (dyn > dyn_max) return hipErrorInvalidValue;
     switch (hidden / 512u) {
-        case 1: REDHIP_GUS(1); break;
-        case 2: REDHIP_GUS(2); break;
-        case 4: REDHIP_GUS(4); break;
-        case 8: REDHIP_GUS(8); break;
+        case 1: REDHIP_GUS_FMT(1); break;
+        case 2: REDHIP_GUS_FMT(2); break;
+        case 4: REDHIP_GUS_FMT(4); break;
+        case 8: REDHIP_GUS_FMT(8); break;
         default: return hipErrorInvalidValue;
     }
+#undef REDHIP_GUS_FMT
 #undef REDHIP_GUS
     return hipGetLastError();
 }

@@ -24,6 +24,7 @@ inline bool pool_quant_supported(uint32_t t) { return pool_block_bytes(t) != 0u;
 // tables before every launch; callers whose tables differ must not run at the same time
 hipError_t set_caller_grids(const int8_t *iq2_xs, const int8_t *iq1_m, const void *owner = nullptr);
 void forget_caller_grids(const void *owner);
+const int8_t *caller_grid_device(uint32_t type);      // device address of the process's codebook of IQ2_XS / IQ1_M, nullptr for other types
 bool caller_grid_present(uint32_t type);       // true for the formats that carry their own tables
 inline uint64_t row_bytes(uint32_t t, uint32_t ncols) {
     if (!ncols) return 0;
@@ -164,6 +165,14 @@ inline bool fused_iq2_supported(uint32_t hidden, uint32_t ffn) {
 // `count` matrices, raw_stride / packed_stride bytes apart; packed = qs [nrows][K/32] uint2 then ds [nrows][K/256] fp16
 hipError_t launch_repack_iq2xxs(const void *raw, uint64_t raw_stride, uint32_t count, uint32_t nrows, uint32_t K, bool col_major,
                                 void *packed, uint64_t packed_stride, hipStream_t s);
+// gate / up matrices of IQ2_XXS, IQ2_XS or IQ1_M rows into the streams of the one-token gate/up kernel
+hipError_t launch_repack_gateup(uint32_t type, const void *raw, uint64_t raw_stride, uint32_t count, uint32_t nrows, uint32_t K,
+                                void *packed, uint64_t packed_stride, hipStream_t s);
+// bytes of one such matrix: 8 per 32 weights + 2 per 256, IQ2_XS one more per 32
+inline uint64_t packed_matrix_bytes(uint32_t type, uint32_t nrows, uint32_t K) {
+    return (uint64_t)nrows * ((uint64_t)(K / 32u) * (type == T_IQ2_XS ? 9u : 8u) + (uint64_t)(K / 256u) * 2u);
+}
+hipError_t launch_dequant_packed(uint32_t type, const void *packed, uint32_t nrows, uint32_t K, const int8_t *grid, float *out, hipStream_t s);
 hipError_t launch_dequant_packed_iq2xxs(const void *packed, uint32_t nrows, uint32_t K, bool col_major, float *out, hipStream_t s);
 
 // logits [ntok][n_expert + 1] (entry n_expert = gate_inp . x) and the fp16 split of x: xh, xl [ntok][hidden], xexp [ntok]
@@ -192,11 +201,13 @@ hipError_t launch_batch_packed(const void *experts, uint64_t stride, const void 
 hipError_t launch_gateup_select(const void *experts, uint64_t stride, const void *shared, const void *shared_q6k, const float *x,
                                 const float *shared_gu, const float *logits, const uint32_t *ids_in, uint32_t *ids_out, float *weights_out,
                                 float *scalar_out, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l, int *act_exp,
-                                uint32_t hidden, uint32_t ffn, uint32_t n_expert, uint32_t top_k, hipStream_t s, uint32_t ntok = 1u);
+                                uint32_t hidden, uint32_t ffn, uint32_t n_expert, uint32_t top_k, hipStream_t s, uint32_t ntok = 1u,
+                                uint32_t gate_up_type = T_IQ2_XXS, const int8_t *grid = nullptr);
 // down + weighted combine for layouts whose down matrices are raw GGUF rows of any supported type
 hipError_t launch_down_combine_raw(uint32_t down_type, uint32_t shared_down_type, const void *experts, uint64_t stride, const void *shared,
                                    const uint32_t *ids, const float *weights, const float *scalar, const void *act_h, const void *act_l,
-                                   const int *act_exp, float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, hipStream_t s, uint32_t ntok = 1u);
+                                   const int *act_exp, float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, hipStream_t s, uint32_t ntok = 1u,
+                                   const int8_t *grid = nullptr);
 // single token: out[r] = sum_k weights[k] * down_{ids[k]}[r] . act[k] + scalar * shared_down[r] . act[top_k], k in order
 hipError_t launch_down_combine(const void *experts, uint64_t stride, const void *shared, const uint32_t *ids, const float *weights,
                                const float *scalar, const void *act_h, const void *act_l, const int *act_exp, float *out,

@@ -23,8 +23,8 @@ static inline uint32_t padded_floats(uint32_t n) { return n + (n >> 5); }
 
 // The reference hands these codebooks to its kernels as arguments (native/redmetal_ffn.m:223-227); here they live in
 // device memory of this translation unit, uploaded by the pool / one-shot surfaces before they launch.
-__device__ int8_t g_iq2xs_grid[512 * 8];
-__device__ int8_t g_iq1m_grid[2048 * 8];
+__device__ __attribute__((aligned(16))) int8_t g_iq2xs_grid[512 * 8];
+__device__ __attribute__((aligned(16))) int8_t g_iq1m_grid[2048 * 8];
 
 static std::mutex g_grid_mu;
 static const void *g_grid_owner = nullptr;      // whose tables the device holds; nullptr: nobody's in particular
@@ -51,49 +51,15 @@ void forget_caller_grids(const void *owner) {
     if (g_grid_owner == owner) g_grid_owner = nullptr;
 }
 
-template <> struct Fmt<T_IQ2_XS> { static constexpr uint32_t kBlock = 74u; };
-template <> struct Fmt<T_IQ1_M> { static constexpr uint32_t kBlock = 56u; };
+template <> __device__ __forceinline__ void decode32<T_IQ2_XS>(const uint8_t *row, uint32_t chunk, float *w) { decode32_cb<T_IQ2_XS>(row, chunk, w, g_iq2xs_grid); }
+template <> __device__ __forceinline__ void decode32<T_IQ1_M>(const uint8_t *row, uint32_t chunk, float *w) { decode32_cb<T_IQ1_M>(row, chunk, w, g_iq1m_grid); }
 
-// IQ2_XS, native/redlite_native_reference.c:116-142: block = f16 d, 32 x u16 (9-bit codebook index + 7 sign bits, the
-// eighth sign is their parity), 8 bytes of 4-bit scales (one per 16 weights); weight = d * (0.5 + scale) * 0.25 * entry * sign
-template <> __device__ __forceinline__ void decode32<T_IQ2_XS>(const uint8_t *row, uint32_t chunk, float *w) {
-    const uint8_t *bp = row + (size_t)(chunk >> 3) * 74u;
-    const uint32_t cb = chunk & 7u;
-    const float d = half_bits_to_f32(ld_u16(bp));
-    const uint32_t sc = bp[66u + cb];
-    const float db0 = d * (0.5f + (float)(sc & 15u)) * 0.25f, db1 = d * (0.5f + (float)(sc >> 4)) * 0.25f;
-#pragma unroll
-    for (uint32_t k = 0; k < 4u; ++k) {
-        const uint32_t q = ld_u16(bp + 2u + 2u * (4u * cb + k));
-        const int8_t *entry = g_iq2xs_grid + (q & 511u) * 8u;
-        const uint32_t s7 = (q >> 9) & 127u, s8 = s7 | ((__popc(s7) & 1u) << 7);
-        const float db = k < 2u ? db0 : db1;
-#pragma unroll
-        for (uint32_t j = 0; j < 8u; ++j) w[8u * k + j] = apply_sign(db * (float)entry[j], (s8 >> j) & 1u);
-    }
-}
-
-// IQ1_M, native/redlite_native_reference.c:149-170: block = 32 index bytes, 16 bytes of nibbles (3 high index bits + the
-// sign of the 1/8 offset), four u16 with 3-bit scales (one per 16 weights) and the f16 d spread over their top nibbles;
-// weight = d * (2 * scale + 1) * (entry + or - 0.125), entry in {-1, 0, 1}
-template <> __device__ __forceinline__ void decode32<T_IQ1_M>(const uint8_t *row, uint32_t chunk, float *w) {
-    const uint8_t *bp = row + (size_t)(chunk >> 3) * 56u;
-    const uint32_t cb = chunk & 7u;
-    uint32_t sc[4];
-#pragma unroll
-    for (uint32_t i = 0; i < 4u; ++i) sc[i] = ld_u16(bp + 48u + 2u * i);
-    const float d = half_bits_to_f32((sc[0] >> 12) | ((sc[1] >> 8) & 0x00f0u) | ((sc[2] >> 4) & 0x0f00u) | (sc[3] & 0xf000u));
-#pragma unroll
-    for (uint32_t k = 0; k < 4u; ++k) {
-        const uint32_t group = 4u * cb + k;
-        const uint32_t nibble = ((uint32_t)bp[32u + (group >> 1)] >> (4u * (group & 1u))) & 15u;
-        const int8_t *entry = g_iq1m_grid + ((uint32_t)bp[group] | ((nibble & 7u) << 8)) * 8u;
-        const float delta = (nibble & 8u) ? -0.125f : 0.125f;
-        const uint32_t si = group >> 1;
-        const float dl = d * (float)(2u * ((sc[si >> 2] >> (3u * (si & 3u))) & 7u) + 1u);
-#pragma unroll
-        for (uint32_t j = 0; j < 8u; ++j) w[8u * k + j] = dl * ((float)entry[j] + delta);
-    }
+// device address of the codebook the process holds for `type` (nullptr: the type has none)
+const int8_t *caller_grid_device(uint32_t type) {
+    void *p = nullptr;
+    if (type == T_IQ2_XS) { if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_iq2xs_grid)) != hipSuccess) return nullptr; }
+    else if (type == T_IQ1_M) { if (hipGetSymbolAddress(&p, HIP_SYMBOL(g_iq1m_grid)) != hipSuccess) return nullptr; }
+    return static_cast<const int8_t *>(p);
 }
 
 template <uint32_t T>

@@ -46,6 +46,8 @@ struct Moe {
     redhip_moe_config cfg;
     uint32_t gu_type, dn_type, sh_gu_type, sh_dn_type;
     uint64_t gate_bytes, down_bytes, expert_stride;          // routed expert
+    uint64_t pk_gate_bytes = 0;                              // one gate / up matrix in the packed streams of the one-token kernel
+    const int8_t *gu_grid = nullptr, *dn_grid = nullptr;     // device copies of the caller's codebooks (IQ2_XS / IQ1_M matrices)
     uint64_t sh_gate_bytes, sh_down_bytes;                   // shared expert
     uint64_t router_bytes;
     uint64_t resident = 0;
@@ -57,8 +59,8 @@ struct Moe {
     uint8_t *ws = nullptr;
     // single-token fused path (all matrices IQ2_XXS, shapes the fused kernel tiles)
     bool fused = false;
-    // mixed-precision layouts (gate/up IQ2_XXS, other matrices of other types): the routed gate/up matrices are packed
-    // for the MFMA gate/up kernel, the down matrices stay raw GGUF rows; one token at a time
+    // mixed-precision layouts (gate/up IQ2_XXS, IQ2_XS or IQ1_M, other matrices of other types): the routed gate/up matrices
+    // are packed for the MFMA gate/up kernel, the down matrices stay raw GGUF rows; one token at a time
     bool mixed = false;
     uint64_t packed_stride = 0;              // bytes between experts in `packed`
     bool packed_gu() const { return fused || mixed; }
@@ -72,7 +74,7 @@ struct Moe {
     bool tiled_router(uint32_t ntok) const {
         return packed_gu() && ntok >= 16u && (cfg.router_type == T_F32 || mixed);
     }
-    bool tiles_resident() const { return packed_gu() && cfg.max_tokens > 8u && cfg.ffn <= 512u && cfg.hidden / 512u <= 4u; }
+    bool tiles_resident() const { return packed_gu() && gu_type == T_IQ2_XXS && cfg.max_tokens > 8u && cfg.ffn <= 512u && cfg.hidden / 512u <= 4u; }
     // a chunk on a mixed layout: the routed gate/up matrices (packed IQ2_XXS) run on the prefill tiles, the rest on raw rows
     bool mixed_chunk(uint32_t ntok) const { return mixed && ntok > 8u && tiles_resident(); }
     uint64_t tiled_down_stride() const { return ((uint64_t)cfg.hidden * (cfg.ffn / 32u) * 16u + (uint64_t)cfg.hidden * (cfg.ffn / 256u) * 2u + 255u) & ~255ull; }
@@ -215,7 +217,7 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
         HIP_OK(launch_gateup_select(L.packed, m->packed_stride, L.shared_packed, L.shared, x, select_here && m->shared_gu_ready ? m->act : nullptr,
                                     select_here ? m->logits : nullptr, ids, m->ids,
                                     m->weights, m->scalar, m->xh, m->xl, m->xexp, m->act_h, m->act_l, m->act_exp, c.hidden, c.ffn, c.n_expert,
-                                    c.top_k, s, ntok), "gate/up launch");      // ntok > 1: a small batch on a mixed layout, one grid layer per token
+                                    c.top_k, s, ntok, m->gu_type, m->gu_grid), "gate/up launch");      // ntok > 1: a small batch on a mixed layout, one grid layer per token
         prof_set_stage(ST_DOWN_COMBINE);
         if (m->fused)
             HIP_OK(launch_down_combine(L.packed, m->expert_stride, L.shared_packed, select_here ? m->ids : ids, select_here ? m->weights : weights,
@@ -223,7 +225,7 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
         else
             HIP_OK(launch_down_combine_raw(m->dn_type, m->sh_dn_type, L.experts + 2u * m->gate_bytes, m->expert_stride, L.shared + 2u * m->sh_gate_bytes,
                                            select_here ? m->ids : ids, select_here ? m->weights : weights, m->scalar, m->act_h, m->act_l,
-                                           m->act_exp, out, c.hidden, c.ffn, c.top_k, s, ntok), "down/combine launch");
+                                           m->act_exp, out, c.hidden, c.ffn, c.top_k, s, ntok, m->dn_grid), "down/combine launch");
         prof_set_stage(ST_OTHER);
         return 1;
     }
@@ -279,9 +281,16 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
     m->layers.resize(c.n_layer);
     m->fused = gu == T_IQ2_XXS && dn == T_IQ2_XXS && sgu == T_IQ2_XXS && sdn == T_IQ2_XXS && fused_iq2_supported(c.hidden, c.ffn);
     // (the raw-row down kernel stages 8 rows per slot in LDS: keep that within the default 64 KB)
-    m->mixed = !m->fused && gu == T_IQ2_XXS && (sgu == T_IQ2_XXS || sgu == T_Q6_K) && fused_iq2_supported(c.hidden, c.ffn) &&
-               (size_t)(c.top_k + 1u) * 8u * (c.ffn / 256u) * 210u <= 64u * 1024u && (sgu != T_Q6_K || (size_t)64u * (c.hidden / 256u) * 210u + (size_t)(c.hidden + c.hidden / 32u + c.hidden / 16u) * 4u <= 144u * 1024u);
-    m->packed_stride = m->fused ? m->expert_stride : align256(2u * m->gate_bytes);
+    // IQ2_XS / IQ1_M gate/up matrices have a packed form of their own (a shared expert beside them is Q6_K; the gate/up kernel keeps
+    // their fp16 codebook in LDS next to the staged Q6_K rows: 32 KB for IQ1_M)
+    const bool gu_codebook = gu == T_IQ2_XS || gu == T_IQ1_M;
+    m->mixed = !m->fused && (gu == T_IQ2_XXS || gu_codebook) && (sgu == T_Q6_K || (sgu == T_IQ2_XXS && !gu_codebook)) && fused_iq2_supported(c.hidden, c.ffn) &&
+               (size_t)(c.top_k + 1u) * 8u * (c.ffn / 256u) * 210u + (dn == T_IQ1_M ? 17u * 1024u : dn == T_IQ2_XS ? 5u * 1024u : 0u) <= 64u * 1024u &&
+               (sgu != T_Q6_K || (size_t)64u * (c.hidden / 256u) * 210u + (size_t)(c.hidden + c.hidden / 32u + c.hidden / 16u) * 4u <= (gu == T_IQ1_M ? 120u : 144u) * 1024u);
+    m->pk_gate_bytes = packed_matrix_bytes(gu, c.ffn, c.hidden);
+    m->packed_stride = m->fused ? m->expert_stride : align256(2u * m->pk_gate_bytes);
+    m->gu_grid = caller_grid_device(gu);
+    m->dn_grid = caller_grid_device(dn);
     bool ok = true;
     for (uint32_t l = 0; l < c.n_layer && ok; ++l) {
         Layer &L = m->layers[l];
@@ -477,8 +486,8 @@ static int stage_and_pack(Moe *m, uint32_t layer, uint32_t first, uint32_t count
     if (m->packed_gu()) {
         const redhip_moe_config &c = m->cfg;
         uint8_t *pk = m->layers[layer].packed + (uint64_t)first * m->packed_stride;
-        HIP_OK(launch_repack_iq2xxs(dst, m->expert_stride, count, c.ffn, c.hidden, false, pk, m->packed_stride, nullptr), "expert gate repack");
-        HIP_OK(launch_repack_iq2xxs(dst + m->gate_bytes, m->expert_stride, count, c.ffn, c.hidden, false, pk + m->gate_bytes, m->packed_stride, nullptr), "expert up repack");
+        HIP_OK(launch_repack_gateup(m->gu_type, dst, m->expert_stride, count, c.ffn, c.hidden, pk, m->packed_stride, nullptr), "expert gate repack");
+        HIP_OK(launch_repack_gateup(m->gu_type, dst + m->gate_bytes, m->expert_stride, count, c.ffn, c.hidden, pk + m->pk_gate_bytes, m->packed_stride, nullptr), "expert up repack");
         if (m->fused)
             HIP_OK(launch_repack_iq2xxs(dst + 2u * m->gate_bytes, m->expert_stride, count, c.hidden, c.ffn, false, pk + 2u * m->gate_bytes, m->packed_stride, nullptr), "expert down repack");
         if (m->layers[layer].tiled) {
@@ -674,8 +683,8 @@ int redhip_moe_dequant_resident(redhip_moe_t h, uint32_t layer, uint32_t expert,
     const bool sh = expert == c.n_expert;
     if (m->fused || (m->mixed && which < 2u && (!sh || L.shared_packed))) {        // the layout the MFMA kernels read
         const uint8_t *pk = sh ? L.shared_packed : L.packed + (uint64_t)expert * m->packed_stride;
-        const uint64_t gbytes = m->gate_bytes;
-        if (which < 2u) HIP_OK(launch_dequant_packed_iq2xxs(pk + which * gbytes, c.ffn, c.hidden, false, out_dev, s), "packed gate/up dequant");
+        const uint64_t gbytes = m->pk_gate_bytes;
+        if (which < 2u) HIP_OK(launch_dequant_packed(m->gu_type, pk + which * gbytes, c.ffn, c.hidden, m->gu_grid, out_dev, s), "packed gate/up dequant");
         else HIP_OK(launch_dequant_packed_iq2xxs(pk + 2u * gbytes, c.hidden, c.ffn, false, out_dev, s), "packed down dequant");
         return 1;
     }
