@@ -1135,11 +1135,10 @@ __global__ __launch_bounds__(NW * 64) void down_combine_raw_kernel(DownRawArgs a
     __shared__ __attribute__((aligned(16))) int8_t cb[kGridBytes ? kGridBytes : 16u];
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
     const uint32_t F = a.ffn, FG = F / 32u, FB = F / 256u, n_slot = a.top_k + 1u;
-    uint4 cbv[2] = {};                                 // requested first, stored once the wave's rows are on their way
+    uint4 cb0 = make_uint4(0u, 0u, 0u, 0u), cb1 = cb0;   // requested first, stored once the wave's rows are on their way
     if constexpr (kGridBytes != 0u) {
-#pragma unroll
-        for (uint32_t i = 0; i < 2u; ++i)
-            if (tid + i * NW * 64u < kGridBytes / 16u) cbv[i] = reinterpret_cast<const uint4 *>(a.grid)[tid + i * NW * 64u];
+        if (tid < kGridBytes / 16u) cb0 = reinterpret_cast<const uint4 *>(a.grid)[tid];
+        if (tid + NW * 64u < kGridBytes / 16u) cb1 = reinterpret_cast<const uint4 *>(a.grid)[tid + NW * 64u];
     }
     if (const uint32_t tok = blockIdx.y) {             // several tokens in one launch
         const uint64_t t = tok;
@@ -1162,9 +1161,8 @@ __global__ __launch_bounds__(NW * 64) void down_combine_raw_kernel(DownRawArgs a
         wave_stage(mine, rows, 8u * row_bytes, lane);          // 8 rows x FB blocks of 56 .. 210 bytes: a multiple of 16
     }
     if constexpr (kGridBytes != 0u) {
-#pragma unroll
-        for (uint32_t i = 0; i < 2u; ++i)
-            if (tid + i * NW * 64u < kGridBytes / 16u) reinterpret_cast<uint4 *>(cb)[tid + i * NW * 64u] = cbv[i];
+        if (tid < kGridBytes / 16u) reinterpret_cast<uint4 *>(cb)[tid] = cb0;
+        if (tid + NW * 64u < kGridBytes / 16u) reinterpret_cast<uint4 *>(cb)[tid + NW * 64u] = cb1;
         __syncthreads();
     }
     if (wave < n_slot) {
