@@ -460,7 +460,7 @@ __global__ __launch_bounds__(256) void router_quant_kernel(const uint8_t *w, Rou
 hipError_t launch_router_gemv(uint32_t router_type, const void *w, const float *x, const float *gate_inp, uint32_t ntok, uint32_t hidden,
                               uint32_t n_expert, float *logits, void *xh, void *xl, int *xexp, const void *sh_q6k, float *sh_gu, uint32_t ffn,
                               hipStream_t s, const float *sh_dense) {
-    if (!ntok || !hidden || hidden % 256u || !n_expert || n_expert > 1024u) return hipErrorInvalidValue;
+    if (!ntok || !hidden || hidden % 256u || (!n_expert && !sh_dense) || n_expert > 1024u) return hipErrorInvalidValue;      // n_expert 0: only the shared expert's rows
     const bool with_shared = sh_q6k && sh_gu && router_type == T_Q6_K && ntok <= 8u && ffn % 4u == 0u;      // sh_gu: [ntok][2 * ffn]
     const BlockContext &bc = block_context();
     if (bc.branch && (!bc.norm_w || !bc.xn_out)) return hipErrorInvalidValue;
@@ -1233,6 +1233,261 @@ hipError_t launch_down_combine_raw(uint32_t down_type, uint32_t shared_down_type
     }
 }
 
+// ---------------------------------------------------------------- IQ3_S down matrices of mixed layouts on the matrix units
+//
+// "Word-packed IQ3_S" (built at upload): one 32-bit word per eight weights - two 9-bit grid indices (the qh bit folded in) in bits 0-8
+// and 9-17, the eight sign bits in 18-25, the group's scale nibble in 26-29 - as one uint4 per 32 weights, [row][K/32], followed by
+// d as fp16 [row][K/256]. 130 bytes per 256 weights instead of 110, every load naturally aligned. A weight is
+// sign * grid byte * (2 * nibble + 1) * d: the four grid bytes of an entry come as exact fp16 values from an LDS table (512 x 8 bytes),
+// the signs are placed as in the IQ2_XXS kernels, and the same 4x4x4 MFMA multiplies them with the fp16 halves of the activations.
+constexpr uint32_t kIq3TableBytes = 512u * 8u;
+
+__global__ void repack_iq3s_words_kernel(const uint8_t *raw0, uint64_t raw_stride, uint32_t nrows, uint32_t K, uint8_t *packed0, uint64_t packed_stride) {
+    const uint32_t groups = K / 32u, blocks = K / 256u;
+    const uint8_t *raw = raw0 + (uint64_t)blockIdx.y * raw_stride;
+    uint8_t *pk = packed0 + (uint64_t)blockIdx.y * packed_stride;
+    const uint64_t gid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= (uint64_t)nrows * groups) return;
+    const uint32_t r = (uint32_t)(gid / groups), g = (uint32_t)(gid % groups), sub = g & 7u;
+    const uint8_t *bp = raw + ((uint64_t)r * blocks + (g >> 3)) * 110u;
+    const uint32_t nib = ((uint32_t)bp[106u + (sub >> 1)] >> (4u * (sub & 1u))) & 15u, qh = bp[66u + sub];
+    uint32_t w[4];
+    for (uint32_t l = 0; l < 4u; ++l) {
+        const uint32_t ia = (uint32_t)bp[2u + 8u * sub + 2u * l] | ((qh << (8u - 2u * l)) & 256u);
+        const uint32_t ib = (uint32_t)bp[3u + 8u * sub + 2u * l] | ((qh << (7u - 2u * l)) & 256u);
+        w[l] = ia | (ib << 9) | ((uint32_t)bp[74u + 4u * sub + l] << 18) | (nib << 26);
+    }
+    reinterpret_cast<uint4 *>(pk)[gid] = make_uint4(w[0], w[1], w[2], w[3]);
+    if (sub == 0u) reinterpret_cast<uint16_t *>(pk + (uint64_t)nrows * groups * 16u)[(uint64_t)r * blocks + (g >> 3)] = (uint16_t)ld_u16(bp);
+}
+
+hipError_t launch_repack_iq3s_words(const void *raw, uint64_t raw_stride, uint32_t count, uint32_t nrows, uint32_t K, void *packed, uint64_t packed_stride, hipStream_t s) {
+    if (!nrows || !K || K % 256u || !count || count > 65535u) return hipErrorInvalidValue;
+    const uint64_t total = (uint64_t)nrows * (K / 32u);
+    REDHIP_LAUNCH(repack_iq3s_words_kernel, dim3((uint32_t)((total + 255u) / 256u), count), dim3(256), 0, s, static_cast<const uint8_t *>(raw), raw_stride, nrows, K,
+                  static_cast<uint8_t *>(packed), packed_stride);
+    return hipGetLastError();
+}
+
+// parity tap: f32 dequantisation from the words, arithmetic as decode32<T_IQ3_S>
+__global__ void dequant_iq3s_words_kernel(const uint8_t *pk, uint32_t nrows, uint32_t K, float *out) {
+    const uint32_t groups = K / 32u, blocks = K / 256u;
+    const uint64_t gid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    if (gid >= (uint64_t)nrows * groups) return;
+    const uint32_t r = (uint32_t)(gid / groups), g = (uint32_t)(gid % groups);
+    const uint4 v = reinterpret_cast<const uint4 *>(pk)[gid];
+    const float d = half_bits_to_f32(reinterpret_cast<const uint16_t *>(pk + (uint64_t)nrows * groups * 16u)[(uint64_t)r * blocks + (g >> 3)]);
+    const float db = d * (float)(1u + 2u * ((v.x >> 26) & 15u));
+    const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
+    float *o = out + (uint64_t)r * K + 32u * g;
+    for (uint32_t l = 0; l < 4u; ++l) {
+        const uint32_t wa = redhip_iq3s_grid[w4[l] & 511u], wb = redhip_iq3s_grid[(w4[l] >> 9) & 511u], sg = (w4[l] >> 18) & 255u;
+        for (uint32_t j = 0; j < 4u; ++j) {
+            o[8u * l + j] = apply_sign(db * (float)((wa >> (8u * j)) & 255u), (sg >> j) & 1u);
+            o[8u * l + 4u + j] = apply_sign(db * (float)((wb >> (8u * j)) & 255u), (sg >> (4u + j)) & 1u);
+        }
+    }
+}
+
+hipError_t launch_dequant_iq3s_words(const void *packed, uint32_t nrows, uint32_t K, float *out, hipStream_t s) {
+    if (!nrows || !K || K % 256u) return hipErrorInvalidValue;
+    const uint64_t total = (uint64_t)nrows * (K / 32u);
+    REDHIP_LAUNCH(dequant_iq3s_words_kernel, dim3((uint32_t)((total + 255u) / 256u)), dim3(256), 0, s, static_cast<const uint8_t *>(packed), nrows, K, out);
+    return hipGetLastError();
+}
+
+// LDS table: the four bytes of every grid entry as fp16; built by the first 512 lanes of a workgroup
+__device__ __forceinline__ void build_iq3s_quads(uint8_t *lds, uint32_t tid) {
+    if (tid < 512u) {
+        const uint32_t e = redhip_iq3s_grid[tid];
+        uint32_t w2[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const _Float16 lo = (_Float16)(float)((e >> (16 * i)) & 255u), hi = (_Float16)(float)((e >> (16 * i + 8)) & 255u);
+            w2[i] = (uint32_t)__builtin_bit_cast(uint16_t, lo) | ((uint32_t)__builtin_bit_cast(uint16_t, hi) << 16);
+        }
+        *reinterpret_cast<uint2 *>(lds + (size_t)tid * 8u) = make_uint2(w2[0], w2[1]);
+    }
+}
+
+// 32 weights (one uint4 of words) against an activation operand that carries one token (rows 0, 1 = hi, lo) or two (rows 2, 3 the
+// second): va = first token's product, vb = the second's; scale nibble applied, d is not.
+__device__ __forceinline__ void iq3s_group_dot(uint4 q, const half4_t *ax, const uint8_t *lds, float &va, float &vb) {
+    const uint32_t w4[4] = {q.x, q.y, q.z, q.w};
+    float4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (uint32_t l = 0; l < 4u; ++l) {
+        const uint2 ma = *reinterpret_cast<const uint2 *>(lds + ((w4[l] & 511u) << 3)), mb = *reinterpret_cast<const uint2 *>(lds + (((w4[l] >> 9) & 511u) << 3));
+        const uint32_t s8s = ((w4[l] >> 18) & 255u) << 8;          // sign bit k of the eight at bit 8 + k, as place_signs takes them
+        WeightQuad b0, b1;
+        b0.u[0] = (__umul24(s8s, (1u << 7) | (1u << 22)) & 0x80008000u) | ma.x;
+        b0.u[1] = (__umul24(s8s, (1u << 5) | (1u << 20)) & 0x80008000u) | ma.y;
+        b1.u[0] = (__umul24(s8s, (1u << 3) | (1u << 18)) & 0x80008000u) | mb.x;
+        b1.u[1] = (__umul24(s8s, (1u << 1) | (1u << 16)) & 0x80008000u) | mb.y;
+        acc = __builtin_amdgcn_mfma_f32_4x4x4f16(ax[2u * l], b0.h, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_4x4x4f16(ax[2u * l + 1u], b1.h, acc, 0, 0, 0);
+    }
+    const float sc = (float)(2u * ((q.x >> 26) & 15u) + 1u);
+    va = (acc[0] + acc[1] * 4.8828125e-4f) * sc;
+    vb = (acc[2] + acc[3] * 4.8828125e-4f) * sc;
+}
+
+// One row of a dense f32 matrix against an activation vector kept as fp16 halves + one exponent per 32 columns: the LPR lanes that
+// share a row take every LPR-th float4 and meet by butterfly adds. Returns the row's product in every one of those lanes.
+template <uint32_t LPR>
+__device__ __forceinline__ float dense_row_dot(const float *row, const _Float16 *ah, const _Float16 *al, const int *aexp, uint32_t F, uint32_t part) {
+    float acc = 0.0f;
+    for (uint32_t c0 = part; c0 < F / 4u; c0 += 8u * LPR) {      // eight float4 per lane and round, all requested before the first is used
+        float4 w[8];
+        uint2 hv[8], lv[8];
+        int ev[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t cr = c0 + LPR * (uint32_t)i, c4 = cr < F / 4u ? cr : F / 4u - 1u;
+            w[i] = reinterpret_cast<const float4 *>(row)[c4];
+            if (cr >= F / 4u) w[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            hv[i] = reinterpret_cast<const uint2 *>(ah)[c4];
+            lv[i] = reinterpret_cast<const uint2 *>(al)[c4];
+            ev[i] = aexp[c4 >> 3];
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            union { uint2 u; _Float16 h[4]; } hh, ll;
+            hh.u = hv[i];
+            ll.u = lv[i];
+            float t = w[i].x * fmaf((float)ll.h[0], 4.8828125e-4f, (float)hh.h[0]);
+            t = fmaf(w[i].y, fmaf((float)ll.h[1], 4.8828125e-4f, (float)hh.h[1]), t);
+            t = fmaf(w[i].z, fmaf((float)ll.h[2], 4.8828125e-4f, (float)hh.h[2]), t);
+            t = fmaf(w[i].w, fmaf((float)ll.h[3], 4.8828125e-4f, (float)hh.h[3]), t);
+            acc = fmaf(t, exp2i(ev[i]), acc);
+        }
+    }
+#pragma unroll
+    for (uint32_t o = 1u; o < LPR; o <<= 1) acc += __shfl_xor(acc, (int)o, 64);
+    return acc;
+}
+
+// Down + combine of one token on a mixed layout whose routed down matrices are word-packed IQ3_S: 8 output rows per workgroup, wave s <
+// top_k owns the selected expert s (both row quads against all ffn columns, as down_combine_kernel), wave top_k the shared expert, read
+// from its dense f32 copy [hidden][ffn]. blockIdx.y = token (small batches run one grid layer per token).
+struct DownWordsArgs {
+    const uint8_t *experts;    // word-packed down matrix of expert e at experts + e * stride
+    uint64_t stride;
+    const float *shared;       // dense f32 down matrix of the shared expert
+    const uint32_t *ids;
+    const float *weights, *scalar;
+    const _Float16 *act_h, *act_l;
+    const int *act_exp;
+    float *out;
+    uint32_t hidden, ffn, top_k;
+    const float *resid_a, *resid_b;
+};
+
+template <int NW>
+__global__ __launch_bounds__(NW * 64) void down_combine_words_kernel(DownWordsArgs a) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds[kIq3TableBytes];
+    __shared__ float part[17 * 8];
+    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
+    const uint32_t F = a.ffn, FG = F / 32u, FB = F / 256u, n_slot = a.top_k + 1u;
+    if (const uint32_t tok = blockIdx.y) {
+        const uint64_t t = tok;
+        a.ids += t * a.top_k;
+        a.weights += t * a.top_k;
+        a.scalar += t;
+        a.act_h += t * n_slot * F;
+        a.act_l += t * n_slot * F;
+        a.act_exp += t * n_slot * FG;
+        a.out += t * a.hidden;
+        if (a.resid_a) { a.resid_a += t * a.hidden; a.resid_b += t * a.hidden; }
+    }
+    const uint32_t row0 = 8u * blockIdx.x;
+    const uint32_t n_chunk = (FG + 15u) / 16u;         // ffn <= 1024
+    uint4 dq[2][2];
+    uint32_t dd[2][2];
+    half4_t ax[2][8];
+    float sc[2] = {0.0f, 0.0f};
+    const bool routed = wave < a.top_k;
+    if (routed) {
+        const uint8_t *ex = a.experts + (uint64_t)a.ids[wave] * a.stride;
+        const uint4 *qs = reinterpret_cast<const uint4 *>(ex);                                            // [hidden][FG]
+        const uint16_t *ds = reinterpret_cast<const uint16_t *>(ex + (uint64_t)a.hidden * FG * 16u);      // [hidden][FB]
+#pragma unroll
+        for (int q = 0; q < 2; ++q)
+#pragma unroll
+            for (int c = 0; c < 2; ++c) {
+                const uint32_t r = row0 + 4u * q + j, G = 16u * c + blk;
+                if ((uint32_t)c < n_chunk && G < FG) { dq[q][c] = qs[(uint64_t)r * FG + G]; dd[q][c] = ds[(uint64_t)r * FB + (G >> 3)]; }
+            }
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            const uint32_t G = 16u * c + blk;
+            if ((uint32_t)c < n_chunk && G < FG) {
+                load_act_operand(ax[c], a.act_h + (uint64_t)wave * F + 32u * G, a.act_l + (uint64_t)wave * F + 32u * G, j);
+                sc[c] = exp2i(a.act_exp[wave * FG + G]);
+            }
+        }
+    } else {                                           // the waves behind the routed ones share the shared expert's 8 rows
+        const uint32_t spare = (uint32_t)NW - a.top_k, k = a.top_k, sw = wave - a.top_k;
+        const _Float16 *ah = a.act_h + (uint64_t)k * F, *al = a.act_l + (uint64_t)k * F;
+        const int *ae = a.act_exp + k * FG;
+        if (spare >= 4u) {
+            if (sw < 4u) {
+                const uint32_t row = 2u * sw + (lane >> 5);
+                const float r = dense_row_dot<32>(a.shared + (uint64_t)(row0 + row) * F, ah, al, ae, F, lane & 31u);
+                if ((lane & 31u) == 0u) part[k * 8u + row] = r;
+            }
+        } else if (spare >= 2u) {
+            if (sw < 2u) {
+                const uint32_t row = 4u * sw + (lane >> 4);
+                const float r = dense_row_dot<16>(a.shared + (uint64_t)(row0 + row) * F, ah, al, ae, F, lane & 15u);
+                if ((lane & 15u) == 0u) part[k * 8u + row] = r;
+            }
+        } else if (sw == 0u) {
+            const uint32_t row = lane >> 3;
+            const float r = dense_row_dot<8>(a.shared + (uint64_t)(row0 + row) * F, ah, al, ae, F, lane & 7u);
+            if ((lane & 7u) == 0u) part[k * 8u + row] = r;
+        }
+    }
+    build_iq3s_quads(lds, tid);
+    __syncthreads();
+    if (routed) {
+        float tot[2] = {0.0f, 0.0f};
+#pragma unroll
+        for (int c = 0; c < 2; ++c) {
+            const uint32_t G = 16u * c + blk;
+            if ((uint32_t)c < n_chunk && G < FG) {
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {
+                    float va, vb;
+                    iq3s_group_dot(dq[q][c], ax[c], lds, va, vb);
+                    tot[q] += va * scale_to_f32(dd[q][c]) * sc[c];
+                }
+            }
+        }
+        const float r = quad_column_reduce<2>(tot, lane);
+        if (reduced_writer<2>(lane)) part[wave * 8u + 4u * reduced_unit<2>(lane) + j] = r;
+    }
+    __syncthreads();
+    if (tid < 8u) {
+        float sum = 0.0f;
+        for (uint32_t s = 0; s < a.top_k; ++s) sum = fmaf(a.weights[s], part[s * 8u + tid], sum);
+        sum = fmaf(a.scalar[0], part[a.top_k * 8u + tid], sum);
+        a.out[row0 + tid] = a.resid_a ? (a.resid_a[row0 + tid] + a.resid_b[row0 + tid]) + sum : sum;
+    }
+}
+
+hipError_t launch_down_combine_words(const void *experts, uint64_t stride, const float *shared_dense, const uint32_t *ids, const float *weights,
+                                     const float *scalar, const void *act_h, const void *act_l, const int *act_exp, float *out, uint32_t hidden,
+                                     uint32_t ffn, uint32_t top_k, hipStream_t s, uint32_t ntok) {
+    if (!hidden || hidden % 8u || !ffn || ffn % 256u || ffn > 1024u || top_k + 1u > (uint32_t)kWaves || !ntok || ntok > 65535u || !shared_dense) return hipErrorInvalidValue;
+    const DownWordsArgs a{static_cast<const uint8_t *>(experts), stride, shared_dense, ids, weights, scalar, static_cast<const _Float16 *>(act_h),
+                          static_cast<const _Float16 *>(act_l), act_exp, out, hidden, ffn, top_k, block_context().resid_a, block_context().resid_b};
+    const dim3 grid(hidden / 8u, ntok);
+    if (top_k + 1u <= 12u) REDHIP_LAUNCH(down_combine_words_kernel<12>, grid, dim3(12 * 64), 0, s, a);
+    else REDHIP_LAUNCH(down_combine_words_kernel<kWaves>, grid, dim3(kWaves * 64), 0, s, a);
+    return hipGetLastError();
+}
+
 // ---------------------------------------------------------------- small batches (2..16 tokens): select + group, batched gate/up, batched down
 
 // One workgroup: wave t selects the experts of token t, then the (token, k) pairs are grouped by expert. Same
@@ -1364,6 +1619,7 @@ struct BatchArgs {
     float *out;                    // [ntok][hidden]
     uint32_t hidden, ffn, top_k, ntok;
     const float *resid_a, *resid_b;     // when set: out = (resid_a + resid_b) + layer output, [ntok][hidden] each
+    const float *shared_gu;             // shared == nullptr: the shared expert's gate . x and up . x, [ntok][2 ffn] f32, already computed
 };
 
 // Persistent workgroups walk the units (u, g) = (group of pairs, 32 FFN columns): 32 gate + 32 up rows of the
@@ -1403,7 +1659,7 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_batch_kernel(BatchArgs a) 
         meta_expert[tid] = sh ? 0xffffffffu : a.uid[u];
         const uint32_t p0 = sh ? P : a.expert_start[u], p1 = sh ? P + a.ntok : a.expert_start[u + 1u];
         meta_p0[tid] = p0;
-        meta_n[tid] = p1 - p0;
+        meta_n[tid] = sh && !a.shared ? 0u : p1 - p0;      // a shared expert that is not packed has no passes: its products are an input
         for (uint32_t i = 0; i < p1 - p0 && i < (uint32_t)kMaxTok; ++i) meta_tok[tid][i] = (uint8_t)(sh ? i : a.pair_token[p0 + i]);
     }
     if (tid >= 64u && tid < 64u + a.ntok) tok_scale[tid - 64u] = 0.125f * exp2i(a.xexp[tid - 64u]);
@@ -1429,7 +1685,7 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_batch_kernel(BatchArgs a) 
     auto load_weights = [&](uint32_t k, uint2 *q, uint32_t *d) {
         const uint32_t g = (blockIdx.x + k * gridDim.x) % FG;
         const uint32_t e = __builtin_amdgcn_readfirstlane(meta_expert[k]);
-        const uint8_t *ex = e == 0xffffffffu ? a.shared : a.experts + (uint64_t)e * a.stride;
+        const uint8_t *ex = e == 0xffffffffu ? (a.shared ? a.shared : a.experts) : a.experts + (uint64_t)e * a.stride;   // (never-used weights of a unit without passes)
 #pragma unroll
         for (int un = 0; un < UPW; ++un) {
             const uint32_t quad = q0 + (NW / NKC) * un;
@@ -1509,6 +1765,18 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_batch_kernel(BatchArgs a) 
                     if (c == 0u) a.act_exp[pr * FG + g] = e;
                 }
             }
+        }
+        if (!a.shared && meta_expert[k] == 0xffffffffu && tid < 32u * a.ntok) {      // SwiGLU of the given products, token t at pair P + t
+            const uint32_t t = tid >> 5, c = tid & 31u;
+            const float gsum = a.shared_gu[(uint64_t)t * 2u * F + 32u * g + c], usum = a.shared_gu[(uint64_t)t * 2u * F + F + 32u * g + c];
+            const float act = (gsum / (1.0f + expf(-gsum))) * usum;
+            float amax = fabsf(act);
+#pragma unroll
+            for (int o = 16; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+            const int e = prescale_exp(amax);
+            const uint64_t pr = P + t;
+            split_hi_lo(act, exp2i(-e), a.act_h + pr * F + 32u * g + c, a.act_l + pr * F + 32u * g + c);
+            if (c == 0u) a.act_exp[pr * FG + g] = e;
         }
 #pragma unroll
         for (int un = 0; un < UPW; ++un) { wq[un] = wq_next[un]; wd[un] = wd_next[un]; }
@@ -1623,6 +1891,105 @@ __global__ __launch_bounds__(kWaves * 64) void down_batch_kernel(BatchArgs a) {
     }
 }
 
+// Batched down + combine on raw GGUF rows (mixed layouts): the work split of down_batch_kernel (8 output rows per workgroup, wave w owns
+// the groups w, w + 16, ..., the last group is the shared expert with every token) with the decode of down_combine_raw_kernel. A wave
+// stages the 8 rows of its group in LDS (the next group's rows are requested into registers before the current group is computed),
+// decodes a row's chunk once and applies it to every pair of the group, so a matrix is read once however many tokens selected it.
+struct DownBatchRawArgs {
+    const uint8_t *experts;    // expert e's raw down rows at experts + e * stride
+    uint64_t stride;
+    const uint8_t *shared;     // raw down rows of the shared expert
+    const uint32_t *uid, *expert_start, *n_unique;
+    const float *pair_weight;
+    const uint32_t *tok_pair;
+    const float *scalar;
+    const _Float16 *act_h, *act_l;     // [P + ntok][ffn]
+    const int *act_exp;
+    float *out;
+    uint32_t hidden, ffn, top_k, ntok;
+    const float *resid_a, *resid_b;
+};
+
+template <uint32_t TD, uint32_t TS>
+__global__ __launch_bounds__(kWaves * 64) void down_batch_raw_kernel(DownBatchRawArgs a) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t raw_rows[];     // [wave][8 rows of the wave's current group]
+    __shared__ float part[144 * 8];
+    constexpr uint32_t kMaxBlock = Fmt<TD>::kBlock > Fmt<TS>::kBlock ? Fmt<TD>::kBlock : Fmt<TS>::kBlock;
+    constexpr int kVec = 5;                            // 16-byte pieces per lane of one group's rows: 8 rows x 3 blocks x 210 bytes at most
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t H = a.hidden, F = a.ffn, FG = F / 32u, FB = F / 256u, P = a.ntok * a.top_k;
+    const uint32_t row0 = 8u * blockIdx.x, U = __builtin_amdgcn_readfirstlane(a.n_unique[0]);
+    uint8_t *mine = raw_rows + wave * 8u * FB * kMaxBlock;
+    uint4 nxt[kVec];
+    auto fetch = [&](uint32_t u) {                      // rows of group u (clamped: the last request repeats the shared expert's)
+        const uint32_t uc = u < U ? u : U;
+        const bool sh = uc == U;
+        const uint32_t row_bytes = FB * (sh ? Fmt<TS>::kBlock : Fmt<TD>::kBlock), nvec = 8u * row_bytes / 16u;
+        const uint32_t e = __builtin_amdgcn_readfirstlane(a.uid[sh ? 0u : uc]);
+        const uint4 *src = reinterpret_cast<const uint4 *>((sh ? a.shared : a.experts + (uint64_t)e * a.stride) + (uint64_t)row0 * row_bytes);
+#pragma unroll
+        for (int i = 0; i < kVec; ++i) {
+            const uint32_t at = lane + 64u * (uint32_t)i;
+            nxt[i] = src[at < nvec ? at : nvec - 1u];
+        }
+    };
+    fetch(wave);
+    for (uint32_t u = wave; u <= U; u += 16u) {
+        const bool sh = u == U;
+        const uint32_t row_bytes = FB * (sh ? Fmt<TS>::kBlock : Fmt<TD>::kBlock), nvec = 8u * row_bytes / 16u;
+        const uint32_t p0 = sh ? P : __builtin_amdgcn_readfirstlane(a.expert_start[u]);
+        const uint32_t p1 = sh ? P + a.ntok : __builtin_amdgcn_readfirstlane(a.expert_start[u + 1u]);
+        wave_lds_sync();                               // the previous group's reads of `mine` are done
+#pragma unroll
+        for (int i = 0; i < kVec; ++i) {
+            const uint32_t at = lane + 64u * (uint32_t)i;
+            if (at < nvec) reinterpret_cast<uint4 *>(mine)[at] = nxt[i];
+        }
+        fetch(u + 16u);                                // always issued: a conditional request would be waited for at once
+        wave_lds_sync();
+        for (uint32_t G = blk; G < FG; G += 16u) {
+#pragma unroll
+            for (int q = 0; q < 2; ++q) {
+                float w[32];
+                const uint8_t *row = mine + (4u * (uint32_t)q + j) * row_bytes;
+                if (sh) decode32<TS>(row, G, w); else decode32<TD>(row, G, w);
+                for (uint32_t p = p0; p < p1; ++p) {
+                    const float sc = exp2i(a.act_exp[p * FG + G]);
+                    const uint4 *ph = reinterpret_cast<const uint4 *>(a.act_h + (uint64_t)p * F + 32u * G), *pl = reinterpret_cast<const uint4 *>(a.act_l + (uint64_t)p * F + 32u * G);
+                    float acc = 0.0f;
+#pragma unroll
+                    for (int v = 0; v < 4; ++v) {
+                        union { uint4 u; _Float16 h[8]; } hh, ll;
+                        hh.u = ph[v];
+                        ll.u = pl[v];
+#pragma unroll
+                        for (int i = 0; i < 8; ++i) acc = fmaf(w[8 * v + i], fmaf((float)ll.h[i], 4.8828125e-4f, (float)hh.h[i]), acc);
+                    }
+                    acc *= sc;
+                    const float r = quad_column_reduce<1>(&acc, lane);      // over the 16 lanes that share j (one chunk each)
+                    if (reduced_writer<1>(lane)) {
+                        float *dst = &part[p * 8u + 4u * (uint32_t)q + j];
+                        *dst = G == blk ? r : *dst + r;
+                    }
+                }
+            }
+        }
+    }
+    __syncthreads();
+    for (uint32_t i = tid; i < a.ntok * 8u; i += kWaves * 64u) {
+        const uint32_t t = i >> 3, r = i & 7u;
+        float sum = 0.0f;
+        for (uint32_t k = 0; k < a.top_k; ++k) {
+            const uint32_t p = a.tok_pair[t * a.top_k + k];
+            sum = fmaf(a.pair_weight[p], part[p * 8u + r], sum);
+        }
+        sum = fmaf(a.scalar[t], part[(P + t) * 8u + r], sum);
+        const uint64_t at = (uint64_t)t * H + row0 + r;
+        a.out[at] = a.resid_a ? (a.resid_a[at] + a.resid_b[at]) + sum : sum;
+    }
+}
+
 static hipError_t launch_gateup_batch_kernel(const BatchArgs &a, uint32_t n_groups, hipStream_t s);
 
 hipError_t launch_batch_packed(const void *experts, uint64_t stride, const void *shared, const uint32_t *uid, const uint32_t *expert_start,
@@ -1633,7 +2000,7 @@ hipError_t launch_batch_packed(const void *experts, uint64_t stride, const void 
     BatchArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(shared), uid, expert_start, pair_token, n_unique,
                 pair_weight, tok_pair, scalar, static_cast<const _Float16 *>(xh), static_cast<const _Float16 *>(xl), xexp,
                 static_cast<_Float16 *>(act_h), static_cast<_Float16 *>(act_l), act_exp, out, hidden, ffn, top_k, ntok,
-                block_context().resid_a, block_context().resid_b};
+                block_context().resid_a, block_context().resid_b, nullptr};
     const uint32_t P = ntok * top_k, n_groups = (P < n_expert ? P : n_expert) + 1u;
     hipError_t e = launch_gateup_batch_kernel(a, n_groups, s);
     if (e != hipSuccess) return e;
@@ -1649,6 +2016,60 @@ hipError_t launch_batch_packed(const void *experts, uint64_t stride, const void 
 }
 
 // the persistent gate/up kernel of a small batch over n_groups groups of pairs (the shared expert included when a.shared is set)
+template <uint32_t TD>
+static hipError_t launch_down_batch_raw_shared(uint32_t ts, const DownBatchRawArgs &a, hipStream_t s) {
+    const dim3 grid(a.hidden / 8u), block(kWaves * 64);
+    const size_t lds = (size_t)kWaves * 8u * (a.ffn / 256u) * 210u;       // sized for the largest block type: 53,760 bytes at ffn 512
+#define REDHIP_DBR(TSV)                                                                                                     \
+    do {                                                                                                                    \
+        static bool attr = false;                                                                                            \
+        if (!attr) {                                                                                                         \
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(down_batch_raw_kernel<TD, TSV>), hipFuncAttributeMaxDynamicSharedMemorySize, 96 * 1024); \
+            if (e != hipSuccess) return e;                                                                                   \
+            attr = true;                                                                                                     \
+        }                                                                                                                    \
+        REDHIP_LAUNCH((down_batch_raw_kernel<TD, TSV>), grid, block, lds, s, a);                                              \
+    } while (0)
+    switch (ts) {
+        case T_IQ2_XXS: REDHIP_DBR(T_IQ2_XXS); break;
+        case T_IQ3_S: REDHIP_DBR(T_IQ3_S); break;
+        case T_Q6_K: REDHIP_DBR(T_Q6_K); break;
+        default: return hipErrorInvalidValue;
+    }
+#undef REDHIP_DBR
+    return hipGetLastError();
+}
+
+// Small batch on a mixed layout, pairs grouped by expert: packed IQ2_XXS gate/up matrices on the batched MFMA kernel (the shared
+// expert's gate / up products come in as shared_gu [ntok][2 ffn]), raw down matrices of any built-in type on the batched raw-row kernel.
+hipError_t launch_batch_mixed(const void *packed, uint64_t packed_stride, const float *shared_gu, uint32_t down_type, uint32_t shared_down_type,
+                              const void *raw_down, uint64_t raw_stride, const void *shared_down, const uint32_t *uid, const uint32_t *expert_start,
+                              const uint32_t *pair_token, const uint32_t *n_unique, const float *pair_weight, const uint32_t *tok_pair,
+                              const float *scalar, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l, int *act_exp,
+                              float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s) {
+    if (!fused_iq2_supported(hidden, ffn) || !ntok || ntok > (uint32_t)kMaxTok || ntok * top_k + ntok > 144u || ffn > 768u || !shared_gu) return hipErrorInvalidValue;
+    // the staged rows move in 16-byte pieces
+    const uint32_t rbd = (ffn / 256u) * block_bytes(down_type), rbs = (ffn / 256u) * block_bytes(shared_down_type);
+    if (!rbd || !rbs || (8u * rbd) % 16u || (8u * rbs) % 16u || raw_stride % 16u || (uintptr_t)raw_down % 16u || (uintptr_t)shared_down % 16u) return hipErrorInvalidValue;
+    BatchArgs a{static_cast<const uint8_t *>(packed), packed_stride, nullptr, uid, expert_start, pair_token, n_unique,
+                pair_weight, tok_pair, scalar, static_cast<const _Float16 *>(xh), static_cast<const _Float16 *>(xl), xexp,
+                static_cast<_Float16 *>(act_h), static_cast<_Float16 *>(act_l), act_exp, out, hidden, ffn, top_k, ntok,
+                nullptr, nullptr, shared_gu};
+    const uint32_t P = ntok * top_k, n_groups = (P < n_expert ? P : n_expert) + 1u;
+    hipError_t e = launch_gateup_batch_kernel(a, n_groups, s);
+    if (e != hipSuccess) return e;
+    prof_set_stage(ST_BATCH_DOWN);
+    const DownBatchRawArgs d{static_cast<const uint8_t *>(raw_down), raw_stride, static_cast<const uint8_t *>(shared_down), uid, expert_start, n_unique,
+                             pair_weight, tok_pair, scalar, static_cast<const _Float16 *>(act_h), static_cast<const _Float16 *>(act_l), act_exp, out,
+                             hidden, ffn, top_k, ntok, block_context().resid_a, block_context().resid_b};
+    switch (down_type) {
+        case T_IQ2_XXS: return launch_down_batch_raw_shared<T_IQ2_XXS>(shared_down_type, d, s);
+        case T_IQ3_S: return launch_down_batch_raw_shared<T_IQ3_S>(shared_down_type, d, s);
+        case T_Q6_K: return launch_down_batch_raw_shared<T_Q6_K>(shared_down_type, d, s);
+        default: return hipErrorInvalidValue;
+    }
+}
+
 static hipError_t launch_gateup_batch_kernel(const BatchArgs &a, uint32_t n_groups, hipStream_t s) {
     const uint32_t hidden = a.hidden, ffn = a.ffn, ntok = a.ntok;
     const uint32_t unit_bound = n_groups * (ffn / 32u);

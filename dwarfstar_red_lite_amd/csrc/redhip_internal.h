@@ -203,6 +203,21 @@ hipError_t launch_gateup_select(const void *experts, uint64_t stride, const void
                                 float *scalar_out, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l, int *act_exp,
                                 uint32_t hidden, uint32_t ffn, uint32_t n_expert, uint32_t top_k, hipStream_t s, uint32_t ntok = 1u,
                                 uint32_t gate_up_type = T_IQ2_XXS, const int8_t *grid = nullptr);
+// small batch on a mixed layout with the pairs grouped by expert: batched MFMA gate/up on the packed IQ2_XXS matrices (shared expert's
+// products given), batched raw-row down of the built-in block types; every distinct expert is read once
+hipError_t launch_batch_mixed(const void *packed, uint64_t packed_stride, const float *shared_gu, uint32_t down_type, uint32_t shared_down_type,
+                              const void *raw_down, uint64_t raw_stride, const void *shared_down, const uint32_t *uid, const uint32_t *expert_start,
+                              const uint32_t *pair_token, const uint32_t *n_unique, const float *pair_weight, const uint32_t *tok_pair,
+                              const float *scalar, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l, int *act_exp,
+                              float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s);
+// IQ3_S down matrices of mixed layouts as one word per eight weights (uint4 per 32, [row][K/32], then d as fp16 [row][K/256])
+hipError_t launch_repack_iq3s_words(const void *raw, uint64_t raw_stride, uint32_t count, uint32_t nrows, uint32_t K, void *packed, uint64_t packed_stride, hipStream_t s);
+hipError_t launch_dequant_iq3s_words(const void *packed, uint32_t nrows, uint32_t K, float *out, hipStream_t s);
+inline uint64_t iq3s_words_bytes(uint32_t nrows, uint32_t K) { return (uint64_t)nrows * ((uint64_t)(K / 32u) * 16u + (uint64_t)(K / 256u) * 2u); }
+// down + combine of one token (ntok > 1: one grid layer per token) on word-packed IQ3_S routed matrices and the shared expert's dense f32 copy
+hipError_t launch_down_combine_words(const void *experts, uint64_t stride, const float *shared_dense, const uint32_t *ids, const float *weights,
+                                     const float *scalar, const void *act_h, const void *act_l, const int *act_exp, float *out, uint32_t hidden,
+                                     uint32_t ffn, uint32_t top_k, hipStream_t s, uint32_t ntok = 1u);
 // down + weighted combine for layouts whose down matrices are raw GGUF rows of any supported type
 hipError_t launch_down_combine_raw(uint32_t down_type, uint32_t shared_down_type, const void *experts, uint64_t stride, const void *shared,
                                    const uint32_t *ids, const float *weights, const float *scalar, const void *act_h, const void *act_l,

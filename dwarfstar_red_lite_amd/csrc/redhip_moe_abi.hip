@@ -40,6 +40,7 @@ struct Layer {
     // kernel: router [n_expert][hidden] (when it is quantised), shared gate | up [2 ffn][hidden], shared down [hidden][ffn]
     float *dense_router = nullptr, *dense_gu = nullptr, *dense_down = nullptr;
     uint8_t *tiled_down = nullptr;   // mixed layouts with IQ3_S down matrices that take chunks: their tile-major copy
+    uint8_t *words_down = nullptr;   // mixed layouts with IQ3_S down matrices: one word per eight weights, for the MFMA down kernels of up to 8 tokens
 };
 
 struct Moe {
@@ -77,6 +78,7 @@ struct Moe {
     bool tiles_resident() const { return packed_gu() && gu_type == T_IQ2_XXS && cfg.max_tokens > 8u && cfg.ffn <= 512u && cfg.hidden / 512u <= 4u; }
     // a chunk on a mixed layout: the routed gate/up matrices (packed IQ2_XXS) run on the prefill tiles, the rest on raw rows
     bool mixed_chunk(uint32_t ntok) const { return mixed && ntok > 8u && tiles_resident(); }
+    uint64_t words_down_stride() const { return (iq3s_words_bytes(cfg.hidden, cfg.ffn) + 255u) & ~255ull; }
     uint64_t tiled_down_stride() const { return ((uint64_t)cfg.hidden * (cfg.ffn / 32u) * 16u + (uint64_t)cfg.hidden * (cfg.ffn / 256u) * 2u + 255u) & ~255ull; }
     // the one-launch router kernels (logits of every expert + the shared expert's gate logit, optional residual + norm) and the
     // one-wave selection serve every layout whose router they tile; the per-row GEMV + generic selection are what is left
@@ -104,6 +106,15 @@ struct Moe {
     // expert at these sizes, so reading a shared expert twice costs less than the pair sort and the per-pair kernels)
     bool small_batch_mixed(uint32_t ntok) const {
         return mixed && ntok >= 2u && ntok <= 8u && ntok * cfg.top_k <= 128u && ntok * (cfg.top_k + 1u) <= 144u && cfg.hidden / 512u <= 4u;
+    }
+    // from kGroupedMin tokens on such a batch is grouped by expert instead when its formats allow (packed IQ2_XXS gate/up on the batched
+    // MFMA kernel, built-in down types on the batched raw-row kernel): every distinct expert is read once. Needs the router launch of the
+    // same forward() for the shared expert's gate / up products.
+    static constexpr uint32_t kGroupedMin = 3u;
+    bool grouped_mixed(uint32_t ntok) const {
+        const uint32_t rbd = (cfg.ffn / 256u) * block_bytes(dn_type), rbs = (cfg.ffn / 256u) * block_bytes(sh_dn_type);
+        return small_batch_mixed(ntok) && ntok >= kGroupedMin && gu_type == T_IQ2_XXS && quant_supported(dn_type) && cfg.ffn <= 768u &&
+               (8u * rbd) % 16u == 0u && (8u * rbs) % 16u == 0u && (2u * gate_bytes) % 16u == 0u && (2u * sh_gate_bytes) % 16u == 0u;
     }
     // every batch size runs on the packed layout when the layer has one (decode kernel, small-batch kernels, prefill tiles)
     bool packed_path(uint32_t ntok) const { return (fused && (ntok == 1u || small_batch(ntok) || cfg.hidden / 512u <= 4u)) || (mixed && ntok == 1u); }
@@ -151,6 +162,20 @@ __global__ __launch_bounds__(256) void resid_rms_kernel(const float *x, const fl
 int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const uint32_t *ids, const float *weights,
                     float *out, hipStream_t s, bool select_here = false, bool grouped = false) {
     const redhip_moe_config &c = m->cfg;
+    if (m->grouped_mixed(ntok) && m->shared_gu_ready) {      // xh / xl / xexp / scalar and the shared gate | up products (m->act) come from the router launch
+        const Layer &L = m->layers[layer];
+        if (!grouped) {
+            prof_set_stage(ST_GROUP);
+            HIP_OK(launch_group_pairs(ids, weights, ntok, c.top_k, c.n_expert, m->uid, m->expert_start, m->pair_token, m->pair_weight,
+                                      m->tok_pair, m->n_unique, s), "grouping launch");
+        }
+        HIP_OK(launch_batch_mixed(L.packed, m->packed_stride, m->act, m->dn_type, m->sh_dn_type, L.experts + 2u * m->gate_bytes, m->expert_stride,
+                                  L.shared + 2u * m->sh_gate_bytes, m->uid, m->expert_start, m->pair_token, m->n_unique, m->pair_weight, m->tok_pair,
+                                  m->scalar, m->xh, m->xl, m->xexp, m->act_h, m->act_l, m->act_exp, out, c.hidden, c.ffn, c.top_k, ntok, c.n_expert, s),
+               "grouped mixed batch launch");
+        prof_set_stage(ST_OTHER);
+        return 1;
+    }
     if (ntok > 1u && !m->small_batch_mixed(ntok)) {       // group the (token, expert) pairs by expert, run each distinct expert once over its tokens
         const uint32_t P = ntok * c.top_k, n_groups = P < c.n_expert ? P : c.n_expert;
         const ExpertSet ex = m->routed(layer), sh = m->shared(layer);
@@ -222,6 +247,9 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
         if (m->fused)
             HIP_OK(launch_down_combine(L.packed, m->expert_stride, L.shared_packed, select_here ? m->ids : ids, select_here ? m->weights : weights,
                                        m->scalar, m->act_h, m->act_l, m->act_exp, out, c.hidden, c.ffn, c.top_k, s), "down/combine launch");
+        else if (L.words_down && L.dense_down)
+            HIP_OK(launch_down_combine_words(L.words_down, m->words_down_stride(), L.dense_down, select_here ? m->ids : ids, select_here ? m->weights : weights,
+                                             m->scalar, m->act_h, m->act_l, m->act_exp, out, c.hidden, c.ffn, c.top_k, s, ntok), "down/combine launch");
         else
             HIP_OK(launch_down_combine_raw(m->dn_type, m->sh_dn_type, L.experts + 2u * m->gate_bytes, m->expert_stride, L.shared + 2u * m->sh_gate_bytes,
                                            select_here ? m->ids : ids, select_here ? m->weights : weights, m->scalar, m->act_h, m->act_l,
@@ -320,6 +348,10 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
                 m->resident += align256(rb) + align256(gb) + align256(db);
             }
         }
+        if (ok && m->mixed && dn == T_IQ3_S && c.ffn <= 1024u) {
+            ok = hipMalloc(reinterpret_cast<void **>(&L.words_down), (size_t)c.n_expert * m->words_down_stride()) == hipSuccess;
+            m->resident += (uint64_t)c.n_expert * m->words_down_stride();
+        }
         if (ok && m->mixed && m->tiles_resident() && dn == T_IQ3_S) {
             ok = hipMalloc(reinterpret_cast<void **>(&L.tiled_down), (size_t)c.n_expert * m->tiled_down_stride()) == hipSuccess;
             m->resident += (uint64_t)c.n_expert * m->tiled_down_stride();
@@ -395,6 +427,7 @@ void redhip_moe_destroy(redhip_moe_t h) {
         if (L.dense_gu) (void)hipFree(L.dense_router ? L.dense_router : L.dense_gu);
         if (L.tiled) (void)hipFree(L.tiled);
         if (L.tiled_down) (void)hipFree(L.tiled_down);
+        if (L.words_down) (void)hipFree(L.words_down);
         if (L.shared_tiled) (void)hipFree(L.shared_tiled);
     }
     if (m->ws) (void)hipFree(m->ws);
@@ -497,6 +530,9 @@ static int stage_and_pack(Moe *m, uint32_t layer, uint32_t first, uint32_t count
             if (m->fused)
                 HIP_OK(launch_tile_packed(pk + 2u * m->gate_bytes, m->packed_stride, count, c.hidden, c.ffn, tl + 2u * m->gate_bytes, m->packed_stride, nullptr), "expert down tiling");
         }
+        if (m->layers[layer].words_down)
+            HIP_OK(launch_repack_iq3s_words(dst + 2u * m->gate_bytes, m->expert_stride, count, c.hidden, c.ffn,
+                                            m->layers[layer].words_down + (uint64_t)first * m->words_down_stride(), m->words_down_stride(), nullptr), "expert down words");
         if (m->layers[layer].tiled_down)
             HIP_OK(launch_tile_iq3s(dst + 2u * m->gate_bytes, m->expert_stride, count, c.hidden, c.ffn,
                                     m->layers[layer].tiled_down + (uint64_t)first * m->tiled_down_stride(), m->tiled_down_stride(), nullptr), "expert down tiling");
@@ -565,10 +601,22 @@ int redhip_moe_experts(redhip_moe_t h, uint32_t layer, const float *x_dev, uint3
     if (!check_layer(m, layer)) return 0;
     if (!x_dev || !ids_dev || !weights_dev || !out_dev || !ntok || ntok > m->cfg.max_tokens) { moe_err("invalid expert execution arguments"); return 0; }
     hipStream_t s = static_cast<hipStream_t>(stream);
+    m->shared_gu_ready = false;
     if (m->packed_path(ntok) || m->small_batch_mixed(ntok) || m->mixed_chunk(ntok)) {
         prof_set_stage(ST_OTHER);
         HIP_OK(launch_prep(x_dev, m->layers[layer].gate_inp, ntok, m->cfg.hidden, m->xh, m->xl, m->xexp, m->scalar, s), "prep launch");
-        return experts_enqueue(m, layer, x_dev, ntok, ids_dev, weights_dev, out_dev, s);
+        const Layer &L = m->layers[layer];
+        const uint32_t nv = m->cfg.hidden / 256u;
+        if (m->grouped_mixed(ntok) && L.dense_gu && (nv == 2u || nv == 4u || nv == 8u || nv == 16u)) {
+            // the grouped kernels take the shared expert's gate | up products as an input: one f32 GEMV over its f32 copy (no router rows)
+            prof_set_stage(ST_SHARED_GATEUP);
+            HIP_OK(launch_router_gemv(T_F32, L.dense_gu, x_dev, L.gate_inp, ntok, m->cfg.hidden, 0u, m->logits, m->xh, m->xl, m->xexp, nullptr, m->act,
+                                      m->cfg.ffn, s, L.dense_gu), "shared gate/up launch");
+            m->shared_gu_ready = true;
+        }
+        const int ok = experts_enqueue(m, layer, x_dev, ntok, ids_dev, weights_dev, out_dev, s);
+        m->shared_gu_ready = false;
+        return ok;
     }
     scalar_gate_kernel<<<ntok, 256, 0, s>>>(m->layers[layer].gate_inp, x_dev, m->cfg.hidden, m->scalar);
     HIP_OK(hipGetLastError(), "scalar gate launch");
@@ -579,8 +627,8 @@ int redhip_moe_forward(redhip_moe_t h, uint32_t layer, const float *x_dev, uint3
     Moe *m = moe_of(h);
     if (!check_layer(m, layer)) return 0;
     if (!x_dev || !out_dev) { moe_err("null activation pointer"); return 0; }
-    const bool select_in_gateup = m->packed_gu() && (ntok == 1u || m->small_batch_mixed(ntok));
-    const bool group_in_select = m->small_batch(ntok);
+    const bool group_in_select = m->small_batch(ntok) || m->grouped_mixed(ntok);
+    const bool select_in_gateup = m->packed_gu() && (ntok == 1u || m->small_batch_mixed(ntok)) && !group_in_select;
     m->skip_select = select_in_gateup;
     m->select_and_group = group_in_select;
     const int routed = redhip_moe_route(h, layer, x_dev, ntok, nullptr, nullptr, nullptr, stream);
@@ -608,8 +656,8 @@ int redhip_moe_forward_block(redhip_moe_t h, uint32_t layer, const float *x_dev,
         if (hipGetLastError() != hipSuccess) { moe_err("residual + norm launch failed"); ok = 0; }
     }
     if (ok) {
-        const bool select_in_gateup = m->packed_gu() && (ntok == 1u || m->small_batch_mixed(ntok));
-        const bool group_in_select = m->small_batch(ntok);
+        const bool group_in_select = m->small_batch(ntok) || m->grouped_mixed(ntok);
+        const bool select_in_gateup = m->packed_gu() && (ntok == 1u || m->small_batch_mixed(ntok)) && !group_in_select;
         m->skip_select = select_in_gateup;
         m->select_and_group = group_in_select;
         if (in_router) { bc.branch = branch_dev; bc.norm_w = post_norm_dev; bc.eps = eps; bc.xn_out = m->xn; }
@@ -686,6 +734,10 @@ int redhip_moe_dequant_resident(redhip_moe_t h, uint32_t layer, uint32_t expert,
         const uint64_t gbytes = m->pk_gate_bytes;
         if (which < 2u) HIP_OK(launch_dequant_packed(m->gu_type, pk + which * gbytes, c.ffn, c.hidden, m->gu_grid, out_dev, s), "packed gate/up dequant");
         else HIP_OK(launch_dequant_packed_iq2xxs(pk + 2u * gbytes, c.hidden, c.ffn, false, out_dev, s), "packed down dequant");
+        return 1;
+    }
+    if (which == 2u && !sh && L.words_down) {       // the copy the MFMA down kernels read
+        HIP_OK(launch_dequant_iq3s_words(L.words_down + (uint64_t)expert * m->words_down_stride(), c.hidden, c.ffn, out_dev, s), "word-packed down dequant");
         return 1;
     }
     const uint8_t *base = sh ? L.shared : L.experts + (uint64_t)expert * m->expert_stride;

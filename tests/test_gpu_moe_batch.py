@@ -60,6 +60,18 @@ def test_ragged_small_batches_hot_experts(layout):
     assert np.array_equal(got[0], got[1])
     for t in range(5):
         assert rel_l2(got[t], want[t]) <= REL_L2_TOL
+    # a full batch in which three requests carry the same row: groups of one, two and three pairs, read once each
+    x = synth.normed_x(rng, 8, cfg["hidden"])
+    x[3] = x[0]
+    x[6] = x[0]
+    x[7] = x[2]
+    got = m.forward(0, torch.from_numpy(x).cuda()).cpu().numpy()
+    gids, gw, glog = m.last_route(8)
+    want, cids, cw, clog = orc.Layer(cfg, **lay).forward(x, threads=8)
+    assert np.array_equal(gids, cids)
+    assert np.array_equal(got[0], got[3]) and np.array_equal(got[0], got[6]) and np.array_equal(got[2], got[7])
+    for t in range(8):
+        assert rel_l2(got[t], want[t]) <= REL_L2_TOL, (layout, t)
     m.close()
 
 
