@@ -1891,6 +1891,131 @@ __global__ __launch_bounds__(kWaves * 64) void down_batch_kernel(BatchArgs a) {
     }
 }
 
+// The same kernel for mixed layouts whose routed down matrices are word-packed IQ3_S; the shared expert's rows come from its dense f32
+// copy (token t's product on wave 15 - t, ahead of that wave's routed groups).
+struct BatchWordsArgs {
+    const uint8_t *experts;    // word-packed down matrix of expert e at experts + e * stride
+    uint64_t stride;
+    const float *shared;       // dense f32 [hidden][ffn]
+    const uint32_t *uid, *expert_start, *n_unique;
+    const float *pair_weight;
+    const uint32_t *tok_pair;
+    const float *scalar;
+    const _Float16 *act_h, *act_l;
+    const int *act_exp;
+    float *out;
+    uint32_t hidden, ffn, top_k, ntok;
+    const float *resid_a, *resid_b;
+};
+
+template <int MAXPAIR, int NCH, int GPW>     // GPW: groups of a wave whose weights are in registers at once
+__global__ __launch_bounds__(kWaves * 64) void down_batch_words_kernel(BatchWordsArgs a) {
+    __shared__ __attribute__((aligned(16))) uint8_t lds[kIq3TableBytes];
+    __shared__ float part[MAXPAIR * 8];
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
+    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t H = a.hidden, F = a.ffn, FG = F / 32u, FB = F / 256u, P = a.ntok * a.top_k;
+    const uint32_t row0 = 8u * blockIdx.x, U = __builtin_amdgcn_readfirstlane(a.n_unique[0]);
+    const uint64_t qs_bytes = (uint64_t)H * FG * 16u;
+
+    uint4 wq[GPW][NCH][2];
+    uint32_t wd[GPW][NCH], gp0[GPW], gp1[GPW];      // wd: the two rows' block scales, 16 bits each
+    // metadata and weights of groups first, first + 16, ...; indices are clamped so that every request is valid
+    auto request = [&](uint32_t first) {
+#pragma unroll
+        for (int i = 0; i < GPW; ++i) {
+            const uint32_t u = first + 16u * (uint32_t)i, uc = u < U ? u : U - 1u;      // routed groups only (U >= 1)
+            // wave-uniform values: kept in scalar registers
+            const uint32_t e = __builtin_amdgcn_readfirstlane(a.uid[uc]), es0 = __builtin_amdgcn_readfirstlane(a.expert_start[uc]),
+                           es1 = __builtin_amdgcn_readfirstlane(a.expert_start[uc + 1u]);
+            gp0[i] = es0;
+            gp1[i] = u < U ? es1 : es0;
+            const uint8_t *dn = a.experts + (uint64_t)e * a.stride;
+#pragma unroll
+            for (int c = 0; c < NCH; ++c) {
+                const uint32_t G = 16u * (uint32_t)c + blk, Gc = G < FG ? G : FG - 1u;
+                uint32_t d2 = 0u;
+#pragma unroll
+                for (int q = 0; q < 2; ++q) {
+                    const uint32_t r = row0 + 4u * (uint32_t)q + j;
+                    wq[i][c][q] = reinterpret_cast<const uint4 *>(dn)[(uint64_t)r * FG + Gc];
+                    d2 |= (uint32_t)reinterpret_cast<const uint16_t *>(dn + qs_bytes)[(uint64_t)r * FB + (Gc >> 3)] << (16 * q);
+                }
+                wd[i][c] = d2;
+            }
+        }
+    };
+    struct Pass { half4_t ax[NCH][8]; float sa[NCH], sb[NCH]; };
+    // activations of pairs pp (and pp + 1 if it belongs to the group); pp is clamped into the buffer
+    auto load_pass = [&](uint32_t pp, uint32_t p1, Pass &ps) {
+        const uint32_t last = P + a.ntok - 1u, pa = pp < last ? pp : last, pb = pa + 1u < p1 ? pa + 1u : pa;
+        const bool have_b = pp + 1u < p1;
+#pragma unroll
+        for (int c = 0; c < NCH; ++c) {
+            const uint32_t G = 16u * (uint32_t)c + blk, Gc = G < FG ? G : FG - 1u;
+            load_act_operand2(ps.ax[c], a.act_h, a.act_l, (uint64_t)pa * F, (uint64_t)pb * F, true, 32u * Gc, j);
+            const float live = G < FG ? 1.0f : 0.0f;
+            ps.sa[c] = live * exp2i(a.act_exp[pa * FG + Gc]);
+            ps.sb[c] = have_b ? live * exp2i(a.act_exp[pb * FG + Gc]) : 0.0f;
+        }
+    };
+    // the shared expert: its 8 rows from the dense copy; token t on wave 15 - t, before that wave's routed groups take their registers
+    if (15u - wave < a.ntok) {
+        const uint32_t p = P + (15u - wave), row = lane >> 3;
+        const float r = dense_row_dot<8>(a.shared + (uint64_t)(row0 + row) * F, a.act_h + (uint64_t)p * F, a.act_l + (uint64_t)p * F, a.act_exp + p * FG, F, lane & 7u);
+        if ((lane & 7u) == 0u) part[p * 8u + row] = r;
+    }
+    request(wave);
+    build_iq3s_quads(lds, tid);
+    __syncthreads();
+
+    for (uint32_t first = wave; first < U; first += 16u * GPW) {
+        if (first != wave) request(first);
+        Pass buf[2];                                     // activations of the current and of the next group
+        load_pass(gp0[0], gp1[0], buf[0]);
+#pragma unroll
+        for (int i = 0; i < GPW; ++i) {
+            Pass &cur = buf[NCH == 1 ? i & 1 : 0];
+            if (NCH == 1 && i + 1 < GPW) load_pass(gp0[i + 1 < GPW ? i + 1 : i], gp1[i + 1 < GPW ? i + 1 : i], buf[(i + 1) & 1]);
+            if (NCH != 1 && i > 0) load_pass(gp0[i], gp1[i], cur);
+            for (uint32_t pp = gp0[i]; pp < gp1[i]; pp += 2u) {
+                if (pp != gp0[i]) load_pass(pp, gp1[i], cur);            // further passes of a large group
+                const bool have_b = pp + 1u < gp1[i];
+                float tot_a[2] = {0.0f, 0.0f}, tot_b[2] = {0.0f, 0.0f};
+#pragma unroll
+                for (int c = 0; c < NCH; ++c) {
+#pragma unroll
+                    for (int q = 0; q < 2; ++q) {
+                        const float d = scale_to_f32(wd[i][c] >> (16 * q));
+                        float va, vb;
+                        iq3s_group_dot(wq[i][c][q], cur.ax[c], lds, va, vb);
+                        tot_a[q] += va * d * cur.sa[c];
+                        tot_b[q] += vb * d * cur.sb[c];
+                    }
+                }
+                const float ra = quad_column_reduce<2>(tot_a, lane), rb = quad_column_reduce<2>(tot_b, lane);
+                if (reduced_writer<2>(lane)) {
+                    const uint32_t rr = 4u * reduced_unit<2>(lane) + j;
+                    part[pp * 8u + rr] = ra;
+                    if (have_b) part[(pp + 1u) * 8u + rr] = rb;
+                }
+            }
+        }
+    }
+    __syncthreads();
+    for (uint32_t i = tid; i < a.ntok * 8u; i += kWaves * 64u) {
+        const uint32_t t = i >> 3, r = i & 7u;
+        float sum = 0.0f;
+        for (uint32_t k = 0; k < a.top_k; ++k) {
+            const uint32_t p = a.tok_pair[t * a.top_k + k];
+            sum = fmaf(a.pair_weight[p], part[p * 8u + r], sum);
+        }
+        sum = fmaf(a.scalar[t], part[(P + t) * 8u + r], sum);
+        const uint64_t at = (uint64_t)t * H + row0 + r;
+        a.out[at] = a.resid_a ? (a.resid_a[at] + a.resid_b[at]) + sum : sum;
+    }
+}
+
 // Batched down + combine on raw GGUF rows (mixed layouts): the work split of down_batch_kernel (8 output rows per workgroup, wave w owns
 // the groups w, w + 16, ..., the last group is the shared expert with every token) with the decode of down_combine_raw_kernel. A wave
 // stages the 8 rows of its group in LDS (the next group's rows are requested into registers before the current group is computed),
@@ -2043,7 +2168,8 @@ static hipError_t launch_down_batch_raw_shared(uint32_t ts, const DownBatchRawAr
 // Small batch on a mixed layout, pairs grouped by expert: packed IQ2_XXS gate/up matrices on the batched MFMA kernel (the shared
 // expert's gate / up products come in as shared_gu [ntok][2 ffn]), raw down matrices of any built-in type on the batched raw-row kernel.
 hipError_t launch_batch_mixed(const void *packed, uint64_t packed_stride, const float *shared_gu, uint32_t down_type, uint32_t shared_down_type,
-                              const void *raw_down, uint64_t raw_stride, const void *shared_down, const uint32_t *uid, const uint32_t *expert_start,
+                              const void *raw_down, uint64_t raw_stride, const void *shared_down, const void *words_down, uint64_t words_stride,
+                              const float *dense_down, const uint32_t *uid, const uint32_t *expert_start,
                               const uint32_t *pair_token, const uint32_t *n_unique, const float *pair_weight, const uint32_t *tok_pair,
                               const float *scalar, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l, int *act_exp,
                               float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s) {
@@ -2059,6 +2185,18 @@ hipError_t launch_batch_mixed(const void *packed, uint64_t packed_stride, const 
     hipError_t e = launch_gateup_batch_kernel(a, n_groups, s);
     if (e != hipSuccess) return e;
     prof_set_stage(ST_BATCH_DOWN);
+    if (words_down && dense_down && down_type == T_IQ3_S) {      // word-packed IQ3_S on the matrix units, the shared expert's rows from its f32 copy
+        const BatchWordsArgs w{static_cast<const uint8_t *>(words_down), words_stride, dense_down, uid, expert_start, n_unique, pair_weight, tok_pair, scalar,
+                               static_cast<const _Float16 *>(act_h), static_cast<const _Float16 *>(act_l), act_exp, out, hidden, ffn, top_k, ntok,
+                               block_context().resid_a, block_context().resid_b};
+        const uint32_t groups_per_wave = (n_groups + kWaves - 1u) / kWaves;
+        const dim3 dgrid(hidden / 8u), dblock(kWaves * 64);
+        // (the words take twice the registers of the IQ2_XXS groups: at most three groups of a wave in flight)
+        if (ffn > 512u) REDHIP_LAUNCH((down_batch_words_kernel<144, 2, 1>), dgrid, dblock, 0, s, w);
+        else if (groups_per_wave <= 2u) REDHIP_LAUNCH((down_batch_words_kernel<144, 1, 2>), dgrid, dblock, 0, s, w);
+        else REDHIP_LAUNCH((down_batch_words_kernel<144, 1, 3>), dgrid, dblock, 0, s, w);
+        return hipGetLastError();
+    }
     const DownBatchRawArgs d{static_cast<const uint8_t *>(raw_down), raw_stride, static_cast<const uint8_t *>(shared_down), uid, expert_start, n_unique,
                              pair_weight, tok_pair, scalar, static_cast<const _Float16 *>(act_h), static_cast<const _Float16 *>(act_l), act_exp, out,
                              hidden, ffn, top_k, ntok, block_context().resid_a, block_context().resid_b};

@@ -206,7 +206,8 @@ hipError_t launch_gateup_select(const void *experts, uint64_t stride, const void
 // small batch on a mixed layout with the pairs grouped by expert: batched MFMA gate/up on the packed IQ2_XXS matrices (shared expert's
 // products given), batched raw-row down of the built-in block types; every distinct expert is read once
 hipError_t launch_batch_mixed(const void *packed, uint64_t packed_stride, const float *shared_gu, uint32_t down_type, uint32_t shared_down_type,
-                              const void *raw_down, uint64_t raw_stride, const void *shared_down, const uint32_t *uid, const uint32_t *expert_start,
+                              const void *raw_down, uint64_t raw_stride, const void *shared_down, const void *words_down, uint64_t words_stride,
+                              const float *dense_down, const uint32_t *uid, const uint32_t *expert_start,
                               const uint32_t *pair_token, const uint32_t *n_unique, const float *pair_weight, const uint32_t *tok_pair,
                               const float *scalar, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l, int *act_exp,
                               float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s);

@@ -170,7 +170,7 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
                                       m->tok_pair, m->n_unique, s), "grouping launch");
         }
         HIP_OK(launch_batch_mixed(L.packed, m->packed_stride, m->act, m->dn_type, m->sh_dn_type, L.experts + 2u * m->gate_bytes, m->expert_stride,
-                                  L.shared + 2u * m->sh_gate_bytes, m->uid, m->expert_start, m->pair_token, m->n_unique, m->pair_weight, m->tok_pair,
+                                  L.shared + 2u * m->sh_gate_bytes, L.words_down, m->words_down_stride(), L.dense_down, m->uid, m->expert_start, m->pair_token, m->n_unique, m->pair_weight, m->tok_pair,
                                   m->scalar, m->xh, m->xl, m->xexp, m->act_h, m->act_l, m->act_exp, out, c.hidden, c.ffn, c.top_k, ntok, c.n_expert, s),
                "grouped mixed batch launch");
         prof_set_stage(ST_OTHER);
