@@ -883,11 +883,12 @@ __device__ __forceinline__ float group_dot_fmt(uint2 q, uint32_t sc, const half4
     }
 }
 
-// fp16 copy of a caller-supplied codebook (int8 [entries][8]) in LDS, 16 bytes per entry; built by every wave but the first
+// fp16 copy of a caller-supplied codebook (int8 [entries][8]) in LDS, 16 bytes per entry; built by `builders` lanes starting at lane `first`
+// of the workgroup (the gate/up kernel: every wave but the first, which selects meanwhile)
 template <int FMT>
-__device__ __forceinline__ void build_codebook_table(uint8_t *lds, uint32_t tid, const int8_t *grid) {
+__device__ __forceinline__ void build_codebook_table(uint8_t *lds, uint32_t tid, const int8_t *grid, uint32_t first = 64u, uint32_t builders = (kWaves - 1) * 64u) {
     constexpr uint32_t kEntries = FMT == 1 ? 512u : 2048u;
-    for (uint32_t i = tid - 64u; i < kEntries; i += (kWaves - 1) * 64u) {      // tid < 64 wraps past the bound
+    for (uint32_t i = tid - first; i < kEntries; i += builders) {      // tid < first wraps past the bound
         const uint64_t e = reinterpret_cast<const uint64_t *>(grid)[i];
         uint32_t w4[4];
 #pragma unroll
@@ -1175,6 +1176,68 @@ __global__ __launch_bounds__(kWaves * 64) void down_combine_kernel(DownArgs a) {
     }
 }
 
+// One row of a dense f32 matrix against an activation vector kept as fp16 halves + one exponent per 32 columns: the LPR lanes that
+// share a row take every LPR-th float4 and meet by butterfly adds. Returns the row's product in every one of those lanes.
+template <uint32_t LPR>
+__device__ __forceinline__ float dense_row_dot(const float *row, const _Float16 *ah, const _Float16 *al, const int *aexp, uint32_t F, uint32_t part) {
+    float acc = 0.0f;
+    for (uint32_t c0 = part; c0 < F / 4u; c0 += 8u * LPR) {      // eight float4 per lane and round, all requested before the first is used
+        float4 w[8];
+        uint2 hv[8], lv[8];
+        int ev[8];
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            const uint32_t cr = c0 + LPR * (uint32_t)i, c4 = cr < F / 4u ? cr : F / 4u - 1u;
+            w[i] = reinterpret_cast<const float4 *>(row)[c4];
+            if (cr >= F / 4u) w[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            hv[i] = reinterpret_cast<const uint2 *>(ah)[c4];
+            lv[i] = reinterpret_cast<const uint2 *>(al)[c4];
+            ev[i] = aexp[c4 >> 3];
+        }
+#pragma unroll
+        for (int i = 0; i < 8; ++i) {
+            union { uint2 u; _Float16 h[4]; } hh, ll;
+            hh.u = hv[i];
+            ll.u = lv[i];
+            float t = w[i].x * fmaf((float)ll.h[0], 4.8828125e-4f, (float)hh.h[0]);
+            t = fmaf(w[i].y, fmaf((float)ll.h[1], 4.8828125e-4f, (float)hh.h[1]), t);
+            t = fmaf(w[i].z, fmaf((float)ll.h[2], 4.8828125e-4f, (float)hh.h[2]), t);
+            t = fmaf(w[i].w, fmaf((float)ll.h[3], 4.8828125e-4f, (float)hh.h[3]), t);
+            acc = fmaf(t, exp2i(ev[i]), acc);
+        }
+    }
+#pragma unroll
+    for (uint32_t o = 1u; o < LPR; o <<= 1) acc += __shfl_xor(acc, (int)o, 64);
+    return acc;
+}
+
+// The waves behind the routed ones (wave >= top_k of NW) share the shared expert's 8 output rows, read from its dense f32 copy
+// [hidden][ffn]; the activations are slot top_k of act_h / act_l / act_exp. Row sums go to part[top_k * 8 + row].
+template <int NW>
+__device__ __forceinline__ void shared_rows_dense(const float *shared, uint32_t row0, uint32_t F, uint32_t top_k, const _Float16 *act_h, const _Float16 *act_l,
+                                                  const int *act_exp, uint32_t wave, uint32_t lane, float *part) {
+    const uint32_t spare = (uint32_t)NW - top_k, k = top_k, sw = wave - top_k;
+    const _Float16 *ah = act_h + (uint64_t)k * F, *al = act_l + (uint64_t)k * F;
+    const int *ae = act_exp + k * (F / 32u);
+    if (spare >= 4u) {
+        if (sw < 4u) {
+            const uint32_t row = 2u * sw + (lane >> 5);
+            const float r = dense_row_dot<32>(shared + (uint64_t)(row0 + row) * F, ah, al, ae, F, lane & 31u);
+            if ((lane & 31u) == 0u) part[k * 8u + row] = r;
+        }
+    } else if (spare >= 2u) {
+        if (sw < 2u) {
+            const uint32_t row = 4u * sw + (lane >> 4);
+            const float r = dense_row_dot<16>(shared + (uint64_t)(row0 + row) * F, ah, al, ae, F, lane & 15u);
+            if ((lane & 15u) == 0u) part[k * 8u + row] = r;
+        }
+    } else if (sw == 0u) {
+        const uint32_t row = lane >> 3;
+        const float r = dense_row_dot<8>(shared + (uint64_t)(row0 + row) * F, ah, al, ae, F, lane & 7u);
+        if ((lane & 7u) == 0u) part[k * 8u + row] = r;
+    }
+}
+
 // Down + combine when the down matrices are not IQ2_XXS (mixed-precision layouts: IQ3_S routed, Q6_K shared): same
 // work split as down_combine_kernel (8 rows per workgroup, wave = slot, lane = (32-column chunk, row)), weights
 // decoded from the raw GGUF rows and multiplied in f32 against the activation rebuilt from its fp16 halves.
@@ -1190,6 +1253,7 @@ struct DownRawArgs {
     uint32_t hidden, ffn, top_k;
     const float *resid_a, *resid_b;
     const int8_t *grid;        // the caller's codebook of the routed down format (IQ2_XS, IQ1_M) or nullptr
+    const float *shared_dense; // when set: the shared expert's down matrix as dense f32 [hidden][ffn], read instead of `shared`
 };
 
 template <uint32_t T>
@@ -1237,7 +1301,9 @@ __global__ __launch_bounds__(NW * 64) void down_combine_raw_kernel(DownRawArgs a
     const bool is_shared = wave == a.top_k;
     const uint32_t row_bytes = FB * (is_shared ? Fmt<TS>::kBlock : Fmt<TD>::kBlock);
     uint8_t *mine = raw_rows + wave * 8u * FB * kMaxBlock;
-    if (wave < n_slot) {
+    const uint32_t n_raw = a.shared_dense ? a.top_k : n_slot;      // slots decoded from staged raw rows
+    if (a.shared_dense && wave >= a.top_k) shared_rows_dense<NW>(a.shared_dense, row0, F, a.top_k, a.act_h, a.act_l, a.act_exp, wave, lane, part);
+    if (wave < n_raw) {
         const uint8_t *rows = (is_shared ? a.shared : a.experts + (uint64_t)a.ids[wave] * a.stride) + (uint64_t)row0 * row_bytes;
         wave_stage(mine, rows, 8u * row_bytes, lane);          // 8 rows x FB blocks of 56 .. 210 bytes: a multiple of 16
     }
@@ -1246,7 +1312,7 @@ __global__ __launch_bounds__(NW * 64) void down_combine_raw_kernel(DownRawArgs a
         if (tid + NW * 64u < kGridBytes / 16u) reinterpret_cast<uint4 *>(cb)[tid + NW * 64u] = cb1;
         __syncthreads();
     }
-    if (wave < n_slot) {
+    if (wave < n_raw) {
         float tot[2] = {0.0f, 0.0f};
         for (uint32_t G = blk; G < FG; G += 16u) {
             float av[32];
@@ -1298,12 +1364,12 @@ static hipError_t launch_down_raw_shared(uint32_t ts, const DownRawArgs &a, uint
 hipError_t launch_down_combine_raw(uint32_t down_type, uint32_t shared_down_type, const void *experts, uint64_t stride, const void *shared,
                                    const uint32_t *ids, const float *weights, const float *scalar, const void *act_h, const void *act_l,
                                    const int *act_exp, float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, hipStream_t s, uint32_t ntok,
-                                   const int8_t *grid) {
+                                   const int8_t *grid, const float *shared_dense) {
     if (!hidden || hidden % 8u || !ffn || ffn % 256u || top_k + 1u > (uint32_t)kWaves || !ntok || ntok > 65535u) return hipErrorInvalidValue;
     if ((down_type == T_IQ2_XS || down_type == T_IQ1_M) && !grid) return hipErrorInvalidValue;
     const DownRawArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(shared), ids, weights, scalar,
                         static_cast<const _Float16 *>(act_h), static_cast<const _Float16 *>(act_l), act_exp, out, hidden, ffn, top_k,
-                        block_context().resid_a, block_context().resid_b, grid};
+                        block_context().resid_a, block_context().resid_b, grid, shared_dense};
     switch (down_type) {
         case T_IQ2_XXS: return launch_down_raw_shared<T_IQ2_XXS>(shared_down_type, a, ntok, s);
         case T_IQ3_S: return launch_down_raw_shared<T_IQ3_S>(shared_down_type, a, ntok, s);
@@ -1413,47 +1479,13 @@ __device__ __forceinline__ void iq3s_group_dot(uint4 q, const half4_t *ax, const
     vb = (acc[2] + acc[3] * 4.8828125e-4f) * sc;
 }
 
-// One row of a dense f32 matrix against an activation vector kept as fp16 halves + one exponent per 32 columns: the LPR lanes that
-// share a row take every LPR-th float4 and meet by butterfly adds. Returns the row's product in every one of those lanes.
-template <uint32_t LPR>
-__device__ __forceinline__ float dense_row_dot(const float *row, const _Float16 *ah, const _Float16 *al, const int *aexp, uint32_t F, uint32_t part) {
-    float acc = 0.0f;
-    for (uint32_t c0 = part; c0 < F / 4u; c0 += 8u * LPR) {      // eight float4 per lane and round, all requested before the first is used
-        float4 w[8];
-        uint2 hv[8], lv[8];
-        int ev[8];
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            const uint32_t cr = c0 + LPR * (uint32_t)i, c4 = cr < F / 4u ? cr : F / 4u - 1u;
-            w[i] = reinterpret_cast<const float4 *>(row)[c4];
-            if (cr >= F / 4u) w[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
-            hv[i] = reinterpret_cast<const uint2 *>(ah)[c4];
-            lv[i] = reinterpret_cast<const uint2 *>(al)[c4];
-            ev[i] = aexp[c4 >> 3];
-        }
-#pragma unroll
-        for (int i = 0; i < 8; ++i) {
-            union { uint2 u; _Float16 h[4]; } hh, ll;
-            hh.u = hv[i];
-            ll.u = lv[i];
-            float t = w[i].x * fmaf((float)ll.h[0], 4.8828125e-4f, (float)hh.h[0]);
-            t = fmaf(w[i].y, fmaf((float)ll.h[1], 4.8828125e-4f, (float)hh.h[1]), t);
-            t = fmaf(w[i].z, fmaf((float)ll.h[2], 4.8828125e-4f, (float)hh.h[2]), t);
-            t = fmaf(w[i].w, fmaf((float)ll.h[3], 4.8828125e-4f, (float)hh.h[3]), t);
-            acc = fmaf(t, exp2i(ev[i]), acc);
-        }
-    }
-#pragma unroll
-    for (uint32_t o = 1u; o < LPR; o <<= 1) acc += __shfl_xor(acc, (int)o, 64);
-    return acc;
-}
-
 // Down + combine of one token on a mixed layout whose routed down matrices are word-packed IQ3_S: 8 output rows per workgroup, wave s <
 // top_k owns the selected expert s (both row quads against all ffn columns, as down_combine_kernel), wave top_k the shared expert, read
 // from its dense f32 copy [hidden][ffn]. blockIdx.y = token (small batches run one grid layer per token).
 struct DownWordsArgs {
-    const uint8_t *experts;    // word-packed down matrix of expert e at experts + e * stride
+    const uint8_t *experts;    // word-packed (IQ3_S) or stream-packed (IQ2_XS, IQ1_M: as their gate / up matrices) down matrix of expert e at experts + e * stride
     uint64_t stride;
+    const int8_t *grid;        // the caller's codebook of IQ2_XS / IQ1_M down matrices
     const float *shared;       // dense f32 down matrix of the shared expert
     const uint32_t *ids;
     const float *weights, *scalar;
@@ -1464,9 +1496,9 @@ struct DownWordsArgs {
     const float *resid_a, *resid_b;
 };
 
-template <int NW>
+template <int NW, int FMT>       // FMT: 0 word-packed IQ3_S, 1 stream-packed IQ2_XS, 2 stream-packed IQ1_M
 __global__ __launch_bounds__(NW * 64) void down_combine_words_kernel(DownWordsArgs a) {
-    __shared__ __attribute__((aligned(16))) uint8_t lds[kIq3TableBytes];
+    __shared__ __attribute__((aligned(16))) uint8_t lds[FMT == 0 ? kIq3TableBytes : FMT == 1 ? 512u * 16u : 2048u * 16u];
     __shared__ float part[17 * 8];
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
     const uint32_t F = a.ffn, FG = F / 32u, FB = F / 256u, n_slot = a.top_k + 1u;
@@ -1483,21 +1515,30 @@ __global__ __launch_bounds__(NW * 64) void down_combine_words_kernel(DownWordsAr
     }
     const uint32_t row0 = 8u * blockIdx.x;
     const uint32_t n_chunk = (FG + 15u) / 16u;         // ffn <= 1024
-    uint4 dq[2][2];
+    uint4 dq[2][2];            // IQ2_XS / IQ1_M: x, y = the group's uint2, z = the IQ2_XS scale byte
     uint32_t dd[2][2];
     half4_t ax[2][8];
     float sc[2] = {0.0f, 0.0f};
     const bool routed = wave < a.top_k;
     if (routed) {
         const uint8_t *ex = a.experts + (uint64_t)a.ids[wave] * a.stride;
-        const uint4 *qs = reinterpret_cast<const uint4 *>(ex);                                            // [hidden][FG]
-        const uint16_t *ds = reinterpret_cast<const uint16_t *>(ex + (uint64_t)a.hidden * FG * 16u);      // [hidden][FB]
+        constexpr uint32_t kGroupBytes = FMT == 0 ? 16u : 8u;
+        const uint16_t *ds = reinterpret_cast<const uint16_t *>(ex + (uint64_t)a.hidden * FG * kGroupBytes);      // [hidden][FB]
+        const uint8_t *scs = ex + (uint64_t)a.hidden * FG * kGroupBytes + (uint64_t)a.hidden * FB * 2u;           // IQ2_XS: [hidden][FG]
 #pragma unroll
         for (int q = 0; q < 2; ++q)
 #pragma unroll
             for (int c = 0; c < 2; ++c) {
                 const uint32_t r = row0 + 4u * q + j, G = 16u * c + blk;
-                if ((uint32_t)c < n_chunk && G < FG) { dq[q][c] = qs[(uint64_t)r * FG + G]; dd[q][c] = ds[(uint64_t)r * FB + (G >> 3)]; }
+                if ((uint32_t)c < n_chunk && G < FG) {
+                    if constexpr (FMT == 0) {
+                        dq[q][c] = reinterpret_cast<const uint4 *>(ex)[(uint64_t)r * FG + G];
+                    } else {
+                        const uint2 v = reinterpret_cast<const uint2 *>(ex)[(uint64_t)r * FG + G];
+                        dq[q][c] = make_uint4(v.x, v.y, FMT == 1 ? (uint32_t)scs[(uint64_t)r * FG + G] : 0u, 0u);
+                    }
+                    dd[q][c] = ds[(uint64_t)r * FB + (G >> 3)];
+                }
             }
 #pragma unroll
         for (int c = 0; c < 2; ++c) {
@@ -1507,29 +1548,11 @@ __global__ __launch_bounds__(NW * 64) void down_combine_words_kernel(DownWordsAr
                 sc[c] = exp2i(a.act_exp[wave * FG + G]);
             }
         }
-    } else {                                           // the waves behind the routed ones share the shared expert's 8 rows
-        const uint32_t spare = (uint32_t)NW - a.top_k, k = a.top_k, sw = wave - a.top_k;
-        const _Float16 *ah = a.act_h + (uint64_t)k * F, *al = a.act_l + (uint64_t)k * F;
-        const int *ae = a.act_exp + k * FG;
-        if (spare >= 4u) {
-            if (sw < 4u) {
-                const uint32_t row = 2u * sw + (lane >> 5);
-                const float r = dense_row_dot<32>(a.shared + (uint64_t)(row0 + row) * F, ah, al, ae, F, lane & 31u);
-                if ((lane & 31u) == 0u) part[k * 8u + row] = r;
-            }
-        } else if (spare >= 2u) {
-            if (sw < 2u) {
-                const uint32_t row = 4u * sw + (lane >> 4);
-                const float r = dense_row_dot<16>(a.shared + (uint64_t)(row0 + row) * F, ah, al, ae, F, lane & 15u);
-                if ((lane & 15u) == 0u) part[k * 8u + row] = r;
-            }
-        } else if (sw == 0u) {
-            const uint32_t row = lane >> 3;
-            const float r = dense_row_dot<8>(a.shared + (uint64_t)(row0 + row) * F, ah, al, ae, F, lane & 7u);
-            if ((lane & 7u) == 0u) part[k * 8u + row] = r;
-        }
+    } else {
+        shared_rows_dense<NW>(a.shared, row0, F, a.top_k, a.act_h, a.act_l, a.act_exp, wave, lane, part);
     }
-    build_iq3s_quads(lds, tid);
+    if constexpr (FMT == 0) build_iq3s_quads(lds, tid);
+    else build_codebook_table<FMT>(lds, tid, a.grid, 0u, (uint32_t)NW * 64u);
     __syncthreads();
     if (routed) {
         float tot[2] = {0.0f, 0.0f};
@@ -1540,7 +1563,8 @@ __global__ __launch_bounds__(NW * 64) void down_combine_words_kernel(DownWordsAr
 #pragma unroll
                 for (int q = 0; q < 2; ++q) {
                     float va, vb;
-                    iq3s_group_dot(dq[q][c], ax[c], lds, va, vb);
+                    if constexpr (FMT == 0) iq3s_group_dot(dq[q][c], ax[c], lds, va, vb);
+                    else va = group_dot_fmt<FMT>(make_uint2(dq[q][c].x, dq[q][c].y), dq[q][c].z, ax[c], lds) * (FMT == 1 ? 0.125f : 1.0f);
                     tot[q] += va * scale_to_f32(dd[q][c]) * sc[c];
                 }
             }
@@ -1557,15 +1581,27 @@ __global__ __launch_bounds__(NW * 64) void down_combine_words_kernel(DownWordsAr
     }
 }
 
-hipError_t launch_down_combine_words(const void *experts, uint64_t stride, const float *shared_dense, const uint32_t *ids, const float *weights,
-                                     const float *scalar, const void *act_h, const void *act_l, const int *act_exp, float *out, uint32_t hidden,
-                                     uint32_t ffn, uint32_t top_k, hipStream_t s, uint32_t ntok) {
+hipError_t launch_down_combine_words(uint32_t down_type, const int8_t *grid, const void *experts, uint64_t stride, const float *shared_dense, const uint32_t *ids,
+                                     const float *weights, const float *scalar, const void *act_h, const void *act_l, const int *act_exp, float *out,
+                                     uint32_t hidden, uint32_t ffn, uint32_t top_k, hipStream_t s, uint32_t ntok) {
     if (!hidden || hidden % 8u || !ffn || ffn % 256u || ffn > 1024u || top_k + 1u > (uint32_t)kWaves || !ntok || ntok > 65535u || !shared_dense) return hipErrorInvalidValue;
-    const DownWordsArgs a{static_cast<const uint8_t *>(experts), stride, shared_dense, ids, weights, scalar, static_cast<const _Float16 *>(act_h),
+    if ((down_type == T_IQ2_XS || down_type == T_IQ1_M) && !grid) return hipErrorInvalidValue;
+    const DownWordsArgs a{static_cast<const uint8_t *>(experts), stride, grid, shared_dense, ids, weights, scalar, static_cast<const _Float16 *>(act_h),
                           static_cast<const _Float16 *>(act_l), act_exp, out, hidden, ffn, top_k, block_context().resid_a, block_context().resid_b};
-    const dim3 grid(hidden / 8u, ntok);
-    if (top_k + 1u <= 12u) REDHIP_LAUNCH(down_combine_words_kernel<12>, grid, dim3(12 * 64), 0, s, a);
-    else REDHIP_LAUNCH(down_combine_words_kernel<kWaves>, grid, dim3(kWaves * 64), 0, s, a);
+    const dim3 grid_dim(hidden / 8u, ntok);
+    const bool narrow = top_k + 1u <= 12u;
+#define REDHIP_DCW(FMT)                                                                                              \
+    do {                                                                                                             \
+        if (narrow) REDHIP_LAUNCH((down_combine_words_kernel<12, FMT>), grid_dim, dim3(12 * 64), 0, s, a);           \
+        else REDHIP_LAUNCH((down_combine_words_kernel<kWaves, FMT>), grid_dim, dim3(kWaves * 64), 0, s, a);          \
+    } while (0)
+    switch (down_type) {
+        case T_IQ3_S: REDHIP_DCW(0); break;
+        case T_IQ2_XS: REDHIP_DCW(1); break;
+        case T_IQ1_M: REDHIP_DCW(2); break;
+        default: return hipErrorInvalidValue;
+    }
+#undef REDHIP_DCW
     return hipGetLastError();
 }
 

@@ -216,14 +216,15 @@ hipError_t launch_repack_iq3s_words(const void *raw, uint64_t raw_stride, uint32
 hipError_t launch_dequant_iq3s_words(const void *packed, uint32_t nrows, uint32_t K, float *out, hipStream_t s);
 inline uint64_t iq3s_words_bytes(uint32_t nrows, uint32_t K) { return (uint64_t)nrows * ((uint64_t)(K / 32u) * 16u + (uint64_t)(K / 256u) * 2u); }
 // down + combine of one token (ntok > 1: one grid layer per token) on word-packed IQ3_S routed matrices and the shared expert's dense f32 copy
-hipError_t launch_down_combine_words(const void *experts, uint64_t stride, const float *shared_dense, const uint32_t *ids, const float *weights,
-                                     const float *scalar, const void *act_h, const void *act_l, const int *act_exp, float *out, uint32_t hidden,
-                                     uint32_t ffn, uint32_t top_k, hipStream_t s, uint32_t ntok = 1u);
+// (IQ2_XS / IQ1_M down matrices: the streams of launch_repack_gateup and the caller's codebook)
+hipError_t launch_down_combine_words(uint32_t down_type, const int8_t *grid, const void *experts, uint64_t stride, const float *shared_dense, const uint32_t *ids,
+                                     const float *weights, const float *scalar, const void *act_h, const void *act_l, const int *act_exp, float *out,
+                                     uint32_t hidden, uint32_t ffn, uint32_t top_k, hipStream_t s, uint32_t ntok = 1u);
 // down + weighted combine for layouts whose down matrices are raw GGUF rows of any supported type
 hipError_t launch_down_combine_raw(uint32_t down_type, uint32_t shared_down_type, const void *experts, uint64_t stride, const void *shared,
                                    const uint32_t *ids, const float *weights, const float *scalar, const void *act_h, const void *act_l,
                                    const int *act_exp, float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, hipStream_t s, uint32_t ntok = 1u,
-                                   const int8_t *grid = nullptr);
+                                   const int8_t *grid = nullptr, const float *shared_dense = nullptr);
 // single token: out[r] = sum_k weights[k] * down_{ids[k]}[r] . act[k] + scalar * shared_down[r] . act[top_k], k in order
 hipError_t launch_down_combine(const void *experts, uint64_t stride, const void *shared, const uint32_t *ids, const float *weights,
                                const float *scalar, const void *act_h, const void *act_l, const int *act_exp, float *out,

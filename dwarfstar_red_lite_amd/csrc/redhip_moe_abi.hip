@@ -78,7 +78,9 @@ struct Moe {
     bool tiles_resident() const { return packed_gu() && gu_type == T_IQ2_XXS && cfg.max_tokens > 8u && cfg.ffn <= 512u && cfg.hidden / 512u <= 4u; }
     // a chunk on a mixed layout: the routed gate/up matrices (packed IQ2_XXS) run on the prefill tiles, the rest on raw rows
     bool mixed_chunk(uint32_t ntok) const { return mixed && ntok > 8u && tiles_resident(); }
-    uint64_t words_down_stride() const { return (iq3s_words_bytes(cfg.hidden, cfg.ffn) + 255u) & ~255ull; }
+    uint64_t words_down_stride() const {
+        return ((dn_type == T_IQ3_S ? iq3s_words_bytes(cfg.hidden, cfg.ffn) : packed_matrix_bytes(dn_type, cfg.hidden, cfg.ffn)) + 255u) & ~255ull;
+    }
     uint64_t tiled_down_stride() const { return ((uint64_t)cfg.hidden * (cfg.ffn / 32u) * 16u + (uint64_t)cfg.hidden * (cfg.ffn / 256u) * 2u + 255u) & ~255ull; }
     // the one-launch router kernels (logits of every expert + the shared expert's gate logit, optional residual + norm) and the
     // one-wave selection serve every layout whose router they tile; the per-row GEMV + generic selection are what is left
@@ -248,12 +250,12 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
             HIP_OK(launch_down_combine(L.packed, m->expert_stride, L.shared_packed, select_here ? m->ids : ids, select_here ? m->weights : weights,
                                        m->scalar, m->act_h, m->act_l, m->act_exp, out, c.hidden, c.ffn, c.top_k, s), "down/combine launch");
         else if (L.words_down && L.dense_down)
-            HIP_OK(launch_down_combine_words(L.words_down, m->words_down_stride(), L.dense_down, select_here ? m->ids : ids, select_here ? m->weights : weights,
+            HIP_OK(launch_down_combine_words(m->dn_type, m->dn_grid, L.words_down, m->words_down_stride(), L.dense_down, select_here ? m->ids : ids, select_here ? m->weights : weights,
                                              m->scalar, m->act_h, m->act_l, m->act_exp, out, c.hidden, c.ffn, c.top_k, s, ntok), "down/combine launch");
         else
             HIP_OK(launch_down_combine_raw(m->dn_type, m->sh_dn_type, L.experts + 2u * m->gate_bytes, m->expert_stride, L.shared + 2u * m->sh_gate_bytes,
                                            select_here ? m->ids : ids, select_here ? m->weights : weights, m->scalar, m->act_h, m->act_l,
-                                           m->act_exp, out, c.hidden, c.ffn, c.top_k, s, ntok, m->dn_grid), "down/combine launch");
+                                           m->act_exp, out, c.hidden, c.ffn, c.top_k, s, ntok, m->dn_grid, L.dense_down), "down/combine launch");
         prof_set_stage(ST_OTHER);
         return 1;
     }
@@ -348,7 +350,7 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
                 m->resident += align256(rb) + align256(gb) + align256(db);
             }
         }
-        if (ok && m->mixed && dn == T_IQ3_S && c.ffn <= 1024u) {
+        if (ok && m->mixed && (dn == T_IQ3_S || dn == T_IQ2_XS || dn == T_IQ1_M) && c.ffn <= 1024u) {
             ok = hipMalloc(reinterpret_cast<void **>(&L.words_down), (size_t)c.n_expert * m->words_down_stride()) == hipSuccess;
             m->resident += (uint64_t)c.n_expert * m->words_down_stride();
         }
@@ -530,9 +532,11 @@ static int stage_and_pack(Moe *m, uint32_t layer, uint32_t first, uint32_t count
             if (m->fused)
                 HIP_OK(launch_tile_packed(pk + 2u * m->gate_bytes, m->packed_stride, count, c.hidden, c.ffn, tl + 2u * m->gate_bytes, m->packed_stride, nullptr), "expert down tiling");
         }
-        if (m->layers[layer].words_down)
-            HIP_OK(launch_repack_iq3s_words(dst + 2u * m->gate_bytes, m->expert_stride, count, c.hidden, c.ffn,
-                                            m->layers[layer].words_down + (uint64_t)first * m->words_down_stride(), m->words_down_stride(), nullptr), "expert down words");
+        if (m->layers[layer].words_down) {
+            uint8_t *wd = m->layers[layer].words_down + (uint64_t)first * m->words_down_stride();
+            if (m->dn_type == T_IQ3_S) HIP_OK(launch_repack_iq3s_words(dst + 2u * m->gate_bytes, m->expert_stride, count, c.hidden, c.ffn, wd, m->words_down_stride(), nullptr), "expert down words");
+            else HIP_OK(launch_repack_gateup(m->dn_type, dst + 2u * m->gate_bytes, m->expert_stride, count, c.hidden, c.ffn, wd, m->words_down_stride(), nullptr), "expert down streams");
+        }
         if (m->layers[layer].tiled_down)
             HIP_OK(launch_tile_iq3s(dst + 2u * m->gate_bytes, m->expert_stride, count, c.hidden, c.ffn,
                                     m->layers[layer].tiled_down + (uint64_t)first * m->tiled_down_stride(), m->tiled_down_stride(), nullptr), "expert down tiling");
@@ -737,7 +741,9 @@ int redhip_moe_dequant_resident(redhip_moe_t h, uint32_t layer, uint32_t expert,
         return 1;
     }
     if (which == 2u && !sh && L.words_down) {       // the copy the MFMA down kernels read
-        HIP_OK(launch_dequant_iq3s_words(L.words_down + (uint64_t)expert * m->words_down_stride(), c.hidden, c.ffn, out_dev, s), "word-packed down dequant");
+        const uint8_t *wd = L.words_down + (uint64_t)expert * m->words_down_stride();
+        if (m->dn_type == T_IQ3_S) HIP_OK(launch_dequant_iq3s_words(wd, c.hidden, c.ffn, out_dev, s), "word-packed down dequant");
+        else HIP_OK(launch_dequant_packed(m->dn_type, wd, c.hidden, c.ffn, m->dn_grid, out_dev, s), "stream-packed down dequant");
         return 1;
     }
     const uint8_t *base = sh ? L.shared : L.experts + (uint64_t)expert * m->expert_stride;
