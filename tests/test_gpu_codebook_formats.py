@@ -192,3 +192,36 @@ def test_resident_layer(layout, shape, grids):
             assert ids_match_up_to_ties(gids[i], cids[i], clog[i])
             assert rel_l2(out[i], want[i]) <= REL_L2_TOL, (layout, shape, ntok, i)
     m.close()
+
+
+@pytest.mark.parametrize("layout", ["f2", "xs", "m"])
+@pytest.mark.parametrize("shape", [(1024, 768, 24, 12), (4096, 1024, 16, 2), (512, 256, 16, 4)])
+def test_mixed_layouts_other_shapes(layout, shape, grids):
+    """mixed-precision layers away from the benchmark shape: 13 slots (the 16-wave kernels), ffn 768 / 1024 (two column chunks per
+    lane), hidden 512 .. 4096; one token, a pair, grouped batches, with dequantisation from the copies the kernels read"""
+    from dwarfstar_red_lite_amd.moe import ResidentMoe
+    from test_gpu_moe_layer import ids_match_up_to_ties
+    orc.set_codebooks(*grids)
+    H, F, E, K = shape
+    cfg = synth.layer_config(hidden=H, ffn=F, n_expert=E, top_k=K, layout=layout)
+    m = ResidentMoe(cfg, n_layer=1, max_tokens=8)
+    lay = synth.make_layer(90 + H + F, cfg)
+    m.load_layer(0, lay)
+    ref = orc.Layer(cfg, **lay)
+    for e, which in ((1, 0), (E - 1, 1), (E // 2, 2), (0, 2)):
+        t = cfg["gate_up_type" if which < 2 else "down_type"]
+        want = orc.dequant_rows(t, lay[("gate", "up", "down")[which]][e].reshape(-1), H if which < 2 else F)
+        got = m.dequant_resident(0, e, which).cpu().numpy()
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (layout, shape, e, which)
+    xs = synth.normed_x(np.random.default_rng(17), 8, H)
+    xs[5] = xs[1]                                        # two requests with the same row: groups of two pairs
+    for ntok in (1, 2, 5, 8):
+        out = m.forward(0, torch.from_numpy(xs[:ntok].copy()).cuda()).cpu().numpy()
+        gids, gw, glog = m.last_route(ntok)
+        want, cids, cw, clog = ref.forward(xs[:ntok], threads=8)
+        for i in range(ntok):
+            assert ids_match_up_to_ties(gids[i], cids[i], clog[i])
+            assert rel_l2(out[i], want[i]) <= REL_L2_TOL, (layout, shape, ntok, i)
+        if ntok == 8:
+            assert np.array_equal(out[5], out[1])
+    m.close()
