@@ -854,11 +854,11 @@ __device__ __forceinline__ float group_dot(uint2 q, const half4_t *ax, const uin
 // `sc`) and the packed IQ1_M group (FMT 2: 11-bit indices into the caller's 2048-entry codebook of -1 / 0 / 1, plus or minus 1/8 per
 // eight weights added as packed fp16, exact; 3-bit scales per 16 weights in q.y). `lds` is the fp16 copy of the codebook.
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+// va: the product with the token in rows 0, 1 (hi, lo) of the activation operand, vb: with the one in rows 2, 3 (if any)
 template <int FMT>
-__device__ __forceinline__ float group_dot_fmt(uint2 q, uint32_t sc, const half4_t *ax, const uint8_t *lds) {
-    if constexpr (FMT == 0) {
-        return group_dot(q, ax, lds);
-    } else {
+__device__ __forceinline__ void group_dot_fmt2(uint2 q, uint32_t sc, const half4_t *ax, const uint8_t *lds, float &va, float &vb) {
+    static_assert(FMT == 1 || FMT == 2, "codebook formats");
+    {
         float4_t acc[2] = {{0.0f, 0.0f, 0.0f, 0.0f}, {0.0f, 0.0f, 0.0f, 0.0f}};
 #pragma unroll
         for (uint32_t l = 0; l < 4u; ++l) {
@@ -879,7 +879,19 @@ __device__ __forceinline__ float group_dot_fmt(uint2 q, uint32_t sc, const half4
             acc[l >> 1] = __builtin_amdgcn_mfma_f32_4x4x4f16(ax[2u * l + 1u], b1.h, acc[l >> 1], 0, 0, 0);
         }
         const uint32_t s0 = FMT == 1 ? (sc & 15u) : ((q.y >> 16) & 7u), s1 = FMT == 1 ? (sc >> 4) : ((q.y >> 19) & 7u);
-        return (acc[0][0] + acc[0][1] * 4.8828125e-4f) * (float)(2u * s0 + 1u) + (acc[1][0] + acc[1][1] * 4.8828125e-4f) * (float)(2u * s1 + 1u);
+        const float f0 = (float)(2u * s0 + 1u), f1 = (float)(2u * s1 + 1u);
+        va = (acc[0][0] + acc[0][1] * 4.8828125e-4f) * f0 + (acc[1][0] + acc[1][1] * 4.8828125e-4f) * f1;
+        vb = (acc[0][2] + acc[0][3] * 4.8828125e-4f) * f0 + (acc[1][2] + acc[1][3] * 4.8828125e-4f) * f1;
+    }
+}
+template <int FMT>
+__device__ __forceinline__ float group_dot_fmt(uint2 q, uint32_t sc, const half4_t *ax, const uint8_t *lds) {
+    if constexpr (FMT == 0) {
+        return group_dot(q, ax, lds);
+    } else {
+        float va, vb;
+        group_dot_fmt2<FMT>(q, sc, ax, lds, va, vb);
+        return va;
     }
 }
 
@@ -1737,6 +1749,7 @@ struct BatchArgs {
     uint32_t hidden, ffn, top_k, ntok;
     const float *resid_a, *resid_b;     // when set: out = (resid_a + resid_b) + layer output, [ntok][hidden] each
     const float *shared_gu;             // shared == nullptr: the shared expert's gate . x and up . x, [ntok][2 ffn] f32, already computed
+    const int8_t *grid;                 // the caller's codebook when the gate / up matrices are IQ2_XS / IQ1_M streams
 };
 
 // Persistent workgroups walk the units (u, g) = (group of pairs, 32 FFN columns): 32 gate + 32 up rows of the
@@ -1746,12 +1759,13 @@ struct BatchArgs {
 constexpr int kMaxUnits = 16;      // units per workgroup
 constexpr int kMaxTok = 8;         // tokens of a small batch
 
-template <int NKC, int NTP>
+template <int NKC, int NTP, int FMT = 0>      // FMT: 0 IQ2_XXS, 1 IQ2_XS, 2 IQ1_M streams (the latter two: one token pair per pass, no packed shared expert)
 __global__ __launch_bounds__(kWaves * 64) void gateup_batch_kernel(BatchArgs a) {
     constexpr int NW = kWaves;
     constexpr int UPW = 16 * NKC / NW;
+    static_assert(FMT == 0 || NTP == 1, "the codebook formats run one token pair per pass");
     extern __shared__ __attribute__((aligned(16))) uint8_t dyn[];                  // activation planes of all tokens
-    __shared__ __attribute__((aligned(16))) uint8_t lds[kMagBytes];
+    __shared__ __attribute__((aligned(16))) uint8_t lds[FMT == 0 ? kMagBytes : FMT == 1 ? 512u * 16u : 2048u * 16u];
     __shared__ float part[2][2 * NTP][NKC * 64];                                   // alternating between passes
     __shared__ uint32_t meta_expert[kMaxUnits], meta_p0[kMaxUnits], meta_n[kMaxUnits];
     __shared__ uint8_t meta_tok[kMaxUnits][kMaxTok];
@@ -1759,7 +1773,7 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_batch_kernel(BatchArgs a) 
     const uint32_t tid = threadIdx.x, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t H = a.hidden, F = a.ffn, HG = H / 32u, HB = H / 256u, FG = F / 32u, P = a.ntok * a.top_k;
-    const uint64_t grid_entry = tid < 256u ? redhip_iq2xxs_grid[tid] : 0ull;
+    const uint64_t grid_entry = FMT == 0 && tid < 256u ? redhip_iq2xxs_grid[tid] : 0ull;
     const uint32_t U = a.n_unique[0], n_units = (U + 1u) * FG;
     uint32_t count = 0u;
     if (blockIdx.x < n_units) count = (n_units - blockIdx.x + gridDim.x - 1u) / gridDim.x;
@@ -1779,7 +1793,7 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_batch_kernel(BatchArgs a) 
         meta_n[tid] = sh && !a.shared ? 0u : p1 - p0;      // a shared expert that is not packed has no passes: its products are an input
         for (uint32_t i = 0; i < p1 - p0 && i < (uint32_t)kMaxTok; ++i) meta_tok[tid][i] = (uint8_t)(sh ? i : a.pair_token[p0 + i]);
     }
-    if (tid >= 64u && tid < 64u + a.ntok) tok_scale[tid - 64u] = 0.125f * exp2i(a.xexp[tid - 64u]);
+    if (tid >= 64u && tid < 64u + a.ntok) tok_scale[tid - 64u] = (FMT == 2 ? 1.0f : 0.125f) * exp2i(a.xexp[tid - 64u]);
     for (uint32_t i = tid; i < a.ntok * H / 8u; i += NW * 64u) {
         const uint32_t t = i / (H / 8u), c = i % (H / 8u), at = (2u * (c & 3u)) * SS + 2u * t * PLS + (c >> 2);
         const uint4 vh = reinterpret_cast<const uint4 *>(a.xh)[i], vl = reinterpret_cast<const uint4 *>(a.xl)[i];
@@ -1789,15 +1803,16 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_batch_kernel(BatchArgs a) 
         xs[at + PLS + SS] = make_uint2(vl.z, vl.w);
     }
     for (uint32_t i = tid; i < 8u * PLS; i += NW * 64u) xs[(i / PLS) * SS + ZP * PLS + i % PLS] = make_uint2(0u, 0u);
-    build_tables(lds, tid, grid_entry);
+    if constexpr (FMT == 0) build_tables(lds, tid, grid_entry);
+    else build_codebook_table<FMT>(lds, tid, a.grid, 0u, NW * 64u);
     __syncthreads();
 
-    const uint64_t qs_bytes = (uint64_t)F * HG * 8u, gate_bytes = qs_bytes + (uint64_t)F * HB * 2u;
+    const uint64_t qs_bytes = (uint64_t)F * HG * 8u, sc_off = qs_bytes + (uint64_t)F * HB * 2u, gate_bytes = sc_off + (FMT == 1 ? (uint64_t)F * HG : 0u);
     const uint32_t kc = wave % NKC, q0 = wave / NKC;              // wave-uniform: they stay in scalar registers
     const uint32_t G = 16u * kc + blk;
     const uint32_t lane_q = (j * HG + blk) * 8u, lane_d = (j * HB + (blk >> 3)) * 2u;
     uint2 wq[UPW], wq_next[UPW];
-    uint32_t wd[UPW], wd_next[UPW];
+    uint32_t wd[UPW], wd_next[UPW];               // bits 0-15: d; IQ2_XS: bits 16-23 the group's scale byte
     // uniform row base + one lane offset for all units of the wave
     auto load_weights = [&](uint32_t k, uint2 *q, uint32_t *d) {
         const uint32_t g = (blockIdx.x + k * gridDim.x) % FG;
@@ -1810,6 +1825,7 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_batch_kernel(BatchArgs a) 
             const uint8_t *mat = ex + (quad < 8u ? 0u : gate_bytes);
             q[un] = *reinterpret_cast<const uint2 *>(mat + ((uint64_t)row * HG + 16u * kc) * 8u + lane_q);
             d[un] = *reinterpret_cast<const uint16_t *>(mat + qs_bytes + ((uint64_t)row * HB + 2u * kc) * 2u + lane_d);
+            if constexpr (FMT == 1) d[un] |= (uint32_t)(mat + sc_off)[(uint64_t)row * HG + 16u * kc + (lane_q >> 3)] << 16;
         }
     };
     load_weights(0u, wq, wd);
@@ -1844,14 +1860,20 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_batch_kernel(BatchArgs a) 
                 q[un] = wq[un];
                 asm volatile("" : "+v"(q[un].x), "+v"(q[un].y));   // table addresses are formed here, not hoisted out of the pass loop
             }
+            if constexpr (FMT == 0) {
 #pragma unroll
-            for (int un = 0; un < kAhead; ++un) group_lookup(q[un], lds, m[un]);
+                for (int un = 0; un < kAhead; ++un) group_lookup(q[un], lds, m[un]);
+            }
 #pragma unroll
             for (int un = 0; un < UPW; ++un) {
-                if (un + kAhead < UPW) group_lookup(q[un + kAhead], lds, m[un + kAhead]);
                 float va[NTP], vb[NTP];
-                group_consume<NTP>(q[un], m[un], ax, va, vb);
-                const float d = scale_to_f32(wd[un]);
+                if constexpr (FMT == 0) {
+                    if (un + kAhead < UPW) group_lookup(q[un + kAhead], lds, m[un + kAhead]);
+                    group_consume<NTP>(q[un], m[un], ax, va, vb);
+                } else {
+                    group_dot_fmt2<FMT>(q[un], wd[un] >> 16, ax[0], lds, va[0], vb[0]);
+                }
+                const float d = scale_to_f32(wd[un] & 0xffffu);
 #pragma unroll
                 for (int t = 0; t < NTP; ++t) { v[2 * t][un] = va[t] * d; v[2 * t + 1][un] = vb[t] * d; }
             }
@@ -2008,11 +2030,12 @@ __global__ __launch_bounds__(kWaves * 64) void down_batch_kernel(BatchArgs a) {
     }
 }
 
-// The same kernel for mixed layouts whose routed down matrices are word-packed IQ3_S; the shared expert's rows come from its dense f32
-// copy (token t's product on wave 15 - t, ahead of that wave's routed groups).
+// The same kernel with the shared expert's rows taken from its dense f32 copy (token t's product on wave 15 - t, ahead of that wave's
+// routed groups), for routed down matrices that are word-packed IQ3_S (FMT 0), IQ2_XS / IQ1_M streams (1 / 2) or IQ2_XXS streams (3).
 struct BatchWordsArgs {
-    const uint8_t *experts;    // word-packed down matrix of expert e at experts + e * stride
+    const uint8_t *experts;    // packed down matrix of expert e at experts + e * stride
     uint64_t stride;
+    const int8_t *grid;        // the caller's codebook (IQ2_XS / IQ1_M)
     const float *shared;       // dense f32 [hidden][ffn]
     const uint32_t *uid, *expert_start, *n_unique;
     const float *pair_weight;
@@ -2025,15 +2048,16 @@ struct BatchWordsArgs {
     const float *resid_a, *resid_b;
 };
 
-template <int MAXPAIR, int NCH, int GPW>     // GPW: groups of a wave whose weights are in registers at once
+template <int MAXPAIR, int NCH, int GPW, int FMT>     // GPW: groups of a wave whose weights are in registers at once
 __global__ __launch_bounds__(kWaves * 64) void down_batch_words_kernel(BatchWordsArgs a) {
-    __shared__ __attribute__((aligned(16))) uint8_t lds[kIq3TableBytes];
+    __shared__ __attribute__((aligned(16))) uint8_t lds[FMT == 0 ? kIq3TableBytes : FMT == 1 ? 512u * 16u : FMT == 2 ? 2048u * 16u : kMagBytes];
     __shared__ float part[MAXPAIR * 8];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t H = a.hidden, F = a.ffn, FG = F / 32u, FB = F / 256u, P = a.ntok * a.top_k;
     const uint32_t row0 = 8u * blockIdx.x, U = __builtin_amdgcn_readfirstlane(a.n_unique[0]);
-    const uint64_t qs_bytes = (uint64_t)H * FG * 16u;
+    const uint64_t qs_bytes = (uint64_t)H * FG * (FMT == 0 ? 16u : 8u), sc_off = qs_bytes + (uint64_t)H * FB * 2u;      // IQ2_XS: scale bytes [hidden][FG] behind d
+    const uint64_t grid_entry = FMT == 3 && tid < 256u ? redhip_iq2xxs_grid[tid] : 0ull;
 
     uint4 wq[GPW][NCH][2];
     uint32_t wd[GPW][NCH], gp0[GPW], gp1[GPW];      // wd: the two rows' block scales, 16 bits each
@@ -2055,7 +2079,12 @@ __global__ __launch_bounds__(kWaves * 64) void down_batch_words_kernel(BatchWord
 #pragma unroll
                 for (int q = 0; q < 2; ++q) {
                     const uint32_t r = row0 + 4u * (uint32_t)q + j;
-                    wq[i][c][q] = reinterpret_cast<const uint4 *>(dn)[(uint64_t)r * FG + Gc];
+                    if constexpr (FMT == 0) {
+                        wq[i][c][q] = reinterpret_cast<const uint4 *>(dn)[(uint64_t)r * FG + Gc];
+                    } else {
+                        const uint2 v = reinterpret_cast<const uint2 *>(dn)[(uint64_t)r * FG + Gc];
+                        wq[i][c][q] = make_uint4(v.x, v.y, FMT == 1 ? (uint32_t)(dn + sc_off)[(uint64_t)r * FG + Gc] : 0u, 0u);
+                    }
                     d2 |= (uint32_t)reinterpret_cast<const uint16_t *>(dn + qs_bytes)[(uint64_t)r * FB + (Gc >> 3)] << (16 * q);
                 }
                 wd[i][c] = d2;
@@ -2083,7 +2112,9 @@ __global__ __launch_bounds__(kWaves * 64) void down_batch_words_kernel(BatchWord
         if ((lane & 7u) == 0u) part[p * 8u + row] = r;
     }
     request(wave);
-    build_iq3s_quads(lds, tid);
+    if constexpr (FMT == 0) build_iq3s_quads(lds, tid);
+    else if constexpr (FMT == 3) build_tables(lds, tid, grid_entry);
+    else build_codebook_table<FMT>(lds, tid, a.grid, 0u, kWaves * 64u);
     __syncthreads();
 
     for (uint32_t first = wave; first < U; first += 16u * GPW) {
@@ -2105,7 +2136,10 @@ __global__ __launch_bounds__(kWaves * 64) void down_batch_words_kernel(BatchWord
                     for (int q = 0; q < 2; ++q) {
                         const float d = scale_to_f32(wd[i][c] >> (16 * q));
                         float va, vb;
-                        iq3s_group_dot(wq[i][c][q], cur.ax[c], lds, va, vb);
+                        const uint4 w = wq[i][c][q];
+                        if constexpr (FMT == 0) iq3s_group_dot(w, cur.ax[c], lds, va, vb);
+                        else if constexpr (FMT == 3) group_dot_multi<1>(make_uint2(w.x, w.y), reinterpret_cast<const half4_t (*)[8]>(cur.ax[c]), lds, &va, &vb);
+                        else group_dot_fmt2<FMT>(make_uint2(w.x, w.y), w.z, cur.ax[c], lds, va, vb);
                         tot_a[q] += va * d * cur.sa[c];
                         tot_b[q] += vb * d * cur.sb[c];
                     }
@@ -2125,7 +2159,7 @@ __global__ __launch_bounds__(kWaves * 64) void down_batch_words_kernel(BatchWord
         float sum = 0.0f;
         for (uint32_t k = 0; k < a.top_k; ++k) {
             const uint32_t p = a.tok_pair[t * a.top_k + k];
-            sum = fmaf(a.pair_weight[p], part[p * 8u + r], sum);
+            sum = fmaf(a.pair_weight[p] * (FMT == 1 || FMT == 3 ? 0.125f : 1.0f), part[p * 8u + r], sum);      // d/8 formats
         }
         sum = fmaf(a.scalar[t], part[(P + t) * 8u + r], sum);
         const uint64_t at = (uint64_t)t * H + row0 + r;
@@ -2232,7 +2266,7 @@ __global__ __launch_bounds__(kWaves * 64) void down_batch_raw_kernel(DownBatchRa
     }
 }
 
-static hipError_t launch_gateup_batch_kernel(const BatchArgs &a, uint32_t n_groups, hipStream_t s);
+static hipError_t launch_gateup_batch_kernel(const BatchArgs &a, uint32_t n_groups, hipStream_t s, uint32_t gate_up_type = T_IQ2_XXS);
 
 hipError_t launch_batch_packed(const void *experts, uint64_t stride, const void *shared, const uint32_t *uid, const uint32_t *expert_start,
                                const uint32_t *pair_token, const uint32_t *n_unique, const float *pair_weight, const uint32_t *tok_pair,
@@ -2242,7 +2276,7 @@ hipError_t launch_batch_packed(const void *experts, uint64_t stride, const void 
     BatchArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(shared), uid, expert_start, pair_token, n_unique,
                 pair_weight, tok_pair, scalar, static_cast<const _Float16 *>(xh), static_cast<const _Float16 *>(xl), xexp,
                 static_cast<_Float16 *>(act_h), static_cast<_Float16 *>(act_l), act_exp, out, hidden, ffn, top_k, ntok,
-                block_context().resid_a, block_context().resid_b, nullptr};
+                block_context().resid_a, block_context().resid_b, nullptr, nullptr};
     const uint32_t P = ntok * top_k, n_groups = (P < n_expert ? P : n_expert) + 1u;
     hipError_t e = launch_gateup_batch_kernel(a, n_groups, s);
     if (e != hipSuccess) return e;
@@ -2284,34 +2318,49 @@ static hipError_t launch_down_batch_raw_shared(uint32_t ts, const DownBatchRawAr
 
 // Small batch on a mixed layout, pairs grouped by expert: packed IQ2_XXS gate/up matrices on the batched MFMA kernel (the shared
 // expert's gate / up products come in as shared_gu [ntok][2 ffn]), raw down matrices of any built-in type on the batched raw-row kernel.
-hipError_t launch_batch_mixed(const void *packed, uint64_t packed_stride, const float *shared_gu, uint32_t down_type, uint32_t shared_down_type,
+hipError_t launch_batch_mixed(uint32_t gate_up_type, const int8_t *gate_up_grid, const void *packed, uint64_t packed_stride, const float *shared_gu,
+                              uint32_t down_type, const int8_t *down_grid, uint32_t shared_down_type,
                               const void *raw_down, uint64_t raw_stride, const void *shared_down, const void *words_down, uint64_t words_stride,
                               const float *dense_down, const uint32_t *uid, const uint32_t *expert_start,
                               const uint32_t *pair_token, const uint32_t *n_unique, const float *pair_weight, const uint32_t *tok_pair,
                               const float *scalar, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l, int *act_exp,
                               float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s) {
     if (!fused_iq2_supported(hidden, ffn) || !ntok || ntok > (uint32_t)kMaxTok || ntok * top_k + ntok > 144u || ffn > 768u || !shared_gu) return hipErrorInvalidValue;
-    // the staged rows move in 16-byte pieces
-    const uint32_t rbd = (ffn / 256u) * block_bytes(down_type), rbs = (ffn / 256u) * block_bytes(shared_down_type);
-    if (!rbd || !rbs || (8u * rbd) % 16u || (8u * rbs) % 16u || raw_stride % 16u || (uintptr_t)raw_down % 16u || (uintptr_t)shared_down % 16u) return hipErrorInvalidValue;
+    const bool gu_codebook = gate_up_type == T_IQ2_XS || gate_up_type == T_IQ1_M, dn_codebook = down_type == T_IQ2_XS || down_type == T_IQ1_M;
+    if ((gate_up_type != T_IQ2_XXS && !gu_codebook) || (gu_codebook && !gate_up_grid) || (dn_codebook && !down_grid)) return hipErrorInvalidValue;
+    const bool on_mfma = words_down && dense_down && (down_type == T_IQ3_S || dn_codebook || down_type == T_IQ2_XXS);
+    if (!on_mfma) {                                    // the staged raw rows move in 16-byte pieces
+        const uint32_t rbd = (ffn / 256u) * block_bytes(down_type), rbs = (ffn / 256u) * block_bytes(shared_down_type);
+        if (!rbd || !rbs || (8u * rbd) % 16u || (8u * rbs) % 16u || raw_stride % 16u || (uintptr_t)raw_down % 16u || (uintptr_t)shared_down % 16u) return hipErrorInvalidValue;
+    }
     BatchArgs a{static_cast<const uint8_t *>(packed), packed_stride, nullptr, uid, expert_start, pair_token, n_unique,
                 pair_weight, tok_pair, scalar, static_cast<const _Float16 *>(xh), static_cast<const _Float16 *>(xl), xexp,
                 static_cast<_Float16 *>(act_h), static_cast<_Float16 *>(act_l), act_exp, out, hidden, ffn, top_k, ntok,
-                nullptr, nullptr, shared_gu};
+                nullptr, nullptr, shared_gu, gate_up_grid};
     const uint32_t P = ntok * top_k, n_groups = (P < n_expert ? P : n_expert) + 1u;
-    hipError_t e = launch_gateup_batch_kernel(a, n_groups, s);
+    hipError_t e = launch_gateup_batch_kernel(a, n_groups, s, gate_up_type);
     if (e != hipSuccess) return e;
     prof_set_stage(ST_BATCH_DOWN);
-    if (words_down && dense_down && down_type == T_IQ3_S) {      // word-packed IQ3_S on the matrix units, the shared expert's rows from its f32 copy
-        const BatchWordsArgs w{static_cast<const uint8_t *>(words_down), words_stride, dense_down, uid, expert_start, n_unique, pair_weight, tok_pair, scalar,
+    if (on_mfma) {      // packed down matrices on the matrix units, the shared expert's rows from its f32 copy
+        const BatchWordsArgs w{static_cast<const uint8_t *>(words_down), words_stride, down_grid, dense_down, uid, expert_start, n_unique, pair_weight, tok_pair, scalar,
                                static_cast<const _Float16 *>(act_h), static_cast<const _Float16 *>(act_l), act_exp, out, hidden, ffn, top_k, ntok,
                                block_context().resid_a, block_context().resid_b};
         const uint32_t groups_per_wave = (n_groups + kWaves - 1u) / kWaves;
         const dim3 dgrid(hidden / 8u), dblock(kWaves * 64);
-        // (the words take twice the registers of the IQ2_XXS groups: at most three groups of a wave in flight)
-        if (ffn > 512u) REDHIP_LAUNCH((down_batch_words_kernel<144, 2, 1>), dgrid, dblock, 0, s, w);
-        else if (groups_per_wave <= 2u) REDHIP_LAUNCH((down_batch_words_kernel<144, 1, 2>), dgrid, dblock, 0, s, w);
-        else REDHIP_LAUNCH((down_batch_words_kernel<144, 1, 3>), dgrid, dblock, 0, s, w);
+        // (IQ3_S words take twice the registers of the 8-byte groups: at most three groups of a wave in flight)
+#define REDHIP_DBW(FMT)                                                                                                          \
+    do {                                                                                                                         \
+        if (ffn > 512u) REDHIP_LAUNCH((down_batch_words_kernel<144, 2, 1, FMT>), dgrid, dblock, 0, s, w);                         \
+        else if (groups_per_wave <= 2u) REDHIP_LAUNCH((down_batch_words_kernel<144, 1, 2, FMT>), dgrid, dblock, 0, s, w);         \
+        else REDHIP_LAUNCH((down_batch_words_kernel<144, 1, 3, FMT>), dgrid, dblock, 0, s, w);                                    \
+    } while (0)
+        switch (down_type) {
+            case T_IQ3_S: REDHIP_DBW(0); break;
+            case T_IQ2_XS: REDHIP_DBW(1); break;
+            case T_IQ1_M: REDHIP_DBW(2); break;
+            default: REDHIP_DBW(3); break;
+        }
+#undef REDHIP_DBW
         return hipGetLastError();
     }
     const DownBatchRawArgs d{static_cast<const uint8_t *>(raw_down), raw_stride, static_cast<const uint8_t *>(shared_down), uid, expert_start, n_unique,
@@ -2325,26 +2374,33 @@ hipError_t launch_batch_mixed(const void *packed, uint64_t packed_stride, const 
     }
 }
 
-static hipError_t launch_gateup_batch_kernel(const BatchArgs &a, uint32_t n_groups, hipStream_t s) {
+static hipError_t launch_gateup_batch_kernel(const BatchArgs &a, uint32_t n_groups, hipStream_t s, uint32_t gate_up_type) {
     const uint32_t hidden = a.hidden, ffn = a.ffn, ntok = a.ntok;
     const uint32_t unit_bound = n_groups * (ffn / 32u);
     const dim3 grid(256u * ((unit_bound + 256u * kMaxUnits - 1u) / (256u * kMaxUnits)));
     const size_t dyn_lds = (size_t)(2u * ntok + 1u) * (hidden / 32u + 8u) * 64u;   // hi and lo plane per token + a zero plane, 8 pieces of 8 bytes per group
+    const bool codebook = gate_up_type == T_IQ2_XS || gate_up_type == T_IQ1_M;
+    if (codebook && (ntok > 8u || a.shared || !a.grid)) return hipErrorInvalidValue;
     prof_set_stage(ST_BATCH_GATEUP);
+#define REDHIP_GUB_ONE(NKC, NTP, FMT)                                                                                      \
+    do {                                                                                                                  \
+        static bool attr = false;                                                                                          \
+        if (!attr) {                                                                                                       \
+            hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void *>(gateup_batch_kernel<NKC, NTP, FMT>), hipFuncAttributeMaxDynamicSharedMemorySize, (FMT == 2 ? 112 : 128) * 1024); \
+            if (e1 != hipSuccess) return e1;                                                                               \
+            attr = true;                                                                                                   \
+        }                                                                                                                  \
+        REDHIP_LAUNCH((gateup_batch_kernel<NKC, NTP, FMT>), grid, dim3(kWaves * 64), dyn_lds, s, a);                        \
+    } while (0)
 #define REDHIP_GUB(NKC)                                                                                                   \
     do {                                                                                                                  \
         /* two token pairs per pass keep the kernel inside 128 VGPRs; larger groups take more passes */                  \
-        static bool attr = false;                                                                                          \
-        if (!attr) {                                                                                                       \
-            hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void *>(gateup_batch_kernel<NKC, 1>), hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024); \
-            hipError_t e2 = hipFuncSetAttribute(reinterpret_cast<const void *>(gateup_batch_kernel<NKC, 2>), hipFuncAttributeMaxDynamicSharedMemorySize, 128 * 1024); \
-            if (e1 != hipSuccess) return e1;                                                                               \
-            if (e2 != hipSuccess) return e2;                                                                               \
-            attr = true;                                                                                                   \
-        }                                                                                                                  \
-        if (ntok <= 8u) REDHIP_LAUNCH((gateup_batch_kernel<NKC, 1>), grid, dim3(kWaves * 64), dyn_lds, s, a);              \
-        else REDHIP_LAUNCH((gateup_batch_kernel<NKC, 2>), grid, dim3(kWaves * 64), dyn_lds, s, a);                         \
+        if (gate_up_type == T_IQ2_XS) REDHIP_GUB_ONE(NKC, 1, 1);                                                          \
+        else if (gate_up_type == T_IQ1_M) REDHIP_GUB_ONE(NKC, 1, 2);                                                      \
+        else if (ntok <= 8u) REDHIP_GUB_ONE(NKC, 1, 0);                                                                   \
+        else REDHIP_GUB_ONE(NKC, 2, 0);                                                                                   \
     } while (0)
+    if (dyn_lds > (gate_up_type == T_IQ1_M ? 112u : 128u) * 1024u) return hipErrorInvalidValue;
     switch (hidden / 512u) {
         case 1: REDHIP_GUB(1); break;
         case 2: REDHIP_GUB(2); break;
@@ -2352,6 +2408,7 @@ static hipError_t launch_gateup_batch_kernel(const BatchArgs &a, uint32_t n_grou
         default: return hipErrorInvalidValue;
     }
 #undef REDHIP_GUB
+#undef REDHIP_GUB_ONE
     return hipGetLastError();
 }
 

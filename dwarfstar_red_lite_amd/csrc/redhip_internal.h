@@ -203,9 +203,11 @@ hipError_t launch_gateup_select(const void *experts, uint64_t stride, const void
                                 float *scalar_out, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l, int *act_exp,
                                 uint32_t hidden, uint32_t ffn, uint32_t n_expert, uint32_t top_k, hipStream_t s, uint32_t ntok = 1u,
                                 uint32_t gate_up_type = T_IQ2_XXS, const int8_t *grid = nullptr);
-// small batch on a mixed layout with the pairs grouped by expert: batched MFMA gate/up on the packed IQ2_XXS matrices (shared expert's
-// products given), batched raw-row down of the built-in block types; every distinct expert is read once
-hipError_t launch_batch_mixed(const void *packed, uint64_t packed_stride, const float *shared_gu, uint32_t down_type, uint32_t shared_down_type,
+// small batch on a mixed layout with the pairs grouped by expert: batched MFMA gate/up on the packed IQ2_XXS / IQ2_XS / IQ1_M matrices
+// (shared expert's products given), batched MFMA down on the packed copy (`words_down`: IQ3_S words or the streams of the other three
+// formats) with the shared rows from `dense_down`, else batched raw-row down of the built-in block types; every distinct expert is read once
+hipError_t launch_batch_mixed(uint32_t gate_up_type, const int8_t *gate_up_grid, const void *packed, uint64_t packed_stride, const float *shared_gu,
+                              uint32_t down_type, const int8_t *down_grid, uint32_t shared_down_type,
                               const void *raw_down, uint64_t raw_stride, const void *shared_down, const void *words_down, uint64_t words_stride,
                               const float *dense_down, const uint32_t *uid, const uint32_t *expert_start,
                               const uint32_t *pair_token, const uint32_t *n_unique, const float *pair_weight, const uint32_t *tok_pair,

@@ -115,8 +115,9 @@ struct Moe {
     static constexpr uint32_t kGroupedMin = 3u;
     bool grouped_mixed(uint32_t ntok) const {
         const uint32_t rbd = (cfg.ffn / 256u) * block_bytes(dn_type), rbs = (cfg.ffn / 256u) * block_bytes(sh_dn_type);
-        return small_batch_mixed(ntok) && ntok >= kGroupedMin && gu_type == T_IQ2_XXS && quant_supported(dn_type) && cfg.ffn <= 768u &&
-               (8u * rbd) % 16u == 0u && (8u * rbs) % 16u == 0u && (2u * gate_bytes) % 16u == 0u && (2u * sh_gate_bytes) % 16u == 0u;
+        const bool words = (dn_type == T_IQ3_S || dn_type == T_IQ2_XS || dn_type == T_IQ1_M) && cfg.ffn <= 1024u;      // then the layers hold a packed down copy
+        return small_batch_mixed(ntok) && ntok >= kGroupedMin && cfg.ffn <= 768u &&
+               (words || (quant_supported(dn_type) && (8u * rbd) % 16u == 0u && (8u * rbs) % 16u == 0u && (2u * gate_bytes) % 16u == 0u && (2u * sh_gate_bytes) % 16u == 0u));
     }
     // every batch size runs on the packed layout when the layer has one (decode kernel, small-batch kernels, prefill tiles)
     bool packed_path(uint32_t ntok) const { return (fused && (ntok == 1u || small_batch(ntok) || cfg.hidden / 512u <= 4u)) || (mixed && ntok == 1u); }
@@ -171,7 +172,7 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
             HIP_OK(launch_group_pairs(ids, weights, ntok, c.top_k, c.n_expert, m->uid, m->expert_start, m->pair_token, m->pair_weight,
                                       m->tok_pair, m->n_unique, s), "grouping launch");
         }
-        HIP_OK(launch_batch_mixed(L.packed, m->packed_stride, m->act, m->dn_type, m->sh_dn_type, L.experts + 2u * m->gate_bytes, m->expert_stride,
+        HIP_OK(launch_batch_mixed(m->gu_type, m->gu_grid, L.packed, m->packed_stride, m->act, m->dn_type, m->dn_grid, m->sh_dn_type, L.experts + 2u * m->gate_bytes, m->expert_stride,
                                   L.shared + 2u * m->sh_gate_bytes, L.words_down, m->words_down_stride(), L.dense_down, m->uid, m->expert_start, m->pair_token, m->n_unique, m->pair_weight, m->tok_pair,
                                   m->scalar, m->xh, m->xl, m->xexp, m->act_h, m->act_l, m->act_exp, out, c.hidden, c.ffn, c.top_k, ntok, c.n_expert, s),
                "grouped mixed batch launch");
