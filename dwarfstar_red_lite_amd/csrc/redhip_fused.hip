@@ -2031,7 +2031,7 @@ __global__ __launch_bounds__(kWaves * 64) void down_batch_kernel(BatchArgs a) {
 }
 
 // The same kernel with the shared expert's rows taken from its dense f32 copy (token t's product on wave 15 - t, ahead of that wave's
-// routed groups), for routed down matrices that are word-packed IQ3_S (FMT 0), IQ2_XS / IQ1_M streams (1 / 2) or IQ2_XXS streams (3).
+// routed groups), for routed down matrices that are word-packed IQ3_S (FMT 0) or IQ2_XS / IQ1_M streams (1 / 2).
 struct BatchWordsArgs {
     const uint8_t *experts;    // packed down matrix of expert e at experts + e * stride
     uint64_t stride;
@@ -2050,14 +2050,13 @@ struct BatchWordsArgs {
 
 template <int MAXPAIR, int NCH, int GPW, int FMT>     // GPW: groups of a wave whose weights are in registers at once
 __global__ __launch_bounds__(kWaves * 64) void down_batch_words_kernel(BatchWordsArgs a) {
-    __shared__ __attribute__((aligned(16))) uint8_t lds[FMT == 0 ? kIq3TableBytes : FMT == 1 ? 512u * 16u : FMT == 2 ? 2048u * 16u : kMagBytes];
+    __shared__ __attribute__((aligned(16))) uint8_t lds[FMT == 0 ? kIq3TableBytes : FMT == 1 ? 512u * 16u : 2048u * 16u];
     __shared__ float part[MAXPAIR * 8];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t H = a.hidden, F = a.ffn, FG = F / 32u, FB = F / 256u, P = a.ntok * a.top_k;
     const uint32_t row0 = 8u * blockIdx.x, U = __builtin_amdgcn_readfirstlane(a.n_unique[0]);
     const uint64_t qs_bytes = (uint64_t)H * FG * (FMT == 0 ? 16u : 8u), sc_off = qs_bytes + (uint64_t)H * FB * 2u;      // IQ2_XS: scale bytes [hidden][FG] behind d
-    const uint64_t grid_entry = FMT == 3 && tid < 256u ? redhip_iq2xxs_grid[tid] : 0ull;
 
     uint4 wq[GPW][NCH][2];
     uint32_t wd[GPW][NCH], gp0[GPW], gp1[GPW];      // wd: the two rows' block scales, 16 bits each
@@ -2113,7 +2112,6 @@ __global__ __launch_bounds__(kWaves * 64) void down_batch_words_kernel(BatchWord
     }
     request(wave);
     if constexpr (FMT == 0) build_iq3s_quads(lds, tid);
-    else if constexpr (FMT == 3) build_tables(lds, tid, grid_entry);
     else build_codebook_table<FMT>(lds, tid, a.grid, 0u, kWaves * 64u);
     __syncthreads();
 
@@ -2138,7 +2136,6 @@ __global__ __launch_bounds__(kWaves * 64) void down_batch_words_kernel(BatchWord
                         float va, vb;
                         const uint4 w = wq[i][c][q];
                         if constexpr (FMT == 0) iq3s_group_dot(w, cur.ax[c], lds, va, vb);
-                        else if constexpr (FMT == 3) group_dot_multi<1>(make_uint2(w.x, w.y), reinterpret_cast<const half4_t (*)[8]>(cur.ax[c]), lds, &va, &vb);
                         else group_dot_fmt2<FMT>(make_uint2(w.x, w.y), w.z, cur.ax[c], lds, va, vb);
                         tot_a[q] += va * d * cur.sa[c];
                         tot_b[q] += vb * d * cur.sb[c];
@@ -2159,7 +2156,7 @@ __global__ __launch_bounds__(kWaves * 64) void down_batch_words_kernel(BatchWord
         float sum = 0.0f;
         for (uint32_t k = 0; k < a.top_k; ++k) {
             const uint32_t p = a.tok_pair[t * a.top_k + k];
-            sum = fmaf(a.pair_weight[p] * (FMT == 1 || FMT == 3 ? 0.125f : 1.0f), part[p * 8u + r], sum);      // d/8 formats
+            sum = fmaf(a.pair_weight[p] * (FMT == 1 ? 0.125f : 1.0f), part[p * 8u + r], sum);      // IQ2_XS: d/8
         }
         sum = fmaf(a.scalar[t], part[(P + t) * 8u + r], sum);
         const uint64_t at = (uint64_t)t * H + row0 + r;
@@ -2325,11 +2322,12 @@ hipError_t launch_batch_mixed(uint32_t gate_up_type, const int8_t *gate_up_grid,
                               const uint32_t *pair_token, const uint32_t *n_unique, const float *pair_weight, const uint32_t *tok_pair,
                               const float *scalar, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l, int *act_exp,
                               float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s) {
-    if (!fused_iq2_supported(hidden, ffn) || !ntok || ntok > (uint32_t)kMaxTok || ntok * top_k + ntok > 144u || ffn > 768u || !shared_gu) return hipErrorInvalidValue;
+    if (!fused_iq2_supported(hidden, ffn) || !ntok || ntok > (uint32_t)kMaxTok || ntok * top_k + ntok > 144u || !shared_gu) return hipErrorInvalidValue;
     const bool gu_codebook = gate_up_type == T_IQ2_XS || gate_up_type == T_IQ1_M, dn_codebook = down_type == T_IQ2_XS || down_type == T_IQ1_M;
     if ((gate_up_type != T_IQ2_XXS && !gu_codebook) || (gu_codebook && !gate_up_grid) || (dn_codebook && !down_grid)) return hipErrorInvalidValue;
-    const bool on_mfma = words_down && dense_down && (down_type == T_IQ3_S || dn_codebook || down_type == T_IQ2_XXS);
-    if (!on_mfma) {                                    // the staged raw rows move in 16-byte pieces
+    const bool on_mfma = words_down && dense_down && (down_type == T_IQ3_S || dn_codebook);
+    if (!on_mfma) {                                    // the staged raw rows move in 16-byte pieces, five per lane at most
+        if (ffn > 768u) return hipErrorInvalidValue;
         const uint32_t rbd = (ffn / 256u) * block_bytes(down_type), rbs = (ffn / 256u) * block_bytes(shared_down_type);
         if (!rbd || !rbs || (8u * rbd) % 16u || (8u * rbs) % 16u || raw_stride % 16u || (uintptr_t)raw_down % 16u || (uintptr_t)shared_down % 16u) return hipErrorInvalidValue;
     }
@@ -2347,7 +2345,7 @@ hipError_t launch_batch_mixed(uint32_t gate_up_type, const int8_t *gate_up_grid,
                                block_context().resid_a, block_context().resid_b};
         const uint32_t groups_per_wave = (n_groups + kWaves - 1u) / kWaves;
         const dim3 dgrid(hidden / 8u), dblock(kWaves * 64);
-        // (IQ3_S words take twice the registers of the 8-byte groups: at most three groups of a wave in flight)
+        // (at most three groups of a wave in flight: IQ3_S words take twice the registers of the IQ2_XXS groups)
 #define REDHIP_DBW(FMT)                                                                                                          \
     do {                                                                                                                         \
         if (ffn > 512u) REDHIP_LAUNCH((down_batch_words_kernel<144, 2, 1, FMT>), dgrid, dblock, 0, s, w);                         \
@@ -2357,8 +2355,7 @@ hipError_t launch_batch_mixed(uint32_t gate_up_type, const int8_t *gate_up_grid,
         switch (down_type) {
             case T_IQ3_S: REDHIP_DBW(0); break;
             case T_IQ2_XS: REDHIP_DBW(1); break;
-            case T_IQ1_M: REDHIP_DBW(2); break;
-            default: REDHIP_DBW(3); break;
+            default: REDHIP_DBW(2); break;
         }
 #undef REDHIP_DBW
         return hipGetLastError();

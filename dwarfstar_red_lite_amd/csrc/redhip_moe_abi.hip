@@ -116,7 +116,7 @@ struct Moe {
     bool grouped_mixed(uint32_t ntok) const {
         const uint32_t rbd = (cfg.ffn / 256u) * block_bytes(dn_type), rbs = (cfg.ffn / 256u) * block_bytes(sh_dn_type);
         const bool words = (dn_type == T_IQ3_S || dn_type == T_IQ2_XS || dn_type == T_IQ1_M) && cfg.ffn <= 1024u;      // then the layers hold a packed down copy
-        return small_batch_mixed(ntok) && ntok >= kGroupedMin && cfg.ffn <= 768u &&
+        return small_batch_mixed(ntok) && ntok >= kGroupedMin && (words || cfg.ffn <= 768u) &&
                (words || (quant_supported(dn_type) && (8u * rbd) % 16u == 0u && (8u * rbs) % 16u == 0u && (2u * gate_bytes) % 16u == 0u && (2u * sh_gate_bytes) % 16u == 0u));
     }
     // every batch size runs on the packed layout when the layer has one (decode kernel, small-batch kernels, prefill tiles)
