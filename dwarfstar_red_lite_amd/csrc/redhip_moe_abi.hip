@@ -119,6 +119,16 @@ struct Moe {
         return small_batch_mixed(ntok) && ntok >= kGroupedMin && (words || cfg.ffn <= 768u) &&
                (words || (quant_supported(dn_type) && (8u * rbd) % 16u == 0u && (8u * rbs) % 16u == 0u && (2u * gate_bytes) % 16u == 0u && (2u * sh_gate_bytes) % 16u == 0u));
     }
+    // a chunk on a mixed layout that has no tile kernels (IQ2_XS / IQ1_M gate/up, ffn > 512) runs as slices of 8 tokens on the grouped
+    // small-batch kernels, far ahead of the generic per-pair kernels on raw rows
+    static constexpr uint32_t kSlice = 8u;
+    bool sliced(uint32_t ntok) const { return mixed && ntok > kSlice && !tiles_resident() && grouped_mixed(kSlice); }
+    // the workspace entries a caller can read back (redhip_moe_last_route) of the slice that starts at token t0 sit at their place in the chunk
+    void shift_route_outputs(int64_t t0) {
+        ids += t0 * (int64_t)cfg.top_k;
+        weights += t0 * (int64_t)cfg.top_k;
+        logits += t0 * (int64_t)(cfg.n_expert + 1u);
+    }
     // every batch size runs on the packed layout when the layer has one (decode kernel, small-batch kernels, prefill tiles)
     bool packed_path(uint32_t ntok) const { return (fused && (ntok == 1u || small_batch(ntok) || cfg.hidden / 512u <= 4u)) || (mixed && ntok == 1u); }
     ExpertSet routed(uint32_t l) const { return ExpertSet{layers[l].experts, expert_stride, gate_bytes, gate_bytes, gu_type, dn_type}; }
@@ -632,6 +642,16 @@ int redhip_moe_forward(redhip_moe_t h, uint32_t layer, const float *x_dev, uint3
     Moe *m = moe_of(h);
     if (!check_layer(m, layer)) return 0;
     if (!x_dev || !out_dev) { moe_err("null activation pointer"); return 0; }
+    if (m->sliced(ntok) && ntok <= m->cfg.max_tokens) {
+        int ok = 1;
+        for (uint32_t t0 = 0; t0 < ntok && ok; t0 += Moe::kSlice) {
+            const uint32_t n = ntok - t0 < Moe::kSlice ? ntok - t0 : Moe::kSlice;
+            m->shift_route_outputs(t0);
+            ok = redhip_moe_forward(h, layer, x_dev + (size_t)t0 * m->cfg.hidden, n, out_dev + (size_t)t0 * m->cfg.hidden, stream);
+            m->shift_route_outputs(-(int64_t)t0);
+        }
+        return ok;
+    }
     const bool group_in_select = m->small_batch(ntok) || m->grouped_mixed(ntok);
     const bool select_in_gateup = m->packed_gu() && (ntok == 1u || m->small_batch_mixed(ntok)) && !group_in_select;
     m->skip_select = select_in_gateup;
@@ -649,6 +669,20 @@ int redhip_moe_forward_block(redhip_moe_t h, uint32_t layer, const float *x_dev,
     if (!check_layer(m, layer)) return 0;
     if (!x_dev || !branch_dev || !post_norm_dev || !x_out_dev || !ntok || ntok > m->cfg.max_tokens) { moe_err("invalid block step arguments"); return 0; }
     const redhip_moe_config &c = m->cfg;
+    if (m->sliced(ntok)) {
+        int ok = 1;
+        for (uint32_t t0 = 0; t0 < ntok && ok; t0 += Moe::kSlice) {
+            const uint32_t n = ntok - t0 < Moe::kSlice ? ntok - t0 : Moe::kSlice;
+            const size_t off = (size_t)t0 * c.hidden;
+            m->shift_route_outputs(t0);
+            float *xn = m->xn;
+            m->xn += off;                                // the normalised rows of the slice at their place in the chunk too
+            ok = redhip_moe_forward_block(h, layer, x_dev + off, branch_dev + off, post_norm_dev, eps, n, x_out_dev + off, stream);
+            m->xn = xn;
+            m->shift_route_outputs(-(int64_t)t0);
+        }
+        return ok;
+    }
     hipStream_t s = static_cast<hipStream_t>(stream);
     BlockContext &bc = block_context();
     bc = BlockContext{};
