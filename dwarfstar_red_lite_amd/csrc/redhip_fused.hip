@@ -895,23 +895,6 @@ __device__ __forceinline__ float group_dot_fmt(uint2 q, uint32_t sc, const half4
     }
 }
 
-// fp16 copy of a caller-supplied codebook (int8 [entries][8]) in LDS, 16 bytes per entry; built by `builders` lanes starting at lane `first`
-// of the workgroup (the gate/up kernel: every wave but the first, which selects meanwhile)
-template <int FMT>
-__device__ __forceinline__ void build_codebook_table(uint8_t *lds, uint32_t tid, const int8_t *grid, uint32_t first = 64u, uint32_t builders = (kWaves - 1) * 64u) {
-    constexpr uint32_t kEntries = FMT == 1 ? 512u : 2048u;
-    for (uint32_t i = tid - first; i < kEntries; i += builders) {      // tid < first wraps past the bound
-        const uint64_t e = reinterpret_cast<const uint64_t *>(grid)[i];
-        uint32_t w4[4];
-#pragma unroll
-        for (int k = 0; k < 4; ++k) {
-            const _Float16 lo = (_Float16)(float)(int8_t)(e >> (16 * k)), hi = (_Float16)(float)(int8_t)(e >> (16 * k + 8));
-            w4[k] = (uint32_t)__builtin_bit_cast(uint16_t, lo) | ((uint32_t)__builtin_bit_cast(uint16_t, hi) << 16);
-        }
-        *reinterpret_cast<uint4 *>(lds + (size_t)i * 16u) = make_uint4(w4[0], w4[1], w4[2], w4[3]);
-    }
-}
-
 // the lane's activation operand: 32 values starting at src (fp16), lanes j = 0 / 1 carry hi / lo, others zero
 __device__ __forceinline__ void load_act_operand(half4_t *ax, const _Float16 *hi, const _Float16 *lo, uint32_t j) {
     const _Float16 *src = j == 0u ? hi : lo;

@@ -140,6 +140,12 @@ hipError_t launch_prefill_gateup_tiled(const void *tiled_experts, uint64_t strid
                                        int *act_exp, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s);
 // tile-major IQ3_S matrices (one 32-bit word per eight weights) from raw GGUF rows, and the routed down projection of a chunk on them
 hipError_t launch_tile_iq3s(const void *raw, uint64_t raw_stride, uint32_t count, uint32_t nrows, uint32_t K, void *tiled, uint64_t tiled_stride, hipStream_t s);
+// routed matrices of a chunk whose experts are IQ2_XS / IQ1_M: tile kernels on the row-major streams (gate | up at `packed`, down at `down`)
+hipError_t launch_prefill_streams(uint32_t gate_up_type, const int8_t *gate_up_grid, const void *packed, uint64_t packed_stride, uint32_t down_type,
+                                  const int8_t *down_grid, const void *down, uint64_t down_stride, const uint32_t *uid, const uint32_t *expert_start,
+                                  const uint32_t *pair_token, const uint32_t *n_unique, uint32_t *tile_group, uint32_t *tile_pair0, uint32_t *tile_n,
+                                  uint32_t *n_tiles, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l, int *act_exp, float *tmp,
+                                  uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s);
 hipError_t launch_prefill_down_iq3s(const void *tiled_down, uint64_t stride, const uint32_t *uid, const uint32_t *n_unique, const uint32_t *tile_group,
                                     const uint32_t *tile_pair0, const uint32_t *tile_n, const uint32_t *n_tiles, const void *act_h, const void *act_l,
                                     const int *act_exp, float *tmp, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert,

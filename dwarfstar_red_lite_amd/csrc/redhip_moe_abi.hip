@@ -119,10 +119,16 @@ struct Moe {
         return small_batch_mixed(ntok) && ntok >= kGroupedMin && (words || cfg.ffn <= 768u) &&
                (words || (quant_supported(dn_type) && (8u * rbd) % 16u == 0u && (8u * rbs) % 16u == 0u && (2u * gate_bytes) % 16u == 0u && (2u * sh_gate_bytes) % 16u == 0u));
     }
-    // a chunk on a mixed layout that has no tile kernels (IQ2_XS / IQ1_M gate/up, ffn > 512) runs as slices of 8 tokens on the grouped
-    // small-batch kernels, far ahead of the generic per-pair kernels on raw rows
+    // a chunk on a layout whose experts are IQ2_XS / IQ1_M: the tile kernels on the row-major streams of the routed matrices, the shared
+    // expert and the router as dense f32 products
+    bool stream_chunk(uint32_t ntok) const {
+        const bool gu_cb = gu_type == T_IQ2_XS || gu_type == T_IQ1_M, dn_cb = dn_type == T_IQ2_XS || dn_type == T_IQ1_M;
+        return mixed && ntok > 8u && gu_cb && dn_cb && (cfg.ffn == 256u || cfg.ffn == 512u) && cfg.hidden / 512u <= 4u && cfg.max_tokens > 8u;
+    }
+    // a chunk on a mixed layout that has no tile kernels (ffn > 512, or IQ2_XS / IQ1_M gate/up beside another down format) runs as slices
+    // of 8 tokens on the grouped small-batch kernels, far ahead of the generic per-pair kernels on raw rows
     static constexpr uint32_t kSlice = 8u;
-    bool sliced(uint32_t ntok) const { return mixed && ntok > kSlice && !tiles_resident() && grouped_mixed(kSlice); }
+    bool sliced(uint32_t ntok) const { return mixed && ntok > kSlice && !tiles_resident() && !stream_chunk(ntok) && grouped_mixed(kSlice); }
     // the workspace entries a caller can read back (redhip_moe_last_route) of the slice that starts at token t0 sit at their place in the chunk
     void shift_route_outputs(int64_t t0) {
         ids += t0 * (int64_t)cfg.top_k;
@@ -210,6 +216,22 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
             HIP_OK(launch_prefill_packed(L.packed, m->expert_stride, L.shared_packed, L.tiled, L.shared_tiled, m->uid, m->expert_start, m->pair_token, m->n_unique,
                                          m->tile_group, m->tile_pair0, m->tile_n, m->n_tiles, m->xh, m->xl, m->xexp, m->act_h, m->act_l,
                                          m->act_exp, m->tmp, m->sh_tmp, c.hidden, c.ffn, c.top_k, ntok, c.n_expert, s), "prefill launch");
+            prof_set_stage(ST_BATCH_COMBINE);
+            HIP_OK(launch_batch_combine(m->tmp, m->pair_weight, m->tok_pair, ntok, c.top_k, m->sh_tmp, m->scalar, c.hidden, out, s), "batched combine launch");
+            prof_set_stage(ST_OTHER);
+            return 1;
+        }
+        if (m->stream_chunk(ntok) && m->layers[layer].words_down && m->layers[layer].dense_gu) {
+            const Layer &L = m->layers[layer];
+            float *gu = m->tmp;                          // [ntok][2 ffn]; free until the routed down kernel writes tmp (2 ffn <= top_k * hidden)
+            prof_set_stage(ST_BATCH_GATEUP);
+            HIP_OK(launch_f32_tiles(L.dense_gu, nullptr, x, ntok, c.hidden, 2u * c.ffn, gu, 2u * c.ffn, nullptr, nullptr, nullptr, s), "shared gate/up tiles");
+            HIP_OK(launch_swiglu_rows(gu, 2u * c.ffn, ntok, c.ffn, m->sh_act, s), "shared SwiGLU");
+            HIP_OK(launch_prefill_streams(m->gu_type, m->gu_grid, L.packed, m->packed_stride, m->dn_type, m->dn_grid, L.words_down, m->words_down_stride(), m->uid,
+                                          m->expert_start, m->pair_token, m->n_unique, m->tile_group, m->tile_pair0, m->tile_n, m->n_tiles, m->xh, m->xl, m->xexp,
+                                          m->act_h, m->act_l, m->act_exp, m->tmp, c.hidden, c.ffn, c.top_k, ntok, c.n_expert, s), "stream tile launch");
+            prof_set_stage(ST_BATCH_DOWN);
+            HIP_OK(launch_f32_tiles(L.dense_down, nullptr, m->sh_act, ntok, c.ffn, c.hidden, m->sh_tmp, c.hidden, nullptr, nullptr, nullptr, s), "shared down tiles");
             prof_set_stage(ST_BATCH_COMBINE);
             HIP_OK(launch_batch_combine(m->tmp, m->pair_weight, m->tok_pair, ntok, c.top_k, m->sh_tmp, m->scalar, c.hidden, out, s), "batched combine launch");
             prof_set_stage(ST_OTHER);
@@ -617,7 +639,7 @@ int redhip_moe_experts(redhip_moe_t h, uint32_t layer, const float *x_dev, uint3
     if (!x_dev || !ids_dev || !weights_dev || !out_dev || !ntok || ntok > m->cfg.max_tokens) { moe_err("invalid expert execution arguments"); return 0; }
     hipStream_t s = static_cast<hipStream_t>(stream);
     m->shared_gu_ready = false;
-    if (m->packed_path(ntok) || m->small_batch_mixed(ntok) || m->mixed_chunk(ntok)) {
+    if (m->packed_path(ntok) || m->small_batch_mixed(ntok) || m->mixed_chunk(ntok) || m->stream_chunk(ntok)) {
         prof_set_stage(ST_OTHER);
         HIP_OK(launch_prep(x_dev, m->layers[layer].gate_inp, ntok, m->cfg.hidden, m->xh, m->xl, m->xexp, m->scalar, s), "prep launch");
         const Layer &L = m->layers[layer];

@@ -386,34 +386,97 @@ __device__ __forceinline__ half8_t decode_scaled(uint2 w, uint32_t q, const uint
     return r.v;
 }
 
-struct RowChunk { uint4 a, b; uint32_t d; };      // four groups (32 bytes) of one packed row and the block scale over them
+struct RowChunk { uint4 a, b; uint32_t d, sc; };      // four groups (32 bytes) of one packed row, the block scale over them, IQ2_XS: their four scale bytes
 
 struct TiledArgs {
     PrefillArgs p;
     const uint8_t *experts, *shared;      // tile-major copies; same expert stride and matrix offsets as the packed layout
     float *act_f32;                       // gate/up kernel: when set, the SwiGLU activations go here as f32 [pairs][ffn] (kernels on raw rows follow)
+    const int8_t *grid;                   // FMT 1 / 2: the caller's codebook; `experts` are then the row-major streams of the format
+    uint64_t down_off;                    // down kernel, FMT 1 / 2: offset of the down matrix inside an expert's slot
 };
+
+// The same kernels serve IQ2_XS (FMT 1) and IQ1_M (FMT 2) matrices, read from their row-major streams (uint2 per 32 weights, d per 256,
+// IQ2_XS a scale byte per 32) - 16 rows x 32 bytes per wave-wide load instead of 512 contiguous bytes. Their codebooks are too large to
+// be multiplied out with every group scale, so the table holds the plain fp16 entries (8 KB / 32 KB) and the scale (per 16 weights) is
+// applied to the eight weights by packed fp16 multiplies, exact: IQ2_XS entry * (2 s + 1) <= 43 * 31, IQ1_M (entry +- 1/8) * (2 s + 1)
+// in eighths <= 135. The d/8 of IQ2_XS stays in the activation scale, IQ1_M has none.
+typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
+template <int FMT> constexpr uint32_t reg_table_bytes() { return FMT == 0 ? kSignBytes + kScaledMagBytes : FMT == 1 ? kSignBytes + 512u * 16u : 2048u * 16u; }
+
+__device__ __forceinline__ void build_sign_table(uint8_t *sgn, uint32_t tid, uint32_t nthreads) {
+    for (uint32_t s7 = tid; s7 < 128u; s7 += nthreads) {
+        const uint32_t s8 = s7 | ((__popc(s7) & 1u) << 7);
+        uint32_t w4[4];
+#pragma unroll
+        for (uint32_t i = 0; i < 4u; ++i) w4[i] = (((s8 >> (2u * i)) & 1u) << 15) | (((s8 >> (2u * i + 1u)) & 1u) << 31);
+        *reinterpret_cast<uint4 *>(sgn + (size_t)s7 * 16u) = make_uint4(w4[0], w4[1], w4[2], w4[3]);
+    }
+}
+// tables of a format at `tables`: FMT 0 signs | scaled magnitudes, FMT 1 signs | fp16 codebook, FMT 2 fp16 codebook
+template <int FMT>
+__device__ __forceinline__ void build_reg_tables(uint8_t *tables, uint32_t tid, uint32_t nthreads, const int8_t *grid) {
+    if constexpr (FMT == 0) {
+        build_scaled_tables(tables + kSignBytes, tables, tid, nthreads);
+    } else if constexpr (FMT == 1) {
+        build_sign_table(tables, tid, nthreads);
+        build_codebook_table<1>(tables + kSignBytes, tid, grid, 0u, nthreads);
+    } else {
+        build_codebook_table<2>(tables, tid, grid, 0u, nthreads);
+    }
+}
+// odd integer 2 s + 1 (s < 16) as two equal fp16 halves
+__device__ __forceinline__ uint32_t odd_scale_splat(uint32_t s) {
+    const uint32_t h = __builtin_bit_cast(uint16_t, (_Float16)(float)(2u * s + 1u));
+    return h | (h << 16);
+}
+// the eight signed, scaled fp16 weights of entry q (eight columns) of a group: w = the group's uint2, sc = its IQ2_XS scale byte
+template <int FMT>
+__device__ __forceinline__ half8_t decode_reg(uint2 w, uint32_t sc, uint32_t q, const uint8_t *tables) {
+    if constexpr (FMT == 0) {
+        return decode_scaled(w, q, tables + kSignBytes, tables);
+    } else if constexpr (FMT == 1) {
+        const uint32_t w16 = (((q & 2u) ? w.y : w.x) >> (16u * (q & 1u))) & 0xffffu;
+        const uint4 m = *reinterpret_cast<const uint4 *>(tables + kSignBytes + ((w16 & 511u) << 4));
+        const uint4 g = *reinterpret_cast<const uint4 *>(tables + ((w16 >> 9) << 4));
+        const half2_t f = __builtin_bit_cast(half2_t, odd_scale_splat((sc >> (4u * (q >> 1))) & 15u));
+        Half8 r;
+        r.u = make_uint4(__builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, m.x ^ g.x) * f), __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, m.y ^ g.y) * f),
+                         __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, m.z ^ g.z) * f), __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, m.w ^ g.w) * f));
+        return r.v;
+    } else {
+        const uint32_t idx = ((w.x >> (8u * q)) & 255u) | (((w.y >> (4u * q)) & 7u) << 8);
+        const uint4 m = *reinterpret_cast<const uint4 *>(tables + (idx << 4));
+        const uint32_t fs = odd_scale_splat((w.y >> (16u + 3u * (q >> 1))) & 7u);
+        const half2_t f = __builtin_bit_cast(half2_t, fs);
+        // (2 s + 1) / 8 with the sign of the offset: three exponent steps down (2 s + 1 >= 1 is a normal number), sign bit by xor
+        const half2_t off = __builtin_bit_cast(half2_t, (fs - 0x0c000c00u) ^ (((w.y >> (4u * q + 3u)) & 1u) * 0x80008000u));
+        Half8 r;
+        r.u = make_uint4(__builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, m.x) * f + off), __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, m.y) * f + off),
+                         __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, m.z) * f + off), __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, m.w) * f + off));
+        return r.v;
+    }
+}
 
 // gate/up + SwiGLU. Wave = (K quarter kc, column half rh): for the unit of 32 FFN columns j it computes the gate row and the
 // up row of column 32 j + 16 rh + r against its quarter of the hidden dimension; the quarters meet in LDS (double-buffered:
 // one barrier per unit).
-template <int NKC>          // hidden = 512 * NKC
+template <int NKC, int FMT>          // hidden = 512 * NKC; FMT 0: tile-major packed IQ2_XXS, 1 / 2: row-major IQ2_XS / IQ1_M streams
 __global__ __launch_bounds__(kRegWaves * 64) void prefill_gateup_reg_kernel(TiledArgs ta) {
     const PrefillArgs &a = ta.p;
     constexpr uint32_t H = 512u * NKC, HG = H / 32u, HB = H / 256u, GQ = HG / 4u, NC = H / 128u;   // GQ: groups per K quarter = 4 NKC
     extern __shared__ __attribute__((aligned(16))) uint8_t dyn[];          // acts: [16][F + 4] f32
-    __shared__ __attribute__((aligned(16))) uint8_t tables[kSignBytes + kScaledMagBytes];      // static: table reads take immediate offsets
+    __shared__ __attribute__((aligned(16))) uint8_t tables[reg_table_bytes<FMT>()];      // static: table reads take immediate offsets
     __shared__ float part[2][4][kTile][68];                // [unit parity][K quarter][pair][gate 0..31 | up 0..31], padded
     __shared__ float tok_scale[kTile];
     __shared__ uint32_t tok_of[kTile];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, r = lane & 15u, q = lane >> 4;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6), kc = wave & 3u, rh = wave >> 2;
     const uint32_t F = a.ffn, FG = F / 32u, P = a.ntok * a.top_k, AROW = F + 4u;
-    const uint8_t *sgn = tables, *mag = tables + kSignBytes;
     float *acts = reinterpret_cast<float *>(dyn);
-    build_scaled_tables(tables + kSignBytes, tables, tid, kRegWaves * 64u);
+    build_reg_tables<FMT>(tables, tid, kRegWaves * 64u, ta.grid);
     const uint32_t T = a.n_tiles[0], U = a.n_unique[0];
-    const uint64_t qs_bytes = (uint64_t)F * HG * 8u, gate_bytes = qs_bytes + (uint64_t)F * HB * 2u;
+    const uint64_t qs_bytes = (uint64_t)F * HG * 8u, sc_off = qs_bytes + (uint64_t)F * HB * 2u, gate_bytes = sc_off + (FMT == 1 ? (uint64_t)F * HG : 0u);
 
     // Work items are half tiles (one half of the FFN columns, with an activation exponent of its own) so that the last round of
     // the persistent workgroups is short; a workgroup takes a contiguous range of items and keeps its A operands when two of
@@ -432,7 +495,7 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_gateup_reg_kernel(Tile
             if (tid < kTile) {
                 const uint32_t p = p0 + tid, tok = tid < n ? (p < P ? a.pair_token[p] : p - P) : 0u;
                 tok_of[tid] = tok;
-                tok_scale[tid] = tid < n ? 0.125f * exp2i(a.xexp[tok]) : 0.0f;
+                tok_scale[tid] = tid < n ? (FMT == 2 ? 1.0f : 0.125f) * exp2i(a.xexp[tok]) : 0.0f;
             }
             __syncthreads();
             // this lane's A operands for the whole tile: token of pair r, columns 8 q .. 8 q + 7 of each group of the wave's quarter
@@ -450,9 +513,16 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_gateup_reg_kernel(Tile
         }
         auto load_chunk = [&](const uint8_t *mat, uint32_t j, uint32_t c) {
             const uint32_t rtile = 2u * j + rh, chunk = kc * NKC + c;
-            const uint4 *qp = reinterpret_cast<const uint4 *>(mat + (((uint64_t)rtile * NC + chunk) * 16u + r) * 32u);
-            const uint16_t *dp = reinterpret_cast<const uint16_t *>(mat + qs_bytes) + ((uint64_t)rtile * HB + chunk / 2u) * 16u + r;
-            return RowChunk{qp[0], qp[1], *dp};
+            if constexpr (FMT == 0) {
+                const uint4 *qp = reinterpret_cast<const uint4 *>(mat + (((uint64_t)rtile * NC + chunk) * 16u + r) * 32u);
+                const uint16_t *dp = reinterpret_cast<const uint16_t *>(mat + qs_bytes) + ((uint64_t)rtile * HB + chunk / 2u) * 16u + r;
+                return RowChunk{qp[0], qp[1], *dp, 0u};
+            } else {
+                const uint64_t row = 16u * rtile + r;
+                const uint4 *qp = reinterpret_cast<const uint4 *>(mat + (row * HG + 4u * chunk) * 8u);
+                const uint32_t d = reinterpret_cast<const uint16_t *>(mat + qs_bytes)[row * HB + chunk / 2u];
+                return RowChunk{qp[0], qp[1], d, FMT == 1 ? *reinterpret_cast<const uint32_t *>(mat + sc_off + row * HG + 4u * chunk) : 0u};
+            }
         };
         const uint8_t *gmat = ex, *umat = ex + gate_bytes;
         RowChunk cg = load_chunk(gmat, j0, 0u), cu = load_chunk(umat, j0, 0u);
@@ -473,7 +543,7 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_gateup_reg_kernel(Tile
 #pragma unroll
                 for (uint32_t k = 0; k < 4u; ++k) {
                     const uint32_t g = 4u * c + k;
-                    const half8_t bg = decode_scaled(wg4[k], q, mag, sgn), bu = decode_scaled(wu4[k], q, mag, sgn);
+                    const half8_t bg = decode_reg<FMT>(wg4[k], cg.sc >> (8u * k), q, tables), bu = decode_reg<FMT>(wu4[k], cu.sc >> (8u * k), q, tables);
                     gh = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[g].v, bg, gh, 0, 0, 0);
                     gl = __builtin_amdgcn_mfma_f32_16x16x32_f16(xb[g].v, bg, gl, 0, 0, 0);
                     uh = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[g].v, bu, uh, 0, 0, 0);
@@ -527,19 +597,19 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_gateup_reg_kernel(Tile
 }
 
 // down. Wave w computes rows 128 b + 16 w + r for b = 0, 1, ... against all ffn columns of the tile; no reduction across waves.
-template <int NFG>          // ffn = 32 * NFG, NFG <= 16
+template <int NFG, int FMT>          // ffn = 32 * NFG, NFG <= 16; FMT as in the gate/up kernel
 __global__ __launch_bounds__(kRegWaves * 64) void prefill_down_reg_kernel(TiledArgs ta) {
     const PrefillArgs &a = ta.p;
     constexpr uint32_t F = 32u * NFG, FB = F / 256u, NCK = NFG / 4u;
-    __shared__ __attribute__((aligned(16))) uint8_t tables[kSignBytes + kScaledMagBytes];      // static: table reads take immediate offsets
+    __shared__ __attribute__((aligned(16))) uint8_t tables[reg_table_bytes<FMT>()];      // static: table reads take immediate offsets
     __shared__ __attribute__((aligned(16))) float pair_scale[2][kTile];      // per column half of the activations
     const uint32_t tid = threadIdx.x, lane = tid & 63u, r = lane & 15u, q = lane >> 4;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t H = a.hidden, P = a.ntok * a.top_k;
-    const uint8_t *sgn = tables, *mag = tables + kSignBytes;
-    build_scaled_tables(tables + kSignBytes, tables, tid, kRegWaves * 64u);
+    build_reg_tables<FMT>(tables, tid, kRegWaves * 64u, ta.grid);
     const uint32_t T = a.n_tiles[0], U = a.n_unique[0];
-    const uint64_t down_off = 2u * ((uint64_t)F * (H / 32u) * 8u + (uint64_t)F * (H / 256u) * 2u), qs_bytes = (uint64_t)H * NFG * 8u;
+    const uint64_t down_off = FMT == 0 ? 2u * ((uint64_t)F * (H / 32u) * 8u + (uint64_t)F * (H / 256u) * 2u) : ta.down_off, qs_bytes = (uint64_t)H * NFG * 8u;
+    const uint64_t sc_off = qs_bytes + (uint64_t)H * FB * 2u;
     constexpr uint32_t kRowsPerPass = 16u * kRegWaves;
 
     // Work items are half tiles (the row passes of a tile cut in two) so that the last round of the persistent workgroups is
@@ -556,7 +626,7 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_down_reg_kernel(TiledA
         if (tile != have_tile) {
             have_tile = tile;
             __syncthreads();
-            if (tid < 2u * kTile) pair_scale[tid & 1u][tid >> 1] = (tid >> 1) < n ? 0.125f * exp2i(a.act_exp[2u * p0 + tid]) : 0.0f;
+            if (tid < 2u * kTile) pair_scale[tid & 1u][tid >> 1] = (tid >> 1) < n ? (FMT == 2 ? 1.0f : 0.125f) * exp2i(a.act_exp[2u * p0 + tid]) : 0.0f;
             __syncthreads();
             const uint64_t base = (uint64_t)(p0 + r) * F + 8u * q;
             const bool live = r < n;
@@ -573,9 +643,16 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_down_reg_kernel(TiledA
         const float4_t ps0 = *reinterpret_cast<const float4_t *>(&pair_scale[0][4u * q]), ps1 = *reinterpret_cast<const float4_t *>(&pair_scale[1][4u * q]);
         auto load_chunk = [&](uint32_t b, uint32_t c) {
             const uint32_t rtile = kRegWaves * (pass0 + b) + wave;
-            const uint4 *qp = reinterpret_cast<const uint4 *>(dn + (((uint64_t)rtile * NCK + c) * 16u + r) * 32u);
-            const uint16_t *dp = reinterpret_cast<const uint16_t *>(dn + qs_bytes) + ((uint64_t)rtile * FB + c / 2u) * 16u + r;
-            return RowChunk{qp[0], qp[1], *dp};
+            if constexpr (FMT == 0) {
+                const uint4 *qp = reinterpret_cast<const uint4 *>(dn + (((uint64_t)rtile * NCK + c) * 16u + r) * 32u);
+                const uint16_t *dp = reinterpret_cast<const uint16_t *>(dn + qs_bytes) + ((uint64_t)rtile * FB + c / 2u) * 16u + r;
+                return RowChunk{qp[0], qp[1], *dp, 0u};
+            } else {
+                const uint64_t row = 16u * rtile + r;
+                const uint4 *qp = reinterpret_cast<const uint4 *>(dn + (row * NFG + 4u * c) * 8u);
+                const uint32_t d = reinterpret_cast<const uint16_t *>(dn + qs_bytes)[row * FB + c / 2u];
+                return RowChunk{qp[0], qp[1], d, FMT == 1 ? *reinterpret_cast<const uint32_t *>(dn + sc_off + row * NFG + 4u * c) : 0u};
+            }
         };
         // One buffer per chunk of a pass, reloaded with the same chunk of the next pass as soon as it has been decoded: every load
         // has a whole pass of work to arrive.
@@ -590,13 +667,14 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_down_reg_kernel(TiledA
             for (uint32_t c = 0; c < NCK; ++c) {
                 const uint2 w4[4] = {make_uint2(cw[c].a.x, cw[c].a.y), make_uint2(cw[c].a.z, cw[c].a.w), make_uint2(cw[c].b.x, cw[c].b.y), make_uint2(cw[c].b.z, cw[c].b.w)};
                 const float d = scale_to_f32(cw[c].d);
+                const uint32_t sc4 = cw[c].sc;
                 cw[c] = load_chunk(nb, c);
                 __builtin_amdgcn_sched_barrier(0);         // keeps the loads here: the scheduler otherwise sinks them to the end of the pass
                 float4_t hi = {0.0f, 0.0f, 0.0f, 0.0f}, lo = hi;
 #pragma unroll
                 for (uint32_t k = 0; k < 4u; ++k) {
                     const uint32_t g = 4u * c + k;
-                    const half8_t bw = decode_scaled(w4[k], q, mag, sgn);
+                    const half8_t bw = decode_reg<FMT>(w4[k], sc4 >> (8u * k), q, tables);
                     hi = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[g].v, bw, hi, 0, 0, 0);
                     lo = __builtin_amdgcn_mfma_f32_16x16x32_f16(xb[g].v, bw, lo, 0, 0, 0);
                 }
@@ -867,20 +945,26 @@ hipError_t launch_swiglu_rows(const float *gu, uint32_t gu_stride, uint32_t ntok
     return hipGetLastError();
 }
 
-static hipError_t launch_gateup_reg(const TiledArgs &ta, dim3 grid, hipStream_t s) {
+static hipError_t launch_gateup_reg(const TiledArgs &ta, dim3 grid, hipStream_t s, uint32_t fmt = 0u) {
     const uint32_t hidden = ta.p.hidden, ffn = ta.p.ffn;
     const size_t acts_lds = (size_t)kTile * (ffn + 4u) * sizeof(float);
     hipError_t e = hipSuccess;
     prof_set_stage(ST_PREFILL_GATEUP);
-#define REDHIP_PGR(NKC)                                                                                                                   \
+#define REDHIP_PGR_ONE(NKC, FMT)                                                                                                          \
     do {                                                                                                                                  \
         static bool attr = false;                                                                                                          \
         if (!attr) {                                                                                                                       \
-            e = hipFuncSetAttribute(reinterpret_cast<const void *>(prefill_gateup_reg_kernel<NKC>), hipFuncAttributeMaxDynamicSharedMemorySize, 40 * 1024); \
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(prefill_gateup_reg_kernel<NKC, FMT>), hipFuncAttributeMaxDynamicSharedMemorySize, 40 * 1024); \
             if (e != hipSuccess) return e;                                                                                                 \
             attr = true;                                                                                                                   \
         }                                                                                                                                  \
-        REDHIP_LAUNCH(prefill_gateup_reg_kernel<NKC>, grid, dim3(kRegWaves * 64), acts_lds, s, ta);                                        \
+        REDHIP_LAUNCH((prefill_gateup_reg_kernel<NKC, FMT>), grid, dim3(kRegWaves * 64), acts_lds, s, ta);                                 \
+    } while (0)
+#define REDHIP_PGR(NKC)                                                                                                                   \
+    do {                                                                                                                                  \
+        if (fmt == 1u) REDHIP_PGR_ONE(NKC, 1);                                                                                             \
+        else if (fmt == 2u) REDHIP_PGR_ONE(NKC, 2);                                                                                        \
+        else REDHIP_PGR_ONE(NKC, 0);                                                                                                       \
     } while (0)
     switch (hidden / 512u) {
         case 1: REDHIP_PGR(1); break;
@@ -889,6 +973,7 @@ static hipError_t launch_gateup_reg(const TiledArgs &ta, dim3 grid, hipStream_t 
         default: return hipErrorInvalidValue;
     }
 #undef REDHIP_PGR
+#undef REDHIP_PGR_ONE
     return hipGetLastError();
 }
 
@@ -909,9 +994,47 @@ hipError_t launch_prefill_gateup_tiled(const void *tiled_experts, uint64_t strid
     PrefillArgs a{nullptr, stride, nullptr, uid, pair_token, n_unique, tile_group, tile_pair0, tile_n, n_tiles, static_cast<const _Float16 *>(xh),
                   static_cast<const _Float16 *>(xl), xexp, static_cast<_Float16 *>(act_h), static_cast<_Float16 *>(act_l), act_exp, nullptr, nullptr, hidden,
                   ffn, top_k, ntok};
-    const TiledArgs ta{a, static_cast<const uint8_t *>(tiled_experts), nullptr, act};
+    const TiledArgs ta{a, static_cast<const uint8_t *>(tiled_experts), nullptr, act, nullptr, 0u};
     const uint32_t tile_bound = prefill_tile_bound(ntok, top_k, n_expert);
     return launch_gateup_reg(ta, dim3(tile_bound < 256u ? tile_bound : 256u), s);
+}
+
+// The routed gate/up and down matrices of a chunk on a layout whose experts are IQ2_XS / IQ1_M: the same tile kernels on the row-major
+// streams of the format (gate | up per expert at `packed`, the down matrix at `down`), decoded through the caller's codebooks. The
+// tile list is built here (no shared tiles); outputs as the IQ2_XXS tile kernels: fp16 activations per pair, then tmp [pairs][hidden].
+hipError_t launch_prefill_streams(uint32_t gate_up_type, const int8_t *gate_up_grid, const void *packed, uint64_t packed_stride, uint32_t down_type,
+                                  const int8_t *down_grid, const void *down, uint64_t down_stride, const uint32_t *uid, const uint32_t *expert_start,
+                                  const uint32_t *pair_token, const uint32_t *n_unique, uint32_t *tile_group, uint32_t *tile_pair0, uint32_t *tile_n,
+                                  uint32_t *n_tiles, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l, int *act_exp, float *tmp,
+                                  uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s) {
+    const auto fmt_of = [](uint32_t t) { return t == T_IQ2_XS ? 1u : t == T_IQ1_M ? 2u : 0u; };
+    const uint32_t fg = fmt_of(gate_up_type), fd = fmt_of(down_type);
+    if (!fg || !fd || !gate_up_grid || !down_grid || !packed || !down || !fused_iq2_supported(hidden, ffn) || hidden / 512u > 4u || (ffn != 256u && ffn != 512u) || !ntok)
+        return hipErrorInvalidValue;
+    const uint32_t P = ntok * top_k;
+    prof_set_stage(ST_GROUP);
+    REDHIP_LAUNCH(build_tiles_kernel, dim3(1), dim3(1024), 0, s, expert_start, n_unique, P, 0u, tile_group, tile_pair0, tile_n, n_tiles);      // no shared tiles
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    PrefillArgs a{nullptr, packed_stride, nullptr, uid, pair_token, n_unique, tile_group, tile_pair0, tile_n, n_tiles, static_cast<const _Float16 *>(xh),
+                  static_cast<const _Float16 *>(xl), xexp, static_cast<_Float16 *>(act_h), static_cast<_Float16 *>(act_l), act_exp, tmp, nullptr, hidden,
+                  ffn, top_k, ntok};
+    const uint32_t tile_bound = prefill_tile_bound(ntok, top_k, n_expert);
+    const dim3 grid(tile_bound < 256u ? tile_bound : 256u), rblock(kRegWaves * 64);
+    const TiledArgs tg{a, static_cast<const uint8_t *>(packed), nullptr, nullptr, gate_up_grid, 0u};
+    e = launch_gateup_reg(tg, grid, s, fg);
+    if (e != hipSuccess) return e;
+    a.stride = down_stride;
+    const TiledArgs td{a, static_cast<const uint8_t *>(down), nullptr, nullptr, down_grid, 0u};
+    prof_set_stage(ST_PREFILL_DOWN);
+    if (ffn == 256u) {
+        if (fd == 1u) REDHIP_LAUNCH((prefill_down_reg_kernel<8, 1>), grid, rblock, 0, s, td);
+        else REDHIP_LAUNCH((prefill_down_reg_kernel<8, 2>), grid, rblock, 0, s, td);
+    } else {
+        if (fd == 1u) REDHIP_LAUNCH((prefill_down_reg_kernel<16, 1>), grid, rblock, 0, s, td);
+        else REDHIP_LAUNCH((prefill_down_reg_kernel<16, 2>), grid, rblock, 0, s, td);
+    }
+    return hipGetLastError();
 }
 
 // routed down projection of a chunk on tile-major IQ3_S matrices, behind launch_prefill_gateup_tiled (its tile list and fp16 activations)
@@ -950,13 +1073,13 @@ hipError_t launch_prefill_packed(const void *experts, uint64_t stride, const voi
     const uint32_t tile_bound = prefill_tile_bound(ntok, top_k, n_expert);
     const dim3 grid(tile_bound < 256u ? tile_bound : 256u), block(kWaves * 64);
     if (tiled_experts && tiled_shared && ffn <= 512u) {          // tile-major copy present: activations of a tile in registers
-        const TiledArgs ta{a, static_cast<const uint8_t *>(tiled_experts), static_cast<const uint8_t *>(tiled_shared), nullptr};
+        const TiledArgs ta{a, static_cast<const uint8_t *>(tiled_experts), static_cast<const uint8_t *>(tiled_shared), nullptr, nullptr, 0u};
         const dim3 rblock(kRegWaves * 64);
         e = launch_gateup_reg(ta, grid, s);
         if (e != hipSuccess) return e;
         prof_set_stage(ST_PREFILL_DOWN);
-        if (ffn == 256u) REDHIP_LAUNCH(prefill_down_reg_kernel<8>, grid, rblock, 0, s, ta);
-        else REDHIP_LAUNCH(prefill_down_reg_kernel<16>, grid, rblock, 0, s, ta);
+        if (ffn == 256u) REDHIP_LAUNCH((prefill_down_reg_kernel<8, 0>), grid, rblock, 0, s, ta);
+        else REDHIP_LAUNCH((prefill_down_reg_kernel<16, 0>), grid, rblock, 0, s, ta);
         return hipGetLastError();
     }
     const size_t dyn_lds = (size_t)2u * kTile * (hidden + kRowPad) * 2u;

@@ -225,3 +225,28 @@ def test_mixed_layouts_other_shapes(layout, shape, grids):
         if ntok == 8:
             assert np.array_equal(out[5], out[1])
     m.close()
+
+
+@pytest.mark.parametrize("layout", ["xs", "m"])
+@pytest.mark.parametrize("shape,ntok", [((1024, 512, 16, 4), 48), ((512, 256, 16, 4), 33)])
+def test_codebook_layout_chunks(layout, shape, ntok, grids):
+    """prefill chunks on IQ2_XS / IQ1_M layers (tile kernels on the row-major streams): experts with several tiles (twenty requests carry
+    the same row), partial last tiles, experts nobody selected"""
+    from dwarfstar_red_lite_amd.moe import ResidentMoe
+    from test_gpu_moe_layer import ids_match_up_to_ties
+    orc.set_codebooks(*grids)
+    H, F, E, K = shape
+    cfg = synth.layer_config(hidden=H, ffn=F, n_expert=E, top_k=K, layout=layout)
+    m = ResidentMoe(cfg, n_layer=1, max_tokens=ntok)
+    lay = synth.make_layer(7 + H, cfg)
+    m.load_layer(0, lay)
+    xs = synth.normed_x(np.random.default_rng(23), ntok, H)
+    xs[5:25] = xs[4]
+    out = m.forward(0, torch.from_numpy(xs).cuda()).cpu().numpy()
+    gids, gw, glog = m.last_route(ntok)
+    want, cids, cw, clog = orc.Layer(cfg, **lay).forward(xs, threads=8)
+    for i in range(ntok):
+        assert ids_match_up_to_ties(gids[i], cids[i], clog[i])
+        assert rel_l2(out[i], want[i]) <= REL_L2_TOL, (layout, shape, i)
+    assert np.array_equal(out[7], out[4])
+    m.close()
