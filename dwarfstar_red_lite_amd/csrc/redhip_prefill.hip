@@ -850,18 +850,22 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_down_iq3s_kernel(Iq3Do
 
 // ---------------------------------------------------------------- router logits of a token chunk
 
-// logits[tok][e] = W[e] . x[tok] for an f32 router as a tiled product on v_mfma_f32_16x16x4_f32 (full fp32
-// multiply-add): a workgroup owns 16 router rows x 16 tokens and its four waves each take a quarter of the hidden dimension,
-// so that a compute unit holds enough waves to cover the load latency; the four partial tiles meet in LDS and are added in a
-// fixed order. Lane (r = l % 16, q = l / 16) loads four consecutive k of row r and of token r per 16 k and feeds them to four
-// MFMAs (A[i = r][k = q], B[k = q][j = r], D[i = 4q .. 4q + 3][j = r]); with `gate_inp` set, row E is that vector (the shared
-// expert's gate). A second kind of workgroup (blockIdx.x beyond the row tiles, launched when xh is set) does the fp16 split of
-// its tokens' activations. The same kernel multiplies any f32 matrix [E][H] with a chunk of activations (dense shared expert).
+// logits[tok][e] = W[e] . x[tok] for an f32 router as a tiled product on v_mfma_f32_16x16x4_f32 (full fp32 multiply-add): a workgroup
+// owns 32 rows x 32 tokens, wave (wr, wt) the 16 x 16 block of rows 16 wr .. and tokens 16 wt .. over the whole hidden dimension. Both
+// operands pass through LDS in slices of 64 k (double-buffered, one barrier per slice: the next two slices are in registers while this one
+// is multiplied), so a row or an activation vector is read from L2 once per workgroup instead of once per 16 x 16 block. Lane
+// (r = l % 16, q = l / 16) reads four consecutive k of row r and of token r per 16 k and feeds them to four MFMAs (A[i = r][k = q],
+// B[k = q][j = r], D[i = 4q .. 4q + 3][j = r]; the order of k inside a slice does not matter as long as both operands agree). With
+// `gate_inp` set, row E is that vector (the shared expert's gate). A second kind of workgroup (blockIdx.x beyond the row tiles,
+// launched when xh is set) does the fp16 split of its tokens' activations. The same kernel multiplies any f32 matrix [E][H] with a
+// chunk of activations (dense shared expert).
+constexpr uint32_t kGemmTile = 32u, kGemmK = 64u, kGemmRow = kGemmK + 4u;      // LDS row of 68 floats: the eight lanes of a 16-byte read pass hit different banks
+
 __global__ __launch_bounds__(256) void router_f32_tile_kernel(const float *w, const float *gate_inp, const float *x, float *logits, uint32_t out_stride,
                                                               _Float16 *xh, _Float16 *xl, int *xexp, uint32_t H, uint32_t E, uint32_t ntok) {
-    __shared__ float part[4][16][17];
+    __shared__ __attribute__((aligned(16))) float ws[2][kGemmTile][kGemmRow], xs[2][kGemmTile][kGemmRow];
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, r = lane & 15u, q = lane >> 4;
-    const uint32_t n_rows = E + (gate_inp ? 1u : 0u), row_tiles = (n_rows + 15u) / 16u;
+    const uint32_t n_rows = E + (gate_inp ? 1u : 0u), row_tiles = (n_rows + kGemmTile - 1u) / kGemmTile;
     if (blockIdx.x >= row_tiles) {                         // split job: one wave per token, 4 tokens per workgroup
         const uint32_t tok = 4u * (blockIdx.y * (gridDim.x - row_tiles) + (blockIdx.x - row_tiles)) + wave;
         if (tok >= ntok) return;
@@ -876,42 +880,63 @@ __global__ __launch_bounds__(256) void router_f32_tile_kernel(const float *w, co
         if (lane == 0u) xexp[tok] = e;
         return;
     }
-    const uint32_t row = 16u * blockIdx.x + r, tok = 16u * blockIdx.y + r, kq = H / 4u;          // this wave: k in [wave * kq, (wave + 1) * kq)
-    const float *wr = (row < E ? w + (uint64_t)row * H : gate_inp ? gate_inp : w) + wave * kq;      // rows beyond the last one repeat another and are not stored
-    const float *xt = x + (uint64_t)(tok < ntok ? tok : ntok - 1u) * H + wave * kq;
-    // 64 k per step: four loads of 16 bytes per operand, those of the next step in flight while this one is multiplied;
-    // two accumulators halve the chain of dependent MFMAs
+    // staging: thread t moves rows t / 16 and t / 16 + 16 of both operands, 16 bytes at column 4 (t % 16); rows beyond the last one
+    // repeat another and are not stored
+    const uint32_t srow = tid >> 4, scol = 4u * (tid & 15u);
+    const uint32_t row_a = kGemmTile * blockIdx.x + srow, row_b = row_a + 16u, tok_a = kGemmTile * blockIdx.y + srow, tok_b = tok_a + 16u;
+    const float *wsrc_a = (row_a < E ? w + (uint64_t)row_a * H : gate_inp ? gate_inp : w) + scol;
+    const float *wsrc_b = (row_b < E ? w + (uint64_t)row_b * H : gate_inp ? gate_inp : w) + scol;
+    const float *xsrc_a = x + (uint64_t)(tok_a < ntok ? tok_a : ntok - 1u) * H + scol;
+    const float *xsrc_b = x + (uint64_t)(tok_b < ntok ? tok_b : ntok - 1u) * H + scol;
+    const uint32_t wr = wave & 1u, wt = wave >> 1, n_slice = H / kGemmK;      // hidden is a multiple of 256: an even number of slices
+    // two register sets, one per LDS buffer: the loads of slice sl + 2 are issued while slice sl is multiplied, so an L2 round trip has two
+    // slices of arithmetic to hide behind (plain variables: arrays of them end up in scratch memory)
+    float4 w0a = *reinterpret_cast<const float4 *>(wsrc_a), w0b = *reinterpret_cast<const float4 *>(wsrc_b);
+    float4 x0a = *reinterpret_cast<const float4 *>(xsrc_a), x0b = *reinterpret_cast<const float4 *>(xsrc_b);
+    float4 w1a = *reinterpret_cast<const float4 *>(wsrc_a + kGemmK), w1b = *reinterpret_cast<const float4 *>(wsrc_b + kGemmK);
+    float4 x1a = *reinterpret_cast<const float4 *>(xsrc_a + kGemmK), x1b = *reinterpret_cast<const float4 *>(xsrc_b + kGemmK);
     float4_t acc0 = {0.0f, 0.0f, 0.0f, 0.0f}, acc1 = acc0;
-    float4 av[4], bv[4], an[4], bn[4];
+    auto multiply = [&](uint32_t buf) {
 #pragma unroll
-    for (int u = 0; u < 4; ++u) {
-        av[u] = *reinterpret_cast<const float4 *>(wr + 16u * u + 4u * q);
-        bv[u] = *reinterpret_cast<const float4 *>(xt + 16u * u + 4u * q);
-    }
-    for (uint32_t k0 = 0; k0 < kq; k0 += 64u) {
-        const uint32_t kn = k0 + 64u < kq ? k0 + 64u : k0;          // the last step reloads itself: no branch around the loads
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            an[u] = *reinterpret_cast<const float4 *>(wr + kn + 16u * u + 4u * q);
-            bn[u] = *reinterpret_cast<const float4 *>(xt + kn + 16u * u + 4u * q);
+        for (uint32_t u = 0; u < kGemmK / 16u; ++u) {
+            const float4 av = *reinterpret_cast<const float4 *>(&ws[buf][16u * wr + r][16u * u + 4u * q]);
+            const float4 bv = *reinterpret_cast<const float4 *>(&xs[buf][16u * wt + r][16u * u + 4u * q]);
+            acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(av.x, bv.x, acc0, 0, 0, 0);
+            acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(av.y, bv.y, acc1, 0, 0, 0);
+            acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(av.z, bv.z, acc0, 0, 0, 0);
+            acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(av.w, bv.w, acc1, 0, 0, 0);
         }
-#pragma unroll
-        for (int u = 0; u < 4; ++u) {
-            acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(av[u].x, bv[u].x, acc0, 0, 0, 0);
-            acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(av[u].y, bv[u].y, acc1, 0, 0, 0);
-            acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(av[u].z, bv[u].z, acc0, 0, 0, 0);
-            acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(av[u].w, bv[u].w, acc1, 0, 0, 0);
-        }
-#pragma unroll
-        for (int u = 0; u < 4; ++u) { av[u] = an[u]; bv[u] = bn[u]; }
+    };
+    for (uint32_t sl = 0; sl < n_slice; sl += 2u) {
+        *reinterpret_cast<float4 *>(&ws[0][srow][scol]) = w0a;
+        *reinterpret_cast<float4 *>(&ws[0][srow + 16u][scol]) = w0b;
+        *reinterpret_cast<float4 *>(&xs[0][srow][scol]) = x0a;
+        *reinterpret_cast<float4 *>(&xs[0][srow + 16u][scol]) = x0b;
+        __syncthreads();                                   // slice sl is in place; the readers of the other buffer (slice sl - 1) are past their barrier
+        const uint32_t k2 = (sl + 2u < n_slice ? sl + 2u : sl) * kGemmK;          // the last slices reload themselves: no branch around the loads
+        w0a = *reinterpret_cast<const float4 *>(wsrc_a + k2);
+        w0b = *reinterpret_cast<const float4 *>(wsrc_b + k2);
+        x0a = *reinterpret_cast<const float4 *>(xsrc_a + k2);
+        x0b = *reinterpret_cast<const float4 *>(xsrc_b + k2);
+        multiply(0u);
+        *reinterpret_cast<float4 *>(&ws[1][srow][scol]) = w1a;
+        *reinterpret_cast<float4 *>(&ws[1][srow + 16u][scol]) = w1b;
+        *reinterpret_cast<float4 *>(&xs[1][srow][scol]) = x1a;
+        *reinterpret_cast<float4 *>(&xs[1][srow + 16u][scol]) = x1b;
+        __syncthreads();
+        const uint32_t k3 = (sl + 3u < n_slice ? sl + 3u : sl + 1u) * kGemmK;
+        w1a = *reinterpret_cast<const float4 *>(wsrc_a + k3);
+        w1b = *reinterpret_cast<const float4 *>(wsrc_b + k3);
+        x1a = *reinterpret_cast<const float4 *>(xsrc_a + k3);
+        x1b = *reinterpret_cast<const float4 *>(xsrc_b + k3);
+        multiply(1u);
     }
+    const uint32_t out_tok = kGemmTile * blockIdx.y + 16u * wt + r;
 #pragma unroll
-    for (uint32_t t = 0; t < 4u; ++t) part[wave][r][4u * q + t] = acc0[t] + acc1[t];          // [token j][row i]
-    __syncthreads();
-    const uint32_t i = tid & 15u, j = tid >> 4;             // consecutive threads store consecutive rows of one token
-    const uint32_t out_row = 16u * blockIdx.x + i, out_tok = 16u * blockIdx.y + j;
-    if (out_tok < ntok && out_row < n_rows)
-        logits[(uint64_t)out_tok * out_stride + out_row] = (part[0][j][i] + part[1][j][i]) + (part[2][j][i] + part[3][j][i]);
+    for (uint32_t t = 0; t < 4u; ++t) {
+        const uint32_t out_row = kGemmTile * blockIdx.x + 16u * wr + 4u * q + t;
+        if (out_tok < ntok && out_row < n_rows) logits[(uint64_t)out_tok * out_stride + out_row] = acc0[t] + acc1[t];
+    }
 }
 
 // out[tok][row] = W[row] . x[tok] for an f32 matrix W [n_rows][K] and a chunk of activations x [ntok][K]; extra_row (optional) is one more
@@ -919,7 +944,7 @@ __global__ __launch_bounds__(256) void router_f32_tile_kernel(const float *w, co
 hipError_t launch_f32_tiles(const float *w, const float *extra_row, const float *x, uint32_t ntok, uint32_t K, uint32_t n_rows, float *out,
                             uint32_t out_stride, void *xh, void *xl, int *xexp, hipStream_t s) {
     if (!ntok || !K || K % 256u || !n_rows || !w || !x || !out) return hipErrorInvalidValue;
-    const uint32_t row_tiles = (n_rows + (extra_row ? 1u : 0u) + 15u) / 16u, tok_tiles = (ntok + 15u) / 16u;
+    const uint32_t row_tiles = (n_rows + (extra_row ? 1u : 0u) + kGemmTile - 1u) / kGemmTile, tok_tiles = (ntok + kGemmTile - 1u) / kGemmTile;
     if (tok_tiles > 65535u) return hipErrorInvalidValue;
     const uint32_t split_wgs = xh ? ((ntok + 3u) / 4u + tok_tiles - 1u) / tok_tiles : 0u;            // per blockIdx.y
     REDHIP_LAUNCH(router_f32_tile_kernel, dim3(row_tiles + split_wgs, tok_tiles), dim3(256), 0, s, w, extra_row, x, out, out_stride,
