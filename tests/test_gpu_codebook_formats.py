@@ -250,3 +250,28 @@ def test_codebook_layout_chunks(layout, shape, ntok, grids):
         assert rel_l2(out[i], want[i]) <= REL_L2_TOL, (layout, shape, i)
     assert np.array_equal(out[7], out[4])
     m.close()
+
+
+@pytest.mark.parametrize("layout", ["xs", "m"])
+def test_codebook_layout_given_routing(layout, grids):
+    """caller-given routing (drawn logits with hot experts, so tokens share experts) on IQ2_XS / IQ1_M layers: batches of 2 (single-token
+    kernels), 3 and 8 (grouped kernels) and a chunk of 40 tokens, against the oracle run token by token"""
+    from dwarfstar_red_lite_amd.moe import ResidentMoe
+    from test_gpu_moe_batch import oracle_tokens
+    orc.set_codebooks(*grids)
+    cfg = synth.layer_config(hidden=1024, ffn=512, n_expert=64, top_k=6, layout=layout)
+    lay = synth.make_layer(321, cfg)
+    m = ResidentMoe(cfg, n_layer=1, max_tokens=40)
+    m.load_layer(0, lay)
+    rng = np.random.default_rng(77)
+    for ntok in (2, 3, 8, 40):
+        x = synth.normed_x(rng, ntok, cfg["hidden"])
+        logits = synth.hot_logits(rng, ntok, cfg["n_expert"])
+        sel = [orc.router_select(logits[t], cfg["top_k"]) for t in range(ntok)]
+        ids = np.stack([s[0] for s in sel])
+        w = np.stack([s[1] for s in sel])
+        got = m.experts(0, torch.from_numpy(x).cuda(), torch.from_numpy(ids.astype(np.int32)).cuda(), torch.from_numpy(w).cuda()).cpu().numpy()
+        want = oracle_tokens(cfg, lay, x, ids, w)
+        for t in range(ntok):
+            assert rel_l2(got[t], want[t]) <= REL_L2_TOL, (layout, ntok, t)
+    m.close()
