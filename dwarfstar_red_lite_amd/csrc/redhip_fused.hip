@@ -543,12 +543,25 @@ hipError_t launch_router_gemv(uint32_t router_type, const void *w, const float *
         const float *wf = static_cast<const float *>(w);
         const dim3 mgrid((n_expert + 1u + 2u * ffn + 7u) / 8u);
         const size_t lds = (size_t)ntok * hidden * 4u;
+        // (64 KB of activations at 8 tokens of 2048, beside a few static bytes: the limit is raised explicitly)
+#define REDHIP_RMULTI(NV)                                                                                                                                  \
+    do {                                                                                                                                                   \
+        static bool attr = false;                                                                                                                           \
+        if (!attr) {                                                                                                                                        \
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(router_f32_multi_kernel<NV, 8>), hipFuncAttributeMaxDynamicSharedMemorySize, 72 * 1024); \
+            if (e != hipSuccess) return e;                                                                                                                  \
+            attr = true;                                                                                                                                    \
+        }                                                                                                                                                   \
+        REDHIP_LAUNCH((router_f32_multi_kernel<NV, 8>), mgrid, dim3(512), lds, s, wf, a, ntok);                                                             \
+        return hipGetLastError();                                                                                                                           \
+    } while (0)
         switch (hidden / 256u) {
-            case 2: REDHIP_LAUNCH((router_f32_multi_kernel<2, 8>), mgrid, dim3(512), lds, s, wf, a, ntok); return hipGetLastError();
-            case 4: REDHIP_LAUNCH((router_f32_multi_kernel<4, 8>), mgrid, dim3(512), lds, s, wf, a, ntok); return hipGetLastError();
-            case 8: REDHIP_LAUNCH((router_f32_multi_kernel<8, 8>), mgrid, dim3(512), lds, s, wf, a, ntok); return hipGetLastError();
+            case 2: REDHIP_RMULTI(2);
+            case 4: REDHIP_RMULTI(4);
+            case 8: REDHIP_RMULTI(8);
             default: break;
         }
+#undef REDHIP_RMULTI
     }
     if (router_type == T_F32) {
         const float *wf = static_cast<const float *>(w);
