@@ -71,9 +71,10 @@ struct Moe {
     uint8_t *stage = nullptr;                // upload staging for handles that do not keep the raw rows: kStageExperts slots
     static constexpr uint32_t kStageExperts = 64u;
     // handles that can be given chunks keep a tile-major copy for the prefill kernels that hold a tile's activations in registers
-    // chunks of 16 tokens and more take the router as a tiled f32 product (a quantised router through its f32 copy)
+    // larger chunks take the router as a tiled f32 product (a quantised router through its f32 copy)
+    // (an F32 router below 48 tokens is quicker one token per grid layer: 32 x 32 tiles leave most of the chip idle there)
     bool tiled_router(uint32_t ntok) const {
-        return packed_gu() && ntok >= 16u && (cfg.router_type == T_F32 || mixed);
+        return packed_gu() && ntok >= (cfg.router_type == T_F32 ? 48u : 16u) && (cfg.router_type == T_F32 || mixed);
     }
     bool tiles_resident() const { return packed_gu() && gu_type == T_IQ2_XXS && cfg.max_tokens > 8u && cfg.ffn <= 512u && cfg.hidden / 512u <= 4u; }
     // a chunk on a mixed layout: the routed gate/up matrices (packed IQ2_XXS) run on the prefill tiles, the rest on raw rows
