@@ -129,7 +129,13 @@ struct Moe {
     // a chunk on a mixed layout that has no tile kernels (ffn > 512, or IQ2_XS / IQ1_M gate/up beside another down format) runs as slices
     // of 8 tokens on the grouped small-batch kernels, far ahead of the generic per-pair kernels on raw rows
     static constexpr uint32_t kSlice = 8u;
-    bool sliced(uint32_t ntok) const { return mixed && ntok > kSlice && !tiles_resident() && !stream_chunk(ntok) && grouped_mixed(kSlice); }
+    // So does every layout from 9 to 16 tokens: two small batches are quicker than one chunk, whose tile kernels leave most workgroups
+    // without work at that size.
+    bool sliced(uint32_t ntok) const {
+        if (ntok <= kSlice) return false;
+        if (ntok <= 2u * kSlice && (small_batch(kSlice) || grouped_mixed(kSlice))) return true;
+        return mixed && !tiles_resident() && !stream_chunk(ntok) && grouped_mixed(kSlice);
+    }
     // the workspace entries a caller can read back (redhip_moe_last_route) of the slice that starts at token t0 sit at their place in the chunk
     void shift_route_outputs(int64_t t0) {
         ids += t0 * (int64_t)cfg.top_k;

@@ -21,7 +21,7 @@ def oracle_block(cfg, lay, x, branch, w, eps):
     return (resid + ffn.astype(np.float32)).astype(np.float32), normed, ids
 
 
-@pytest.mark.parametrize("layout,ntok", [("iq2", 1), ("f2", 1), ("iq2", 3), ("f2", 2), ("f2", 6), ("iq2", 24)])
+@pytest.mark.parametrize("layout,ntok", [("iq2", 1), ("f2", 1), ("iq2", 3), ("f2", 2), ("f2", 6), ("iq2", 12), ("f2", 13), ("iq2", 24)])
 def test_block_step_matches_cpu(layout, ntok):
     """one token (norm inside the router launch, residual in the down kernel) on both layouts, a small batch, a batch on the
     generic kernels, and a chunk (separate norm kernel, tiled router, MFMA tiles, residual in the combine kernel)"""
