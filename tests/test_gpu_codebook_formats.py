@@ -195,7 +195,7 @@ def test_resident_layer(layout, shape, grids):
 
 
 @pytest.mark.parametrize("layout", ["f2", "xs", "m"])
-@pytest.mark.parametrize("shape", [(1024, 768, 24, 12), (4096, 1024, 16, 2), (2048, 1024, 16, 4), (512, 256, 16, 4)])
+@pytest.mark.parametrize("shape", [(1024, 768, 24, 12), (4096, 1024, 16, 2), (2048, 1024, 16, 4), (512, 256, 16, 4), (512, 256, 4, 1), (1024, 256, 2, 2)])
 def test_mixed_layouts_other_shapes(layout, shape, grids):
     """mixed-precision layers away from the benchmark shape: 13 slots (the 16-wave kernels), ffn 768 / 1024 (two column chunks per
     lane), hidden 512 .. 4096; one token, a pair, grouped batches, with dequantisation from the copies the kernels read"""
