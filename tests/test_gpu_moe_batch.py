@@ -138,3 +138,28 @@ def test_prefill_chunk_forward_config_shape(layout):
     assert np.abs(gw - cw).max() <= 1e-5
     assert max(rel_l2(got[t], want[t]) for t in range(ntok)) <= REL_L2_TOL
     m.close()
+
+
+@pytest.mark.parametrize("down_type", [synth.TYPE_Q6_K, synth.TYPE_IQ2_XXS])
+def test_mixed_layout_raw_down_rows(down_type):
+    """mixed layers whose routed down matrices have no packed copy (Q6_K, or IQ2_XXS beside a Q6_K shared expert): the raw-row down
+    kernels for one token, a pair, grouped batches and a chunk"""
+    from dwarfstar_red_lite_amd.moe import ResidentMoe
+    cfg = synth.layer_config(hidden=1024, ffn=512, n_expert=32, top_k=6, layout="f2")
+    cfg["down_type"] = down_type
+    lay = synth.make_layer(911, cfg)
+    m = ResidentMoe(cfg, n_layer=1, max_tokens=20)
+    m.load_layer(0, lay)
+    ref = orc.Layer(cfg, **lay)
+    xs = synth.normed_x(np.random.default_rng(3), 20, cfg["hidden"])
+    xs[6] = xs[2]
+    for ntok in (1, 2, 5, 8, 20):
+        out = m.forward(0, torch.from_numpy(xs[:ntok].copy()).cuda()).cpu().numpy()
+        gids, gw, glog = m.last_route(ntok)
+        want, cids, cw, clog = ref.forward(xs[:ntok], threads=8)
+        assert np.array_equal(gids, cids)
+        for i in range(ntok):
+            assert rel_l2(out[i], want[i]) <= REL_L2_TOL, (down_type, ntok, i)
+        if ntok >= 8:
+            assert np.array_equal(out[6], out[2])
+    m.close()
