@@ -163,3 +163,22 @@ def test_mixed_layout_raw_down_rows(down_type):
         if ntok >= 8:
             assert np.array_equal(out[6], out[2])
     m.close()
+
+
+def test_chunk_as_slices_of_small_batches():
+    """a layout without tile kernels (ffn 768): forward() of 20 tokens runs as slices of 8 on the grouped small-batch kernels, the route
+    of every token at its place in the chunk"""
+    from dwarfstar_red_lite_amd.moe import ResidentMoe
+    cfg = synth.layer_config(hidden=1024, ffn=768, n_expert=24, top_k=12, layout="f2")
+    lay = synth.make_layer(505, cfg)
+    m = ResidentMoe(cfg, n_layer=1, max_tokens=20)
+    m.load_layer(0, lay)
+    xs = synth.normed_x(np.random.default_rng(9), 20, cfg["hidden"])
+    out = m.forward(0, torch.from_numpy(xs).cuda()).cpu().numpy()
+    gids, gw, glog = m.last_route(20)
+    want, cids, cw, clog = orc.Layer(cfg, **lay).forward(xs, threads=8)
+    assert np.array_equal(gids, cids)
+    assert np.all(np.abs(gw - cw) <= 1e-6 + 1e-5 * cw)
+    for i in range(20):
+        assert rel_l2(out[i], want[i]) <= REL_L2_TOL, i
+    m.close()
