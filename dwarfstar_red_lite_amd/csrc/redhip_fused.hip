@@ -295,6 +295,7 @@ struct RouterArgs {
     const float *branch, *norm_w;
     float eps;
     float *xn_out;             // [ntok][hidden]
+    float *scalar_out;         // optional [ntok]: sigmoid of the gate logit (row n_expert), for callers that bring their own routing
 };
 
 // fp16 split of x, spread over the whole grid (every workgroup knows the largest |x| of its token)
@@ -364,6 +365,7 @@ __global__ __launch_bounds__(256) void router_f32_kernel(const float *w, RouterA
     acc = wave_sum(acc);
     if (lane == 0u && r <= a.n_expert) a.logits[(uint64_t)tok * (a.n_expert + 1u) + r] = acc;
     else if (lane == 0u && r < n_rows) a.sh_gu[(uint64_t)tok * 2u * a.ffn + (r - a.n_expert - 1u)] = acc;
+    if (lane == 0u && r == a.n_expert && a.scalar_out) a.scalar_out[tok] = 1.0f / (1.0f + expf(-acc));      // as the selection computes it
     split_x_job(a, tok, wave_max(amax), norm_inv);
 }
 
@@ -431,6 +433,7 @@ __global__ __launch_bounds__(NWV * 64) void router_f32_multi_kernel(const float 
         acc = wave_sum(acc);
         if (lane == 0u && r <= a.n_expert) a.logits[(uint64_t)tok * (a.n_expert + 1u) + r] = acc;
         else if (lane == 0u && r < n_rows) a.sh_gu[(uint64_t)tok * 2u * a.ffn + (r - a.n_expert - 1u)] = acc;
+        if (lane == 0u && r == a.n_expert && a.scalar_out) a.scalar_out[tok] = 1.0f / (1.0f + expf(-acc));      // as the selection computes it
         split_x_job(a, tok, s_amax[tok], s_ninv[tok]);
     }
 }
@@ -527,7 +530,7 @@ __global__ __launch_bounds__(256) void router_quant_kernel(const uint8_t *w, Rou
 
 hipError_t launch_router_gemv(uint32_t router_type, const void *w, const float *x, const float *gate_inp, uint32_t ntok, uint32_t hidden,
                               uint32_t n_expert, float *logits, void *xh, void *xl, int *xexp, const void *sh_q6k, float *sh_gu, uint32_t ffn,
-                              hipStream_t s, const float *sh_dense) {
+                              hipStream_t s, const float *sh_dense, float *scalar_out) {
     if (!ntok || !hidden || hidden % 256u || (!n_expert && !sh_dense) || n_expert > 1024u) return hipErrorInvalidValue;      // n_expert 0: only the shared expert's rows
     const bool with_shared = sh_q6k && sh_gu && router_type == T_Q6_K && ntok <= 8u && ffn % 4u == 0u;      // sh_gu: [ntok][2 * ffn]
     const BlockContext &bc = block_context();
@@ -535,7 +538,7 @@ hipError_t launch_router_gemv(uint32_t router_type, const void *w, const float *
     const bool with_dense = sh_dense && sh_gu && router_type == T_F32 && ntok <= 8u;      // sh_gu: [ntok][2 * ffn]
     RouterArgs a{x, gate_inp, logits, static_cast<_Float16 *>(xh), static_cast<_Float16 *>(xl), xexp, hidden, n_expert,
                  with_shared ? static_cast<const uint8_t *>(sh_q6k) : nullptr, with_dense ? sh_dense : nullptr, sh_gu, ffn, bc.branch, bc.norm_w, bc.eps,
-                 bc.xn_out};
+                 bc.xn_out, scalar_out};
     const dim3 grid((n_expert + 1u + (with_dense ? 2u * ffn : 0u) + 3u) / 4u, ntok);
     // with the shared expert's rows behind the router's (1537 rows at the benchmark shape) a row is read once for the whole batch; the
     // router's own 513 rows are quicker one token per grid layer (their re-reads hit the L2)

@@ -184,7 +184,7 @@ hipError_t launch_dequant_packed_iq2xxs(const void *packed, uint32_t nrows, uint
 // logits [ntok][n_expert + 1] (entry n_expert = gate_inp . x) and the fp16 split of x: xh, xl [ntok][hidden], xexp [ntok]
 hipError_t launch_router_gemv(uint32_t router_type, const void *w, const float *x, const float *gate_inp, uint32_t ntok, uint32_t hidden,
                               uint32_t n_expert, float *logits, void *xh, void *xl, int *xexp, const void *sh_q6k, float *sh_gu, uint32_t ffn,
-                              hipStream_t s, const float *sh_dense = nullptr);      // sh_dense: f32 [2 ffn][hidden] shared gate | up rows (F32 router, <= 8 tokens)
+                              hipStream_t s, const float *sh_dense = nullptr, float *scalar_out = nullptr);      // sh_dense: f32 [2 ffn][hidden] shared gate | up rows (F32 router, <= 8 tokens)
 // softmax top-k of logits [ntok][n_expert + 1]; scalar[t] = sigmoid(logits[t][n_expert]); optional probs [ntok][n_expert]
 hipError_t launch_select(const float *logits, uint32_t ntok, uint32_t n_expert, uint32_t top_k, uint32_t *ids, float *weights, float *scalar,
                          float *probs, hipStream_t s);

@@ -647,16 +647,18 @@ int redhip_moe_experts(redhip_moe_t h, uint32_t layer, const float *x_dev, uint3
     hipStream_t s = static_cast<hipStream_t>(stream);
     m->shared_gu_ready = false;
     if (m->packed_path(ntok) || m->small_batch_mixed(ntok) || m->mixed_chunk(ntok) || m->stream_chunk(ntok)) {
-        prof_set_stage(ST_OTHER);
-        HIP_OK(launch_prep(x_dev, m->layers[layer].gate_inp, ntok, m->cfg.hidden, m->xh, m->xl, m->xexp, m->scalar, s), "prep launch");
         const Layer &L = m->layers[layer];
         const uint32_t nv = m->cfg.hidden / 256u;
         if (m->grouped_mixed(ntok) && L.dense_gu && (nv == 2u || nv == 4u || nv == 8u || nv == 16u)) {
-            // the grouped kernels take the shared expert's gate | up products as an input: one f32 GEMV over its f32 copy (no router rows)
+            // the grouped kernels take the shared expert's gate | up products as an input: one f32 GEMV over its f32 copy (no router rows),
+            // which also leaves the fp16 halves of x and the shared expert's scalar gate
             prof_set_stage(ST_SHARED_GATEUP);
             HIP_OK(launch_router_gemv(T_F32, L.dense_gu, x_dev, L.gate_inp, ntok, m->cfg.hidden, 0u, m->logits, m->xh, m->xl, m->xexp, nullptr, m->act,
-                                      m->cfg.ffn, s, L.dense_gu), "shared gate/up launch");
+                                      m->cfg.ffn, s, L.dense_gu, m->scalar), "shared gate/up launch");
             m->shared_gu_ready = true;
+        } else {
+            prof_set_stage(ST_OTHER);
+            HIP_OK(launch_prep(x_dev, L.gate_inp, ntok, m->cfg.hidden, m->xh, m->xl, m->xexp, m->scalar, s), "prep launch");
         }
         const int ok = experts_enqueue(m, layer, x_dev, ntok, ids_dev, weights_dev, out_dev, s);
         m->shared_gu_ready = false;
