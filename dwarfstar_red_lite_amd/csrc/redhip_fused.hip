@@ -276,6 +276,62 @@ __device__ __forceinline__ float q6k_dot32(const uint8_t *row, uint32_t chunk, c
     return d * (s0 * fmaf(-32.0f, sx0, acc0) + s1 * fmaf(-32.0f, sx1, acc1));
 }
 
+// ---------------------------------------------------------------- grouping of at most 128 (token, k) pairs by expert
+
+// Same outputs as the host pair sort it replaces: groups in first-appearance order, pairs of a group in token order.
+// A table in LDS holds, per expert, the set of tokens that selected it (a token selects an expert at most once): the
+// position of a pair inside its group and the group's size are bit counts of that set, the order of the groups a
+// bit count over the "first pair of its expert" flags, the group offsets one prefix sum. Run by a whole workgroup
+// of at least 128 threads (every thread reaches the barriers); at most 16 tokens, 128 pairs, 1024 experts.
+constexpr uint32_t kGroupLdsWords = 1024u + 4u;
+template <class PairId, class PairWeight>
+__device__ __forceinline__ void group_small(const GroupJob &g, uint32_t *lds, PairId pair_id, PairWeight pair_w) {
+    uint32_t *token_set = lds;                           // per expert: bit t = token t selected it; later the group's offset
+    uint32_t *first_count = lds + 1024, *size_total = lds + 1026;
+    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, K = g.top_k;
+    for (uint32_t i = tid; i < g.n_expert; i += blockDim.x) token_set[i] = 0u;
+    __syncthreads();
+    const uint32_t P = g.ntok * K, pr = tid;             // pair index (waves 0 and 1)
+    const bool live = pr < P;
+    const uint32_t t = live ? pr / K : 0u;
+    const uint32_t e = live ? pair_id(t, pr % K) : 0u;
+    if (live) atomicOr(&token_set[e], 1u << t);
+    __syncthreads();
+    const uint32_t set = live ? token_set[e] : 0u;
+    const uint32_t n = (uint32_t)__popc(set), before = (uint32_t)__popc(set & ((1u << t) - 1u));
+    const bool first = live && before == 0u;
+    uint32_t scan = first ? n : 0u;                      // inclusive prefix sum of the group sizes in pair order
+    if (wave < 2u) {
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const uint32_t up = __shfl_up(scan, o, 64);
+            if (lane >= (uint32_t)o) scan += up;
+        }
+        const uint64_t fm = __ballot(first);
+        if (lane == 63u) { first_count[wave] = (uint32_t)__popcll(fm); size_total[wave] = scan; }
+    }
+    const uint64_t first_mask = __ballot(first);
+    __syncthreads();
+    const uint32_t grp = (wave == 1u ? first_count[0] : 0u) + __builtin_amdgcn_mbcnt_hi((uint32_t)(first_mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)first_mask, 0u));
+    const uint32_t start = (wave == 1u ? size_total[0] : 0u) + scan - (first ? n : 0u);
+    if (first) { token_set[e] = start; g.uid[grp] = e; g.expert_start[grp] = start; }
+    if (tid == 0u) { const uint32_t U = first_count[0] + first_count[1]; g.expert_start[U] = P; g.n_unique[0] = U; }
+    __syncthreads();
+    if (live) {
+        const uint32_t pos = token_set[e] + before;
+        g.pair_token[pos] = t;
+        g.pair_weight[pos] = pair_w(t, pr % K);
+        g.tok_pair[pr] = pos;
+    }
+}
+// the same from routing held in device memory (kernels that carry the grouping as a side job of one extra workgroup)
+__device__ __forceinline__ void group_small_given(const GroupJob &g, uint32_t *lds) {
+    group_small(g, lds, [&](uint32_t t, uint32_t k) { return g.ids[t * g.top_k + k]; }, [&](uint32_t t, uint32_t k) { return g.weights[t * g.top_k + k]; });
+}
+__host__ inline bool group_job_fits(const GroupJob &g) {
+    return g.ids && g.weights && g.ntok && g.ntok <= 16u && g.top_k && g.top_k <= 16u && g.ntok * g.top_k <= 128u && g.n_expert && g.n_expert <= 1024u;
+}
+
 // ---------------------------------------------------------------- router GEMV
 
 struct RouterArgs {
@@ -299,8 +355,8 @@ struct RouterArgs {
 };
 
 // fp16 split of x, spread over the whole grid (every workgroup knows the largest |x| of its token)
-__device__ __forceinline__ void split_x_job(const RouterArgs &a, uint32_t tok, float amax, float norm_inv) {
-    const uint32_t gt = blockIdx.x * blockDim.x + threadIdx.x, nt = gridDim.x * blockDim.x;
+__device__ __forceinline__ void split_x_job(const RouterArgs &a, uint32_t tok, float amax, float norm_inv, uint32_t n_blocks) {
+    const uint32_t gt = blockIdx.x * blockDim.x + threadIdx.x, nt = n_blocks * blockDim.x;
     const int e = prescale_exp(amax);
     const float inv = exp2i(-e);
     const uint64_t base = (uint64_t)tok * a.hidden;
@@ -366,15 +422,20 @@ __global__ __launch_bounds__(256) void router_f32_kernel(const float *w, RouterA
     if (lane == 0u && r <= a.n_expert) a.logits[(uint64_t)tok * (a.n_expert + 1u) + r] = acc;
     else if (lane == 0u && r < n_rows) a.sh_gu[(uint64_t)tok * 2u * a.ffn + (r - a.n_expert - 1u)] = acc;
     if (lane == 0u && r == a.n_expert && a.scalar_out) a.scalar_out[tok] = 1.0f / (1.0f + expf(-acc));      // as the selection computes it
-    split_x_job(a, tok, wave_max(amax), norm_inv);
+    split_x_job(a, tok, wave_max(amax), norm_inv, gridDim.x);
 }
 
 // The same product for 2..8 tokens at once: a wave keeps its row in registers and walks the tokens, whose activation vectors (after the
 // optional residual + norm, done by wave t for token t) sit in LDS, so a row is read once per batch instead of once per token.
 template <int NV, int NWV>          // NWV waves (rows) per workgroup
-__global__ __launch_bounds__(NWV * 64) void router_f32_multi_kernel(const float *w, RouterArgs a, uint32_t ntok) {
+__global__ __launch_bounds__(NWV * 64) void router_f32_multi_kernel(const float *w, RouterArgs a, uint32_t ntok, GroupJob job) {
     extern __shared__ __attribute__((aligned(16))) float xs_all[];      // [ntok][hidden]
     __shared__ float s_amax[8], s_ninv[8];
+    const uint32_t n_blocks = gridDim.x - (job.ids ? 1u : 0u);
+    if (blockIdx.x == n_blocks) {                        // the extra workgroup: pair sort of the caller's routing
+        group_small_given(job, reinterpret_cast<uint32_t *>(xs_all));
+        return;
+    }
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63u, H = a.hidden;
     const uint32_t r = blockIdx.x * (uint32_t)NWV + wave;
     const uint32_t n_rows = a.n_expert + 1u + (a.sh_dense ? 2u * a.ffn : 0u);
@@ -434,7 +495,7 @@ __global__ __launch_bounds__(NWV * 64) void router_f32_multi_kernel(const float 
         if (lane == 0u && r <= a.n_expert) a.logits[(uint64_t)tok * (a.n_expert + 1u) + r] = acc;
         else if (lane == 0u && r < n_rows) a.sh_gu[(uint64_t)tok * 2u * a.ffn + (r - a.n_expert - 1u)] = acc;
         if (lane == 0u && r == a.n_expert && a.scalar_out) a.scalar_out[tok] = 1.0f / (1.0f + expf(-acc));      // as the selection computes it
-        split_x_job(a, tok, s_amax[tok], s_ninv[tok]);
+        split_x_job(a, tok, s_amax[tok], s_ninv[tok], n_blocks);
     }
 }
 
@@ -525,17 +586,18 @@ __global__ __launch_bounds__(256) void router_quant_kernel(const uint8_t *w, Rou
         acc = wave_sum(acc);
         if (lane == 0u) a.logits[(uint64_t)tok * (a.n_expert + 1u) + r] = acc;
     }
-    split_x_job(a, tok, amax, norm_inv);
+    split_x_job(a, tok, amax, norm_inv, gridDim.x);
 }
 
 hipError_t launch_router_gemv(uint32_t router_type, const void *w, const float *x, const float *gate_inp, uint32_t ntok, uint32_t hidden,
                               uint32_t n_expert, float *logits, void *xh, void *xl, int *xexp, const void *sh_q6k, float *sh_gu, uint32_t ffn,
-                              hipStream_t s, const float *sh_dense, float *scalar_out) {
+                              hipStream_t s, const float *sh_dense, float *scalar_out, const GroupJob *job, bool *job_done) {
     if (!ntok || !hidden || hidden % 256u || (!n_expert && !sh_dense) || n_expert > 1024u) return hipErrorInvalidValue;      // n_expert 0: only the shared expert's rows
     const bool with_shared = sh_q6k && sh_gu && router_type == T_Q6_K && ntok <= 8u && ffn % 4u == 0u;      // sh_gu: [ntok][2 * ffn]
     const BlockContext &bc = block_context();
     if (bc.branch && (!bc.norm_w || !bc.xn_out)) return hipErrorInvalidValue;
     const bool with_dense = sh_dense && sh_gu && router_type == T_F32 && ntok <= 8u;      // sh_gu: [ntok][2 * ffn]
+    if (job_done) *job_done = false;
     RouterArgs a{x, gate_inp, logits, static_cast<_Float16 *>(xh), static_cast<_Float16 *>(xl), xexp, hidden, n_expert,
                  with_shared ? static_cast<const uint8_t *>(sh_q6k) : nullptr, with_dense ? sh_dense : nullptr, sh_gu, ffn, bc.branch, bc.norm_w, bc.eps,
                  bc.xn_out, scalar_out};
@@ -544,8 +606,11 @@ hipError_t launch_router_gemv(uint32_t router_type, const void *w, const float *
     // router's own 513 rows are quicker one token per grid layer (their re-reads hit the L2)
     if (router_type == T_F32 && with_dense && ntok >= 2u && (size_t)ntok * hidden * 4u <= 64u * 1024u) {
         const float *wf = static_cast<const float *>(w);
-        const dim3 mgrid((n_expert + 1u + 2u * ffn + 7u) / 8u);
-        const size_t lds = (size_t)ntok * hidden * 4u;
+        const bool with_job = job && job_done && group_job_fits(*job);
+        const dim3 mgrid((n_expert + 1u + 2u * ffn + 7u) / 8u + (with_job ? 1u : 0u));
+        size_t lds = (size_t)ntok * hidden * 4u;
+        if (with_job && lds < kGroupLdsWords * 4u) lds = kGroupLdsWords * 4u;
+        const GroupJob gj = with_job ? *job : GroupJob{};
         // (64 KB of activations at 8 tokens of 2048, beside a few static bytes: the limit is raised explicitly)
 #define REDHIP_RMULTI(NV)                                                                                                                                  \
     do {                                                                                                                                                   \
@@ -555,7 +620,8 @@ hipError_t launch_router_gemv(uint32_t router_type, const void *w, const float *
             if (e != hipSuccess) return e;                                                                                                                  \
             attr = true;                                                                                                                                    \
         }                                                                                                                                                   \
-        REDHIP_LAUNCH((router_f32_multi_kernel<NV, 8>), mgrid, dim3(512), lds, s, wf, a, ntok);                                                             \
+        REDHIP_LAUNCH((router_f32_multi_kernel<NV, 8>), mgrid, dim3(512), lds, s, wf, a, ntok, gj);                                                         \
+        if (with_job) *job_done = true;                                                                                                                     \
         return hipGetLastError();                                                                                                                           \
     } while (0)
         switch (hidden / 256u) {
@@ -763,9 +829,15 @@ hipError_t launch_select(const float *logits, uint32_t ntok, uint32_t n_expert, 
 }
 
 // without a router (callers that bring their own routing): fp16 split of x and the scalar gate, one workgroup per token
-__global__ __launch_bounds__(256) void prep_kernel(const float *x, const float *gate_inp, uint32_t H, _Float16 *xh, _Float16 *xl, int *xexp, float *scalar) {
+__global__ __launch_bounds__(256) void prep_kernel(const float *x, const float *gate_inp, uint32_t H, _Float16 *xh, _Float16 *xl, int *xexp, float *scalar,
+                                                   uint32_t ntok, GroupJob job) {
     __shared__ float red[4];
+    __shared__ uint32_t group_lds[kGroupLdsWords];
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63u, tok = blockIdx.x;
+    if (tok == ntok) {                                   // the extra workgroup: pair sort of the caller's routing
+        group_small_given(job, group_lds);
+        return;
+    }
     const float *xt = x + (uint64_t)tok * H;
     float amax = 0.0f, acc = 0.0f;
     for (uint32_t i = threadIdx.x; i < H; i += 256u) { const float v = xt[i]; amax = fmaxf(amax, fabsf(v)); acc = fmaf(gate_inp[i], v, acc); }
@@ -784,8 +856,12 @@ __global__ __launch_bounds__(256) void prep_kernel(const float *x, const float *
     if (threadIdx.x == 0u) xexp[tok] = e;
 }
 
-hipError_t launch_prep(const float *x, const float *gate_inp, uint32_t ntok, uint32_t hidden, void *xh, void *xl, int *xexp, float *scalar, hipStream_t s) {
-    REDHIP_LAUNCH(prep_kernel, dim3(ntok), dim3(256), 0, s, x, gate_inp, hidden, static_cast<_Float16 *>(xh), static_cast<_Float16 *>(xl), xexp, scalar);
+hipError_t launch_prep(const float *x, const float *gate_inp, uint32_t ntok, uint32_t hidden, void *xh, void *xl, int *xexp, float *scalar, hipStream_t s,
+                       const GroupJob *job, bool *job_done) {
+    const bool with_job = job && job_done && group_job_fits(*job);
+    REDHIP_LAUNCH(prep_kernel, dim3(ntok + (with_job ? 1u : 0u)), dim3(256), 0, s, x, gate_inp, hidden, static_cast<_Float16 *>(xh), static_cast<_Float16 *>(xl), xexp,
+                  scalar, ntok, with_job ? *job : GroupJob{});
+    if (job_done) *job_done = with_job;
     return hipGetLastError();
 }
 
@@ -1618,20 +1694,14 @@ hipError_t launch_down_combine_words(uint32_t down_type, const int8_t *grid, con
 
 // ---------------------------------------------------------------- small batches (2..16 tokens): select + group, batched gate/up, batched down
 
-// One workgroup: wave t selects the experts of token t, then the (token, k) pairs are grouped by expert. Same
-// outputs as the host pair sort it replaces: groups in first-appearance order, pairs of a group in token order.
-// A table in LDS holds, per expert, the set of tokens that selected it (a token selects an expert at most once): the
-// position of a pair inside its group and the group's size are bit counts of that set, the order of the groups a
-// bit count over the "first pair of its expert" flags, the group offsets one prefix sum. At most 128 pairs.
+// One workgroup: wave t selects the experts of token t, then the (token, k) pairs are grouped by expert (group_small).
 __global__ __launch_bounds__(1024) void select_group_kernel(const float *logits, uint32_t ntok, uint32_t E, uint32_t K,
                                                             uint32_t *ids, float *weights, float *scalar, uint32_t *uid,
                                                             uint32_t *expert_start, uint32_t *pair_token, float *pair_weight,
                                                             uint32_t *tok_pair, uint32_t *n_unique) {
     __shared__ SelectOut sel[16];
-    __shared__ uint32_t token_set[1024];                 // per expert: bit t = token t selected it; later the group's offset
-    __shared__ uint32_t first_count[2], size_total[2];
+    __shared__ uint32_t group_lds[kGroupLdsWords];
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
-    if (tid < E) token_set[tid] = 0u;
     if (wave < ntok) {
         const float *l = logits + (uint64_t)wave * (E + 1u);
         if (E <= 512u) wave_select_topk<8>(l, E, K, &sel[wave]); else wave_select_topk<16>(l, E, K, &sel[wave]);
@@ -1640,38 +1710,8 @@ __global__ __launch_bounds__(1024) void select_group_kernel(const float *logits,
         if (lane == 0u) scalar[wave] = sel[wave].scalar;
     }
     __syncthreads();
-    const uint32_t P = ntok * K, pr = tid;               // pair index (waves 0 and 1)
-    const bool live = pr < P;
-    const uint32_t t = live ? pr / K : 0u;
-    const uint32_t e = live ? sel[t].ids[pr % K] : 0u;
-    if (live) atomicOr(&token_set[e], 1u << t);
-    __syncthreads();
-    const uint32_t set = live ? token_set[e] : 0u;
-    const uint32_t n = (uint32_t)__popc(set), before = (uint32_t)__popc(set & ((1u << t) - 1u));
-    const bool first = live && before == 0u;
-    uint32_t scan = first ? n : 0u;                      // inclusive prefix sum of the group sizes in pair order
-    if (wave < 2u) {
-#pragma unroll
-        for (int o = 1; o < 64; o <<= 1) {
-            const uint32_t up = __shfl_up(scan, o, 64);
-            if (lane >= (uint32_t)o) scan += up;
-        }
-        const uint64_t fm = __ballot(first);
-        if (lane == 63u) { first_count[wave] = (uint32_t)__popcll(fm); size_total[wave] = scan; }
-    }
-    const uint64_t first_mask = __ballot(first);
-    __syncthreads();
-    const uint32_t grp = (wave == 1u ? first_count[0] : 0u) + __builtin_amdgcn_mbcnt_hi((uint32_t)(first_mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)first_mask, 0u));
-    const uint32_t start = (wave == 1u ? size_total[0] : 0u) + scan - (first ? n : 0u);
-    if (first) { token_set[e] = start; uid[grp] = e; expert_start[grp] = start; }
-    if (tid == 0u) { const uint32_t U = first_count[0] + first_count[1]; expert_start[U] = P; n_unique[0] = U; }
-    __syncthreads();
-    if (live) {
-        const uint32_t pos = token_set[e] + before;
-        pair_token[pos] = t;
-        pair_weight[pos] = sel[t].w[pr % K];
-        tok_pair[pr] = pos;
-    }
+    const GroupJob g{nullptr, nullptr, ntok, K, E, uid, expert_start, pair_token, pair_weight, tok_pair, n_unique};
+    group_small(g, group_lds, [&](uint32_t t, uint32_t k) { return sel[t].ids[k]; }, [&](uint32_t t, uint32_t k) { return sel[t].w[k]; });
 }
 
 hipError_t launch_select_group(const float *logits, uint32_t ntok, uint32_t n_expert, uint32_t top_k, uint32_t *ids, float *weights,

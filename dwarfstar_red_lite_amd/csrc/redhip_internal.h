@@ -181,15 +181,30 @@ inline uint64_t packed_matrix_bytes(uint32_t type, uint32_t nrows, uint32_t K) {
 hipError_t launch_dequant_packed(uint32_t type, const void *packed, uint32_t nrows, uint32_t K, const int8_t *grid, float *out, hipStream_t s);
 hipError_t launch_dequant_packed_iq2xxs(const void *packed, uint32_t nrows, uint32_t K, bool col_major, float *out, hipStream_t s);
 
+// Pair sort of caller-given routing (at most 16 tokens, 128 pairs, 1024 experts) as a side job of another launch: one extra
+// workgroup groups ids / weights [ntok][top_k] by expert while the others do the launch's own work. Outputs as launch_group_pairs.
+struct GroupJob {
+    const uint32_t *ids;
+    const float *weights;
+    uint32_t ntok, top_k, n_expert;
+    uint32_t *uid, *expert_start, *pair_token;
+    float *pair_weight;
+    uint32_t *tok_pair, *n_unique;
+};
+
 // logits [ntok][n_expert + 1] (entry n_expert = gate_inp . x) and the fp16 split of x: xh, xl [ntok][hidden], xexp [ntok]
+// sh_dense: f32 [2 ffn][hidden] shared gate | up rows (F32 router, <= 8 tokens). job / job_done: the launch carries the pair sort
+// when its kernel can (*job_done says whether it did).
 hipError_t launch_router_gemv(uint32_t router_type, const void *w, const float *x, const float *gate_inp, uint32_t ntok, uint32_t hidden,
                               uint32_t n_expert, float *logits, void *xh, void *xl, int *xexp, const void *sh_q6k, float *sh_gu, uint32_t ffn,
-                              hipStream_t s, const float *sh_dense = nullptr, float *scalar_out = nullptr);      // sh_dense: f32 [2 ffn][hidden] shared gate | up rows (F32 router, <= 8 tokens)
+                              hipStream_t s, const float *sh_dense = nullptr, float *scalar_out = nullptr, const GroupJob *job = nullptr,
+                              bool *job_done = nullptr);
 // softmax top-k of logits [ntok][n_expert + 1]; scalar[t] = sigmoid(logits[t][n_expert]); optional probs [ntok][n_expert]
 hipError_t launch_select(const float *logits, uint32_t ntok, uint32_t n_expert, uint32_t top_k, uint32_t *ids, float *weights, float *scalar,
                          float *probs, hipStream_t s);
-// fp16 split of x and the scalar gate without a router
-hipError_t launch_prep(const float *x, const float *gate_inp, uint32_t ntok, uint32_t hidden, void *xh, void *xl, int *xexp, float *scalar, hipStream_t s);
+// fp16 split of x and the scalar gate without a router; with a job that fits, one more workgroup does the pair sort (*job_done)
+hipError_t launch_prep(const float *x, const float *gate_inp, uint32_t ntok, uint32_t hidden, void *xh, void *xl, int *xexp, float *scalar, hipStream_t s,
+                       const GroupJob *job = nullptr, bool *job_done = nullptr);
 
 // 2..16 tokens (at most 128 pairs): per-token selection and the pair sort in one launch
 hipError_t launch_select_group(const float *logits, uint32_t ntok, uint32_t n_expert, uint32_t top_k, uint32_t *ids, float *weights,

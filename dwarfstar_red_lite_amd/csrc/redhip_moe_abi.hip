@@ -114,10 +114,10 @@ struct Moe {
     // MFMA kernel, built-in down types on the batched raw-row kernel): every distinct expert is read once. Needs the router launch of the
     // same forward() for the shared expert's gate / up products.
     static constexpr uint32_t kGroupedMin = 3u;
-    bool grouped_mixed(uint32_t ntok) const {
+    bool grouped_mixed(uint32_t ntok, uint32_t from = kGroupedMin) const {
         const uint32_t rbd = (cfg.ffn / 256u) * block_bytes(dn_type), rbs = (cfg.ffn / 256u) * block_bytes(sh_dn_type);
         const bool words = (dn_type == T_IQ3_S || dn_type == T_IQ2_XS || dn_type == T_IQ1_M) && cfg.ffn <= 1024u;      // then the layers hold a packed down copy
-        return small_batch_mixed(ntok) && ntok >= kGroupedMin && (words || cfg.ffn <= 768u) &&
+        return small_batch_mixed(ntok) && ntok >= from && (words || cfg.ffn <= 768u) &&
                (words || (quant_supported(dn_type) && (8u * rbd) % 16u == 0u && (8u * rbs) % 16u == 0u && (2u * gate_bytes) % 16u == 0u && (2u * sh_gate_bytes) % 16u == 0u));
     }
     // a chunk on a layout whose experts are IQ2_XS / IQ1_M: the tile kernels on the row-major streams of the routed matrices, the shared
@@ -188,7 +188,7 @@ __global__ __launch_bounds__(256) void resid_rms_kernel(const float *x, const fl
 int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const uint32_t *ids, const float *weights,
                     float *out, hipStream_t s, bool select_here = false, bool grouped = false) {
     const redhip_moe_config &c = m->cfg;
-    if (m->grouped_mixed(ntok) && m->shared_gu_ready) {      // xh / xl / xexp / scalar and the shared gate | up products (m->act) come from the router launch
+    if (m->grouped_mixed(ntok, grouped ? 2u : Moe::kGroupedMin) && m->shared_gu_ready) {      // xh / xl / xexp / scalar and the shared gate | up products (m->act) come from the router launch
         const Layer &L = m->layers[layer];
         if (!grouped) {
             prof_set_stage(ST_GROUP);
@@ -649,18 +649,23 @@ int redhip_moe_experts(redhip_moe_t h, uint32_t layer, const float *x_dev, uint3
     if (m->packed_path(ntok) || m->small_batch_mixed(ntok) || m->mixed_chunk(ntok) || m->stream_chunk(ntok)) {
         const Layer &L = m->layers[layer];
         const uint32_t nv = m->cfg.hidden / 256u;
-        if (m->grouped_mixed(ntok) && L.dense_gu && (nv == 2u || nv == 4u || nv == 8u || nv == 16u)) {
+        // batches whose pairs are grouped by expert next: the pair sort rides in the same launch as one more workgroup
+        // (with the routing given, grouping pays from two tokens on: the pair sort costs no launch of its own)
+        const bool to_group = m->small_batch(ntok) || m->grouped_mixed(ntok, 2u);
+        const GroupJob job{ids_dev, weights_dev, ntok, m->cfg.top_k, m->cfg.n_expert, m->uid, m->expert_start, m->pair_token, m->pair_weight, m->tok_pair, m->n_unique};
+        bool grouped = false;
+        if (m->grouped_mixed(ntok, 2u) && L.dense_gu && (nv == 2u || nv == 4u || nv == 8u || nv == 16u)) {
             // the grouped kernels take the shared expert's gate | up products as an input: one f32 GEMV over its f32 copy (no router rows),
             // which also leaves the fp16 halves of x and the shared expert's scalar gate
             prof_set_stage(ST_SHARED_GATEUP);
             HIP_OK(launch_router_gemv(T_F32, L.dense_gu, x_dev, L.gate_inp, ntok, m->cfg.hidden, 0u, m->logits, m->xh, m->xl, m->xexp, nullptr, m->act,
-                                      m->cfg.ffn, s, L.dense_gu, m->scalar), "shared gate/up launch");
+                                      m->cfg.ffn, s, L.dense_gu, m->scalar, to_group ? &job : nullptr, &grouped), "shared gate/up launch");
             m->shared_gu_ready = true;
         } else {
             prof_set_stage(ST_OTHER);
-            HIP_OK(launch_prep(x_dev, L.gate_inp, ntok, m->cfg.hidden, m->xh, m->xl, m->xexp, m->scalar, s), "prep launch");
+            HIP_OK(launch_prep(x_dev, L.gate_inp, ntok, m->cfg.hidden, m->xh, m->xl, m->xexp, m->scalar, s, to_group ? &job : nullptr, &grouped), "prep launch");
         }
-        const int ok = experts_enqueue(m, layer, x_dev, ntok, ids_dev, weights_dev, out_dev, s);
+        const int ok = experts_enqueue(m, layer, x_dev, ntok, ids_dev, weights_dev, out_dev, s, false, grouped);
         m->shared_gu_ready = false;
         return ok;
     }

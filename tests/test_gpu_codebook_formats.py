@@ -254,8 +254,8 @@ def test_codebook_layout_chunks(layout, shape, ntok, grids):
 
 @pytest.mark.parametrize("layout", ["xs", "m"])
 def test_codebook_layout_given_routing(layout, grids):
-    """caller-given routing (drawn logits with hot experts, so tokens share experts) on IQ2_XS / IQ1_M layers: batches of 2 (single-token
-    kernels), 3 and 8 (grouped kernels) and a chunk of 40 tokens, against the oracle run token by token"""
+    """caller-given routing (drawn logits with hot experts, so tokens share experts) on IQ2_XS / IQ1_M layers: batches of 2, 3
+    and 8 (grouped kernels, the pair sort riding in the shared gate/up launch) and a chunk of 40 tokens, against the oracle run token by token"""
     from dwarfstar_red_lite_amd.moe import ResidentMoe
     from test_gpu_moe_batch import oracle_tokens
     orc.set_codebooks(*grids)
