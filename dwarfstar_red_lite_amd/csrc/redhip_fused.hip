@@ -11,8 +11,8 @@
 //   down_combine_kernel    8 output rows per workgroup, one wave per selected expert; weighted sum in selection
 //                          order + shared expert * scalar gate: deterministic (down_combine_raw_kernel when the down
 //                          matrices are raw IQ3_S / Q6_K rows)
-// Two to eight tokens: select_group_kernel (selection per token + pair sort), gateup_batch_kernel (persistent
-// workgroups, every distinct expert read once), down_batch_kernel.
+// Two to eight tokens: gateup_batch_kernel (every workgroup repeats the selection per token and the pair sort, then persistent
+// workgroups read every distinct expert once), down_batch_kernel.
 //
 // Arithmetic: a weight is (sign * magnitude * (2*scale+1)) * d/8; the eight magnitudes of a grid entry are exact fp16
 // values from an LDS table, the sign bits are placed by integer arithmetic; an activation vector is split into two
@@ -1694,35 +1694,6 @@ hipError_t launch_down_combine_words(uint32_t down_type, const int8_t *grid, con
 
 // ---------------------------------------------------------------- small batches (2..16 tokens): select + group, batched gate/up, batched down
 
-// One workgroup: wave t selects the experts of token t, then the (token, k) pairs are grouped by expert (group_small).
-__global__ __launch_bounds__(1024) void select_group_kernel(const float *logits, uint32_t ntok, uint32_t E, uint32_t K,
-                                                            uint32_t *ids, float *weights, float *scalar, uint32_t *uid,
-                                                            uint32_t *expert_start, uint32_t *pair_token, float *pair_weight,
-                                                            uint32_t *tok_pair, uint32_t *n_unique) {
-    __shared__ SelectOut sel[16];
-    __shared__ uint32_t group_lds[kGroupLdsWords];
-    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
-    if (wave < ntok) {
-        const float *l = logits + (uint64_t)wave * (E + 1u);
-        if (E <= 512u) wave_select_topk<8>(l, E, K, &sel[wave]); else wave_select_topk<16>(l, E, K, &sel[wave]);
-        wave_lds_sync();
-        if (lane < K) { ids[wave * K + lane] = sel[wave].ids[lane]; weights[wave * K + lane] = sel[wave].w[lane]; }
-        if (lane == 0u) scalar[wave] = sel[wave].scalar;
-    }
-    __syncthreads();
-    const GroupJob g{nullptr, nullptr, ntok, K, E, uid, expert_start, pair_token, pair_weight, tok_pair, n_unique};
-    group_small(g, group_lds, [&](uint32_t t, uint32_t k) { return sel[t].ids[k]; }, [&](uint32_t t, uint32_t k) { return sel[t].w[k]; });
-}
-
-hipError_t launch_select_group(const float *logits, uint32_t ntok, uint32_t n_expert, uint32_t top_k, uint32_t *ids, float *weights,
-                               float *scalar, uint32_t *uid, uint32_t *expert_start, uint32_t *pair_token, float *pair_weight,
-                               uint32_t *tok_pair, uint32_t *n_unique, hipStream_t s) {
-    if (!ntok || ntok > 16u || ntok * top_k > 128u || !n_expert || n_expert > 1024u || !top_k || top_k > 16u || top_k > n_expert) return hipErrorInvalidValue;
-    REDHIP_LAUNCH(select_group_kernel, dim3(1), dim3(1024), 0, s, logits, ntok, n_expert, top_k, ids, weights, scalar, uid, expert_start,
-                  pair_token, pair_weight, tok_pair, n_unique);
-    return hipGetLastError();
-}
-
 // 32 weights of one group against NTP activation operands, each carrying two tokens (rows 0,1 = hi,lo of the
 // first, rows 2,3 of the second): the table lookups are done once, the MFMAs once per token pair. The lookups are
 // a separate step so that a caller can have those of several groups in flight before it consumes the first.
@@ -1789,6 +1760,9 @@ struct BatchArgs {
     const float *resid_a, *resid_b;     // when set: out = (resid_a + resid_b) + layer output, [ntok][hidden] each
     const float *shared_gu;             // shared == nullptr: the shared expert's gate . x and up . x, [ntok][2 ffn] f32, already computed
     const int8_t *grid;                 // the caller's codebook when the gate / up matrices are IQ2_XS / IQ1_M streams
+    // selection inside the gate/up kernel: logits [ntok][n_expert + 1] from the router launch; the routing (ids, weights, scalar) and its
+    // grouping (uid .. n_unique above) are then outputs of the gate/up kernel, written identically by every workgroup
+    BatchSelect sel;
 };
 
 // Persistent workgroups walk the units (u, g) = (group of pairs, 32 FFN columns): 32 gate + 32 up rows of the
@@ -1809,10 +1783,30 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_batch_kernel(BatchArgs a) 
     __shared__ uint32_t meta_expert[kMaxUnits], meta_p0[kMaxUnits], meta_n[kMaxUnits];
     __shared__ uint8_t meta_tok[kMaxUnits][kMaxTok];
     __shared__ float tok_scale[kMaxTok];
+    __shared__ SelectOut sel[kMaxTok];
+    __shared__ uint32_t group_lds[kGroupLdsWords];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t H = a.hidden, F = a.ffn, HG = H / 32u, HB = H / 256u, FG = F / 32u, P = a.ntok * a.top_k;
     const uint64_t grid_entry = FMT == 0 && tid < 256u ? redhip_iq2xxs_grid[tid] : 0ull;
+    if (a.sel.logits) {
+        // Every workgroup selects and groups for itself (wave t the experts of token t), in place of a launch of its
+        // own, and writes the same routing and grouping to device memory: the barrier behind it makes the workgroup's own writes visible
+        // to its reads below, and another workgroup's writes carry the same values.
+        const uint32_t E = a.sel.n_expert, K = a.top_k;
+        if (wave < a.ntok) {
+            const float *l = a.sel.logits + (uint64_t)wave * (E + 1u);
+            if (E <= 512u) wave_select_topk<8>(l, E, K, &sel[wave]); else wave_select_topk<16>(l, E, K, &sel[wave]);
+            wave_lds_sync();
+            if (lane < K) { a.sel.ids[wave * K + lane] = sel[wave].ids[lane]; a.sel.weights[wave * K + lane] = sel[wave].w[lane]; }
+            if (lane == 0u) a.sel.scalar[wave] = sel[wave].scalar;
+        }
+        __syncthreads();
+        const GroupJob gj{nullptr, nullptr, a.ntok, K, E, const_cast<uint32_t *>(a.uid), const_cast<uint32_t *>(a.expert_start), const_cast<uint32_t *>(a.pair_token),
+                          const_cast<float *>(a.pair_weight), const_cast<uint32_t *>(a.tok_pair), const_cast<uint32_t *>(a.n_unique)};
+        group_small(gj, group_lds, [&](uint32_t t, uint32_t k) { return sel[t].ids[k]; }, [&](uint32_t t, uint32_t k) { return sel[t].w[k]; });
+        __syncthreads();
+    }
     const uint32_t U = a.n_unique[0], n_units = (U + 1u) * FG;
     uint32_t count = 0u;
     if (blockIdx.x < n_units) count = (n_units - blockIdx.x + gridDim.x - 1u) / gridDim.x;
@@ -2303,16 +2297,22 @@ __global__ __launch_bounds__(kWaves * 64) void down_batch_raw_kernel(DownBatchRa
 }
 
 static hipError_t launch_gateup_batch_kernel(const BatchArgs &a, uint32_t n_groups, hipStream_t s, uint32_t gate_up_type = T_IQ2_XXS);
+static bool batch_select_ok(const BatchSelect &b, uint32_t ntok, uint32_t top_k, uint32_t n_expert) {
+    return b.logits && b.ids && b.weights && b.scalar && b.n_expert == n_expert && n_expert <= 1024u && top_k <= 16u && top_k <= n_expert && ntok * top_k <= 128u;
+}
 
 hipError_t launch_batch_packed(const void *experts, uint64_t stride, const void *shared, const uint32_t *uid, const uint32_t *expert_start,
                                const uint32_t *pair_token, const uint32_t *n_unique, const float *pair_weight, const uint32_t *tok_pair,
                                const float *scalar, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l, int *act_exp,
-                               float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s) {
+                               float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s,
+                               const BatchSelect *select) {
     if (!fused_iq2_supported(hidden, ffn) || !ntok || ntok > (uint32_t)kMaxTok || ntok * top_k + ntok > 144u) return hipErrorInvalidValue;
     BatchArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(shared), uid, expert_start, pair_token, n_unique,
                 pair_weight, tok_pair, scalar, static_cast<const _Float16 *>(xh), static_cast<const _Float16 *>(xl), xexp,
                 static_cast<_Float16 *>(act_h), static_cast<_Float16 *>(act_l), act_exp, out, hidden, ffn, top_k, ntok,
-                block_context().resid_a, block_context().resid_b, nullptr, nullptr};
+                block_context().resid_a, block_context().resid_b, nullptr, nullptr, BatchSelect{}};
+    if (select && !batch_select_ok(*select, ntok, top_k, n_expert)) return hipErrorInvalidValue;
+    if (select) a.sel = *select;
     const uint32_t P = ntok * top_k, n_groups = (P < n_expert ? P : n_expert) + 1u;
     hipError_t e = launch_gateup_batch_kernel(a, n_groups, s);
     if (e != hipSuccess) return e;
@@ -2360,7 +2360,8 @@ hipError_t launch_batch_mixed(uint32_t gate_up_type, const int8_t *gate_up_grid,
                               const float *dense_down, const uint32_t *uid, const uint32_t *expert_start,
                               const uint32_t *pair_token, const uint32_t *n_unique, const float *pair_weight, const uint32_t *tok_pair,
                               const float *scalar, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l, int *act_exp,
-                              float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s) {
+                              float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s,
+                              const BatchSelect *select) {
     if (!fused_iq2_supported(hidden, ffn) || !ntok || ntok > (uint32_t)kMaxTok || ntok * top_k + ntok > 144u || !shared_gu) return hipErrorInvalidValue;
     const bool gu_codebook = gate_up_type == T_IQ2_XS || gate_up_type == T_IQ1_M, dn_codebook = down_type == T_IQ2_XS || down_type == T_IQ1_M;
     if ((gate_up_type != T_IQ2_XXS && !gu_codebook) || (gu_codebook && !gate_up_grid) || (dn_codebook && !down_grid)) return hipErrorInvalidValue;
@@ -2373,7 +2374,9 @@ hipError_t launch_batch_mixed(uint32_t gate_up_type, const int8_t *gate_up_grid,
     BatchArgs a{static_cast<const uint8_t *>(packed), packed_stride, nullptr, uid, expert_start, pair_token, n_unique,
                 pair_weight, tok_pair, scalar, static_cast<const _Float16 *>(xh), static_cast<const _Float16 *>(xl), xexp,
                 static_cast<_Float16 *>(act_h), static_cast<_Float16 *>(act_l), act_exp, out, hidden, ffn, top_k, ntok,
-                nullptr, nullptr, shared_gu, gate_up_grid};
+                nullptr, nullptr, shared_gu, gate_up_grid, BatchSelect{}};
+    if (select && !batch_select_ok(*select, ntok, top_k, n_expert)) return hipErrorInvalidValue;
+    if (select) a.sel = *select;
     const uint32_t P = ntok * top_k, n_groups = (P < n_expert ? P : n_expert) + 1u;
     hipError_t e = launch_gateup_batch_kernel(a, n_groups, s, gate_up_type);
     if (e != hipSuccess) return e;
@@ -2422,7 +2425,7 @@ static hipError_t launch_gateup_batch_kernel(const BatchArgs &a, uint32_t n_grou
     do {                                                                                                                  \
         static bool attr = false;                                                                                          \
         if (!attr) {                                                                                                       \
-            hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void *>(gateup_batch_kernel<NKC, NTP, FMT>), hipFuncAttributeMaxDynamicSharedMemorySize, (FMT == 2 ? 112 : 128) * 1024); \
+            hipError_t e1 = hipFuncSetAttribute(reinterpret_cast<const void *>(gateup_batch_kernel<NKC, NTP, FMT>), hipFuncAttributeMaxDynamicSharedMemorySize, (FMT == 2 ? 104 : 128) * 1024); \
             if (e1 != hipSuccess) return e1;                                                                               \
             attr = true;                                                                                                   \
         }                                                                                                                  \
@@ -2436,7 +2439,8 @@ static hipError_t launch_gateup_batch_kernel(const BatchArgs &a, uint32_t n_grou
         else if (ntok <= 8u) REDHIP_GUB_ONE(NKC, 1, 0);                                                                   \
         else REDHIP_GUB_ONE(NKC, 2, 0);                                                                                   \
     } while (0)
-    if (dyn_lds > (gate_up_type == T_IQ1_M ? 112u : 128u) * 1024u) return hipErrorInvalidValue;
+    // (beside the static tables: 51 KB with the IQ1_M codebook, 27 KB otherwise, of 160 KB per workgroup)
+    if (dyn_lds > (gate_up_type == T_IQ1_M ? 104u : 128u) * 1024u) return hipErrorInvalidValue;
     switch (hidden / 512u) {
         case 1: REDHIP_GUB(1); break;
         case 2: REDHIP_GUB(2); break;

@@ -192,6 +192,16 @@ struct GroupJob {
     uint32_t *tok_pair, *n_unique;
 };
 
+// Selection inside the batched gate/up kernel: logits [ntok][n_expert + 1] in, the routing out (ids, weights [ntok][top_k], scalar [ntok]);
+// the grouping arrays handed to the launcher are then outputs too.
+struct BatchSelect {
+    const float *logits;
+    uint32_t n_expert;
+    uint32_t *ids;
+    float *weights;
+    float *scalar;
+};
+
 // logits [ntok][n_expert + 1] (entry n_expert = gate_inp . x) and the fp16 split of x: xh, xl [ntok][hidden], xexp [ntok]
 // sh_dense: f32 [2 ffn][hidden] shared gate | up rows (F32 router, <= 8 tokens). job / job_done: the launch carries the pair sort
 // when its kernel can (*job_done says whether it did).
@@ -206,16 +216,13 @@ hipError_t launch_select(const float *logits, uint32_t ntok, uint32_t n_expert, 
 hipError_t launch_prep(const float *x, const float *gate_inp, uint32_t ntok, uint32_t hidden, void *xh, void *xl, int *xexp, float *scalar, hipStream_t s,
                        const GroupJob *job = nullptr, bool *job_done = nullptr);
 
-// 2..16 tokens (at most 128 pairs): per-token selection and the pair sort in one launch
-hipError_t launch_select_group(const float *logits, uint32_t ntok, uint32_t n_expert, uint32_t top_k, uint32_t *ids, float *weights,
-                               float *scalar, uint32_t *uid, uint32_t *expert_start, uint32_t *pair_token, float *pair_weight,
-                               uint32_t *tok_pair, uint32_t *n_unique, hipStream_t s);
 // batched gate/up + down/combine over grouped pairs, packed IQ2_XXS, small batches (ntok * (top_k + 1) <= 144).
 // act buffers hold ntok * (top_k + 1) rows (routed pairs, then one row per token for the shared expert).
 hipError_t launch_batch_packed(const void *experts, uint64_t stride, const void *shared, const uint32_t *uid, const uint32_t *expert_start,
                                const uint32_t *pair_token, const uint32_t *n_unique, const float *pair_weight, const uint32_t *tok_pair,
                                const float *scalar, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l, int *act_exp,
-                               float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s);
+                               float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s,
+                               const BatchSelect *select = nullptr);
 
 // single token: act[slot] = SwiGLU(gate . x, up . x) as fp16 halves with one exponent per 32 values. With `logits` the
 // kernel selects the experts itself (and writes ids / weights / scalar); with logits == nullptr it takes ids_in.
@@ -233,7 +240,8 @@ hipError_t launch_batch_mixed(uint32_t gate_up_type, const int8_t *gate_up_grid,
                               const float *dense_down, const uint32_t *uid, const uint32_t *expert_start,
                               const uint32_t *pair_token, const uint32_t *n_unique, const float *pair_weight, const uint32_t *tok_pair,
                               const float *scalar, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l, int *act_exp,
-                              float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s);
+                              float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s,
+                              const BatchSelect *select = nullptr);
 // IQ3_S down matrices of mixed layouts as one word per eight weights (uint4 per 32, [row][K/32], then d as fp16 [row][K/256])
 hipError_t launch_repack_iq3s_words(const void *raw, uint64_t raw_stride, uint32_t count, uint32_t nrows, uint32_t K, void *packed, uint64_t packed_stride, hipStream_t s);
 hipError_t launch_dequant_iq3s_words(const void *packed, uint32_t nrows, uint32_t K, float *out, hipStream_t s);

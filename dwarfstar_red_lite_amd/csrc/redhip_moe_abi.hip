@@ -91,7 +91,6 @@ struct Moe {
     }
     void *xh = nullptr, *xl = nullptr;       // fp16 [hidden] each
     int *xexp = nullptr;
-    bool select_and_group = false;           // forward() of a small batch: one launch selects and sorts the pairs
     bool skip_select = false;                // forward(): the gate/up kernel selects, route() skips its own selection
     bool shared_gu_ready = false;            // the router launch of this forward() has left the shared expert's gate / up products in `act`
     // batched path (ntok > 1): pairs grouped by expert
@@ -188,6 +187,9 @@ __global__ __launch_bounds__(256) void resid_rms_kernel(const float *x, const fl
 int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const uint32_t *ids, const float *weights,
                     float *out, hipStream_t s, bool select_here = false, bool grouped = false) {
     const redhip_moe_config &c = m->cfg;
+    // select_here && grouped: selection and pair sort both happen inside the batched gate/up kernel, from m->logits
+    const BatchSelect bsel{m->logits, c.n_expert, m->ids, m->weights, m->scalar};
+    const BatchSelect *in_batch = select_here && grouped ? &bsel : nullptr;
     if (m->grouped_mixed(ntok, grouped ? 2u : Moe::kGroupedMin) && m->shared_gu_ready) {      // xh / xl / xexp / scalar and the shared gate | up products (m->act) come from the router launch
         const Layer &L = m->layers[layer];
         if (!grouped) {
@@ -197,7 +199,7 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
         }
         HIP_OK(launch_batch_mixed(m->gu_type, m->gu_grid, L.packed, m->packed_stride, m->act, m->dn_type, m->dn_grid, m->sh_dn_type, L.experts + 2u * m->gate_bytes, m->expert_stride,
                                   L.shared + 2u * m->sh_gate_bytes, L.words_down, m->words_down_stride(), L.dense_down, m->uid, m->expert_start, m->pair_token, m->n_unique, m->pair_weight, m->tok_pair,
-                                  m->scalar, m->xh, m->xl, m->xexp, m->act_h, m->act_l, m->act_exp, out, c.hidden, c.ffn, c.top_k, ntok, c.n_expert, s),
+                                  m->scalar, m->xh, m->xl, m->xexp, m->act_h, m->act_l, m->act_exp, out, c.hidden, c.ffn, c.top_k, ntok, c.n_expert, s, in_batch),
                "grouped mixed batch launch");
         prof_set_stage(ST_OTHER);
         return 1;
@@ -214,7 +216,7 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
             const Layer &L = m->layers[layer];
             HIP_OK(launch_batch_packed(L.packed, m->expert_stride, L.shared_packed, m->uid, m->expert_start, m->pair_token, m->n_unique,
                                        m->pair_weight, m->tok_pair, m->scalar, m->xh, m->xl, m->xexp, m->act_h, m->act_l, m->act_exp, out,
-                                       c.hidden, c.ffn, c.top_k, ntok, c.n_expert, s), "batched packed launch");
+                                       c.hidden, c.ffn, c.top_k, ntok, c.n_expert, s, in_batch), "batched packed launch");
             prof_set_stage(ST_OTHER);
             return 1;
         }
@@ -614,11 +616,7 @@ int redhip_moe_route(redhip_moe_t h, uint32_t layer, const float *x_dev, uint32_
             HIP_OK(launch_router_gemv(c.router_type, m->layers[layer].router, x_dev, m->layers[layer].gate_inp, ntok, c.hidden, c.n_expert,
                                       m->logits, m->xh, m->xl, m->xexp, m->shared_gu_ready ? m->layers[layer].shared : nullptr, m->act, c.ffn, s),
                    "router launch");
-        if (m->select_and_group) {
-            prof_set_stage(ST_ROUTE_SELECT);
-            HIP_OK(launch_select_group(m->logits, ntok, c.n_expert, c.top_k, m->ids, m->weights, m->scalar, m->uid, m->expert_start,
-                                       m->pair_token, m->pair_weight, m->tok_pair, m->n_unique, s), "selection + grouping launch");
-        } else if (!m->skip_select) {
+        if (!m->skip_select) {
             prof_set_stage(ST_ROUTE_SELECT);
             HIP_OK(launch_select(m->logits, ntok, c.n_expert, c.top_k, ids_dev ? ids_dev : m->ids, weights_dev ? weights_dev : m->weights,
                                  m->scalar, nullptr, s), "selection launch");
@@ -690,13 +688,11 @@ int redhip_moe_forward(redhip_moe_t h, uint32_t layer, const float *x_dev, uint3
     }
     const bool group_in_select = m->small_batch(ntok) || m->grouped_mixed(ntok);
     const bool select_in_gateup = m->packed_gu() && (ntok == 1u || m->small_batch_mixed(ntok)) && !group_in_select;
-    m->skip_select = select_in_gateup;
-    m->select_and_group = group_in_select;
+    m->skip_select = select_in_gateup || group_in_select;      // small batches: the batched gate/up kernel selects and sorts the pairs itself
     const int routed = redhip_moe_route(h, layer, x_dev, ntok, nullptr, nullptr, nullptr, stream);
     m->skip_select = false;
-    m->select_and_group = false;
     if (!routed) return 0;
-    return experts_enqueue(m, layer, x_dev, ntok, m->ids, m->weights, out_dev, static_cast<hipStream_t>(stream), select_in_gateup, group_in_select);
+    return experts_enqueue(m, layer, x_dev, ntok, m->ids, m->weights, out_dev, static_cast<hipStream_t>(stream), select_in_gateup || group_in_select, group_in_select);
 }
 
 int redhip_moe_forward_block(redhip_moe_t h, uint32_t layer, const float *x_dev, const float *branch_dev, const float *post_norm_dev, float eps,
@@ -733,18 +729,16 @@ int redhip_moe_forward_block(redhip_moe_t h, uint32_t layer, const float *x_dev,
     if (ok) {
         const bool group_in_select = m->small_batch(ntok) || m->grouped_mixed(ntok);
         const bool select_in_gateup = m->packed_gu() && (ntok == 1u || m->small_batch_mixed(ntok)) && !group_in_select;
-        m->skip_select = select_in_gateup;
-        m->select_and_group = group_in_select;
+        m->skip_select = select_in_gateup || group_in_select;
         if (in_router) { bc.branch = branch_dev; bc.norm_w = post_norm_dev; bc.eps = eps; bc.xn_out = m->xn; }
         ok = redhip_moe_route(h, layer, in_router ? x_dev : m->xn, ntok, nullptr, nullptr, nullptr, stream);
         bc.branch = bc.norm_w = nullptr;
         bc.xn_out = nullptr;
         m->skip_select = false;
-        m->select_and_group = false;
-        if (ok) {
+            if (ok) {
             bc.resid_a = x_dev;                              // the path's last kernel adds x + branch to its output
             bc.resid_b = branch_dev;
-            ok = experts_enqueue(m, layer, m->xn, ntok, m->ids, m->weights, x_out_dev, s, select_in_gateup, group_in_select);
+            ok = experts_enqueue(m, layer, m->xn, ntok, m->ids, m->weights, x_out_dev, s, select_in_gateup || group_in_select, group_in_select);
         }
     }
     bc = BlockContext{};
