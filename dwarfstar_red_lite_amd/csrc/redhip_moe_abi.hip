@@ -97,6 +97,11 @@ struct Moe {
     uint32_t *uid = nullptr, *expert_start = nullptr, *pair_token = nullptr, *tok_pair = nullptr, *n_unique = nullptr;
     uint32_t *tile_group = nullptr, *tile_pair0 = nullptr, *tile_n = nullptr, *n_tiles = nullptr;      // prefill tiles
     float *pair_weight = nullptr, *tmp = nullptr, *sh_tmp = nullptr;
+    // chunks on mixed layouts: the shared expert's dense products (x -> sh_gu -> sh_act -> sh_tmp) run on a stream of their own beside
+    // the routed experts' tile kernels, which leave most of the machine's issue slots free; forked and joined with events
+    float *sh_gu = nullptr;                  // [max_tokens][2 ffn]
+    hipStream_t side = nullptr;
+    hipEvent_t ev_fork = nullptr, ev_join = nullptr;
     void *act_h = nullptr, *act_l = nullptr; // fp16 [top_k + 1][ffn] each
     int *act_exp = nullptr;                  // [top_k + 1][ffn / 32]
 
@@ -182,6 +187,25 @@ __global__ __launch_bounds__(256) void resid_rms_kernel(const float *x, const fl
     for (uint32_t i = threadIdx.x; i < hidden; i += 256u) xn[base + i] = ((x[base + i] + branch[base + i]) * inv) * w[i];
 }
 
+// The shared expert of a chunk on a mixed layout as dense f32 products (gate | up, SwiGLU, down) on the side stream: forked from s here,
+// joined by join_shared_dense before the combine. Reads x, writes sh_gu, sh_act, sh_tmp, which nothing on s touches in between.
+int fork_shared_dense(Moe *m, const Layer &L, const float *x, uint32_t ntok, hipStream_t s) {
+    const redhip_moe_config &c = m->cfg;
+    HIP_OK(hipEventRecord(m->ev_fork, s), "fork event");
+    HIP_OK(hipStreamWaitEvent(m->side, m->ev_fork, 0), "fork wait");
+    prof_set_stage(ST_BATCH_GATEUP);
+    HIP_OK(launch_f32_tiles(L.dense_gu, nullptr, x, ntok, c.hidden, 2u * c.ffn, m->sh_gu, 2u * c.ffn, nullptr, nullptr, nullptr, m->side), "shared gate/up tiles");
+    HIP_OK(launch_swiglu_rows(m->sh_gu, 2u * c.ffn, ntok, c.ffn, m->sh_act, m->side), "shared SwiGLU");
+    prof_set_stage(ST_BATCH_DOWN);
+    HIP_OK(launch_f32_tiles(L.dense_down, nullptr, m->sh_act, ntok, c.ffn, c.hidden, m->sh_tmp, c.hidden, nullptr, nullptr, nullptr, m->side), "shared down tiles");
+    HIP_OK(hipEventRecord(m->ev_join, m->side), "join event");
+    return 1;
+}
+int join_shared_dense(Moe *m, hipStream_t s) {
+    HIP_OK(hipStreamWaitEvent(s, m->ev_join, 0), "join wait");
+    return 1;
+}
+
 // select_here: the gate/up kernel selects the experts from m->logits itself (ids / weights are then outputs)
 // grouped: the pair sort of (ids, weights) is already in the workspace
 int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const uint32_t *ids, const float *weights,
@@ -207,6 +231,11 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
     if (ntok > 1u && !m->small_batch_mixed(ntok)) {       // group the (token, expert) pairs by expert, run each distinct expert once over its tokens
         const uint32_t P = ntok * c.top_k, n_groups = P < c.n_expert ? P : c.n_expert;
         const ExpertSet ex = m->routed(layer), sh = m->shared(layer);
+        const Layer &Ld = m->layers[layer];
+        const bool stream_tiles = m->stream_chunk(ntok) && Ld.words_down && Ld.dense_gu && m->side;
+        // the shared expert as dense f32 products on the fp32 matrix units, started before the pair sort (one workgroup on an idle machine)
+        const bool dense_shared = (stream_tiles || (m->mixed_chunk(ntok) && Ld.dense_gu && m->side));
+        if (dense_shared && !fork_shared_dense(m, Ld, x, ntok, s)) return 0;
         if (!grouped) {
             prof_set_stage(ST_GROUP);
             HIP_OK(launch_group_pairs(ids, weights, ntok, c.top_k, c.n_expert, m->uid, m->expert_start, m->pair_token, m->pair_weight,
@@ -230,17 +259,13 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
             prof_set_stage(ST_OTHER);
             return 1;
         }
-        if (m->stream_chunk(ntok) && m->layers[layer].words_down && m->layers[layer].dense_gu) {
-            const Layer &L = m->layers[layer];
-            float *gu = m->tmp;                          // [ntok][2 ffn]; free until the routed down kernel writes tmp (2 ffn <= top_k * hidden)
+        if (stream_tiles) {
+            const Layer &L = Ld;
             prof_set_stage(ST_BATCH_GATEUP);
-            HIP_OK(launch_f32_tiles(L.dense_gu, nullptr, x, ntok, c.hidden, 2u * c.ffn, gu, 2u * c.ffn, nullptr, nullptr, nullptr, s), "shared gate/up tiles");
-            HIP_OK(launch_swiglu_rows(gu, 2u * c.ffn, ntok, c.ffn, m->sh_act, s), "shared SwiGLU");
             HIP_OK(launch_prefill_streams(m->gu_type, m->gu_grid, L.packed, m->packed_stride, m->dn_type, m->dn_grid, L.words_down, m->words_down_stride(), m->uid,
                                           m->expert_start, m->pair_token, m->n_unique, m->tile_group, m->tile_pair0, m->tile_n, m->n_tiles, m->xh, m->xl, m->xexp,
                                           m->act_h, m->act_l, m->act_exp, m->tmp, c.hidden, c.ffn, c.top_k, ntok, c.n_expert, s), "stream tile launch");
-            prof_set_stage(ST_BATCH_DOWN);
-            HIP_OK(launch_f32_tiles(L.dense_down, nullptr, m->sh_act, ntok, c.ffn, c.hidden, m->sh_tmp, c.hidden, nullptr, nullptr, nullptr, s), "shared down tiles");
+            if (!join_shared_dense(m, s)) return 0;
             prof_set_stage(ST_BATCH_COMBINE);
             HIP_OK(launch_batch_combine(m->tmp, m->pair_weight, m->tok_pair, ntok, c.top_k, m->sh_tmp, m->scalar, c.hidden, out, s), "batched combine launch");
             prof_set_stage(ST_OTHER);
@@ -255,13 +280,7 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
         else
             HIP_OK(launch_batch_gateup(ex, m->uid, m->expert_start, m->pair_token, m->n_unique, n_groups, P, c.hidden, c.ffn, x, m->act, s), "batched gate/up launch");
         prof_set_stage(ST_BATCH_GATEUP);
-        const Layer &Ld = m->layers[layer];
-        const bool dense_shared = m->mixed_chunk(ntok) && Ld.dense_gu;      // the shared expert as two dense f32 products on the fp32 matrix units
-        if (dense_shared) {
-            float *gu = m->tmp;                          // [ntok][2 ffn]; free until the routed down kernel writes tmp (2 ffn <= top_k * hidden)
-            HIP_OK(launch_f32_tiles(Ld.dense_gu, nullptr, x, ntok, c.hidden, 2u * c.ffn, gu, 2u * c.ffn, nullptr, nullptr, nullptr, s), "shared gate/up tiles");
-            HIP_OK(launch_swiglu_rows(gu, 2u * c.ffn, ntok, c.ffn, m->sh_act, s), "shared SwiGLU");
-        } else {
+        if (!dense_shared) {
             HIP_OK(launch_batch_gateup(sh, nullptr, nullptr, nullptr, nullptr, 1u, ntok, c.hidden, c.ffn, x, m->sh_act, s), "batched shared gate/up launch");
         }
         prof_set_stage(ST_BATCH_DOWN);
@@ -271,9 +290,9 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
         else
             HIP_OK(launch_batch_down(ex, m->uid, m->expert_start, m->n_unique, n_groups, P, c.hidden, c.ffn, m->act, m->tmp, s), "batched down launch");
         prof_set_stage(ST_BATCH_DOWN);
-        if (dense_shared)
-            HIP_OK(launch_f32_tiles(Ld.dense_down, nullptr, m->sh_act, ntok, c.ffn, c.hidden, m->sh_tmp, c.hidden, nullptr, nullptr, nullptr, s), "shared down tiles");
-        else
+        if (dense_shared) {
+            if (!join_shared_dense(m, s)) return 0;
+        } else
             HIP_OK(launch_batch_down(sh, nullptr, nullptr, nullptr, 1u, ntok, c.hidden, c.ffn, m->sh_act, m->sh_tmp, s), "batched shared down launch");
         prof_set_stage(ST_BATCH_COMBINE);
         HIP_OK(launch_batch_combine(m->tmp, m->pair_weight, m->tok_pair, ntok, c.top_k, m->sh_tmp, m->scalar, c.hidden, out, s), "batched combine launch");
@@ -411,6 +430,7 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
                             align256(T * c.top_k * c.ffn * 4u) + align256(T * c.ffn * 4u) +
                             2u * align256(2u * T * c.hidden) + align256(4u * T) + 2u * align256(2u * T * (c.top_k + 1u) * c.ffn) +
                             align256(4u * T * (c.top_k + 1u) * (c.ffn / 32u)) +
+                            (T > 8u && m->mixed ? align256(8u * T * c.ffn) : 0u) +
                             (T > 1u ? 6u * align256(4u * (T * c.top_k + 2u)) + align256(4u * T * c.top_k * c.hidden) + align256(4u * T * c.hidden) +
                                           4u * align256(4u * (size_t)prefill_tile_bound(c.max_tokens, c.top_k, c.n_expert)) : 0u);
     ok = ok && hipMalloc(reinterpret_cast<void **>(&m->ws), ws_bytes) == hipSuccess;
@@ -433,6 +453,15 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
     m->act_h = w; w += align256(2u * T * (c.top_k + 1u) * c.ffn);
     m->act_l = w; w += align256(2u * T * (c.top_k + 1u) * c.ffn);
     m->act_exp = reinterpret_cast<int *>(w); w += align256(4u * T * (c.top_k + 1u) * (c.ffn / 32u));
+    if (T > 8u && m->mixed) {
+        m->sh_gu = reinterpret_cast<float *>(w); w += align256(8u * T * c.ffn);
+        if (hipStreamCreateWithFlags(&m->side, hipStreamNonBlocking) != hipSuccess || hipEventCreateWithFlags(&m->ev_fork, hipEventDisableTiming) != hipSuccess ||
+            hipEventCreateWithFlags(&m->ev_join, hipEventDisableTiming) != hipSuccess) {
+            moe_err("failed to create the side stream of the shared expert");
+            redhip_moe_destroy(m);
+            return nullptr;
+        }
+    }
     if (T > 1u) {
         const size_t pw = align256(4u * (T * c.top_k + 2u));
         m->uid = reinterpret_cast<uint32_t *>(w); w += pw;
@@ -474,6 +503,9 @@ void redhip_moe_destroy(redhip_moe_t h) {
         if (L.words_down) (void)hipFree(L.words_down);
         if (L.shared_tiled) (void)hipFree(L.shared_tiled);
     }
+    if (m->ev_fork) (void)hipEventDestroy(m->ev_fork);
+    if (m->ev_join) (void)hipEventDestroy(m->ev_join);
+    if (m->side) (void)hipStreamDestroy(m->side);
     if (m->ws) (void)hipFree(m->ws);
     if (m->stage) (void)hipFree(m->stage);
     delete m;

@@ -14,6 +14,8 @@
  * (thread-local), abi_version() == 1, handles made and destroyed by the caller, destroy(NULL) is a no-op.
  * `*_dev` arguments are device pointers; `stream` is a hipStream_t (NULL = the default stream). Calls that
  * take a stream only enqueue work. One forward at a time per handle: the handle owns the workspace.
+ * Chunks (more than 8 tokens) on mixed-precision layouts run part of their work on a second stream that the
+ * handle owns, forked from `stream` and joined to it again with events inside the same call (capturable).
  */
 #pragma once
 #include <stdint.h>

@@ -275,3 +275,56 @@ def test_codebook_layout_given_routing(layout, grids):
         for t in range(ntok):
             assert rel_l2(got[t], want[t]) <= REL_L2_TOL, (layout, ntok, t)
     m.close()
+
+
+@pytest.mark.parametrize("layout", ["f2", "xs"])
+def test_chunk_in_a_graph_with_the_shared_expert_on_its_own_stream(layout, grids):
+    """A chunk on a mixed layout forks the shared expert's dense products onto a second stream and joins them before the combine.
+    Captured into a HIP graph (two layers, so that a fork follows a join) and replayed with new inputs, eager work and
+    synchronisations in between: every replay must equal the eager result bit for bit, and the eager result the oracle."""
+    from dwarfstar_red_lite_amd.moe import ResidentMoe
+    orc.set_codebooks(*grids)
+    cfg = synth.layer_config(hidden=1024, ffn=512, n_expert=32, top_k=6, layout=layout)
+    lays = [synth.make_layer(900 + i, cfg) for i in range(2)]
+    ntok = 40
+    m = ResidentMoe(cfg, n_layer=2, max_tokens=ntok)
+    for i, lay in enumerate(lays):
+        m.load_layer(i, lay)
+    rng = np.random.default_rng(5)
+    xs = [synth.normed_x(rng, ntok, cfg["hidden"]) for _ in range(3)]
+    x_dev = torch.empty((ntok, cfg["hidden"]), dtype=torch.float32, device="cuda")
+    mid = torch.empty_like(x_dev)
+    out = torch.empty_like(x_dev)
+
+    def two_layers():
+        m.forward(0, x_dev, out=mid)
+        m.forward(1, mid, out=out)
+
+    eager = []
+    for x in xs:
+        x_dev.copy_(torch.from_numpy(x))
+        two_layers()
+        torch.cuda.synchronize()
+        eager.append((mid.clone(), out.clone()))
+    want0, *_ = orc.Layer(cfg, **lays[0]).forward(xs[0], threads=8)
+    for t in range(ntok):
+        assert rel_l2(eager[0][0][t].cpu().numpy(), want0[t]) <= REL_L2_TOL, (layout, t)
+    stream = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    stream.wait_stream(torch.cuda.current_stream())
+    with torch.cuda.stream(stream):
+        two_layers()                                # warm-up on the capture stream
+    torch.cuda.synchronize()
+    with torch.cuda.graph(graph, stream=stream):
+        two_layers()
+    for rnd in range(2):
+        for x, (e_mid, e_out) in zip(xs, eager):
+            x_dev.copy_(torch.from_numpy(x))
+            torch.cuda.synchronize()
+            graph.replay()
+            torch.cuda.synchronize()
+            assert torch.equal(mid, e_mid) and torch.equal(out, e_out), (layout, rnd)
+            two_layers()                            # the program's own eager work between replays
+            torch.cuda.synchronize()
+            assert torch.equal(out, e_out), (layout, rnd)
+    m.close()

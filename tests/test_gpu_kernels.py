@@ -118,9 +118,9 @@ def test_router_select_random_and_ties():
 def test_grouping_matches_host_sort():
     from dwarfstar_red_lite_amd import moe
     cfg = synth.layer_config(hidden=256, ffn=256, n_expert=512, top_k=10)
-    m = moe.ResidentMoe(cfg, n_layer=1, max_tokens=512)
+    m = moe.ResidentMoe(cfg, n_layer=1, max_tokens=1600)
     rng = np.random.default_rng(12)
-    for ntok in (1, 2, 3, 8, 33, 512):
+    for ntok in (1, 2, 3, 8, 33, 512, 1600):
         l = synth.hot_logits(rng, ntok, 512)
         sel = [orc.router_select(l[t], 10) for t in range(ntok)]
         ids = np.stack([s[0] for s in sel])

@@ -182,3 +182,4 @@ def test_chunk_as_slices_of_small_batches():
     for i in range(20):
         assert rel_l2(out[i], want[i]) <= REL_L2_TOL, i
     m.close()
+
