@@ -215,7 +215,7 @@ def main():
         torch.cuda.synchronize()
         t1 = time.perf_counter()
         eager_ms_per_step = (t1 - t0) * 1e3 / K
-    ms_per_step, launch_mode = eager_ms_per_step, "eager"
+    ms_per_step, launch_mode, graph_ms_per_step = eager_ms_per_step, "eager", None
     if not args.no_graph:
         # the same K steps recorded once into a HIP graph (kernel launches only, no memset nodes) and replayed: this
         # is how a decode loop would issue them; the replay is checked against the eager outputs before it is timed
@@ -236,7 +236,10 @@ def main():
             graph.replay()
             torch.cuda.synchronize()
             t1 = time.perf_counter()
-            ms_per_step, launch_mode = (t1 - t0) * 1e3 / K, "hip_graph"
+            graph_ms_per_step = (t1 - t0) * 1e3 / K
+            # (chunks that fork work onto a second stream replay a little slower than they launch: the quicker mode is the one reported)
+            if graph_ms_per_step <= eager_ms_per_step:
+                ms_per_step, launch_mode = graph_ms_per_step, "hip_graph"
     with torch.cuda.stream(stream):
 
         # the same K steps again with per-kernel begin/end timestamps (HIP events on the launch stream)
@@ -320,7 +323,8 @@ def main():
     result = {
         "metric": "moe_ffn_layer_us_per_token", "value": round(us_per_token, 3), "unit": "us/token", "n_gpus": 1,
         "steps": K, "warmup": W, "ms_per_step": round(ms_per_step, 6), "launch_mode": launch_mode,
-        "eager_ms_per_step": round(eager_ms_per_step, 6), "higher_is_better": False, "scaling": "weak",
+        "eager_ms_per_step": round(eager_ms_per_step, 6),
+        "graph_ms_per_step": None if graph_ms_per_step is None else round(graph_ms_per_step, 6), "higher_is_better": False, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "%s: one MoE FFN layer, B=%d decode token(s), hidden 2048, 512 experts top-10 + shared, ffn 512, layout %s, "
                                "all experts of %d layers resident" % ({"iq2": "config1", "f2": "config2"}.get(args.layout, "target-file expert format"),
