@@ -1789,6 +1789,26 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_batch_kernel(BatchArgs a) 
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t H = a.hidden, F = a.ffn, HG = H / 32u, HB = H / 256u, FG = F / 32u, P = a.ntok * a.top_k;
     const uint64_t grid_entry = FMT == 0 && tid < 256u ? redhip_iq2xxs_grid[tid] : 0ull;
+    // x operand in LDS as [piece s of 8 bytes][plane][group], plane = 2 * token + (hi, lo) and one more plane of
+    // zeros for lanes without a token: the 64 lanes of a wave read the same piece of consecutive groups, and the
+    // plane stride of HG + 8 keeps the hi and lo planes on different banks
+    const uint32_t PLS = HG + 8u, ZP = 2u * a.ntok, SS = (ZP + 1u) * PLS;
+    uint2 *xs = reinterpret_cast<uint2 *>(dyn);
+    // staged by the threads from `first` on (the waves below it select meanwhile, when the kernel selects)
+    auto stage_x = [&](uint32_t first) {
+        const uint32_t st = tid - first, nst = NW * 64u - first;
+        if (st < a.ntok) tok_scale[st] = (FMT == 2 ? 1.0f : 0.125f) * exp2i(a.xexp[st]);
+        for (uint32_t i = st; i < a.ntok * H / 8u; i += nst) {
+            const uint32_t t = i / (H / 8u), c = i % (H / 8u), at = (2u * (c & 3u)) * SS + 2u * t * PLS + (c >> 2);
+            const uint4 vh = reinterpret_cast<const uint4 *>(a.xh)[i], vl = reinterpret_cast<const uint4 *>(a.xl)[i];
+            xs[at] = make_uint2(vh.x, vh.y);
+            xs[at + SS] = make_uint2(vh.z, vh.w);
+            xs[at + PLS] = make_uint2(vl.x, vl.y);
+            xs[at + PLS + SS] = make_uint2(vl.z, vl.w);
+        }
+        for (uint32_t i = st; i < 8u * PLS; i += nst) xs[(i / PLS) * SS + ZP * PLS + i % PLS] = make_uint2(0u, 0u);
+        if constexpr (FMT != 0) build_codebook_table<FMT>(lds, tid, a.grid, first, nst);
+    };
     if (a.sel.logits) {
         // Every workgroup selects and groups for itself (wave t the experts of token t), in place of a launch of its
         // own, and writes the same routing and grouping to device memory: the barrier behind it makes the workgroup's own writes visible
@@ -1800,6 +1820,8 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_batch_kernel(BatchArgs a) 
             wave_lds_sync();
             if (lane < K) { a.sel.ids[wave * K + lane] = sel[wave].ids[lane]; a.sel.weights[wave * K + lane] = sel[wave].w[lane]; }
             if (lane == 0u) a.sel.scalar[wave] = sel[wave].scalar;
+        } else {
+            stage_x(a.ntok * 64u);
         }
         __syncthreads();
         const GroupJob gj{nullptr, nullptr, a.ntok, K, E, const_cast<uint32_t *>(a.uid), const_cast<uint32_t *>(a.expert_start), const_cast<uint32_t *>(a.pair_token),
@@ -1812,11 +1834,6 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_batch_kernel(BatchArgs a) 
     if (blockIdx.x < n_units) count = (n_units - blockIdx.x + gridDim.x - 1u) / gridDim.x;
     if (count > (uint32_t)kMaxUnits) count = kMaxUnits;
     if (count == 0u) return;
-    // x operand in LDS as [piece s of 8 bytes][plane][group], plane = 2 * token + (hi, lo) and one more plane of
-    // zeros for lanes without a token: the 64 lanes of a wave read the same piece of consecutive groups, and the
-    // plane stride of HG + 8 keeps the hi and lo planes on different banks
-    const uint32_t PLS = HG + 8u, ZP = 2u * a.ntok, SS = (ZP + 1u) * PLS;
-    uint2 *xs = reinterpret_cast<uint2 *>(dyn);
     if (tid < count) {
         const uint32_t u = (blockIdx.x + tid * gridDim.x) / FG;
         const bool sh = u == U;
@@ -1826,18 +1843,8 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_batch_kernel(BatchArgs a) 
         meta_n[tid] = sh && !a.shared ? 0u : p1 - p0;      // a shared expert that is not packed has no passes: its products are an input
         for (uint32_t i = 0; i < p1 - p0 && i < (uint32_t)kMaxTok; ++i) meta_tok[tid][i] = (uint8_t)(sh ? i : a.pair_token[p0 + i]);
     }
-    if (tid >= 64u && tid < 64u + a.ntok) tok_scale[tid - 64u] = (FMT == 2 ? 1.0f : 0.125f) * exp2i(a.xexp[tid - 64u]);
-    for (uint32_t i = tid; i < a.ntok * H / 8u; i += NW * 64u) {
-        const uint32_t t = i / (H / 8u), c = i % (H / 8u), at = (2u * (c & 3u)) * SS + 2u * t * PLS + (c >> 2);
-        const uint4 vh = reinterpret_cast<const uint4 *>(a.xh)[i], vl = reinterpret_cast<const uint4 *>(a.xl)[i];
-        xs[at] = make_uint2(vh.x, vh.y);
-        xs[at + SS] = make_uint2(vh.z, vh.w);
-        xs[at + PLS] = make_uint2(vl.x, vl.y);
-        xs[at + PLS + SS] = make_uint2(vl.z, vl.w);
-    }
-    for (uint32_t i = tid; i < 8u * PLS; i += NW * 64u) xs[(i / PLS) * SS + ZP * PLS + i % PLS] = make_uint2(0u, 0u);
+    if (!a.sel.logits) stage_x(0u);
     if constexpr (FMT == 0) build_tables(lds, tid, grid_entry);
-    else build_codebook_table<FMT>(lds, tid, a.grid, 0u, NW * 64u);
     __syncthreads();
 
     const uint64_t qs_bytes = (uint64_t)F * HG * 8u, sc_off = qs_bytes + (uint64_t)F * HB * 2u, gate_bytes = sc_off + (FMT == 1 ? (uint64_t)F * HG : 0u);
