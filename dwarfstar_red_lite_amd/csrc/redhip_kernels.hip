@@ -670,8 +670,12 @@ __device__ __forceinline__ uint32_t block_scan_1024(uint32_t v, uint32_t *wave_t
 // One workgroup. For every (token, k) pair p = t * top_k + k:
 //   first[e]   = smallest p that names expert e            -> experts numbered in first-appearance order
 //   member[e]  = bitmap over tokens that selected e        -> rank of a pair inside its expert = popcount below t
-// which gives the stable counting sort of the host loop it replaces without a serial pass.
-__global__ __launch_bounds__(1024) void group_pairs_kernel(const uint32_t *ids, const float *weights, uint32_t ntok, uint32_t top_k,
+// which gives the stable counting sort of the host loop it replaces without a serial pass. All of it runs on one
+// compute unit, so the instruction count is what it costs: the token of a pair comes from a multiply-high by
+// ceil(2^32 / top_k) (exact while pairs * top_k < 2^32), and with PREFIX the bit counts of the words below a token's word come
+// from a table made once per expert (which also yields the expert's pair count) instead of a loop per pair.
+template <bool PREFIX>
+__global__ __launch_bounds__(1024) void group_pairs_kernel(const uint32_t *ids, const float *weights, uint32_t ntok, uint32_t top_k, uint32_t top_k_magic,
                                                            uint32_t n_expert, uint32_t *uid, uint32_t *expert_start,
                                                            uint32_t *pair_token, float *pair_weight, uint32_t *tok_pair,
                                                            uint32_t *n_unique) {
@@ -684,16 +688,25 @@ __global__ __launch_bounds__(1024) void group_pairs_kernel(const uint32_t *ids, 
     uint32_t *uid_l = start + n_expert + 1u;       // [1024] experts by dense index (n_expert <= 1024)
     uint32_t *wave_tot = uid_l + 1024u;            // [17]
     uint32_t *member = wave_tot + 17u;             // [n_expert][words]
+    uint32_t *below = member + n_expert * words;   // [n_expert][words] when PREFIX: members in the words before this one
+    auto token_of = [&](uint32_t p) { return top_k == 1u ? p : __umulhi(p, top_k_magic); };
     for (uint32_t i = tid; i < n_expert; i += 1024u) { first[i] = 0xffffffffu; count[i] = 0u; dense[i] = 0u; }
     for (uint32_t i = tid; i < n_expert * words; i += 1024u) member[i] = 0u;
     __syncthreads();
     for (uint32_t p = tid; p < P; p += 1024u) {
-        const uint32_t e = ids[p], t = p / top_k;
+        const uint32_t e = ids[p], t = token_of(p);
         atomicMin(&first[e], p);
-        atomicAdd(&count[e], 1u);
+        if constexpr (!PREFIX) atomicAdd(&count[e], 1u);
         atomicOr(&member[e * words + (t >> 5)], 1u << (t & 31u));
     }
     __syncthreads();
+    if constexpr (PREFIX) {
+        for (uint32_t e = tid; e < n_expert; e += 1024u) {
+            uint32_t run = 0u;
+            for (uint32_t w = 0; w < words; ++w) { below[e * words + w] = run; run += __popc(member[e * words + w]); }
+            count[e] = run;
+        }
+    }
     // exclusive scan of "pair p is the first appearance of its expert", P elements in per-thread runs
     const uint32_t per = (P + 1023u) / 1024u;
     uint32_t mine = 0u;
@@ -712,10 +725,11 @@ __global__ __launch_bounds__(1024) void group_pairs_kernel(const uint32_t *ids, 
     if (tid == 0u) { start[U] = all; expert_start[U] = all; n_unique[0] = U; }
     __syncthreads();
     for (uint32_t p = tid; p < P; p += 1024u) {
-        const uint32_t e = ids[p], t = p / top_k;
+        const uint32_t e = ids[p], t = token_of(p);
         const uint32_t *bits = member + e * words;
         uint32_t rank = __popc(bits[t >> 5] & ((1u << (t & 31u)) - 1u));
-        for (uint32_t w = 0; w < (t >> 5); ++w) rank += __popc(bits[w]);
+        if constexpr (PREFIX) rank += below[e * words + (t >> 5)];
+        else for (uint32_t w = 0; w < (t >> 5); ++w) rank += __popc(bits[w]);
         const uint32_t pos = start[dense[e]] + rank;
         pair_token[pos] = t;
         pair_weight[pos] = weights[p];
@@ -726,17 +740,23 @@ __global__ __launch_bounds__(1024) void group_pairs_kernel(const uint32_t *ids, 
 hipError_t launch_group_pairs(const uint32_t *ids, const float *weights, uint32_t ntok, uint32_t top_k, uint32_t n_expert,
                               uint32_t *uid, uint32_t *expert_start, uint32_t *pair_token, float *pair_weight,
                               uint32_t *tok_pair, uint32_t *n_unique, hipStream_t s) {
-    if (!ntok || !top_k || !n_expert || n_expert > 1024u) return hipErrorInvalidValue;
+    if (!ntok || !top_k || !n_expert || n_expert > 1024u || (uint64_t)ntok * top_k * top_k >= (1ull << 32)) return hipErrorInvalidValue;
     const uint32_t words = (ntok + 31u) / 32u;
     const size_t lds = sizeof(uint32_t) * ((size_t)4u * n_expert + 1u + 1024u + 17u + (size_t)n_expert * words);
     if (lds > 160u * 1024u) return hipErrorInvalidValue;
+    const size_t lds_prefix = lds + sizeof(uint32_t) * (size_t)n_expert * words;
+    const uint32_t magic = (uint32_t)(((1ull << 32) + top_k - 1u) / top_k);      // top_k == 1 needs none (and would not fit)
     static bool attr_set = false;
     if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(group_pairs_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(group_pairs_kernel<false>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void *>(group_pairs_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
         if (e != hipSuccess) return e;
         attr_set = true;
     }
-    REDHIP_LAUNCH(group_pairs_kernel, dim3(1), dim3(1024), lds, s, ids, weights, ntok, top_k, n_expert, uid, expert_start, pair_token, pair_weight, tok_pair, n_unique);
+    if (lds_prefix <= 160u * 1024u)
+        REDHIP_LAUNCH(group_pairs_kernel<true>, dim3(1), dim3(1024), lds_prefix, s, ids, weights, ntok, top_k, magic, n_expert, uid, expert_start, pair_token, pair_weight, tok_pair, n_unique);
+    else
+        REDHIP_LAUNCH(group_pairs_kernel<false>, dim3(1), dim3(1024), lds, s, ids, weights, ntok, top_k, magic, n_expert, uid, expert_start, pair_token, pair_weight, tok_pair, n_unique);
     return hipGetLastError();
 }
 
