@@ -828,10 +828,13 @@ hipError_t launch_select(const float *logits, uint32_t ntok, uint32_t n_expert, 
     return hipGetLastError();
 }
 
-// without a router (callers that bring their own routing): fp16 split of x and the scalar gate, one workgroup per token
+// without a router (callers that bring their own routing): fp16 split of x and the scalar gate, one workgroup per token.
+// NV > 0: hidden = 256 * NV and a thread keeps its NV activations in registers, so x is read once and the two block-wide
+// reductions (largest |x|, gate_inp . x) share one barrier; NV == 0: any hidden, x read twice.
+template <int NV>
 __global__ __launch_bounds__(256) void prep_kernel(const float *x, const float *gate_inp, uint32_t H, _Float16 *xh, _Float16 *xl, int *xexp, float *scalar,
                                                    uint32_t ntok, GroupJob job) {
-    __shared__ float red[4];
+    __shared__ float red[8];
     __shared__ uint32_t group_lds[kGroupLdsWords];
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63u, tok = blockIdx.x;
     if (tok == ntok) {                                   // the extra workgroup: pair sort of the caller's routing
@@ -840,27 +843,46 @@ __global__ __launch_bounds__(256) void prep_kernel(const float *x, const float *
     }
     const float *xt = x + (uint64_t)tok * H;
     float amax = 0.0f, acc = 0.0f;
-    for (uint32_t i = threadIdx.x; i < H; i += 256u) { const float v = xt[i]; amax = fmaxf(amax, fabsf(v)); acc = fmaf(gate_inp[i], v, acc); }
+    float xv[NV > 0 ? NV : 1];
+    if constexpr (NV > 0) {
+        float gv[NV];
+#pragma unroll
+        for (int k = 0; k < NV; ++k) { xv[k] = xt[threadIdx.x + 256u * k]; gv[k] = gate_inp[threadIdx.x + 256u * k]; }
+#pragma unroll
+        for (int k = 0; k < NV; ++k) { amax = fmaxf(amax, fabsf(xv[k])); acc = fmaf(gv[k], xv[k], acc); }
+    } else {
+        for (uint32_t i = threadIdx.x; i < H; i += 256u) { const float v = xt[i]; amax = fmaxf(amax, fabsf(v)); acc = fmaf(gate_inp[i], v, acc); }
+    }
     amax = wave_max(amax);
     acc = wave_sum(acc);
-    if (lane == 0u) red[wave] = amax;
+    if (lane == 0u) { red[wave] = amax; red[4u + wave] = acc; }
     __syncthreads();
     amax = fmaxf(fmaxf(red[0], red[1]), fmaxf(red[2], red[3]));
-    __syncthreads();
-    if (lane == 0u) red[wave] = acc;
-    __syncthreads();
-    if (threadIdx.x == 0u) scalar[tok] = 1.0f / (1.0f + expf(-((red[0] + red[1]) + (red[2] + red[3]))));
+    if (threadIdx.x == 0u) scalar[tok] = 1.0f / (1.0f + expf(-((red[4] + red[5]) + (red[6] + red[7]))));
     const int e = prescale_exp(amax);
     const float inv = exp2i(-e);
-    for (uint32_t i = threadIdx.x; i < H; i += 256u) split_hi_lo(xt[i], inv, xh + (uint64_t)tok * H + i, xl + (uint64_t)tok * H + i);
+    if constexpr (NV > 0) {
+#pragma unroll
+        for (int k = 0; k < NV; ++k) split_hi_lo(xv[k], inv, xh + (uint64_t)tok * H + threadIdx.x + 256u * k, xl + (uint64_t)tok * H + threadIdx.x + 256u * k);
+    } else {
+        for (uint32_t i = threadIdx.x; i < H; i += 256u) split_hi_lo(xt[i], inv, xh + (uint64_t)tok * H + i, xl + (uint64_t)tok * H + i);
+    }
     if (threadIdx.x == 0u) xexp[tok] = e;
 }
 
 hipError_t launch_prep(const float *x, const float *gate_inp, uint32_t ntok, uint32_t hidden, void *xh, void *xl, int *xexp, float *scalar, hipStream_t s,
                        const GroupJob *job, bool *job_done) {
     const bool with_job = job && job_done && group_job_fits(*job);
-    REDHIP_LAUNCH(prep_kernel, dim3(ntok + (with_job ? 1u : 0u)), dim3(256), 0, s, x, gate_inp, hidden, static_cast<_Float16 *>(xh), static_cast<_Float16 *>(xl), xexp,
-                  scalar, ntok, with_job ? *job : GroupJob{});
+    const dim3 grid(ntok + (with_job ? 1u : 0u));
+    const GroupJob gj = with_job ? *job : GroupJob{};
+    _Float16 *h = static_cast<_Float16 *>(xh), *l = static_cast<_Float16 *>(xl);
+    switch (hidden) {
+        case 512: REDHIP_LAUNCH(prep_kernel<2>, grid, dim3(256), 0, s, x, gate_inp, hidden, h, l, xexp, scalar, ntok, gj); break;
+        case 1024: REDHIP_LAUNCH(prep_kernel<4>, grid, dim3(256), 0, s, x, gate_inp, hidden, h, l, xexp, scalar, ntok, gj); break;
+        case 2048: REDHIP_LAUNCH(prep_kernel<8>, grid, dim3(256), 0, s, x, gate_inp, hidden, h, l, xexp, scalar, ntok, gj); break;
+        case 4096: REDHIP_LAUNCH(prep_kernel<16>, grid, dim3(256), 0, s, x, gate_inp, hidden, h, l, xexp, scalar, ntok, gj); break;
+        default: REDHIP_LAUNCH(prep_kernel<0>, grid, dim3(256), 0, s, x, gate_inp, hidden, h, l, xexp, scalar, ntok, gj); break;
+    }
     if (job_done) *job_done = with_job;
     return hipGetLastError();
 }
