@@ -430,7 +430,7 @@ __global__ __launch_bounds__(256) void router_f32_kernel(const float *w, RouterA
 template <int NV, int NWV>          // NWV waves (rows) per workgroup
 __global__ __launch_bounds__(NWV * 64) void router_f32_multi_kernel(const float *w, RouterArgs a, uint32_t ntok, GroupJob job) {
     extern __shared__ __attribute__((aligned(16))) float xs_all[];      // [ntok][hidden]
-    __shared__ float s_amax[8], s_ninv[8];
+    __shared__ float s_amax[8];
     const uint32_t n_blocks = gridDim.x - (job.ids ? 1u : 0u);
     if (blockIdx.x == n_blocks) {                        // the extra workgroup: pair sort of the caller's routing
         group_small_given(job, reinterpret_cast<uint32_t *>(xs_all));
@@ -477,9 +477,17 @@ __global__ __launch_bounds__(NWV * 64) void router_f32_multi_kernel(const float 
             reinterpret_cast<float4 *>(xs_all + (uint64_t)tok * H)[lane + 64u * k] = xq[k];
         }
         amax = wave_max(amax);
-        if (lane == 0u) { s_amax[tok] = amax; s_ninv[tok] = norm_inv; }
+        if (lane == 0u) s_amax[tok] = amax;
     }
     __syncthreads();
+    // fp16 split of all tokens, one element per thread over the first workgroups, from the copy in LDS (the values the products use)
+    for (uint32_t idx = blockIdx.x * blockDim.x + threadIdx.x; idx < ntok * H; idx += n_blocks * blockDim.x) {
+        const uint32_t tok = idx / H;
+        const float v = xs_all[idx];
+        if (a.branch) a.xn_out[idx] = v;
+        split_hi_lo(v, exp2i(-prescale_exp(s_amax[tok])), a.xh + idx, a.xl + idx);
+        if (idx == tok * H) a.xexp[tok] = prescale_exp(s_amax[tok]);
+    }
     for (uint32_t tok = 0; tok < ntok; ++tok) {
         const float4 *xq = reinterpret_cast<const float4 *>(xs_all + (uint64_t)tok * H);
         float acc = 0.0f;
@@ -495,7 +503,6 @@ __global__ __launch_bounds__(NWV * 64) void router_f32_multi_kernel(const float 
         if (lane == 0u && r <= a.n_expert) a.logits[(uint64_t)tok * (a.n_expert + 1u) + r] = acc;
         else if (lane == 0u && r < n_rows) a.sh_gu[(uint64_t)tok * 2u * a.ffn + (r - a.n_expert - 1u)] = acc;
         if (lane == 0u && r == a.n_expert && a.scalar_out) a.scalar_out[tok] = 1.0f / (1.0f + expf(-acc));      // as the selection computes it
-        split_x_job(a, tok, s_amax[tok], s_ninv[tok], n_blocks);
     }
 }
 
