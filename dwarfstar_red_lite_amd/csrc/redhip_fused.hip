@@ -1795,7 +1795,7 @@ struct BatchArgs {
 };
 
 // Persistent workgroups walk the units (u, g) = (group of pairs, 32 FFN columns): 32 gate + 32 up rows of the
-// group's expert (u == U: the shared expert, all tokens) for every token that selected it, NTP token pairs per
+// group's expert (u >= U: the shared expert, two tokens per group when it is packed) for every token that selected it, NTP token pairs per
 // pass. The fp16 halves of all tokens sit in LDS, the routing metadata of the workgroup's units too, and the
 // weights of the next unit are requested while the current one is computed.
 constexpr int kMaxUnits = 16;      // units per workgroup
@@ -1858,19 +1858,22 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_batch_kernel(BatchArgs a) 
         group_small(gj, group_lds, [&](uint32_t t, uint32_t k) { return sel[t].ids[k]; }, [&](uint32_t t, uint32_t k) { return sel[t].w[k]; });
         __syncthreads();
     }
-    const uint32_t U = a.n_unique[0], n_units = (U + 1u) * FG;
+    // a packed shared expert is split into groups of two tokens (one pass each) so that no workgroup gets a unit of ntok / 2 passes
+    const uint32_t S = a.shared ? (a.ntok + 1u) / 2u : 1u;
+    const uint32_t U = a.n_unique[0], n_units = (U + S) * FG;
     uint32_t count = 0u;
     if (blockIdx.x < n_units) count = (n_units - blockIdx.x + gridDim.x - 1u) / gridDim.x;
     if (count > (uint32_t)kMaxUnits) count = kMaxUnits;
     if (count == 0u) return;
     if (tid < count) {
         const uint32_t u = (blockIdx.x + tid * gridDim.x) / FG;
-        const bool sh = u == U;
+        const bool sh = u >= U;
         meta_expert[tid] = sh ? 0xffffffffu : a.uid[u];
-        const uint32_t p0 = sh ? P : a.expert_start[u], p1 = sh ? P + a.ntok : a.expert_start[u + 1u];
+        const uint32_t sp0 = P + (a.shared ? 2u * (u - U) : 0u), sp1 = a.shared && sp0 + 2u < P + a.ntok ? sp0 + 2u : P + a.ntok;
+        const uint32_t p0 = sh ? sp0 : a.expert_start[u], p1 = sh ? sp1 : a.expert_start[u + 1u];
         meta_p0[tid] = p0;
         meta_n[tid] = sh && !a.shared ? 0u : p1 - p0;      // a shared expert that is not packed has no passes: its products are an input
-        for (uint32_t i = 0; i < p1 - p0 && i < (uint32_t)kMaxTok; ++i) meta_tok[tid][i] = (uint8_t)(sh ? i : a.pair_token[p0 + i]);
+        for (uint32_t i = 0; i < p1 - p0 && i < (uint32_t)kMaxTok; ++i) meta_tok[tid][i] = (uint8_t)(sh ? p0 - P + i : a.pair_token[p0 + i]);
     }
     if (!a.sel.logits) stage_x(0u);
     if constexpr (FMT == 0) build_tables(lds, tid, grid_entry);
@@ -2350,7 +2353,7 @@ hipError_t launch_batch_packed(const void *experts, uint64_t stride, const void 
     if (select && !batch_select_ok(*select, ntok, top_k, n_expert)) return hipErrorInvalidValue;
     if (select) a.sel = *select;
     const uint32_t P = ntok * top_k, n_groups = (P < n_expert ? P : n_expert) + 1u;
-    hipError_t e = launch_gateup_batch_kernel(a, n_groups, s);
+    hipError_t e = launch_gateup_batch_kernel(a, n_groups + (shared ? (ntok + 1u) / 2u - 1u : 0u), s);      // the shared expert counts as one group per two tokens
     if (e != hipSuccess) return e;
     prof_set_stage(ST_BATCH_DOWN);
     const uint32_t groups_per_wave = (n_groups + kWaves - 1u) / kWaves;     // bound known on the host: min(pairs, experts) + 1 groups
