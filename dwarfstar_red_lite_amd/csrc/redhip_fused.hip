@@ -2007,6 +2007,7 @@ __global__ __launch_bounds__(kWaves * 64) void down_batch_kernel(BatchArgs a) {
     const uint32_t H = a.hidden, F = a.ffn, FG = F / 32u, FB = F / 256u, P = a.ntok * a.top_k;
     const uint64_t grid_entry = tid < 256u ? redhip_iq2xxs_grid[tid] : 0ull;
     const uint32_t row0 = 8u * blockIdx.x, U = __builtin_amdgcn_readfirstlane(a.n_unique[0]);
+    const uint32_t S = (a.ntok + 1u) / 2u;           // the shared expert as S groups of two tokens: one pass each, on S different waves
     const uint64_t down_off = 2u * ((uint64_t)F * (H / 32u) * 8u + (uint64_t)F * (H / 256u) * 2u), qs_bytes = (uint64_t)H * FG * 8u;
 
     uint2 wq[GPW][NCH][2];
@@ -2020,8 +2021,10 @@ __global__ __launch_bounds__(kWaves * 64) void down_batch_kernel(BatchArgs a) {
             // wave-uniform values: kept in scalar registers
             const uint32_t e = __builtin_amdgcn_readfirstlane(a.uid[sh ? 0u : uc]), es0 = __builtin_amdgcn_readfirstlane(a.expert_start[uc]),
                            es1 = __builtin_amdgcn_readfirstlane(a.expert_start[sh ? U : uc + 1u]);
-            gp0[i] = sh ? P : es0;
-            gp1[i] = u > U ? gp0[i] : sh ? P + a.ntok : es1;
+            // groups U .. U + S - 1: the shared expert, two tokens each (its pairs follow the routed ones); beyond: empty
+            const uint32_t sub = u - U, sp0 = P + 2u * sub, sp1 = sp0 + 2u < P + a.ntok ? sp0 + 2u : P + a.ntok;
+            gp0[i] = sh ? (sub < S ? sp0 : P) : es0;
+            gp1[i] = sh ? (sub < S ? sp1 : gp0[i]) : es1;
             const uint8_t *dn = (sh ? a.shared : a.experts + (uint64_t)e * a.stride) + down_off;
 #pragma unroll
             for (int c = 0; c < NCH; ++c) {
@@ -2055,7 +2058,7 @@ __global__ __launch_bounds__(kWaves * 64) void down_batch_kernel(BatchArgs a) {
     build_tables(lds, tid, grid_entry);
     __syncthreads();
 
-    for (uint32_t first = wave; first <= U; first += 16u * GPW) {
+    for (uint32_t first = wave; first < U + S; first += 16u * GPW) {
         if (first != wave) request(first);
         Pass buf[2];                                     // activations of the current and of the next group
         load_pass(gp0[0], gp1[0], buf[0]);
@@ -2356,7 +2359,7 @@ hipError_t launch_batch_packed(const void *experts, uint64_t stride, const void 
     hipError_t e = launch_gateup_batch_kernel(a, n_groups + (shared ? (ntok + 1u) / 2u - 1u : 0u), s);      // the shared expert counts as one group per two tokens
     if (e != hipSuccess) return e;
     prof_set_stage(ST_BATCH_DOWN);
-    const uint32_t groups_per_wave = (n_groups + kWaves - 1u) / kWaves;     // bound known on the host: min(pairs, experts) + 1 groups
+    const uint32_t groups_per_wave = (n_groups + (ntok + 1u) / 2u - 1u + kWaves - 1u) / kWaves;     // bound known on the host: min(pairs, experts) groups + the shared expert's
     const dim3 dgrid(hidden / 8u), dblock(kWaves * 64);
     if (ffn > 512u) REDHIP_LAUNCH((down_batch_kernel<144, 2, 2>), dgrid, dblock, 0, s, a);
     else if (groups_per_wave <= 2u) REDHIP_LAUNCH((down_batch_kernel<144, 1, 2>), dgrid, dblock, 0, s, a);
