@@ -1814,6 +1814,7 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_batch_kernel(BatchArgs a) 
     __shared__ float tok_scale[kMaxTok];
     __shared__ SelectOut sel[kMaxTok];
     __shared__ uint32_t group_lds[kGroupLdsWords];
+    __shared__ uint32_t pass_start[130];                 // [128]: passes in all, [129]: whether any group has more than one
     const uint32_t tid = threadIdx.x, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t H = a.hidden, F = a.ffn, HG = H / 32u, HB = H / 256u, FG = F / 32u, P = a.ntok * a.top_k;
@@ -1860,17 +1861,50 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_batch_kernel(BatchArgs a) 
     }
     // a packed shared expert is split into groups of two tokens (one pass each) so that no workgroup gets a unit of ntok / 2 passes
     const uint32_t S = a.shared ? (a.ntok + 1u) / 2u : 1u;
-    const uint32_t U = a.n_unique[0], n_units = (U + S) * FG;
+    // Routed groups too are scheduled pass by pass (2 * NTP tokens of one expert): pass_start[u] = passes of the groups before u, so
+    // that a popular expert's tokens spread over workgroups instead of making one unit of several passes.
+    const uint32_t U = a.n_unique[0];
+    if (wave == 0u) {                                    // at most 128 groups: two per lane, prefix sums by lane shifts
+        constexpr uint32_t TPP = 2u * NTP;
+        const uint32_t u0 = lane, u1 = lane + 64u;
+        const uint32_t c0 = u0 < U ? (a.expert_start[u0 + 1u] - a.expert_start[u0] + TPP - 1u) / TPP : 0u;
+        const uint32_t c1 = u1 < U ? (a.expert_start[u1 + 1u] - a.expert_start[u1] + TPP - 1u) / TPP : 0u;
+        if (__ballot(c0 > 1u || c1 > 1u) == 0ull) {      // every group is one pass (the usual case without popular experts): pass = group
+            pass_start[u0] = u0 < U ? u0 : U;
+            pass_start[u1] = u1 < U ? u1 : U;
+            if (lane == 63u) { pass_start[128] = U; pass_start[129] = 0u; }
+        } else {
+            uint32_t s0 = c0, s1 = c1;
+#pragma unroll
+            for (int o = 1; o < 64; o <<= 1) {
+                const uint32_t n0 = __shfl_up(s0, o, 64), n1 = __shfl_up(s1, o, 64);
+                if (lane >= (uint32_t)o) { s0 += n0; s1 += n1; }
+            }
+            const uint32_t half = __shfl(s0, 63, 64);
+            pass_start[u0] = s0 - c0;
+            pass_start[u1] = half + s1 - c1;
+            if (lane == 63u) { pass_start[128] = half + s1; pass_start[129] = 1u; }
+        }
+    }
+    __syncthreads();
+    const uint32_t V = pass_start[128], n_units = (V + S) * FG;
     uint32_t count = 0u;
     if (blockIdx.x < n_units) count = (n_units - blockIdx.x + gridDim.x - 1u) / gridDim.x;
     if (count > (uint32_t)kMaxUnits) count = kMaxUnits;
     if (count == 0u) return;
     if (tid < count) {
-        const uint32_t u = (blockIdx.x + tid * gridDim.x) / FG;
-        const bool sh = u >= U;
+        const uint32_t v = (blockIdx.x + tid * gridDim.x) / FG;      // pass number: routed passes, then the shared expert's
+        const bool sh = v >= V;
+        uint32_t u = sh ? 0u : v;                        // the group of pass v: the last one with pass_start[u] <= v
+        if (pass_start[129]) {
+            u = 0u;
+#pragma unroll
+            for (uint32_t step = 64u; step > 0u; step >>= 1) { if (u + step < U && pass_start[u + step] <= v) u += step; }
+        }
         meta_expert[tid] = sh ? 0xffffffffu : a.uid[u];
-        const uint32_t sp0 = P + (a.shared ? 2u * (u - U) : 0u), sp1 = a.shared && sp0 + 2u < P + a.ntok ? sp0 + 2u : P + a.ntok;
-        const uint32_t p0 = sh ? sp0 : a.expert_start[u], p1 = sh ? sp1 : a.expert_start[u + 1u];
+        const uint32_t sp0 = P + (a.shared ? 2u * (v - V) : 0u), sp1 = a.shared && sp0 + 2u < P + a.ntok ? sp0 + 2u : P + a.ntok;
+        const uint32_t rp0 = sh ? 0u : a.expert_start[u] + 2u * NTP * (v - pass_start[u]), rend = sh ? 0u : a.expert_start[u + 1u];
+        const uint32_t p0 = sh ? sp0 : rp0, p1 = sh ? sp1 : (rp0 + 2u * NTP < rend ? rp0 + 2u * NTP : rend);
         meta_p0[tid] = p0;
         meta_n[tid] = sh && !a.shared ? 0u : p1 - p0;      // a shared expert that is not packed has no passes: its products are an input
         for (uint32_t i = 0; i < p1 - p0 && i < (uint32_t)kMaxTok; ++i) meta_tok[tid][i] = (uint8_t)(sh ? p0 - P + i : a.pair_token[p0 + i]);
@@ -2356,7 +2390,8 @@ hipError_t launch_batch_packed(const void *experts, uint64_t stride, const void 
     if (select && !batch_select_ok(*select, ntok, top_k, n_expert)) return hipErrorInvalidValue;
     if (select) a.sel = *select;
     const uint32_t P = ntok * top_k, n_groups = (P < n_expert ? P : n_expert) + 1u;
-    hipError_t e = launch_gateup_batch_kernel(a, n_groups + (shared ? (ntok + 1u) / 2u - 1u : 0u), s);      // the shared expert counts as one group per two tokens
+    // units are passes of two tokens: at most (pairs + groups) / 2 routed ones, then the shared expert's, one per two tokens
+    hipError_t e = launch_gateup_batch_kernel(a, (P + (P < n_expert ? P : n_expert) + 1u) / 2u + (ntok + 1u) / 2u, s);
     if (e != hipSuccess) return e;
     prof_set_stage(ST_BATCH_DOWN);
     const uint32_t groups_per_wave = (n_groups + (ntok + 1u) / 2u - 1u + kWaves - 1u) / kWaves;     // bound known on the host: min(pairs, experts) groups + the shared expert's
@@ -2420,7 +2455,7 @@ hipError_t launch_batch_mixed(uint32_t gate_up_type, const int8_t *gate_up_grid,
     if (select && !batch_select_ok(*select, ntok, top_k, n_expert)) return hipErrorInvalidValue;
     if (select) a.sel = *select;
     const uint32_t P = ntok * top_k, n_groups = (P < n_expert ? P : n_expert) + 1u;
-    hipError_t e = launch_gateup_batch_kernel(a, n_groups, s, gate_up_type);
+    hipError_t e = launch_gateup_batch_kernel(a, (P + (P < n_expert ? P : n_expert) + 1u) / 2u + 1u, s, gate_up_type);      // passes of two tokens + the shared expert's SwiGLU unit
     if (e != hipSuccess) return e;
     prof_set_stage(ST_BATCH_DOWN);
     if (on_mfma) {      // packed down matrices on the matrix units, the shared expert's rows from its f32 copy
