@@ -302,7 +302,7 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
     if (m->packed_gu()) {    // xh / xl / scalar come from the router kernel or the prep kernel
         const Layer &L = m->layers[layer];
         prof_set_stage(ST_GATEUP);
-        HIP_OK(launch_gateup_select(L.packed, m->packed_stride, L.shared_packed, L.shared, x, select_here && m->shared_gu_ready ? m->act : nullptr,
+        HIP_OK(launch_gateup_select(L.packed, m->packed_stride, L.shared_packed, L.shared, x, m->shared_gu_ready ? m->act : nullptr,
                                     select_here ? m->logits : nullptr, ids, m->ids,
                                     m->weights, m->scalar, m->xh, m->xl, m->xexp, m->act_h, m->act_l, m->act_exp, c.hidden, c.ffn, c.n_expert,
                                     c.top_k, s, ntok, m->gu_type, m->gu_grid), "gate/up launch");      // ntok > 1: a small batch on a mixed layout, one grid layer per token
@@ -684,9 +684,9 @@ int redhip_moe_experts(redhip_moe_t h, uint32_t layer, const float *x_dev, uint3
         const bool to_group = m->small_batch(ntok) || m->grouped_mixed(ntok, 2u);
         const GroupJob job{ids_dev, weights_dev, ntok, m->cfg.top_k, m->cfg.n_expert, m->uid, m->expert_start, m->pair_token, m->pair_weight, m->tok_pair, m->n_unique};
         bool grouped = false;
-        if (m->grouped_mixed(ntok, 2u) && L.dense_gu && (nv == 2u || nv == 4u || nv == 8u || nv == 16u)) {
-            // the grouped kernels take the shared expert's gate | up products as an input: one f32 GEMV over its f32 copy (no router rows),
-            // which also leaves the fp16 halves of x and the shared expert's scalar gate
+        if (m->mixed && m->packed_gu() && (ntok == 1u || m->small_batch_mixed(ntok)) && L.dense_gu && (nv == 2u || nv == 4u || nv == 8u || nv == 16u)) {
+            // one token or a small batch on a mixed layout: the kernels take the shared expert's gate | up products as an input: one f32
+            // GEMV over its f32 copy (no router rows), which also leaves the fp16 halves of x and the shared expert's scalar gate
             prof_set_stage(ST_SHARED_GATEUP);
             HIP_OK(launch_router_gemv(T_F32, L.dense_gu, x_dev, L.gate_inp, ntok, m->cfg.hidden, 0u, m->logits, m->xh, m->xl, m->xexp, nullptr, m->act,
                                       m->cfg.ffn, s, L.dense_gu, m->scalar, to_group ? &job : nullptr, &grouped), "shared gate/up launch");

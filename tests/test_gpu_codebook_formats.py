@@ -254,7 +254,7 @@ def test_codebook_layout_chunks(layout, shape, ntok, grids):
 
 @pytest.mark.parametrize("layout", ["xs", "m"])
 def test_codebook_layout_given_routing(layout, grids):
-    """caller-given routing (drawn logits with hot experts, so tokens share experts) on IQ2_XS / IQ1_M layers: batches of 2, 3
+    """caller-given routing (drawn logits with hot experts, so tokens share experts) on IQ2_XS / IQ1_M layers: one token (single-token kernels), batches of 2, 3
     and 8 (grouped kernels, the pair sort riding in the shared gate/up launch) and a chunk of 40 tokens, against the oracle run token by token"""
     from dwarfstar_red_lite_amd.moe import ResidentMoe
     from test_gpu_moe_batch import oracle_tokens
@@ -264,7 +264,7 @@ def test_codebook_layout_given_routing(layout, grids):
     m = ResidentMoe(cfg, n_layer=1, max_tokens=40)
     m.load_layer(0, lay)
     rng = np.random.default_rng(77)
-    for ntok in (2, 3, 8, 40):
+    for ntok in (1, 2, 3, 8, 40):
         x = synth.normed_x(rng, ntok, cfg["hidden"])
         logits = synth.hot_logits(rng, ntok, cfg["n_expert"])
         sel = [orc.router_select(logits[t], cfg["top_k"]) for t in range(ntok)]

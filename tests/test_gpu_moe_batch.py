@@ -39,13 +39,13 @@ def test_ragged_small_batches_hot_experts(layout):
     m = ResidentMoe(cfg, n_layer=1, max_tokens=8)
     m.load_layer(0, lay)
     rng = np.random.default_rng(31)
-    for ntok in (2, 3, 8):
+    for ntok in (1, 2, 3, 8):                                                      # (one token: the caller's routing on the single-token kernels)
         x = synth.normed_x(rng, ntok, cfg["hidden"])
         logits = synth.hot_logits(rng, ntok, cfg["n_expert"])
         sel = [orc.router_select(logits[t], cfg["top_k"]) for t in range(ntok)]
         ids = np.stack([s[0] for s in sel])
         w = np.stack([s[1] for s in sel])
-        assert len(set(ids.ravel().tolist())) < ntok * cfg["top_k"]            # tokens do share experts
+        assert ntok == 1 or len(set(ids.ravel().tolist())) < ntok * cfg["top_k"]            # tokens do share experts
         got = m.experts(0, torch.from_numpy(x).cuda(), torch.from_numpy(ids.astype(np.int32)).cuda(), torch.from_numpy(w).cuda()).cpu().numpy()
         want = oracle_tokens(cfg, lay, x, ids, w)
         for t in range(ntok):
