@@ -45,42 +45,9 @@ def parse():
     ap.add_argument("--no-micro", action="store_true", help="skip the single-GEMV microbench (only run for --layout iq2 --batch 1)")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--calibrate", action="store_true", help="also run the plain copy kernel of known size (for rocprofv3 --pmc runs)")
+    ap.add_argument("--no-sweep", action="store_true", help="skip the B=2/4/8 hot-routing sweep that the default (B=1, own router) run appends")
+    ap.add_argument("--prime", type=int, default=2000, help="untimed steps before the warm-up that bring the clocks up (reported as clock_priming_steps)")
     return ap.parse_args()
-
-
-def synth_layer_on_gpu(torch, gen, cfg):
-    """Random-valid blocks generated on the GPU (same construction as dwarfstar_red_lite_amd.synth, torch RNG)."""
-    from dwarfstar_red_lite_amd import synth
-
-    def rows(t, nrows, ncols, d_range=None):
-        bb = synth.BLOCK_BYTES[t]
-        nb = nrows * (ncols // 256)
-        raw = torch.randint(0, 256, (nb, bb), dtype=torch.uint8, device="cuda", generator=gen)
-        lo, hi = d_range or synth.D_RANGE[t]
-        d = (lo + (hi - lo) * torch.rand(nb, device="cuda", generator=gen)).to(torch.float16).view(torch.uint8).reshape(nb, 2)
-        if t == synth.TYPE_IQ1_M:          # d sits in the top nibbles of the four 16-bit scale words (bytes 48..55)
-            for i in range(4):
-                nib = (d[:, i // 2] >> (4 * (i % 2))) & 15
-                raw[:, 49 + 2 * i] = (raw[:, 49 + 2 * i] & 0x0F) | (nib << 4)
-        else:
-            off = synth.D_OFFSET[t]
-            raw[:, off:off + 2] = d
-        return raw.reshape(nrows, -1)
-
-    H, F, E = cfg["hidden"], cfg["ffn"], cfg["n_expert"]
-    a = {}
-    if cfg["router_type"] == 0:
-        a["router"] = 0.02 * torch.randn((E, H), device="cuda", generator=gen)
-    else:
-        a["router"] = rows(cfg["router_type"], E, H, d_range=(1e-5, 3e-5))
-    a["gate"] = rows(cfg["gate_up_type"], E * F, H).reshape(E, -1)
-    a["up"] = rows(cfg["gate_up_type"], E * F, H).reshape(E, -1)
-    a["down"] = rows(cfg["down_type"], E * H, F).reshape(E, -1)
-    a["sh_gate"] = rows(cfg["sh_gate_up_type"], F, H)
-    a["sh_up"] = rows(cfg["sh_gate_up_type"], F, H)
-    a["sh_down"] = rows(cfg["sh_down_type"], H, F)
-    a["sh_gate_inp"] = 0.02 * torch.randn(H, device="cuda", generator=gen)
-    return a
 
 
 def layer_bytes(cfg, distinct_experts, batch):
@@ -112,97 +79,11 @@ def oracle_given_routing(orc, cfg, lay, x, ids, w, threads):
     return out
 
 
-def main():
-    args = parse()
-    if args.gpus != 1:
-        print("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)" % args.gpus, file=sys.stderr)
-        sys.exit(2)
-    import numpy as np
-    import torch
-
-    from dwarfstar_red_lite_amd import load, synth
-    from dwarfstar_red_lite_amd.moe import ResidentMoe
-
-    lib = load()
-    torch.cuda.init()
-    cfg = synth.layer_config(layout=args.layout)
-    B, NL = args.batch, args.layers
-    if args.layout in ("xs", "m"):          # these two decode through codebooks the caller supplies: the reference's, from the fixture
-        import oracle_lib as orc
-        from dwarfstar_red_lite_amd import moe as moe_api
-        g = json.load(open(os.path.join(ROOT, "tests", "golden", "iq_grids.json")))
-        grids = [np.frombuffer(bytes.fromhex(g[k]), np.int8) for k in ("iq2_xs", "iq1_m")]
-        moe_api.set_codebooks(*grids)
-        orc.set_codebooks(*grids)
-    moe = ResidentMoe(cfg, n_layer=NL, max_tokens=B)
-    gen = torch.Generator(device="cuda")
-    gen.manual_seed(20241125)
-    layer0 = None
-    for l in range(NL):
-        a = synth_layer_on_gpu(torch, gen, cfg)
-        moe.load_layer(l, a)
-        if l == 0:
-            layer0 = {k: v.cpu().numpy() for k, v in a.items()}
-            if cfg["router_type"] != 0:
-                layer0["router"] = layer0["router"].view(np.uint8)
-        del a
-    torch.cuda.synchronize()
-
-    NX = 64
-    xs_host = synth.normed_x(np.random.default_rng(99), NX * B, cfg["hidden"]).reshape(NX, B, cfg["hidden"])
-    xs = torch.from_numpy(xs_host).cuda()
-    outs = torch.empty_like(xs)
-    stream = torch.cuda.Stream()
-
-    # drawn routing (configs 3 and 4): ids / weights per activation set, made on the host
-    route_ids = route_w = None
-    if args.routing != "router":
-        import oracle_lib as orc
-        rr = np.random.default_rng(7)
-        K_, E_ = cfg["top_k"], cfg["n_expert"]
-        ids_h = np.empty((NX, B, K_), np.uint32)
-        w_h = np.empty((NX, B, K_), np.float32)
-        for i in range(NX):
-            if args.routing == "hot":
-                lg = synth.hot_logits(rr, B, E_)
-                for t in range(B):
-                    ids_h[i, t], w_h[i, t] = orc.router_select(lg[t], K_)
-            else:
-                ids_h[i] = synth.zipf_topk(rr, B, E_, K_)
-                ww = rr.random((B, K_)).astype(np.float32) + 0.1
-                w_h[i] = ww / ww.sum(axis=1, keepdims=True)
-        route_ids = torch.from_numpy(ids_h.astype(np.int32)).cuda()
-        route_w = torch.from_numpy(w_h).cuda()
-
-    def step(i):
-        if route_ids is None:
-            moe.forward(i % NL, xs[i % NX], outs[i % NX])
-        else:
-            moe.experts(i % NL, xs[i % NX], route_ids[i % NX], route_w[i % NX], outs[i % NX])
-
-    # ---- parity gate on the very tensors the timed steps use (layer 0, CPU oracle) ----
-    import oracle_lib as orc
-    ref = orc.Layer(cfg, **layer0)
-    with torch.cuda.stream(stream):
-        step(0)
-        if route_ids is None:
-            gids, _, _ = moe.last_route(B)
-    if route_ids is None:
-        want, cids, _, _ = ref.forward(xs_host[0], threads=os.cpu_count() or 1)
-        got = outs[0].cpu().numpy()
-        ids_ok = bool(np.array_equal(gids, cids))
-    else:           # drawn routing: the oracle's routed experts + gated shared expert for the first tokens of the step
-        n_chk = min(B, 8)
-        want = oracle_given_routing(orc, cfg, layer0, xs_host[0][:n_chk], ids_h[0][:n_chk], w_h[0][:n_chk], os.cpu_count() or 1)
-        got = outs[0][:n_chk].cpu().numpy()
-        ids_ok = True
-    rel = float(np.linalg.norm(got - want) / np.linalg.norm(want))
-    if not rel <= 1e-3 or not ids_ok:
-        print("PARITY FAILURE: rel L2 %.3g vs the CPU oracle, router ids identical: %s" % (rel, ids_ok), file=sys.stderr)
-        sys.exit(1)
-
-    # ---- timed region ----
-    K, W = args.steps, args.warmup
+def time_steps(torch, stream, step, K, W, outs, rows_written, use_graph, replays=15):
+    """W untimed + exactly K timed eager steps (synchronised on both sides); then the same K steps recorded once into a HIP graph
+    (kernel launches only) and replayed: every replay is checked bit for bit against the eager outputs on the rows the K steps write,
+    and the median over `replays` timed replays (each exactly K steps between two synchronisations) is what a decode loop that issues
+    graphs would see."""
     with torch.cuda.stream(stream):
         for i in range(W):
             step(i)
@@ -213,65 +94,56 @@ def main():
             step(W + i)
         stream.synchronize()
         torch.cuda.synchronize()
+        eager_ms = (time.perf_counter() - t0) * 1e3 / K
+    res = {"eager_ms": eager_ms, "graph_ms": None, "ms": eager_ms, "mode": "eager", "replays_timed": 0}
+    if not use_graph:
+        return res
+    idx = torch.tensor(sorted(rows_written), device="cuda")
+    eager_rows = outs[idx].clone()
+    graph = torch.cuda.CUDAGraph()
+    with torch.cuda.graph(graph, stream=stream):
+        for i in range(K):
+            step(W + i)
+    times = []
+    for r in range(2 + replays):                # the first two replays are untimed (the first one uploads the graph)
+        outs.zero_()
+        torch.cuda.synchronize()
+        t0 = time.perf_counter()
+        graph.replay()
+        torch.cuda.synchronize()
         t1 = time.perf_counter()
-        eager_ms_per_step = (t1 - t0) * 1e3 / K
-    ms_per_step, launch_mode, graph_ms_per_step = eager_ms_per_step, "eager", None
-    if not args.no_graph:
-        # the same K steps recorded once into a HIP graph (kernel launches only, no memset nodes) and replayed: this
-        # is how a decode loop would issue them; the replay is checked against the eager outputs before it is timed
-        eager_out = outs.clone()
-        graph = torch.cuda.CUDAGraph()
-        with torch.cuda.graph(graph, stream=stream):
-            for i in range(K):
-                step(W + i)
-        for _ in range(2):                      # untimed replays (the first one uploads the graph)
-            graph.replay()
-            torch.cuda.synchronize()
-            if not torch.equal(outs, eager_out):
-                print("GRAPH REPLAY MISMATCH: falling back to eager timing", file=sys.stderr)
-                break
-        else:
-            torch.cuda.synchronize()
-            t0 = time.perf_counter()
-            graph.replay()
-            torch.cuda.synchronize()
-            t1 = time.perf_counter()
-            graph_ms_per_step = (t1 - t0) * 1e3 / K
-            # (chunks that fork work onto a second stream replay a little slower than they launch: the quicker mode is the one reported)
-            if graph_ms_per_step <= eager_ms_per_step:
-                ms_per_step, launch_mode = graph_ms_per_step, "hip_graph"
-    with torch.cuda.stream(stream):
+        if not torch.equal(outs[idx], eager_rows):
+            print("GRAPH REPLAY MISMATCH on replay %d: the eager timing is reported" % r, file=sys.stderr)
+            res["replay_mismatch"] = True
+            return res
+        if r >= 2:
+            times.append((t1 - t0) * 1e3 / K)
+    times.sort()
+    res["graph_ms"] = times[len(times) // 2]
+    res["graph_ms_min"] = times[0]
+    res["replays_timed"] = len(times)
+    # (chunks that fork work onto a second stream replay a little slower than they launch: the quicker mode is the one reported)
+    if res["graph_ms"] <= eager_ms:
+        res["ms"], res["mode"] = res["graph_ms"], "hip_graph"
+    return res
 
-        # the same K steps again with per-kernel begin/end timestamps (HIP events on the launch stream)
-        n_stage = lib.redhip_profile_stage_count()
+
+def stage_profile(lib, stream, torch, step, K, W):
+    """the same K steps with per-kernel begin/end timestamps (HIP events on the launch stream)"""
+    n_stage = lib.redhip_profile_stage_count()
+    with torch.cuda.stream(stream):
         lib.redhip_profile_begin()
         for i in range(K):
             step(W + i)
         stage_ms = (C.c_double * n_stage)()
         stage_n = (C.c_uint32 * n_stage)()
         lib.redhip_profile_end(stage_ms, stage_n, n_stage)
-        # distinct routed experts per step (B > 1 shares experts between tokens)
-        distinct = []
-        for i in range(min(K, NX)):
-            if route_ids is None:
-                step(W + i)
-                ids, _, _ = moe.last_route(B)
-            else:
-                ids = ids_h[(W + i) % NX]
-            distinct.append(len(set(ids.ravel().tolist())))
-    if args.calibrate:         # yardstick for FETCH_SIZE / WRITE_SIZE: copies of exactly CAL_BYTES in, CAL_BYTES out
-        cal_src = torch.empty(CAL_BYTES, dtype=torch.uint8, device="cuda").random_(0, 256)
-        cal_dst = torch.empty_like(cal_src)
-        for _ in range(4):
-            assert lib.redhip_calibration_copy(cal_dst.data_ptr(), cal_src.data_ptr(), CAL_BYTES, None)
-        torch.cuda.synchronize()
-    stages = {lib.redhip_profile_stage_name(s).decode(): {"ms_total": stage_ms[s], "launches": int(stage_n[s]),
-                                                        "us_avg": 1e3 * stage_ms[s] / stage_n[s]}
-              for s in range(n_stage) if stage_n[s]}
-    mean_distinct = float(np.mean(distinct))
-    lb = layer_bytes(cfg, mean_distinct, B)
+    return {lib.redhip_profile_stage_name(s).decode(): {"ms_total": stage_ms[s], "launches": int(stage_n[s]), "us_avg": 1e3 * stage_ms[s] / stage_n[s]}
+            for s in range(n_stage) if stage_n[s]}
 
-    # dominant kernel = the stage with the largest total time; its algorithmic bytes per launch
+
+def kernel_roofline(cfg, synth, stages, K, B, mean_distinct, lb, traffic_key):
+    """the stage with the largest summed kernel time, its algorithmic bytes (or flops) per launch and what it achieves"""
     dom = max(stages, key=lambda k: stages[k]["ms_total"])
     H, F = cfg["hidden"], cfg["ffn"]
     gate_up = lb["one_expert"] - H * synth.row_bytes(cfg["down_type"], F)
@@ -297,34 +169,163 @@ def main():
     traffic = None
     try:
         with open(os.path.join(ROOT, "profiles", "hbm_traffic.json")) as fh:
-            rec = json.load(fh).get("%s_b%d" % (args.layout, B), {}).get("stages", {}).get(dom)
+            rec = json.load(fh).get(traffic_key, {}).get("stages", {}).get(dom)
         if rec:
             traffic = int(rec["fetch_bytes"] + rec["write_bytes"])
     except (OSError, ValueError, KeyError):
         traffic = None
-    roofline = None
     if dom in ("prefill_gateup", "prefill_down"):
         # prefill tiles run on the MFMA units: algorithmic flops of the stage (2 per multiply-add, every (token, expert) pair
         # and every token's shared expert once; the fp16 hi/lo split that doubles the issued MFMAs is not counted)
         pairs = B * (cfg["top_k"] + 1)
         flops = pairs * 2.0 * H * F * (2 if dom == "prefill_gateup" else 1)
         achieved = flops / (dom_us * 1e-6) / 1e12
-        roofline = {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 2), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
-                    "frac": round(achieved / MFMA_F16_PEAK_TFLOPS, 4), "traffic": traffic, "flops_per_launch": int(flops),
-                    "launch_us": round(dom_us, 3)}
-    elif dom_bytes:
+        return {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 2), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
+                "frac": round(achieved / MFMA_F16_PEAK_TFLOPS, 4), "traffic": traffic, "flops_per_launch": int(flops), "launch_us": round(dom_us, 3)}
+    if dom_bytes:
         achieved = dom_bytes / (dom_us * 1e-6) / 1e9
-        roofline = {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
-                    "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic,
-                    "bytes_per_launch": int(dom_bytes), "launch_us": round(dom_us, 3)}
+        return {"bound": "hbm", "kernel": dom, "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                "frac": round(achieved / HBM_PEAK_GBS, 4), "traffic": traffic, "bytes_per_launch": int(dom_bytes), "launch_us": round(dom_us, 3)}
+    return None
+
+
+def main():
+    args = parse()
+    if args.gpus != 1:
+        print("bench.py measures one GPU: this build has no multi-GPU path (--gpus %d refused)" % args.gpus, file=sys.stderr)
+        sys.exit(2)
+    import numpy as np
+    import torch
+
+    import oracle_lib as orc
+    from dwarfstar_red_lite_amd import load, synth
+    from dwarfstar_red_lite_amd.moe import ResidentMoe
+
+    lib = load()
+    torch.cuda.init()
+    cfg = synth.layer_config(layout=args.layout)
+    B, NL = args.batch, args.layers
+    K, W = args.steps, args.warmup
+    H, F = cfg["hidden"], cfg["ffn"]
+    if args.layout in ("xs", "m"):          # these two decode through codebooks the caller supplies: the reference's, from the fixture
+        from dwarfstar_red_lite_amd import moe as moe_api
+        g = json.load(open(os.path.join(ROOT, "tests", "golden", "iq_grids.json")))
+        grids = [np.frombuffer(bytes.fromhex(g[k]), np.int8) for k in ("iq2_xs", "iq1_m")]
+        moe_api.set_codebooks(*grids)
+        orc.set_codebooks(*grids)
+    # the default run (one token, the layer's own router) appends the small-batch sweep on the same resident handle
+    sweep = [] if (args.no_sweep or B != 1 or args.routing != "router") else [2, 4, 8]
+    moe = ResidentMoe(cfg, n_layer=NL, max_tokens=max([B] + sweep))
+    gen = torch.Generator(device="cuda")
+    gen.manual_seed(20241125)
+    layer0 = None
+    for l in range(NL):
+        a = synth.make_layer_gpu(torch, gen, cfg)
+        moe.load_layer(l, a)
+        if l == 0:
+            layer0 = synth.layer_to_host(a, cfg)
+        del a
+    torch.cuda.synchronize()
+    ref = orc.Layer(cfg, **layer0)
+    stream = torch.cuda.Stream()
+    NX = 64
+
+    def run_workload(B, routing, micro_xs=None):
+        """parity gate on layer 0, then timing, per-kernel profile and the dominant kernel's roofline for batches of B tokens"""
+        xs_host = synth.normed_x(np.random.default_rng(99 + B), NX * B, H).reshape(NX, B, H)
+        xs = torch.from_numpy(xs_host).cuda()
+        outs = torch.zeros_like(xs)
+        # drawn routing (the ragged small-batch and prefill-chunk configurations): ids / weights per activation set, made on the host
+        route_ids = route_w = ids_h = w_h = None
+        if routing != "router":
+            rr = np.random.default_rng(7)
+            K_, E_ = cfg["top_k"], cfg["n_expert"]
+            ids_h = np.empty((NX, B, K_), np.uint32)
+            w_h = np.empty((NX, B, K_), np.float32)
+            for i in range(NX):
+                if routing == "hot":
+                    lg = synth.hot_logits(rr, B, E_)
+                    for t in range(B):
+                        ids_h[i, t], w_h[i, t] = orc.router_select(lg[t], K_)
+                else:
+                    ids_h[i] = synth.zipf_topk(rr, B, E_, K_)
+                    ww = rr.random((B, K_)).astype(np.float32) + 0.1
+                    w_h[i] = ww / ww.sum(axis=1, keepdims=True)
+            route_ids = torch.from_numpy(ids_h.astype(np.int32)).cuda()
+            route_w = torch.from_numpy(w_h).cuda()
+
+        def step(i):
+            if route_ids is None:
+                moe.forward(i % NL, xs[i % NX], outs[i % NX])
+            else:
+                moe.experts(i % NL, xs[i % NX], route_ids[i % NX], route_w[i % NX], outs[i % NX])
+
+        # ---- parity gate on the very tensors the timed steps use (layer 0, CPU oracle) ----
+        torch.cuda.synchronize()
+        with torch.cuda.stream(stream):
+            step(0)
+            if route_ids is None:
+                gids, _, _ = moe.last_route(B)
+            stream.synchronize()
+        if route_ids is None:
+            want, cids, _, _ = ref.forward(xs_host[0], threads=os.cpu_count() or 1)
+            got = outs[0].cpu().numpy()
+            ids_ok = bool(np.array_equal(gids, cids))
+        else:           # drawn routing: the oracle's routed experts + gated shared expert for the first tokens of the step
+            n_chk = min(B, 8)
+            want = oracle_given_routing(orc, cfg, layer0, xs_host[0][:n_chk], ids_h[0][:n_chk], w_h[0][:n_chk], os.cpu_count() or 1)
+            got = outs[0][:n_chk].cpu().numpy()
+            ids_ok = True
+        rel = float(np.linalg.norm(got - want) / np.linalg.norm(want))
+        if not rel <= 1e-3 or not ids_ok:
+            print("PARITY FAILURE (B=%d, routing %s): rel L2 %.3g vs the CPU oracle, router ids identical: %s" % (B, routing, rel, ids_ok), file=sys.stderr)
+            sys.exit(1)
+
+        # ---- untimed clock priming, then the timed region ----
+        with torch.cuda.stream(stream):
+            for i in range(args.prime):
+                step(i)
+            stream.synchronize()
+        rows_written = {(W + i) % NX for i in range(K)}
+        tm = time_steps(torch, stream, step, K, W, outs, rows_written, not args.no_graph)
+        stages = stage_profile(lib, stream, torch, step, K, W)
+        # distinct routed experts per step (B > 1 shares experts between tokens)
+        distinct = []
+        with torch.cuda.stream(stream):
+            for i in range(min(K, NX)):
+                if route_ids is None:
+                    step(W + i)
+                    ids, _, _ = moe.last_route(B)
+                else:
+                    ids = ids_h[(W + i) % NX]
+                distinct.append(len(set(ids.ravel().tolist())))
+        mean_distinct = float(np.mean(distinct))
+        lb = layer_bytes(cfg, mean_distinct, B)
+        roof = kernel_roofline(cfg, synth, stages, K, B, mean_distinct, lb, "%s_b%d" % (args.layout, B))
+        return {"B": B, "routing": routing, "timing": tm, "stages": stages, "mean_distinct": mean_distinct, "lb": lb, "roofline": roof, "rel": rel,
+                "ids_ok": ids_ok, "xs": xs, "xs_host": xs_host}
+
+    head = run_workload(B, args.routing)
+    tm, stages, lb, mean_distinct = head["timing"], head["stages"], head["lb"], head["mean_distinct"]
+    ms_per_step = tm["ms"]
+    xs, xs_host = head["xs"], head["xs_host"]
+    n_stage = lib.redhip_profile_stage_count()
+    if args.calibrate:         # yardstick for FETCH_SIZE / WRITE_SIZE: copies of exactly CAL_BYTES in, CAL_BYTES out
+        cal_src = torch.empty(CAL_BYTES, dtype=torch.uint8, device="cuda").random_(0, 256)
+        cal_dst = torch.empty_like(cal_src)
+        for _ in range(4):
+            assert lib.redhip_calibration_copy(cal_dst.data_ptr(), cal_src.data_ptr(), CAL_BYTES, None)
+        torch.cuda.synchronize()
 
     us_per_token = ms_per_step * 1e3 / B
     total_bytes = lb["expert_bytes"] + lb["router_bytes"] + lb["gate_inp_bytes"] + lb["act_bytes"]
     result = {
         "metric": "moe_ffn_layer_us_per_token", "value": round(us_per_token, 3), "unit": "us/token", "n_gpus": 1,
-        "steps": K, "warmup": W, "ms_per_step": round(ms_per_step, 6), "launch_mode": launch_mode,
-        "eager_ms_per_step": round(eager_ms_per_step, 6),
-        "graph_ms_per_step": None if graph_ms_per_step is None else round(graph_ms_per_step, 6), "higher_is_better": False, "scaling": "weak",
+        "steps": K, "warmup": W, "ms_per_step": round(ms_per_step, 6), "launch_mode": tm["mode"],
+        "eager_ms_per_step": round(tm["eager_ms"], 6),
+        "graph_ms_per_step": None if tm["graph_ms"] is None else round(tm["graph_ms"], 6),
+        "graph_replays_timed": tm["replays_timed"], "clock_priming_steps": args.prime,
+        "higher_is_better": False, "scaling": "weak",
         "vs_baseline": None, "dtype": "f32", "data": "synthetic",
         "config": {"workload": "%s: one MoE FFN layer, B=%d decode token(s), hidden 2048, 512 experts top-10 + shared, ffn 512, layout %s, "
                                "all experts of %d layers resident" % ({"iq2": "config1", "f2": "config2"}.get(args.layout, "target-file expert format"),
@@ -336,9 +337,48 @@ def main():
                        "layer_gbps": round(total_bytes / (ms_per_step * 1e-3) / 1e9, 1),
                        "frac_of_peak_on_expert_bytes": round(lb["expert_bytes"] / (ms_per_step * 1e-3) / 1e9 / HBM_PEAK_GBS, 4)},
         "stages_us": {k: round(v["us_avg"] * v["launches"] / K, 3) for k, v in stages.items()},
-        "parity": {"rel_l2_vs_cpu_oracle": rel, "router_ids_identical": ids_ok},
-        "roofline": roofline,
+        "parity": {"rel_l2_vs_cpu_oracle": head["rel"], "router_ids_identical": head["ids_ok"]},
+        "roofline": head["roofline"],
     }
+
+    # ---- what the launches alone cost on this machine: the same number of dependent launches per step with the same grids, empty kernels ----
+    if B == 1 and not args.no_graph:
+        shapes = [(129, 256), (176, 1024), (256, 1024)]
+        with torch.cuda.stream(stream):
+            for g_, b_ in shapes:
+                assert lib.redhip_calibration_empty(g_, b_, stream.cuda_stream)
+            stream.synchronize()
+            gf = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(gf, stream=stream):
+                for _ in range(K):
+                    for g_, b_ in shapes:
+                        lib.redhip_calibration_empty(g_, b_, stream.cuda_stream)
+        ts = []
+        for r in range(12):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            gf.replay()
+            torch.cuda.synchronize()
+            ts.append((time.perf_counter() - t0) * 1e6 / K)
+        ts = sorted(ts[2:])
+        result["launch_floor_us"] = round(ts[len(ts) // 2], 3)
+        result["launch_floor_note"] = "three dependent launches of empty kernels per step (grids of %s), %d steps per graph replay, median of %d replays" % (
+            " / ".join("%dx%d" % sh for sh in shapes), K, len(ts))
+
+    # ---- the ragged small-batch configuration on the same resident handle: B = 2, 4, 8, drawn logits with 32 hot experts ----
+    if sweep:
+        result["batch_sweep"] = []
+        for b in sweep:
+            r = run_workload(b, "hot")
+            t = r["timing"]
+            rf = r["roofline"] or {}
+            result["batch_sweep"].append({
+                "batch": b, "routing": "hot", "us_per_step": round(t["ms"] * 1e3, 3), "us_per_token": round(t["ms"] * 1e3 / b, 3), "launch_mode": t["mode"],
+                "eager_us_per_step": round(t["eager_ms"] * 1e3, 3), "mean_distinct_routed_experts": r["mean_distinct"],
+                "stages_us": {k: round(v["us_avg"] * v["launches"] / K, 3) for k, v in r["stages"].items()},
+                "dominant_kernel": rf.get("kernel"), "kernel_us": rf.get("launch_us"), "kernel_gbps": rf.get("achieved"), "kernel_frac_of_peak": rf.get("frac"),
+                "expert_bytes": int(r["lb"]["expert_bytes"]), "rel_l2_vs_cpu_oracle": r["rel"]})
+            del r
 
     # ---- per-kernel microbench of config 1: one IQ2_XXS dequant-GEMV [512 x 2048] x [2048] on raw GGUF rows ----
     if args.layout == "iq2" and B == 1 and not args.no_micro:

@@ -73,6 +73,7 @@ ABI = {
     "redhip_profile_begin": (i32, []),
     "redhip_profile_end": (i32, [C.POINTER(dbl), C.POINTER(u32), u32]),
     "redhip_calibration_copy": (i32, [vp, vp, u64, vp]),
+    "redhip_calibration_empty": (i32, [u32, u32, vp]),
 }
 
 _lib = None

@@ -1,28 +1,56 @@
 """Builds libredmetal_hip.so (gfx950) in-tree with hipcc. Run on the CPU-only build machine; the GPU box loads the
-prebuilt library."""
+prebuilt library. Every source is compiled to an object of its own (in parallel), then linked."""
 import os
 import subprocess
+import sys
+from concurrent.futures import ThreadPoolExecutor
 
 HERE = os.path.dirname(os.path.abspath(__file__))
 CSRC = os.path.join(HERE, "csrc")
+OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libredmetal_hip.so")
-SOURCES = ["redhip_kernels.hip", "redhip_fused.hip", "redhip_prefill.hip", "redhip_pool_abi.hip", "redhip_moe_abi.hip", "redhip_gguf.hip", "redhip_profile.hip"]
+SOURCES = ["redhip_kernels.hip", "redhip_fused.hip", "redhip_prefill.hip", "redhip_pool_abi.hip", "redhip_moe_abi.hip",
+           "redhip_gguf.hip", "redhip_profile.hip"]
 # -packed-fp32-ops off: v_pk_*_f32 forms are not used on this pool of machines
-FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-shared", "-std=c++17",
+FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-Wextra", "-Wno-unused-parameter"]
 
 
-def build_library(verbose=False):
-    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    cmd = [hipcc] + FLAGS + ["-o", LIB] + [os.path.join(CSRC, s) for s in SOURCES]
+def _run(cmd):
     res = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     out = "\n".join(l for l in res.stdout.splitlines() if "is not a recognized feature for this target" not in l)
     if res.returncode != 0:
-        raise RuntimeError("hipcc failed:\n" + out)
-    if verbose and out.strip():
-        print(out)
+        raise RuntimeError("hipcc failed: %s\n%s" % (" ".join(cmd[-3:]), out))
+    return out
+
+
+def _stale(obj, src, deps):
+    if not os.path.exists(obj):
+        return True
+    t = os.path.getmtime(obj)
+    return any(os.path.getmtime(d) > t for d in [src] + deps)
+
+
+def build_library(verbose=False, incremental=False):
+    """incremental: recompile only the sources that changed (or whose headers did) since their object was built"""
+    hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    os.makedirs(OBJ, exist_ok=True)
+    headers = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")]
+    headers += [os.path.join(HERE, "..", "include", f) for f in os.listdir(os.path.join(HERE, "..", "include")) if f.endswith(".h")]
+    jobs = []
+    for s in SOURCES:
+        src, obj = os.path.join(CSRC, s), os.path.join(OBJ, s[:-4] + ".o")
+        if not incremental or _stale(obj, src, headers):
+            jobs.append([hipcc] + FLAGS + ["-c", "-o", obj, src])
+    with ThreadPoolExecutor(max(1, min(8, len(jobs) or 1))) as ex:
+        outs = list(ex.map(_run, jobs))
+    outs.append(_run([hipcc, "--offload-arch=gfx950", "-shared", "-fPIC", "-o", LIB] + [os.path.join(OBJ, s[:-4] + ".o") for s in SOURCES]))
+    if verbose:
+        text = "\n".join(o for o in outs if o.strip())
+        if text:
+            print(text)
     return LIB
 
 
 if __name__ == "__main__":
-    print(build_library(verbose=True))
+    print(build_library(verbose=True, incremental="--incremental" in sys.argv))

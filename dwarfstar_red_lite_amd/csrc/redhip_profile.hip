@@ -56,6 +56,8 @@ namespace redhip {
 __global__ __launch_bounds__(256) void calibration_copy_kernel(uint4 *dst, const uint4 *src, uint64_t n16) {
     for (uint64_t i = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x; i < n16; i += (uint64_t)gridDim.x * blockDim.x) dst[i] = src[i];
 }
+// nothing at all: what a launch of a given grid costs by itself
+__global__ void calibration_empty_kernel(int) {}
 }  // namespace redhip
 
 extern "C" {
@@ -98,6 +100,13 @@ int redhip_calibration_copy(void *dst_dev, const void *src_dev, uint64_t bytes, 
     redhip::prof_set_stage(redhip::ST_OTHER);
     REDHIP_LAUNCH(redhip::calibration_copy_kernel, dim3(2048), dim3(256), 0, static_cast<hipStream_t>(stream), static_cast<uint4 *>(dst_dev),
                   static_cast<const uint4 *>(src_dev), bytes / 16u);
+    return hipGetLastError() == hipSuccess;
+}
+
+int redhip_calibration_empty(uint32_t grid, uint32_t block, void *stream) {
+    if (!grid || !block || block > 1024u) return 0;
+    redhip::prof_set_stage(redhip::ST_OTHER);
+    REDHIP_LAUNCH(redhip::calibration_empty_kernel, dim3(grid), dim3(block), 0, static_cast<hipStream_t>(stream), 0);
     return hipGetLastError() == hipSuccess;
 }
 

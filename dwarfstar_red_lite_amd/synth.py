@@ -101,3 +101,45 @@ def zipf_topk(rng, ntok, n_expert, top_k, s=1.1):
     for t in range(ntok):
         ids[t] = perm[rng.choice(n_expert, size=top_k, replace=False, p=p)]
     return ids
+
+
+def make_layer_gpu(torch, gen, cfg):
+    """The same construction as make_layer with torch's generator on the GPU (dict of CUDA tensors): random-valid blocks,
+    d drawn from the format's range. For resident stacks too large to draw on the host in reasonable time."""
+    def rows(t, nrows, ncols, d_range=None):
+        bb = BLOCK_BYTES[t]
+        nb = nrows * (ncols // 256)
+        raw = torch.randint(0, 256, (nb, bb), dtype=torch.uint8, device="cuda", generator=gen)
+        lo, hi = d_range or D_RANGE[t]
+        d = (lo + (hi - lo) * torch.rand(nb, device="cuda", generator=gen)).to(torch.float16).view(torch.uint8).reshape(nb, 2)
+        if t == TYPE_IQ1_M:          # d sits in the top nibbles of the four 16-bit scale words (bytes 48..55)
+            for i in range(4):
+                nib = (d[:, i // 2] >> (4 * (i % 2))) & 15
+                raw[:, 49 + 2 * i] = (raw[:, 49 + 2 * i] & 0x0F) | (nib << 4)
+        else:
+            off = D_OFFSET[t]
+            raw[:, off:off + 2] = d
+        return raw.reshape(nrows, -1)
+
+    H, F, E = cfg["hidden"], cfg["ffn"], cfg["n_expert"]
+    a = {}
+    if cfg["router_type"] == TYPE_F32:
+        a["router"] = 0.02 * torch.randn((E, H), device="cuda", generator=gen)
+    else:
+        a["router"] = rows(cfg["router_type"], E, H, d_range=(1e-5, 3e-5))
+    a["gate"] = rows(cfg["gate_up_type"], E * F, H).reshape(E, -1)
+    a["up"] = rows(cfg["gate_up_type"], E * F, H).reshape(E, -1)
+    a["down"] = rows(cfg["down_type"], E * H, F).reshape(E, -1)
+    a["sh_gate"] = rows(cfg["sh_gate_up_type"], F, H)
+    a["sh_up"] = rows(cfg["sh_gate_up_type"], F, H)
+    a["sh_down"] = rows(cfg["sh_down_type"], H, F)
+    a["sh_gate_inp"] = 0.02 * torch.randn(H, device="cuda", generator=gen)
+    return a
+
+
+def layer_to_host(a, cfg):
+    """make_layer_gpu's tensors as the numpy arrays make_layer returns"""
+    out = {k: v.cpu().numpy() for k, v in a.items()}
+    if cfg["router_type"] != TYPE_F32:
+        out["router"] = out["router"].view(np.uint8)
+    return out

@@ -127,6 +127,9 @@ int redhip_profile_end(double *stage_ms, uint32_t *stage_launches, uint32_t n_st
  * `bytes` bytes (a multiple of 16), reading and writing exactly that much. Memory-traffic counters collected for
  * the kernels above are scaled by what they read for this kernel of known size. */
 int redhip_calibration_copy(void *dst_dev, const void *src_dev, uint64_t bytes, void *stream);
+/* Launch-cost calibration (no counterpart in the reference): one launch of `grid` workgroups of `block` lanes of a kernel that does
+ * nothing. A chain of such launches with a path's grids is the time the path's dependent launches cost before any work. */
+int redhip_calibration_empty(uint32_t grid, uint32_t block, void *stream);
 
 #ifdef __cplusplus
 }
