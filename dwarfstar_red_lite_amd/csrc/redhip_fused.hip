@@ -294,8 +294,8 @@ __device__ __forceinline__ void group_small(const GroupJob &g, uint32_t *lds, Pa
     const uint32_t P = g.ntok * K, pr = tid;             // pair index (waves 0 and 1)
     const bool live = pr < P;
     const uint32_t t = live ? pr / K : 0u;
-    const uint32_t e = live ? pair_id(t, pr % K) : 0u;
-    if (live) atomicOr(&token_set[e], 1u << t);
+    const uint32_t e = live ? guarded_id(pair_id(t, pr % K), g.n_expert, g.status) : 0u;
+    if (live && (atomicOr(&token_set[e], 1u << t) & (1u << t)) && g.status) atomicOr(g.status, 2u);      // the token names this expert twice
     __syncthreads();
     const uint32_t set = live ? token_set[e] : 0u;
     const uint32_t n = (uint32_t)__popc(set), before = (uint32_t)__popc(set & ((1u << t) - 1u));
@@ -1045,6 +1045,7 @@ struct GateUpArgs {
     _Float16 *act_h, *act_l;   // [top_k + 1][ffn]
     int *act_exp;              // [top_k + 1][ffn / 32]
     uint32_t hidden, ffn, n_expert, top_k;
+    uint32_t *status;          // RouteGuard::status when ids_in is the caller's
 };
 
 // FMT: format of the routed (and a packed shared) expert's gate / up matrices: 0 IQ2_XXS, 1 IQ2_XS, 2 IQ1_M
@@ -1119,7 +1120,7 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_select_kernel(GateUpArgs a
             if (tid == 0u) a.scalar_out[0] = sel.scalar;
         }
     } else {
-        expert = a.ids_in[slot];
+        expert = guarded_id(a.ids_in[slot], a.n_expert, a.status);
         __syncthreads();                               // tables
     }
     if (is_shared && !a.shared && a.shared_gu) {           // the router launch has already multiplied the shared expert's rows
@@ -1226,6 +1227,7 @@ struct DownArgs {
     float *out;                // [hidden]
     uint32_t hidden, ffn, top_k;
     const float *resid_a, *resid_b;     // when set: out[i] = (resid_a[i] + resid_b[i]) + layer output
+    uint32_t id_limit;                  // ids are clamped to id_limit - 1 (RouteGuard)
 };
 
 // 8 output rows per workgroup; wave s (< top_k + 1) owns slot s: both row quads of the workgroup against all
@@ -1244,7 +1246,7 @@ __global__ __launch_bounds__(kWaves * 64) void down_combine_kernel(DownArgs a) {
     const bool active = wave < n_slot;
     const uint8_t *ex = nullptr;
     if (active) {
-        ex = wave < a.top_k ? a.experts + (uint64_t)a.ids[wave] * a.stride : a.shared;
+        ex = wave < a.top_k ? a.experts + (uint64_t)guarded_id(a.ids[wave], a.id_limit, nullptr) * a.stride : a.shared;
         const uint64_t gate_bytes = (uint64_t)F * (H / 32u) * 8u + (uint64_t)F * (H / 256u) * 2u;
         const uint2 *qs = reinterpret_cast<const uint2 *>(ex + 2u * gate_bytes);                         // [hidden][FG]
         const uint16_t *ds = reinterpret_cast<const uint16_t *>(ex + 2u * gate_bytes + (uint64_t)H * FG * 8u);   // [hidden][FB]
@@ -1370,6 +1372,7 @@ struct DownRawArgs {
     const float *resid_a, *resid_b;
     const int8_t *grid;        // the caller's codebook of the routed down format (IQ2_XS, IQ1_M) or nullptr
     const float *shared_dense; // when set: the shared expert's down matrix as dense f32 [hidden][ffn], read instead of `shared`
+    uint32_t id_limit;         // ids are clamped to id_limit - 1 (RouteGuard)
 };
 
 template <uint32_t T>
@@ -1420,7 +1423,7 @@ __global__ __launch_bounds__(NW * 64) void down_combine_raw_kernel(DownRawArgs a
     const uint32_t n_raw = a.shared_dense ? a.top_k : n_slot;      // slots decoded from staged raw rows
     if (a.shared_dense && wave >= a.top_k) shared_rows_dense<NW>(a.shared_dense, row0, F, a.top_k, a.act_h, a.act_l, a.act_exp, wave, lane, part);
     if (wave < n_raw) {
-        const uint8_t *rows = (is_shared ? a.shared : a.experts + (uint64_t)a.ids[wave] * a.stride) + (uint64_t)row0 * row_bytes;
+        const uint8_t *rows = (is_shared ? a.shared : a.experts + (uint64_t)guarded_id(a.ids[wave], a.id_limit, nullptr) * a.stride) + (uint64_t)row0 * row_bytes;
         wave_stage(mine, rows, 8u * row_bytes, lane);          // 8 rows x FB blocks of 56 .. 210 bytes: a multiple of 16
     }
     if constexpr (kGridBytes != 0u) {
@@ -1485,7 +1488,7 @@ hipError_t launch_down_combine_raw(uint32_t down_type, uint32_t shared_down_type
     if ((down_type == T_IQ2_XS || down_type == T_IQ1_M) && !grid) return hipErrorInvalidValue;
     const DownRawArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(shared), ids, weights, scalar,
                         static_cast<const _Float16 *>(act_h), static_cast<const _Float16 *>(act_l), act_exp, out, hidden, ffn, top_k,
-                        block_context().resid_a, block_context().resid_b, grid, shared_dense};
+                        block_context().resid_a, block_context().resid_b, grid, shared_dense, route_guard().id_limit};
     switch (down_type) {
         case T_IQ2_XXS: return launch_down_raw_shared<T_IQ2_XXS>(shared_down_type, a, ntok, s);
         case T_IQ3_S: return launch_down_raw_shared<T_IQ3_S>(shared_down_type, a, ntok, s);
@@ -1610,6 +1613,7 @@ struct DownWordsArgs {
     float *out;
     uint32_t hidden, ffn, top_k;
     const float *resid_a, *resid_b;
+    uint32_t id_limit;         // ids are clamped to id_limit - 1 (RouteGuard)
 };
 
 template <int NW, int FMT>       // FMT: 0 word-packed IQ3_S, 1 stream-packed IQ2_XS, 2 stream-packed IQ1_M
@@ -1637,7 +1641,7 @@ __global__ __launch_bounds__(NW * 64) void down_combine_words_kernel(DownWordsAr
     float sc[2] = {0.0f, 0.0f};
     const bool routed = wave < a.top_k;
     if (routed) {
-        const uint8_t *ex = a.experts + (uint64_t)a.ids[wave] * a.stride;
+        const uint8_t *ex = a.experts + (uint64_t)guarded_id(a.ids[wave], a.id_limit, nullptr) * a.stride;
         constexpr uint32_t kGroupBytes = FMT == 0 ? 16u : 8u;
         const uint16_t *ds = reinterpret_cast<const uint16_t *>(ex + (uint64_t)a.hidden * FG * kGroupBytes);      // [hidden][FB]
         const uint8_t *scs = ex + (uint64_t)a.hidden * FG * kGroupBytes + (uint64_t)a.hidden * FB * 2u;           // IQ2_XS: [hidden][FG]
@@ -1703,7 +1707,7 @@ hipError_t launch_down_combine_words(uint32_t down_type, const int8_t *grid, con
     if (!hidden || hidden % 8u || !ffn || ffn % 256u || ffn > 1024u || top_k + 1u > (uint32_t)kWaves || !ntok || ntok > 65535u || !shared_dense) return hipErrorInvalidValue;
     if ((down_type == T_IQ2_XS || down_type == T_IQ1_M) && !grid) return hipErrorInvalidValue;
     const DownWordsArgs a{static_cast<const uint8_t *>(experts), stride, grid, shared_dense, ids, weights, scalar, static_cast<const _Float16 *>(act_h),
-                          static_cast<const _Float16 *>(act_l), act_exp, out, hidden, ffn, top_k, block_context().resid_a, block_context().resid_b};
+                          static_cast<const _Float16 *>(act_l), act_exp, out, hidden, ffn, top_k, block_context().resid_a, block_context().resid_b, route_guard().id_limit};
     const dim3 grid_dim(hidden / 8u, ntok);
     const bool narrow = top_k + 1u <= 12u;
 #define REDHIP_DCW(FMT)                                                                                              \
@@ -2540,7 +2544,7 @@ hipError_t launch_gateup_select(const void *experts, uint64_t stride, const void
     if ((gate_up_type != T_IQ2_XXS && !codebook) || (codebook && (!grid || shared))) return hipErrorInvalidValue;
     GateUpArgs a{static_cast<const uint8_t *>(experts), stride, grid, static_cast<const uint8_t *>(shared), static_cast<const uint8_t *>(shared_q6k), x,
                  shared_gu, logits, ids_in, ids_out, weights_out, scalar_out, static_cast<const _Float16 *>(xh), static_cast<const _Float16 *>(xl),
-                 xexp, static_cast<_Float16 *>(act_h), static_cast<_Float16 *>(act_l), act_exp, hidden, ffn, n_expert, top_k};
+                 xexp, static_cast<_Float16 *>(act_h), static_cast<_Float16 *>(act_l), act_exp, hidden, ffn, n_expert, top_k, route_guard().status};
     const dim3 grid_dim(ffn / 32u, top_k + 1u, ntok);
     const size_t dyn = shared || shared_gu ? 0u : (size_t)64u * (hidden / 256u) * 210u + (size_t)(hidden + hidden / 32u + hidden / 16u) * 4u;   // raw Q6_K rows of one unit of the shared expert, x, sums of 16 x
     const size_t dyn_max = gate_up_type == T_IQ1_M ? 120u * 1024u : 144u * 1024u;      // beside the static decode table (32 KB for IQ1_M)
@@ -2579,7 +2583,7 @@ hipError_t launch_down_combine(const void *experts, uint64_t stride, const void 
     if (!fused_iq2_supported(hidden, ffn) || top_k + 1u > (uint32_t)kWaves) return hipErrorInvalidValue;
     DownArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(shared), ids, weights, scalar,
                static_cast<const _Float16 *>(act_h), static_cast<const _Float16 *>(act_l), act_exp, out, hidden, ffn, top_k,
-               block_context().resid_a, block_context().resid_b};
+               block_context().resid_a, block_context().resid_b, route_guard().id_limit};
     REDHIP_LAUNCH(down_combine_kernel, dim3(hidden / 8u), dim3(kWaves * 64), 0, s, a);
     return hipGetLastError();
 }

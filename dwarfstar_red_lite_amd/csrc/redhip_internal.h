@@ -5,7 +5,11 @@
 #include <stddef.h>
 #include <stdint.h>
 
+#include <mutex>
+
 namespace redhip {
+
+std::mutex &caller_grid_mutex();      // serialises uploads of the caller-supplied codebooks (and one-shot launches that must see their own)
 
 enum : uint32_t { T_F32 = 0u, T_Q6_K = 14u, T_IQ2_XXS = 16u, T_IQ2_XS = 17u, T_IQ3_S = 21u, T_IQ1_M = 29u };
 
@@ -20,10 +24,14 @@ inline uint64_t pool_row_bytes(uint32_t t, uint32_t ncols) {
 }
 inline bool pool_quant_supported(uint32_t t) { return pool_block_bytes(t) != 0u; }
 // device copies of the caller's IQ2_XS (512 x 8) / IQ1_M (2048 x 8) int8 codebooks; either may be null (left as is).
-// One copy per process: `owner` (a pool) makes a repeated call by the same owner free, so each pool can ask for its own
-// tables before every launch; callers whose tables differ must not run at the same time
-hipError_t set_caller_grids(const int8_t *iq2_xs, const int8_t *iq1_m, const void *owner = nullptr);
+// One pair per process. `bind_owner` (a pool, a resident-layer handle) binds itself to the content it uploads; while anybody is bound an
+// upload of different content returns hipErrorContextAlreadyInUse (report it with kCodebookConflict) instead of changing what the bound
+// users decode through; the same content again is free. forget_caller_grids unbinds.
+hipError_t set_caller_grids(const int8_t *iq2_xs, const int8_t *iq1_m, const void *bind_owner = nullptr);
+hipError_t set_caller_grids_locked(const int8_t *iq2_xs, const int8_t *iq1_m, const void *bind_owner = nullptr);      // caller holds caller_grid_mutex()
+bool caller_grids_bound(const void *owner);
 void forget_caller_grids(const void *owner);
+constexpr const char *kCodebookConflict = "IQ2_XS / IQ1_M codebooks differ from the ones this process holds while pools or resident layers that decode through them are alive";
 const int8_t *caller_grid_device(uint32_t type);      // device address of the process's codebook of IQ2_XS / IQ1_M, nullptr for other types
 bool caller_grid_present(uint32_t type);       // true for the formats that carry their own tables
 inline uint64_t row_bytes(uint32_t t, uint32_t ncols) {
@@ -57,6 +65,23 @@ struct BlockContext {
     const float *resid_a = nullptr, *resid_b = nullptr;   // output side
 };
 BlockContext &block_context();
+
+// Routing that a caller hands in (redhip_moe_experts, redhip_moe_group) is untrusted: every kernel that turns an expert id into an
+// address clamps it to id_limit - 1 first and, when it had to, sets bit 0 of *status; the pair sort sets bit 1 when a token names an
+// expert twice (its bitmap ranks assume distinct ids per token). Context of the calling thread, picked up by the launchers; the default
+// clamps nothing and reports nowhere (ids the library selected itself).
+struct RouteGuard {
+    uint32_t id_limit = 0xffffffffu;      // n_expert
+    uint32_t *status = nullptr;           // device word
+};
+RouteGuard &route_guard();
+#if defined(__HIPCC__)
+__device__ __forceinline__ uint32_t guarded_id(uint32_t id, uint32_t id_limit, uint32_t *status) {
+    if (id < id_limit) return id;
+    if (status) atomicOr(status, 1u);
+    return id_limit - 1u;
+}
+#endif
 void prof_events(hipEvent_t *start, hipEvent_t *stop);     // both nullptr when profiling is off
 
 #define REDHIP_LAUNCH(kern, grid, block, lds, stream, ...)                                         \
@@ -190,6 +215,7 @@ struct GroupJob {
     uint32_t *uid, *expert_start, *pair_token;
     float *pair_weight;
     uint32_t *tok_pair, *n_unique;
+    uint32_t *status = nullptr;      // RouteGuard::status of the call (ids are clamped to n_expert - 1 either way)
 };
 
 // Selection inside the batched gate/up kernel: logits [ntok][n_expert + 1] in, the routing out (ids, weights [ntok][top_k], scalar [ntok]);

@@ -4,7 +4,10 @@
 // partial sums meet in a butterfly of cross-lane shuffles.
 #include "redhip_decode.h"
 
+#include <string.h>
+
 #include <mutex>
+#include <vector>
 
 namespace redhip {
 
@@ -22,33 +25,60 @@ static inline uint32_t padded_floats(uint32_t n) { return n + (n >> 5); }
 // ---------------------------------------------------------------- IQ2_XS / IQ1_M (caller-supplied codebooks)
 
 // The reference hands these codebooks to its kernels as arguments (native/redmetal_ffn.m:223-227); here they live in
-// device memory of this translation unit, uploaded by the pool / one-shot surfaces before they launch.
+// device memory of this translation unit, uploaded by the pool / one-shot / resident-layer surfaces.
 __device__ __attribute__((aligned(16))) int8_t g_iq2xs_grid[512 * 8];
 __device__ __attribute__((aligned(16))) int8_t g_iq1m_grid[2048 * 8];
 
+// One pair of tables per process. Pools and resident layers that decode through them bind to their content; while any is bound,
+// an upload of different content is refused (the bound users would silently decode through the wrong tables), an upload of the same
+// content is free. With nobody bound an upload replaces the tables.
 static std::mutex g_grid_mu;
-static const void *g_grid_owner = nullptr;      // whose tables the device holds; nullptr: nobody's in particular
-static bool g_grid_have[2] = {false, false};    // IQ2_XS, IQ1_M uploaded at least once
+static std::vector<int8_t> g_grid_host[2];      // what the device holds: IQ2_XS, IQ1_M (empty: never uploaded)
+static std::vector<const void *> g_grid_bound;  // the owners bound to that content
+
+std::mutex &caller_grid_mutex() { return g_grid_mu; }
 
 bool caller_grid_present(uint32_t type) {
     std::lock_guard<std::mutex> lk(g_grid_mu);
-    return type == T_IQ2_XS ? g_grid_have[0] : type == T_IQ1_M ? g_grid_have[1] : true;
+    return type == T_IQ2_XS ? !g_grid_host[0].empty() : type == T_IQ1_M ? !g_grid_host[1].empty() : true;
 }
 
-hipError_t set_caller_grids(const int8_t *iq2_xs, const int8_t *iq1_m, const void *owner) {
-    std::lock_guard<std::mutex> lk(g_grid_mu);
-    if (owner && owner == g_grid_owner) return hipSuccess;
+static bool grid_is_bound(const void *owner) {
+    for (const void *o : g_grid_bound) if (o == owner) return true;
+    return false;
+}
+
+hipError_t set_caller_grids_locked(const int8_t *iq2_xs, const int8_t *iq1_m, const void *bind_owner) {
+    if (bind_owner && grid_is_bound(bind_owner)) return hipSuccess;
+    const int8_t *src[2] = {iq2_xs, iq1_m};
+    const size_t n[2] = {sizeof(g_iq2xs_grid), sizeof(g_iq1m_grid)};
+    bool differs[2] = {false, false};
+    for (int k = 0; k < 2; ++k)
+        differs[k] = src[k] && (g_grid_host[k].size() != n[k] || memcmp(g_grid_host[k].data(), src[k], n[k]) != 0);
+    if ((differs[0] || differs[1]) && !g_grid_bound.empty()) return hipErrorContextAlreadyInUse;      // see caller_grid_conflict()
     hipError_t e = hipSuccess;
-    if (iq2_xs) e = hipMemcpyToSymbol(HIP_SYMBOL(g_iq2xs_grid), iq2_xs, sizeof(g_iq2xs_grid));
-    if (e == hipSuccess && iq1_m) e = hipMemcpyToSymbol(HIP_SYMBOL(g_iq1m_grid), iq1_m, sizeof(g_iq1m_grid));
-    g_grid_owner = e == hipSuccess ? owner : nullptr;
-    if (e == hipSuccess) { g_grid_have[0] |= iq2_xs != nullptr; g_grid_have[1] |= iq1_m != nullptr; }
+    if (differs[0]) e = hipMemcpyToSymbol(HIP_SYMBOL(g_iq2xs_grid), iq2_xs, n[0]);
+    if (e == hipSuccess && differs[0]) g_grid_host[0].assign(iq2_xs, iq2_xs + n[0]);
+    if (e == hipSuccess && differs[1]) e = hipMemcpyToSymbol(HIP_SYMBOL(g_iq1m_grid), iq1_m, n[1]);
+    if (e == hipSuccess && differs[1]) g_grid_host[1].assign(iq1_m, iq1_m + n[1]);
+    if (e == hipSuccess && bind_owner) g_grid_bound.push_back(bind_owner);
     return e;
+}
+
+hipError_t set_caller_grids(const int8_t *iq2_xs, const int8_t *iq1_m, const void *bind_owner) {
+    std::lock_guard<std::mutex> lk(g_grid_mu);
+    return set_caller_grids_locked(iq2_xs, iq1_m, bind_owner);
+}
+
+bool caller_grids_bound(const void *owner) {
+    std::lock_guard<std::mutex> lk(g_grid_mu);
+    return grid_is_bound(owner);
 }
 
 void forget_caller_grids(const void *owner) {
     std::lock_guard<std::mutex> lk(g_grid_mu);
-    if (g_grid_owner == owner) g_grid_owner = nullptr;
+    for (size_t i = 0; i < g_grid_bound.size(); ++i)
+        if (g_grid_bound[i] == owner) { g_grid_bound.erase(g_grid_bound.begin() + (long)i); break; }
 }
 
 template <> __device__ __forceinline__ void decode32<T_IQ2_XS>(const uint8_t *row, uint32_t chunk, float *w) { decode32_cb<T_IQ2_XS>(row, chunk, w, g_iq2xs_grid); }
@@ -294,11 +324,11 @@ hipError_t launch_route_select(const float *logits, uint32_t ntok, uint32_t n_ex
 template <uint32_t T, int LPR>
 __global__ __launch_bounds__(256) void moe_gateup_kernel(const uint8_t *base, uint64_t stride, uint64_t gate_bytes,
                                                          const uint32_t *ids, uint32_t hidden, uint32_t ffn,
-                                                         const float *x, float *act) {
+                                                         const float *x, float *act, uint32_t id_limit, uint32_t *status) {
     extern __shared__ float xs[];
     for (uint32_t i = threadIdx.x; i < hidden; i += 256u) xs[pad32(i)] = x[i];
     __syncthreads();
-    const uint32_t slot = blockIdx.y, e = ids ? ids[slot] : slot;
+    const uint32_t slot = blockIdx.y, e = ids ? guarded_id(ids[slot], id_limit, status) : slot;
     const uint32_t sub = threadIdx.x % LPR, r = blockIdx.x * (256u / LPR) + threadIdx.x / LPR;
     const uint64_t rb = (uint64_t)(hidden / 256u) * Fmt<T>::kBlock;
     float g = 0.0f, u = 0.0f;
@@ -322,10 +352,10 @@ static hipError_t gateup_dispatch(const ExpertSet &ex, const uint32_t *ids, uint
     const dim3 grid((ffn + 256u / lpr - 1u) / (256u / lpr), n_slot);
     const size_t lds = padded_floats(hidden) * sizeof(float);
     switch (lpr) {
-        case 64: REDHIP_LAUNCH((moe_gateup_kernel<T, 64>), dim3(grid), dim3(256), lds, s, ex.base, ex.stride, ex.gate_bytes, ids, hidden, ffn, x, act); break;
-        case 32: REDHIP_LAUNCH((moe_gateup_kernel<T, 32>), dim3(grid), dim3(256), lds, s, ex.base, ex.stride, ex.gate_bytes, ids, hidden, ffn, x, act); break;
-        case 16: REDHIP_LAUNCH((moe_gateup_kernel<T, 16>), dim3(grid), dim3(256), lds, s, ex.base, ex.stride, ex.gate_bytes, ids, hidden, ffn, x, act); break;
-        default: REDHIP_LAUNCH((moe_gateup_kernel<T, 8>), dim3(grid), dim3(256), lds, s, ex.base, ex.stride, ex.gate_bytes, ids, hidden, ffn, x, act); break;
+        case 64: REDHIP_LAUNCH((moe_gateup_kernel<T, 64>), dim3(grid), dim3(256), lds, s, ex.base, ex.stride, ex.gate_bytes, ids, hidden, ffn, x, act, route_guard().id_limit, route_guard().status); break;
+        case 32: REDHIP_LAUNCH((moe_gateup_kernel<T, 32>), dim3(grid), dim3(256), lds, s, ex.base, ex.stride, ex.gate_bytes, ids, hidden, ffn, x, act, route_guard().id_limit, route_guard().status); break;
+        case 16: REDHIP_LAUNCH((moe_gateup_kernel<T, 16>), dim3(grid), dim3(256), lds, s, ex.base, ex.stride, ex.gate_bytes, ids, hidden, ffn, x, act, route_guard().id_limit, route_guard().status); break;
+        default: REDHIP_LAUNCH((moe_gateup_kernel<T, 8>), dim3(grid), dim3(256), lds, s, ex.base, ex.stride, ex.gate_bytes, ids, hidden, ffn, x, act, route_guard().id_limit, route_guard().status); break;
     }
     return hipGetLastError();
 }
@@ -354,7 +384,7 @@ __global__ __launch_bounds__(256) void moe_down_combine_kernel(const uint8_t *ba
                                                                const uint8_t *sh_down, const float *scalar,
                                                                uint32_t hidden, uint32_t ffn,
                                                                const float *act, const float *sh_act, float *out,
-                                                               const float *resid_a, const float *resid_b) {
+                                                               const float *resid_a, const float *resid_b, uint32_t id_limit) {
     extern __shared__ float as[];                          // [top_k + 1][padded ffn], then [4][64 / LPR] partial sums
     constexpr uint32_t kRows = 64u / LPR;
     const uint32_t fp = ffn + (ffn >> 5);
@@ -373,7 +403,7 @@ __global__ __launch_bounds__(256) void moe_down_combine_kernel(const uint8_t *ba
         float part = 0.0f;
         if (r < hidden) {
             if (k < top_k) {
-                const uint8_t *row = base + (uint64_t)ids[k] * stride + down_off + (uint64_t)r * rbd;
+                const uint8_t *row = base + (uint64_t)guarded_id(ids[k], id_limit, nullptr) * stride + down_off + (uint64_t)r * rbd;
                 for (uint32_t c = sub; c < ffn / 32u; c += LPR) part += chunk_dot<TD>(row, c, as + k * fp + 33u * c);
             } else {
                 const uint8_t *row = sh_down + (uint64_t)r * rbs;
@@ -400,7 +430,7 @@ static hipError_t down_dispatch(const ExpertSet &ex, const uint32_t *ids, const 
     const size_t lds = ((size_t)(top_k + 1u) * padded_floats(ffn) + 4u * (64u / lpr)) * sizeof(float);
     const uint8_t *shd = sh.base ? sh.base + sh.gate_bytes + sh.up_bytes : nullptr;
     const uint64_t off = ex.gate_bytes + ex.up_bytes;
-#define REDHIP_DOWN(L) REDHIP_LAUNCH((moe_down_combine_kernel<TD, TS, L>), dim3(grid), dim3(256), lds, s, ex.base, ex.stride, off, ids, weights, top_k, shd, scalar, hidden, ffn, act, sh_act, out, block_context().resid_a, block_context().resid_b)
+#define REDHIP_DOWN(L) REDHIP_LAUNCH((moe_down_combine_kernel<TD, TS, L>), dim3(grid), dim3(256), lds, s, ex.base, ex.stride, off, ids, weights, top_k, shd, scalar, hidden, ffn, act, sh_act, out, block_context().resid_a, block_context().resid_b, route_guard().id_limit)
     switch (lpr) {
         case 64: REDHIP_DOWN(64); break;
         case 32: REDHIP_DOWN(32); break;
@@ -678,7 +708,7 @@ template <bool PREFIX>
 __global__ __launch_bounds__(1024) void group_pairs_kernel(const uint32_t *ids, const float *weights, uint32_t ntok, uint32_t top_k, uint32_t top_k_magic,
                                                            uint32_t n_expert, uint32_t *uid, uint32_t *expert_start,
                                                            uint32_t *pair_token, float *pair_weight, uint32_t *tok_pair,
-                                                           uint32_t *n_unique) {
+                                                           uint32_t *n_unique, uint32_t *status) {
     extern __shared__ uint32_t sm[];
     const uint32_t words = (ntok + 31u) / 32u, P = ntok * top_k, tid = threadIdx.x;
     uint32_t *first = sm;                          // [n_expert]
@@ -690,14 +720,16 @@ __global__ __launch_bounds__(1024) void group_pairs_kernel(const uint32_t *ids, 
     uint32_t *member = wave_tot + 17u;             // [n_expert][words]
     uint32_t *below = member + n_expert * words;   // [n_expert][words] when PREFIX: members in the words before this one
     auto token_of = [&](uint32_t p) { return top_k == 1u ? p : __umulhi(p, top_k_magic); };
+    // the ids are the caller's: clamped into the tables (reported once, in the first pass)
+    auto id_of = [&](uint32_t p) { const uint32_t e = ids[p]; return e < n_expert ? e : n_expert - 1u; };
     for (uint32_t i = tid; i < n_expert; i += 1024u) { first[i] = 0xffffffffu; count[i] = 0u; dense[i] = 0u; }
     for (uint32_t i = tid; i < n_expert * words; i += 1024u) member[i] = 0u;
     __syncthreads();
     for (uint32_t p = tid; p < P; p += 1024u) {
-        const uint32_t e = ids[p], t = token_of(p);
+        const uint32_t e = guarded_id(ids[p], n_expert, status), t = token_of(p);
         atomicMin(&first[e], p);
         if constexpr (!PREFIX) atomicAdd(&count[e], 1u);
-        atomicOr(&member[e * words + (t >> 5)], 1u << (t & 31u));
+        if ((atomicOr(&member[e * words + (t >> 5)], 1u << (t & 31u)) & (1u << (t & 31u))) && status) atomicOr(status, 2u);      // the token names this expert twice
     }
     __syncthreads();
     if constexpr (PREFIX) {
@@ -710,12 +742,12 @@ __global__ __launch_bounds__(1024) void group_pairs_kernel(const uint32_t *ids, 
     // exclusive scan of "pair p is the first appearance of its expert", P elements in per-thread runs
     const uint32_t per = (P + 1023u) / 1024u;
     uint32_t mine = 0u;
-    for (uint32_t j = 0; j < per; ++j) { const uint32_t p = tid * per + j; if (p < P && first[ids[p]] == p) ++mine; }
+    for (uint32_t j = 0; j < per; ++j) { const uint32_t p = tid * per + j; if (p < P && first[id_of(p)] == p) ++mine; }
     uint32_t U = 0u;
     uint32_t run = block_scan_1024(mine, wave_tot, U);
     for (uint32_t j = 0; j < per; ++j) {
         const uint32_t p = tid * per + j;
-        if (p < P && first[ids[p]] == p) { const uint32_t e = ids[p]; dense[e] = run; uid_l[run] = e; uid[run] = e; ++run; }
+        if (p < P && first[id_of(p)] == p) { const uint32_t e = id_of(p); dense[e] = run; uid_l[run] = e; uid[run] = e; ++run; }
     }
     __syncthreads();
     // exclusive scan of the per-expert pair counts in dense order (U <= n_expert <= 1024: one per thread)
@@ -725,7 +757,7 @@ __global__ __launch_bounds__(1024) void group_pairs_kernel(const uint32_t *ids, 
     if (tid == 0u) { start[U] = all; expert_start[U] = all; n_unique[0] = U; }
     __syncthreads();
     for (uint32_t p = tid; p < P; p += 1024u) {
-        const uint32_t e = ids[p], t = token_of(p);
+        const uint32_t e = id_of(p), t = token_of(p);
         const uint32_t *bits = member + e * words;
         uint32_t rank = __popc(bits[t >> 5] & ((1u << (t & 31u)) - 1u));
         if constexpr (PREFIX) rank += below[e * words + (t >> 5)];
@@ -754,9 +786,9 @@ hipError_t launch_group_pairs(const uint32_t *ids, const float *weights, uint32_
         attr_set = true;
     }
     if (lds_prefix <= 160u * 1024u)
-        REDHIP_LAUNCH(group_pairs_kernel<true>, dim3(1), dim3(1024), lds_prefix, s, ids, weights, ntok, top_k, magic, n_expert, uid, expert_start, pair_token, pair_weight, tok_pair, n_unique);
+        REDHIP_LAUNCH(group_pairs_kernel<true>, dim3(1), dim3(1024), lds_prefix, s, ids, weights, ntok, top_k, magic, n_expert, uid, expert_start, pair_token, pair_weight, tok_pair, n_unique, route_guard().status);
     else
-        REDHIP_LAUNCH(group_pairs_kernel<false>, dim3(1), dim3(1024), lds, s, ids, weights, ntok, top_k, magic, n_expert, uid, expert_start, pair_token, pair_weight, tok_pair, n_unique);
+        REDHIP_LAUNCH(group_pairs_kernel<false>, dim3(1), dim3(1024), lds, s, ids, weights, ntok, top_k, magic, n_expert, uid, expert_start, pair_token, pair_weight, tok_pair, n_unique, route_guard().status);
     return hipGetLastError();
 }
 

@@ -57,6 +57,7 @@ struct Moe {
     float *logits = nullptr, *weights = nullptr, *scalar = nullptr, *act = nullptr, *sh_act = nullptr;
     float *xn = nullptr;                     // [max_tokens][hidden]: normalised activations of redhip_moe_forward_block
     uint32_t *ids = nullptr;
+    uint32_t *status = nullptr;              // device word: bit 0 an expert id of the caller's routing was out of range (clamped), bit 1 a token named an expert twice
     uint8_t *ws = nullptr;
     // single-token fused path (all matrices IQ2_XXS, shapes the fused kernel tiles)
     bool fused = false;
@@ -370,18 +371,22 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
     m->sh_down_bytes = (uint64_t)c.hidden * row_bytes(sdn, c.ffn);
     m->router_bytes = (uint64_t)c.n_expert * row_bytes(c.router_type, c.hidden);
     m->layers.resize(c.n_layer);
-    m->fused = gu == T_IQ2_XXS && dn == T_IQ2_XXS && sgu == T_IQ2_XXS && sdn == T_IQ2_XXS && fused_iq2_supported(c.hidden, c.ffn);
+    // the one-token kernels of the packed paths give every slot (top_k routed + the shared expert) a wave of a 16-wave workgroup, and the mixed
+    // ones keep the shared expert's gate | up products in the activation rows of two routed slots: other top_k run on the generic kernels
+    const bool slots_fit = c.top_k + 1u <= 16u;
+    m->fused = gu == T_IQ2_XXS && dn == T_IQ2_XXS && sgu == T_IQ2_XXS && sdn == T_IQ2_XXS && fused_iq2_supported(c.hidden, c.ffn) && slots_fit;
     // (the raw-row down kernel stages 8 rows per slot in LDS: keep that within the default 64 KB)
     // IQ2_XS / IQ1_M gate/up matrices have a packed form of their own (a shared expert beside them is Q6_K; the gate/up kernel keeps
     // their fp16 codebook in LDS next to the staged Q6_K rows: 32 KB for IQ1_M)
     const bool gu_codebook = gu == T_IQ2_XS || gu == T_IQ1_M;
-    m->mixed = !m->fused && (gu == T_IQ2_XXS || gu_codebook) && (sgu == T_Q6_K || (sgu == T_IQ2_XXS && !gu_codebook)) && fused_iq2_supported(c.hidden, c.ffn) &&
+    m->mixed = !m->fused && slots_fit && c.top_k >= 2u && (gu == T_IQ2_XXS || gu_codebook) && (sgu == T_Q6_K || (sgu == T_IQ2_XXS && !gu_codebook)) && fused_iq2_supported(c.hidden, c.ffn) &&
                (size_t)(c.top_k + 1u) * 8u * (c.ffn / 256u) * 210u + (dn == T_IQ1_M ? 17u * 1024u : dn == T_IQ2_XS ? 5u * 1024u : 0u) <= 64u * 1024u &&
                (sgu != T_Q6_K || (size_t)64u * (c.hidden / 256u) * 210u + (size_t)(c.hidden + c.hidden / 32u + c.hidden / 16u) * 4u <= (gu == T_IQ1_M ? 120u : 144u) * 1024u);
     m->pk_gate_bytes = packed_matrix_bytes(gu, c.ffn, c.hidden);
     m->packed_stride = m->fused ? m->expert_stride : align256(2u * m->pk_gate_bytes);
     m->gu_grid = caller_grid_device(gu);
     m->dn_grid = caller_grid_device(dn);
+    if (m->gu_grid || m->dn_grid) (void)set_caller_grids(nullptr, nullptr, m);      // bound to the tables the process holds now: they cannot change under this handle
     bool ok = true;
     for (uint32_t l = 0; l < c.n_layer && ok; ++l) {
         Layer &L = m->layers[l];
@@ -426,7 +431,7 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
         }
     }
     const size_t T = c.max_tokens;
-    const size_t ws_bytes = align256(T * c.hidden * 4u) + align256(T * (c.n_expert + 1u) * 4u) + 2u * align256(T * c.top_k * 4u) + align256(T * 4u) +
+    const size_t ws_bytes = align256(4u) + align256(T * c.hidden * 4u) + align256(T * (c.n_expert + 1u) * 4u) + 2u * align256(T * c.top_k * 4u) + align256(T * 4u) +
                             align256(T * c.top_k * c.ffn * 4u) + align256(T * c.ffn * 4u) +
                             2u * align256(2u * T * c.hidden) + align256(4u * T) + 2u * align256(2u * T * (c.top_k + 1u) * c.ffn) +
                             align256(4u * T * (c.top_k + 1u) * (c.ffn / 32u)) +
@@ -440,6 +445,7 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
         return nullptr;
     }
     uint8_t *w = m->ws;
+    m->status = reinterpret_cast<uint32_t *>(w); w += align256(4u);
     m->xn = reinterpret_cast<float *>(w); w += align256(T * c.hidden * 4u);
     m->logits = reinterpret_cast<float *>(w); w += align256(T * (c.n_expert + 1u) * 4u);
     m->ids = reinterpret_cast<uint32_t *>(w); w += align256(T * c.top_k * 4u);
@@ -492,6 +498,7 @@ void redhip_moe_destroy(redhip_moe_t h) {
     Moe *m = moe_of(h);
     if (!m) return;
     (void)hipDeviceSynchronize();
+    forget_caller_grids(m);
     for (Layer &L : m->layers) {
         if (L.router) (void)hipFree(L.router);
         if (L.experts) (void)hipFree(L.experts);
@@ -676,13 +683,17 @@ int redhip_moe_experts(redhip_moe_t h, uint32_t layer, const float *x_dev, uint3
     if (!x_dev || !ids_dev || !weights_dev || !out_dev || !ntok || ntok > m->cfg.max_tokens) { moe_err("invalid expert execution arguments"); return 0; }
     hipStream_t s = static_cast<hipStream_t>(stream);
     m->shared_gu_ready = false;
+    struct GuardScope {          // the caller's ids are clamped and reported by every kernel that reads them during this call
+        GuardScope(uint32_t n, uint32_t *st) { route_guard() = RouteGuard{n, st}; }
+        ~GuardScope() { route_guard() = RouteGuard{}; }
+    } guard_scope(m->cfg.n_expert, m->status);
     if (m->packed_path(ntok) || m->small_batch_mixed(ntok) || m->mixed_chunk(ntok) || m->stream_chunk(ntok)) {
         const Layer &L = m->layers[layer];
         const uint32_t nv = m->cfg.hidden / 256u;
         // batches whose pairs are grouped by expert next: the pair sort rides in the same launch as one more workgroup
         // (with the routing given, grouping pays from two tokens on: the pair sort costs no launch of its own)
         const bool to_group = m->small_batch(ntok) || m->grouped_mixed(ntok, 2u);
-        const GroupJob job{ids_dev, weights_dev, ntok, m->cfg.top_k, m->cfg.n_expert, m->uid, m->expert_start, m->pair_token, m->pair_weight, m->tok_pair, m->n_unique};
+        const GroupJob job{ids_dev, weights_dev, ntok, m->cfg.top_k, m->cfg.n_expert, m->uid, m->expert_start, m->pair_token, m->pair_weight, m->tok_pair, m->n_unique, m->status};
         bool grouped = false;
         if (m->mixed && m->packed_gu() && (ntok == 1u || m->small_batch_mixed(ntok)) && L.dense_gu && (nv == 2u || nv == 4u || nv == 8u || nv == 16u)) {
             // one token or a small batch on a mixed layout: the kernels take the shared expert's gate | up products as an input: one f32
@@ -782,6 +793,14 @@ int redhip_moe_last_route(redhip_moe_t h, uint32_t ntok, uint32_t *ids, float *w
     if (!m || !ntok || ntok > m->cfg.max_tokens) { moe_err("invalid last-route request"); return 0; }
     HIP_OK(hipStreamSynchronize(static_cast<hipStream_t>(stream)), "stream synchronise");
     const redhip_moe_config &c = m->cfg;
+    uint32_t status = 0u;
+    HIP_OK(hipMemcpy(&status, m->status, 4u, hipMemcpyDeviceToHost), "status download");
+    if (status) {
+        HIP_OK(hipMemset(m->status, 0, 4u), "status reset");
+        moe_err("routing given to redhip_moe_experts / redhip_moe_group broke its contract:%s%s (ids were clamped; the outputs of those calls are not meaningful)",
+                (status & 1u) ? " an expert id was >= n_expert" : "", (status & 2u) ? " a token named an expert twice" : "");
+        return 0;
+    }
     if (ids) HIP_OK(hipMemcpy(ids, m->ids, (size_t)ntok * c.top_k * 4u, hipMemcpyDeviceToHost), "ids download");
     if (weights) HIP_OK(hipMemcpy(weights, m->weights, (size_t)ntok * c.top_k * 4u, hipMemcpyDeviceToHost), "weights download");
     if (logits) {
@@ -801,8 +820,11 @@ int redhip_moe_group(redhip_moe_t h, const uint32_t *ids_dev, const float *weigh
         return 0;
     }
     prof_set_stage(ST_GROUP);
-    HIP_OK(launch_group_pairs(ids_dev, weights_dev, ntok, m->cfg.top_k, m->cfg.n_expert, uid_dev, expert_start_dev, pair_token_dev,
-                              pair_weight_dev, tok_pair_dev, n_unique_dev, static_cast<hipStream_t>(stream)), "grouping launch");
+    route_guard() = RouteGuard{m->cfg.n_expert, m->status};
+    const hipError_t ge = launch_group_pairs(ids_dev, weights_dev, ntok, m->cfg.top_k, m->cfg.n_expert, uid_dev, expert_start_dev, pair_token_dev,
+                                             pair_weight_dev, tok_pair_dev, n_unique_dev, static_cast<hipStream_t>(stream));
+    route_guard() = RouteGuard{};
+    HIP_OK(ge, "grouping launch");
     return 1;
 }
 
@@ -811,7 +833,9 @@ int redhip_set_codebooks(const int8_t *iq2_xs_grid, uint32_t iq2_xs_count, const
         moe_err("codebook size mismatch: IQ2_XS takes 4096 values, IQ1_M 16384");
         return 0;
     }
-    HIP_OK(set_caller_grids(iq2_xs_grid, iq1_m_grid), "codebook upload");
+    const hipError_t e = set_caller_grids(iq2_xs_grid, iq1_m_grid);
+    if (e == hipErrorContextAlreadyInUse) { moe_err("%s", kCodebookConflict); return 0; }
+    HIP_OK(e, "codebook upload");
     return 1;
 }
 

@@ -300,6 +300,7 @@ int redmetal_ffn_pool_execute_expert(redmetal_ffn_pool_t h, uint32_t slot_id, ui
     if (e != hipSuccess) { FFN_ERR("FFN input upload failed: %s", hipGetErrorString(e)); return 0; }
     if (gu == T_IQ2_XS || gu == T_IQ1_M || dn == T_IQ2_XS || dn == T_IQ1_M) {      // this pool's codebooks on the device (free when they already are)
         e = set_caller_grids(p->iq2_xs.data(), p->iq1_m.data(), p);
+        if (e == hipErrorContextAlreadyInUse) { FFN_ERR("%s", kCodebookConflict); return 0; }
         if (e != hipSuccess) { FFN_ERR("failed to upload the IQ2_XS / IQ1_M codebooks: %s", hipGetErrorString(e)); return 0; }
     }
     p->mark(slot_id, 1);
@@ -331,10 +332,13 @@ int redmetal_quant_rows(const char *model_path, uint64_t matrix_file_offset, uin
     if (ggml_type == T_IQ2_XS || ggml_type == T_IQ1_M) {      // these two decode through the caller's codebook, as in the reference
         const uint32_t want = ggml_type == T_IQ2_XS ? 512u * 8u : 2048u * 8u;
         if (!grid || grid_count != want) { QUANT_ERR("mixed-quant grid size mismatch: got %u expected %u", grid_count, want); return 0; }
-        if (set_caller_grids(ggml_type == T_IQ2_XS ? grid : nullptr, ggml_type == T_IQ1_M ? grid : nullptr) != hipSuccess) {
-            QUANT_ERR("failed to upload the codebook");
-            return 0;
-        }
+    }
+    // a one-shot call binds nothing: it holds the codebook lock from its upload to the end of its kernel instead
+    std::unique_lock<std::mutex> grid_lock(caller_grid_mutex(), std::defer_lock);
+    if (ggml_type == T_IQ2_XS || ggml_type == T_IQ1_M) {
+        grid_lock.lock();
+        const hipError_t ge = set_caller_grids_locked(ggml_type == T_IQ2_XS ? grid : nullptr, ggml_type == T_IQ1_M ? grid : nullptr);
+        if (ge != hipSuccess) { QUANT_ERR("%s", ge == hipErrorContextAlreadyInUse ? kCodebookConflict : "failed to upload the codebook"); return 0; }
     }
     if (!ncols || ncols % 256u || !nrows || !row_count || row_start >= nrows || row_count > nrows - row_start ||
         input_count != ncols || output_count < row_count) {

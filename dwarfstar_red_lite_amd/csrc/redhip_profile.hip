@@ -32,6 +32,11 @@ BlockContext &block_context() {
     return ctx;
 }
 
+RouteGuard &route_guard() {
+    static thread_local RouteGuard g;
+    return g;
+}
+
 void prof_events(hipEvent_t *start, hipEvent_t *stop) {
     *start = *stop = nullptr;
     if (!g_prof.on) return;

@@ -30,12 +30,13 @@ typedef struct {
     uint32_t hidden;            /* multiple of 256 */
     uint32_t ffn;               /* multiple of 256 */
     uint32_t n_expert;          /* <= 1024 */
-    uint32_t top_k;             /* <= 16 */
+    uint32_t top_k;             /* <= 16 (the one-token and small-batch MFMA kernels serve 2..15, other values run on the generic kernels) */
     uint32_t n_layer;
     uint32_t max_tokens;        /* largest ntok of redhip_moe_forward */
     uint32_t router_type;       /* 0 (F32) or 14 (Q6_K) */
-    uint32_t expert_type_word;  /* gate_up | down << 8, as native/redlite_native_metal.h:69-73; types 16, 21, 14 */
-    uint32_t shared_type_word;  /* same encoding for the shared expert */
+    uint32_t expert_type_word;  /* gate_up | down << 8, as native/redlite_native_metal.h:69-73; types 16 (IQ2_XXS), 21 (IQ3_S), 14 (Q6_K), and
+                                   17 (IQ2_XS) / 29 (IQ1_M) after redhip_set_codebooks */
+    uint32_t shared_type_word;  /* same encoding for the shared expert; types 16, 21, 14 */
     uint32_t reserved;
 } redhip_moe_config;
 
@@ -59,13 +60,19 @@ int redhip_moe_load_experts(redhip_moe_t moe, uint32_t layer, uint32_t first_exp
 int redhip_moe_forward(redhip_moe_t moe, uint32_t layer, const float *x_dev, uint32_t ntok, float *out_dev, void *stream);
 
 /* Stream-ordered pieces of the same path (what forward chains), for callers that interleave their own work and
- * for parity taps. ids_dev [ntok][top_k] u32, weights_dev [ntok][top_k] f32, logits_dev [ntok][n_expert] f32. */
+ * for parity taps. ids_dev [ntok][top_k] u32, weights_dev [ntok][top_k] f32, logits_dev [ntok][n_expert] f32.
+ * Contract of routing a caller hands in (redhip_moe_experts, redhip_moe_group), as the reference checks its host-side lists
+ * (native/redmetal_topk.m:1313,1635-1636): every id < n_expert, and the ids of one token distinct. The ids live in device memory
+ * and cannot be checked before the kernels run, so the kernels guard themselves: an id >= n_expert is clamped to n_expert - 1
+ * (no out-of-bounds access), and both violations set a status word that makes the next redhip_moe_last_route on the handle fail
+ * with a message (and clears it). Outputs of a call that broke the contract are not meaningful. */
 int redhip_moe_route(redhip_moe_t moe, uint32_t layer, const float *x_dev, uint32_t ntok,
     uint32_t *ids_dev, float *weights_dev, float *logits_dev, void *stream);
 int redhip_moe_experts(redhip_moe_t moe, uint32_t layer, const float *x_dev, uint32_t ntok,
     const uint32_t *ids_dev, const float *weights_dev, float *out_dev, void *stream);
 
-/* Routing of the last forward / route on this handle, copied to host after synchronising `stream`. Any may be NULL. */
+/* Routing of the last forward / route on this handle, copied to host after synchronising `stream`. Any may be NULL. Fails (0, message)
+ * when a call since the last one was given routing that broke the contract above. */
 int redhip_moe_last_route(redhip_moe_t moe, uint32_t ntok, uint32_t *ids, float *weights, float *logits, void *stream);
 
 /* GGUF side (the role of native/redlite_native_gguf.c:196-440 and the tensor checks of
@@ -102,7 +109,9 @@ int redhip_moe_group(redhip_moe_t moe, const uint32_t *ids_dev, const float *wei
 /* The int8 codebooks of IQ2_XS (512 x 8) and IQ1_M (2048 x 8) that type 17 / 29 rows decode through, copied to the device
  * for the taps below; either may be NULL to keep what is there. The reference hands the same two tables to
  * redmetal_ffn_pool_create and redmetal_quant_rows (native/redmetal_ffn.h:9-18, native/redmetal_quant.h:9-27), which upload
- * them too. Process-wide; synchronous. */
+ * them too. Process-wide and synchronous: the process holds one pair of tables. Resident layers with such experts, and pools that have run
+ * one, are bound to the tables' content: while any of them is alive, a call (here, or through a pool / redmetal_quant_rows) that brings
+ * different tables fails with a message instead of changing what they decode through; the same content again is free. */
 int redhip_set_codebooks(const int8_t *iq2_xs_grid, uint32_t iq2_xs_count, const int8_t *iq1_m_grid, uint32_t iq1_m_count);
 
 /* Parity tap: f32 dequantisation of `rows` rows of `ncols` weights of raw GGUF blocks (device pointers). */

@@ -5,11 +5,13 @@
  * native/redmetal_ffn.m:425-706. Names, argument meaning, return convention (1 = success, 0 = failure,
  * message through redmetal_ffn_last_error(), thread-local) and the slot layout gate|up|down are kept, so a
  * caller of the reference binds this library unchanged. Differences, all additive:
- *   - ggml_type accepts IQ2_XXS (16), IQ3_S (21), Q6_K (14) and the reference's two-type word
- *     gate_up | down << 8 (native/redlite_native_metal.h:69-73). IQ2_XS (17) / IQ1_M (29) are rejected with
- *     a message: they are outside this path.
- *   - the two grid arguments of pool_create are accepted as the reference requires them (non-NULL, exact
- *     counts, native/redmetal_ffn.m:223-227) and otherwise unused: the codebooks are built in.
+ *   - ggml_type accepts the reference's IQ2_XS (17) / IQ1_M (29), decoded through the two codebooks handed to pool_create
+ *     exactly as the reference takes them (non-NULL, exact counts, native/redmetal_ffn.m:223-227), plus IQ2_XXS (16),
+ *     IQ3_S (21), Q6_K (14), whose tables are built in, and the reference's two-type word gate_up | down << 8
+ *     (native/redlite_native_metal.h:69-73) mixing any of them.
+ *   - the process holds one device copy of the two codebooks: a pool binds to their content the first time it runs an
+ *     IQ2_XS / IQ1_M expert, and while bound pools or resident layers are alive a pool with different tables fails with a
+ *     message instead of decoding through the wrong ones (the reference keeps two buffers per pool).
  *   - slots live in device memory (HBM); load_expert reads the file into pinned host memory and copies.
  * All pointers are host pointers; every call is synchronous.
  */

@@ -4,8 +4,9 @@
  * Replaces native/redmetal_quant.h:9-28 (implementation native/redmetal_quant.m:146-303): reads a row-major
  * quantised matrix from a file and returns rows [row_start, row_start + row_count) of W . x. Same signature
  * and error convention (1/0, redmetal_quant_last_error(), thread-local, cleared on entry).
- * ggml_type: F32 (0), Q6_K (14), IQ2_XXS (16), IQ3_S (21). `grid` / `grid_count` are kept for signature
- * compatibility; they may be NULL / 0 because these formats carry built-in codebooks.
+ * ggml_type: the reference's IQ2_XS (17) / IQ1_M (29), decoded through the caller's `grid` (512 x 8 resp. 2048 x 8 int8 values, exact
+ * count required, as native/redmetal_quant.m:160-170), plus F32 (0), Q6_K (14), IQ2_XXS (16), IQ3_S (21), for which `grid` may be
+ * NULL / 0: these formats carry built-in codebooks.
  */
 #pragma once
 #include <stdint.h>

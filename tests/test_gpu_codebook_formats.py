@@ -163,6 +163,45 @@ def test_ffn_pool(model_file, grids):
         with pytest.raises(ValueError, match="need the pool created with"):
             pool.execute(0, lay, T_XS, H, F, 0, H, x)
 
+def test_pools_with_different_codebooks_do_not_decode_through_each_others_tables(model_file, grids):
+    """the process holds one device copy of the two codebooks: while a pool that has run an IQ2_XS expert is alive, a pool (or a one-shot
+    GEMV) that brings other tables is refused with a message; once the first pool is gone the second one runs on its own tables"""
+    from dwarfstar_red_lite_amd import moe
+    from dwarfstar_red_lite_amd._lib import RedHipError
+    from dwarfstar_red_lite_amd.redmetal_ffn import ExpertLayout, RedMetalFfnPool
+    from dwarfstar_red_lite_amd.redmetal_quant import RedMetalQuantBridge
+    path, blob, index, H, F = model_file
+    xs, m = grids
+    xs2 = np.roll(xs.reshape(512, 8), 1, axis=0).copy().reshape(-1)          # the same entries under other indices
+    x = synth.normed_x(np.random.default_rng(16), 1, H)[0]
+    slot_bytes = sum(index["xs." + n][1] for n in ("gate", "up", "down"))
+    lay = ExpertLayout(*index["xs.gate"], *index["xs.up"], *index["xs.down"])
+    sl = lambda o, n: blob[o:o + n]
+    want = {id(g): orc.expert_ffn_grid(T_XS, T_XS, sl(lay.gate_offset, lay.gate_bytes), sl(lay.up_offset, lay.up_bytes),
+                                       sl(lay.down_offset, lay.down_bytes), H, F, x, g, m) for g in (xs, xs2)}
+    first = RedMetalFfnPool(path, 2 * (slot_bytes + 4096), slot_bytes, iq2_xs_grid=xs, iq1_m_grid=m)
+    second = RedMetalFfnPool(path, 2 * (slot_bytes + 4096), slot_bytes, iq2_xs_grid=xs2, iq1_m_grid=m)
+    try:
+        first.load(0, lay)
+        second.load(0, lay)
+        out, _ = first.execute(0, lay, T_XS, H, F, 0, H, x)
+        assert rel_l2(out, want[id(xs)]) <= REL_L2_TOL
+        with pytest.raises(RedHipError, match="codebooks differ"):
+            second.execute(0, lay, T_XS, H, F, 0, H, x)
+        off, n = index["xs.gate"]
+        with pytest.raises(RedHipError, match="codebooks differ"):
+            RedMetalQuantBridge().rows(path, off, n, T_XS, H, F, 0, 4, x, grid=xs2)
+        out, _ = first.execute(0, lay, T_XS, H, F, 0, H, x)                   # the bound pool is unaffected
+        assert rel_l2(out, want[id(xs)]) <= REL_L2_TOL
+        first.close()
+        out2, _ = second.execute(0, lay, T_XS, H, F, 0, H, x)
+        assert rel_l2(out2, want[id(xs2)]) <= REL_L2_TOL
+        assert rel_l2(out2, want[id(xs)]) > 10 * REL_L2_TOL                   # (the two tables do decode differently)
+    finally:
+        first.close()
+        second.close()
+    moe.set_codebooks(xs, m)                                                  # what the tests after this one expect on the device
+
 
 @pytest.mark.parametrize("layout", ["xs", "m"])
 @pytest.mark.parametrize("shape", [(512, 256, 16, 4), (2048, 512, 64, 10)])

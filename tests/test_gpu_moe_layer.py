@@ -73,6 +73,6 @@ def test_layer_full_size_config0():
         x = torch.from_numpy(xs[t:t + 1]).cuda()
         ids, w, logits = m.route(0, x)
         out2 = m.experts(0, x, ids, w).cpu().numpy()[0]
-        # the fused kernel accumulates expert slices with float atomics: same terms, order of addition may differ
-        assert rel_l2(out2, out) <= 1e-5
+        # the same kernels as forward() with the selection as a launch of its own: same terms, same order of addition
+        assert np.array_equal(out2, out)
     m.close()

@@ -270,6 +270,20 @@ def test_expert_ffn_grid_composition(golden_dir):
         assert np.all(np.abs(got - want) <= bound + 1e-300), (gu, dn)
         win = orc.expert_ffn_grid(gu, dn, gate, up, down, H, F, x, xs, m, row_start=500, row_count=12)
         assert np.array_equal(win, got[500:])
+    # a Q6_K (and an IQ2_XXS, an IQ3_S) down matrix fed double activations: the row dot with a double input vector against a numpy
+    # double product over the exactly dequantised row (each term is one rounding of an exact product, the sum is sequential)
+    for dn in (14, 16, 21):
+        down = synth.quant_rows(rng, dn, H, F)
+        act = rng.standard_normal(F) * np.exp(rng.uniform(-3, 3, F))
+        wd = orc.dequant_rows(dn, down, F).astype(np.float64)
+        got = np.array([orc.row_dot(dn, down[r], act) for r in range(H)])          # float64 input: orc_row_dot_d
+        bound = 1e-12 * (np.abs(wd) @ np.abs(act))
+        assert np.all(np.abs(got - wd @ act) <= bound + 1e-300), dn
+        # and it is what the expert FFN feeds its down projection with
+        gate, up = synth.quant_rows(rng, 16, F, H), synth.quant_rows(rng, 16, F, H)
+        a64 = np.array([orc.lib().orc_silu_mul(orc.row_dot(16, gate[r], x), orc.row_dot(16, up[r], x)) for r in range(F)])
+        ffn = orc.expert_ffn(16, dn, gate, up, down, H, F, x)
+        assert np.array_equal(ffn, np.array([orc.row_dot(dn, down[r], a64) for r in range(H)])), dn
 
 
 def test_kept_codebooks_match_grid_arguments(golden_dir):
