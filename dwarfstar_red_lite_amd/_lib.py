@@ -42,6 +42,7 @@ ABI = {
     "redmetal_ffn_pool_load_expert": (i32, [vp, u32, u64, u64, u64, u64, u64, u64, C.POINTER(u64), C.POINTER(dbl)]),
     "redmetal_ffn_pool_slot_addresses": (i32, [vp, u32, u64, u64, u64, C.POINTER(u64), C.POINTER(u64), C.POINTER(u64)]),
     "redmetal_ffn_pool_execute_expert": (i32, [vp, u32, u32, u64, u64, u64, u32, u32, u32, u32, vp, u32, vp, u32, C.POINTER(dbl)]),
+    "redmetal_ffn_pool_execute_expert_noalloc": (i32, [vp, u32, u32, u64, u64, u64, u32, u32, u32, u32, vp, u32, vp, u32, vp]),
     "redmetal_quant_abi_version": (u32, []),
     "redmetal_quant_last_error": (C.c_char_p, []),
     "redmetal_quant_rows": (i32, [C.c_char_p, u64, u64, u32, u32, u32, u32, u32, vp, u32, vp, u32, vp, u32, C.POINTER(dbl), C.POINTER(dbl)]),

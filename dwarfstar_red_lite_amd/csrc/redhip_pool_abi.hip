@@ -111,6 +111,12 @@ struct FfnPool {
         }
         return slabs[slab] + (uint64_t)(slot % slots_per_slab) * slot_bytes;
     }
+    uint8_t *slot_base_existing(uint32_t slot) {  // nullptr when the slot's slab has not been created yet; allocates nothing
+        if (slot >= capacity) return nullptr;
+        std::lock_guard<std::mutex> lk(mu);
+        const uint32_t slab = slot / slots_per_slab;
+        return slab < slabs.size() ? slabs[slab] + (uint64_t)(slot % slots_per_slab) * slot_bytes : nullptr;
+    }
     void mark(uint32_t slot, int delta) {
         std::lock_guard<std::mutex> lk(mu);
         if (delta > 0) inflight[slot] += (uint32_t)delta;
@@ -119,6 +125,30 @@ struct FfnPool {
 };
 
 FfnPool *pool_of(redmetal_ffn_pool_t h) { return static_cast<FfnPool *>(h); }
+
+// ---- scratch of redmetal_ffn_pool_execute_expert_noalloc: the SwiGLU activations between its two launches live in one array that is
+// part of the library's device image, so the call never allocates. Every GPU holds its own copy at its own address; the address is
+// looked up once per device (with that device current) and host code uses only that pointer, never the array's name.
+constexpr uint32_t kNoAllocMaxFfn = 16384u;                                  // 64 KB per GPU, held until the process ends
+static __device__ __align__(256) float scratch[kNoAllocMaxFfn];
+constexpr int kMaxDevices = 64;
+float *g_scratch_ptr[kMaxDevices];
+std::mutex g_scratch_mu;
+
+// the current device's copy of `scratch`; nullptr + message on failure
+float *scratch_of_current_device(char *err, size_t cap) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess || dev < 0 || dev >= kMaxDevices) { set_err(err, cap, "no usable current HIP device for the static scratch (device %d): %s", dev, hipGetErrorString(e)); return nullptr; }
+    std::lock_guard<std::mutex> lk(g_scratch_mu);
+    if (!g_scratch_ptr[dev]) {
+        void *p = nullptr;
+        e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+        if (e != hipSuccess || !p) { set_err(err, cap, "hipGetSymbolAddress of the static scratch failed on device %d: %s", dev, hipGetErrorString(e)); return nullptr; }
+        g_scratch_ptr[dev] = static_cast<float *>(p);
+    }
+    return g_scratch_ptr[dev];
+}
 
 bool sizes_overflow(uint64_t a, uint64_t b, uint64_t c) { return a > UINT64_MAX - b || a + b > UINT64_MAX - c; }
 
@@ -145,6 +175,7 @@ redmetal_ffn_pool_t redmetal_ffn_pool_create(const char *model_path, uint64_t bu
     if (!aligned || aligned > budget_bytes) { FFN_ERR("FFN cache budget cannot fit one aligned expert slot"); return nullptr; }
     int ndev = 0;
     if (hipGetDeviceCount(&ndev) != hipSuccess || ndev < 1) { FFN_ERR("no HIP device available"); return nullptr; }
+    if (!scratch_of_current_device(g_ffn_error, sizeof(g_ffn_error))) return nullptr;      // set-up of the entry point that allocates nothing
     FfnPool *p = new FfnPool();
     p->iq2_xs.assign(iq2_xs_grid, iq2_xs_grid + iq2_xs_grid_count);      // uploaded when an IQ2_XS / IQ1_M expert is executed
     p->iq1_m.assign(iq1_m_grid, iq1_m_grid + iq1_m_grid_count);
@@ -315,6 +346,56 @@ int redmetal_ffn_pool_execute_expert(redmetal_ffn_pool_t h, uint32_t slot_id, ui
     e = hipMemcpy(output, dout, n_out * sizeof(float), hipMemcpyDeviceToHost);
     if (e != hipSuccess) { FFN_ERR("FFN output download failed: %s", hipGetErrorString(e)); return 0; }
     if (elapsed_ms) *elapsed_ms = ms;
+    return 1;
+}
+
+int redmetal_ffn_pool_execute_expert_noalloc(redmetal_ffn_pool_t h, uint32_t slot_id, uint32_t ggml_type,
+        uint64_t gate_bytes, uint64_t up_bytes, uint64_t down_bytes, uint32_t hidden_size, uint32_t ffn_size,
+        uint32_t output_row_start, uint32_t output_row_count, const float *input_dev, uint32_t input_count,
+        float *output_dev, uint32_t output_count, void *stream) {
+    FfnPool *p = pool_of(h);
+    if (!p || !input_dev || !output_dev || slot_id >= p->capacity) { FFN_ERR("invalid arguments of the non-allocating FFN call"); return 0; }
+    const uint32_t gu = word_gate_up(ggml_type), dn = word_down(ggml_type);
+    if (!pool_quant_supported(gu) || !pool_quant_supported(dn) || (ggml_type >> 16)) {
+        FFN_ERR("unsupported FFN GGML type word 0x%x (supported: IQ2_XS 17, IQ1_M 29, IQ2_XXS 16, IQ3_S 21, Q6_K 14)", ggml_type);
+        return 0;
+    }
+    if (ffn_size > kNoAllocMaxFfn) {
+        FFN_ERR("ffn %u exceeds the static scratch of the non-allocating FFN call (at most %u activations)", ffn_size, kNoAllocMaxFfn);
+        return 0;
+    }
+    if (!hidden_size || hidden_size % 256u || !ffn_size || ffn_size % 256u || input_count != hidden_size ||
+        !output_row_count || output_row_start >= hidden_size || output_row_count > hidden_size - output_row_start ||
+        output_count < output_row_count) {
+        FFN_ERR("invalid FFN dimensions hidden=%u ffn=%u start=%u count=%u", hidden_size, ffn_size, output_row_start, output_row_count);
+        return 0;
+    }
+    const uint64_t expect_gate = (uint64_t)ffn_size * pool_row_bytes(gu, hidden_size);
+    const uint64_t expect_down = (uint64_t)hidden_size * pool_row_bytes(dn, ffn_size);
+    if (gate_bytes != expect_gate || up_bytes != expect_gate || down_bytes != expect_down) {
+        FFN_ERR("FFN matrix byte mismatch gate=%llu/%llu up=%llu/%llu down=%llu/%llu", (unsigned long long)gate_bytes,
+                (unsigned long long)expect_gate, (unsigned long long)up_bytes, (unsigned long long)expect_gate,
+                (unsigned long long)down_bytes, (unsigned long long)expect_down);
+        return 0;
+    }
+    if (sizes_overflow(gate_bytes, up_bytes, down_bytes) || gate_bytes + up_bytes + down_bytes > p->slot_bytes) {
+        FFN_ERR("FFN resident expert exceeds slot bounds");
+        return 0;
+    }
+    uint8_t *base = p->slot_base_existing(slot_id);
+    if (!base) { FFN_ERR("FFN slot %u holds no expert yet: load it before the non-allocating call", slot_id); return 0; }
+    if ((gu == T_IQ2_XS || gu == T_IQ1_M || dn == T_IQ2_XS || dn == T_IQ1_M) && !caller_grids_bound(p)) {
+        FFN_ERR("the pool's IQ2_XS / IQ1_M codebooks are not on the device yet: run redmetal_ffn_pool_execute_expert on such an expert once first");
+        return 0;
+    }
+    float *act = scratch_of_current_device(g_ffn_error, sizeof(g_ffn_error));      // looked up at pool_create; a table read here
+    if (!act) return 0;
+    hipStream_t s = static_cast<hipStream_t>(stream);
+    // gate/up + SwiGLU writes act[0 .. ffn), the down rows read exactly that range: nothing in the scratch has to start at zero
+    const ExpertSet ex{base, 0, gate_bytes, up_bytes, gu, dn};
+    hipError_t e = launch_moe_gateup(ex, nullptr, 1u, hidden_size, ffn_size, input_dev, act, s);
+    if (e == hipSuccess) e = launch_gemv_rows(dn, base + gate_bytes + up_bytes, ffn_size, output_row_start, output_row_count, act, output_dev, s);
+    if (e != hipSuccess) { FFN_ERR("FFN HIP command failed: %s", hipGetErrorString(e)); return 0; }
     return 1;
 }
 

@@ -82,6 +82,15 @@ class RedMetalFfnPool:
             raise RedHipError(self._last_error())
         return out[:output_row_count], float(ms.value)
 
+    def execute_noalloc(self, slot_id, layout, ggml_type, hidden_size, ffn_size, output_row_start, output_row_count, x_dev, out_dev, stream=None):
+        """The same computation enqueued on `stream` (a hipStream_t value) with device pointers and no device allocation: x_dev / out_dev are
+        device addresses (int) of float32 [hidden] / [output_row_count]. Returns once the two launches are enqueued."""
+        ok = self.lib.redmetal_ffn_pool_execute_expert_noalloc(self.handle, slot_id, int(ggml_type), layout.gate_bytes, layout.up_bytes,
+                                                               layout.down_bytes, hidden_size, ffn_size, output_row_start, output_row_count,
+                                                               int(x_dev), hidden_size, int(out_dev), output_row_count, stream)
+        if not ok:
+            raise RedHipError(self._last_error())
+
     def telemetry(self):
         L, h = self.lib, self.handle
         return {"capacity": self.capacity, "slab_count": int(L.redmetal_ffn_pool_slab_count(h)),

@@ -61,6 +61,20 @@ int redmetal_ffn_pool_execute_expert(redmetal_ffn_pool_t pool, uint32_t slot_id,
     uint32_t output_row_start, uint32_t output_row_count, const float *input, uint32_t input_count,
     float *output, uint32_t output_count, double *elapsed_ms);
 
+/* No counterpart in the reference. For callers that cannot allocate device memory (code under HIP graph capture, tight serving
+ * loops, harnesses that forbid hipMalloc): the same computation as redmetal_ffn_pool_execute_expert, stream-ordered on device
+ * pointers - input_dev [hidden] f32, output_dev [output_row_count] f32, `stream` a hipStream_t (NULL = the default stream), no host
+ * synchronisation - and it calls no hipMalloc / hipFree. The SwiGLU activations between its two launches live in a 64 KB array
+ * that is part of the library's device image (one copy per GPU, held until the process ends): ffn_size is limited to 16384
+ * (larger: 0 + message). Every call on a GPU shares that GPU's array, so calls that overlap on one GPU (different streams,
+ * threads or pools) race; calls on one stream are ordered. The slot must have been loaded (its slab exists); the slot is not
+ * marked in flight, so the caller must not reload it before the stream has passed the call. IQ2_XS / IQ1_M experts need the
+ * pool's codebooks on the device already (redmetal_ffn_pool_execute_expert on such an expert puts them there). */
+int redmetal_ffn_pool_execute_expert_noalloc(redmetal_ffn_pool_t pool, uint32_t slot_id, uint32_t ggml_type,
+    uint64_t gate_bytes, uint64_t up_bytes, uint64_t down_bytes, uint32_t hidden_size, uint32_t ffn_size,
+    uint32_t output_row_start, uint32_t output_row_count, const float *input_dev, uint32_t input_count,
+    float *output_dev, uint32_t output_count, void *stream);
+
 #ifdef __cplusplus
 }
 #endif
