@@ -813,6 +813,145 @@ __device__ __forceinline__ void wave_select_topk(const float *logits, uint32_t E
     if (lane == 0u) out->scalar = 1.0f / (1.0f + expf(-gate_logit));
 }
 
+// ---------------------------------------------------------------- softmax top-k selection by a whole workgroup
+//
+// The same selection spread over the waves of a 1024-lane workgroup (one logit per lane in the first ceil(E / 64) waves), three
+// barriers deep: a lone wave issues about one instruction per five clocks, so the single-wave routine above costs its instruction
+// count; here every wave runs a short chain.
+//   1. every selecting wave reads all logits for the maximum (same addresses in every wave, no barrier), then its own lane's
+//      e = expf(l - max); per-wave double sums and the maxima of the 2 * NS half waves go to LDS.
+//   2. denominator = the wave sums added in wave order; p = e * (float)(1 / denominator) as the CPU path forms it. The K-th largest
+//      half-wave maximum (minus a few ulps: two different e can round to one p) bounds the K-th largest e from below, so the winners
+//      are among the lanes at or above it, typically a dozen; each wave lists its candidates (p bits above the complemented index).
+//   3. every candidate counts the candidates that beat it under (p descending, index ascending): that count is its place in selection
+//      order, and the K lowest are the selected experts - the set and order of the CPU's argmax loop with ties to the lower index.
+// Ties and degenerate inputs only lengthen the candidate lists (all-equal logits: every lane is a candidate), never change the result.
+struct BlockSelect {
+    double sum_part[16];
+    uint32_t half_max[32];
+    uint32_t cand_n[16];
+    uint32_t ids[16];
+    float p[16];
+    uint64_t cand[16][64];      // per wave: its candidates in lane order; entries n .. kCandHead - 1 are zero (a zero beats nobody)
+};
+constexpr uint32_t kCandHead = 4u;      // candidates per wave that the ranking reads unconditionally (a wave rarely lists more)
+
+__device__ __forceinline__ uint32_t umax32(uint32_t a, uint32_t b) { return a > b ? a : b; }
+template <int CTRL> __device__ __forceinline__ uint32_t dpp_u32(uint32_t v) { return (uint32_t)__builtin_amdgcn_update_dpp(0, (int)v, CTRL, 0xf, 0xf, false); }
+__device__ __forceinline__ uint32_t half_wave_max_u32(uint32_t v) {
+    v = umax32(v, dpp_u32<kDppXor1>(v));
+    v = umax32(v, dpp_u32<kDppXor2>(v));
+    v = umax32(v, dpp_u32<kDppRor4>(v));
+    v = umax32(v, dpp_u32<kDppRor8>(v));
+    const auto r = __builtin_amdgcn_permlane16_swap(v, v, false, false);      // rows 0 | 1 and rows 2 | 3 meet
+    return umax32((uint32_t)r[0], (uint32_t)r[1]);
+}
+
+// Called by every thread of a workgroup of 16 waves; on return (behind a barrier) bs->ids[k], bs->p[k], k < K, hold the selection.
+// NSM: upper bound of the waves that hold logits (8 for E <= 512, else 16). Every loop over waves is unrolled to it with predicates, so
+// that the loads of one step (device memory for the logits, LDS afterwards) are all in flight together instead of one round trip each.
+template <int NSM>
+__device__ __forceinline__ void block_select_topk(const float *logits, uint32_t E, uint32_t K, BlockSelect *bs, float *probs = nullptr) {
+    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
+    const uint32_t NS = (E + 63u) >> 6;                      // waves that hold logits (<= NSM)
+    const bool valid = tid < E;
+    float e = 0.0f;
+    uint32_t ekey = 0u;
+    if (wave < NS) {
+        float lv[NSM];
+#pragma unroll
+        for (int s = 0; s < NSM; ++s) { const uint32_t q = lane + 64u * s; lv[s] = q < E ? logits[q] : -INFINITY; }
+        const float l = valid ? logits[tid] : -INFINITY;
+        float m = lv[0];
+#pragma unroll
+        for (int s = 1; s < NSM; ++s) m = fmaxf(m, lv[s]);
+        m = wave_max(m);
+        e = valid ? expf(l - m) : 0.0f;
+        const double part = wave_sum_d((double)e);
+        ekey = valid ? (__float_as_uint(e) | 0x80000000u) : 0u;      // valid keys have the top bit set: padding never counts
+        const uint32_t hm = half_wave_max_u32(ekey);
+        if (lane == 0u) bs->sum_part[wave] = part;
+        if ((lane & 31u) == 0u) bs->half_max[2u * wave + (lane >> 5)] = hm;
+    }
+    __syncthreads();
+    float p = 0.0f;
+    uint64_t word = 0ull;
+    bool take = false;
+    if (wave < NS) {
+        double sp[NSM];
+#pragma unroll
+        for (int w = 0; w < NSM; ++w) sp[w] = bs->sum_part[w];
+        uint32_t hmx[2 * NSM];
+#pragma unroll
+        for (int q = 0; q < 2 * NSM; ++q) hmx[q] = bs->half_max[q];
+        double denom = 0.0;
+#pragma unroll
+        for (int w = 0; w < NSM; ++w) denom += (uint32_t)w < NS ? sp[w] : 0.0;      // wave order
+        const bool bad = !(denom > 0.0) || isinf(denom) || isnan(denom);
+        p = e * (bad ? 0.0f : reciprocal_as_float(denom));
+        const uint32_t key = valid ? (__float_as_uint(p) | 0x80000000u) : 0u;
+        if (probs && valid) probs[tid] = p;
+        const uint32_t NH = 2u * NS;
+        uint32_t tau = 0x80000000u;                          // no bound: every valid lane is a candidate
+        if (K <= NH) {
+            const uint32_t v = lane < NH ? bs->half_max[lane] : 0u;
+            uint32_t above = 0u;
+#pragma unroll
+            for (int q = 0; q < 2 * NSM; ++q) above += ((uint32_t)q < NH && (hmx[q] > v || (hmx[q] == v && (uint32_t)q < lane))) ? 1u : 0u;
+            const uint64_t hit = __ballot(lane < NH && above == K - 1u);      // exactly one lane
+            const uint32_t kth = (uint32_t)__shfl((int)v, __ffsll((long long)hit) - 1, 64);
+            tau = kth > 0x80000004u ? kth - 4u : 0x80000000u;
+        }
+        take = valid && ekey >= tau;
+        word = ((uint64_t)key << 32) | (uint64_t)(~tid);     // larger word <=> earlier in selection order
+        const uint64_t mask = __ballot(take);
+        const uint32_t n = (uint32_t)__popcll(mask);
+        if (take) bs->cand[wave][__builtin_amdgcn_mbcnt_hi((uint32_t)(mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)mask, 0u))] = word;
+        if (lane >= n && lane < kCandHead) bs->cand[wave][lane] = 0ull;
+        if (lane == 0u) bs->cand_n[wave] = n;
+    }
+    __syncthreads();
+    if (wave < NS) {
+        uint32_t rank = 0u;
+#pragma unroll
+        for (int w0 = 0; w0 < NSM; w0 += 8) {          // eight waves' lists at a time: 32 words in registers
+            if ((uint32_t)w0 < NS) {
+                uint64_t head[8][kCandHead];
+                uint32_t cn[8];
+#pragma unroll
+                for (int w = 0; w < 8; ++w) {
+                    cn[w] = bs->cand_n[w0 + w];
+#pragma unroll
+                    for (uint32_t q = 0; q < kCandHead; ++q) head[w][q] = bs->cand[w0 + w][q];
+                }
+#pragma unroll
+                for (int w = 0; w < 8; ++w) {
+                    if ((uint32_t)(w0 + w) < NS) {
+#pragma unroll
+                        for (uint32_t q = 0; q < kCandHead; ++q) rank += head[w][q] > word ? 1u : 0u;
+                        const uint32_t n = (uint32_t)__builtin_amdgcn_readfirstlane((int)cn[w]);
+                        for (uint32_t q = kCandHead; q < n; ++q) rank += bs->cand[w0 + w][q] > word ? 1u : 0u;      // a crowded wave: the rest of its list
+                    }
+                }
+            }
+            __builtin_amdgcn_sched_barrier(0);
+        }
+        if (take && rank < K) { bs->ids[rank] = tid; bs->p[rank] = p; }
+    }
+    __syncthreads();
+}
+// weight of selected expert k: p_k * (float)(1 / sum of the selected p in selection order, in double); NaN flags an invalid softmax
+__device__ __forceinline__ float block_select_weight(const BlockSelect *bs, uint32_t K, uint32_t k) {
+    float pp[16];
+#pragma unroll
+    for (int q = 0; q < 16; ++q) pp[q] = bs->p[q];           // entries K .. 15 are never written: not added below
+    double sum = 0.0;
+#pragma unroll
+    for (int q = 0; q < 16; ++q) sum += (uint32_t)q < K ? (double)pp[q] : 0.0;
+    const bool bad = !(sum > 0.0) || isinf(sum) || isnan(sum);
+    return bs->p[k] * (bad ? __uint_as_float(0x7fc00000u) : reciprocal_as_float(sum));
+}
+
 // stand-alone selection (one wave per token): ids / weights [ntok][top_k], scalar [ntok]
 __global__ __launch_bounds__(64) void select_kernel(const float *logits, uint32_t E, uint32_t K, uint32_t *ids, float *weights, float *scalar,
                                                     float *probs) {
@@ -828,10 +967,26 @@ __global__ __launch_bounds__(64) void select_kernel(const float *logits, uint32_
     if (threadIdx.x == 0u && scalar) scalar[blockIdx.x] = sel.scalar;
 }
 
+// the same by a workgroup of 16 waves per token
+__global__ __launch_bounds__(kWaves * 64) void select_block_kernel(const float *logits, uint32_t E, uint32_t K, uint32_t *ids, float *weights, float *scalar,
+                                                                   float *probs) {
+    __shared__ BlockSelect bs;
+    const float *l = logits + (uint64_t)blockIdx.x * (E + 1u);
+    float *pr = probs ? probs + (uint64_t)blockIdx.x * E : nullptr;
+    if (E <= 512u) block_select_topk<8>(l, E, K, &bs, pr); else block_select_topk<16>(l, E, K, &bs, pr);
+    if (threadIdx.x < K) {
+        ids[(uint64_t)blockIdx.x * K + threadIdx.x] = bs.ids[threadIdx.x];
+        weights[(uint64_t)blockIdx.x * K + threadIdx.x] = block_select_weight(&bs, K, threadIdx.x);
+    }
+    if (threadIdx.x == 0u && scalar) scalar[blockIdx.x] = 1.0f / (1.0f + expf(-l[E]));
+}
+
 hipError_t launch_select(const float *logits, uint32_t ntok, uint32_t n_expert, uint32_t top_k, uint32_t *ids, float *weights, float *scalar,
                          float *probs, hipStream_t s) {
     if (!ntok || !n_expert || n_expert > 1024u || !top_k || top_k > 16u || top_k > n_expert) return hipErrorInvalidValue;
-    REDHIP_LAUNCH(select_kernel, dim3(ntok), dim3(64), 0, s, logits, n_expert, top_k, ids, weights, scalar, probs);
+    // few tokens: one workgroup of 16 waves each (short chains per wave); many tokens: one wave each (the machine is full either way)
+    if (ntok <= 64u) REDHIP_LAUNCH(select_block_kernel, dim3(ntok), dim3(kWaves * 64), 0, s, logits, n_expert, top_k, ids, weights, scalar, probs);
+    else REDHIP_LAUNCH(select_kernel, dim3(ntok), dim3(64), 0, s, logits, n_expert, top_k, ids, weights, scalar, probs);
     return hipGetLastError();
 }
 
@@ -1292,6 +1447,293 @@ __global__ __launch_bounds__(kWaves * 64) void down_combine_kernel(DownArgs a) {
         for (uint32_t s = 0; s < n_slot; ++s) sum = fmaf(comb[s], part[s * 8u + tid], sum);      // selection order, the shared expert last
         a.out[row0 + tid] = a.resid_a ? (a.resid_a[row0 + tid] + a.resid_b[row0 + tid]) + sum : sum;
     }
+}
+
+// ---------------------------------------------------------------- one token on all-IQ2_XXS layers: expert slices
+//
+// One workgroup per (slot, 32 ffn columns): it selects (or takes the caller's routing), multiplies its 32 gate rows and 32 up rows
+// of the slot's expert, applies SwiGLU, keeps the 32 activations in LDS and multiplies them straight away with the matching 32
+// columns of the expert's down matrix - all `hidden` rows - weighted by the slot's router weight. Gate / up and down weights are
+// requested together, right after the selection, so the launch waits for weights once, and the activations never leave the
+// compute unit. What leaves it is one partial output vector per workgroup, partial[slot][column group][hidden]; slice_sum_kernel
+// adds the (top_k + 1) * ffn / 32 partial vectors in a fixed order. The down matrices are read from a column-sliced copy
+// (qs [ffn / 32][hidden] uint2, ds [ffn / 256][hidden] fp16) so that a workgroup's slice is contiguous.
+//
+// REP copies of every entry of the magnitude table sit side by side in LDS, lane l reads copy l % REP: with REP = 16 the sixteen
+// lanes that the LDS serves together always hit sixteen different 16-byte bank groups, whatever entries they ask for.
+struct SliceArgs {
+    const uint8_t *experts;        // packed experts: gate | up streams (row-major), expert e at experts + e * stride
+    uint64_t stride;
+    const uint8_t *down_cm;        // column-sliced packed down matrices, expert e at down_cm + e * down_stride
+    uint64_t down_stride;
+    const uint8_t *shared;         // packed shared expert: gate | up
+    const uint8_t *shared_down_cm;
+    const float *logits;           // [n_expert + 1]: selection happens here; or nullptr: the caller's routing below
+    const uint32_t *ids_in;        // [top_k]
+    const float *weights_in;       // [top_k]
+    const float *scalar_in;        // [1] sigmoid of the shared expert's gate logit
+    uint32_t *ids_out;             // [top_k] written by workgroup (0, 0) when selecting
+    float *weights_out;            // [top_k]
+    float *scalar_out;             // [1]
+    const _Float16 *xh, *xl;       // [hidden]
+    const int *xexp;               // [1]
+    float *partial;                // [top_k + 1][ffn / 32][hidden]
+    uint32_t hidden, ffn, n_expert, top_k;
+    uint32_t *status;              // RouteGuard::status when ids_in is the caller's
+};
+
+// Built by NB whole waves (NB = 8 or 16; `bw` = index of this wave among them, other waves pass bw >= NB and do nothing). Wave bw owns
+// 256 / NB grid entries: its first lanes convert one entry each into a compact strip (`strip`, 4 KB, entry i at 16 i), then the wave copies
+// every entry to its REP slots with lane % 16 = copy and lane / 16 = entry, so that the sixteen lanes the LDS serves together write (and
+// later read) sixteen different 16-byte bank groups. REP = 16; nothing but the wave's own strip entries is read: no workgroup barrier.
+template <int REP, int NB>
+__device__ __forceinline__ void build_tables_rep(uint8_t *lds, uint8_t *strip, uint32_t bw, uint32_t lane) {
+    static_assert(REP == 16 && (NB == 8 || NB == 16), "replication layout");
+    if (bw >= (uint32_t)NB) return;
+    constexpr uint32_t kOwn = 256u / NB;                 // entries of this wave
+    if (lane < kOwn) {
+        const uint32_t idx = bw * kOwn + lane;
+        const uint64_t grid_entry = redhip_iq2xxs_grid[idx];
+        uint32_t w4[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) {
+            const _Float16 lo = (_Float16)(float)((uint32_t)(grid_entry >> (16 * i)) & 255u), hi = (_Float16)(float)((uint32_t)(grid_entry >> (16 * i + 8)) & 255u);
+            w4[i] = (uint32_t)__builtin_bit_cast(uint16_t, lo) | ((uint32_t)__builtin_bit_cast(uint16_t, hi) << 16);
+        }
+        *reinterpret_cast<uint4 *>(strip + (size_t)idx * 16u) = make_uint4(w4[0], w4[1], w4[2], w4[3]);
+    }
+    wave_lds_sync();
+#pragma unroll
+    for (uint32_t k = 0; k < kOwn / 4u; ++k) {
+        const uint32_t idx = bw * kOwn + 4u * k + (lane >> 4);
+        const uint4 e = *reinterpret_cast<const uint4 *>(strip + (size_t)idx * 16u);
+        *reinterpret_cast<uint4 *>(lds + ((size_t)idx * REP + (lane & 15u)) * 16u) = e;
+    }
+}
+// group_dot on the replicated table: `tab` is the table's base plus this lane's copy offset
+template <int REP>
+__device__ __forceinline__ float group_dot_rep(uint2 q, const half4_t *ax, const uint8_t *tab) {
+    float4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (uint32_t l = 0; l < 4u; ++l) {
+        const uint32_t idx = (q.x >> (8u * l)) & 255u, s7 = (q.y >> (7u * l)) & 127u;
+        WeightQuad b0, b1;
+        place_signs(*reinterpret_cast<const uint4 *>(tab + idx * (16u * REP)), s7, b0, b1);
+        acc = __builtin_amdgcn_mfma_f32_4x4x4f16(ax[2u * l], b0.h, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_4x4x4f16(ax[2u * l + 1u], b1.h, acc, 0, 0, 0);
+    }
+    return (acc[0] + acc[1] * 4.8828125e-4f) * (float)(2u * (q.y >> 28) + 1u);
+}
+
+template <int NKC, int REP>        // hidden = 512 * NKC
+__global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(SliceArgs a) {
+    constexpr int NW = kWaves;
+    constexpr int UPW = 16 * NKC / NW;                 // (row-quad, K-chunk) units of gate / up per wave
+    constexpr int DU = (8 * NKC + NW - 1) / NW;        // units of 64 down rows per wave
+    static_assert(UPW >= 1 && UPW * NW == 16 * NKC, "waves must tile the 16 row-quads x NKC chunks");
+    extern __shared__ __attribute__((aligned(16))) uint8_t dyn[];
+    uint8_t *lds = dyn;                                                    // REP * 4 KB magnitude table
+    uint8_t *strip = dyn + REP * kMagBytes;                                // 4 KB: the table once, as its builders convert it
+    float *part = reinterpret_cast<float *>(strip + kMagBytes);            // [NKC][64]
+    _Float16 *act_hl = reinterpret_cast<_Float16 *>(part + NKC * 64);      // [2][32]: hi, lo halves of the 32 activations
+    float *act_scale = reinterpret_cast<float *>(act_hl + 64);             // [4]
+    SelectOut *sel = reinterpret_cast<SelectOut *>(act_scale + 4);
+
+    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
+    const uint32_t H = a.hidden, F = a.ffn, HG = H / 32u, HB = H / 256u, FG = F / 32u;
+    const uint32_t g = blockIdx.x, slot = blockIdx.y;
+    const bool is_shared = slot >= a.top_k;
+
+    // activation operand of the gate / up rows: independent of the routing, requested first
+    const uint32_t kc = wave % NKC, q0 = wave / NKC;
+    const uint32_t G = 16u * kc + blk;
+    half4_t ax[8];
+    load_act_operand(ax, a.xh + 32u * G, a.xl + 32u * G, j);
+    // the table is first read behind the barrier that ends the selection: wave 0 selects, waves 8..15 build meanwhile
+    const bool selecting = !is_shared && a.logits;
+    if (selecting) build_tables_rep<REP, 8>(lds, strip, wave - 8u, lane); else build_tables_rep<REP, 16>(lds, strip, wave, lane);
+    const uint8_t *tab = lds + (lane % REP) * 16u;
+
+    uint32_t expert = 0u;
+    float comb;                                        // the slot's weight in the layer's output
+    if (is_shared) {
+        comb = a.logits ? 1.0f / (1.0f + expf(-a.logits[a.n_expert])) : a.scalar_in[0];
+        __syncthreads();                               // table
+    } else if (a.logits) {
+        if (wave == 0u) {
+            if (a.n_expert <= 512u) wave_select_topk<8>(a.logits, a.n_expert, a.top_k, sel);
+            else wave_select_topk<16>(a.logits, a.n_expert, a.top_k, sel);
+        }
+        __syncthreads();                               // selection and table
+        expert = sel->ids[slot];
+        comb = sel->w[slot];
+        if (g == 0u && slot == 0u) {
+            if (tid < a.top_k) { a.ids_out[tid] = sel->ids[tid]; a.weights_out[tid] = sel->w[tid]; }
+            if (tid == 0u) a.scalar_out[0] = sel->scalar;
+        }
+    } else {
+        expert = guarded_id(a.ids_in[slot], a.n_expert, a.status);
+        comb = a.weights_in[slot];
+        __syncthreads();                               // table
+    }
+    const uint8_t *ex = is_shared ? a.shared : a.experts + (uint64_t)expert * a.stride;
+    const uint8_t *dn = is_shared ? a.shared_down_cm : a.down_cm + (uint64_t)expert * a.down_stride;
+    const uint64_t gate_bytes = (uint64_t)F * HG * 8u + (uint64_t)F * HB * 2u;
+    const uint2 *gate_qs = reinterpret_cast<const uint2 *>(ex);
+    const uint16_t *gate_ds = reinterpret_cast<const uint16_t *>(ex + (uint64_t)F * HG * 8u);
+    const uint2 *up_qs = reinterpret_cast<const uint2 *>(ex + gate_bytes);
+    const uint16_t *up_ds = reinterpret_cast<const uint16_t *>(ex + gate_bytes + (uint64_t)F * HG * 8u);
+    const uint2 *down_qs = reinterpret_cast<const uint2 *>(dn) + (uint64_t)g * H;                                        // [FG][H]
+    const uint16_t *down_ds = reinterpret_cast<const uint16_t *>(dn + (uint64_t)FG * H * 8u) + (uint64_t)(g >> 3) * H;    // [F / 256][H]
+
+    // every weight this workgroup needs is requested here: gate / up units, then the down slice
+    uint2 wq[UPW];
+    uint32_t wd[UPW];
+#pragma unroll
+    for (int u = 0; u < UPW; ++u) {
+        const uint32_t quad = q0 + (NW / NKC) * u;     // 0..7 gate, 8..15 up
+        const uint32_t r = 32u * g + 4u * (quad & 7u) + j;
+        const uint2 *qs = quad < 8u ? gate_qs : up_qs;
+        const uint16_t *ds = quad < 8u ? gate_ds : up_ds;
+        wq[u] = qs[(uint64_t)r * HG + G];
+        wd[u] = ds[(uint64_t)r * HB + (G >> 3)];
+    }
+    uint2 dq[DU];
+    uint32_t dd[DU];
+#pragma unroll
+    for (int k = 0; k < DU; ++k) {
+        const uint32_t unit = wave + NW * k;           // 64 output rows each
+        const uint32_t row = 64u * (unit < 8u * NKC ? unit : 0u) + lane;
+        dq[k] = down_qs[row];
+        dd[k] = down_ds[row];
+    }
+    float v[UPW];
+#pragma unroll
+    for (int u = 0; u < UPW; ++u) v[u] = group_dot_rep<REP>(wq[u], ax, tab) * scale_to_f32(wd[u]);
+    const float tot = quad_column_reduce<UPW>(v, lane);
+    if (reduced_writer<UPW>(lane)) {
+        const uint32_t quad = q0 + (NW / NKC) * reduced_unit<UPW>(lane);
+        part[kc * 64u + 4u * quad + j] = tot;
+    }
+    __syncthreads();
+    if (tid < 32u) {
+        float gsum = 0.0f, usum = 0.0f;
+#pragma unroll
+        for (int c = 0; c < NKC; ++c) { gsum += part[c * 64 + tid]; usum += part[c * 64 + 32 + tid]; }
+        const float xs = 0.125f * exp2i(a.xexp[0]);      // d / 8 and the pre-scale of x
+        gsum *= xs;
+        usum *= xs;
+        const float act = (gsum / (1.0f + expf(-gsum))) * usum;
+        float amax = fabsf(act);
+#pragma unroll
+        for (int o = 16; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+        const int e = prescale_exp(amax);
+        split_hi_lo(act, exp2i(-e), act_hl + tid, act_hl + 32u + tid);
+        if (tid == 0u) act_scale[0] = exp2i(e);
+    }
+    __syncthreads();
+    // down slice: lane = output row of the unit, the 32 activations are the same operand for every lane block
+    half4_t ad[8];
+    {
+        const _Float16 *src = act_hl + (j == 1u ? 32u : 0u);
+#pragma unroll
+        for (int s8 = 0; s8 < 8; ++s8) {
+            half4_t t = {(_Float16)0, (_Float16)0, (_Float16)0, (_Float16)0};
+            if (j < 2u) t = *reinterpret_cast<const half4_t *>(src + 4 * s8);
+            ad[s8] = t;
+        }
+    }
+    const float post = act_scale[0] * comb * 0.125f;     // the activations' pre-scale, the slot's weight, d / 8
+    float *out = a.partial + ((uint64_t)slot * FG + g) * H;
+#pragma unroll
+    for (int k = 0; k < DU; ++k) {
+        const uint32_t unit = wave + NW * k;
+        if (unit < 8u * NKC) out[64u * unit + lane] = group_dot_rep<REP>(dq[k], ad, tab) * scale_to_f32(dd[k]) * post;
+    }
+}
+
+// out[r] = sum over slots (selection order, the shared expert last) and column groups of partial[slot][group][r] (+ the residual of the
+// block step). 32 rows per workgroup as eight float4 columns; a thread adds every 32nd partial vector, the 32 threads of a column
+// meet by shuffles and through LDS in a fixed order.
+__global__ __launch_bounds__(256) void slice_sum_kernel(const float *partial, uint32_t n_part, uint32_t H, float *out, const float *resid_a, const float *resid_b) {
+    __shared__ float4 red[4][8];
+    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, c8 = tid & 7u, pl = tid >> 3;      // pl 0..31
+    const uint32_t col = blockIdx.x * 8u + c8;          // float4 column
+    const float4 *p4 = reinterpret_cast<const float4 *>(partial);
+    const uint32_t H4 = H / 4u;
+    float4 v[8];
+    uint32_t n = 0u;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) {
+        const uint32_t pp = pl + 32u * i;
+        v[i] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (pp < n_part) { v[i] = p4[(uint64_t)pp * H4 + col]; n = i + 1; }
+    }
+    float4 acc = v[0];
+#pragma unroll
+    for (int i = 1; i < 8; ++i) { acc.x += v[i].x; acc.y += v[i].y; acc.z += v[i].z; acc.w += v[i].w; }
+    for (uint32_t base = 256u; base < n_part; base += 256u) {      // more than 256 partial vectors (large top_k x ffn)
+        for (uint32_t pp = base + pl; pp < n_part && pp < base + 256u; pp += 32u) {
+            const float4 t = p4[(uint64_t)pp * H4 + col];
+            acc.x += t.x; acc.y += t.y; acc.z += t.z; acc.w += t.w;
+        }
+    }
+    (void)n;
+#pragma unroll
+    for (int o = 8; o < 64; o <<= 1) {                  // lanes of a wave that share c8: lane bits 3..5
+        acc.x += __shfl_xor(acc.x, o, 64); acc.y += __shfl_xor(acc.y, o, 64); acc.z += __shfl_xor(acc.z, o, 64); acc.w += __shfl_xor(acc.w, o, 64);
+    }
+    if (lane < 8u) red[wave][lane] = acc;
+    __syncthreads();
+    if (tid < 8u) {
+        const float4 a0 = red[0][tid], a1 = red[1][tid], a2 = red[2][tid], a3 = red[3][tid];
+        float4 sum = make_float4((a0.x + a1.x) + (a2.x + a3.x), (a0.y + a1.y) + (a2.y + a3.y), (a0.z + a1.z) + (a2.z + a3.z), (a0.w + a1.w) + (a2.w + a3.w));
+        if (resid_a) {
+            const float4 ra = reinterpret_cast<const float4 *>(resid_a)[col], rb = reinterpret_cast<const float4 *>(resid_b)[col];
+            sum = make_float4((ra.x + rb.x) + sum.x, (ra.y + rb.y) + sum.y, (ra.z + rb.z) + sum.z, (ra.w + rb.w) + sum.w);
+        }
+        reinterpret_cast<float4 *>(out)[col] = sum;
+    }
+}
+
+constexpr int kSliceRep = 16;
+inline size_t slice_lds_bytes(int nkc, int rep) { return (size_t)(rep + 1) * kMagBytes + (size_t)nkc * 64u * 4u + 128u + 16u + sizeof(SelectOut); }
+
+hipError_t launch_expert_slices(const void *experts, uint64_t stride, const void *down_cm, uint64_t down_stride, const void *shared, const void *shared_down_cm,
+                                const float *logits, const uint32_t *ids_in, const float *weights_in, const float *scalar_in, uint32_t *ids_out,
+                                float *weights_out, float *scalar_out, const void *xh, const void *xl, const int *xexp, float *partial, float *out,
+                                uint32_t hidden, uint32_t ffn, uint32_t n_expert, uint32_t top_k, hipStream_t s) {
+    if (!fused_iq2_supported(hidden, ffn) || top_k + 1u > (uint32_t)kWaves || n_expert > 1024u || hidden % 32u) return hipErrorInvalidValue;
+    if (!logits && (!ids_in || !weights_in || !scalar_in)) return hipErrorInvalidValue;
+    const SliceArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(down_cm), down_stride, static_cast<const uint8_t *>(shared),
+                      static_cast<const uint8_t *>(shared_down_cm), logits, ids_in, weights_in, scalar_in, ids_out, weights_out, scalar_out,
+                      static_cast<const _Float16 *>(xh), static_cast<const _Float16 *>(xl), xexp, partial, hidden, ffn, n_expert, top_k, route_guard().status};
+    const dim3 grid_dim(ffn / 32u, top_k + 1u);
+#define REDHIP_SLICE(NKC)                                                                                                              \
+    do {                                                                                                                               \
+        static bool attr = false;                                                                                                       \
+        const size_t dyn = slice_lds_bytes(NKC, kSliceRep);                                                                             \
+        if (!attr) {                                                                                                                    \
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(expert_slice_kernel<NKC, kSliceRep>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn); \
+            if (e != hipSuccess) return e;                                                                                              \
+            attr = true;                                                                                                                \
+        }                                                                                                                               \
+        REDHIP_LAUNCH((expert_slice_kernel<NKC, kSliceRep>), grid_dim, dim3(kWaves * 64), dyn, s, a);                                     \
+    } while (0)
+    prof_set_stage(ST_FUSED_EXPERTS);
+    switch (hidden / 512u) {
+        case 1: REDHIP_SLICE(1); break;
+        case 2: REDHIP_SLICE(2); break;
+        case 4: REDHIP_SLICE(4); break;
+        case 8: REDHIP_SLICE(8); break;
+        default: return hipErrorInvalidValue;
+    }
+#undef REDHIP_SLICE
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    prof_set_stage(ST_SLICE_SUM);
+    REDHIP_LAUNCH(slice_sum_kernel, dim3(hidden / 32u), dim3(256), 0, s, partial, (top_k + 1u) * (ffn / 32u), hidden, out, block_context().resid_a, block_context().resid_b);
+    return hipGetLastError();
 }
 
 // One row of a dense f32 matrix against an activation vector kept as fp16 halves + one exponent per 32 columns: the LPR lanes that

@@ -50,7 +50,7 @@ inline uint32_t word_down(uint32_t w) { return ((w >> 8) & 255u) ? ((w >> 8) & 2
 // and end, so a stage's time is kernel execution only, not launch latency.
 enum Stage : uint32_t {
     ST_OTHER = 0, ST_ROUTER_GEMV, ST_ROUTE_SELECT, ST_GROUP, ST_GATEUP, ST_SHARED_GATEUP, ST_DOWN_COMBINE,
-    ST_FUSED_EXPERTS, ST_BATCH_GATEUP, ST_BATCH_DOWN, ST_BATCH_COMBINE, ST_PREFILL_GATEUP, ST_PREFILL_DOWN, ST_COUNT
+    ST_FUSED_EXPERTS, ST_BATCH_GATEUP, ST_BATCH_DOWN, ST_BATCH_COMBINE, ST_PREFILL_GATEUP, ST_PREFILL_DOWN, ST_SLICE_SUM, ST_COUNT
 };
 void prof_set_stage(uint32_t stage);                       // label of the launches that follow (calling thread)
 
@@ -282,6 +282,13 @@ hipError_t launch_down_combine_raw(uint32_t down_type, uint32_t shared_down_type
                                    const uint32_t *ids, const float *weights, const float *scalar, const void *act_h, const void *act_l,
                                    const int *act_exp, float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, hipStream_t s, uint32_t ntok = 1u,
                                    const int8_t *grid = nullptr, const float *shared_dense = nullptr);
+// single token on all-IQ2_XXS layers, two launches: expert slices (selection from `logits`, or the caller's ids_in / weights_in / scalar_in;
+// gate / up / SwiGLU / the matching columns of the down matrix from its column-sliced copy; partial [top_k + 1][ffn / 32][hidden]), then
+// the sum of the partial vectors into out [hidden]
+hipError_t launch_expert_slices(const void *experts, uint64_t stride, const void *down_cm, uint64_t down_stride, const void *shared, const void *shared_down_cm,
+                                const float *logits, const uint32_t *ids_in, const float *weights_in, const float *scalar_in, uint32_t *ids_out,
+                                float *weights_out, float *scalar_out, const void *xh, const void *xl, const int *xexp, float *partial, float *out,
+                                uint32_t hidden, uint32_t ffn, uint32_t n_expert, uint32_t top_k, hipStream_t s);
 // single token: out[r] = sum_k weights[k] * down_{ids[k]}[r] . act[k] + scalar * shared_down[r] . act[top_k], k in order
 hipError_t launch_down_combine(const void *experts, uint64_t stride, const void *shared, const uint32_t *ids, const float *weights,
                                const float *scalar, const void *act_h, const void *act_l, const int *act_exp, float *out,

@@ -34,6 +34,8 @@ struct Layer {
     uint8_t *experts = nullptr;      // n_expert slots of expert_stride bytes, each gate | up | down
     uint8_t *packed = nullptr;       // same slots in the packed IQ2_XXS layout of the fused kernel (fused path only)
     uint8_t *shared_packed = nullptr;
+    uint8_t *down_cm = nullptr;      // all-IQ2_XXS layers: the packed down matrices once more, column-sliced (qs [ffn / 32][hidden], ds [ffn / 256][hidden]), for the
+    uint8_t *shared_down_cm = nullptr;      // one-token kernel whose workgroups each take 32 columns of a down matrix
     uint8_t *tiled = nullptr;        // third copy, tile-major, read by the prefill kernels (handles that take chunks only)
     uint8_t *shared_tiled = nullptr;
     // mixed layouts that take chunks: f32 copies of the small dense matrices (dequantised once at upload) for the fp32 tile
@@ -47,6 +49,8 @@ struct Moe {
     redhip_moe_config cfg;
     uint32_t gu_type, dn_type, sh_gu_type, sh_dn_type;
     uint64_t gate_bytes, down_bytes, expert_stride;          // routed expert
+    uint64_t down_cm_stride() const { return (down_bytes + 255u) & ~255ull; }
+    float *partial = nullptr;                                // [top_k + 1][ffn / 32][hidden]: partial output vectors of the one-token expert slices
     uint64_t pk_gate_bytes = 0;                              // one gate / up matrix in the packed streams of the one-token kernel
     const int8_t *gu_grid = nullptr, *dn_grid = nullptr;     // device copies of the caller's codebooks (IQ2_XS / IQ1_M matrices)
     uint64_t sh_gate_bytes, sh_down_bytes;                   // shared expert
@@ -300,6 +304,14 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
         prof_set_stage(ST_OTHER);
         return 1;
     }
+    if (m->fused && ntok == 1u) {    // expert slices + their sum; xh / xl (and the scalar gate of a caller's routing) come from the router kernel or the prep kernel
+        const Layer &L = m->layers[layer];
+        HIP_OK(launch_expert_slices(L.packed, m->expert_stride, L.down_cm, m->down_cm_stride(), L.shared_packed, L.shared_down_cm, select_here ? m->logits : nullptr,
+                                    ids, weights, m->scalar, m->ids, m->weights, m->scalar, m->xh, m->xl, m->xexp, m->partial, out, c.hidden, c.ffn, c.n_expert,
+                                    c.top_k, s), "expert slice launch");
+        prof_set_stage(ST_OTHER);
+        return 1;
+    }
     if (m->packed_gu()) {    // xh / xl / scalar come from the router kernel or the prep kernel
         const Layer &L = m->layers[layer];
         prof_set_stage(ST_GATEUP);
@@ -405,6 +417,11 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
                  (!sh_packed || hipMalloc(reinterpret_cast<void **>(&L.shared_packed), align256(2u * m->sh_gate_bytes + m->sh_down_bytes)) == hipSuccess);
             m->resident += (uint64_t)c.n_expert * m->packed_stride + (sh_packed ? align256(2u * m->sh_gate_bytes + m->sh_down_bytes) : 0u);
         }
+        if (ok && m->fused) {
+            ok = hipMalloc(reinterpret_cast<void **>(&L.down_cm), (size_t)c.n_expert * m->down_cm_stride()) == hipSuccess &&
+                 hipMalloc(reinterpret_cast<void **>(&L.shared_down_cm), m->down_cm_stride()) == hipSuccess;
+            m->resident += (uint64_t)(c.n_expert + 1u) * m->down_cm_stride();
+        }
         if (ok && m->mixed) {
             const size_t rb = c.router_type == T_F32 ? 0u : (size_t)c.n_expert * c.hidden * 4u, gb = (size_t)2u * c.ffn * c.hidden * 4u, db = (size_t)c.hidden * c.ffn * 4u;
             float *d = nullptr;
@@ -431,7 +448,8 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
         }
     }
     const size_t T = c.max_tokens;
-    const size_t ws_bytes = align256(4u) + align256(T * c.hidden * 4u) + align256(T * (c.n_expert + 1u) * 4u) + 2u * align256(T * c.top_k * 4u) + align256(T * 4u) +
+    const size_t partial_bytes = m->fused ? align256((size_t)(c.top_k + 1u) * (c.ffn / 32u) * c.hidden * 4u) : 0u;
+    const size_t ws_bytes = partial_bytes + align256(4u) + align256(T * c.hidden * 4u) + align256(T * (c.n_expert + 1u) * 4u) + 2u * align256(T * c.top_k * 4u) + align256(T * 4u) +
                             align256(T * c.top_k * c.ffn * 4u) + align256(T * c.ffn * 4u) +
                             2u * align256(2u * T * c.hidden) + align256(4u * T) + 2u * align256(2u * T * (c.top_k + 1u) * c.ffn) +
                             align256(4u * T * (c.top_k + 1u) * (c.ffn / 32u)) +
@@ -446,6 +464,7 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
     }
     uint8_t *w = m->ws;
     m->status = reinterpret_cast<uint32_t *>(w); w += align256(4u);
+    if (partial_bytes) { m->partial = reinterpret_cast<float *>(w); w += partial_bytes; }
     m->xn = reinterpret_cast<float *>(w); w += align256(T * c.hidden * 4u);
     m->logits = reinterpret_cast<float *>(w); w += align256(T * (c.n_expert + 1u) * 4u);
     m->ids = reinterpret_cast<uint32_t *>(w); w += align256(T * c.top_k * 4u);
@@ -504,6 +523,8 @@ void redhip_moe_destroy(redhip_moe_t h) {
         if (L.experts) (void)hipFree(L.experts);
         if (L.packed) (void)hipFree(L.packed);
         if (L.shared_packed) (void)hipFree(L.shared_packed);
+        if (L.down_cm) (void)hipFree(L.down_cm);
+        if (L.shared_down_cm) (void)hipFree(L.shared_down_cm);
         if (L.dense_gu) (void)hipFree(L.dense_router ? L.dense_router : L.dense_gu);
         if (L.tiled) (void)hipFree(L.tiled);
         if (L.tiled_down) (void)hipFree(L.tiled_down);
@@ -556,8 +577,10 @@ int redhip_moe_load_shared(redhip_moe_t h, uint32_t layer, const float *gate_inp
     if (L.shared_packed) {
         const redhip_moe_config &c = m->cfg;
         HIP_OK(launch_repack_iq2xxs(L.shared, gate_bytes, 2u, c.ffn, c.hidden, false, L.shared_packed, gate_bytes, nullptr), "shared gate/up repack");
-        if (m->fused)
+        if (m->fused) {
             HIP_OK(launch_repack_iq2xxs(L.shared + 2u * gate_bytes, 0u, 1u, c.hidden, c.ffn, false, L.shared_packed + 2u * gate_bytes, 0u, nullptr), "shared down repack");
+            HIP_OK(launch_repack_iq2xxs(L.shared + 2u * gate_bytes, 0u, 1u, c.hidden, c.ffn, true, L.shared_down_cm, 0u, nullptr), "shared down column slices");
+        }
         if (L.shared_tiled) {
             HIP_OK(launch_tile_packed(L.shared_packed, gate_bytes, 2u, c.ffn, c.hidden, L.shared_tiled, gate_bytes, nullptr), "shared gate/up tiling");
             HIP_OK(launch_tile_packed(L.shared_packed + 2u * gate_bytes, 0u, 1u, c.hidden, c.ffn, L.shared_tiled + 2u * gate_bytes, 0u, nullptr), "shared down tiling");
@@ -604,8 +627,11 @@ static int stage_and_pack(Moe *m, uint32_t layer, uint32_t first, uint32_t count
         uint8_t *pk = m->layers[layer].packed + (uint64_t)first * m->packed_stride;
         HIP_OK(launch_repack_gateup(m->gu_type, dst, m->expert_stride, count, c.ffn, c.hidden, pk, m->packed_stride, nullptr), "expert gate repack");
         HIP_OK(launch_repack_gateup(m->gu_type, dst + m->gate_bytes, m->expert_stride, count, c.ffn, c.hidden, pk + m->pk_gate_bytes, m->packed_stride, nullptr), "expert up repack");
-        if (m->fused)
+        if (m->fused) {
             HIP_OK(launch_repack_iq2xxs(dst + 2u * m->gate_bytes, m->expert_stride, count, c.hidden, c.ffn, false, pk + 2u * m->gate_bytes, m->packed_stride, nullptr), "expert down repack");
+            HIP_OK(launch_repack_iq2xxs(dst + 2u * m->gate_bytes, m->expert_stride, count, c.hidden, c.ffn, true,
+                                        m->layers[layer].down_cm + (uint64_t)first * m->down_cm_stride(), m->down_cm_stride(), nullptr), "expert down column slices");
+        }
         if (m->layers[layer].tiled) {
             uint8_t *tl = m->layers[layer].tiled + (uint64_t)first * m->packed_stride;
             HIP_OK(launch_tile_packed(pk, m->packed_stride, count, c.ffn, c.hidden, tl, m->packed_stride, nullptr), "expert gate tiling");
@@ -849,11 +875,16 @@ int redhip_moe_dequant_resident(redhip_moe_t h, uint32_t layer, uint32_t expert,
     Moe *m = moe_of(h);
     if (!check_layer(m, layer)) return 0;
     const redhip_moe_config &c = m->cfg;
-    if (!out_dev || which > 3u || (which < 3u && expert > c.n_expert)) { moe_err("invalid resident matrix request"); return 0; }
+    if (!out_dev || which > 4u || (which != 3u && expert > c.n_expert)) { moe_err("invalid resident matrix request"); return 0; }
     const Layer &L = m->layers[layer];
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (which == 3u) { HIP_OK(launch_dequant_rows(c.router_type, L.router, c.n_expert, c.hidden, out_dev, s), "router dequant"); return 1; }
     const bool sh = expert == c.n_expert;
+    if (which == 4u) {                                      // the column-sliced copy of a down matrix (all-IQ2_XXS layers)
+        if (!m->fused) { moe_err("only all-IQ2_XXS layers keep column-sliced down matrices"); return 0; }
+        HIP_OK(launch_dequant_packed_iq2xxs(sh ? L.shared_down_cm : L.down_cm + (uint64_t)expert * m->down_cm_stride(), c.hidden, c.ffn, true, out_dev, s), "column-sliced down dequant");
+        return 1;
+    }
     if (m->fused || (m->mixed && which < 2u && (!sh || L.shared_packed))) {        // the layout the MFMA kernels read
         const uint8_t *pk = sh ? L.shared_packed : L.packed + (uint64_t)expert * m->packed_stride;
         const uint64_t gbytes = m->pk_gate_bytes;

@@ -22,7 +22,7 @@ Profiler g_prof;
 thread_local uint32_t t_stage = ST_OTHER;
 const char *const kStageNames[ST_COUNT] = {
     "other", "router_gemv", "route_select", "group_pairs", "gateup", "shared_gateup", "down_combine",
-    "fused_experts", "batch_gateup", "batch_down", "batch_combine", "prefill_gateup", "prefill_down"};
+    "fused_experts", "batch_gateup", "batch_down", "batch_combine", "prefill_gateup", "prefill_down", "slice_sum"};
 }  // namespace
 
 void prof_set_stage(uint32_t stage) { t_stage = stage < ST_COUNT ? stage : ST_OTHER; }

@@ -154,7 +154,7 @@ class ResidentMoe:
 
     def dequant_resident(self, layer, expert, which):
         H, F, E = self.cfg["hidden"], self.cfg["ffn"], self.cfg["n_expert"]
-        shape = (E, H) if which == 3 else ((F, H) if which < 2 else (H, F))
+        shape = (E, H) if which == 3 else ((F, H) if which < 2 else (H, F))      # which 4: the column-sliced copy of a down matrix
         out = torch.empty(shape, dtype=torch.float32, device="cuda")
         self._check(self.lib.redhip_moe_dequant_resident(self.handle, layer, expert, which, out.data_ptr(), _stream()))
         return out

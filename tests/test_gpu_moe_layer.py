@@ -43,6 +43,9 @@ def test_layer_single_token(layout, shape):
             want = orc.dequant_rows(t, raw.reshape(-1), H if which < 2 else F)
             got = m.dequant_resident(l, e, which).cpu().numpy()
             assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
+            if which == 2 and layout == "iq2":               # and from the column-sliced copy that the one-token kernel reads
+                got = m.dequant_resident(l, e, 4).cpu().numpy()
+                assert np.array_equal(got.view(np.uint32), want.view(np.uint32))
         for t in range(3):
             out = m.forward(l, torch.from_numpy(xs[t:t + 1]).cuda()).cpu().numpy()[0]
             gids, gw, glog = m.last_route(1)
