@@ -283,11 +283,14 @@ __device__ __forceinline__ float q6k_dot32(const uint8_t *row, uint32_t chunk, c
 // position of a pair inside its group and the group's size are bit counts of that set, the order of the groups a
 // bit count over the "first pair of its expert" flags, the group offsets one prefix sum. Run by a whole workgroup
 // of at least 128 threads (every thread reaches the barriers); at most 16 tokens, 128 pairs, 1024 experts.
-constexpr uint32_t kGroupLdsWords = 1024u + 4u;
+constexpr uint32_t kGroupLdsWords = 1024u + 6u;
+// Optionally also the pass list of the batched expert-slice kernel (g.pass_list != nullptr): a pass = up to two consecutive pairs of one
+// group. Entry v: x = expert | pairs in the pass << 16 | position of its first pair << 24; y = four bytes: the (token * top_k + k) index
+// of its first and second pair, then their tokens. Passes follow the groups' order; *g.n_pass = their number.
 template <class PairId, class PairWeight>
 __device__ __forceinline__ void group_small(const GroupJob &g, uint32_t *lds, PairId pair_id, PairWeight pair_w) {
-    uint32_t *token_set = lds;                           // per expert: bit t = token t selected it; later the group's offset
-    uint32_t *first_count = lds + 1024, *size_total = lds + 1026;
+    uint32_t *token_set = lds;                           // per expert: bit t = token t selected it; later the group's offset (| its first pass << 16)
+    uint32_t *first_count = lds + 1024, *size_total = lds + 1026, *pass_total = lds + 1028;
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, K = g.top_k;
     for (uint32_t i = tid; i < g.n_expert; i += blockDim.x) token_set[i] = 0u;
     __syncthreads();
@@ -301,27 +304,42 @@ __device__ __forceinline__ void group_small(const GroupJob &g, uint32_t *lds, Pa
     const uint32_t n = (uint32_t)__popc(set), before = (uint32_t)__popc(set & ((1u << t) - 1u));
     const bool first = live && before == 0u;
     uint32_t scan = first ? n : 0u;                      // inclusive prefix sum of the group sizes in pair order
+    const uint32_t n_pass_mine = first ? (n + 1u) >> 1 : 0u;
+    uint32_t pscan = n_pass_mine;                        // the same of the groups' pass counts
     if (wave < 2u) {
 #pragma unroll
         for (int o = 1; o < 64; o <<= 1) {
-            const uint32_t up = __shfl_up(scan, o, 64);
-            if (lane >= (uint32_t)o) scan += up;
+            const uint32_t up = __shfl_up(scan, o, 64), pup = __shfl_up(pscan, o, 64);
+            if (lane >= (uint32_t)o) { scan += up; pscan += pup; }
         }
         const uint64_t fm = __ballot(first);
-        if (lane == 63u) { first_count[wave] = (uint32_t)__popcll(fm); size_total[wave] = scan; }
+        if (lane == 63u) { first_count[wave] = (uint32_t)__popcll(fm); size_total[wave] = scan; pass_total[wave] = pscan; }
     }
     const uint64_t first_mask = __ballot(first);
     __syncthreads();
     const uint32_t grp = (wave == 1u ? first_count[0] : 0u) + __builtin_amdgcn_mbcnt_hi((uint32_t)(first_mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)first_mask, 0u));
     const uint32_t start = (wave == 1u ? size_total[0] : 0u) + scan - (first ? n : 0u);
-    if (first) { token_set[e] = start; g.uid[grp] = e; g.expert_start[grp] = start; }
-    if (tid == 0u) { const uint32_t U = first_count[0] + first_count[1]; g.expert_start[U] = P; g.n_unique[0] = U; }
+    const uint32_t pass0 = (wave == 1u ? pass_total[0] : 0u) + pscan - n_pass_mine;
+    if (first) { token_set[e] = start | (pass0 << 16); g.uid[grp] = e; g.expert_start[grp] = start; }
+    if (tid == 0u) {
+        const uint32_t U = first_count[0] + first_count[1];
+        g.expert_start[U] = P;
+        g.n_unique[0] = U;
+        if (g.n_pass) g.n_pass[0] = pass_total[0] + pass_total[1];
+    }
     __syncthreads();
     if (live) {
-        const uint32_t pos = token_set[e] + before;
+        const uint32_t word = token_set[e], pos = (word & 0xffffu) + before;
         g.pair_token[pos] = t;
         g.pair_weight[pos] = pair_w(t, pr % K);
         g.tok_pair[pr] = pos;
+        if (g.pass_list) {
+            const uint32_t v = (word >> 16) + (before >> 1), half = before & 1u;
+            uint8_t *entry = reinterpret_cast<uint8_t *>(g.pass_list + v);
+            if (half == 0u) reinterpret_cast<uint32_t *>(entry)[0] = e | ((n - before >= 2u ? 2u : 1u) << 16) | (pos << 24);
+            entry[4u + half] = (uint8_t)pr;
+            entry[6u + half] = (uint8_t)t;
+        }
     }
 }
 // the same from routing held in device memory (kernels that carry the grouping as a side job of one extra workgroup)
@@ -1482,15 +1500,24 @@ struct SliceArgs {
     uint32_t *status;              // RouteGuard::status when ids_in is the caller's
 };
 
+// Two tables, REP copies of every 16-byte entry side by side (entry i, copy c at (i * REP + c) * 16), lane l reads copy l % REP: with
+// REP = 16 the sixteen lanes that the LDS serves together always hit sixteen different 16-byte bank groups, whatever entries they ask for.
+//   magnitudes: 256 entries, the eight fp16 magnitudes of a grid entry;
+//   sign masks: 128 entries, for a 7-bit sign field (the eighth sign is its parity) the four words that flip the fp16 sign bits of the
+//               eight weights (bit 15 / 31 of word i = sign of weight 2 i / 2 i + 1) - one read and four XORs in place of a dozen integer
+//               operations per eight weights.
 // Built by NB whole waves (NB = 8 or 16; `bw` = index of this wave among them, other waves pass bw >= NB and do nothing). Wave bw owns
-// 256 / NB grid entries: its first lanes convert one entry each into a compact strip (`strip`, 4 KB, entry i at 16 i), then the wave copies
-// every entry to its REP slots with lane % 16 = copy and lane / 16 = entry, so that the sixteen lanes the LDS serves together write (and
-// later read) sixteen different 16-byte bank groups. REP = 16; nothing but the wave's own strip entries is read: no workgroup barrier.
-template <int REP, int NB>
+// 256 / NB grid entries and 128 / NB sign fields: its first lanes make one entry each in a compact strip (`strip`: 4 KB + 2 KB), then the
+// wave copies every entry to its REP slots with lane % 16 = copy and lane / 16 = entry (conflict-free writes too). Nothing but the
+// wave's own strip entries is read: no workgroup barrier inside.
+constexpr uint32_t kSignBytes = 128u * 16u;
+// SREP: copies of the sign table (16, or 8 where LDS is short: lanes l and l + 8 then share a copy and sometimes collide)
+template <int REP, int NB, int SREP = REP>
 __device__ __forceinline__ void build_tables_rep(uint8_t *lds, uint8_t *strip, uint32_t bw, uint32_t lane) {
-    static_assert(REP == 16 && (NB == 8 || NB == 16), "replication layout");
+    static_assert((REP == 16 || REP == 8) && (SREP == 16 || SREP == 8 || SREP == 0) && (NB == 8 || NB == 16), "replication layout");
     if (bw >= (uint32_t)NB) return;
-    constexpr uint32_t kOwn = 256u / NB;                 // entries of this wave
+    constexpr uint32_t kOwn = 256u / NB, kOwnS = 128u / NB;      // entries of this wave
+    uint8_t *sign_lds = lds + REP * kMagBytes, *sign_strip = strip + kMagBytes;
     if (lane < kOwn) {
         const uint32_t idx = bw * kOwn + lane;
         const uint64_t grid_entry = redhip_iq2xxs_grid[idx];
@@ -1501,24 +1528,50 @@ __device__ __forceinline__ void build_tables_rep(uint8_t *lds, uint8_t *strip, u
             w4[i] = (uint32_t)__builtin_bit_cast(uint16_t, lo) | ((uint32_t)__builtin_bit_cast(uint16_t, hi) << 16);
         }
         *reinterpret_cast<uint4 *>(strip + (size_t)idx * 16u) = make_uint4(w4[0], w4[1], w4[2], w4[3]);
+    } else if (SREP != 0 && lane - 32u < kOwnS) {        // (kOwn <= 32)
+        const uint32_t s7 = bw * kOwnS + lane - 32u, s8 = s7 | ((__popc(s7) & 1u) << 7);
+        uint32_t w4[4];
+#pragma unroll
+        for (int i = 0; i < 4; ++i) w4[i] = (((s8 >> (2 * i)) & 1u) << 15) | (((s8 >> (2 * i + 1)) & 1u) << 31);
+        *reinterpret_cast<uint4 *>(sign_strip + (size_t)s7 * 16u) = make_uint4(w4[0], w4[1], w4[2], w4[3]);
     }
     wave_lds_sync();
+    constexpr uint32_t kPerM = 64u / REP;                // entries per copy instruction
 #pragma unroll
-    for (uint32_t k = 0; k < kOwn / 4u; ++k) {
-        const uint32_t idx = bw * kOwn + 4u * k + (lane >> 4);
+    for (uint32_t k = 0; k < kOwn / kPerM; ++k) {
+        const uint32_t idx = bw * kOwn + kPerM * k + lane / REP;
         const uint4 e = *reinterpret_cast<const uint4 *>(strip + (size_t)idx * 16u);
-        *reinterpret_cast<uint4 *>(lds + ((size_t)idx * REP + (lane & 15u)) * 16u) = e;
+        *reinterpret_cast<uint4 *>(lds + ((size_t)idx * REP + lane % REP) * 16u) = e;
+    }
+    if constexpr (SREP != 0) {
+        constexpr uint32_t kPer = 64u / (SREP ? SREP : 1);
+#pragma unroll
+        for (uint32_t k = 0; k < kOwnS / kPer; ++k) {
+            const uint32_t s7 = bw * kOwnS + kPer * k + lane / (SREP ? SREP : 1);
+            const uint4 e = *reinterpret_cast<const uint4 *>(sign_strip + (size_t)s7 * 16u);
+            *reinterpret_cast<uint4 *>(sign_lds + ((size_t)s7 * SREP + lane % (SREP ? SREP : 1)) * 16u) = e;
+        }
     }
 }
-// group_dot on the replicated table: `tab` is the table's base plus this lane's copy offset
-template <int REP>
-__device__ __forceinline__ float group_dot_rep(uint2 q, const half4_t *ax, const uint8_t *tab) {
+// eight signed fp16 weights from the two replicated tables; `tab` / `stab` = base of the magnitude / sign table + this lane's copy offset
+template <int REP, int SREP>
+__device__ __forceinline__ void signed_weights_rep(const uint8_t *tab, const uint8_t *stab, uint32_t idx, uint32_t s7, WeightQuad &b0, WeightQuad &b1) {
+    const uint4 m = *reinterpret_cast<const uint4 *>(tab + idx * (16u * REP));
+    const uint4 sg = *reinterpret_cast<const uint4 *>(stab + s7 * (16u * SREP));
+    b0.u[0] = m.x ^ sg.x;
+    b0.u[1] = m.y ^ sg.y;
+    b1.u[0] = m.z ^ sg.z;
+    b1.u[1] = m.w ^ sg.w;
+}
+// group_dot on the replicated tables
+template <int REP, int SREP>
+__device__ __forceinline__ float group_dot_rep(uint2 q, const half4_t *ax, const uint8_t *tab, const uint8_t *stab) {
     float4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
 #pragma unroll
     for (uint32_t l = 0; l < 4u; ++l) {
         const uint32_t idx = (q.x >> (8u * l)) & 255u, s7 = (q.y >> (7u * l)) & 127u;
         WeightQuad b0, b1;
-        place_signs(*reinterpret_cast<const uint4 *>(tab + idx * (16u * REP)), s7, b0, b1);
+        signed_weights_rep<REP, SREP>(tab, stab, idx, s7, b0, b1);
         acc = __builtin_amdgcn_mfma_f32_4x4x4f16(ax[2u * l], b0.h, acc, 0, 0, 0);
         acc = __builtin_amdgcn_mfma_f32_4x4x4f16(ax[2u * l + 1u], b1.h, acc, 0, 0, 0);
     }
@@ -1532,9 +1585,9 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(SliceArgs a) 
     constexpr int DU = (8 * NKC + NW - 1) / NW;        // units of 64 down rows per wave
     static_assert(UPW >= 1 && UPW * NW == 16 * NKC, "waves must tile the 16 row-quads x NKC chunks");
     extern __shared__ __attribute__((aligned(16))) uint8_t dyn[];
-    uint8_t *lds = dyn;                                                    // REP * 4 KB magnitude table
-    uint8_t *strip = dyn + REP * kMagBytes;                                // 4 KB: the table once, as its builders convert it
-    float *part = reinterpret_cast<float *>(strip + kMagBytes);            // [NKC][64]
+    uint8_t *lds = dyn;                                                    // REP * (4 KB magnitude table + 2 KB sign masks)
+    uint8_t *strip = dyn + REP * (kMagBytes + kSignBytes);                 // 4 KB + 2 KB: the tables once, as their builders make them
+    float *part = reinterpret_cast<float *>(strip + kMagBytes + kSignBytes);      // [NKC][64]
     _Float16 *act_hl = reinterpret_cast<_Float16 *>(part + NKC * 64);      // [2][32]: hi, lo halves of the 32 activations
     float *act_scale = reinterpret_cast<float *>(act_hl + 64);             // [4]
     SelectOut *sel = reinterpret_cast<SelectOut *>(act_scale + 4);
@@ -1552,7 +1605,7 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(SliceArgs a) 
     // the table is first read behind the barrier that ends the selection: wave 0 selects, waves 8..15 build meanwhile
     const bool selecting = !is_shared && a.logits;
     if (selecting) build_tables_rep<REP, 8>(lds, strip, wave - 8u, lane); else build_tables_rep<REP, 16>(lds, strip, wave, lane);
-    const uint8_t *tab = lds + (lane % REP) * 16u;
+    const uint8_t *tab = lds + (lane % REP) * 16u, *stab = tab + REP * kMagBytes;
 
     uint32_t expert = 0u;
     float comb;                                        // the slot's weight in the layer's output
@@ -1609,7 +1662,7 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(SliceArgs a) 
     }
     float v[UPW];
 #pragma unroll
-    for (int u = 0; u < UPW; ++u) v[u] = group_dot_rep<REP>(wq[u], ax, tab) * scale_to_f32(wd[u]);
+    for (int u = 0; u < UPW; ++u) v[u] = group_dot_rep<REP, REP>(wq[u], ax, tab, stab) * scale_to_f32(wd[u]);
     const float tot = quad_column_reduce<UPW>(v, lane);
     if (reduced_writer<UPW>(lane)) {
         const uint32_t quad = q0 + (NW / NKC) * reduced_unit<UPW>(lane);
@@ -1648,7 +1701,7 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(SliceArgs a) 
 #pragma unroll
     for (int k = 0; k < DU; ++k) {
         const uint32_t unit = wave + NW * k;
-        if (unit < 8u * NKC) out[64u * unit + lane] = group_dot_rep<REP>(dq[k], ad, tab) * scale_to_f32(dd[k]) * post;
+        if (unit < 8u * NKC) out[64u * unit + lane] = group_dot_rep<REP, REP>(dq[k], ad, tab, stab) * scale_to_f32(dd[k]) * post;
     }
 }
 
@@ -1659,8 +1712,10 @@ __global__ __launch_bounds__(256) void slice_sum_kernel(const float *partial, ui
     __shared__ float4 red[4][8];
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, c8 = tid & 7u, pl = tid >> 3;      // pl 0..31
     const uint32_t col = blockIdx.x * 8u + c8;          // float4 column
-    const float4 *p4 = reinterpret_cast<const float4 *>(partial);
     const uint32_t H4 = H / 4u;
+    const float4 *p4 = reinterpret_cast<const float4 *>(partial) + (uint64_t)blockIdx.y * n_part * H4;      // blockIdx.y = token
+    out += (uint64_t)blockIdx.y * H;
+    if (resid_a) { resid_a += (uint64_t)blockIdx.y * H; resid_b += (uint64_t)blockIdx.y * H; }
     float4 v[8];
     uint32_t n = 0u;
 #pragma unroll
@@ -1696,8 +1751,180 @@ __global__ __launch_bounds__(256) void slice_sum_kernel(const float *partial, ui
     }
 }
 
+// ---------------------------------------------------------------- two to eight tokens on all-IQ2_XXS layers: expert slices per pass
+//
+// The same slices for a small batch whose pairs are grouped by expert. A pass = up to two pairs (tokens) of one expert; one workgroup
+// per (pass, 32 ffn columns): the two tokens ride in rows 0, 1 and 2, 3 of the MFMA's activation operand, so every weight is decoded
+// once for both. A popular expert's tokens spread over several workgroups (its weights come from L2 after the first), the shared
+// expert is one pass per two tokens. Partial vectors land at partial[token][k][column group][hidden] (k = top_k: the shared expert), so
+// that the sum kernel reads one contiguous block per token.
+struct BatchSliceArgs {
+    const uint8_t *experts;
+    uint64_t stride;
+    const uint8_t *down_cm;
+    uint64_t down_stride;
+    const uint8_t *shared;
+    const uint8_t *shared_down_cm;
+    const uint2 *pass_list;        // from the pair sort (GroupJob::pass_list)
+    const uint32_t *n_pass;
+    const float *weights;          // [ntok][top_k] router weights, indexed token * top_k + k
+    const float *scalar;           // [ntok]
+    const _Float16 *xh, *xl;       // [ntok][hidden]
+    const int *xexp;               // [ntok]
+    float *partial;                // [ntok][top_k + 1][ffn / 32][hidden]
+    uint32_t hidden, ffn, top_k, ntok;
+};
+
+// two tokens' results of one group: va for the token in rows 0, 1 of the operand, vb for the one in rows 2, 3
+template <int REP, int SREP>
+__device__ __forceinline__ void group_dot2_rep(uint2 q, const half4_t *ax, const uint8_t *tab, const uint8_t *stab, float &va, float &vb) {
+    float4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (uint32_t l = 0; l < 4u; ++l) {
+        const uint32_t idx = (q.x >> (8u * l)) & 255u, s7 = (q.y >> (7u * l)) & 127u;
+        WeightQuad b0, b1;
+        if constexpr (SREP == 0) place_signs(*reinterpret_cast<const uint4 *>(tab + idx * (16u * REP)), s7, b0, b1);
+        else signed_weights_rep<REP, SREP>(tab, stab, idx, s7, b0, b1);
+        acc = __builtin_amdgcn_mfma_f32_4x4x4f16(ax[2u * l], b0.h, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_4x4x4f16(ax[2u * l + 1u], b1.h, acc, 0, 0, 0);
+    }
+    const float sc = (float)(2u * (q.y >> 28) + 1u);
+    va = (acc[0] + acc[1] * 4.8828125e-4f) * sc;
+    vb = (acc[2] + acc[3] * 4.8828125e-4f) * sc;
+}
+
+// One workgroup per (pass, column group) - the hardware's own dispatch balances the units over the compute units (persistent workgroups
+// that walked a unit list with the next unit's weights requested ahead were measured too: slower at 2, 4 and 8 tokens, their start-up
+// and the coarser balance cost more than the requests they hide).
+// Both tables eight times here (lanes l and l + 8 share a copy and collide now and then): 56 KB of LDS and at most 64 registers per lane,
+// so that two workgroups fit a compute unit and one's weight requests and barriers hide behind the other's arithmetic.
+constexpr int kBatchRep = 16, kBatchSignRep = 0;
+template <int NKC, int REP>
+__global__ __launch_bounds__(kWaves * 64, 8) void batch_slice_kernel(BatchSliceArgs a) {
+    constexpr int NW = kWaves;
+    constexpr int UPW = 16 * NKC / NW;
+    constexpr int DU = (8 * NKC + NW - 1) / NW;
+    constexpr int SREP = kBatchSignRep;
+    extern __shared__ __attribute__((aligned(16))) uint8_t dyn[];
+    uint8_t *lds = dyn;
+    uint8_t *strip = dyn + REP * kMagBytes + SREP * kSignBytes;
+    float *part = reinterpret_cast<float *>(strip + kMagBytes + kSignBytes);      // [2 tokens][NKC][64]
+    _Float16 *act_hl = reinterpret_cast<_Float16 *>(part + 2 * NKC * 64);  // [2 tokens][2 halves][32]
+    float *act_scale = reinterpret_cast<float *>(act_hl + 128);            // [2] (+ 2 unused)
+
+    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
+    const uint32_t H = a.hidden, F = a.ffn, HG = H / 32u, HB = H / 256u, FG = F / 32u, K = a.top_k;
+    const uint32_t g = blockIdx.x, v = blockIdx.y;
+    const uint32_t n_pass = a.n_pass[0];
+    if (v >= n_pass + ((a.ntok + 1u) >> 1)) return;    // the grid covers the largest possible number of passes
+    const bool sh = v >= n_pass;
+    uint2 e;
+    if (sh) {                                          // the shared expert: tokens 2 s, 2 s + 1; k = top_k
+        const uint32_t t0 = 2u * (v - n_pass), t1 = t0 + 1u < a.ntok ? t0 + 1u : t0;
+        e.x = 0xffffu | ((t0 + 1u < a.ntok ? 2u : 1u) << 16);
+        e.y = (t0 << 16) | (t1 << 24);
+    } else {
+        e = a.pass_list[v];
+        if (((e.x >> 16) & 255u) < 2u) e.y = (e.y & 0x00ff00ffu) * 0x101u;      // a lone token: its twin computes the same and is not stored
+    }
+    const uint32_t expert = e.x & 0xffffu, cnt = (e.x >> 16) & 255u, tok0 = (e.y >> 16) & 255u, tok1 = e.y >> 24;
+    const uint32_t k0 = sh ? K : (e.y & 255u) - tok0 * K, k1 = sh ? K : ((e.y >> 8) & 255u) - tok1 * K;
+
+    const uint32_t kc = wave % NKC, q0 = wave / NKC;
+    const uint32_t G = 16u * kc + blk;
+    half4_t ax[8];
+    {
+        const uint32_t t = (j >> 1) ? tok1 : tok0;
+        const _Float16 *src = ((j & 1u) ? a.xl : a.xh) + (uint64_t)t * H + 32u * G;
+#pragma unroll
+        for (int s8 = 0; s8 < 8; ++s8) ax[s8] = *reinterpret_cast<const half4_t *>(src + 4 * s8);
+    }
+    const uint8_t *ex = sh ? a.shared : a.experts + (uint64_t)expert * a.stride;
+    const uint8_t *dn = sh ? a.shared_down_cm : a.down_cm + (uint64_t)expert * a.down_stride;
+    const uint64_t gate_bytes = (uint64_t)F * HG * 8u + (uint64_t)F * HB * 2u;
+    uint2 wq[UPW];
+    uint32_t wd[UPW];
+#pragma unroll
+    for (int u = 0; u < UPW; ++u) {
+        const uint32_t quad = q0 + (NW / NKC) * u;
+        const uint32_t r = 32u * g + 4u * (quad & 7u) + j;
+        const uint8_t *mat = ex + (quad < 8u ? 0u : gate_bytes);
+        wq[u] = reinterpret_cast<const uint2 *>(mat)[(uint64_t)r * HG + G];
+        wd[u] = reinterpret_cast<const uint16_t *>(mat + (uint64_t)F * HG * 8u)[(uint64_t)r * HB + (G >> 3)];
+    }
+    const uint2 *down_qs = reinterpret_cast<const uint2 *>(dn) + (uint64_t)g * H;
+    const uint16_t *down_ds = reinterpret_cast<const uint16_t *>(dn + (uint64_t)FG * H * 8u) + (uint64_t)(g >> 3) * H;
+    uint2 dq[DU];
+    uint32_t dd[DU];
+#pragma unroll
+    for (int kk = 0; kk < DU; ++kk) {
+        const uint32_t unit = wave + NW * kk;
+        const uint32_t r = 64u * (unit < 8u * NKC ? unit : 0u) + lane;
+        dq[kk] = down_qs[r];
+        dd[kk] = down_ds[r];
+    }
+    const float w0 = sh ? a.scalar[tok0] : a.weights[tok0 * K + k0], w1 = sh ? a.scalar[tok1] : a.weights[tok1 * K + k1];
+    const float xs0 = 0.125f * exp2i(a.xexp[tok0]), xs1 = 0.125f * exp2i(a.xexp[tok1]);
+    build_tables_rep<REP, 16, SREP>(lds, strip, wave, lane);
+    const uint8_t *tab = lds + (lane % REP) * 16u, *stab = lds + REP * kMagBytes + (lane % (SREP ? SREP : 1)) * 16u;
+    __syncthreads();                                   // tables
+
+    float va[UPW], vb[UPW];
+#pragma unroll
+    for (int u = 0; u < UPW; ++u) {
+        group_dot2_rep<REP, SREP>(wq[u], ax, tab, stab, va[u], vb[u]);
+        const float d = scale_to_f32(wd[u]);
+        va[u] *= d;
+        vb[u] *= d;
+    }
+    const float ta = quad_column_reduce<UPW>(va, lane), tb = quad_column_reduce<UPW>(vb, lane);
+    if (reduced_writer<UPW>(lane)) {
+        const uint32_t quad = q0 + (NW / NKC) * reduced_unit<UPW>(lane);
+        part[kc * 64u + 4u * quad + j] = ta;
+        part[NKC * 64u + kc * 64u + 4u * quad + j] = tb;
+    }
+    __syncthreads();
+    if (tid < 64u) {
+        const uint32_t t = tid >> 5, c = tid & 31u;
+        const float *pt = part + t * NKC * 64u;
+        float gsum = 0.0f, usum = 0.0f;
+#pragma unroll
+        for (int kk = 0; kk < NKC; ++kk) { gsum += pt[kk * 64 + c]; usum += pt[kk * 64 + 32 + c]; }
+        const float xs = t ? xs1 : xs0;
+        gsum *= xs;
+        usum *= xs;
+        const float act = (gsum / (1.0f + expf(-gsum))) * usum;
+        float amax = fabsf(act);
+#pragma unroll
+        for (int o = 16; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+        const int ee = prescale_exp(amax);
+        split_hi_lo(act, exp2i(-ee), act_hl + t * 64u + c, act_hl + t * 64u + 32u + c);
+        if (c == 0u) act_scale[t] = exp2i(ee);
+    }
+    __syncthreads();
+    half4_t ad[8];
+    {
+        const _Float16 *src = act_hl + (j >> 1) * 64u + (j & 1u) * 32u;
+#pragma unroll
+        for (int s8 = 0; s8 < 8; ++s8) ad[s8] = *reinterpret_cast<const half4_t *>(src + 4 * s8);
+    }
+    const float post0 = act_scale[0] * w0 * 0.125f, post1 = act_scale[1] * w1 * 0.125f;
+    float *out0 = a.partial + ((uint64_t)(tok0 * (K + 1u) + k0) * FG + g) * H, *out1 = a.partial + ((uint64_t)(tok1 * (K + 1u) + k1) * FG + g) * H;
+#pragma unroll
+    for (int kk = 0; kk < DU; ++kk) {
+        const uint32_t unit = wave + NW * kk;
+        if (unit < 8u * NKC) {
+            float da, db;
+            group_dot2_rep<REP, SREP>(dq[kk], ad, tab, stab, da, db);
+            const float d = scale_to_f32(dd[kk]);
+            out0[64u * unit + lane] = da * d * post0;
+            if (cnt > 1u) out1[64u * unit + lane] = db * d * post1;
+        }
+    }
+}
+
 constexpr int kSliceRep = 16;
-inline size_t slice_lds_bytes(int nkc, int rep) { return (size_t)(rep + 1) * kMagBytes + (size_t)nkc * 64u * 4u + 128u + 16u + sizeof(SelectOut); }
+inline size_t slice_lds_bytes(int nkc, int rep) { return (size_t)(rep + 1) * (kMagBytes + kSignBytes) + (size_t)nkc * 64u * 4u + 128u + 16u + sizeof(SelectOut); }
 
 hipError_t launch_expert_slices(const void *experts, uint64_t stride, const void *down_cm, uint64_t down_stride, const void *shared, const void *shared_down_cm,
                                 const float *logits, const uint32_t *ids_in, const float *weights_in, const float *scalar_in, uint32_t *ids_out,
@@ -1733,6 +1960,40 @@ hipError_t launch_expert_slices(const void *experts, uint64_t stride, const void
     if (e != hipSuccess) return e;
     prof_set_stage(ST_SLICE_SUM);
     REDHIP_LAUNCH(slice_sum_kernel, dim3(hidden / 32u), dim3(256), 0, s, partial, (top_k + 1u) * (ffn / 32u), hidden, out, block_context().resid_a, block_context().resid_b);
+    return hipGetLastError();
+}
+
+hipError_t launch_batch_slices(const void *experts, uint64_t stride, const void *down_cm, uint64_t down_stride, const void *shared, const void *shared_down_cm,
+                               const void *pass_list, const uint32_t *n_pass, const float *weights, const float *scalar, const void *xh, const void *xl,
+                               const int *xexp, float *partial, float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, hipStream_t s) {
+    if (!fused_iq2_supported(hidden, ffn) || hidden % 32u || !ntok || ntok > 16u || ntok * top_k > 128u || !pass_list || !n_pass) return hipErrorInvalidValue;
+    const BatchSliceArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(down_cm), down_stride, static_cast<const uint8_t *>(shared),
+                           static_cast<const uint8_t *>(shared_down_cm), static_cast<const uint2 *>(pass_list), n_pass, weights, scalar,
+                           static_cast<const _Float16 *>(xh), static_cast<const _Float16 *>(xl), xexp, partial, hidden, ffn, top_k, ntok};
+    const dim3 grid_dim(ffn / 32u, ntok * top_k + (ntok + 1u) / 2u);      // every pair a pass of its own at most, then the shared expert's passes
+#define REDHIP_BSLICE(NKC)                                                                                                             \
+    do {                                                                                                                               \
+        static bool attr = false;                                                                                                       \
+        const size_t dyn = (size_t)kBatchRep * kMagBytes + (size_t)kBatchSignRep * kSignBytes + kMagBytes + kSignBytes + (size_t)2u * NKC * 64u * 4u + 256u + 16u; \
+        if (!attr) {                                                                                                                    \
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(batch_slice_kernel<NKC, kBatchRep>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn); \
+            if (e != hipSuccess) return e;                                                                                              \
+            attr = true;                                                                                                                \
+        }                                                                                                                               \
+        REDHIP_LAUNCH((batch_slice_kernel<NKC, kBatchRep>), grid_dim, dim3(kWaves * 64), dyn, s, a);                                      \
+    } while (0)
+    prof_set_stage(ST_FUSED_EXPERTS);
+    switch (hidden / 512u) {
+        case 1: REDHIP_BSLICE(1); break;
+        case 2: REDHIP_BSLICE(2); break;
+        case 4: REDHIP_BSLICE(4); break;
+        default: return hipErrorInvalidValue;      // (hidden 4096 would spill registers: such layers take their batches on other kernels)
+    }
+#undef REDHIP_BSLICE
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    prof_set_stage(ST_SLICE_SUM);
+    REDHIP_LAUNCH(slice_sum_kernel, dim3(hidden / 32u, ntok), dim3(256), 0, s, partial, (top_k + 1u) * (ffn / 32u), hidden, out, block_context().resid_a, block_context().resid_b);
     return hipGetLastError();
 }
 

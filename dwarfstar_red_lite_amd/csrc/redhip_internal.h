@@ -216,6 +216,8 @@ struct GroupJob {
     float *pair_weight;
     uint32_t *tok_pair, *n_unique;
     uint32_t *status = nullptr;      // RouteGuard::status of the call (ids are clamped to n_expert - 1 either way)
+    uint2 *pass_list = nullptr;      // optional: the pass list of the batched expert-slice kernel, at most ntok * top_k entries, and
+    uint32_t *n_pass = nullptr;      // their number
 };
 
 // Selection inside the batched gate/up kernel: logits [ntok][n_expert + 1] in, the routing out (ids, weights [ntok][top_k], scalar [ntok]);
@@ -289,6 +291,11 @@ hipError_t launch_expert_slices(const void *experts, uint64_t stride, const void
                                 const float *logits, const uint32_t *ids_in, const float *weights_in, const float *scalar_in, uint32_t *ids_out,
                                 float *weights_out, float *scalar_out, const void *xh, const void *xl, const int *xexp, float *partial, float *out,
                                 uint32_t hidden, uint32_t ffn, uint32_t n_expert, uint32_t top_k, hipStream_t s);
+// the same for 2..16 tokens (at most 128 pairs) whose pairs are grouped by expert: pass_list / n_pass from the pair sort (GroupJob), weights
+// [ntok][top_k] and scalar [ntok] of the routing; partial [ntok][top_k + 1][ffn / 32][hidden]
+hipError_t launch_batch_slices(const void *experts, uint64_t stride, const void *down_cm, uint64_t down_stride, const void *shared, const void *shared_down_cm,
+                               const void *pass_list, const uint32_t *n_pass, const float *weights, const float *scalar, const void *xh, const void *xl,
+                               const int *xexp, float *partial, float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, hipStream_t s);
 // single token: out[r] = sum_k weights[k] * down_{ids[k]}[r] . act[k] + scalar * shared_down[r] . act[top_k], k in order
 hipError_t launch_down_combine(const void *experts, uint64_t stride, const void *shared, const uint32_t *ids, const float *weights,
                                const float *scalar, const void *act_h, const void *act_l, const int *act_exp, float *out,

@@ -50,7 +50,9 @@ struct Moe {
     uint32_t gu_type, dn_type, sh_gu_type, sh_dn_type;
     uint64_t gate_bytes, down_bytes, expert_stride;          // routed expert
     uint64_t down_cm_stride() const { return (down_bytes + 255u) & ~255ull; }
-    float *partial = nullptr;                                // [top_k + 1][ffn / 32][hidden]: partial output vectors of the one-token expert slices
+    float *partial = nullptr;                                // [tokens <= 8][top_k + 1][ffn / 32][hidden]: partial output vectors of the expert slices
+    uint2 *pass_list = nullptr;                              // small batches: the passes (two pairs of one expert) of the batched expert slices
+    uint32_t *n_pass = nullptr;
     uint64_t pk_gate_bytes = 0;                              // one gate / up matrix in the packed streams of the one-token kernel
     const int8_t *gu_grid = nullptr, *dn_grid = nullptr;     // device copies of the caller's codebooks (IQ2_XS / IQ1_M matrices)
     uint64_t sh_gate_bytes, sh_down_bytes;                   // shared expert
@@ -245,6 +247,13 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
             prof_set_stage(ST_GROUP);
             HIP_OK(launch_group_pairs(ids, weights, ntok, c.top_k, c.n_expert, m->uid, m->expert_start, m->pair_token, m->pair_weight,
                                       m->tok_pair, m->n_unique, s), "grouping launch");
+        }
+        if (m->small_batch(ntok) && grouped && !select_here) {     // the caller's routing, sorted (with its pass list) by the prep launch: expert slices per pass
+            const Layer &L = m->layers[layer];
+            HIP_OK(launch_batch_slices(L.packed, m->expert_stride, L.down_cm, m->down_cm_stride(), L.shared_packed, L.shared_down_cm, m->pass_list, m->n_pass,
+                                       weights, m->scalar, m->xh, m->xl, m->xexp, m->partial, out, c.hidden, c.ffn, c.top_k, ntok, s), "batched expert slice launch");
+            prof_set_stage(ST_OTHER);
+            return 1;
         }
         if (m->small_batch(ntok)) {     // packed IQ2_XXS, MFMA kernels; xh / xl / xexp / scalar come from the router or prep kernel
             const Layer &L = m->layers[layer];
@@ -448,8 +457,8 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
         }
     }
     const size_t T = c.max_tokens;
-    const size_t partial_bytes = m->fused ? align256((size_t)(c.top_k + 1u) * (c.ffn / 32u) * c.hidden * 4u) : 0u;
-    const size_t ws_bytes = partial_bytes + align256(4u) + align256(T * c.hidden * 4u) + align256(T * (c.n_expert + 1u) * 4u) + 2u * align256(T * c.top_k * 4u) + align256(T * 4u) +
+    const size_t partial_bytes = m->fused ? align256((size_t)(c.max_tokens < 8u ? c.max_tokens : 8u) * (c.top_k + 1u) * (c.ffn / 32u) * c.hidden * 4u) : 0u;
+    const size_t ws_bytes = partial_bytes + align256(8u * 128u) + align256(4u) + align256(4u) + align256(T * c.hidden * 4u) + align256(T * (c.n_expert + 1u) * 4u) + 2u * align256(T * c.top_k * 4u) + align256(T * 4u) +
                             align256(T * c.top_k * c.ffn * 4u) + align256(T * c.ffn * 4u) +
                             2u * align256(2u * T * c.hidden) + align256(4u * T) + 2u * align256(2u * T * (c.top_k + 1u) * c.ffn) +
                             align256(4u * T * (c.top_k + 1u) * (c.ffn / 32u)) +
@@ -465,6 +474,8 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
     uint8_t *w = m->ws;
     m->status = reinterpret_cast<uint32_t *>(w); w += align256(4u);
     if (partial_bytes) { m->partial = reinterpret_cast<float *>(w); w += partial_bytes; }
+    m->pass_list = reinterpret_cast<uint2 *>(w); w += align256(8u * 128u);
+    m->n_pass = reinterpret_cast<uint32_t *>(w); w += align256(4u);
     m->xn = reinterpret_cast<float *>(w); w += align256(T * c.hidden * 4u);
     m->logits = reinterpret_cast<float *>(w); w += align256(T * (c.n_expert + 1u) * 4u);
     m->ids = reinterpret_cast<uint32_t *>(w); w += align256(T * c.top_k * 4u);
@@ -719,7 +730,8 @@ int redhip_moe_experts(redhip_moe_t h, uint32_t layer, const float *x_dev, uint3
         // batches whose pairs are grouped by expert next: the pair sort rides in the same launch as one more workgroup
         // (with the routing given, grouping pays from two tokens on: the pair sort costs no launch of its own)
         const bool to_group = m->small_batch(ntok) || m->grouped_mixed(ntok, 2u);
-        const GroupJob job{ids_dev, weights_dev, ntok, m->cfg.top_k, m->cfg.n_expert, m->uid, m->expert_start, m->pair_token, m->pair_weight, m->tok_pair, m->n_unique, m->status};
+        const GroupJob job{ids_dev, weights_dev, ntok, m->cfg.top_k, m->cfg.n_expert, m->uid, m->expert_start, m->pair_token, m->pair_weight, m->tok_pair, m->n_unique, m->status,
+                           m->small_batch(ntok) ? m->pass_list : nullptr, m->small_batch(ntok) ? m->n_pass : nullptr};
         bool grouped = false;
         if (m->mixed && m->packed_gu() && (ntok == 1u || m->small_batch_mixed(ntok)) && L.dense_gu && (nv == 2u || nv == 4u || nv == 8u || nv == 16u)) {
             // one token or a small batch on a mixed layout: the kernels take the shared expert's gate | up products as an input: one f32
