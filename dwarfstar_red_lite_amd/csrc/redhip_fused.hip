@@ -393,10 +393,10 @@ __device__ __forceinline__ float norm_scale(double ss, uint32_t n, float eps) { 
 
 // F32 router: one wave per row (row n_expert is the shared expert's gate vector), the row and x read as float4
 // with lanes interleaved; every wave sees all of x, so the pre-scale exponent needs no extra pass. blockIdx.y = token.
-template <int NV>          // float4 per lane: hidden = 256 * NV
-__global__ __launch_bounds__(256) void router_f32_kernel(const float *w, RouterArgs a) {
+template <int NV, int WPB = 4>          // float4 per lane: hidden = 256 * NV; WPB waves (rows) per workgroup
+__global__ __launch_bounds__(WPB * 64) void router_f32_kernel(const float *w, RouterArgs a) {
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63u, H = a.hidden, tok = blockIdx.y;
-    const uint32_t r = blockIdx.x * 4u + wave;
+    const uint32_t r = blockIdx.x * WPB + wave;
     const uint32_t n_rows = a.n_expert + 1u + (a.sh_dense ? 2u * a.ffn : 0u);      // router rows, the gate vector, then the shared expert's gate | up rows
     const float4 *wr = reinterpret_cast<const float4 *>(r < a.n_expert ? w + (uint64_t)r * H : r == a.n_expert ? a.gate_inp
                                                         : a.sh_dense + (uint64_t)(r < n_rows ? r - a.n_expert - 1u : 0u) * H);
@@ -627,6 +627,9 @@ hipError_t launch_router_gemv(uint32_t router_type, const void *w, const float *
                  with_shared ? static_cast<const uint8_t *>(sh_q6k) : nullptr, with_dense ? sh_dense : nullptr, sh_gu, ffn, bc.branch, bc.norm_w, bc.eps,
                  bc.xn_out, scalar_out};
     const dim3 grid((n_expert + 1u + (with_dense ? 2u * ffn : 0u) + 3u) / 4u, ntok);
+    // F32 rows: a multiple of eight workgroups per token. Workgroups go to the eight XCDs in turn, so a row block then lands on the same
+    // XCD for every token of the batch and all tokens but the first find it in that XCD's L2 instead of fetching the rows once per XCD.
+    const dim3 grid8((grid.x + 7u) & ~7u, ntok);
     // with the shared expert's rows behind the router's (1537 rows at the benchmark shape) a row is read once for the whole batch; the
     // router's own 513 rows are quicker one token per grid layer (their re-reads hit the L2)
     if (router_type == T_F32 && with_dense && ntok >= 2u && (size_t)ntok * hidden * 4u <= 64u * 1024u) {
@@ -660,10 +663,10 @@ hipError_t launch_router_gemv(uint32_t router_type, const void *w, const float *
     if (router_type == T_F32) {
         const float *wf = static_cast<const float *>(w);
         switch (hidden / 256u) {
-            case 2: REDHIP_LAUNCH(router_f32_kernel<2>, grid, dim3(256), 0, s, wf, a); break;
-            case 4: REDHIP_LAUNCH(router_f32_kernel<4>, grid, dim3(256), 0, s, wf, a); break;
-            case 8: REDHIP_LAUNCH(router_f32_kernel<8>, grid, dim3(256), 0, s, wf, a); break;
-            case 16: REDHIP_LAUNCH(router_f32_kernel<16>, grid, dim3(256), 0, s, wf, a); break;
+            case 2: REDHIP_LAUNCH(router_f32_kernel<2>, grid8, dim3(256), 0, s, wf, a); break;
+            case 4: REDHIP_LAUNCH(router_f32_kernel<4>, grid8, dim3(256), 0, s, wf, a); break;
+            case 8: REDHIP_LAUNCH(router_f32_kernel<8>, grid8, dim3(256), 0, s, wf, a); break;      // (one or two rows per workgroup instead of four: no difference)
+            case 16: REDHIP_LAUNCH(router_f32_kernel<16>, grid8, dim3(256), 0, s, wf, a); break;
             default: return hipErrorInvalidValue;
         }
     } else if (router_type == T_Q6_K) {
@@ -1005,6 +1008,35 @@ hipError_t launch_select(const float *logits, uint32_t ntok, uint32_t n_expert, 
     // few tokens: one workgroup of 16 waves each (short chains per wave); many tokens: one wave each (the machine is full either way)
     if (ntok <= 64u) REDHIP_LAUNCH(select_block_kernel, dim3(ntok), dim3(kWaves * 64), 0, s, logits, n_expert, top_k, ids, weights, scalar, probs);
     else REDHIP_LAUNCH(select_kernel, dim3(ntok), dim3(64), 0, s, logits, n_expert, top_k, ids, weights, scalar, probs);
+    return hipGetLastError();
+}
+
+// Small batches routed by the layer's own router: wave t selects the experts of token t, then the whole workgroup sorts the pairs by
+// expert (with the pass list of the batched expert-slice kernel). One workgroup; logits [ntok][n_expert + 1].
+__global__ __launch_bounds__(kWaves * 64) void select_group_kernel(const float *logits, uint32_t ntok, uint32_t E, uint32_t K, uint32_t *ids, float *weights,
+                                                                   float *scalar, GroupJob job) {
+    __shared__ SelectOut sel[8];
+    __shared__ uint32_t group_lds[kGroupLdsWords];
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63u;
+    if (wave < ntok) {
+        const float *l = logits + (uint64_t)wave * (E + 1u);
+        if (E <= 512u) wave_select_topk<8>(l, E, K, &sel[wave]); else wave_select_topk<16>(l, E, K, &sel[wave]);
+        wave_lds_sync();
+        if (lane < K) { ids[wave * K + lane] = sel[wave].ids[lane]; weights[wave * K + lane] = sel[wave].w[lane]; }
+        if (lane == 0u) scalar[wave] = sel[wave].scalar;
+    }
+    __syncthreads();
+    group_small(job, group_lds, [&](uint32_t t, uint32_t k) { return sel[t].ids[k]; }, [&](uint32_t t, uint32_t k) { return sel[t].w[k]; });
+}
+
+hipError_t launch_select_group(const float *logits, uint32_t ntok, uint32_t n_expert, uint32_t top_k, uint32_t *ids, float *weights, float *scalar,
+                               const GroupJob &job, hipStream_t s) {
+    if (!ntok || ntok > 8u || !n_expert || n_expert > 1024u || !top_k || top_k > 16u || top_k > n_expert || ntok * top_k > 128u) return hipErrorInvalidValue;
+    GroupJob gj = job;
+    gj.ids = nullptr;
+    gj.weights = nullptr;
+    gj.ntok = ntok; gj.top_k = top_k; gj.n_expert = n_expert;
+    REDHIP_LAUNCH(select_group_kernel, dim3(1), dim3(kWaves * 64), 0, s, logits, ntok, n_expert, top_k, ids, weights, scalar, gj);
     return hipGetLastError();
 }
 

@@ -240,6 +240,9 @@ hipError_t launch_router_gemv(uint32_t router_type, const void *w, const float *
 // softmax top-k of logits [ntok][n_expert + 1]; scalar[t] = sigmoid(logits[t][n_expert]); optional probs [ntok][n_expert]
 hipError_t launch_select(const float *logits, uint32_t ntok, uint32_t n_expert, uint32_t top_k, uint32_t *ids, float *weights, float *scalar,
                          float *probs, hipStream_t s);
+// 2..8 tokens: softmax top-k per token and the pair sort (outputs of `job`, pass list included) in one launch of one workgroup
+hipError_t launch_select_group(const float *logits, uint32_t ntok, uint32_t n_expert, uint32_t top_k, uint32_t *ids, float *weights, float *scalar,
+                               const GroupJob &job, hipStream_t s);
 // fp16 split of x and the scalar gate without a router; with a job that fits, one more workgroup does the pair sort (*job_done)
 hipError_t launch_prep(const float *x, const float *gate_inp, uint32_t ntok, uint32_t hidden, void *xh, void *xl, int *xexp, float *scalar, hipStream_t s,
                        const GroupJob *job = nullptr, bool *job_done = nullptr);

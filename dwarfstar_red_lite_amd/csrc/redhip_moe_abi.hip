@@ -353,6 +353,16 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
     return 1;
 }
 
+// a small batch on an all-IQ2_XXS layer behind the router launch: selection + pair sort (one launch), expert slices per pass, their sum
+int select_group_slices(Moe *m, uint32_t layer, const float *x, uint32_t ntok, float *out, hipStream_t s) {
+    const redhip_moe_config &c = m->cfg;
+    const GroupJob job{nullptr, nullptr, ntok, c.top_k, c.n_expert, m->uid, m->expert_start, m->pair_token, m->pair_weight, m->tok_pair, m->n_unique, nullptr,
+                       m->pass_list, m->n_pass};
+    prof_set_stage(ST_ROUTE_SELECT);
+    HIP_OK(launch_select_group(m->logits, ntok, c.n_expert, c.top_k, m->ids, m->weights, m->scalar, job, s), "selection + pair sort launch");
+    return experts_enqueue(m, layer, x, ntok, m->ids, m->weights, out, s, false, true);
+}
+
 }  // namespace
 
 extern "C" {
@@ -773,6 +783,7 @@ int redhip_moe_forward(redhip_moe_t h, uint32_t layer, const float *x_dev, uint3
     const int routed = redhip_moe_route(h, layer, x_dev, ntok, nullptr, nullptr, nullptr, stream);
     m->skip_select = false;
     if (!routed) return 0;
+    if (m->small_batch(ntok)) return select_group_slices(m, layer, x_dev, ntok, out_dev, static_cast<hipStream_t>(stream));
     return experts_enqueue(m, layer, x_dev, ntok, m->ids, m->weights, out_dev, static_cast<hipStream_t>(stream), select_in_gateup || group_in_select, group_in_select);
 }
 
@@ -819,7 +830,8 @@ int redhip_moe_forward_block(redhip_moe_t h, uint32_t layer, const float *x_dev,
             if (ok) {
             bc.resid_a = x_dev;                              // the path's last kernel adds x + branch to its output
             bc.resid_b = branch_dev;
-            ok = experts_enqueue(m, layer, m->xn, ntok, m->ids, m->weights, x_out_dev, s, select_in_gateup || group_in_select, group_in_select);
+            ok = m->small_batch(ntok) ? select_group_slices(m, layer, m->xn, ntok, x_out_dev, s)
+                                      : experts_enqueue(m, layer, m->xn, ntok, m->ids, m->weights, x_out_dev, s, select_in_gateup || group_in_select, group_in_select);
         }
     }
     bc = BlockContext{};
