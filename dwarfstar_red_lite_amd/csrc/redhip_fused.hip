@@ -5,14 +5,18 @@
 // One token, three launches per layer:
 //   router_*_kernel        logits of every expert (plus the shared expert's gate logit) and the fp16 split of x; for a
 //                          Q6_K shared expert also its gate and up products, in extra workgroups
-//   gateup_select_kernel   every routed workgroup repeats the cheap softmax top-k from the logits on one wave, then
-//                          computes 32 gate rows + 32 up rows of one selected expert (or the shared expert) ->
-//                          SwiGLU -> fp16 halves
-//   down_combine_kernel    8 output rows per workgroup, one wave per selected expert; weighted sum in selection
-//                          order + shared expert * scalar gate: deterministic (down_combine_raw_kernel when the down
-//                          matrices are raw IQ3_S / Q6_K rows)
-// Two to eight tokens: gateup_batch_kernel (every workgroup repeats the selection per token and the pair sort, then persistent
-// workgroups read every distinct expert once), down_batch_kernel.
+//   all matrices IQ2_XXS:
+//   expert_slice_kernel    one workgroup per (slot, 32 ffn columns): softmax top-k on one wave, the slot's 32 gate + 32 up rows,
+//                          SwiGLU, then the matching 32 columns of its down matrix (column-sliced copy), weighted -> a partial
+//                          output vector per workgroup
+//   slice_sum_kernel       the (top_k + 1) * ffn / 32 partial vectors added in a fixed order: deterministic
+//   mixed layouts:
+//   gateup_select_kernel   the same selection, then 32 gate rows + 32 up rows of one selected expert -> SwiGLU -> fp16 halves
+//   down_combine_*_kernel  8 output rows per workgroup, one wave per selected expert; weighted sum in selection order + shared
+//                          expert * scalar gate (word-packed IQ3_S / stream-packed IQ2_XS, IQ1_M on the MFMA, other types raw rows)
+// Two to eight tokens: pairs grouped by expert (group_small, in the first launch or with the selection in one of its own), then
+// batch_slice_kernel + slice_sum_kernel (all IQ2_XXS: a pass = two tokens of one expert) or gateup_batch_kernel + down_batch_*_kernel
+// (mixed layouts: persistent workgroups, every distinct expert read once).
 //
 // Arithmetic: a weight is (sign * magnitude * (2*scale+1)) * d/8; the eight magnitudes of a grid entry are exact fp16
 // values from an LDS table, the sign bits are placed by integer arithmetic; an activation vector is split into two
@@ -1420,85 +1424,6 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_select_kernel(GateUpArgs a
     }
 }
 
-struct DownArgs {
-    const uint8_t *experts;
-    uint64_t stride;
-    const uint8_t *shared;
-    const uint32_t *ids;       // [top_k]
-    const float *weights;      // [top_k]
-    const float *scalar;       // [1]
-    const _Float16 *act_h, *act_l;
-    const int *act_exp;
-    float *out;                // [hidden]
-    uint32_t hidden, ffn, top_k;
-    const float *resid_a, *resid_b;     // when set: out[i] = (resid_a[i] + resid_b[i]) + layer output
-    uint32_t id_limit;                  // ids are clamped to id_limit - 1 (RouteGuard)
-};
-
-// 8 output rows per workgroup; wave s (< top_k + 1) owns slot s: both row quads of the workgroup against all
-// ffn columns (ffn = 512: 16 groups = the 16 lane blocks of a wave). Slots are then added in selection order.
-__global__ __launch_bounds__(kWaves * 64) void down_combine_kernel(DownArgs a) {
-    __shared__ __attribute__((aligned(16))) uint8_t lds[kMagBytes];
-    __shared__ float part[17 * 8], comb[17];
-    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
-    const uint32_t H = a.hidden, F = a.ffn, FG = F / 32u, FB = F / 256u, n_slot = a.top_k + 1u;
-    const uint64_t grid_entry = tid < 256u ? redhip_iq2xxs_grid[tid] : 0ull;
-    const uint32_t row0 = 8u * blockIdx.x;
-    float tot[2] = {0.0f, 0.0f};
-    uint2 dq[2][2];            // [row quad][column chunk of 16 groups] (ffn <= 1024)
-    uint32_t dd[2][2];
-    const uint32_t n_chunk = (FG + 15u) / 16u;
-    const bool active = wave < n_slot;
-    const uint8_t *ex = nullptr;
-    if (active) {
-        ex = wave < a.top_k ? a.experts + (uint64_t)guarded_id(a.ids[wave], a.id_limit, nullptr) * a.stride : a.shared;
-        const uint64_t gate_bytes = (uint64_t)F * (H / 32u) * 8u + (uint64_t)F * (H / 256u) * 2u;
-        const uint2 *qs = reinterpret_cast<const uint2 *>(ex + 2u * gate_bytes);                         // [hidden][FG]
-        const uint16_t *ds = reinterpret_cast<const uint16_t *>(ex + 2u * gate_bytes + (uint64_t)H * FG * 8u);   // [hidden][FB]
-#pragma unroll
-        for (int q = 0; q < 2; ++q)
-#pragma unroll
-            for (int c = 0; c < 2; ++c) {
-                const uint32_t r = row0 + 4u * q + j, G = 16u * c + blk;
-                if ((uint32_t)c < n_chunk && G < FG) { dq[q][c] = qs[(uint64_t)r * FG + G]; dd[q][c] = ds[(uint64_t)r * FB + (G >> 3)]; }
-            }
-    }
-    // activations and combine weights are requested before the table barrier: nothing below waits for memory twice
-    half4_t ax[2][8];
-    float sc[2] = {0.0f, 0.0f};
-    if (active) {
-#pragma unroll
-        for (int c = 0; c < 2; ++c) {
-            const uint32_t G = 16u * c + blk;
-            if ((uint32_t)c < n_chunk && G < FG) {
-                load_act_operand(ax[c], a.act_h + (uint64_t)wave * F + 32u * G, a.act_l + (uint64_t)wave * F + 32u * G, j);
-                sc[c] = exp2i(a.act_exp[wave * FG + G]);
-            }
-        }
-    }
-    if (tid < n_slot) comb[tid] = 0.125f * (tid < a.top_k ? a.weights[tid] : a.scalar[0]);
-    build_tables(lds, tid, grid_entry);
-    __syncthreads();
-    if (active) {
-#pragma unroll
-        for (int c = 0; c < 2; ++c) {
-            const uint32_t G = 16u * c + blk;
-            if ((uint32_t)c < n_chunk && G < FG) {
-#pragma unroll
-                for (int q = 0; q < 2; ++q) tot[q] += group_dot(dq[q][c], ax[c], lds) * scale_to_f32(dd[q][c]) * sc[c];
-            }
-        }
-        const float r = quad_column_reduce<2>(tot, lane);
-        if (reduced_writer<2>(lane)) part[wave * 8u + 4u * reduced_unit<2>(lane) + j] = r;
-    }
-    __syncthreads();
-    if (tid < 8u) {
-        float sum = 0.0f;
-        for (uint32_t s = 0; s < n_slot; ++s) sum = fmaf(comb[s], part[s * 8u + tid], sum);      // selection order, the shared expert last
-        a.out[row0 + tid] = a.resid_a ? (a.resid_a[row0 + tid] + a.resid_b[row0 + tid]) + sum : sum;
-    }
-}
-
 // ---------------------------------------------------------------- one token on all-IQ2_XXS layers: expert slices
 //
 // One workgroup per (slot, 32 ffn columns): it selects (or takes the caller's routing), multiplies its 32 gate rows and 32 up rows
@@ -2092,7 +2017,7 @@ __device__ __forceinline__ void shared_rows_dense(const float *shared, uint32_t 
 }
 
 // Down + combine when the down matrices are not IQ2_XXS (mixed-precision layouts: IQ3_S routed, Q6_K shared): same
-// work split as down_combine_kernel (8 rows per workgroup, wave = slot, lane = (32-column chunk, row)), weights
+// 8 output rows per workgroup, wave = slot, lane = (32-column chunk, row); weights
 // decoded from the raw GGUF rows and multiplied in f32 against the activation rebuilt from its fp16 halves.
 struct DownRawArgs {
     const uint8_t *experts;    // expert e's raw down rows at experts + e * stride
@@ -2334,7 +2259,7 @@ __device__ __forceinline__ void iq3s_group_dot(uint4 q, const half4_t *ax, const
 }
 
 // Down + combine of one token on a mixed layout whose routed down matrices are word-packed IQ3_S: 8 output rows per workgroup, wave s <
-// top_k owns the selected expert s (both row quads against all ffn columns, as down_combine_kernel), wave top_k the shared expert, read
+// top_k owns the selected expert s (both row quads of the workgroup against all ffn columns), wave top_k the shared expert, read
 // from its dense f32 copy [hidden][ffn]. blockIdx.y = token (small batches run one grid layer per token).
 struct DownWordsArgs {
     const uint8_t *experts;    // word-packed (IQ3_S) or stream-packed (IQ2_XS, IQ1_M: as their gate / up matrices) down matrix of expert e at experts + e * stride
@@ -2767,119 +2692,6 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_batch_kernel(BatchArgs a) 
     }
 }
 
-// Workgroup = 8 output rows; wave w owns the groups u = w, w + 16, ... (the last one is the shared expert) and,
-// for each, every pair of tokens that selected it. All weights of the wave's groups are requested at once, right at
-// the start, and the activations of a group while the one before it is computed, so the memory round trips overlap
-// instead of adding up. Per-pair partial rows meet in LDS and each token's sum is taken in its own selection order.
-template <int MAXPAIR, int NCH, int GPW>     // GPW: groups of a wave whose weights are in registers at once
-__global__ __launch_bounds__(kWaves * 64) void down_batch_kernel(BatchArgs a) {
-    __shared__ __attribute__((aligned(16))) uint8_t lds[kMagBytes];
-    __shared__ float part[MAXPAIR * 8];
-    const uint32_t tid = threadIdx.x, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
-    const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
-    const uint32_t H = a.hidden, F = a.ffn, FG = F / 32u, FB = F / 256u, P = a.ntok * a.top_k;
-    const uint64_t grid_entry = tid < 256u ? redhip_iq2xxs_grid[tid] : 0ull;
-    const uint32_t row0 = 8u * blockIdx.x, U = __builtin_amdgcn_readfirstlane(a.n_unique[0]);
-    const uint32_t S = (a.ntok + 1u) / 2u;           // the shared expert as S groups of two tokens: one pass each, on S different waves
-    const uint64_t down_off = 2u * ((uint64_t)F * (H / 32u) * 8u + (uint64_t)F * (H / 256u) * 2u), qs_bytes = (uint64_t)H * FG * 8u;
-
-    uint2 wq[GPW][NCH][2];
-    uint32_t wd[GPW][NCH], gp0[GPW], gp1[GPW];      // wd: the two rows' block scales, 16 bits each
-    // metadata and weights of groups first, first + 16, ...; indices are clamped so that every request is valid
-    auto request = [&](uint32_t first) {
-#pragma unroll
-        for (int i = 0; i < GPW; ++i) {
-            const uint32_t u = first + 16u * (uint32_t)i, uc = u < U ? u : U;
-            const bool sh = uc == U;
-            // wave-uniform values: kept in scalar registers
-            const uint32_t e = __builtin_amdgcn_readfirstlane(a.uid[sh ? 0u : uc]), es0 = __builtin_amdgcn_readfirstlane(a.expert_start[uc]),
-                           es1 = __builtin_amdgcn_readfirstlane(a.expert_start[sh ? U : uc + 1u]);
-            // groups U .. U + S - 1: the shared expert, two tokens each (its pairs follow the routed ones); beyond: empty
-            const uint32_t sub = u - U, sp0 = P + 2u * sub, sp1 = sp0 + 2u < P + a.ntok ? sp0 + 2u : P + a.ntok;
-            gp0[i] = sh ? (sub < S ? sp0 : P) : es0;
-            gp1[i] = sh ? (sub < S ? sp1 : gp0[i]) : es1;
-            const uint8_t *dn = (sh ? a.shared : a.experts + (uint64_t)e * a.stride) + down_off;
-#pragma unroll
-            for (int c = 0; c < NCH; ++c) {
-                const uint32_t G = 16u * (uint32_t)c + blk, Gc = G < FG ? G : FG - 1u;
-                uint32_t d2 = 0u;
-#pragma unroll
-                for (int q = 0; q < 2; ++q) {
-                    const uint32_t r = row0 + 4u * (uint32_t)q + j;
-                    wq[i][c][q] = reinterpret_cast<const uint2 *>(dn)[(uint64_t)r * FG + Gc];
-                    d2 |= (uint32_t)reinterpret_cast<const uint16_t *>(dn + qs_bytes)[(uint64_t)r * FB + (Gc >> 3)] << (16 * q);
-                }
-                wd[i][c] = d2;
-            }
-        }
-    };
-    struct Pass { half4_t ax[NCH][8]; float sa[NCH], sb[NCH]; };
-    // activations of pairs pp (and pp + 1 if it belongs to the group); pp is clamped into the buffer
-    auto load_pass = [&](uint32_t pp, uint32_t p1, Pass &ps) {
-        const uint32_t last = P + a.ntok - 1u, pa = pp < last ? pp : last, pb = pa + 1u < p1 ? pa + 1u : pa;
-        const bool have_b = pp + 1u < p1;
-#pragma unroll
-        for (int c = 0; c < NCH; ++c) {
-            const uint32_t G = 16u * (uint32_t)c + blk, Gc = G < FG ? G : FG - 1u;
-            load_act_operand2(ps.ax[c], a.act_h, a.act_l, (uint64_t)pa * F, (uint64_t)pb * F, true, 32u * Gc, j);
-            const float live = G < FG ? 1.0f : 0.0f;
-            ps.sa[c] = live * exp2i(a.act_exp[pa * FG + Gc]);
-            ps.sb[c] = have_b ? live * exp2i(a.act_exp[pb * FG + Gc]) : 0.0f;
-        }
-    };
-    request(wave);
-    build_tables(lds, tid, grid_entry);
-    __syncthreads();
-
-    for (uint32_t first = wave; first < U + S; first += 16u * GPW) {
-        if (first != wave) request(first);
-        Pass buf[2];                                     // activations of the current and of the next group
-        load_pass(gp0[0], gp1[0], buf[0]);
-#pragma unroll
-        for (int i = 0; i < GPW; ++i) {
-            Pass &cur = buf[NCH == 1 ? i & 1 : 0];
-            if (NCH == 1 && i + 1 < GPW) load_pass(gp0[i + 1 < GPW ? i + 1 : i], gp1[i + 1 < GPW ? i + 1 : i], buf[(i + 1) & 1]);
-            if (NCH != 1 && i > 0) load_pass(gp0[i], gp1[i], cur);
-            for (uint32_t pp = gp0[i]; pp < gp1[i]; pp += 2u) {
-                if (pp != gp0[i]) load_pass(pp, gp1[i], cur);            // further passes of a large group
-                const bool have_b = pp + 1u < gp1[i];
-                float tot_a[2] = {0.0f, 0.0f}, tot_b[2] = {0.0f, 0.0f};
-#pragma unroll
-                for (int c = 0; c < NCH; ++c) {
-#pragma unroll
-                    for (int q = 0; q < 2; ++q) {
-                        const float d = scale_to_f32(wd[i][c] >> (16 * q));
-                        float va[1], vb[1];
-                        group_dot_multi<1>(wq[i][c][q], reinterpret_cast<const half4_t (*)[8]>(cur.ax[c]), lds, va, vb);
-                        tot_a[q] += va[0] * d * cur.sa[c];
-                        tot_b[q] += vb[0] * d * cur.sb[c];
-                    }
-                }
-                const float ra = quad_column_reduce<2>(tot_a, lane), rb = quad_column_reduce<2>(tot_b, lane);
-                if (reduced_writer<2>(lane)) {
-                    const uint32_t rr = 4u * reduced_unit<2>(lane) + j;
-                    part[pp * 8u + rr] = ra;
-                    if (have_b) part[(pp + 1u) * 8u + rr] = rb;
-                }
-            }
-        }
-    }
-    __syncthreads();
-    for (uint32_t i = tid; i < a.ntok * 8u; i += kWaves * 64u) {
-        const uint32_t t = i >> 3, r = i & 7u;
-        float sum = 0.0f;
-        for (uint32_t k = 0; k < a.top_k; ++k) {
-            const uint32_t p = a.tok_pair[t * a.top_k + k];
-            sum = fmaf(a.pair_weight[p] * 0.125f, part[p * 8u + r], sum);
-        }
-        sum = fmaf(a.scalar[t] * 0.125f, part[(P + t) * 8u + r], sum);
-        const uint64_t at = (uint64_t)t * H + row0 + r;
-        a.out[at] = a.resid_a ? (a.resid_a[at] + a.resid_b[at]) + sum : sum;
-    }
-}
-
-// The same kernel with the shared expert's rows taken from its dense f32 copy (token t's product on wave 15 - t, ahead of that wave's
-// routed groups), for routed down matrices that are word-packed IQ3_S (FMT 0) or IQ2_XS / IQ1_M streams (1 / 2).
 struct BatchWordsArgs {
     const uint8_t *experts;    // packed down matrix of expert e at experts + e * stride
     uint64_t stride;
@@ -3012,7 +2824,7 @@ __global__ __launch_bounds__(kWaves * 64) void down_batch_words_kernel(BatchWord
     }
 }
 
-// Batched down + combine on raw GGUF rows (mixed layouts): the work split of down_batch_kernel (8 output rows per workgroup, wave w owns
+// Batched down + combine on raw GGUF rows (mixed layouts): 8 output rows per workgroup, wave w owns
 // the groups w, w + 16, ..., the last group is the shared expert with every token) with the decode of down_combine_raw_kernel. A wave
 // stages the 8 rows of its group in LDS (the next group's rows are requested into registers before the current group is computed),
 // decodes a row's chunk once and applies it to every pair of the group, so a matrix is read once however many tokens selected it.
@@ -3116,34 +2928,6 @@ static bool batch_select_ok(const BatchSelect &b, uint32_t ntok, uint32_t top_k,
     return b.logits && b.ids && b.weights && b.scalar && b.n_expert == n_expert && n_expert <= 1024u && top_k <= 16u && top_k <= n_expert && ntok * top_k <= 128u;
 }
 
-hipError_t launch_batch_packed(const void *experts, uint64_t stride, const void *shared, const uint32_t *uid, const uint32_t *expert_start,
-                               const uint32_t *pair_token, const uint32_t *n_unique, const float *pair_weight, const uint32_t *tok_pair,
-                               const float *scalar, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l, int *act_exp,
-                               float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s,
-                               const BatchSelect *select) {
-    if (!fused_iq2_supported(hidden, ffn) || !ntok || ntok > (uint32_t)kMaxTok || ntok * top_k + ntok > 144u) return hipErrorInvalidValue;
-    BatchArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(shared), uid, expert_start, pair_token, n_unique,
-                pair_weight, tok_pair, scalar, static_cast<const _Float16 *>(xh), static_cast<const _Float16 *>(xl), xexp,
-                static_cast<_Float16 *>(act_h), static_cast<_Float16 *>(act_l), act_exp, out, hidden, ffn, top_k, ntok,
-                block_context().resid_a, block_context().resid_b, nullptr, nullptr, BatchSelect{}};
-    if (select && !batch_select_ok(*select, ntok, top_k, n_expert)) return hipErrorInvalidValue;
-    if (select) a.sel = *select;
-    const uint32_t P = ntok * top_k, n_groups = (P < n_expert ? P : n_expert) + 1u;
-    // units are passes of two tokens: at most (pairs + groups) / 2 routed ones, then the shared expert's, one per two tokens
-    hipError_t e = launch_gateup_batch_kernel(a, (P + (P < n_expert ? P : n_expert) + 1u) / 2u + (ntok + 1u) / 2u, s);
-    if (e != hipSuccess) return e;
-    prof_set_stage(ST_BATCH_DOWN);
-    const uint32_t groups_per_wave = (n_groups + (ntok + 1u) / 2u - 1u + kWaves - 1u) / kWaves;     // bound known on the host: min(pairs, experts) groups + the shared expert's
-    const dim3 dgrid(hidden / 8u), dblock(kWaves * 64);
-    if (ffn > 512u) REDHIP_LAUNCH((down_batch_kernel<144, 2, 2>), dgrid, dblock, 0, s, a);
-    else if (groups_per_wave <= 2u) REDHIP_LAUNCH((down_batch_kernel<144, 1, 2>), dgrid, dblock, 0, s, a);
-    else if (groups_per_wave <= 3u) REDHIP_LAUNCH((down_batch_kernel<144, 1, 3>), dgrid, dblock, 0, s, a);
-    else if (groups_per_wave <= 4u) REDHIP_LAUNCH((down_batch_kernel<144, 1, 4>), dgrid, dblock, 0, s, a);
-    else REDHIP_LAUNCH((down_batch_kernel<144, 1, 6>), dgrid, dblock, 0, s, a);
-    return hipGetLastError();
-}
-
-// the persistent gate/up kernel of a small batch over n_groups groups of pairs (the shared expert included when a.shared is set)
 template <uint32_t TD>
 static hipError_t launch_down_batch_raw_shared(uint32_t ts, const DownBatchRawArgs &a, hipStream_t s) {
     const dim3 grid(a.hidden / 8u), block(kWaves * 64);
@@ -3309,17 +3093,6 @@ hipError_t launch_gateup_select(const void *experts, uint64_t stride, const void
     }
 #undef REDHIP_GUS_FMT
 #undef REDHIP_GUS
-    return hipGetLastError();
-}
-
-hipError_t launch_down_combine(const void *experts, uint64_t stride, const void *shared, const uint32_t *ids, const float *weights,
-                               const float *scalar, const void *act_h, const void *act_l, const int *act_exp, float *out,
-                               uint32_t hidden, uint32_t ffn, uint32_t top_k, hipStream_t s) {
-    if (!fused_iq2_supported(hidden, ffn) || top_k + 1u > (uint32_t)kWaves) return hipErrorInvalidValue;
-    DownArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(shared), ids, weights, scalar,
-               static_cast<const _Float16 *>(act_h), static_cast<const _Float16 *>(act_l), act_exp, out, hidden, ffn, top_k,
-               block_context().resid_a, block_context().resid_b, route_guard().id_limit};
-    REDHIP_LAUNCH(down_combine_kernel, dim3(hidden / 8u), dim3(kWaves * 64), 0, s, a);
     return hipGetLastError();
 }
 

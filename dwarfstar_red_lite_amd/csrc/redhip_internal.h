@@ -247,14 +247,6 @@ hipError_t launch_select_group(const float *logits, uint32_t ntok, uint32_t n_ex
 hipError_t launch_prep(const float *x, const float *gate_inp, uint32_t ntok, uint32_t hidden, void *xh, void *xl, int *xexp, float *scalar, hipStream_t s,
                        const GroupJob *job = nullptr, bool *job_done = nullptr);
 
-// batched gate/up + down/combine over grouped pairs, packed IQ2_XXS, small batches (ntok * (top_k + 1) <= 144).
-// act buffers hold ntok * (top_k + 1) rows (routed pairs, then one row per token for the shared expert).
-hipError_t launch_batch_packed(const void *experts, uint64_t stride, const void *shared, const uint32_t *uid, const uint32_t *expert_start,
-                               const uint32_t *pair_token, const uint32_t *n_unique, const float *pair_weight, const uint32_t *tok_pair,
-                               const float *scalar, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l, int *act_exp,
-                               float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s,
-                               const BatchSelect *select = nullptr);
-
 // single token: act[slot] = SwiGLU(gate . x, up . x) as fp16 halves with one exponent per 32 values. With `logits` the
 // kernel selects the experts itself (and writes ids / weights / scalar); with logits == nullptr it takes ids_in.
 hipError_t launch_gateup_select(const void *experts, uint64_t stride, const void *shared, const void *shared_q6k, const float *x,
@@ -299,9 +291,5 @@ hipError_t launch_expert_slices(const void *experts, uint64_t stride, const void
 hipError_t launch_batch_slices(const void *experts, uint64_t stride, const void *down_cm, uint64_t down_stride, const void *shared, const void *shared_down_cm,
                                const void *pass_list, const uint32_t *n_pass, const float *weights, const float *scalar, const void *xh, const void *xl,
                                const int *xexp, float *partial, float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, hipStream_t s);
-// single token: out[r] = sum_k weights[k] * down_{ids[k]}[r] . act[k] + scalar * shared_down[r] . act[top_k], k in order
-hipError_t launch_down_combine(const void *experts, uint64_t stride, const void *shared, const uint32_t *ids, const float *weights,
-                               const float *scalar, const void *act_h, const void *act_l, const int *act_exp, float *out,
-                               uint32_t hidden, uint32_t ffn, uint32_t top_k, hipStream_t s);
 
 }  // namespace redhip

@@ -75,6 +75,11 @@ struct Moe {
     // every path of an all-IQ2_XXS handle of these shapes reads the packed copies: the raw GGUF rows of the routed experts only pass
     // through a staging buffer at upload
     bool keep_raw() const { return !(fused && cfg.hidden / 512u <= 4u); }
+    // all-IQ2_XXS layers of the shapes whose chunks run on the tile-major copies read their down matrices from the column-sliced copy (one
+    // token, small batches) or the tile-major one (chunks): the row-major packed down matrices are not kept (they pass through a second
+    // staging buffer on their way to the tile-major copy)
+    bool rowmajor_down() const { return !(fused && cfg.ffn <= 512u && cfg.hidden / 512u <= 4u); }
+    uint8_t *stage_down = nullptr;           // row-major packed down matrices of kStageExperts experts, source of their tile-major copy
     uint8_t *stage = nullptr;                // upload staging for handles that do not keep the raw rows: kStageExperts slots
     static constexpr uint32_t kStageExperts = 64u;
     // handles that can be given chunks keep a tile-major copy for the prefill kernels that hold a tile's activations in registers
@@ -83,6 +88,7 @@ struct Moe {
     bool tiled_router(uint32_t ntok) const {
         return packed_gu() && ntok >= (cfg.router_type == T_F32 ? 48u : 16u) && (cfg.router_type == T_F32 || mixed);
     }
+    uint64_t tiled_stride() const { return fused ? expert_stride : packed_stride; }      // bytes between experts in `tiled`
     bool tiles_resident() const { return packed_gu() && gu_type == T_IQ2_XXS && cfg.max_tokens > 8u && cfg.ffn <= 512u && cfg.hidden / 512u <= 4u; }
     // a chunk on a mixed layout: the routed gate/up matrices (packed IQ2_XXS) run on the prefill tiles, the rest on raw rows
     bool mixed_chunk(uint32_t ntok) const { return mixed && ntok > 8u && tiles_resident(); }
@@ -250,19 +256,12 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
         }
         if (m->small_batch(ntok) && grouped && !select_here) {     // the caller's routing, sorted (with its pass list) by the prep launch: expert slices per pass
             const Layer &L = m->layers[layer];
-            HIP_OK(launch_batch_slices(L.packed, m->expert_stride, L.down_cm, m->down_cm_stride(), L.shared_packed, L.shared_down_cm, m->pass_list, m->n_pass,
+            HIP_OK(launch_batch_slices(L.packed, m->packed_stride, L.down_cm, m->down_cm_stride(), L.shared_packed, L.shared_down_cm, m->pass_list, m->n_pass,
                                        weights, m->scalar, m->xh, m->xl, m->xexp, m->partial, out, c.hidden, c.ffn, c.top_k, ntok, s), "batched expert slice launch");
             prof_set_stage(ST_OTHER);
             return 1;
         }
-        if (m->small_batch(ntok)) {     // packed IQ2_XXS, MFMA kernels; xh / xl / xexp / scalar come from the router or prep kernel
-            const Layer &L = m->layers[layer];
-            HIP_OK(launch_batch_packed(L.packed, m->expert_stride, L.shared_packed, m->uid, m->expert_start, m->pair_token, m->n_unique,
-                                       m->pair_weight, m->tok_pair, m->scalar, m->xh, m->xl, m->xexp, m->act_h, m->act_l, m->act_exp, out,
-                                       c.hidden, c.ffn, c.top_k, ntok, c.n_expert, s, in_batch), "batched packed launch");
-            prof_set_stage(ST_OTHER);
-            return 1;
-        }
+        if (m->small_batch(ntok)) { moe_err("internal: a small batch reached the expert kernels without its pass list"); return 0; }
         if (m->packed_path(ntok)) {     // prefill chunk: tiles of 16 pairs per expert on the MFMA units
             const Layer &L = m->layers[layer];
             HIP_OK(launch_prefill_packed(L.packed, m->expert_stride, L.shared_packed, L.tiled, L.shared_tiled, m->uid, m->expert_start, m->pair_token, m->n_unique,
@@ -315,7 +314,7 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
     }
     if (m->fused && ntok == 1u) {    // expert slices + their sum; xh / xl (and the scalar gate of a caller's routing) come from the router kernel or the prep kernel
         const Layer &L = m->layers[layer];
-        HIP_OK(launch_expert_slices(L.packed, m->expert_stride, L.down_cm, m->down_cm_stride(), L.shared_packed, L.shared_down_cm, select_here ? m->logits : nullptr,
+        HIP_OK(launch_expert_slices(L.packed, m->packed_stride, L.down_cm, m->down_cm_stride(), L.shared_packed, L.shared_down_cm, select_here ? m->logits : nullptr,
                                     ids, weights, m->scalar, m->ids, m->weights, m->scalar, m->xh, m->xl, m->xexp, m->partial, out, c.hidden, c.ffn, c.n_expert,
                                     c.top_k, s), "expert slice launch");
         prof_set_stage(ST_OTHER);
@@ -329,10 +328,7 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
                                     m->weights, m->scalar, m->xh, m->xl, m->xexp, m->act_h, m->act_l, m->act_exp, c.hidden, c.ffn, c.n_expert,
                                     c.top_k, s, ntok, m->gu_type, m->gu_grid), "gate/up launch");      // ntok > 1: a small batch on a mixed layout, one grid layer per token
         prof_set_stage(ST_DOWN_COMBINE);
-        if (m->fused)
-            HIP_OK(launch_down_combine(L.packed, m->expert_stride, L.shared_packed, select_here ? m->ids : ids, select_here ? m->weights : weights,
-                                       m->scalar, m->act_h, m->act_l, m->act_exp, out, c.hidden, c.ffn, c.top_k, s), "down/combine launch");
-        else if (L.words_down && L.dense_down)
+        if (L.words_down && L.dense_down)
             HIP_OK(launch_down_combine_words(m->dn_type, m->dn_grid, L.words_down, m->words_down_stride(), L.dense_down, select_here ? m->ids : ids, select_here ? m->weights : weights,
                                              m->scalar, m->act_h, m->act_l, m->act_exp, out, c.hidden, c.ffn, c.top_k, s, ntok), "down/combine launch");
         else
@@ -414,7 +410,7 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
                (size_t)(c.top_k + 1u) * 8u * (c.ffn / 256u) * 210u + (dn == T_IQ1_M ? 17u * 1024u : dn == T_IQ2_XS ? 5u * 1024u : 0u) <= 64u * 1024u &&
                (sgu != T_Q6_K || (size_t)64u * (c.hidden / 256u) * 210u + (size_t)(c.hidden + c.hidden / 32u + c.hidden / 16u) * 4u <= (gu == T_IQ1_M ? 120u : 144u) * 1024u);
     m->pk_gate_bytes = packed_matrix_bytes(gu, c.ffn, c.hidden);
-    m->packed_stride = m->fused ? m->expert_stride : align256(2u * m->pk_gate_bytes);
+    m->packed_stride = m->fused && m->rowmajor_down() ? m->expert_stride : align256(2u * m->pk_gate_bytes);
     m->gu_grid = caller_grid_device(gu);
     m->dn_grid = caller_grid_device(dn);
     if (m->gu_grid || m->dn_grid) (void)set_caller_grids(nullptr, nullptr, m);      // bound to the tables the process holds now: they cannot change under this handle
@@ -461,9 +457,9 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
             m->resident += (uint64_t)c.n_expert * m->tiled_down_stride();
         }
         if (ok && m->tiles_resident()) {
-            ok = hipMalloc(reinterpret_cast<void **>(&L.tiled), (size_t)c.n_expert * m->packed_stride) == hipSuccess &&
+            ok = hipMalloc(reinterpret_cast<void **>(&L.tiled), (size_t)c.n_expert * m->tiled_stride()) == hipSuccess &&
                  (!m->fused || hipMalloc(reinterpret_cast<void **>(&L.shared_tiled), align256(2u * m->sh_gate_bytes + m->sh_down_bytes)) == hipSuccess);
-            m->resident += (uint64_t)c.n_expert * m->packed_stride + (m->fused ? align256(2u * m->sh_gate_bytes + m->sh_down_bytes) : 0u);
+            m->resident += (uint64_t)c.n_expert * m->tiled_stride() + (m->fused ? align256(2u * m->sh_gate_bytes + m->sh_down_bytes) : 0u);
         }
     }
     const size_t T = c.max_tokens;
@@ -557,6 +553,7 @@ void redhip_moe_destroy(redhip_moe_t h) {
     if (m->side) (void)hipStreamDestroy(m->side);
     if (m->ws) (void)hipFree(m->ws);
     if (m->stage) (void)hipFree(m->stage);
+    if (m->stage_down) (void)hipFree(m->stage_down);
     delete m;
 }
 
@@ -625,6 +622,10 @@ int redhip_moe_load_experts(redhip_moe_t h, uint32_t layer, uint32_t first, uint
             HIP_OK(hipMalloc(reinterpret_cast<void **>(&m->stage), (size_t)Moe::kStageExperts * m->expert_stride), "staging allocation");
             m->resident += (uint64_t)Moe::kStageExperts * m->expert_stride;
         }
+        if (!m->stage_down && !m->rowmajor_down() && m->tiles_resident()) {
+            HIP_OK(hipMalloc(reinterpret_cast<void **>(&m->stage_down), (size_t)Moe::kStageExperts * m->down_cm_stride()), "down staging allocation");
+            m->resident += (uint64_t)Moe::kStageExperts * m->down_cm_stride();
+        }
         for (uint32_t done = 0; done < count; done += Moe::kStageExperts) {
             const uint32_t n = count - done < Moe::kStageExperts ? count - done : Moe::kStageExperts;
             if (!stage_and_pack(m, layer, first + done, n, m->stage, static_cast<const uint8_t *>(gate) + (uint64_t)done * m->gate_bytes,
@@ -648,17 +649,30 @@ static int stage_and_pack(Moe *m, uint32_t layer, uint32_t first, uint32_t count
         uint8_t *pk = m->layers[layer].packed + (uint64_t)first * m->packed_stride;
         HIP_OK(launch_repack_gateup(m->gu_type, dst, m->expert_stride, count, c.ffn, c.hidden, pk, m->packed_stride, nullptr), "expert gate repack");
         HIP_OK(launch_repack_gateup(m->gu_type, dst + m->gate_bytes, m->expert_stride, count, c.ffn, c.hidden, pk + m->pk_gate_bytes, m->packed_stride, nullptr), "expert up repack");
+        // row-major packed down matrices: beside gate | up where the layout keeps them, else in the staging buffer (source of the tiles only)
+        const uint8_t *pk_down = nullptr;
+        uint64_t pk_down_stride = 0;
         if (m->fused) {
-            HIP_OK(launch_repack_iq2xxs(dst + 2u * m->gate_bytes, m->expert_stride, count, c.hidden, c.ffn, false, pk + 2u * m->gate_bytes, m->packed_stride, nullptr), "expert down repack");
+            if (m->rowmajor_down()) {
+                HIP_OK(launch_repack_iq2xxs(dst + 2u * m->gate_bytes, m->expert_stride, count, c.hidden, c.ffn, false, pk + 2u * m->gate_bytes, m->packed_stride, nullptr), "expert down repack");
+                pk_down = pk + 2u * m->gate_bytes;
+                pk_down_stride = m->packed_stride;
+            } else if (m->layers[layer].tiled) {
+                if (!m->stage_down || count > Moe::kStageExperts) { moe_err("down staging buffer missing"); return 0; }
+                HIP_OK(launch_repack_iq2xxs(dst + 2u * m->gate_bytes, m->expert_stride, count, c.hidden, c.ffn, false, m->stage_down, m->down_cm_stride(), nullptr), "expert down repack");
+                pk_down = m->stage_down;
+                pk_down_stride = m->down_cm_stride();
+            }
             HIP_OK(launch_repack_iq2xxs(dst + 2u * m->gate_bytes, m->expert_stride, count, c.hidden, c.ffn, true,
                                         m->layers[layer].down_cm + (uint64_t)first * m->down_cm_stride(), m->down_cm_stride(), nullptr), "expert down column slices");
         }
-        if (m->layers[layer].tiled) {
-            uint8_t *tl = m->layers[layer].tiled + (uint64_t)first * m->packed_stride;
-            HIP_OK(launch_tile_packed(pk, m->packed_stride, count, c.ffn, c.hidden, tl, m->packed_stride, nullptr), "expert gate tiling");
-            HIP_OK(launch_tile_packed(pk + m->gate_bytes, m->packed_stride, count, c.ffn, c.hidden, tl + m->gate_bytes, m->packed_stride, nullptr), "expert up tiling");
+        if (m->layers[layer].tiled) {      // (the tile-major copy keeps the gate | up | down slots of the raw layout)
+            const uint64_t tstride = m->tiled_stride();
+            uint8_t *tl = m->layers[layer].tiled + (uint64_t)first * tstride;
+            HIP_OK(launch_tile_packed(pk, m->packed_stride, count, c.ffn, c.hidden, tl, tstride, nullptr), "expert gate tiling");
+            HIP_OK(launch_tile_packed(pk + m->gate_bytes, m->packed_stride, count, c.ffn, c.hidden, tl + m->gate_bytes, tstride, nullptr), "expert up tiling");
             if (m->fused)
-                HIP_OK(launch_tile_packed(pk + 2u * m->gate_bytes, m->packed_stride, count, c.hidden, c.ffn, tl + 2u * m->gate_bytes, m->packed_stride, nullptr), "expert down tiling");
+                HIP_OK(launch_tile_packed(pk_down, pk_down_stride, count, c.hidden, c.ffn, tl + 2u * m->gate_bytes, tstride, nullptr), "expert down tiling");
         }
         if (m->layers[layer].words_down) {
             uint8_t *wd = m->layers[layer].words_down + (uint64_t)first * m->words_down_stride();
@@ -913,7 +927,8 @@ int redhip_moe_dequant_resident(redhip_moe_t h, uint32_t layer, uint32_t expert,
         const uint8_t *pk = sh ? L.shared_packed : L.packed + (uint64_t)expert * m->packed_stride;
         const uint64_t gbytes = m->pk_gate_bytes;
         if (which < 2u) HIP_OK(launch_dequant_packed(m->gu_type, pk + which * gbytes, c.ffn, c.hidden, m->gu_grid, out_dev, s), "packed gate/up dequant");
-        else HIP_OK(launch_dequant_packed_iq2xxs(pk + 2u * gbytes, c.hidden, c.ffn, false, out_dev, s), "packed down dequant");
+        else if (sh || m->rowmajor_down()) HIP_OK(launch_dequant_packed_iq2xxs(pk + 2u * gbytes, c.hidden, c.ffn, false, out_dev, s), "packed down dequant");
+        else HIP_OK(launch_dequant_packed_iq2xxs(L.down_cm + (uint64_t)expert * m->down_cm_stride(), c.hidden, c.ffn, true, out_dev, s), "column-sliced down dequant");
         return 1;
     }
     if (which == 2u && !sh && L.words_down) {       // the copy the MFMA down kernels read
