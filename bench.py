@@ -303,7 +303,7 @@ def main():
                 distinct.append(len(set(ids.ravel().tolist())))
         mean_distinct = float(np.mean(distinct))
         lb = layer_bytes(cfg, mean_distinct, B)
-        roof = kernel_roofline(cfg, synth, stages, K, B, mean_distinct, lb, "%s_b%d" % (args.layout, B))
+        roof = kernel_roofline(cfg, synth, stages, K, B, mean_distinct, lb, "%s_b%d" % (args.layout, B) + ("" if routing == "router" else "_" + routing))
         return {"B": B, "routing": routing, "timing": tm, "stages": stages, "mean_distinct": mean_distinct, "lb": lb, "roofline": roof, "rel": rel,
                 "ids_ok": ids_ok, "xs": xs, "xs_host": xs_host}
 
@@ -345,7 +345,7 @@ def main():
 
     # ---- what the launches alone cost on this machine: the same number of dependent launches per step with the same grids, empty kernels ----
     if B == 1 and not args.no_graph:
-        shapes = [(129, 256), (176, 1024), (256, 1024)]
+        shapes = [(136, 256), (176, 1024), (64, 256)]          # router, expert slices, sum of the partial vectors
         with torch.cuda.stream(stream):
             for g_, b_ in shapes:
                 assert lib.redhip_calibration_empty(g_, b_, stream.cuda_stream)

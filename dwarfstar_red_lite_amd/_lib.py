@@ -25,6 +25,11 @@ class MoeConfig(C.Structure):             # include/redhip_moe.h
                                           "expert_type_word", "shared_type_word", "reserved")]
 
 
+class GgufExpertLayout(C.Structure):      # include/redhip_moe.h; the reference's rl_expert_layout (native/redlite_native_gguf.h:47-59)
+    _fields_ = [(n, C.c_uint32) for n in ("layer", "expert", "ggml_type", "down_type")] + \
+               [(n, C.c_uint64) for n in ("gate_offset", "gate_bytes", "up_offset", "up_bytes", "down_offset", "down_bytes", "total_bytes")]
+
+
 # every symbol the headers declare: name -> (restype, argtypes)
 u32, u64, vp, dbl, i32 = C.c_uint32, C.c_uint64, C.c_void_p, C.c_double, C.c_int
 ABI = {
@@ -59,6 +64,7 @@ ABI = {
     "redhip_gguf_last_error": (C.c_char_p, []),
     "redhip_gguf_moe_config": (i32, [C.c_char_p, u32, C.POINTER(MoeConfig)]),
     "redhip_moe_load_gguf": (i32, [vp, C.c_char_p, u32, u32, C.POINTER(MoeConfig)]),
+    "redhip_gguf_expert_layout": (i32, [C.c_char_p, u32, u32, u32, C.POINTER(GgufExpertLayout)]),
     "redhip_moe_forward": (i32, [vp, u32, vp, u32, vp, vp]),
     "redhip_moe_forward_block": (i32, [vp, u32, vp, vp, vp, C.c_float, u32, vp, vp]),
     "redhip_moe_route": (i32, [vp, u32, vp, u32, vp, vp, vp, vp]),

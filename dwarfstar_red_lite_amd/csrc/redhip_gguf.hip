@@ -240,6 +240,39 @@ int redhip_gguf_moe_config(const char *path, uint32_t first_layer, redhip_moe_co
     return 1;
 }
 
+int redhip_gguf_expert_layout(const char *path, uint32_t expected_experts, uint32_t layer, uint32_t expert, redhip_gguf_expert_layout_t *out) {
+    g_gguf_error[0] = '\0';
+    if (!path || !out || !expected_experts || expert >= expected_experts) { gguf_err("invalid expert layout request"); return 0; }
+    File f;
+    Directory d;
+    if (!parse(path, f, d)) return 0;
+    const Tensor *t[3] = {find(d, layer, "ffn_gate_exps.weight"), find(d, layer, "ffn_up_exps.weight"), find(d, layer, "ffn_down_exps.weight")};
+    if (!t[0] || !t[1] || !t[2]) { gguf_err("layer %u does not contain routed gate/up/down tensors", layer); return 0; }
+    uint64_t per[3];
+    for (int k = 0; k < 3; ++k) {
+        // the expert index is the slowest dimension, so one expert is a contiguous range of the tensor
+        if (t[k]->n_dims < 2 || t[k]->dims[t[k]->n_dims - 1] != expected_experts || !t[k]->bytes || t[k]->bytes % expected_experts) {
+            gguf_err("layer %u: a routed tensor is not sliceable by expert (expert count %u is not its last dimension, or its type is not sized here)", layer, expected_experts);
+            return 0;
+        }
+        per[k] = t[k]->bytes / expected_experts;
+    }
+    if (t[0]->type != t[1]->type) { gguf_err("layer %u: routed gate and up tensors must share one quantisation type", layer); return 0; }
+    memset(out, 0, sizeof(*out));
+    out->layer = layer;
+    out->expert = expert;
+    out->ggml_type = t[0]->type;
+    out->down_type = t[2]->type;
+    out->gate_offset = t[0]->offset + expert * per[0];
+    out->gate_bytes = per[0];
+    out->up_offset = t[1]->offset + expert * per[1];
+    out->up_bytes = per[1];
+    out->down_offset = t[2]->offset + expert * per[2];
+    out->down_bytes = per[2];
+    out->total_bytes = per[0] + per[1] + per[2];
+    return 1;
+}
+
 int redhip_moe_load_gguf(redhip_moe_t moe, const char *path, uint32_t first_layer, uint32_t n_layer, const redhip_moe_config *cfg) {
     g_gguf_error[0] = '\0';
     if (!moe || !path || !cfg || !n_layer || n_layer > cfg->n_layer) { gguf_err("invalid GGUF load request"); return 0; }

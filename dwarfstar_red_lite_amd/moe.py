@@ -173,6 +173,17 @@ def gguf_moe_config(path, first_layer=0):
     return cfg, c.n_layer
 
 
+def gguf_expert_layout(path, n_expert, layer, expert):
+    """dict of the reference's rl_expert_layout fields (native/redlite_native_gguf.h:47-59) for one routed expert of a GGUF file:
+    quantisation types and the absolute byte ranges of its gate / up / down matrices. Host only."""
+    from ._lib import GgufExpertLayout
+    lib = load()
+    out = GgufExpertLayout()
+    if not lib.redhip_gguf_expert_layout(os.fsencode(path), n_expert, layer, expert, C.byref(out)):
+        raise RedHipError(lib.redhip_gguf_last_error().decode("utf-8", errors="replace"))
+    return {n: int(getattr(out, n)) for n, _ in GgufExpertLayout._fields_}
+
+
 def set_codebooks(iq2_xs_grid=None, iq1_m_grid=None):
     """upload the int8 codebooks (512 x 8 and 2048 x 8 values) that IQ2_XS / IQ1_M rows decode through."""
     lib = load()

@@ -89,6 +89,24 @@ const char *redhip_gguf_last_error(void);
 int redhip_gguf_moe_config(const char *path, uint32_t first_layer, redhip_moe_config *out);
 int redhip_moe_load_gguf(redhip_moe_t moe, const char *path, uint32_t first_layer, uint32_t n_layer, const redhip_moe_config *cfg);
 
+/* Where the bytes of one routed expert lie in the file: the answer of rl_native_build_expert_map + rl_native_expert_layout
+ * (native/redlite_native_gguf.c:199-397 and :399-440; struct rl_expert_layout of native/redlite_native_gguf.h:47-59, same
+ * fields in the same order) as this library's reader sees the file, i.e. the byte ranges redhip_moe_load_gguf uploads.
+ * Offsets are absolute file offsets. `expected_experts` is checked against the last dimension of the three tensors.
+ * Fails (0, redhip_gguf_last_error) for an expert beyond the count, a layer without its gate / up / down tensors, or gate
+ * and up tensors of different types, as the reference does. Host code only: no GPU is touched. */
+typedef struct {
+    uint32_t layer;
+    uint32_t expert;
+    uint32_t ggml_type;      /* gate and up */
+    uint32_t down_type;
+    uint64_t gate_offset, gate_bytes;
+    uint64_t up_offset, up_bytes;
+    uint64_t down_offset, down_bytes;
+    uint64_t total_bytes;
+} redhip_gguf_expert_layout_t;
+int redhip_gguf_expert_layout(const char *path, uint32_t expected_experts, uint32_t layer, uint32_t expert, redhip_gguf_expert_layout_t *out);
+
 /* The layer with the steps on either side of it, one call per layer and token batch
  * (native/redlite_native_engine_cpu.c:418-427; Metal rl_resid_rms native/redmetal_engine.m:95-105 in front and
  * rl_moe_tail :61-69 behind): resid = x + branch (the attention / DeltaNet branch output), the layer's input is

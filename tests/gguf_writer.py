@@ -29,7 +29,7 @@ def write_moe_gguf(path, cfg, layers, first_layer=0, alignment=32, arch="qwen3ne
             ("blk.%d.ffn_up_shexp.weight" % l, lay["sh_up"], (H, F), cfg["sh_gate_up_type"]),
             ("blk.%d.ffn_down_shexp.weight" % l, lay["sh_down"], (F, H), cfg["sh_down_type"]),
             ("blk.%d.ffn_gate_exps.weight" % l, lay["gate"], (H, F, E), cfg["gate_up_type"]),
-            ("blk.%d.ffn_up_exps.weight" % l, lay["up"], (H, F, E), cfg["gate_up_type"]),
+            ("blk.%d.ffn_up_exps.weight" % l, lay["up"], (H, F, E), cfg.get("up_type", cfg["gate_up_type"])),
             ("blk.%d.ffn_down_exps.weight" % l, lay["down"], (F, H, E), cfg["down_type"]),
         ]
     kv = [("general.architecture", GGUF_STRING, arch), ("general.alignment", GGUF_U32, alignment),
@@ -59,3 +59,22 @@ def write_moe_gguf(path, cfg, layers, first_layer=0, alignment=32, arch="qwen3ne
             fh.seek(start + o)
             fh.write(raw)
         fh.truncate(start + off)
+
+
+def write_case(path, spec):
+    """One of the fixture files of tests/golden/gguf_expert_layout.json, rebuilt from its `spec` (the same bytes every time: the
+    fixture holds the file's CRC-32). Returns (list of per-layer configurations, list of layers)."""
+    from dwarfstar_red_lite_amd import synth
+    cfgs = []
+    for layout in spec["layouts"]:
+        c = synth.layer_config(hidden=spec["hidden"], ffn=spec["ffn"], n_expert=spec["n_expert"], top_k=spec["top_k"], layout=layout)
+        if spec.get("up_type") is not None:
+            c["up_type"] = spec["up_type"]                   # a file the reference refuses: gate and up of different types
+        cfgs.append(c)
+    layers = [synth.make_layer(spec["seed"] + i, c) for i, c in enumerate(cfgs)]
+    extra = [("token_embd.weight", np.arange(spec["extra_floats"], dtype=np.float32))] if spec.get("extra_floats") else []
+    write_moe_gguf(path, cfgs, layers, first_layer=spec["first_layer"], alignment=spec["alignment"], extra_tensors=extra)
+    if spec.get("trailing_bytes"):
+        with open(path, "ab") as fh:
+            fh.write(b"\xa5" * spec["trailing_bytes"])
+    return cfgs, layers
