@@ -81,6 +81,39 @@ ABI = {
     "redhip_profile_end": (i32, [C.POINTER(dbl), C.POINTER(u32), u32]),
     "redhip_calibration_copy": (i32, [vp, vp, u64, vp]),
     "redhip_calibration_empty": (i32, [u32, u32, vp]),
+    # include/redmetal_topk.h
+    "redmetal_topk_abi_version": (u32, []),
+    "redmetal_topk_last_error": (C.c_char_p, []),
+    "redmetal_topk_pool_create": (vp, [C.c_char_p, u64, u64, u32, vp, u32, vp, u32]),
+    "redmetal_topk_pool_destroy": (None, [vp]),
+    "redmetal_topk_pool_set_classes": (i32, [vp, u32, vp, vp]),
+    "redmetal_topk_pool_capacity": (u32, [vp]),
+    "redmetal_topk_pool_slab_count": (u32, [vp]),
+    "redmetal_topk_pool_allocated_bytes": (u64, [vp]),
+    "redmetal_topk_pool_bytes_read": (u64, [vp]),
+    "redmetal_topk_pool_read_calls": (u64, [vp]),
+    "redmetal_topk_pool_read_ms": (dbl, [vp]),
+    "redmetal_topk_pool_slot_generation": (u32, [vp, u32]),
+    "redmetal_topk_pool_slot_inflight": (i32, [vp, u32]),
+    "redmetal_topk_pool_load_expert": (i32, [vp, u32, u64, u64, u64, u64, u64, u64, C.POINTER(u64), C.POINTER(dbl)]),
+    "redmetal_topk_pool_slot_addresses": (i32, [vp, u32, u64, u64, u64, C.POINTER(u64), C.POINTER(u64), C.POINTER(u64)]),
+    "redmetal_topk_pool_execute": (i32, [vp, vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, u32, vp, u32, vp, u32, C.POINTER(dbl)]),
+    "redmetal_topk_pool_encode": (i32, [vp, vp, vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, u32, vp, u64, vp, u64]),
+    "redmetal_topk_pool_release": (None, [vp, vp, u32]),
+    "redmetal_topk_pool_residency_table_init": (i32, [vp, u32, u32]),
+    "redmetal_topk_pool_residency_table": (vp, [vp]),
+    "redmetal_topk_pool_residency_set": (i32, [vp, u32, u32, u32]),
+    "redmetal_topk_pool_residency_clear": (None, [vp, u32, u32]),
+    "redmetal_topk_pool_slab_residency_set": (vp, [vp]),
+    "redmetal_topk_pool_allocate_all": (i32, [vp]),
+    "redmetal_topk_pool_use_all_slabs": (None, [vp, vp]),
+    "redmetal_topk_pool_tmp_buffer": (vp, [vp]),
+    "redmetal_topk_pool_encode_device": (i32, [vp, vp, vp, u64, vp, u64, u32, u32, u32, u32, u64, u64, vp, u64, vp, u64]),
+    "redmetal_topk_pool_encode_device_into": (i32, [vp, vp, vp, u64, vp, u64, u32, u32, u32, u32, u64, u64, vp, u64, vp, u64]),
+    "redmetal_topk_pool_encode_device_into2": (i32, [vp, vp, vp, u64, vp, u64, u32, u32, u32, u32, u64, u64, vp, u64, vp, u64, vp, u64, u32]),
+    "redmetal_topk_pool_encode_device_tail": (i32, [vp, vp, vp, u64, vp, u64, u32, u32, u32, u32, u64, u64, vp, u64, vp, vp, vp, vp, vp, u64]),
+    "redmetal_topk_pool_encode_batched": (i32, [vp, vp, vp, vp, vp, vp, u32, u32, u32, u32, u32, u32, u32, u32, vp, vp, vp, vp, vp, u64, vp, u64]),
+    "redmetal_topk_pool_encode_mapped": (i32, [vp, vp, vp, u64, vp, u64, vp, u64, u64, u64, u64, vp, u32, u32, u32, u32, u32, u32, u32, u32, vp, vp, vp, vp, vp, u64, vp, u64]),
 }
 
 _lib = None
@@ -97,7 +130,7 @@ def load():
             fn = getattr(lib, name)          # AttributeError here = header/library mismatch
             fn.restype = res
             fn.argtypes = args
-        for fam in ("redmetal_ffn", "redmetal_quant", "redhip_moe"):
+        for fam in ("redmetal_ffn", "redmetal_quant", "redmetal_topk", "redhip_moe"):
             if getattr(lib, fam + "_abi_version")() != 1:
                 raise RedHipError("unsupported %s ABI version" % fam)
         _lib = lib

@@ -10,7 +10,7 @@ CSRC = os.path.join(HERE, "csrc")
 OBJ = os.path.join(HERE, "build")
 LIB = os.path.join(HERE, "libredmetal_hip.so")
 SOURCES = ["redhip_kernels.hip", "redhip_fused.hip", "redhip_prefill.hip", "redhip_pool_abi.hip", "redhip_moe_abi.hip",
-           "redhip_gguf.hip", "redhip_profile.hip"]
+           "redhip_gguf.hip", "redhip_profile.hip", "redhip_topk_abi.hip"]
 # -packed-fp32-ops off: v_pk_*_f32 forms are not used on this pool of machines
 FLAGS = ["-O3", "--offload-arch=gfx950", "-fPIC", "-std=c++17",
          "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops", "-Wall", "-Wextra", "-Wno-unused-parameter"]

@@ -113,11 +113,17 @@ struct ExpertSet {               // where the experts of one layer live (raw GGU
     uint64_t stride;
     uint64_t gate_bytes, up_bytes;
     uint32_t gate_up_type, down_type;
+    const uint64_t *table = nullptr;   // device array of expert base addresses (a slot table), or nullptr. When set, slot / group i
+                                       // reads its expert at table[i]; base, stride and the ids / uid arrays are not used
 };
 
 // act[slot][r] = SiLU(gate_e[r] . x) * (up_e[r] . x) for slot < n_slot, e = ids ? ids[slot] : slot
+// With x1, slots from x_split on read x1 instead of x (two activation vectors in one launch).
 hipError_t launch_moe_gateup(const ExpertSet &ex, const uint32_t *ids, uint32_t n_slot, uint32_t hidden, uint32_t ffn,
-                             const float *x, float *act, hipStream_t s);
+                             const float *x, float *act, hipStream_t s, const float *x1 = nullptr, uint32_t x_split = 0u);
+// out[i] = sum_k weights[k] * tmp[k][row_start + i], k in order (tmp [top_k][hidden], i < row_count)
+hipError_t launch_weighted_sum(const float *tmp, const float *weights, uint32_t top_k, uint32_t hidden, uint32_t row_start,
+                               uint32_t row_count, float *out, hipStream_t s);
 
 // out[r] = sum_k weights[k] * (down_{ids[k]}[r] . act[k]) + scalar[0] * (shared_down[r] . shared_act), k in selection order
 hipError_t launch_moe_down_combine(const ExpertSet &ex, const uint32_t *ids, const float *weights, uint32_t top_k,

@@ -324,16 +324,19 @@ hipError_t launch_route_select(const float *logits, uint32_t ntok, uint32_t n_ex
 template <uint32_t T, int LPR>
 __global__ __launch_bounds__(256) void moe_gateup_kernel(const uint8_t *base, uint64_t stride, uint64_t gate_bytes,
                                                          const uint32_t *ids, uint32_t hidden, uint32_t ffn,
-                                                         const float *x, float *act, uint32_t id_limit, uint32_t *status) {
+                                                         const float *x, float *act, uint32_t id_limit, uint32_t *status,
+                                                         const uint64_t *table, const float *x1, uint32_t x_split) {
     extern __shared__ float xs[];
-    for (uint32_t i = threadIdx.x; i < hidden; i += 256u) xs[pad32(i)] = x[i];
-    __syncthreads();
     const uint32_t slot = blockIdx.y, e = ids ? guarded_id(ids[slot], id_limit, status) : slot;
+    const float *xin = x1 && slot >= x_split ? x1 : x;
+    for (uint32_t i = threadIdx.x; i < hidden; i += 256u) xs[pad32(i)] = xin[i];
+    __syncthreads();
+    const uint8_t *ebase = table ? reinterpret_cast<const uint8_t *>(table[slot]) : base + (uint64_t)e * stride;
     const uint32_t sub = threadIdx.x % LPR, r = blockIdx.x * (256u / LPR) + threadIdx.x / LPR;
     const uint64_t rb = (uint64_t)(hidden / 256u) * Fmt<T>::kBlock;
     float g = 0.0f, u = 0.0f;
     if (r < ffn) {
-        const uint8_t *grow = base + (uint64_t)e * stride + (uint64_t)r * rb;
+        const uint8_t *grow = ebase + (uint64_t)r * rb;
         const uint8_t *urow = grow + gate_bytes;
         for (uint32_t c = sub; c < hidden / 32u; c += LPR) {
             g += chunk_dot<T>(grow, c, xs + 33u * c);
@@ -347,30 +350,30 @@ __global__ __launch_bounds__(256) void moe_gateup_kernel(const uint8_t *base, ui
 
 template <uint32_t T>
 static hipError_t gateup_dispatch(const ExpertSet &ex, const uint32_t *ids, uint32_t n_slot, uint32_t hidden, uint32_t ffn,
-                                  const float *x, float *act, hipStream_t s) {
+                                  const float *x, float *act, hipStream_t s, const float *x1, uint32_t x_split) {
     const uint32_t lpr = lanes_per_row(hidden);
     const dim3 grid((ffn + 256u / lpr - 1u) / (256u / lpr), n_slot);
     const size_t lds = padded_floats(hidden) * sizeof(float);
     switch (lpr) {
-        case 64: REDHIP_LAUNCH((moe_gateup_kernel<T, 64>), dim3(grid), dim3(256), lds, s, ex.base, ex.stride, ex.gate_bytes, ids, hidden, ffn, x, act, route_guard().id_limit, route_guard().status); break;
-        case 32: REDHIP_LAUNCH((moe_gateup_kernel<T, 32>), dim3(grid), dim3(256), lds, s, ex.base, ex.stride, ex.gate_bytes, ids, hidden, ffn, x, act, route_guard().id_limit, route_guard().status); break;
-        case 16: REDHIP_LAUNCH((moe_gateup_kernel<T, 16>), dim3(grid), dim3(256), lds, s, ex.base, ex.stride, ex.gate_bytes, ids, hidden, ffn, x, act, route_guard().id_limit, route_guard().status); break;
-        default: REDHIP_LAUNCH((moe_gateup_kernel<T, 8>), dim3(grid), dim3(256), lds, s, ex.base, ex.stride, ex.gate_bytes, ids, hidden, ffn, x, act, route_guard().id_limit, route_guard().status); break;
+        case 64: REDHIP_LAUNCH((moe_gateup_kernel<T, 64>), dim3(grid), dim3(256), lds, s, ex.base, ex.stride, ex.gate_bytes, ids, hidden, ffn, x, act, route_guard().id_limit, route_guard().status, ex.table, x1, x_split); break;
+        case 32: REDHIP_LAUNCH((moe_gateup_kernel<T, 32>), dim3(grid), dim3(256), lds, s, ex.base, ex.stride, ex.gate_bytes, ids, hidden, ffn, x, act, route_guard().id_limit, route_guard().status, ex.table, x1, x_split); break;
+        case 16: REDHIP_LAUNCH((moe_gateup_kernel<T, 16>), dim3(grid), dim3(256), lds, s, ex.base, ex.stride, ex.gate_bytes, ids, hidden, ffn, x, act, route_guard().id_limit, route_guard().status, ex.table, x1, x_split); break;
+        default: REDHIP_LAUNCH((moe_gateup_kernel<T, 8>), dim3(grid), dim3(256), lds, s, ex.base, ex.stride, ex.gate_bytes, ids, hidden, ffn, x, act, route_guard().id_limit, route_guard().status, ex.table, x1, x_split); break;
     }
     return hipGetLastError();
 }
 
 hipError_t launch_moe_gateup(const ExpertSet &ex, const uint32_t *ids, uint32_t n_slot, uint32_t hidden, uint32_t ffn,
-                             const float *x, float *act, hipStream_t s) {
+                             const float *x, float *act, hipStream_t s, const float *x1, uint32_t x_split) {
     hipError_t e = ensure_tables();
     if (e != hipSuccess) return e;
     if (!n_slot || hidden % 256u || ffn % 256u) return hipErrorInvalidValue;
     switch (ex.gate_up_type) {
-        case T_IQ2_XXS: return gateup_dispatch<T_IQ2_XXS>(ex, ids, n_slot, hidden, ffn, x, act, s);
-        case T_IQ3_S: return gateup_dispatch<T_IQ3_S>(ex, ids, n_slot, hidden, ffn, x, act, s);
-        case T_Q6_K: return gateup_dispatch<T_Q6_K>(ex, ids, n_slot, hidden, ffn, x, act, s);
-        case T_IQ2_XS: return gateup_dispatch<T_IQ2_XS>(ex, ids, n_slot, hidden, ffn, x, act, s);
-        case T_IQ1_M: return gateup_dispatch<T_IQ1_M>(ex, ids, n_slot, hidden, ffn, x, act, s);
+        case T_IQ2_XXS: return gateup_dispatch<T_IQ2_XXS>(ex, ids, n_slot, hidden, ffn, x, act, s, x1, x_split);
+        case T_IQ3_S: return gateup_dispatch<T_IQ3_S>(ex, ids, n_slot, hidden, ffn, x, act, s, x1, x_split);
+        case T_Q6_K: return gateup_dispatch<T_Q6_K>(ex, ids, n_slot, hidden, ffn, x, act, s, x1, x_split);
+        case T_IQ2_XS: return gateup_dispatch<T_IQ2_XS>(ex, ids, n_slot, hidden, ffn, x, act, s, x1, x_split);
+        case T_IQ1_M: return gateup_dispatch<T_IQ1_M>(ex, ids, n_slot, hidden, ffn, x, act, s, x1, x_split);
         default: return hipErrorInvalidValue;
     }
 }
@@ -485,6 +488,7 @@ struct PairArgs {
     const uint32_t *pair_token;    // [P] token of each pair, or nullptr: pair p is token p
     const uint32_t *n_unique;      // [1] number of groups, or nullptr: one group
     uint32_t n_pairs_total;        // used when expert_start == nullptr: one group of this many pairs
+    const uint64_t *table;         // [U] base address of group u's expert (a slot table), or nullptr: base + e * stride
 };
 
 template <uint32_t T, int LPR>
@@ -497,8 +501,9 @@ __global__ __launch_bounds__(256) void batch_gateup_kernel(PairArgs a, uint32_t 
     const uint32_t hp = hidden + (hidden >> 5);
     const uint32_t sub = threadIdx.x % LPR, r = blockIdx.x * (256u / LPR) + threadIdx.x / LPR;
     const uint64_t rb = (uint64_t)(hidden / 256u) * Fmt<T>::kBlock;
-    const uint8_t *grow = a.base + (uint64_t)e * a.stride + a.matrix_off + (uint64_t)r * rb;
-    const uint8_t *urow = a.base + (uint64_t)e * a.stride + a.second_off + (uint64_t)r * rb;
+    const uint8_t *ebase = a.table ? reinterpret_cast<const uint8_t *>(a.table[u]) : a.base + (uint64_t)e * a.stride;
+    const uint8_t *grow = ebase + a.matrix_off + (uint64_t)r * rb;
+    const uint8_t *urow = ebase + a.second_off + (uint64_t)r * rb;
     for (uint32_t c0 = p0; c0 < p1; c0 += kPairTile) {
         const uint32_t nb = p1 - c0 < (uint32_t)kPairTile ? p1 - c0 : (uint32_t)kPairTile;
         __syncthreads();
@@ -549,7 +554,7 @@ __global__ __launch_bounds__(256) void batch_down_kernel(PairArgs a, uint32_t hi
     const uint32_t fp = ffn + (ffn >> 5);
     const uint32_t sub = threadIdx.x % LPR, r = blockIdx.x * (256u / LPR) + threadIdx.x / LPR;
     const uint64_t rb = (uint64_t)(ffn / 256u) * Fmt<T>::kBlock;
-    const uint8_t *row = a.base + (uint64_t)e * a.stride + a.matrix_off + (uint64_t)r * rb;
+    const uint8_t *row = (a.table ? reinterpret_cast<const uint8_t *>(a.table[u]) : a.base + (uint64_t)e * a.stride) + a.matrix_off + (uint64_t)r * rb;
     for (uint32_t c0 = p0; c0 < p1; c0 += kPairTile) {
         const uint32_t nb = p1 - c0 < (uint32_t)kPairTile ? p1 - c0 : (uint32_t)kPairTile;
         __syncthreads();
@@ -643,7 +648,7 @@ hipError_t launch_batch_gateup(const ExpertSet &ex, const uint32_t *uid, const u
                                const uint32_t *n_unique, uint32_t n_groups, uint32_t n_pairs_total, uint32_t hidden, uint32_t ffn,
                                const float *x, float *act, hipStream_t s) {
     if (!n_groups || hidden % 256u || ffn % 256u || (size_t)kPairTile * padded_floats(hidden) * 4u > 160u * 1024u || n_groups > 65535u) return hipErrorInvalidValue;
-    const PairArgs a{ex.base, ex.stride, 0u, ex.gate_bytes, uid, expert_start, pair_token, n_unique, n_pairs_total};
+    const PairArgs a{ex.base, ex.stride, 0u, ex.gate_bytes, uid, expert_start, pair_token, n_unique, n_pairs_total, ex.table};
     switch (ex.gate_up_type) {
         case T_IQ2_XXS: return batch_gateup_dispatch<T_IQ2_XXS>(a, n_groups, hidden, ffn, x, act, s);
         case T_IQ3_S: return batch_gateup_dispatch<T_IQ3_S>(a, n_groups, hidden, ffn, x, act, s);
@@ -657,7 +662,7 @@ hipError_t launch_batch_gateup(const ExpertSet &ex, const uint32_t *uid, const u
 hipError_t launch_batch_down(const ExpertSet &ex, const uint32_t *uid, const uint32_t *expert_start, const uint32_t *n_unique,
                              uint32_t n_groups, uint32_t n_pairs_total, uint32_t hidden, uint32_t ffn, const float *act, float *tmp, hipStream_t s) {
     if (!n_groups || hidden % 256u || ffn % 256u || n_groups > 65535u) return hipErrorInvalidValue;
-    const PairArgs a{ex.base, ex.stride, ex.gate_bytes + ex.up_bytes, 0u, uid, expert_start, nullptr, n_unique, n_pairs_total};
+    const PairArgs a{ex.base, ex.stride, ex.gate_bytes + ex.up_bytes, 0u, uid, expert_start, nullptr, n_unique, n_pairs_total, ex.table};
     switch (ex.down_type) {
         case T_IQ2_XXS: return batch_down_dispatch<T_IQ2_XXS>(a, n_groups, hidden, ffn, act, tmp, s);
         case T_IQ3_S: return batch_down_dispatch<T_IQ3_S>(a, n_groups, hidden, ffn, act, tmp, s);
@@ -671,6 +676,23 @@ hipError_t launch_batch_down(const ExpertSet &ex, const uint32_t *uid, const uin
 hipError_t launch_batch_combine(const float *tmp, const float *pair_weight, const uint32_t *tok_pair, uint32_t ntok, uint32_t top_k,
                                 const float *sh_tmp, const float *scalar, uint32_t hidden, float *out, hipStream_t s) {
     REDHIP_LAUNCH(batch_combine_kernel, dim3((hidden + 255u) / 256u, ntok), dim3(256), 0, s, tmp, pair_weight, tok_pair, top_k, sh_tmp, scalar, hidden, out, block_context().resid_a, block_context().resid_b);
+    return hipGetLastError();
+}
+
+// out[i] = sum_k weights[k] * tmp[k][row_start + i], experts accumulated in the order of the list
+__global__ __launch_bounds__(256) void weighted_sum_kernel(const float *tmp, const float *weights, uint32_t top_k, uint32_t hidden,
+                                                           uint32_t row_start, uint32_t row_count, float *out) {
+    const uint32_t i = blockIdx.x * 256u + threadIdx.x;
+    if (i >= row_count) return;
+    float acc = 0.0f;
+    for (uint32_t k = 0; k < top_k; ++k) acc = fmaf(weights[k], tmp[(uint64_t)k * hidden + row_start + i], acc);
+    out[i] = acc;
+}
+
+hipError_t launch_weighted_sum(const float *tmp, const float *weights, uint32_t top_k, uint32_t hidden, uint32_t row_start,
+                               uint32_t row_count, float *out, hipStream_t s) {
+    if (!top_k || !row_count || row_start >= hidden || row_count > hidden - row_start) return hipErrorInvalidValue;
+    REDHIP_LAUNCH(weighted_sum_kernel, dim3((row_count + 255u) / 256u), dim3(256), 0, s, tmp, weights, top_k, hidden, row_start, row_count, out);
     return hipGetLastError();
 }
 

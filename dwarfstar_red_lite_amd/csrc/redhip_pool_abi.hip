@@ -17,70 +17,18 @@
 #include "../../include/redmetal_ffn.h"
 #include "../../include/redmetal_quant.h"
 #include "../../include/redmetal_router.h"
+#include "redhip_host_util.h"
 #include "redhip_internal.h"
 
 using namespace redhip;
 
 namespace {
 
-double now_ms() {
-    struct timespec ts;
-    clock_gettime(CLOCK_MONOTONIC, &ts);
-    return (double)ts.tv_sec * 1000.0 + (double)ts.tv_nsec / 1.0e6;
-}
-
 thread_local char g_ffn_error[512];
 thread_local char g_quant_error[512];
 
-void set_err(char *dst, size_t cap, const char *fmt, ...) {
-    if (!dst || !cap) return;
-    va_list ap;
-    va_start(ap, fmt);
-    vsnprintf(dst, cap, fmt, ap);
-    va_end(ap);
-}
 #define FFN_ERR(...) set_err(g_ffn_error, sizeof(g_ffn_error), __VA_ARGS__)
 #define QUANT_ERR(...) set_err(g_quant_error, sizeof(g_quant_error), __VA_ARGS__)
-
-// whole-range pread with EINTR retry; counts calls and bytes
-bool pread_range(int fd, uint64_t file_size, uint64_t offset, uint64_t len, uint8_t *dst, uint64_t *bytes, uint64_t *calls,
-                 char *err, size_t cap) {
-    if (!dst || offset > file_size || len > file_size - offset) {
-        set_err(err, cap, "invalid pread range offset=%llu len=%llu file_size=%llu", (unsigned long long)offset,
-                (unsigned long long)len, (unsigned long long)file_size);
-        return false;
-    }
-    uint64_t pos = 0;
-    while (pos < len) {
-        const uint64_t rem = len - pos;
-        const size_t want = rem > (uint64_t)SSIZE_MAX ? (size_t)SSIZE_MAX : (size_t)rem;
-        ssize_t n;
-        do { n = pread(fd, dst + pos, want, (off_t)(offset + pos)); } while (n < 0 && errno == EINTR);
-        if (calls) ++*calls;
-        if (n <= 0) {
-            set_err(err, cap, n < 0 ? "pread failed: %s" : "unexpected end of file%s", n < 0 ? strerror(errno) : "");
-            return false;
-        }
-        pos += (uint64_t)n;
-    }
-    if (bytes) *bytes += len;
-    return true;
-}
-
-struct DevBuf {                       // grow-only device scratch
-    void *p = nullptr;
-    size_t cap = 0;
-    bool reserve(size_t n) {
-        if (n <= cap) return true;
-        if (p) (void)hipFree(p);
-        p = nullptr;
-        cap = 0;
-        if (hipMalloc(&p, n) != hipSuccess) { p = nullptr; return false; }
-        cap = n;
-        return true;
-    }
-    ~DevBuf() { if (p) (void)hipFree(p); }
-};
 
 struct FfnPool {
     int fd = -1;
@@ -149,8 +97,6 @@ float *scratch_of_current_device(char *err, size_t cap) {
     }
     return g_scratch_ptr[dev];
 }
-
-bool sizes_overflow(uint64_t a, uint64_t b, uint64_t c) { return a > UINT64_MAX - b || a + b > UINT64_MAX - c; }
 
 }  // namespace
 

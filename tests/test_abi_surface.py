@@ -41,6 +41,11 @@ def test_error_strings_without_device_work():
     lib.redhip_moe_destroy(None)
     assert lib.redhip_moe_create(None) is None
     assert b"null MoE config" in lib.redhip_moe_last_error()
+    assert lib.redmetal_topk_pool_create(None, 0, 0, 0, None, 0, None, 0) is None
+    assert b"invalid Red Metal top-k pool arguments" in lib.redmetal_topk_last_error()
+    lib.redmetal_topk_pool_destroy(None)
+    assert lib.redmetal_topk_pool_capacity(None) == 0 and lib.redmetal_topk_pool_tmp_buffer(None) is None
+    assert lib.redmetal_topk_pool_slab_residency_set(None) is None
     assert lib.redmetal_quant_rows(None, 0, 0, 16, 256, 1, 0, 1, None, 256, None, 0, None, 1, None, None) == 0
     assert b"invalid Red Metal mixed-quant arguments" in lib.redmetal_quant_last_error()
 

@@ -1,0 +1,295 @@
+"""The resident top-k expert pool (redmetal_topk_*) through the C ABI against the CPU path: experts are read from a GGUF file into
+slots at the byte ranges the file's directory gives, then the weighted top-k FFN runs over slot lists - host arrays (execute),
+stream-ordered with host lists (encode, encode_batched, encode_mapped) and with the slot table and weights read on the device
+(encode_device_into / _into2 / _tail). Expected values: the CPU path's expert FFN in double, summed in list order."""
+import json
+import os
+
+import numpy as np
+import pytest
+
+import oracle_lib as orc
+from dwarfstar_red_lite_amd import synth
+from dwarfstar_red_lite_amd._lib import RedHipError
+from gguf_writer import write_moe_gguf
+from gpu_common import REL_L2_TOL, rel_l2
+
+pytestmark = pytest.mark.gpu
+torch = pytest.importorskip("torch")
+
+
+@pytest.fixture(scope="module")
+def grids(golden_dir):
+    g = json.load(open(os.path.join(golden_dir, "iq_grids.json")))
+    xs = np.frombuffer(bytes.fromhex(g["iq2_xs"]), np.int8)
+    m = np.frombuffer(bytes.fromhex(g["iq1_m"]), np.int8)
+    orc.set_codebooks(xs, m)
+    return xs, m
+
+
+def read_device(ptr, nbytes, dtype):
+    """bytes at a device address the library handed out (not a torch allocation), through the library's own copy kernel"""
+    from dwarfstar_red_lite_amd._lib import load
+    assert nbytes % 16 == 0
+    dst = torch.empty(nbytes, dtype=torch.uint8, device="cuda")
+    assert load().redhip_calibration_copy(dst.data_ptr(), ptr, nbytes, torch.cuda.current_stream().cuda_stream)
+    return dst.cpu().numpy().view(dtype)
+
+
+def type_word(cfg):
+    return cfg["gate_up_type"] if cfg["gate_up_type"] == cfg["down_type"] else cfg["gate_up_type"] | (cfg["down_type"] << 8)
+
+
+class Case:
+    """a one-layer GGUF file of `layout`, a pool over it, experts 0 .. n_load - 1 loaded into slots in a scrambled order"""
+
+    def __init__(self, tmp_path, grids, layout, hidden=512, ffn=256, n_expert=16, n_load=None, seed=700, **pool_kw):
+        from dwarfstar_red_lite_amd.moe import gguf_expert_layout
+        from dwarfstar_red_lite_amd.redmetal_topk import ExpertLayout, RedMetalTopKPool
+        self.cfg = cfg = synth.layer_config(hidden=hidden, ffn=ffn, n_expert=n_expert, top_k=4, layout=layout)
+        self.lay = synth.make_layer(seed, cfg)
+        self.path = str(tmp_path / ("topk_%s_%d.gguf" % (layout, hidden)))
+        write_moe_gguf(self.path, cfg, [self.lay])
+        self.layouts = []
+        for e in range(n_expert):
+            d = gguf_expert_layout(self.path, n_expert, 0, e)
+            self.layouts.append(ExpertLayout(d["gate_offset"], d["gate_bytes"], d["up_offset"], d["up_bytes"], d["down_offset"], d["down_bytes"]))
+        self.slot_bytes = self.layouts[0].gate_bytes * 2 + self.layouts[0].down_bytes
+        n_load = n_expert if n_load is None else n_load
+        kw = dict(slots_per_slab=5)
+        kw.update(pool_kw)
+        self.pool = RedMetalTopKPool(self.path, (n_load + 3) * ((self.slot_bytes + 4095) // 4096 * 4096), self.slot_bytes,
+                                     iq2_xs_grid=grids[0], iq1_m_grid=grids[1], **kw)
+        self.slot_of = {}
+        for i, e in enumerate(np.random.default_rng(seed).permutation(n_load)):
+            self.slot_of[int(e)] = i
+            got = self.pool.load(i, self.layouts[e])
+            assert got["bytes_read"] == self.slot_bytes
+        self.word = type_word(cfg)
+
+    def want(self, experts, weights, x, row_start=0, row_count=None):
+        cfg, lay = self.cfg, self.lay
+        acc = None
+        for e, w in zip(experts, weights):
+            y = orc.expert_ffn(cfg["gate_up_type"], cfg["down_type"], lay["gate"][e], lay["up"][e], lay["down"][e], cfg["hidden"], cfg["ffn"], x,
+                               row_start, row_count)
+            acc = float(w) * y if acc is None else acc + float(w) * y
+        return acc
+
+
+@pytest.mark.parametrize("layout", ["iq2", "f2", "xs", "m"])
+def test_execute_against_cpu_path(tmp_path, grids, layout):
+    c = Case(tmp_path, grids, layout)
+    H, F = c.cfg["hidden"], c.cfg["ffn"]
+    rng = np.random.default_rng(5)
+    for top_k, row_start, row_count in ((4, 0, H), (1, 0, H), (7, 128, 200), (16, H - 1, 1)):
+        experts = rng.permutation(16)[:top_k]
+        w = rng.random(top_k).astype(np.float32) + 0.05
+        x = synth.normed_x(rng, 1, H)[0]
+        got, ms = c.pool.execute([c.slot_of[int(e)] for e in experts], [c.layouts[e] for e in experts], w, c.word, H, F, row_start, row_count, x)
+        assert got.shape == (row_count,) and ms > 0.0
+        assert rel_l2(got, c.want(experts, w, x, row_start, row_count)) <= REL_L2_TOL, (layout, top_k, row_start)
+        assert not any(c.pool.slot_inflight(s) for s in range(c.pool.capacity))
+    t = c.pool.telemetry()
+    assert t["bytes_read"] == 16 * c.slot_bytes and t["read_calls"] >= 48 and t["slab_count"] == 4 and t["capacity"] == 19
+    c.pool.close()
+
+
+def test_execute_full_shape_top10(tmp_path, grids):
+    """hidden 2048, ffn 512, ten experts of the mixed-precision layout (gate/up IQ2_XXS, down IQ3_S)"""
+    c = Case(tmp_path, grids, "f2", hidden=2048, ffn=512, n_expert=12)
+    rng = np.random.default_rng(6)
+    experts = rng.permutation(12)[:10]
+    w = rng.random(10).astype(np.float32)
+    w /= w.sum()
+    x = synth.normed_x(rng, 1, 2048)[0]
+    got, _ = c.pool.execute([c.slot_of[int(e)] for e in experts], [c.layouts[e] for e in experts], w, c.word, 2048, 512, 0, 2048, x)
+    assert rel_l2(got, c.want(experts, w, x)) <= REL_L2_TOL
+    c.pool.close()
+
+
+def test_validation_and_slot_bookkeeping(tmp_path, grids):
+    c = Case(tmp_path, grids, "iq2", n_load=6)
+    H, F, L = c.cfg["hidden"], c.cfg["ffn"], c.layouts
+    x = np.zeros(H, np.float32)
+    ok = lambda ids, lays, w, **kw: c.pool.execute(ids, lays, w, kw.get("word", c.word), kw.get("H", H), F, kw.get("start", 0), kw.get("count", H), kw.get("x", x))
+    with pytest.raises(RedHipError, match="duplicate slot 2"):
+        ok([1, 2, 2], [L[0]] * 3, [1, 1, 1])
+    with pytest.raises(RedHipError, match="exceeds capacity"):
+        ok([1, 99], [L[0]] * 2, [1, 1])
+    with pytest.raises(RedHipError, match=r"top_k=0 must be in \[1,512\]"):
+        ok([], [], [])
+    with pytest.raises(RedHipError, match="matrix byte mismatch"):
+        ok([1], [L[0]._replace(down_bytes=L[0].down_bytes - 2)], [1])
+    with pytest.raises(RedHipError, match="invalid top-k dimensions"):
+        ok([1], [L[0]], [1], start=H)
+    with pytest.raises(RedHipError, match="unsupported top-k GGML type word"):
+        ok([1], [L[0]], [1], word=2)
+    # generations count the loads of a slot; a slot in flight is not overwritten
+    assert c.pool.slot_generation(0) == 1 and c.pool.slot_generation(8) == 0
+    c.pool.load(0, L[3])
+    assert c.pool.slot_generation(0) == 2
+    xd, od = torch.zeros(H, device="cuda"), torch.zeros(H, device="cuda")
+    c.pool.encode(None, [0, 1], [L[3], L[0]], [0.5, 0.5], c.word, H, F, 0, H, xd.data_ptr(), od.data_ptr())
+    assert c.pool.slot_inflight(0) and c.pool.slot_inflight(1) and not c.pool.slot_inflight(2)
+    with pytest.raises(RedHipError, match="refusing to overwrite in-flight top-k slot 0"):
+        c.pool.load(0, L[2])
+    torch.cuda.synchronize()
+    c.pool.release([0, 1])
+    assert not c.pool.slot_inflight(0)
+    c.pool.load(0, L[2])
+    with pytest.raises(RedHipError, match="payload exceeds slot size"):
+        c.pool.load(1, L[0]._replace(gate_bytes=L[0].gate_bytes + 8192))
+    with pytest.raises(RedHipError, match="invalid pread range"):
+        c.pool.load(1, L[0]._replace(gate_offset=10 ** 12))
+    with pytest.raises(RedHipError, match="must be set before any slab"):
+        c.pool.set_classes([c.slot_bytes], [4])
+    c.pool.close()
+
+
+def test_slot_classes_and_budget(tmp_path, grids):
+    from dwarfstar_red_lite_amd.redmetal_topk import RedMetalTopKPool
+    c = Case(tmp_path, grids, "f2", n_load=0)
+    big = (c.slot_bytes + 4095) // 4096 * 4096
+    pool = RedMetalTopKPool(c.path, 10 * big, c.slot_bytes, slots_per_slab=2, iq2_xs_grid=grids[0], iq1_m_grid=grids[1])
+    assert pool.capacity == 10
+    with pytest.raises(RedHipError, match="exceed the cache budget"):
+        pool.set_classes([big, 4096], [10, 1])
+    pool.set_classes([8192, c.slot_bytes], [3, 5])                  # slots 0..2 small, 3..7 expert sized
+    assert pool.capacity == 8
+    with pytest.raises(RedHipError, match="payload exceeds slot size"):
+        pool.load(1, c.layouts[0])
+    pool.load(3, c.layouts[4])
+    pool.load(7, c.layouts[9])
+    g3, u3, d3 = pool.addresses(3, c.layouts[4])
+    g4, _, _ = pool.addresses(4, c.layouts[4])
+    assert u3 - g3 == c.layouts[4].gate_bytes and d3 - u3 == c.layouts[4].up_bytes and g4 - g3 == big
+    t = pool.telemetry()
+    assert t["slab_count"] == 2 and t["allocated_bytes"] == 2 * big + 1 * big       # slab of slots 3,4 and slab of slot 7 alone
+    rng = np.random.default_rng(8)
+    x = synth.normed_x(rng, 1, c.cfg["hidden"])[0]
+    got, _ = pool.execute([7, 3], [c.layouts[9], c.layouts[4]], [0.25, 0.75], c.word, c.cfg["hidden"], c.cfg["ffn"], 0, c.cfg["hidden"], x)
+    assert rel_l2(got, c.want([9, 4], [0.25, 0.75], x)) <= REL_L2_TOL
+    pool.allocate_all()
+    assert pool.telemetry()["slab_count"] == 2 + 3
+    pool.close()
+    c.pool.close()
+
+
+@pytest.mark.parametrize("layout", ["iq2", "f2"])
+def test_device_driven_forms(tmp_path, grids, layout):
+    """slot addresses gathered on the device from the residency table, weights on the device: into, into with the sum left to the
+    caller, two input vectors, and the fused tail; replayed from a HIP graph as well (these forms copy nothing from the host)"""
+    c = Case(tmp_path, grids, layout)
+    H, F, E = c.cfg["hidden"], c.cfg["ffn"], 16
+    gb = c.layouts[0].gate_bytes
+    table_ptr = c.pool.residency_table_init(3, E)
+    for e in range(E):
+        c.pool.residency_set(1, e, c.slot_of[e])
+    c.pool.residency_clear(1, 5)
+    g_addr = [c.pool.addresses(c.slot_of[e], c.layouts[e])[0] for e in range(E)]
+    host_table = read_device(table_ptr, 3 * E * 8, np.uint64).reshape(3, E)
+    assert host_table[0].sum() == 0 and host_table[2].sum() == 0 and host_table[1][5] == 0
+    assert all(int(host_table[1][e]) == g_addr[e] for e in range(E) if e != 5)
+    rng = np.random.default_rng(9)
+    experts = np.array([3, 11, 0, 7, 9, 14])
+    w = (rng.random(6).astype(np.float32) + 0.1)
+    x = synth.normed_x(rng, 2, H)
+    slots_dev = torch.from_numpy(np.array([g_addr[e] for e in experts], np.uint64).view(np.int64)).cuda()
+    w_dev, x_dev = torch.from_numpy(w).cuda(), torch.from_numpy(x).cuda()
+    out = torch.zeros(H, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    c.pool.encode_device_into(stream, slots_dev.data_ptr(), w_dev.data_ptr(), 6, c.word, H, F, gb, gb, x_dev.data_ptr(), out.data_ptr())
+    want0 = c.want(experts, w, x[0])
+    assert rel_l2(out.cpu().numpy(), want0) <= REL_L2_TOL
+    # the sum left to the caller: tmp[e][r] in the pool's buffer
+    c.pool.encode_device_into(stream, slots_dev.data_ptr(), w_dev.data_ptr(), 6, c.word, H, F, gb, gb, x_dev.data_ptr(), None)
+    torch.cuda.synchronize()
+    tmp = read_device(c.pool.tmp_buffer(), 6 * H * 4, np.float32).reshape(6, H)
+    for k, e in enumerate(experts):
+        assert rel_l2(tmp[k], c.want([e], [1.0], x[0])) <= REL_L2_TOL
+    # two input vectors: experts 0..3 on x[0], 4..5 on x[1]
+    c.pool.encode_device_into(stream, slots_dev.data_ptr(), w_dev.data_ptr(), 6, c.word, H, F, gb, gb, x_dev[0].data_ptr(), out.data_ptr(),
+                              x1_dev=x_dev[1].data_ptr(), x_split=4)
+    want2 = c.want(experts[:4], w[:4], x[0]) + c.want(experts[4:], w[4:], x[1])
+    assert rel_l2(out.cpu().numpy(), want2) <= REL_L2_TOL
+    # fused tail: x = layer_out = resid + (routed + shared * scalar)
+    resid, shared = torch.from_numpy(synth.normed_x(rng, 2, H)).cuda()
+    scalar = torch.tensor([0.37], device="cuda")
+    x_out, layer_out = torch.zeros(H, device="cuda"), torch.zeros(H, device="cuda")
+    assert c.pool.encode_device_tail(stream, slots_dev.data_ptr(), w_dev.data_ptr(), 6, c.word, H, F, gb, gb, x_dev.data_ptr(), resid.data_ptr(),
+                                     shared.data_ptr(), scalar.data_ptr(), x_out.data_ptr(), layer_out.data_ptr()) == 1
+    want_tail = resid.cpu().numpy().astype(np.float64) + (want0 + shared.cpu().numpy().astype(np.float64) * 0.37)
+    assert torch.equal(x_out, layer_out) and rel_l2(x_out.cpu().numpy(), want_tail) <= REL_L2_TOL
+    big = torch.zeros(65, dtype=torch.int64, device="cuda")
+    assert c.pool.encode_device_tail(stream, big.data_ptr(), w_dev.data_ptr(), 65, c.word, H, F, gb, gb, x_dev.data_ptr(), resid.data_ptr(),
+                                     shared.data_ptr(), scalar.data_ptr(), x_out.data_ptr(), layer_out.data_ptr()) == -1
+    with pytest.raises(RedHipError, match="matrix byte mismatch"):
+        c.pool.encode_device_into(stream, slots_dev.data_ptr(), w_dev.data_ptr(), 6, c.word, H, F, gb + 66, gb, x_dev.data_ptr(), out.data_ptr())
+    # graph replays of the device-driven form against its eager result
+    eager = torch.zeros(H, device="cuda")
+    c.pool.encode_device_into(stream, slots_dev.data_ptr(), w_dev.data_ptr(), 6, c.word, H, F, gb, gb, x_dev.data_ptr(), eager.data_ptr())
+    torch.cuda.synchronize()
+    side = torch.cuda.Stream()
+    graph = torch.cuda.CUDAGraph()
+    gout = torch.zeros(H, device="cuda")
+    with torch.cuda.stream(side):
+        with torch.cuda.graph(graph, stream=side):
+            c.pool.encode_device_into(side.cuda_stream, slots_dev.data_ptr(), w_dev.data_ptr(), 6, c.word, H, F, gb, gb, x_dev.data_ptr(), gout.data_ptr())
+    for _ in range(3):
+        gout.zero_()
+        torch.cuda.synchronize()
+        graph.replay()
+        torch.cuda.synchronize()
+        assert torch.equal(gout, eager)
+        c.pool.encode_device_into(stream, slots_dev.data_ptr(), w_dev.data_ptr(), 6, c.word, H, F, gb, gb, x_dev[1].data_ptr(), out.data_ptr())
+        torch.cuda.synchronize()
+    del graph
+    c.pool.close()
+
+
+@pytest.mark.parametrize("layout", ["iq2", "f2", "xs"])
+def test_batched_and_mapped_pairs(tmp_path, grids, layout):
+    """prefill form: pairs sorted by expert over a ragged routing (an expert with 19 pairs, experts with one, experts with none), tokens
+    tok_first .. of a larger buffer; the same pairs on experts read in place from device copies of the whole tensors"""
+    c = Case(tmp_path, grids, layout)
+    H, F, E, K = c.cfg["hidden"], c.cfg["ffn"], 16, 3
+    rng = np.random.default_rng(10)
+    tok_first, ntok = 2, 21
+    ids = np.stack([rng.permutation(12)[:K] for _ in range(ntok)]).astype(np.uint32)
+    ids[:19, 1] = 13                                                   # a popular expert: three slices of eight pairs
+    ids[:19, 0] = np.where(ids[:19, 0] == 13, 14, ids[:19, 0])
+    ids[:19, 2] = np.where(ids[:19, 2] == 13, 15, ids[:19, 2])
+    for t in range(ntok):
+        assert len(set(ids[t].tolist())) == K
+    w = (rng.random((ntok, K)).astype(np.float32) + 0.1)
+    uid, start, ptok, pw, tp = orc.group_pairs(ids, w, E)
+    x = synth.normed_x(rng, tok_first + ntok, H)
+    x_dev = torch.from_numpy(x).cuda()
+    out = torch.full((tok_first + ntok, H), 7.0, device="cuda")
+    stream = torch.cuda.current_stream().cuda_stream
+    slots = [c.slot_of[int(e)] for e in uid]
+    c.pool.encode_batched(stream, slots, [c.layouts[int(e)] for e in uid], c.word, H, F, tok_first, ntok, K, ptok + tok_first, pw, start, tp,
+                          x_dev.data_ptr(), out.data_ptr())
+    assert all(c.pool.slot_inflight(s) for s in slots)
+    torch.cuda.synchronize()
+    c.pool.release(slots)
+    got = out.cpu().numpy()
+    assert (got[:tok_first] == 7.0).all()                              # rows before tok_first are not written
+    for t in range(ntok):
+        assert rel_l2(got[tok_first + t], c.want(ids[t], w[t], x[tok_first + t])) <= REL_L2_TOL, t
+    # mapped: whole tensors on the device, experts addressed by id
+    g_dev, u_dev, d_dev = (torch.from_numpy(np.ascontiguousarray(c.lay[k])).cuda() for k in ("gate", "up", "down"))
+    out2 = torch.zeros_like(out)
+    L0 = c.layouts[0]
+    c.pool.encode_mapped(stream, g_dev.data_ptr(), u_dev.data_ptr(), d_dev.data_ptr(), L0.gate_bytes, L0.up_bytes, L0.down_bytes, uid, c.word, H, F,
+                         tok_first, ntok, K, ptok + tok_first, pw, start, tp, x_dev.data_ptr(), out2.data_ptr())
+    torch.cuda.synchronize()
+    assert torch.equal(out2[tok_first:], out[tok_first:])              # same kernels on the same bytes
+    with pytest.raises(RedHipError, match="expert_start is inconsistent"):
+        c.pool.encode_batched(stream, slots, [c.layouts[int(e)] for e in uid], c.word, H, F, tok_first, ntok, K, ptok + tok_first, pw, start[::-1].copy(), tp,
+                              x_dev.data_ptr(), out.data_ptr())
+    with pytest.raises(RedHipError, match="pair token out of range"):
+        c.pool.encode_batched(stream, slots, [c.layouts[int(e)] for e in uid], c.word, H, F, 0, ntok, K, ptok + tok_first, pw, start, tp,
+                              x_dev.data_ptr(), out.data_ptr())
+    c.pool.close()
