@@ -322,6 +322,9 @@ __global__ __launch_bounds__(kWaves * 64) void prefill_down_kernel(PrefillArgs a
 // scales its sums once per chunk instead of once per group (22 bits below the largest activation of 256 columns is ample
 // for a dot product).
 constexpr int kRegWaves = 8;
+// The gate/up tile kernel works in items of kItemUnits units of 32 FFN columns (= one 128-column chunk of the down kernels) and leaves
+// one activation exponent per pair and item: kExpPerPair ints per pair (ffn <= 512).
+constexpr uint32_t kItemUnits = 4u, kExpPerPair = 4u;
 constexpr uint32_t kScaledMagBytes = 16u * 256u * 16u;      // [group scale s][grid entry]
 constexpr uint32_t kSignBytes = 128u * 16u;                 // [seven sign bits] (the eighth sign is their parity)
 
@@ -465,28 +468,29 @@ template <int NKC, int FMT>          // hidden = 512 * NKC; FMT 0: tile-major pa
 __global__ __launch_bounds__(kRegWaves * 64) void prefill_gateup_reg_kernel(TiledArgs ta) {
     const PrefillArgs &a = ta.p;
     constexpr uint32_t H = 512u * NKC, HG = H / 32u, HB = H / 256u, GQ = HG / 4u, NC = H / 128u;   // GQ: groups per K quarter = 4 NKC
-    extern __shared__ __attribute__((aligned(16))) uint8_t dyn[];          // acts: [16][F + 4] f32
+    extern __shared__ __attribute__((aligned(16))) uint8_t dyn[];          // acts: [16][128 + 4] f32
     __shared__ __attribute__((aligned(16))) uint8_t tables[reg_table_bytes<FMT>()];      // static: table reads take immediate offsets
     __shared__ float part[2][4][kTile][68];                // [unit parity][K quarter][pair][gate 0..31 | up 0..31], padded
     __shared__ float tok_scale[kTile];
     __shared__ uint32_t tok_of[kTile];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, r = lane & 15u, q = lane >> 4;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6), kc = wave & 3u, rh = wave >> 2;
-    const uint32_t F = a.ffn, FG = F / 32u, P = a.ntok * a.top_k, AROW = F + 4u;
+    const uint32_t F = a.ffn, FG = F / 32u, P = a.ntok * a.top_k;
+    constexpr uint32_t FGH = kItemUnits, AROW = 32u * kItemUnits + 4u;
     float *acts = reinterpret_cast<float *>(dyn);
     build_reg_tables<FMT>(tables, tid, kRegWaves * 64u, ta.grid);
     const uint32_t T = a.n_tiles[0], U = a.n_unique[0];
     const uint64_t qs_bytes = (uint64_t)F * HG * 8u, sc_off = qs_bytes + (uint64_t)F * HB * 2u, gate_bytes = sc_off + (FMT == 1 ? (uint64_t)F * HG : 0u);
 
-    // Work items are half tiles (one half of the FFN columns, with an activation exponent of its own) so that the last round of
-    // the persistent workgroups is short; a workgroup takes a contiguous range of items and keeps its A operands when two of
-    // them share a tile.
-    const uint32_t items = 2u * T, FGH = FG / 2u;
+    // Work items are parts of tiles (128 of the FFN columns, with an activation exponent of their own) so that the last round of
+    // the persistent workgroups is short (with half tiles as items a chunk of 544 tiles gave four items to some workgroups and five
+    // to others); a workgroup takes a contiguous range of items and keeps its A operands when consecutive ones share a tile.
+    const uint32_t parts = FG / FGH, items = parts * T;
     const uint32_t item_begin = (uint32_t)(((uint64_t)blockIdx.x * items) / gridDim.x), item_end = (uint32_t)(((uint64_t)(blockIdx.x + 1u) * items) / gridDim.x);
     Half8 xa[GQ], xb[GQ];
     uint32_t have_tile = 0xffffffffu;
     for (uint32_t item = item_begin; item < item_end; ++item) {
-        const uint32_t tile = item >> 1, half = item & 1u, j0 = half * FGH;
+        const uint32_t tile = item / parts, ipart = item % parts, j0 = ipart * FGH;
         const uint32_t u = a.tile_group[tile], p0 = a.tile_pair0[tile], n = a.tile_n[tile];
         const uint8_t *ex = u == U ? ta.shared : ta.experts + (uint64_t)a.uid[u] * a.stride;
         __syncthreads();                                   // the previous item's readers are done with acts / tok_of; tables are built
@@ -569,29 +573,29 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_gateup_reg_kernel(Tile
                 const uint32_t i = tid >> 5, c = tid & 31u;
                 const float gsum = ((pt[0][i][c] + pt[1][i][c]) + (pt[2][i][c] + pt[3][i][c])) * tok_scale[i];
                 const float usum = ((pt[0][i][32u + c] + pt[1][i][32u + c]) + (pt[2][i][32u + c] + pt[3][i][32u + c])) * tok_scale[i];
-                acts[i * AROW + 32u * j + c] = (gsum / (1.0f + expf(-gsum))) * usum;
+                acts[i * AROW + 32u * (j - j0) + c] = (gsum / (1.0f + expf(-gsum))) * usum;
             }
         }
         __syncthreads();
-        // one exponent per pair and column half, then the fp16 halves: wave w takes pairs 2 w and 2 w + 1
+        // one exponent per pair and part, then the fp16 halves: wave w takes pairs 2 w and 2 w + 1
         const uint32_t c0 = 32u * j0, c1 = c0 + 32u * FGH;
 #pragma unroll
         for (uint32_t h = 0; h < 2u; ++h) {
             const uint32_t i = 2u * wave + h;
             if (i >= n) continue;                          // wave-uniform
             if (ta.act_f32) {
-                for (uint32_t c = c0 + lane; c < c1; c += 64u) ta.act_f32[(uint64_t)(p0 + i) * F + c] = acts[i * AROW + c];
+                for (uint32_t c = c0 + lane; c < c1; c += 64u) ta.act_f32[(uint64_t)(p0 + i) * F + c] = acts[i * AROW + c - c0];
                 continue;
             }
             float amax = 0.0f;
-            for (uint32_t c = c0 + lane; c < c1; c += 64u) amax = fmaxf(amax, fabsf(acts[i * AROW + c]));
+            for (uint32_t c = c0 + lane; c < c1; c += 64u) amax = fmaxf(amax, fabsf(acts[i * AROW + c - c0]));
 #pragma unroll
             for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
             const int e = prescale_exp(amax);
             const float inv = exp2i(-e);
             const uint64_t pr = p0 + i;
-            for (uint32_t c = c0 + lane; c < c1; c += 64u) split_hi_lo(acts[i * AROW + c], inv, a.act_h + pr * F + c, a.act_l + pr * F + c);
-            if (lane == 0u) a.act_exp[2u * pr + half] = e;
+            for (uint32_t c = c0 + lane; c < c1; c += 64u) split_hi_lo(acts[i * AROW + c - c0], inv, a.act_h + pr * F + c, a.act_l + pr * F + c);
+            if (lane == 0u) a.act_exp[kExpPerPair * pr + ipart] = e;
         }
     }
 }
@@ -602,7 +606,7 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_down_reg_kernel(TiledA
     const PrefillArgs &a = ta.p;
     constexpr uint32_t F = 32u * NFG, FB = F / 256u, NCK = NFG / 4u;
     __shared__ __attribute__((aligned(16))) uint8_t tables[reg_table_bytes<FMT>()];      // static: table reads take immediate offsets
-    __shared__ __attribute__((aligned(16))) float pair_scale[2][kTile];      // per column half of the activations
+    __shared__ __attribute__((aligned(16))) float pair_scale[kExpPerPair][kTile];      // per 128-column chunk of the activations
     const uint32_t tid = threadIdx.x, lane = tid & 63u, r = lane & 15u, q = lane >> 4;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t H = a.hidden, P = a.ntok * a.top_k;
@@ -612,9 +616,9 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_down_reg_kernel(TiledA
     const uint64_t sc_off = qs_bytes + (uint64_t)H * FB * 2u;
     constexpr uint32_t kRowsPerPass = 16u * kRegWaves;
 
-    // Work items are half tiles (the row passes of a tile cut in two) so that the last round of the persistent workgroups is
-    // short; a workgroup takes a contiguous range of items and keeps the activations when two of them share a tile.
-    const uint32_t n_pass_tile = H / kRowsPerPass, parts = n_pass_tile % 2u == 0u ? 2u : 1u, n_pass = n_pass_tile / parts;
+    // Work items are quarter tiles (the row passes of a tile cut in four) so that the last round of the persistent workgroups is
+    // short; a workgroup takes a contiguous range of items and keeps the activations when consecutive ones share a tile.
+    const uint32_t n_pass_tile = H / kRowsPerPass, parts = n_pass_tile % 4u == 0u ? 4u : n_pass_tile % 2u == 0u ? 2u : 1u, n_pass = n_pass_tile / parts;
     const uint32_t items = T * parts;
     const uint32_t item_begin = (uint32_t)(((uint64_t)blockIdx.x * items) / gridDim.x), item_end = (uint32_t)(((uint64_t)(blockIdx.x + 1u) * items) / gridDim.x);
     Half8 xa[NFG], xb[NFG];
@@ -626,7 +630,7 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_down_reg_kernel(TiledA
         if (tile != have_tile) {
             have_tile = tile;
             __syncthreads();
-            if (tid < 2u * kTile) pair_scale[tid & 1u][tid >> 1] = (tid >> 1) < n ? (FMT == 2 ? 1.0f : 0.125f) * exp2i(a.act_exp[2u * p0 + tid]) : 0.0f;
+            if (tid < kExpPerPair * kTile && (tid & 3u) < NCK) pair_scale[tid & 3u][tid >> 2] = (tid >> 2) < n ? (FMT == 2 ? 1.0f : 0.125f) * exp2i(a.act_exp[kExpPerPair * p0 + tid]) : 0.0f;
             __syncthreads();
             const uint64_t base = (uint64_t)(p0 + r) * F + 8u * q;
             const bool live = r < n;
@@ -640,7 +644,6 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_down_reg_kernel(TiledA
                 }
             }
         }
-        const float4_t ps0 = *reinterpret_cast<const float4_t *>(&pair_scale[0][4u * q]), ps1 = *reinterpret_cast<const float4_t *>(&pair_scale[1][4u * q]);
         auto load_chunk = [&](uint32_t b, uint32_t c) {
             const uint32_t rtile = kRegWaves * (pass0 + b) + wave;
             if constexpr (FMT == 0) {
@@ -678,8 +681,9 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_down_reg_kernel(TiledA
                     hi = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[g].v, bw, hi, 0, 0, 0);
                     lo = __builtin_amdgcn_mfma_f32_16x16x32_f16(xb[g].v, bw, lo, 0, 0, 0);
                 }
+                const float4_t ps = *reinterpret_cast<const float4_t *>(&pair_scale[c][4u * q]);
 #pragma unroll
-                for (int t = 0; t < 4; ++t) tot[t] = fmaf(fmaf(lo[t], 4.8828125e-4f, hi[t]) * d, 2u * c < NCK ? ps0[t] : ps1[t], tot[t]);
+                for (int t = 0; t < 4; ++t) tot[t] = fmaf(fmaf(lo[t], 4.8828125e-4f, hi[t]) * d, ps[t], tot[t]);
             }
             const uint32_t row = kRowsPerPass * (pass0 + b) + 16u * wave + r;
 #pragma unroll
@@ -760,7 +764,7 @@ __device__ __forceinline__ half8_t decode_iq3s(uint32_t w, const uint8_t *sgn, c
 }
 
 struct Iq3DownArgs {
-    PrefillArgs p;                 // act_h / act_l / act_exp (two exponents per pair) from the gate/up kernel, tmp out; routed tiles only
+    PrefillArgs p;                 // act_h / act_l / act_exp (kExpPerPair exponents per pair) from the gate/up kernel, tmp out; routed tiles only
     const uint8_t *experts;        // tile-major IQ3_S down matrices
     uint64_t stride;
 };
@@ -771,7 +775,7 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_down_iq3s_kernel(Iq3Do
     const PrefillArgs &a = da.p;
     constexpr uint32_t F = 32u * NFG, FB = F / 256u, NCK = NFG / 4u;
     __shared__ __attribute__((aligned(16))) uint8_t tables[kIq3SignBytes + kIq3MagBytes];      // static: table reads take immediate offsets
-    __shared__ __attribute__((aligned(16))) float pair_scale[2][kTile];
+    __shared__ __attribute__((aligned(16))) float pair_scale[kExpPerPair][kTile];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, r = lane & 15u, q = lane >> 4;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     const uint32_t H = a.hidden;
@@ -780,7 +784,7 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_down_iq3s_kernel(Iq3Do
     const uint32_t T = a.n_tiles[0];
     const uint64_t qs_bytes = (uint64_t)H * NFG * 16u;
     constexpr uint32_t kRowsPerPass = 16u * kRegWaves;
-    const uint32_t n_pass_tile = H / kRowsPerPass, parts = n_pass_tile % 2u == 0u ? 2u : 1u, n_pass = n_pass_tile / parts;
+    const uint32_t n_pass_tile = H / kRowsPerPass, parts = n_pass_tile % 4u == 0u ? 4u : n_pass_tile % 2u == 0u ? 2u : 1u, n_pass = n_pass_tile / parts;
     const uint32_t items = T * parts;
     const uint32_t item_begin = (uint32_t)(((uint64_t)blockIdx.x * items) / gridDim.x), item_end = (uint32_t)(((uint64_t)(blockIdx.x + 1u) * items) / gridDim.x);
     Half8 xa[NFG], xb[NFG];
@@ -792,7 +796,7 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_down_iq3s_kernel(Iq3Do
         if (tile != have_tile) {
             have_tile = tile;
             __syncthreads();
-            if (tid < 2u * kTile) pair_scale[tid & 1u][tid >> 1] = (tid >> 1) < n ? exp2i(a.act_exp[2u * p0 + tid]) : 0.0f;      // IQ3_S: weight = d (1 + 2 nibble) grid, no 1/8
+            if (tid < kExpPerPair * kTile && (tid & 3u) < NCK) pair_scale[tid & 3u][tid >> 2] = (tid >> 2) < n ? exp2i(a.act_exp[kExpPerPair * p0 + tid]) : 0.0f;      // IQ3_S: weight = d (1 + 2 nibble) grid, no 1/8
             __syncthreads();
             const uint64_t base = (uint64_t)(p0 + r) * F + 8u * q;
             const bool live = r < n;
@@ -806,7 +810,6 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_down_iq3s_kernel(Iq3Do
                 }
             }
         }
-        const float4_t ps0 = *reinterpret_cast<const float4_t *>(&pair_scale[0][4u * q]), ps1 = *reinterpret_cast<const float4_t *>(&pair_scale[1][4u * q]);
         struct Chunk { uint4 w; uint32_t d; };
         auto load_chunk = [&](uint32_t b, uint32_t c) {
             const uint32_t rtile = kRegWaves * (pass0 + b) + wave;
@@ -835,8 +838,9 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_down_iq3s_kernel(Iq3Do
                     hi = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[g].v, bw, hi, 0, 0, 0);
                     lo = __builtin_amdgcn_mfma_f32_16x16x32_f16(xb[g].v, bw, lo, 0, 0, 0);
                 }
+                const float4_t ps = *reinterpret_cast<const float4_t *>(&pair_scale[c][4u * q]);
 #pragma unroll
-                for (int t = 0; t < 4; ++t) tot[t] = fmaf(fmaf(lo[t], 4.8828125e-4f, hi[t]) * d, 2u * c < NCK ? ps0[t] : ps1[t], tot[t]);
+                for (int t = 0; t < 4; ++t) tot[t] = fmaf(fmaf(lo[t], 4.8828125e-4f, hi[t]) * d, ps[t], tot[t]);
             }
             const uint32_t row = kRowsPerPass * (pass0 + b) + 16u * wave + r;
 #pragma unroll
@@ -971,8 +975,8 @@ hipError_t launch_swiglu_rows(const float *gu, uint32_t gu_stride, uint32_t ntok
 }
 
 static hipError_t launch_gateup_reg(const TiledArgs &ta, dim3 grid, hipStream_t s, uint32_t fmt = 0u) {
-    const uint32_t hidden = ta.p.hidden, ffn = ta.p.ffn;
-    const size_t acts_lds = (size_t)kTile * (ffn + 4u) * sizeof(float);
+    const uint32_t hidden = ta.p.hidden;
+    const size_t acts_lds = (size_t)kTile * (32u * kItemUnits + 4u) * sizeof(float);
     hipError_t e = hipSuccess;
     prof_set_stage(ST_PREFILL_GATEUP);
 #define REDHIP_PGR_ONE(NKC, FMT)                                                                                                          \
