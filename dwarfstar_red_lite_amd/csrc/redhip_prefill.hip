@@ -433,7 +433,48 @@ __device__ __forceinline__ uint32_t odd_scale_splat(uint32_t s) {
     const uint32_t h = __builtin_bit_cast(uint16_t, (_Float16)(float)(2u * s + 1u));
     return h | (h << 16);
 }
-// the eight signed, scaled fp16 weights of entry q (eight columns) of a group: w = the group's uint2, sc = its IQ2_XS scale byte
+// The decode in two steps, so that a kernel can have the table reads of the next groups in flight while it finishes this one:
+// fetch_reg issues the LDS reads of entry q (eight columns) of a group, finish_reg turns what they returned into the eight signed,
+// scaled fp16 weights. w = the group's uint2, sc = its IQ2_XS scale byte.
+struct RawEntry { uint4 m, g; };
+template <int FMT>
+__device__ __forceinline__ RawEntry fetch_reg(uint2 w, uint32_t q, const uint8_t *tables) {
+    RawEntry e;
+    if constexpr (FMT == 0) {
+        const uint32_t idx = __builtin_amdgcn_ubfe(w.x, 8u * q, 8u), s7 = __builtin_amdgcn_ubfe(w.y, 7u * q, 7u);
+        e.m = *reinterpret_cast<const uint4 *>(tables + kSignBytes + ((((w.y >> 28) << 8) | idx) << 4));
+        e.g = *reinterpret_cast<const uint4 *>(tables + (s7 << 4));
+    } else if constexpr (FMT == 1) {
+        const uint32_t w16 = (((q & 2u) ? w.y : w.x) >> (16u * (q & 1u))) & 0xffffu;
+        e.m = *reinterpret_cast<const uint4 *>(tables + kSignBytes + ((w16 & 511u) << 4));
+        e.g = *reinterpret_cast<const uint4 *>(tables + ((w16 >> 9) << 4));
+    } else {
+        const uint32_t idx = ((w.x >> (8u * q)) & 255u) | (((w.y >> (4u * q)) & 7u) << 8);
+        e.m = *reinterpret_cast<const uint4 *>(tables + (idx << 4));
+        e.g = e.m;
+    }
+    return e;
+}
+template <int FMT>
+__device__ __forceinline__ half8_t finish_reg(const RawEntry &e, uint2 w, uint32_t sc, uint32_t q) {
+    const uint4 m = e.m, g = e.g;
+    Half8 r;
+    if constexpr (FMT == 0) {
+        r.u = make_uint4(m.x ^ g.x, m.y ^ g.y, m.z ^ g.z, m.w ^ g.w);
+    } else if constexpr (FMT == 1) {
+        const half2_t f = __builtin_bit_cast(half2_t, odd_scale_splat((sc >> (4u * (q >> 1))) & 15u));
+        r.u = make_uint4(__builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, m.x ^ g.x) * f), __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, m.y ^ g.y) * f),
+                         __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, m.z ^ g.z) * f), __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, m.w ^ g.w) * f));
+    } else {
+        const uint32_t fs = odd_scale_splat((w.y >> (16u + 3u * (q >> 1))) & 7u);
+        const half2_t f = __builtin_bit_cast(half2_t, fs);
+        const half2_t off = __builtin_bit_cast(half2_t, (fs - 0x0c000c00u) ^ (((w.y >> (4u * q + 3u)) & 1u) * 0x80008000u));
+        r.u = make_uint4(__builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, m.x) * f + off), __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, m.y) * f + off),
+                         __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, m.z) * f + off), __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, m.w) * f + off));
+    }
+    return r.v;
+}
+// both steps at once
 template <int FMT>
 __device__ __forceinline__ half8_t decode_reg(uint2 w, uint32_t sc, uint32_t q, const uint8_t *tables) {
     if constexpr (FMT == 0) {
@@ -544,10 +585,20 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_gateup_reg_kernel(Tile
                 // the four groups of the chunk share the block scale d: their products add up in the matrix units, activations
                 // hi and lo in accumulators of their own
                 float4_t gh = {0.0f, 0.0f, 0.0f, 0.0f}, gl = gh, uh = gh, ul = gh;
+                // the table reads run two groups ahead of the arithmetic: a wave that waits for every read before it issues the next
+                // spends most of its time on LDS round trips (two waves per SIMD do not hide them)
+                RawEntry rg0 = fetch_reg<FMT>(wg4[0], q, tables), ru0 = fetch_reg<FMT>(wu4[0], q, tables);
+                RawEntry rg1 = fetch_reg<FMT>(wg4[1], q, tables), ru1 = fetch_reg<FMT>(wu4[1], q, tables);
 #pragma unroll
                 for (uint32_t k = 0; k < 4u; ++k) {
                     const uint32_t g = 4u * c + k;
-                    const half8_t bg = decode_reg<FMT>(wg4[k], cg.sc >> (8u * k), q, tables), bu = decode_reg<FMT>(wu4[k], cu.sc >> (8u * k), q, tables);
+                    __builtin_amdgcn_sched_barrier(0);
+                    const half8_t bg = finish_reg<FMT>(k & 1u ? rg1 : rg0, wg4[k], cg.sc >> (8u * k), q), bu = finish_reg<FMT>(k & 1u ? ru1 : ru0, wu4[k], cu.sc >> (8u * k), q);
+                    if (k + 2u < 4u) {
+                        if (k & 1u) { rg1 = fetch_reg<FMT>(wg4[k + 2u], q, tables); ru1 = fetch_reg<FMT>(wu4[k + 2u], q, tables); }
+                        else { rg0 = fetch_reg<FMT>(wg4[k + 2u], q, tables); ru0 = fetch_reg<FMT>(wu4[k + 2u], q, tables); }
+                    }
+                    __builtin_amdgcn_sched_barrier(0);
                     gh = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[g].v, bg, gh, 0, 0, 0);
                     gl = __builtin_amdgcn_mfma_f32_16x16x32_f16(xb[g].v, bg, gl, 0, 0, 0);
                     uh = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[g].v, bu, uh, 0, 0, 0);
