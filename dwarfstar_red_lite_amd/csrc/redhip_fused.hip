@@ -1753,8 +1753,11 @@ __device__ __forceinline__ void group_dot2_rep(uint2 q, const half4_t *ax, const
 // One workgroup per (pass, column group) - the hardware's own dispatch balances the units over the compute units (persistent workgroups
 // that walked a unit list with the next unit's weights requested ahead were measured too: slower at 2, 4 and 8 tokens, their start-up
 // and the coarser balance cost more than the requests they hide).
-// Both tables eight times here (lanes l and l + 8 share a copy and collide now and then): 56 KB of LDS and at most 64 registers per lane,
-// so that two workgroups fit a compute unit and one's weight requests and barriers hide behind the other's arithmetic.
+// The magnitude table sixteen times, the signs placed by integer arithmetic (no sign table): 74 KB of LDS and at most 64 registers per
+// lane, so that two workgroups fit a compute unit and one's weight requests and barriers hide behind the other's arithmetic. Measured
+// at 8 tokens with 32 hot experts: this 27.7 us; eight copies of the magnitude table 28.3 us (38 % of its LDS cycles are bank
+// conflicts: the LDS serves sixteen lanes of a 16-byte read together); eight copies of both tables 34.3 us (a fifth fewer vector
+// instructions, 70 % more LDS reads); sixteen copies of both at one workgroup per compute unit 43.5 us.
 constexpr int kBatchRep = 16, kBatchSignRep = 0;
 template <int NKC, int REP>
 __global__ __launch_bounds__(kWaves * 64, 8) void batch_slice_kernel(BatchSliceArgs a) {
