@@ -36,6 +36,7 @@ struct TopkPool {
     std::vector<uint32_t> inflight, generation;
     std::mutex mu;                                // counters, slab creation, marks, residency mirror
     std::mutex exec_mu;                           // `execute` stages through buffers of the pool: one at a time
+    std::recursive_mutex enc_mu;                  // an encode call sizes and fills buffers of the pool: host side one call at a time
     uint64_t bytes_read = 0, read_calls = 0;
     double read_ms = 0.0;
     std::vector<int8_t> iq2_xs, iq1_m;
@@ -160,6 +161,7 @@ __global__ __launch_bounds__(256) void topk_tail_kernel(const float *tmp, const 
 bool enqueue_token(TopkPool *p, hipStream_t s, const uint64_t *table_dev, const float *weights_dev, uint32_t top_k, uint32_t type_word,
                    uint32_t hidden, uint32_t ffn, uint64_t gate_bytes, uint64_t up_bytes, uint32_t row_start, uint32_t row_count,
                    const float *x, const float *x1, uint32_t x_split, float *out, const Tail *tail) {
+    std::lock_guard<std::recursive_mutex> lk(p->enc_mu);
     if (!bind_grids(p, type_word) || !ensure_scratch(p, REDMETAL_TOPK_MAX, hidden, ffn)) return false;
     ExpertSet ex{nullptr, 0, gate_bytes, up_bytes, word_gate_up(type_word), word_down(type_word)};
     ex.table = table_dev;
@@ -229,6 +231,7 @@ bool enqueue_pairs(TopkPool *p, hipStream_t s, const std::vector<uint64_t> &gate
                    uint64_t up_delta, uint64_t down_off, uint32_t n_expert, uint32_t type_word, uint32_t hidden, uint32_t ffn,
                    uint32_t tok_first, uint32_t ntok, uint32_t top_k, uint32_t n_pairs, const uint32_t *pair_token,
                    const float *pair_weight, const uint32_t *expert_start, const uint32_t *tok_pair, const float *x, float *out) {
+    std::lock_guard<std::recursive_mutex> lk(p->enc_mu);
     if (!bind_grids(p, type_word) || !ensure_scratch(p, n_pairs, hidden, ffn)) return false;
     std::vector<uint64_t> table(gate_table);
     table.insert(table.end(), down_table.begin(), down_table.end());
@@ -504,6 +507,7 @@ int redmetal_topk_pool_encode(redmetal_topk_pool_t h, void *stream, const uint32
         table[i] = (uint64_t)(uintptr_t)base;
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
+    std::lock_guard<std::recursive_mutex> lk(p->enc_mu);
     Staged st;
     if (!stage_lists(p, s, table, router_weights, top_k, {}, &st)) return 0;
     const bool ok = enqueue_token(p, s, st.table, st.w, top_k, ggml_type, hidden_size, ffn_size, gate_bytes[0], up_bytes[0], output_row_start,
