@@ -26,6 +26,7 @@
 // Layout ("packed IQ2_XXS"): the 66-byte blocks are split at upload into an 8-byte stream [row][group] (4 grid
 // indices + 28 sign bits + 4 scale bits per 32 weights) and an fp16 stream [row][block] (d per 256 weights), both
 // naturally aligned. Same total bytes as the GGUF blocks.
+#include <type_traits>
 #include <hip/hip_fp16.h>
 
 #include "redhip_decode.h"
@@ -1424,6 +1425,44 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_select_kernel(GateUpArgs a
     }
 }
 
+// ---- word-packed IQ3_S (see the section on IQ3_S down matrices below for the format): the decode shared by the kernels that read it
+constexpr uint32_t kIq3TableBytes = 512u * 8u;
+// LDS table: the four bytes of every grid entry as fp16; built by the first 512 lanes of a workgroup
+__device__ __forceinline__ void build_iq3s_quads(uint8_t *lds, uint32_t tid) {
+    if (tid < 512u) {
+        const uint32_t e = redhip_iq3s_grid[tid];
+        uint32_t w2[2];
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const _Float16 lo = (_Float16)(float)((e >> (16 * i)) & 255u), hi = (_Float16)(float)((e >> (16 * i + 8)) & 255u);
+            w2[i] = (uint32_t)__builtin_bit_cast(uint16_t, lo) | ((uint32_t)__builtin_bit_cast(uint16_t, hi) << 16);
+        }
+        *reinterpret_cast<uint2 *>(lds + (size_t)tid * 8u) = make_uint2(w2[0], w2[1]);
+    }
+}
+
+// 32 weights (one uint4 of words) against an activation operand that carries one token (rows 0, 1 = hi, lo) or two (rows 2, 3 the
+// second): va = first token's product, vb = the second's; scale nibble applied, d is not.
+__device__ __forceinline__ void iq3s_group_dot(uint4 q, const half4_t *ax, const uint8_t *lds, float &va, float &vb) {
+    const uint32_t w4[4] = {q.x, q.y, q.z, q.w};
+    float4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+#pragma unroll
+    for (uint32_t l = 0; l < 4u; ++l) {
+        const uint2 ma = *reinterpret_cast<const uint2 *>(lds + ((w4[l] & 511u) << 3)), mb = *reinterpret_cast<const uint2 *>(lds + (((w4[l] >> 9) & 511u) << 3));
+        const uint32_t s8s = ((w4[l] >> 18) & 255u) << 8;          // sign bit k of the eight at bit 8 + k, as place_signs takes them
+        WeightQuad b0, b1;
+        b0.u[0] = (__umul24(s8s, (1u << 7) | (1u << 22)) & 0x80008000u) | ma.x;
+        b0.u[1] = (__umul24(s8s, (1u << 5) | (1u << 20)) & 0x80008000u) | ma.y;
+        b1.u[0] = (__umul24(s8s, (1u << 3) | (1u << 18)) & 0x80008000u) | mb.x;
+        b1.u[1] = (__umul24(s8s, (1u << 1) | (1u << 16)) & 0x80008000u) | mb.y;
+        acc = __builtin_amdgcn_mfma_f32_4x4x4f16(ax[2u * l], b0.h, acc, 0, 0, 0);
+        acc = __builtin_amdgcn_mfma_f32_4x4x4f16(ax[2u * l + 1u], b1.h, acc, 0, 0, 0);
+    }
+    const float sc = (float)(2u * ((q.x >> 26) & 15u) + 1u);
+    va = (acc[0] + acc[1] * 4.8828125e-4f) * sc;
+    vb = (acc[2] + acc[3] * 4.8828125e-4f) * sc;
+}
+
 // ---------------------------------------------------------------- one token on all-IQ2_XXS layers: expert slices
 //
 // One workgroup per (slot, 32 ffn columns): it selects (or takes the caller's routing), multiplies its 32 gate rows and 32 up rows
@@ -1730,6 +1769,9 @@ struct BatchSliceArgs {
     const int *xexp;               // [ntok]
     float *partial;                // [ntok][top_k + 1][ffn / 32][hidden]
     uint32_t hidden, ffn, top_k, ntok;
+    // mixed layouts (MIX): down_cm holds column-sliced word-packed IQ3_S matrices; the shared expert comes as its gate . x and up . x
+    // products [ntok][2 ffn] f32 (left by the router launch) and the dense f32 copy [hidden][ffn] of its down matrix
+    const float *shared_gu, *shared_dense;
 };
 
 // two tokens' results of one group: va for the token in rows 0, 1 of the operand, vb for the one in rows 2, 3
@@ -1759,7 +1801,7 @@ __device__ __forceinline__ void group_dot2_rep(uint2 q, const half4_t *ax, const
 // conflicts: the LDS serves sixteen lanes of a 16-byte read together); eight copies of both tables 34.3 us (a fifth fewer vector
 // instructions, 70 % more LDS reads); sixteen copies of both at one workgroup per compute unit 43.5 us.
 constexpr int kBatchRep = 16, kBatchSignRep = 0;
-template <int NKC, int REP>
+template <int NKC, int REP, int MIX>       // MIX 0: every matrix packed IQ2_XXS; 1: IQ3_S down matrices, dense shared expert (see BatchSliceArgs)
 __global__ __launch_bounds__(kWaves * 64, 8) void batch_slice_kernel(BatchSliceArgs a) {
     constexpr int NW = kWaves;
     constexpr int UPW = 16 * NKC / NW;
@@ -1771,6 +1813,7 @@ __global__ __launch_bounds__(kWaves * 64, 8) void batch_slice_kernel(BatchSliceA
     float *part = reinterpret_cast<float *>(strip + kMagBytes + kSignBytes);      // [2 tokens][NKC][64]
     _Float16 *act_hl = reinterpret_cast<_Float16 *>(part + 2 * NKC * 64);  // [2 tokens][2 halves][32]
     float *act_scale = reinterpret_cast<float *>(act_hl + 128);            // [2] (+ 2 unused)
+    uint8_t *iq3_tab = reinterpret_cast<uint8_t *>(act_scale + 4);         // MIX: 4 KB, the IQ3_S grid as fp16
 
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
     const uint32_t H = a.hidden, F = a.ffn, HG = H / 32u, HB = H / 256u, FG = F / 32u, K = a.top_k;
@@ -1789,6 +1832,45 @@ __global__ __launch_bounds__(kWaves * 64, 8) void batch_slice_kernel(BatchSliceA
     }
     const uint32_t expert = e.x & 0xffffu, cnt = (e.x >> 16) & 255u, tok0 = (e.y >> 16) & 255u, tok1 = e.y >> 24;
     const uint32_t k0 = sh ? K : (e.y & 255u) - tok0 * K, k1 = sh ? K : ((e.y >> 8) & 255u) - tok1 * K;
+    float *out0 = a.partial + ((uint64_t)(tok0 * (K + 1u) + k0) * FG + g) * H, *out1 = a.partial + ((uint64_t)(tok1 * (K + 1u) + k1) * FG + g) * H;
+
+    if constexpr (MIX != 0) {
+        if (sh) {      // the shared expert's slice from dense f32 data: SwiGLU of the 32 columns, then their part of every output row
+            if (tid < 64u) {
+                const uint32_t t = tid >> 5, c = tid & 31u;
+                const float *gu = a.shared_gu + (uint64_t)(t ? tok1 : tok0) * 2u * F + 32u * g + c;
+                const float gv = gu[0], uv = gu[F];
+                part[tid] = (gv / (1.0f + expf(-gv))) * uv;
+            }
+            __syncthreads();
+            // a lane pair per output row, each lane 16 of the 32 columns for both tokens: its 32 activations stay in registers
+            const uint32_t half = tid & 1u;
+            float4 av[4], bv[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                av[i] = *reinterpret_cast<const float4 *>(part + 16u * half + 4 * i);
+                bv[i] = *reinterpret_cast<const float4 *>(part + 32u + 16u * half + 4 * i);
+            }
+            const float s0 = a.scalar[tok0], s1 = a.scalar[tok1];
+            for (uint32_t h = tid >> 1; h < H; h += (uint32_t)NW * 32u) {
+                const float4 *wr = reinterpret_cast<const float4 *>(a.shared_dense + (uint64_t)h * F + 32u * g + 16u * half);
+                float4 w4[4];
+#pragma unroll
+                for (int i = 0; i < 4; ++i) w4[i] = wr[i];
+                float acc0 = 0.0f, acc1 = 0.0f;
+#pragma unroll
+                for (int i = 0; i < 4; ++i) {
+                    acc0 = fmaf(w4[i].w, av[i].w, fmaf(w4[i].z, av[i].z, fmaf(w4[i].y, av[i].y, fmaf(w4[i].x, av[i].x, acc0))));
+                    acc1 = fmaf(w4[i].w, bv[i].w, fmaf(w4[i].z, bv[i].z, fmaf(w4[i].y, bv[i].y, fmaf(w4[i].x, bv[i].x, acc1))));
+                }
+                acc0 += __shfl_xor(acc0, 1, 64);
+                acc1 += __shfl_xor(acc1, 1, 64);
+                if (half == 0u) out0[h] = acc0 * s0;
+                else if (cnt > 1u) out1[h] = acc1 * s1;
+            }
+            return;
+        }
+    }
 
     const uint32_t kc = wave % NKC, q0 = wave / NKC;
     const uint32_t G = 16u * kc + blk;
@@ -1812,9 +1894,10 @@ __global__ __launch_bounds__(kWaves * 64, 8) void batch_slice_kernel(BatchSliceA
         wq[u] = reinterpret_cast<const uint2 *>(mat)[(uint64_t)r * HG + G];
         wd[u] = reinterpret_cast<const uint16_t *>(mat + (uint64_t)F * HG * 8u)[(uint64_t)r * HB + (G >> 3)];
     }
-    const uint2 *down_qs = reinterpret_cast<const uint2 *>(dn) + (uint64_t)g * H;
-    const uint16_t *down_ds = reinterpret_cast<const uint16_t *>(dn + (uint64_t)FG * H * 8u) + (uint64_t)(g >> 3) * H;
-    uint2 dq[DU];
+    using DownGroup = typename std::conditional<MIX != 0, uint4, uint2>::type;      // one row's 32 weights of the slice
+    const DownGroup *down_qs = reinterpret_cast<const DownGroup *>(dn) + (uint64_t)g * H;
+    const uint16_t *down_ds = reinterpret_cast<const uint16_t *>(dn + (uint64_t)FG * H * sizeof(DownGroup)) + (uint64_t)(g >> 3) * H;
+    DownGroup dq[DU];
     uint32_t dd[DU];
 #pragma unroll
     for (int kk = 0; kk < DU; ++kk) {
@@ -1823,6 +1906,7 @@ __global__ __launch_bounds__(kWaves * 64, 8) void batch_slice_kernel(BatchSliceA
         dq[kk] = down_qs[r];
         dd[kk] = down_ds[r];
     }
+    if constexpr (MIX != 0) build_iq3s_quads(iq3_tab, tid);
     const float w0 = sh ? a.scalar[tok0] : a.weights[tok0 * K + k0], w1 = sh ? a.scalar[tok1] : a.weights[tok1 * K + k1];
     const float xs0 = 0.125f * exp2i(a.xexp[tok0]), xs1 = 0.125f * exp2i(a.xexp[tok1]);
     build_tables_rep<REP, 16, SREP>(lds, strip, wave, lane);
@@ -1868,14 +1952,15 @@ __global__ __launch_bounds__(kWaves * 64, 8) void batch_slice_kernel(BatchSliceA
 #pragma unroll
         for (int s8 = 0; s8 < 8; ++s8) ad[s8] = *reinterpret_cast<const half4_t *>(src + 4 * s8);
     }
-    const float post0 = act_scale[0] * w0 * 0.125f, post1 = act_scale[1] * w1 * 0.125f;
-    float *out0 = a.partial + ((uint64_t)(tok0 * (K + 1u) + k0) * FG + g) * H, *out1 = a.partial + ((uint64_t)(tok1 * (K + 1u) + k1) * FG + g) * H;
+    // (an IQ3_S weight is d (1 + 2 nibble) grid byte: no 1 / 8)
+    const float post0 = act_scale[0] * w0 * (MIX != 0 ? 1.0f : 0.125f), post1 = act_scale[1] * w1 * (MIX != 0 ? 1.0f : 0.125f);
 #pragma unroll
     for (int kk = 0; kk < DU; ++kk) {
         const uint32_t unit = wave + NW * kk;
         if (unit < 8u * NKC) {
             float da, db;
-            group_dot2_rep<REP, SREP>(dq[kk], ad, tab, stab, da, db);
+            if constexpr (MIX != 0) iq3s_group_dot(dq[kk], ad, iq3_tab, da, db);
+            else group_dot2_rep<REP, SREP>(dq[kk], ad, tab, stab, da, db);
             const float d = scale_to_f32(dd[kk]);
             out0[64u * unit + lane] = da * d * post0;
             if (cnt > 1u) out1[64u * unit + lane] = db * d * post1;
@@ -1925,23 +2010,28 @@ hipError_t launch_expert_slices(const void *experts, uint64_t stride, const void
 
 hipError_t launch_batch_slices(const void *experts, uint64_t stride, const void *down_cm, uint64_t down_stride, const void *shared, const void *shared_down_cm,
                                const void *pass_list, const uint32_t *n_pass, const float *weights, const float *scalar, const void *xh, const void *xl,
-                               const int *xexp, float *partial, float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, hipStream_t s) {
+                               const int *xexp, float *partial, float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, hipStream_t s,
+                               const float *shared_gu, const float *shared_dense) {
     if (!fused_iq2_supported(hidden, ffn) || hidden % 32u || !ntok || ntok > 16u || ntok * top_k > 128u || !pass_list || !n_pass) return hipErrorInvalidValue;
+    const bool mix = shared_gu != nullptr;
+    if (mix ? !shared_dense : (!shared || !shared_down_cm)) return hipErrorInvalidValue;
     const BatchSliceArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(down_cm), down_stride, static_cast<const uint8_t *>(shared),
                            static_cast<const uint8_t *>(shared_down_cm), static_cast<const uint2 *>(pass_list), n_pass, weights, scalar,
-                           static_cast<const _Float16 *>(xh), static_cast<const _Float16 *>(xl), xexp, partial, hidden, ffn, top_k, ntok};
+                           static_cast<const _Float16 *>(xh), static_cast<const _Float16 *>(xl), xexp, partial, hidden, ffn, top_k, ntok, shared_gu, shared_dense};
     const dim3 grid_dim(ffn / 32u, ntok * top_k + (ntok + 1u) / 2u);      // every pair a pass of its own at most, then the shared expert's passes
-#define REDHIP_BSLICE(NKC)                                                                                                             \
+#define REDHIP_BSLICE_ONE(NKC, MIX)                                                                                                    \
     do {                                                                                                                               \
         static bool attr = false;                                                                                                       \
-        const size_t dyn = (size_t)kBatchRep * kMagBytes + (size_t)kBatchSignRep * kSignBytes + kMagBytes + kSignBytes + (size_t)2u * NKC * 64u * 4u + 256u + 16u; \
+        const size_t dyn = (size_t)kBatchRep * kMagBytes + (size_t)kBatchSignRep * kSignBytes + kMagBytes + kSignBytes + (size_t)2u * NKC * 64u * 4u + 256u + 16u + \
+                           (MIX ? kIq3TableBytes : 0u);                                                                                 \
         if (!attr) {                                                                                                                    \
-            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(batch_slice_kernel<NKC, kBatchRep>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn); \
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(batch_slice_kernel<NKC, kBatchRep, MIX>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn); \
             if (e != hipSuccess) return e;                                                                                              \
             attr = true;                                                                                                                \
         }                                                                                                                               \
-        REDHIP_LAUNCH((batch_slice_kernel<NKC, kBatchRep>), grid_dim, dim3(kWaves * 64), dyn, s, a);                                      \
+        REDHIP_LAUNCH((batch_slice_kernel<NKC, kBatchRep, MIX>), grid_dim, dim3(kWaves * 64), dyn, s, a);                                 \
     } while (0)
+#define REDHIP_BSLICE(NKC) do { if (mix) REDHIP_BSLICE_ONE(NKC, 1); else REDHIP_BSLICE_ONE(NKC, 0); } while (0)
     prof_set_stage(ST_FUSED_EXPERTS);
     switch (hidden / 512u) {
         case 1: REDHIP_BSLICE(1); break;
@@ -1950,6 +2040,7 @@ hipError_t launch_batch_slices(const void *experts, uint64_t stride, const void 
         default: return hipErrorInvalidValue;      // (hidden 4096 would spill registers: such layers take their batches on other kernels)
     }
 #undef REDHIP_BSLICE
+#undef REDHIP_BSLICE_ONE
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     prof_set_stage(ST_SLICE_SUM);
@@ -2169,9 +2260,9 @@ hipError_t launch_down_combine_raw(uint32_t down_type, uint32_t shared_down_type
 // d as fp16 [row][K/256]. 130 bytes per 256 weights instead of 110, every load naturally aligned. A weight is
 // sign * grid byte * (2 * nibble + 1) * d: the four grid bytes of an entry come as exact fp16 values from an LDS table (512 x 8 bytes),
 // the signs are placed as in the IQ2_XXS kernels, and the same 4x4x4 MFMA multiplies them with the fp16 halves of the activations.
-constexpr uint32_t kIq3TableBytes = 512u * 8u;
 
-__global__ void repack_iq3s_words_kernel(const uint8_t *raw0, uint64_t raw_stride, uint32_t nrows, uint32_t K, uint8_t *packed0, uint64_t packed_stride) {
+// col_major: the same words stored [K / 32][nrows] (and d [K / 256][nrows]): the column slices of a down matrix, one group of every output row side by side
+__global__ void repack_iq3s_words_kernel(const uint8_t *raw0, uint64_t raw_stride, uint32_t nrows, uint32_t K, uint8_t *packed0, uint64_t packed_stride, int col_major) {
     const uint32_t groups = K / 32u, blocks = K / 256u;
     const uint8_t *raw = raw0 + (uint64_t)blockIdx.y * raw_stride;
     uint8_t *pk = packed0 + (uint64_t)blockIdx.y * packed_stride;
@@ -2186,26 +2277,26 @@ __global__ void repack_iq3s_words_kernel(const uint8_t *raw0, uint64_t raw_strid
         const uint32_t ib = (uint32_t)bp[3u + 8u * sub + 2u * l] | ((qh << (7u - 2u * l)) & 256u);
         w[l] = ia | (ib << 9) | ((uint32_t)bp[74u + 4u * sub + l] << 18) | (nib << 26);
     }
-    reinterpret_cast<uint4 *>(pk)[gid] = make_uint4(w[0], w[1], w[2], w[3]);
-    if (sub == 0u) reinterpret_cast<uint16_t *>(pk + (uint64_t)nrows * groups * 16u)[(uint64_t)r * blocks + (g >> 3)] = (uint16_t)ld_u16(bp);
+    reinterpret_cast<uint4 *>(pk)[col_major ? (uint64_t)g * nrows + r : gid] = make_uint4(w[0], w[1], w[2], w[3]);
+    if (sub == 0u) reinterpret_cast<uint16_t *>(pk + (uint64_t)nrows * groups * 16u)[col_major ? (uint64_t)(g >> 3) * nrows + r : (uint64_t)r * blocks + (g >> 3)] = (uint16_t)ld_u16(bp);
 }
 
-hipError_t launch_repack_iq3s_words(const void *raw, uint64_t raw_stride, uint32_t count, uint32_t nrows, uint32_t K, void *packed, uint64_t packed_stride, hipStream_t s) {
+hipError_t launch_repack_iq3s_words(const void *raw, uint64_t raw_stride, uint32_t count, uint32_t nrows, uint32_t K, void *packed, uint64_t packed_stride, hipStream_t s, bool col_major) {
     if (!nrows || !K || K % 256u || !count || count > 65535u) return hipErrorInvalidValue;
     const uint64_t total = (uint64_t)nrows * (K / 32u);
     REDHIP_LAUNCH(repack_iq3s_words_kernel, dim3((uint32_t)((total + 255u) / 256u), count), dim3(256), 0, s, static_cast<const uint8_t *>(raw), raw_stride, nrows, K,
-                  static_cast<uint8_t *>(packed), packed_stride);
+                  static_cast<uint8_t *>(packed), packed_stride, col_major ? 1 : 0);
     return hipGetLastError();
 }
 
 // parity tap: f32 dequantisation from the words, arithmetic as decode32<T_IQ3_S>
-__global__ void dequant_iq3s_words_kernel(const uint8_t *pk, uint32_t nrows, uint32_t K, float *out) {
+__global__ void dequant_iq3s_words_kernel(const uint8_t *pk, uint32_t nrows, uint32_t K, float *out, int col_major) {
     const uint32_t groups = K / 32u, blocks = K / 256u;
     const uint64_t gid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (gid >= (uint64_t)nrows * groups) return;
     const uint32_t r = (uint32_t)(gid / groups), g = (uint32_t)(gid % groups);
-    const uint4 v = reinterpret_cast<const uint4 *>(pk)[gid];
-    const float d = half_bits_to_f32(reinterpret_cast<const uint16_t *>(pk + (uint64_t)nrows * groups * 16u)[(uint64_t)r * blocks + (g >> 3)]);
+    const uint4 v = reinterpret_cast<const uint4 *>(pk)[col_major ? (uint64_t)g * nrows + r : gid];
+    const float d = half_bits_to_f32(reinterpret_cast<const uint16_t *>(pk + (uint64_t)nrows * groups * 16u)[col_major ? (uint64_t)(g >> 3) * nrows + r : (uint64_t)r * blocks + (g >> 3)]);
     const float db = d * (float)(1u + 2u * ((v.x >> 26) & 15u));
     const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
     float *o = out + (uint64_t)r * K + 32u * g;
@@ -2218,47 +2309,11 @@ __global__ void dequant_iq3s_words_kernel(const uint8_t *pk, uint32_t nrows, uin
     }
 }
 
-hipError_t launch_dequant_iq3s_words(const void *packed, uint32_t nrows, uint32_t K, float *out, hipStream_t s) {
+hipError_t launch_dequant_iq3s_words(const void *packed, uint32_t nrows, uint32_t K, float *out, hipStream_t s, bool col_major) {
     if (!nrows || !K || K % 256u) return hipErrorInvalidValue;
     const uint64_t total = (uint64_t)nrows * (K / 32u);
-    REDHIP_LAUNCH(dequant_iq3s_words_kernel, dim3((uint32_t)((total + 255u) / 256u)), dim3(256), 0, s, static_cast<const uint8_t *>(packed), nrows, K, out);
+    REDHIP_LAUNCH(dequant_iq3s_words_kernel, dim3((uint32_t)((total + 255u) / 256u)), dim3(256), 0, s, static_cast<const uint8_t *>(packed), nrows, K, out, col_major ? 1 : 0);
     return hipGetLastError();
-}
-
-// LDS table: the four bytes of every grid entry as fp16; built by the first 512 lanes of a workgroup
-__device__ __forceinline__ void build_iq3s_quads(uint8_t *lds, uint32_t tid) {
-    if (tid < 512u) {
-        const uint32_t e = redhip_iq3s_grid[tid];
-        uint32_t w2[2];
-#pragma unroll
-        for (int i = 0; i < 2; ++i) {
-            const _Float16 lo = (_Float16)(float)((e >> (16 * i)) & 255u), hi = (_Float16)(float)((e >> (16 * i + 8)) & 255u);
-            w2[i] = (uint32_t)__builtin_bit_cast(uint16_t, lo) | ((uint32_t)__builtin_bit_cast(uint16_t, hi) << 16);
-        }
-        *reinterpret_cast<uint2 *>(lds + (size_t)tid * 8u) = make_uint2(w2[0], w2[1]);
-    }
-}
-
-// 32 weights (one uint4 of words) against an activation operand that carries one token (rows 0, 1 = hi, lo) or two (rows 2, 3 the
-// second): va = first token's product, vb = the second's; scale nibble applied, d is not.
-__device__ __forceinline__ void iq3s_group_dot(uint4 q, const half4_t *ax, const uint8_t *lds, float &va, float &vb) {
-    const uint32_t w4[4] = {q.x, q.y, q.z, q.w};
-    float4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
-#pragma unroll
-    for (uint32_t l = 0; l < 4u; ++l) {
-        const uint2 ma = *reinterpret_cast<const uint2 *>(lds + ((w4[l] & 511u) << 3)), mb = *reinterpret_cast<const uint2 *>(lds + (((w4[l] >> 9) & 511u) << 3));
-        const uint32_t s8s = ((w4[l] >> 18) & 255u) << 8;          // sign bit k of the eight at bit 8 + k, as place_signs takes them
-        WeightQuad b0, b1;
-        b0.u[0] = (__umul24(s8s, (1u << 7) | (1u << 22)) & 0x80008000u) | ma.x;
-        b0.u[1] = (__umul24(s8s, (1u << 5) | (1u << 20)) & 0x80008000u) | ma.y;
-        b1.u[0] = (__umul24(s8s, (1u << 3) | (1u << 18)) & 0x80008000u) | mb.x;
-        b1.u[1] = (__umul24(s8s, (1u << 1) | (1u << 16)) & 0x80008000u) | mb.y;
-        acc = __builtin_amdgcn_mfma_f32_4x4x4f16(ax[2u * l], b0.h, acc, 0, 0, 0);
-        acc = __builtin_amdgcn_mfma_f32_4x4x4f16(ax[2u * l + 1u], b1.h, acc, 0, 0, 0);
-    }
-    const float sc = (float)(2u * ((q.x >> 26) & 15u) + 1u);
-    va = (acc[0] + acc[1] * 4.8828125e-4f) * sc;
-    vb = (acc[2] + acc[3] * 4.8828125e-4f) * sc;
 }
 
 // Down + combine of one token on a mixed layout whose routed down matrices are word-packed IQ3_S: 8 output rows per workgroup, wave s <

@@ -272,8 +272,9 @@ hipError_t launch_batch_mixed(uint32_t gate_up_type, const int8_t *gate_up_grid,
                               float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s,
                               const BatchSelect *select = nullptr);
 // IQ3_S down matrices of mixed layouts as one word per eight weights (uint4 per 32, [row][K/32], then d as fp16 [row][K/256])
-hipError_t launch_repack_iq3s_words(const void *raw, uint64_t raw_stride, uint32_t count, uint32_t nrows, uint32_t K, void *packed, uint64_t packed_stride, hipStream_t s);
-hipError_t launch_dequant_iq3s_words(const void *packed, uint32_t nrows, uint32_t K, float *out, hipStream_t s);
+hipError_t launch_repack_iq3s_words(const void *raw, uint64_t raw_stride, uint32_t count, uint32_t nrows, uint32_t K, void *packed, uint64_t packed_stride, hipStream_t s,
+                                    bool col_major = false);      // col_major: words [K / 32][nrows], d [K / 256][nrows]
+hipError_t launch_dequant_iq3s_words(const void *packed, uint32_t nrows, uint32_t K, float *out, hipStream_t s, bool col_major = false);
 inline uint64_t iq3s_words_bytes(uint32_t nrows, uint32_t K) { return (uint64_t)nrows * ((uint64_t)(K / 32u) * 16u + (uint64_t)(K / 256u) * 2u); }
 // down + combine of one token (ntok > 1: one grid layer per token) on word-packed IQ3_S routed matrices and the shared expert's dense f32 copy
 // (IQ2_XS / IQ1_M down matrices: the streams of launch_repack_gateup and the caller's codebook)
@@ -296,6 +297,9 @@ hipError_t launch_expert_slices(const void *experts, uint64_t stride, const void
 // [ntok][top_k] and scalar [ntok] of the routing; partial [ntok][top_k + 1][ffn / 32][hidden]
 hipError_t launch_batch_slices(const void *experts, uint64_t stride, const void *down_cm, uint64_t down_stride, const void *shared, const void *shared_down_cm,
                                const void *pass_list, const uint32_t *n_pass, const float *weights, const float *scalar, const void *xh, const void *xl,
-                               const int *xexp, float *partial, float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, hipStream_t s);
+                               const int *xexp, float *partial, float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, hipStream_t s,
+                               const float *shared_gu = nullptr, const float *shared_dense = nullptr);
+// (with shared_gu / shared_dense: a mixed layout - gate / up packed IQ2_XXS in `experts`, down_cm column-sliced word-packed IQ3_S, the shared
+// expert as its gate | up products [ntok][2 ffn] and the dense f32 copy [hidden][ffn] of its down matrix; shared / shared_down_cm unused)
 
 }  // namespace redhip

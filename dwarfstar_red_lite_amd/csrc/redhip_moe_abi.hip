@@ -35,7 +35,8 @@ struct Layer {
     uint8_t *packed = nullptr;       // same slots in the packed IQ2_XXS layout of the fused kernel (fused path only)
     uint8_t *shared_packed = nullptr;
     uint8_t *down_cm = nullptr;      // all-IQ2_XXS layers: the packed down matrices once more, column-sliced (qs [ffn / 32][hidden], ds [ffn / 256][hidden]), for the
-    uint8_t *shared_down_cm = nullptr;      // one-token kernel whose workgroups each take 32 columns of a down matrix
+    uint8_t *shared_down_cm = nullptr;      // slice kernels whose workgroups each take 32 columns of a down matrix; mixed layouts with IQ3_S down matrices
+                                            // whose small batches run as slices: their word-packed down matrices column-sliced (no shared_down_cm)
     uint8_t *tiled = nullptr;        // third copy, tile-major, read by the prefill kernels (handles that take chunks only)
     uint8_t *shared_tiled = nullptr;
     // mixed layouts that take chunks: f32 copies of the small dense matrices (dequantised once at upload) for the fp32 tile
@@ -49,7 +50,7 @@ struct Moe {
     redhip_moe_config cfg;
     uint32_t gu_type, dn_type, sh_gu_type, sh_dn_type;
     uint64_t gate_bytes, down_bytes, expert_stride;          // routed expert
-    uint64_t down_cm_stride() const { return (down_bytes + 255u) & ~255ull; }
+    uint64_t down_cm_stride() const { return mixed ? words_down_stride() : (down_bytes + 255u) & ~255ull; }
     float *partial = nullptr;                                // [tokens <= 8][top_k + 1][ffn / 32][hidden]: partial output vectors of the expert slices
     uint2 *pass_list = nullptr;                              // small batches: the passes (two pairs of one expert) of the batched expert slices
     uint32_t *n_pass = nullptr;
@@ -118,9 +119,12 @@ struct Moe {
     void *act_h = nullptr, *act_l = nullptr; // fp16 [top_k + 1][ffn] each
     int *act_exp = nullptr;                  // [top_k + 1][ffn / 32]
 
-    // batches the packed MFMA kernels take: 2..16 tokens, at most 128 pairs
+    // mixed layouts whose batches of 2..8 tokens run as expert slices: gate/up packed IQ2_XXS, down IQ3_S (column-sliced words), the shared
+    // expert from its dense f32 copies, an f32 router (or the f32 copy of a quantised one) in the launch that leaves the shared gate | up products
+    bool mixed_slices = false;
+    // batches that run as expert slices per pass: 2..8 tokens, at most 128 pairs
     bool small_batch(uint32_t ntok) const {
-        return fused && ntok >= 2u && ntok <= 8u && ntok * cfg.top_k <= 128u && ntok * (cfg.top_k + 1u) <= 144u && cfg.hidden / 512u <= 4u;
+        return (fused || mixed_slices) && ntok >= 2u && ntok <= 8u && ntok * cfg.top_k <= 128u && ntok * (cfg.top_k + 1u) <= 144u && cfg.hidden / 512u <= 4u;
     }
     // the same batches on a mixed layout run on the single-token kernels, one grid layer per token (tokens rarely share an
     // expert at these sizes, so reading a shared expert twice costs less than the pair sort and the per-pair kernels)
@@ -227,6 +231,14 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
     // select_here && grouped: selection and pair sort both happen inside the batched gate/up kernel, from m->logits
     const BatchSelect bsel{m->logits, c.n_expert, m->ids, m->weights, m->scalar};
     const BatchSelect *in_batch = select_here && grouped ? &bsel : nullptr;
+    if (m->mixed_slices && m->small_batch(ntok)) {     // pairs sorted (with their pass list) by the launch before; the shared gate | up products are in m->act
+        if (!grouped || select_here || !m->shared_gu_ready) { moe_err("internal: a small batch reached the expert slices without its pass list"); return 0; }
+        const Layer &L = m->layers[layer];
+        HIP_OK(launch_batch_slices(L.packed, m->packed_stride, L.down_cm, m->down_cm_stride(), nullptr, nullptr, m->pass_list, m->n_pass, weights, m->scalar,
+                                   m->xh, m->xl, m->xexp, m->partial, out, c.hidden, c.ffn, c.top_k, ntok, s, m->act, L.dense_down), "batched expert slice launch");
+        prof_set_stage(ST_OTHER);
+        return 1;
+    }
     if (m->grouped_mixed(ntok, grouped ? 2u : Moe::kGroupedMin) && m->shared_gu_ready) {      // xh / xl / xexp / scalar and the shared gate | up products (m->act) come from the router launch
         const Layer &L = m->layers[layer];
         if (!grouped) {
@@ -409,6 +421,11 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
     m->mixed = !m->fused && slots_fit && c.top_k >= 2u && (gu == T_IQ2_XXS || gu_codebook) && (sgu == T_Q6_K || (sgu == T_IQ2_XXS && !gu_codebook)) && fused_iq2_supported(c.hidden, c.ffn) &&
                (size_t)(c.top_k + 1u) * 8u * (c.ffn / 256u) * 210u + (dn == T_IQ1_M ? 17u * 1024u : dn == T_IQ2_XS ? 5u * 1024u : 0u) <= 64u * 1024u &&
                (sgu != T_Q6_K || (size_t)64u * (c.hidden / 256u) * 210u + (size_t)(c.hidden + c.hidden / 32u + c.hidden / 16u) * 4u <= (gu == T_IQ1_M ? 120u : 144u) * 1024u);
+    {
+        const uint32_t nv = c.hidden / 256u;
+        m->mixed_slices = m->mixed && gu == T_IQ2_XXS && dn == T_IQ3_S && c.ffn <= 512u && c.hidden / 512u <= 4u && (nv == 2u || nv == 4u || nv == 8u || nv == 16u) &&
+                          c.max_tokens >= 2u;
+    }
     m->pk_gate_bytes = packed_matrix_bytes(gu, c.ffn, c.hidden);
     m->packed_stride = m->fused && m->rowmajor_down() ? m->expert_stride : align256(2u * m->pk_gate_bytes);
     m->gu_grid = caller_grid_device(gu);
@@ -448,6 +465,10 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
                 m->resident += align256(rb) + align256(gb) + align256(db);
             }
         }
+        if (ok && m->mixed_slices) {
+            ok = hipMalloc(reinterpret_cast<void **>(&L.down_cm), (size_t)c.n_expert * m->down_cm_stride()) == hipSuccess;
+            m->resident += (uint64_t)c.n_expert * m->down_cm_stride();
+        }
         if (ok && m->mixed && (dn == T_IQ3_S || dn == T_IQ2_XS || dn == T_IQ1_M) && c.ffn <= 1024u) {
             ok = hipMalloc(reinterpret_cast<void **>(&L.words_down), (size_t)c.n_expert * m->words_down_stride()) == hipSuccess;
             m->resident += (uint64_t)c.n_expert * m->words_down_stride();
@@ -463,7 +484,7 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
         }
     }
     const size_t T = c.max_tokens;
-    const size_t partial_bytes = m->fused ? align256((size_t)(c.max_tokens < 8u ? c.max_tokens : 8u) * (c.top_k + 1u) * (c.ffn / 32u) * c.hidden * 4u) : 0u;
+    const size_t partial_bytes = m->fused || m->mixed_slices ? align256((size_t)(c.max_tokens < 8u ? c.max_tokens : 8u) * (c.top_k + 1u) * (c.ffn / 32u) * c.hidden * 4u) : 0u;
     const size_t ws_bytes = partial_bytes + align256(8u * 128u) + align256(4u) + align256(4u) + align256(T * c.hidden * 4u) + align256(T * (c.n_expert + 1u) * 4u) + 2u * align256(T * c.top_k * 4u) + align256(T * 4u) +
                             align256(T * c.top_k * c.ffn * 4u) + align256(T * c.ffn * 4u) +
                             2u * align256(2u * T * c.hidden) + align256(4u * T) + 2u * align256(2u * T * (c.top_k + 1u) * c.ffn) +
@@ -679,6 +700,9 @@ static int stage_and_pack(Moe *m, uint32_t layer, uint32_t first, uint32_t count
             if (m->dn_type == T_IQ3_S) HIP_OK(launch_repack_iq3s_words(dst + 2u * m->gate_bytes, m->expert_stride, count, c.hidden, c.ffn, wd, m->words_down_stride(), nullptr), "expert down words");
             else HIP_OK(launch_repack_gateup(m->dn_type, dst + 2u * m->gate_bytes, m->expert_stride, count, c.hidden, c.ffn, wd, m->words_down_stride(), nullptr), "expert down streams");
         }
+        if (m->mixed_slices)
+            HIP_OK(launch_repack_iq3s_words(dst + 2u * m->gate_bytes, m->expert_stride, count, c.hidden, c.ffn, m->layers[layer].down_cm + (uint64_t)first * m->down_cm_stride(),
+                                            m->down_cm_stride(), nullptr, true), "expert down column slices");
         if (m->layers[layer].tiled_down)
             HIP_OK(launch_tile_iq3s(dst + 2u * m->gate_bytes, m->expert_stride, count, c.hidden, c.ffn,
                                     m->layers[layer].tiled_down + (uint64_t)first * m->tiled_down_stride(), m->tiled_down_stride(), nullptr), "expert down tiling");
@@ -918,8 +942,12 @@ int redhip_moe_dequant_resident(redhip_moe_t h, uint32_t layer, uint32_t expert,
     hipStream_t s = static_cast<hipStream_t>(stream);
     if (which == 3u) { HIP_OK(launch_dequant_rows(c.router_type, L.router, c.n_expert, c.hidden, out_dev, s), "router dequant"); return 1; }
     const bool sh = expert == c.n_expert;
-    if (which == 4u) {                                      // the column-sliced copy of a down matrix (all-IQ2_XXS layers)
-        if (!m->fused) { moe_err("only all-IQ2_XXS layers keep column-sliced down matrices"); return 0; }
+    if (which == 4u) {                                      // the column-sliced copy of a down matrix
+        if (m->mixed_slices && !sh) {
+            HIP_OK(launch_dequant_iq3s_words(L.down_cm + (uint64_t)expert * m->down_cm_stride(), c.hidden, c.ffn, out_dev, s, true), "column-sliced down dequant");
+            return 1;
+        }
+        if (!m->fused) { moe_err("this layout keeps no column-sliced copy of that down matrix"); return 0; }
         HIP_OK(launch_dequant_packed_iq2xxs(sh ? L.shared_down_cm : L.down_cm + (uint64_t)expert * m->down_cm_stride(), c.hidden, c.ffn, true, out_dev, s), "column-sliced down dequant");
         return 1;
     }

@@ -38,6 +38,11 @@ def test_ragged_small_batches_hot_experts(layout):
     lay = synth.make_layer(77, cfg)
     m = ResidentMoe(cfg, n_layer=1, max_tokens=8)
     m.load_layer(0, lay)
+    # the column-sliced copies of the routed down matrices that these batches read dequantise bit-exactly
+    for e in (0, 311, cfg["n_expert"] - 1):
+        want = orc.dequant_rows(cfg["down_type"], lay["down"][e].reshape(-1), cfg["ffn"])
+        got = m.dequant_resident(0, e, 4).cpu().numpy()
+        assert np.array_equal(got.view(np.uint32), want.view(np.uint32)), (layout, e)
     rng = np.random.default_rng(31)
     for ntok in (1, 2, 3, 8):                                                      # (one token: the caller's routing on the single-token kernels)
         x = synth.normed_x(rng, ntok, cfg["hidden"])
