@@ -1427,6 +1427,17 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_select_kernel(GateUpArgs a
 
 // ---- word-packed IQ3_S (see the section on IQ3_S down matrices below for the format): the decode shared by the kernels that read it
 constexpr uint32_t kIq3TableBytes = 512u * 8u;
+// Column-sliced copy of a word-packed matrix: group g of row r. Eight rows of one group side by side (128 bytes), then the next group of the
+// same eight rows: the workgroups that take one group of many rows (expert slices) read whole 128-byte lines, those that take every
+// group of eight rows (one-token down kernel) one contiguous block.
+__device__ __forceinline__ uint64_t iq3s_sliced_index(uint32_t g, uint32_t r, uint32_t groups, uint32_t nrows) {
+#ifdef IQ3_PLAIN_CM
+    return (uint64_t)g * nrows + r;
+#else
+    (void)nrows;
+    return ((uint64_t)(r >> 3) * groups + g) * 8u + (r & 7u);
+#endif
+}
 // LDS table: the four bytes of every grid entry as fp16; built by the first 512 lanes of a workgroup
 __device__ __forceinline__ void build_iq3s_quads(uint8_t *lds, uint32_t tid) {
     if (tid < 512u) {
@@ -1895,7 +1906,7 @@ __global__ __launch_bounds__(kWaves * 64, 8) void batch_slice_kernel(BatchSliceA
         wd[u] = reinterpret_cast<const uint16_t *>(mat + (uint64_t)F * HG * 8u)[(uint64_t)r * HB + (G >> 3)];
     }
     using DownGroup = typename std::conditional<MIX != 0, uint4, uint2>::type;      // one row's 32 weights of the slice
-    const DownGroup *down_qs = reinterpret_cast<const DownGroup *>(dn) + (uint64_t)g * H;
+    const DownGroup *down_qs = reinterpret_cast<const DownGroup *>(dn) + (MIX != 0 ? 0u : (uint64_t)g * H);
     const uint16_t *down_ds = reinterpret_cast<const uint16_t *>(dn + (uint64_t)FG * H * sizeof(DownGroup)) + (uint64_t)(g >> 3) * H;
     DownGroup dq[DU];
     uint32_t dd[DU];
@@ -1903,7 +1914,7 @@ __global__ __launch_bounds__(kWaves * 64, 8) void batch_slice_kernel(BatchSliceA
     for (int kk = 0; kk < DU; ++kk) {
         const uint32_t unit = wave + NW * kk;
         const uint32_t r = 64u * (unit < 8u * NKC ? unit : 0u) + lane;
-        dq[kk] = down_qs[r];
+        dq[kk] = down_qs[MIX != 0 ? iq3s_sliced_index(g, r, FG, H) : (uint64_t)r];
         dd[kk] = down_ds[r];
     }
     if constexpr (MIX != 0) build_iq3s_quads(iq3_tab, tid);
@@ -2261,7 +2272,7 @@ hipError_t launch_down_combine_raw(uint32_t down_type, uint32_t shared_down_type
 // sign * grid byte * (2 * nibble + 1) * d: the four grid bytes of an entry come as exact fp16 values from an LDS table (512 x 8 bytes),
 // the signs are placed as in the IQ2_XXS kernels, and the same 4x4x4 MFMA multiplies them with the fp16 halves of the activations.
 
-// col_major: the same words stored [K / 32][nrows] (and d [K / 256][nrows]): the column slices of a down matrix, one group of every output row side by side
+// col_major: the same words stored column-sliced (iq3s_sliced_index; d [K / 256][nrows])
 __global__ void repack_iq3s_words_kernel(const uint8_t *raw0, uint64_t raw_stride, uint32_t nrows, uint32_t K, uint8_t *packed0, uint64_t packed_stride, int col_major) {
     const uint32_t groups = K / 32u, blocks = K / 256u;
     const uint8_t *raw = raw0 + (uint64_t)blockIdx.y * raw_stride;
@@ -2277,7 +2288,7 @@ __global__ void repack_iq3s_words_kernel(const uint8_t *raw0, uint64_t raw_strid
         const uint32_t ib = (uint32_t)bp[3u + 8u * sub + 2u * l] | ((qh << (7u - 2u * l)) & 256u);
         w[l] = ia | (ib << 9) | ((uint32_t)bp[74u + 4u * sub + l] << 18) | (nib << 26);
     }
-    reinterpret_cast<uint4 *>(pk)[col_major ? (uint64_t)g * nrows + r : gid] = make_uint4(w[0], w[1], w[2], w[3]);
+    reinterpret_cast<uint4 *>(pk)[col_major ? iq3s_sliced_index(g, r, groups, nrows) : gid] = make_uint4(w[0], w[1], w[2], w[3]);
     if (sub == 0u) reinterpret_cast<uint16_t *>(pk + (uint64_t)nrows * groups * 16u)[col_major ? (uint64_t)(g >> 3) * nrows + r : (uint64_t)r * blocks + (g >> 3)] = (uint16_t)ld_u16(bp);
 }
 
@@ -2295,7 +2306,7 @@ __global__ void dequant_iq3s_words_kernel(const uint8_t *pk, uint32_t nrows, uin
     const uint64_t gid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (gid >= (uint64_t)nrows * groups) return;
     const uint32_t r = (uint32_t)(gid / groups), g = (uint32_t)(gid % groups);
-    const uint4 v = reinterpret_cast<const uint4 *>(pk)[col_major ? (uint64_t)g * nrows + r : gid];
+    const uint4 v = reinterpret_cast<const uint4 *>(pk)[col_major ? iq3s_sliced_index(g, r, groups, nrows) : gid];
     const float d = half_bits_to_f32(reinterpret_cast<const uint16_t *>(pk + (uint64_t)nrows * groups * 16u)[col_major ? (uint64_t)(g >> 3) * nrows + r : (uint64_t)r * blocks + (g >> 3)]);
     const float db = d * (float)(1u + 2u * ((v.x >> 26) & 15u));
     const uint32_t w4[4] = {v.x, v.y, v.z, v.w};
@@ -2334,8 +2345,11 @@ struct DownWordsArgs {
     uint32_t id_limit;         // ids are clamped to id_limit - 1 (RouteGuard)
 };
 
-template <int NW, int FMT>       // FMT: 0 word-packed IQ3_S, 1 stream-packed IQ2_XS, 2 stream-packed IQ1_M
+// FMT: 0 word-packed IQ3_S, 1 stream-packed IQ2_XS, 2 stream-packed IQ1_M; CM (IQ3_S): the words stored column-sliced
+// (iq3s_sliced_index, d [ffn / 256][hidden]), the copy that the expert slices of small batches read
+template <int NW, int FMT, int CM = 0>
 __global__ __launch_bounds__(NW * 64) void down_combine_words_kernel(DownWordsArgs a) {
+    static_assert(CM == 0 || FMT == 0, "column-sliced copies exist of IQ3_S words only");
     __shared__ __attribute__((aligned(16))) uint8_t lds[FMT == 0 ? kIq3TableBytes : FMT == 1 ? 512u * 16u : 2048u * 16u];
     __shared__ float part[17 * 8];
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
@@ -2370,12 +2384,12 @@ __global__ __launch_bounds__(NW * 64) void down_combine_words_kernel(DownWordsAr
                 const uint32_t r = row0 + 4u * q + j, G = 16u * c + blk;
                 if ((uint32_t)c < n_chunk && G < FG) {
                     if constexpr (FMT == 0) {
-                        dq[q][c] = reinterpret_cast<const uint4 *>(ex)[(uint64_t)r * FG + G];
+                        dq[q][c] = reinterpret_cast<const uint4 *>(ex)[CM != 0 ? iq3s_sliced_index(G, r, FG, a.hidden) : (uint64_t)r * FG + G];
                     } else {
                         const uint2 v = reinterpret_cast<const uint2 *>(ex)[(uint64_t)r * FG + G];
                         dq[q][c] = make_uint4(v.x, v.y, FMT == 1 ? (uint32_t)scs[(uint64_t)r * FG + G] : 0u, 0u);
                     }
-                    dd[q][c] = ds[(uint64_t)r * FB + (G >> 3)];
+                    dd[q][c] = ds[CM != 0 ? (uint64_t)(G >> 3) * a.hidden + r : (uint64_t)r * FB + (G >> 3)];
                 }
             }
 #pragma unroll
@@ -2421,22 +2435,22 @@ __global__ __launch_bounds__(NW * 64) void down_combine_words_kernel(DownWordsAr
 
 hipError_t launch_down_combine_words(uint32_t down_type, const int8_t *grid, const void *experts, uint64_t stride, const float *shared_dense, const uint32_t *ids,
                                      const float *weights, const float *scalar, const void *act_h, const void *act_l, const int *act_exp, float *out,
-                                     uint32_t hidden, uint32_t ffn, uint32_t top_k, hipStream_t s, uint32_t ntok) {
+                                     uint32_t hidden, uint32_t ffn, uint32_t top_k, hipStream_t s, uint32_t ntok, bool col_major) {
     if (!hidden || hidden % 8u || !ffn || ffn % 256u || ffn > 1024u || top_k + 1u > (uint32_t)kWaves || !ntok || ntok > 65535u || !shared_dense) return hipErrorInvalidValue;
-    if ((down_type == T_IQ2_XS || down_type == T_IQ1_M) && !grid) return hipErrorInvalidValue;
+    if ((down_type == T_IQ2_XS || down_type == T_IQ1_M) && (!grid || col_major)) return hipErrorInvalidValue;
     const DownWordsArgs a{static_cast<const uint8_t *>(experts), stride, grid, shared_dense, ids, weights, scalar, static_cast<const _Float16 *>(act_h),
                           static_cast<const _Float16 *>(act_l), act_exp, out, hidden, ffn, top_k, block_context().resid_a, block_context().resid_b, route_guard().id_limit};
     const dim3 grid_dim(hidden / 8u, ntok);
     const bool narrow = top_k + 1u <= 12u;
-#define REDHIP_DCW(FMT)                                                                                              \
+#define REDHIP_DCW(FMT, CM)                                                                                          \
     do {                                                                                                             \
-        if (narrow) REDHIP_LAUNCH((down_combine_words_kernel<12, FMT>), grid_dim, dim3(12 * 64), 0, s, a);           \
-        else REDHIP_LAUNCH((down_combine_words_kernel<kWaves, FMT>), grid_dim, dim3(kWaves * 64), 0, s, a);          \
+        if (narrow) REDHIP_LAUNCH((down_combine_words_kernel<12, FMT, CM>), grid_dim, dim3(12 * 64), 0, s, a);       \
+        else REDHIP_LAUNCH((down_combine_words_kernel<kWaves, FMT, CM>), grid_dim, dim3(kWaves * 64), 0, s, a);      \
     } while (0)
     switch (down_type) {
-        case T_IQ3_S: REDHIP_DCW(0); break;
-        case T_IQ2_XS: REDHIP_DCW(1); break;
-        case T_IQ1_M: REDHIP_DCW(2); break;
+        case T_IQ3_S: if (col_major) REDHIP_DCW(0, 1); else REDHIP_DCW(0, 0); break;
+        case T_IQ2_XS: REDHIP_DCW(1, 0); break;
+        case T_IQ1_M: REDHIP_DCW(2, 0); break;
         default: return hipErrorInvalidValue;
     }
 #undef REDHIP_DCW

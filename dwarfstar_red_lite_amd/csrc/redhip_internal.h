@@ -280,7 +280,8 @@ inline uint64_t iq3s_words_bytes(uint32_t nrows, uint32_t K) { return (uint64_t)
 // (IQ2_XS / IQ1_M down matrices: the streams of launch_repack_gateup and the caller's codebook)
 hipError_t launch_down_combine_words(uint32_t down_type, const int8_t *grid, const void *experts, uint64_t stride, const float *shared_dense, const uint32_t *ids,
                                      const float *weights, const float *scalar, const void *act_h, const void *act_l, const int *act_exp, float *out,
-                                     uint32_t hidden, uint32_t ffn, uint32_t top_k, hipStream_t s, uint32_t ntok = 1u);
+                                     uint32_t hidden, uint32_t ffn, uint32_t top_k, hipStream_t s, uint32_t ntok = 1u,
+                                     bool col_major = false);      // col_major (IQ3_S): the column-sliced copy of launch_repack_iq3s_words
 // down + weighted combine for layouts whose down matrices are raw GGUF rows of any supported type
 hipError_t launch_down_combine_raw(uint32_t down_type, uint32_t shared_down_type, const void *experts, uint64_t stride, const void *shared,
                                    const uint32_t *ids, const float *weights, const float *scalar, const void *act_h, const void *act_l,

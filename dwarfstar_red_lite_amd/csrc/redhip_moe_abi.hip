@@ -43,7 +43,7 @@ struct Layer {
     // kernel: router [n_expert][hidden] (when it is quantised), shared gate | up [2 ffn][hidden], shared down [hidden][ffn]
     float *dense_router = nullptr, *dense_gu = nullptr, *dense_down = nullptr;
     uint8_t *tiled_down = nullptr;   // mixed layouts with IQ3_S down matrices that take chunks: their tile-major copy
-    uint8_t *words_down = nullptr;   // mixed layouts with IQ3_S down matrices: one word per eight weights, for the MFMA down kernels of up to 8 tokens
+    uint8_t *words_down = nullptr;   // mixed layouts with IQ3_S / IQ2_XS / IQ1_M down matrices, row-major words or streams for the MFMA down kernels of up to 8 tokens (layers with a column-sliced IQ3_S copy read that one instead)
 };
 
 struct Moe {
@@ -340,9 +340,10 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
                                     m->weights, m->scalar, m->xh, m->xl, m->xexp, m->act_h, m->act_l, m->act_exp, c.hidden, c.ffn, c.n_expert,
                                     c.top_k, s, ntok, m->gu_type, m->gu_grid), "gate/up launch");      // ntok > 1: a small batch on a mixed layout, one grid layer per token
         prof_set_stage(ST_DOWN_COMBINE);
-        if (L.words_down && L.dense_down)
-            HIP_OK(launch_down_combine_words(m->dn_type, m->dn_grid, L.words_down, m->words_down_stride(), L.dense_down, select_here ? m->ids : ids, select_here ? m->weights : weights,
-                                             m->scalar, m->act_h, m->act_l, m->act_exp, out, c.hidden, c.ffn, c.top_k, s, ntok), "down/combine launch");
+        if ((L.words_down || m->mixed_slices) && L.dense_down)      // (layers whose small batches run as slices keep their IQ3_S words column-sliced only)
+            HIP_OK(launch_down_combine_words(m->dn_type, m->dn_grid, m->mixed_slices ? L.down_cm : L.words_down, m->words_down_stride(), L.dense_down,
+                                             select_here ? m->ids : ids, select_here ? m->weights : weights,
+                                             m->scalar, m->act_h, m->act_l, m->act_exp, out, c.hidden, c.ffn, c.top_k, s, ntok, m->mixed_slices), "down/combine launch");
         else
             HIP_OK(launch_down_combine_raw(m->dn_type, m->sh_dn_type, L.experts + 2u * m->gate_bytes, m->expert_stride, L.shared + 2u * m->sh_gate_bytes,
                                            select_here ? m->ids : ids, select_here ? m->weights : weights, m->scalar, m->act_h, m->act_l,
@@ -423,8 +424,7 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
                (sgu != T_Q6_K || (size_t)64u * (c.hidden / 256u) * 210u + (size_t)(c.hidden + c.hidden / 32u + c.hidden / 16u) * 4u <= (gu == T_IQ1_M ? 120u : 144u) * 1024u);
     {
         const uint32_t nv = c.hidden / 256u;
-        m->mixed_slices = m->mixed && gu == T_IQ2_XXS && dn == T_IQ3_S && c.ffn <= 512u && c.hidden / 512u <= 4u && (nv == 2u || nv == 4u || nv == 8u || nv == 16u) &&
-                          c.max_tokens >= 2u;
+        m->mixed_slices = m->mixed && gu == T_IQ2_XXS && dn == T_IQ3_S && c.ffn <= 512u && c.hidden / 512u <= 4u && (nv == 2u || nv == 4u || nv == 8u || nv == 16u);
     }
     m->pk_gate_bytes = packed_matrix_bytes(gu, c.ffn, c.hidden);
     m->packed_stride = m->fused && m->rowmajor_down() ? m->expert_stride : align256(2u * m->pk_gate_bytes);
@@ -469,7 +469,7 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
             ok = hipMalloc(reinterpret_cast<void **>(&L.down_cm), (size_t)c.n_expert * m->down_cm_stride()) == hipSuccess;
             m->resident += (uint64_t)c.n_expert * m->down_cm_stride();
         }
-        if (ok && m->mixed && (dn == T_IQ3_S || dn == T_IQ2_XS || dn == T_IQ1_M) && c.ffn <= 1024u) {
+        if (ok && m->mixed && !m->mixed_slices && (dn == T_IQ3_S || dn == T_IQ2_XS || dn == T_IQ1_M) && c.ffn <= 1024u) {
             ok = hipMalloc(reinterpret_cast<void **>(&L.words_down), (size_t)c.n_expert * m->words_down_stride()) == hipSuccess;
             m->resident += (uint64_t)c.n_expert * m->words_down_stride();
         }
@@ -957,6 +957,10 @@ int redhip_moe_dequant_resident(redhip_moe_t h, uint32_t layer, uint32_t expert,
         if (which < 2u) HIP_OK(launch_dequant_packed(m->gu_type, pk + which * gbytes, c.ffn, c.hidden, m->gu_grid, out_dev, s), "packed gate/up dequant");
         else if (sh || m->rowmajor_down()) HIP_OK(launch_dequant_packed_iq2xxs(pk + 2u * gbytes, c.hidden, c.ffn, false, out_dev, s), "packed down dequant");
         else HIP_OK(launch_dequant_packed_iq2xxs(L.down_cm + (uint64_t)expert * m->down_cm_stride(), c.hidden, c.ffn, true, out_dev, s), "column-sliced down dequant");
+        return 1;
+    }
+    if (which == 2u && !sh && m->mixed_slices) {
+        HIP_OK(launch_dequant_iq3s_words(L.down_cm + (uint64_t)expert * m->down_cm_stride(), c.hidden, c.ffn, out_dev, s, true), "column-sliced down dequant");
         return 1;
     }
     if (which == 2u && !sh && L.words_down) {       // the copy the MFMA down kernels read
