@@ -45,6 +45,7 @@ def parse():
     ap.add_argument("--no-micro", action="store_true", help="skip the single-GEMV microbench (only run for --layout iq2 --batch 1)")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--calibrate", action="store_true", help="also run the plain copy kernel of known size (for rocprofv3 --pmc runs)")
+    ap.add_argument("--f2-layers", type=int, default=48, help="layers of the F2 handle that the default run's sweep adds (0: leave the F2 sweep out)")
     ap.add_argument("--no-sweep", action="store_true", help="skip the B=2/4/8 hot-routing sweep that the default (B=1, own router) run appends")
     ap.add_argument("--prime", type=int, default=2000, help="untimed steps before the warm-up that bring the clocks up (reported as clock_priming_steps)")
     return ap.parse_args()
@@ -205,10 +206,8 @@ def main():
 
     lib = load()
     torch.cuda.init()
-    cfg = synth.layer_config(layout=args.layout)
     B, NL = args.batch, args.layers
     K, W = args.steps, args.warmup
-    H, F = cfg["hidden"], cfg["ffn"]
     if args.layout in ("xs", "m"):          # these two decode through codebooks the caller supplies: the reference's, from the fixture
         from dwarfstar_red_lite_amd import moe as moe_api
         g = json.load(open(os.path.join(ROOT, "tests", "golden", "iq_grids.json")))
@@ -217,22 +216,28 @@ def main():
         orc.set_codebooks(*grids)
     # the default run (one token, the layer's own router) appends the small-batch sweep on the same resident handle
     sweep = [] if (args.no_sweep or B != 1 or args.routing != "router") else [2, 4, 8]
-    moe = ResidentMoe(cfg, n_layer=NL, max_tokens=max([B] + sweep))
     gen = torch.Generator(device="cuda")
     gen.manual_seed(20241125)
-    layer0 = None
-    for l in range(NL):
-        a = synth.make_layer_gpu(torch, gen, cfg)
-        moe.load_layer(l, a)
-        if l == 0:
-            layer0 = synth.layer_to_host(a, cfg)
-        del a
-    torch.cuda.synchronize()
-    ref = orc.Layer(cfg, **layer0)
     stream = torch.cuda.Stream()
     NX = 64
 
-    def run_workload(B, routing, micro_xs=None):
+    def resident_handle(layout, NL, max_tokens):
+        """a handle with NL layers of the layout resident (weights drawn on the GPU), layer 0 also on the host for the oracle"""
+        cfg = synth.layer_config(layout=layout)
+        moe = ResidentMoe(cfg, n_layer=NL, max_tokens=max_tokens)
+        layer0 = None
+        for l in range(NL):
+            a = synth.make_layer_gpu(torch, gen, cfg)
+            moe.load_layer(l, a)
+            if l == 0:
+                layer0 = synth.layer_to_host(a, cfg)
+            del a
+        torch.cuda.synchronize()
+        return {"layout": layout, "cfg": cfg, "moe": moe, "NL": NL, "layer0": layer0, "ref": orc.Layer(cfg, **layer0)}
+
+    def run_workload(ctx, B, routing):
+        cfg, moe, NL, layer0, ref = ctx["cfg"], ctx["moe"], ctx["NL"], ctx["layer0"], ctx["ref"]
+        H = cfg["hidden"]
         """parity gate on layer 0, then timing, per-kernel profile and the dominant kernel's roofline for batches of B tokens"""
         xs_host = synth.normed_x(np.random.default_rng(99 + B), NX * B, H).reshape(NX, B, H)
         xs = torch.from_numpy(xs_host).cuda()
@@ -303,11 +308,15 @@ def main():
                 distinct.append(len(set(ids.ravel().tolist())))
         mean_distinct = float(np.mean(distinct))
         lb = layer_bytes(cfg, mean_distinct, B)
-        roof = kernel_roofline(cfg, synth, stages, K, B, mean_distinct, lb, "%s_b%d" % (args.layout, B) + ("" if routing == "router" else "_" + routing))
+        roof = kernel_roofline(cfg, synth, stages, K, B, mean_distinct, lb, "%s_b%d" % (ctx["layout"], B) + ("" if routing == "router" else "_" + routing))
         return {"B": B, "routing": routing, "timing": tm, "stages": stages, "mean_distinct": mean_distinct, "lb": lb, "roofline": roof, "rel": rel,
                 "ids_ok": ids_ok, "xs": xs, "xs_host": xs_host}
 
-    head = run_workload(B, args.routing)
+    main_ctx = resident_handle(args.layout, NL, max([B] + sweep))
+    cfg, moe = main_ctx["cfg"], main_ctx["moe"]
+    H, F = cfg["hidden"], cfg["ffn"]
+    ref = main_ctx["ref"]
+    head = run_workload(main_ctx, B, args.routing)
     tm, stages, lb, mean_distinct = head["timing"], head["stages"], head["lb"], head["mean_distinct"]
     ms_per_step = tm["ms"]
     xs, xs_host = head["xs"], head["xs_host"]
@@ -368,19 +377,26 @@ def main():
             " / ".join("%dx%d" % sh for sh in shapes), K, len(ts))
 
     # ---- the ragged small-batch configuration on the same resident handle: B = 2, 4, 8, drawn logits with 32 hot experts ----
-    if sweep:
-        result["batch_sweep"] = []
-        for b in sweep:
-            r = run_workload(b, "hot")
-            t = r["timing"]
-            rf = r["roofline"] or {}
-            result["batch_sweep"].append({
-                "batch": b, "routing": "hot", "us_per_step": round(t["ms"] * 1e3, 3), "us_per_token": round(t["ms"] * 1e3 / b, 3), "launch_mode": t["mode"],
+    def sweep_entry(ctx, b, routing):
+        r = run_workload(ctx, b, routing)
+        t = r["timing"]
+        rf = r["roofline"] or {}
+        return {"batch": b, "routing": routing, "us_per_step": round(t["ms"] * 1e3, 3), "us_per_token": round(t["ms"] * 1e3 / b, 3), "launch_mode": t["mode"],
                 "eager_us_per_step": round(t["eager_ms"] * 1e3, 3), "mean_distinct_routed_experts": r["mean_distinct"],
                 "stages_us": {k: round(v["us_avg"] * v["launches"] / K, 3) for k, v in r["stages"].items()},
                 "dominant_kernel": rf.get("kernel"), "kernel_us": rf.get("launch_us"), "kernel_gbps": rf.get("achieved"), "kernel_frac_of_peak": rf.get("frac"),
-                "expert_bytes": int(r["lb"]["expert_bytes"]), "rel_l2_vs_cpu_oracle": r["rel"]})
-            del r
+                "expert_bytes": int(r["lb"]["expert_bytes"]), "rel_l2_vs_cpu_oracle": r["rel"]}
+
+    if sweep:
+        result["batch_sweep"] = [sweep_entry(main_ctx, b, "hot") for b in sweep]
+        # ---- the mixed-precision layout of the target files (config 2) on a handle of its own: one token with the layer's own router, then
+        # the same ragged batches; all 48 layers resident like the headline handle ----
+        if args.layout == "iq2" and args.f2_layers > 0:
+            f2 = resident_handle("f2", args.f2_layers, max(sweep))
+            result["f2_sweep"] = {"resident_layers": args.f2_layers, "resident_gb": round(f2["moe"].resident_bytes / 1e9, 2),
+                                  "runs": [sweep_entry(f2, 1, "router")] + [sweep_entry(f2, b, "hot") for b in sweep]}
+            f2["moe"].close()
+            del f2
 
     # ---- per-kernel microbench of config 1: one IQ2_XXS dequant-GEMV [512 x 2048] x [2048] on raw GGUF rows ----
     if args.layout == "iq2" and B == 1 and not args.no_micro:

@@ -126,6 +126,9 @@ struct Moe {
     bool small_batch(uint32_t ntok) const {
         return (fused || mixed_slices) && ntok >= 2u && ntok <= 8u && ntok * cfg.top_k <= 128u && ntok * (cfg.top_k + 1u) <= 144u && cfg.hidden / 512u <= 4u;
     }
+    // ... with the layer's own router: on a mixed layout two tokens are quicker on the single-token kernels (three launches, the selection
+    // inside the gate/up kernel) than as slices behind a selection + pair sort launch of their own (four): 30.7 against 32.7 us
+    bool slices_after_router(uint32_t ntok) const { return small_batch(ntok) && (fused || ntok >= kGroupedMin); }
     // the same batches on a mixed layout run on the single-token kernels, one grid layer per token (tokens rarely share an
     // expert at these sizes, so reading a shared expert twice costs less than the pair sort and the per-pair kernels)
     bool small_batch_mixed(uint32_t ntok) const {
@@ -231,8 +234,8 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
     // select_here && grouped: selection and pair sort both happen inside the batched gate/up kernel, from m->logits
     const BatchSelect bsel{m->logits, c.n_expert, m->ids, m->weights, m->scalar};
     const BatchSelect *in_batch = select_here && grouped ? &bsel : nullptr;
-    if (m->mixed_slices && m->small_batch(ntok)) {     // pairs sorted (with their pass list) by the launch before; the shared gate | up products are in m->act
-        if (!grouped || select_here || !m->shared_gu_ready) { moe_err("internal: a small batch reached the expert slices without its pass list"); return 0; }
+    if (m->mixed_slices && m->small_batch(ntok) && grouped) {     // pairs sorted (with their pass list) by the launch before; the shared gate | up products are in m->act
+        if (select_here || !m->shared_gu_ready) { moe_err("internal: a small batch reached the expert slices without its routing or the shared expert's products"); return 0; }
         const Layer &L = m->layers[layer];
         HIP_OK(launch_batch_slices(L.packed, m->packed_stride, L.down_cm, m->down_cm_stride(), nullptr, nullptr, m->pass_list, m->n_pass, weights, m->scalar,
                                    m->xh, m->xl, m->xexp, m->partial, out, c.hidden, c.ffn, c.top_k, ntok, s, m->act, L.dense_down), "batched expert slice launch");
@@ -815,13 +818,13 @@ int redhip_moe_forward(redhip_moe_t h, uint32_t layer, const float *x_dev, uint3
         }
         return ok;
     }
-    const bool group_in_select = m->small_batch(ntok) || m->grouped_mixed(ntok);
+    const bool group_in_select = m->slices_after_router(ntok) || m->grouped_mixed(ntok);
     const bool select_in_gateup = m->packed_gu() && (ntok == 1u || m->small_batch_mixed(ntok)) && !group_in_select;
     m->skip_select = select_in_gateup || group_in_select;      // small batches: the batched gate/up kernel selects and sorts the pairs itself
     const int routed = redhip_moe_route(h, layer, x_dev, ntok, nullptr, nullptr, nullptr, stream);
     m->skip_select = false;
     if (!routed) return 0;
-    if (m->small_batch(ntok)) return select_group_slices(m, layer, x_dev, ntok, out_dev, static_cast<hipStream_t>(stream));
+    if (m->slices_after_router(ntok)) return select_group_slices(m, layer, x_dev, ntok, out_dev, static_cast<hipStream_t>(stream));
     return experts_enqueue(m, layer, x_dev, ntok, m->ids, m->weights, out_dev, static_cast<hipStream_t>(stream), select_in_gateup || group_in_select, group_in_select);
 }
 
@@ -857,7 +860,7 @@ int redhip_moe_forward_block(redhip_moe_t h, uint32_t layer, const float *x_dev,
         if (hipGetLastError() != hipSuccess) { moe_err("residual + norm launch failed"); ok = 0; }
     }
     if (ok) {
-        const bool group_in_select = m->small_batch(ntok) || m->grouped_mixed(ntok);
+        const bool group_in_select = m->slices_after_router(ntok) || m->grouped_mixed(ntok);
         const bool select_in_gateup = m->packed_gu() && (ntok == 1u || m->small_batch_mixed(ntok)) && !group_in_select;
         m->skip_select = select_in_gateup || group_in_select;
         if (in_router) { bc.branch = branch_dev; bc.norm_w = post_norm_dev; bc.eps = eps; bc.xn_out = m->xn; }
@@ -868,7 +871,7 @@ int redhip_moe_forward_block(redhip_moe_t h, uint32_t layer, const float *x_dev,
             if (ok) {
             bc.resid_a = x_dev;                              // the path's last kernel adds x + branch to its output
             bc.resid_b = branch_dev;
-            ok = m->small_batch(ntok) ? select_group_slices(m, layer, m->xn, ntok, x_out_dev, s)
+            ok = m->slices_after_router(ntok) ? select_group_slices(m, layer, m->xn, ntok, x_out_dev, s)
                                       : experts_enqueue(m, layer, m->xn, ntok, m->ids, m->weights, x_out_dev, s, select_in_gateup || group_in_select, group_in_select);
         }
     }
