@@ -730,7 +730,7 @@ template <bool PREFIX>
 __global__ __launch_bounds__(1024) void group_pairs_kernel(const uint32_t *ids, const float *weights, uint32_t ntok, uint32_t top_k, uint32_t top_k_magic,
                                                            uint32_t n_expert, uint32_t *uid, uint32_t *expert_start,
                                                            uint32_t *pair_token, float *pair_weight, uint32_t *tok_pair,
-                                                           uint32_t *n_unique, uint32_t *status) {
+                                                           uint32_t *n_unique, uint32_t *status, uint32_t cache_ids) {
     extern __shared__ uint32_t sm[];
     const uint32_t words = (ntok + 31u) / 32u, P = ntok * top_k, tid = threadIdx.x;
     uint32_t *first = sm;                          // [n_expert]
@@ -741,14 +741,16 @@ __global__ __launch_bounds__(1024) void group_pairs_kernel(const uint32_t *ids, 
     uint32_t *wave_tot = uid_l + 1024u;            // [17]
     uint32_t *member = wave_tot + 17u;             // [n_expert][words]
     uint32_t *below = member + n_expert * words;   // [n_expert][words] when PREFIX: members in the words before this one
+    uint32_t *ids_l = cache_ids ? below + (PREFIX ? n_expert * words : 0u) : nullptr;      // [P] the clamped ids, when LDS has room: the later passes need no second trip to device memory
     auto token_of = [&](uint32_t p) { return top_k == 1u ? p : __umulhi(p, top_k_magic); };
     // the ids are the caller's: clamped into the tables (reported once, in the first pass)
-    auto id_of = [&](uint32_t p) { const uint32_t e = ids[p]; return e < n_expert ? e : n_expert - 1u; };
+    auto id_of = [&](uint32_t p) { if (ids_l) return ids_l[p]; const uint32_t e = ids[p]; return e < n_expert ? e : n_expert - 1u; };
     for (uint32_t i = tid; i < n_expert; i += 1024u) { first[i] = 0xffffffffu; count[i] = 0u; dense[i] = 0u; }
     for (uint32_t i = tid; i < n_expert * words; i += 1024u) member[i] = 0u;
     __syncthreads();
     for (uint32_t p = tid; p < P; p += 1024u) {
         const uint32_t e = guarded_id(ids[p], n_expert, status), t = token_of(p);
+        if (ids_l) ids_l[p] = e;
         atomicMin(&first[e], p);
         if constexpr (!PREFIX) atomicAdd(&count[e], 1u);
         if ((atomicOr(&member[e * words + (t >> 5)], 1u << (t & 31u)) & (1u << (t & 31u))) && status) atomicOr(status, 2u);      // the token names this expert twice
@@ -807,10 +809,16 @@ hipError_t launch_group_pairs(const uint32_t *ids, const float *weights, uint32_
         if (e != hipSuccess) return e;
         attr_set = true;
     }
-    if (lds_prefix <= 160u * 1024u)
-        REDHIP_LAUNCH(group_pairs_kernel<true>, dim3(1), dim3(1024), lds_prefix, s, ids, weights, ntok, top_k, magic, n_expert, uid, expert_start, pair_token, pair_weight, tok_pair, n_unique, route_guard().status);
-    else
-        REDHIP_LAUNCH(group_pairs_kernel<false>, dim3(1), dim3(1024), lds, s, ids, weights, ntok, top_k, magic, n_expert, uid, expert_start, pair_token, pair_weight, tok_pair, n_unique, route_guard().status);
+    const size_t ids_bytes = sizeof(uint32_t) * (size_t)ntok * top_k;
+    if (lds_prefix <= 160u * 1024u) {
+        const bool cache = lds_prefix + ids_bytes <= 160u * 1024u;
+        REDHIP_LAUNCH(group_pairs_kernel<true>, dim3(1), dim3(1024), lds_prefix + (cache ? ids_bytes : 0u), s, ids, weights, ntok, top_k, magic, n_expert, uid, expert_start, pair_token,
+                      pair_weight, tok_pair, n_unique, route_guard().status, cache ? 1u : 0u);
+    } else {
+        const bool cache = lds + ids_bytes <= 160u * 1024u;
+        REDHIP_LAUNCH(group_pairs_kernel<false>, dim3(1), dim3(1024), lds + (cache ? ids_bytes : 0u), s, ids, weights, ntok, top_k, magic, n_expert, uid, expert_start, pair_token,
+                      pair_weight, tok_pair, n_unique, route_guard().status, cache ? 1u : 0u);
+    }
     return hipGetLastError();
 }
 

@@ -912,85 +912,142 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_down_iq3s_kernel(Iq3Do
 // (r = l % 16, q = l / 16) reads four consecutive k of row r and of token r per 16 k and feeds them to four MFMAs (A[i = r][k = q],
 // B[k = q][j = r], D[i = 4q .. 4q + 3][j = r]; the order of k inside a slice does not matter as long as both operands agree). With
 // `gate_inp` set, row E is that vector (the shared expert's gate). A second kind of workgroup (blockIdx.x beyond the row tiles,
-// launched when xh is set) does the fp16 split of its tokens' activations. The same kernel multiplies any f32 matrix [E][H] with a
-// chunk of activations (dense shared expert).
+// launched when xh is set) does the fp16 split of its tokens' activations; it then also multiplies them with the gate vector, so the
+// row tiles cover the E matrix rows only (512 experts x 512 tokens: 16 x 16 tiles, one per compute unit, instead of a seventeenth row of
+// tiles for the one vector). The same kernel multiplies any f32 matrix [E][H] with a chunk of activations (dense shared expert).
 constexpr uint32_t kGemmTile = 32u, kGemmK = 64u, kGemmRow = kGemmK + 4u;      // LDS row of 68 floats: the eight lanes of a 16-byte read pass hit different banks
 
-__global__ __launch_bounds__(256) void router_f32_tile_kernel(const float *w, const float *gate_inp, const float *x, float *logits, uint32_t out_stride,
+// Eight waves: waves 0..3 take the even slices of 64 k, waves 4..7 the odd ones (each set one 16 x 16 block per wave, as described above);
+// the two partial blocks meet in LDS at the end. Two waves per SIMD, so one's MFMAs run while the other waits at the barrier or for LDS,
+// and half as many barriers as slices.
+__global__ __launch_bounds__(512) void router_f32_tile_kernel(const float *w, const float *gate_inp, const float *x, float *logits, uint32_t out_stride,
                                                               _Float16 *xh, _Float16 *xl, int *xexp, uint32_t H, uint32_t E, uint32_t ntok) {
-    __shared__ __attribute__((aligned(16))) float ws[2][kGemmTile][kGemmRow], xs[2][kGemmTile][kGemmRow];
+    __shared__ __attribute__((aligned(16))) float ws[2][2][kGemmTile][kGemmRow], xs[2][2][kGemmTile][kGemmRow];      // [buffer][k half]
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, r = lane & 15u, q = lane >> 4;
-    const uint32_t n_rows = E + (gate_inp ? 1u : 0u), row_tiles = (n_rows + kGemmTile - 1u) / kGemmTile;
-    if (blockIdx.x >= row_tiles) {                         // split job: one wave per token, 4 tokens per workgroup
-        const uint32_t tok = 4u * (blockIdx.y * (gridDim.x - row_tiles) + (blockIdx.x - row_tiles)) + wave;
+    const uint32_t n_rows = E + (gate_inp && !xh ? 1u : 0u), row_tiles = (n_rows + kGemmTile - 1u) / kGemmTile, tok_tiles = (ntok + kGemmTile - 1u) / kGemmTile;
+    const uint32_t n_tile = row_tiles * tok_tiles;
+    if (blockIdx.x >= n_tile) {                            // split job: one wave per token, 8 tokens per workgroup
+        const uint32_t tok = 8u * (blockIdx.x - n_tile) + wave;
         if (tok >= ntok) return;
-        const float *xt = x + (uint64_t)tok * H;
-        float amax = 0.0f;
-        for (uint32_t i = lane; i < H; i += 64u) amax = fmaxf(amax, fabsf(xt[i]));
+        // the vector as float4 per lane, eight requested at a time (2048 elements per pass: one round trip for the usual widths)
+        const float4 *xt = reinterpret_cast<const float4 *>(x + (uint64_t)tok * H), *gv = reinterpret_cast<const float4 *>(gate_inp);
+        const uint32_t H4 = H / 4u;
+        float amax = 0.0f, gate = 0.0f;
+        for (uint32_t base = 0; base < H4; base += 512u) {
+            float4 v[8], g[8];
 #pragma unroll
-        for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+            for (int k = 0; k < 8; ++k) {
+                const uint32_t i = base + 64u * k + lane;
+                v[k] = i < H4 ? xt[i] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+                g[k] = gate_inp && i < H4 ? gv[i] : make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            }
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                amax = fmaxf(fmaxf(amax, fmaxf(fabsf(v[k].x), fabsf(v[k].y))), fmaxf(fabsf(v[k].z), fabsf(v[k].w)));
+                gate = fmaf(g[k].w, v[k].w, fmaf(g[k].z, v[k].z, fmaf(g[k].y, v[k].y, fmaf(g[k].x, v[k].x, gate))));
+            }
+        }
+#pragma unroll
+        for (int o = 32; o > 0; o >>= 1) { amax = fmaxf(amax, __shfl_xor(amax, o, 64)); gate += __shfl_xor(gate, o, 64); }
         const int e = prescale_exp(amax);
         const float inv = exp2i(-e);
-        for (uint32_t i = lane; i < H; i += 64u) split_hi_lo(xt[i], inv, xh + (uint64_t)tok * H + i, xl + (uint64_t)tok * H + i);
-        if (lane == 0u) xexp[tok] = e;
+        for (uint32_t base = 0; base < H4; base += 512u) {
+            float4 v[8];
+#pragma unroll
+            for (int k = 0; k < 8; ++k) { const uint32_t i = base + 64u * k + lane; v[k] = xt[i < H4 ? i : 0u]; }
+#pragma unroll
+            for (int k = 0; k < 8; ++k) {
+                const uint32_t i = base + 64u * k + lane;
+                if (i >= H4) continue;
+                const float f[4] = {v[k].x, v[k].y, v[k].z, v[k].w};
+                half4_t h4, l4;
+#pragma unroll
+                for (int c = 0; c < 4; ++c) { _Float16 hh, ll; split_hi_lo(f[c], inv, &hh, &ll); h4[c] = hh; l4[c] = ll; }
+                *reinterpret_cast<half4_t *>(xh + (uint64_t)tok * H + 4u * i) = h4;
+                *reinterpret_cast<half4_t *>(xl + (uint64_t)tok * H + 4u * i) = l4;
+            }
+        }
+        if (lane == 0u) {
+            xexp[tok] = e;
+            if (gate_inp) logits[(uint64_t)tok * out_stride + E] = gate;
+        }
         return;
     }
-    // staging: thread t moves rows t / 16 and t / 16 + 16 of both operands, 16 bytes at column 4 (t % 16); rows beyond the last one
-    // repeat another and are not stored
-    const uint32_t srow = tid >> 4, scol = 4u * (tid & 15u);
-    const uint32_t row_a = kGemmTile * blockIdx.x + srow, row_b = row_a + 16u, tok_a = kGemmTile * blockIdx.y + srow, tok_b = tok_a + 16u;
-    const float *wsrc_a = (row_a < E ? w + (uint64_t)row_a * H : gate_inp ? gate_inp : w) + scol;
-    const float *wsrc_b = (row_b < E ? w + (uint64_t)row_b * H : gate_inp ? gate_inp : w) + scol;
-    const float *xsrc_a = x + (uint64_t)(tok_a < ntok ? tok_a : ntok - 1u) * H + scol;
-    const float *xsrc_b = x + (uint64_t)(tok_b < ntok ? tok_b : ntok - 1u) * H + scol;
-    const uint32_t wr = wave & 1u, wt = wave >> 1, n_slice = H / kGemmK;      // hidden is a multiple of 256: an even number of slices
-    // two register sets, one per LDS buffer: the loads of slice sl + 2 are issued while slice sl is multiplied, so an L2 round trip has two
-    // slices of arithmetic to hide behind (plain variables: arrays of them end up in scratch memory)
+    // staging: thread t of k half h = t / 256 moves rows (t % 256) / 16 and + 16 of both operands, 16 bytes at column 4 (t % 16) of its half's
+    // slice; rows beyond the last one repeat another and are not stored
+    // Workgroups are dealt to the eight XCDs in turn, each with its own L2: workgroup i lands on XCD i % 8. The tiles of one XCD form a
+    // compact block of the tile grid (a quarter of the row tiles x half of the token tiles), so that an XCD fetches a quarter of the
+    // matrix and half of the activations instead of all of both. (A different dealing order would only cost this locality.)
+    uint32_t tile_r = blockIdx.x % row_tiles, tile_t = blockIdx.x / row_tiles;
+    if (row_tiles % 4u == 0u && tok_tiles % 2u == 0u) {
+        const uint32_t xcd = blockIdx.x & 7u, slot = blockIdx.x >> 3, br = row_tiles / 4u, bt = tok_tiles / 2u;
+        tile_r = (xcd & 3u) * br + slot % br;
+        tile_t = (xcd >> 2) * bt + slot / br;
+    }
+    const uint32_t kh = tid >> 8, srow = (tid & 255u) >> 4, scol = 4u * (tid & 15u);
+    const uint32_t row_a = kGemmTile * tile_r + srow, row_b = row_a + 16u, tok_a = kGemmTile * tile_t + srow, tok_b = tok_a + 16u;
+    const float *wsrc_a = (row_a < E ? w + (uint64_t)row_a * H : gate_inp ? gate_inp : w) + scol + kh * kGemmK;
+    const float *wsrc_b = (row_b < E ? w + (uint64_t)row_b * H : gate_inp ? gate_inp : w) + scol + kh * kGemmK;
+    const float *xsrc_a = x + (uint64_t)(tok_a < ntok ? tok_a : ntok - 1u) * H + scol + kh * kGemmK;
+    const float *xsrc_b = x + (uint64_t)(tok_b < ntok ? tok_b : ntok - 1u) * H + scol + kh * kGemmK;
+    const uint32_t wr = wave & 1u, wt = (wave >> 1) & 1u, n_round = H / (2u * kGemmK);      // hidden is a multiple of 256: an even number of rounds
+    constexpr uint32_t kStep = 2u * kGemmK;                // k per round
+    // two register sets, one per LDS buffer: the loads of round rd + 2 are issued while round rd is multiplied, so a round trip has two
+    // rounds of arithmetic to hide behind (plain variables: arrays of them end up in scratch memory)
     float4 w0a = *reinterpret_cast<const float4 *>(wsrc_a), w0b = *reinterpret_cast<const float4 *>(wsrc_b);
     float4 x0a = *reinterpret_cast<const float4 *>(xsrc_a), x0b = *reinterpret_cast<const float4 *>(xsrc_b);
-    float4 w1a = *reinterpret_cast<const float4 *>(wsrc_a + kGemmK), w1b = *reinterpret_cast<const float4 *>(wsrc_b + kGemmK);
-    float4 x1a = *reinterpret_cast<const float4 *>(xsrc_a + kGemmK), x1b = *reinterpret_cast<const float4 *>(xsrc_b + kGemmK);
+    float4 w1a = *reinterpret_cast<const float4 *>(wsrc_a + kStep), w1b = *reinterpret_cast<const float4 *>(wsrc_b + kStep);
+    float4 x1a = *reinterpret_cast<const float4 *>(xsrc_a + kStep), x1b = *reinterpret_cast<const float4 *>(xsrc_b + kStep);
     float4_t acc0 = {0.0f, 0.0f, 0.0f, 0.0f}, acc1 = acc0;
+    const uint32_t mh = wave >> 2;                         // the k half this wave multiplies
     auto multiply = [&](uint32_t buf) {
 #pragma unroll
         for (uint32_t u = 0; u < kGemmK / 16u; ++u) {
-            const float4 av = *reinterpret_cast<const float4 *>(&ws[buf][16u * wr + r][16u * u + 4u * q]);
-            const float4 bv = *reinterpret_cast<const float4 *>(&xs[buf][16u * wt + r][16u * u + 4u * q]);
+            const float4 av = *reinterpret_cast<const float4 *>(&ws[buf][mh][16u * wr + r][16u * u + 4u * q]);
+            const float4 bv = *reinterpret_cast<const float4 *>(&xs[buf][mh][16u * wt + r][16u * u + 4u * q]);
             acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(av.x, bv.x, acc0, 0, 0, 0);
             acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(av.y, bv.y, acc1, 0, 0, 0);
             acc0 = __builtin_amdgcn_mfma_f32_16x16x4f32(av.z, bv.z, acc0, 0, 0, 0);
             acc1 = __builtin_amdgcn_mfma_f32_16x16x4f32(av.w, bv.w, acc1, 0, 0, 0);
         }
     };
-    for (uint32_t sl = 0; sl < n_slice; sl += 2u) {
-        *reinterpret_cast<float4 *>(&ws[0][srow][scol]) = w0a;
-        *reinterpret_cast<float4 *>(&ws[0][srow + 16u][scol]) = w0b;
-        *reinterpret_cast<float4 *>(&xs[0][srow][scol]) = x0a;
-        *reinterpret_cast<float4 *>(&xs[0][srow + 16u][scol]) = x0b;
-        __syncthreads();                                   // slice sl is in place; the readers of the other buffer (slice sl - 1) are past their barrier
-        const uint32_t k2 = (sl + 2u < n_slice ? sl + 2u : sl) * kGemmK;          // the last slices reload themselves: no branch around the loads
+    for (uint32_t rd = 0; rd < n_round; rd += 2u) {
+        *reinterpret_cast<float4 *>(&ws[0][kh][srow][scol]) = w0a;
+        *reinterpret_cast<float4 *>(&ws[0][kh][srow + 16u][scol]) = w0b;
+        *reinterpret_cast<float4 *>(&xs[0][kh][srow][scol]) = x0a;
+        *reinterpret_cast<float4 *>(&xs[0][kh][srow + 16u][scol]) = x0b;
+        __syncthreads();                                   // round rd is in place; the readers of the other buffer (round rd - 1) are past their barrier
+        const uint32_t k2 = (rd + 2u < n_round ? rd + 2u : rd) * kStep;          // the last rounds reload themselves: no branch around the loads
         w0a = *reinterpret_cast<const float4 *>(wsrc_a + k2);
         w0b = *reinterpret_cast<const float4 *>(wsrc_b + k2);
         x0a = *reinterpret_cast<const float4 *>(xsrc_a + k2);
         x0b = *reinterpret_cast<const float4 *>(xsrc_b + k2);
         multiply(0u);
-        *reinterpret_cast<float4 *>(&ws[1][srow][scol]) = w1a;
-        *reinterpret_cast<float4 *>(&ws[1][srow + 16u][scol]) = w1b;
-        *reinterpret_cast<float4 *>(&xs[1][srow][scol]) = x1a;
-        *reinterpret_cast<float4 *>(&xs[1][srow + 16u][scol]) = x1b;
+        *reinterpret_cast<float4 *>(&ws[1][kh][srow][scol]) = w1a;
+        *reinterpret_cast<float4 *>(&ws[1][kh][srow + 16u][scol]) = w1b;
+        *reinterpret_cast<float4 *>(&xs[1][kh][srow][scol]) = x1a;
+        *reinterpret_cast<float4 *>(&xs[1][kh][srow + 16u][scol]) = x1b;
         __syncthreads();
-        const uint32_t k3 = (sl + 3u < n_slice ? sl + 3u : sl + 1u) * kGemmK;
+        const uint32_t k3 = (rd + 3u < n_round ? rd + 3u : rd + 1u) * kStep;
         w1a = *reinterpret_cast<const float4 *>(wsrc_a + k3);
         w1b = *reinterpret_cast<const float4 *>(wsrc_b + k3);
         x1a = *reinterpret_cast<const float4 *>(xsrc_a + k3);
         x1b = *reinterpret_cast<const float4 *>(xsrc_b + k3);
         multiply(1u);
     }
-    const uint32_t out_tok = kGemmTile * blockIdx.y + 16u * wt + r;
+    // the odd slices' blocks go through LDS (buffer 0 was last read two barriers ago) to the waves that hold the even ones
+    float *meet = &ws[0][0][0][0];                         // [4 blocks][64 lanes] float4
+    __syncthreads();
+    if (mh == 1u) *reinterpret_cast<float4 *>(meet + ((wave & 3u) * 64u + lane) * 4u) = make_float4(acc0[0] + acc1[0], acc0[1] + acc1[1], acc0[2] + acc1[2], acc0[3] + acc1[3]);
+    __syncthreads();
+    if (mh == 1u) return;
+    const float4 other = *reinterpret_cast<const float4 *>(meet + (wave * 64u + lane) * 4u);
+    const float oth[4] = {other.x, other.y, other.z, other.w};
+    const uint32_t out_tok = kGemmTile * tile_t + 16u * wt + r;
 #pragma unroll
     for (uint32_t t = 0; t < 4u; ++t) {
-        const uint32_t out_row = kGemmTile * blockIdx.x + 16u * wr + 4u * q + t;
-        if (out_tok < ntok && out_row < n_rows) logits[(uint64_t)out_tok * out_stride + out_row] = acc0[t] + acc1[t];
+        const uint32_t out_row = kGemmTile * tile_r + 16u * wr + 4u * q + t;
+        if (out_tok < ntok && out_row < n_rows) logits[(uint64_t)out_tok * out_stride + out_row] = (acc0[t] + acc1[t]) + oth[t];
     }
 }
 
@@ -999,10 +1056,10 @@ __global__ __launch_bounds__(256) void router_f32_tile_kernel(const float *w, co
 hipError_t launch_f32_tiles(const float *w, const float *extra_row, const float *x, uint32_t ntok, uint32_t K, uint32_t n_rows, float *out,
                             uint32_t out_stride, void *xh, void *xl, int *xexp, hipStream_t s) {
     if (!ntok || !K || K % 256u || !n_rows || !w || !x || !out) return hipErrorInvalidValue;
-    const uint32_t row_tiles = (n_rows + (extra_row ? 1u : 0u) + kGemmTile - 1u) / kGemmTile, tok_tiles = (ntok + kGemmTile - 1u) / kGemmTile;
-    if (tok_tiles > 65535u) return hipErrorInvalidValue;
-    const uint32_t split_wgs = xh ? ((ntok + 3u) / 4u + tok_tiles - 1u) / tok_tiles : 0u;            // per blockIdx.y
-    REDHIP_LAUNCH(router_f32_tile_kernel, dim3(row_tiles + split_wgs, tok_tiles), dim3(256), 0, s, w, extra_row, x, out, out_stride,
+    const uint32_t row_tiles = (n_rows + (extra_row && !xh ? 1u : 0u) + kGemmTile - 1u) / kGemmTile, tok_tiles = (ntok + kGemmTile - 1u) / kGemmTile;      // (as in the kernel)
+    if ((uint64_t)row_tiles * tok_tiles + ntok > 0x7fffffffull) return hipErrorInvalidValue;
+    const uint32_t split_wgs = xh ? (ntok + 7u) / 8u : 0u;            // behind the tiles
+    REDHIP_LAUNCH(router_f32_tile_kernel, dim3(row_tiles * tok_tiles + split_wgs), dim3(512), 0, s, w, extra_row, x, out, out_stride,
                   static_cast<_Float16 *>(xh), static_cast<_Float16 *>(xl), xexp, K, n_rows, ntok);
     return hipGetLastError();
 }
