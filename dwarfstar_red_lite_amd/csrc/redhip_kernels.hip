@@ -745,15 +745,36 @@ __global__ __launch_bounds__(1024) void group_pairs_kernel(const uint32_t *ids, 
     auto token_of = [&](uint32_t p) { return top_k == 1u ? p : __umulhi(p, top_k_magic); };
     // the ids are the caller's: clamped into the tables (reported once, in the first pass)
     auto id_of = [&](uint32_t p) { if (ids_l) return ids_l[p]; const uint32_t e = ids[p]; return e < n_expert ? e : n_expert - 1u; };
+    // Up to eight pairs per thread (chunks of up to 8192 pairs) are requested here, ids and weights, before anything else: read inside the
+    // passes below, each would be a round trip of its own (the stores of the last pass keep the loads of the next pair behind them).
+    constexpr uint32_t kRegPairs = 8u;
+    const bool in_regs = P <= kRegPairs * 1024u;
+    uint32_t ereg[kRegPairs];
+    float wreg[kRegPairs];
+    if (in_regs) {
+#pragma unroll
+        for (uint32_t j = 0; j < kRegPairs; ++j) {
+            const uint32_t p = tid + 1024u * j;
+            ereg[j] = p < P ? ids[p] : 0u;
+            wreg[j] = p < P ? weights[p] : 0.0f;
+        }
+    }
     for (uint32_t i = tid; i < n_expert; i += 1024u) { first[i] = 0xffffffffu; count[i] = 0u; dense[i] = 0u; }
     for (uint32_t i = tid; i < n_expert * words; i += 1024u) member[i] = 0u;
     __syncthreads();
-    for (uint32_t p = tid; p < P; p += 1024u) {
-        const uint32_t e = guarded_id(ids[p], n_expert, status), t = token_of(p);
+    auto enter = [&](uint32_t p, uint32_t raw) {
+        const uint32_t e = guarded_id(raw, n_expert, status), t = token_of(p);
         if (ids_l) ids_l[p] = e;
         atomicMin(&first[e], p);
         if constexpr (!PREFIX) atomicAdd(&count[e], 1u);
         if ((atomicOr(&member[e * words + (t >> 5)], 1u << (t & 31u)) & (1u << (t & 31u))) && status) atomicOr(status, 2u);      // the token names this expert twice
+        return e;
+    };
+    if (in_regs) {
+#pragma unroll
+        for (uint32_t j = 0; j < kRegPairs; ++j) { const uint32_t p = tid + 1024u * j; if (p < P) ereg[j] = enter(p, ereg[j]); }
+    } else {
+        for (uint32_t p = tid; p < P; p += 1024u) enter(p, ids[p]);
     }
     __syncthreads();
     if constexpr (PREFIX) {
@@ -780,16 +801,22 @@ __global__ __launch_bounds__(1024) void group_pairs_kernel(const uint32_t *ids, 
     if (tid < U) { start[tid] = my_start; expert_start[tid] = my_start; }
     if (tid == 0u) { start[U] = all; expert_start[U] = all; n_unique[0] = U; }
     __syncthreads();
-    for (uint32_t p = tid; p < P; p += 1024u) {
-        const uint32_t e = id_of(p), t = token_of(p);
+    auto place = [&](uint32_t p, uint32_t e, float wt) {
+        const uint32_t t = token_of(p);
         const uint32_t *bits = member + e * words;
         uint32_t rank = __popc(bits[t >> 5] & ((1u << (t & 31u)) - 1u));
         if constexpr (PREFIX) rank += below[e * words + (t >> 5)];
         else for (uint32_t w = 0; w < (t >> 5); ++w) rank += __popc(bits[w]);
         const uint32_t pos = start[dense[e]] + rank;
         pair_token[pos] = t;
-        pair_weight[pos] = weights[p];
+        pair_weight[pos] = wt;
         tok_pair[p] = pos;
+    };
+    if (in_regs) {
+#pragma unroll
+        for (uint32_t j = 0; j < kRegPairs; ++j) { const uint32_t p = tid + 1024u * j; if (p < P) place(p, ereg[j], wreg[j]); }
+    } else {
+        for (uint32_t p = tid; p < P; p += 1024u) place(p, id_of(p), weights[p]);
     }
 }
 
