@@ -494,7 +494,7 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
                             align256(4u * T * (c.top_k + 1u) * (c.ffn / 32u)) +
                             (T > 8u && m->mixed ? align256(8u * T * c.ffn) : 0u) +
                             (T > 1u ? 6u * align256(4u * (T * c.top_k + 2u)) + align256(4u * T * c.top_k * c.hidden) + align256(4u * T * c.hidden) +
-                                          4u * align256(4u * (size_t)prefill_tile_bound(c.max_tokens, c.top_k, c.n_expert)) : 0u);
+                                          4u * align256(12u * (size_t)prefill_tile_bound(c.max_tokens, c.top_k, c.n_expert)) : 0u);      // (three tile lists)
     ok = ok && hipMalloc(reinterpret_cast<void **>(&m->ws), ws_bytes) == hipSuccess;
     if (!ok) {
         moe_err("failed to allocate resident MoE memory (%llu bytes so far)", (unsigned long long)m->resident);
@@ -538,7 +538,7 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
         m->pair_weight = reinterpret_cast<float *>(w); w += pw;
         m->tmp = reinterpret_cast<float *>(w); w += align256(4u * T * c.top_k * c.hidden);
         m->sh_tmp = reinterpret_cast<float *>(w); w += align256(4u * T * c.hidden);
-        const size_t tw = align256(4u * (size_t)prefill_tile_bound(c.max_tokens, c.top_k, c.n_expert));
+        const size_t tw = align256(12u * (size_t)prefill_tile_bound(c.max_tokens, c.top_k, c.n_expert));
         m->tile_group = reinterpret_cast<uint32_t *>(w); w += tw;
         m->tile_pair0 = reinterpret_cast<uint32_t *>(w); w += tw;
         m->tile_n = reinterpret_cast<uint32_t *>(w); w += tw;

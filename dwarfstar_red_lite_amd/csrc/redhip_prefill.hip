@@ -25,39 +25,59 @@ constexpr uint32_t kRowPad = 32u;               // fp16 elements of padding per 
 // ---------------------------------------------------------------- tile list
 
 // groups 0..U-1 are the distinct routed experts (pairs expert_start[u] .. expert_start[u + 1]), group U is the shared
-// expert with pairs P .. P + ntok. One workgroup: exclusive prefix sum of the tiles per group, then every group writes
-// its tiles: (group, first pair, number of pairs).
+// expert with pairs P .. P + ntok. One workgroup: exclusive prefix sums of the tiles per group, then every group writes
+// its tiles: (group, first pair, number of pairs). Three lists in the same arrays, list l from entry l * list_stride on, its length in
+// n_tiles[l]:
+//   0  tiles of kTile pairs (the down kernels; the gate/up kernel of hidden 512)
+//   1  "wide" tiles of 17 .. kWideTile pairs: a group's runs of 32 pairs, and its remainder when that is more than 16
+//   2  "narrow" tiles: the remainders of 1 .. 16 pairs
+// Lists 1 and 2 together cover every pair once: the gate/up kernels take the wide tiles on the kernel that multiplies two sets of 16
+// pairs with every decoded weight, the narrow ones on the kernel for 16.
+constexpr uint32_t kWideTile = 32u;
 __global__ __launch_bounds__(1024) void build_tiles_kernel(const uint32_t *expert_start, const uint32_t *n_unique, uint32_t P, uint32_t ntok,
-                                                           uint32_t *tile_group, uint32_t *tile_pair0, uint32_t *tile_n, uint32_t *n_tiles) {
-    __shared__ uint32_t wave_total[16];
+                                                           uint32_t *tile_group, uint32_t *tile_pair0, uint32_t *tile_n, uint32_t *n_tiles, uint32_t list_stride) {
+    __shared__ uint32_t wave_total[3][16];
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
     const uint32_t U = n_unique[0];
     uint32_t p0 = 0u, n = 0u;
     if (tid < U) { p0 = expert_start[tid]; n = expert_start[tid + 1u] - p0; }
-    const uint32_t mine = (n + kTile - 1u) / kTile;
-    uint32_t scan = mine;
+    auto counts = [](uint32_t m, uint32_t *c) {            // tiles of m pairs in the three lists
+        const uint32_t rem = m % kWideTile;
+        c[0] = (m + kTile - 1u) / kTile;
+        c[1] = m / kWideTile + (rem > kTile ? 1u : 0u);
+        c[2] = rem > 0u && rem <= kTile ? 1u : 0u;
+    };
+    uint32_t mine[3], scan[3];
+    counts(n, mine);
 #pragma unroll
-    for (int o = 1; o < 64; o <<= 1) {
-        const uint32_t up = __shfl_up(scan, o, 64);
-        if (lane >= (uint32_t)o) scan += up;
+    for (int l = 0; l < 3; ++l) {
+        scan[l] = mine[l];
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const uint32_t up = __shfl_up(scan[l], o, 64);
+            if (lane >= (uint32_t)o) scan[l] += up;
+        }
+        if (lane == 63u) wave_total[l][wave] = scan[l];
     }
-    if (lane == 63u) wave_total[wave] = scan;
     __syncthreads();
-    uint32_t base = 0u, routed_tiles = 0u;
-    for (uint32_t w = 0; w < 16u; ++w) { if (w < wave) base += wave_total[w]; routed_tiles += wave_total[w]; }
-    const uint32_t first = base + scan - mine;
-    for (uint32_t t = 0; t < mine; ++t) {
-        tile_group[first + t] = tid;
-        tile_pair0[first + t] = p0 + kTile * t;
-        tile_n[first + t] = n - kTile * t < kTile ? n - kTile * t : kTile;
+    uint32_t sh[3];
+    counts(ntok, sh);
+#pragma unroll
+    for (int l = 0; l < 3; ++l) {
+        uint32_t base = 0u, routed_tiles = 0u;
+        for (uint32_t w = 0; w < 16u; ++w) { if (w < wave) base += wave_total[l][w]; routed_tiles += wave_total[l][w]; }
+        const uint32_t off = (uint32_t)l * list_stride, first = off + base + scan[l] - mine[l];
+        // tile t of a run of m pairs that starts at pair q0, in list l
+        auto put = [&](uint32_t at, uint32_t group, uint32_t q0, uint32_t m, uint32_t t) {
+            const uint32_t size = l == 0 ? kTile : kWideTile, start = l == 2 ? m - m % kWideTile : size * t;
+            tile_group[at] = group;
+            tile_pair0[at] = q0 + start;
+            tile_n[at] = m - start < size ? m - start : size;
+        };
+        for (uint32_t t = 0; t < mine[l]; ++t) put(first + t, tid, p0, n, t);
+        for (uint32_t t = tid; t < sh[l]; t += 1024u) put(off + routed_tiles + t, U, P, ntok, t);
+        if (tid == 0u) n_tiles[l] = routed_tiles + sh[l];
     }
-    const uint32_t shared_tiles = (ntok + kTile - 1u) / kTile;
-    for (uint32_t t = tid; t < shared_tiles; t += 1024u) {
-        tile_group[routed_tiles + t] = U;
-        tile_pair0[routed_tiles + t] = P + kTile * t;
-        tile_n[routed_tiles + t] = ntok - kTile * t < kTile ? ntok - kTile * t : kTile;
-    }
-    if (tid == 0u) n_tiles[0] = routed_tiles + shared_tiles;
 }
 
 struct PrefillArgs {
@@ -505,29 +525,27 @@ __device__ __forceinline__ half8_t decode_reg(uint2 w, uint32_t sc, uint32_t q, 
 // gate/up + SwiGLU. Wave = (K quarter kc, column half rh): for the unit of 32 FFN columns j it computes the gate row and the
 // up row of column 32 j + 16 rh + r against its quarter of the hidden dimension; the quarters meet in LDS (double-buffered:
 // one barrier per unit).
+// Work items are parts of tiles (128 of the FFN columns, with an activation exponent of their own) so that the last round of
+// the persistent workgroups is short (with half tiles as items a chunk of 544 tiles gave four items to some workgroups and five
+// to others); a workgroup takes a contiguous range of items and keeps its A operands when consecutive ones share a tile.
+// Items item_begin .. item_end - 1 (item = tile * parts + part) of the tile list in ta.p; `tables` built by the caller (a barrier of this
+// function comes before their first use); lds: [16][128 + 4] f32 activations, then the partial sums [unit parity][K quarter][pair][gate
+// 0..31 | up 0..31, padded to 68] f32; tok_scale / tok_of: 16 entries each.
+constexpr size_t kNarrowLds = ((size_t)kTile * (32u * kItemUnits + 4u) + (size_t)2u * 4u * kTile * 68u) * sizeof(float);
 template <int NKC, int FMT>          // hidden = 512 * NKC; FMT 0: tile-major packed IQ2_XXS, 1 / 2: row-major IQ2_XS / IQ1_M streams
-__global__ __launch_bounds__(kRegWaves * 64) void prefill_gateup_reg_kernel(TiledArgs ta) {
+__device__ __forceinline__ void gateup_narrow_items(const TiledArgs &ta, uint32_t item_begin, uint32_t item_end, const uint8_t *tables, uint8_t *lds,
+                                                    float *tok_scale, uint32_t *tok_of) {
     const PrefillArgs &a = ta.p;
     constexpr uint32_t H = 512u * NKC, HG = H / 32u, HB = H / 256u, GQ = HG / 4u, NC = H / 128u;   // GQ: groups per K quarter = 4 NKC
-    extern __shared__ __attribute__((aligned(16))) uint8_t dyn[];          // acts: [16][128 + 4] f32
-    __shared__ __attribute__((aligned(16))) uint8_t tables[reg_table_bytes<FMT>()];      // static: table reads take immediate offsets
-    __shared__ float part[2][4][kTile][68];                // [unit parity][K quarter][pair][gate 0..31 | up 0..31], padded
-    __shared__ float tok_scale[kTile];
-    __shared__ uint32_t tok_of[kTile];
     const uint32_t tid = threadIdx.x, lane = tid & 63u, r = lane & 15u, q = lane >> 4;
     const uint32_t wave = __builtin_amdgcn_readfirstlane(tid >> 6), kc = wave & 3u, rh = wave >> 2;
     const uint32_t F = a.ffn, FG = F / 32u, P = a.ntok * a.top_k;
     constexpr uint32_t FGH = kItemUnits, AROW = 32u * kItemUnits + 4u;
-    float *acts = reinterpret_cast<float *>(dyn);
-    build_reg_tables<FMT>(tables, tid, kRegWaves * 64u, ta.grid);
-    const uint32_t T = a.n_tiles[0], U = a.n_unique[0];
+    float *acts = reinterpret_cast<float *>(lds);
+    float (*part)[4][kTile][68] = reinterpret_cast<float (*)[4][kTile][68]>(acts + kTile * AROW);
+    const uint32_t U = a.n_unique[0];
     const uint64_t qs_bytes = (uint64_t)F * HG * 8u, sc_off = qs_bytes + (uint64_t)F * HB * 2u, gate_bytes = sc_off + (FMT == 1 ? (uint64_t)F * HG : 0u);
-
-    // Work items are parts of tiles (128 of the FFN columns, with an activation exponent of their own) so that the last round of
-    // the persistent workgroups is short (with half tiles as items a chunk of 544 tiles gave four items to some workgroups and five
-    // to others); a workgroup takes a contiguous range of items and keeps its A operands when consecutive ones share a tile.
-    const uint32_t parts = FG / FGH, items = parts * T;
-    const uint32_t item_begin = (uint32_t)(((uint64_t)blockIdx.x * items) / gridDim.x), item_end = (uint32_t)(((uint64_t)(blockIdx.x + 1u) * items) / gridDim.x);
+    const uint32_t parts = FG / FGH;
     Half8 xa[GQ], xb[GQ];
     uint32_t have_tile = 0xffffffffu;
     for (uint32_t item = item_begin; item < item_end; ++item) {
@@ -649,6 +667,215 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_gateup_reg_kernel(Tile
             if (lane == 0u) a.act_exp[kExpPerPair * pr + ipart] = e;
         }
     }
+}
+
+// the kernel of hidden 512: all items of the list in ta.p
+template <int NKC, int FMT>
+__global__ __launch_bounds__(kRegWaves * 64) void prefill_gateup_reg_kernel(TiledArgs ta) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t dyn[];
+    __shared__ __attribute__((aligned(16))) uint8_t tables[reg_table_bytes<FMT>()];      // static: table reads take immediate offsets
+    __shared__ float tok_scale[kTile];
+    __shared__ uint32_t tok_of[kTile];
+    build_reg_tables<FMT>(tables, threadIdx.x, kRegWaves * 64u, ta.grid);
+    const uint32_t items = (ta.p.ffn / 32u / kItemUnits) * ta.p.n_tiles[0];
+    gateup_narrow_items<NKC, FMT>(ta, (uint32_t)(((uint64_t)blockIdx.x * items) / gridDim.x), (uint32_t)(((uint64_t)(blockIdx.x + 1u) * items) / gridDim.x), tables, dyn,
+                                  tok_scale, tok_of);
+}
+
+// The same gate/up + SwiGLU on the wide tiles (17 .. 32 pairs, list 1 of build_tiles_kernel): a wave owns an eighth of the hidden
+// dimension and keeps the activations of two sets of 16 pairs for it in registers (the same 128 registers as a quarter for one set); for
+// every unit of 32 FFN columns it decodes both row halves of its eighth and multiplies each decoded operand with both sets, so an expert
+// with many pairs in the chunk is decoded once per 32 of them. The eight partial sums per (pair, column) meet in LDS, single-buffered:
+// two barriers per unit. (On tiles of 16 or fewer pairs this layout was measured a quarter slower than the kernel above: they stay there.)
+// lds: [32][128 + 4] f32 activations, then the partial sums [8 K eighths][32 pairs][gate 0..31 | up 0..31, padded to 68] f32; tok_scale /
+// tok_of: 32 entries each; the rest as gateup_narrow_items.
+constexpr size_t kWideLds = ((size_t)kWideTile * (32u * kItemUnits + 4u) + (size_t)8u * kWideTile * 68u) * sizeof(float);
+template <int NKC, int FMT>          // hidden = 512 * NKC, NKC even
+__device__ __forceinline__ void gateup_wide_items(const TiledArgs &ta, uint32_t item_begin, uint32_t item_end, const uint8_t *tables, uint8_t *lds,
+                                                  float *tok_scale, uint32_t *tok_of) {
+    static_assert(NKC % 2 == 0 && kRegWaves == 8, "a wave takes NKC / 2 chunks of 128 columns");
+    const PrefillArgs &a = ta.p;
+    constexpr uint32_t H = 512u * NKC, HG = H / 32u, HB = H / 256u, GE = HG / 8u, NC = H / 128u, CW = NKC / 2u;   // GE: groups per K eighth = 2 NKC; CW: chunks per wave
+    constexpr uint32_t FGH = kItemUnits, AROW = 32u * kItemUnits + 4u;
+    const uint32_t tid = threadIdx.x, lane = tid & 63u, r = lane & 15u, q = lane >> 4;
+    const uint32_t kc = __builtin_amdgcn_readfirstlane(tid >> 6);
+    const uint32_t F = a.ffn, FG = F / 32u, P = a.ntok * a.top_k;
+    float *acts = reinterpret_cast<float *>(lds);
+    float (*part)[kWideTile][68] = reinterpret_cast<float (*)[kWideTile][68]>(acts + kWideTile * AROW);
+    const uint32_t U = a.n_unique[0];
+    const uint64_t qs_bytes = (uint64_t)F * HG * 8u, sc_off = qs_bytes + (uint64_t)F * HB * 2u, gate_bytes = sc_off + (FMT == 1 ? (uint64_t)F * HG : 0u);
+    const uint32_t parts = FG / FGH;
+    Half8 xa[2][GE], xb[2][GE];
+    uint32_t have_tile = 0xffffffffu;
+    for (uint32_t item = item_begin; item < item_end; ++item) {
+        const uint32_t tile = item / parts, ipart = item % parts, j0 = ipart * FGH;
+        const uint32_t u = a.tile_group[tile], p0 = a.tile_pair0[tile], n = a.tile_n[tile];
+        const uint8_t *ex = u == U ? ta.shared : ta.experts + (uint64_t)a.uid[u] * a.stride;
+        __syncthreads();                                   // the previous item's readers are done with acts / tok_of; tables are built
+        if (tile != have_tile) {
+            have_tile = tile;
+            if (tid < kWideTile) {
+                const uint32_t p = p0 + tid, tok = tid < n ? (p < P ? a.pair_token[p] : p - P) : 0u;
+                tok_of[tid] = tok;
+                tok_scale[tid] = tid < n ? (FMT == 2 ? 1.0f : 0.125f) * exp2i(a.xexp[tok]) : 0.0f;
+            }
+            __syncthreads();
+#pragma unroll
+            for (uint32_t s2 = 0; s2 < 2u; ++s2) {
+                const uint64_t base = (uint64_t)tok_of[16u * s2 + r] * H + 32u * (kc * GE) + 8u * q;
+                const bool live = 16u * s2 + r < n;
+#pragma unroll
+                for (uint32_t g = 0; g < GE; ++g) {
+                    xa[s2][g].u = make_uint4(0u, 0u, 0u, 0u);
+                    xb[s2][g].u = xa[s2][g].u;
+                    if (live) {
+                        xa[s2][g].u = *reinterpret_cast<const uint4 *>(a.xh + base + 32u * g);
+                        xb[s2][g].u = *reinterpret_cast<const uint4 *>(a.xl + base + 32u * g);
+                    }
+                }
+            }
+            // The low halves are stored times 2^11; here they go back to their own scale (exact: the largest |x| of a token sits in
+            // [2^13, 2^14), so a low half below the fp16 normal range belongs to an element 2^-16 of that), and a product's high and low
+            // parts add up in one accumulator.
+#pragma unroll
+            for (uint32_t s2 = 0; s2 < 2u; ++s2)
+#pragma unroll
+                for (uint32_t g = 0; g < GE; ++g) xb[s2][g].v = xb[s2][g].v * (_Float16)4.8828125e-4f;
+        }
+        // half step hs of the item: unit j0 + hs / 2, row half hs % 2; chunks c = 0 .. CW - 1 of the wave's eighth inside it
+        constexpr uint32_t kHalfSteps = FGH * 2u;
+        auto load_chunk = [&](const uint8_t *mat, uint32_t hs, uint32_t c) {
+            const uint32_t rtile = 2u * j0 + hs, chunk = kc * CW + c;      // (2 (j0 + hs / 2) + hs % 2)
+            if constexpr (FMT == 0) {
+                const uint4 *qp = reinterpret_cast<const uint4 *>(mat + (((uint64_t)rtile * NC + chunk) * 16u + r) * 32u);
+                const uint16_t *dp = reinterpret_cast<const uint16_t *>(mat + qs_bytes) + ((uint64_t)rtile * HB + chunk / 2u) * 16u + r;
+                return RowChunk{qp[0], qp[1], *dp, 0u};
+            } else {
+                const uint64_t row = 16u * rtile + r;
+                const uint4 *qp = reinterpret_cast<const uint4 *>(mat + (row * HG + 4u * chunk) * 8u);
+                const uint32_t d = reinterpret_cast<const uint16_t *>(mat + qs_bytes)[row * HB + chunk / 2u];
+                return RowChunk{qp[0], qp[1], d, FMT == 1 ? *reinterpret_cast<const uint32_t *>(mat + sc_off + row * HG + 4u * chunk) : 0u};
+            }
+        };
+        const uint8_t *gmat = ex, *umat = ex + gate_bytes;
+        RowChunk cg = load_chunk(gmat, 0u, 0u), cu = load_chunk(umat, 0u, 0u);
+#pragma unroll 1
+        for (uint32_t hs = 0; hs < kHalfSteps; ++hs) {
+            const uint32_t rh = hs & 1u, j = j0 + (hs >> 1);
+            float4_t totg[2], totu[2];
+#pragma unroll
+            for (int s2 = 0; s2 < 2; ++s2) { totg[s2] = float4_t{0.0f, 0.0f, 0.0f, 0.0f}; totu[s2] = totg[s2]; }
+#pragma unroll
+            for (uint32_t c = 0; c < CW; ++c) {
+                // the chunk after this one (same half step, or the first of the next; the last one reloads itself) is in flight
+                const uint32_t nh = c + 1u < CW ? hs : (hs + 1u < kHalfSteps ? hs + 1u : hs), nc = c + 1u < CW ? c + 1u : 0u;
+                const RowChunk ng = load_chunk(gmat, nh, nc), nu = load_chunk(umat, nh, nc);
+                __builtin_amdgcn_sched_barrier(0);         // keeps the loads ahead of the chunk's arithmetic
+                const uint2 wg4[4] = {make_uint2(cg.a.x, cg.a.y), make_uint2(cg.a.z, cg.a.w), make_uint2(cg.b.x, cg.b.y), make_uint2(cg.b.z, cg.b.w)};
+                const uint2 wu4[4] = {make_uint2(cu.a.x, cu.a.y), make_uint2(cu.a.z, cu.a.w), make_uint2(cu.b.x, cu.b.y), make_uint2(cu.b.z, cu.b.w)};
+                float4_t ga[2], ua[2];
+#pragma unroll
+                for (int s2 = 0; s2 < 2; ++s2) { ga[s2] = float4_t{0.0f, 0.0f, 0.0f, 0.0f}; ua[s2] = ga[s2]; }
+                RawEntry rg0 = fetch_reg<FMT>(wg4[0], q, tables), ru0 = fetch_reg<FMT>(wu4[0], q, tables);
+#pragma unroll
+                for (uint32_t k = 0; k < 4u; ++k) {
+                    const uint32_t g = 4u * c + k;
+                    __builtin_amdgcn_sched_barrier(0);
+                    const half8_t bg = finish_reg<FMT>(rg0, wg4[k], cg.sc >> (8u * k), q), bu = finish_reg<FMT>(ru0, wu4[k], cu.sc >> (8u * k), q);
+                    if (k + 1u < 4u) { rg0 = fetch_reg<FMT>(wg4[k + 1u], q, tables); ru0 = fetch_reg<FMT>(wu4[k + 1u], q, tables); }
+                    __builtin_amdgcn_sched_barrier(0);
+                    ga[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[0][g].v, bg, ga[0], 0, 0, 0);
+                    ua[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[0][g].v, bu, ua[0], 0, 0, 0);
+                    ga[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[1][g].v, bg, ga[1], 0, 0, 0);
+                    ua[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xa[1][g].v, bu, ua[1], 0, 0, 0);
+                    ga[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xb[0][g].v, bg, ga[0], 0, 0, 0);
+                    ua[0] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xb[0][g].v, bu, ua[0], 0, 0, 0);
+                    ga[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xb[1][g].v, bg, ga[1], 0, 0, 0);
+                    ua[1] = __builtin_amdgcn_mfma_f32_16x16x32_f16(xb[1][g].v, bu, ua[1], 0, 0, 0);
+                }
+                const float dg = scale_to_f32(cg.d), du = scale_to_f32(cu.d);
+#pragma unroll
+                for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+                    for (int t = 0; t < 4; ++t) {
+                        totg[s2][t] = fmaf(ga[s2][t], dg, totg[s2][t]);
+                        totu[s2][t] = fmaf(ua[s2][t], du, totu[s2][t]);
+                    }
+                cg = ng;
+                cu = nu;
+            }
+            // this row half of the unit is complete for the wave's eighth
+#pragma unroll
+            for (uint32_t s2 = 0; s2 < 2u; ++s2)
+#pragma unroll
+                for (uint32_t t = 0; t < 4u; ++t) {
+                    part[kc][16u * s2 + 4u * q + t][16u * rh + r] = totg[s2][t];
+                    part[kc][16u * s2 + 4u * q + t][32u + 16u * rh + r] = totu[s2][t];
+                }
+            if (rh == 0u) continue;
+            __syncthreads();
+            for (uint32_t i = tid >> 5; i < kWideTile; i += 16u) {      // (pair i, column cc) per thread: the eight eighths, the token's scale, SwiGLU
+                const uint32_t cc = tid & 31u;
+                float gs[8], us[8];
+#pragma unroll
+                for (int e8 = 0; e8 < 8; ++e8) { gs[e8] = part[e8][i][cc]; us[e8] = part[e8][i][32u + cc]; }
+                const float gsum = (((gs[0] + gs[1]) + (gs[2] + gs[3])) + ((gs[4] + gs[5]) + (gs[6] + gs[7]))) * tok_scale[i];
+                const float usum = (((us[0] + us[1]) + (us[2] + us[3])) + ((us[4] + us[5]) + (us[6] + us[7]))) * tok_scale[i];
+                acts[i * AROW + 32u * (j - j0) + cc] = (gsum / (1.0f + expf(-gsum))) * usum;
+            }
+            __syncthreads();                               // the partial sums may be overwritten
+        }
+        // one exponent per pair and part, then the fp16 halves: wave w takes pairs 4 w .. 4 w + 3
+        const uint32_t c0 = 32u * j0, c1 = c0 + 32u * FGH;
+#pragma unroll
+        for (uint32_t h = 0; h < 4u; ++h) {
+            const uint32_t i = 4u * kc + h;
+            if (i >= n) continue;                          // wave-uniform
+            if (ta.act_f32) {
+                for (uint32_t c = c0 + lane; c < c1; c += 64u) ta.act_f32[(uint64_t)(p0 + i) * F + c] = acts[i * AROW + c - c0];
+                continue;
+            }
+            float amax = 0.0f;
+            for (uint32_t c = c0 + lane; c < c1; c += 64u) amax = fmaxf(amax, fabsf(acts[i * AROW + c - c0]));
+#pragma unroll
+            for (int o = 32; o > 0; o >>= 1) amax = fmaxf(amax, __shfl_xor(amax, o, 64));
+            const int e = prescale_exp(amax);
+            const float inv = exp2i(-e);
+            const uint64_t pr = p0 + i;
+            for (uint32_t c = c0 + lane; c < c1; c += 64u) split_hi_lo(acts[i * AROW + c - c0], inv, a.act_h + pr * F + c, a.act_l + pr * F + c);
+            if (lane == 0u) a.act_exp[kExpPerPair * pr + ipart] = e;
+        }
+    }
+}
+
+// Gate/up of a chunk in one launch: the wide tiles (list 1, at ta.p's tile arrays + list_stride) and the narrow ones (list 2). The
+// persistent workgroups cut one line of work into equal pieces: first the wide items at 3 units each, then the narrow ones at 2 (a wide
+// item was measured at 1.4 narrow ones); a workgroup runs the items that start inside its piece, so every compute unit is busy whatever
+// the mix (as two launches the wide tiles of a chunk with few of them left half of the device idle: 171 against 157 us).
+template <int NKC, int FMT>
+__global__ __launch_bounds__(kRegWaves * 64) void prefill_gateup_mixed_kernel(TiledArgs ta, uint32_t list_stride) {
+    extern __shared__ __attribute__((aligned(16))) uint8_t dyn[];          // kWideLds
+    __shared__ __attribute__((aligned(16))) uint8_t tables[reg_table_bytes<FMT>()];      // static: table reads take immediate offsets
+    __shared__ float tok_scale[kWideTile];
+    __shared__ uint32_t tok_of[kWideTile];
+    build_reg_tables<FMT>(tables, threadIdx.x, kRegWaves * 64u, ta.grid);
+    const uint32_t parts = ta.p.ffn / 32u / kItemUnits, n_wide = parts * ta.p.n_tiles[1], n_narrow = parts * ta.p.n_tiles[2];
+    const uint64_t line = 3ull * n_wide + 2ull * n_narrow;
+    const uint64_t lo = (uint64_t)blockIdx.x * line / gridDim.x, hi = (uint64_t)(blockIdx.x + 1u) * line / gridDim.x;
+    // items whose start (3 i, or 3 n_wide + 2 j) lies in [lo, hi)
+    const auto first_at = [](uint64_t x, uint64_t base, uint64_t unit, uint32_t n) { const uint64_t i = x <= base ? 0u : (x - base + unit - 1u) / unit; return (uint32_t)(i < n ? i : n); };
+    const uint32_t w0 = first_at(lo, 0u, 3u, n_wide), w1 = first_at(hi, 0u, 3u, n_wide);
+    const uint32_t m0 = first_at(lo, 3ull * n_wide, 2u, n_narrow), m1 = first_at(hi, 3ull * n_wide, 2u, n_narrow);
+    TiledArgs tl = ta;
+    const auto use_list = [&](uint32_t l) {
+        tl.p.tile_group = ta.p.tile_group + l * list_stride;
+        tl.p.tile_pair0 = ta.p.tile_pair0 + l * list_stride;
+        tl.p.tile_n = ta.p.tile_n + l * list_stride;
+    };
+    use_list(1u);
+    gateup_wide_items<NKC, FMT>(tl, w0, w1, tables, dyn, tok_scale, tok_of);
+    use_list(2u);
+    gateup_narrow_items<NKC, FMT>(tl, m0, m1, tables, dyn, tok_scale, tok_of);
 }
 
 // down. Wave w computes rows 128 b + 16 w + r for b = 0, 1, ... against all ffn columns of the tile; no reduction across waves.
@@ -1082,16 +1309,40 @@ hipError_t launch_swiglu_rows(const float *gu, uint32_t gu_stride, uint32_t ntok
     return hipGetLastError();
 }
 
-static hipError_t launch_gateup_reg(const TiledArgs &ta, dim3 grid, hipStream_t s, uint32_t fmt = 0u) {
+// list_stride: distance of the tile lists in the tile arrays (build_tiles_kernel). hidden >= 1024: wide and narrow tiles in one launch;
+// hidden 512: list 0 on the kernel for 16 pairs.
+static hipError_t launch_gateup_reg(const TiledArgs &ta, dim3 grid, hipStream_t s, uint32_t list_stride, uint32_t fmt = 0u) {
     const uint32_t hidden = ta.p.hidden;
-    const size_t acts_lds = (size_t)kTile * (32u * kItemUnits + 4u) * sizeof(float);
     hipError_t e = hipSuccess;
     prof_set_stage(ST_PREFILL_GATEUP);
+    if (hidden / 512u == 2u || hidden / 512u == 4u) {
+#define REDHIP_PGW_ONE(NKC, FMT)                                                                                                          \
+    do {                                                                                                                                  \
+        static bool attr = false;                                                                                                          \
+        if (!attr) {                                                                                                                       \
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(prefill_gateup_mixed_kernel<NKC, FMT>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kWideLds); \
+            if (e != hipSuccess) return e;                                                                                                 \
+            attr = true;                                                                                                                   \
+        }                                                                                                                                  \
+        REDHIP_LAUNCH((prefill_gateup_mixed_kernel<NKC, FMT>), grid, dim3(kRegWaves * 64), kWideLds, s, ta, list_stride);                  \
+    } while (0)
+#define REDHIP_PGW(NKC)                                                                                                                   \
+    do {                                                                                                                                  \
+        if (fmt == 1u) REDHIP_PGW_ONE(NKC, 1);                                                                                             \
+        else if (fmt == 2u) REDHIP_PGW_ONE(NKC, 2);                                                                                        \
+        else REDHIP_PGW_ONE(NKC, 0);                                                                                                       \
+    } while (0)
+        if (hidden / 512u == 2u) REDHIP_PGW(2); else REDHIP_PGW(4);
+#undef REDHIP_PGW
+#undef REDHIP_PGW_ONE
+        return hipGetLastError();
+    }
+    const size_t acts_lds = kNarrowLds;
 #define REDHIP_PGR_ONE(NKC, FMT)                                                                                                          \
     do {                                                                                                                                  \
         static bool attr = false;                                                                                                          \
         if (!attr) {                                                                                                                       \
-            e = hipFuncSetAttribute(reinterpret_cast<const void *>(prefill_gateup_reg_kernel<NKC, FMT>), hipFuncAttributeMaxDynamicSharedMemorySize, 40 * 1024); \
+            e = hipFuncSetAttribute(reinterpret_cast<const void *>(prefill_gateup_reg_kernel<NKC, FMT>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kNarrowLds); \
             if (e != hipSuccess) return e;                                                                                                 \
             attr = true;                                                                                                                   \
         }                                                                                                                                  \
@@ -1125,7 +1376,7 @@ hipError_t launch_prefill_gateup_tiled(const void *tiled_experts, uint64_t strid
         return hipErrorInvalidValue;
     const uint32_t P = ntok * top_k;
     prof_set_stage(ST_GROUP);
-    REDHIP_LAUNCH(build_tiles_kernel, dim3(1), dim3(1024), 0, s, expert_start, n_unique, P, 0u, tile_group, tile_pair0, tile_n, n_tiles);      // no shared tiles
+    REDHIP_LAUNCH(build_tiles_kernel, dim3(1), dim3(1024), 0, s, expert_start, n_unique, P, 0u, tile_group, tile_pair0, tile_n, n_tiles, prefill_tile_bound(ntok, top_k, n_expert));      // no shared tiles
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     PrefillArgs a{nullptr, stride, nullptr, uid, pair_token, n_unique, tile_group, tile_pair0, tile_n, n_tiles, static_cast<const _Float16 *>(xh),
@@ -1133,7 +1384,7 @@ hipError_t launch_prefill_gateup_tiled(const void *tiled_experts, uint64_t strid
                   ffn, top_k, ntok};
     const TiledArgs ta{a, static_cast<const uint8_t *>(tiled_experts), nullptr, act, nullptr, 0u};
     const uint32_t tile_bound = prefill_tile_bound(ntok, top_k, n_expert);
-    return launch_gateup_reg(ta, dim3(tile_bound < 256u ? tile_bound : 256u), s);
+    return launch_gateup_reg(ta, dim3(tile_bound < 256u ? tile_bound : 256u), s, tile_bound);
 }
 
 // The routed gate/up and down matrices of a chunk on a layout whose experts are IQ2_XS / IQ1_M: the same tile kernels on the row-major
@@ -1150,7 +1401,7 @@ hipError_t launch_prefill_streams(uint32_t gate_up_type, const int8_t *gate_up_g
         return hipErrorInvalidValue;
     const uint32_t P = ntok * top_k;
     prof_set_stage(ST_GROUP);
-    REDHIP_LAUNCH(build_tiles_kernel, dim3(1), dim3(1024), 0, s, expert_start, n_unique, P, 0u, tile_group, tile_pair0, tile_n, n_tiles);      // no shared tiles
+    REDHIP_LAUNCH(build_tiles_kernel, dim3(1), dim3(1024), 0, s, expert_start, n_unique, P, 0u, tile_group, tile_pair0, tile_n, n_tiles, prefill_tile_bound(ntok, top_k, n_expert));      // no shared tiles
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     PrefillArgs a{nullptr, packed_stride, nullptr, uid, pair_token, n_unique, tile_group, tile_pair0, tile_n, n_tiles, static_cast<const _Float16 *>(xh),
@@ -1159,7 +1410,7 @@ hipError_t launch_prefill_streams(uint32_t gate_up_type, const int8_t *gate_up_g
     const uint32_t tile_bound = prefill_tile_bound(ntok, top_k, n_expert);
     const dim3 grid(tile_bound < 256u ? tile_bound : 256u), rblock(kRegWaves * 64);
     const TiledArgs tg{a, static_cast<const uint8_t *>(packed), nullptr, nullptr, gate_up_grid, 0u};
-    e = launch_gateup_reg(tg, grid, s, fg);
+    e = launch_gateup_reg(tg, grid, s, tile_bound, fg);
     if (e != hipSuccess) return e;
     a.stride = down_stride;
     const TiledArgs td{a, static_cast<const uint8_t *>(down), nullptr, nullptr, down_grid, 0u};
@@ -1201,7 +1452,7 @@ hipError_t launch_prefill_packed(const void *experts, uint64_t stride, const voi
     if (!fused_iq2_supported(hidden, ffn) || hidden / 512u > 4u || !ntok) return hipErrorInvalidValue;
     const uint32_t P = ntok * top_k;
     prof_set_stage(ST_GROUP);
-    REDHIP_LAUNCH(build_tiles_kernel, dim3(1), dim3(1024), 0, s, expert_start, n_unique, P, ntok, tile_group, tile_pair0, tile_n, n_tiles);
+    REDHIP_LAUNCH(build_tiles_kernel, dim3(1), dim3(1024), 0, s, expert_start, n_unique, P, ntok, tile_group, tile_pair0, tile_n, n_tiles, prefill_tile_bound(ntok, top_k, n_expert));
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     PrefillArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(shared), uid, pair_token, n_unique,
@@ -1212,7 +1463,7 @@ hipError_t launch_prefill_packed(const void *experts, uint64_t stride, const voi
     if (tiled_experts && tiled_shared && ffn <= 512u) {          // tile-major copy present: activations of a tile in registers
         const TiledArgs ta{a, static_cast<const uint8_t *>(tiled_experts), static_cast<const uint8_t *>(tiled_shared), nullptr, nullptr, 0u};
         const dim3 rblock(kRegWaves * 64);
-        e = launch_gateup_reg(ta, grid, s);
+        e = launch_gateup_reg(ta, grid, s, tile_bound);
         if (e != hipSuccess) return e;
         prof_set_stage(ST_PREFILL_DOWN);
         if (ffn == 256u) REDHIP_LAUNCH((prefill_down_reg_kernel<8, 0>), grid, rblock, 0, s, ta);

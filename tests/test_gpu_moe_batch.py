@@ -124,6 +124,33 @@ def test_prefill_chunk_packed_tiles(hidden, ffn, ntok):
     m.close()
 
 
+@pytest.mark.parametrize("layout,hidden", [("iq2", 1024), ("f2", 2048)])
+def test_prefill_chunk_tile_list_edges(layout, hidden):
+    """Experts with exactly 16, 17, 32, 33, 48 and 49 pairs in one chunk: the gate/up tiles are cut into runs of 32 pairs (two sets of 16
+    share every decoded weight) with remainders of 17 .. 31 as one more such tile and remainders of 1 .. 16 on the 16-pair kernel; the
+    down tiles stay 16 pairs. Every boundary of that split in one call."""
+    from dwarfstar_red_lite_amd.moe import ResidentMoe
+    ntok, E, K = 128, 64, 2
+    cfg = synth.layer_config(hidden=hidden, ffn=512, n_expert=E, top_k=K, layout=layout)
+    lay = synth.make_layer(12, cfg)
+    m = ResidentMoe(cfg, n_layer=1, max_tokens=ntok)
+    m.load_layer(0, lay)
+    order = [0] * 16 + [1] * 17 + [2] * 32 + [3] * 33 + [4] * 48 + [5] * 49
+    order += [6 + i % (E - 6) for i in range(ntok * K - len(order))]
+    ids = np.stack([order[:ntok], order[ntok:]], axis=1).astype(np.uint32)             # token t: pairs t and t + ntok of the run list
+    assert all(ids[t, 0] != ids[t, 1] for t in range(ntok))
+    counts = np.bincount(ids.ravel(), minlength=E)
+    assert list(counts[:6]) == [16, 17, 32, 33, 48, 49]
+    rng = np.random.default_rng(13)
+    x = synth.normed_x(rng, ntok, hidden)
+    w = rng.random((ntok, K)).astype(np.float32) + 0.1
+    w /= w.sum(axis=1, keepdims=True)
+    got = m.experts(0, torch.from_numpy(x).cuda(), torch.from_numpy(ids.astype(np.int32)).cuda(), torch.from_numpy(w).cuda()).cpu().numpy()
+    want = oracle_tokens(cfg, lay, x, ids, w)
+    assert max(rel_l2(got[t], want[t]) for t in range(ntok)) <= REL_L2_TOL
+    m.close()
+
+
 @pytest.mark.parametrize("layout", ["iq2", "f2"])
 def test_prefill_chunk_forward_config_shape(layout):
     """A 24-token chunk at the benchmark shape through forward(): router (tiled, a Q6_K router through its f32 copy), selection, grouping,
