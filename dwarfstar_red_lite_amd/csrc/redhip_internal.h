@@ -168,7 +168,7 @@ hipError_t launch_tile_packed(const void *packed, uint64_t packed_stride, uint32
 hipError_t launch_prefill_gateup_tiled(const void *tiled_experts, uint64_t stride, const uint32_t *uid, const uint32_t *expert_start,
                                        const uint32_t *pair_token, const uint32_t *n_unique, uint32_t *tile_group, uint32_t *tile_pair0, uint32_t *tile_n,
                                        uint32_t *n_tiles, const void *xh, const void *xl, const int *xexp, float *act, void *act_h, void *act_l,
-                                       int *act_exp, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s);
+                                       int *act_exp, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s, bool tiles_built = false);      // tiles_built: launch_group_pairs wrote the tile lists
 // tile-major IQ3_S matrices (one 32-bit word per eight weights) from raw GGUF rows, and the routed down projection of a chunk on them
 hipError_t launch_tile_iq3s(const void *raw, uint64_t raw_stride, uint32_t count, uint32_t nrows, uint32_t K, void *tiled, uint64_t tiled_stride, hipStream_t s);
 // routed matrices of a chunk whose experts are IQ2_XS / IQ1_M: tile kernels on the row-major streams (gate | up at `packed`, down at `down`)
@@ -176,7 +176,7 @@ hipError_t launch_prefill_streams(uint32_t gate_up_type, const int8_t *gate_up_g
                                   const int8_t *down_grid, const void *down, uint64_t down_stride, const uint32_t *uid, const uint32_t *expert_start,
                                   const uint32_t *pair_token, const uint32_t *n_unique, uint32_t *tile_group, uint32_t *tile_pair0, uint32_t *tile_n,
                                   uint32_t *n_tiles, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l, int *act_exp, float *tmp,
-                                  uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s);
+                                  uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s, bool tiles_built = false);      // tiles_built: launch_group_pairs wrote the tile lists
 hipError_t launch_prefill_down_iq3s(const void *tiled_down, uint64_t stride, const uint32_t *uid, const uint32_t *n_unique, const uint32_t *tile_group,
                                     const uint32_t *tile_pair0, const uint32_t *tile_n, const uint32_t *n_tiles, const void *act_h, const void *act_l,
                                     const int *act_exp, float *tmp, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert,
@@ -186,10 +186,69 @@ hipError_t launch_prefill_packed(const void *experts, uint64_t stride, const voi
                                  const uint32_t *pair_token, const uint32_t *n_unique, uint32_t *tile_group, uint32_t *tile_pair0,
                                  uint32_t *tile_n, uint32_t *n_tiles, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l,
                                  int *act_exp, float *tmp, float *sh_tmp, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok,
-                                 uint32_t n_expert, hipStream_t s);
+                                 uint32_t n_expert, hipStream_t s, bool tiles_built = false);      // tiles_built: launch_group_pairs wrote the tile lists
+// Tile lists of a chunk for the prefill kernels. Groups 0..U-1 are the distinct routed experts (pairs expert_start[u] ..
+// expert_start[u + 1]), group U is the shared expert with pairs P .. P + shared_ntok (0: no shared tiles). A tile = (group, first pair,
+// number of pairs). Three lists in the same arrays, list l from entry l * list_stride on (list_stride = prefill_tile_bound of the call),
+// its length in n_tiles[l]:
+//   0  tiles of kPrefillTile pairs (the down kernels; the gate/up kernel of hidden 512)
+//   1  "wide" tiles of 17 .. kPrefillWideTile pairs: a group's runs of 32 pairs, and its remainder when that is more than 16
+//   2  "narrow" tiles: the remainders of 1 .. 16 pairs
+// Lists 1 and 2 together cover every pair once: the gate/up kernel takes the wide tiles on the path that multiplies two sets of 16 pairs
+// with every decoded weight, the narrow ones on the path for 16.
+constexpr uint32_t kPrefillTile = 16u, kPrefillWideTile = 32u;
+struct TileLists {
+    uint32_t *tile_group, *tile_pair0, *tile_n, *n_tiles;
+    uint32_t list_stride, shared_ntok;
+};
+#ifdef __HIPCC__
+// By all 1024 threads of one workgroup: thread u < U brings its group's run (first pair p0, n pairs), the others n = 0; wave_total:
+// LDS scratch. Exclusive prefix sums of the tiles per group, then every group writes its tiles.
+__device__ __forceinline__ void build_tile_lists(uint32_t U, uint32_t p0, uint32_t n, uint32_t P, const TileLists &tl, uint32_t (*wave_total)[16]) {
+    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
+    auto counts = [](uint32_t m, uint32_t *c) {            // tiles of m pairs in the three lists
+        const uint32_t rem = m % kPrefillWideTile;
+        c[0] = (m + kPrefillTile - 1u) / kPrefillTile;
+        c[1] = m / kPrefillWideTile + (rem > kPrefillTile ? 1u : 0u);
+        c[2] = rem > 0u && rem <= kPrefillTile ? 1u : 0u;
+    };
+    uint32_t mine[3], scan[3];
+    counts(n, mine);
+#pragma unroll
+    for (int l = 0; l < 3; ++l) {
+        scan[l] = mine[l];
+#pragma unroll
+        for (int o = 1; o < 64; o <<= 1) {
+            const uint32_t up = __shfl_up(scan[l], o, 64);
+            if (lane >= (uint32_t)o) scan[l] += up;
+        }
+        if (lane == 63u) wave_total[l][wave] = scan[l];
+    }
+    __syncthreads();
+    uint32_t sh[3];
+    counts(tl.shared_ntok, sh);
+#pragma unroll
+    for (int l = 0; l < 3; ++l) {
+        uint32_t base = 0u, routed_tiles = 0u;
+        for (uint32_t w = 0; w < 16u; ++w) { if (w < wave) base += wave_total[l][w]; routed_tiles += wave_total[l][w]; }
+        const uint32_t off = (uint32_t)l * tl.list_stride, first = off + base + scan[l] - mine[l];
+        // tile t of a run of m pairs that starts at pair q0, in list l
+        auto put = [&](uint32_t at, uint32_t group, uint32_t q0, uint32_t m, uint32_t t) {
+            const uint32_t size = l == 0 ? kPrefillTile : kPrefillWideTile, start = l == 2 ? m - m % kPrefillWideTile : size * t;
+            tl.tile_group[at] = group;
+            tl.tile_pair0[at] = q0 + start;
+            tl.tile_n[at] = m - start < size ? m - start : size;
+        };
+        for (uint32_t t = 0; t < mine[l]; ++t) put(first + t, tid, p0, n, t);
+        for (uint32_t t = tid; t < sh[l]; t += 1024u) put(off + routed_tiles + t, U, P, tl.shared_ntok, t);
+        if (tid == 0u) tl.n_tiles[l] = routed_tiles + sh[l];
+    }
+}
+#endif
+// tiles: also write the tile lists of the chunk (the prefill launchers then take tiles_built = true and launch no build_tiles_kernel)
 hipError_t launch_group_pairs(const uint32_t *ids, const float *weights, uint32_t ntok, uint32_t top_k, uint32_t n_expert,
                               uint32_t *uid, uint32_t *expert_start, uint32_t *pair_token, float *pair_weight,
-                              uint32_t *tok_pair, uint32_t *n_unique, hipStream_t s);
+                              uint32_t *tok_pair, uint32_t *n_unique, hipStream_t s, const TileLists *tiles = nullptr);
 
 // ---- decode path over packed IQ2_XXS (redhip_fused.hip) ----
 

@@ -730,8 +730,9 @@ template <bool PREFIX>
 __global__ __launch_bounds__(1024) void group_pairs_kernel(const uint32_t *ids, const float *weights, uint32_t ntok, uint32_t top_k, uint32_t top_k_magic,
                                                            uint32_t n_expert, uint32_t *uid, uint32_t *expert_start,
                                                            uint32_t *pair_token, float *pair_weight, uint32_t *tok_pair,
-                                                           uint32_t *n_unique, uint32_t *status, uint32_t cache_ids) {
+                                                           uint32_t *n_unique, uint32_t *status, uint32_t cache_ids, TileLists tiles) {
     extern __shared__ uint32_t sm[];
+    __shared__ uint32_t tile_tot[3][16];
     const uint32_t words = (ntok + 31u) / 32u, P = ntok * top_k, tid = threadIdx.x;
     uint32_t *first = sm;                          // [n_expert]
     uint32_t *count = first + n_expert;            // [n_expert]
@@ -818,33 +819,37 @@ __global__ __launch_bounds__(1024) void group_pairs_kernel(const uint32_t *ids, 
     } else {
         for (uint32_t p = tid; p < P; p += 1024u) place(p, id_of(p), weights[p]);
     }
+    // the tile lists of the prefill kernels, from the group starts still in LDS: no launch of their own
+    if (tiles.tile_group) build_tile_lists(U, tid < U ? start[tid] : 0u, tid < U ? start[tid + 1u] - start[tid] : 0u, P, tiles, tile_tot);
 }
 
 hipError_t launch_group_pairs(const uint32_t *ids, const float *weights, uint32_t ntok, uint32_t top_k, uint32_t n_expert,
                               uint32_t *uid, uint32_t *expert_start, uint32_t *pair_token, float *pair_weight,
-                              uint32_t *tok_pair, uint32_t *n_unique, hipStream_t s) {
+                              uint32_t *tok_pair, uint32_t *n_unique, hipStream_t s, const TileLists *tiles) {
     if (!ntok || !top_k || !n_expert || n_expert > 1024u || (uint64_t)ntok * top_k * top_k >= (1ull << 32)) return hipErrorInvalidValue;
+    const TileLists tl = tiles ? *tiles : TileLists{};
     const uint32_t words = (ntok + 31u) / 32u;
     const size_t lds = sizeof(uint32_t) * ((size_t)4u * n_expert + 1u + 1024u + 17u + (size_t)n_expert * words);
-    if (lds > 160u * 1024u) return hipErrorInvalidValue;
+    constexpr size_t kGroupDynLds = 159u * 1024u;      // (the kernel has a little static LDS beside it)
+    if (lds > kGroupDynLds) return hipErrorInvalidValue;
     const size_t lds_prefix = lds + sizeof(uint32_t) * (size_t)n_expert * words;
     const uint32_t magic = (uint32_t)(((1ull << 32) + top_k - 1u) / top_k);      // top_k == 1 needs none (and would not fit)
     static bool attr_set = false;
     if (!attr_set) {
-        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(group_pairs_kernel<false>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
-        if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void *>(group_pairs_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024);
+        hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(group_pairs_kernel<false>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGroupDynLds);
+        if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void *>(group_pairs_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGroupDynLds);
         if (e != hipSuccess) return e;
         attr_set = true;
     }
     const size_t ids_bytes = sizeof(uint32_t) * (size_t)ntok * top_k;
-    if (lds_prefix <= 160u * 1024u) {
-        const bool cache = lds_prefix + ids_bytes <= 160u * 1024u;
+    if (lds_prefix <= kGroupDynLds) {
+        const bool cache = lds_prefix + ids_bytes <= kGroupDynLds;
         REDHIP_LAUNCH(group_pairs_kernel<true>, dim3(1), dim3(1024), lds_prefix + (cache ? ids_bytes : 0u), s, ids, weights, ntok, top_k, magic, n_expert, uid, expert_start, pair_token,
-                      pair_weight, tok_pair, n_unique, route_guard().status, cache ? 1u : 0u);
+                      pair_weight, tok_pair, n_unique, route_guard().status, cache ? 1u : 0u, tl);
     } else {
-        const bool cache = lds + ids_bytes <= 160u * 1024u;
+        const bool cache = lds + ids_bytes <= kGroupDynLds;
         REDHIP_LAUNCH(group_pairs_kernel<false>, dim3(1), dim3(1024), lds + (cache ? ids_bytes : 0u), s, ids, weights, ntok, top_k, magic, n_expert, uid, expert_start, pair_token,
-                      pair_weight, tok_pair, n_unique, route_guard().status, cache ? 1u : 0u);
+                      pair_weight, tok_pair, n_unique, route_guard().status, cache ? 1u : 0u, tl);
     }
     return hipGetLastError();
 }

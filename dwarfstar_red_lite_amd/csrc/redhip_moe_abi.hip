@@ -264,10 +264,14 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
         // the shared expert as dense f32 products on the fp32 matrix units, started before the pair sort (one workgroup on an idle machine)
         const bool dense_shared = (stream_tiles || (m->mixed_chunk(ntok) && Ld.dense_gu && m->side));
         if (dense_shared && !fork_shared_dense(m, Ld, x, ntok, s)) return 0;
+        // the pair sort also writes the tile lists of the tile kernels that follow (all-IQ2_XXS layers: with the shared expert's tiles)
+        const bool tile_path = !m->small_batch(ntok) && (m->packed_path(ntok) || stream_tiles || m->mixed_chunk(ntok));
+        const TileLists tl{m->tile_group, m->tile_pair0, m->tile_n, m->n_tiles, prefill_tile_bound(ntok, c.top_k, c.n_expert), m->packed_path(ntok) ? ntok : 0u};
+        const bool tiles_built = !grouped && tile_path;
         if (!grouped) {
             prof_set_stage(ST_GROUP);
             HIP_OK(launch_group_pairs(ids, weights, ntok, c.top_k, c.n_expert, m->uid, m->expert_start, m->pair_token, m->pair_weight,
-                                      m->tok_pair, m->n_unique, s), "grouping launch");
+                                      m->tok_pair, m->n_unique, s, tile_path ? &tl : nullptr), "grouping launch");
         }
         if (m->small_batch(ntok) && grouped && !select_here) {     // the caller's routing, sorted (with its pass list) by the prep launch: expert slices per pass
             const Layer &L = m->layers[layer];
@@ -281,7 +285,7 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
             const Layer &L = m->layers[layer];
             HIP_OK(launch_prefill_packed(L.packed, m->expert_stride, L.shared_packed, L.tiled, L.shared_tiled, m->uid, m->expert_start, m->pair_token, m->n_unique,
                                          m->tile_group, m->tile_pair0, m->tile_n, m->n_tiles, m->xh, m->xl, m->xexp, m->act_h, m->act_l,
-                                         m->act_exp, m->tmp, m->sh_tmp, c.hidden, c.ffn, c.top_k, ntok, c.n_expert, s), "prefill launch");
+                                         m->act_exp, m->tmp, m->sh_tmp, c.hidden, c.ffn, c.top_k, ntok, c.n_expert, s, tiles_built), "prefill launch");
             prof_set_stage(ST_BATCH_COMBINE);
             HIP_OK(launch_batch_combine(m->tmp, m->pair_weight, m->tok_pair, ntok, c.top_k, m->sh_tmp, m->scalar, c.hidden, out, s), "batched combine launch");
             prof_set_stage(ST_OTHER);
@@ -292,7 +296,7 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
             prof_set_stage(ST_BATCH_GATEUP);
             HIP_OK(launch_prefill_streams(m->gu_type, m->gu_grid, L.packed, m->packed_stride, m->dn_type, m->dn_grid, L.words_down, m->words_down_stride(), m->uid,
                                           m->expert_start, m->pair_token, m->n_unique, m->tile_group, m->tile_pair0, m->tile_n, m->n_tiles, m->xh, m->xl, m->xexp,
-                                          m->act_h, m->act_l, m->act_exp, m->tmp, c.hidden, c.ffn, c.top_k, ntok, c.n_expert, s), "stream tile launch");
+                                          m->act_h, m->act_l, m->act_exp, m->tmp, c.hidden, c.ffn, c.top_k, ntok, c.n_expert, s, tiles_built), "stream tile launch");
             if (!join_shared_dense(m, s)) return 0;
             prof_set_stage(ST_BATCH_COMBINE);
             HIP_OK(launch_batch_combine(m->tmp, m->pair_weight, m->tok_pair, ntok, c.top_k, m->sh_tmp, m->scalar, c.hidden, out, s), "batched combine launch");
@@ -304,7 +308,7 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
         if (m->mixed_chunk(ntok))      // xh / xl / xexp come from the router kernel or the prep kernel
             HIP_OK(launch_prefill_gateup_tiled(m->layers[layer].tiled, m->packed_stride, m->uid, m->expert_start, m->pair_token, m->n_unique, m->tile_group,
                                                m->tile_pair0, m->tile_n, m->n_tiles, m->xh, m->xl, m->xexp, tiled_down ? nullptr : m->act, m->act_h, m->act_l,
-                                               m->act_exp, c.hidden, c.ffn, c.top_k, ntok, c.n_expert, s), "tiled gate/up launch");
+                                               m->act_exp, c.hidden, c.ffn, c.top_k, ntok, c.n_expert, s, tiles_built), "tiled gate/up launch");
         else
             HIP_OK(launch_batch_gateup(ex, m->uid, m->expert_start, m->pair_token, m->n_unique, n_groups, P, c.hidden, c.ffn, x, m->act, s), "batched gate/up launch");
         prof_set_stage(ST_BATCH_GATEUP);

@@ -19,65 +19,19 @@
 
 namespace redhip {
 
-constexpr uint32_t kTile = 16u;                 // pairs per tile
+constexpr uint32_t kTile = kPrefillTile;         // pairs per tile
 constexpr uint32_t kRowPad = 32u;               // fp16 elements of padding per staged activation row (64 B: spreads the rows over the banks)
 
 // ---------------------------------------------------------------- tile list
 
-// groups 0..U-1 are the distinct routed experts (pairs expert_start[u] .. expert_start[u + 1]), group U is the shared
-// expert with pairs P .. P + ntok. One workgroup: exclusive prefix sums of the tiles per group, then every group writes
-// its tiles: (group, first pair, number of pairs). Three lists in the same arrays, list l from entry l * list_stride on, its length in
-// n_tiles[l]:
-//   0  tiles of kTile pairs (the down kernels; the gate/up kernel of hidden 512)
-//   1  "wide" tiles of 17 .. kWideTile pairs: a group's runs of 32 pairs, and its remainder when that is more than 16
-//   2  "narrow" tiles: the remainders of 1 .. 16 pairs
-// Lists 1 and 2 together cover every pair once: the gate/up kernels take the wide tiles on the kernel that multiplies two sets of 16
-// pairs with every decoded weight, the narrow ones on the kernel for 16.
-constexpr uint32_t kWideTile = 32u;
-__global__ __launch_bounds__(1024) void build_tiles_kernel(const uint32_t *expert_start, const uint32_t *n_unique, uint32_t P, uint32_t ntok,
-                                                           uint32_t *tile_group, uint32_t *tile_pair0, uint32_t *tile_n, uint32_t *n_tiles, uint32_t list_stride) {
+// the tile lists (TileLists) as a launch of their own, for callers whose pair sort did not write them
+constexpr uint32_t kWideTile = kPrefillWideTile;
+__global__ __launch_bounds__(1024) void build_tiles_kernel(const uint32_t *expert_start, const uint32_t *n_unique, uint32_t P, TileLists tl) {
     __shared__ uint32_t wave_total[3][16];
-    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u;
-    const uint32_t U = n_unique[0];
+    const uint32_t tid = threadIdx.x, U = n_unique[0];
     uint32_t p0 = 0u, n = 0u;
     if (tid < U) { p0 = expert_start[tid]; n = expert_start[tid + 1u] - p0; }
-    auto counts = [](uint32_t m, uint32_t *c) {            // tiles of m pairs in the three lists
-        const uint32_t rem = m % kWideTile;
-        c[0] = (m + kTile - 1u) / kTile;
-        c[1] = m / kWideTile + (rem > kTile ? 1u : 0u);
-        c[2] = rem > 0u && rem <= kTile ? 1u : 0u;
-    };
-    uint32_t mine[3], scan[3];
-    counts(n, mine);
-#pragma unroll
-    for (int l = 0; l < 3; ++l) {
-        scan[l] = mine[l];
-#pragma unroll
-        for (int o = 1; o < 64; o <<= 1) {
-            const uint32_t up = __shfl_up(scan[l], o, 64);
-            if (lane >= (uint32_t)o) scan[l] += up;
-        }
-        if (lane == 63u) wave_total[l][wave] = scan[l];
-    }
-    __syncthreads();
-    uint32_t sh[3];
-    counts(ntok, sh);
-#pragma unroll
-    for (int l = 0; l < 3; ++l) {
-        uint32_t base = 0u, routed_tiles = 0u;
-        for (uint32_t w = 0; w < 16u; ++w) { if (w < wave) base += wave_total[l][w]; routed_tiles += wave_total[l][w]; }
-        const uint32_t off = (uint32_t)l * list_stride, first = off + base + scan[l] - mine[l];
-        // tile t of a run of m pairs that starts at pair q0, in list l
-        auto put = [&](uint32_t at, uint32_t group, uint32_t q0, uint32_t m, uint32_t t) {
-            const uint32_t size = l == 0 ? kTile : kWideTile, start = l == 2 ? m - m % kWideTile : size * t;
-            tile_group[at] = group;
-            tile_pair0[at] = q0 + start;
-            tile_n[at] = m - start < size ? m - start : size;
-        };
-        for (uint32_t t = 0; t < mine[l]; ++t) put(first + t, tid, p0, n, t);
-        for (uint32_t t = tid; t < sh[l]; t += 1024u) put(off + routed_tiles + t, U, P, ntok, t);
-        if (tid == 0u) n_tiles[l] = routed_tiles + sh[l];
-    }
+    build_tile_lists(U, p0, n, P, tl, wave_total);
 }
 
 struct PrefillArgs {
@@ -1371,14 +1325,18 @@ static hipError_t launch_gateup_reg(const TiledArgs &ta, dim3 grid, hipStream_t 
 hipError_t launch_prefill_gateup_tiled(const void *tiled_experts, uint64_t stride, const uint32_t *uid, const uint32_t *expert_start,
                                        const uint32_t *pair_token, const uint32_t *n_unique, uint32_t *tile_group, uint32_t *tile_pair0, uint32_t *tile_n,
                                        uint32_t *n_tiles, const void *xh, const void *xl, const int *xexp, float *act, void *act_h, void *act_l,
-                                       int *act_exp, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s) {
+                                       int *act_exp, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s, bool tiles_built) {
     if (!fused_iq2_supported(hidden, ffn) || hidden / 512u > 4u || ffn > 512u || !ntok || !tiled_experts || (!act && (!act_h || !act_l || !act_exp)))
         return hipErrorInvalidValue;
     const uint32_t P = ntok * top_k;
-    prof_set_stage(ST_GROUP);
-    REDHIP_LAUNCH(build_tiles_kernel, dim3(1), dim3(1024), 0, s, expert_start, n_unique, P, 0u, tile_group, tile_pair0, tile_n, n_tiles, prefill_tile_bound(ntok, top_k, n_expert));      // no shared tiles
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return e;
+    hipError_t e = hipSuccess;
+    if (!tiles_built) {
+        prof_set_stage(ST_GROUP);
+        const TileLists tl{tile_group, tile_pair0, tile_n, n_tiles, prefill_tile_bound(ntok, top_k, n_expert), 0u};      // no shared tiles
+        REDHIP_LAUNCH(build_tiles_kernel, dim3(1), dim3(1024), 0, s, expert_start, n_unique, P, tl);
+        e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
     PrefillArgs a{nullptr, stride, nullptr, uid, pair_token, n_unique, tile_group, tile_pair0, tile_n, n_tiles, static_cast<const _Float16 *>(xh),
                   static_cast<const _Float16 *>(xl), xexp, static_cast<_Float16 *>(act_h), static_cast<_Float16 *>(act_l), act_exp, nullptr, nullptr, hidden,
                   ffn, top_k, ntok};
@@ -1394,16 +1352,20 @@ hipError_t launch_prefill_streams(uint32_t gate_up_type, const int8_t *gate_up_g
                                   const int8_t *down_grid, const void *down, uint64_t down_stride, const uint32_t *uid, const uint32_t *expert_start,
                                   const uint32_t *pair_token, const uint32_t *n_unique, uint32_t *tile_group, uint32_t *tile_pair0, uint32_t *tile_n,
                                   uint32_t *n_tiles, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l, int *act_exp, float *tmp,
-                                  uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s) {
+                                  uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, uint32_t n_expert, hipStream_t s, bool tiles_built) {
     const auto fmt_of = [](uint32_t t) { return t == T_IQ2_XS ? 1u : t == T_IQ1_M ? 2u : 0u; };
     const uint32_t fg = fmt_of(gate_up_type), fd = fmt_of(down_type);
     if (!fg || !fd || !gate_up_grid || !down_grid || !packed || !down || !fused_iq2_supported(hidden, ffn) || hidden / 512u > 4u || (ffn != 256u && ffn != 512u) || !ntok)
         return hipErrorInvalidValue;
     const uint32_t P = ntok * top_k;
-    prof_set_stage(ST_GROUP);
-    REDHIP_LAUNCH(build_tiles_kernel, dim3(1), dim3(1024), 0, s, expert_start, n_unique, P, 0u, tile_group, tile_pair0, tile_n, n_tiles, prefill_tile_bound(ntok, top_k, n_expert));      // no shared tiles
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return e;
+    hipError_t e = hipSuccess;
+    if (!tiles_built) {
+        prof_set_stage(ST_GROUP);
+        const TileLists tl{tile_group, tile_pair0, tile_n, n_tiles, prefill_tile_bound(ntok, top_k, n_expert), 0u};      // no shared tiles
+        REDHIP_LAUNCH(build_tiles_kernel, dim3(1), dim3(1024), 0, s, expert_start, n_unique, P, tl);
+        e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
     PrefillArgs a{nullptr, packed_stride, nullptr, uid, pair_token, n_unique, tile_group, tile_pair0, tile_n, n_tiles, static_cast<const _Float16 *>(xh),
                   static_cast<const _Float16 *>(xl), xexp, static_cast<_Float16 *>(act_h), static_cast<_Float16 *>(act_l), act_exp, tmp, nullptr, hidden,
                   ffn, top_k, ntok};
@@ -1448,13 +1410,17 @@ hipError_t launch_prefill_packed(const void *experts, uint64_t stride, const voi
                                  const uint32_t *pair_token, const uint32_t *n_unique, uint32_t *tile_group, uint32_t *tile_pair0,
                                  uint32_t *tile_n, uint32_t *n_tiles, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l,
                                  int *act_exp, float *tmp, float *sh_tmp, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok,
-                                 uint32_t n_expert, hipStream_t s) {
+                                 uint32_t n_expert, hipStream_t s, bool tiles_built) {
     if (!fused_iq2_supported(hidden, ffn) || hidden / 512u > 4u || !ntok) return hipErrorInvalidValue;
     const uint32_t P = ntok * top_k;
-    prof_set_stage(ST_GROUP);
-    REDHIP_LAUNCH(build_tiles_kernel, dim3(1), dim3(1024), 0, s, expert_start, n_unique, P, ntok, tile_group, tile_pair0, tile_n, n_tiles, prefill_tile_bound(ntok, top_k, n_expert));
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return e;
+    hipError_t e = hipSuccess;
+    if (!tiles_built) {
+        prof_set_stage(ST_GROUP);
+        const TileLists tl{tile_group, tile_pair0, tile_n, n_tiles, prefill_tile_bound(ntok, top_k, n_expert), ntok};
+        REDHIP_LAUNCH(build_tiles_kernel, dim3(1), dim3(1024), 0, s, expert_start, n_unique, P, tl);
+        e = hipGetLastError();
+        if (e != hipSuccess) return e;
+    }
     PrefillArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(shared), uid, pair_token, n_unique,
                   tile_group, tile_pair0, tile_n, n_tiles, static_cast<const _Float16 *>(xh), static_cast<const _Float16 *>(xl), xexp,
                   static_cast<_Float16 *>(act_h), static_cast<_Float16 *>(act_l), act_exp, tmp, sh_tmp, hidden, ffn, top_k, ntok};
