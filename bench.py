@@ -456,7 +456,7 @@ def main():
     if not args.no_cpu:
         cores = min(os.cpu_count() or 1, 64)
         reps, t_cpu, budget = 0, 0.0, 12.0
-        while t_cpu < budget and reps < 400:
+        while t_cpu < budget and reps < 2000:
             tc = time.perf_counter()
             ref.forward(xs_host[reps % NX], threads=cores)
             t_cpu += time.perf_counter() - tc
