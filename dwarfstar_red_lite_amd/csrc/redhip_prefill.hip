@@ -502,10 +502,37 @@ __device__ __forceinline__ void gateup_narrow_items(const TiledArgs &ta, uint32_
     const uint32_t parts = FG / FGH;
     Half8 xa[GQ], xb[GQ];
     uint32_t have_tile = 0xffffffffu;
+    // An item's tile entry, its expert's address and its first weight chunks are three dependent round trips: those of the next item are
+    // requested while this one is multiplied (the last chunk step of an item fetches the next item's first chunks instead of its own again).
+    struct ItemInfo { uint32_t p0, n; const uint8_t *ex; };
+    auto info_of = [&](uint32_t item) {
+        const uint32_t tile = item / parts;
+        const uint32_t u = a.tile_group[tile];
+        return ItemInfo{a.tile_pair0[tile], a.tile_n[tile], u == U ? ta.shared : ta.experts + (uint64_t)a.uid[u] * a.stride};
+    };
+    auto load_chunk = [&](const uint8_t *mat, uint32_t j, uint32_t c) {
+        const uint32_t rtile = 2u * j + rh, chunk = kc * NKC + c;
+        if constexpr (FMT == 0) {
+            const uint4 *qp = reinterpret_cast<const uint4 *>(mat + (((uint64_t)rtile * NC + chunk) * 16u + r) * 32u);
+            const uint16_t *dp = reinterpret_cast<const uint16_t *>(mat + qs_bytes) + ((uint64_t)rtile * HB + chunk / 2u) * 16u + r;
+            return RowChunk{qp[0], qp[1], *dp, 0u};
+        } else {
+            const uint64_t row = 16u * rtile + r;
+            const uint4 *qp = reinterpret_cast<const uint4 *>(mat + (row * HG + 4u * chunk) * 8u);
+            const uint32_t d = reinterpret_cast<const uint16_t *>(mat + qs_bytes)[row * HB + chunk / 2u];
+            return RowChunk{qp[0], qp[1], d, FMT == 1 ? *reinterpret_cast<const uint32_t *>(mat + sc_off + row * HG + 4u * chunk) : 0u};
+        }
+    };
+    if (item_begin >= item_end) return;
+    ItemInfo cur = info_of(item_begin);
+    RowChunk cg = load_chunk(cur.ex, (item_begin % parts) * FGH, 0u), cu = load_chunk(cur.ex + gate_bytes, (item_begin % parts) * FGH, 0u);
     for (uint32_t item = item_begin; item < item_end; ++item) {
         const uint32_t tile = item / parts, ipart = item % parts, j0 = ipart * FGH;
-        const uint32_t u = a.tile_group[tile], p0 = a.tile_pair0[tile], n = a.tile_n[tile];
-        const uint8_t *ex = u == U ? ta.shared : ta.experts + (uint64_t)a.uid[u] * a.stride;
+        const uint32_t p0 = cur.p0, n = cur.n;
+        const uint8_t *ex = cur.ex;
+        const uint32_t next_item = item + 1u < item_end ? item + 1u : item;
+        const ItemInfo nxt = info_of(next_item);
+        const uint32_t next_j0 = (next_item % parts) * FGH;
         __syncthreads();                                   // the previous item's readers are done with acts / tok_of; tables are built
         if (tile != have_tile) {
             have_tile = tile;
@@ -528,29 +555,17 @@ __device__ __forceinline__ void gateup_narrow_items(const TiledArgs &ta, uint32_
                 }
             }
         }
-        auto load_chunk = [&](const uint8_t *mat, uint32_t j, uint32_t c) {
-            const uint32_t rtile = 2u * j + rh, chunk = kc * NKC + c;
-            if constexpr (FMT == 0) {
-                const uint4 *qp = reinterpret_cast<const uint4 *>(mat + (((uint64_t)rtile * NC + chunk) * 16u + r) * 32u);
-                const uint16_t *dp = reinterpret_cast<const uint16_t *>(mat + qs_bytes) + ((uint64_t)rtile * HB + chunk / 2u) * 16u + r;
-                return RowChunk{qp[0], qp[1], *dp, 0u};
-            } else {
-                const uint64_t row = 16u * rtile + r;
-                const uint4 *qp = reinterpret_cast<const uint4 *>(mat + (row * HG + 4u * chunk) * 8u);
-                const uint32_t d = reinterpret_cast<const uint16_t *>(mat + qs_bytes)[row * HB + chunk / 2u];
-                return RowChunk{qp[0], qp[1], d, FMT == 1 ? *reinterpret_cast<const uint32_t *>(mat + sc_off + row * HG + 4u * chunk) : 0u};
-            }
-        };
         const uint8_t *gmat = ex, *umat = ex + gate_bytes;
-        RowChunk cg = load_chunk(gmat, j0, 0u), cu = load_chunk(umat, j0, 0u);
 #pragma unroll 1
         for (uint32_t j = j0; j < j0 + FGH; ++j) {
             float4_t totg = {0.0f, 0.0f, 0.0f, 0.0f}, totu = totg;
 #pragma unroll
             for (uint32_t c = 0; c < (uint32_t)NKC; ++c) {
-                // the chunk after this one (same unit, or the first of the next unit; the last unit reloads itself) is in flight
-                const uint32_t nj = c + 1u < (uint32_t)NKC ? j : (j + 1u < j0 + FGH ? j + 1u : j), nc = c + 1u < (uint32_t)NKC ? c + 1u : 0u;
-                const RowChunk ng = load_chunk(gmat, nj, nc), nu = load_chunk(umat, nj, nc);
+                // the chunk after this one (same unit, the first of the next unit, or the first of the next item) is in flight
+                const bool to_next_item = c + 1u == (uint32_t)NKC && j + 1u == j0 + FGH;
+                const uint32_t nj = c + 1u < (uint32_t)NKC ? j : (to_next_item ? next_j0 : j + 1u), nc = c + 1u < (uint32_t)NKC ? c + 1u : 0u;
+                const uint8_t *ngm = to_next_item ? nxt.ex : gmat;
+                const RowChunk ng = load_chunk(ngm, nj, nc), nu = load_chunk(ngm + gate_bytes, nj, nc);
                 __builtin_amdgcn_sched_barrier(0);         // keeps the loads ahead of the chunk's arithmetic
                 const uint2 wg4[4] = {make_uint2(cg.a.x, cg.a.y), make_uint2(cg.a.z, cg.a.w), make_uint2(cg.b.x, cg.b.y), make_uint2(cg.b.z, cg.b.w)};
                 const uint2 wu4[4] = {make_uint2(cu.a.x, cu.a.y), make_uint2(cu.a.z, cu.a.w), make_uint2(cu.b.x, cu.b.y), make_uint2(cu.b.z, cu.b.w)};
@@ -620,6 +635,7 @@ __device__ __forceinline__ void gateup_narrow_items(const TiledArgs &ta, uint32_
             for (uint32_t c = c0 + lane; c < c1; c += 64u) split_hi_lo(acts[i * AROW + c - c0], inv, a.act_h + pr * F + c, a.act_l + pr * F + c);
             if (lane == 0u) a.act_exp[kExpPerPair * pr + ipart] = e;
         }
+        cur = nxt;
     }
 }
 
