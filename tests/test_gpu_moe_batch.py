@@ -151,6 +151,44 @@ def test_prefill_chunk_tile_list_edges(layout, hidden):
     m.close()
 
 
+@pytest.mark.parametrize("layout", ["iq2", "f2", "xs", "m"])
+def test_drawn_routing_every_batch_size_class(layout, golden_dir):
+    """Seeded routing at every batch size class of the dispatch (one token, small batches, two small batches, chunks), spread over all
+    experts or concentrated on top_k of them (every token the same experts: the largest tiles a chunk can have), on every layout:
+    caller-given routing and the layer's own router against the CPU path."""
+    import json
+    import os
+    from dwarfstar_red_lite_amd import moe as moe_api
+    from dwarfstar_red_lite_amd.moe import ResidentMoe
+    if layout in ("xs", "m"):
+        g = json.load(open(os.path.join(golden_dir, "iq_grids.json")))
+        grids = [np.frombuffer(bytes.fromhex(g[k]), np.int8) for k in ("iq2_xs", "iq1_m")]
+        moe_api.set_codebooks(*grids)
+        orc.set_codebooks(*grids)
+    H, F, E, K = 1024, 256, 24, 6
+    cfg = synth.layer_config(hidden=H, ffn=F, n_expert=E, top_k=K, layout=layout)
+    lay = synth.make_layer(21, cfg)
+    m = ResidentMoe(cfg, n_layer=1, max_tokens=130)
+    m.load_layer(0, lay)
+    ref = orc.Layer(cfg, **lay)
+    rng = np.random.default_rng(22)
+    for ntok, hot in ((1, E), (2, K), (7, E), (9, K), (16, 11), (33, K), (130, K), (130, E)):
+        x = synth.normed_x(rng, ntok, H)
+        ids = np.stack([rng.permutation(hot)[:K] for _ in range(ntok)]).astype(np.uint32)
+        w = rng.random((ntok, K)).astype(np.float32) + 0.05
+        w /= w.sum(axis=1, keepdims=True)
+        got = m.experts(0, torch.from_numpy(x).cuda(), torch.from_numpy(ids.astype(np.int32)).cuda(), torch.from_numpy(w).cuda()).cpu().numpy()
+        want = oracle_tokens(cfg, lay, x, ids, w)
+        assert max(rel_l2(got[t], want[t]) for t in range(ntok)) <= REL_L2_TOL, (layout, ntok, hot)
+        got = m.forward(0, torch.from_numpy(x).cuda()).cpu().numpy()
+        gids, _, _ = m.last_route(ntok)
+        want, cids, _, _ = ref.forward(x, threads=8)
+        agree = [t for t in range(ntok) if np.array_equal(gids[t], cids[t])]             # (a near tie in the logits may order two experts differently)
+        assert len(agree) >= ntok - 1
+        assert max(rel_l2(got[t], want[t]) for t in agree) <= REL_L2_TOL, (layout, ntok)
+    m.close()
+
+
 @pytest.mark.parametrize("layout", ["iq2", "f2"])
 def test_prefill_chunk_forward_config_shape(layout):
     """A 24-token chunk at the benchmark shape through forward(): router (tiled, a Q6_K router through its f32 copy), selection, grouping,
