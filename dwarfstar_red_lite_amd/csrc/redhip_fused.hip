@@ -67,14 +67,14 @@ hipError_t launch_repack_iq2xxs(const void *raw, uint64_t raw_stride, uint32_t c
     return hipGetLastError();
 }
 
-// The same split for the two formats that decode through caller-supplied codebooks, row-major only:
+// The same split for the two formats that decode through caller-supplied codebooks (col_major as above: every array [group or block][row]):
 //   IQ2_XS (74-byte blocks): qs [nrows][K/32] uint2 = the group's four u16 (9-bit index + 7 sign bits each), ds [nrows][K/256] u16,
 //                            sc [nrows][K/32] u8 = the group's two 4-bit scales (one per 16 weights)
 //   IQ1_M (56-byte blocks):  qs [nrows][K/32] uint2: x = the group's four low index bytes, y = its four nibbles (3 high index bits +
 //                            offset sign) | scale of the first 16 weights << 16 | scale of the second 16 << 19; ds [nrows][K/256] u16 = d
 //                            gathered from the top nibbles of the block's four scale words
 template <uint32_t T>
-__global__ void repack_codebook_kernel(const uint8_t *raw0, uint64_t raw_stride, uint32_t nrows, uint32_t K, uint8_t *packed0, uint64_t packed_stride) {
+__global__ void repack_codebook_kernel(const uint8_t *raw0, uint64_t raw_stride, uint32_t nrows, uint32_t K, int col_major, uint8_t *packed0, uint64_t packed_stride) {
     const uint32_t groups = K / 32u, blocks = K / 256u;
     const uint8_t *raw = raw0 + (uint64_t)blockIdx.y * raw_stride;
     uint8_t *pk = packed0 + (uint64_t)blockIdx.y * packed_stride;
@@ -85,31 +85,32 @@ __global__ void repack_codebook_kernel(const uint8_t *raw0, uint64_t raw_stride,
     if (gid >= (uint64_t)nrows * groups) return;
     const uint32_t r = (uint32_t)(gid / groups), g = (uint32_t)(gid % groups), gb = g & 7u;
     const uint8_t *bp = raw + ((uint64_t)r * blocks + (g >> 3)) * Fmt<T>::kBlock;
+    const uint64_t at = col_major ? (uint64_t)g * nrows + r : gid, d_at = col_major ? (uint64_t)(g >> 3) * nrows + r : (uint64_t)r * blocks + (g >> 3);
     if constexpr (T == T_IQ2_XS) {
-        qs[gid] = make_uint2(ld_u32_a2(bp + 2u + 8u * gb), ld_u32_a2(bp + 6u + 8u * gb));
-        sc[gid] = bp[66u + gb];
-        if (gb == 0u) ds[(uint64_t)r * blocks + (g >> 3)] = (uint16_t)ld_u16(bp);
+        qs[at] = make_uint2(ld_u32_a2(bp + 2u + 8u * gb), ld_u32_a2(bp + 6u + 8u * gb));
+        sc[at] = bp[66u + gb];
+        if (gb == 0u) ds[d_at] = (uint16_t)ld_u16(bp);
     } else {
         const uint32_t word = ld_u16(bp + 48u + 2u * (gb >> 1)), sh = 6u * (gb & 1u);
-        qs[gid] = make_uint2(ld_u32_a2(bp + 4u * gb), ld_u16(bp + 32u + 2u * gb) | (((word >> sh) & 7u) << 16) | (((word >> (sh + 3u)) & 7u) << 19));
+        qs[at] = make_uint2(ld_u32_a2(bp + 4u * gb), ld_u16(bp + 32u + 2u * gb) | (((word >> sh) & 7u) << 16) | (((word >> (sh + 3u)) & 7u) << 19));
         if (gb == 0u) {
             const uint32_t s0 = ld_u16(bp + 48u), s1 = ld_u16(bp + 50u), s2 = ld_u16(bp + 52u), s3 = ld_u16(bp + 54u);
-            ds[(uint64_t)r * blocks + (g >> 3)] = (uint16_t)((s0 >> 12) | ((s1 >> 8) & 0x00f0u) | ((s2 >> 4) & 0x0f00u) | (s3 & 0xf000u));
+            ds[d_at] = (uint16_t)((s0 >> 12) | ((s1 >> 8) & 0x00f0u) | ((s2 >> 4) & 0x0f00u) | (s3 & 0xf000u));
         }
     }
 }
 
 // gate / up matrices of `type` (IQ2_XXS, IQ2_XS, IQ1_M) into the streams the one-token gate/up kernel reads; packed_matrix_bytes() each
 hipError_t launch_repack_gateup(uint32_t type, const void *raw, uint64_t raw_stride, uint32_t count, uint32_t nrows, uint32_t K,
-                                void *packed, uint64_t packed_stride, hipStream_t s) {
-    if (type == T_IQ2_XXS) return launch_repack_iq2xxs(raw, raw_stride, count, nrows, K, false, packed, packed_stride, s);
+                                void *packed, uint64_t packed_stride, hipStream_t s, bool col_major) {
+    if (type == T_IQ2_XXS) return launch_repack_iq2xxs(raw, raw_stride, count, nrows, K, col_major, packed, packed_stride, s);
     if (!nrows || !K || K % 256u || !count || count > 65535u) return hipErrorInvalidValue;
     const uint64_t total = (uint64_t)nrows * (K / 32u);
     const dim3 grid((uint32_t)((total + 255u) / 256u), count);
     if (type == T_IQ2_XS)
-        REDHIP_LAUNCH(repack_codebook_kernel<T_IQ2_XS>, grid, dim3(256), 0, s, static_cast<const uint8_t *>(raw), raw_stride, nrows, K, static_cast<uint8_t *>(packed), packed_stride);
+        REDHIP_LAUNCH(repack_codebook_kernel<T_IQ2_XS>, grid, dim3(256), 0, s, static_cast<const uint8_t *>(raw), raw_stride, nrows, K, col_major ? 1 : 0, static_cast<uint8_t *>(packed), packed_stride);
     else if (type == T_IQ1_M)
-        REDHIP_LAUNCH(repack_codebook_kernel<T_IQ1_M>, grid, dim3(256), 0, s, static_cast<const uint8_t *>(raw), raw_stride, nrows, K, static_cast<uint8_t *>(packed), packed_stride);
+        REDHIP_LAUNCH(repack_codebook_kernel<T_IQ1_M>, grid, dim3(256), 0, s, static_cast<const uint8_t *>(raw), raw_stride, nrows, K, col_major ? 1 : 0, static_cast<uint8_t *>(packed), packed_stride);
     else
         return hipErrorInvalidValue;
     return hipGetLastError();
@@ -143,16 +144,17 @@ hipError_t launch_dequant_packed_iq2xxs(const void *packed, uint32_t nrows, uint
 
 // the same tap for the packed IQ2_XS / IQ1_M streams; arithmetic as decode32_cb
 template <uint32_t T>
-__global__ void dequant_packed_codebook_kernel(const uint8_t *pk, uint32_t nrows, uint32_t K, const int8_t *grid, float *out) {
+__global__ void dequant_packed_codebook_kernel(const uint8_t *pk, uint32_t nrows, uint32_t K, const int8_t *grid, float *out, int col_major) {
     const uint32_t groups = K / 32u, blocks = K / 256u;
     const uint64_t gid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (gid >= (uint64_t)nrows * groups) return;
     const uint32_t r = (uint32_t)(gid / groups), g = (uint32_t)(gid % groups);
-    const uint2 v = reinterpret_cast<const uint2 *>(pk)[gid];
-    const float d = half_bits_to_f32(reinterpret_cast<const uint16_t *>(pk + (uint64_t)nrows * groups * 8u)[(uint64_t)r * blocks + (g >> 3)]);
+    const uint64_t at = col_major ? (uint64_t)g * nrows + r : gid, d_at = col_major ? (uint64_t)(g >> 3) * nrows + r : (uint64_t)r * blocks + (g >> 3);
+    const uint2 v = reinterpret_cast<const uint2 *>(pk)[at];
+    const float d = half_bits_to_f32(reinterpret_cast<const uint16_t *>(pk + (uint64_t)nrows * groups * 8u)[d_at]);
     float *o = out + (uint64_t)r * K + 32u * g;
     if constexpr (T == T_IQ2_XS) {
-        const uint32_t sc = (pk + (uint64_t)nrows * groups * 8u + (uint64_t)nrows * blocks * 2u)[gid];
+        const uint32_t sc = (pk + (uint64_t)nrows * groups * 8u + (uint64_t)nrows * blocks * 2u)[at];
         for (uint32_t l = 0; l < 4u; ++l) {
             const uint32_t w16 = ((l < 2u ? v.x : v.y) >> (16u * (l & 1u))) & 0xffffu;
             const int8_t *entry = grid + (w16 & 511u) * 8u;
@@ -170,13 +172,13 @@ __global__ void dequant_packed_codebook_kernel(const uint8_t *pk, uint32_t nrows
     }
 }
 
-hipError_t launch_dequant_packed(uint32_t type, const void *packed, uint32_t nrows, uint32_t K, const int8_t *grid, float *out, hipStream_t s) {
-    if (type == T_IQ2_XXS) return launch_dequant_packed_iq2xxs(packed, nrows, K, false, out, s);
+hipError_t launch_dequant_packed(uint32_t type, const void *packed, uint32_t nrows, uint32_t K, const int8_t *grid, float *out, hipStream_t s, bool col_major) {
+    if (type == T_IQ2_XXS) return launch_dequant_packed_iq2xxs(packed, nrows, K, col_major, out, s);
     if (!nrows || !K || K % 256u || !grid) return hipErrorInvalidValue;
     const uint64_t total = (uint64_t)nrows * (K / 32u);
     const dim3 grid_dim((uint32_t)((total + 255u) / 256u));
-    if (type == T_IQ2_XS) REDHIP_LAUNCH(dequant_packed_codebook_kernel<T_IQ2_XS>, grid_dim, dim3(256), 0, s, static_cast<const uint8_t *>(packed), nrows, K, grid, out);
-    else if (type == T_IQ1_M) REDHIP_LAUNCH(dequant_packed_codebook_kernel<T_IQ1_M>, grid_dim, dim3(256), 0, s, static_cast<const uint8_t *>(packed), nrows, K, grid, out);
+    if (type == T_IQ2_XS) REDHIP_LAUNCH(dequant_packed_codebook_kernel<T_IQ2_XS>, grid_dim, dim3(256), 0, s, static_cast<const uint8_t *>(packed), nrows, K, grid, out, col_major ? 1 : 0);
+    else if (type == T_IQ1_M) REDHIP_LAUNCH(dequant_packed_codebook_kernel<T_IQ1_M>, grid_dim, dim3(256), 0, s, static_cast<const uint8_t *>(packed), nrows, K, grid, out, col_major ? 1 : 0);
     else return hipErrorInvalidValue;
     return hipGetLastError();
 }
@@ -1783,6 +1785,9 @@ struct BatchSliceArgs {
     // mixed layouts (MIX): down_cm holds column-sliced word-packed IQ3_S matrices; the shared expert comes as its gate . x and up . x
     // products [ntok][2 ffn] f32 (left by the router launch) and the dense f32 copy [hidden][ffn] of its down matrix
     const float *shared_gu, *shared_dense;
+    // MIX 2 / 3: `experts` holds the row-major IQ2_XS / IQ1_M streams of gate | up, down_cm the column-sliced streams of the down matrices,
+    // grid the caller's codebook; the shared expert as for MIX 1
+    const int8_t *grid;
 };
 
 // two tokens' results of one group: va for the token in rows 0, 1 of the operand, vb for the one in rows 2, 3
@@ -1812,16 +1817,22 @@ __device__ __forceinline__ void group_dot2_rep(uint2 q, const half4_t *ax, const
 // conflicts: the LDS serves sixteen lanes of a 16-byte read together); eight copies of both tables 34.3 us (a fifth fewer vector
 // instructions, 70 % more LDS reads); sixteen copies of both at one workgroup per compute unit 43.5 us.
 constexpr int kBatchRep = 16, kBatchSignRep = 0;
-template <int NKC, int REP, int MIX>       // MIX 0: every matrix packed IQ2_XXS; 1: IQ3_S down matrices, dense shared expert (see BatchSliceArgs)
+// LDS bytes of the decode tables at the head of the kernel's dynamic LDS
+template <int REP, int MIX> constexpr uint32_t batch_slice_table_bytes() {
+    return MIX == 2 ? 512u * 16u : MIX == 3 ? 2048u * 16u : (uint32_t)(REP + 1) * kMagBytes + (uint32_t)(kBatchSignRep + 1) * kSignBytes;
+}
+// MIX 0: every matrix packed IQ2_XXS; 1: IQ3_S down matrices, dense shared expert; 2 / 3: IQ2_XS / IQ1_M streams, dense shared expert (see BatchSliceArgs)
+template <int NKC, int REP, int MIX>
 __global__ __launch_bounds__(kWaves * 64, 8) void batch_slice_kernel(BatchSliceArgs a) {
     constexpr int NW = kWaves;
     constexpr int UPW = 16 * NKC / NW;
     constexpr int DU = (8 * NKC + NW - 1) / NW;
     constexpr int SREP = kBatchSignRep;
+    constexpr int FMT = MIX >= 2 ? MIX - 1 : 0;            // format of the routed matrices as group_dot_fmt2 numbers them
     extern __shared__ __attribute__((aligned(16))) uint8_t dyn[];
     uint8_t *lds = dyn;
     uint8_t *strip = dyn + REP * kMagBytes + SREP * kSignBytes;
-    float *part = reinterpret_cast<float *>(strip + kMagBytes + kSignBytes);      // [2 tokens][NKC][64]
+    float *part = reinterpret_cast<float *>(dyn + batch_slice_table_bytes<REP, MIX>());      // [2 tokens][NKC][64]
     _Float16 *act_hl = reinterpret_cast<_Float16 *>(part + 2 * NKC * 64);  // [2 tokens][2 halves][32]
     float *act_scale = reinterpret_cast<float *>(act_hl + 128);            // [2] (+ 2 unused)
     uint8_t *iq3_tab = reinterpret_cast<uint8_t *>(act_scale + 4);         // MIX: 4 KB, the IQ3_S grid as fp16
@@ -1894,9 +1905,10 @@ __global__ __launch_bounds__(kWaves * 64, 8) void batch_slice_kernel(BatchSliceA
     }
     const uint8_t *ex = sh ? a.shared : a.experts + (uint64_t)expert * a.stride;
     const uint8_t *dn = sh ? a.shared_down_cm : a.down_cm + (uint64_t)expert * a.down_stride;
-    const uint64_t gate_bytes = (uint64_t)F * HG * 8u + (uint64_t)F * HB * 2u;
+    const uint64_t gate_sc = (uint64_t)F * HG * 8u + (uint64_t)F * HB * 2u;       // IQ2_XS: the scale bytes [row][group] behind qs and ds
+    const uint64_t gate_bytes = gate_sc + (MIX == 2 ? (uint64_t)F * HG : 0u);
     uint2 wq[UPW];
-    uint32_t wd[UPW];
+    uint32_t wd[UPW];                                    // block scale d (fp16 bits); IQ2_XS: the group's scale byte above it
 #pragma unroll
     for (int u = 0; u < UPW; ++u) {
         const uint32_t quad = q0 + (NW / NKC) * u;
@@ -1904,30 +1916,36 @@ __global__ __launch_bounds__(kWaves * 64, 8) void batch_slice_kernel(BatchSliceA
         const uint8_t *mat = ex + (quad < 8u ? 0u : gate_bytes);
         wq[u] = reinterpret_cast<const uint2 *>(mat)[(uint64_t)r * HG + G];
         wd[u] = reinterpret_cast<const uint16_t *>(mat + (uint64_t)F * HG * 8u)[(uint64_t)r * HB + (G >> 3)];
+        if constexpr (MIX == 2) wd[u] |= (uint32_t)(mat + gate_sc)[(uint64_t)r * HG + G] << 16;
     }
-    using DownGroup = typename std::conditional<MIX != 0, uint4, uint2>::type;      // one row's 32 weights of the slice
-    const DownGroup *down_qs = reinterpret_cast<const DownGroup *>(dn) + (MIX != 0 ? 0u : (uint64_t)g * H);
+    using DownGroup = typename std::conditional<MIX == 1, uint4, uint2>::type;      // one row's 32 weights of the slice
+    const DownGroup *down_qs = reinterpret_cast<const DownGroup *>(dn) + (MIX == 1 ? 0u : (uint64_t)g * H);
     const uint16_t *down_ds = reinterpret_cast<const uint16_t *>(dn + (uint64_t)FG * H * sizeof(DownGroup)) + (uint64_t)(g >> 3) * H;
+    const uint8_t *down_sc = dn + (uint64_t)FG * H * 8u + (uint64_t)(FG >> 3) * H * 2u + (uint64_t)g * H;      // MIX 2
     DownGroup dq[DU];
-    uint32_t dd[DU];
+    uint32_t dd[DU];                                     // as wd
 #pragma unroll
     for (int kk = 0; kk < DU; ++kk) {
         const uint32_t unit = wave + NW * kk;
         const uint32_t r = 64u * (unit < 8u * NKC ? unit : 0u) + lane;
-        dq[kk] = down_qs[MIX != 0 ? iq3s_sliced_index(g, r, FG, H) : (uint64_t)r];
+        dq[kk] = down_qs[MIX == 1 ? iq3s_sliced_index(g, r, FG, H) : (uint64_t)r];
         dd[kk] = down_ds[r];
+        if constexpr (MIX == 2) dd[kk] |= (uint32_t)down_sc[r] << 16;
     }
-    if constexpr (MIX != 0) build_iq3s_quads(iq3_tab, tid);
+    if constexpr (MIX == 1) build_iq3s_quads(iq3_tab, tid);
     const float w0 = sh ? a.scalar[tok0] : a.weights[tok0 * K + k0], w1 = sh ? a.scalar[tok1] : a.weights[tok1 * K + k1];
-    const float xs0 = 0.125f * exp2i(a.xexp[tok0]), xs1 = 0.125f * exp2i(a.xexp[tok1]);
-    build_tables_rep<REP, 16, SREP>(lds, strip, wave, lane);
+    // (an IQ1_M weight is d (2 s + 1) (entry +- 1/8): no 1 / 8)
+    const float xs0 = (MIX == 3 ? 1.0f : 0.125f) * exp2i(a.xexp[tok0]), xs1 = (MIX == 3 ? 1.0f : 0.125f) * exp2i(a.xexp[tok1]);
+    if constexpr (MIX >= 2) build_codebook_table<FMT>(lds, tid, a.grid, 0u, (uint32_t)NW * 64u);
+    else build_tables_rep<REP, 16, SREP>(lds, strip, wave, lane);
     const uint8_t *tab = lds + (lane % REP) * 16u, *stab = lds + REP * kMagBytes + (lane % (SREP ? SREP : 1)) * 16u;
     __syncthreads();                                   // tables
 
     float va[UPW], vb[UPW];
 #pragma unroll
     for (int u = 0; u < UPW; ++u) {
-        group_dot2_rep<REP, SREP>(wq[u], ax, tab, stab, va[u], vb[u]);
+        if constexpr (MIX >= 2) group_dot_fmt2<FMT>(wq[u], wd[u] >> 16, ax, lds, va[u], vb[u]);
+        else group_dot2_rep<REP, SREP>(wq[u], ax, tab, stab, va[u], vb[u]);
         const float d = scale_to_f32(wd[u]);
         va[u] *= d;
         vb[u] *= d;
@@ -1963,14 +1981,15 @@ __global__ __launch_bounds__(kWaves * 64, 8) void batch_slice_kernel(BatchSliceA
 #pragma unroll
         for (int s8 = 0; s8 < 8; ++s8) ad[s8] = *reinterpret_cast<const half4_t *>(src + 4 * s8);
     }
-    // (an IQ3_S weight is d (1 + 2 nibble) grid byte: no 1 / 8)
-    const float post0 = act_scale[0] * w0 * (MIX != 0 ? 1.0f : 0.125f), post1 = act_scale[1] * w1 * (MIX != 0 ? 1.0f : 0.125f);
+    // (an IQ3_S weight is d (1 + 2 nibble) grid byte, an IQ1_M weight as above: no 1 / 8)
+    const float post0 = act_scale[0] * w0 * (MIX == 1 || MIX == 3 ? 1.0f : 0.125f), post1 = act_scale[1] * w1 * (MIX == 1 || MIX == 3 ? 1.0f : 0.125f);
 #pragma unroll
     for (int kk = 0; kk < DU; ++kk) {
         const uint32_t unit = wave + NW * kk;
         if (unit < 8u * NKC) {
             float da, db;
-            if constexpr (MIX != 0) iq3s_group_dot(dq[kk], ad, iq3_tab, da, db);
+            if constexpr (MIX == 1) iq3s_group_dot(dq[kk], ad, iq3_tab, da, db);
+            else if constexpr (MIX >= 2) group_dot_fmt2<FMT>(dq[kk], dd[kk] >> 16, ad, lds, da, db);
             else group_dot2_rep<REP, SREP>(dq[kk], ad, tab, stab, da, db);
             const float d = scale_to_f32(dd[kk]);
             out0[64u * unit + lane] = da * d * post0;
@@ -2022,19 +2041,20 @@ hipError_t launch_expert_slices(const void *experts, uint64_t stride, const void
 hipError_t launch_batch_slices(const void *experts, uint64_t stride, const void *down_cm, uint64_t down_stride, const void *shared, const void *shared_down_cm,
                                const void *pass_list, const uint32_t *n_pass, const float *weights, const float *scalar, const void *xh, const void *xl,
                                const int *xexp, float *partial, float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, hipStream_t s,
-                               const float *shared_gu, const float *shared_dense) {
+                               const float *shared_gu, const float *shared_dense, uint32_t stream_type, const int8_t *grid) {
     if (!fused_iq2_supported(hidden, ffn) || hidden % 32u || !ntok || ntok > 16u || ntok * top_k > 128u || !pass_list || !n_pass) return hipErrorInvalidValue;
     const bool mix = shared_gu != nullptr;
     if (mix ? !shared_dense : (!shared || !shared_down_cm)) return hipErrorInvalidValue;
+    if (stream_type && ((stream_type != T_IQ2_XS && stream_type != T_IQ1_M) || !grid || !mix)) return hipErrorInvalidValue;
+    const int kind = stream_type == T_IQ2_XS ? 2 : stream_type == T_IQ1_M ? 3 : mix ? 1 : 0;
     const BatchSliceArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(down_cm), down_stride, static_cast<const uint8_t *>(shared),
                            static_cast<const uint8_t *>(shared_down_cm), static_cast<const uint2 *>(pass_list), n_pass, weights, scalar,
-                           static_cast<const _Float16 *>(xh), static_cast<const _Float16 *>(xl), xexp, partial, hidden, ffn, top_k, ntok, shared_gu, shared_dense};
+                           static_cast<const _Float16 *>(xh), static_cast<const _Float16 *>(xl), xexp, partial, hidden, ffn, top_k, ntok, shared_gu, shared_dense, grid};
     const dim3 grid_dim(ffn / 32u, ntok * top_k + (ntok + 1u) / 2u);      // every pair a pass of its own at most, then the shared expert's passes
 #define REDHIP_BSLICE_ONE(NKC, MIX)                                                                                                    \
     do {                                                                                                                               \
         static bool attr = false;                                                                                                       \
-        const size_t dyn = (size_t)kBatchRep * kMagBytes + (size_t)kBatchSignRep * kSignBytes + kMagBytes + kSignBytes + (size_t)2u * NKC * 64u * 4u + 256u + 16u + \
-                           (MIX ? kIq3TableBytes : 0u);                                                                                 \
+        const size_t dyn = (size_t)batch_slice_table_bytes<kBatchRep, MIX>() + (size_t)2u * NKC * 64u * 4u + 256u + 16u + (MIX == 1 ? kIq3TableBytes : 0u); \
         if (!attr) {                                                                                                                    \
             const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(batch_slice_kernel<NKC, kBatchRep, MIX>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn); \
             if (e != hipSuccess) return e;                                                                                              \
@@ -2042,7 +2062,10 @@ hipError_t launch_batch_slices(const void *experts, uint64_t stride, const void 
         }                                                                                                                               \
         REDHIP_LAUNCH((batch_slice_kernel<NKC, kBatchRep, MIX>), grid_dim, dim3(kWaves * 64), dyn, s, a);                                 \
     } while (0)
-#define REDHIP_BSLICE(NKC) do { if (mix) REDHIP_BSLICE_ONE(NKC, 1); else REDHIP_BSLICE_ONE(NKC, 0); } while (0)
+#define REDHIP_BSLICE(NKC)                                                                                                             \
+    do {                                                                                                                               \
+        if (kind == 3) REDHIP_BSLICE_ONE(NKC, 3); else if (kind == 2) REDHIP_BSLICE_ONE(NKC, 2); else if (kind == 1) REDHIP_BSLICE_ONE(NKC, 1); else REDHIP_BSLICE_ONE(NKC, 0); \
+    } while (0)
     prof_set_stage(ST_FUSED_EXPERTS);
     switch (hidden / 512u) {
         case 1: REDHIP_BSLICE(1); break;

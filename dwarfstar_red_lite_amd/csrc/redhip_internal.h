@@ -261,14 +261,15 @@ inline bool fused_iq2_supported(uint32_t hidden, uint32_t ffn) {
 // `count` matrices, raw_stride / packed_stride bytes apart; packed = qs [nrows][K/32] uint2 then ds [nrows][K/256] fp16
 hipError_t launch_repack_iq2xxs(const void *raw, uint64_t raw_stride, uint32_t count, uint32_t nrows, uint32_t K, bool col_major,
                                 void *packed, uint64_t packed_stride, hipStream_t s);
-// gate / up matrices of IQ2_XXS, IQ2_XS or IQ1_M rows into the streams of the one-token gate/up kernel
+// gate / up matrices of IQ2_XXS, IQ2_XS or IQ1_M rows into the streams of the one-token gate/up kernel (col_major: every array
+// [group or block][row] instead of [row][group or block], the column-sliced form of a down matrix)
 hipError_t launch_repack_gateup(uint32_t type, const void *raw, uint64_t raw_stride, uint32_t count, uint32_t nrows, uint32_t K,
-                                void *packed, uint64_t packed_stride, hipStream_t s);
+                                void *packed, uint64_t packed_stride, hipStream_t s, bool col_major = false);
 // bytes of one such matrix: 8 per 32 weights + 2 per 256, IQ2_XS one more per 32
 inline uint64_t packed_matrix_bytes(uint32_t type, uint32_t nrows, uint32_t K) {
     return (uint64_t)nrows * ((uint64_t)(K / 32u) * (type == T_IQ2_XS ? 9u : 8u) + (uint64_t)(K / 256u) * 2u);
 }
-hipError_t launch_dequant_packed(uint32_t type, const void *packed, uint32_t nrows, uint32_t K, const int8_t *grid, float *out, hipStream_t s);
+hipError_t launch_dequant_packed(uint32_t type, const void *packed, uint32_t nrows, uint32_t K, const int8_t *grid, float *out, hipStream_t s, bool col_major = false);
 hipError_t launch_dequant_packed_iq2xxs(const void *packed, uint32_t nrows, uint32_t K, bool col_major, float *out, hipStream_t s);
 
 // Pair sort of caller-given routing (at most 16 tokens, 128 pairs, 1024 experts) as a side job of another launch: one extra
@@ -358,8 +359,9 @@ hipError_t launch_expert_slices(const void *experts, uint64_t stride, const void
 hipError_t launch_batch_slices(const void *experts, uint64_t stride, const void *down_cm, uint64_t down_stride, const void *shared, const void *shared_down_cm,
                                const void *pass_list, const uint32_t *n_pass, const float *weights, const float *scalar, const void *xh, const void *xl,
                                const int *xexp, float *partial, float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, hipStream_t s,
-                               const float *shared_gu = nullptr, const float *shared_dense = nullptr);
+                               const float *shared_gu = nullptr, const float *shared_dense = nullptr, uint32_t stream_type = 0u, const int8_t *grid = nullptr);
 // (with shared_gu / shared_dense: a mixed layout - gate / up packed IQ2_XXS in `experts`, down_cm column-sliced word-packed IQ3_S, the shared
-// expert as its gate | up products [ntok][2 ffn] and the dense f32 copy [hidden][ffn] of its down matrix; shared / shared_down_cm unused)
+// expert as its gate | up products [ntok][2 ffn] and the dense f32 copy [hidden][ffn] of its down matrix; shared / shared_down_cm unused.
+// With stream_type IQ2_XS / IQ1_M and the caller's codebook besides: `experts` and down_cm hold that format's streams, down_cm column-sliced)
 
 }  // namespace redhip

@@ -120,8 +120,13 @@ struct Moe {
     int *act_exp = nullptr;                  // [top_k + 1][ffn / 32]
 
     // mixed layouts whose batches of 2..8 tokens run as expert slices: gate/up packed IQ2_XXS, down IQ3_S (column-sliced words), the shared
-    // expert from its dense f32 copies, an f32 router (or the f32 copy of a quantised one) in the launch that leaves the shared gate | up products
+    // expert from its dense f32 copies, an f32 router (or the f32 copy of a quantised one) in the launch that leaves the shared gate | up products;
+    // or every routed matrix IQ2_XS, or every one IQ1_M (gate | up as row-major streams, the down streams once more column-sliced)
     bool mixed_slices = false;
+    // ... whose IQ3_S down matrices are kept column-sliced only (the one-token kernel reads that copy too)
+    bool sliced_words() const { return mixed_slices && dn_type == T_IQ3_S; }
+    // ... whose down matrices are IQ2_XS / IQ1_M streams: a column-sliced copy beside the row-major one
+    bool sliced_streams() const { return mixed_slices && dn_type != T_IQ3_S; }
     // batches that run as expert slices per pass: 2..8 tokens, at most 128 pairs
     bool small_batch(uint32_t ntok) const {
         return (fused || mixed_slices) && ntok >= 2u && ntok <= 8u && ntok * cfg.top_k <= 128u && ntok * (cfg.top_k + 1u) <= 144u && cfg.hidden / 512u <= 4u;
@@ -238,7 +243,8 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
         if (select_here || !m->shared_gu_ready) { moe_err("internal: a small batch reached the expert slices without its routing or the shared expert's products"); return 0; }
         const Layer &L = m->layers[layer];
         HIP_OK(launch_batch_slices(L.packed, m->packed_stride, L.down_cm, m->down_cm_stride(), nullptr, nullptr, m->pass_list, m->n_pass, weights, m->scalar,
-                                   m->xh, m->xl, m->xexp, m->partial, out, c.hidden, c.ffn, c.top_k, ntok, s, m->act, L.dense_down), "batched expert slice launch");
+                                   m->xh, m->xl, m->xexp, m->partial, out, c.hidden, c.ffn, c.top_k, ntok, s, m->act, L.dense_down,
+                                   m->sliced_streams() ? m->dn_type : 0u, m->sliced_streams() ? m->dn_grid : nullptr), "batched expert slice launch");
         prof_set_stage(ST_OTHER);
         return 1;
     }
@@ -347,10 +353,10 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
                                     m->weights, m->scalar, m->xh, m->xl, m->xexp, m->act_h, m->act_l, m->act_exp, c.hidden, c.ffn, c.n_expert,
                                     c.top_k, s, ntok, m->gu_type, m->gu_grid), "gate/up launch");      // ntok > 1: a small batch on a mixed layout, one grid layer per token
         prof_set_stage(ST_DOWN_COMBINE);
-        if ((L.words_down || m->mixed_slices) && L.dense_down)      // (layers whose small batches run as slices keep their IQ3_S words column-sliced only)
-            HIP_OK(launch_down_combine_words(m->dn_type, m->dn_grid, m->mixed_slices ? L.down_cm : L.words_down, m->words_down_stride(), L.dense_down,
+        if ((L.words_down || m->sliced_words()) && L.dense_down)      // (layers whose small batches run as slices keep their IQ3_S words column-sliced only)
+            HIP_OK(launch_down_combine_words(m->dn_type, m->dn_grid, m->sliced_words() ? L.down_cm : L.words_down, m->words_down_stride(), L.dense_down,
                                              select_here ? m->ids : ids, select_here ? m->weights : weights,
-                                             m->scalar, m->act_h, m->act_l, m->act_exp, out, c.hidden, c.ffn, c.top_k, s, ntok, m->mixed_slices), "down/combine launch");
+                                             m->scalar, m->act_h, m->act_l, m->act_exp, out, c.hidden, c.ffn, c.top_k, s, ntok, m->sliced_words()), "down/combine launch");
         else
             HIP_OK(launch_down_combine_raw(m->dn_type, m->sh_dn_type, L.experts + 2u * m->gate_bytes, m->expert_stride, L.shared + 2u * m->sh_gate_bytes,
                                            select_here ? m->ids : ids, select_here ? m->weights : weights, m->scalar, m->act_h, m->act_l,
@@ -431,7 +437,8 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
                (sgu != T_Q6_K || (size_t)64u * (c.hidden / 256u) * 210u + (size_t)(c.hidden + c.hidden / 32u + c.hidden / 16u) * 4u <= (gu == T_IQ1_M ? 120u : 144u) * 1024u);
     {
         const uint32_t nv = c.hidden / 256u;
-        m->mixed_slices = m->mixed && gu == T_IQ2_XXS && dn == T_IQ3_S && c.ffn <= 512u && c.hidden / 512u <= 4u && (nv == 2u || nv == 4u || nv == 8u || nv == 16u);
+        m->mixed_slices = m->mixed && ((gu == T_IQ2_XXS && dn == T_IQ3_S) || (gu_codebook && dn == gu && sgu == T_Q6_K)) && c.ffn <= 512u && c.hidden / 512u <= 4u &&
+                          (nv == 2u || nv == 4u || nv == 8u || nv == 16u);
     }
     m->pk_gate_bytes = packed_matrix_bytes(gu, c.ffn, c.hidden);
     m->packed_stride = m->fused && m->rowmajor_down() ? m->expert_stride : align256(2u * m->pk_gate_bytes);
@@ -476,7 +483,7 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
             ok = hipMalloc(reinterpret_cast<void **>(&L.down_cm), (size_t)c.n_expert * m->down_cm_stride()) == hipSuccess;
             m->resident += (uint64_t)c.n_expert * m->down_cm_stride();
         }
-        if (ok && m->mixed && !m->mixed_slices && (dn == T_IQ3_S || dn == T_IQ2_XS || dn == T_IQ1_M) && c.ffn <= 1024u) {
+        if (ok && m->mixed && !m->sliced_words() && (dn == T_IQ3_S || dn == T_IQ2_XS || dn == T_IQ1_M) && c.ffn <= 1024u) {
             ok = hipMalloc(reinterpret_cast<void **>(&L.words_down), (size_t)c.n_expert * m->words_down_stride()) == hipSuccess;
             m->resident += (uint64_t)c.n_expert * m->words_down_stride();
         }
@@ -707,9 +714,12 @@ static int stage_and_pack(Moe *m, uint32_t layer, uint32_t first, uint32_t count
             if (m->dn_type == T_IQ3_S) HIP_OK(launch_repack_iq3s_words(dst + 2u * m->gate_bytes, m->expert_stride, count, c.hidden, c.ffn, wd, m->words_down_stride(), nullptr), "expert down words");
             else HIP_OK(launch_repack_gateup(m->dn_type, dst + 2u * m->gate_bytes, m->expert_stride, count, c.hidden, c.ffn, wd, m->words_down_stride(), nullptr), "expert down streams");
         }
-        if (m->mixed_slices)
+        if (m->sliced_words())
             HIP_OK(launch_repack_iq3s_words(dst + 2u * m->gate_bytes, m->expert_stride, count, c.hidden, c.ffn, m->layers[layer].down_cm + (uint64_t)first * m->down_cm_stride(),
                                             m->down_cm_stride(), nullptr, true), "expert down column slices");
+        if (m->sliced_streams())
+            HIP_OK(launch_repack_gateup(m->dn_type, dst + 2u * m->gate_bytes, m->expert_stride, count, c.hidden, c.ffn,
+                                        m->layers[layer].down_cm + (uint64_t)first * m->down_cm_stride(), m->down_cm_stride(), nullptr, true), "expert down column slices");
         if (m->layers[layer].tiled_down)
             HIP_OK(launch_tile_iq3s(dst + 2u * m->gate_bytes, m->expert_stride, count, c.hidden, c.ffn,
                                     m->layers[layer].tiled_down + (uint64_t)first * m->tiled_down_stride(), m->tiled_down_stride(), nullptr), "expert down tiling");
@@ -950,8 +960,12 @@ int redhip_moe_dequant_resident(redhip_moe_t h, uint32_t layer, uint32_t expert,
     if (which == 3u) { HIP_OK(launch_dequant_rows(c.router_type, L.router, c.n_expert, c.hidden, out_dev, s), "router dequant"); return 1; }
     const bool sh = expert == c.n_expert;
     if (which == 4u) {                                      // the column-sliced copy of a down matrix
-        if (m->mixed_slices && !sh) {
+        if (m->sliced_words() && !sh) {
             HIP_OK(launch_dequant_iq3s_words(L.down_cm + (uint64_t)expert * m->down_cm_stride(), c.hidden, c.ffn, out_dev, s, true), "column-sliced down dequant");
+            return 1;
+        }
+        if (m->sliced_streams() && !sh) {
+            HIP_OK(launch_dequant_packed(m->dn_type, L.down_cm + (uint64_t)expert * m->down_cm_stride(), c.hidden, c.ffn, m->dn_grid, out_dev, s, true), "column-sliced down dequant");
             return 1;
         }
         if (!m->fused) { moe_err("this layout keeps no column-sliced copy of that down matrix"); return 0; }
@@ -966,7 +980,7 @@ int redhip_moe_dequant_resident(redhip_moe_t h, uint32_t layer, uint32_t expert,
         else HIP_OK(launch_dequant_packed_iq2xxs(L.down_cm + (uint64_t)expert * m->down_cm_stride(), c.hidden, c.ffn, true, out_dev, s), "column-sliced down dequant");
         return 1;
     }
-    if (which == 2u && !sh && m->mixed_slices) {
+    if (which == 2u && !sh && m->sliced_words()) {
         HIP_OK(launch_dequant_iq3s_words(L.down_cm + (uint64_t)expert * m->down_cm_stride(), c.hidden, c.ffn, out_dev, s, true), "column-sliced down dequant");
         return 1;
     }

@@ -30,10 +30,18 @@ def oracle_tokens(cfg, lay, x, ids, w):
     return out
 
 
-@pytest.mark.parametrize("layout", ["iq2", "f2"])
-def test_ragged_small_batches_hot_experts(layout):
+@pytest.mark.parametrize("layout", ["iq2", "f2", "xs", "m"])
+def test_ragged_small_batches_hot_experts(layout, golden_dir):
     """Ragged small batches: 2..8 tokens, logits N(0,1) + 2.0 on 32 hot experts, benchmark layer shape."""
+    import json
+    import os
+    from dwarfstar_red_lite_amd import moe as moe_api
     from dwarfstar_red_lite_amd.moe import ResidentMoe
+    if layout in ("xs", "m"):
+        g = json.load(open(os.path.join(golden_dir, "iq_grids.json")))
+        grids = [np.frombuffer(bytes.fromhex(g[k]), np.int8) for k in ("iq2_xs", "iq1_m")]
+        moe_api.set_codebooks(*grids)
+        orc.set_codebooks(*grids)
     cfg = synth.layer_config(layout=layout)
     lay = synth.make_layer(77, cfg)
     m = ResidentMoe(cfg, n_layer=1, max_tokens=8)
