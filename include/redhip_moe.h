@@ -136,7 +136,8 @@ int redhip_set_codebooks(const int8_t *iq2_xs_grid, uint32_t iq2_xs_count, const
 int redhip_dequant_rows(uint32_t ggml_type, const void *rows_dev, uint32_t nrows, uint32_t ncols, float *out_dev, void *stream);
 /* Parity tap: dequantise one resident matrix (which: 0 gate, 1 up, 2 down; expert == n_expert: shared expert;
  * which == 3: the router; which == 4: the down matrix from the column-sliced copy that the expert-slice kernels read - all-IQ2_XXS
- * layers, and the routed experts of layers with IQ2_XXS gate/up and IQ3_S down matrices) from the layout the kernels read.
+ * layers, and the routed experts of layers with IQ2_XXS gate/up and IQ3_S down matrices or with every routed matrix IQ2_XS or IQ1_M)
+ * from the layout the kernels read.
  * out_dev holds rows x cols floats. */
 int redhip_moe_dequant_resident(redhip_moe_t moe, uint32_t layer, uint32_t expert, uint32_t which, float *out_dev, void *stream);
 
