@@ -45,7 +45,9 @@ def parse():
     ap.add_argument("--no-micro", action="store_true", help="skip the single-GEMV microbench (only run for --layout iq2 --batch 1)")
     ap.add_argument("--no-graph", action="store_true", help="launch eagerly instead of replaying a HIP graph")
     ap.add_argument("--calibrate", action="store_true", help="also run the plain copy kernel of known size (for rocprofv3 --pmc runs)")
-    ap.add_argument("--f2-layers", type=int, default=48, help="layers of the F2 handle that the default run's sweep adds (0: leave the F2 sweep out)")
+    ap.add_argument("--f2-layers", type=int, default=48, help="layers of the handles of the other layouts that the default run's sweep adds (0: leave those sweeps out)")
+    ap.add_argument("--sweep-layouts", default="f2,xs,m", help="layouts the default run adds a sweep for on handles of their own (one token through the layer's "
+                                                               "own router, then B=2/4/8 with hot routing); key <layout>_sweep of the result")
     ap.add_argument("--no-sweep", action="store_true", help="skip the B=2/4/8 hot-routing sweep that the default (B=1, own router) run appends")
     ap.add_argument("--prime", type=int, default=2000, help="untimed steps before the warm-up that bring the clocks up (reported as clock_priming_steps)")
     return ap.parse_args()
@@ -211,7 +213,8 @@ def main():
     torch.cuda.init()
     B, NL = args.batch, args.layers
     K, W = args.steps, args.warmup
-    if args.layout in ("xs", "m"):          # these two decode through codebooks the caller supplies: the reference's, from the fixture
+    if args.layout in ("xs", "m") or "xs" in args.sweep_layouts.split(",") or "m" in args.sweep_layouts.split(","):
+        # these two decode through codebooks the caller supplies: the reference's, from the fixture
         from dwarfstar_red_lite_amd import moe as moe_api
         g = json.load(open(os.path.join(ROOT, "tests", "golden", "iq_grids.json")))
         grids = [np.frombuffer(bytes.fromhex(g[k]), np.int8) for k in ("iq2_xs", "iq1_m")]
@@ -219,6 +222,10 @@ def main():
         orc.set_codebooks(*grids)
     # the default run (one token, the layer's own router) appends the small-batch sweep on the same resident handle
     sweep = [] if (args.no_sweep or B != 1 or args.routing != "router") else [2, 4, 8]
+    sweep_layouts = [l for l in args.sweep_layouts.split(",") if l] if (sweep and args.layout == "iq2" and args.f2_layers > 0) else []
+    for l in sweep_layouts:
+        if l not in ("f2", "xs", "m"):
+            raise SystemExit("bench.py: unknown layout %r in --sweep-layouts" % l)
     gen = torch.Generator(device="cuda")
     gen.manual_seed(20241125)
     stream = torch.cuda.Stream()
@@ -392,14 +399,16 @@ def main():
 
     if sweep:
         result["batch_sweep"] = [sweep_entry(main_ctx, b, "hot") for b in sweep]
-        # ---- the mixed-precision layout of the target files (config 2) on a handle of its own: one token with the layer's own router, then
-        # the same ragged batches; all 48 layers resident like the headline handle ----
-        if args.layout == "iq2" and args.f2_layers > 0:
-            f2 = resident_handle("f2", args.f2_layers, max(sweep))
-            result["f2_sweep"] = {"resident_layers": args.f2_layers, "resident_gb": round(f2["moe"].resident_bytes / 1e9, 2),
-                                  "runs": [sweep_entry(f2, 1, "router")] + [sweep_entry(f2, b, "hot") for b in sweep]}
-            f2["moe"].close()
-            del f2
+        # ---- the other layouts, each on a handle of its own: the mixed-precision layout of config 2 (f2) and the layouts with the expert
+        # formats of the reference's target file (xs: IQ2_XS, m: IQ1_M experts). One token with the layer's own router, then the same ragged
+        # batches; all 48 layers resident like the headline handle ----
+        for lay in sweep_layouts:
+            ctx = resident_handle(lay, args.f2_layers, max(sweep))
+            result[lay + "_sweep"] = {"resident_layers": args.f2_layers, "resident_gb": round(ctx["moe"].resident_bytes / 1e9, 2),
+                                      "runs": [sweep_entry(ctx, 1, "router")] + [sweep_entry(ctx, b, "hot") for b in sweep]}
+            ctx["moe"].close()
+            del ctx
+            torch.cuda.empty_cache()
 
     # ---- per-kernel microbench of config 1: one IQ2_XXS dequant-GEMV [512 x 2048] x [2048] on raw GGUF rows ----
     if args.layout == "iq2" and B == 1 and not args.no_micro:
