@@ -162,7 +162,7 @@ inline uint32_t prefill_tile_bound(uint32_t ntok, uint32_t top_k, uint32_t n_exp
 // tiled_experts / tiled_shared: optional tile-major copies (launch_tile_packed) of the same matrices, same stride and offsets; with
 // them and ffn <= 512 the kernels that keep a tile's activations in registers run.
 hipError_t launch_tile_packed(const void *packed, uint64_t packed_stride, uint32_t count, uint32_t nrows, uint32_t K, void *tiled, uint64_t tiled_stride,
-                              hipStream_t s);
+                              hipStream_t s, bool with_sc = false);
 // routed gate/up + SwiGLU of a chunk on the tile-major copy of packed IQ2_XXS gate/up matrices (mixed layouts); act: f32 [pairs][ffn], or
 // nullptr for fp16 halves + two exponents per pair in act_h / act_l / act_exp
 hipError_t launch_prefill_gateup_tiled(const void *tiled_experts, uint64_t stride, const uint32_t *uid, const uint32_t *expert_start,

@@ -42,7 +42,7 @@ struct Layer {
     // mixed layouts that take chunks: f32 copies of the small dense matrices (dequantised once at upload) for the fp32 tile
     // kernel: router [n_expert][hidden] (when it is quantised), shared gate | up [2 ffn][hidden], shared down [hidden][ffn]
     float *dense_router = nullptr, *dense_gu = nullptr, *dense_down = nullptr;
-    uint8_t *tiled_down = nullptr;   // mixed layouts with IQ3_S down matrices that take chunks: their tile-major copy
+    uint8_t *tiled_down = nullptr;   // mixed layouts with IQ3_S, IQ2_XS or IQ1_M down matrices that take chunks on tile kernels: their tile-major copy
     uint8_t *words_down = nullptr;   // mixed layouts with IQ3_S / IQ2_XS / IQ1_M down matrices, row-major words or streams for the MFMA down kernels of up to 8 tokens (layers with a column-sliced IQ3_S copy read that one instead)
 };
 
@@ -151,9 +151,11 @@ struct Moe {
     }
     // a chunk on a layout whose experts are IQ2_XS / IQ1_M: the tile kernels on the row-major streams of the routed matrices, the shared
     // expert and the router as dense f32 products
-    bool stream_chunk(uint32_t ntok) const {
+    bool stream_chunk(uint32_t ntok) const { return ntok > 8u && stream_tiles_resident(); }
+    // ... such a handle keeps tile-major copies of the gate | up streams (`tiled`) and of the down streams (`tiled_down`)
+    bool stream_tiles_resident() const {
         const bool gu_cb = gu_type == T_IQ2_XS || gu_type == T_IQ1_M, dn_cb = dn_type == T_IQ2_XS || dn_type == T_IQ1_M;
-        return mixed && ntok > 8u && gu_cb && dn_cb && (cfg.ffn == 256u || cfg.ffn == 512u) && cfg.hidden / 512u <= 4u && cfg.max_tokens > 8u;
+        return mixed && gu_cb && dn_cb && (cfg.ffn == 256u || cfg.ffn == 512u) && cfg.hidden / 512u <= 4u && cfg.max_tokens > 8u;
     }
     // a chunk on a mixed layout that has no tile kernels (ffn > 512, or IQ2_XS / IQ1_M gate/up beside another down format) runs as slices
     // of 8 tokens on the grouped small-batch kernels, far ahead of the generic per-pair kernels on raw rows
@@ -266,7 +268,7 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
         const uint32_t P = ntok * c.top_k, n_groups = P < c.n_expert ? P : c.n_expert;
         const ExpertSet ex = m->routed(layer), sh = m->shared(layer);
         const Layer &Ld = m->layers[layer];
-        const bool stream_tiles = m->stream_chunk(ntok) && Ld.words_down && Ld.dense_gu && m->side;
+        const bool stream_tiles = m->stream_chunk(ntok) && Ld.tiled && Ld.tiled_down && Ld.dense_gu && m->side;
         // the shared expert as dense f32 products on the fp32 matrix units, started before the pair sort (one workgroup on an idle machine)
         const bool dense_shared = (stream_tiles || (m->mixed_chunk(ntok) && Ld.dense_gu && m->side));
         if (dense_shared && !fork_shared_dense(m, Ld, x, ntok, s)) return 0;
@@ -300,7 +302,7 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
         if (stream_tiles) {
             const Layer &L = Ld;
             prof_set_stage(ST_BATCH_GATEUP);
-            HIP_OK(launch_prefill_streams(m->gu_type, m->gu_grid, L.packed, m->packed_stride, m->dn_type, m->dn_grid, L.words_down, m->words_down_stride(), m->uid,
+            HIP_OK(launch_prefill_streams(m->gu_type, m->gu_grid, L.tiled, m->packed_stride, m->dn_type, m->dn_grid, L.tiled_down, m->words_down_stride(), m->uid,
                                           m->expert_start, m->pair_token, m->n_unique, m->tile_group, m->tile_pair0, m->tile_n, m->n_tiles, m->xh, m->xl, m->xexp,
                                           m->act_h, m->act_l, m->act_exp, m->tmp, c.hidden, c.ffn, c.top_k, ntok, c.n_expert, s, tiles_built), "stream tile launch");
             if (!join_shared_dense(m, s)) return 0;
@@ -490,6 +492,11 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
         if (ok && m->mixed && m->tiles_resident() && dn == T_IQ3_S) {
             ok = hipMalloc(reinterpret_cast<void **>(&L.tiled_down), (size_t)c.n_expert * m->tiled_down_stride()) == hipSuccess;
             m->resident += (uint64_t)c.n_expert * m->tiled_down_stride();
+        }
+        if (ok && m->stream_tiles_resident()) {
+            ok = hipMalloc(reinterpret_cast<void **>(&L.tiled), (size_t)c.n_expert * m->tiled_stride()) == hipSuccess &&
+                 hipMalloc(reinterpret_cast<void **>(&L.tiled_down), (size_t)c.n_expert * m->words_down_stride()) == hipSuccess;
+            m->resident += (uint64_t)c.n_expert * (m->tiled_stride() + m->words_down_stride());
         }
         if (ok && m->tiles_resident()) {
             ok = hipMalloc(reinterpret_cast<void **>(&L.tiled), (size_t)c.n_expert * m->tiled_stride()) == hipSuccess &&
@@ -704,8 +711,9 @@ static int stage_and_pack(Moe *m, uint32_t layer, uint32_t first, uint32_t count
         if (m->layers[layer].tiled) {      // (the tile-major copy keeps the gate | up | down slots of the raw layout)
             const uint64_t tstride = m->tiled_stride();
             uint8_t *tl = m->layers[layer].tiled + (uint64_t)first * tstride;
-            HIP_OK(launch_tile_packed(pk, m->packed_stride, count, c.ffn, c.hidden, tl, tstride, nullptr), "expert gate tiling");
-            HIP_OK(launch_tile_packed(pk + m->gate_bytes, m->packed_stride, count, c.ffn, c.hidden, tl + m->gate_bytes, tstride, nullptr), "expert up tiling");
+            const bool gu_sc = m->gu_type == T_IQ2_XS;          // its streams carry a scale byte per group
+            HIP_OK(launch_tile_packed(pk, m->packed_stride, count, c.ffn, c.hidden, tl, tstride, nullptr, gu_sc), "expert gate tiling");
+            HIP_OK(launch_tile_packed(pk + m->pk_gate_bytes, m->packed_stride, count, c.ffn, c.hidden, tl + m->pk_gate_bytes, tstride, nullptr, gu_sc), "expert up tiling");
             if (m->fused)
                 HIP_OK(launch_tile_packed(pk_down, pk_down_stride, count, c.hidden, c.ffn, tl + 2u * m->gate_bytes, tstride, nullptr), "expert down tiling");
         }
@@ -720,9 +728,15 @@ static int stage_and_pack(Moe *m, uint32_t layer, uint32_t first, uint32_t count
         if (m->sliced_streams())
             HIP_OK(launch_repack_gateup(m->dn_type, dst + 2u * m->gate_bytes, m->expert_stride, count, c.hidden, c.ffn,
                                         m->layers[layer].down_cm + (uint64_t)first * m->down_cm_stride(), m->down_cm_stride(), nullptr, true), "expert down column slices");
-        if (m->layers[layer].tiled_down)
+        if (m->layers[layer].tiled_down && m->dn_type == T_IQ3_S)
             HIP_OK(launch_tile_iq3s(dst + 2u * m->gate_bytes, m->expert_stride, count, c.hidden, c.ffn,
                                     m->layers[layer].tiled_down + (uint64_t)first * m->tiled_down_stride(), m->tiled_down_stride(), nullptr), "expert down tiling");
+        if (m->layers[layer].tiled_down && m->dn_type != T_IQ3_S) {      // IQ2_XS / IQ1_M: the tile-major copy of the row-major streams written above
+            if (!m->layers[layer].words_down) { moe_err("internal: no row-major down streams to tile"); return 0; }
+            HIP_OK(launch_tile_packed(m->layers[layer].words_down + (uint64_t)first * m->words_down_stride(), m->words_down_stride(), count, c.hidden, c.ffn,
+                                      m->layers[layer].tiled_down + (uint64_t)first * m->words_down_stride(), m->words_down_stride(), nullptr, m->dn_type == T_IQ2_XS),
+                   "expert down tiling");
+        }
         HIP_OK(hipStreamSynchronize(nullptr), "expert repack");
     }
     return 1;

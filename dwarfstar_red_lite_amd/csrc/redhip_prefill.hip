@@ -302,8 +302,9 @@ constexpr uint32_t kItemUnits = 4u, kExpPerPair = 4u;
 constexpr uint32_t kScaledMagBytes = 16u * 256u * 16u;      // [group scale s][grid entry]
 constexpr uint32_t kSignBytes = 128u * 16u;                 // [seven sign bits] (the eighth sign is their parity)
 
-// row-major packed matrix -> tile-major copy; one thread per 32-byte chunk, the scales ride along
-__global__ void tile_packed_kernel(const uint8_t *packed, uint64_t packed_stride, uint32_t nrows, uint32_t K, uint8_t *tiled, uint64_t tiled_stride) {
+// row-major packed matrix -> tile-major copy; one thread per 32-byte chunk, the scales ride along (with_sc: an IQ2_XS stream, whose scale
+// bytes [row][group] follow qs and ds; the four of a chunk become one 32-bit word at (tile, chunk, row) like the chunk itself)
+__global__ void tile_packed_kernel(const uint8_t *packed, uint64_t packed_stride, uint32_t nrows, uint32_t K, uint8_t *tiled, uint64_t tiled_stride, int with_sc) {
     const uint32_t NC = K / 128u, NB = K / 256u;
     const uint64_t gid = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
     if (gid >= (uint64_t)nrows * NC) return;
@@ -320,14 +321,19 @@ __global__ void tile_packed_kernel(const uint8_t *packed, uint64_t packed_stride
         reinterpret_cast<uint16_t *>(dst + qs_bytes)[((uint64_t)(row / 16u) * NB + b) * 16u + row % 16u] =
             reinterpret_cast<const uint16_t *>(src + qs_bytes)[(uint64_t)row * NB + b];
     }
+    if (with_sc) {
+        const uint64_t sc_off = qs_bytes + (uint64_t)nrows * NB * 2u;
+        reinterpret_cast<uint32_t *>(dst + sc_off)[((uint64_t)(row / 16u) * NC + c) * 16u + row % 16u] =
+            *reinterpret_cast<const uint32_t *>(src + sc_off + (uint64_t)row * (K / 32u) + 4u * c);
+    }
 }
 
 hipError_t launch_tile_packed(const void *packed, uint64_t packed_stride, uint32_t count, uint32_t nrows, uint32_t K, void *tiled, uint64_t tiled_stride,
-                              hipStream_t s) {
+                              hipStream_t s, bool with_sc) {
     if (!nrows || nrows % 16u || !K || K % 256u || !count || count > 65535u) return hipErrorInvalidValue;
     const uint64_t total = (uint64_t)nrows * (K / 128u);
     REDHIP_LAUNCH(tile_packed_kernel, dim3((uint32_t)((total + 255u) / 256u), count), dim3(256), 0, s, static_cast<const uint8_t *>(packed), packed_stride,
-                  nrows, K, static_cast<uint8_t *>(tiled), tiled_stride);
+                  nrows, K, static_cast<uint8_t *>(tiled), tiled_stride, with_sc ? 1 : 0);
     return hipGetLastError();
 }
 
@@ -373,8 +379,9 @@ struct TiledArgs {
     uint64_t down_off;                    // down kernel, FMT 1 / 2: offset of the down matrix inside an expert's slot
 };
 
-// The same kernels serve IQ2_XS (FMT 1) and IQ1_M (FMT 2) matrices, read from their row-major streams (uint2 per 32 weights, d per 256,
-// IQ2_XS a scale byte per 32) - 16 rows x 32 bytes per wave-wide load instead of 512 contiguous bytes. Their codebooks are too large to
+// The same kernels serve IQ2_XS (FMT 1) and IQ1_M (FMT 2) matrices, read from tile-major copies of their streams (uint2 per 32 weights, d
+// per 256, IQ2_XS a scale byte per 32, laid out as tile_packed_kernel writes them: a wave-wide load is 512 contiguous bytes; from the
+// row-major streams, 16 rows x 32 bytes per load, the IQ2_XS down kernel took 140 us per chunk of 512 tokens). Their codebooks are too large to
 // be multiplied out with every group scale, so the table holds the plain fp16 entries (8 KB / 32 KB) and the scale (per 16 weights) is
 // applied to the eight weights by packed fp16 multiplies, exact: IQ2_XS entry * (2 s + 1) <= 43 * 31, IQ1_M (entry +- 1/8) * (2 s + 1)
 // in eighths <= 135. The d/8 of IQ2_XS stays in the activation scale, IQ1_M has none.
@@ -512,16 +519,10 @@ __device__ __forceinline__ void gateup_narrow_items(const TiledArgs &ta, uint32_
     };
     auto load_chunk = [&](const uint8_t *mat, uint32_t j, uint32_t c) {
         const uint32_t rtile = 2u * j + rh, chunk = kc * NKC + c;
-        if constexpr (FMT == 0) {
-            const uint4 *qp = reinterpret_cast<const uint4 *>(mat + (((uint64_t)rtile * NC + chunk) * 16u + r) * 32u);
-            const uint16_t *dp = reinterpret_cast<const uint16_t *>(mat + qs_bytes) + ((uint64_t)rtile * HB + chunk / 2u) * 16u + r;
-            return RowChunk{qp[0], qp[1], *dp, 0u};
-        } else {
-            const uint64_t row = 16u * rtile + r;
-            const uint4 *qp = reinterpret_cast<const uint4 *>(mat + (row * HG + 4u * chunk) * 8u);
-            const uint32_t d = reinterpret_cast<const uint16_t *>(mat + qs_bytes)[row * HB + chunk / 2u];
-            return RowChunk{qp[0], qp[1], d, FMT == 1 ? *reinterpret_cast<const uint32_t *>(mat + sc_off + row * HG + 4u * chunk) : 0u};
-        }
+        const uint64_t at = ((uint64_t)rtile * NC + chunk) * 16u + r;
+        const uint4 *qp = reinterpret_cast<const uint4 *>(mat + at * 32u);
+        const uint16_t *dp = reinterpret_cast<const uint16_t *>(mat + qs_bytes) + ((uint64_t)rtile * HB + chunk / 2u) * 16u + r;
+        return RowChunk{qp[0], qp[1], *dp, FMT == 1 ? reinterpret_cast<const uint32_t *>(mat + sc_off)[at] : 0u};
     };
     if (item_begin >= item_end) return;
     ItemInfo cur = info_of(item_begin);
@@ -716,16 +717,10 @@ __device__ __forceinline__ void gateup_wide_items(const TiledArgs &ta, uint32_t 
         constexpr uint32_t kHalfSteps = FGH * 2u;
         auto load_chunk = [&](const uint8_t *mat, uint32_t hs, uint32_t c) {
             const uint32_t rtile = 2u * j0 + hs, chunk = kc * CW + c;      // (2 (j0 + hs / 2) + hs % 2)
-            if constexpr (FMT == 0) {
-                const uint4 *qp = reinterpret_cast<const uint4 *>(mat + (((uint64_t)rtile * NC + chunk) * 16u + r) * 32u);
-                const uint16_t *dp = reinterpret_cast<const uint16_t *>(mat + qs_bytes) + ((uint64_t)rtile * HB + chunk / 2u) * 16u + r;
-                return RowChunk{qp[0], qp[1], *dp, 0u};
-            } else {
-                const uint64_t row = 16u * rtile + r;
-                const uint4 *qp = reinterpret_cast<const uint4 *>(mat + (row * HG + 4u * chunk) * 8u);
-                const uint32_t d = reinterpret_cast<const uint16_t *>(mat + qs_bytes)[row * HB + chunk / 2u];
-                return RowChunk{qp[0], qp[1], d, FMT == 1 ? *reinterpret_cast<const uint32_t *>(mat + sc_off + row * HG + 4u * chunk) : 0u};
-            }
+            const uint64_t at = ((uint64_t)rtile * NC + chunk) * 16u + r;
+            const uint4 *qp = reinterpret_cast<const uint4 *>(mat + at * 32u);
+            const uint16_t *dp = reinterpret_cast<const uint16_t *>(mat + qs_bytes) + ((uint64_t)rtile * HB + chunk / 2u) * 16u + r;
+            return RowChunk{qp[0], qp[1], *dp, FMT == 1 ? reinterpret_cast<const uint32_t *>(mat + sc_off)[at] : 0u};
         };
         const uint8_t *gmat = ex, *umat = ex + gate_bytes;
         RowChunk cg = load_chunk(gmat, 0u, 0u), cu = load_chunk(umat, 0u, 0u);
@@ -894,16 +889,10 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_down_reg_kernel(TiledA
         }
         auto load_chunk = [&](uint32_t b, uint32_t c) {
             const uint32_t rtile = kRegWaves * (pass0 + b) + wave;
-            if constexpr (FMT == 0) {
-                const uint4 *qp = reinterpret_cast<const uint4 *>(dn + (((uint64_t)rtile * NCK + c) * 16u + r) * 32u);
-                const uint16_t *dp = reinterpret_cast<const uint16_t *>(dn + qs_bytes) + ((uint64_t)rtile * FB + c / 2u) * 16u + r;
-                return RowChunk{qp[0], qp[1], *dp, 0u};
-            } else {
-                const uint64_t row = 16u * rtile + r;
-                const uint4 *qp = reinterpret_cast<const uint4 *>(dn + (row * NFG + 4u * c) * 8u);
-                const uint32_t d = reinterpret_cast<const uint16_t *>(dn + qs_bytes)[row * FB + c / 2u];
-                return RowChunk{qp[0], qp[1], d, FMT == 1 ? *reinterpret_cast<const uint32_t *>(dn + sc_off + row * NFG + 4u * c) : 0u};
-            }
+            const uint64_t at = ((uint64_t)rtile * NCK + c) * 16u + r;
+            const uint4 *qp = reinterpret_cast<const uint4 *>(dn + at * 32u);
+            const uint16_t *dp = reinterpret_cast<const uint16_t *>(dn + qs_bytes) + ((uint64_t)rtile * FB + c / 2u) * 16u + r;
+            return RowChunk{qp[0], qp[1], *dp, FMT == 1 ? reinterpret_cast<const uint32_t *>(dn + sc_off)[at] : 0u};
         };
         // One buffer per chunk of a pass, reloaded with the same chunk of the next pass as soon as it has been decoded: every load
         // has a whole pass of work to arrive.
