@@ -386,7 +386,12 @@ struct TiledArgs {
 // applied to the eight weights by packed fp16 multiplies, exact: IQ2_XS entry * (2 s + 1) <= 43 * 31, IQ1_M (entry +- 1/8) * (2 s + 1)
 // in eighths <= 135. The d/8 of IQ2_XS stays in the activation scale, IQ1_M has none.
 typedef _Float16 half2_t __attribute__((ext_vector_type(2)));
-template <int FMT> constexpr uint32_t reg_table_bytes() { return FMT == 0 ? kSignBytes + kScaledMagBytes : FMT == 1 ? kSignBytes + 512u * 16u : 2048u * 16u; }
+// (FMT 3: IQ2_XS streams like FMT 1, decoded through a table of the codebook multiplied out with the sixteen odd scales, 128 KB: for
+// kernels that have the LDS to spare, it saves the four packed multiplies per eight weights)
+constexpr uint32_t kScaledXsBytes = 16u * 512u * 16u;       // [scale nibble][codebook entry]
+template <int FMT> constexpr uint32_t reg_table_bytes() {
+    return FMT == 0 ? kSignBytes + kScaledMagBytes : FMT == 1 ? kSignBytes + 512u * 16u : FMT == 3 ? kSignBytes + kScaledXsBytes : 2048u * 16u;
+}
 
 __device__ __forceinline__ void build_sign_table(uint8_t *sgn, uint32_t tid, uint32_t nthreads) {
     for (uint32_t s7 = tid; s7 < 128u; s7 += nthreads) {
@@ -405,6 +410,19 @@ __device__ __forceinline__ void build_reg_tables(uint8_t *tables, uint32_t tid, 
     } else if constexpr (FMT == 1) {
         build_sign_table(tables, tid, nthreads);
         build_codebook_table<1>(tables + kSignBytes, tid, grid, 0u, nthreads);
+    } else if constexpr (FMT == 3) {
+        build_sign_table(tables, tid, nthreads);
+        for (uint32_t e = tid; e < 16u * 512u; e += nthreads) {      // entries are at most 43, scales at most 31: exact in fp16
+            const uint64_t ge = reinterpret_cast<const uint64_t *>(grid)[e & 511u];
+            const float f = (float)(2u * (e >> 9) + 1u);
+            uint32_t w4[4];
+#pragma unroll
+            for (int i = 0; i < 4; ++i) {
+                const _Float16 lo = (_Float16)(f * (float)(int8_t)(ge >> (16 * i))), hi = (_Float16)(f * (float)(int8_t)(ge >> (16 * i + 8)));
+                w4[i] = (uint32_t)__builtin_bit_cast(uint16_t, lo) | ((uint32_t)__builtin_bit_cast(uint16_t, hi) << 16);
+            }
+            *reinterpret_cast<uint4 *>(tables + kSignBytes + (size_t)e * 16u) = make_uint4(w4[0], w4[1], w4[2], w4[3]);
+        }
     } else {
         build_codebook_table<2>(tables, tid, grid, 0u, nthreads);
     }
@@ -468,6 +486,14 @@ __device__ __forceinline__ half8_t decode_reg(uint2 w, uint32_t sc, uint32_t q, 
         Half8 r;
         r.u = make_uint4(__builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, m.x ^ g.x) * f), __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, m.y ^ g.y) * f),
                          __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, m.z ^ g.z) * f), __builtin_bit_cast(uint32_t, __builtin_bit_cast(half2_t, m.w ^ g.w) * f));
+        return r.v;
+    } else if constexpr (FMT == 3) {
+        const uint32_t w16 = (((q & 2u) ? w.y : w.x) >> (16u * (q & 1u))) & 0xffffu;
+        const uint32_t nib = (sc >> (4u * (q >> 1))) & 15u;
+        const uint4 m = *reinterpret_cast<const uint4 *>(tables + kSignBytes + (((nib << 9) | (w16 & 511u)) << 4));
+        const uint4 g = *reinterpret_cast<const uint4 *>(tables + ((w16 >> 9) << 4));
+        Half8 r;
+        r.u = make_uint4(m.x ^ g.x, m.y ^ g.y, m.z ^ g.z, m.w ^ g.w);
         return r.v;
     } else {
         const uint32_t idx = ((w.x >> (8u * q)) & 255u) | (((w.y >> (4u * q)) & 7u) << 8);
@@ -892,7 +918,7 @@ __global__ __launch_bounds__(kRegWaves * 64) void prefill_down_reg_kernel(TiledA
             const uint64_t at = ((uint64_t)rtile * NCK + c) * 16u + r;
             const uint4 *qp = reinterpret_cast<const uint4 *>(dn + at * 32u);
             const uint16_t *dp = reinterpret_cast<const uint16_t *>(dn + qs_bytes) + ((uint64_t)rtile * FB + c / 2u) * 16u + r;
-            return RowChunk{qp[0], qp[1], *dp, FMT == 1 ? reinterpret_cast<const uint32_t *>(dn + sc_off)[at] : 0u};
+            return RowChunk{qp[0], qp[1], *dp, FMT == 1 || FMT == 3 ? reinterpret_cast<const uint32_t *>(dn + sc_off)[at] : 0u};
         };
         // One buffer per chunk of a pass, reloaded with the same chunk of the next pass as soon as it has been decoded: every load
         // has a whole pass of work to arrive.
@@ -1383,10 +1409,10 @@ hipError_t launch_prefill_streams(uint32_t gate_up_type, const int8_t *gate_up_g
     const TiledArgs td{a, static_cast<const uint8_t *>(down), nullptr, nullptr, down_grid, 0u};
     prof_set_stage(ST_PREFILL_DOWN);
     if (ffn == 256u) {
-        if (fd == 1u) REDHIP_LAUNCH((prefill_down_reg_kernel<8, 1>), grid, rblock, 0, s, td);
+        if (fd == 1u) REDHIP_LAUNCH((prefill_down_reg_kernel<8, 3>), grid, rblock, 0, s, td);      // (IQ2_XS: the scale-folded table, 130 KB of LDS)
         else REDHIP_LAUNCH((prefill_down_reg_kernel<8, 2>), grid, rblock, 0, s, td);
     } else {
-        if (fd == 1u) REDHIP_LAUNCH((prefill_down_reg_kernel<16, 1>), grid, rblock, 0, s, td);
+        if (fd == 1u) REDHIP_LAUNCH((prefill_down_reg_kernel<16, 3>), grid, rblock, 0, s, td);
         else REDHIP_LAUNCH((prefill_down_reg_kernel<16, 2>), grid, rblock, 0, s, td);
     }
     return hipGetLastError();
