@@ -1865,30 +1865,31 @@ __global__ __launch_bounds__(kWaves * 64, 8) void batch_slice_kernel(BatchSliceA
                 part[tid] = (gv / (1.0f + expf(-gv))) * uv;
             }
             __syncthreads();
-            // a lane pair per output row, each lane 16 of the 32 columns for both tokens: its 32 activations stay in registers
-            const uint32_t half = tid & 1u;
-            float4 av[4], bv[4];
-#pragma unroll
-            for (int i = 0; i < 4; ++i) {
-                av[i] = *reinterpret_cast<const float4 *>(part + 16u * half + 4 * i);
-                bv[i] = *reinterpret_cast<const float4 *>(part + 32u + 16u * half + 4 * i);
-            }
+            // Eight lanes per output row, each lane four of the 32 columns for both tokens: a wave-wide load reads the 128-byte slices of
+            // eight consecutive rows whole (a lane pair per row, 16 columns each, touched 32 cache lines per load instruction)
+            const uint32_t sub = tid & 7u;
+            const float4 av = *reinterpret_cast<const float4 *>(part + 4u * sub), bv = *reinterpret_cast<const float4 *>(part + 32u + 4u * sub);
             const float s0 = a.scalar[tok0], s1 = a.scalar[tok1];
-            for (uint32_t h = tid >> 1; h < H; h += (uint32_t)NW * 32u) {
-                const float4 *wr = reinterpret_cast<const float4 *>(a.shared_dense + (uint64_t)h * F + 32u * g + 16u * half);
+            constexpr uint32_t kRows = (uint32_t)NW * 8u;      // rows per round of the workgroup
+            for (uint32_t h0 = tid >> 3; h0 < H; h0 += 4u * kRows) {      // four rounds' loads in flight
                 float4 w4[4];
 #pragma unroll
-                for (int i = 0; i < 4; ++i) w4[i] = wr[i];
-                float acc0 = 0.0f, acc1 = 0.0f;
-#pragma unroll
-                for (int i = 0; i < 4; ++i) {
-                    acc0 = fmaf(w4[i].w, av[i].w, fmaf(w4[i].z, av[i].z, fmaf(w4[i].y, av[i].y, fmaf(w4[i].x, av[i].x, acc0))));
-                    acc1 = fmaf(w4[i].w, bv[i].w, fmaf(w4[i].z, bv[i].z, fmaf(w4[i].y, bv[i].y, fmaf(w4[i].x, bv[i].x, acc1))));
+                for (uint32_t i = 0; i < 4u; ++i) {
+                    const uint32_t h = h0 + i * kRows;
+                    w4[i] = *reinterpret_cast<const float4 *>(a.shared_dense + (uint64_t)(h < H ? h : h0) * F + 32u * g + 4u * sub);
                 }
-                acc0 += __shfl_xor(acc0, 1, 64);
-                acc1 += __shfl_xor(acc1, 1, 64);
-                if (half == 0u) out0[h] = acc0 * s0;
-                else if (cnt > 1u) out1[h] = acc1 * s1;
+#pragma unroll
+                for (uint32_t i = 0; i < 4u; ++i) {
+                    const uint32_t h = h0 + i * kRows;
+                    float acc0 = fmaf(w4[i].w, av.w, fmaf(w4[i].z, av.z, fmaf(w4[i].y, av.y, w4[i].x * av.x)));
+                    float acc1 = fmaf(w4[i].w, bv.w, fmaf(w4[i].z, bv.z, fmaf(w4[i].y, bv.y, w4[i].x * bv.x)));
+#pragma unroll
+                    for (int o = 1; o < 8; o <<= 1) { acc0 += __shfl_xor(acc0, o, 64); acc1 += __shfl_xor(acc1, o, 64); }
+                    if (h < H) {
+                        if (sub == 0u) out0[h] = acc0 * s0;
+                        else if (sub == 1u && cnt > 1u) out1[h] = acc1 * s1;
+                    }
+                }
             }
             return;
         }
