@@ -823,6 +823,104 @@ __global__ __launch_bounds__(1024) void group_pairs_kernel(const uint32_t *ids, 
     if (tiles.tile_group) build_tile_lists(U, tid < U ? start[tid] : 0u, tid < U ? start[tid + 1u] - start[tid] : 0u, P, tiles, tile_tot);
 }
 
+// The same sort for chunks of more than 512 tokens, whose token bitmaps per expert would not fit the LDS (2048 tokens x 512 experts: 128
+// KB, and as much again for the prefix counts - without them a pair's rank is a loop over up to 64 words, 300 us per chunk): the first
+// appearances and the pair counts of the experts come from one pass over all pairs, then the pairs are placed block by block of 512
+// tokens - bitmaps and prefix counts of one block (32 KB each), a cursor per expert that advances by the block's count. Same outputs in
+// the same (stable) order; one workgroup, the time grows with the number of blocks.
+constexpr uint32_t kGroupBlockTokens = 512u, kGroupBlockWords = kGroupBlockTokens / 32u;
+__global__ __launch_bounds__(1024) void group_pairs_blocked_kernel(const uint32_t *ids, const float *weights, uint32_t ntok, uint32_t top_k, uint32_t top_k_magic,
+                                                                   uint32_t n_expert, uint32_t *uid, uint32_t *expert_start,
+                                                                   uint32_t *pair_token, float *pair_weight, uint32_t *tok_pair,
+                                                                   uint32_t *n_unique, uint32_t *status, uint32_t cache_ids, TileLists tiles) {
+    extern __shared__ uint32_t sm[];
+    __shared__ uint32_t tile_tot[3][16];
+    constexpr uint32_t WB = kGroupBlockWords;
+    const uint32_t P = ntok * top_k, tid = threadIdx.x;
+    uint32_t *first = sm;                          // [n_expert]
+    uint32_t *count = first + n_expert;            // [n_expert]
+    uint32_t *dense = count + n_expert;            // [n_expert]
+    uint32_t *cursor = dense + n_expert;           // [n_expert] pairs of the expert placed by the blocks before
+    uint32_t *start = cursor + n_expert;           // [n_expert + 1] by dense index
+    uint32_t *uid_l = start + n_expert + 1u;       // [1024]
+    uint32_t *wave_tot = uid_l + 1024u;            // [17]
+    uint32_t *member = wave_tot + 17u;             // [n_expert][WB] tokens of the block that selected the expert
+    uint32_t *below = member + n_expert * WB;      // [n_expert][WB] members in the words before this one
+    uint32_t *ids_l = cache_ids ? below + n_expert * WB : nullptr;      // [P] the clamped ids
+    auto token_of = [&](uint32_t p) { return top_k == 1u ? p : __umulhi(p, top_k_magic); };
+    auto id_of = [&](uint32_t p) { if (ids_l) return ids_l[p]; const uint32_t e = ids[p]; return e < n_expert ? e : n_expert - 1u; };
+    for (uint32_t i = tid; i < n_expert; i += 1024u) { first[i] = 0xffffffffu; count[i] = 0u; dense[i] = 0u; cursor[i] = 0u; }
+    __syncthreads();
+    for (uint32_t pb = tid; pb < P; pb += 8u * 1024u) {      // eight ids per thread requested together
+        uint32_t raw[8];
+#pragma unroll
+        for (uint32_t j = 0; j < 8u; ++j) { const uint32_t p = pb + 1024u * j; raw[j] = p < P ? ids[p] : 0u; }
+#pragma unroll
+        for (uint32_t j = 0; j < 8u; ++j) {
+            const uint32_t p = pb + 1024u * j;
+            if (p < P) {
+                const uint32_t e = guarded_id(raw[j], n_expert, status);
+                if (ids_l) ids_l[p] = e;
+                atomicMin(&first[e], p);
+                atomicAdd(&count[e], 1u);
+            }
+        }
+    }
+    __syncthreads();
+    // experts numbered in first-appearance order: exclusive scan of "pair p is the first appearance of its expert" in per-thread runs
+    const uint32_t per = (P + 1023u) / 1024u;
+    uint32_t mine = 0u;
+    for (uint32_t j = 0; j < per; ++j) { const uint32_t p = tid * per + j; if (p < P && first[id_of(p)] == p) ++mine; }
+    uint32_t U = 0u;
+    uint32_t run = block_scan_1024(mine, wave_tot, U);
+    for (uint32_t j = 0; j < per; ++j) {
+        const uint32_t p = tid * per + j;
+        if (p < P && first[id_of(p)] == p) { const uint32_t e = id_of(p); dense[e] = run; uid_l[run] = e; uid[run] = e; ++run; }
+    }
+    __syncthreads();
+    uint32_t all = 0u;
+    const uint32_t my_start = block_scan_1024(tid < U ? count[uid_l[tid]] : 0u, wave_tot, all);
+    if (tid < U) { start[tid] = my_start; expert_start[tid] = my_start; }
+    if (tid == 0u) { start[U] = all; expert_start[U] = all; n_unique[0] = U; }
+    __syncthreads();
+    for (uint32_t t0 = 0; t0 < ntok; t0 += kGroupBlockTokens) {
+        const uint32_t t1 = t0 + kGroupBlockTokens < ntok ? t0 + kGroupBlockTokens : ntok, p0 = t0 * top_k, p1 = t1 * top_k;
+        // the block's weights (at most 512 x 16 pairs: eight per thread) are requested here and stored behind the bitmap passes
+        float wreg[8];
+#pragma unroll
+        for (uint32_t j = 0; j < 8u; ++j) { const uint32_t p = p0 + tid + 1024u * j; wreg[j] = p < p1 ? weights[p] : 0.0f; }
+        for (uint32_t i = tid; i < n_expert * WB; i += 1024u) member[i] = 0u;
+        __syncthreads();
+        for (uint32_t p = p0 + tid; p < p1; p += 1024u) {
+            const uint32_t e = id_of(p), t = token_of(p) - t0, bit = 1u << (t & 31u);
+            if ((atomicOr(&member[e * WB + (t >> 5)], bit) & bit) && status) atomicOr(status, 2u);      // the token names this expert twice
+        }
+        __syncthreads();
+        uint32_t block_count = 0u;                     // of expert tid (n_expert <= 1024)
+        if (tid < n_expert) {
+#pragma unroll
+            for (uint32_t w = 0; w < WB; ++w) { below[tid * WB + w] = block_count; block_count += __popc(member[tid * WB + w]); }
+        }
+        __syncthreads();
+#pragma unroll
+        for (uint32_t j = 0; j < 8u; ++j) {
+            const uint32_t p = p0 + tid + 1024u * j;
+            if (p < p1) {
+                const uint32_t e = id_of(p), tok = token_of(p), t = tok - t0;
+                const uint32_t rank = below[e * WB + (t >> 5)] + __popc(member[e * WB + (t >> 5)] & ((1u << (t & 31u)) - 1u));
+                const uint32_t pos = start[dense[e]] + cursor[e] + rank;
+                pair_token[pos] = tok;
+                pair_weight[pos] = wreg[j];
+                tok_pair[p] = pos;
+            }
+        }
+        __syncthreads();
+        if (tid < n_expert) cursor[tid] += block_count;
+    }
+    __syncthreads();
+    if (tiles.tile_group) build_tile_lists(U, tid < U ? start[tid] : 0u, tid < U ? start[tid + 1u] - start[tid] : 0u, P, tiles, tile_tot);
+}
+
 hipError_t launch_group_pairs(const uint32_t *ids, const float *weights, uint32_t ntok, uint32_t top_k, uint32_t n_expert,
                               uint32_t *uid, uint32_t *expert_start, uint32_t *pair_token, float *pair_weight,
                               uint32_t *tok_pair, uint32_t *n_unique, hipStream_t s, const TileLists *tiles) {
@@ -831,7 +929,6 @@ hipError_t launch_group_pairs(const uint32_t *ids, const float *weights, uint32_
     const uint32_t words = (ntok + 31u) / 32u;
     const size_t lds = sizeof(uint32_t) * ((size_t)4u * n_expert + 1u + 1024u + 17u + (size_t)n_expert * words);
     constexpr size_t kGroupDynLds = 159u * 1024u;      // (the kernel has a little static LDS beside it)
-    if (lds > kGroupDynLds) return hipErrorInvalidValue;
     const size_t lds_prefix = lds + sizeof(uint32_t) * (size_t)n_expert * words;
     const uint32_t magic = (uint32_t)(((1ull << 32) + top_k - 1u) / top_k);      // top_k == 1 needs none (and would not fit)
     static bool attr_set = false;
@@ -842,6 +939,20 @@ hipError_t launch_group_pairs(const uint32_t *ids, const float *weights, uint32_
         attr_set = true;
     }
     const size_t ids_bytes = sizeof(uint32_t) * (size_t)ntok * top_k;
+    const size_t lds_blocked = sizeof(uint32_t) * ((size_t)5u * n_expert + 1u + 1024u + 17u + (size_t)2u * n_expert * kGroupBlockWords);
+    if (ntok > kGroupBlockTokens && lds_blocked <= kGroupDynLds) {       // larger chunks: block by block
+        static bool blocked_attr = false;
+        if (!blocked_attr) {
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(group_pairs_blocked_kernel), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGroupDynLds);
+            if (e != hipSuccess) return e;
+            blocked_attr = true;
+        }
+        const bool cache = lds_blocked + ids_bytes <= kGroupDynLds;
+        REDHIP_LAUNCH(group_pairs_blocked_kernel, dim3(1), dim3(1024), lds_blocked + (cache ? ids_bytes : 0u), s, ids, weights, ntok, top_k, magic, n_expert, uid, expert_start,
+                      pair_token, pair_weight, tok_pair, n_unique, route_guard().status, cache ? 1u : 0u, tl);
+        return hipGetLastError();
+    }
+    if (lds > kGroupDynLds) return hipErrorInvalidValue;
     if (lds_prefix <= kGroupDynLds) {
         const bool cache = lds_prefix + ids_bytes <= kGroupDynLds;
         REDHIP_LAUNCH(group_pairs_kernel<true>, dim3(1), dim3(1024), lds_prefix + (cache ? ids_bytes : 0u), s, ids, weights, ntok, top_k, magic, n_expert, uid, expert_start, pair_token,

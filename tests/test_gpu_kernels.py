@@ -118,9 +118,9 @@ def test_router_select_random_and_ties():
 def test_grouping_matches_host_sort():
     from dwarfstar_red_lite_amd import moe
     cfg = synth.layer_config(hidden=256, ffn=256, n_expert=512, top_k=10)
-    m = moe.ResidentMoe(cfg, n_layer=1, max_tokens=1600)
+    m = moe.ResidentMoe(cfg, n_layer=1, max_tokens=2048)
     rng = np.random.default_rng(12)
-    for ntok in (1, 2, 3, 8, 33, 512, 1600):
+    for ntok in (1, 2, 3, 8, 33, 512, 513, 1024, 1600, 2048):          # (more than 512 tokens: the pair sort places block by block)
         l = synth.hot_logits(rng, ntok, 512)
         sel = [orc.router_select(l[t], 10) for t in range(ntok)]
         ids = np.stack([s[0] for s in sel])
@@ -129,9 +129,20 @@ def test_grouping_matches_host_sort():
         got = m.group(dev(ids.astype(np.int32)), dev(w))
         for a, b in zip(got, want):
             assert np.array_equal(a.cpu().numpy().view(b.dtype), b), ntok
-    ids = synth.zipf_topk(rng, 512, 512, 10)
-    w = rng.random((512, 10)).astype(np.float32)
-    want = orc.group_pairs(ids, w, 512)
+    for ntok in (512, 2048):
+        ids = synth.zipf_topk(rng, ntok, 512, 10)
+        w = rng.random((ntok, 10)).astype(np.float32)
+        want = orc.group_pairs(ids, w, 512)
+        got = m.group(dev(ids.astype(np.int32)), dev(w))
+        for a, b in zip(got, want):
+            assert np.array_equal(a.cpu().numpy().view(b.dtype), b), ntok
+    m.close()
+    # the widest expert table (1024) with a partial last block of tokens
+    cfg = synth.layer_config(hidden=256, ffn=256, n_expert=1024, top_k=4)
+    m = moe.ResidentMoe(cfg, n_layer=1, max_tokens=1500)
+    ids = synth.zipf_topk(rng, 1500, 1024, 4)
+    w = rng.random((1500, 4)).astype(np.float32)
+    want = orc.group_pairs(ids, w, 1024)
     got = m.group(dev(ids.astype(np.int32)), dev(w))
     for a, b in zip(got, want):
         assert np.array_equal(a.cpu().numpy().view(b.dtype), b)
