@@ -582,7 +582,7 @@ __device__ __forceinline__ void gateup_narrow_items(const TiledArgs &ta, uint32_
                 }
             }
         }
-        const uint8_t *gmat = ex, *umat = ex + gate_bytes;
+        const uint8_t *gmat = ex;
 #pragma unroll 1
         for (uint32_t j = j0; j < j0 + FGH; ++j) {
             float4_t totg = {0.0f, 0.0f, 0.0f, 0.0f}, totu = totg;
@@ -748,7 +748,7 @@ __device__ __forceinline__ void gateup_wide_items(const TiledArgs &ta, uint32_t 
             const uint16_t *dp = reinterpret_cast<const uint16_t *>(mat + qs_bytes) + ((uint64_t)rtile * HB + chunk / 2u) * 16u + r;
             return RowChunk{qp[0], qp[1], *dp, FMT == 1 ? reinterpret_cast<const uint32_t *>(mat + sc_off)[at] : 0u};
         };
-        const uint8_t *gmat = ex, *umat = ex + gate_bytes;
+        const uint8_t *gmat = ex;
         RowChunk cg = load_chunk(gmat, 0u, 0u), cu = load_chunk(umat, 0u, 0u);
 #pragma unroll 1
         for (uint32_t hs = 0; hs < kHalfSteps; ++hs) {
