@@ -748,7 +748,7 @@ __device__ __forceinline__ void gateup_wide_items(const TiledArgs &ta, uint32_t 
             const uint16_t *dp = reinterpret_cast<const uint16_t *>(mat + qs_bytes) + ((uint64_t)rtile * HB + chunk / 2u) * 16u + r;
             return RowChunk{qp[0], qp[1], *dp, FMT == 1 ? reinterpret_cast<const uint32_t *>(mat + sc_off)[at] : 0u};
         };
-        const uint8_t *gmat = ex;
+        const uint8_t *gmat = ex, *umat = ex + gate_bytes;
         RowChunk cg = load_chunk(gmat, 0u, 0u), cu = load_chunk(umat, 0u, 0u);
 #pragma unroll 1
         for (uint32_t hs = 0; hs < kHalfSteps; ++hs) {
@@ -1353,6 +1353,10 @@ static hipError_t launch_gateup_reg(const TiledArgs &ta, dim3 grid, hipStream_t 
 // routed gate/up + SwiGLU of a chunk on the tile-major copy of packed IQ2_XXS gate/up matrices: the front half of a layer whose other
 // matrices are of other types. Activations out as f32 [pairs][ffn] (`act`, for kernels on raw rows) or, with act == nullptr, as fp16 halves
 // with two exponents per pair (for launch_prefill_down_iq3s). Needs the pair grouping; builds the tile list; the shared expert is not touched.
+// Persistent workgroups of the tile kernels: a tile is cut into up to four work items, so small chunks fill more workgroups than they
+// have tiles (17 tokens: 152 tiles, 608 items - three rounds on 256 workgroups instead of four on 183)
+static inline uint32_t tile_grid(uint32_t tile_bound) { return 4u * tile_bound < 256u ? 4u * tile_bound : 256u; }
+
 hipError_t launch_prefill_gateup_tiled(const void *tiled_experts, uint64_t stride, const uint32_t *uid, const uint32_t *expert_start,
                                        const uint32_t *pair_token, const uint32_t *n_unique, uint32_t *tile_group, uint32_t *tile_pair0, uint32_t *tile_n,
                                        uint32_t *n_tiles, const void *xh, const void *xl, const int *xexp, float *act, void *act_h, void *act_l,
@@ -1373,7 +1377,7 @@ hipError_t launch_prefill_gateup_tiled(const void *tiled_experts, uint64_t strid
                   ffn, top_k, ntok};
     const TiledArgs ta{a, static_cast<const uint8_t *>(tiled_experts), nullptr, act, nullptr, 0u};
     const uint32_t tile_bound = prefill_tile_bound(ntok, top_k, n_expert);
-    return launch_gateup_reg(ta, dim3(tile_bound < 256u ? tile_bound : 256u), s, tile_bound);
+    return launch_gateup_reg(ta, dim3(tile_grid(tile_bound)), s, tile_bound);
 }
 
 // The routed gate/up and down matrices of a chunk on a layout whose experts are IQ2_XS / IQ1_M: the same tile kernels on the row-major
@@ -1401,7 +1405,7 @@ hipError_t launch_prefill_streams(uint32_t gate_up_type, const int8_t *gate_up_g
                   static_cast<const _Float16 *>(xl), xexp, static_cast<_Float16 *>(act_h), static_cast<_Float16 *>(act_l), act_exp, tmp, nullptr, hidden,
                   ffn, top_k, ntok};
     const uint32_t tile_bound = prefill_tile_bound(ntok, top_k, n_expert);
-    const dim3 grid(tile_bound < 256u ? tile_bound : 256u), rblock(kRegWaves * 64);
+    const dim3 grid(tile_grid(tile_bound)), rblock(kRegWaves * 64);
     const TiledArgs tg{a, static_cast<const uint8_t *>(packed), nullptr, nullptr, gate_up_grid, 0u};
     e = launch_gateup_reg(tg, grid, s, tile_bound, fg);
     if (e != hipSuccess) return e;
@@ -1429,7 +1433,7 @@ hipError_t launch_prefill_down_iq3s(const void *tiled_down, uint64_t stride, con
                   nullptr, hidden, ffn, top_k, ntok};
     const Iq3DownArgs da{a, static_cast<const uint8_t *>(tiled_down), stride};
     const uint32_t tile_bound = prefill_tile_bound(ntok, top_k, n_expert);
-    const dim3 grid(tile_bound < 256u ? tile_bound : 256u);
+    const dim3 grid(tile_grid(tile_bound));
     prof_set_stage(ST_PREFILL_DOWN);
     if (ffn == 256u) REDHIP_LAUNCH(prefill_down_iq3s_kernel<8>, grid, dim3(kRegWaves * 64), 0, s, da);
     else REDHIP_LAUNCH(prefill_down_iq3s_kernel<16>, grid, dim3(kRegWaves * 64), 0, s, da);
@@ -1459,12 +1463,12 @@ hipError_t launch_prefill_packed(const void *experts, uint64_t stride, const voi
     const dim3 grid(tile_bound < 256u ? tile_bound : 256u), block(kWaves * 64);
     if (tiled_experts && tiled_shared && ffn <= 512u) {          // tile-major copy present: activations of a tile in registers
         const TiledArgs ta{a, static_cast<const uint8_t *>(tiled_experts), static_cast<const uint8_t *>(tiled_shared), nullptr, nullptr, 0u};
-        const dim3 rblock(kRegWaves * 64);
-        e = launch_gateup_reg(ta, grid, s, tile_bound);
+        const dim3 rblock(kRegWaves * 64), rgrid(tile_grid(tile_bound));
+        e = launch_gateup_reg(ta, rgrid, s, tile_bound);
         if (e != hipSuccess) return e;
         prof_set_stage(ST_PREFILL_DOWN);
-        if (ffn == 256u) REDHIP_LAUNCH((prefill_down_reg_kernel<8, 0>), grid, rblock, 0, s, ta);
-        else REDHIP_LAUNCH((prefill_down_reg_kernel<16, 0>), grid, rblock, 0, s, ta);
+        if (ffn == 256u) REDHIP_LAUNCH((prefill_down_reg_kernel<8, 0>), rgrid, rblock, 0, s, ta);
+        else REDHIP_LAUNCH((prefill_down_reg_kernel<16, 0>), rgrid, rblock, 0, s, ta);
         return hipGetLastError();
     }
     const size_t dyn_lds = (size_t)2u * kTile * (hidden + kRowPad) * 2u;
