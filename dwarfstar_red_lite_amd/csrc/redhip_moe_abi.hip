@@ -85,10 +85,9 @@ struct Moe {
     static constexpr uint32_t kStageExperts = 64u;
     // handles that can be given chunks keep a tile-major copy for the prefill kernels that hold a tile's activations in registers
     // larger chunks take the router as a tiled f32 product (a quantised router through its f32 copy)
-    // (an F32 router below 48 tokens is quicker one token per grid layer: 32 x 32 tiles leave most of the chip idle there)
-    bool tiled_router(uint32_t ntok) const {
-        return packed_gu() && ntok >= (cfg.router_type == T_F32 ? 48u : 16u) && (cfg.router_type == T_F32 || mixed);
-    }
+    // (below 40 tokens the f32 rows are quicker one token per grid layer - 12.1 against 14.0 us at 32 tokens, 14.4 against 13.8 at 40:
+    // 32 x 32 tiles leave most of the chip idle there)
+    bool tiled_router(uint32_t ntok) const { return packed_gu() && ntok >= 40u && (cfg.router_type == T_F32 || mixed); }
     uint64_t tiled_stride() const { return fused ? expert_stride : packed_stride; }      // bytes between experts in `tiled`
     bool tiles_resident() const { return packed_gu() && gu_type == T_IQ2_XXS && cfg.max_tokens > 8u && cfg.ffn <= 512u && cfg.hidden / 512u <= 4u; }
     // a chunk on a mixed layout: the routed gate/up matrices (packed IQ2_XXS) run on the prefill tiles, the rest on raw rows
@@ -767,6 +766,11 @@ int redhip_moe_route(redhip_moe_t h, uint32_t layer, const float *x_dev, uint32_
         else if (dense_small)
             HIP_OK(launch_router_gemv(T_F32, router_f32, x_dev, m->layers[layer].gate_inp, ntok, c.hidden, c.n_expert, m->logits, m->xh, m->xl, m->xexp,
                                       nullptr, m->act, c.ffn, s, m->layers[layer].dense_gu), "router launch");
+        else if (m->mixed && c.router_type != T_F32 && router_f32 && ntok > 8u && (nv == 2u || nv == 4u || nv == 8u || nv == 16u))
+            // a small chunk on a layout with a quantised router: the f32 copy of its rows, one token per grid layer (no shared rows: the
+            // shared expert of a chunk runs as dense products on the second stream)
+            HIP_OK(launch_router_gemv(T_F32, router_f32, x_dev, m->layers[layer].gate_inp, ntok, c.hidden, c.n_expert, m->logits, m->xh, m->xl, m->xexp,
+                                      nullptr, nullptr, c.ffn, s), "router launch");
         else
             HIP_OK(launch_router_gemv(c.router_type, m->layers[layer].router, x_dev, m->layers[layer].gate_inp, ntok, c.hidden, c.n_expert,
                                       m->logits, m->xh, m->xl, m->xexp, m->shared_gu_ready ? m->layers[layer].shared : nullptr, m->act, c.ffn, s),
