@@ -438,8 +438,9 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
                (sgu != T_Q6_K || (size_t)64u * (c.hidden / 256u) * 210u + (size_t)(c.hidden + c.hidden / 32u + c.hidden / 16u) * 4u <= (gu == T_IQ1_M ? 120u : 144u) * 1024u);
     {
         const uint32_t nv = c.hidden / 256u;
-        m->mixed_slices = m->mixed && ((gu == T_IQ2_XXS && dn == T_IQ3_S) || (gu_codebook && dn == gu && sgu == T_Q6_K)) && c.ffn <= 512u && c.hidden / 512u <= 4u &&
-                          (nv == 2u || nv == 4u || nv == 8u || nv == 16u);
+        // (a handle for one token at a time needs no second copy of IQ2_XS / IQ1_M down streams: only the slices read the column-sliced one)
+        m->mixed_slices = m->mixed && ((gu == T_IQ2_XXS && dn == T_IQ3_S) || (gu_codebook && dn == gu && sgu == T_Q6_K && c.max_tokens >= 2u)) && c.ffn <= 512u &&
+                          c.hidden / 512u <= 4u && (nv == 2u || nv == 4u || nv == 8u || nv == 16u);
     }
     m->pk_gate_bytes = packed_matrix_bytes(gu, c.ffn, c.hidden);
     m->packed_stride = m->fused && m->rowmajor_down() ? m->expert_stride : align256(2u * m->pk_gate_bytes);
