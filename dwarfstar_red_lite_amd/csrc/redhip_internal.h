@@ -245,10 +245,24 @@ __device__ __forceinline__ void build_tile_lists(uint32_t U, uint32_t p0, uint32
     }
 }
 #endif
+// Device scratch of the pair sort of large chunks (more than 512 tokens), which runs as three launches over blocks of kGroupSpan tokens:
+// count_blk / blk_off [blocks][n_expert], first_key / expert_base [n_expert]. All zero before the first use (the sort leaves first_key
+// zero again); `blocks` = the capacity in blocks.
+constexpr uint32_t kGroupSpan = 64u;
+struct GroupScratch { uint32_t *count_blk, *blk_off, *first_key, *expert_base; uint32_t blocks; };
+inline size_t group_scratch_bytes(uint32_t max_tokens, uint32_t n_expert) {
+    return sizeof(uint32_t) * ((size_t)2u * ((max_tokens + kGroupSpan - 1u) / kGroupSpan) + 2u) * n_expert;
+}
+inline GroupScratch group_scratch_at(void *base, uint32_t max_tokens, uint32_t n_expert) {
+    const uint32_t nb = (max_tokens + kGroupSpan - 1u) / kGroupSpan;
+    uint32_t *p = static_cast<uint32_t *>(base);
+    return GroupScratch{p, p + (size_t)nb * n_expert, p + (size_t)2u * nb * n_expert, p + (size_t)2u * nb * n_expert + n_expert, nb};
+}
 // tiles: also write the tile lists of the chunk (the prefill launchers then take tiles_built = true and launch no build_tiles_kernel)
+// scratch: when given, chunks of more than 512 tokens are sorted by many workgroups (three launches) instead of one
 hipError_t launch_group_pairs(const uint32_t *ids, const float *weights, uint32_t ntok, uint32_t top_k, uint32_t n_expert,
                               uint32_t *uid, uint32_t *expert_start, uint32_t *pair_token, float *pair_weight,
-                              uint32_t *tok_pair, uint32_t *n_unique, hipStream_t s, const TileLists *tiles = nullptr);
+                              uint32_t *tok_pair, uint32_t *n_unique, hipStream_t s, const TileLists *tiles = nullptr, const GroupScratch *scratch = nullptr);
 
 // ---- decode path over packed IQ2_XXS (redhip_fused.hip) ----
 

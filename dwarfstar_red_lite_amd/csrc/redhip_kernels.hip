@@ -921,9 +921,117 @@ __global__ __launch_bounds__(1024) void group_pairs_blocked_kernel(const uint32_
     if (tiles.tile_group) build_tile_lists(U, tid < U ? start[tid] : 0u, tid < U ? start[tid + 1u] - start[tid] : 0u, P, tiles, tile_tot);
 }
 
+// ---- the same sort by many workgroups, for large chunks: spans of kGroupSpan tokens, three launches
+//   group_count_kernel  one workgroup per span: pairs per expert of the span, and the first pair of every expert (a maximum over ~p, so
+//                       that the all-zero scratch means "no pair yet")
+//   group_plan_kernel   one workgroup: experts in first-appearance order, their starts, every span's offset inside its expert, the tile
+//                       lists; leaves first_key zero for the next chunk
+//   group_place_kernel  one workgroup per span: a pair's place = its expert's start + the pairs of the spans before + the tokens of this
+//                       span before it that chose the expert (bitmap of the span's tokens per expert in LDS)
+// Same outputs in the same stable order as the single-workgroup kernels.
+__global__ __launch_bounds__(256) void group_count_kernel(const uint32_t *ids, uint32_t ntok, uint32_t top_k, uint32_t n_expert, GroupScratch gs, uint32_t *status) {
+    __shared__ uint32_t hist[1024], key[1024];
+    const uint32_t tid = threadIdx.x, b = blockIdx.x;
+    const uint32_t t0 = b * kGroupSpan, t1 = t0 + kGroupSpan < ntok ? t0 + kGroupSpan : ntok, p0 = t0 * top_k, p1 = t1 * top_k;
+    for (uint32_t e = tid; e < n_expert; e += 256u) { hist[e] = 0u; key[e] = 0u; }
+    __syncthreads();
+    for (uint32_t p = p0 + tid; p < p1; p += 256u) {
+        const uint32_t e = guarded_id(ids[p], n_expert, status);
+        atomicAdd(&hist[e], 1u);
+        atomicMax(&key[e], ~p);
+    }
+    __syncthreads();
+    for (uint32_t e = tid; e < n_expert; e += 256u) {
+        gs.count_blk[(uint64_t)b * n_expert + e] = hist[e];
+        if (key[e]) atomicMax(&gs.first_key[e], key[e]);
+    }
+}
+
+__global__ __launch_bounds__(1024) void group_plan_kernel(GroupScratch gs, uint32_t nb, uint32_t n_expert, uint32_t P, uint32_t *uid, uint32_t *expert_start,
+                                                          uint32_t *n_unique, TileLists tiles) {
+    __shared__ uint32_t key_l[1024], cnt[1024], uid_l[1024], start[1025], wave_tot[17];
+    __shared__ uint32_t tile_tot[3][16];
+    const uint32_t tid = threadIdx.x;
+    uint32_t my_key = 0u, total = 0u;
+    if (tid < n_expert) {
+        my_key = gs.first_key[tid];
+        gs.first_key[tid] = 0u;                            // ready for the next chunk
+        for (uint32_t b0 = 0; b0 < nb; b0 += 16u) {      // sixteen spans' counts requested together, then their running sums stored
+            uint32_t c[16];
+#pragma unroll
+            for (uint32_t i = 0; i < 16u; ++i) c[i] = b0 + i < nb ? gs.count_blk[(uint64_t)(b0 + i) * n_expert + tid] : 0u;
+#pragma unroll
+            for (uint32_t i = 0; i < 16u; ++i) {
+                if (b0 + i < nb) gs.blk_off[(uint64_t)(b0 + i) * n_expert + tid] = total;
+                total += c[i];
+            }
+        }
+    }
+    key_l[tid] = my_key;
+    cnt[tid] = total;
+    __syncthreads();
+    // first-appearance order: the experts with an earlier first pair (a larger key) come before this one
+    uint32_t d = 0u;
+    if (my_key) for (uint32_t e = 0; e < n_expert; ++e) d += key_l[e] > my_key ? 1u : 0u;
+    uint32_t U = 0u;
+    (void)block_scan_1024(my_key ? 1u : 0u, wave_tot, U);
+    if (my_key) { uid_l[d] = tid; uid[d] = tid; }
+    __syncthreads();
+    uint32_t all = 0u;
+    const uint32_t my_start = block_scan_1024(tid < U ? cnt[uid_l[tid]] : 0u, wave_tot, all);
+    if (tid < U) { start[tid] = my_start; expert_start[tid] = my_start; gs.expert_base[uid_l[tid]] = my_start; }
+    if (tid == 0u) { start[U] = all; expert_start[U] = all; n_unique[0] = U; }
+    __syncthreads();
+    if (tiles.tile_group) build_tile_lists(U, tid < U ? start[tid] : 0u, tid < U ? start[tid + 1u] - start[tid] : 0u, P, tiles, tile_tot);
+}
+
+__global__ __launch_bounds__(256) void group_place_kernel(const uint32_t *ids, const float *weights, uint32_t ntok, uint32_t top_k, uint32_t top_k_magic,
+                                                          uint32_t n_expert, GroupScratch gs, uint32_t *pair_token, float *pair_weight, uint32_t *tok_pair,
+                                                          uint32_t *status) {
+    constexpr uint32_t W = kGroupSpan / 32u;
+    __shared__ uint32_t member[1024 * W];
+    const uint32_t tid = threadIdx.x, b = blockIdx.x;
+    const uint32_t t0 = b * kGroupSpan, t1 = t0 + kGroupSpan < ntok ? t0 + kGroupSpan : ntok, p0 = t0 * top_k, p1 = t1 * top_k;
+    auto token_of = [&](uint32_t p) { return top_k == 1u ? p : __umulhi(p, top_k_magic); };
+    // at most kGroupSpan x 16 pairs per span: four per thread, ids and weights requested up front
+    uint32_t ereg[4];
+    float wreg[4];
+#pragma unroll
+    for (uint32_t j = 0; j < 4u; ++j) {
+        const uint32_t p = p0 + tid + 256u * j;
+        const uint32_t e = p < p1 ? ids[p] : 0u;
+        ereg[j] = e < n_expert ? e : n_expert - 1u;        // (reported by the counting launch)
+        wreg[j] = p < p1 ? weights[p] : 0.0f;
+    }
+    for (uint32_t i = tid; i < n_expert * W; i += 256u) member[i] = 0u;
+    __syncthreads();
+#pragma unroll
+    for (uint32_t j = 0; j < 4u; ++j) {
+        const uint32_t p = p0 + tid + 256u * j;
+        if (p < p1) {
+            const uint32_t t = token_of(p) - t0, bit = 1u << (t & 31u);
+            if ((atomicOr(&member[ereg[j] * W + (t >> 5)], bit) & bit) && status) atomicOr(status, 2u);      // the token names this expert twice
+        }
+    }
+    __syncthreads();
+#pragma unroll
+    for (uint32_t j = 0; j < 4u; ++j) {
+        const uint32_t p = p0 + tid + 256u * j;
+        if (p < p1) {
+            const uint32_t e = ereg[j], tok = token_of(p), t = tok - t0;
+            uint32_t rank = __popc(member[e * W + (t >> 5)] & ((1u << (t & 31u)) - 1u));
+            for (uint32_t w = 0; w < (t >> 5); ++w) rank += __popc(member[e * W + w]);
+            const uint32_t pos = gs.expert_base[e] + gs.blk_off[(uint64_t)b * n_expert + e] + rank;
+            pair_token[pos] = tok;
+            pair_weight[pos] = wreg[j];
+            tok_pair[p] = pos;
+        }
+    }
+}
+
 hipError_t launch_group_pairs(const uint32_t *ids, const float *weights, uint32_t ntok, uint32_t top_k, uint32_t n_expert,
                               uint32_t *uid, uint32_t *expert_start, uint32_t *pair_token, float *pair_weight,
-                              uint32_t *tok_pair, uint32_t *n_unique, hipStream_t s, const TileLists *tiles) {
+                              uint32_t *tok_pair, uint32_t *n_unique, hipStream_t s, const TileLists *tiles, const GroupScratch *scratch) {
     if (!ntok || !top_k || !n_expert || n_expert > 1024u || (uint64_t)ntok * top_k * top_k >= (1ull << 32)) return hipErrorInvalidValue;
     const TileLists tl = tiles ? *tiles : TileLists{};
     const uint32_t words = (ntok + 31u) / 32u;
@@ -937,6 +1045,14 @@ hipError_t launch_group_pairs(const uint32_t *ids, const float *weights, uint32_
         if (e == hipSuccess) e = hipFuncSetAttribute(reinterpret_cast<const void *>(group_pairs_kernel<true>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)kGroupDynLds);
         if (e != hipSuccess) return e;
         attr_set = true;
+    }
+    if (scratch && ntok > kGroupBlockTokens && (ntok + kGroupSpan - 1u) / kGroupSpan <= scratch->blocks && top_k <= 16u) {      // many workgroups, three launches
+        const uint32_t nb = (ntok + kGroupSpan - 1u) / kGroupSpan;
+        REDHIP_LAUNCH(group_count_kernel, dim3(nb), dim3(256), 0, s, ids, ntok, top_k, n_expert, *scratch, route_guard().status);
+        REDHIP_LAUNCH(group_plan_kernel, dim3(1), dim3(1024), 0, s, *scratch, nb, n_expert, ntok * top_k, uid, expert_start, n_unique, tl);
+        REDHIP_LAUNCH(group_place_kernel, dim3(nb), dim3(256), 0, s, ids, weights, ntok, top_k, magic, n_expert, *scratch, pair_token, pair_weight, tok_pair,
+                      route_guard().status);
+        return hipGetLastError();
     }
     const size_t ids_bytes = sizeof(uint32_t) * (size_t)ntok * top_k;
     const size_t lds_blocked = sizeof(uint32_t) * ((size_t)5u * n_expert + 1u + 1024u + 17u + (size_t)2u * n_expert * kGroupBlockWords);

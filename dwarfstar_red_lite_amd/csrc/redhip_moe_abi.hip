@@ -109,6 +109,9 @@ struct Moe {
     // batched path (ntok > 1): pairs grouped by expert
     uint32_t *uid = nullptr, *expert_start = nullptr, *pair_token = nullptr, *tok_pair = nullptr, *n_unique = nullptr;
     uint32_t *tile_group = nullptr, *tile_pair0 = nullptr, *tile_n = nullptr, *n_tiles = nullptr;      // prefill tiles
+    void *group_mem = nullptr;               // handles that take more than 512 tokens: scratch of the pair sort by many workgroups
+    GroupScratch group_scratch{};
+    const GroupScratch *group_scratch_ptr() const { return group_mem ? &group_scratch : nullptr; }
     float *pair_weight = nullptr, *tmp = nullptr, *sh_tmp = nullptr;
     // chunks on mixed layouts: the shared expert's dense products (x -> sh_gu -> sh_act -> sh_tmp) run on a stream of their own beside
     // the routed experts' tile kernels, which leave most of the machine's issue slots free; forked and joined with events
@@ -268,7 +271,9 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
         const ExpertSet ex = m->routed(layer), sh = m->shared(layer);
         const Layer &Ld = m->layers[layer];
         const bool stream_tiles = m->stream_chunk(ntok) && Ld.tiled && Ld.tiled_down && Ld.dense_gu && m->side;
-        // the shared expert as dense f32 products on the fp32 matrix units, started before the pair sort (one workgroup on an idle machine)
+        // the shared expert as dense f32 products on the fp32 matrix units, started before the pair sort (one workgroup on an idle machine;
+        // the many-workgroup sort of a large chunk then queues behind the dense tiles - 73 against 22 us at 2048 tokens - but started
+        // behind the sort the dense products slow the down tiles by more: 787 against 760 us per chunk)
         const bool dense_shared = (stream_tiles || (m->mixed_chunk(ntok) && Ld.dense_gu && m->side));
         if (dense_shared && !fork_shared_dense(m, Ld, x, ntok, s)) return 0;
         // the pair sort also writes the tile lists of the tile kernels that follow (all-IQ2_XXS layers: with the shared expert's tiles)
@@ -278,7 +283,7 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
         if (!grouped) {
             prof_set_stage(ST_GROUP);
             HIP_OK(launch_group_pairs(ids, weights, ntok, c.top_k, c.n_expert, m->uid, m->expert_start, m->pair_token, m->pair_weight,
-                                      m->tok_pair, m->n_unique, s, tile_path ? &tl : nullptr), "grouping launch");
+                                      m->tok_pair, m->n_unique, s, tile_path ? &tl : nullptr, m->group_scratch_ptr()), "grouping launch");
         }
         if (m->small_batch(ntok) && grouped && !select_here) {     // the caller's routing, sorted (with its pass list) by the prep launch: expert slices per pass
             const Layer &L = m->layers[layer];
@@ -563,6 +568,16 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
         m->n_tiles = reinterpret_cast<uint32_t *>(w);
     }
     if (hipMemset(m->ws, 0, ws_bytes) != hipSuccess) { moe_err("failed to clear the MoE workspace"); redhip_moe_destroy(m); return nullptr; }
+    if (T > 512u) {
+        const size_t gb = group_scratch_bytes(c.max_tokens, c.n_expert);
+        if (hipMalloc(&m->group_mem, gb) != hipSuccess || hipMemset(m->group_mem, 0, gb) != hipSuccess) {
+            moe_err("failed to allocate the pair sort scratch");
+            redhip_moe_destroy(m);
+            return nullptr;
+        }
+        m->group_scratch = group_scratch_at(m->group_mem, c.max_tokens, c.n_expert);
+        m->resident += gb;
+    }
     // first launches copy the codebooks to the device; do it here so that forward never synchronises
     if (launch_dequant_rows(T_F32, m->ws, 1u, 32u, m->logits, nullptr) != hipSuccess || hipDeviceSynchronize() != hipSuccess) {
         moe_err("failed to initialise device codebooks");
@@ -594,6 +609,7 @@ void redhip_moe_destroy(redhip_moe_t h) {
     if (m->ev_join) (void)hipEventDestroy(m->ev_join);
     if (m->side) (void)hipStreamDestroy(m->side);
     if (m->ws) (void)hipFree(m->ws);
+    if (m->group_mem) (void)hipFree(m->group_mem);
     if (m->stage) (void)hipFree(m->stage);
     if (m->stage_down) (void)hipFree(m->stage_down);
     delete m;
@@ -946,7 +962,8 @@ int redhip_moe_group(redhip_moe_t h, const uint32_t *ids_dev, const float *weigh
     prof_set_stage(ST_GROUP);
     route_guard() = RouteGuard{m->cfg.n_expert, m->status};
     const hipError_t ge = launch_group_pairs(ids_dev, weights_dev, ntok, m->cfg.top_k, m->cfg.n_expert, uid_dev, expert_start_dev, pair_token_dev,
-                                             pair_weight_dev, tok_pair_dev, n_unique_dev, static_cast<hipStream_t>(stream));
+                                             pair_weight_dev, tok_pair_dev, n_unique_dev, static_cast<hipStream_t>(stream), nullptr,
+                                             ntok <= m->cfg.max_tokens ? m->group_scratch_ptr() : nullptr);
     route_guard() = RouteGuard{};
     HIP_OK(ge, "grouping launch");
     return 1;

@@ -13,6 +13,41 @@ pytestmark = pytest.mark.gpu
 torch = pytest.importorskip("torch")
 
 
+def test_pair_sort_of_a_large_chunk_reports_the_same_way():
+    """More than 512 tokens: the pair sort runs on many workgroups (spans of 64 tokens); an id out of range in one span and an expert named
+    twice in another are clamped / reported, the sorted arrays are those of the clamped routing."""
+    from dwarfstar_red_lite_amd.moe import ResidentMoe
+    E, K, ntok = 64, 4, 700
+    cfg = synth.layer_config(hidden=512, ffn=256, n_expert=E, top_k=K, layout="iq2")
+    m = ResidentMoe(cfg, n_layer=1, max_tokens=ntok)
+    rng = np.random.default_rng(3)
+    ids = np.stack([rng.choice(E - 1, size=K, replace=False) for _ in range(ntok)]).astype(np.uint32)      # (expert E - 1 unused: the clamp lands there)
+    w = rng.random((ntok, K)).astype(np.float32)
+    got = m.group(torch.from_numpy(ids.astype(np.int32)).cuda(), torch.from_numpy(w).cuda())
+    m.last_route(1)                                          # no report
+    for a, b in zip(got, orc.group_pairs(ids, w, E)):
+        assert np.array_equal(a.cpu().numpy().view(b.dtype), b)
+    bad = ids.copy()
+    bad[650, 2] = E + 77
+    got = m.group(torch.from_numpy(bad.astype(np.int32)).cuda(), torch.from_numpy(w).cuda())
+    with pytest.raises(RedHipError, match="n_expert"):
+        m.last_route(1)
+    clamped = bad.copy()
+    clamped[650, 2] = E - 1
+    for a, b in zip(got, orc.group_pairs(clamped, w, E)):
+        assert np.array_equal(a.cpu().numpy().view(b.dtype), b)
+    dup = ids.copy()
+    dup[130, 3] = dup[130, 1]
+    m.group(torch.from_numpy(dup.astype(np.int32)).cuda(), torch.from_numpy(w).cuda())
+    with pytest.raises(RedHipError, match="twice"):
+        m.last_route(1)
+    got = m.group(torch.from_numpy(ids.astype(np.int32)).cuda(), torch.from_numpy(w).cuda())               # the scratch is ready for the next chunk
+    m.last_route(1)
+    for a, b in zip(got, orc.group_pairs(ids, w, E)):
+        assert np.array_equal(a.cpu().numpy().view(b.dtype), b)
+    m.close()
+
+
 @pytest.mark.parametrize("layout,shape", [("iq2", (512, 256, 32, 4)), ("f2", (512, 256, 32, 4)), ("f2", (768, 256, 24, 3))])
 def test_out_of_range_and_repeated_ids_are_clamped_and_reported(layout, shape):
     from dwarfstar_red_lite_amd.moe import ResidentMoe
