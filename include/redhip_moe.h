@@ -32,7 +32,10 @@ typedef struct {
     uint32_t n_expert;          /* <= 1024 */
     uint32_t top_k;             /* <= 16 (the one-token and small-batch MFMA kernels serve 2..15, other values run on the generic kernels) */
     uint32_t n_layer;
-    uint32_t max_tokens;        /* largest ntok of redhip_moe_forward */
+    uint32_t max_tokens;        /* largest ntok of redhip_moe_forward (the reference's prefill hands over chunks of up to 2048 tokens,
+                                   native/redmetal_engine_prefill.m:1246-1277). It also decides which copies of the weights the handle keeps
+                                   beside the raw blocks: 1 - the streams of the one-token kernels; 2..8 - also the column-sliced down copy of
+                                   the small-batch kernels; more than 8 - also the tile-major copies of the chunk kernels */
     uint32_t router_type;       /* 0 (F32) or 14 (Q6_K) */
     uint32_t expert_type_word;  /* gate_up | down << 8, as native/redlite_native_metal.h:69-73; types 16 (IQ2_XXS), 21 (IQ3_S), 14 (Q6_K), and
                                    17 (IQ2_XS) / 29 (IQ1_M) after redhip_set_codebooks */
