@@ -590,19 +590,45 @@ __global__ __launch_bounds__(256) void batch_down_kernel(PairArgs a, uint32_t hi
 }
 
 // out[t][r] = sum_k pair_weight[p_k] * tmp[p_k][r] (p_k = tok_pair[t][k], selection order) + scalar[t] * sh_tmp[t][r]
+// Four rows per thread; a token's pair indices, weights and rows (top_k <= 16) are all requested before the first is used - as a loop
+// over k every term was three dependent round trips - and added in selection order as before.
 __global__ __launch_bounds__(256) void batch_combine_kernel(const float *tmp, const float *pair_weight, const uint32_t *tok_pair, uint32_t top_k,
                                                             const float *sh_tmp, const float *scalar, uint32_t hidden, float *out,
                                                             const float *resid_a, const float *resid_b) {
-    const uint32_t r = blockIdx.x * 256u + threadIdx.x, t = blockIdx.y;
-    if (r >= hidden) return;
-    float acc = 0.0f;
-    for (uint32_t k = 0; k < top_k; ++k) {
-        const uint32_t p = tok_pair[(uint64_t)t * top_k + k];
-        acc = fmaf(pair_weight[p], tmp[(uint64_t)p * hidden + r], acc);
+    const uint32_t c = blockIdx.x * 256u + threadIdx.x, t = blockIdx.y, H4 = hidden / 4u;
+    if (c >= H4) return;
+    uint32_t p[16];
+    float w[16];
+    float4 v[16];
+#pragma unroll
+    for (uint32_t k = 0; k < 16u; ++k) p[k] = k < top_k ? tok_pair[(uint64_t)t * top_k + k] : 0u;
+#pragma unroll
+    for (uint32_t k = 0; k < 16u; ++k) {
+        w[k] = 0.0f;
+        v[k] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+        if (k < top_k) {                                   // (uniform: no row is read for the unused terms)
+            w[k] = pair_weight[p[k]];
+            v[k] = reinterpret_cast<const float4 *>(tmp)[(uint64_t)p[k] * H4 + c];
+        }
     }
-    if (sh_tmp) acc = fmaf(scalar[t], sh_tmp[(uint64_t)t * hidden + r], acc);
-    const uint64_t at = (uint64_t)t * hidden + r;
-    out[at] = resid_a ? (resid_a[at] + resid_b[at]) + acc : acc;
+    float4 sh = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    const float sc = sh_tmp ? scalar[t] : 0.0f;
+    if (sh_tmp) sh = reinterpret_cast<const float4 *>(sh_tmp)[(uint64_t)t * H4 + c];
+    float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+#pragma unroll
+    for (uint32_t k = 0; k < 16u; ++k) {
+        if (k < top_k) {
+            acc.x = fmaf(w[k], v[k].x, acc.x); acc.y = fmaf(w[k], v[k].y, acc.y);
+            acc.z = fmaf(w[k], v[k].z, acc.z); acc.w = fmaf(w[k], v[k].w, acc.w);
+        }
+    }
+    if (sh_tmp) { acc.x = fmaf(sc, sh.x, acc.x); acc.y = fmaf(sc, sh.y, acc.y); acc.z = fmaf(sc, sh.z, acc.z); acc.w = fmaf(sc, sh.w, acc.w); }
+    const uint64_t at = (uint64_t)t * H4 + c;
+    if (resid_a) {
+        const float4 ra = reinterpret_cast<const float4 *>(resid_a)[at], rb = reinterpret_cast<const float4 *>(resid_b)[at];
+        acc = make_float4((ra.x + rb.x) + acc.x, (ra.y + rb.y) + acc.y, (ra.z + rb.z) + acc.z, (ra.w + rb.w) + acc.w);
+    }
+    reinterpret_cast<float4 *>(out)[at] = acc;
 }
 
 template <uint32_t T>
@@ -675,7 +701,8 @@ hipError_t launch_batch_down(const ExpertSet &ex, const uint32_t *uid, const uin
 
 hipError_t launch_batch_combine(const float *tmp, const float *pair_weight, const uint32_t *tok_pair, uint32_t ntok, uint32_t top_k,
                                 const float *sh_tmp, const float *scalar, uint32_t hidden, float *out, hipStream_t s) {
-    REDHIP_LAUNCH(batch_combine_kernel, dim3((hidden + 255u) / 256u, ntok), dim3(256), 0, s, tmp, pair_weight, tok_pair, top_k, sh_tmp, scalar, hidden, out, block_context().resid_a, block_context().resid_b);
+    if (hidden % 4u || top_k > 16u) return hipErrorInvalidValue;
+    REDHIP_LAUNCH(batch_combine_kernel, dim3((hidden / 4u + 255u) / 256u, ntok), dim3(256), 0, s, tmp, pair_weight, tok_pair, top_k, sh_tmp, scalar, hidden, out, block_context().resid_a, block_context().resid_b);
     return hipGetLastError();
 }
 
@@ -685,7 +712,17 @@ __global__ __launch_bounds__(256) void weighted_sum_kernel(const float *tmp, con
     const uint32_t i = blockIdx.x * 256u + threadIdx.x;
     if (i >= row_count) return;
     float acc = 0.0f;
-    for (uint32_t k = 0; k < top_k; ++k) acc = fmaf(weights[k], tmp[(uint64_t)k * hidden + row_start + i], acc);
+    for (uint32_t k0 = 0; k0 < top_k; k0 += 16u) {      // sixteen terms requested together, added in the order of the list
+        float w[16], v[16];
+#pragma unroll
+        for (uint32_t k = 0; k < 16u; ++k) {
+            w[k] = 0.0f;
+            v[k] = 0.0f;
+            if (k0 + k < top_k) { w[k] = weights[k0 + k]; v[k] = tmp[(uint64_t)(k0 + k) * hidden + row_start + i]; }
+        }
+#pragma unroll
+        for (uint32_t k = 0; k < 16u; ++k) if (k0 + k < top_k) acc = fmaf(w[k], v[k], acc);
+    }
     out[i] = acc;
 }
 
