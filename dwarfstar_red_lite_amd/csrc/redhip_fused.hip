@@ -305,11 +305,15 @@ __device__ __forceinline__ void group_small(const GroupJob &g, uint32_t *lds, Pa
     const bool live = pr < P;
     const uint32_t t = live ? pr / K : 0u;
     const uint32_t e = live ? guarded_id(pair_id(t, pr % K), g.n_expert, g.status) : 0u;
-    if (live && (atomicOr(&token_set[e], 1u << t) & (1u << t)) && g.status) atomicOr(g.status, 2u);      // the token names this expert twice
+    // A token that names an expert twice breaks the caller's contract: reported, and the repeated pair takes no place of its own in the
+    // group arrays (it shares its twin's position, so every index stays inside the arrays of ntok * top_k pairs; expert_start[U] is then
+    // the number of pairs placed, less than ntok * top_k)
+    const bool dup = live && (atomicOr(&token_set[e], 1u << t) & (1u << t)) != 0u;
+    if (dup && g.status) atomicOr(g.status, 2u);
     __syncthreads();
     const uint32_t set = live ? token_set[e] : 0u;
     const uint32_t n = (uint32_t)__popc(set), before = (uint32_t)__popc(set & ((1u << t) - 1u));
-    const bool first = live && before == 0u;
+    const bool first = live && !dup && before == 0u;
     uint32_t scan = first ? n : 0u;                      // inclusive prefix sum of the group sizes in pair order
     const uint32_t n_pass_mine = first ? (n + 1u) >> 1 : 0u;
     uint32_t pscan = n_pass_mine;                        // the same of the groups' pass counts
@@ -330,17 +334,19 @@ __device__ __forceinline__ void group_small(const GroupJob &g, uint32_t *lds, Pa
     if (first) { token_set[e] = start | (pass0 << 16); g.uid[grp] = e; g.expert_start[grp] = start; }
     if (tid == 0u) {
         const uint32_t U = first_count[0] + first_count[1];
-        g.expert_start[U] = P;
+        g.expert_start[U] = size_total[0] + size_total[1];      // = P unless a token repeated an expert
         g.n_unique[0] = U;
         if (g.n_pass) g.n_pass[0] = pass_total[0] + pass_total[1];
     }
     __syncthreads();
     if (live) {
         const uint32_t word = token_set[e], pos = (word & 0xffffu) + before;
-        g.pair_token[pos] = t;
-        g.pair_weight[pos] = pair_w(t, pr % K);
         g.tok_pair[pr] = pos;
-        if (g.pass_list) {
+        if (!dup) {
+            g.pair_token[pos] = t;
+            g.pair_weight[pos] = pair_w(t, pr % K);
+        }
+        if (g.pass_list && !dup) {
             const uint32_t v = (word >> 16) + (before >> 1), half = before & 1u;
             uint8_t *entry = reinterpret_cast<uint8_t *>(g.pass_list + v);
             if (half == 0u) reinterpret_cast<uint32_t *>(entry)[0] = e | ((n - before >= 2u ? 2u : 1u) << 16) | (pos << 24);

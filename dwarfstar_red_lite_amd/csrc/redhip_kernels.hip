@@ -367,7 +367,7 @@ hipError_t launch_moe_gateup(const ExpertSet &ex, const uint32_t *ids, uint32_t 
                              const float *x, float *act, hipStream_t s, const float *x1, uint32_t x_split) {
     hipError_t e = ensure_tables();
     if (e != hipSuccess) return e;
-    if (!n_slot || hidden % 256u || ffn % 256u) return hipErrorInvalidValue;
+    if (!n_slot || hidden % 256u || ffn % 256u || (size_t)padded_floats(hidden) * 4u > 64u * 1024u) return hipErrorInvalidValue;
     switch (ex.gate_up_type) {
         case T_IQ2_XXS: return gateup_dispatch<T_IQ2_XXS>(ex, ids, n_slot, hidden, ffn, x, act, s, x1, x_split);
         case T_IQ3_S: return gateup_dispatch<T_IQ3_S>(ex, ids, n_slot, hidden, ffn, x, act, s, x1, x_split);
@@ -631,6 +631,49 @@ __global__ __launch_bounds__(256) void batch_combine_kernel(const float *tmp, co
     reinterpret_cast<float4 *>(out)[at] = acc;
 }
 
+// the same sum for top_k > 16: blocks of sixteen terms requested together, every term added in selection order
+__global__ __launch_bounds__(256) void batch_combine_loop_kernel(const float *tmp, const float *pair_weight, const uint32_t *tok_pair, uint32_t top_k,
+                                                                 const float *sh_tmp, const float *scalar, uint32_t hidden, float *out,
+                                                                 const float *resid_a, const float *resid_b) {
+    const uint32_t c = blockIdx.x * 256u + threadIdx.x, t = blockIdx.y, H4 = hidden / 4u;
+    if (c >= H4) return;
+    float4 acc = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+    for (uint32_t k0 = 0; k0 < top_k; k0 += 16u) {
+        uint32_t p[16];
+        float w[16];
+        float4 v[16];
+#pragma unroll
+        for (uint32_t k = 0; k < 16u; ++k) p[k] = k0 + k < top_k ? tok_pair[(uint64_t)t * top_k + k0 + k] : 0u;
+#pragma unroll
+        for (uint32_t k = 0; k < 16u; ++k) {
+            w[k] = 0.0f;
+            v[k] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if (k0 + k < top_k) {
+                w[k] = pair_weight[p[k]];
+                v[k] = reinterpret_cast<const float4 *>(tmp)[(uint64_t)p[k] * H4 + c];
+            }
+        }
+#pragma unroll
+        for (uint32_t k = 0; k < 16u; ++k) {
+            if (k0 + k < top_k) {
+                acc.x = fmaf(w[k], v[k].x, acc.x); acc.y = fmaf(w[k], v[k].y, acc.y);
+                acc.z = fmaf(w[k], v[k].z, acc.z); acc.w = fmaf(w[k], v[k].w, acc.w);
+            }
+        }
+    }
+    if (sh_tmp) {
+        const float sc = scalar[t];
+        const float4 sh = reinterpret_cast<const float4 *>(sh_tmp)[(uint64_t)t * H4 + c];
+        acc.x = fmaf(sc, sh.x, acc.x); acc.y = fmaf(sc, sh.y, acc.y); acc.z = fmaf(sc, sh.z, acc.z); acc.w = fmaf(sc, sh.w, acc.w);
+    }
+    const uint64_t at = (uint64_t)t * H4 + c;
+    if (resid_a) {
+        const float4 ra = reinterpret_cast<const float4 *>(resid_a)[at], rb = reinterpret_cast<const float4 *>(resid_b)[at];
+        acc = make_float4((ra.x + rb.x) + acc.x, (ra.y + rb.y) + acc.y, (ra.z + rb.z) + acc.z, (ra.w + rb.w) + acc.w);
+    }
+    reinterpret_cast<float4 *>(out)[at] = acc;
+}
+
 template <uint32_t T>
 static hipError_t batch_gateup_dispatch(const PairArgs &a, uint32_t n_groups, uint32_t hidden, uint32_t ffn, const float *x, float *act, hipStream_t s) {
     const uint32_t lpr = lanes_per_row(hidden);
@@ -661,12 +704,23 @@ static hipError_t batch_down_dispatch(const PairArgs &a, uint32_t n_groups, uint
     const uint32_t lpr = lanes_per_row(ffn);
     const dim3 grid((hidden + 256u / lpr - 1u) / (256u / lpr), n_groups);
     const size_t lds = (size_t)kPairTile * padded_floats(ffn) * sizeof(float);
+#define REDHIP_BDN(L)                                                                                                              \
+    do {                                                                                                                           \
+        static bool attr = false;                                                                                                  \
+        if (!attr) {      /* (the default limit is 64 KB: ffn >= 2048 needs more) */                                               \
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(batch_down_kernel<T, L>), hipFuncAttributeMaxDynamicSharedMemorySize, 160 * 1024); \
+            if (e != hipSuccess) return e;                                                                                         \
+            attr = true;                                                                                                           \
+        }                                                                                                                          \
+        REDHIP_LAUNCH((batch_down_kernel<T, L>), grid, dim3(256), lds, s, a, hidden, ffn, act, tmp);                               \
+    } while (0)
     switch (lpr) {
-        case 64: REDHIP_LAUNCH((batch_down_kernel<T, 64>), grid, dim3(256), lds, s, a, hidden, ffn, act, tmp); break;
-        case 32: REDHIP_LAUNCH((batch_down_kernel<T, 32>), grid, dim3(256), lds, s, a, hidden, ffn, act, tmp); break;
-        case 16: REDHIP_LAUNCH((batch_down_kernel<T, 16>), grid, dim3(256), lds, s, a, hidden, ffn, act, tmp); break;
-        default: REDHIP_LAUNCH((batch_down_kernel<T, 8>), grid, dim3(256), lds, s, a, hidden, ffn, act, tmp); break;
+        case 64: REDHIP_BDN(64); break;
+        case 32: REDHIP_BDN(32); break;
+        case 16: REDHIP_BDN(16); break;
+        default: REDHIP_BDN(8); break;
     }
+#undef REDHIP_BDN
     return hipGetLastError();
 }
 
@@ -687,7 +741,7 @@ hipError_t launch_batch_gateup(const ExpertSet &ex, const uint32_t *uid, const u
 
 hipError_t launch_batch_down(const ExpertSet &ex, const uint32_t *uid, const uint32_t *expert_start, const uint32_t *n_unique,
                              uint32_t n_groups, uint32_t n_pairs_total, uint32_t hidden, uint32_t ffn, const float *act, float *tmp, hipStream_t s) {
-    if (!n_groups || hidden % 256u || ffn % 256u || n_groups > 65535u) return hipErrorInvalidValue;
+    if (!n_groups || hidden % 256u || ffn % 256u || (size_t)kPairTile * padded_floats(ffn) * 4u > 160u * 1024u || n_groups > 65535u) return hipErrorInvalidValue;
     const PairArgs a{ex.base, ex.stride, ex.gate_bytes + ex.up_bytes, 0u, uid, expert_start, nullptr, n_unique, n_pairs_total, ex.table};
     switch (ex.down_type) {
         case T_IQ2_XXS: return batch_down_dispatch<T_IQ2_XXS>(a, n_groups, hidden, ffn, act, tmp, s);
@@ -701,8 +755,10 @@ hipError_t launch_batch_down(const ExpertSet &ex, const uint32_t *uid, const uin
 
 hipError_t launch_batch_combine(const float *tmp, const float *pair_weight, const uint32_t *tok_pair, uint32_t ntok, uint32_t top_k,
                                 const float *sh_tmp, const float *scalar, uint32_t hidden, float *out, hipStream_t s) {
-    if (hidden % 4u || top_k > 16u) return hipErrorInvalidValue;
-    REDHIP_LAUNCH(batch_combine_kernel, dim3((hidden / 4u + 255u) / 256u, ntok), dim3(256), 0, s, tmp, pair_weight, tok_pair, top_k, sh_tmp, scalar, hidden, out, block_context().resid_a, block_context().resid_b);
+    if (hidden % 4u || !top_k) return hipErrorInvalidValue;
+    const dim3 grid((hidden / 4u + 255u) / 256u, ntok);
+    if (top_k <= 16u) REDHIP_LAUNCH(batch_combine_kernel, grid, dim3(256), 0, s, tmp, pair_weight, tok_pair, top_k, sh_tmp, scalar, hidden, out, block_context().resid_a, block_context().resid_b);
+    else REDHIP_LAUNCH(batch_combine_loop_kernel, grid, dim3(256), 0, s, tmp, pair_weight, tok_pair, top_k, sh_tmp, scalar, hidden, out, block_context().resid_a, block_context().resid_b);
     return hipGetLastError();
 }
 

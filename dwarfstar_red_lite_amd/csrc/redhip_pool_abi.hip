@@ -36,7 +36,8 @@ struct FfnPool {
     uint32_t capacity = 0, slots_per_slab = 0;
     std::vector<uint8_t *> slabs;                 // device memory, created on first use of a slot in the slab
     std::vector<uint32_t> inflight;
-    std::mutex mu;                                // counters, slab creation, in-flight marks
+    std::vector<uint64_t> loaded_bytes;           // per slot: payload bytes of the last successful load_expert (0: never loaded)
+    std::mutex mu;                                // counters, slab creation, in-flight marks, loaded_bytes
     std::mutex exec_mu;                           // the scratch below serves one execute at a time
     DevBuf scratch;
     uint64_t bytes_read = 0, read_calls = 0;
@@ -142,6 +143,7 @@ redmetal_ffn_pool_t redmetal_ffn_pool_create(const char *model_path, uint64_t bu
     }
     p->file_size = (uint64_t)st.st_size;
     p->inflight.assign(p->capacity, 0u);
+    p->loaded_bytes.assign(p->capacity, 0u);
     return p;
 }
 
@@ -217,6 +219,7 @@ int redmetal_ffn_pool_load_expert(redmetal_ffn_pool_t h, uint32_t slot_id,
         p->bytes_read += local_bytes;
         p->read_calls += local_calls;
         p->read_ms += ms;
+        p->loaded_bytes[slot_id] = payload;
     }
     if (bytes_read) *bytes_read = local_bytes;
     if (elapsed_ms) *elapsed_ms = ms;
@@ -329,7 +332,13 @@ int redmetal_ffn_pool_execute_expert_noalloc(redmetal_ffn_pool_t h, uint32_t slo
         return 0;
     }
     uint8_t *base = p->slot_base_existing(slot_id);
-    if (!base) { FFN_ERR("FFN slot %u holds no expert yet: load it before the non-allocating call", slot_id); return 0; }
+    uint64_t loaded = 0;
+    if (base) { std::lock_guard<std::mutex> lk(p->mu); loaded = p->loaded_bytes[slot_id]; }
+    if (!base || !loaded) { FFN_ERR("FFN slot %u holds no expert yet: load it before the non-allocating call", slot_id); return 0; }
+    if (gate_bytes + up_bytes + down_bytes > loaded) {
+        FFN_ERR("FFN slot %u holds %llu bytes, the call names %llu", slot_id, (unsigned long long)loaded, (unsigned long long)(gate_bytes + up_bytes + down_bytes));
+        return 0;
+    }
     if ((gu == T_IQ2_XS || gu == T_IQ1_M || dn == T_IQ2_XS || dn == T_IQ1_M) && !caller_grids_bound(p)) {
         FFN_ERR("the pool's IQ2_XS / IQ1_M codebooks are not on the device yet: run redmetal_ffn_pool_execute_expert on such an expert once first");
         return 0;

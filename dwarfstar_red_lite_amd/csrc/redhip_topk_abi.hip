@@ -42,6 +42,9 @@ struct TopkPool {
     std::vector<int8_t> iq2_xs, iq1_m;
     // buffers between the launches of a call (grow-only)
     DevBuf act, tmp, io;
+    // the batched / mapped forms keep buffers of their own (the reference's _tmpB): growing them for a large chunk never moves `tmp`,
+    // whose address callers hold through redmetal_topk_pool_tmp_buffer
+    DevBuf act_b, tmp_b;
     // host lists of a call (slot addresses, weights, pair arrays) travel through a ring of pinned host buffers, each with a
     // device buffer of its own; an event recorded behind the call's last launch says when both may be used again
     struct Stage {
@@ -95,6 +98,18 @@ struct TopkPool {
 
 TopkPool *pool_of(redmetal_topk_pool_t h) { return static_cast<TopkPool *>(h); }
 
+// What the raw-row kernels of this pool can stage in LDS: one token keeps its activation vector (hidden floats, padded) within the
+// default 64 KB; the batched forms and the down rows keep eight pairs' vectors within 160 KB. Checked before anything is enqueued.
+constexpr uint32_t kPoolMaxHiddenToken = 15360u, kPoolMaxBatched = 4864u;
+bool pool_shape_ok(uint32_t hidden, uint32_t ffn, bool batched) {
+    const uint32_t max_hidden = batched ? kPoolMaxBatched : kPoolMaxHiddenToken;
+    if (hidden > max_hidden || ffn > kPoolMaxBatched) {
+        TOPK_ERR("top-k shape hidden=%u ffn=%u exceeds what this pool's kernels stage in LDS (hidden <= %u, ffn <= %u for this call)", hidden, ffn, max_hidden, kPoolMaxBatched);
+        return false;
+    }
+    return true;
+}
+
 bool type_word_ok(uint32_t w) { return !(w >> 16) && pool_quant_supported(word_gate_up(w)) && pool_quant_supported(word_down(w)); }
 
 // this pool's codebooks on the device before an IQ2_XS / IQ1_M expert runs (free when they already are)
@@ -109,7 +124,7 @@ bool bind_grids(TopkPool *p, uint32_t type_word) {
 
 // native/redmetal_topk.m:1291-1336
 bool validate(TopkPool *p, const uint32_t *slot_ids, const uint64_t *gate_bytes, const uint64_t *up_bytes, const uint64_t *down_bytes,
-              uint32_t top_k, uint32_t type_word, uint32_t hidden, uint32_t ffn, uint32_t row_start, uint32_t row_count) {
+              uint32_t top_k, uint32_t type_word, uint32_t hidden, uint32_t ffn, uint32_t row_start, uint32_t row_count, bool batched = false) {
     if (!p || !slot_ids || !gate_bytes || !up_bytes || !down_bytes) return false;
     if (!top_k || top_k > REDMETAL_TOPK_MAX) { TOPK_ERR("top_k=%u must be in [1,%u]", top_k, REDMETAL_TOPK_MAX); return false; }
     if (!type_word_ok(type_word)) { TOPK_ERR("unsupported top-k GGML type word 0x%x (supported: IQ2_XS 17, IQ1_M 29, IQ2_XXS 16, IQ3_S 21, Q6_K 14)", type_word); return false; }
@@ -117,6 +132,7 @@ bool validate(TopkPool *p, const uint32_t *slot_ids, const uint64_t *gate_bytes,
         TOPK_ERR("invalid top-k dimensions hidden=%u ffn=%u start=%u count=%u", hidden, ffn, row_start, row_count);
         return false;
     }
+    if (!pool_shape_ok(hidden, ffn, batched)) return false;
     for (uint32_t i = 0; i < top_k; ++i) {
         if (slot_ids[i] >= p->capacity) { TOPK_ERR("top-k slot %u exceeds capacity %u", slot_ids[i], p->capacity); return false; }
         for (uint32_t j = 0; j < i; ++j)
@@ -134,8 +150,9 @@ bool validate(TopkPool *p, const uint32_t *slot_ids, const uint64_t *gate_bytes,
     return true;
 }
 
-bool ensure_scratch(TopkPool *p, uint32_t n_act_rows, uint32_t hidden, uint32_t ffn) {
-    if (!p->act.reserve((size_t)n_act_rows * ffn * sizeof(float)) || !p->tmp.reserve((size_t)n_act_rows * hidden * sizeof(float))) {
+bool ensure_scratch(TopkPool *p, uint32_t n_act_rows, uint32_t hidden, uint32_t ffn, bool batched = false) {
+    DevBuf &act = batched ? p->act_b : p->act, &tmp = batched ? p->tmp_b : p->tmp;
+    if (!act.reserve((size_t)n_act_rows * ffn * sizeof(float)) || !tmp.reserve((size_t)n_act_rows * hidden * sizeof(float))) {
         TOPK_ERR("failed to allocate top-k activation buffers");
         return false;
     }
@@ -232,7 +249,7 @@ bool enqueue_pairs(TopkPool *p, hipStream_t s, const std::vector<uint64_t> &gate
                    uint32_t tok_first, uint32_t ntok, uint32_t top_k, uint32_t n_pairs, const uint32_t *pair_token,
                    const float *pair_weight, const uint32_t *expert_start, const uint32_t *tok_pair, const float *x, float *out) {
     std::lock_guard<std::recursive_mutex> lk(p->enc_mu);
-    if (!bind_grids(p, type_word) || !ensure_scratch(p, n_pairs, hidden, ffn)) return false;
+    if (!bind_grids(p, type_word) || !ensure_scratch(p, n_pairs, hidden, ffn, true)) return false;
     std::vector<uint64_t> table(gate_table);
     table.insert(table.end(), down_table.begin(), down_table.end());
     std::vector<uint32_t> u;
@@ -243,7 +260,7 @@ bool enqueue_pairs(TopkPool *p, hipStream_t s, const std::vector<uint64_t> &gate
     Staged st;
     if (!stage_lists(p, s, table, pair_weight, n_pairs, u, &st)) return false;
     const uint32_t *d_pair_token = st.u, *d_start = st.u + n_pairs, *d_tok_pair = d_start + n_expert + 1u;
-    float *act = static_cast<float *>(p->act.p), *tmp = static_cast<float *>(p->tmp.p);
+    float *act = static_cast<float *>(p->act_b.p), *tmp = static_cast<float *>(p->tmp_b.p);
     ExpertSet gu{nullptr, 0, up_delta, 0, word_gate_up(type_word), word_down(type_word)};
     gu.table = st.table;
     ExpertSet dn{nullptr, 0, down_off, 0, word_gate_up(type_word), word_down(type_word)};
@@ -283,6 +300,7 @@ int encode_device_impl(redmetal_topk_pool_t h, void *stream, void *slot_table_de
         TOPK_ERR("device-driven top-k matrix byte mismatch");
         return 0;
     }
+    if (!pool_shape_ok(hidden, ffn, false)) return 0;
     const uint64_t *table = reinterpret_cast<const uint64_t *>(static_cast<uint8_t *>(slot_table_dev) + slot_table_offset);
     return enqueue_token(p, static_cast<hipStream_t>(stream), table, at(weight_dev, weight_offset), top_k, type_word, hidden, ffn,
                          gate_bytes, up_bytes, 0u, hidden, at(input_dev, input_offset), input1_dev ? at(input1_dev, input1_offset) : nullptr,
@@ -643,7 +661,7 @@ int redmetal_topk_pool_encode_batched(redmetal_topk_pool_t h, void *stream, cons
     TopkPool *p = pool_of(h);
     if (!p || !input_dev || !output_dev || !pair_token || !pair_weight || !expert_start || !tok_pair) return 0;
     if (!ntok || !top_k || !n_pairs || (uint64_t)ntok * top_k != n_pairs || n_pairs > REDMETAL_TOPK_MAX * 64u) { TOPK_ERR("invalid batched top-k pair layout"); return 0; }
-    if (!validate(p, slot_ids, gate_bytes, up_bytes, down_bytes, n_expert, ggml_type, hidden_size, ffn_size, 0u, hidden_size)) return 0;
+    if (!validate(p, slot_ids, gate_bytes, up_bytes, down_bytes, n_expert, ggml_type, hidden_size, ffn_size, 0u, hidden_size, true)) return 0;
     if (!pair_layout_ok("batched", n_expert, tok_first, ntok, top_k, n_pairs, pair_token, expert_start, tok_pair)) return 0;
     std::vector<uint64_t> table(n_expert);
     for (uint32_t i = 0; i < n_expert; ++i) {
@@ -670,6 +688,7 @@ int redmetal_topk_pool_encode_mapped(redmetal_topk_pool_t h, void *stream,
     if (!type_word_ok(ggml_type) || !hidden_size || hidden_size % 256u || !ffn_size || ffn_size % 256u) { TOPK_ERR("mapped top-k needs a supported type word and 256-aligned sizes"); return 0; }
     if (gate_bytes != (uint64_t)ffn_size * pool_row_bytes(word_gate_up(ggml_type), hidden_size) || up_bytes != gate_bytes ||
         down_bytes != (uint64_t)hidden_size * pool_row_bytes(word_down(ggml_type), ffn_size)) { TOPK_ERR("mapped top-k matrix byte mismatch"); return 0; }
+    if (!pool_shape_ok(hidden_size, ffn_size, true)) return 0;
     if (!pair_layout_ok("mapped", n_expert, tok_first, ntok, top_k, n_pairs, pair_token, expert_start, tok_pair)) return 0;
     std::vector<uint64_t> gate(n_expert), down(n_expert);
     for (uint32_t i = 0; i < n_expert; ++i) {

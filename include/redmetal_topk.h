@@ -117,7 +117,10 @@ int redmetal_topk_pool_encode_device_into(redmetal_topk_pool_t pool, void *strea
     void *slot_table_dev, uint64_t slot_table_offset, void *weight_dev, uint64_t weight_offset,
     uint32_t top_k, uint32_t ggml_type, uint32_t hidden_size, uint32_t ffn_size, uint64_t gate_bytes, uint64_t up_bytes,
     void *input_dev, uint64_t input_offset, void *output_dev, uint64_t output_offset);
-void *redmetal_topk_pool_tmp_buffer(redmetal_topk_pool_t pool);         /* device pointer; NULL before the first encode */
+/* Device pointer; NULL before the first single-token encode. Sized REDMETAL_TOPK_MAX * hidden_size floats by the single-token
+ * encodes only: the pointer stays valid until an encode with a larger hidden_size (or ffn_size) than any before it; the batched /
+ * mapped forms use buffers of their own and never move it. */
+void *redmetal_topk_pool_tmp_buffer(redmetal_topk_pool_t pool);
 
 /* native/redmetal_topk.h:156-161, native/redmetal_topk.m:1997-2016 (kernel :209-252): as encode_device_into, but the experts
  * from index x_split on read the second input vector (two-row verify). */

@@ -78,3 +78,14 @@ def write_case(path, spec):
         with open(path, "ab") as fh:
             fh.write(b"\xa5" * spec["trailing_bytes"])
     return cfgs, layers
+
+
+def write_topk_case(path, spec):
+    """One of the fixture files of tests/golden/reference_topk.json: a single layer whose routed experts have the given gate/up and
+    down formats (the same bytes every time). Returns (configuration, layer)."""
+    from dwarfstar_red_lite_amd import synth
+    c = synth.layer_config(hidden=spec["hidden"], ffn=spec["ffn"], n_expert=spec["n_expert"], top_k=2, layout="xs")
+    c["gate_up_type"], c["down_type"] = spec["gate_up_type"], spec["down_type"]
+    layer = synth.make_layer(spec["seed"], c)
+    write_moe_gguf(path, c, [layer])
+    return c, layer

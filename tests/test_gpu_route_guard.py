@@ -97,6 +97,38 @@ def test_out_of_range_and_repeated_ids_are_clamped_and_reported(layout, shape):
     m.close()
 
 
+@pytest.mark.parametrize("layout", ["iq2", "f2"])
+def test_worst_case_repeats_stay_inside_the_pair_arrays(layout):
+    """The fullest small batch (8 tokens x top_k 15 = 120 of at most 128 pairs) whose first token names one expert fifteen times, an expert
+    that every other token names too: the repeated pairs take no place of their own in the group arrays (before, each counted the whole
+    group again and the pair / pass lists ran past their ends into the neighbouring scratch). Reported, and the next valid call on the
+    same handle is right."""
+    from dwarfstar_red_lite_amd.moe import ResidentMoe
+    from test_gpu_moe_batch import oracle_tokens
+    H, F, E, K, ntok = 512, 256, 32, 15, 8
+    cfg = synth.layer_config(hidden=H, ffn=F, n_expert=E, top_k=K, layout=layout)
+    lay = synth.make_layer(99, cfg)
+    m = ResidentMoe(cfg, n_layer=1, max_tokens=ntok)
+    m.load_layer(0, lay)
+    rng = np.random.default_rng(12)
+    x = synth.normed_x(rng, ntok, H)
+    ids = np.stack([np.concatenate([[5], rng.choice(np.setdiff1d(np.arange(E), [5]), size=K - 1, replace=False)]) for _ in range(ntok)]).astype(np.uint32)
+    w = rng.random((ntok, K)).astype(np.float32) + 0.1
+    w /= w.sum(axis=1, keepdims=True)
+    xd, wd = torch.from_numpy(x).cuda(), torch.from_numpy(w).cuda()
+    for bad_tok in (0, 3, ntok - 1):
+        bad = ids.copy()
+        bad[bad_tok, :] = 5
+        m.experts(0, xd, torch.from_numpy(bad.astype(np.int32)).cuda(), wd)
+        with pytest.raises(RedHipError, match="twice"):
+            m.last_route(ntok)
+        got = m.experts(0, xd, torch.from_numpy(ids.astype(np.int32)).cuda(), wd).cpu().numpy()
+        m.last_route(ntok)
+        want = oracle_tokens(cfg, lay, x, ids, w)
+        assert max(rel_l2(got[t], want[t]) for t in range(ntok)) <= REL_L2_TOL
+    m.close()
+
+
 def test_top_k_limits_are_settled_at_create():
     """top_k = 16 (17 slots with the shared expert) and top_k = 1 run on the generic kernels instead of failing mid-forward"""
     from dwarfstar_red_lite_amd.moe import ResidentMoe

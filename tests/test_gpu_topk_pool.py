@@ -293,3 +293,27 @@ def test_batched_and_mapped_pairs(tmp_path, grids, layout):
         c.pool.encode_batched(stream, slots, [c.layouts[int(e)] for e in uid], c.word, H, F, 0, ntok, K, ptok + tok_first, pw, start, tp,
                               x_dev.data_ptr(), out.data_ptr())
     c.pool.close()
+
+
+def test_batched_pairs_with_more_than_sixteen_experts_per_token(tmp_path, grids):
+    """the batched form takes any top_k the pool does (the reference's sum loops over top_k): 17 and 20 experts per token run the looped
+    combine, in selection order, against the CPU path"""
+    c = Case(tmp_path, grids, "iq2", n_expert=24)
+    H, F, E = c.cfg["hidden"], c.cfg["ffn"], 24
+    rng = np.random.default_rng(44)
+    stream = torch.cuda.current_stream().cuda_stream
+    for K, ntok in ((17, 3), (20, 5)):
+        ids = np.stack([rng.permutation(E)[:K] for _ in range(ntok)]).astype(np.uint32)
+        w = rng.random((ntok, K)).astype(np.float32) + 0.1
+        uid, start, ptok, pw, tp = orc.group_pairs(ids, w, E)
+        x = synth.normed_x(rng, ntok, H)
+        x_dev = torch.from_numpy(x).cuda()
+        out = torch.zeros((ntok, H), device="cuda")
+        slots = [c.slot_of[int(e)] for e in uid]
+        c.pool.encode_batched(stream, slots, [c.layouts[int(e)] for e in uid], c.word, H, F, 0, ntok, K, ptok, pw, start, tp, x_dev.data_ptr(), out.data_ptr())
+        torch.cuda.synchronize()
+        c.pool.release(slots)
+        got = out.cpu().numpy()
+        for t in range(ntok):
+            assert rel_l2(got[t], c.want(ids[t], w[t], x[t])) <= REL_L2_TOL, (K, t)
+    c.pool.close()

@@ -215,3 +215,42 @@ def test_rmsnorm():
     out = np.empty(8, np.float32)
     orc.lib().orc_rmsnorm(x.ctypes.data, None, 8, 1e-6, out.ctypes.data)
     assert np.allclose(out, x / math.sqrt(float((x.astype(np.float64) ** 2).mean()) + 1e-6), rtol=1e-7)
+
+
+def test_routed_topk_against_the_compiled_reference(golden_dir, tmp_path):
+    """orc_routed_topk / orc_expert_ffn_grid bit for bit against rl_native_reference_topk (native/redlite_native_reference.c:251-382) on the
+    formats that function accepts: IQ2_XS, IQ1_M, IQ3_S and two mixed gate/up vs down pairings. This is the direct pin of the expert step
+    (gate and up in double, SiLU * up in double, down rows on double activations, experts added in selection order)."""
+    import sys
+    import zlib
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    from gguf_writer import write_topk_case
+    grids = json.load(open(os.path.join(golden_dir, "iq_grids.json")))
+    xs_grid, m_grid = (np.frombuffer(bytes.fromhex(grids[k]), np.int8) for k in ("iq2_xs", "iq1_m"))
+    orc.set_codebooks(xs_grid, m_grid)
+    g = json.load(open(os.path.join(golden_dir, "reference_topk.json")))
+    assert len(g["cases"]) == 5
+    for c in g["cases"]:
+        spec = c["spec"]
+        path = str(tmp_path / (spec["name"] + ".gguf"))
+        cfg, lay = write_topk_case(path, spec)
+        assert zlib.crc32(open(path, "rb").read()) == c["file_crc32"], spec["name"]      # the very bytes the reference read
+        H, F = spec["hidden"], spec["ffn"]
+        i = np.arange(H, dtype=np.int64)
+        x = (((i * 17 + 3) % 61 - 30) / 32.0).astype(np.float32)
+        L = orc.lib()
+        p = lambda a: a.ctypes.data_as(orc.C.c_void_p)
+        for call in c["calls"]:
+            ids, w = np.asarray(call["ids"], np.uint32), unhex(call["weights_f32_hex"], np.float32)
+            want = unhex(call["output_f64_hex"], np.float64)
+            r0, n = call["row_start"], call["row_count"]
+            full = np.zeros(H, np.float64)
+            assert L.orc_routed_topk(spec["gate_up_type"], spec["down_type"], p(lay["gate"]), p(lay["up"]), p(lay["down"]), lay["gate"][0].nbytes,
+                                     lay["up"][0].nbytes, lay["down"][0].nbytes, p(ids), p(w), ids.size, H, F, p(x), p(full))
+            assert np.array_equal(full[r0:r0 + n].view(np.uint64), want.view(np.uint64)), (spec["name"], call["ids"])
+            # the single-expert form on the same row window, weighted and added in selection order as the reference does
+            acc = np.zeros(n, np.float64)
+            for e, we in zip(ids, w):
+                acc += np.float64(we) * orc.expert_ffn_grid(spec["gate_up_type"], spec["down_type"], lay["gate"][e], lay["up"][e], lay["down"][e], H, F, x,
+                                                            xs_grid, m_grid, r0, n)
+            assert np.array_equal(acc.view(np.uint64), want.view(np.uint64)), (spec["name"], "windowed")

@@ -40,6 +40,11 @@ def test_noalloc_matches_execute_expert_on_two_calls_in_a_row(tmp_path):
         with pytest.raises(RedHipError, match="holds no expert"):
             pool.execute_noalloc(0, lays[0], expert_type_word(T_IQ2, T_IQ3), 1024, 512, 0, 1024, torch.zeros(1024, device="cuda").data_ptr(),
                                  torch.zeros(1024, device="cuda").data_ptr(), stream.cuda_stream)
+        # nor does a slot whose slab exists (slot 0 shares it) but which itself was never loaded pass
+        pool.load(0, lays[0])
+        with pytest.raises(RedHipError, match="holds no expert"):
+            pool.execute_noalloc(1, lays[1], expert_type_word(T_Q6K, T_Q6K), 512, 256, 0, 512, torch.zeros(512, device="cuda").data_ptr(),
+                                 torch.zeros(512, device="cuda").data_ptr(), stream.cuda_stream)
         for slot, lay in enumerate(lays):
             pool.load(slot, lay)
         want = [pool.execute(slot, lays[slot], expert_type_word(gu, dn), H, F, 0, H, xs[slot])[0] for slot, (H, F, gu, dn) in enumerate(shapes)]
