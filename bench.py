@@ -7,8 +7,14 @@ A step is one pass of the hot path over one batch: router GEMV -> softmax top-k 
 the router picks different experts every step. Inputs are resident in HBM before the timed region starts.
 
 Prints one JSON line (metric: microseconds per token for one MoE layer; lower is better), with
-  roofline      the dominant kernel's algorithmic bytes per launch / its measured launch duration, vs 8 TB/s
-  cpu_baseline  the CPU oracle (a port of the reference's scalar double-accumulating path) on this host's cores
+  roofline       the dominant kernel's algorithmic bytes per launch / its measured launch duration, vs 8 TB/s
+  cpu_baseline   the CPU oracle (a port of the reference's scalar double-accumulating path) on this host's cores
+  batch_sweep    the ragged small batches (B = 2, 4, 8): drawn hot routing as an input, and the layer's own router
+  <layout>_sweep the same on the mixed-precision layout and the two layouts with the expert formats of the reference's target file
+  prefill_sweep  chunks of 512 / 2048 tokens on the MFMA tile kernels: TFLOP/s against the fp16 matrix-core peak and the HBM cap
+  stack          48 layers back to back for one token (residual + RMS-norm around every layer), us per token and GB/s
+  yardsticks     this machine's own streaming-read rate and fp16 matrix-core rate, measured in the same run
+The headline is timed as HIP graph replays (what a decode loop issues); the eager figure is printed beside it.
 """
 import argparse
 import ctypes as C
@@ -49,6 +55,9 @@ def parse():
     ap.add_argument("--sweep-layouts", default="f2,xs,m", help="layouts the default run adds a sweep for on handles of their own (one token through the layer's "
                                                                "own router, then B=2/4/8 with hot routing); key <layout>_sweep of the result")
     ap.add_argument("--no-sweep", action="store_true", help="skip the B=2/4/8 hot-routing sweep that the default (B=1, own router) run appends")
+    ap.add_argument("--no-prefill", action="store_true", help="skip the prefill-chunk sweep (512 / 2048 tokens) that the default run appends")
+    ap.add_argument("--prefill-layers", type=int, default=8, help="resident layers of the chunk handles (a chunk reads about 0.4 GB of experts per layer)")
+    ap.add_argument("--no-yardsticks", action="store_true", help="skip the streaming-read and matrix-core yardsticks")
     ap.add_argument("--prime", type=int, default=2000, help="untimed steps before the warm-up that bring the clocks up (reported as clock_priming_steps)")
     return ap.parse_args()
 
@@ -86,7 +95,7 @@ def time_steps(torch, stream, step, K, W, outs, rows_written, use_graph, replays
     """W untimed + exactly K timed eager steps (synchronised on both sides); then the same K steps recorded once into a HIP graph
     (kernel launches only) and replayed: every replay is checked bit for bit against the eager outputs on the rows the K steps write,
     and the median over `replays` timed replays (each exactly K steps between two synchronisations) is what a decode loop that issues
-    graphs would see."""
+    graphs would see. That median is the reported time whenever the replays are bit-identical to the eager run."""
     with torch.cuda.stream(stream):
         for i in range(W):
             step(i)
@@ -125,9 +134,8 @@ def time_steps(torch, stream, step, K, W, outs, rows_written, use_graph, replays
     res["graph_ms"] = times[len(times) // 2]
     res["graph_ms_min"] = times[0]
     res["replays_timed"] = len(times)
-    # (chunks that fork work onto a second stream replay a little slower than they launch: the quicker mode is the one reported)
-    if res["graph_ms"] <= eager_ms:
-        res["ms"], res["mode"] = res["graph_ms"], "hip_graph"
+    # one fixed mode: graph replay (the eager figure is reported beside it)
+    res["ms"], res["mode"] = res["graph_ms"], "hip_graph"
     return res
 
 
@@ -185,7 +193,7 @@ def kernel_roofline(cfg, synth, stages, K, B, mean_distinct, lb, traffic_key):
     if dom in ("prefill_gateup", "prefill_down"):
         # prefill tiles run on the MFMA units: algorithmic flops of the stage (2 per multiply-add, every (token, expert) pair
         # and every token's shared expert once; the fp16 hi/lo split that doubles the issued MFMAs is not counted)
-        pairs = B * (cfg["top_k"] + 1)
+        pairs = B * (cfg["top_k"] + (0 if "batch_gateup" in stages else 1))      # (mixed layouts: the shared expert runs as dense f32 products beside the tiles)
         flops = pairs * 2.0 * H * F * (2 if dom == "prefill_gateup" else 1)
         achieved = flops / (dom_us * 1e-6) / 1e12
         return {"bound": "mfma", "kernel": dom, "achieved": round(achieved, 2), "peak": MFMA_F16_PEAK_TFLOPS, "unit": "TFLOP/s",
@@ -229,7 +237,7 @@ def main():
     gen = torch.Generator(device="cuda")
     gen.manual_seed(20241125)
     stream = torch.cuda.Stream()
-    NX = 64
+    NX_DECODE = 64
 
     def resident_handle(layout, NL, max_tokens):
         """a handle with NL layers of the layout resident (weights drawn on the GPU), layer 0 also on the host for the oracle"""
@@ -246,9 +254,11 @@ def main():
         return {"layout": layout, "cfg": cfg, "moe": moe, "NL": NL, "layer0": layer0, "ref": orc.Layer(cfg, **layer0)}
 
     def run_workload(ctx, B, routing):
+        """parity gate on layer 0, then timing, per-kernel profile and the dominant kernel's roofline for batches of B tokens"""
         cfg, moe, NL, layer0, ref = ctx["cfg"], ctx["moe"], ctx["NL"], ctx["layer0"], ctx["ref"]
         H = cfg["hidden"]
-        """parity gate on layer 0, then timing, per-kernel profile and the dominant kernel's roofline for batches of B tokens"""
+        NX = NX_DECODE if B <= 64 else max(4, 4096 // B)          # activation sets the steps cycle through (chunks: fewer, larger ones)
+        prime = args.prime if B <= 64 else max(50, args.prime // 10)
         xs_host = synth.normed_x(np.random.default_rng(99 + B), NX * B, H).reshape(NX, B, H)
         xs = torch.from_numpy(xs_host).cuda()
         outs = torch.zeros_like(xs)
@@ -284,10 +294,11 @@ def main():
             if route_ids is None:
                 gids, _, _ = moe.last_route(B)
             stream.synchronize()
-        if route_ids is None:
-            want, cids, _, _ = ref.forward(xs_host[0], threads=os.cpu_count() or 1)
-            got = outs[0].cpu().numpy()
-            ids_ok = bool(np.array_equal(gids, cids))
+        if route_ids is None:           # (chunks: the first eight tokens - tokens are independent of each other)
+            n_chk = min(B, 8)
+            want, cids, _, _ = ref.forward(xs_host[0][:n_chk], threads=os.cpu_count() or 1)
+            got = outs[0][:n_chk].cpu().numpy()
+            ids_ok = bool(np.array_equal(gids[:n_chk], cids))
         else:           # drawn routing: the oracle's routed experts + gated shared expert for the first tokens of the step
             n_chk = min(B, 8)
             want = oracle_given_routing(orc, cfg, layer0, xs_host[0][:n_chk], ids_h[0][:n_chk], w_h[0][:n_chk], os.cpu_count() or 1)
@@ -300,7 +311,7 @@ def main():
 
         # ---- untimed clock priming, then the timed region ----
         with torch.cuda.stream(stream):
-            for i in range(args.prime):
+            for i in range(prime):
                 step(i)
             stream.synchronize()
         rows_written = {(W + i) % NX for i in range(K)}
@@ -320,7 +331,7 @@ def main():
         lb = layer_bytes(cfg, mean_distinct, B)
         roof = kernel_roofline(cfg, synth, stages, K, B, mean_distinct, lb, "%s_b%d" % (ctx["layout"], B) + ("" if routing == "router" else "_" + routing))
         return {"B": B, "routing": routing, "timing": tm, "stages": stages, "mean_distinct": mean_distinct, "lb": lb, "roofline": roof, "rel": rel,
-                "ids_ok": ids_ok, "xs": xs, "xs_host": xs_host}
+                "ids_ok": ids_ok, "xs": xs, "xs_host": xs_host, "NX": NX}
 
     main_ctx = resident_handle(args.layout, NL, max([B] + sweep))
     cfg, moe = main_ctx["cfg"], main_ctx["moe"]
@@ -352,7 +363,9 @@ def main():
                                "all experts of %d layers resident" % ({"iq2": "config1", "f2": "config2"}.get(args.layout, "target-file expert format"),
                                                                       B, args.layout, NL),
                    "layout": args.layout, "batch": B, "routing": args.routing, "resident_layers": NL, "resident_gb": round(moe.resident_bytes / 1e9, 2),
-                   "mean_distinct_routed_experts": mean_distinct},
+                   "mean_distinct_routed_experts": mean_distinct,
+                   "arithmetic": "weights exact in fp16 (integer codebook values, block scales applied in f32), activations as fp16 hi + lo halves "
+                                 "(22 significant bits), f32 accumulation"},
         "layer_gbps": {"expert_bytes": int(lb["expert_bytes"]), "layer_bytes": int(total_bytes),
                        "expert_gbps": round(lb["expert_bytes"] / (ms_per_step * 1e-3) / 1e9, 1),
                        "layer_gbps": round(total_bytes / (ms_per_step * 1e-3) / 1e9, 1),
@@ -386,7 +399,8 @@ def main():
         result["launch_floor_note"] = "three dependent launches of empty kernels per step (grids of %s), %d steps per graph replay, median of %d replays" % (
             " / ".join("%dx%d" % sh for sh in shapes), K, len(ts))
 
-    # ---- the ragged small-batch configuration on the same resident handle: B = 2, 4, 8, drawn logits with 32 hot experts ----
+    # ---- the ragged small-batch configuration on the same resident handle: B = 2, 4, 8; drawn logits with 32 hot experts (the routing is an
+    # input, as the configuration defines it), and the same batches through the layer's own router (router GEMV + selection in the step) ----
     def sweep_entry(ctx, b, routing):
         r = run_workload(ctx, b, routing)
         t = r["timing"]
@@ -395,20 +409,159 @@ def main():
                 "eager_us_per_step": round(t["eager_ms"] * 1e3, 3), "mean_distinct_routed_experts": r["mean_distinct"],
                 "stages_us": {k: round(v["us_avg"] * v["launches"] / K, 3) for k, v in r["stages"].items()},
                 "dominant_kernel": rf.get("kernel"), "kernel_us": rf.get("launch_us"), "kernel_gbps": rf.get("achieved"), "kernel_frac_of_peak": rf.get("frac"),
-                "expert_bytes": int(r["lb"]["expert_bytes"]), "rel_l2_vs_cpu_oracle": r["rel"]}
+                "kernel_traffic_bytes": rf.get("traffic"), "expert_bytes": int(r["lb"]["expert_bytes"]),
+                "step_gbps_on_expert_bytes": round(r["lb"]["expert_bytes"] / (t["ms"] * 1e-3) / 1e9, 1), "rel_l2_vs_cpu_oracle": r["rel"]}
+
+    # ---- prefill chunks on the MFMA tile kernels: algorithmic flops (2 per multiply-add, every (token, expert) pair's three products and every
+    # token's shared expert once; the fp16 hi / lo split doubles the MFMAs issued and is not counted) against the dense fp16 matrix-core peak,
+    # and the HBM cap: the bytes of the distinct experts the chunk touches (+ shared expert + router) against 8 TB/s ----
+    def chunk_entry(ctx, ntok, routing):
+        r = run_workload(ctx, ntok, routing)
+        c, t, lb = ctx["cfg"], r["timing"], r["lb"]
+        us = t["ms"] * 1e3
+        flops = ntok * (c["top_k"] + 1) * 3 * 2.0 * c["hidden"] * c["ffn"]
+        cap_bytes = lb["expert_bytes"] + lb["router_bytes"] + lb["gate_inp_bytes"] + lb["act_bytes"]
+        return {"layout": ctx["layout"], "tokens": ntok, "routing": routing, "us_per_chunk": round(us, 2), "us_per_token": round(us / ntok, 4),
+                "launch_mode": t["mode"], "eager_us_per_chunk": round(t["eager_ms"] * 1e3, 2), "resident_layers": ctx["NL"],
+                "mean_distinct_routed_experts": r["mean_distinct"],
+                "stages_us": {k: round(v["us_avg"] * v["launches"] / K, 3) for k, v in r["stages"].items()},
+                "roofline": r["roofline"],
+                "chunk_flops": int(flops), "chunk_tflops": round(flops / (us * 1e-6) / 1e12, 2),
+                "chunk_frac_of_mfma_peak": round(flops / (us * 1e-6) / 1e12 / MFMA_F16_PEAK_TFLOPS, 4),
+                "hbm_cap": {"bytes": int(cap_bytes), "us_at_peak": round(cap_bytes / HBM_PEAK_GBS / 1e3, 2), "achieved_gbps": round(cap_bytes / (us * 1e-6) / 1e9, 1),
+                            "frac": round(cap_bytes / (us * 1e-6) / 1e9 / HBM_PEAK_GBS, 4)},
+                "rel_l2_vs_cpu_oracle": r["rel"], "router_ids_identical": r["ids_ok"]}
+
+    # ---- 48 layers back to back for one token: x <- (x + branch) + layer_l(rmsnorm(x + branch)) for l = 0 .. NL - 1, every layer's input the
+    # previous layer's output (the residual add and RMS-norm ride in the layer's own launches). Gate: layer 0's block step against the oracle. ----
+    def stack_entry(ctx, n_tok=10):
+        c, m, NL = ctx["cfg"], ctx["moe"], ctx["NL"]
+        Hc = c["hidden"]
+        rs = np.random.default_rng(4242)
+        x0 = (2.0 * rs.standard_normal((1, Hc))).astype(np.float32)
+        br = (0.5 * rs.standard_normal((NX_DECODE, 1, Hc))).astype(np.float32)
+        pw = np.ones(Hc, np.float32)
+        brd, pwd = torch.from_numpy(br).cuda(), torch.from_numpy(pw).cuda()
+        xd = torch.from_numpy(x0).cuda()
+        with torch.cuda.stream(stream):
+            got = m.forward_block(0, xd, brd[0], pwd, 1e-6).cpu().numpy()
+            gids, _, _ = m.last_route(1)
+        resid = (x0 + br[0]).astype(np.float32)
+        normed = np.empty_like(resid)
+        orc.lib().orc_rmsnorm(resid[0].ctypes.data, pw.ctypes.data, Hc, 1e-6, normed[0].ctypes.data)
+        ffn, cids, _, _ = ctx["ref"].forward(normed, threads=os.cpu_count() or 1)
+        want = resid + ffn.astype(np.float32)
+        rel = float(np.linalg.norm((got - resid) - (want - resid)) / np.linalg.norm(want - resid))
+        if not rel <= 1e-3 or not np.array_equal(gids, cids):
+            print("PARITY FAILURE (stack, %s): block step of layer 0 rel L2 %.3g" % (ctx["layout"], rel), file=sys.stderr)
+            sys.exit(1)
+
+        def token(i):
+            for l in range(NL):
+                m.forward_block(l, xd, brd[(i * NL + l) % NX_DECODE], pwd, 1e-6, out=xd)
+        with torch.cuda.stream(stream):
+            for i in range(20):
+                token(i)
+            stream.synchronize()
+            t0 = time.perf_counter()
+            for i in range(n_tok):
+                token(i)
+            stream.synchronize()
+            eager_us = (time.perf_counter() - t0) * 1e6 / n_tok
+            g = torch.cuda.CUDAGraph()
+            with torch.cuda.graph(g, stream=stream):
+                for i in range(n_tok):
+                    token(i)
+        ts = []
+        for rpl in range(12):
+            torch.cuda.synchronize()
+            t0 = time.perf_counter()
+            g.replay()
+            torch.cuda.synchronize()
+            ts.append((time.perf_counter() - t0) * 1e6 / n_tok)
+        ts = sorted(ts[2:])
+        us = ts[len(ts) // 2]
+        finite = bool(torch.isfinite(xd).all().item())
+        lb1 = layer_bytes(c, c["top_k"], 1)
+        per_layer = lb1["expert_bytes"] + lb1["router_bytes"] + lb1["gate_inp_bytes"]
+        return {"layout": ctx["layout"], "layers": NL, "batch": 1, "us_per_token": round(us, 2), "us_per_layer": round(us / NL, 3), "launch_mode": "hip_graph",
+                "eager_us_per_token": round(eager_us, 2), "tokens_per_replay": n_tok, "replays_timed": len(ts),
+                "bytes_per_token": int(per_layer * NL), "gbps": round(per_layer * NL / us / 1e3, 1), "frac_of_hbm_peak": round(per_layer * NL / us / 1e3 / HBM_PEAK_GBS, 4),
+                "us_at_60pct_of_peak": round(per_layer * NL / (0.6 * HBM_PEAK_GBS) / 1e3, 1), "output_finite": finite,
+                "rel_l2_vs_cpu_oracle_layer0_block": rel}
 
     if sweep:
-        result["batch_sweep"] = [sweep_entry(main_ctx, b, "hot") for b in sweep]
+        result["batch_sweep"] = [sweep_entry(main_ctx, b, "hot") for b in sweep] + [sweep_entry(main_ctx, b, "router") for b in sweep]
+        if NL >= 48:
+            result["stack"] = [stack_entry(main_ctx)]
         # ---- the other layouts, each on a handle of its own: the mixed-precision layout of config 2 (f2) and the layouts with the expert
         # formats of the reference's target file (xs: IQ2_XS, m: IQ1_M experts). One token with the layer's own router, then the same ragged
         # batches; all 48 layers resident like the headline handle ----
         for lay in sweep_layouts:
             ctx = resident_handle(lay, args.f2_layers, max(sweep))
             result[lay + "_sweep"] = {"resident_layers": args.f2_layers, "resident_gb": round(ctx["moe"].resident_bytes / 1e9, 2),
-                                      "runs": [sweep_entry(ctx, 1, "router")] + [sweep_entry(ctx, b, "hot") for b in sweep]}
+                                      "runs": [sweep_entry(ctx, 1, "router")] + [sweep_entry(ctx, b, "hot") for b in sweep] +
+                                              ([sweep_entry(ctx, b, "router") for b in sweep] if lay == "f2" else [])}
+            if lay == "f2" and args.f2_layers >= 48:
+                result.setdefault("stack", []).append(stack_entry(ctx))
             ctx["moe"].close()
             del ctx
             torch.cuda.empty_cache()
+
+    # ---- prefill chunks (handles of their own, made for chunks: they also hold the tile-major copies) ----
+    if sweep and not args.no_prefill:
+        moe.close()                                   # the headline handle is no longer needed: its memory goes to the chunk handles
+        main_ctx["moe"] = None
+        torch.cuda.empty_cache()
+        pre = []
+        ctx = resident_handle("iq2", args.prefill_layers, 2048)
+        pre.append(chunk_entry(ctx, 512, "router"))
+        pre.append(chunk_entry(ctx, 512, "zipf"))
+        pre.append(chunk_entry(ctx, 2048, "router"))
+        ctx["moe"].close()
+        del ctx
+        torch.cuda.empty_cache()
+        ctx = resident_handle("f2", args.prefill_layers, 2048)
+        pre.append(chunk_entry(ctx, 512, "zipf"))
+        pre.append(chunk_entry(ctx, 512, "router"))
+        pre.append(chunk_entry(ctx, 2048, "zipf"))
+        ctx["moe"].close()
+        del ctx
+        torch.cuda.empty_cache()
+        result["prefill_sweep"] = pre
+
+    # ---- this machine's own yardsticks, in the same run: streaming read of 1 GiB (four times the 256 MB last-level cache) and a dense fp16
+    # matrix-core loop on register operands ----
+    if not args.no_yardsticks:
+        n_stage_ = lib.redhip_profile_stage_count()
+        buf = torch.empty(1 << 30, dtype=torch.uint8, device="cuda").random_(0, 256)
+        sink = torch.zeros(4, dtype=torch.float32, device="cuda")
+        torch.cuda.synchronize()
+
+        def timed(launch, reps):
+            with torch.cuda.stream(stream):
+                for _ in range(2):
+                    launch()
+                stream.synchronize()
+                lib.redhip_profile_begin()
+                for _ in range(reps):
+                    launch()
+                sm_, sn_ = (C.c_double * n_stage_)(), (C.c_uint32 * n_stage_)()
+                lib.redhip_profile_end(sm_, sn_, n_stage_)
+            return 1e3 * sum(sm_) / max(sum(sn_), 1)          # average kernel duration in us
+        rd_us = timed(lambda: lib.redhip_calibration_read(buf.data_ptr(), buf.numel(), sink.data_ptr(), stream.cuda_stream), 8)
+        cp_src, cp_dst = buf[:CAL_BYTES], torch.empty(CAL_BYTES, dtype=torch.uint8, device="cuda")
+        cp_us = timed(lambda: lib.redhip_calibration_copy(cp_dst.data_ptr(), cp_src.data_ptr(), CAL_BYTES, stream.cuda_stream), 8)
+        fl = C.c_uint64(0)
+        mf_us = timed(lambda: lib.redhip_calibration_mfma(2048, 2048, sink.data_ptr(), C.byref(fl), stream.cuda_stream), 4)
+        result["yardsticks"] = {
+            "streaming_read": {"bytes": int(buf.numel()), "us": round(rd_us, 2), "gbps": round(buf.numel() / rd_us / 1e3, 1),
+                               "frac_of_published_peak": round(buf.numel() / rd_us / 1e3 / HBM_PEAK_GBS, 4)},
+            "copy": {"bytes_in": CAL_BYTES, "bytes_out": CAL_BYTES, "us": round(cp_us, 2), "gbps_in_plus_out": round(2 * CAL_BYTES / cp_us / 1e3, 1)},
+            "mfma_f16_16x16x32": {"flops": int(fl.value), "us": round(mf_us, 2), "tflops": round(fl.value / mf_us / 1e6, 1),
+                                  "frac_of_published_peak": round(fl.value / mf_us / 1e6 / MFMA_F16_PEAK_TFLOPS, 4)},
+            "note": "kernel durations from the dispatches' own timestamps; published peaks: HBM 8 TB/s, dense fp16 MFMA 2.5 PFLOP/s"}
+        del buf, cp_dst
 
     # ---- per-kernel microbench of config 1: one IQ2_XXS dequant-GEMV [512 x 2048] x [2048] on raw GGUF rows ----
     if args.layout == "iq2" and B == 1 and not args.no_micro:
@@ -467,7 +620,7 @@ def main():
         reps, t_cpu, budget = 0, 0.0, 12.0
         while t_cpu < budget and reps < 2000:
             tc = time.perf_counter()
-            ref.forward(xs_host[reps % NX], threads=cores)
+            ref.forward(xs_host[reps % head["NX"]], threads=cores)
             t_cpu += time.perf_counter() - tc
             reps += 1
         cpu_us = t_cpu * 1e6 / (reps * B)

@@ -81,6 +81,8 @@ ABI = {
     "redhip_profile_end": (i32, [C.POINTER(dbl), C.POINTER(u32), u32]),
     "redhip_calibration_copy": (i32, [vp, vp, u64, vp]),
     "redhip_calibration_empty": (i32, [u32, u32, vp]),
+    "redhip_calibration_read": (i32, [vp, u64, vp, vp]),
+    "redhip_calibration_mfma": (i32, [u32, u32, vp, C.POINTER(C.c_uint64), vp]),
     # include/redmetal_topk.h
     "redmetal_topk_abi_version": (u32, []),
     "redmetal_topk_last_error": (C.c_char_p, []),

@@ -63,6 +63,45 @@ __global__ __launch_bounds__(256) void calibration_copy_kernel(uint4 *dst, const
 }
 // nothing at all: what a launch of a given grid costs by itself
 __global__ void calibration_empty_kernel(int) {}
+
+// Streaming read of known size: every lane keeps eight 16-byte loads in flight, nothing is written unless the XOR of everything
+// read is a value the caller chose (so the loads cannot be dropped). The machine's own read rate beside the published 8 TB/s.
+__global__ __launch_bounds__(256) void calibration_read_kernel(const uint4 *src, uint64_t n16, uint32_t *sink, uint32_t magic) {
+    const uint64_t nthr = (uint64_t)gridDim.x * blockDim.x, t = (uint64_t)blockIdx.x * blockDim.x + threadIdx.x;
+    uint4 acc = make_uint4(0u, 0u, 0u, 0u);
+    uint64_t i = t;
+    for (; i + 7u * nthr < n16; i += 8u * nthr) {
+        uint4 v[8];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) v[k] = src[i + (uint64_t)k * nthr];
+#pragma unroll
+        for (int k = 0; k < 8; ++k) { acc.x ^= v[k].x; acc.y ^= v[k].y; acc.z ^= v[k].z; acc.w ^= v[k].w; }
+    }
+    for (; i < n16; i += nthr) { const uint4 v = src[i]; acc.x ^= v.x; acc.y ^= v.y; acc.z ^= v.z; acc.w ^= v.w; }
+    const uint32_t h = acc.x ^ acc.y ^ acc.z ^ acc.w;
+    if (h == magic) sink[0] = h;
+}
+
+// Dense fp16 matrix-core loop: every wave issues `iters` rounds of eight independent v_mfma_f32_16x16x32_f16 on operands that stay in
+// registers (no memory traffic at all); 16 * 16 * 32 * 2 flops each. The machine's own MFMA rate beside the published 2.5 PFLOP/s.
+typedef _Float16 cal_half8 __attribute__((ext_vector_type(8)));
+typedef float cal_float4 __attribute__((ext_vector_type(4)));
+__global__ __launch_bounds__(256) void calibration_mfma_kernel(uint32_t iters, float seed, float *sink) {
+    cal_half8 a, b;
+#pragma unroll
+    for (int i = 0; i < 8; ++i) { a[i] = (_Float16)(seed * (float)(threadIdx.x % 7u + i)); b[i] = (_Float16)(seed * (float)(threadIdx.x % 5u + i)); }
+    cal_float4 c[8];
+#pragma unroll
+    for (int k = 0; k < 8; ++k) c[k] = cal_float4{0.0f, 0.0f, 0.0f, 0.0f};
+    for (uint32_t it = 0; it < iters; ++it) {
+#pragma unroll
+        for (int k = 0; k < 8; ++k) c[k] = __builtin_amdgcn_mfma_f32_16x16x32_f16(a, b, c[k], 0, 0, 0);
+    }
+    float tot = 0.0f;
+#pragma unroll
+    for (int k = 0; k < 8; ++k) tot += c[k][0] + c[k][1] + c[k][2] + c[k][3];
+    if (tot == 12345.678f) sink[0] = tot;
+}
 }  // namespace redhip
 
 extern "C" {
@@ -105,6 +144,22 @@ int redhip_calibration_copy(void *dst_dev, const void *src_dev, uint64_t bytes, 
     redhip::prof_set_stage(redhip::ST_OTHER);
     REDHIP_LAUNCH(redhip::calibration_copy_kernel, dim3(2048), dim3(256), 0, static_cast<hipStream_t>(stream), static_cast<uint4 *>(dst_dev),
                   static_cast<const uint4 *>(src_dev), bytes / 16u);
+    return hipGetLastError() == hipSuccess;
+}
+
+int redhip_calibration_read(const void *src_dev, uint64_t bytes, void *sink_dev, void *stream) {
+    if (!src_dev || !sink_dev || !bytes || bytes % 16u) return 0;
+    redhip::prof_set_stage(redhip::ST_OTHER);
+    REDHIP_LAUNCH(redhip::calibration_read_kernel, dim3(4096), dim3(256), 0, static_cast<hipStream_t>(stream), static_cast<const uint4 *>(src_dev),
+                  bytes / 16u, static_cast<uint32_t *>(sink_dev), 0x9e3779b9u);
+    return hipGetLastError() == hipSuccess;
+}
+
+int redhip_calibration_mfma(uint32_t grid, uint32_t iters, void *sink_dev, uint64_t *flops, void *stream) {
+    if (!grid || !iters || !sink_dev) return 0;
+    redhip::prof_set_stage(redhip::ST_OTHER);
+    REDHIP_LAUNCH(redhip::calibration_mfma_kernel, dim3(grid), dim3(256), 0, static_cast<hipStream_t>(stream), iters, 0.0f, static_cast<float *>(sink_dev));
+    if (flops) *flops = (uint64_t)grid * 4u * iters * 8u * (2ull * 16u * 16u * 32u);      // four waves per workgroup
     return hipGetLastError() == hipSuccess;
 }
 

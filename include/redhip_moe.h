@@ -160,6 +160,12 @@ int redhip_profile_end(double *stage_ms, uint32_t *stage_launches, uint32_t n_st
  * `bytes` bytes (a multiple of 16), reading and writing exactly that much. Memory-traffic counters collected for
  * the kernels above are scaled by what they read for this kernel of known size. */
 int redhip_calibration_copy(void *dst_dev, const void *src_dev, uint64_t bytes, void *stream);
+/* The machine's own yardsticks (the counterpart of the reference's kernel-bench, native/redmetal_engine_selftest.m:295-462): a
+ * streaming read of `bytes` bytes (a multiple of 16; nothing is written; sink_dev: four bytes of device memory), and a dense fp16
+ * matrix-core loop on register operands (`grid` workgroups of four waves, `iters` rounds of eight 16x16x32 MFMAs per wave;
+ * *flops = what the launch computes). Time them with events around the call or with the stage profile above. */
+int redhip_calibration_read(const void *src_dev, uint64_t bytes, void *sink_dev, void *stream);
+int redhip_calibration_mfma(uint32_t grid, uint32_t iters, void *sink_dev, uint64_t *flops, void *stream);
 /* Launch-cost calibration (no counterpart in the reference): one launch of `grid` workgroups of `block` lanes of a kernel that does
  * nothing. A chain of such launches with a path's grids is the time the path's dependent launches cost before any work. */
 int redhip_calibration_empty(uint32_t grid, uint32_t block, void *stream);
