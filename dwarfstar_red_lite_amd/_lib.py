@@ -4,7 +4,8 @@ import ctypes as C
 import os
 
 HERE = os.path.dirname(os.path.abspath(__file__))
-LIB_PATH = os.path.join(HERE, "libredmetal_hip.so")
+# REDHIP_LIBRARY: another build of the same library (the one with phase stamps, build.py --timeline)
+LIB_PATH = os.environ.get("REDHIP_LIBRARY") or os.path.join(HERE, "libredmetal_hip.so")
 
 
 class RedHipError(RuntimeError):
@@ -79,6 +80,7 @@ ABI = {
     "redhip_profile_stage_name": (C.c_char_p, [u32]),
     "redhip_profile_begin": (i32, []),
     "redhip_profile_end": (i32, [C.POINTER(dbl), C.POINTER(u32), u32]),
+    "redhip_timeline_read": (i32, [C.POINTER(u64), u32, u32]),
     "redhip_calibration_copy": (i32, [vp, vp, u64, vp]),
     "redhip_calibration_empty": (i32, [u32, u32, vp]),
     "redhip_calibration_read": (i32, [vp, u64, vp, vp]),

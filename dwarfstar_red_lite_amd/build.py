@@ -31,9 +31,14 @@ def _stale(obj, src, deps):
     return any(os.path.getmtime(d) > t for d in [src] + deps)
 
 
-def build_library(verbose=False, incremental=False):
-    """incremental: recompile only the sources that changed (or whose headers did) since their object was built"""
+def build_library(verbose=False, incremental=False, timeline=False):
+    """incremental: recompile only the sources that changed (or whose headers did) since their object was built.
+    timeline: a second library, libredmetal_hip_timeline.so, whose expert kernels store phase stamps (-DREDHIP_TIMELINE; see
+    redhip_timeline_read); load it by pointing REDHIP_LIBRARY at it. The ordinary library is not touched."""
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
+    OBJ = os.path.join(HERE, "build_timeline" if timeline else "build")
+    LIB = os.path.join(HERE, "libredmetal_hip_timeline.so" if timeline else "libredmetal_hip.so")
+    FLAGS = globals()["FLAGS"] + (["-DREDHIP_TIMELINE"] if timeline else [])
     os.makedirs(OBJ, exist_ok=True)
     headers = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")]
     headers += [os.path.join(HERE, "..", "include", f) for f in os.listdir(os.path.join(HERE, "..", "include")) if f.endswith(".h")]
@@ -53,4 +58,4 @@ def build_library(verbose=False, incremental=False):
 
 
 if __name__ == "__main__":
-    print(build_library(verbose=True, incremental="--incremental" in sys.argv))
+    print(build_library(verbose=True, incremental="--incremental" in sys.argv, timeline="--timeline" in sys.argv))

@@ -34,6 +34,31 @@
 
 namespace redhip {
 
+// ---- in-kernel phase stamps (only in a library built with -DREDHIP_TIMELINE; the counterpart of the reference's RL_ENGINE_PROFILE for what
+// happens inside one launch) ----
+// REDHIP_STAMP(slot) in a kernel: lane 0 of the workgroup stores the 100 MHz wall clock into timeline[workgroup][slot] (workgroup = its
+// linear index in the grid, the first kTimelineGroups of them; slot < kTimelineSlots; slot kTimelineSlots - 1 holds the compute unit the
+// workgroup ran on, slots 13 and 14 the shader clock counter at stamps 3 and 4: with the wall clock of the same stamps, the clock rate).
+// redhip_timeline_read copies the array out. Without the flag the macro is empty and the array does not exist.
+[[maybe_unused]] constexpr uint32_t kTimelineGroups = 2048u, kTimelineSlots = 16u;
+#if defined(REDHIP_TIMELINE) && defined(__HIPCC__)
+__device__ unsigned long long g_timeline[kTimelineGroups * kTimelineSlots];      // (device symbols are private to a source file here: the stamps and their reader live in this one)
+__device__ __forceinline__ void timeline_stamp(uint32_t slot) {
+    if (threadIdx.x == 0u) {
+        const uint32_t wg = (blockIdx.z * gridDim.y + blockIdx.y) * gridDim.x + blockIdx.x;
+        if (wg < kTimelineGroups) {
+            g_timeline[wg * kTimelineSlots + slot] = wall_clock64();
+            if (slot == 0u) g_timeline[wg * kTimelineSlots + kTimelineSlots - 1u] = __smid();
+            if (slot == 3u || slot == 4u) g_timeline[wg * kTimelineSlots + 10u + slot] = clock64();      // slots 13, 14: the shader clock around one phase
+        }
+    }
+}
+#define REDHIP_STAMP(slot) ::redhip::timeline_stamp(slot)
+#else
+#define REDHIP_STAMP(slot) do {} while (0)
+#endif
+
+
 
 
 // ---------------------------------------------------------------- repacking (upload time)
@@ -1447,9 +1472,9 @@ __device__ __forceinline__ uint64_t iq3s_sliced_index(uint32_t g, uint32_t r, ui
 #endif
 }
 // LDS table: the four bytes of every grid entry as fp16; built by the first 512 lanes of a workgroup
-__device__ __forceinline__ void build_iq3s_quads(uint8_t *lds, uint32_t tid) {
+__device__ __forceinline__ uint32_t iq3s_quads_seed(uint32_t tid) { return tid < 512u ? redhip_iq3s_grid[tid] : 0u; }
+__device__ __forceinline__ void build_iq3s_quads_from(uint8_t *lds, uint32_t tid, uint32_t e) {
     if (tid < 512u) {
-        const uint32_t e = redhip_iq3s_grid[tid];
         uint32_t w2[2];
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
@@ -1459,6 +1484,7 @@ __device__ __forceinline__ void build_iq3s_quads(uint8_t *lds, uint32_t tid) {
         *reinterpret_cast<uint2 *>(lds + (size_t)tid * 8u) = make_uint2(w2[0], w2[1]);
     }
 }
+__device__ __forceinline__ void build_iq3s_quads(uint8_t *lds, uint32_t tid) { build_iq3s_quads_from(lds, tid, iq3s_quads_seed(tid)); }
 
 // 32 weights (one uint4 of words) against an activation operand that carries one token (rows 0, 1 = hi, lo) or two (rows 2, 3 the
 // second): va = first token's product, vb = the second's; scale nibble applied, d is not.
@@ -1527,15 +1553,21 @@ struct SliceArgs {
 // wave's own strip entries is read: no workgroup barrier inside.
 constexpr uint32_t kSignBytes = 128u * 16u;
 // SREP: copies of the sign table (16, or 8 where LDS is short: lanes l and l + 8 then share a copy and sometimes collide)
+// The grid entry a lane turns into its strip entry comes from device memory: table_seed requests it (a kernel whose routing arrives by
+// a load of its own asks for the seed first, so that both round trips are one), build_tables_rep_from does the rest.
+template <int NB>
+__device__ __forceinline__ uint64_t table_seed(uint32_t bw, uint32_t lane) {
+    constexpr uint32_t kOwn = 256u / NB;
+    return (bw < (uint32_t)NB && lane < kOwn) ? redhip_iq2xxs_grid[bw * kOwn + lane] : 0ull;
+}
 template <int REP, int NB, int SREP = REP>
-__device__ __forceinline__ void build_tables_rep(uint8_t *lds, uint8_t *strip, uint32_t bw, uint32_t lane) {
+__device__ __forceinline__ void build_tables_rep_from(uint8_t *lds, uint8_t *strip, uint32_t bw, uint32_t lane, uint64_t grid_entry) {
     static_assert((REP == 16 || REP == 8) && (SREP == 16 || SREP == 8 || SREP == 0) && (NB == 8 || NB == 16), "replication layout");
     if (bw >= (uint32_t)NB) return;
     constexpr uint32_t kOwn = 256u / NB, kOwnS = 128u / NB;      // entries of this wave
     uint8_t *sign_lds = lds + REP * kMagBytes, *sign_strip = strip + kMagBytes;
     if (lane < kOwn) {
         const uint32_t idx = bw * kOwn + lane;
-        const uint64_t grid_entry = redhip_iq2xxs_grid[idx];
         uint32_t w4[4];
 #pragma unroll
         for (int i = 0; i < 4; ++i) {
@@ -1568,6 +1600,10 @@ __device__ __forceinline__ void build_tables_rep(uint8_t *lds, uint8_t *strip, u
         }
     }
 }
+template <int REP, int NB, int SREP = REP>
+__device__ __forceinline__ void build_tables_rep(uint8_t *lds, uint8_t *strip, uint32_t bw, uint32_t lane) {
+    build_tables_rep_from<REP, NB, SREP>(lds, strip, bw, lane, table_seed<NB>(bw, lane));
+}
 // eight signed fp16 weights from the two replicated tables; `tab` / `stab` = base of the magnitude / sign table + this lane's copy offset
 template <int REP, int SREP>
 __device__ __forceinline__ void signed_weights_rep(const uint8_t *tab, const uint8_t *stab, uint32_t idx, uint32_t s7, WeightQuad &b0, WeightQuad &b1) {
@@ -1593,6 +1629,110 @@ __device__ __forceinline__ float group_dot_rep(uint2 q, const half4_t *ax, const
     return (acc[0] + acc[1] * 4.8828125e-4f) * (float)(2u * (q.y >> 28) + 1u);
 }
 
+// Signs from a small table instead of a table of whole masks: entry s7 is ONE word that holds the eight sign bits of the field (the eighth
+// = its parity) where shifts of 0..3 put them on the fp16 sign positions of the four weight pairs - bit 15 - i / 31 - i = sign of weight
+// 2 i / 2 i + 1. A pair of signed weights is then (entry << i) & 0x80008000 | magnitudes: seven operations per eight weights and a 4-byte
+// read, against a 16-byte read and four XORs for the table of masks, or thirteen operations without a table.
+// LR copies of every entry side by side (entry s7, copy c at (s7 * LR + c) * 4), lane l reads copy l % LR.
+__device__ __forceinline__ uint32_t spread_signs(uint32_t s7) {
+    const uint32_t s8 = s7 | ((__popc(s7) & 1u) << 7);
+    uint32_t e = 0u;
+#pragma unroll
+    for (uint32_t i = 0; i < 4u; ++i) e |= (((s8 >> (2u * i)) & 1u) << (15u - i)) | (((s8 >> (2u * i + 1u)) & 1u) << (31u - i));
+    return e;
+}
+template <int LR>      // written by `builders` lanes starting at lane `first` of the workgroup (lanes before `first` wrap past the bound and write nothing)
+__device__ __forceinline__ void build_sign_lut(uint32_t *lut, uint32_t tid, uint32_t first = 0u, uint32_t builders = (uint32_t)kWaves * 64u) {
+    for (uint32_t n = tid - first; n < 128u * LR; n += builders) lut[n] = spread_signs(n / LR);
+}
+// The same words as data, for kernels that would rather request a word early than compute it (thirty operations per word)
+struct SignWordTable { uint32_t w[128]; };
+constexpr SignWordTable make_sign_words() {
+    SignWordTable t{};
+    for (uint32_t s7 = 0; s7 < 128u; ++s7) {
+        uint32_t par = 0u;
+        for (uint32_t b = 0; b < 7u; ++b) par ^= (s7 >> b) & 1u;
+        const uint32_t s8 = s7 | (par << 7);
+        uint32_t e = 0u;
+        for (uint32_t i = 0; i < 4u; ++i) e |= (((s8 >> (2u * i)) & 1u) << (15u - i)) | (((s8 >> (2u * i + 1u)) & 1u) << (31u - i));
+        t.w[s7] = e;
+    }
+    return t;
+}
+__device__ const SignWordTable redhip_sign_words = make_sign_words();
+// Where the two tables lie for a lane, as 32-bit LDS addresses with the lane's copy offset added in. The copy offsets occupy the address
+// bits below the entry index and the table bases the bits above it - magnitudes (64 KB-aligned): entry << 8 | (lane % 16) << 4; sign
+// words (aligned to their size): field << (2 + log2 LR) | (lane % LR) << 2 - so that an address is one byte permute resp. a shift and an
+// and-or of the packed group word, with no add.
+struct LaneTables { uint32_t mag_lane, lut_lane; };
+typedef uint32_t lds_u32x4 __attribute__((ext_vector_type(4)));
+typedef __attribute__((address_space(3))) const lds_u32x4 *lds_u32x4_ptr;
+typedef __attribute__((address_space(3))) const uint32_t *lds_u32_ptr;
+__device__ __forceinline__ uint32_t lds_address(const void *p) { return (uint32_t)(uintptr_t)(__attribute__((address_space(3))) const void *)p; }
+template <int REP, int LR>
+__device__ __forceinline__ LaneTables lane_tables(const uint8_t *mag, const uint8_t *lut, uint32_t lane) {
+    static_assert(REP == 16 && (LR == 8 || LR == 16 || LR == 32), "address bit layout");
+    return LaneTables{lds_address(mag) + (lane % (uint32_t)REP) * 16u, lds_address(lut) + (lane % (uint32_t)LR) * 4u};
+}
+// eight signed weights: group word pair q, index / sign field L (0..3)
+template <int REP, int LR, uint32_t L>
+__device__ __forceinline__ void signed_weights_lut(const LaneTables &t, uint2 q, WeightQuad &b0, WeightQuad &b1) {
+    constexpr uint32_t kLutShift = LR == 8 ? 5u : LR == 16 ? 6u : 7u;      // log2 of the bytes per sign field
+    // bytes of the magnitude address: [low byte of the lane's base, index byte L of q.x, upper two bytes of the lane's base]
+    const uint32_t mag_at = __builtin_amdgcn_perm(q.x, t.mag_lane, 0x03020000u | ((4u + L) << 8));
+    const uint32_t field = 7u * L < kLutShift ? q.y << (kLutShift - 7u * L) : q.y >> (7u * L - kLutShift);
+    const uint32_t lut_at = (field & (127u << kLutShift)) | t.lut_lane;
+#ifdef EXP_NO_LDS
+    const lds_u32x4 m = {mag_at, lut_at, mag_at ^ 0x1234u, lut_at + 7u};
+    const uint32_t e = lut_at ^ mag_at;
+#else
+    const lds_u32x4 m = *reinterpret_cast<lds_u32x4_ptr>((uintptr_t)mag_at);
+    const uint32_t e = *reinterpret_cast<lds_u32_ptr>((uintptr_t)lut_at);
+#endif
+#ifdef EXP_NO_SIGN
+    b0.u[0] = m.x ^ e; b0.u[1] = m.y; b1.u[0] = m.z; b1.u[1] = m.w;
+#else
+    b0.u[0] = (e & 0x80008000u) | m.x;
+    b0.u[1] = ((e << 1) & 0x80008000u) | m.y;
+    b1.u[0] = ((e << 2) & 0x80008000u) | m.z;
+    b1.u[1] = ((e << 3) & 0x80008000u) | m.w;
+#endif
+}
+template <int REP, int LR, uint32_t L>
+__device__ __forceinline__ float4_t group_step_lut(const LaneTables &t, uint2 q, const half4_t *ax, float4_t acc) {
+    WeightQuad b0, b1;
+    signed_weights_lut<REP, LR, L>(t, q, b0, b1);
+#ifdef EXP_NO_MFMA
+    asm volatile("" :: "v"(b0.u[0]), "v"(b0.u[1]), "v"(b1.u[0]), "v"(b1.u[1]));
+    return acc;
+#else
+    acc = __builtin_amdgcn_mfma_f32_4x4x4f16(ax[2u * L], b0.h, acc, 0, 0, 0);
+    return __builtin_amdgcn_mfma_f32_4x4x4f16(ax[2u * L + 1u], b1.h, acc, 0, 0, 0);
+#endif
+}
+// group_dot / group_dot2 on the replicated magnitude table and the sign words
+template <int REP, int LR>
+__device__ __forceinline__ float4_t group_acc_lut(const LaneTables &t, uint2 q, const half4_t *ax) {
+    float4_t acc = {0.0f, 0.0f, 0.0f, 0.0f};
+    acc = group_step_lut<REP, LR, 0u>(t, q, ax, acc);
+    acc = group_step_lut<REP, LR, 1u>(t, q, ax, acc);
+    acc = group_step_lut<REP, LR, 2u>(t, q, ax, acc);
+    return group_step_lut<REP, LR, 3u>(t, q, ax, acc);
+}
+template <int REP, int LR>
+__device__ __forceinline__ float group_dot_lut(uint2 q, const half4_t *ax, const LaneTables &t) {
+    const float4_t acc = group_acc_lut<REP, LR>(t, q, ax);
+    return (acc[0] + acc[1] * 4.8828125e-4f) * (float)(2u * (q.y >> 28) + 1u);
+}
+template <int REP, int LR>
+__device__ __forceinline__ void group_dot2_lut(uint2 q, const half4_t *ax, const LaneTables &t, float &va, float &vb) {
+    const float4_t acc = group_acc_lut<REP, LR>(t, q, ax);
+    const float sc = (float)(2u * (q.y >> 28) + 1u);
+    va = (acc[0] + acc[1] * 4.8828125e-4f) * sc;
+    vb = (acc[2] + acc[3] * 4.8828125e-4f) * sc;
+}
+
+constexpr int kSliceLut = 32;      // copies of the sign words in the one-token kernel: 16 KB, every lane of a half wave its own bank
 template <int NKC, int REP>        // hidden = 512 * NKC
 __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(SliceArgs a) {
     constexpr int NW = kWaves;
@@ -1600,9 +1740,10 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(SliceArgs a) 
     constexpr int DU = (8 * NKC + NW - 1) / NW;        // units of 64 down rows per wave
     static_assert(UPW >= 1 && UPW * NW == 16 * NKC, "waves must tile the 16 row-quads x NKC chunks");
     extern __shared__ __attribute__((aligned(16))) uint8_t dyn[];
-    uint8_t *lds = dyn;                                                    // REP * (4 KB magnitude table + 2 KB sign masks)
-    uint8_t *strip = dyn + REP * (kMagBytes + kSignBytes);                 // 4 KB + 2 KB: the tables once, as their builders make them
-    float *part = reinterpret_cast<float *>(strip + kMagBytes + kSignBytes);      // [NKC][64]
+    uint8_t *lds = dyn;                                                    // REP copies of the 4 KB magnitude table
+    uint8_t *sign_lut = dyn + REP * kMagBytes;                             // kSliceLut copies of the 128 sign words (aligned to their size)
+    uint8_t *strip = sign_lut + 128u * 4u * kSliceLut;                     // 4 KB: the magnitude table once, as its builders make it
+    float *part = reinterpret_cast<float *>(strip + kMagBytes);            // [NKC][64]
     _Float16 *act_hl = reinterpret_cast<_Float16 *>(part + NKC * 64);      // [2][32]: hi, lo halves of the 32 activations
     float *act_scale = reinterpret_cast<float *>(act_hl + 64);             // [4]
     SelectOut *sel = reinterpret_cast<SelectOut *>(act_scale + 4);
@@ -1611,6 +1752,7 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(SliceArgs a) 
     const uint32_t H = a.hidden, F = a.ffn, HG = H / 32u, HB = H / 256u, FG = F / 32u;
     const uint32_t g = blockIdx.x, slot = blockIdx.y;
     const bool is_shared = slot >= a.top_k;
+    REDHIP_STAMP(0);
 
     // activation operand of the gate / up rows: independent of the routing, requested first
     const uint32_t kc = wave % NKC, q0 = wave / NKC;
@@ -1619,8 +1761,10 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(SliceArgs a) 
     load_act_operand(ax, a.xh + 32u * G, a.xl + 32u * G, j);
     // the table is first read behind the barrier that ends the selection: wave 0 selects, waves 8..15 build meanwhile
     const bool selecting = !is_shared && a.logits;
-    if (selecting) build_tables_rep<REP, 8>(lds, strip, wave - 8u, lane); else build_tables_rep<REP, 16>(lds, strip, wave, lane);
-    const uint8_t *tab = lds + (lane % REP) * 16u, *stab = tab + REP * kMagBytes;
+    // (and waves 1..7 write the sign words)
+    if (selecting) { build_tables_rep<REP, 8, 0>(lds, strip, wave - 8u, lane); if (wave < 8u) build_sign_lut<kSliceLut>(reinterpret_cast<uint32_t *>(sign_lut), tid, 64u, 7u * 64u); }
+    else { build_tables_rep<REP, 16, 0>(lds, strip, wave, lane); build_sign_lut<kSliceLut>(reinterpret_cast<uint32_t *>(sign_lut), tid); }
+    const LaneTables lt = lane_tables<REP, kSliceLut>(lds, sign_lut, lane);
 
     uint32_t expert = 0u;
     float comb;                                        // the slot's weight in the layer's output
@@ -1644,6 +1788,7 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(SliceArgs a) 
         comb = a.weights_in[slot];
         __syncthreads();                               // table
     }
+    REDHIP_STAMP(1);                                   // selection (or the caller's routing) and tables are here
     const uint8_t *ex = is_shared ? a.shared : a.experts + (uint64_t)expert * a.stride;
     const uint8_t *dn = is_shared ? a.shared_down_cm : a.down_cm + (uint64_t)expert * a.down_stride;
     const uint64_t gate_bytes = (uint64_t)F * HG * 8u + (uint64_t)F * HB * 2u;
@@ -1676,14 +1821,20 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(SliceArgs a) 
         dd[k] = down_ds[row];
     }
     float v[UPW];
+    REDHIP_STAMP(2);                                   // every weight requested
 #pragma unroll
-    for (int u = 0; u < UPW; ++u) v[u] = group_dot_rep<REP, REP>(wq[u], ax, tab, stab) * scale_to_f32(wd[u]);
+    for (int u = 0; u < UPW; ++u) {
+        v[u] = group_dot_lut<REP, kSliceLut>(wq[u], ax, lt) * scale_to_f32(wd[u]);
+        if (u == 0) REDHIP_STAMP(3);                   // the first unit's weights arrived and are multiplied
+    }
     const float tot = quad_column_reduce<UPW>(v, lane);
+    REDHIP_STAMP(4);                                   // gate / up rows of wave 0 multiplied
     if (reduced_writer<UPW>(lane)) {
         const uint32_t quad = q0 + (NW / NKC) * reduced_unit<UPW>(lane);
         part[kc * 64u + 4u * quad + j] = tot;
     }
     __syncthreads();
+    REDHIP_STAMP(5);                                   // ... of every wave
     if (tid < 32u) {
         float gsum = 0.0f, usum = 0.0f;
 #pragma unroll
@@ -1700,6 +1851,7 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(SliceArgs a) 
         if (tid == 0u) act_scale[0] = exp2i(e);
     }
     __syncthreads();
+    REDHIP_STAMP(6);                                   // activations exchanged
     // down slice: lane = output row of the unit, the 32 activations are the same operand for every lane block
     half4_t ad[8];
     {
@@ -1716,8 +1868,9 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(SliceArgs a) 
 #pragma unroll
     for (int k = 0; k < DU; ++k) {
         const uint32_t unit = wave + NW * k;
-        if (unit < 8u * NKC) out[64u * unit + lane] = group_dot_rep<REP, REP>(dq[k], ad, tab, stab) * scale_to_f32(dd[k]) * post;
+        if (unit < 8u * NKC) out[64u * unit + lane] = group_dot_lut<REP, kSliceLut>(dq[k], ad, lt) * scale_to_f32(dd[k]) * post;
     }
+    REDHIP_STAMP(7);                                   // down slice of wave 0 multiplied, stores issued
 }
 
 // out[r] = sum over slots (selection order, the shared expert last) and column groups of partial[slot][group][r] (+ the residual of the
@@ -1822,10 +1975,10 @@ __device__ __forceinline__ void group_dot2_rep(uint2 q, const half4_t *ax, const
 // at 8 tokens with 32 hot experts: this 27.7 us; eight copies of the magnitude table 28.3 us (38 % of its LDS cycles are bank
 // conflicts: the LDS serves sixteen lanes of a 16-byte read together); eight copies of both tables 34.3 us (a fifth fewer vector
 // instructions, 70 % more LDS reads); sixteen copies of both at one workgroup per compute unit 43.5 us.
-constexpr int kBatchRep = 16, kBatchSignRep = 0;
+constexpr int kBatchRep = 16, kBatchSignRep = 0, kBatchLut = 8;      // (kBatchLut copies of the 128 sign words: 4 KB)
 // LDS bytes of the decode tables at the head of the kernel's dynamic LDS
 template <int REP, int MIX> constexpr uint32_t batch_slice_table_bytes() {
-    return MIX == 2 ? 512u * 16u : MIX == 3 ? 2048u * 16u : (uint32_t)(REP + 1) * kMagBytes + (uint32_t)(kBatchSignRep + 1) * kSignBytes;
+    return MIX == 2 ? 512u * 16u : MIX == 3 ? 2048u * 16u : (uint32_t)(REP + 1) * kMagBytes + (uint32_t)kBatchSignRep * kSignBytes + 128u * 4u * (uint32_t)kBatchLut;
 }
 // MIX 0: every matrix packed IQ2_XXS; 1: IQ3_S down matrices, dense shared expert; 2 / 3: IQ2_XS / IQ1_M streams, dense shared expert (see BatchSliceArgs)
 template <int NKC, int REP, int MIX>
@@ -1837,28 +1990,43 @@ __global__ __launch_bounds__(kWaves * 64, 8) void batch_slice_kernel(BatchSliceA
     constexpr int FMT = MIX >= 2 ? MIX - 1 : 0;            // format of the routed matrices as group_dot_fmt2 numbers them
     extern __shared__ __attribute__((aligned(16))) uint8_t dyn[];
     uint8_t *lds = dyn;
-    uint8_t *strip = dyn + REP * kMagBytes + SREP * kSignBytes;
+    uint8_t *strip = dyn + REP * kMagBytes + SREP * kSignBytes;            // 4 KB: the magnitude table once, as its builders make it
+    uint8_t *sign_lut = strip + kMagBytes;                                 // kBatchLut copies of the sign words
     float *part = reinterpret_cast<float *>(dyn + batch_slice_table_bytes<REP, MIX>());      // [2 tokens][NKC][64]
     _Float16 *act_hl = reinterpret_cast<_Float16 *>(part + 2 * NKC * 64);  // [2 tokens][2 halves][32]
     float *act_scale = reinterpret_cast<float *>(act_hl + 128);            // [2] (+ 2 unused)
     uint8_t *iq3_tab = reinterpret_cast<uint8_t *>(act_scale + 4);         // MIX: 4 KB, the IQ3_S grid as fp16
 
-    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
+    const uint32_t tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63u, blk = lane >> 2, j = lane & 3u;      // (wave: in a scalar register)
     const uint32_t H = a.hidden, F = a.ffn, HG = H / 32u, HB = H / 256u, FG = F / 32u, K = a.top_k;
     const uint32_t g = blockIdx.x, v = blockIdx.y;
+    REDHIP_STAMP(0);
+    // Three requests leave together, so that the workgroup waits for one round trip before it knows its weights' addresses: the number of
+    // passes, this workgroup's entry of the pass list (read whether or not it turns out to be one: the index is clamped into the list) and
+    // the codebook entries its lanes turn into the LDS tables. The tables are then written while the weights are on their way: loads
+    // return in order, so a table seed requested behind the weights would not be usable before they have all arrived.
+    const uint32_t n_pairs = a.ntok * K;
     const uint32_t n_pass = a.n_pass[0];
+    uint2 e = a.pass_list[v < n_pairs ? v : n_pairs - 1u];
+    uint64_t seed_cb[2] = {0ull, 0ull};
+    uint64_t seed_mag = 0ull;
+    uint32_t seed_q3 = 0u;
+    uint32_t seed_sign = 0u;                           // kBatchLut = 8 copies of 128 words: one word per lane of the workgroup
+    static_assert(kBatchLut * 128 == kWaves * 64, "one sign word per lane");
+    if constexpr (MIX >= 2) codebook_seed<FMT>(tid, a.grid, seed_cb);
+    else { seed_mag = table_seed<16>(wave, lane); seed_sign = redhip_sign_words.w[tid / (uint32_t)kBatchLut]; }
+    if constexpr (MIX == 1) seed_q3 = iq3s_quads_seed(tid);
     if (v >= n_pass + ((a.ntok + 1u) >> 1)) return;    // the grid covers the largest possible number of passes
     const bool sh = v >= n_pass;
-    uint2 e;
     if (sh) {                                          // the shared expert: tokens 2 s, 2 s + 1; k = top_k
         const uint32_t t0 = 2u * (v - n_pass), t1 = t0 + 1u < a.ntok ? t0 + 1u : t0;
         e.x = 0xffffu | ((t0 + 1u < a.ntok ? 2u : 1u) << 16);
         e.y = (t0 << 16) | (t1 << 24);
-    } else {
-        e = a.pass_list[v];
-        if (((e.x >> 16) & 255u) < 2u) e.y = (e.y & 0x00ff00ffu) * 0x101u;      // a lone token: its twin computes the same and is not stored
+    } else if (((e.x >> 16) & 255u) < 2u) {
+        e.y = (e.y & 0x00ff00ffu) * 0x101u;            // a lone token: its twin computes the same and is not stored
     }
     const uint32_t expert = e.x & 0xffffu, cnt = (e.x >> 16) & 255u, tok0 = (e.y >> 16) & 255u, tok1 = e.y >> 24;
+    REDHIP_STAMP(1);                                   // the pass entry is here
     const uint32_t k0 = sh ? K : (e.y & 255u) - tok0 * K, k1 = sh ? K : ((e.y >> 8) & 255u) - tok1 * K;
     float *out0 = a.partial + ((uint64_t)(tok0 * (K + 1u) + k0) * FG + g) * H, *out1 = a.partial + ((uint64_t)(tok1 * (K + 1u) + k1) * FG + g) * H;
 
@@ -1920,50 +2088,57 @@ __global__ __launch_bounds__(kWaves * 64, 8) void batch_slice_kernel(BatchSliceA
     for (int u = 0; u < UPW; ++u) {
         const uint32_t quad = q0 + (NW / NKC) * u;
         const uint32_t r = 32u * g + 4u * (quad & 7u) + j;
-        const uint8_t *mat = ex + (quad < 8u ? 0u : gate_bytes);
-        wq[u] = reinterpret_cast<const uint2 *>(mat)[(uint64_t)r * HG + G];
-        wd[u] = reinterpret_cast<const uint16_t *>(mat + (uint64_t)F * HG * 8u)[(uint64_t)r * HB + (G >> 3)];
-        if constexpr (MIX == 2) wd[u] |= (uint32_t)(mat + gate_sc)[(uint64_t)r * HG + G] << 16;
+        const uint8_t *mat = ex + (quad < 8u ? 0u : gate_bytes);         // (the same in every lane of the wave; a matrix is far below 4 GB: 32-bit offsets)
+        wq[u] = *reinterpret_cast<const uint2 *>(mat + (r * HG + G) * 8u);
+        wd[u] = *reinterpret_cast<const uint16_t *>(mat + (F * HG * 8u + (r * HB + (G >> 3)) * 2u));
+        if constexpr (MIX == 2) wd[u] |= (uint32_t)mat[(uint32_t)gate_sc + r * HG + G] << 16;
     }
     using DownGroup = typename std::conditional<MIX == 1, uint4, uint2>::type;      // one row's 32 weights of the slice
-    const DownGroup *down_qs = reinterpret_cast<const DownGroup *>(dn) + (MIX == 1 ? 0u : (uint64_t)g * H);
-    const uint16_t *down_ds = reinterpret_cast<const uint16_t *>(dn + (uint64_t)FG * H * sizeof(DownGroup)) + (uint64_t)(g >> 3) * H;
-    const uint8_t *down_sc = dn + (uint64_t)FG * H * 8u + (uint64_t)(FG >> 3) * H * 2u + (uint64_t)g * H;      // MIX 2
+    const uint8_t *down_qs = dn + (MIX == 1 ? 0u : g * H * (uint32_t)sizeof(DownGroup));
+    const uint8_t *down_ds = dn + (FG * H * (uint32_t)sizeof(DownGroup) + (g >> 3) * H * 2u);
+    const uint8_t *down_sc = dn + (FG * H * 8u + (FG >> 3) * H * 2u + g * H);      // MIX 2
     DownGroup dq[DU];
     uint32_t dd[DU];                                     // as wd
 #pragma unroll
     for (int kk = 0; kk < DU; ++kk) {
         const uint32_t unit = wave + NW * kk;
         const uint32_t r = 64u * (unit < 8u * NKC ? unit : 0u) + lane;
-        dq[kk] = down_qs[MIX == 1 ? iq3s_sliced_index(g, r, FG, H) : (uint64_t)r];
-        dd[kk] = down_ds[r];
+        dq[kk] = *reinterpret_cast<const DownGroup *>(down_qs + (MIX == 1 ? (uint32_t)iq3s_sliced_index(g, r, FG, H) : r) * (uint32_t)sizeof(DownGroup));
+        dd[kk] = *reinterpret_cast<const uint16_t *>(down_ds + r * 2u);
         if constexpr (MIX == 2) dd[kk] |= (uint32_t)down_sc[r] << 16;
     }
-    if constexpr (MIX == 1) build_iq3s_quads(iq3_tab, tid);
+    if constexpr (MIX == 1) build_iq3s_quads_from(iq3_tab, tid, seed_q3);
     const float w0 = sh ? a.scalar[tok0] : a.weights[tok0 * K + k0], w1 = sh ? a.scalar[tok1] : a.weights[tok1 * K + k1];
     // (an IQ1_M weight is d (2 s + 1) (entry +- 1/8): no 1 / 8)
     const float xs0 = (MIX == 3 ? 1.0f : 0.125f) * exp2i(a.xexp[tok0]), xs1 = (MIX == 3 ? 1.0f : 0.125f) * exp2i(a.xexp[tok1]);
-    if constexpr (MIX >= 2) build_codebook_table<FMT>(lds, tid, a.grid, 0u, (uint32_t)NW * 64u);
-    else build_tables_rep<REP, 16, SREP>(lds, strip, wave, lane);
-    const uint8_t *tab = lds + (lane % REP) * 16u, *stab = lds + REP * kMagBytes + (lane % (SREP ? SREP : 1)) * 16u;
+    if constexpr (MIX >= 2) build_codebook_table_from<FMT>(lds, tid, seed_cb);
+    else {
+        build_tables_rep_from<REP, 16, SREP>(lds, strip, wave, lane, seed_mag);
+        reinterpret_cast<uint32_t *>(sign_lut)[tid] = seed_sign;
+    }
+    const LaneTables lt = lane_tables<REP, kBatchLut>(lds, sign_lut, lane);
+    REDHIP_STAMP(2);                                   // loads requested, tables written
     __syncthreads();                                   // tables
+    REDHIP_STAMP(3);
 
     float va[UPW], vb[UPW];
 #pragma unroll
     for (int u = 0; u < UPW; ++u) {
         if constexpr (MIX >= 2) group_dot_fmt2<FMT>(wq[u], wd[u] >> 16, ax, lds, va[u], vb[u]);
-        else group_dot2_rep<REP, SREP>(wq[u], ax, tab, stab, va[u], vb[u]);
+        else group_dot2_lut<REP, kBatchLut>(wq[u], ax, lt, va[u], vb[u]);
         const float d = scale_to_f32(wd[u]);
         va[u] *= d;
         vb[u] *= d;
     }
     const float ta = quad_column_reduce<UPW>(va, lane), tb = quad_column_reduce<UPW>(vb, lane);
+    REDHIP_STAMP(4);                                   // gate / up rows of wave 0 multiplied
     if (reduced_writer<UPW>(lane)) {
         const uint32_t quad = q0 + (NW / NKC) * reduced_unit<UPW>(lane);
         part[kc * 64u + 4u * quad + j] = ta;
         part[NKC * 64u + kc * 64u + 4u * quad + j] = tb;
     }
     __syncthreads();
+    REDHIP_STAMP(5);                                   // ... of every wave
     if (tid < 64u) {
         const uint32_t t = tid >> 5, c = tid & 31u;
         const float *pt = part + t * NKC * 64u;
@@ -1982,6 +2157,7 @@ __global__ __launch_bounds__(kWaves * 64, 8) void batch_slice_kernel(BatchSliceA
         if (c == 0u) act_scale[t] = exp2i(ee);
     }
     __syncthreads();
+    REDHIP_STAMP(6);                                   // activations exchanged
     half4_t ad[8];
     {
         const _Float16 *src = act_hl + (j >> 1) * 64u + (j & 1u) * 32u;
@@ -1997,16 +2173,17 @@ __global__ __launch_bounds__(kWaves * 64, 8) void batch_slice_kernel(BatchSliceA
             float da, db;
             if constexpr (MIX == 1) iq3s_group_dot(dq[kk], ad, iq3_tab, da, db);
             else if constexpr (MIX >= 2) group_dot_fmt2<FMT>(dq[kk], dd[kk] >> 16, ad, lds, da, db);
-            else group_dot2_rep<REP, SREP>(dq[kk], ad, tab, stab, da, db);
+            else group_dot2_lut<REP, kBatchLut>(dq[kk], ad, lt, da, db);
             const float d = scale_to_f32(dd[kk]);
             out0[64u * unit + lane] = da * d * post0;
             if (cnt > 1u) out1[64u * unit + lane] = db * d * post1;
         }
     }
+    REDHIP_STAMP(7);                                   // down slice of wave 0 multiplied, stores issued
 }
 
 constexpr int kSliceRep = 16;
-inline size_t slice_lds_bytes(int nkc, int rep) { return (size_t)(rep + 1) * (kMagBytes + kSignBytes) + (size_t)nkc * 64u * 4u + 128u + 16u + sizeof(SelectOut); }
+inline size_t slice_lds_bytes(int nkc, int rep) { return (size_t)(rep + 1) * kMagBytes + 128u * 4u * (size_t)kSliceLut + (size_t)nkc * 64u * 4u + 128u + 16u + sizeof(SelectOut); }
 
 hipError_t launch_expert_slices(const void *experts, uint64_t stride, const void *down_cm, uint64_t down_stride, const void *shared, const void *shared_down_cm,
                                 const float *logits, const uint32_t *ids_in, const float *weights_in, const float *scalar_in, uint32_t *ids_out,
@@ -3199,3 +3376,20 @@ hipError_t launch_gateup_select(const void *experts, uint64_t stride, const void
 }
 
 }  // namespace redhip
+
+extern "C" int redhip_timeline_read(uint64_t *stamps, uint32_t n_groups, uint32_t clear) {
+#ifdef REDHIP_TIMELINE
+    if (!stamps || !n_groups || n_groups > redhip::kTimelineGroups) return 0;
+    if (hipDeviceSynchronize() != hipSuccess) return 0;
+    const size_t bytes = (size_t)n_groups * redhip::kTimelineSlots * sizeof(uint64_t);
+    if (hipMemcpyFromSymbol(stamps, HIP_SYMBOL(redhip::g_timeline), bytes) != hipSuccess) return 0;
+    if (clear) {
+        void *p = nullptr;
+        if (hipGetSymbolAddress(&p, HIP_SYMBOL(redhip::g_timeline)) != hipSuccess || hipMemset(p, 0, sizeof(uint64_t) * redhip::kTimelineGroups * redhip::kTimelineSlots) != hipSuccess) return 0;
+    }
+    return 1;
+#else
+    (void)stamps; (void)n_groups; (void)clear;
+    return 0;                                            // this library was built without the phase stamps
+#endif
+}

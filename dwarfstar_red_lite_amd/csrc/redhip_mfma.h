@@ -80,5 +80,31 @@ __device__ __forceinline__ void build_codebook_table(uint8_t *lds, uint32_t tid,
         *reinterpret_cast<uint4 *>(lds + (size_t)i * 16u) = make_uint4(w4[0], w4[1], w4[2], w4[3]);
     }
 }
+// The same table built by all 1024 lanes of a workgroup in two steps: codebook_seed requests a lane's entries (tid, and tid + 1024 for the
+// 2048-entry codebook), build_codebook_table_from converts and stores them - for kernels that want the request in flight early.
+template <int FMT>
+__device__ __forceinline__ void codebook_seed(uint32_t tid, const int8_t *grid, uint64_t (&seed)[2]) {
+    constexpr uint32_t kEntries = FMT == 1 ? 512u : 2048u;
+    seed[0] = tid < kEntries ? reinterpret_cast<const uint64_t *>(grid)[tid] : 0ull;
+    seed[1] = tid + 1024u < kEntries ? reinterpret_cast<const uint64_t *>(grid)[tid + 1024u] : 0ull;
+}
+template <int FMT>
+__device__ __forceinline__ void build_codebook_table_from(uint8_t *lds, uint32_t tid, const uint64_t (&seed)[2]) {
+    constexpr uint32_t kEntries = FMT == 1 ? 512u : 2048u;
+#pragma unroll
+    for (uint32_t r = 0; r < 2u; ++r) {
+        const uint32_t i = tid + 1024u * r;
+        if (i < kEntries) {
+            const uint64_t e = seed[r];
+            uint32_t w4[4];
+#pragma unroll
+            for (int k = 0; k < 4; ++k) {
+                const _Float16 lo = (_Float16)(float)(int8_t)(e >> (16 * k)), hi = (_Float16)(float)(int8_t)(e >> (16 * k + 8));
+                w4[k] = (uint32_t)__builtin_bit_cast(uint16_t, lo) | ((uint32_t)__builtin_bit_cast(uint16_t, hi) << 16);
+            }
+            *reinterpret_cast<uint4 *>(lds + (size_t)i * 16u) = make_uint4(w4[0], w4[1], w4[2], w4[3]);
+        }
+    }
+}
 
 }  // namespace redhip

@@ -156,6 +156,11 @@ uint32_t redhip_profile_stage_count(void);
 const char *redhip_profile_stage_name(uint32_t stage);
 int redhip_profile_begin(void);
 int redhip_profile_end(double *stage_ms, uint32_t *stage_launches, uint32_t n_stage);
+/* Phase stamps inside the expert kernels (no counterpart in the reference's C surface; its RL_ENGINE_PROFILE stops at whole stages): a
+ * library built with -DREDHIP_TIMELINE (python dwarfstar_red_lite_amd/build.py --timeline) stores, per workgroup of the last expert launch,
+ * the 100 MHz wall clock at every phase boundary: stamps[workgroup * 16 + slot], slot 15 = the compute unit. Synchronises the device.
+ * Returns 0 in an ordinary build. */
+int redhip_timeline_read(uint64_t *stamps, uint32_t n_groups, uint32_t clear);
 /* Counter calibration (no counterpart in the reference): one plain copy kernel, dst_dev[i] = src_dev[i] for
  * `bytes` bytes (a multiple of 16), reading and writing exactly that much. Memory-traffic counters collected for
  * the kernels above are scaled by what they read for this kernel of known size. */
