@@ -75,7 +75,15 @@ struct Moe {
     bool packed_gu() const { return fused || mixed; }
     // every path of an all-IQ2_XXS handle of these shapes reads the packed copies: the raw GGUF rows of the routed experts only pass
     // through a staging buffer at upload
-    bool keep_raw() const { return !(fused && cfg.hidden / 512u <= 4u); }
+    // So do the mixed layouts whose batches run as expert slices, when every size they can be given has kernels on the packed copies:
+    // one token (packed gate | up, word- or stream-packed down), 2..8 tokens (slices), 9..16 (two small batches), larger chunks only
+    // with the tile-major copies (a handle made for more than 16 tokens on a shape without tile kernels keeps the raw rows for the
+    // raw-row kernels). Any kernel that would read raw rows on such a handle is refused on the host (raw_rows below).
+    bool keep_raw() const {
+        if (fused && cfg.hidden / 512u <= 4u) return false;
+        if (mixed_slices && (cfg.max_tokens <= 2u * kSlice || (sliced_words() ? tiles_resident() : stream_tiles_resident()))) return false;
+        return true;
+    }
     // all-IQ2_XXS layers of the shapes whose chunks run on the tile-major copies read their down matrices from the column-sliced copy (one
     // token, small batches) or the tile-major one (chunks): the row-major packed down matrices are not kept (they pass through a second
     // staging buffer on their way to the tile-major copy)
@@ -183,6 +191,13 @@ struct Moe {
 
 Moe *moe_of(redhip_moe_t h) { return static_cast<Moe *>(h); }
 
+// the raw GGUF rows of a layer's routed experts, for the kernels that read them; nullptr + message on a handle that keeps none
+const uint8_t *raw_rows(const Moe *m, uint32_t layer) {
+    const uint8_t *p = m->layers[layer].experts;
+    if (!p) moe_err("internal: this handle keeps no raw rows of its routed experts, and a kernel that reads them was chosen (layer %u)", layer);
+    return p;
+}
+
 size_t align256(size_t n) { return (n + 255u) & ~(size_t)255u; }
 
 bool check_layer(Moe *m, uint32_t layer) {
@@ -259,7 +274,8 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
             HIP_OK(launch_group_pairs(ids, weights, ntok, c.top_k, c.n_expert, m->uid, m->expert_start, m->pair_token, m->pair_weight,
                                       m->tok_pair, m->n_unique, s), "grouping launch");
         }
-        HIP_OK(launch_batch_mixed(m->gu_type, m->gu_grid, L.packed, m->packed_stride, m->act, m->dn_type, m->dn_grid, m->sh_dn_type, L.experts + 2u * m->gate_bytes, m->expert_stride,
+        if (!L.words_down && !raw_rows(m, layer)) return 0;          // (the batched down kernel reads the packed copy when there is one)
+        HIP_OK(launch_batch_mixed(m->gu_type, m->gu_grid, L.packed, m->packed_stride, m->act, m->dn_type, m->dn_grid, m->sh_dn_type, L.experts ? L.experts + 2u * m->gate_bytes : nullptr, m->expert_stride,
                                   L.shared + 2u * m->sh_gate_bytes, L.words_down, m->words_down_stride(), L.dense_down, m->uid, m->expert_start, m->pair_token, m->n_unique, m->pair_weight, m->tok_pair,
                                   m->scalar, m->xh, m->xl, m->xexp, m->act_h, m->act_l, m->act_exp, out, c.hidden, c.ffn, c.top_k, ntok, c.n_expert, s, in_batch),
                "grouped mixed batch launch");
@@ -317,6 +333,7 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
         }
         prof_set_stage(ST_BATCH_GATEUP);
         const bool tiled_down = m->mixed_chunk(ntok) && m->layers[layer].tiled_down;      // then the activations stay fp16 halves for the IQ3_S tile kernel
+        if (!(m->mixed_chunk(ntok) && tiled_down) && !raw_rows(m, layer)) return 0;       // (the per-pair kernels below read raw rows)
         if (m->mixed_chunk(ntok))      // xh / xl / xexp come from the router kernel or the prep kernel
             HIP_OK(launch_prefill_gateup_tiled(m->layers[layer].tiled, m->packed_stride, m->uid, m->expert_start, m->pair_token, m->n_unique, m->tile_group,
                                                m->tile_pair0, m->tile_n, m->n_tiles, m->xh, m->xl, m->xexp, tiled_down ? nullptr : m->act, m->act_h, m->act_l,
@@ -363,6 +380,8 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
             HIP_OK(launch_down_combine_words(m->dn_type, m->dn_grid, m->sliced_words() ? L.down_cm : L.words_down, m->words_down_stride(), L.dense_down,
                                              select_here ? m->ids : ids, select_here ? m->weights : weights,
                                              m->scalar, m->act_h, m->act_l, m->act_exp, out, c.hidden, c.ffn, c.top_k, s, ntok, m->sliced_words()), "down/combine launch");
+        else if (!raw_rows(m, layer))
+            return 0;
         else
             HIP_OK(launch_down_combine_raw(m->dn_type, m->sh_dn_type, L.experts + 2u * m->gate_bytes, m->expert_stride, L.shared + 2u * m->sh_gate_bytes,
                                            select_here ? m->ids : ids, select_here ? m->weights : weights, m->scalar, m->act_h, m->act_l,
@@ -370,6 +389,7 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
         prof_set_stage(ST_OTHER);
         return 1;
     }
+    if (!raw_rows(m, layer)) return 0;
     const ExpertSet ex = m->routed(layer), sh = m->shared(layer);
     prof_set_stage(ST_GATEUP);
     HIP_OK(launch_moe_gateup(ex, ids, c.top_k, c.hidden, c.ffn, x, m->act, s), "routed gate/up launch");
@@ -1026,6 +1046,7 @@ int redhip_moe_dequant_resident(redhip_moe_t h, uint32_t layer, uint32_t expert,
         else HIP_OK(launch_dequant_packed(m->dn_type, wd, c.hidden, c.ffn, m->dn_grid, out_dev, s), "stream-packed down dequant");
         return 1;
     }
+    if (!sh && !raw_rows(m, layer)) return 0;
     const uint8_t *base = sh ? L.shared : L.experts + (uint64_t)expert * m->expert_stride;
     const uint64_t gb = sh ? m->sh_gate_bytes : m->gate_bytes;
     const uint32_t gu = sh ? m->sh_gu_type : m->gu_type, dn = sh ? m->sh_dn_type : m->dn_type;

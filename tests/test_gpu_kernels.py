@@ -115,6 +115,50 @@ def test_router_select_random_and_ties():
         assert np.all(np.abs(w - cw) <= 1e-6 + 1e-5 * cw)
 
 
+def test_router_select_adversarial(golden_dir):
+    """The selection must pick what the CPU's argmax loop over probabilities picks, also where different logits share a probability:
+    logits one to a few ulps apart around the K-th place (the lower index a little smaller, so that logit order and the CPU's order
+    differ whenever the probabilities collapse), tight clusters, logits spread until the tail underflows, all equal, and the golden
+    cases of the reference (here without the probabilities output)."""
+    from dwarfstar_red_lite_amd import redmetal_quant as rq
+    rng = np.random.default_rng(2024)
+    cases = []
+    for c in json.load(open(os.path.join(golden_dir, "router_select.json")))["cases"]:
+        cases.append((np.frombuffer(bytes.fromhex(c["logits"]), np.float32).copy(), c["top_k"]))
+    for case in range(96):
+        E, K = (512, 10) if case % 3 else (64, 4)
+        l = (rng.standard_normal(E) * (0.9, 3.0, 40.0, 300.0)[case % 4]).astype(np.float32)
+        order = np.argsort(-l)
+        kind = case % 6
+        if kind == 0:            # the K-th and (K+1)-th one ulp apart, the smaller logit at the lower index
+            hi, lo = sorted((int(order[K - 1]), int(order[K])))
+            l[hi] = l[order[K - 1]]
+            l[lo] = np.nextafter(l[hi], np.float32(-np.inf))
+        elif kind == 1:          # a ladder of ulps through the top K + 4
+            base = l[order[0]]
+            for r, i in enumerate(sorted(int(j) for j in order[:K + 4])):
+                v = base
+                for _ in range(3 * r):
+                    v = np.nextafter(v, np.float32(-np.inf))
+                l[i] = v
+        elif kind == 2:          # twenty logits within 1e-6 of each other at the top
+            top = order[:20]
+            l[top] = l[order[0]] + (rng.random(20) * 1e-6).astype(np.float32)
+        elif kind == 3:          # exact ties across the boundary
+            l[order[K - 3:K + 5]] = l[order[K - 1]]
+        elif kind == 4:          # fewer than K probabilities above zero: the tail is picked by index
+            l = (rng.standard_normal(E) * 400.0).astype(np.float32)
+        # kind 5: plain random
+        cases.append((l, K))
+    cases.append((np.zeros(512, np.float32), 10))
+    cases.append((np.full(512, -3.25, np.float32), 10))
+    for n, (l, K) in enumerate(cases):
+        ids, w = rq.router_select(l, K)
+        ci, cw = orc.router_select(l, K)
+        assert np.array_equal(ids, ci), (n, ids, ci)
+        assert np.all(np.abs(w - cw) <= 1e-6 + 1e-5 * cw), n
+
+
 def test_grouping_matches_host_sort():
     from dwarfstar_red_lite_amd import moe
     cfg = synth.layer_config(hidden=256, ffn=256, n_expert=512, top_k=10)
