@@ -314,19 +314,20 @@ __device__ __forceinline__ float q6k_dot32(const uint8_t *row, uint32_t chunk, c
 // A table in LDS holds, per expert, the set of tokens that selected it (a token selects an expert at most once): the
 // position of a pair inside its group and the group's size are bit counts of that set, the order of the groups a
 // bit count over the "first pair of its expert" flags, the group offsets one prefix sum. Run by a whole workgroup
-// of at least 128 threads (every thread reaches the barriers); at most 16 tokens, 128 pairs, 1024 experts.
-constexpr uint32_t kGroupLdsWords = 1024u + 6u;
+// of at least 256 threads (every thread reaches the barriers); at most 16 tokens, 256 pairs (one per lane of the first four waves), 1024 experts.
+constexpr uint32_t kGroupLdsWords = 1024u + 12u;
+constexpr uint32_t kGroupSmallPairs = 256u;
 // Optionally also the pass list of the batched expert-slice kernel (g.pass_list != nullptr): a pass = up to two consecutive pairs of one
 // group. Entry v: x = expert | pairs in the pass << 16 | position of its first pair << 24; y = four bytes: the (token * top_k + k) index
 // of its first and second pair, then their tokens. Passes follow the groups' order; *g.n_pass = their number.
 template <class PairId, class PairWeight>
 __device__ __forceinline__ void group_small(const GroupJob &g, uint32_t *lds, PairId pair_id, PairWeight pair_w) {
     uint32_t *token_set = lds;                           // per expert: bit t = token t selected it; later the group's offset (| its first pass << 16)
-    uint32_t *first_count = lds + 1024, *size_total = lds + 1026, *pass_total = lds + 1028;
+    uint32_t *first_count = lds + 1024, *size_total = lds + 1028, *pass_total = lds + 1032;      // per wave of pairs (four)
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, K = g.top_k;
     for (uint32_t i = tid; i < g.n_expert; i += blockDim.x) token_set[i] = 0u;
     __syncthreads();
-    const uint32_t P = g.ntok * K, pr = tid;             // pair index (waves 0 and 1)
+    const uint32_t P = g.ntok * K, pr = tid;             // pair index (waves 0..3)
     const bool live = pr < P;
     const uint32_t t = live ? pr / K : 0u;
     const uint32_t e = live ? guarded_id(pair_id(t, pr % K), g.n_expert, g.status) : 0u;
@@ -342,7 +343,7 @@ __device__ __forceinline__ void group_small(const GroupJob &g, uint32_t *lds, Pa
     uint32_t scan = first ? n : 0u;                      // inclusive prefix sum of the group sizes in pair order
     const uint32_t n_pass_mine = first ? (n + 1u) >> 1 : 0u;
     uint32_t pscan = n_pass_mine;                        // the same of the groups' pass counts
-    if (wave < 2u) {
+    if (wave < 4u) {
 #pragma unroll
         for (int o = 1; o < 64; o <<= 1) {
             const uint32_t up = __shfl_up(scan, o, 64), pup = __shfl_up(pscan, o, 64);
@@ -353,15 +354,19 @@ __device__ __forceinline__ void group_small(const GroupJob &g, uint32_t *lds, Pa
     }
     const uint64_t first_mask = __ballot(first);
     __syncthreads();
-    const uint32_t grp = (wave == 1u ? first_count[0] : 0u) + __builtin_amdgcn_mbcnt_hi((uint32_t)(first_mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)first_mask, 0u));
-    const uint32_t start = (wave == 1u ? size_total[0] : 0u) + scan - (first ? n : 0u);
-    const uint32_t pass0 = (wave == 1u ? pass_total[0] : 0u) + pscan - n_pass_mine;
+    uint32_t groups_before = 0u, size_before = 0u, pass_before = 0u;      // totals of the waves of pairs before this one
+#pragma unroll
+    for (uint32_t w = 0; w < 3u; ++w)
+        if (w < wave && wave < 4u) { groups_before += first_count[w]; size_before += size_total[w]; pass_before += pass_total[w]; }
+    const uint32_t grp = groups_before + __builtin_amdgcn_mbcnt_hi((uint32_t)(first_mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)first_mask, 0u));
+    const uint32_t start = size_before + scan - (first ? n : 0u);
+    const uint32_t pass0 = pass_before + pscan - n_pass_mine;
     if (first) { token_set[e] = start | (pass0 << 16); g.uid[grp] = e; g.expert_start[grp] = start; }
     if (tid == 0u) {
-        const uint32_t U = first_count[0] + first_count[1];
-        g.expert_start[U] = size_total[0] + size_total[1];      // = P unless a token repeated an expert
+        const uint32_t U = (first_count[0] + first_count[1]) + (first_count[2] + first_count[3]);
+        g.expert_start[U] = (size_total[0] + size_total[1]) + (size_total[2] + size_total[3]);      // = P unless a token repeated an expert
         g.n_unique[0] = U;
-        if (g.n_pass) g.n_pass[0] = pass_total[0] + pass_total[1];
+        if (g.n_pass) g.n_pass[0] = (pass_total[0] + pass_total[1]) + (pass_total[2] + pass_total[3]);
     }
     __syncthreads();
     if (live) {
@@ -385,7 +390,7 @@ __device__ __forceinline__ void group_small_given(const GroupJob &g, uint32_t *l
     group_small(g, lds, [&](uint32_t t, uint32_t k) { return g.ids[t * g.top_k + k]; }, [&](uint32_t t, uint32_t k) { return g.weights[t * g.top_k + k]; });
 }
 __host__ inline bool group_job_fits(const GroupJob &g) {
-    return g.ids && g.weights && g.ntok && g.ntok <= 16u && g.top_k && g.top_k <= 16u && g.ntok * g.top_k <= 128u && g.n_expert && g.n_expert <= 1024u;
+    return g.ids && g.weights && g.ntok && g.ntok <= 16u && g.top_k && g.top_k <= 16u && g.ntok * g.top_k <= kGroupSmallPairs && g.n_expert && g.n_expert <= 1024u;
 }
 
 // ---------------------------------------------------------------- router GEMV
@@ -1053,7 +1058,7 @@ hipError_t launch_select(const float *logits, uint32_t ntok, uint32_t n_expert, 
 // expert (with the pass list of the batched expert-slice kernel). One workgroup; logits [ntok][n_expert + 1].
 __global__ __launch_bounds__(kWaves * 64) void select_group_kernel(const float *logits, uint32_t ntok, uint32_t E, uint32_t K, uint32_t *ids, float *weights,
                                                                    float *scalar, GroupJob job) {
-    __shared__ SelectOut sel[8];
+    __shared__ SelectOut sel[kWaves];
     __shared__ uint32_t group_lds[kGroupLdsWords];
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63u;
     if (wave < ntok) {
@@ -1069,7 +1074,7 @@ __global__ __launch_bounds__(kWaves * 64) void select_group_kernel(const float *
 
 hipError_t launch_select_group(const float *logits, uint32_t ntok, uint32_t n_expert, uint32_t top_k, uint32_t *ids, float *weights, float *scalar,
                                const GroupJob &job, hipStream_t s) {
-    if (!ntok || ntok > 8u || !n_expert || n_expert > 1024u || !top_k || top_k > 16u || top_k > n_expert || ntok * top_k > 128u) return hipErrorInvalidValue;
+    if (!ntok || ntok > (uint32_t)kWaves || !n_expert || n_expert > 1024u || !top_k || top_k > 16u || top_k > n_expert || ntok * top_k > kGroupSmallPairs) return hipErrorInvalidValue;
     GroupJob gj = job;
     gj.ids = nullptr;
     gj.weights = nullptr;
@@ -2226,7 +2231,7 @@ hipError_t launch_batch_slices(const void *experts, uint64_t stride, const void 
                                const void *pass_list, const uint32_t *n_pass, const float *weights, const float *scalar, const void *xh, const void *xl,
                                const int *xexp, float *partial, float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, hipStream_t s,
                                const float *shared_gu, const float *shared_dense, uint32_t stream_type, const int8_t *grid) {
-    if (!fused_iq2_supported(hidden, ffn) || hidden % 32u || !ntok || ntok > 16u || ntok * top_k > 128u || !pass_list || !n_pass) return hipErrorInvalidValue;
+    if (!fused_iq2_supported(hidden, ffn) || hidden % 32u || !ntok || ntok > 16u || ntok * top_k > kGroupSmallPairs || !pass_list || !n_pass) return hipErrorInvalidValue;
     const bool mix = shared_gu != nullptr;
     if (mix ? !shared_dense : (!shared || !shared_down_cm)) return hipErrorInvalidValue;
     if (stream_type && ((stream_type != T_IQ2_XS && stream_type != T_IQ1_M) || !grid || !mix)) return hipErrorInvalidValue;

@@ -137,9 +137,13 @@ struct Moe {
     bool sliced_words() const { return mixed_slices && dn_type == T_IQ3_S; }
     // ... whose down matrices are IQ2_XS / IQ1_M streams: a column-sliced copy beside the row-major one
     bool sliced_streams() const { return mixed_slices && dn_type != T_IQ3_S; }
-    // batches that run as expert slices per pass: 2..8 tokens, at most 128 pairs
+    // batches that run as expert slices per pass: 2..8 tokens and at most 128 pairs on mixed layouts (their first launch multiplies the
+    // shared expert's gate | up rows for up to eight tokens), 2..16 tokens and at most 256 pairs on all-IQ2_XXS layers
+    static constexpr uint32_t kSmallMaxFused = 16u;
     bool small_batch(uint32_t ntok) const {
-        return (fused || mixed_slices) && ntok >= 2u && ntok <= 8u && ntok * cfg.top_k <= 128u && ntok * (cfg.top_k + 1u) <= 144u && cfg.hidden / 512u <= 4u;
+        if (ntok < 2u || cfg.hidden / 512u > 4u) return false;
+        if (fused) return ntok <= kSmallMaxFused && ntok * cfg.top_k <= 256u;
+        return mixed_slices && ntok <= 8u && ntok * cfg.top_k <= 128u && ntok * (cfg.top_k + 1u) <= 144u;
     }
     // ... with the layer's own router: on a mixed layout two tokens are quicker on the single-token kernels (three launches, the selection
     // inside the gate/up kernel) than as slices behind a selection + pair sort launch of their own (four): 30.7 against 32.7 us
@@ -173,7 +177,7 @@ struct Moe {
     // So does every layout from 9 to 16 tokens: two small batches are quicker than one chunk, whose tile kernels leave most workgroups
     // without work at that size.
     bool sliced(uint32_t ntok) const {
-        if (ntok <= kSlice) return false;
+        if (ntok <= kSlice || small_batch(ntok)) return false;      // (all-IQ2_XXS layers take up to 16 tokens as one small batch)
         if (ntok <= 2u * kSlice && (small_batch(kSlice) || grouped_mixed(kSlice))) return true;
         return mixed && !tiles_resident() && !stream_chunk(ntok) && grouped_mixed(kSlice);
     }
@@ -530,8 +534,9 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
         }
     }
     const size_t T = c.max_tokens;
-    const size_t partial_bytes = m->fused || m->mixed_slices ? align256((size_t)(c.max_tokens < 8u ? c.max_tokens : 8u) * (c.top_k + 1u) * (c.ffn / 32u) * c.hidden * 4u) : 0u;
-    const size_t ws_bytes = partial_bytes + align256(8u * 128u) + align256(4u) + align256(4u) + align256(T * c.hidden * 4u) + align256(T * (c.n_expert + 1u) * 4u) + 2u * align256(T * c.top_k * 4u) + align256(T * 4u) +
+    const size_t partial_tokens = m->fused ? Moe::kSmallMaxFused : 8u;      // the largest batch that runs as expert slices
+    const size_t partial_bytes = m->fused || m->mixed_slices ? align256((size_t)(c.max_tokens < partial_tokens ? c.max_tokens : partial_tokens) * (c.top_k + 1u) * (c.ffn / 32u) * c.hidden * 4u) : 0u;
+    const size_t ws_bytes = partial_bytes + align256(8u * 256u) + align256(4u) + align256(4u) + align256(T * c.hidden * 4u) + align256(T * (c.n_expert + 1u) * 4u) + 2u * align256(T * c.top_k * 4u) + align256(T * 4u) +
                             align256(T * c.top_k * c.ffn * 4u) + align256(T * c.ffn * 4u) +
                             2u * align256(2u * T * c.hidden) + align256(4u * T) + 2u * align256(2u * T * (c.top_k + 1u) * c.ffn) +
                             align256(4u * T * (c.top_k + 1u) * (c.ffn / 32u)) +
@@ -547,7 +552,7 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
     uint8_t *w = m->ws;
     m->status = reinterpret_cast<uint32_t *>(w); w += align256(4u);
     if (partial_bytes) { m->partial = reinterpret_cast<float *>(w); w += partial_bytes; }
-    m->pass_list = reinterpret_cast<uint2 *>(w); w += align256(8u * 128u);
+    m->pass_list = reinterpret_cast<uint2 *>(w); w += align256(8u * 256u);
     m->n_pass = reinterpret_cast<uint32_t *>(w); w += align256(4u);
     m->xn = reinterpret_cast<float *>(w); w += align256(T * c.hidden * 4u);
     m->logits = reinterpret_cast<float *>(w); w += align256(T * (c.n_expert + 1u) * 4u);
