@@ -269,6 +269,14 @@ __device__ __forceinline__ void wave_lds_sync() {
     __builtin_amdgcn_wave_barrier();
     __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "wavefront");
 }
+// Workgroup barrier for data exchanged through LDS only: waits for this wave's LDS operations, not for its outstanding global loads
+// (__syncthreads waits for those too, so a workgroup that has requested its weights would sit at the barrier until the last of them has
+// arrived; with this one every wave goes on to its first weights as soon as THEY are there).
+__device__ __forceinline__ void lds_barrier() {
+    __builtin_amdgcn_fence(__ATOMIC_RELEASE, "workgroup", "local");
+    __builtin_amdgcn_s_barrier();
+    __builtin_amdgcn_fence(__ATOMIC_ACQUIRE, "workgroup", "local");
+}
 __device__ __forceinline__ uint32_t wave_count(bool pred) { return (uint32_t)__popcll(__ballot(pred)); }
 // Raw GGUF rows are decoded from LDS: a wave copies `bytes` (a multiple of 16, both addresses 16-byte aligned) with
 // coalesced 16-byte loads, so the many one- and two-byte fields of a block never go to memory one by one.
@@ -2123,7 +2131,7 @@ __global__ __launch_bounds__(kWaves * 64, 8) void batch_slice_kernel(BatchSliceA
     }
     const LaneTables lt = lane_tables<REP, kBatchLut>(lds, sign_lut, lane);
     REDHIP_STAMP(2);                                   // loads requested, tables written
-    __syncthreads();                                   // tables
+    lds_barrier();                                   // tables
     REDHIP_STAMP(3);
 
     float va[UPW], vb[UPW];
@@ -2142,7 +2150,7 @@ __global__ __launch_bounds__(kWaves * 64, 8) void batch_slice_kernel(BatchSliceA
         part[kc * 64u + 4u * quad + j] = ta;
         part[NKC * 64u + kc * 64u + 4u * quad + j] = tb;
     }
-    __syncthreads();
+    lds_barrier();
     REDHIP_STAMP(5);                                   // ... of every wave
     if (tid < 64u) {
         const uint32_t t = tid >> 5, c = tid & 31u;
@@ -2161,7 +2169,7 @@ __global__ __launch_bounds__(kWaves * 64, 8) void batch_slice_kernel(BatchSliceA
         split_hi_lo(act, exp2i(-ee), act_hl + t * 64u + c, act_hl + t * 64u + 32u + c);
         if (c == 0u) act_scale[t] = exp2i(ee);
     }
-    __syncthreads();
+    lds_barrier();
     REDHIP_STAMP(6);                                   // activations exchanged
     half4_t ad[8];
     {
