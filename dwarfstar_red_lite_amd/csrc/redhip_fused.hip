@@ -769,6 +769,7 @@ __device__ __forceinline__ void wave_select_topk(const float *logits, uint32_t E
     }
     const float gate_logit = logits[E];                      // shared expert's gate logit rides along
     m = wave_max(m);
+    REDHIP_STAMP(8);                                   // logits here, maximum known
     float p[PER];
     double part = 0.0;
 #pragma unroll
@@ -779,6 +780,7 @@ __device__ __forceinline__ void wave_select_topk(const float *logits, uint32_t E
     const double denom = wave_sum_d(part);
     const bool bad = !(denom > 0.0) || isinf(denom) || isnan(denom);
     const float inv = bad ? 0.0f : reciprocal_as_float(denom);
+    REDHIP_STAMP(9);                                   // exponentials and their sum
     uint32_t key[PER];
 #pragma unroll
     for (int s = 0; s < PER; ++s) {
@@ -803,6 +805,7 @@ __device__ __forceinline__ void wave_select_topk(const float *logits, uint32_t E
     uint32_t n_c = 0u;
 #pragma unroll
     for (int s = 0; s < PER; ++s) n_c += wave_count(key[s] >= tau);
+    REDHIP_STAMP(10);                                  // threshold and candidate count
     uint32_t mine = 0xffffffffu, kmine = 0u, rank = 0u;
     if (n_c <= 64u) {
         // Level 2: candidates to LDS in index order, one per lane, ranked against each other with lane broadcasts:
@@ -874,6 +877,7 @@ __device__ __forceinline__ void wave_select_topk(const float *logits, uint32_t E
         if (lane >= K) rank = 0xffffffffu;
     }
     const bool selected = rank < K;
+    REDHIP_STAMP(11);                                  // candidates ranked
     const float pm = __uint_as_float(kmine & 0x7fffffffu);
     const double sum = wave_sum_d(selected ? (double)pm : 0.0);
     const bool bad2 = bad || !(sum > 0.0) || isinf(sum) || isnan(sum);
@@ -883,6 +887,7 @@ __device__ __forceinline__ void wave_select_topk(const float *logits, uint32_t E
         out->w[rank] = pm * invs;
     }
     if (lane == 0u) out->scalar = 1.0f / (1.0f + expf(-gate_logit));
+    REDHIP_STAMP(12);                                  // weights written
 }
 
 // ---------------------------------------------------------------- softmax top-k selection by a whole workgroup

@@ -80,6 +80,12 @@ def main():
     print("|---|---|---|---|---|")
     for k, name in enumerate(names):
         print("| %s | %.2f | %.2f | %.2f | %.2f |" % (name, d[:, k].mean(), np.median(d[:, k]), np.percentile(d[:, k], 90), d[:, k].max()))
+    if B == 1 and args.routing == "router" and (t[:, 12] > 0).any():      # the selecting wave's own stamps (workgroups of routed slots)
+        sel = t[t[:, 12] > t[:, 0]]
+        ds = np.stack([sel[:, 8] - sel[:, 0], sel[:, 9] - sel[:, 8], sel[:, 10] - sel[:, 9], sel[:, 11] - sel[:, 10], sel[:, 12] - sel[:, 11], sel[:, 1] - sel[:, 12]], axis=1) * 0.01
+        for k, name in enumerate(["selection: entry -> logits loaded, maximum", "selection: exponentials, denominator", "selection: threshold, candidate count",
+                                  "selection: candidates compacted and ranked", "selection: weights", "selection: end -> barrier passed"]):
+            print("| %s | %.2f | %.2f | %.2f | %.2f |" % (name, ds[:, k].mean(), np.median(ds[:, k]), np.percentile(ds[:, k], 90), ds[:, k].max()))
     life = (t[:, 7] - t[:, 0]) * 0.01
     start = (t[:, 0] - t0) * 0.01
     print("| workgroup lifetime | %.2f | %.2f | %.2f | %.2f |" % (life.mean(), np.median(life), np.percentile(life, 90), life.max()))
