@@ -1557,6 +1557,12 @@ struct SliceArgs {
     float *partial;                // [top_k + 1][ffn / 32][hidden]
     uint32_t hidden, ffn, n_expert, top_k;
     uint32_t *status;              // RouteGuard::status when ids_in is the caller's
+    // SLOTS variant: the experts of a pool of slots. slot_table[k] = address of slot k's raw bytes, its re-laid copy (packed gate | up,
+    // column-sliced down) lies shadow_off behind it; x / x1 = f32 activations (experts from x_split on read x1), split to fp16 halves here
+    const uint64_t *slot_table;
+    uint64_t shadow_off;
+    const float *x, *x1;
+    uint32_t x_split;
 };
 
 // Two tables, REP copies of every 16-byte entry side by side (entry i, copy c at (i * REP + c) * 16), lane l reads copy l % REP: with
@@ -1751,7 +1757,7 @@ __device__ __forceinline__ void group_dot2_lut(uint2 q, const half4_t *ax, const
 }
 
 constexpr int kSliceLut = 32;      // copies of the sign words in the one-token kernel: 16 KB, every lane of a half wave its own bank
-template <int NKC, int REP>        // hidden = 512 * NKC
+template <int NKC, int REP, bool SLOTS = false>        // hidden = 512 * NKC
 __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(SliceArgs a) {
     constexpr int NW = kWaves;
     constexpr int UPW = 16 * NKC / NW;                 // (row-quad, K-chunk) units of gate / up per wave
@@ -1776,9 +1782,26 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(SliceArgs a) 
     const uint32_t kc = wave % NKC, q0 = wave / NKC;
     const uint32_t G = 16u * kc + blk;
     half4_t ax[8];
-    load_act_operand(ax, a.xh + 32u * G, a.xl + 32u * G, j);
+    float4 xf[SLOTS ? 8 : 1];                          // SLOTS: the lane's 32 activations as f32 (lanes j = 0, 1), split behind the barrier
+    uint64_t slot_base = 0u;
+    if constexpr (SLOTS) {
+        slot_base = a.slot_table[slot];
+        const float *xs = (a.x1 && slot >= a.x_split ? a.x1 : a.x) + 32u * G;
+        float amax = 0.0f;
+#pragma unroll
+        for (int s8 = 0; s8 < 8; ++s8) {
+            xf[s8] = make_float4(0.0f, 0.0f, 0.0f, 0.0f);
+            if (j < 2u) xf[s8] = *reinterpret_cast<const float4 *>(xs + 4 * s8);
+        }
+#pragma unroll
+        for (int s8 = 0; s8 < 8; ++s8) amax = fmaxf(fmaxf(amax, fmaxf(fabsf(xf[s8].x), fabsf(xf[s8].y))), fmaxf(fabsf(xf[s8].z), fabsf(xf[s8].w)));
+        amax = wave_max(amax);                         // waves kc = 0 .. NKC - 1 cover the whole vector between them
+        if (lane == 0u) reinterpret_cast<float *>(sel)[wave] = amax;
+    } else {
+        load_act_operand(ax, a.xh + 32u * G, a.xl + 32u * G, j);
+    }
     // the table is first read behind the barrier that ends the selection: wave 0 selects, waves 8..15 build meanwhile
-    const bool selecting = !is_shared && a.logits;
+    const bool selecting = !SLOTS && !is_shared && a.logits;
     // (and waves 1..7 write the sign words)
     if (selecting) { build_tables_rep<REP, 8, 0>(lds, strip, wave - 8u, lane); if (wave < 8u) build_sign_lut<kSliceLut>(reinterpret_cast<uint32_t *>(sign_lut), tid, 64u, 7u * 64u); }
     else { build_tables_rep<REP, 16, 0>(lds, strip, wave, lane); build_sign_lut<kSliceLut>(reinterpret_cast<uint32_t *>(sign_lut), tid); }
@@ -1786,7 +1809,25 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(SliceArgs a) 
 
     uint32_t expert = 0u;
     float comb;                                        // the slot's weight in the layer's output
-    if (is_shared) {
+    int x_exp = 0;
+    if constexpr (SLOTS) {
+        comb = a.weights_in[slot];
+        __syncthreads();                               // table, the waves' largest |x|
+        float amax = 0.0f;
+#pragma unroll
+        for (int w = 0; w < NW; ++w) amax = fmaxf(amax, reinterpret_cast<const float *>(sel)[w]);
+        x_exp = prescale_exp(amax);
+        const float inv = exp2i(-x_exp);
+#pragma unroll
+        for (int s8 = 0; s8 < 8; ++s8) {
+            const float t[4] = {xf[s8].x * inv, xf[s8].y * inv, xf[s8].z * inv, xf[s8].w * inv};
+#pragma unroll
+            for (int c = 0; c < 4; ++c) {
+                const _Float16 h = (_Float16)t[c];
+                ax[s8][c] = j == 0u ? h : (_Float16)((t[c] - (float)h) * 2048.0f);      // (lanes j >= 2 hold zeros: both halves are zero)
+            }
+        }
+    } else if (is_shared) {
         comb = a.logits ? 1.0f / (1.0f + expf(-a.logits[a.n_expert])) : a.scalar_in[0];
         __syncthreads();                               // table
     } else if (a.logits) {
@@ -1807,9 +1848,13 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(SliceArgs a) 
         __syncthreads();                               // table
     }
     REDHIP_STAMP(1);                                   // selection (or the caller's routing) and tables are here
+    const uint64_t gate_bytes = (uint64_t)F * HG * 8u + (uint64_t)F * HB * 2u;
     const uint8_t *ex = is_shared ? a.shared : a.experts + (uint64_t)expert * a.stride;
     const uint8_t *dn = is_shared ? a.shared_down_cm : a.down_cm + (uint64_t)expert * a.down_stride;
-    const uint64_t gate_bytes = (uint64_t)F * HG * 8u + (uint64_t)F * HB * 2u;
+    if constexpr (SLOTS) {
+        ex = reinterpret_cast<const uint8_t *>(slot_base + a.shadow_off);
+        dn = ex + 2u * gate_bytes;
+    }
     const uint2 *gate_qs = reinterpret_cast<const uint2 *>(ex);
     const uint16_t *gate_ds = reinterpret_cast<const uint16_t *>(ex + (uint64_t)F * HG * 8u);
     const uint2 *up_qs = reinterpret_cast<const uint2 *>(ex + gate_bytes);
@@ -1857,7 +1902,7 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(SliceArgs a) 
         float gsum = 0.0f, usum = 0.0f;
 #pragma unroll
         for (int c = 0; c < NKC; ++c) { gsum += part[c * 64 + tid]; usum += part[c * 64 + 32 + tid]; }
-        const float xs = 0.125f * exp2i(a.xexp[0]);      // d / 8 and the pre-scale of x
+        const float xs = 0.125f * exp2i(SLOTS ? x_exp : a.xexp[0]);      // d / 8 and the pre-scale of x
         gsum *= xs;
         usum *= xs;
         const float act = (gsum / (1.0f + expf(-gsum))) * usum;
@@ -1894,7 +1939,9 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(SliceArgs a) 
 // out[r] = sum over slots (selection order, the shared expert last) and column groups of partial[slot][group][r] (+ the residual of the
 // block step). 32 rows per workgroup as eight float4 columns; a thread adds every 32nd partial vector, the 32 threads of a column
 // meet by shuffles and through LDS in a fixed order.
-__global__ __launch_bounds__(256) void slice_sum_kernel(const float *partial, uint32_t n_part, uint32_t H, float *out, const float *resid_a, const float *resid_b) {
+struct SumTail { const float *resid, *shared, *scalar; float *out2; };      // out = out2 = resid + (sum + shared * scalar[0]); all nullptr: none
+__global__ __launch_bounds__(256) void slice_sum_kernel(const float *partial, uint32_t n_part, uint32_t H, float *out, const float *resid_a, const float *resid_b,
+                                                        SumTail tail) {
     __shared__ float4 red[4][8];
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, c8 = tid & 7u, pl = tid >> 3;      // pl 0..31
     const uint32_t col = blockIdx.x * 8u + c8;          // float4 column
@@ -1932,6 +1979,12 @@ __global__ __launch_bounds__(256) void slice_sum_kernel(const float *partial, ui
         if (resid_a) {
             const float4 ra = reinterpret_cast<const float4 *>(resid_a)[col], rb = reinterpret_cast<const float4 *>(resid_b)[col];
             sum = make_float4((ra.x + rb.x) + sum.x, (ra.y + rb.y) + sum.y, (ra.z + rb.z) + sum.z, (ra.w + rb.w) + sum.w);
+        }
+        if (tail.resid) {
+            const float4 r = reinterpret_cast<const float4 *>(tail.resid)[col], sh = reinterpret_cast<const float4 *>(tail.shared)[col];
+            const float sc = tail.scalar[0];
+            sum = make_float4(r.x + fmaf(sh.x, sc, sum.x), r.y + fmaf(sh.y, sc, sum.y), r.z + fmaf(sh.z, sc, sum.z), r.w + fmaf(sh.w, sc, sum.w));
+            reinterpret_cast<float4 *>(tail.out2)[col] = sum;
         }
         reinterpret_cast<float4 *>(out)[col] = sum;
     }
@@ -2211,7 +2264,8 @@ hipError_t launch_expert_slices(const void *experts, uint64_t stride, const void
     if (!logits && (!ids_in || !weights_in || !scalar_in)) return hipErrorInvalidValue;
     const SliceArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(down_cm), down_stride, static_cast<const uint8_t *>(shared),
                       static_cast<const uint8_t *>(shared_down_cm), logits, ids_in, weights_in, scalar_in, ids_out, weights_out, scalar_out,
-                      static_cast<const _Float16 *>(xh), static_cast<const _Float16 *>(xl), xexp, partial, hidden, ffn, n_expert, top_k, route_guard().status};
+                      static_cast<const _Float16 *>(xh), static_cast<const _Float16 *>(xl), xexp, partial, hidden, ffn, n_expert, top_k, route_guard().status,
+                      nullptr, 0u, nullptr, nullptr, 0u};
     const dim3 grid_dim(ffn / 32u, top_k + 1u);
 #define REDHIP_SLICE(NKC)                                                                                                              \
     do {                                                                                                                               \
@@ -2236,7 +2290,49 @@ hipError_t launch_expert_slices(const void *experts, uint64_t stride, const void
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     prof_set_stage(ST_SLICE_SUM);
-    REDHIP_LAUNCH(slice_sum_kernel, dim3(hidden / 32u), dim3(256), 0, s, partial, (top_k + 1u) * (ffn / 32u), hidden, out, block_context().resid_a, block_context().resid_b);
+    REDHIP_LAUNCH(slice_sum_kernel, dim3(hidden / 32u), dim3(256), 0, s, partial, (top_k + 1u) * (ffn / 32u), hidden, out, block_context().resid_a, block_context().resid_b, SumTail{nullptr, nullptr, nullptr, nullptr});
+    return hipGetLastError();
+}
+
+// One token over the slots of a pool: slot_table[k] = address of slot k's raw bytes, whose re-laid IQ2_XXS copy lies shadow_off behind.
+// Two launches: slices (partial [top_k][ffn / 32][hidden]) and their sum into out (and, with a tail, out = out2 = resid + (sum + shared * scalar)).
+hipError_t launch_slot_slices(const uint64_t *slot_table, uint64_t shadow_off, const float *weights, uint32_t top_k, uint32_t hidden, uint32_t ffn,
+                              const float *x, const float *x1, uint32_t x_split, float *partial, float *out, const float *tail_resid,
+                              const float *tail_shared, const float *tail_scalar, float *tail_out2, hipStream_t s) {
+    if (!fused_iq2_supported(hidden, ffn) || hidden % 32u || !top_k || top_k > 64u || !slot_table || !weights || !x || !partial || !out) return hipErrorInvalidValue;
+    SliceArgs a{};
+    a.weights_in = weights;
+    a.partial = partial;
+    a.hidden = hidden; a.ffn = ffn; a.n_expert = 0u; a.top_k = top_k;
+    a.slot_table = slot_table;
+    a.shadow_off = shadow_off;
+    a.x = x; a.x1 = x1; a.x_split = x_split;
+    const dim3 grid_dim(ffn / 32u, top_k);
+#define REDHIP_SLOT_SLICE(NKC)                                                                                                         \
+    do {                                                                                                                               \
+        static bool attr = false;                                                                                                       \
+        const size_t dyn = slice_lds_bytes(NKC, kSliceRep);                                                                             \
+        if (!attr) {                                                                                                                    \
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(expert_slice_kernel<NKC, kSliceRep, true>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn); \
+            if (e != hipSuccess) return e;                                                                                              \
+            attr = true;                                                                                                                \
+        }                                                                                                                               \
+        REDHIP_LAUNCH((expert_slice_kernel<NKC, kSliceRep, true>), grid_dim, dim3(kWaves * 64), dyn, s, a);                               \
+    } while (0)
+    prof_set_stage(ST_FUSED_EXPERTS);
+    switch (hidden / 512u) {
+        case 1: REDHIP_SLOT_SLICE(1); break;
+        case 2: REDHIP_SLOT_SLICE(2); break;
+        case 4: REDHIP_SLOT_SLICE(4); break;
+        case 8: REDHIP_SLOT_SLICE(8); break;
+        default: return hipErrorInvalidValue;
+    }
+#undef REDHIP_SLOT_SLICE
+    hipError_t e = hipGetLastError();
+    if (e != hipSuccess) return e;
+    prof_set_stage(ST_SLICE_SUM);
+    const SumTail tail{tail_resid, tail_shared, tail_scalar, tail_out2};
+    REDHIP_LAUNCH(slice_sum_kernel, dim3(hidden / 32u), dim3(256), 0, s, partial, top_k * (ffn / 32u), hidden, out, nullptr, nullptr, tail);
     return hipGetLastError();
 }
 
@@ -2280,7 +2376,7 @@ hipError_t launch_batch_slices(const void *experts, uint64_t stride, const void 
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     prof_set_stage(ST_SLICE_SUM);
-    REDHIP_LAUNCH(slice_sum_kernel, dim3(hidden / 32u, ntok), dim3(256), 0, s, partial, (top_k + 1u) * (ffn / 32u), hidden, out, block_context().resid_a, block_context().resid_b);
+    REDHIP_LAUNCH(slice_sum_kernel, dim3(hidden / 32u, ntok), dim3(256), 0, s, partial, (top_k + 1u) * (ffn / 32u), hidden, out, block_context().resid_a, block_context().resid_b, SumTail{nullptr, nullptr, nullptr, nullptr});
     return hipGetLastError();
 }
 

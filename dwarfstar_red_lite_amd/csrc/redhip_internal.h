@@ -368,6 +368,12 @@ hipError_t launch_expert_slices(const void *experts, uint64_t stride, const void
                                 const float *logits, const uint32_t *ids_in, const float *weights_in, const float *scalar_in, uint32_t *ids_out,
                                 float *weights_out, float *scalar_out, const void *xh, const void *xl, const int *xexp, float *partial, float *out,
                                 uint32_t hidden, uint32_t ffn, uint32_t n_expert, uint32_t top_k, hipStream_t s);
+// one token over slots of a pool whose re-laid IQ2_XXS copies (packed gate | up, column-sliced down) lie shadow_off behind the raw bytes
+// that slot_table [top_k] points at; x split to fp16 halves inside the kernel (experts from x_split on read x1 when given); partial
+// [top_k][ffn / 32][hidden]; with tail_resid: out = tail_out2 = tail_resid + (sum + tail_shared * tail_scalar[0]). top_k <= 64
+hipError_t launch_slot_slices(const uint64_t *slot_table, uint64_t shadow_off, const float *weights, uint32_t top_k, uint32_t hidden, uint32_t ffn,
+                              const float *x, const float *x1, uint32_t x_split, float *partial, float *out, const float *tail_resid,
+                              const float *tail_shared, const float *tail_scalar, float *tail_out2, hipStream_t s);
 // the same for 2..16 tokens (at most 128 pairs) whose pairs are grouped by expert: pass_list / n_pass from the pair sort (GroupJob), weights
 // [ntok][top_k] and scalar [ntok] of the routing; partial [ntok][top_k + 1][ffn / 32][hidden]
 hipError_t launch_batch_slices(const void *experts, uint64_t stride, const void *down_cm, uint64_t down_stride, const void *shared, const void *shared_down_cm,

@@ -56,6 +56,16 @@ struct TopkPool {
     static constexpr int kStages = 4;
     Stage stage[kStages];
     int next_stage = 0;
+    // Opt-in fast path for one declared expert shape (all IQ2_XXS): behind the raw bytes of a slot lies a second copy in the layout the
+    // slice kernels read (packed gate | up streams, column-sliced down), written when the slot is loaded. The copy of a slot starts
+    // shadow_off behind the slot's address, the same distance in every slot, so a device-side slot table needs no second table.
+    struct FastShape { uint32_t word = 0, hidden = 0, ffn = 0; uint64_t gate = 0, down = 0, shadow_off = 0, shadow_bytes = 0; };
+    bool fast = false;
+    FastShape fs;
+    uint64_t cls_shadow[RL_TOPK_MAX_CLASSES] = {0};   // bytes behind each slot of the class for its copy (0: the class holds none)
+    std::vector<uint8_t> shadow_ok;               // by slot: the copy matches the slot's raw bytes
+    DevBuf partial;                               // partial output vectors of the slice kernels
+    uint64_t phys(uint32_t c) const { return cls_bytes[c] + cls_shadow[c]; }
     uint32_t *iota = nullptr;                     // device [REDMETAL_TOPK_MAX + 1]: 0, 1, 2, .. (one pair per expert)
     uint64_t *residency = nullptr;                // device [layers][experts]
     uint32_t res_layers = 0, res_experts = 0;
@@ -75,7 +85,7 @@ struct TopkPool {
         std::lock_guard<std::mutex> lk(mu);
         if (!slab_of[slab]) {
             const uint32_t first = in_class / slots_per_slab * slots_per_slab, remaining = (cls_first[c + 1u] - cls_first[c]) - first;
-            const uint64_t bytes = (uint64_t)(remaining < slots_per_slab ? remaining : slots_per_slab) * cls_bytes[c];
+            const uint64_t bytes = (uint64_t)(remaining < slots_per_slab ? remaining : slots_per_slab) * phys(c);
             if (!bytes || allocated > budget - bytes) { TOPK_ERR("top-k slab allocation would exceed hard budget"); return nullptr; }
             void *p = nullptr;
             const hipError_t e = hipMalloc(&p, (size_t)bytes);
@@ -84,7 +94,11 @@ struct TopkPool {
             allocated += bytes;
             ++slabs_made;
         }
-        return slab_of[slab] + (uint64_t)local * cls_bytes[c];
+        return slab_of[slab] + (uint64_t)local * phys(c);
+    }
+    // may calls of this shape run on the slice kernels? (the copies of the slots they name are checked by the caller where it knows them)
+    bool fast_shape(uint32_t word, uint32_t hidden, uint32_t ffn) const {
+        return fast && hidden == fs.hidden && ffn == fs.ffn && word_gate_up(word) == T_IQ2_XXS && word_down(word) == T_IQ2_XXS;
     }
     void mark(const uint32_t *slots, uint32_t n, int delta) {
         std::lock_guard<std::mutex> lk(mu);
@@ -163,6 +177,7 @@ bool ensure_scratch(TopkPool *p, uint32_t n_act_rows, uint32_t hidden, uint32_t 
 // weighted sum in list order (native/redmetal_topk.m:1338-1415 and :1858-1943). x1: experts from x_split on read it. With
 // out == nullptr the sum is left to the caller; with a tail the last launch also adds the residual and the shared expert.
 struct Tail { const float *resid, *shared, *scalar; float *x, *layer_out; };
+constexpr uint32_t kFastMaxTopK = 64u;             // experts per call on the slice kernels (sizes the partial vectors)
 
 __global__ __launch_bounds__(256) void topk_tail_kernel(const float *tmp, const float *weights, uint32_t top_k, uint32_t n,
                                                         const float *resid, const float *shared, const float *scalar, float *x, float *layer_out) {
@@ -177,8 +192,18 @@ __global__ __launch_bounds__(256) void topk_tail_kernel(const float *tmp, const 
 
 bool enqueue_token(TopkPool *p, hipStream_t s, const uint64_t *table_dev, const float *weights_dev, uint32_t top_k, uint32_t type_word,
                    uint32_t hidden, uint32_t ffn, uint64_t gate_bytes, uint64_t up_bytes, uint32_t row_start, uint32_t row_count,
-                   const float *x, const float *x1, uint32_t x_split, float *out, const Tail *tail) {
+                   const float *x, const float *x1, uint32_t x_split, float *out, const Tail *tail, bool slots_fast) {
     std::lock_guard<std::recursive_mutex> lk(p->enc_mu);
+    if (slots_fast && top_k <= kFastMaxTopK && row_start == 0u && row_count == hidden && (out || tail) && p->fast_shape(type_word, hidden, ffn)) {
+        // two launches on the slots' re-laid copies: expert slices, then the sum of their partial vectors (with the tail when asked)
+        float *partial = static_cast<float *>(p->partial.p);
+        const hipError_t e = tail ? launch_slot_slices(table_dev, p->fs.shadow_off, weights_dev, top_k, hidden, ffn, x, x1, x_split, partial, tail->x,
+                                                       tail->resid, tail->shared, tail->scalar, tail->layer_out, s)
+                                  : launch_slot_slices(table_dev, p->fs.shadow_off, weights_dev, top_k, hidden, ffn, x, x1, x_split, partial, out,
+                                                       nullptr, nullptr, nullptr, nullptr, s);
+        if (e != hipSuccess) { TOPK_ERR("top-k HIP command failed: %s", hipGetErrorString(e)); return false; }
+        return true;
+    }
     if (!bind_grids(p, type_word) || !ensure_scratch(p, REDMETAL_TOPK_MAX, hidden, ffn)) return false;
     ExpertSet ex{nullptr, 0, gate_bytes, up_bytes, word_gate_up(type_word), word_down(type_word)};
     ex.table = table_dev;
@@ -304,7 +329,7 @@ int encode_device_impl(redmetal_topk_pool_t h, void *stream, void *slot_table_de
     const uint64_t *table = reinterpret_cast<const uint64_t *>(static_cast<uint8_t *>(slot_table_dev) + slot_table_offset);
     return enqueue_token(p, static_cast<hipStream_t>(stream), table, at(weight_dev, weight_offset), top_k, type_word, hidden, ffn,
                          gate_bytes, up_bytes, 0u, hidden, at(input_dev, input_offset), input1_dev ? at(input1_dev, input1_offset) : nullptr,
-                         x_split, output_dev ? at(output_dev, output_offset) : nullptr, tail) ? 1 : 0;
+                         x_split, output_dev ? at(output_dev, output_offset) : nullptr, tail, true) ? 1 : 0;
 }
 
 }  // namespace
@@ -391,6 +416,7 @@ int redmetal_topk_pool_set_classes(redmetal_topk_pool_t handle, uint32_t n, cons
     if (!n || n > RL_TOPK_MAX_CLASSES || !slot_bytes || !capacity) { TOPK_ERR("invalid top-k slot classes"); return 0; }
     std::lock_guard<std::mutex> lk(p->mu);
     if (p->slabs_made) { TOPK_ERR("top-k slot classes must be set before any slab is allocated"); return 0; }
+    if (p->fast) { TOPK_ERR("top-k slot classes must be set before the fast path is enabled"); return 0; }
     uint64_t total = 0, sz[RL_TOPK_MAX_CLASSES];
     uint32_t slots = 0, slabs = 0, first[RL_TOPK_MAX_CLASSES + 1], slab[RL_TOPK_MAX_CLASSES + 1];
     for (uint32_t c = 0; c < n; ++c) {
@@ -414,6 +440,58 @@ int redmetal_topk_pool_set_classes(redmetal_topk_pool_t handle, uint32_t n, cons
     p->inflight.assign(slots, 0u);
     p->generation.assign(slots, 0u);
     p->slab_of.assign(slabs, nullptr);
+    return 1;
+}
+
+int redhip_topk_pool_enable_fast_path(redmetal_topk_pool_t handle, uint32_t ggml_type, uint32_t hidden_size, uint32_t ffn_size) {
+    TopkPool *p = pool_of(handle);
+    if (!p) return 0;
+    if (!type_word_ok(ggml_type) || word_gate_up(ggml_type) != T_IQ2_XXS || word_down(ggml_type) != T_IQ2_XXS || !fused_iq2_supported(hidden_size, ffn_size) || hidden_size % 32u) {
+        TOPK_ERR("the top-k fast path takes all-IQ2_XXS experts with hidden in {512, 1024, 2048, 4096} and ffn a multiple of 256 up to 1024 (asked: type word 0x%x, hidden=%u, ffn=%u)",
+                 ggml_type, hidden_size, ffn_size);
+        return 0;
+    }
+    std::lock_guard<std::mutex> lk(p->mu);
+    if (p->slabs_made) { TOPK_ERR("the top-k fast path must be enabled before any slab is allocated"); return 0; }
+    if (p->fast) { TOPK_ERR("the top-k fast path is already enabled"); return 0; }
+    TopkPool::FastShape f;
+    f.word = ggml_type; f.hidden = hidden_size; f.ffn = ffn_size;
+    f.gate = (uint64_t)ffn_size * pool_row_bytes(T_IQ2_XXS, hidden_size);
+    f.down = (uint64_t)hidden_size * pool_row_bytes(T_IQ2_XXS, ffn_size);
+    f.shadow_off = round_up(2u * f.gate + f.down, 256u);
+    f.shadow_bytes = 2u * f.gate + f.down;
+    // classes that can hold an expert of this shape grow by the room for its copy; the budget covers both
+    uint64_t shadow[RL_TOPK_MAX_CLASSES] = {0}, total = 0;
+    bool any = false;
+    for (uint32_t c = 0; c < p->n_cls; ++c) {
+        if (p->cls_bytes[c] >= 2u * f.gate + f.down) {
+            const uint64_t need = round_up(f.shadow_off + f.shadow_bytes, 4096u);
+            shadow[c] = need > p->cls_bytes[c] ? need - p->cls_bytes[c] : 0u;
+            any = true;
+        }
+        total += (p->cls_bytes[c] + shadow[c]) * (uint64_t)(p->cls_first[c + 1u] - p->cls_first[c]);
+    }
+    if (!any) { TOPK_ERR("no top-k slot class holds an expert of the fast path's shape"); return 0; }
+    if (p->n_cls == 1u) {
+        // one class sized by the budget: fewer, larger slots
+        const uint64_t cap64 = p->budget / (p->cls_bytes[0] + shadow[0]);
+        if (!cap64) { TOPK_ERR("top-k cache budget cannot fit one expert slot with its copy"); return 0; }
+        p->capacity = cap64 > 0xffffffffull ? 0xffffffffu : (uint32_t)cap64;
+        if (p->slots_per_slab > p->capacity) p->slots_per_slab = p->capacity;
+        p->cls_first[1] = p->capacity;
+        p->cls_slab[1] = (p->capacity + p->slots_per_slab - 1u) / p->slots_per_slab;
+        p->inflight.assign(p->capacity, 0u);
+        p->generation.assign(p->capacity, 0u);
+        p->slab_of.assign(p->cls_slab[1], nullptr);
+    } else if (total > p->budget) {
+        TOPK_ERR("top-k slot classes with the fast path's copies exceed the cache budget");
+        return 0;
+    }
+    if (!p->partial.reserve((size_t)kFastMaxTopK * (ffn_size / 32u) * hidden_size * sizeof(float))) { TOPK_ERR("failed to allocate top-k activation buffers"); return 0; }
+    for (uint32_t c = 0; c < p->n_cls; ++c) p->cls_shadow[c] = shadow[c];
+    p->shadow_ok.assign(p->capacity, 0u);
+    p->fs = f;
+    p->fast = true;
     return 1;
 }
 
@@ -483,6 +561,21 @@ int redmetal_topk_pool_load_expert(redmetal_topk_pool_t h, uint32_t slot_id,
         const hipError_t e = hipMemcpy(base, host.data(), (size_t)payload, hipMemcpyHostToDevice);
         if (e != hipSuccess) { TOPK_ERR("top-k slot upload failed: %s", hipGetErrorString(e)); return 0; }
     }
+    if (p->fast) {
+        // the slot's copy for the slice kernels, when the expert has the declared shape and the slot's class has room for it
+        const TopkPool::FastShape &f = p->fs;
+        bool ok_copy = false;
+        if (gate_bytes == f.gate && up_bytes == f.gate && down_bytes == f.down && f.shadow_off + f.shadow_bytes <= p->phys(p->class_of(slot_id))) {
+            uint8_t *copy = base + f.shadow_off;
+            hipError_t e = launch_repack_iq2xxs(base, f.gate, 2u, f.ffn, f.hidden, false, copy, f.gate, nullptr);
+            if (e == hipSuccess) e = launch_repack_iq2xxs(base + 2u * f.gate, 0u, 1u, f.hidden, f.ffn, true, copy + 2u * f.gate, 0u, nullptr);
+            if (e == hipSuccess) e = hipStreamSynchronize(nullptr);
+            if (e != hipSuccess) { TOPK_ERR("top-k slot re-layout failed: %s", hipGetErrorString(e)); return 0; }
+            ok_copy = true;
+        }
+        std::lock_guard<std::mutex> lk(p->mu);
+        p->shadow_ok[slot_id] = ok_copy ? 1u : 0u;
+    }
     const double ms = now_ms() - t0;
     {
         std::lock_guard<std::mutex> lk(p->mu);
@@ -526,10 +619,15 @@ int redmetal_topk_pool_encode(redmetal_topk_pool_t h, void *stream, const uint32
     }
     hipStream_t s = static_cast<hipStream_t>(stream);
     std::lock_guard<std::recursive_mutex> lk(p->enc_mu);
+    bool copies = p->fast;
+    if (copies) {
+        std::lock_guard<std::mutex> lk2(p->mu);
+        for (uint32_t i = 0; i < top_k; ++i) copies = copies && p->shadow_ok[slot_ids[i]];
+    }
     Staged st;
     if (!stage_lists(p, s, table, router_weights, top_k, {}, &st)) return 0;
     const bool ok = enqueue_token(p, s, st.table, st.w, top_k, ggml_type, hidden_size, ffn_size, gate_bytes[0], up_bytes[0], output_row_start,
-                                  output_row_count, at(input_dev, input_offset), nullptr, 0u, at(output_dev, output_offset), nullptr);
+                                  output_row_count, at(input_dev, input_offset), nullptr, 0u, at(output_dev, output_offset), nullptr, copies);
     stage_done(st, s);
     if (!ok) return 0;
     p->mark(slot_ids, top_k, +1);

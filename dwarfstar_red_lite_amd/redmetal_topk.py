@@ -61,6 +61,11 @@ class RedMetalTopKPool:
         sb, cp = _u64(slot_bytes), _u32(capacity)
         self._check(self.lib.redmetal_topk_pool_set_classes(self.handle, sb.size, sb.ctypes.data, cp.ctypes.data))
 
+    def enable_fast_path(self, type_word, hidden, ffn):
+        """experts of this shape (all IQ2_XXS) also keep a copy in the fused kernels' layout behind their slot's raw bytes (written at
+        load); their single-token calls then run on it. Before the first slab exists; the copies count against the budget."""
+        self._check(self.lib.redhip_topk_pool_enable_fast_path(self.handle, int(type_word), int(hidden), int(ffn)))
+
     def slot_inflight(self, slot_id):
         return bool(self.lib.redmetal_topk_pool_slot_inflight(self.handle, slot_id))
 

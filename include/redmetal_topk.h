@@ -163,6 +163,18 @@ int redmetal_topk_pool_encode_mapped(redmetal_topk_pool_t pool, void *stream,
     uint32_t n_pairs, const uint32_t *pair_token, const float *pair_weight, const uint32_t *expert_start,
     const uint32_t *tok_pair, void *input_dev, uint64_t input_offset, void *output_dev, uint64_t output_offset);
 
+/* No counterpart in the reference. Opt-in, after redmetal_topk_pool_set_classes (if used) and before the first slab exists (no load,
+ * no slot_addresses, no allocate_all yet): experts of one declared shape - every matrix IQ2_XXS (type word 16), hidden_size in
+ * {512, 1024, 2048, 4096}, ffn_size a multiple of 256 up to 1024 - also keep, behind the raw bytes of their slot, a copy in the
+ * layout this library's fused kernels read (packed gate | up streams, column-sliced down matrix), written by
+ * redmetal_topk_pool_load_expert. The single-token calls (encode, execute, encode_device, _into, _into2 with an output, _tail) of that
+ * shape with whole output rows and top_k <= 64 then run as two launches on those copies instead of three on the raw rows; every other
+ * call runs as before, and redmetal_topk_pool_slot_addresses keeps returning the raw bytes. The copies count against the budget: a
+ * slot class that holds such experts grows to twice the expert's bytes (a single-class pool's capacity shrinks accordingly; with
+ * classes set, the call fails when they no longer fit). With the device-driven forms the slot table must hold addresses of this
+ * pool's slots loaded with experts of the declared shape. Returns 1, or 0 with redmetal_topk_last_error(). */
+int redhip_topk_pool_enable_fast_path(redmetal_topk_pool_t pool, uint32_t ggml_type, uint32_t hidden_size, uint32_t ffn_size);
+
 #ifdef __cplusplus
 }
 #endif

@@ -43,7 +43,7 @@ def type_word(cfg):
 class Case:
     """a one-layer GGUF file of `layout`, a pool over it, experts 0 .. n_load - 1 loaded into slots in a scrambled order"""
 
-    def __init__(self, tmp_path, grids, layout, hidden=512, ffn=256, n_expert=16, n_load=None, seed=700, **pool_kw):
+    def __init__(self, tmp_path, grids, layout, hidden=512, ffn=256, n_expert=16, n_load=None, seed=700, fast=False, **pool_kw):
         from dwarfstar_red_lite_amd.moe import gguf_expert_layout
         from dwarfstar_red_lite_amd.redmetal_topk import ExpertLayout, RedMetalTopKPool
         self.cfg = cfg = synth.layer_config(hidden=hidden, ffn=ffn, n_expert=n_expert, top_k=4, layout=layout)
@@ -58,14 +58,20 @@ class Case:
         n_load = n_expert if n_load is None else n_load
         kw = dict(slots_per_slab=5)
         kw.update(pool_kw)
-        self.pool = RedMetalTopKPool(self.path, (n_load + 3) * ((self.slot_bytes + 4095) // 4096 * 4096), self.slot_bytes,
-                                     iq2_xs_grid=grids[0], iq1_m_grid=grids[1], **kw)
+        up = lambda v, a: (v + a - 1) // a * a
+        # with the fast path a slot also holds the re-laid copy of its expert, 256-aligned behind the raw bytes
+        self.slot_phys = up(up(self.slot_bytes, 256) + self.slot_bytes, 4096) if fast else up(self.slot_bytes, 4096)
+        self.pool = RedMetalTopKPool(self.path, (n_load + 3) * self.slot_phys, self.slot_bytes, iq2_xs_grid=grids[0], iq1_m_grid=grids[1], **kw)
+        self.word = type_word(cfg)
+        if fast:
+            assert self.pool.capacity > n_load + 3
+            self.pool.enable_fast_path(self.word, hidden, ffn)
+            assert self.pool.capacity == n_load + 3
         self.slot_of = {}
         for i, e in enumerate(np.random.default_rng(seed).permutation(n_load)):
             self.slot_of[int(e)] = i
             got = self.pool.load(i, self.layouts[e])
             assert got["bytes_read"] == self.slot_bytes
-        self.word = type_word(cfg)
 
     def want(self, experts, weights, x, row_start=0, row_count=None):
         cfg, lay = self.cfg, self.lay
@@ -77,9 +83,10 @@ class Case:
         return acc
 
 
-@pytest.mark.parametrize("layout", ["iq2", "f2", "xs", "m"])
-def test_execute_against_cpu_path(tmp_path, grids, layout):
-    c = Case(tmp_path, grids, layout)
+@pytest.mark.parametrize("layout,fast", [("iq2", False), ("f2", False), ("xs", False), ("m", False), ("iq2", True)])
+def test_execute_against_cpu_path(tmp_path, grids, layout, fast):
+    """fast: the calls with whole output rows run on the slots' re-laid copies, the row windows on the raw rows"""
+    c = Case(tmp_path, grids, layout, fast=fast)
     H, F = c.cfg["hidden"], c.cfg["ffn"]
     rng = np.random.default_rng(5)
     for top_k, row_start, row_count in ((4, 0, H), (1, 0, H), (7, 128, 200), (16, H - 1, 1)):
@@ -176,11 +183,12 @@ def test_slot_classes_and_budget(tmp_path, grids):
     c.pool.close()
 
 
-@pytest.mark.parametrize("layout", ["iq2", "f2"])
-def test_device_driven_forms(tmp_path, grids, layout):
+@pytest.mark.parametrize("layout,fast", [("iq2", False), ("f2", False), ("iq2", True)])
+def test_device_driven_forms(tmp_path, grids, layout, fast):
     """slot addresses gathered on the device from the residency table, weights on the device: into, into with the sum left to the
-    caller, two input vectors, and the fused tail; replayed from a HIP graph as well (these forms copy nothing from the host)"""
-    c = Case(tmp_path, grids, layout)
+    caller, two input vectors, and the fused tail; replayed from a HIP graph as well (these forms copy nothing from the host).
+    fast: on the slots' re-laid copies (the sum left to the caller stays on the raw rows)"""
+    c = Case(tmp_path, grids, layout, fast=fast)
     H, F, E = c.cfg["hidden"], c.cfg["ffn"], 16
     gb = c.layouts[0].gate_bytes
     table_ptr = c.pool.residency_table_init(3, E)
@@ -317,3 +325,41 @@ def test_batched_pairs_with_more_than_sixteen_experts_per_token(tmp_path, grids)
         for t in range(ntok):
             assert rel_l2(got[t], c.want(ids[t], w[t], x[t])) <= REL_L2_TOL, (K, t)
     c.pool.close()
+
+
+def test_fast_path_copies_follow_the_slots(tmp_path, grids):
+    """the re-laid copy of a slot is rewritten whenever the slot is loaded: after a slot changes its expert, calls through the copies
+    (whole rows) and through the raw rows (a row window) both see the new expert; shapes and moments the fast path refuses"""
+    from dwarfstar_red_lite_amd.redmetal_topk import RedMetalTopKPool
+    c = Case(tmp_path, grids, "iq2", hidden=1024, ffn=512, n_expert=12, n_load=8, fast=True)
+    H, F, L = 1024, 512, c.layouts
+    rng = np.random.default_rng(71)
+    x = synth.normed_x(rng, 1, H)[0]
+    w = rng.random(5).astype(np.float32) + 0.1
+    experts = [0, 3, 5, 6, 7]
+    slots = [c.slot_of[e] for e in experts]
+    got, _ = c.pool.execute(slots, [L[e] for e in experts], w, c.word, H, F, 0, H, x)
+    assert rel_l2(got, c.want(experts, w, x)) <= REL_L2_TOL
+    # slot of expert 3 now holds expert 10, the slot of expert 6 expert 11
+    c.pool.load(c.slot_of[3], L[10])
+    c.pool.load(c.slot_of[6], L[11])
+    now = [0, 10, 5, 11, 7]
+    got, _ = c.pool.execute(slots, [L[e] for e in now], w, c.word, H, F, 0, H, x)
+    assert rel_l2(got, c.want(now, w, x)) <= REL_L2_TOL
+    part, _ = c.pool.execute(slots, [L[e] for e in now], w, c.word, H, F, 100, 300, x)
+    assert rel_l2(part, c.want(now, w, x, 100, 300)) <= REL_L2_TOL
+    assert rel_l2(part, got[100:400]) <= 2 * REL_L2_TOL
+    with pytest.raises(RedHipError, match="before any slab"):
+        c.pool.enable_fast_path(c.word, H, F)
+    c.pool.close()
+    pool = RedMetalTopKPool(c.path, 8 * c.slot_phys, c.slot_bytes, iq2_xs_grid=grids[0], iq1_m_grid=grids[1])
+    with pytest.raises(RedHipError, match="all-IQ2_XXS"):
+        pool.enable_fast_path(16 | (21 << 8), H, F)
+    with pytest.raises(RedHipError, match="all-IQ2_XXS"):
+        pool.enable_fast_path(16, 768, F)
+    pool.enable_fast_path(16, H, F)
+    with pytest.raises(RedHipError, match="already enabled"):
+        pool.enable_fast_path(16, H, F)
+    with pytest.raises(RedHipError, match="before the fast path"):
+        pool.set_classes([c.slot_bytes], [2])
+    pool.close()
