@@ -91,7 +91,7 @@ ABI = {
     "redmetal_topk_pool_create": (vp, [C.c_char_p, u64, u64, u32, vp, u32, vp, u32]),
     "redmetal_topk_pool_destroy": (None, [vp]),
     "redmetal_topk_pool_set_classes": (i32, [vp, u32, vp, vp]),
-    "redhip_topk_pool_enable_fast_path": (i32, [vp, u32, u32, u32]),
+    "redhip_topk_pool_enable_fast_path": (i32, [vp, u32, u32, u32, u32]),
     "redmetal_topk_pool_capacity": (u32, [vp]),
     "redmetal_topk_pool_slab_count": (u32, [vp]),
     "redmetal_topk_pool_allocated_bytes": (u64, [vp]),

@@ -186,7 +186,7 @@ hipError_t launch_prefill_packed(const void *experts, uint64_t stride, const voi
                                  const uint32_t *pair_token, const uint32_t *n_unique, uint32_t *tile_group, uint32_t *tile_pair0,
                                  uint32_t *tile_n, uint32_t *n_tiles, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l,
                                  int *act_exp, float *tmp, float *sh_tmp, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok,
-                                 uint32_t n_expert, hipStream_t s, bool tiles_built = false);      // tiles_built: launch_group_pairs wrote the tile lists
+                                 uint32_t n_expert, hipStream_t s, bool tiles_built = false, bool with_shared = true);      // without: no shared expert's tiles (shared, tiled_shared, sh_tmp unused)      // tiles_built: launch_group_pairs wrote the tile lists
 // Tile lists of a chunk for the prefill kernels. Groups 0..U-1 are the distinct routed experts (pairs expert_start[u] ..
 // expert_start[u + 1]), group U is the shared expert with pairs P .. P + shared_ntok (0: no shared tiles). A tile = (group, first pair,
 // number of pairs). Three lists in the same arrays, list l from entry l * list_stride on (list_stride = prefill_tile_bound of the call),

@@ -1445,13 +1445,13 @@ hipError_t launch_prefill_packed(const void *experts, uint64_t stride, const voi
                                  const uint32_t *pair_token, const uint32_t *n_unique, uint32_t *tile_group, uint32_t *tile_pair0,
                                  uint32_t *tile_n, uint32_t *n_tiles, const void *xh, const void *xl, const int *xexp, void *act_h, void *act_l,
                                  int *act_exp, float *tmp, float *sh_tmp, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok,
-                                 uint32_t n_expert, hipStream_t s, bool tiles_built) {
+                                 uint32_t n_expert, hipStream_t s, bool tiles_built, bool with_shared) {
     if (!fused_iq2_supported(hidden, ffn) || hidden / 512u > 4u || !ntok) return hipErrorInvalidValue;
     const uint32_t P = ntok * top_k;
     hipError_t e = hipSuccess;
     if (!tiles_built) {
         prof_set_stage(ST_GROUP);
-        const TileLists tl{tile_group, tile_pair0, tile_n, n_tiles, prefill_tile_bound(ntok, top_k, n_expert), ntok};
+        const TileLists tl{tile_group, tile_pair0, tile_n, n_tiles, prefill_tile_bound(ntok, top_k, n_expert), with_shared ? ntok : 0u};
         REDHIP_LAUNCH(build_tiles_kernel, dim3(1), dim3(1024), 0, s, expert_start, n_unique, P, tl);
         e = hipGetLastError();
         if (e != hipSuccess) return e;
@@ -1461,7 +1461,7 @@ hipError_t launch_prefill_packed(const void *experts, uint64_t stride, const voi
                   static_cast<_Float16 *>(act_h), static_cast<_Float16 *>(act_l), act_exp, tmp, sh_tmp, hidden, ffn, top_k, ntok};
     const uint32_t tile_bound = prefill_tile_bound(ntok, top_k, n_expert);
     const dim3 grid(tile_bound < 256u ? tile_bound : 256u), block(kWaves * 64);
-    if (tiled_experts && tiled_shared && ffn <= 512u) {          // tile-major copy present: activations of a tile in registers
+    if (tiled_experts && (tiled_shared || !with_shared) && ffn <= 512u) {          // tile-major copy present: activations of a tile in registers
         const TiledArgs ta{a, static_cast<const uint8_t *>(tiled_experts), static_cast<const uint8_t *>(tiled_shared), nullptr, nullptr, 0u};
         const dim3 rblock(kRegWaves * 64), rgrid(tile_grid(tile_bound));
         e = launch_gateup_reg(ta, rgrid, s, tile_bound);

@@ -7,6 +7,7 @@
 #include <fcntl.h>
 #include <sys/stat.h>
 
+#include <algorithm>
 #include <mutex>
 #include <vector>
 
@@ -48,7 +49,7 @@ struct TopkPool {
     // host lists of a call (slot addresses, weights, pair arrays) travel through a ring of pinned host buffers, each with a
     // device buffer of its own; an event recorded behind the call's last launch says when both may be used again
     struct Stage {
-        void *host = nullptr, *dev = nullptr;
+        void *host = nullptr, *host_dev = nullptr, *dev = nullptr;      // host_dev: the pinned buffer as the device addresses it
         size_t cap = 0;
         hipEvent_t done = nullptr;
         bool used = false;
@@ -59,12 +60,16 @@ struct TopkPool {
     // Opt-in fast path for one declared expert shape (all IQ2_XXS): behind the raw bytes of a slot lies a second copy in the layout the
     // slice kernels read (packed gate | up streams, column-sliced down), written when the slot is loaded. The copy of a slot starts
     // shadow_off behind the slot's address, the same distance in every slot, so a device-side slot table needs no second table.
-    struct FastShape { uint32_t word = 0, hidden = 0, ffn = 0; uint64_t gate = 0, down = 0, shadow_off = 0, shadow_bytes = 0; };
+    // With REDHIP_TOPK_FAST_TILES a third copy follows tile_off behind the slot's address: the three matrices tile-major, as the prefill
+    // tile kernels read them; the batched form then runs on those kernels.
+    struct FastShape { uint32_t word = 0, hidden = 0, ffn = 0; uint64_t gate = 0, down = 0, shadow_off = 0, tile_off = 0, slot_need = 0; bool tiles = false; };
     bool fast = false;
     FastShape fs;
     uint64_t cls_shadow[RL_TOPK_MAX_CLASSES] = {0};   // bytes behind each slot of the class for its copy (0: the class holds none)
     std::vector<uint8_t> shadow_ok;               // by slot: the copy matches the slot's raw bytes
     DevBuf partial;                               // partial output vectors of the slice kernels
+    DevBuf stage_down;                            // load: the row-major packed down matrix on its way to the tile-major copy
+    DevBuf chunk;                                 // batched form on the tile kernels: fp16 halves of x and of the activations, tile lists
     uint64_t phys(uint32_t c) const { return cls_bytes[c] + cls_shadow[c]; }
     uint32_t *iota = nullptr;                     // device [REDMETAL_TOPK_MAX + 1]: 0, 1, 2, .. (one pair per expert)
     uint64_t *residency = nullptr;                // device [layers][experts]
@@ -147,10 +152,18 @@ bool validate(TopkPool *p, const uint32_t *slot_ids, const uint64_t *gate_bytes,
         return false;
     }
     if (!pool_shape_ok(hidden, ffn, batched)) return false;
-    for (uint32_t i = 0; i < top_k; ++i) {
-        if (slot_ids[i] >= p->capacity) { TOPK_ERR("top-k slot %u exceeds capacity %u", slot_ids[i], p->capacity); return false; }
-        for (uint32_t j = 0; j < i; ++j)
-            if (slot_ids[i] == slot_ids[j]) { TOPK_ERR("top-k slot list contains duplicate slot %u", slot_ids[i]); return false; }
+    if (top_k <= 32u) {
+        for (uint32_t i = 0; i < top_k; ++i) {
+            if (slot_ids[i] >= p->capacity) { TOPK_ERR("top-k slot %u exceeds capacity %u", slot_ids[i], p->capacity); return false; }
+            for (uint32_t j = 0; j < i; ++j)
+                if (slot_ids[i] == slot_ids[j]) { TOPK_ERR("top-k slot list contains duplicate slot %u", slot_ids[i]); return false; }
+        }
+    } else {                                            // long lists (the batched form): one pass over a sorted copy's neighbours
+        std::vector<uint32_t> sorted(slot_ids, slot_ids + top_k);
+        for (uint32_t v : sorted) if (v >= p->capacity) { TOPK_ERR("top-k slot %u exceeds capacity %u", v, p->capacity); return false; }
+        std::sort(sorted.begin(), sorted.end());
+        for (uint32_t i = 1; i < top_k; ++i)
+            if (sorted[i] == sorted[i - 1u]) { TOPK_ERR("top-k slot list contains duplicate slot %u", sorted[i]); return false; }
     }
     const uint64_t expect_gate = (uint64_t)ffn * pool_row_bytes(word_gate_up(type_word), hidden);
     const uint64_t expect_down = (uint64_t)hidden * pool_row_bytes(word_down(type_word), ffn);
@@ -222,6 +235,10 @@ bool enqueue_token(TopkPool *p, hipStream_t s, const uint64_t *table_dev, const 
     return true;
 }
 
+__global__ __launch_bounds__(256) void stage_copy_kernel(uint4 *dst, const uint4 *src, uint32_t n16) {
+    for (uint32_t i = blockIdx.x * 256u + threadIdx.x; i < n16; i += gridDim.x * 256u) dst[i] = src[i];
+}
+
 // host lists of one call -> device through the next pinned stage. Layout: table u64 [n_table] | weights f32 [n_w] | u32 lists.
 // The caller records the stage's event behind its last launch (stage_done).
 struct Staged { uint64_t *table; float *w; uint32_t *u; TopkPool::Stage *stage; };
@@ -241,8 +258,9 @@ bool stage_lists(TopkPool *p, hipStream_t s, const std::vector<uint64_t> &table,
         if (st->dev) (void)hipFree(st->dev);
         st->host = st->dev = nullptr;
         st->cap = 0;
-        const size_t want = total < 65536u ? 65536u : total;
-        if (hipHostMalloc(&st->host, want, hipHostMallocDefault) != hipSuccess || hipMalloc(&st->dev, want) != hipSuccess ||
+        const size_t want = ((total < 65536u ? 65536u : total) + 15u) & ~(size_t)15u;
+        if (hipHostMalloc(&st->host, want, hipHostMallocDefault) != hipSuccess || hipHostGetDevicePointer(&st->host_dev, st->host, 0) != hipSuccess ||
+            hipMalloc(&st->dev, want) != hipSuccess ||
             (!st->done && hipEventCreateWithFlags(&st->done, hipEventDisableTiming) != hipSuccess)) {
             TOPK_ERR("failed to allocate top-k table buffers");
             return false;
@@ -253,7 +271,12 @@ bool stage_lists(TopkPool *p, hipStream_t s, const std::vector<uint64_t> &table,
     memcpy(host, table.data(), tb);
     if (n_w) memcpy(host + tb, w, n_w * 4u);
     if (ub) memcpy(host + tb + wb, u.data(), ub);
-    const hipError_t e = hipMemcpyAsync(base, host, total, hipMemcpyHostToDevice, s);
+    // a kernel reads the pinned buffer: the launches behind it follow in the same queue, without the hand-over between the copy engine
+    // and the compute queue that a stream-ordered memcpy costs (tens of microseconds per call)
+    const uint32_t n16 = (uint32_t)((total + 15u) / 16u);
+    hipLaunchKernelGGL(stage_copy_kernel, dim3((n16 + 255u) / 256u < 64u ? (n16 + 255u) / 256u : 64u), dim3(256), 0, s, reinterpret_cast<uint4 *>(base),
+                       static_cast<const uint4 *>(st->host_dev), n16);
+    const hipError_t e = hipGetLastError();
     if (e != hipSuccess) { TOPK_ERR("top-k table upload failed: %s", hipGetErrorString(e)); return false; }
     out->table = reinterpret_cast<uint64_t *>(base);
     out->w = reinterpret_cast<float *>(base + tb);
@@ -292,6 +315,62 @@ bool enqueue_pairs(TopkPool *p, hipStream_t s, const std::vector<uint64_t> &gate
     dn.table = st.table + n_expert;
     hipError_t e = launch_batch_gateup(gu, nullptr, d_start, d_pair_token, nullptr, n_expert, n_pairs, hidden, ffn, x, act, s);
     if (e == hipSuccess) e = launch_batch_down(dn, nullptr, d_start, nullptr, n_expert, n_pairs, hidden, ffn, act, tmp, s);
+    if (e == hipSuccess) e = launch_batch_combine(tmp, st.w, d_tok_pair, ntok, top_k, nullptr, nullptr, hidden, out + (uint64_t)tok_first * hidden, s);
+    stage_done(st, s);
+    if (e != hipSuccess) { TOPK_ERR("batched top-k HIP command failed: %s", hipGetErrorString(e)); return false; }
+    return true;
+}
+
+// The same pairs on the prefill tile kernels, for slots that hold tile-major copies: x split to fp16 halves per token, tiles of up to 32
+// pairs per expert on the MFMA units (gate / up + SwiGLU, then down rows into tmp[pair]), combine in selection order. An expert is named
+// by the distance of its slot from the lowest slot of the call, in units of 256 bytes (slots are 4096-aligned, HBM is far below 1 TB).
+bool enqueue_pairs_tiles(TopkPool *p, hipStream_t s, const std::vector<uint64_t> &slot_addr, uint32_t n_expert, uint32_t hidden, uint32_t ffn,
+                         uint32_t tok_first, uint32_t ntok, uint32_t top_k, uint32_t n_pairs, const uint32_t *pair_token, const float *pair_weight,
+                         const uint32_t *expert_start, const uint32_t *tok_pair, const float *x, float *out) {
+    std::lock_guard<std::recursive_mutex> lk(p->enc_mu);
+    uint64_t lowest = slot_addr[0];
+    for (uint64_t a : slot_addr) lowest = a < lowest ? a : lowest;
+    std::vector<uint32_t> u;
+    u.reserve((size_t)n_pairs * 2u + 2u * n_expert + 2u);
+    u.insert(u.end(), pair_token, pair_token + n_pairs);
+    u.insert(u.end(), expert_start, expert_start + n_expert + 1u);
+    u.insert(u.end(), tok_pair, tok_pair + (size_t)ntok * top_k);
+    for (uint64_t a : slot_addr) {
+        const uint64_t d = a - lowest;
+        if ((d & 255u) || (d >> 8) > 0xffffffffull) { TOPK_ERR("top-k slots of one call lie too far apart"); return false; }
+        u.push_back((uint32_t)(d >> 8));
+    }
+    u.push_back(n_expert);
+    // scratch of the call: rows of x up to the last token of the call, n_pairs activation rows
+    const size_t rows = (size_t)tok_first + ntok, arows = (size_t)n_pairs + ntok;
+    const uint32_t bound = prefill_tile_bound(ntok, top_k, n_expert);
+    auto a256 = [](size_t v) { return (v + 255u) & ~(size_t)255u; };
+    const size_t x_half = a256(rows * hidden * 2u), x_exp = a256(rows * 4u), a_half = a256(arows * ffn * 2u), a_exp = a256(arows * (ffn / 32u) * 4u), tl = a256(12u * (size_t)bound);
+    if (!p->chunk.reserve(2u * x_half + 2u * x_exp + 2u * a_half + a_exp + 4u * tl) || !p->tmp_b.reserve((size_t)n_pairs * hidden * sizeof(float))) {
+        TOPK_ERR("failed to allocate top-k activation buffers");
+        return false;
+    }
+    uint8_t *w = static_cast<uint8_t *>(p->chunk.p);
+    void *xh = w; w += x_half;
+    void *xl = w; w += x_half;
+    int *xexp = reinterpret_cast<int *>(w); w += x_exp;
+    float *gate_unused = reinterpret_cast<float *>(w); w += x_exp;
+    void *act_h = w; w += a_half;
+    void *act_l = w; w += a_half;
+    int *act_exp = reinterpret_cast<int *>(w); w += a_exp;
+    uint32_t *tile_group = reinterpret_cast<uint32_t *>(w); w += tl;
+    uint32_t *tile_pair0 = reinterpret_cast<uint32_t *>(w); w += tl;
+    uint32_t *tile_n = reinterpret_cast<uint32_t *>(w); w += tl;
+    uint32_t *n_tiles = reinterpret_cast<uint32_t *>(w);
+    Staged st;
+    if (!stage_lists(p, s, {}, pair_weight, n_pairs, u, &st)) return false;
+    const uint32_t *d_pair_token = st.u, *d_start = st.u + n_pairs, *d_tok_pair = d_start + n_expert + 1u, *d_uid = d_tok_pair + (size_t)ntok * top_k, *d_unique = d_uid + n_expert;
+    float *tmp = static_cast<float *>(p->tmp_b.p);
+    const uint8_t *tiles = reinterpret_cast<const uint8_t *>(lowest + p->fs.tile_off);
+    // (the split kernel also forms a gate logit per row from a second vector: x itself stands in, the result is not used)
+    hipError_t e = launch_prep(x, x, (uint32_t)rows, hidden, xh, xl, xexp, gate_unused, s, nullptr, nullptr);
+    if (e == hipSuccess) e = launch_prefill_packed(nullptr, 256u, nullptr, tiles, nullptr, d_uid, d_start, d_pair_token, d_unique, tile_group, tile_pair0, tile_n, n_tiles,
+                                                   xh, xl, xexp, act_h, act_l, act_exp, tmp, nullptr, hidden, ffn, top_k, ntok, n_expert, s, false, false);
     if (e == hipSuccess) e = launch_batch_combine(tmp, st.w, d_tok_pair, ntok, top_k, nullptr, nullptr, hidden, out + (uint64_t)tok_first * hidden, s);
     stage_done(st, s);
     if (e != hipSuccess) { TOPK_ERR("batched top-k HIP command failed: %s", hipGetErrorString(e)); return false; }
@@ -443,12 +522,16 @@ int redmetal_topk_pool_set_classes(redmetal_topk_pool_t handle, uint32_t n, cons
     return 1;
 }
 
-int redhip_topk_pool_enable_fast_path(redmetal_topk_pool_t handle, uint32_t ggml_type, uint32_t hidden_size, uint32_t ffn_size) {
+int redhip_topk_pool_enable_fast_path(redmetal_topk_pool_t handle, uint32_t ggml_type, uint32_t hidden_size, uint32_t ffn_size, uint32_t flags) {
     TopkPool *p = pool_of(handle);
     if (!p) return 0;
     if (!type_word_ok(ggml_type) || word_gate_up(ggml_type) != T_IQ2_XXS || word_down(ggml_type) != T_IQ2_XXS || !fused_iq2_supported(hidden_size, ffn_size) || hidden_size % 32u) {
         TOPK_ERR("the top-k fast path takes all-IQ2_XXS experts with hidden in {512, 1024, 2048, 4096} and ffn a multiple of 256 up to 1024 (asked: type word 0x%x, hidden=%u, ffn=%u)",
                  ggml_type, hidden_size, ffn_size);
+        return 0;
+    }
+    if ((flags & ~REDHIP_TOPK_FAST_TILES) || ((flags & REDHIP_TOPK_FAST_TILES) && (ffn_size > 512u || hidden_size > 2048u))) {
+        TOPK_ERR("the top-k fast path keeps tile-major copies for hidden <= 2048 and ffn <= 512 only (asked: hidden=%u, ffn=%u, flags 0x%x)", hidden_size, ffn_size, flags);
         return 0;
     }
     std::lock_guard<std::mutex> lk(p->mu);
@@ -458,15 +541,17 @@ int redhip_topk_pool_enable_fast_path(redmetal_topk_pool_t handle, uint32_t ggml
     f.word = ggml_type; f.hidden = hidden_size; f.ffn = ffn_size;
     f.gate = (uint64_t)ffn_size * pool_row_bytes(T_IQ2_XXS, hidden_size);
     f.down = (uint64_t)hidden_size * pool_row_bytes(T_IQ2_XXS, ffn_size);
-    f.shadow_off = round_up(2u * f.gate + f.down, 256u);
-    f.shadow_bytes = 2u * f.gate + f.down;
+    const uint64_t payload = 2u * f.gate + f.down;
+    f.tiles = (flags & REDHIP_TOPK_FAST_TILES) != 0u;
+    f.shadow_off = round_up(payload, 256u);
+    f.tile_off = 2u * f.shadow_off;
+    f.slot_need = round_up((f.tiles ? f.tile_off : f.shadow_off) + payload, 4096u);
     // classes that can hold an expert of this shape grow by the room for its copy; the budget covers both
     uint64_t shadow[RL_TOPK_MAX_CLASSES] = {0}, total = 0;
     bool any = false;
     for (uint32_t c = 0; c < p->n_cls; ++c) {
-        if (p->cls_bytes[c] >= 2u * f.gate + f.down) {
-            const uint64_t need = round_up(f.shadow_off + f.shadow_bytes, 4096u);
-            shadow[c] = need > p->cls_bytes[c] ? need - p->cls_bytes[c] : 0u;
+        if (p->cls_bytes[c] >= payload) {
+            shadow[c] = f.slot_need > p->cls_bytes[c] ? f.slot_need - p->cls_bytes[c] : 0u;
             any = true;
         }
         total += (p->cls_bytes[c] + shadow[c]) * (uint64_t)(p->cls_first[c + 1u] - p->cls_first[c]);
@@ -487,7 +572,10 @@ int redhip_topk_pool_enable_fast_path(redmetal_topk_pool_t handle, uint32_t ggml
         TOPK_ERR("top-k slot classes with the fast path's copies exceed the cache budget");
         return 0;
     }
-    if (!p->partial.reserve((size_t)kFastMaxTopK * (ffn_size / 32u) * hidden_size * sizeof(float))) { TOPK_ERR("failed to allocate top-k activation buffers"); return 0; }
+    if (!p->partial.reserve((size_t)kFastMaxTopK * (ffn_size / 32u) * hidden_size * sizeof(float)) || (f.tiles && !p->stage_down.reserve((size_t)f.down))) {
+        TOPK_ERR("failed to allocate top-k activation buffers");
+        return 0;
+    }
     for (uint32_t c = 0; c < p->n_cls; ++c) p->cls_shadow[c] = shadow[c];
     p->shadow_ok.assign(p->capacity, 0u);
     p->fs = f;
@@ -565,10 +653,15 @@ int redmetal_topk_pool_load_expert(redmetal_topk_pool_t h, uint32_t slot_id,
         // the slot's copy for the slice kernels, when the expert has the declared shape and the slot's class has room for it
         const TopkPool::FastShape &f = p->fs;
         bool ok_copy = false;
-        if (gate_bytes == f.gate && up_bytes == f.gate && down_bytes == f.down && f.shadow_off + f.shadow_bytes <= p->phys(p->class_of(slot_id))) {
-            uint8_t *copy = base + f.shadow_off;
+        if (gate_bytes == f.gate && up_bytes == f.gate && down_bytes == f.down && f.slot_need <= p->phys(p->class_of(slot_id))) {
+            uint8_t *copy = base + f.shadow_off, *tiles = base + f.tile_off;
             hipError_t e = launch_repack_iq2xxs(base, f.gate, 2u, f.ffn, f.hidden, false, copy, f.gate, nullptr);
             if (e == hipSuccess) e = launch_repack_iq2xxs(base + 2u * f.gate, 0u, 1u, f.hidden, f.ffn, true, copy + 2u * f.gate, 0u, nullptr);
+            if (f.tiles) {
+                if (e == hipSuccess) e = launch_tile_packed(copy, f.gate, 2u, f.ffn, f.hidden, tiles, f.gate, nullptr);
+                if (e == hipSuccess) e = launch_repack_iq2xxs(base + 2u * f.gate, 0u, 1u, f.hidden, f.ffn, false, p->stage_down.p, 0u, nullptr);
+                if (e == hipSuccess) e = launch_tile_packed(p->stage_down.p, 0u, 1u, f.hidden, f.ffn, tiles + 2u * f.gate, 0u, nullptr);
+            }
             if (e == hipSuccess) e = hipStreamSynchronize(nullptr);
             if (e != hipSuccess) { TOPK_ERR("top-k slot re-layout failed: %s", hipGetErrorString(e)); return 0; }
             ok_copy = true;
@@ -767,9 +860,16 @@ int redmetal_topk_pool_encode_batched(redmetal_topk_pool_t h, void *stream, cons
         if (!base) return 0;
         table[i] = (uint64_t)(uintptr_t)base;
     }
-    if (!enqueue_pairs(p, static_cast<hipStream_t>(stream), table, table, gate_bytes[0], gate_bytes[0] + up_bytes[0], n_expert, ggml_type,
-                       hidden_size, ffn_size, tok_first, ntok, top_k, n_pairs, pair_token, pair_weight, expert_start, tok_pair,
-                       at(input_dev, input_offset), at(output_dev, output_offset))) return 0;
+    bool tiles = p->fast && p->fs.tiles && p->fast_shape(ggml_type, hidden_size, ffn_size) && n_expert <= 1024u;
+    if (tiles) {
+        std::lock_guard<std::mutex> lk(p->mu);
+        for (uint32_t i = 0; i < n_expert; ++i) tiles = tiles && p->shadow_ok[slot_ids[i]];
+    }
+    if (tiles ? !enqueue_pairs_tiles(p, static_cast<hipStream_t>(stream), table, n_expert, hidden_size, ffn_size, tok_first, ntok, top_k, n_pairs, pair_token,
+                                     pair_weight, expert_start, tok_pair, at(input_dev, input_offset), at(output_dev, output_offset))
+              : !enqueue_pairs(p, static_cast<hipStream_t>(stream), table, table, gate_bytes[0], gate_bytes[0] + up_bytes[0], n_expert, ggml_type,
+                               hidden_size, ffn_size, tok_first, ntok, top_k, n_pairs, pair_token, pair_weight, expert_start, tok_pair,
+                               at(input_dev, input_offset), at(output_dev, output_offset))) return 0;
     p->mark(slot_ids, n_expert, +1);
     return 1;
 }

@@ -61,10 +61,11 @@ class RedMetalTopKPool:
         sb, cp = _u64(slot_bytes), _u32(capacity)
         self._check(self.lib.redmetal_topk_pool_set_classes(self.handle, sb.size, sb.ctypes.data, cp.ctypes.data))
 
-    def enable_fast_path(self, type_word, hidden, ffn):
+    def enable_fast_path(self, type_word, hidden, ffn, tiles=False):
         """experts of this shape (all IQ2_XXS) also keep a copy in the fused kernels' layout behind their slot's raw bytes (written at
-        load); their single-token calls then run on it. Before the first slab exists; the copies count against the budget."""
-        self._check(self.lib.redhip_topk_pool_enable_fast_path(self.handle, int(type_word), int(hidden), int(ffn)))
+        load); their single-token calls then run on it, and with `tiles` (a third, tile-major copy) the batched form runs on the prefill
+        tile kernels. Before the first slab exists; the copies count against the budget."""
+        self._check(self.lib.redhip_topk_pool_enable_fast_path(self.handle, int(type_word), int(hidden), int(ffn), 1 if tiles else 0))
 
     def slot_inflight(self, slot_id):
         return bool(self.lib.redmetal_topk_pool_slot_inflight(self.handle, slot_id))

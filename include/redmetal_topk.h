@@ -172,8 +172,12 @@ int redmetal_topk_pool_encode_mapped(redmetal_topk_pool_t pool, void *stream,
  * call runs as before, and redmetal_topk_pool_slot_addresses keeps returning the raw bytes. The copies count against the budget: a
  * slot class that holds such experts grows to twice the expert's bytes (a single-class pool's capacity shrinks accordingly; with
  * classes set, the call fails when they no longer fit). With the device-driven forms the slot table must hold addresses of this
- * pool's slots loaded with experts of the declared shape. Returns 1, or 0 with redmetal_topk_last_error(). */
-int redhip_topk_pool_enable_fast_path(redmetal_topk_pool_t pool, uint32_t ggml_type, uint32_t hidden_size, uint32_t ffn_size);
+ * pool's slots loaded with experts of the declared shape. flags: REDHIP_TOPK_FAST_TILES (hidden_size <= 2048 and ffn_size <= 512)
+ * adds a third copy per slot, tile-major as this library's prefill kernels read it (the slot class grows to three times the expert's
+ * bytes); redmetal_topk_pool_encode_batched of that shape then runs on those kernels - tiles of up to 32 pairs per expert on the
+ * matrix units - when every slot it names holds its copies; 0: none. Returns 1, or 0 with redmetal_topk_last_error(). */
+#define REDHIP_TOPK_FAST_TILES 1u
+int redhip_topk_pool_enable_fast_path(redmetal_topk_pool_t pool, uint32_t ggml_type, uint32_t hidden_size, uint32_t ffn_size, uint32_t flags);
 
 #ifdef __cplusplus
 }

@@ -43,7 +43,7 @@ def type_word(cfg):
 class Case:
     """a one-layer GGUF file of `layout`, a pool over it, experts 0 .. n_load - 1 loaded into slots in a scrambled order"""
 
-    def __init__(self, tmp_path, grids, layout, hidden=512, ffn=256, n_expert=16, n_load=None, seed=700, fast=False, **pool_kw):
+    def __init__(self, tmp_path, grids, layout, hidden=512, ffn=256, n_expert=16, n_load=None, seed=700, fast=False, tiles=False, **pool_kw):
         from dwarfstar_red_lite_amd.moe import gguf_expert_layout
         from dwarfstar_red_lite_amd.redmetal_topk import ExpertLayout, RedMetalTopKPool
         self.cfg = cfg = synth.layer_config(hidden=hidden, ffn=ffn, n_expert=n_expert, top_k=4, layout=layout)
@@ -60,12 +60,13 @@ class Case:
         kw.update(pool_kw)
         up = lambda v, a: (v + a - 1) // a * a
         # with the fast path a slot also holds the re-laid copy of its expert, 256-aligned behind the raw bytes
-        self.slot_phys = up(up(self.slot_bytes, 256) + self.slot_bytes, 4096) if fast else up(self.slot_bytes, 4096)
+        # (and with tiles a third, tile-major one)
+        self.slot_phys = up((2 if tiles else 1) * up(self.slot_bytes, 256) + self.slot_bytes, 4096) if fast else up(self.slot_bytes, 4096)
         self.pool = RedMetalTopKPool(self.path, (n_load + 3) * self.slot_phys, self.slot_bytes, iq2_xs_grid=grids[0], iq1_m_grid=grids[1], **kw)
         self.word = type_word(cfg)
         if fast:
             assert self.pool.capacity > n_load + 3
-            self.pool.enable_fast_path(self.word, hidden, ffn)
+            self.pool.enable_fast_path(self.word, hidden, ffn, tiles=tiles)
             assert self.pool.capacity == n_load + 3
         self.slot_of = {}
         for i, e in enumerate(np.random.default_rng(seed).permutation(n_load)):
@@ -256,11 +257,12 @@ def test_device_driven_forms(tmp_path, grids, layout, fast):
     c.pool.close()
 
 
-@pytest.mark.parametrize("layout", ["iq2", "f2", "xs"])
-def test_batched_and_mapped_pairs(tmp_path, grids, layout):
+@pytest.mark.parametrize("layout,tiles", [("iq2", False), ("f2", False), ("xs", False), ("iq2", True)])
+def test_batched_and_mapped_pairs(tmp_path, grids, layout, tiles):
     """prefill form: pairs sorted by expert over a ragged routing (an expert with 19 pairs, experts with one, experts with none), tokens
-    tok_first .. of a larger buffer; the same pairs on experts read in place from device copies of the whole tensors"""
-    c = Case(tmp_path, grids, layout)
+    tok_first .. of a larger buffer; the same pairs on experts read in place from device copies of the whole tensors.
+    tiles: the batched form on the tile-major copies of the slots (the mapped form, which has no slots, stays on the raw rows)"""
+    c = Case(tmp_path, grids, layout, fast=tiles, tiles=tiles)
     H, F, E, K = c.cfg["hidden"], c.cfg["ffn"], 16, 3
     rng = np.random.default_rng(10)
     tok_first, ntok = 2, 21
@@ -293,7 +295,10 @@ def test_batched_and_mapped_pairs(tmp_path, grids, layout):
     c.pool.encode_mapped(stream, g_dev.data_ptr(), u_dev.data_ptr(), d_dev.data_ptr(), L0.gate_bytes, L0.up_bytes, L0.down_bytes, uid, c.word, H, F,
                          tok_first, ntok, K, ptok + tok_first, pw, start, tp, x_dev.data_ptr(), out2.data_ptr())
     torch.cuda.synchronize()
-    assert torch.equal(out2[tok_first:], out[tok_first:])              # same kernels on the same bytes
+    if tiles:
+        assert rel_l2(out2[tok_first:].cpu().numpy(), out[tok_first:].cpu().numpy()) <= REL_L2_TOL
+    else:
+        assert torch.equal(out2[tok_first:], out[tok_first:])          # same kernels on the same bytes
     with pytest.raises(RedHipError, match="expert_start is inconsistent"):
         c.pool.encode_batched(stream, slots, [c.layouts[int(e)] for e in uid], c.word, H, F, tok_first, ntok, K, ptok + tok_first, pw, start[::-1].copy(), tp,
                               x_dev.data_ptr(), out.data_ptr())
@@ -363,3 +368,36 @@ def test_fast_path_copies_follow_the_slots(tmp_path, grids):
     with pytest.raises(RedHipError, match="before the fast path"):
         pool.set_classes([c.slot_bytes], [2])
     pool.close()
+
+
+def test_batched_chunk_of_512_tokens_on_the_tile_copies(tmp_path, grids):
+    """a prefill chunk at the full expert shape (hidden 2048, ffn 512, ten of 48 experts per token, 512 tokens) through the batched form
+    on the slots' tile-major copies: every 16th token against the CPU path, every token against the same call on a pool without copies
+    (the raw-row kernels)"""
+    H, F, E, K, ntok = 2048, 512, 48, 10, 512
+    fast = Case(tmp_path, grids, "iq2", hidden=H, ffn=F, n_expert=E, fast=True, tiles=True, slots_per_slab=7)
+    (tmp_path / "raw").mkdir()
+    raw = Case(tmp_path / "raw", grids, "iq2", hidden=H, ffn=F, n_expert=E)
+    rng = np.random.default_rng(12)
+    logits = rng.standard_normal((ntok, E)) + 1.5 * (np.arange(E) < 3)                # three popular experts: wide tiles, narrow ones, singles
+    ids = np.argsort(-logits, axis=1)[:, :K].astype(np.uint32)
+    w = rng.random((ntok, K)).astype(np.float32) + 0.05
+    w /= w.sum(axis=1, keepdims=True)
+    uid, start, ptok, pw, tp = orc.group_pairs(ids, w, E)
+    x = synth.normed_x(rng, ntok, H)
+    x_dev = torch.from_numpy(x).cuda()
+    stream = torch.cuda.current_stream().cuda_stream
+    outs = []
+    for c in (fast, raw):
+        out = torch.zeros((ntok, H), device="cuda")
+        slots = [c.slot_of[int(e)] for e in uid]
+        c.pool.encode_batched(stream, slots, [c.layouts[int(e)] for e in uid], c.word, H, F, 0, ntok, K, ptok, pw, start, tp, x_dev.data_ptr(), out.data_ptr())
+        torch.cuda.synchronize()
+        c.pool.release(slots)
+        outs.append(out.cpu().numpy())
+    for t in range(0, ntok, 16):
+        assert rel_l2(outs[0][t], fast.want(ids[t], w[t], x[t])) <= REL_L2_TOL, t
+    for t in range(ntok):
+        assert rel_l2(outs[0][t], outs[1][t]) <= REL_L2_TOL, t
+    fast.pool.close()
+    raw.pool.close()
