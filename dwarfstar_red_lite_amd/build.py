@@ -31,14 +31,23 @@ def _stale(obj, src, deps):
     return any(os.path.getmtime(d) > t for d in [src] + deps)
 
 
-def build_library(verbose=False, incremental=False, timeline=False):
+ABLATIONS = {"no_mfma": "REDHIP_ABLATE_NO_MFMA", "no_lds": "REDHIP_ABLATE_NO_LDS", "no_sign": "REDHIP_ABLATE_NO_SIGN"}
+
+
+def build_library(verbose=False, incremental=False, timeline=False, ablate=()):
     """incremental: recompile only the sources that changed (or whose headers did) since their object was built.
     timeline: a second library, libredmetal_hip_timeline.so, whose expert kernels store phase stamps (-DREDHIP_TIMELINE; see
-    redhip_timeline_read); load it by pointing REDHIP_LIBRARY at it. The ordinary library is not touched."""
+    redhip_timeline_read); load it by pointing REDHIP_LIBRARY at it. The ordinary library is not touched.
+    ablate (with timeline): names from ABLATIONS; the slice kernels of libredmetal_hip_timeline_<names>.so leave that part of the decode
+    out (matrix instructions, table reads, sign placement). Their results are wrong on purpose: for `timeline.py` only, which times
+    phases and checks no values."""
     hipcc = os.environ.get("HIPCC", "/opt/rocm/bin/hipcc")
-    OBJ = os.path.join(HERE, "build_timeline" if timeline else "build")
-    LIB = os.path.join(HERE, "libredmetal_hip_timeline.so" if timeline else "libredmetal_hip.so")
-    FLAGS = globals()["FLAGS"] + (["-DREDHIP_TIMELINE"] if timeline else [])
+    if ablate and not timeline:
+        raise ValueError("--ablate builds are measurement builds: combine with --timeline")
+    tag = "_timeline" + "".join("_" + a for a in ablate) if timeline else ""
+    OBJ = os.path.join(HERE, "build" + tag)
+    LIB = os.path.join(HERE, "libredmetal_hip%s.so" % tag)
+    FLAGS = globals()["FLAGS"] + (["-DREDHIP_TIMELINE"] if timeline else []) + ["-D" + ABLATIONS[a] for a in ablate]
     os.makedirs(OBJ, exist_ok=True)
     headers = [os.path.join(CSRC, f) for f in os.listdir(CSRC) if f.endswith(".h")]
     headers += [os.path.join(HERE, "..", "include", f) for f in os.listdir(os.path.join(HERE, "..", "include")) if f.endswith(".h")]
@@ -58,4 +67,5 @@ def build_library(verbose=False, incremental=False, timeline=False):
 
 
 if __name__ == "__main__":
-    print(build_library(verbose=True, incremental="--incremental" in sys.argv, timeline="--timeline" in sys.argv))
+    _ablate = tuple(sys.argv[i + 1] for i, a in enumerate(sys.argv[:-1]) if a == "--ablate")
+    print(build_library(verbose=True, incremental="--incremental" in sys.argv, timeline="--timeline" in sys.argv, ablate=_ablate))

@@ -1706,14 +1706,14 @@ __device__ __forceinline__ void signed_weights_lut(const LaneTables &t, uint2 q,
     const uint32_t mag_at = __builtin_amdgcn_perm(q.x, t.mag_lane, 0x03020000u | ((4u + L) << 8));
     const uint32_t field = 7u * L < kLutShift ? q.y << (kLutShift - 7u * L) : q.y >> (7u * L - kLutShift);
     const uint32_t lut_at = (field & (127u << kLutShift)) | t.lut_lane;
-#ifdef EXP_NO_LDS
+#ifdef REDHIP_ABLATE_NO_LDS      // measurement builds only (build.py --ablate): the table reads replaced by register moves, results wrong
     const lds_u32x4 m = {mag_at, lut_at, mag_at ^ 0x1234u, lut_at + 7u};
     const uint32_t e = lut_at ^ mag_at;
 #else
     const lds_u32x4 m = *reinterpret_cast<lds_u32x4_ptr>((uintptr_t)mag_at);
     const uint32_t e = *reinterpret_cast<lds_u32_ptr>((uintptr_t)lut_at);
 #endif
-#ifdef EXP_NO_SIGN
+#ifdef REDHIP_ABLATE_NO_SIGN     // ... the sign placement left out
     b0.u[0] = m.x ^ e; b0.u[1] = m.y; b1.u[0] = m.z; b1.u[1] = m.w;
 #else
     b0.u[0] = (e & 0x80008000u) | m.x;
@@ -1726,7 +1726,7 @@ template <int REP, int LR, uint32_t L>
 __device__ __forceinline__ float4_t group_step_lut(const LaneTables &t, uint2 q, const half4_t *ax, float4_t acc) {
     WeightQuad b0, b1;
     signed_weights_lut<REP, LR, L>(t, q, b0, b1);
-#ifdef EXP_NO_MFMA
+#ifdef REDHIP_ABLATE_NO_MFMA     // ... the matrix instructions left out (the decoded weights stay live)
     asm volatile("" :: "v"(b0.u[0]), "v"(b0.u[1]), "v"(b1.u[0]), "v"(b1.u[1]));
     return acc;
 #else

@@ -70,6 +70,7 @@ def main():
     ran = t[:, 7] > 0                                   # workgroups that reached the last stamp in the last launch that wrote any
     last = t[ran][:, 0].max()
     ran &= t[:, 0] > last - 100000                      # ... within a millisecond of the newest start (older launches had other grids)
+    ran &= (np.diff(t[:, :8], axis=1) >= 0).all(axis=1)  # a workgroup that left early this time still shows an older launch's later stamps
     t = t[ran]
     t0 = t[:, 0].min()
     print("workload: layout %s, %d token(s), routing %s; %d workgroups ran all phases; kernel span %.2f us (first start to last end)" % (
