@@ -445,20 +445,26 @@ __device__ __forceinline__ float norm_scale(double ss, uint32_t n, float eps) { 
 // F32 router: one wave per row (row n_expert is the shared expert's gate vector), the row and x read as float4
 // with lanes interleaved; every wave sees all of x, so the pre-scale exponent needs no extra pass. blockIdx.y = token.
 template <int NV, int WPB = 4>          // float4 per lane: hidden = 256 * NV; WPB waves (rows) per workgroup
-__global__ __launch_bounds__(WPB * 64) void router_f32_kernel(const float *w, RouterArgs a) {
-    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63u, H = a.hidden, tok = blockIdx.y;
+__global__ __launch_bounds__(WPB * 64) void router_f32_kernel(const float *w, const float *x_first, uint32_t hidden_first, uint32_t n_expert_first, RouterArgs a) {
+    // (x_first, hidden_first, n_expert_first repeat a.x, a.hidden, a.n_expert: leading scalar arguments can reach a wave in registers at
+    // its start, so the requests for the activations and for a router row leave before the argument block has come from memory)
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63u, H = hidden_first, tok = blockIdx.y;
     const uint32_t r = blockIdx.x * WPB + wave;
-    const uint32_t n_rows = a.n_expert + 1u + (a.sh_dense ? 2u * a.ffn : 0u);      // router rows, the gate vector, then the shared expert's gate | up rows
-    const float4 *wr = reinterpret_cast<const float4 *>(r < a.n_expert ? w + (uint64_t)r * H : r == a.n_expert ? a.gate_inp
-                                                        : a.sh_dense + (uint64_t)(r < n_rows ? r - a.n_expert - 1u : 0u) * H);
-    const float4 *xv = reinterpret_cast<const float4 *>(a.x + (uint64_t)tok * H);
+    const float4 *xv = reinterpret_cast<const float4 *>(x_first + (uint64_t)tok * H);
     float4 wv[NV], xq[NV];
-    if (r < n_rows) {
+#pragma unroll
+    for (int k = 0; k < NV; ++k) xq[k] = xv[lane + 64u * k];
+    if (r < n_expert_first) {
+        const float4 *wr = reinterpret_cast<const float4 *>(w + (uint64_t)r * H);
 #pragma unroll
         for (int k = 0; k < NV; ++k) wv[k] = wr[lane + 64u * k];
     }
+    const uint32_t n_rows = a.n_expert + 1u + (a.sh_dense ? 2u * a.ffn : 0u);      // router rows, the gate vector, then the shared expert's gate | up rows
+    if (r >= a.n_expert && r < n_rows) {
+        const float4 *wr = reinterpret_cast<const float4 *>(r == a.n_expert ? a.gate_inp : a.sh_dense + (uint64_t)(r - a.n_expert - 1u) * H);
 #pragma unroll
-    for (int k = 0; k < NV; ++k) xq[k] = xv[lane + 64u * k];
+        for (int k = 0; k < NV; ++k) wv[k] = wr[lane + 64u * k];
+    }
     float norm_inv = 1.0f;
     if (a.branch) {                                        // every wave holds the whole vector: the norm needs no workgroup barrier
         const float4 *bv = reinterpret_cast<const float4 *>(a.branch + (uint64_t)tok * H), *nw = reinterpret_cast<const float4 *>(a.norm_w);
@@ -714,10 +720,10 @@ hipError_t launch_router_gemv(uint32_t router_type, const void *w, const float *
     if (router_type == T_F32) {
         const float *wf = static_cast<const float *>(w);
         switch (hidden / 256u) {
-            case 2: REDHIP_LAUNCH(router_f32_kernel<2>, grid8, dim3(256), 0, s, wf, a); break;
-            case 4: REDHIP_LAUNCH(router_f32_kernel<4>, grid8, dim3(256), 0, s, wf, a); break;
-            case 8: REDHIP_LAUNCH(router_f32_kernel<8>, grid8, dim3(256), 0, s, wf, a); break;      // (one or two rows per workgroup instead of four: no difference)
-            case 16: REDHIP_LAUNCH(router_f32_kernel<16>, grid8, dim3(256), 0, s, wf, a); break;
+            case 2: REDHIP_LAUNCH(router_f32_kernel<2>, grid8, dim3(256), 0, s, wf, a.x, a.hidden, a.n_expert, a); break;
+            case 4: REDHIP_LAUNCH(router_f32_kernel<4>, grid8, dim3(256), 0, s, wf, a.x, a.hidden, a.n_expert, a); break;
+            case 8: REDHIP_LAUNCH(router_f32_kernel<8>, grid8, dim3(256), 0, s, wf, a.x, a.hidden, a.n_expert, a); break;      // (one or two rows per workgroup instead of four: no difference)
+            case 16: REDHIP_LAUNCH(router_f32_kernel<16>, grid8, dim3(256), 0, s, wf, a.x, a.hidden, a.n_expert, a); break;
             default: return hipErrorInvalidValue;
         }
     } else if (router_type == T_Q6_K) {
@@ -1311,7 +1317,7 @@ struct GateUpArgs {
 
 // FMT: format of the routed (and a packed shared) expert's gate / up matrices: 0 IQ2_XXS, 1 IQ2_XS, 2 IQ1_M
 template <int NKC, int FMT>        // K chunks of 512 columns in a gate/up row: hidden = 512 * NKC
-__global__ __launch_bounds__(kWaves * 64) void gateup_select_kernel(GateUpArgs a) {
+__global__ __launch_bounds__(kWaves * 64) void gateup_select_kernel(const float *logits_first, uint32_t n_expert_first, uint32_t top_k_first, GateUpArgs a) {
     constexpr int NW = kWaves;
     constexpr int UPW = 16 * NKC / NW;                 // (row-quad, K-chunk) units per wave
     static_assert(UPW >= 1 && UPW * NW == 16 * NKC, "waves must tile the 16 row-quads x NKC chunks");
@@ -1319,7 +1325,14 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_select_kernel(GateUpArgs a
     __shared__ float part[NKC * 64];
     __shared__ SelectOut sel;
 
-    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
+    const uint32_t tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
+    // The leading kernel arguments repeat a.logits, a.n_expert, a.top_k: they can reach a wave in registers at its start, so the selecting
+    // wave's request for the logits leaves before the argument block has come from memory - and before anything else this wave does.
+    if (blockIdx.y < top_k_first && logits_first && wave == 0u) {
+        const float *lg = logits_first + (uint64_t)blockIdx.z * (n_expert_first + 1u);
+        if (n_expert_first <= 512u) wave_select_topk<8>(lg, n_expert_first, top_k_first, &sel);
+        else wave_select_topk<16>(lg, n_expert_first, top_k_first, &sel);
+    }
     const uint32_t H = a.hidden, F = a.ffn, HG = H / 32u, HB = H / 256u;
     if (const uint32_t tok = blockIdx.z) {             // several tokens in one launch: every token is a layer of the grid with buffers of its own
         const uint64_t t = tok;
@@ -1370,11 +1383,7 @@ __global__ __launch_bounds__(kWaves * 64) void gateup_select_kernel(GateUpArgs a
         }
         __syncthreads();                                   // tables; the shared expert does not depend on the routing
     } else if (a.logits) {
-        if (wave == 0u) {        // the other waves have nothing to do until the expert is known
-            if (a.n_expert <= 512u) wave_select_topk<8>(a.logits, a.n_expert, a.top_k, &sel);
-            else wave_select_topk<16>(a.logits, a.n_expert, a.top_k, &sel);
-        }
-        __syncthreads();
+        __syncthreads();                                   // the selection (wave 0, at the kernel's head) and the tables
         expert = sel.ids[slot];
         if (g == 0u && slot == 0u) {
             if (tid < a.top_k) { a.ids_out[tid] = sel.ids[tid]; a.weights_out[tid] = sel.w[tid]; }
@@ -1758,7 +1767,8 @@ __device__ __forceinline__ void group_dot2_lut(uint2 q, const half4_t *ax, const
 
 constexpr int kSliceLut = 32;      // copies of the sign words in the one-token kernel: 16 KB, every lane of a half wave its own bank
 template <int NKC, int REP, bool SLOTS = false>        // hidden = 512 * NKC
-__global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(SliceArgs a) {
+__global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(const float *logits_first, uint32_t n_expert_first, uint32_t top_k_first, const uint64_t *slot_table_first,
+                                                                   const float *x_first, const float *x1_first, uint32_t x_split_first, SliceArgs a) {
     constexpr int NW = kWaves;
     constexpr int UPW = 16 * NKC / NW;                 // (row-quad, K-chunk) units of gate / up per wave
     constexpr int DU = (8 * NKC + NW - 1) / NW;        // units of 64 down rows per wave
@@ -1772,11 +1782,18 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(SliceArgs a) 
     float *act_scale = reinterpret_cast<float *>(act_hl + 64);             // [4]
     SelectOut *sel = reinterpret_cast<SelectOut *>(act_scale + 4);
 
-    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
-    const uint32_t H = a.hidden, F = a.ffn, HG = H / 32u, HB = H / 256u, FG = F / 32u;
+    const uint32_t tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
     const uint32_t g = blockIdx.x, slot = blockIdx.y;
-    const bool is_shared = slot >= a.top_k;
+    // The three leading kernel arguments repeat a.logits, a.n_expert and a.top_k: leading scalar arguments can be handed to a wave in
+    // registers at its start, so the selecting wave's request for the logits does not wait for the argument block to come from memory.
+    const bool is_shared = slot >= top_k_first;
+    const bool selecting = !SLOTS && !is_shared && logits_first;
     REDHIP_STAMP(0);
+    if (selecting && wave == 0u) {                     // first thing in the kernel: everything else of this wave comes behind the selection
+        if (n_expert_first <= 512u) wave_select_topk<8>(logits_first, n_expert_first, top_k_first, sel);
+        else wave_select_topk<16>(logits_first, n_expert_first, top_k_first, sel);
+    }
+    const uint32_t H = a.hidden, F = a.ffn, HG = H / 32u, HB = H / 256u, FG = F / 32u;
 
     // activation operand of the gate / up rows: independent of the routing, requested first
     const uint32_t kc = wave % NKC, q0 = wave / NKC;
@@ -1785,8 +1802,8 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(SliceArgs a) 
     float4 xf[SLOTS ? 8 : 1];                          // SLOTS: the lane's 32 activations as f32 (lanes j = 0, 1), split behind the barrier
     uint64_t slot_base = 0u;
     if constexpr (SLOTS) {
-        slot_base = a.slot_table[slot];
-        const float *xs = (a.x1 && slot >= a.x_split ? a.x1 : a.x) + 32u * G;
+        slot_base = slot_table_first[slot];            // (leading arguments, like the logits': a.slot_table, a.x, a.x1, a.x_split)
+        const float *xs = (x1_first && slot >= x_split_first ? x1_first : x_first) + 32u * G;
         float amax = 0.0f;
 #pragma unroll
         for (int s8 = 0; s8 < 8; ++s8) {
@@ -1801,7 +1818,6 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(SliceArgs a) 
         load_act_operand(ax, a.xh + 32u * G, a.xl + 32u * G, j);
     }
     // the table is first read behind the barrier that ends the selection: wave 0 selects, waves 8..15 build meanwhile
-    const bool selecting = !SLOTS && !is_shared && a.logits;
     // (and waves 1..7 write the sign words)
     if (selecting) { build_tables_rep<REP, 8, 0>(lds, strip, wave - 8u, lane); if (wave < 8u) build_sign_lut<kSliceLut>(reinterpret_cast<uint32_t *>(sign_lut), tid, 64u, 7u * 64u); }
     else { build_tables_rep<REP, 16, 0>(lds, strip, wave, lane); build_sign_lut<kSliceLut>(reinterpret_cast<uint32_t *>(sign_lut), tid); }
@@ -1831,11 +1847,7 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(SliceArgs a) 
         comb = a.logits ? 1.0f / (1.0f + expf(-a.logits[a.n_expert])) : a.scalar_in[0];
         __syncthreads();                               // table
     } else if (a.logits) {
-        if (wave == 0u) {
-            if (a.n_expert <= 512u) wave_select_topk<8>(a.logits, a.n_expert, a.top_k, sel);
-            else wave_select_topk<16>(a.logits, a.n_expert, a.top_k, sel);
-        }
-        __syncthreads();                               // selection and table
+        __syncthreads();                               // selection (by wave 0, at the kernel's head) and table
         expert = sel->ids[slot];
         comb = sel->w[slot];
         if (g == 0u && slot == 0u) {
@@ -2053,7 +2065,8 @@ template <int REP, int MIX> constexpr uint32_t batch_slice_table_bytes() {
 }
 // MIX 0: every matrix packed IQ2_XXS; 1: IQ3_S down matrices, dense shared expert; 2 / 3: IQ2_XS / IQ1_M streams, dense shared expert (see BatchSliceArgs)
 template <int NKC, int REP, int MIX>
-__global__ __launch_bounds__(kWaves * 64, 8) void batch_slice_kernel(BatchSliceArgs a) {
+__global__ __launch_bounds__(kWaves * 64, 8) void batch_slice_kernel(const uint2 *pass_list_first, const uint32_t *n_pass_first, uint32_t ntok_first, uint32_t top_k_first,
+                                                                     BatchSliceArgs a) {
     constexpr int NW = kWaves;
     constexpr int UPW = 16 * NKC / NW;
     constexpr int DU = (8 * NKC + NW - 1) / NW;
@@ -2069,16 +2082,18 @@ __global__ __launch_bounds__(kWaves * 64, 8) void batch_slice_kernel(BatchSliceA
     uint8_t *iq3_tab = reinterpret_cast<uint8_t *>(act_scale + 4);         // MIX: 4 KB, the IQ3_S grid as fp16
 
     const uint32_t tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63u, blk = lane >> 2, j = lane & 3u;      // (wave: in a scalar register)
-    const uint32_t H = a.hidden, F = a.ffn, HG = H / 32u, HB = H / 256u, FG = F / 32u, K = a.top_k;
-    const uint32_t g = blockIdx.x, v = blockIdx.y;
+    const uint32_t g = blockIdx.x, v = blockIdx.y, K = top_k_first;
     REDHIP_STAMP(0);
     // Three requests leave together, so that the workgroup waits for one round trip before it knows its weights' addresses: the number of
     // passes, this workgroup's entry of the pass list (read whether or not it turns out to be one: the index is clamped into the list) and
     // the codebook entries its lanes turn into the LDS tables. The tables are then written while the weights are on their way: loads
     // return in order, so a table seed requested behind the weights would not be usable before they have all arrived.
-    const uint32_t n_pairs = a.ntok * K;
-    const uint32_t n_pass = a.n_pass[0];
-    uint2 e = a.pass_list[v < n_pairs ? v : n_pairs - 1u];
+    // (the four leading kernel arguments repeat a.pass_list, a.n_pass, ntok_first, top_k_first: they can reach the wave in registers at its start,
+    // so these requests do not wait for the argument block to come from memory)
+    const uint32_t n_pairs = ntok_first * K;
+    const uint32_t n_pass = n_pass_first[0];
+    uint2 e = pass_list_first[v < n_pairs ? v : n_pairs - 1u];
+    const uint32_t H = a.hidden, F = a.ffn, HG = H / 32u, HB = H / 256u, FG = F / 32u;
     uint64_t seed_cb[2] = {0ull, 0ull};
     uint64_t seed_mag = 0ull;
     uint32_t seed_q3 = 0u;
@@ -2087,11 +2102,11 @@ __global__ __launch_bounds__(kWaves * 64, 8) void batch_slice_kernel(BatchSliceA
     if constexpr (MIX >= 2) codebook_seed<FMT>(tid, a.grid, seed_cb);
     else { seed_mag = table_seed<16>(wave, lane); seed_sign = redhip_sign_words.w[tid / (uint32_t)kBatchLut]; }
     if constexpr (MIX == 1) seed_q3 = iq3s_quads_seed(tid);
-    if (v >= n_pass + ((a.ntok + 1u) >> 1)) return;    // the grid covers the largest possible number of passes
+    if (v >= n_pass + ((ntok_first + 1u) >> 1)) return;    // the grid covers the largest possible number of passes
     const bool sh = v >= n_pass;
     if (sh) {                                          // the shared expert: tokens 2 s, 2 s + 1; k = top_k
-        const uint32_t t0 = 2u * (v - n_pass), t1 = t0 + 1u < a.ntok ? t0 + 1u : t0;
-        e.x = 0xffffu | ((t0 + 1u < a.ntok ? 2u : 1u) << 16);
+        const uint32_t t0 = 2u * (v - n_pass), t1 = t0 + 1u < ntok_first ? t0 + 1u : t0;
+        e.x = 0xffffu | ((t0 + 1u < ntok_first ? 2u : 1u) << 16);
         e.y = (t0 << 16) | (t1 << 24);
     } else if (((e.x >> 16) & 255u) < 2u) {
         e.y = (e.y & 0x00ff00ffu) * 0x101u;            // a lone token: its twin computes the same and is not stored
@@ -2276,7 +2291,7 @@ hipError_t launch_expert_slices(const void *experts, uint64_t stride, const void
             if (e != hipSuccess) return e;                                                                                              \
             attr = true;                                                                                                                \
         }                                                                                                                               \
-        REDHIP_LAUNCH((expert_slice_kernel<NKC, kSliceRep>), grid_dim, dim3(kWaves * 64), dyn, s, a);                                     \
+        REDHIP_LAUNCH((expert_slice_kernel<NKC, kSliceRep>), grid_dim, dim3(kWaves * 64), dyn, s, a.logits, a.n_expert, a.top_k, a.slot_table, a.x, a.x1, a.x_split, a); \
     } while (0)
     prof_set_stage(ST_FUSED_EXPERTS);
     switch (hidden / 512u) {
@@ -2317,7 +2332,7 @@ hipError_t launch_slot_slices(const uint64_t *slot_table, uint64_t shadow_off, c
             if (e != hipSuccess) return e;                                                                                              \
             attr = true;                                                                                                                \
         }                                                                                                                               \
-        REDHIP_LAUNCH((expert_slice_kernel<NKC, kSliceRep, true>), grid_dim, dim3(kWaves * 64), dyn, s, a);                               \
+        REDHIP_LAUNCH((expert_slice_kernel<NKC, kSliceRep, true>), grid_dim, dim3(kWaves * 64), dyn, s, a.logits, a.n_expert, a.top_k, a.slot_table, a.x, a.x1, a.x_split, a); \
     } while (0)
     prof_set_stage(ST_FUSED_EXPERTS);
     switch (hidden / 512u) {
@@ -2358,7 +2373,7 @@ hipError_t launch_batch_slices(const void *experts, uint64_t stride, const void 
             if (e != hipSuccess) return e;                                                                                              \
             attr = true;                                                                                                                \
         }                                                                                                                               \
-        REDHIP_LAUNCH((batch_slice_kernel<NKC, kBatchRep, MIX>), grid_dim, dim3(kWaves * 64), dyn, s, a);                                 \
+        REDHIP_LAUNCH((batch_slice_kernel<NKC, kBatchRep, MIX>), grid_dim, dim3(kWaves * 64), dyn, s, a.pass_list, a.n_pass, a.ntok, a.top_k, a); \
     } while (0)
 #define REDHIP_BSLICE(NKC)                                                                                                             \
     do {                                                                                                                               \
@@ -2669,11 +2684,14 @@ struct DownWordsArgs {
 // FMT: 0 word-packed IQ3_S, 1 stream-packed IQ2_XS, 2 stream-packed IQ1_M; CM (IQ3_S): the words stored column-sliced
 // (iq3s_sliced_index, d [ffn / 256][hidden]), the copy that the expert slices of small batches read
 template <int NW, int FMT, int CM = 0>
-__global__ __launch_bounds__(NW * 64) void down_combine_words_kernel(DownWordsArgs a) {
+__global__ __launch_bounds__(NW * 64) void down_combine_words_kernel(const uint32_t *ids_first, uint32_t top_k_first, DownWordsArgs a) {
     static_assert(CM == 0 || FMT == 0, "column-sliced copies exist of IQ3_S words only");
     __shared__ __attribute__((aligned(16))) uint8_t lds[FMT == 0 ? kIq3TableBytes : FMT == 1 ? 512u * 16u : 2048u * 16u];
     __shared__ float part[17 * 8];
-    const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
+    const uint32_t tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
+    // (ids_first, top_k_first repeat a.ids, a.top_k: leading arguments can reach a wave in registers at its start, so the request for
+    // the wave's expert id - the head of a chain of three dependent trips - leaves before the argument block has come from memory)
+    const uint32_t my_id = wave < top_k_first ? ids_first[blockIdx.y * top_k_first + wave] : 0u;
     const uint32_t F = a.ffn, FG = F / 32u, FB = F / 256u, n_slot = a.top_k + 1u;
     if (const uint32_t tok = blockIdx.y) {
         const uint64_t t = tok;
@@ -2694,7 +2712,7 @@ __global__ __launch_bounds__(NW * 64) void down_combine_words_kernel(DownWordsAr
     float sc[2] = {0.0f, 0.0f};
     const bool routed = wave < a.top_k;
     if (routed) {
-        const uint8_t *ex = a.experts + (uint64_t)guarded_id(a.ids[wave], a.id_limit, nullptr) * a.stride;
+        const uint8_t *ex = a.experts + (uint64_t)guarded_id(my_id, a.id_limit, nullptr) * a.stride;
         constexpr uint32_t kGroupBytes = FMT == 0 ? 16u : 8u;
         const uint16_t *ds = reinterpret_cast<const uint16_t *>(ex + (uint64_t)a.hidden * FG * kGroupBytes);      // [hidden][FB]
         const uint8_t *scs = ex + (uint64_t)a.hidden * FG * kGroupBytes + (uint64_t)a.hidden * FB * 2u;           // IQ2_XS: [hidden][FG]
@@ -2765,8 +2783,8 @@ hipError_t launch_down_combine_words(uint32_t down_type, const int8_t *grid, con
     const bool narrow = top_k + 1u <= 12u;
 #define REDHIP_DCW(FMT, CM)                                                                                          \
     do {                                                                                                             \
-        if (narrow) REDHIP_LAUNCH((down_combine_words_kernel<12, FMT, CM>), grid_dim, dim3(12 * 64), 0, s, a);       \
-        else REDHIP_LAUNCH((down_combine_words_kernel<kWaves, FMT, CM>), grid_dim, dim3(kWaves * 64), 0, s, a);      \
+        if (narrow) REDHIP_LAUNCH((down_combine_words_kernel<12, FMT, CM>), grid_dim, dim3(12 * 64), 0, s, a.ids, a.top_k, a);       \
+        else REDHIP_LAUNCH((down_combine_words_kernel<kWaves, FMT, CM>), grid_dim, dim3(kWaves * 64), 0, s, a.ids, a.top_k, a);      \
     } while (0)
     switch (down_type) {
         case T_IQ3_S: if (col_major) REDHIP_DCW(0, 1); else REDHIP_DCW(0, 0); break;
@@ -3468,7 +3486,7 @@ hipError_t launch_gateup_select(const void *experts, uint64_t stride, const void
             if (e != hipSuccess) return e;                                                                                              \
             attr = true;                                                                                                                \
         }                                                                                                                               \
-        REDHIP_LAUNCH((gateup_select_kernel<NKC, FMT>), grid_dim, dim3(kWaves * 64), dyn, s, a);                                          \
+        REDHIP_LAUNCH((gateup_select_kernel<NKC, FMT>), grid_dim, dim3(kWaves * 64), dyn, s, a.logits, a.n_expert, a.top_k, a);           \
     } while (0)
 #define REDHIP_GUS_FMT(NKC)                                                                                                            \
     do {                                                                                                                               \
