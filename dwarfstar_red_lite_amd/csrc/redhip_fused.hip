@@ -1767,8 +1767,8 @@ __device__ __forceinline__ void group_dot2_lut(uint2 q, const half4_t *ax, const
 
 constexpr int kSliceLut = 32;      // copies of the sign words in the one-token kernel: 16 KB, every lane of a half wave its own bank
 template <int NKC, int REP, bool SLOTS = false>        // hidden = 512 * NKC
-__global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(const float *logits_first, uint32_t n_expert_first, uint32_t top_k_first, const uint64_t *slot_table_first,
-                                                                   const float *x_first, const float *x1_first, uint32_t x_split_first, SliceArgs a) {
+__global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(const void *p0_first, uint32_t n_expert_first, uint32_t top_k_first, const void *p1_first,
+                                                                   const void *p2_first, uint32_t u0_first, uint32_t hidden_first, uint32_t ffn_first, SliceArgs a) {
     constexpr int NW = kWaves;
     constexpr int UPW = 16 * NKC / NW;                 // (row-quad, K-chunk) units of gate / up per wave
     constexpr int DU = (8 * NKC + NW - 1) / NW;        // units of 64 down rows per wave
@@ -1784,16 +1784,13 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(const float *
 
     const uint32_t tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
     const uint32_t g = blockIdx.x, slot = blockIdx.y;
-    // The three leading kernel arguments repeat a.logits, a.n_expert and a.top_k: leading scalar arguments can be handed to a wave in
-    // registers at its start, so the selecting wave's request for the logits does not wait for the argument block to come from memory.
+    // The leading kernel arguments repeat what the first requests of the kernel need - a.logits, a.xh, a.xl (SLOTS: a.slot_table, a.x,
+    // a.x1 and a.x_split), a.n_expert, a.top_k: leading scalar arguments can be handed to a wave in registers at its start, so these
+    // requests do not wait for the argument block to come from memory.
+    const float *logits_first = SLOTS ? nullptr : static_cast<const float *>(p0_first);
     const bool is_shared = slot >= top_k_first;
     const bool selecting = !SLOTS && !is_shared && logits_first;
     REDHIP_STAMP(0);
-    if (selecting && wave == 0u) {                     // first thing in the kernel: everything else of this wave comes behind the selection
-        if (n_expert_first <= 512u) wave_select_topk<8>(logits_first, n_expert_first, top_k_first, sel);
-        else wave_select_topk<16>(logits_first, n_expert_first, top_k_first, sel);
-    }
-    const uint32_t H = a.hidden, F = a.ffn, HG = H / 32u, HB = H / 256u, FG = F / 32u;
 
     // activation operand of the gate / up rows: independent of the routing, requested first
     const uint32_t kc = wave % NKC, q0 = wave / NKC;
@@ -1802,8 +1799,9 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(const float *
     float4 xf[SLOTS ? 8 : 1];                          // SLOTS: the lane's 32 activations as f32 (lanes j = 0, 1), split behind the barrier
     uint64_t slot_base = 0u;
     if constexpr (SLOTS) {
-        slot_base = slot_table_first[slot];            // (leading arguments, like the logits': a.slot_table, a.x, a.x1, a.x_split)
-        const float *xs = (x1_first && slot >= x_split_first ? x1_first : x_first) + 32u * G;
+        slot_base = static_cast<const uint64_t *>(p0_first)[slot];
+        const float *x_first = static_cast<const float *>(p1_first), *x1_first = static_cast<const float *>(p2_first);
+        const float *xs = (x1_first && slot >= u0_first ? x1_first : x_first) + 32u * G;
         float amax = 0.0f;
 #pragma unroll
         for (int s8 = 0; s8 < 8; ++s8) {
@@ -1815,8 +1813,19 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(const float *
         amax = wave_max(amax);                         // waves kc = 0 .. NKC - 1 cover the whole vector between them
         if (lane == 0u) reinterpret_cast<float *>(sel)[wave] = amax;
     } else {
-        load_act_operand(ax, a.xh + 32u * G, a.xl + 32u * G, j);
+        const _Float16 *xh_g = static_cast<const _Float16 *>(p1_first) + 32u * G, *xl_g = static_cast<const _Float16 *>(p2_first) + 32u * G;
+        // The selecting wave asks for the logits before anything else and for its activations only behind the selection (requested together,
+        // the logits were measured to arrive 0.5 us later: the wave then waits for all its loads); the barrier behind the selection
+        // waits for LDS only, so those late activations do not hold the workgroup up.
+        if (selecting && wave == 0u) {
+            if (n_expert_first <= 512u) wave_select_topk<8>(logits_first, n_expert_first, top_k_first, sel);
+            else wave_select_topk<16>(logits_first, n_expert_first, top_k_first, sel);
+        }
+        load_act_operand(ax, xh_g, xl_g, j);
     }
+    // (hidden and ffn are leading arguments too, and the branch below tests the leading copy of a.logits: the selecting wave reaches the
+    // barrier without having touched the argument block, whose fetch would otherwise sit between its selection and the barrier)
+    const uint32_t H = hidden_first, F = ffn_first, HG = H / 32u, HB = H / 256u, FG = F / 32u;
     // the table is first read behind the barrier that ends the selection: wave 0 selects, waves 8..15 build meanwhile
     // (and waves 1..7 write the sign words)
     if (selecting) { build_tables_rep<REP, 8, 0>(lds, strip, wave - 8u, lane); if (wave < 8u) build_sign_lut<kSliceLut>(reinterpret_cast<uint32_t *>(sign_lut), tid, 64u, 7u * 64u); }
@@ -1844,18 +1853,18 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(const float *
             }
         }
     } else if (is_shared) {
-        comb = a.logits ? 1.0f / (1.0f + expf(-a.logits[a.n_expert])) : a.scalar_in[0];
+        comb = logits_first ? 1.0f / (1.0f + expf(-logits_first[n_expert_first])) : a.scalar_in[0];
         __syncthreads();                               // table
-    } else if (a.logits) {
-        __syncthreads();                               // selection (by wave 0, at the kernel's head) and table
-        expert = sel->ids[slot];
+    } else if (logits_first) {
+        lds_barrier();                                 // selection (by wave 0, at the kernel's head) and table: both in LDS
+        expert = __builtin_amdgcn_readfirstlane(sel->ids[slot]);      // the same in every lane: the weights' base addresses stay scalar
         comb = sel->w[slot];
         if (g == 0u && slot == 0u) {
             if (tid < a.top_k) { a.ids_out[tid] = sel->ids[tid]; a.weights_out[tid] = sel->w[tid]; }
             if (tid == 0u) a.scalar_out[0] = sel->scalar;
         }
     } else {
-        expert = guarded_id(a.ids_in[slot], a.n_expert, a.status);
+        expert = __builtin_amdgcn_readfirstlane(guarded_id(a.ids_in[slot], a.n_expert, a.status));
         comb = a.weights_in[slot];
         __syncthreads();                               // table
     }
@@ -1864,27 +1873,26 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(const float *
     const uint8_t *ex = is_shared ? a.shared : a.experts + (uint64_t)expert * a.stride;
     const uint8_t *dn = is_shared ? a.shared_down_cm : a.down_cm + (uint64_t)expert * a.down_stride;
     if constexpr (SLOTS) {
-        ex = reinterpret_cast<const uint8_t *>(slot_base + a.shadow_off);
+        // (the builtin returns a signed int: each half goes through uint32_t, or a low half with bit 31 set would sign-extend over the high one)
+        const uint32_t base_lo = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)slot_base), base_hi = (uint32_t)__builtin_amdgcn_readfirstlane((uint32_t)(slot_base >> 32));
+        const uint64_t base = ((uint64_t)base_hi << 32) | base_lo;
+        ex = reinterpret_cast<const uint8_t *>(base + a.shadow_off);
         dn = ex + 2u * gate_bytes;
     }
-    const uint2 *gate_qs = reinterpret_cast<const uint2 *>(ex);
-    const uint16_t *gate_ds = reinterpret_cast<const uint16_t *>(ex + (uint64_t)F * HG * 8u);
-    const uint2 *up_qs = reinterpret_cast<const uint2 *>(ex + gate_bytes);
-    const uint16_t *up_ds = reinterpret_cast<const uint16_t *>(ex + gate_bytes + (uint64_t)F * HG * 8u);
-    const uint2 *down_qs = reinterpret_cast<const uint2 *>(dn) + (uint64_t)g * H;                                        // [FG][H]
-    const uint16_t *down_ds = reinterpret_cast<const uint16_t *>(dn + (uint64_t)FG * H * 8u) + (uint64_t)(g >> 3) * H;    // [F / 256][H]
+    // (bases the same in every lane, 32-bit byte offsets per lane: a matrix is far below 4 GB)
+    const uint8_t *down_qs = dn + (uint64_t)g * H * 8u;                                          // [FG][H] uint2
+    const uint8_t *down_ds = dn + (uint64_t)FG * H * 8u + (uint64_t)(g >> 3) * H * 2u;           // [F / 256][H] fp16
 
     // every weight this workgroup needs is requested here: gate / up units, then the down slice
     uint2 wq[UPW];
     uint32_t wd[UPW];
 #pragma unroll
     for (int u = 0; u < UPW; ++u) {
-        const uint32_t quad = q0 + (NW / NKC) * u;     // 0..7 gate, 8..15 up
+        const uint32_t quad = q0 + (NW / NKC) * u;     // 0..7 gate, 8..15 up (the same in every lane of the wave)
         const uint32_t r = 32u * g + 4u * (quad & 7u) + j;
-        const uint2 *qs = quad < 8u ? gate_qs : up_qs;
-        const uint16_t *ds = quad < 8u ? gate_ds : up_ds;
-        wq[u] = qs[(uint64_t)r * HG + G];
-        wd[u] = ds[(uint64_t)r * HB + (G >> 3)];
+        const uint8_t *mat = ex + (quad < 8u ? 0u : gate_bytes);
+        wq[u] = *reinterpret_cast<const uint2 *>(mat + (r * HG + G) * 8u);
+        wd[u] = *reinterpret_cast<const uint16_t *>(mat + (F * HG * 8u + (r * HB + (G >> 3)) * 2u));
     }
     uint2 dq[DU];
     uint32_t dd[DU];
@@ -1892,8 +1900,8 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(const float *
     for (int k = 0; k < DU; ++k) {
         const uint32_t unit = wave + NW * k;           // 64 output rows each
         const uint32_t row = 64u * (unit < 8u * NKC ? unit : 0u) + lane;
-        dq[k] = down_qs[row];
-        dd[k] = down_ds[row];
+        dq[k] = *reinterpret_cast<const uint2 *>(down_qs + row * 8u);
+        dd[k] = *reinterpret_cast<const uint16_t *>(down_ds + row * 2u);
     }
     float v[UPW];
     REDHIP_STAMP(2);                                   // every weight requested
@@ -2291,7 +2299,7 @@ hipError_t launch_expert_slices(const void *experts, uint64_t stride, const void
             if (e != hipSuccess) return e;                                                                                              \
             attr = true;                                                                                                                \
         }                                                                                                                               \
-        REDHIP_LAUNCH((expert_slice_kernel<NKC, kSliceRep>), grid_dim, dim3(kWaves * 64), dyn, s, a.logits, a.n_expert, a.top_k, a.slot_table, a.x, a.x1, a.x_split, a); \
+        REDHIP_LAUNCH((expert_slice_kernel<NKC, kSliceRep>), grid_dim, dim3(kWaves * 64), dyn, s, (const void *)a.logits, a.n_expert, a.top_k, (const void *)a.xh, (const void *)a.xl, 0u, a.hidden, a.ffn, a); \
     } while (0)
     prof_set_stage(ST_FUSED_EXPERTS);
     switch (hidden / 512u) {
@@ -2332,7 +2340,7 @@ hipError_t launch_slot_slices(const uint64_t *slot_table, uint64_t shadow_off, c
             if (e != hipSuccess) return e;                                                                                              \
             attr = true;                                                                                                                \
         }                                                                                                                               \
-        REDHIP_LAUNCH((expert_slice_kernel<NKC, kSliceRep, true>), grid_dim, dim3(kWaves * 64), dyn, s, a.logits, a.n_expert, a.top_k, a.slot_table, a.x, a.x1, a.x_split, a); \
+        REDHIP_LAUNCH((expert_slice_kernel<NKC, kSliceRep, true>), grid_dim, dim3(kWaves * 64), dyn, s, (const void *)a.slot_table, a.n_expert, a.top_k, (const void *)a.x, (const void *)a.x1, a.x_split, a.hidden, a.ffn, a); \
     } while (0)
     prof_set_stage(ST_FUSED_EXPERTS);
     switch (hidden / 512u) {
