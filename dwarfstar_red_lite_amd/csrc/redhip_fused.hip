@@ -503,26 +503,28 @@ __global__ __launch_bounds__(WPB * 64) void router_f32_kernel(const float *w, co
 // The same product for 2..8 tokens at once: a wave keeps its row in registers and walks the tokens, whose activation vectors (after the
 // optional residual + norm, done by wave t for token t) sit in LDS, so a row is read once per batch instead of once per token.
 template <int NV, int NWV>          // NWV waves (rows) per workgroup
-__global__ __launch_bounds__(NWV * 64) void router_f32_multi_kernel(const float *w, RouterArgs a, uint32_t ntok, GroupJob job) {
+__global__ __launch_bounds__(NWV * 64) void router_f32_multi_kernel(const float *w, const float *x_first, const float *gate_inp_first, const float *sh_dense_first, uint32_t hidden_first,
+                                                                  uint32_t n_expert_first, uint32_t ffn_first, uint32_t ntok, uint32_t n_blocks, RouterArgs a, GroupJob job) {
+    // (the leading arguments repeat a.x, a.gate_inp, a.sh_dense, a.hidden, a.n_expert, a.ffn; n_blocks = the workgroups that multiply rows:
+    // leading scalar arguments can reach a wave in registers at its start, so the requests for its row and the activations leave at once)
     extern __shared__ __attribute__((aligned(16))) float xs_all[];      // [ntok][hidden]
     __shared__ float s_amax[8];
-    const uint32_t n_blocks = gridDim.x - (job.ids ? 1u : 0u);
     if (blockIdx.x == n_blocks) {                        // the extra workgroup: pair sort of the caller's routing
         group_small_given(job, reinterpret_cast<uint32_t *>(xs_all));
         return;
     }
-    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63u, H = a.hidden;
+    const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63u, H = hidden_first;
     const uint32_t r = blockIdx.x * (uint32_t)NWV + wave;
-    const uint32_t n_rows = a.n_expert + 1u + (a.sh_dense ? 2u * a.ffn : 0u);
-    const float4 *wr = reinterpret_cast<const float4 *>(r < a.n_expert ? w + (uint64_t)r * H : r == a.n_expert ? a.gate_inp
-                                                        : a.sh_dense + (uint64_t)(r < n_rows ? r - a.n_expert - 1u : 0u) * H);
+    const uint32_t n_rows = n_expert_first + 1u + (sh_dense_first ? 2u * ffn_first : 0u);
+    const float4 *wr = reinterpret_cast<const float4 *>(r < n_expert_first ? w + (uint64_t)r * H : r == n_expert_first ? gate_inp_first
+                                                        : sh_dense_first + (uint64_t)(r < n_rows ? r - n_expert_first - 1u : 0u) * H);
     float4 wv[NV];
     if (r < n_rows) {
 #pragma unroll
         for (int k = 0; k < NV; ++k) wv[k] = wr[lane + 64u * k];
     }
     for (uint32_t tok = wave; tok < ntok; tok += (uint32_t)NWV) {
-        const float4 *xv = reinterpret_cast<const float4 *>(a.x + (uint64_t)tok * H);
+        const float4 *xv = reinterpret_cast<const float4 *>(x_first + (uint64_t)tok * H);
         float4 xq[NV];
 #pragma unroll
         for (int k = 0; k < NV; ++k) xq[k] = xv[lane + 64u * k];
@@ -705,7 +707,8 @@ hipError_t launch_router_gemv(uint32_t router_type, const void *w, const float *
             if (e != hipSuccess) return e;                                                                                                                  \
             attr = true;                                                                                                                                    \
         }                                                                                                                                                   \
-        REDHIP_LAUNCH((router_f32_multi_kernel<NV, 8>), mgrid, dim3(512), lds, s, wf, a, ntok, gj);                                                         \
+        REDHIP_LAUNCH((router_f32_multi_kernel<NV, 8>), mgrid, dim3(512), lds, s, wf, a.x, a.gate_inp, a.sh_dense, a.hidden, a.n_expert, a.ffn, ntok,       \
+                      mgrid.x - (gj.ids ? 1u : 0u), a, gj);                                                                                                 \
         if (with_job) *job_done = true;                                                                                                                     \
         return hipGetLastError();                                                                                                                           \
     } while (0)
