@@ -14,6 +14,8 @@ Prints one JSON line (metric: microseconds per token for one MoE layer; lower is
   prefill_sweep  chunks of 512 / 2048 tokens on the MFMA tile kernels: TFLOP/s against the fp16 matrix-core peak and the HBM cap
   stack          48 layers back to back for one token (residual + RMS-norm around every layer), us per token and GB/s
   yardsticks     this machine's own streaming-read rate and fp16 matrix-core rate, measured in the same run
+  topk_pool      the file-backed top-k pool (redmetal_topk_*) on a synthetic GGUF file: one token through a device slot table and a chunk of 512
+                 tokens, on raw slots and with the fast path's re-laid copies
 The headline is timed as HIP graph replays (what a decode loop issues); the eager figure is printed beside it.
 """
 import argparse
@@ -58,6 +60,7 @@ def parse():
     ap.add_argument("--no-prefill", action="store_true", help="skip the prefill-chunk sweep (512 / 2048 tokens) that the default run appends")
     ap.add_argument("--prefill-layers", type=int, default=8, help="resident layers of the chunk handles (a chunk reads about 0.4 GB of experts per layer)")
     ap.add_argument("--no-yardsticks", action="store_true", help="skip the streaming-read and matrix-core yardsticks")
+    ap.add_argument("--no-pool", action="store_true", help="skip the file-backed top-k pool entries that the default run appends")
     ap.add_argument("--prime", type=int, default=2000, help="untimed steps before the warm-up that bring the clocks up (reported as clock_priming_steps)")
     return ap.parse_args()
 
@@ -613,6 +616,126 @@ def main():
         if not micro_rel <= 1e-3:
             print("PARITY FAILURE in the GEMV microbench: rel L2 %.3g" % micro_rel, file=sys.stderr)
             sys.exit(1)
+
+    # ---- the file-backed top-k pool (redmetal_topk_*), the surface the reference's engine binds: ten experts for one token through a device
+    # slot table (encode_device_into) and a chunk of 512 tokens x top-10 (encode_batched), on raw GGUF slots and on a pool with the fast
+    # path's re-laid copies; 512 all-IQ2_XXS experts of the config shape read from a synthetic GGUF file ----
+    if args.layout == "iq2" and B == 1 and sweep and not args.no_pool:
+        import tempfile
+
+        from dwarfstar_red_lite_amd.gguf_writer import write_moe_gguf
+        from dwarfstar_red_lite_amd.moe import gguf_expert_layout
+        from dwarfstar_red_lite_amd.redmetal_topk import ExpertLayout, RedMetalTopKPool
+        PE, PK, PT = 512, cfg["top_k"], 512
+        pcfg = synth.layer_config(hidden=H, ffn=F, n_expert=PE, top_k=PK, layout="iq2")
+        play = synth.make_layer(4242, pcfg)
+        tmpd = tempfile.mkdtemp(prefix="redhip_pool_")
+        gguf = os.path.join(tmpd, "pool.gguf")
+        write_moe_gguf(gguf, pcfg, [play])
+        lays = []
+        for e in range(PE):
+            d = gguf_expert_layout(gguf, PE, 0, e)
+            lays.append(ExpertLayout(d["gate_offset"], d["gate_bytes"], d["up_offset"], d["up_bytes"], d["down_offset"], d["down_bytes"]))
+        payload = 2 * lays[0].gate_bytes + lays[0].down_bytes
+        up_ = lambda v, a_: (v + a_ - 1) // a_ * a_
+        zero_xs, zero_m = np.zeros(512 * 8, np.int8), np.zeros(2048 * 8, np.int8)      # (codebooks of formats this file does not use)
+        prng = np.random.default_rng(77)
+        NLIST = 32
+        lists = [prng.permutation(PE)[:PK] for _ in range(NLIST)]
+        pw = [(prng.random(PK).astype(np.float32) + 0.1) for _ in range(NLIST)]
+        px = torch.from_numpy(synth.normed_x(prng, max(NLIST, PT), H)).cuda()
+        logit = prng.standard_normal((PT, PE))
+        bids = np.argsort(-logit, axis=1)[:, :PK].astype(np.uint32)
+        bw = prng.random((PT, PK)).astype(np.float32) + 0.05
+        uid, start, ptok, pweight, tpair = orc.group_pairs(bids, bw, PE)
+        entry = {"experts": PE, "expert_bytes": int(payload), "note": "graph replay of 128 single-token calls over 32 different expert lists; batched: 16 calls "
+                 "queued back to back, device time per call; raw = the pool as the reference defines it (raw GGUF bytes per slot), fast = "
+                 "redhip_topk_pool_enable_fast_path with tile-major copies"}
+        for mode in ("raw", "fast"):
+            phys = up_(2 * up_(payload, 256) + payload, 4096) if mode == "fast" else up_(payload, 4096)
+            pool = RedMetalTopKPool(gguf, (PE + 2) * phys, payload, slots_per_slab=64, iq2_xs_grid=zero_xs, iq1_m_grid=zero_m)
+            if mode == "fast":
+                pool.enable_fast_path(16, H, F, tiles=True)
+            for e in range(PE):
+                pool.load(e, lays[e])
+            addr = [pool.addresses(e, lays[e])[0] for e in range(PE)]
+            tabs = [torch.from_numpy(np.array([addr[e] for e in l], np.uint64).view(np.int64)).cuda() for l in lists]
+            wdev = [torch.from_numpy(w_).cuda() for w_ in pw]
+            pouts = torch.zeros(NLIST, H, device="cuda")
+            gb = lays[0].gate_bytes
+
+            def run_lists(st):
+                for i in range(NLIST):
+                    pool.encode_device_into(st, tabs[i].data_ptr(), wdev[i].data_ptr(), PK, 16, H, F, gb, gb, px[i].data_ptr(), pouts[i].data_ptr())
+            with torch.cuda.stream(stream):
+                run_lists(stream.cuda_stream)
+                stream.synchronize()
+                want = sum(float(w_) * orc.expert_ffn(16, 16, play["gate"][e], play["up"][e], play["down"][e], H, F, px[0].cpu().numpy())
+                           for e, w_ in zip(lists[0], pw[0]))
+                prel = float(np.linalg.norm(pouts[0].cpu().numpy() - want) / np.linalg.norm(want))
+                if not prel <= 1e-3:
+                    print("PARITY FAILURE in the top-k pool (%s): rel L2 %.3g" % (mode, prel), file=sys.stderr)
+                    sys.exit(1)
+                pgraph = torch.cuda.CUDAGraph()
+                with torch.cuda.graph(pgraph, stream=stream):
+                    for _ in range(4):
+                        run_lists(stream.cuda_stream)
+                ts = []
+                for _ in range(10):
+                    stream.synchronize()
+                    t0_ = time.perf_counter()
+                    pgraph.replay()
+                    stream.synchronize()
+                    ts.append((time.perf_counter() - t0_) * 1e6 / (4 * NLIST))
+                one_us_ = sorted(ts[2:])[len(ts[2:]) // 2]
+                del pgraph
+                # the chunk
+                bout = torch.zeros(PT, H, device="cuda")
+                slots_b = [int(e) for e in uid]
+                lays_b = [lays[int(e)] for e in uid]
+
+                # (the C entry point itself, its host arrays made once: the Python bridge spends 0.2 ms per call turning 512 layout tuples into arrays)
+                ids_a = np.ascontiguousarray(slots_b, np.uint32)
+                gb_a, ub_a, db_a = (np.ascontiguousarray([getattr(l_, f_) for l_ in lays_b], np.uint64) for f_ in ("gate_bytes", "up_bytes", "down_bytes"))
+                pt_a, pw_a = np.ascontiguousarray(ptok, np.uint32), np.ascontiguousarray(pweight, np.float32)
+                es_a, tp_a = np.ascontiguousarray(start, np.uint32), np.ascontiguousarray(tpair, np.uint32)
+
+                def run_chunk():
+                    if not pool.lib.redmetal_topk_pool_encode_batched(pool.handle, stream.cuda_stream, ids_a.ctypes.data, gb_a.ctypes.data, ub_a.ctypes.data,
+                                                                      db_a.ctypes.data, ids_a.size, 16, H, F, 0, PT, PK, pt_a.size, pt_a.ctypes.data, pw_a.ctypes.data,
+                                                                      es_a.ctypes.data, tp_a.ctypes.data, px.data_ptr(), 0, bout.data_ptr(), 0):
+                        raise SystemExit("encode_batched failed: " + pool._last_error())
+                for _ in range(2):
+                    run_chunk()
+                stream.synchronize()
+                row = bout[5].cpu().numpy()
+                want_b = sum(float(w_) * orc.expert_ffn(16, 16, play["gate"][e], play["up"][e], play["down"][e], H, F, px[5].cpu().numpy())
+                             for e, w_ in zip(bids[5], bw[5]))
+                brel = float(np.linalg.norm(row - want_b) / np.linalg.norm(want_b))
+                if not brel <= 1e-3:
+                    print("PARITY FAILURE in the batched top-k pool (%s): rel L2 %.3g" % (mode, brel), file=sys.stderr)
+                    sys.exit(1)
+                nrep = 16 if mode == "fast" else 4
+                e0, e1 = torch.cuda.Event(enable_timing=True), torch.cuda.Event(enable_timing=True)
+                e0.record(stream)
+                for _ in range(nrep):
+                    run_chunk()
+                e1.record(stream)
+                stream.synchronize()
+                chunk_us = e0.elapsed_time(e1) * 1e3 / nrep
+                pool.release(slots_b)
+            entry[mode] = {"encode_device_into_us": round(one_us_, 2), "encode_device_into_gbps": round(PK * payload / one_us_ / 1e3, 1),
+                           "encode_batched_512_tokens_us": round(chunk_us, 1), "distinct_experts_in_chunk": int(len(uid)),
+                           "pool_bytes": int(pool.telemetry()["allocated_bytes"]), "rel_l2_vs_cpu_oracle": prel, "rel_l2_batched_row": brel}
+            pool.close()
+            del tabs, wdev, pouts, bout
+            torch.cuda.empty_cache()
+        try:
+            os.remove(gguf)
+            os.rmdir(tmpd)
+        except OSError:
+            pass
+        result["topk_pool"] = entry
 
     # ---- CPU baseline: the oracle on this host's cores, layer 0, same activations ----
     if not args.no_cpu:

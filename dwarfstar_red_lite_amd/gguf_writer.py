@@ -1,4 +1,4 @@
-"""Writes a GGUF v3 file holding the MoE tensors of synthetic layers (test infrastructure). Format as the reference parses it
+"""Writes a GGUF v3 file holding the MoE tensors of synthetic layers (for the tests and the benchmark of the file-backed pool). Format as the reference parses it
 (native/redlite_native_gguf.c:196-330): header, metadata key/values, tensor directory, aligned data."""
 import struct
 

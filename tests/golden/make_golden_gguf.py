@@ -1,5 +1,5 @@
 """Writes tests/golden/gguf_expert_layout.json. Runs ONLY in the build container, where the reference checkout exists: small GGUF
-files are written by tests/gguf_writer.py, parsed by the reference's own C (native/redlite_native_gguf.c, compiled unchanged into
+files are written by dwarfstar_red_lite_amd/gguf_writer.py, parsed by the reference's own C (native/redlite_native_gguf.c, compiled unchanged into
 oracle/_ref/libref.so by oracle/Makefile) through rl_native_build_expert_map (:199-397) and rl_native_expert_layout (:399-440), and
 what the reference answers is stored next to the recipe of each file and the file's CRC-32. The fixture is data: the reference's
 answers; nothing of its source text.
@@ -16,7 +16,7 @@ import zlib
 HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(os.path.dirname(HERE))
 sys.path[:0] = [ROOT, os.path.join(ROOT, "tests")]
-from gguf_writer import write_case      # noqa: E402
+from dwarfstar_red_lite_amd.gguf_writer import write_case      # noqa: E402
 
 
 class ExpertTensor(C.Structure):         # rl_expert_tensor, native/redlite_native_gguf.h:19-31

@@ -1,6 +1,6 @@
 """Writes tests/golden/reference_topk.json. Runs ONLY in the build container, where the reference checkout exists: small GGUF files
 with routed experts in the formats the reference's routed-expert CPU path accepts (IQ2_XS 17, IQ1_M 29, IQ3_S 21, and mixed gate/up
-vs down types) are written by tests/gguf_writer.py, and the reference's own C (native/redlite_native_reference.c:307-382
+vs down types) are written by dwarfstar_red_lite_amd/gguf_writer.py, and the reference's own C (native/redlite_native_reference.c:307-382
 rl_native_reference_topk, compiled unchanged into oracle/_ref/libref.so by oracle/Makefile) computes the weighted top-k expert
 FFN on them in double. The fixture is data: each file's recipe and CRC-32, the routing, and the reference's answers as the hex of
 their float64 bytes; nothing of its source text.
@@ -20,7 +20,7 @@ HERE = os.path.dirname(os.path.abspath(__file__))
 ROOT = os.path.dirname(os.path.dirname(HERE))
 sys.path[:0] = [ROOT, os.path.join(ROOT, "tests"), HERE]
 from make_golden_gguf import ExpertMap      # noqa: E402
-from gguf_writer import write_topk_case      # noqa: E402
+from dwarfstar_red_lite_amd.gguf_writer import write_topk_case      # noqa: E402
 
 # (gate/up type, down type): the reference runs the down rows on double activations (the step no other fixture reaches)
 CASES = [

@@ -5,7 +5,7 @@ import pytest
 
 from dwarfstar_red_lite_amd import synth
 from dwarfstar_red_lite_amd._lib import RedHipError
-from gguf_writer import write_moe_gguf
+from dwarfstar_red_lite_amd.gguf_writer import write_moe_gguf
 
 
 def small_cfg(layout):
@@ -123,7 +123,7 @@ LAYOUT_FIELDS = ("layer", "expert", "ggml_type", "down_type", "gate_offset", "ga
 def test_expert_layout_equals_the_reference_parser(tmp_path, golden_dir):
     import zlib
     from dwarfstar_red_lite_amd.moe import gguf_expert_layout
-    from gguf_writer import write_case
+    from dwarfstar_red_lite_amd.gguf_writer import write_case
     seen = 0
     for case in layout_cases(golden_dir):
         spec = case["spec"]
@@ -168,7 +168,7 @@ def test_layer_loaded_from_file_equals_cpu_path_on_the_reference_byte_ranges(tmp
     import oracle_lib as orc
     from dwarfstar_red_lite_amd.moe import ResidentMoe
     from gpu_common import REL_L2_TOL, rel_l2
-    from gguf_writer import write_case
+    from dwarfstar_red_lite_amd.gguf_writer import write_case
     from test_gpu_moe_layer import ids_match_up_to_ties
     for case in layout_cases(golden_dir)[:2]:
         spec = case["spec"]

@@ -11,7 +11,7 @@ import pytest
 import oracle_lib as orc
 from dwarfstar_red_lite_amd import synth
 from dwarfstar_red_lite_amd._lib import RedHipError
-from gguf_writer import write_moe_gguf
+from dwarfstar_red_lite_amd.gguf_writer import write_moe_gguf
 from gpu_common import REL_L2_TOL, rel_l2
 
 pytestmark = pytest.mark.gpu

@@ -224,7 +224,7 @@ def test_routed_topk_against_the_compiled_reference(golden_dir, tmp_path):
     import sys
     import zlib
     sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
-    from gguf_writer import write_topk_case
+    from dwarfstar_red_lite_amd.gguf_writer import write_topk_case
     grids = json.load(open(os.path.join(golden_dir, "iq_grids.json")))
     xs_grid, m_grid = (np.frombuffer(bytes.fromhex(grids[k]), np.int8) for k in ("iq2_xs", "iq1_m"))
     orc.set_codebooks(xs_grid, m_grid)
