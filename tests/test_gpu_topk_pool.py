@@ -401,3 +401,25 @@ def test_batched_chunk_of_512_tokens_on_the_tile_copies(tmp_path, grids):
         assert rel_l2(outs[0][t], outs[1][t]) <= REL_L2_TOL, t
     fast.pool.close()
     raw.pool.close()
+
+
+def test_fast_path_up_to_64_experts_per_call(tmp_path, grids):
+    """the copies serve calls of up to 64 experts (the partial vectors are sized for that); a call with more runs on the raw rows of the
+    same pool: both against the CPU path, through the device-driven form"""
+    c = Case(tmp_path, grids, "iq2", n_expert=72, fast=True)
+    H, F = c.cfg["hidden"], c.cfg["ffn"]
+    gb = c.layouts[0].gate_bytes
+    rng = np.random.default_rng(81)
+    x = synth.normed_x(rng, 1, H)[0]
+    x_dev = torch.from_numpy(x).cuda()
+    stream = torch.cuda.current_stream().cuda_stream
+    g_addr = [c.pool.addresses(c.slot_of[e], c.layouts[e])[0] for e in range(72)]
+    for top_k in (64, 66):
+        experts = rng.permutation(72)[:top_k]
+        w = rng.random(top_k).astype(np.float32) + 0.05
+        slots_dev = torch.from_numpy(np.array([g_addr[e] for e in experts], np.uint64).view(np.int64)).cuda()
+        w_dev = torch.from_numpy(w).cuda()
+        out = torch.zeros(H, device="cuda")
+        c.pool.encode_device_into(stream, slots_dev.data_ptr(), w_dev.data_ptr(), top_k, c.word, H, F, gb, gb, x_dev.data_ptr(), out.data_ptr())
+        assert rel_l2(out.cpu().numpy(), c.want(experts, w, x)) <= REL_L2_TOL, top_k
+    c.pool.close()
