@@ -1575,6 +1575,10 @@ struct SliceArgs {
     uint64_t shadow_off;
     const float *x, *x1;
     uint32_t x_split;
+    // MIX 1 (IQ2_XXS gate / up, IQ3_S down, dense shared expert): down_cm holds the column-sliced word-packed IQ3_S matrices; the shared
+    // expert comes as its gate . x and up . x products [2 ffn] f32 (left by the router launch) and the dense f32 copy [hidden][ffn] of its
+    // down matrix
+    const float *shared_gu, *shared_dense;
 };
 
 // Two tables, REP copies of every 16-byte entry side by side (entry i, copy c at (i * REP + c) * 16), lane l reads copy l % REP: with
@@ -1769,13 +1773,15 @@ __device__ __forceinline__ void group_dot2_lut(uint2 q, const half4_t *ax, const
 }
 
 constexpr int kSliceLut = 32;      // copies of the sign words in the one-token kernel: 16 KB, every lane of a half wave its own bank
-template <int NKC, int REP, bool SLOTS = false>        // hidden = 512 * NKC
+constexpr uint32_t kSliceSharedParts = 4u;      // workgroups per 32 columns of a dense shared expert (mixed layouts)
+template <int NKC, int REP, bool SLOTS = false, int MIX = 0>        // hidden = 512 * NKC; MIX as in batch_slice_kernel (0 or 1)
 __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(const void *p0_first, uint32_t n_expert_first, uint32_t top_k_first, const void *p1_first,
                                                                    const void *p2_first, uint32_t u0_first, uint32_t hidden_first, uint32_t ffn_first, SliceArgs a) {
     constexpr int NW = kWaves;
     constexpr int UPW = 16 * NKC / NW;                 // (row-quad, K-chunk) units of gate / up per wave
     constexpr int DU = (8 * NKC + NW - 1) / NW;        // units of 64 down rows per wave
     static_assert(UPW >= 1 && UPW * NW == 16 * NKC, "waves must tile the 16 row-quads x NKC chunks");
+    static_assert(MIX == 0 || (MIX == 1 && !SLOTS), "mixed layouts: the resident layer's IQ3_S down slices only");
     extern __shared__ __attribute__((aligned(16))) uint8_t dyn[];
     uint8_t *lds = dyn;                                                    // REP copies of the 4 KB magnitude table
     uint8_t *sign_lut = dyn + REP * kMagBytes;                             // kSliceLut copies of the 128 sign words (aligned to their size)
@@ -1784,9 +1790,12 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(const void *p
     _Float16 *act_hl = reinterpret_cast<_Float16 *>(part + NKC * 64);      // [2][32]: hi, lo halves of the 32 activations
     float *act_scale = reinterpret_cast<float *>(act_hl + 64);             // [4]
     SelectOut *sel = reinterpret_cast<SelectOut *>(act_scale + 4);
+    [[maybe_unused]] uint8_t *iq3_tab = reinterpret_cast<uint8_t *>(sel + 1);      // MIX 1: 4 KB, the IQ3_S grid as fp16
 
     const uint32_t tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
-    const uint32_t g = blockIdx.x, slot = blockIdx.y;
+    // MIX 1: the shared expert's dense slice is kSliceSharedParts workgroups (a quarter of the output rows each: 16 x hidden bytes of f32
+    // per row-quarter would otherwise be the longest-running workgroup); they come first in the grid, the routed slots behind them
+    const uint32_t g = blockIdx.x, slot = MIX == 1 ? (blockIdx.y < kSliceSharedParts ? top_k_first : blockIdx.y - kSliceSharedParts) : blockIdx.y;
     // The leading kernel arguments repeat what the first requests of the kernel need - a.logits, a.xh, a.xl (SLOTS: a.slot_table, a.x,
     // a.x1 and a.x_split), a.n_expert, a.top_k: leading scalar arguments can be handed to a wave in registers at its start, so these
     // requests do not wait for the argument block to come from memory.
@@ -1794,6 +1803,43 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(const void *p
     const bool is_shared = slot >= top_k_first;
     const bool selecting = !SLOTS && !is_shared && logits_first;
     REDHIP_STAMP(0);
+    // (hidden and ffn are leading arguments too, and the branch below tests the leading copy of a.logits: the selecting wave reaches the
+    // barrier without having touched the argument block, whose fetch would otherwise sit between its selection and the barrier)
+    const uint32_t H = hidden_first, F = ffn_first, HG = H / 32u, HB = H / 256u, FG = F / 32u;
+    if constexpr (MIX == 1) {
+        if (is_shared) {       // the shared expert's slice from dense f32 data: SwiGLU of the 32 columns, then their part of every output row
+            if (tid < 32u) {
+                const float *gu = a.shared_gu + 32u * g + tid;
+                const float gv = gu[0], uv = gu[F];
+                part[tid] = (gv / (1.0f + expf(-gv))) * uv;
+            }
+            const float gate = logits_first ? 1.0f / (1.0f + expf(-logits_first[n_expert_first])) : a.scalar_in[0];
+            __syncthreads();
+            // eight lanes per output row, each lane four of the 32 columns: a wave-wide load reads the 128-byte slices of eight rows whole
+            const uint32_t sub = tid & 7u;
+            const float4 av = *reinterpret_cast<const float4 *>(part + 4u * sub);
+            constexpr uint32_t kRows = (uint32_t)NW * 8u;      // rows per round of the workgroup
+            float *out = a.partial + ((uint64_t)slot * FG + g) * H;
+            const uint32_t h_end = (blockIdx.y + 1u) * (H / kSliceSharedParts);      // (hidden is a multiple of 512)
+            for (uint32_t h0 = blockIdx.y * (H / kSliceSharedParts) + (tid >> 3); h0 < h_end; h0 += 4u * kRows) {      // four rounds' loads in flight
+                float4 w4[4];
+#pragma unroll
+                for (uint32_t i = 0; i < 4u; ++i) {
+                    const uint32_t h = h0 + i * kRows;
+                    w4[i] = *reinterpret_cast<const float4 *>(a.shared_dense + (uint64_t)(h < h_end ? h : h0) * F + 32u * g + 4u * sub);
+                }
+#pragma unroll
+                for (uint32_t i = 0; i < 4u; ++i) {
+                    const uint32_t h = h0 + i * kRows;
+                    float acc = fmaf(w4[i].w, av.w, fmaf(w4[i].z, av.z, fmaf(w4[i].y, av.y, w4[i].x * av.x)));
+#pragma unroll
+                    for (int o = 1; o < 8; o <<= 1) acc += __shfl_xor(acc, o, 64);
+                    if (h < h_end && sub == 0u) out[h] = acc * gate;
+                }
+            }
+            return;
+        }
+    }
 
     // activation operand of the gate / up rows: independent of the routing, requested first
     const uint32_t kc = wave % NKC, q0 = wave / NKC;
@@ -1826,14 +1872,14 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(const void *p
         }
         load_act_operand(ax, xh_g, xl_g, j);
     }
-    // (hidden and ffn are leading arguments too, and the branch below tests the leading copy of a.logits: the selecting wave reaches the
-    // barrier without having touched the argument block, whose fetch would otherwise sit between its selection and the barrier)
-    const uint32_t H = hidden_first, F = ffn_first, HG = H / 32u, HB = H / 256u, FG = F / 32u;
+    [[maybe_unused]] uint32_t seed_q3 = 0u;
+    if constexpr (MIX == 1) seed_q3 = iq3s_quads_seed(tid);
     // the table is first read behind the barrier that ends the selection: wave 0 selects, waves 8..15 build meanwhile
     // (and waves 1..7 write the sign words)
     if (selecting) { build_tables_rep<REP, 8, 0>(lds, strip, wave - 8u, lane); if (wave < 8u) build_sign_lut<kSliceLut>(reinterpret_cast<uint32_t *>(sign_lut), tid, 64u, 7u * 64u); }
     else { build_tables_rep<REP, 16, 0>(lds, strip, wave, lane); build_sign_lut<kSliceLut>(reinterpret_cast<uint32_t *>(sign_lut), tid); }
     const LaneTables lt = lane_tables<REP, kSliceLut>(lds, sign_lut, lane);
+    if constexpr (MIX == 1) build_iq3s_quads_from(iq3_tab, tid, seed_q3);
 
     uint32_t expert = 0u;
     float comb;                                        // the slot's weight in the layer's output
@@ -1883,8 +1929,9 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(const void *p
         dn = ex + 2u * gate_bytes;
     }
     // (bases the same in every lane, 32-bit byte offsets per lane: a matrix is far below 4 GB)
-    const uint8_t *down_qs = dn + (uint64_t)g * H * 8u;                                          // [FG][H] uint2
-    const uint8_t *down_ds = dn + (uint64_t)FG * H * 8u + (uint64_t)(g >> 3) * H * 2u;           // [F / 256][H] fp16
+    using DownGroup = typename std::conditional<MIX == 1, uint4, uint2>::type;      // one row's 32 weights of the slice (IQ3_S: four words)
+    const uint8_t *down_qs = dn + (MIX == 1 ? 0u : (uint64_t)g * H * 8u);                        // [FG][H] uint2; IQ3_S: blocks of eight rows per group
+    const uint8_t *down_ds = dn + (uint64_t)FG * H * sizeof(DownGroup) + (uint64_t)(g >> 3) * H * 2u;      // [F / 256][H] fp16
 
     // every weight this workgroup needs is requested here: gate / up units, then the down slice
     uint2 wq[UPW];
@@ -1897,13 +1944,13 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(const void *p
         wq[u] = *reinterpret_cast<const uint2 *>(mat + (r * HG + G) * 8u);
         wd[u] = *reinterpret_cast<const uint16_t *>(mat + (F * HG * 8u + (r * HB + (G >> 3)) * 2u));
     }
-    uint2 dq[DU];
+    DownGroup dq[DU];
     uint32_t dd[DU];
 #pragma unroll
     for (int k = 0; k < DU; ++k) {
         const uint32_t unit = wave + NW * k;           // 64 output rows each
         const uint32_t row = 64u * (unit < 8u * NKC ? unit : 0u) + lane;
-        dq[k] = *reinterpret_cast<const uint2 *>(down_qs + row * 8u);
+        dq[k] = *reinterpret_cast<const DownGroup *>(down_qs + (MIX == 1 ? (uint32_t)iq3s_sliced_index(g, row, FG, H) : row) * (uint32_t)sizeof(DownGroup));
         dd[k] = *reinterpret_cast<const uint16_t *>(down_ds + row * 2u);
     }
     float v[UPW];
@@ -1949,12 +1996,17 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(const void *p
             ad[s8] = t;
         }
     }
-    const float post = act_scale[0] * comb * 0.125f;     // the activations' pre-scale, the slot's weight, d / 8
+    const float post = act_scale[0] * comb * (MIX == 1 ? 1.0f : 0.125f);     // the activations' pre-scale, the slot's weight, d / 8 (an IQ3_S weight is d (1 + 2 nibble) grid byte: no 1 / 8)
     float *out = a.partial + ((uint64_t)slot * FG + g) * H;
 #pragma unroll
     for (int k = 0; k < DU; ++k) {
         const uint32_t unit = wave + NW * k;
-        if (unit < 8u * NKC) out[64u * unit + lane] = group_dot_lut<REP, kSliceLut>(dq[k], ad, lt) * scale_to_f32(dd[k]) * post;
+        if (unit < 8u * NKC) {
+            float dot;
+            if constexpr (MIX == 1) { float other; iq3s_group_dot(dq[k], ad, iq3_tab, dot, other); }
+            else dot = group_dot_lut<REP, kSliceLut>(dq[k], ad, lt);
+            out[64u * unit + lane] = dot * scale_to_f32(dd[k]) * post;
+        }
     }
     REDHIP_STAMP(7);                                   // down slice of wave 0 multiplied, stores issued
 }
@@ -2280,29 +2332,38 @@ __global__ __launch_bounds__(kWaves * 64, 8) void batch_slice_kernel(const uint2
 }
 
 constexpr int kSliceRep = 16;
-inline size_t slice_lds_bytes(int nkc, int rep) { return (size_t)(rep + 1) * kMagBytes + 128u * 4u * (size_t)kSliceLut + (size_t)nkc * 64u * 4u + 128u + 16u + sizeof(SelectOut); }
+inline size_t slice_lds_bytes(int nkc, int rep, bool mix = false) {
+    return (size_t)(rep + 1) * kMagBytes + 128u * 4u * (size_t)kSliceLut + (size_t)nkc * 64u * 4u + 128u + 16u + sizeof(SelectOut) + (mix ? kIq3TableBytes : 0u);
+}
 
 hipError_t launch_expert_slices(const void *experts, uint64_t stride, const void *down_cm, uint64_t down_stride, const void *shared, const void *shared_down_cm,
                                 const float *logits, const uint32_t *ids_in, const float *weights_in, const float *scalar_in, uint32_t *ids_out,
                                 float *weights_out, float *scalar_out, const void *xh, const void *xl, const int *xexp, float *partial, float *out,
-                                uint32_t hidden, uint32_t ffn, uint32_t n_expert, uint32_t top_k, hipStream_t s) {
+                                uint32_t hidden, uint32_t ffn, uint32_t n_expert, uint32_t top_k, hipStream_t s, const float *shared_gu, const float *shared_dense) {
     if (!fused_iq2_supported(hidden, ffn) || top_k + 1u > (uint32_t)kWaves || n_expert > 1024u || hidden % 32u) return hipErrorInvalidValue;
     if (!logits && (!ids_in || !weights_in || !scalar_in)) return hipErrorInvalidValue;
+    const bool mix = shared_gu != nullptr;             // IQ3_S down slices (word-packed, column-sliced) and the dense shared expert
+    if (mix && (!shared_dense || ffn % 256u)) return hipErrorInvalidValue;
     const SliceArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(down_cm), down_stride, static_cast<const uint8_t *>(shared),
                       static_cast<const uint8_t *>(shared_down_cm), logits, ids_in, weights_in, scalar_in, ids_out, weights_out, scalar_out,
                       static_cast<const _Float16 *>(xh), static_cast<const _Float16 *>(xl), xexp, partial, hidden, ffn, n_expert, top_k, route_guard().status,
-                      nullptr, 0u, nullptr, nullptr, 0u};
-    const dim3 grid_dim(ffn / 32u, top_k + 1u);
-#define REDHIP_SLICE(NKC)                                                                                                              \
+                      nullptr, 0u, nullptr, nullptr, 0u, shared_gu, shared_dense};
+    const dim3 grid_dim(ffn / 32u, top_k + (mix ? kSliceSharedParts : 1u));
+#define REDHIP_SLICE_MIX(NKC, MIX)                                                                                                     \
     do {                                                                                                                               \
         static bool attr = false;                                                                                                       \
-        const size_t dyn = slice_lds_bytes(NKC, kSliceRep);                                                                             \
+        const size_t dyn = slice_lds_bytes(NKC, kSliceRep, MIX == 1);                                                                   \
         if (!attr) {                                                                                                                    \
-            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(expert_slice_kernel<NKC, kSliceRep>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn); \
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(expert_slice_kernel<NKC, kSliceRep, false, MIX>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn); \
             if (e != hipSuccess) return e;                                                                                              \
             attr = true;                                                                                                                \
         }                                                                                                                               \
-        REDHIP_LAUNCH((expert_slice_kernel<NKC, kSliceRep>), grid_dim, dim3(kWaves * 64), dyn, s, (const void *)a.logits, a.n_expert, a.top_k, (const void *)a.xh, (const void *)a.xl, 0u, a.hidden, a.ffn, a); \
+        REDHIP_LAUNCH((expert_slice_kernel<NKC, kSliceRep, false, MIX>), grid_dim, dim3(kWaves * 64), dyn, s, (const void *)a.logits, a.n_expert, a.top_k, (const void *)a.xh, (const void *)a.xl, 0u, a.hidden, a.ffn, a); \
+    } while (0)
+#define REDHIP_SLICE(NKC)                                                                                                              \
+    do {                                                                                                                               \
+        if (mix) REDHIP_SLICE_MIX(NKC, 1);                                                                                              \
+        else REDHIP_SLICE_MIX(NKC, 0);                                                                                                  \
     } while (0)
     prof_set_stage(ST_FUSED_EXPERTS);
     switch (hidden / 512u) {
@@ -2313,6 +2374,7 @@ hipError_t launch_expert_slices(const void *experts, uint64_t stride, const void
         default: return hipErrorInvalidValue;
     }
 #undef REDHIP_SLICE
+#undef REDHIP_SLICE_MIX
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     prof_set_stage(ST_SLICE_SUM);

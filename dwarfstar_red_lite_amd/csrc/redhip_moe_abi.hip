@@ -372,6 +372,16 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
         prof_set_stage(ST_OTHER);
         return 1;
     }
+    if (m->sliced_words() && ntok == 1u && m->shared_gu_ready && m->layers[layer].dense_down) {
+        // one token on IQ2_XXS gate / up with IQ3_S down: the same slices, the down matrices from their column-sliced words, the shared
+        // expert from its products (m->act, left by the router launch) and the dense copy of its down matrix
+        const Layer &L = m->layers[layer];
+        HIP_OK(launch_expert_slices(L.packed, m->packed_stride, L.down_cm, m->down_cm_stride(), nullptr, nullptr, select_here ? m->logits : nullptr,
+                                    ids, weights, m->scalar, m->ids, m->weights, m->scalar, m->xh, m->xl, m->xexp, m->partial, out, c.hidden, c.ffn, c.n_expert,
+                                    c.top_k, s, m->act, L.dense_down), "expert slice launch");
+        prof_set_stage(ST_OTHER);
+        return 1;
+    }
     if (m->packed_gu()) {    // xh / xl / scalar come from the router kernel or the prep kernel
         const Layer &L = m->layers[layer];
         prof_set_stage(ST_GATEUP);
