@@ -1579,6 +1579,9 @@ struct SliceArgs {
     // expert comes as its gate . x and up . x products [2 ffn] f32 (left by the router launch) and the dense f32 copy [hidden][ffn] of its
     // down matrix
     const float *shared_gu, *shared_dense;
+    // MIX 2 / 3: `experts` holds the row-major IQ2_XS / IQ1_M streams of gate | up, down_cm the column-sliced streams of the down matrices,
+    // grid the caller's codebook; the shared expert as for MIX 1
+    const int8_t *grid;
 };
 
 // Two tables, REP copies of every 16-byte entry side by side (entry i, copy c at (i * REP + c) * 16), lane l reads copy l % REP: with
@@ -1773,29 +1776,34 @@ __device__ __forceinline__ void group_dot2_lut(uint2 q, const half4_t *ax, const
 }
 
 constexpr int kSliceLut = 32;      // copies of the sign words in the one-token kernel: 16 KB, every lane of a half wave its own bank
+// LDS bytes of the decode tables at the head of the one-token kernel's dynamic LDS
+template <int REP, int MIX> constexpr uint32_t slice_table_bytes() {
+    return MIX == 2 ? 512u * 16u : MIX == 3 ? 2048u * 16u : (uint32_t)(REP + 1) * kMagBytes + 128u * 4u * (uint32_t)kSliceLut;
+}
 constexpr uint32_t kSliceSharedParts = 4u;      // workgroups per 32 columns of a dense shared expert (mixed layouts)
-template <int NKC, int REP, bool SLOTS = false, int MIX = 0>        // hidden = 512 * NKC; MIX as in batch_slice_kernel (0 or 1)
+template <int NKC, int REP, bool SLOTS = false, int MIX = 0>        // hidden = 512 * NKC; MIX as in batch_slice_kernel
 __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(const void *p0_first, uint32_t n_expert_first, uint32_t top_k_first, const void *p1_first,
                                                                    const void *p2_first, uint32_t u0_first, uint32_t hidden_first, uint32_t ffn_first, SliceArgs a) {
     constexpr int NW = kWaves;
     constexpr int UPW = 16 * NKC / NW;                 // (row-quad, K-chunk) units of gate / up per wave
     constexpr int DU = (8 * NKC + NW - 1) / NW;        // units of 64 down rows per wave
     static_assert(UPW >= 1 && UPW * NW == 16 * NKC, "waves must tile the 16 row-quads x NKC chunks");
-    static_assert(MIX == 0 || (MIX == 1 && !SLOTS), "mixed layouts: the resident layer's IQ3_S down slices only");
+    static_assert(MIX == 0 || !SLOTS, "mixed layouts: resident layers only");
+    constexpr int FMT = MIX >= 2 ? MIX - 1 : 0;            // format of the routed matrices as group_dot_fmt2 numbers them
     extern __shared__ __attribute__((aligned(16))) uint8_t dyn[];
-    uint8_t *lds = dyn;                                                    // REP copies of the 4 KB magnitude table
+    uint8_t *lds = dyn;                                                    // REP copies of the 4 KB magnitude table (MIX 2 / 3: the fp16 codebook, once)
     uint8_t *sign_lut = dyn + REP * kMagBytes;                             // kSliceLut copies of the 128 sign words (aligned to their size)
     uint8_t *strip = sign_lut + 128u * 4u * kSliceLut;                     // 4 KB: the magnitude table once, as its builders make it
-    float *part = reinterpret_cast<float *>(strip + kMagBytes);            // [NKC][64]
+    float *part = reinterpret_cast<float *>(dyn + slice_table_bytes<REP, MIX>());      // [NKC][64]
     _Float16 *act_hl = reinterpret_cast<_Float16 *>(part + NKC * 64);      // [2][32]: hi, lo halves of the 32 activations
     float *act_scale = reinterpret_cast<float *>(act_hl + 64);             // [4]
     SelectOut *sel = reinterpret_cast<SelectOut *>(act_scale + 4);
     [[maybe_unused]] uint8_t *iq3_tab = reinterpret_cast<uint8_t *>(sel + 1);      // MIX 1: 4 KB, the IQ3_S grid as fp16
 
     const uint32_t tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
-    // MIX 1: the shared expert's dense slice is kSliceSharedParts workgroups (a quarter of the output rows each: 16 x hidden bytes of f32
+    // Mixed layouts: the shared expert's dense slice is kSliceSharedParts workgroups (a quarter of the output rows each: 16 x hidden bytes of f32
     // per row-quarter would otherwise be the longest-running workgroup); they come first in the grid, the routed slots behind them
-    const uint32_t g = blockIdx.x, slot = MIX == 1 ? (blockIdx.y < kSliceSharedParts ? top_k_first : blockIdx.y - kSliceSharedParts) : blockIdx.y;
+    const uint32_t g = blockIdx.x, slot = MIX != 0 ? (blockIdx.y < kSliceSharedParts ? top_k_first : blockIdx.y - kSliceSharedParts) : blockIdx.y;
     // The leading kernel arguments repeat what the first requests of the kernel need - a.logits, a.xh, a.xl (SLOTS: a.slot_table, a.x,
     // a.x1 and a.x_split), a.n_expert, a.top_k: leading scalar arguments can be handed to a wave in registers at its start, so these
     // requests do not wait for the argument block to come from memory.
@@ -1806,7 +1814,7 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(const void *p
     // (hidden and ffn are leading arguments too, and the branch below tests the leading copy of a.logits: the selecting wave reaches the
     // barrier without having touched the argument block, whose fetch would otherwise sit between its selection and the barrier)
     const uint32_t H = hidden_first, F = ffn_first, HG = H / 32u, HB = H / 256u, FG = F / 32u;
-    if constexpr (MIX == 1) {
+    if constexpr (MIX != 0) {
         if (is_shared) {       // the shared expert's slice from dense f32 data: SwiGLU of the 32 columns, then their part of every output row
             if (tid < 32u) {
                 const float *gu = a.shared_gu + 32u * g + tid;
@@ -1876,9 +1884,15 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(const void *p
     if constexpr (MIX == 1) seed_q3 = iq3s_quads_seed(tid);
     // the table is first read behind the barrier that ends the selection: wave 0 selects, waves 8..15 build meanwhile
     // (and waves 1..7 write the sign words)
-    if (selecting) { build_tables_rep<REP, 8, 0>(lds, strip, wave - 8u, lane); if (wave < 8u) build_sign_lut<kSliceLut>(reinterpret_cast<uint32_t *>(sign_lut), tid, 64u, 7u * 64u); }
-    else { build_tables_rep<REP, 16, 0>(lds, strip, wave, lane); build_sign_lut<kSliceLut>(reinterpret_cast<uint32_t *>(sign_lut), tid); }
-    const LaneTables lt = lane_tables<REP, kSliceLut>(lds, sign_lut, lane);
+    [[maybe_unused]] LaneTables lt{};
+    if constexpr (MIX >= 2) {                          // the codebook as fp16, by the waves that do not select
+        if (selecting) build_codebook_table<FMT>(lds, tid, a.grid);
+        else build_codebook_table<FMT>(lds, tid, a.grid, 0u, (uint32_t)NW * 64u);
+    } else {
+        if (selecting) { build_tables_rep<REP, 8, 0>(lds, strip, wave - 8u, lane); if (wave < 8u) build_sign_lut<kSliceLut>(reinterpret_cast<uint32_t *>(sign_lut), tid, 64u, 7u * 64u); }
+        else { build_tables_rep<REP, 16, 0>(lds, strip, wave, lane); build_sign_lut<kSliceLut>(reinterpret_cast<uint32_t *>(sign_lut), tid); }
+        lt = lane_tables<REP, kSliceLut>(lds, sign_lut, lane);
+    }
     if constexpr (MIX == 1) build_iq3s_quads_from(iq3_tab, tid, seed_q3);
 
     uint32_t expert = 0u;
@@ -1918,7 +1932,8 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(const void *p
         __syncthreads();                               // table
     }
     REDHIP_STAMP(1);                                   // selection (or the caller's routing) and tables are here
-    const uint64_t gate_bytes = (uint64_t)F * HG * 8u + (uint64_t)F * HB * 2u;
+    const uint64_t gate_sc = (uint64_t)F * HG * 8u + (uint64_t)F * HB * 2u;       // IQ2_XS: the scale bytes [row][group] behind qs and ds
+    const uint64_t gate_bytes = gate_sc + (MIX == 2 ? (uint64_t)F * HG : 0u);
     const uint8_t *ex = is_shared ? a.shared : a.experts + (uint64_t)expert * a.stride;
     const uint8_t *dn = is_shared ? a.shared_down_cm : a.down_cm + (uint64_t)expert * a.down_stride;
     if constexpr (SLOTS) {
@@ -1932,10 +1947,11 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(const void *p
     using DownGroup = typename std::conditional<MIX == 1, uint4, uint2>::type;      // one row's 32 weights of the slice (IQ3_S: four words)
     const uint8_t *down_qs = dn + (MIX == 1 ? 0u : (uint64_t)g * H * 8u);                        // [FG][H] uint2; IQ3_S: blocks of eight rows per group
     const uint8_t *down_ds = dn + (uint64_t)FG * H * sizeof(DownGroup) + (uint64_t)(g >> 3) * H * 2u;      // [F / 256][H] fp16
+    [[maybe_unused]] const uint8_t *down_sc = dn + ((uint64_t)FG * H * 8u + (uint64_t)(FG >> 3) * H * 2u + (uint64_t)g * H);      // MIX 2: [FG][H] scale bytes
 
     // every weight this workgroup needs is requested here: gate / up units, then the down slice
     uint2 wq[UPW];
-    uint32_t wd[UPW];
+    uint32_t wd[UPW];                                  // block scale d (fp16 bits); IQ2_XS: the group's scale byte above it
 #pragma unroll
     for (int u = 0; u < UPW; ++u) {
         const uint32_t quad = q0 + (NW / NKC) * u;     // 0..7 gate, 8..15 up (the same in every lane of the wave)
@@ -1943,6 +1959,7 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(const void *p
         const uint8_t *mat = ex + (quad < 8u ? 0u : gate_bytes);
         wq[u] = *reinterpret_cast<const uint2 *>(mat + (r * HG + G) * 8u);
         wd[u] = *reinterpret_cast<const uint16_t *>(mat + (F * HG * 8u + (r * HB + (G >> 3)) * 2u));
+        if constexpr (MIX == 2) wd[u] |= (uint32_t)mat[(uint32_t)gate_sc + r * HG + G] << 16;
     }
     DownGroup dq[DU];
     uint32_t dd[DU];
@@ -1952,12 +1969,14 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(const void *p
         const uint32_t row = 64u * (unit < 8u * NKC ? unit : 0u) + lane;
         dq[k] = *reinterpret_cast<const DownGroup *>(down_qs + (MIX == 1 ? (uint32_t)iq3s_sliced_index(g, row, FG, H) : row) * (uint32_t)sizeof(DownGroup));
         dd[k] = *reinterpret_cast<const uint16_t *>(down_ds + row * 2u);
+        if constexpr (MIX == 2) dd[k] |= (uint32_t)down_sc[row] << 16;
     }
     float v[UPW];
     REDHIP_STAMP(2);                                   // every weight requested
 #pragma unroll
     for (int u = 0; u < UPW; ++u) {
-        v[u] = group_dot_lut<REP, kSliceLut>(wq[u], ax, lt) * scale_to_f32(wd[u]);
+        if constexpr (MIX >= 2) { float other; group_dot_fmt2<FMT>(wq[u], wd[u] >> 16, ax, lds, v[u], other); v[u] *= scale_to_f32(wd[u]); }
+        else v[u] = group_dot_lut<REP, kSliceLut>(wq[u], ax, lt) * scale_to_f32(wd[u]);
         if (u == 0) REDHIP_STAMP(3);                   // the first unit's weights arrived and are multiplied
     }
     const float tot = quad_column_reduce<UPW>(v, lane);
@@ -1972,7 +1991,7 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(const void *p
         float gsum = 0.0f, usum = 0.0f;
 #pragma unroll
         for (int c = 0; c < NKC; ++c) { gsum += part[c * 64 + tid]; usum += part[c * 64 + 32 + tid]; }
-        const float xs = 0.125f * exp2i(SLOTS ? x_exp : a.xexp[0]);      // d / 8 and the pre-scale of x
+        const float xs = (MIX == 3 ? 1.0f : 0.125f) * exp2i(SLOTS ? x_exp : a.xexp[0]);      // d / 8 (an IQ1_M weight is d (2 s + 1) (entry +- 1/8): none) and the pre-scale of x
         gsum *= xs;
         usum *= xs;
         const float act = (gsum / (1.0f + expf(-gsum))) * usum;
@@ -1996,14 +2015,16 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(const void *p
             ad[s8] = t;
         }
     }
-    const float post = act_scale[0] * comb * (MIX == 1 ? 1.0f : 0.125f);     // the activations' pre-scale, the slot's weight, d / 8 (an IQ3_S weight is d (1 + 2 nibble) grid byte: no 1 / 8)
+    const float post = act_scale[0] * comb * (MIX == 1 || MIX == 3 ? 1.0f : 0.125f);     // the activations' pre-scale, the slot's weight, d / 8 (an IQ3_S weight is d (1 + 2 nibble) grid byte: no 1 / 8)
     float *out = a.partial + ((uint64_t)slot * FG + g) * H;
 #pragma unroll
     for (int k = 0; k < DU; ++k) {
         const uint32_t unit = wave + NW * k;
         if (unit < 8u * NKC) {
             float dot;
-            if constexpr (MIX == 1) { float other; iq3s_group_dot(dq[k], ad, iq3_tab, dot, other); }
+            [[maybe_unused]] float other;
+            if constexpr (MIX == 1) iq3s_group_dot(dq[k], ad, iq3_tab, dot, other);
+            else if constexpr (MIX >= 2) group_dot_fmt2<FMT>(dq[k], dd[k] >> 16, ad, lds, dot, other);
             else dot = group_dot_lut<REP, kSliceLut>(dq[k], ad, lt);
             out[64u * unit + lane] = dot * scale_to_f32(dd[k]) * post;
         }
@@ -2332,27 +2353,31 @@ __global__ __launch_bounds__(kWaves * 64, 8) void batch_slice_kernel(const uint2
 }
 
 constexpr int kSliceRep = 16;
-inline size_t slice_lds_bytes(int nkc, int rep, bool mix = false) {
-    return (size_t)(rep + 1) * kMagBytes + 128u * 4u * (size_t)kSliceLut + (size_t)nkc * 64u * 4u + 128u + 16u + sizeof(SelectOut) + (mix ? kIq3TableBytes : 0u);
+template <int MIX = 0> constexpr size_t slice_lds_bytes(int nkc) {
+    return (size_t)slice_table_bytes<kSliceRep, MIX>() + (size_t)nkc * 64u * 4u + 128u + 16u + sizeof(SelectOut) + (MIX == 1 ? kIq3TableBytes : 0u);
 }
 
 hipError_t launch_expert_slices(const void *experts, uint64_t stride, const void *down_cm, uint64_t down_stride, const void *shared, const void *shared_down_cm,
                                 const float *logits, const uint32_t *ids_in, const float *weights_in, const float *scalar_in, uint32_t *ids_out,
                                 float *weights_out, float *scalar_out, const void *xh, const void *xl, const int *xexp, float *partial, float *out,
-                                uint32_t hidden, uint32_t ffn, uint32_t n_expert, uint32_t top_k, hipStream_t s, const float *shared_gu, const float *shared_dense) {
+                                uint32_t hidden, uint32_t ffn, uint32_t n_expert, uint32_t top_k, hipStream_t s, const float *shared_gu, const float *shared_dense,
+                                uint32_t stream_type, const int8_t *grid) {
     if (!fused_iq2_supported(hidden, ffn) || top_k + 1u > (uint32_t)kWaves || n_expert > 1024u || hidden % 32u) return hipErrorInvalidValue;
     if (!logits && (!ids_in || !weights_in || !scalar_in)) return hipErrorInvalidValue;
-    const bool mix = shared_gu != nullptr;             // IQ3_S down slices (word-packed, column-sliced) and the dense shared expert
+    const bool mix = shared_gu != nullptr;             // down slices of another format (column-sliced) and the dense shared expert
     if (mix && (!shared_dense || ffn % 256u)) return hipErrorInvalidValue;
+    // 1: IQ2_XXS gate / up with IQ3_S words; 2 / 3: IQ2_XS / IQ1_M streams throughout
+    const int kind = !mix ? 0 : stream_type == T_IQ2_XS ? 2 : stream_type == T_IQ1_M ? 3 : 1;
+    if (kind >= 2 && !grid) return hipErrorInvalidValue;
     const SliceArgs a{static_cast<const uint8_t *>(experts), stride, static_cast<const uint8_t *>(down_cm), down_stride, static_cast<const uint8_t *>(shared),
                       static_cast<const uint8_t *>(shared_down_cm), logits, ids_in, weights_in, scalar_in, ids_out, weights_out, scalar_out,
                       static_cast<const _Float16 *>(xh), static_cast<const _Float16 *>(xl), xexp, partial, hidden, ffn, n_expert, top_k, route_guard().status,
-                      nullptr, 0u, nullptr, nullptr, 0u, shared_gu, shared_dense};
+                      nullptr, 0u, nullptr, nullptr, 0u, shared_gu, shared_dense, grid};
     const dim3 grid_dim(ffn / 32u, top_k + (mix ? kSliceSharedParts : 1u));
 #define REDHIP_SLICE_MIX(NKC, MIX)                                                                                                     \
     do {                                                                                                                               \
         static bool attr = false;                                                                                                       \
-        const size_t dyn = slice_lds_bytes(NKC, kSliceRep, MIX == 1);                                                                   \
+        const size_t dyn = slice_lds_bytes<MIX>(NKC);                                                                                \
         if (!attr) {                                                                                                                    \
             const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(expert_slice_kernel<NKC, kSliceRep, false, MIX>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn); \
             if (e != hipSuccess) return e;                                                                                              \
@@ -2362,8 +2387,7 @@ hipError_t launch_expert_slices(const void *experts, uint64_t stride, const void
     } while (0)
 #define REDHIP_SLICE(NKC)                                                                                                              \
     do {                                                                                                                               \
-        if (mix) REDHIP_SLICE_MIX(NKC, 1);                                                                                              \
-        else REDHIP_SLICE_MIX(NKC, 0);                                                                                                  \
+        if (kind == 3) REDHIP_SLICE_MIX(NKC, 3); else if (kind == 2) REDHIP_SLICE_MIX(NKC, 2); else if (kind == 1) REDHIP_SLICE_MIX(NKC, 1); else REDHIP_SLICE_MIX(NKC, 0); \
     } while (0)
     prof_set_stage(ST_FUSED_EXPERTS);
     switch (hidden / 512u) {
@@ -2399,7 +2423,7 @@ hipError_t launch_slot_slices(const uint64_t *slot_table, uint64_t shadow_off, c
 #define REDHIP_SLOT_SLICE(NKC)                                                                                                         \
     do {                                                                                                                               \
         static bool attr = false;                                                                                                       \
-        const size_t dyn = slice_lds_bytes(NKC, kSliceRep);                                                                             \
+        const size_t dyn = slice_lds_bytes<0>(NKC);                                                                                     \
         if (!attr) {                                                                                                                    \
             const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(expert_slice_kernel<NKC, kSliceRep, true>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn); \
             if (e != hipSuccess) return e;                                                                                              \

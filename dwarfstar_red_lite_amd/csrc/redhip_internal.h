@@ -368,7 +368,9 @@ hipError_t launch_expert_slices(const void *experts, uint64_t stride, const void
                                 const float *logits, const uint32_t *ids_in, const float *weights_in, const float *scalar_in, uint32_t *ids_out,
                                 float *weights_out, float *scalar_out, const void *xh, const void *xl, const int *xexp, float *partial, float *out,
                                 uint32_t hidden, uint32_t ffn, uint32_t n_expert, uint32_t top_k, hipStream_t s, const float *shared_gu = nullptr,
-                                const float *shared_dense = nullptr);      // both given: down_cm holds column-sliced word-packed IQ3_S, the shared expert is dense
+                                const float *shared_dense = nullptr, uint32_t stream_type = 0u, const int8_t *grid = nullptr);
+// (shared_gu and shared_dense given: a mixed layout as launch_batch_slices takes it - down_cm holds column-sliced word-packed IQ3_S, or with
+// stream_type IQ2_XS / IQ1_M and the codebook `grid`, experts / down_cm hold the row-major / column-sliced streams; the shared expert is dense)
 // one token over slots of a pool whose re-laid IQ2_XXS copies (packed gate | up, column-sliced down) lie shadow_off behind the raw bytes
 // that slot_table [top_k] points at; x split to fp16 halves inside the kernel (experts from x_split on read x1 when given); partial
 // [top_k][ffn / 32][hidden]; with tail_resid: out = tail_out2 = tail_resid + (sum + tail_shared * tail_scalar[0]). top_k <= 64

@@ -372,13 +372,13 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
         prof_set_stage(ST_OTHER);
         return 1;
     }
-    if (m->sliced_words() && ntok == 1u && m->shared_gu_ready && m->layers[layer].dense_down) {
-        // one token on IQ2_XXS gate / up with IQ3_S down: the same slices, the down matrices from their column-sliced words, the shared
-        // expert from its products (m->act, left by the router launch) and the dense copy of its down matrix
+    if (m->mixed_slices && ntok == 1u && m->shared_gu_ready && m->layers[layer].dense_down) {
+        // one token on a mixed layout whose small batches run as slices: the same slices, the down matrices from their column-sliced copy, the
+        // shared expert from its products (m->act, left by the router launch) and the dense copy of its down matrix
         const Layer &L = m->layers[layer];
         HIP_OK(launch_expert_slices(L.packed, m->packed_stride, L.down_cm, m->down_cm_stride(), nullptr, nullptr, select_here ? m->logits : nullptr,
                                     ids, weights, m->scalar, m->ids, m->weights, m->scalar, m->xh, m->xl, m->xexp, m->partial, out, c.hidden, c.ffn, c.n_expert,
-                                    c.top_k, s, m->act, L.dense_down), "expert slice launch");
+                                    c.top_k, s, m->act, L.dense_down, m->sliced_streams() ? m->dn_type : 0u, m->sliced_streams() ? m->dn_grid : nullptr), "expert slice launch");
         prof_set_stage(ST_OTHER);
         return 1;
     }
@@ -478,7 +478,7 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
     {
         const uint32_t nv = c.hidden / 256u;
         // (a handle for one token at a time needs no second copy of IQ2_XS / IQ1_M down streams: only the slices read the column-sliced one)
-        m->mixed_slices = m->mixed && ((gu == T_IQ2_XXS && dn == T_IQ3_S) || (gu_codebook && dn == gu && sgu == T_Q6_K && c.max_tokens >= 2u)) && c.ffn <= 512u &&
+        m->mixed_slices = m->mixed && ((gu == T_IQ2_XXS && dn == T_IQ3_S) || (gu_codebook && dn == gu && sgu == T_Q6_K)) && c.ffn <= 512u &&
                           c.hidden / 512u <= 4u && (nv == 2u || nv == 4u || nv == 8u || nv == 16u);
     }
     m->pk_gate_bytes = packed_matrix_bytes(gu, c.ffn, c.hidden);
