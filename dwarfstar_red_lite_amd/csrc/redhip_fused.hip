@@ -1788,7 +1788,6 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(const void *p
     constexpr int UPW = 16 * NKC / NW;                 // (row-quad, K-chunk) units of gate / up per wave
     constexpr int DU = (8 * NKC + NW - 1) / NW;        // units of 64 down rows per wave
     static_assert(UPW >= 1 && UPW * NW == 16 * NKC, "waves must tile the 16 row-quads x NKC chunks");
-    static_assert(MIX == 0 || !SLOTS, "mixed layouts: resident layers only");
     constexpr int FMT = MIX >= 2 ? MIX - 1 : 0;            // format of the routed matrices as group_dot_fmt2 numbers them
     extern __shared__ __attribute__((aligned(16))) uint8_t dyn[];
     uint8_t *lds = dyn;                                                    // REP copies of the 4 KB magnitude table (MIX 2 / 3: the fp16 codebook, once)
@@ -1803,7 +1802,7 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(const void *p
     const uint32_t tid = threadIdx.x, wave = __builtin_amdgcn_readfirstlane(tid >> 6), lane = tid & 63u, blk = lane >> 2, j = lane & 3u;
     // Mixed layouts: the shared expert's dense slice is kSliceSharedParts workgroups (a quarter of the output rows each: 16 x hidden bytes of f32
     // per row-quarter would otherwise be the longest-running workgroup); they come first in the grid, the routed slots behind them
-    const uint32_t g = blockIdx.x, slot = MIX != 0 ? (blockIdx.y < kSliceSharedParts ? top_k_first : blockIdx.y - kSliceSharedParts) : blockIdx.y;
+    const uint32_t g = blockIdx.x, slot = MIX != 0 && !SLOTS ? (blockIdx.y < kSliceSharedParts ? top_k_first : blockIdx.y - kSliceSharedParts) : blockIdx.y;
     // The leading kernel arguments repeat what the first requests of the kernel need - a.logits, a.xh, a.xl (SLOTS: a.slot_table, a.x,
     // a.x1 and a.x_split), a.n_expert, a.top_k: leading scalar arguments can be handed to a wave in registers at its start, so these
     // requests do not wait for the argument block to come from memory.
@@ -1814,7 +1813,7 @@ __global__ __launch_bounds__(kWaves * 64) void expert_slice_kernel(const void *p
     // (hidden and ffn are leading arguments too, and the branch below tests the leading copy of a.logits: the selecting wave reaches the
     // barrier without having touched the argument block, whose fetch would otherwise sit between its selection and the barrier)
     const uint32_t H = hidden_first, F = ffn_first, HG = H / 32u, HB = H / 256u, FG = F / 32u;
-    if constexpr (MIX != 0) {
+    if constexpr (MIX != 0 && !SLOTS) {
         if (is_shared) {       // the shared expert's slice from dense f32 data: SwiGLU of the 32 columns, then their part of every output row
             if (tid < 32u) {
                 const float *gu = a.shared_gu + 32u * g + tid;
@@ -2410,9 +2409,11 @@ hipError_t launch_expert_slices(const void *experts, uint64_t stride, const void
 // Two launches: slices (partial [top_k][ffn / 32][hidden]) and their sum into out (and, with a tail, out = out2 = resid + (sum + shared * scalar)).
 hipError_t launch_slot_slices(const uint64_t *slot_table, uint64_t shadow_off, const float *weights, uint32_t top_k, uint32_t hidden, uint32_t ffn,
                               const float *x, const float *x1, uint32_t x_split, float *partial, float *out, const float *tail_resid,
-                              const float *tail_shared, const float *tail_scalar, float *tail_out2, hipStream_t s) {
+                              const float *tail_shared, const float *tail_scalar, float *tail_out2, hipStream_t s, uint32_t kind, const int8_t *grid) {
     if (!fused_iq2_supported(hidden, ffn) || hidden % 32u || !top_k || top_k > 64u || !slot_table || !weights || !x || !partial || !out) return hipErrorInvalidValue;
+    if (kind > 3u || (kind >= 2u && !grid) || (kind != 0u && (hidden > 2048u || ffn % 256u))) return hipErrorInvalidValue;
     SliceArgs a{};
+    a.grid = grid;
     a.weights_in = weights;
     a.partial = partial;
     a.hidden = hidden; a.ffn = ffn; a.n_expert = 0u; a.top_k = top_k;
@@ -2420,26 +2421,31 @@ hipError_t launch_slot_slices(const uint64_t *slot_table, uint64_t shadow_off, c
     a.shadow_off = shadow_off;
     a.x = x; a.x1 = x1; a.x_split = x_split;
     const dim3 grid_dim(ffn / 32u, top_k);
-#define REDHIP_SLOT_SLICE(NKC)                                                                                                         \
+#define REDHIP_SLOT_SLICE_MIX(NKC, MIX)                                                                                                \
     do {                                                                                                                               \
         static bool attr = false;                                                                                                       \
-        const size_t dyn = slice_lds_bytes<0>(NKC);                                                                                     \
+        const size_t dyn = slice_lds_bytes<MIX>(NKC);                                                                                   \
         if (!attr) {                                                                                                                    \
-            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(expert_slice_kernel<NKC, kSliceRep, true>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn); \
+            const hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(expert_slice_kernel<NKC, kSliceRep, true, MIX>), hipFuncAttributeMaxDynamicSharedMemorySize, (int)dyn); \
             if (e != hipSuccess) return e;                                                                                              \
             attr = true;                                                                                                                \
         }                                                                                                                               \
-        REDHIP_LAUNCH((expert_slice_kernel<NKC, kSliceRep, true>), grid_dim, dim3(kWaves * 64), dyn, s, (const void *)a.slot_table, a.n_expert, a.top_k, (const void *)a.x, (const void *)a.x1, a.x_split, a.hidden, a.ffn, a); \
+        REDHIP_LAUNCH((expert_slice_kernel<NKC, kSliceRep, true, MIX>), grid_dim, dim3(kWaves * 64), dyn, s, (const void *)a.slot_table, a.n_expert, a.top_k, (const void *)a.x, (const void *)a.x1, a.x_split, a.hidden, a.ffn, a); \
+    } while (0)
+#define REDHIP_SLOT_SLICE(NKC)                                                                                                         \
+    do {                                                                                                                               \
+        if (kind == 3u) REDHIP_SLOT_SLICE_MIX(NKC, 3); else if (kind == 2u) REDHIP_SLOT_SLICE_MIX(NKC, 2); else if (kind == 1u) REDHIP_SLOT_SLICE_MIX(NKC, 1); else REDHIP_SLOT_SLICE_MIX(NKC, 0); \
     } while (0)
     prof_set_stage(ST_FUSED_EXPERTS);
     switch (hidden / 512u) {
         case 1: REDHIP_SLOT_SLICE(1); break;
         case 2: REDHIP_SLOT_SLICE(2); break;
         case 4: REDHIP_SLOT_SLICE(4); break;
-        case 8: REDHIP_SLOT_SLICE(8); break;
+        case 8: REDHIP_SLOT_SLICE_MIX(8, 0); break;
         default: return hipErrorInvalidValue;
     }
 #undef REDHIP_SLOT_SLICE
+#undef REDHIP_SLOT_SLICE_MIX
     hipError_t e = hipGetLastError();
     if (e != hipSuccess) return e;
     prof_set_stage(ST_SLICE_SUM);

@@ -376,7 +376,10 @@ hipError_t launch_expert_slices(const void *experts, uint64_t stride, const void
 // [top_k][ffn / 32][hidden]; with tail_resid: out = tail_out2 = tail_resid + (sum + tail_shared * tail_scalar[0]). top_k <= 64
 hipError_t launch_slot_slices(const uint64_t *slot_table, uint64_t shadow_off, const float *weights, uint32_t top_k, uint32_t hidden, uint32_t ffn,
                               const float *x, const float *x1, uint32_t x_split, float *partial, float *out, const float *tail_resid,
-                              const float *tail_shared, const float *tail_scalar, float *tail_out2, hipStream_t s);
+                              const float *tail_shared, const float *tail_scalar, float *tail_out2, hipStream_t s, uint32_t kind = 0u,
+                              const int8_t *grid = nullptr);
+// (kind 1: the copies hold packed IQ2_XXS gate | up and column-sliced IQ3_S words; 2 / 3: row-major IQ2_XS / IQ1_M streams of gate | up,
+// column-sliced streams of down, decoded through the codebook `grid`; kinds 1..3: hidden <= 2048)
 // the same for 2..16 tokens (at most 128 pairs) whose pairs are grouped by expert: pass_list / n_pass from the pair sort (GroupJob), weights
 // [ntok][top_k] and scalar [ntok] of the routing; partial [ntok][top_k + 1][ffn / 32][hidden]
 hipError_t launch_batch_slices(const void *experts, uint64_t stride, const void *down_cm, uint64_t down_stride, const void *shared, const void *shared_down_cm,

@@ -57,12 +57,18 @@ struct TopkPool {
     static constexpr int kStages = 4;
     Stage stage[kStages];
     int next_stage = 0;
-    // Opt-in fast path for one declared expert shape (all IQ2_XXS): behind the raw bytes of a slot lies a second copy in the layout the
-    // slice kernels read (packed gate | up streams, column-sliced down), written when the slot is loaded. The copy of a slot starts
-    // shadow_off behind the slot's address, the same distance in every slot, so a device-side slot table needs no second table.
-    // With REDHIP_TOPK_FAST_TILES a third copy follows tile_off behind the slot's address: the three matrices tile-major, as the prefill
-    // tile kernels read them; the batched form then runs on those kernels.
-    struct FastShape { uint32_t word = 0, hidden = 0, ffn = 0; uint64_t gate = 0, down = 0, shadow_off = 0, tile_off = 0, slot_need = 0; bool tiles = false; };
+    // Opt-in fast path for one declared expert shape: behind the raw bytes of a slot lies a second copy in the layout the slice kernels
+    // read (packed gate | up streams, column-sliced down), written when the slot is loaded. The copy of a slot starts shadow_off behind
+    // the slot's address, the same distance in every slot, so a device-side slot table needs no second table.
+    // kind 0: all IQ2_XXS; 1: IQ2_XXS gate / up with IQ3_S down (column-sliced words); 2 / 3: all IQ2_XS / all IQ1_M (streams decoded
+    // through the pool's codebooks). gate / down: raw bytes of a matrix, gate_copy / down_copy: bytes of its re-laid form.
+    // With REDHIP_TOPK_FAST_TILES (kind 0) a third copy follows tile_off behind the slot's address: the three matrices tile-major, as the
+    // prefill tile kernels read them; the batched form then runs on those kernels.
+    struct FastShape {
+        uint32_t word = 0, hidden = 0, ffn = 0, kind = 0;
+        uint64_t gate = 0, down = 0, gate_copy = 0, down_copy = 0, shadow_off = 0, tile_off = 0, slot_need = 0;
+        bool tiles = false;
+    };
     bool fast = false;
     FastShape fs;
     uint64_t cls_shadow[RL_TOPK_MAX_CLASSES] = {0};   // bytes behind each slot of the class for its copy (0: the class holds none)
@@ -103,7 +109,7 @@ struct TopkPool {
     }
     // may calls of this shape run on the slice kernels? (the copies of the slots they name are checked by the caller where it knows them)
     bool fast_shape(uint32_t word, uint32_t hidden, uint32_t ffn) const {
-        return fast && hidden == fs.hidden && ffn == fs.ffn && word_gate_up(word) == T_IQ2_XXS && word_down(word) == T_IQ2_XXS;
+        return fast && hidden == fs.hidden && ffn == fs.ffn && word_gate_up(word) == word_gate_up(fs.word) && word_down(word) == word_down(fs.word);
     }
     void mark(const uint32_t *slots, uint32_t n, int delta) {
         std::lock_guard<std::mutex> lk(mu);
@@ -210,10 +216,12 @@ bool enqueue_token(TopkPool *p, hipStream_t s, const uint64_t *table_dev, const 
     if (slots_fast && top_k <= kFastMaxTopK && row_start == 0u && row_count == hidden && (out || tail) && p->fast_shape(type_word, hidden, ffn)) {
         // two launches on the slots' re-laid copies: expert slices, then the sum of their partial vectors (with the tail when asked)
         float *partial = static_cast<float *>(p->partial.p);
+        if (!bind_grids(p, type_word)) return false;
+        const int8_t *grid = p->fs.kind >= 2u ? caller_grid_device(word_gate_up(type_word)) : nullptr;
         const hipError_t e = tail ? launch_slot_slices(table_dev, p->fs.shadow_off, weights_dev, top_k, hidden, ffn, x, x1, x_split, partial, tail->x,
-                                                       tail->resid, tail->shared, tail->scalar, tail->layer_out, s)
+                                                       tail->resid, tail->shared, tail->scalar, tail->layer_out, s, p->fs.kind, grid)
                                   : launch_slot_slices(table_dev, p->fs.shadow_off, weights_dev, top_k, hidden, ffn, x, x1, x_split, partial, out,
-                                                       nullptr, nullptr, nullptr, nullptr, s);
+                                                       nullptr, nullptr, nullptr, nullptr, s, p->fs.kind, grid);
         if (e != hipSuccess) { TOPK_ERR("top-k HIP command failed: %s", hipGetErrorString(e)); return false; }
         return true;
     }
@@ -525,27 +533,32 @@ int redmetal_topk_pool_set_classes(redmetal_topk_pool_t handle, uint32_t n, cons
 int redhip_topk_pool_enable_fast_path(redmetal_topk_pool_t handle, uint32_t ggml_type, uint32_t hidden_size, uint32_t ffn_size, uint32_t flags) {
     TopkPool *p = pool_of(handle);
     if (!p) return 0;
-    if (!type_word_ok(ggml_type) || word_gate_up(ggml_type) != T_IQ2_XXS || word_down(ggml_type) != T_IQ2_XXS || !fused_iq2_supported(hidden_size, ffn_size) || hidden_size % 32u) {
-        TOPK_ERR("the top-k fast path takes all-IQ2_XXS experts with hidden in {512, 1024, 2048, 4096} and ffn a multiple of 256 up to 1024 (asked: type word 0x%x, hidden=%u, ffn=%u)",
-                 ggml_type, hidden_size, ffn_size);
+    const uint32_t gu = type_word_ok(ggml_type) ? word_gate_up(ggml_type) : 0u, dn = type_word_ok(ggml_type) ? word_down(ggml_type) : 0u;
+    const uint32_t kind = gu == T_IQ2_XXS && dn == T_IQ2_XXS ? 0u : gu == T_IQ2_XXS && dn == T_IQ3_S ? 1u : gu == T_IQ2_XS && dn == T_IQ2_XS ? 2u : gu == T_IQ1_M && dn == T_IQ1_M ? 3u : 4u;
+    if (kind > 3u || !fused_iq2_supported(hidden_size, ffn_size) || hidden_size % 32u || (kind != 0u && hidden_size > 2048u)) {
+        TOPK_ERR("the top-k fast path takes all-IQ2_XXS experts with hidden in {512, 1024, 2048, 4096}, or IQ2_XXS gate / up with IQ3_S down, all-IQ2_XS or all-IQ1_M experts with "
+                 "hidden in {512, 1024, 2048}; ffn a multiple of 256 up to 1024 (asked: type word 0x%x, hidden=%u, ffn=%u)", ggml_type, hidden_size, ffn_size);
         return 0;
     }
-    if ((flags & ~REDHIP_TOPK_FAST_TILES) || ((flags & REDHIP_TOPK_FAST_TILES) && (ffn_size > 512u || hidden_size > 2048u))) {
-        TOPK_ERR("the top-k fast path keeps tile-major copies for hidden <= 2048 and ffn <= 512 only (asked: hidden=%u, ffn=%u, flags 0x%x)", hidden_size, ffn_size, flags);
+    if ((flags & ~REDHIP_TOPK_FAST_TILES) || ((flags & REDHIP_TOPK_FAST_TILES) && (kind != 0u || ffn_size > 512u || hidden_size > 2048u))) {
+        TOPK_ERR("the top-k fast path keeps tile-major copies for all-IQ2_XXS experts with hidden <= 2048 and ffn <= 512 only (asked: type word 0x%x, hidden=%u, ffn=%u, flags 0x%x)",
+                 ggml_type, hidden_size, ffn_size, flags);
         return 0;
     }
     std::lock_guard<std::mutex> lk(p->mu);
     if (p->slabs_made) { TOPK_ERR("the top-k fast path must be enabled before any slab is allocated"); return 0; }
     if (p->fast) { TOPK_ERR("the top-k fast path is already enabled"); return 0; }
     TopkPool::FastShape f;
-    f.word = ggml_type; f.hidden = hidden_size; f.ffn = ffn_size;
-    f.gate = (uint64_t)ffn_size * pool_row_bytes(T_IQ2_XXS, hidden_size);
-    f.down = (uint64_t)hidden_size * pool_row_bytes(T_IQ2_XXS, ffn_size);
-    const uint64_t payload = 2u * f.gate + f.down;
+    f.word = ggml_type; f.hidden = hidden_size; f.ffn = ffn_size; f.kind = kind;
+    f.gate = (uint64_t)ffn_size * pool_row_bytes(gu, hidden_size);
+    f.down = (uint64_t)hidden_size * pool_row_bytes(dn, ffn_size);
+    f.gate_copy = packed_matrix_bytes(gu, ffn_size, hidden_size);
+    f.down_copy = kind == 1u ? iq3s_words_bytes(hidden_size, ffn_size) : packed_matrix_bytes(dn, hidden_size, ffn_size);
+    const uint64_t payload = 2u * f.gate + f.down, copy_bytes = 2u * f.gate_copy + f.down_copy;
     f.tiles = (flags & REDHIP_TOPK_FAST_TILES) != 0u;
     f.shadow_off = round_up(payload, 256u);
-    f.tile_off = 2u * f.shadow_off;
-    f.slot_need = round_up((f.tiles ? f.tile_off : f.shadow_off) + payload, 4096u);
+    f.tile_off = f.shadow_off + round_up(copy_bytes, 256u);
+    f.slot_need = round_up(f.tiles ? f.tile_off + payload : f.shadow_off + copy_bytes, 4096u);
     // classes that can hold an expert of this shape grow by the room for its copy; the budget covers both
     uint64_t shadow[RL_TOPK_MAX_CLASSES] = {0}, total = 0;
     bool any = false;
@@ -655,8 +668,13 @@ int redmetal_topk_pool_load_expert(redmetal_topk_pool_t h, uint32_t slot_id,
         bool ok_copy = false;
         if (gate_bytes == f.gate && up_bytes == f.gate && down_bytes == f.down && f.slot_need <= p->phys(p->class_of(slot_id))) {
             uint8_t *copy = base + f.shadow_off, *tiles = base + f.tile_off;
-            hipError_t e = launch_repack_iq2xxs(base, f.gate, 2u, f.ffn, f.hidden, false, copy, f.gate, nullptr);
-            if (e == hipSuccess) e = launch_repack_iq2xxs(base + 2u * f.gate, 0u, 1u, f.hidden, f.ffn, true, copy + 2u * f.gate, 0u, nullptr);
+            const uint32_t gu = word_gate_up(f.word), dn = word_down(f.word);
+            hipError_t e = f.kind <= 1u ? launch_repack_iq2xxs(base, f.gate, 2u, f.ffn, f.hidden, false, copy, f.gate_copy, nullptr)
+                                        : launch_repack_gateup(gu, base, f.gate, 2u, f.ffn, f.hidden, copy, f.gate_copy, nullptr);
+            if (e == hipSuccess)
+                e = f.kind == 0u   ? launch_repack_iq2xxs(base + 2u * f.gate, 0u, 1u, f.hidden, f.ffn, true, copy + 2u * f.gate_copy, 0u, nullptr)
+                    : f.kind == 1u ? launch_repack_iq3s_words(base + 2u * f.gate, 0u, 1u, f.hidden, f.ffn, copy + 2u * f.gate_copy, 0u, nullptr, true)
+                                   : launch_repack_gateup(dn, base + 2u * f.gate, 0u, 1u, f.hidden, f.ffn, copy + 2u * f.gate_copy, 0u, nullptr, true);
             if (f.tiles) {
                 if (e == hipSuccess) e = launch_tile_packed(copy, f.gate, 2u, f.ffn, f.hidden, tiles, f.gate, nullptr);
                 if (e == hipSuccess) e = launch_repack_iq2xxs(base + 2u * f.gate, 0u, 1u, f.hidden, f.ffn, false, p->stage_down.p, 0u, nullptr);

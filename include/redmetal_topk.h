@@ -164,15 +164,18 @@ int redmetal_topk_pool_encode_mapped(redmetal_topk_pool_t pool, void *stream,
     const uint32_t *tok_pair, void *input_dev, uint64_t input_offset, void *output_dev, uint64_t output_offset);
 
 /* No counterpart in the reference. Opt-in, after redmetal_topk_pool_set_classes (if used) and before the first slab exists (no load,
- * no slot_addresses, no allocate_all yet): experts of one declared shape - every matrix IQ2_XXS (type word 16), hidden_size in
- * {512, 1024, 2048, 4096}, ffn_size a multiple of 256 up to 1024 - also keep, behind the raw bytes of their slot, a copy in the
+ * no slot_addresses, no allocate_all yet): experts of one declared shape - every matrix IQ2_XXS (type word 16) with hidden_size in
+ * {512, 1024, 2048, 4096}, or IQ2_XXS gate / up with IQ3_S down (16 | 21 << 8), every matrix IQ2_XS (17) or every matrix IQ1_M (29, the
+ * last two decoded through the pool's codebooks) with hidden_size in {512, 1024, 2048}; ffn_size a multiple of 256 up to 1024 - also
+ * keep, behind the raw bytes of their slot, a copy in the
  * layout this library's fused kernels read (packed gate | up streams, column-sliced down matrix), written by
  * redmetal_topk_pool_load_expert. The single-token calls (encode, execute, encode_device, _into, _into2 with an output, _tail) of that
  * shape with whole output rows and top_k <= 64 then run as two launches on those copies instead of three on the raw rows; every other
  * call runs as before, and redmetal_topk_pool_slot_addresses keeps returning the raw bytes. The copies count against the budget: a
- * slot class that holds such experts grows to twice the expert's bytes (a single-class pool's capacity shrinks accordingly; with
+ * slot class that holds such experts grows to about twice the expert's bytes - the raw bytes rounded up to 256, then the copy: 8 bytes
+ * per 32 weights + 2 per 256 (IQ2_XS 9 per 32, IQ3_S down 16 per 32), the whole rounded up to 4096 - (a single-class pool's capacity shrinks accordingly; with
  * classes set, the call fails when they no longer fit). With the device-driven forms the slot table must hold addresses of this
- * pool's slots loaded with experts of the declared shape. flags: REDHIP_TOPK_FAST_TILES (hidden_size <= 2048 and ffn_size <= 512)
+ * pool's slots loaded with experts of the declared shape. flags: REDHIP_TOPK_FAST_TILES (all IQ2_XXS, hidden_size <= 2048 and ffn_size <= 512)
  * adds a third copy per slot, tile-major as this library's prefill kernels read it (the slot class grows to three times the expert's
  * bytes); redmetal_topk_pool_encode_batched of that shape then runs on those kernels - tiles of up to 32 pairs per expert on the
  * matrix units - when every slot it names holds its copies; 0: none. Returns 1, or 0 with redmetal_topk_last_error(). */

@@ -59,9 +59,15 @@ class Case:
         kw = dict(slots_per_slab=5)
         kw.update(pool_kw)
         up = lambda v, a: (v + a - 1) // a * a
-        # with the fast path a slot also holds the re-laid copy of its expert, 256-aligned behind the raw bytes
-        # (and with tiles a third, tile-major one)
-        self.slot_phys = up((2 if tiles else 1) * up(self.slot_bytes, 256) + self.slot_bytes, 4096) if fast else up(self.slot_bytes, 4096)
+        # with the fast path a slot also holds the re-laid copy of its expert, 256-aligned behind the raw bytes (and with tiles a third,
+        # tile-major one). The copy: 8 bytes per 32 weights + 2 per 256; IQ2_XS 9 per 32; IQ3_S down matrices 16 per 32
+        per32 = lambda t: {17: 9, 21: 16}.get(t, 8)
+        n_w = hidden * ffn
+        self.copy_bytes = 2 * (n_w // 32 * per32(cfg["gate_up_type"]) + n_w // 256 * 2) + n_w // 32 * per32(cfg["down_type"]) + n_w // 256 * 2
+        if tiles:
+            self.slot_phys = up(up(self.slot_bytes, 256) + up(self.copy_bytes, 256) + self.slot_bytes, 4096)
+        else:
+            self.slot_phys = up(up(self.slot_bytes, 256) + self.copy_bytes, 4096) if fast else up(self.slot_bytes, 4096)
         self.pool = RedMetalTopKPool(self.path, (n_load + 3) * self.slot_phys, self.slot_bytes, iq2_xs_grid=grids[0], iq1_m_grid=grids[1], **kw)
         self.word = type_word(cfg)
         if fast:
@@ -84,7 +90,7 @@ class Case:
         return acc
 
 
-@pytest.mark.parametrize("layout,fast", [("iq2", False), ("f2", False), ("xs", False), ("m", False), ("iq2", True)])
+@pytest.mark.parametrize("layout,fast", [("iq2", False), ("f2", False), ("xs", False), ("m", False), ("iq2", True), ("f2", True), ("xs", True), ("m", True)])
 def test_execute_against_cpu_path(tmp_path, grids, layout, fast):
     """fast: the calls with whole output rows run on the slots' re-laid copies, the row windows on the raw rows"""
     c = Case(tmp_path, grids, layout, fast=fast)
@@ -103,9 +109,11 @@ def test_execute_against_cpu_path(tmp_path, grids, layout, fast):
     c.pool.close()
 
 
-def test_execute_full_shape_top10(tmp_path, grids):
-    """hidden 2048, ffn 512, ten experts of the mixed-precision layout (gate/up IQ2_XXS, down IQ3_S)"""
-    c = Case(tmp_path, grids, "f2", hidden=2048, ffn=512, n_expert=12)
+@pytest.mark.parametrize("layout,fast", [("f2", False), ("f2", True), ("xs", True), ("m", True)])
+def test_execute_full_shape_top10(tmp_path, grids, layout, fast):
+    """hidden 2048, ffn 512, ten experts of the mixed-precision layout (gate/up IQ2_XXS, down IQ3_S) and of the IQ2_XS / IQ1_M layouts;
+    fast: on the slots' re-laid copies"""
+    c = Case(tmp_path, grids, layout, hidden=2048, ffn=512, n_expert=12, fast=fast)
     rng = np.random.default_rng(6)
     experts = rng.permutation(12)[:10]
     w = rng.random(10).astype(np.float32)
@@ -184,7 +192,7 @@ def test_slot_classes_and_budget(tmp_path, grids):
     c.pool.close()
 
 
-@pytest.mark.parametrize("layout,fast", [("iq2", False), ("f2", False), ("iq2", True)])
+@pytest.mark.parametrize("layout,fast", [("iq2", False), ("f2", False), ("iq2", True), ("f2", True), ("xs", True), ("m", True)])
 def test_device_driven_forms(tmp_path, grids, layout, fast):
     """slot addresses gathered on the device from the residency table, weights on the device: into, into with the sum left to the
     caller, two input vectors, and the fused tail; replayed from a HIP graph as well (these forms copy nothing from the host).
@@ -359,7 +367,11 @@ def test_fast_path_copies_follow_the_slots(tmp_path, grids):
     c.pool.close()
     pool = RedMetalTopKPool(c.path, 8 * c.slot_phys, c.slot_bytes, iq2_xs_grid=grids[0], iq1_m_grid=grids[1])
     with pytest.raises(RedHipError, match="all-IQ2_XXS"):
-        pool.enable_fast_path(16 | (21 << 8), H, F)
+        pool.enable_fast_path(14, H, F)
+    with pytest.raises(RedHipError, match="all-IQ2_XXS"):
+        pool.enable_fast_path(17 | (29 << 8), H, F)
+    with pytest.raises(RedHipError, match="tile-major copies"):
+        pool.enable_fast_path(17, H, F, tiles=True)
     with pytest.raises(RedHipError, match="all-IQ2_XXS"):
         pool.enable_fast_path(16, 768, F)
     pool.enable_fast_path(16, H, F)
