@@ -62,8 +62,8 @@ struct TopkPool {
     // the slot's address, the same distance in every slot, so a device-side slot table needs no second table.
     // kind 0: all IQ2_XXS; 1: IQ2_XXS gate / up with IQ3_S down (column-sliced words); 2 / 3: all IQ2_XS / all IQ1_M (streams decoded
     // through the pool's codebooks). gate / down: raw bytes of a matrix, gate_copy / down_copy: bytes of its re-laid form.
-    // With REDHIP_TOPK_FAST_TILES (kind 0) a third copy follows tile_off behind the slot's address: the three matrices tile-major, as the
-    // prefill tile kernels read them; the batched form then runs on those kernels.
+    // With REDHIP_TOPK_FAST_TILES (kinds 0, 2, 3) a third copy follows tile_off behind the slot's address: the three matrices tile-major
+    // (as large as the second copy), as the prefill tile kernels read them; the batched form then runs on those kernels.
     struct FastShape {
         uint32_t word = 0, hidden = 0, ffn = 0, kind = 0;
         uint64_t gate = 0, down = 0, gate_copy = 0, down_copy = 0, shadow_off = 0, tile_off = 0, slot_need = 0;
@@ -336,6 +336,7 @@ bool enqueue_pairs_tiles(TopkPool *p, hipStream_t s, const std::vector<uint64_t>
                          uint32_t tok_first, uint32_t ntok, uint32_t top_k, uint32_t n_pairs, const uint32_t *pair_token, const float *pair_weight,
                          const uint32_t *expert_start, const uint32_t *tok_pair, const float *x, float *out) {
     std::lock_guard<std::recursive_mutex> lk(p->enc_mu);
+    if (!bind_grids(p, p->fs.word)) return false;
     uint64_t lowest = slot_addr[0];
     for (uint64_t a : slot_addr) lowest = a < lowest ? a : lowest;
     std::vector<uint32_t> u;
@@ -377,8 +378,14 @@ bool enqueue_pairs_tiles(TopkPool *p, hipStream_t s, const std::vector<uint64_t>
     const uint8_t *tiles = reinterpret_cast<const uint8_t *>(lowest + p->fs.tile_off);
     // (the split kernel also forms a gate logit per row from a second vector: x itself stands in, the result is not used)
     hipError_t e = launch_prep(x, x, (uint32_t)rows, hidden, xh, xl, xexp, gate_unused, s, nullptr, nullptr);
-    if (e == hipSuccess) e = launch_prefill_packed(nullptr, 256u, nullptr, tiles, nullptr, d_uid, d_start, d_pair_token, d_unique, tile_group, tile_pair0, tile_n, n_tiles,
-                                                   xh, xl, xexp, act_h, act_l, act_exp, tmp, nullptr, hidden, ffn, top_k, ntok, n_expert, s, false, false);
+    if (e == hipSuccess && p->fs.kind == 0u)
+        e = launch_prefill_packed(nullptr, 256u, nullptr, tiles, nullptr, d_uid, d_start, d_pair_token, d_unique, tile_group, tile_pair0, tile_n, n_tiles,
+                                  xh, xl, xexp, act_h, act_l, act_exp, tmp, nullptr, hidden, ffn, top_k, ntok, n_expert, s, false, false);
+    else if (e == hipSuccess) {      // IQ2_XS / IQ1_M: the same tile kernels on the tile-major streams, through the pool's codebooks
+        const uint32_t t = word_gate_up(p->fs.word);
+        e = launch_prefill_streams(t, caller_grid_device(t), tiles, 256u, t, caller_grid_device(t), tiles + 2u * p->fs.gate_copy, 256u, d_uid, d_start, d_pair_token,
+                                   d_unique, tile_group, tile_pair0, tile_n, n_tiles, xh, xl, xexp, act_h, act_l, act_exp, tmp, hidden, ffn, top_k, ntok, n_expert, s, false);
+    }
     if (e == hipSuccess) e = launch_batch_combine(tmp, st.w, d_tok_pair, ntok, top_k, nullptr, nullptr, hidden, out + (uint64_t)tok_first * hidden, s);
     stage_done(st, s);
     if (e != hipSuccess) { TOPK_ERR("batched top-k HIP command failed: %s", hipGetErrorString(e)); return false; }
@@ -540,8 +547,8 @@ int redhip_topk_pool_enable_fast_path(redmetal_topk_pool_t handle, uint32_t ggml
                  "hidden in {512, 1024, 2048}; ffn a multiple of 256 up to 1024 (asked: type word 0x%x, hidden=%u, ffn=%u)", ggml_type, hidden_size, ffn_size);
         return 0;
     }
-    if ((flags & ~REDHIP_TOPK_FAST_TILES) || ((flags & REDHIP_TOPK_FAST_TILES) && (kind != 0u || ffn_size > 512u || hidden_size > 2048u))) {
-        TOPK_ERR("the top-k fast path keeps tile-major copies for all-IQ2_XXS experts with hidden <= 2048 and ffn <= 512 only (asked: type word 0x%x, hidden=%u, ffn=%u, flags 0x%x)",
+    if ((flags & ~REDHIP_TOPK_FAST_TILES) || ((flags & REDHIP_TOPK_FAST_TILES) && (kind == 1u || ffn_size > 512u || hidden_size > 2048u))) {
+        TOPK_ERR("the top-k fast path keeps tile-major copies for all-IQ2_XXS, all-IQ2_XS and all-IQ1_M experts with hidden <= 2048 and ffn <= 512 only (asked: type word 0x%x, hidden=%u, ffn=%u, flags 0x%x)",
                  ggml_type, hidden_size, ffn_size, flags);
         return 0;
     }
@@ -558,7 +565,7 @@ int redhip_topk_pool_enable_fast_path(redmetal_topk_pool_t handle, uint32_t ggml
     f.tiles = (flags & REDHIP_TOPK_FAST_TILES) != 0u;
     f.shadow_off = round_up(payload, 256u);
     f.tile_off = f.shadow_off + round_up(copy_bytes, 256u);
-    f.slot_need = round_up(f.tiles ? f.tile_off + payload : f.shadow_off + copy_bytes, 4096u);
+    f.slot_need = round_up(f.tiles ? f.tile_off + copy_bytes : f.shadow_off + copy_bytes, 4096u);
     // classes that can hold an expert of this shape grow by the room for its copy; the budget covers both
     uint64_t shadow[RL_TOPK_MAX_CLASSES] = {0}, total = 0;
     bool any = false;
@@ -585,7 +592,7 @@ int redhip_topk_pool_enable_fast_path(redmetal_topk_pool_t handle, uint32_t ggml
         TOPK_ERR("top-k slot classes with the fast path's copies exceed the cache budget");
         return 0;
     }
-    if (!p->partial.reserve((size_t)kFastMaxTopK * (ffn_size / 32u) * hidden_size * sizeof(float)) || (f.tiles && !p->stage_down.reserve((size_t)f.down))) {
+    if (!p->partial.reserve((size_t)kFastMaxTopK * (ffn_size / 32u) * hidden_size * sizeof(float)) || (f.tiles && !p->stage_down.reserve((size_t)f.down_copy))) {
         TOPK_ERR("failed to allocate top-k activation buffers");
         return 0;
     }
@@ -675,10 +682,12 @@ int redmetal_topk_pool_load_expert(redmetal_topk_pool_t h, uint32_t slot_id,
                 e = f.kind == 0u   ? launch_repack_iq2xxs(base + 2u * f.gate, 0u, 1u, f.hidden, f.ffn, true, copy + 2u * f.gate_copy, 0u, nullptr)
                     : f.kind == 1u ? launch_repack_iq3s_words(base + 2u * f.gate, 0u, 1u, f.hidden, f.ffn, copy + 2u * f.gate_copy, 0u, nullptr, true)
                                    : launch_repack_gateup(dn, base + 2u * f.gate, 0u, 1u, f.hidden, f.ffn, copy + 2u * f.gate_copy, 0u, nullptr, true);
-            if (f.tiles) {
-                if (e == hipSuccess) e = launch_tile_packed(copy, f.gate, 2u, f.ffn, f.hidden, tiles, f.gate, nullptr);
-                if (e == hipSuccess) e = launch_repack_iq2xxs(base + 2u * f.gate, 0u, 1u, f.hidden, f.ffn, false, p->stage_down.p, 0u, nullptr);
-                if (e == hipSuccess) e = launch_tile_packed(p->stage_down.p, 0u, 1u, f.hidden, f.ffn, tiles + 2u * f.gate, 0u, nullptr);
+            if (f.tiles) {      // (kinds 0, 2, 3: the row-major packed down matrix passes through a staging buffer)
+                if (e == hipSuccess) e = launch_tile_packed(copy, f.gate_copy, 2u, f.ffn, f.hidden, tiles, f.gate_copy, nullptr, gu == T_IQ2_XS);
+                if (e == hipSuccess)
+                    e = f.kind == 0u ? launch_repack_iq2xxs(base + 2u * f.gate, 0u, 1u, f.hidden, f.ffn, false, p->stage_down.p, 0u, nullptr)
+                                     : launch_repack_gateup(dn, base + 2u * f.gate, 0u, 1u, f.hidden, f.ffn, p->stage_down.p, 0u, nullptr);
+                if (e == hipSuccess) e = launch_tile_packed(p->stage_down.p, 0u, 1u, f.hidden, f.ffn, tiles + 2u * f.gate_copy, 0u, nullptr, dn == T_IQ2_XS);
             }
             if (e == hipSuccess) e = hipStreamSynchronize(nullptr);
             if (e != hipSuccess) { TOPK_ERR("top-k slot re-layout failed: %s", hipGetErrorString(e)); return 0; }

@@ -65,7 +65,7 @@ class Case:
         n_w = hidden * ffn
         self.copy_bytes = 2 * (n_w // 32 * per32(cfg["gate_up_type"]) + n_w // 256 * 2) + n_w // 32 * per32(cfg["down_type"]) + n_w // 256 * 2
         if tiles:
-            self.slot_phys = up(up(self.slot_bytes, 256) + up(self.copy_bytes, 256) + self.slot_bytes, 4096)
+            self.slot_phys = up(up(self.slot_bytes, 256) + up(self.copy_bytes, 256) + self.copy_bytes, 4096)
         else:
             self.slot_phys = up(up(self.slot_bytes, 256) + self.copy_bytes, 4096) if fast else up(self.slot_bytes, 4096)
         self.pool = RedMetalTopKPool(self.path, (n_load + 3) * self.slot_phys, self.slot_bytes, iq2_xs_grid=grids[0], iq1_m_grid=grids[1], **kw)
@@ -265,7 +265,7 @@ def test_device_driven_forms(tmp_path, grids, layout, fast):
     c.pool.close()
 
 
-@pytest.mark.parametrize("layout,tiles", [("iq2", False), ("f2", False), ("xs", False), ("iq2", True)])
+@pytest.mark.parametrize("layout,tiles", [("iq2", False), ("f2", False), ("xs", False), ("iq2", True), ("xs", True), ("m", True)])
 def test_batched_and_mapped_pairs(tmp_path, grids, layout, tiles):
     """prefill form: pairs sorted by expert over a ragged routing (an expert with 19 pairs, experts with one, experts with none), tokens
     tok_first .. of a larger buffer; the same pairs on experts read in place from device copies of the whole tensors.
@@ -371,7 +371,7 @@ def test_fast_path_copies_follow_the_slots(tmp_path, grids):
     with pytest.raises(RedHipError, match="all-IQ2_XXS"):
         pool.enable_fast_path(17 | (29 << 8), H, F)
     with pytest.raises(RedHipError, match="tile-major copies"):
-        pool.enable_fast_path(17, H, F, tiles=True)
+        pool.enable_fast_path(16 | (21 << 8), H, F, tiles=True)
     with pytest.raises(RedHipError, match="all-IQ2_XXS"):
         pool.enable_fast_path(16, 768, F)
     pool.enable_fast_path(16, H, F)
@@ -382,14 +382,15 @@ def test_fast_path_copies_follow_the_slots(tmp_path, grids):
     pool.close()
 
 
-def test_batched_chunk_of_512_tokens_on_the_tile_copies(tmp_path, grids):
+@pytest.mark.parametrize("layout", ["iq2", "xs"])
+def test_batched_chunk_of_512_tokens_on_the_tile_copies(tmp_path, grids, layout):
     """a prefill chunk at the full expert shape (hidden 2048, ffn 512, ten of 48 experts per token, 512 tokens) through the batched form
     on the slots' tile-major copies: every 16th token against the CPU path, every token against the same call on a pool without copies
     (the raw-row kernels)"""
     H, F, E, K, ntok = 2048, 512, 48, 10, 512
-    fast = Case(tmp_path, grids, "iq2", hidden=H, ffn=F, n_expert=E, fast=True, tiles=True, slots_per_slab=7)
+    fast = Case(tmp_path, grids, layout, hidden=H, ffn=F, n_expert=E, fast=True, tiles=True, slots_per_slab=7)
     (tmp_path / "raw").mkdir()
-    raw = Case(tmp_path / "raw", grids, "iq2", hidden=H, ffn=F, n_expert=E)
+    raw = Case(tmp_path / "raw", grids, layout, hidden=H, ffn=F, n_expert=E)
     rng = np.random.default_rng(12)
     logits = rng.standard_normal((ntok, E)) + 1.5 * (np.arange(E) < 3)                # three popular experts: wide tiles, narrow ones, singles
     ids = np.argsort(-logits, axis=1)[:, :K].astype(np.uint32)
