@@ -62,7 +62,7 @@ struct TopkPool {
     // the slot's address, the same distance in every slot, so a device-side slot table needs no second table.
     // kind 0: all IQ2_XXS; 1: IQ2_XXS gate / up with IQ3_S down (column-sliced words); 2 / 3: all IQ2_XS / all IQ1_M (streams decoded
     // through the pool's codebooks). gate / down: raw bytes of a matrix, gate_copy / down_copy: bytes of its re-laid form.
-    // With REDHIP_TOPK_FAST_TILES (kinds 0, 2, 3) a third copy follows tile_off behind the slot's address: the three matrices tile-major
+    // With REDHIP_TOPK_FAST_TILES a third copy follows tile_off behind the slot's address: the three matrices tile-major
     // (as large as the second copy), as the prefill tile kernels read them; the batched form then runs on those kernels.
     struct FastShape {
         uint32_t word = 0, hidden = 0, ffn = 0, kind = 0;
@@ -381,7 +381,13 @@ bool enqueue_pairs_tiles(TopkPool *p, hipStream_t s, const std::vector<uint64_t>
     if (e == hipSuccess && p->fs.kind == 0u)
         e = launch_prefill_packed(nullptr, 256u, nullptr, tiles, nullptr, d_uid, d_start, d_pair_token, d_unique, tile_group, tile_pair0, tile_n, n_tiles,
                                   xh, xl, xexp, act_h, act_l, act_exp, tmp, nullptr, hidden, ffn, top_k, ntok, n_expert, s, false, false);
-    else if (e == hipSuccess) {      // IQ2_XS / IQ1_M: the same tile kernels on the tile-major streams, through the pool's codebooks
+    else if (e == hipSuccess && p->fs.kind == 1u) {      // IQ2_XXS gate / up tiles, then the IQ3_S down tiles
+        e = launch_prefill_gateup_tiled(tiles, 256u, d_uid, d_start, d_pair_token, d_unique, tile_group, tile_pair0, tile_n, n_tiles, xh, xl, xexp, nullptr, act_h, act_l,
+                                        act_exp, hidden, ffn, top_k, ntok, n_expert, s, false);
+        if (e == hipSuccess)
+            e = launch_prefill_down_iq3s(tiles + 2u * p->fs.gate_copy, 256u, d_uid, d_unique, tile_group, tile_pair0, tile_n, n_tiles, act_h, act_l, act_exp, tmp, hidden, ffn,
+                                         top_k, ntok, n_expert, s);
+    } else if (e == hipSuccess) {      // IQ2_XS / IQ1_M: the same tile kernels on the tile-major streams, through the pool's codebooks
         const uint32_t t = word_gate_up(p->fs.word);
         e = launch_prefill_streams(t, caller_grid_device(t), tiles, 256u, t, caller_grid_device(t), tiles + 2u * p->fs.gate_copy, 256u, d_uid, d_start, d_pair_token,
                                    d_unique, tile_group, tile_pair0, tile_n, n_tiles, xh, xl, xexp, act_h, act_l, act_exp, tmp, hidden, ffn, top_k, ntok, n_expert, s, false);
@@ -547,8 +553,8 @@ int redhip_topk_pool_enable_fast_path(redmetal_topk_pool_t handle, uint32_t ggml
                  "hidden in {512, 1024, 2048}; ffn a multiple of 256 up to 1024 (asked: type word 0x%x, hidden=%u, ffn=%u)", ggml_type, hidden_size, ffn_size);
         return 0;
     }
-    if ((flags & ~REDHIP_TOPK_FAST_TILES) || ((flags & REDHIP_TOPK_FAST_TILES) && (kind == 1u || ffn_size > 512u || hidden_size > 2048u))) {
-        TOPK_ERR("the top-k fast path keeps tile-major copies for all-IQ2_XXS, all-IQ2_XS and all-IQ1_M experts with hidden <= 2048 and ffn <= 512 only (asked: type word 0x%x, hidden=%u, ffn=%u, flags 0x%x)",
+    if ((flags & ~REDHIP_TOPK_FAST_TILES) || ((flags & REDHIP_TOPK_FAST_TILES) && (ffn_size > 512u || hidden_size > 2048u))) {
+        TOPK_ERR("the top-k fast path keeps tile-major copies for hidden <= 2048 and ffn <= 512 only (asked: type word 0x%x, hidden=%u, ffn=%u, flags 0x%x)",
                  ggml_type, hidden_size, ffn_size, flags);
         return 0;
     }
@@ -592,7 +598,7 @@ int redhip_topk_pool_enable_fast_path(redmetal_topk_pool_t handle, uint32_t ggml
         TOPK_ERR("top-k slot classes with the fast path's copies exceed the cache budget");
         return 0;
     }
-    if (!p->partial.reserve((size_t)kFastMaxTopK * (ffn_size / 32u) * hidden_size * sizeof(float)) || (f.tiles && !p->stage_down.reserve((size_t)f.down_copy))) {
+    if (!p->partial.reserve((size_t)kFastMaxTopK * (ffn_size / 32u) * hidden_size * sizeof(float)) || (f.tiles && kind != 1u && !p->stage_down.reserve((size_t)f.down_copy))) {
         TOPK_ERR("failed to allocate top-k activation buffers");
         return 0;
     }
@@ -682,12 +688,13 @@ int redmetal_topk_pool_load_expert(redmetal_topk_pool_t h, uint32_t slot_id,
                 e = f.kind == 0u   ? launch_repack_iq2xxs(base + 2u * f.gate, 0u, 1u, f.hidden, f.ffn, true, copy + 2u * f.gate_copy, 0u, nullptr)
                     : f.kind == 1u ? launch_repack_iq3s_words(base + 2u * f.gate, 0u, 1u, f.hidden, f.ffn, copy + 2u * f.gate_copy, 0u, nullptr, true)
                                    : launch_repack_gateup(dn, base + 2u * f.gate, 0u, 1u, f.hidden, f.ffn, copy + 2u * f.gate_copy, 0u, nullptr, true);
-            if (f.tiles) {      // (kinds 0, 2, 3: the row-major packed down matrix passes through a staging buffer)
+            if (f.tiles) {      // (kinds 0, 2, 3: the row-major packed down matrix passes through a staging buffer; IQ3_S tiles come from the raw rows)
                 if (e == hipSuccess) e = launch_tile_packed(copy, f.gate_copy, 2u, f.ffn, f.hidden, tiles, f.gate_copy, nullptr, gu == T_IQ2_XS);
-                if (e == hipSuccess)
+                if (e == hipSuccess && f.kind == 1u) e = launch_tile_iq3s(base + 2u * f.gate, 0u, 1u, f.hidden, f.ffn, tiles + 2u * f.gate_copy, 0u, nullptr);
+                else if (e == hipSuccess)
                     e = f.kind == 0u ? launch_repack_iq2xxs(base + 2u * f.gate, 0u, 1u, f.hidden, f.ffn, false, p->stage_down.p, 0u, nullptr)
                                      : launch_repack_gateup(dn, base + 2u * f.gate, 0u, 1u, f.hidden, f.ffn, p->stage_down.p, 0u, nullptr);
-                if (e == hipSuccess) e = launch_tile_packed(p->stage_down.p, 0u, 1u, f.hidden, f.ffn, tiles + 2u * f.gate_copy, 0u, nullptr, dn == T_IQ2_XS);
+                if (e == hipSuccess && f.kind != 1u) e = launch_tile_packed(p->stage_down.p, 0u, 1u, f.hidden, f.ffn, tiles + 2u * f.gate_copy, 0u, nullptr, dn == T_IQ2_XS);
             }
             if (e == hipSuccess) e = hipStreamSynchronize(nullptr);
             if (e != hipSuccess) { TOPK_ERR("top-k slot re-layout failed: %s", hipGetErrorString(e)); return 0; }

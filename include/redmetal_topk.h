@@ -175,7 +175,7 @@ int redmetal_topk_pool_encode_mapped(redmetal_topk_pool_t pool, void *stream,
  * slot class that holds such experts grows to about twice the expert's bytes - the raw bytes rounded up to 256, then the copy: 8 bytes
  * per 32 weights + 2 per 256 (IQ2_XS 9 per 32, IQ3_S down 16 per 32), the whole rounded up to 4096 - (a single-class pool's capacity shrinks accordingly; with
  * classes set, the call fails when they no longer fit). With the device-driven forms the slot table must hold addresses of this
- * pool's slots loaded with experts of the declared shape. flags: REDHIP_TOPK_FAST_TILES (all IQ2_XXS, all IQ2_XS or all IQ1_M; hidden_size <= 2048 and ffn_size <= 512)
+ * pool's slots loaded with experts of the declared shape. flags: REDHIP_TOPK_FAST_TILES (hidden_size <= 2048 and ffn_size <= 512)
  * adds a third copy per slot, tile-major as this library's prefill kernels read it (the slot class grows to three times the expert's
  * bytes); redmetal_topk_pool_encode_batched of that shape then runs on those kernels - tiles of up to 32 pairs per expert on the
  * matrix units - when every slot it names holds its copies; 0: none. Returns 1, or 0 with redmetal_topk_last_error(). */

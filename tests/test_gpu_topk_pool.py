@@ -265,7 +265,7 @@ def test_device_driven_forms(tmp_path, grids, layout, fast):
     c.pool.close()
 
 
-@pytest.mark.parametrize("layout,tiles", [("iq2", False), ("f2", False), ("xs", False), ("iq2", True), ("xs", True), ("m", True)])
+@pytest.mark.parametrize("layout,tiles", [("iq2", False), ("f2", False), ("xs", False), ("iq2", True), ("f2", True), ("xs", True), ("m", True)])
 def test_batched_and_mapped_pairs(tmp_path, grids, layout, tiles):
     """prefill form: pairs sorted by expert over a ragged routing (an expert with 19 pairs, experts with one, experts with none), tokens
     tok_first .. of a larger buffer; the same pairs on experts read in place from device copies of the whole tensors.
@@ -371,7 +371,7 @@ def test_fast_path_copies_follow_the_slots(tmp_path, grids):
     with pytest.raises(RedHipError, match="all-IQ2_XXS"):
         pool.enable_fast_path(17 | (29 << 8), H, F)
     with pytest.raises(RedHipError, match="tile-major copies"):
-        pool.enable_fast_path(16 | (21 << 8), H, F, tiles=True)
+        pool.enable_fast_path(16, 4096, F, tiles=True)
     with pytest.raises(RedHipError, match="all-IQ2_XXS"):
         pool.enable_fast_path(16, 768, F)
     pool.enable_fast_path(16, H, F)
@@ -382,7 +382,7 @@ def test_fast_path_copies_follow_the_slots(tmp_path, grids):
     pool.close()
 
 
-@pytest.mark.parametrize("layout", ["iq2", "xs"])
+@pytest.mark.parametrize("layout", ["iq2", "f2", "xs"])
 def test_batched_chunk_of_512_tokens_on_the_tile_copies(tmp_path, grids, layout):
     """a prefill chunk at the full expert shape (hidden 2048, ffn 512, ten of 48 experts per token, 512 tokens) through the batched form
     on the slots' tile-major copies: every 16th token against the CPU path, every token against the same call on a pool without copies
