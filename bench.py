@@ -15,7 +15,7 @@ Prints one JSON line (metric: microseconds per token for one MoE layer; lower is
   stack          48 layers back to back for one token (residual + RMS-norm around every layer), us per token and GB/s
   yardsticks     this machine's own streaming-read rate and fp16 matrix-core rate, measured in the same run
   topk_pool      the file-backed top-k pool (redmetal_topk_*) on a synthetic GGUF file: one token through a device slot table and a chunk of 512
-                 tokens, on raw slots and with the fast path's re-laid copies
+                 tokens, on raw slots and with the fast path's re-laid copies; all-IQ2_XXS experts, and all-IQ2_XS ones (`iq2_xs_experts`)
 The headline is timed as HIP graph replays (what a decode loop issues); the eager figure is printed beside it.
 """
 import argparse
@@ -224,6 +224,7 @@ def main():
     torch.cuda.init()
     B, NL = args.batch, args.layers
     K, W = args.steps, args.warmup
+    grids = None
     if args.layout in ("xs", "m") or "xs" in args.sweep_layouts.split(",") or "m" in args.sweep_layouts.split(","):
         # these two decode through codebooks the caller supplies: the reference's, from the fixture
         from dwarfstar_red_lite_amd import moe as moe_api
@@ -619,15 +620,15 @@ def main():
 
     # ---- the file-backed top-k pool (redmetal_topk_*), the surface the reference's engine binds: ten experts for one token through a device
     # slot table (encode_device_into) and a chunk of 512 tokens x top-10 (encode_batched), on raw GGUF slots and on a pool with the fast
-    # path's re-laid copies; 512 all-IQ2_XXS experts of the config shape read from a synthetic GGUF file ----
-    if args.layout == "iq2" and B == 1 and sweep and not args.no_pool:
+    # path's re-laid copies; 512 experts of the config shape read from a synthetic GGUF file: all IQ2_XXS, and (`iq2_xs_experts`) all IQ2_XS ----
+    def pool_entry(playout, word, codebooks):
         import tempfile
 
         from dwarfstar_red_lite_amd.gguf_writer import write_moe_gguf
         from dwarfstar_red_lite_amd.moe import gguf_expert_layout
         from dwarfstar_red_lite_amd.redmetal_topk import ExpertLayout, RedMetalTopKPool
         PE, PK, PT = 512, cfg["top_k"], 512
-        pcfg = synth.layer_config(hidden=H, ffn=F, n_expert=PE, top_k=PK, layout="iq2")
+        pcfg = synth.layer_config(hidden=H, ffn=F, n_expert=PE, top_k=PK, layout=playout)
         play = synth.make_layer(4242, pcfg)
         tmpd = tempfile.mkdtemp(prefix="redhip_pool_")
         gguf = os.path.join(tmpd, "pool.gguf")
@@ -638,7 +639,7 @@ def main():
             lays.append(ExpertLayout(d["gate_offset"], d["gate_bytes"], d["up_offset"], d["up_bytes"], d["down_offset"], d["down_bytes"]))
         payload = 2 * lays[0].gate_bytes + lays[0].down_bytes
         up_ = lambda v, a_: (v + a_ - 1) // a_ * a_
-        zero_xs, zero_m = np.zeros(512 * 8, np.int8), np.zeros(2048 * 8, np.int8)      # (codebooks of formats this file does not use)
+        cb_xs, cb_m = codebooks
         prng = np.random.default_rng(77)
         NLIST = 32
         lists = [prng.permutation(PE)[:PK] for _ in range(NLIST)]
@@ -652,10 +653,12 @@ def main():
                  "queued back to back, device time per call; raw = the pool as the reference defines it (raw GGUF bytes per slot), fast = "
                  "redhip_topk_pool_enable_fast_path with tile-major copies"}
         for mode in ("raw", "fast"):
-            phys = up_(2 * up_(payload, 256) + payload, 4096) if mode == "fast" else up_(payload, 4096)
-            pool = RedMetalTopKPool(gguf, (PE + 2) * phys, payload, slots_per_slab=64, iq2_xs_grid=zero_xs, iq1_m_grid=zero_m)
+            # (a slot of the fast pool: raw bytes, the re-laid copy - 8 bytes per 32 weights + 2 per 256, IQ2_XS 9 per 32 - and the tile-major one)
+            copy_b = 3 * (H * F // 32 * (9 if word == 17 else 8) + H * F // 256 * 2)
+            phys = up_(up_(payload, 256) + up_(copy_b, 256) + copy_b, 4096) if mode == "fast" else up_(payload, 4096)
+            pool = RedMetalTopKPool(gguf, (PE + 2) * phys, payload, slots_per_slab=64, iq2_xs_grid=cb_xs, iq1_m_grid=cb_m)
             if mode == "fast":
-                pool.enable_fast_path(16, H, F, tiles=True)
+                pool.enable_fast_path(word, H, F, tiles=True)
             for e in range(PE):
                 pool.load(e, lays[e])
             addr = [pool.addresses(e, lays[e])[0] for e in range(PE)]
@@ -666,11 +669,11 @@ def main():
 
             def run_lists(st):
                 for i in range(NLIST):
-                    pool.encode_device_into(st, tabs[i].data_ptr(), wdev[i].data_ptr(), PK, 16, H, F, gb, gb, px[i].data_ptr(), pouts[i].data_ptr())
+                    pool.encode_device_into(st, tabs[i].data_ptr(), wdev[i].data_ptr(), PK, word, H, F, gb, gb, px[i].data_ptr(), pouts[i].data_ptr())
             with torch.cuda.stream(stream):
                 run_lists(stream.cuda_stream)
                 stream.synchronize()
-                want = sum(float(w_) * orc.expert_ffn(16, 16, play["gate"][e], play["up"][e], play["down"][e], H, F, px[0].cpu().numpy())
+                want = sum(float(w_) * orc.expert_ffn(word, word, play["gate"][e], play["up"][e], play["down"][e], H, F, px[0].cpu().numpy())
                            for e, w_ in zip(lists[0], pw[0]))
                 prel = float(np.linalg.norm(pouts[0].cpu().numpy() - want) / np.linalg.norm(want))
                 if not prel <= 1e-3:
@@ -702,14 +705,14 @@ def main():
 
                 def run_chunk():
                     if not pool.lib.redmetal_topk_pool_encode_batched(pool.handle, stream.cuda_stream, ids_a.ctypes.data, gb_a.ctypes.data, ub_a.ctypes.data,
-                                                                      db_a.ctypes.data, ids_a.size, 16, H, F, 0, PT, PK, pt_a.size, pt_a.ctypes.data, pw_a.ctypes.data,
+                                                                      db_a.ctypes.data, ids_a.size, word, H, F, 0, PT, PK, pt_a.size, pt_a.ctypes.data, pw_a.ctypes.data,
                                                                       es_a.ctypes.data, tp_a.ctypes.data, px.data_ptr(), 0, bout.data_ptr(), 0):
                         raise SystemExit("encode_batched failed: " + pool._last_error())
                 for _ in range(2):
                     run_chunk()
                 stream.synchronize()
                 row = bout[5].cpu().numpy()
-                want_b = sum(float(w_) * orc.expert_ffn(16, 16, play["gate"][e], play["up"][e], play["down"][e], H, F, px[5].cpu().numpy())
+                want_b = sum(float(w_) * orc.expert_ffn(word, word, play["gate"][e], play["up"][e], play["down"][e], H, F, px[5].cpu().numpy())
                              for e, w_ in zip(bids[5], bw[5]))
                 brel = float(np.linalg.norm(row - want_b) / np.linalg.norm(want_b))
                 if not brel <= 1e-3:
@@ -735,7 +738,12 @@ def main():
             os.rmdir(tmpd)
         except OSError:
             pass
-        result["topk_pool"] = entry
+        return entry
+
+    if args.layout == "iq2" and B == 1 and sweep and not args.no_pool:
+        result["topk_pool"] = pool_entry("iq2", 16, (np.zeros(512 * 8, np.int8), np.zeros(2048 * 8, np.int8)))      # (codebooks of formats this file does not use)
+        if grids is not None:      # the same with IQ2_XS experts, the format of the reference's target file
+            result["topk_pool"]["iq2_xs_experts"] = pool_entry("xs", 17, grids)
 
     # ---- CPU baseline: the oracle on this host's cores, layer 0, same activations ----
     if not args.no_cpu:
