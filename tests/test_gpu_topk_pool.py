@@ -109,17 +109,18 @@ def test_execute_against_cpu_path(tmp_path, grids, layout, fast):
     c.pool.close()
 
 
-@pytest.mark.parametrize("layout,fast", [("f2", False), ("f2", True), ("xs", True), ("m", True)])
-def test_execute_full_shape_top10(tmp_path, grids, layout, fast):
-    """hidden 2048, ffn 512, ten experts of the mixed-precision layout (gate/up IQ2_XXS, down IQ3_S) and of the IQ2_XS / IQ1_M layouts;
-    fast: on the slots' re-laid copies"""
-    c = Case(tmp_path, grids, layout, hidden=2048, ffn=512, n_expert=12, fast=fast)
+@pytest.mark.parametrize("layout,fast,hidden", [("f2", False, 2048), ("f2", True, 2048), ("xs", True, 2048), ("m", True, 2048),
+                                                ("f2", True, 1024), ("xs", True, 1024), ("m", True, 1024)])
+def test_execute_full_shape_top10(tmp_path, grids, layout, fast, hidden):
+    """hidden 2048 (and 1024), ffn 512, ten experts of the mixed-precision layout (gate/up IQ2_XXS, down IQ3_S) and of the IQ2_XS / IQ1_M
+    layouts; fast: on the slots' re-laid copies"""
+    c = Case(tmp_path, grids, layout, hidden=hidden, ffn=512, n_expert=12, fast=fast)
     rng = np.random.default_rng(6)
     experts = rng.permutation(12)[:10]
     w = rng.random(10).astype(np.float32)
     w /= w.sum()
-    x = synth.normed_x(rng, 1, 2048)[0]
-    got, _ = c.pool.execute([c.slot_of[int(e)] for e in experts], [c.layouts[e] for e in experts], w, c.word, 2048, 512, 0, 2048, x)
+    x = synth.normed_x(rng, 1, hidden)[0]
+    got, _ = c.pool.execute([c.slot_of[int(e)] for e in experts], [c.layouts[e] for e in experts], w, c.word, hidden, 512, 0, hidden, x)
     assert rel_l2(got, c.want(experts, w, x)) <= REL_L2_TOL
     c.pool.close()
 
