@@ -322,20 +322,22 @@ __device__ __forceinline__ float q6k_dot32(const uint8_t *row, uint32_t chunk, c
 // A table in LDS holds, per expert, the set of tokens that selected it (a token selects an expert at most once): the
 // position of a pair inside its group and the group's size are bit counts of that set, the order of the groups a
 // bit count over the "first pair of its expert" flags, the group offsets one prefix sum. Run by a whole workgroup
-// of at least 256 threads (every thread reaches the barriers); at most 16 tokens, 256 pairs (one per lane of the first four waves), 1024 experts.
-constexpr uint32_t kGroupLdsWords = 1024u + 12u;
-constexpr uint32_t kGroupSmallPairs = 256u;
+// of at least 256 threads (every thread reaches the barriers); one pair per lane of the first four waves - 256 pairs - or, in a workgroup
+// of at least 512 threads, of the first eight - 512 pairs; at most 32 tokens (a token set is one word), 1024 experts.
+constexpr uint32_t kGroupLdsWords = 1024u + 24u;
+constexpr uint32_t kGroupSmallPairs = 256u, kGroupMaxPairs = 512u;
 // Optionally also the pass list of the batched expert-slice kernel (g.pass_list != nullptr): a pass = up to two consecutive pairs of one
-// group. Entry v: x = expert | pairs in the pass << 16 | position of its first pair << 24; y = four bytes: the (token * top_k + k) index
-// of its first and second pair, then their tokens. Passes follow the groups' order; *g.n_pass = their number.
+// group. Entry v: x = expert | pairs in the pass << 16; y = four bytes: the place k of the expert in the selection of its first and of
+// its second pair's token, then the two tokens. Passes follow the groups' order; *g.n_pass = their number.
 template <class PairId, class PairWeight>
 __device__ __forceinline__ void group_small(const GroupJob &g, uint32_t *lds, PairId pair_id, PairWeight pair_w) {
     uint32_t *token_set = lds;                           // per expert: bit t = token t selected it; later the group's offset (| its first pass << 16)
-    uint32_t *first_count = lds + 1024, *size_total = lds + 1028, *pass_total = lds + 1032;      // per wave of pairs (four)
+    uint32_t *first_count = lds + 1024, *size_total = lds + 1032, *pass_total = lds + 1040;      // per wave of pairs (four or eight)
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, K = g.top_k;
+    const uint32_t npw = blockDim.x >= 512u ? 8u : 4u;                                            // waves that hold pairs
     for (uint32_t i = tid; i < g.n_expert; i += blockDim.x) token_set[i] = 0u;
     __syncthreads();
-    const uint32_t P = g.ntok * K, pr = tid;             // pair index (waves 0..3)
+    const uint32_t P = g.ntok * K, pr = tid;             // pair index (waves 0 .. npw - 1)
     const bool live = pr < P;
     const uint32_t t = live ? pr / K : 0u;
     const uint32_t e = live ? guarded_id(pair_id(t, pr % K), g.n_expert, g.status) : 0u;
@@ -351,7 +353,7 @@ __device__ __forceinline__ void group_small(const GroupJob &g, uint32_t *lds, Pa
     uint32_t scan = first ? n : 0u;                      // inclusive prefix sum of the group sizes in pair order
     const uint32_t n_pass_mine = first ? (n + 1u) >> 1 : 0u;
     uint32_t pscan = n_pass_mine;                        // the same of the groups' pass counts
-    if (wave < 4u) {
+    if (wave < npw) {
 #pragma unroll
         for (int o = 1; o < 64; o <<= 1) {
             const uint32_t up = __shfl_up(scan, o, 64), pup = __shfl_up(pscan, o, 64);
@@ -364,17 +366,18 @@ __device__ __forceinline__ void group_small(const GroupJob &g, uint32_t *lds, Pa
     __syncthreads();
     uint32_t groups_before = 0u, size_before = 0u, pass_before = 0u;      // totals of the waves of pairs before this one
 #pragma unroll
-    for (uint32_t w = 0; w < 3u; ++w)
-        if (w < wave && wave < 4u) { groups_before += first_count[w]; size_before += size_total[w]; pass_before += pass_total[w]; }
+    for (uint32_t w = 0; w < 7u; ++w)
+        if (w < wave && wave < npw) { groups_before += first_count[w]; size_before += size_total[w]; pass_before += pass_total[w]; }
     const uint32_t grp = groups_before + __builtin_amdgcn_mbcnt_hi((uint32_t)(first_mask >> 32), __builtin_amdgcn_mbcnt_lo((uint32_t)first_mask, 0u));
     const uint32_t start = size_before + scan - (first ? n : 0u);
     const uint32_t pass0 = pass_before + pscan - n_pass_mine;
     if (first) { token_set[e] = start | (pass0 << 16); g.uid[grp] = e; g.expert_start[grp] = start; }
     if (tid == 0u) {
-        const uint32_t U = (first_count[0] + first_count[1]) + (first_count[2] + first_count[3]);
-        g.expert_start[U] = (size_total[0] + size_total[1]) + (size_total[2] + size_total[3]);      // = P unless a token repeated an expert
+        uint32_t U = 0u, placed = 0u, passes = 0u;
+        for (uint32_t w = 0; w < npw; ++w) { U += first_count[w]; placed += size_total[w]; passes += pass_total[w]; }
+        g.expert_start[U] = placed;                      // = P unless a token repeated an expert
         g.n_unique[0] = U;
-        if (g.n_pass) g.n_pass[0] = (pass_total[0] + pass_total[1]) + (pass_total[2] + pass_total[3]);
+        if (g.n_pass) g.n_pass[0] = passes;
     }
     __syncthreads();
     if (live) {
@@ -387,8 +390,8 @@ __device__ __forceinline__ void group_small(const GroupJob &g, uint32_t *lds, Pa
         if (g.pass_list && !dup) {
             const uint32_t v = (word >> 16) + (before >> 1), half = before & 1u;
             uint8_t *entry = reinterpret_cast<uint8_t *>(g.pass_list + v);
-            if (half == 0u) reinterpret_cast<uint32_t *>(entry)[0] = e | ((n - before >= 2u ? 2u : 1u) << 16) | (pos << 24);
-            entry[4u + half] = (uint8_t)pr;
+            if (half == 0u) reinterpret_cast<uint32_t *>(entry)[0] = e | ((n - before >= 2u ? 2u : 1u) << 16);
+            entry[4u + half] = (uint8_t)(pr % K);
             entry[6u + half] = (uint8_t)t;
         }
     }
@@ -1077,18 +1080,20 @@ hipError_t launch_select(const float *logits, uint32_t ntok, uint32_t n_expert, 
 }
 
 // Small batches routed by the layer's own router: wave t selects the experts of token t, then the whole workgroup sorts the pairs by
-// expert (with the pass list of the batched expert-slice kernel). One workgroup; logits [ntok][n_expert + 1].
+// expert (with the pass list of the batched expert-slice kernel). One workgroup; logits [ntok][n_expert + 1]; at most
+// kSelectGroupTokens tokens and kGroupMaxPairs pairs.
+constexpr uint32_t kSelectGroupTokens = 32u;
 __global__ __launch_bounds__(kWaves * 64) void select_group_kernel(const float *logits, uint32_t ntok, uint32_t E, uint32_t K, uint32_t *ids, float *weights,
                                                                    float *scalar, GroupJob job) {
-    __shared__ SelectOut sel[kWaves];
+    __shared__ SelectOut sel[kSelectGroupTokens];
     __shared__ uint32_t group_lds[kGroupLdsWords];
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63u;
-    if (wave < ntok) {
-        const float *l = logits + (uint64_t)wave * (E + 1u);
-        if (E <= 512u) wave_select_topk<8>(l, E, K, &sel[wave]); else wave_select_topk<16>(l, E, K, &sel[wave]);
+    for (uint32_t t = wave; t < ntok; t += (uint32_t)kWaves) {      // (more than sixteen tokens: a wave selects for two)
+        const float *l = logits + (uint64_t)t * (E + 1u);
+        if (E <= 512u) wave_select_topk<8>(l, E, K, &sel[t]); else wave_select_topk<16>(l, E, K, &sel[t]);
         wave_lds_sync();
-        if (lane < K) { ids[wave * K + lane] = sel[wave].ids[lane]; weights[wave * K + lane] = sel[wave].w[lane]; }
-        if (lane == 0u) scalar[wave] = sel[wave].scalar;
+        if (lane < K) { ids[t * K + lane] = sel[t].ids[lane]; weights[t * K + lane] = sel[t].w[lane]; }
+        if (lane == 0u) scalar[t] = sel[t].scalar;
     }
     __syncthreads();
     group_small(job, group_lds, [&](uint32_t t, uint32_t k) { return sel[t].ids[k]; }, [&](uint32_t t, uint32_t k) { return sel[t].w[k]; });
@@ -1096,7 +1101,7 @@ __global__ __launch_bounds__(kWaves * 64) void select_group_kernel(const float *
 
 hipError_t launch_select_group(const float *logits, uint32_t ntok, uint32_t n_expert, uint32_t top_k, uint32_t *ids, float *weights, float *scalar,
                                const GroupJob &job, hipStream_t s) {
-    if (!ntok || ntok > (uint32_t)kWaves || !n_expert || n_expert > 1024u || !top_k || top_k > 16u || top_k > n_expert || ntok * top_k > kGroupSmallPairs) return hipErrorInvalidValue;
+    if (!ntok || ntok > kSelectGroupTokens || !n_expert || n_expert > 1024u || !top_k || top_k > 16u || top_k > n_expert || ntok * top_k > kGroupMaxPairs) return hipErrorInvalidValue;
     GroupJob gj = job;
     gj.ids = nullptr;
     gj.weights = nullptr;
@@ -2196,7 +2201,7 @@ __global__ __launch_bounds__(kWaves * 64, 8) void batch_slice_kernel(const uint2
     }
     const uint32_t expert = e.x & 0xffffu, cnt = (e.x >> 16) & 255u, tok0 = (e.y >> 16) & 255u, tok1 = e.y >> 24;
     REDHIP_STAMP(1);                                   // the pass entry is here
-    const uint32_t k0 = sh ? K : (e.y & 255u) - tok0 * K, k1 = sh ? K : ((e.y >> 8) & 255u) - tok1 * K;
+    const uint32_t k0 = sh ? K : (e.y & 255u), k1 = sh ? K : ((e.y >> 8) & 255u);
     float *out0 = a.partial + ((uint64_t)(tok0 * (K + 1u) + k0) * FG + g) * H, *out1 = a.partial + ((uint64_t)(tok1 * (K + 1u) + k1) * FG + g) * H;
 
     if constexpr (MIX != 0) {
@@ -2458,7 +2463,7 @@ hipError_t launch_batch_slices(const void *experts, uint64_t stride, const void 
                                const void *pass_list, const uint32_t *n_pass, const float *weights, const float *scalar, const void *xh, const void *xl,
                                const int *xexp, float *partial, float *out, uint32_t hidden, uint32_t ffn, uint32_t top_k, uint32_t ntok, hipStream_t s,
                                const float *shared_gu, const float *shared_dense, uint32_t stream_type, const int8_t *grid) {
-    if (!fused_iq2_supported(hidden, ffn) || hidden % 32u || !ntok || ntok > 16u || ntok * top_k > kGroupSmallPairs || !pass_list || !n_pass) return hipErrorInvalidValue;
+    if (!fused_iq2_supported(hidden, ffn) || hidden % 32u || !ntok || ntok > kSelectGroupTokens || ntok * top_k > kGroupMaxPairs || !pass_list || !n_pass) return hipErrorInvalidValue;
     const bool mix = shared_gu != nullptr;
     if (mix ? !shared_dense : (!shared || !shared_down_cm)) return hipErrorInvalidValue;
     if (stream_type && ((stream_type != T_IQ2_XS && stream_type != T_IQ1_M) || !grid || !mix)) return hipErrorInvalidValue;

@@ -138,16 +138,18 @@ struct Moe {
     // ... whose down matrices are IQ2_XS / IQ1_M streams: a column-sliced copy beside the row-major one
     bool sliced_streams() const { return mixed_slices && dn_type != T_IQ3_S; }
     // batches that run as expert slices per pass: 2..8 tokens and at most 128 pairs on mixed layouts (their first launch multiplies the
-    // shared expert's gate | up rows for up to eight tokens), 2..16 tokens and at most 256 pairs on all-IQ2_XXS layers
-    static constexpr uint32_t kSmallMaxFused = 16u;
-    bool small_batch(uint32_t ntok) const {
+    // shared expert's gate | up rows for up to eight tokens), 2..16 tokens and at most 256 pairs on all-IQ2_XXS layers - 2..32 tokens and
+    // 512 pairs behind the layer's own router (own_router: the selection launch sorts that many; a caller's routing is sorted by one more
+    // workgroup of the launch that splits the activations, up to 256 pairs)
+    static constexpr uint32_t kSmallMaxFused = 16u, kSmallMaxRouted = 32u;
+    bool small_batch(uint32_t ntok, bool own_router = false) const {
         if (ntok < 2u || cfg.hidden / 512u > 4u) return false;
-        if (fused) return ntok <= kSmallMaxFused && ntok * cfg.top_k <= 256u;
+        if (fused) return ntok <= (own_router ? kSmallMaxRouted : kSmallMaxFused) && ntok * cfg.top_k <= (own_router ? 512u : 256u);
         return mixed_slices && ntok <= 8u && ntok * cfg.top_k <= 128u && ntok * (cfg.top_k + 1u) <= 144u;
     }
     // ... with the layer's own router: on a mixed layout two tokens are quicker on the single-token kernels (three launches, the selection
     // inside the gate/up kernel) than as slices behind a selection + pair sort launch of their own (four): 30.7 against 32.7 us
-    bool slices_after_router(uint32_t ntok) const { return small_batch(ntok) && (fused || ntok >= kGroupedMin); }
+    bool slices_after_router(uint32_t ntok) const { return small_batch(ntok, true) && (fused || ntok >= kGroupedMin); }
     // the same batches on a mixed layout run on the single-token kernels, one grid layer per token (tokens rarely share an
     // expert at these sizes, so reading a shared expert twice costs less than the pair sort and the per-pair kernels)
     bool small_batch_mixed(uint32_t ntok) const {
@@ -305,7 +307,7 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
             HIP_OK(launch_group_pairs(ids, weights, ntok, c.top_k, c.n_expert, m->uid, m->expert_start, m->pair_token, m->pair_weight,
                                       m->tok_pair, m->n_unique, s, tile_path ? &tl : nullptr, m->group_scratch_ptr()), "grouping launch");
         }
-        if (m->small_batch(ntok) && grouped && !select_here) {     // the caller's routing, sorted (with its pass list) by the prep launch: expert slices per pass
+        if (m->small_batch(ntok, true) && grouped && !select_here) {     // routing sorted (with its pass list) by the prep or the selection launch: expert slices per pass
             const Layer &L = m->layers[layer];
             HIP_OK(launch_batch_slices(L.packed, m->packed_stride, L.down_cm, m->down_cm_stride(), L.shared_packed, L.shared_down_cm, m->pass_list, m->n_pass,
                                        weights, m->scalar, m->xh, m->xl, m->xexp, m->partial, out, c.hidden, c.ffn, c.top_k, ntok, s), "batched expert slice launch");
@@ -544,9 +546,9 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
         }
     }
     const size_t T = c.max_tokens;
-    const size_t partial_tokens = m->fused ? Moe::kSmallMaxFused : 8u;      // the largest batch that runs as expert slices
+    const size_t partial_tokens = m->fused ? Moe::kSmallMaxRouted : 8u;      // the largest batch that runs as expert slices
     const size_t partial_bytes = m->fused || m->mixed_slices ? align256((size_t)(c.max_tokens < partial_tokens ? c.max_tokens : partial_tokens) * (c.top_k + 1u) * (c.ffn / 32u) * c.hidden * 4u) : 0u;
-    const size_t ws_bytes = partial_bytes + align256(8u * 256u) + align256(4u) + align256(4u) + align256(T * c.hidden * 4u) + align256(T * (c.n_expert + 1u) * 4u) + 2u * align256(T * c.top_k * 4u) + align256(T * 4u) +
+    const size_t ws_bytes = partial_bytes + align256(8u * 512u) + align256(4u) + align256(4u) + align256(T * c.hidden * 4u) + align256(T * (c.n_expert + 1u) * 4u) + 2u * align256(T * c.top_k * 4u) + align256(T * 4u) +
                             align256(T * c.top_k * c.ffn * 4u) + align256(T * c.ffn * 4u) +
                             2u * align256(2u * T * c.hidden) + align256(4u * T) + 2u * align256(2u * T * (c.top_k + 1u) * c.ffn) +
                             align256(4u * T * (c.top_k + 1u) * (c.ffn / 32u)) +
@@ -562,7 +564,7 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
     uint8_t *w = m->ws;
     m->status = reinterpret_cast<uint32_t *>(w); w += align256(4u);
     if (partial_bytes) { m->partial = reinterpret_cast<float *>(w); w += partial_bytes; }
-    m->pass_list = reinterpret_cast<uint2 *>(w); w += align256(8u * 256u);
+    m->pass_list = reinterpret_cast<uint2 *>(w); w += align256(8u * 512u);
     m->n_pass = reinterpret_cast<uint32_t *>(w); w += align256(4u);
     m->xn = reinterpret_cast<float *>(w); w += align256(T * c.hidden * 4u);
     m->logits = reinterpret_cast<float *>(w); w += align256(T * (c.n_expert + 1u) * 4u);

@@ -197,6 +197,30 @@ def test_drawn_routing_every_batch_size_class(layout, golden_dir):
     m.close()
 
 
+@pytest.mark.parametrize("shape,sizes", [((2048, 512, 512, 10), (17, 25, 32, 33)), ((1024, 256, 32, 8), (20, 32)), ((512, 256, 64, 16), (31, 32))])
+def test_batches_up_to_32_tokens_behind_the_own_router(shape, sizes):
+    """all-IQ2_XXS layers take up to 32 tokens (512 pairs) through forward() as one batch of expert slices: the selection launch sorts the
+    pairs and writes the pass list. Few experts: every expert serves many tokens (passes of two pairs); 64 experts x top-16: 512 pairs."""
+    from dwarfstar_red_lite_amd.moe import ResidentMoe
+    from test_gpu_moe_layer import ids_match_up_to_ties
+    H, F, E, K = shape
+    cfg = synth.layer_config(hidden=H, ffn=F, n_expert=E, top_k=K, layout="iq2")
+    lay = synth.make_layer(91, cfg)
+    m = ResidentMoe(cfg, n_layer=1, max_tokens=max(sizes))
+    m.load_layer(0, lay)
+    ref = orc.Layer(cfg, **lay)
+    rng = np.random.default_rng(92)
+    for ntok in sizes:
+        x = synth.normed_x(rng, ntok, H)
+        got = m.forward(0, torch.from_numpy(x).cuda()).cpu().numpy()
+        gids, gw, _ = m.last_route(ntok)
+        want, cids, cw, clog = ref.forward(x, threads=8)
+        assert all(ids_match_up_to_ties(gids[t], cids[t], clog[t]) for t in range(ntok)), (shape, ntok)
+        assert np.abs(gw - cw).max() <= 1e-5
+        assert max(rel_l2(got[t], want[t]) for t in range(ntok)) <= REL_L2_TOL, (shape, ntok)
+    m.close()
+
+
 @pytest.mark.parametrize("layout", ["iq2", "f2"])
 def test_prefill_chunk_forward_config_shape(layout):
     """A 24-token chunk at the benchmark shape through forward(): router (tiled, a Q6_K router through its f32 copy), selection, grouping,
