@@ -286,7 +286,7 @@ inline uint64_t packed_matrix_bytes(uint32_t type, uint32_t nrows, uint32_t K) {
 hipError_t launch_dequant_packed(uint32_t type, const void *packed, uint32_t nrows, uint32_t K, const int8_t *grid, float *out, hipStream_t s, bool col_major = false);
 hipError_t launch_dequant_packed_iq2xxs(const void *packed, uint32_t nrows, uint32_t K, bool col_major, float *out, hipStream_t s);
 
-// Pair sort of caller-given routing (at most 16 tokens, 128 pairs, 1024 experts) as a side job of another launch: one extra
+// Pair sort of caller-given routing (at most 16 tokens, 256 pairs, 1024 experts) as a side job of another launch: one extra
 // workgroup groups ids / weights [ntok][top_k] by expert while the others do the launch's own work. Outputs as launch_group_pairs.
 struct GroupJob {
     const uint32_t *ids;
@@ -380,7 +380,7 @@ hipError_t launch_slot_slices(const uint64_t *slot_table, uint64_t shadow_off, c
                               const int8_t *grid = nullptr);
 // (kind 1: the copies hold packed IQ2_XXS gate | up and column-sliced IQ3_S words; 2 / 3: row-major IQ2_XS / IQ1_M streams of gate | up,
 // column-sliced streams of down, decoded through the codebook `grid`; kinds 1..3: hidden <= 2048)
-// the same for 2..16 tokens (at most 128 pairs) whose pairs are grouped by expert: pass_list / n_pass from the pair sort (GroupJob), weights
+// the same for 2..32 tokens (at most 512 pairs) whose pairs are grouped by expert: pass_list / n_pass from the pair sort (GroupJob), weights
 // [ntok][top_k] and scalar [ntok] of the routing; partial [ntok][top_k + 1][ffn / 32][hidden]
 hipError_t launch_batch_slices(const void *experts, uint64_t stride, const void *down_cm, uint64_t down_stride, const void *shared, const void *shared_down_cm,
                                const void *pass_list, const uint32_t *n_pass, const float *weights, const float *scalar, const void *xh, const void *xl,
