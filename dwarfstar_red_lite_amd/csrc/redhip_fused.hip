@@ -1110,6 +1110,20 @@ hipError_t launch_select_group(const float *logits, uint32_t ntok, uint32_t n_ex
     return hipGetLastError();
 }
 
+// The pair sort of a caller's routing as a launch of its own, for batches beyond what the side job of another launch takes (17..32
+// tokens, up to 512 pairs): one workgroup of 16 waves.
+__global__ __launch_bounds__(kWaves * 64) void group_small_kernel(GroupJob job) {
+    __shared__ uint32_t group_lds[kGroupLdsWords];
+    group_small_given(job, group_lds);
+}
+
+hipError_t launch_group_small(const GroupJob &job, hipStream_t s) {
+    if (!job.ids || !job.weights || !job.ntok || job.ntok > kSelectGroupTokens || !job.top_k || job.top_k > 16u || job.ntok * job.top_k > kGroupMaxPairs ||
+        !job.n_expert || job.n_expert > 1024u) return hipErrorInvalidValue;
+    REDHIP_LAUNCH(group_small_kernel, dim3(1), dim3(kWaves * 64), 0, s, job);
+    return hipGetLastError();
+}
+
 // without a router (callers that bring their own routing): fp16 split of x and the scalar gate, one workgroup per token.
 // NV > 0: hidden = 256 * NV and a thread keeps its NV activations in registers, so x is read once and the two block-wide
 // reductions (largest |x|, gate_inp . x) share one barrier; NV == 0: any hidden, x read twice.

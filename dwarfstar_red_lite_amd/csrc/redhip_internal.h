@@ -300,6 +300,9 @@ struct GroupJob {
     uint32_t *n_pass = nullptr;      // their number
 };
 
+// the pair sort (and pass list) of a caller's routing as one launch: up to 32 tokens and 512 pairs
+hipError_t launch_group_small(const GroupJob &job, hipStream_t s);
+
 // Selection inside the batched gate/up kernel: logits [ntok][n_expert + 1] in, the routing out (ids, weights [ntok][top_k], scalar [ntok]);
 // the grouping arrays handed to the launcher are then outputs too.
 struct BatchSelect {

@@ -141,7 +141,7 @@ struct Moe {
     // shared expert's gate | up rows for up to eight tokens), 2..16 tokens and at most 256 pairs on all-IQ2_XXS layers - 2..32 tokens and
     // 512 pairs behind the layer's own router (own_router: the selection launch sorts that many; a caller's routing is sorted by one more
     // workgroup of the launch that splits the activations, up to 256 pairs)
-    static constexpr uint32_t kSmallMaxFused = 16u, kSmallMaxRouted = 32u;
+    static constexpr uint32_t kSmallMaxFused = 16u, kSmallMaxRouted = 32u, kSmallMaxGiven = 24u;
     bool small_batch(uint32_t ntok, bool own_router = false) const {
         if (ntok < 2u || cfg.hidden / 512u > 4u) return false;
         if (fused) return ntok <= (own_router ? kSmallMaxRouted : kSmallMaxFused) && ntok * cfg.top_k <= (own_router ? 512u : 256u);
@@ -880,6 +880,16 @@ int redhip_moe_experts(redhip_moe_t h, uint32_t layer, const float *x_dev, uint3
         } else {
             prof_set_stage(ST_OTHER);
             HIP_OK(launch_prep(x_dev, L.gate_inp, ntok, m->cfg.hidden, m->xh, m->xl, m->xexp, m->scalar, s, to_group ? &job : nullptr, &grouped), "prep launch");
+        }
+        if (m->fused && !grouped && !m->small_batch(ntok) && m->small_batch(ntok, true) && ntok <= Moe::kSmallMaxGiven) {
+            // 17..24 tokens on an all-IQ2_XXS layer: more pairs than the side job above sorts; one more launch sorts them with their pass list.
+            // (The slices cost a pass per two pairs of an expert, the tile kernels a decode per distinct expert: with 32 hot experts the
+            // slices took 58.5 / 74.2 / 93.2 us at 17 / 24 / 32 tokens against 67.9 / 79.2 / 84.5 us on the tiles.)
+            const GroupJob big{ids_dev, weights_dev, ntok, m->cfg.top_k, m->cfg.n_expert, m->uid, m->expert_start, m->pair_token, m->pair_weight, m->tok_pair, m->n_unique,
+                               m->status, m->pass_list, m->n_pass};
+            prof_set_stage(ST_GROUP);
+            HIP_OK(launch_group_small(big, s), "pair sort launch");
+            grouped = true;
         }
         const int ok = experts_enqueue(m, layer, x_dev, ntok, ids_dev, weights_dev, out_dev, s, false, grouped);
         m->shared_gu_ready = false;

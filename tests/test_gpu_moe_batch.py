@@ -199,8 +199,9 @@ def test_drawn_routing_every_batch_size_class(layout, golden_dir):
 
 @pytest.mark.parametrize("shape,sizes", [((2048, 512, 512, 10), (17, 25, 32, 33)), ((1024, 256, 32, 8), (20, 32)), ((512, 256, 64, 16), (31, 32))])
 def test_batches_up_to_32_tokens_behind_the_own_router(shape, sizes):
-    """all-IQ2_XXS layers take up to 32 tokens (512 pairs) through forward() as one batch of expert slices: the selection launch sorts the
-    pairs and writes the pass list. Few experts: every expert serves many tokens (passes of two pairs); 64 experts x top-16: 512 pairs."""
+    """all-IQ2_XXS layers take up to 32 tokens (512 pairs) as one batch of expert slices: through forward() the selection launch sorts the
+    pairs and writes the pass list, with the routing given a launch of its own does. Few experts: every expert serves many tokens
+    (passes of two pairs); 64 experts x top-16: 512 pairs."""
     from dwarfstar_red_lite_amd.moe import ResidentMoe
     from test_gpu_moe_layer import ids_match_up_to_ties
     H, F, E, K = shape
@@ -218,6 +219,14 @@ def test_batches_up_to_32_tokens_behind_the_own_router(shape, sizes):
         assert all(ids_match_up_to_ties(gids[t], cids[t], clog[t]) for t in range(ntok)), (shape, ntok)
         assert np.abs(gw - cw).max() <= 1e-5
         assert max(rel_l2(got[t], want[t]) for t in range(ntok)) <= REL_L2_TOL, (shape, ntok)
+        # the same sizes with the routing given: every token picks among `hot` experts, so an expert serves many tokens of the batch
+        hot = min(E, 3 * K)
+        ids = np.stack([rng.permutation(hot)[:K] for _ in range(ntok)]).astype(np.uint32)
+        w = rng.random((ntok, K)).astype(np.float32) + 0.05
+        w /= w.sum(axis=1, keepdims=True)
+        got = m.experts(0, torch.from_numpy(x).cuda(), torch.from_numpy(ids.astype(np.int32)).cuda(), torch.from_numpy(w).cuda()).cpu().numpy()
+        want = oracle_tokens(cfg, lay, x, ids, w)
+        assert max(rel_l2(got[t], want[t]) for t in range(ntok)) <= REL_L2_TOL, (shape, ntok, "given")
     m.close()
 
 
