@@ -141,10 +141,13 @@ struct Moe {
     // shared expert's gate | up rows for up to eight tokens), 2..16 tokens and at most 256 pairs on all-IQ2_XXS layers - 2..32 tokens and
     // 512 pairs behind the layer's own router (own_router: the selection launch sorts that many; a caller's routing is sorted by one more
     // workgroup of the launch that splits the activations, up to 256 pairs)
-    static constexpr uint32_t kSmallMaxFused = 16u, kSmallMaxRouted = 32u, kSmallMaxGiven = 24u;
+    static constexpr uint32_t kSmallMaxFused = 16u, kSmallMaxRouted = 32u, kSmallMaxGiven = 24u, kSmallMaxMixed = 32u;
+    bool dense_routed = false;               // every layer has f32 copies of its router and of the shared expert's gate | up rows (set at creation)
     bool small_batch(uint32_t ntok, bool own_router = false) const {
         if (ntok < 2u || cfg.hidden / 512u > 4u) return false;
         if (fused) return ntok <= (own_router ? kSmallMaxRouted : kSmallMaxFused) && ntok * cfg.top_k <= (own_router ? 512u : 256u);
+        // (mixed layouts behind their own router: the router launch is repeated per eight tokens, the selection launch sorts up to 512 pairs)
+        if (own_router && ntok > 8u) return mixed_slices && dense_routed && ntok <= kSmallMaxMixed && ntok * cfg.top_k <= 512u;
         return mixed_slices && ntok <= 8u && ntok * cfg.top_k <= 128u && ntok * (cfg.top_k + 1u) <= 144u;
     }
     // ... with the layer's own router: on a mixed layout two tokens are quicker on the single-token kernels (three launches, the selection
@@ -179,7 +182,7 @@ struct Moe {
     // So does every layout from 9 to 16 tokens: two small batches are quicker than one chunk, whose tile kernels leave most workgroups
     // without work at that size.
     bool sliced(uint32_t ntok) const {
-        if (ntok <= kSlice || small_batch(ntok)) return false;      // (all-IQ2_XXS layers take up to 16 tokens as one small batch)
+        if (ntok <= kSlice || small_batch(ntok, true)) return false;      // (one small batch: up to 32 tokens behind the layer's own router)
         if (ntok <= 2u * kSlice && (small_batch(kSlice) || grouped_mixed(kSlice))) return true;
         return mixed && !tiles_resident() && !stream_chunk(ntok) && grouped_mixed(kSlice);
     }
@@ -264,7 +267,7 @@ int experts_enqueue(Moe *m, uint32_t layer, const float *x, uint32_t ntok, const
     // select_here && grouped: selection and pair sort both happen inside the batched gate/up kernel, from m->logits
     const BatchSelect bsel{m->logits, c.n_expert, m->ids, m->weights, m->scalar};
     const BatchSelect *in_batch = select_here && grouped ? &bsel : nullptr;
-    if (m->mixed_slices && m->small_batch(ntok) && grouped) {     // pairs sorted (with their pass list) by the launch before; the shared gate | up products are in m->act
+    if (m->mixed_slices && m->small_batch(ntok, true) && grouped) {     // pairs sorted (with their pass list) by the launch before; the shared gate | up products are in m->act
         if (select_here || !m->shared_gu_ready) { moe_err("internal: a small batch reached the expert slices without its routing or the shared expert's products"); return 0; }
         const Layer &L = m->layers[layer];
         HIP_OK(launch_batch_slices(L.packed, m->packed_stride, L.down_cm, m->down_cm_stride(), nullptr, nullptr, m->pass_list, m->n_pass, weights, m->scalar,
@@ -482,6 +485,7 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
         // (a handle for one token at a time needs no second copy of IQ2_XS / IQ1_M down streams: only the slices read the column-sliced one)
         m->mixed_slices = m->mixed && ((gu == T_IQ2_XXS && dn == T_IQ3_S) || (gu_codebook && dn == gu && sgu == T_Q6_K)) && c.ffn <= 512u &&
                           c.hidden / 512u <= 4u && (nv == 2u || nv == 4u || nv == 8u || nv == 16u);
+        m->dense_routed = m->mixed_slices;      // (every mixed layer gets f32 copies of its shared expert, and of its router unless that is f32 already)
     }
     m->pk_gate_bytes = packed_matrix_bytes(gu, c.ffn, c.hidden);
     m->packed_stride = m->fused && m->rowmajor_down() ? m->expert_stride : align256(2u * m->pk_gate_bytes);
@@ -546,7 +550,7 @@ redhip_moe_t redhip_moe_create(const redhip_moe_config *cfg) {
         }
     }
     const size_t T = c.max_tokens;
-    const size_t partial_tokens = m->fused ? Moe::kSmallMaxRouted : 8u;      // the largest batch that runs as expert slices
+    const size_t partial_tokens = m->fused ? Moe::kSmallMaxRouted : Moe::kSmallMaxMixed;      // the largest batch that runs as expert slices
     const size_t partial_bytes = m->fused || m->mixed_slices ? align256((size_t)(c.max_tokens < partial_tokens ? c.max_tokens : partial_tokens) * (c.top_k + 1u) * (c.ffn / 32u) * c.hidden * 4u) : 0u;
     const size_t ws_bytes = partial_bytes + align256(8u * 512u) + align256(4u) + align256(4u) + align256(T * c.hidden * 4u) + align256(T * (c.n_expert + 1u) * 4u) + 2u * align256(T * c.top_k * 4u) + align256(T * 4u) +
                             align256(T * c.top_k * c.ffn * 4u) + align256(T * c.ffn * 4u) +
@@ -814,7 +818,25 @@ int redhip_moe_route(redhip_moe_t h, uint32_t layer, const float *x_dev, uint32_
                                  (nv == 2u || nv == 4u || nv == 8u || nv == 16u);
         m->shared_gu_ready = dense_small ||
                              (m->mixed && m->sh_gu_type == T_Q6_K && c.router_type == T_Q6_K && (ntok == 1u || m->small_batch_mixed(ntok)) && c.top_k >= 2u);
-        if (m->tiled_router(ntok))
+        const bool dense_multi = !dense_small && m->mixed && ntok > 8u && m->small_batch(ntok, true) && router_f32 && m->layers[layer].dense_gu;
+        if (dense_multi) {
+            // 9..32 tokens on a mixed layout whose batches run as slices: the launch of the eight-token batches once per eight tokens, each
+            // on its own rows of the activations, logits, fp16 halves and shared products (a block step: of the branch and the normalised rows too)
+            BlockContext &bc = block_context();
+            const BlockContext saved = bc;
+            for (uint32_t t0 = 0; t0 < ntok; t0 += 8u) {
+                const uint32_t n = ntok - t0 < 8u ? ntok - t0 : 8u;
+                const size_t row = (size_t)t0 * c.hidden;
+                if (saved.branch) { bc.branch = saved.branch + row; bc.xn_out = saved.xn_out + row; }
+                const hipError_t e = launch_router_gemv(T_F32, router_f32, x_dev + row, m->layers[layer].gate_inp, n, c.hidden, c.n_expert,
+                                                        m->logits + (size_t)t0 * (c.n_expert + 1u), static_cast<uint8_t *>(m->xh) + 2u * row,
+                                                        static_cast<uint8_t *>(m->xl) + 2u * row, m->xexp + t0, nullptr, m->act + (size_t)t0 * 2u * c.ffn, c.ffn, s,
+                                                        m->layers[layer].dense_gu);
+                if (e != hipSuccess) { bc = saved; HIP_OK(e, "router launch"); }
+            }
+            bc = saved;
+            m->shared_gu_ready = true;
+        } else if (m->tiled_router(ntok))
             HIP_OK(launch_router_f32_tiles(router_f32, m->layers[layer].gate_inp, x_dev, ntok, c.hidden,
                                            c.n_expert, m->logits, m->xh, m->xl, m->xexp, s), "router tile launch");
         else if (dense_small)

@@ -230,6 +230,40 @@ def test_batches_up_to_32_tokens_behind_the_own_router(shape, sizes):
     m.close()
 
 
+@pytest.mark.parametrize("layout", ["f2", "xs", "m"])
+@pytest.mark.parametrize("shape,sizes", [((2048, 512, 512, 10), (9, 17, 25, 32, 33)), ((1024, 256, 32, 8), (16, 31))])
+def test_mixed_layout_batches_up_to_32_tokens_behind_the_own_router(layout, shape, sizes, golden_dir):
+    """the mixed layouts whose small batches run as expert slices take 9..32 tokens through forward() as one batch: the router launch of the
+    eight-token batches once per eight tokens, one selection + pair sort launch, slices per pass"""
+    import json
+    import os
+    from dwarfstar_red_lite_amd import moe as moe_api
+    from dwarfstar_red_lite_amd.moe import ResidentMoe
+    from test_gpu_moe_layer import ids_match_up_to_ties
+    if layout in ("xs", "m"):
+        g = json.load(open(os.path.join(golden_dir, "iq_grids.json")))
+        grids = [np.frombuffer(bytes.fromhex(g[k]), np.int8) for k in ("iq2_xs", "iq1_m")]
+        moe_api.set_codebooks(*grids)
+        orc.set_codebooks(*grids)
+    H, F, E, K = shape
+    cfg = synth.layer_config(hidden=H, ffn=F, n_expert=E, top_k=K, layout=layout)
+    lay = synth.make_layer(93, cfg)
+    m = ResidentMoe(cfg, n_layer=1, max_tokens=max(sizes))
+    m.load_layer(0, lay)
+    ref = orc.Layer(cfg, **lay)
+    rng = np.random.default_rng(94)
+    for ntok in sizes:
+        x = synth.normed_x(rng, ntok, H)
+        got = m.forward(0, torch.from_numpy(x).cuda()).cpu().numpy()
+        gids, gw, _ = m.last_route(ntok)
+        want, cids, cw, clog = ref.forward(x, threads=8)
+        assert all(ids_match_up_to_ties(gids[t], cids[t], clog[t]) for t in range(ntok)), (layout, shape, ntok)
+        agree = [t for t in range(ntok) if np.array_equal(gids[t], cids[t])]
+        assert len(agree) >= ntok - 1
+        assert max(rel_l2(got[t], want[t]) for t in agree) <= REL_L2_TOL, (layout, shape, ntok)
+    m.close()
+
+
 @pytest.mark.parametrize("layout", ["iq2", "f2"])
 def test_prefill_chunk_forward_config_shape(layout):
     """A 24-token chunk at the benchmark shape through forward(): router (tiled, a Q6_K router through its f32 copy), selection, grouping,
