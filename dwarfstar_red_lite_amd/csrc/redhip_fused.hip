@@ -334,7 +334,7 @@ __device__ __forceinline__ void group_small(const GroupJob &g, uint32_t *lds, Pa
     uint32_t *token_set = lds;                           // per expert: bit t = token t selected it; later the group's offset (| its first pass << 16)
     uint32_t *first_count = lds + 1024, *size_total = lds + 1032, *pass_total = lds + 1040;      // per wave of pairs (four or eight)
     const uint32_t tid = threadIdx.x, wave = tid >> 6, lane = tid & 63u, K = g.top_k;
-    const uint32_t npw = blockDim.x >= 512u ? 8u : 4u;                                            // waves that hold pairs
+    const uint32_t npw = g.ntok * K > kGroupSmallPairs && blockDim.x >= 512u ? 8u : 4u;          // waves that hold pairs
     for (uint32_t i = tid; i < g.n_expert; i += blockDim.x) token_set[i] = 0u;
     __syncthreads();
     const uint32_t P = g.ntok * K, pr = tid;             // pair index (waves 0 .. npw - 1)
@@ -1083,9 +1083,10 @@ hipError_t launch_select(const float *logits, uint32_t ntok, uint32_t n_expert, 
 // expert (with the pass list of the batched expert-slice kernel). One workgroup; logits [ntok][n_expert + 1]; at most
 // kSelectGroupTokens tokens and kGroupMaxPairs pairs.
 constexpr uint32_t kSelectGroupTokens = 32u;
+template <uint32_t TOK>      // tokens the workgroup has room for: 16 (a wave each) or kSelectGroupTokens
 __global__ __launch_bounds__(kWaves * 64) void select_group_kernel(const float *logits, uint32_t ntok, uint32_t E, uint32_t K, uint32_t *ids, float *weights,
                                                                    float *scalar, GroupJob job) {
-    __shared__ SelectOut sel[kSelectGroupTokens];
+    __shared__ SelectOut sel[TOK];
     __shared__ uint32_t group_lds[kGroupLdsWords];
     const uint32_t wave = threadIdx.x >> 6, lane = threadIdx.x & 63u;
     for (uint32_t t = wave; t < ntok; t += (uint32_t)kWaves) {      // (more than sixteen tokens: a wave selects for two)
@@ -1106,7 +1107,8 @@ hipError_t launch_select_group(const float *logits, uint32_t ntok, uint32_t n_ex
     gj.ids = nullptr;
     gj.weights = nullptr;
     gj.ntok = ntok; gj.top_k = top_k; gj.n_expert = n_expert;
-    REDHIP_LAUNCH(select_group_kernel, dim3(1), dim3(kWaves * 64), 0, s, logits, ntok, n_expert, top_k, ids, weights, scalar, gj);
+    if (ntok <= (uint32_t)kWaves) REDHIP_LAUNCH(select_group_kernel<kWaves>, dim3(1), dim3(kWaves * 64), 0, s, logits, ntok, n_expert, top_k, ids, weights, scalar, gj);
+    else REDHIP_LAUNCH(select_group_kernel<kSelectGroupTokens>, dim3(1), dim3(kWaves * 64), 0, s, logits, ntok, n_expert, top_k, ids, weights, scalar, gj);
     return hipGetLastError();
 }
 
