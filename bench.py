@@ -12,6 +12,7 @@ Prints one JSON line (metric: microseconds per token for one MoE layer; lower is
   batch_sweep    the ragged small batches (B = 2, 4, 8): drawn hot routing as an input, and the layer's own router
   <layout>_sweep the same on the mixed-precision layout and the two layouts with the expert formats of the reference's target file
   prefill_sweep  chunks of 512 / 2048 tokens on the MFMA tile kernels: TFLOP/s against the fp16 matrix-core peak and the HBM cap
+  mid_sweep      12 .. 48 tokens through the layer's own router (iq2; f2 at 16 and 32), between the small batches and the chunks
   stack          48 layers back to back for one token (residual + RMS-norm around every layer), us per token and GB/s
   yardsticks     this machine's own streaming-read rate and fp16 matrix-core rate, measured in the same run
   topk_pool      the file-backed top-k pool (redmetal_topk_*) on a synthetic GGUF file: one token through a device slot table and a chunk of 512
@@ -522,6 +523,8 @@ def main():
         pre.append(chunk_entry(ctx, 512, "router"))
         pre.append(chunk_entry(ctx, 512, "zipf"))
         pre.append(chunk_entry(ctx, 2048, "router"))
+        # between the small batches and the chunks: 12 .. 32 tokens through the layer's own router (one batch of expert slices), 48 on the tiles
+        mid = [dict(sweep_entry(ctx, b, "router"), layout="iq2") for b in (12, 16, 24, 32, 48)]
         ctx["moe"].close()
         del ctx
         torch.cuda.empty_cache()
@@ -529,10 +532,12 @@ def main():
         pre.append(chunk_entry(ctx, 512, "zipf"))
         pre.append(chunk_entry(ctx, 512, "router"))
         pre.append(chunk_entry(ctx, 2048, "zipf"))
+        mid += [dict(sweep_entry(ctx, b, "router"), layout="f2") for b in (16, 32)]
         ctx["moe"].close()
         del ctx
         torch.cuda.empty_cache()
         result["prefill_sweep"] = pre
+        result["mid_sweep"] = mid
 
     # ---- this machine's own yardsticks, in the same run: streaming read of 1 GiB (four times the 256 MB last-level cache) and a dense fp16
     # matrix-core loop on register operands ----

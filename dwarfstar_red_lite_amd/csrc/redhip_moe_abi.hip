@@ -76,7 +76,8 @@ struct Moe {
     // every path of an all-IQ2_XXS handle of these shapes reads the packed copies: the raw GGUF rows of the routed experts only pass
     // through a staging buffer at upload
     // So do the mixed layouts whose batches run as expert slices, when every size they can be given has kernels on the packed copies:
-    // one token (packed gate | up, word- or stream-packed down), 2..8 tokens (slices), 9..16 (two small batches), larger chunks only
+    // one token (packed gate | up, word- or stream-packed down), 2..8 tokens (slices), 9..16 (slices behind the own router, two small
+    // batches or tiles with a caller's routing), larger chunks only
     // with the tile-major copies (a handle made for more than 16 tokens on a shape without tile kernels keeps the raw rows for the
     // raw-row kernels). Any kernel that would read raw rows on such a handle is refused on the host (raw_rows below).
     bool keep_raw() const {
