@@ -511,7 +511,7 @@ __global__ __launch_bounds__(NWV * 64) void router_f32_multi_kernel(const float 
     // (the leading arguments repeat a.x, a.gate_inp, a.sh_dense, a.hidden, a.n_expert, a.ffn; n_blocks = the workgroups that multiply rows:
     // leading scalar arguments can reach a wave in registers at its start, so the requests for its row and the activations leave at once)
     extern __shared__ __attribute__((aligned(16))) float xs_all[];      // [ntok][hidden]
-    __shared__ float s_amax[8];
+    __shared__ float s_amax[16];
     if (blockIdx.x == n_blocks) {                        // the extra workgroup: pair sort of the caller's routing
         group_small_given(job, reinterpret_cast<uint32_t *>(xs_all));
         return;
@@ -683,7 +683,7 @@ hipError_t launch_router_gemv(uint32_t router_type, const void *w, const float *
     const bool with_shared = sh_q6k && sh_gu && router_type == T_Q6_K && ntok <= 8u && ffn % 4u == 0u;      // sh_gu: [ntok][2 * ffn]
     const BlockContext &bc = block_context();
     if (bc.branch && (!bc.norm_w || !bc.xn_out)) return hipErrorInvalidValue;
-    const bool with_dense = sh_dense && sh_gu && router_type == T_F32 && ntok <= 8u;      // sh_gu: [ntok][2 * ffn]
+    const bool with_dense = sh_dense && sh_gu && router_type == T_F32 && ntok <= 16u;      // sh_gu: [ntok][2 * ffn]
     if (job_done) *job_done = false;
     RouterArgs a{x, gate_inp, logits, static_cast<_Float16 *>(xh), static_cast<_Float16 *>(xl), xexp, hidden, n_expert,
                  with_shared ? static_cast<const uint8_t *>(sh_q6k) : nullptr, with_dense ? sh_dense : nullptr, sh_gu, ffn, bc.branch, bc.norm_w, bc.eps,
@@ -694,19 +694,19 @@ hipError_t launch_router_gemv(uint32_t router_type, const void *w, const float *
     const dim3 grid8((grid.x + 7u) & ~7u, ntok);
     // with the shared expert's rows behind the router's (1537 rows at the benchmark shape) a row is read once for the whole batch; the
     // router's own 513 rows are quicker one token per grid layer (their re-reads hit the L2)
-    if (router_type == T_F32 && with_dense && ntok >= 2u && (size_t)ntok * hidden * 4u <= 64u * 1024u) {
+    if (router_type == T_F32 && with_dense && ntok >= 2u && (size_t)ntok * hidden * 4u <= 128u * 1024u) {
         const float *wf = static_cast<const float *>(w);
         const bool with_job = job && job_done && group_job_fits(*job);
         const dim3 mgrid((n_expert + 1u + 2u * ffn + 7u) / 8u + (with_job ? 1u : 0u));
         size_t lds = (size_t)ntok * hidden * 4u;
         if (with_job && lds < kGroupLdsWords * 4u) lds = kGroupLdsWords * 4u;
         const GroupJob gj = with_job ? *job : GroupJob{};
-        // (64 KB of activations at 8 tokens of 2048, beside a few static bytes: the limit is raised explicitly)
+        // (64 KB of activations at 8 tokens of 2048, 128 KB at 16, beside a few static bytes: the limit is raised explicitly)
 #define REDHIP_RMULTI(NV)                                                                                                                                  \
     do {                                                                                                                                                   \
         static bool attr = false;                                                                                                                           \
         if (!attr) {                                                                                                                                        \
-            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(router_f32_multi_kernel<NV, 8>), hipFuncAttributeMaxDynamicSharedMemorySize, 72 * 1024); \
+            hipError_t e = hipFuncSetAttribute(reinterpret_cast<const void *>(router_f32_multi_kernel<NV, 8>), hipFuncAttributeMaxDynamicSharedMemorySize, 136 * 1024); \
             if (e != hipSuccess) return e;                                                                                                                  \
             attr = true;                                                                                                                                    \
         }                                                                                                                                                   \

@@ -821,12 +821,13 @@ int redhip_moe_route(redhip_moe_t h, uint32_t layer, const float *x_dev, uint32_
                              (m->mixed && m->sh_gu_type == T_Q6_K && c.router_type == T_Q6_K && (ntok == 1u || m->small_batch_mixed(ntok)) && c.top_k >= 2u);
         const bool dense_multi = !dense_small && m->mixed && ntok > 8u && m->small_batch(ntok, true) && router_f32 && m->layers[layer].dense_gu;
         if (dense_multi) {
-            // 9..32 tokens on a mixed layout whose batches run as slices: the launch of the eight-token batches once per eight tokens, each
+            // 9..32 tokens on a mixed layout whose batches run as slices: the launch of the small batches once per sixteen tokens, each
             // on its own rows of the activations, logits, fp16 halves and shared products (a block step: of the branch and the normalised rows too)
             BlockContext &bc = block_context();
             const BlockContext saved = bc;
-            for (uint32_t t0 = 0; t0 < ntok; t0 += 8u) {
-                const uint32_t n = ntok - t0 < 8u ? ntok - t0 : 8u;
+            const uint32_t per = (size_t)16u * c.hidden * 4u <= 128u * 1024u ? 16u : 8u;      // tokens whose activations fit the launch's LDS
+            for (uint32_t t0 = 0; t0 < ntok; t0 += per) {
+                const uint32_t n = ntok - t0 < per ? ntok - t0 : per;
                 const size_t row = (size_t)t0 * c.hidden;
                 if (saved.branch) { bc.branch = saved.branch + row; bc.xn_out = saved.xn_out + row; }
                 const hipError_t e = launch_router_gemv(T_F32, router_f32, x_dev + row, m->layers[layer].gate_inp, n, c.hidden, c.n_expert,
