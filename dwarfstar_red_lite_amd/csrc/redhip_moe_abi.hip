@@ -147,7 +147,7 @@ struct Moe {
     bool small_batch(uint32_t ntok, bool own_router = false) const {
         if (ntok < 2u || cfg.hidden / 512u > 4u) return false;
         if (fused) return ntok <= (own_router ? kSmallMaxRouted : kSmallMaxFused) && ntok * cfg.top_k <= (own_router ? 512u : 256u);
-        // (mixed layouts behind their own router: the router launch is repeated per eight tokens, the selection launch sorts up to 512 pairs)
+        // (mixed layouts behind their own router: the router launch is repeated per sixteen tokens, the selection launch sorts up to 512 pairs)
         if (own_router && ntok > 8u) return mixed_slices && dense_routed && ntok <= kSmallMaxMixed && ntok * cfg.top_k <= 512u;
         return mixed_slices && ntok <= 8u && ntok * cfg.top_k <= 128u && ntok * (cfg.top_k + 1u) <= 144u;
     }
