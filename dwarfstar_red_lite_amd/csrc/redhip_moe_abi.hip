@@ -894,7 +894,26 @@ int redhip_moe_experts(redhip_moe_t h, uint32_t layer, const float *x_dev, uint3
         const GroupJob job{ids_dev, weights_dev, ntok, m->cfg.top_k, m->cfg.n_expert, m->uid, m->expert_start, m->pair_token, m->pair_weight, m->tok_pair, m->n_unique, m->status,
                            m->small_batch(ntok) ? m->pass_list : nullptr, m->small_batch(ntok) ? m->n_pass : nullptr};
         bool grouped = false;
-        if (m->mixed && m->packed_gu() && (ntok == 1u || m->small_batch_mixed(ntok)) && L.dense_gu && (nv == 2u || nv == 4u || nv == 8u || nv == 16u)) {
+        const bool mixed_mid = m->mixed_slices && ntok > 8u && ntok <= Moe::kSmallMaxGiven && m->small_batch(ntok, true) && L.dense_gu;
+        if (mixed_mid) {
+            // 9..24 tokens on a mixed layout whose batches run as slices: the shared expert's products, the fp16 halves and the scalar gates
+            // from the launch of the small batches, once per sixteen tokens; then one launch sorts the pairs with their pass list
+            prof_set_stage(ST_SHARED_GATEUP);
+            const uint32_t per = (size_t)16u * m->cfg.hidden * 4u <= 128u * 1024u ? 16u : 8u;      // tokens whose activations fit the launch's LDS
+            for (uint32_t t0 = 0; t0 < ntok; t0 += per) {
+                const uint32_t n = ntok - t0 < per ? ntok - t0 : per;
+                const size_t row = (size_t)t0 * m->cfg.hidden;
+                HIP_OK(launch_router_gemv(T_F32, L.dense_gu, x_dev + row, L.gate_inp, n, m->cfg.hidden, 0u, m->logits + t0, static_cast<uint8_t *>(m->xh) + 2u * row,
+                                          static_cast<uint8_t *>(m->xl) + 2u * row, m->xexp + t0, nullptr, m->act + (size_t)t0 * 2u * m->cfg.ffn, m->cfg.ffn, s, L.dense_gu,
+                                          m->scalar + t0), "shared gate/up launch");
+            }
+            m->shared_gu_ready = true;
+            const GroupJob big{ids_dev, weights_dev, ntok, m->cfg.top_k, m->cfg.n_expert, m->uid, m->expert_start, m->pair_token, m->pair_weight, m->tok_pair, m->n_unique,
+                               m->status, m->pass_list, m->n_pass};
+            prof_set_stage(ST_GROUP);
+            HIP_OK(launch_group_small(big, s), "pair sort launch");
+            grouped = true;
+        } else if (m->mixed && m->packed_gu() && (ntok == 1u || m->small_batch_mixed(ntok)) && L.dense_gu && (nv == 2u || nv == 4u || nv == 8u || nv == 16u)) {
             // one token or a small batch on a mixed layout: the kernels take the shared expert's gate | up products as an input: one f32
             // GEMV over its f32 copy (no router rows), which also leaves the fp16 halves of x and the shared expert's scalar gate
             prof_set_stage(ST_SHARED_GATEUP);

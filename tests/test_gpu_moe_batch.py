@@ -261,6 +261,14 @@ def test_mixed_layout_batches_up_to_32_tokens_behind_the_own_router(layout, shap
         agree = [t for t in range(ntok) if np.array_equal(gids[t], cids[t])]
         assert len(agree) >= ntok - 1
         assert max(rel_l2(got[t], want[t]) for t in agree) <= REL_L2_TOL, (layout, shape, ntok)
+        # the same sizes with the routing given (up to 24 tokens as slices, behind a pair sort launch of its own): few experts, shared by many tokens
+        hot = min(E, 3 * K)
+        ids = np.stack([rng.permutation(hot)[:K] for _ in range(ntok)]).astype(np.uint32)
+        w = rng.random((ntok, K)).astype(np.float32) + 0.05
+        w /= w.sum(axis=1, keepdims=True)
+        got = m.experts(0, torch.from_numpy(x).cuda(), torch.from_numpy(ids.astype(np.int32)).cuda(), torch.from_numpy(w).cuda()).cpu().numpy()
+        want = oracle_tokens(cfg, lay, x, ids, w)
+        assert max(rel_l2(got[t], want[t]) for t in range(ntok)) <= REL_L2_TOL, (layout, shape, ntok, "given")
     m.close()
 
 
