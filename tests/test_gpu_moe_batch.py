@@ -197,7 +197,7 @@ def test_drawn_routing_every_batch_size_class(layout, golden_dir):
     m.close()
 
 
-@pytest.mark.parametrize("shape,sizes", [((2048, 512, 512, 10), (17, 25, 32, 33)), ((1024, 256, 32, 8), (20, 32)), ((512, 256, 64, 16), (31, 32))])
+@pytest.mark.parametrize("shape,sizes", [((2048, 512, 512, 10), (17, 32, 33)), ((1024, 256, 32, 8), (20, 24, 25, 32)), ((512, 256, 64, 16), (31, 32))])
 def test_batches_up_to_32_tokens_behind_the_own_router(shape, sizes):
     """all-IQ2_XXS layers take up to 32 tokens (512 pairs) as one batch of expert slices: through forward() the selection launch sorts the
     pairs and writes the pass list, with the routing given a launch of its own does. Few experts: every expert serves many tokens
@@ -231,7 +231,7 @@ def test_batches_up_to_32_tokens_behind_the_own_router(shape, sizes):
 
 
 @pytest.mark.parametrize("layout", ["f2", "xs", "m"])
-@pytest.mark.parametrize("shape,sizes", [((2048, 512, 512, 10), (9, 17, 25, 32, 33)), ((1024, 256, 32, 8), (16, 31))])
+@pytest.mark.parametrize("shape,sizes", [((2048, 512, 512, 10), (17, 32)), ((1024, 256, 32, 8), (9, 16, 24, 25, 31, 33))])
 def test_mixed_layout_batches_up_to_32_tokens_behind_the_own_router(layout, shape, sizes, golden_dir):
     """the mixed layouts whose small batches run as expert slices take 9..32 tokens through forward() as one batch: the router launch of the
     eight-token batches once per eight tokens, one selection + pair sort launch, slices per pass"""
