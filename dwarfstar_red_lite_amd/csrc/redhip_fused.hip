@@ -10,13 +10,15 @@
 //                          SwiGLU, then the matching 32 columns of its down matrix (column-sliced copy), weighted -> a partial
 //                          output vector per workgroup
 //   slice_sum_kernel       the (top_k + 1) * ffn / 32 partial vectors added in a fixed order: deterministic
-//   mixed layouts:
+//   mixed layouts whose batches run as slices (IQ2_XXS gate / up with IQ3_S down, all IQ2_XS, all IQ1_M): the same two kernels, the
+//   down slices from the column-sliced words / streams, the shared expert from dense f32 copies (its gate / up products by the router launch)
+//   other mixed layouts:
 //   gateup_select_kernel   the same selection, then 32 gate rows + 32 up rows of one selected expert -> SwiGLU -> fp16 halves
 //   down_combine_*_kernel  8 output rows per workgroup, one wave per selected expert; weighted sum in selection order + shared
 //                          expert * scalar gate (word-packed IQ3_S / stream-packed IQ2_XS, IQ1_M on the MFMA, other types raw rows)
-// Two to eight tokens: pairs grouped by expert (group_small, in the first launch or with the selection in one of its own), then
-// batch_slice_kernel + slice_sum_kernel (all IQ2_XXS: a pass = two tokens of one expert) or gateup_batch_kernel + down_batch_*_kernel
-// (mixed layouts: persistent workgroups, every distinct expert read once).
+// Small batches (two to 32 tokens behind the layer's own router, fewer with a caller's routing): pairs grouped by expert (group_small, in
+// the first launch, with the selection in one of its own, or alone), then batch_slice_kernel + slice_sum_kernel (a pass = two tokens of one
+// expert), or gateup_batch_kernel + down_batch_*_kernel (the other mixed layouts: persistent workgroups, every distinct expert read once).
 //
 // Arithmetic: a weight is (sign * magnitude * (2*scale+1)) * d/8; the eight magnitudes of a grid entry are exact fp16
 // values from an LDS table, the sign bits are placed by integer arithmetic; an activation vector is split into two
@@ -1559,8 +1561,10 @@ __device__ __forceinline__ void iq3s_group_dot(uint4 q, const half4_t *ax, const
     vb = (acc[2] + acc[3] * 4.8828125e-4f) * sc;
 }
 
-// ---------------------------------------------------------------- one token on all-IQ2_XXS layers: expert slices
+// ---------------------------------------------------------------- one token: expert slices
 //
+// (Described for all-IQ2_XXS layers; MIX = 1 / 2 / 3 reads the down slices of IQ3_S words or IQ2_XS / IQ1_M streams and takes the shared
+// expert from dense f32 copies, SLOTS takes the experts from the slots of a pool - see SliceArgs.)
 // One workgroup per (slot, 32 ffn columns): it selects (or takes the caller's routing), multiplies its 32 gate rows and 32 up rows
 // of the slot's expert, applies SwiGLU, keeps the 32 activations in LDS and multiplies them straight away with the matching 32
 // columns of the expert's down matrix - all `hidden` rows - weighted by the slot's router weight. Gate / up and down weights are
